@@ -1,0 +1,471 @@
+"""TEST INFRASTRUCTURE — numpy/ctypes bindings for the two CPU checkers.
+
+* ``Oracle``  → oracle/libdloracle.so, this repository's CPU restatement of the
+  reference's FC / batch-(re)norm / activation leaves (oracle/dl_oracle.c).
+* ``Reference`` → oracle/_ref/libdlref.so, the real reference sources compiled by
+  oracle/Makefile.ref (only present where that build was run; the sources do
+  not travel).
+
+Both expose the same leaf interface so a test can be parametrized over them.
+Only tests/, ``__graft_entry__.smoke()`` and ``bench.py``'s cpu_baseline leg may
+import this module; the product (deep-learning_amd/) never does.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+ORACLE_SO = os.path.join(_HERE, "libdloracle.so")
+REF_SO = os.path.join(_HERE, "_ref", "libdlref.so")
+
+c_sz = ctypes.c_size_t
+c_int = ctypes.c_int
+c_f = ctypes.c_float
+c_d = ctypes.c_double
+vp = ctypes.c_void_p
+
+# ACTIVATION / LAYER_NORM / LAYER_DROPOUT / PROPAGATION values of the reference
+# (v1/data/enum/activation.hpp:24-53, layer_norm.hpp:24-26,
+#  layer_dropout.hpp:24-28, propagation.hpp)
+ACT = dict(ELU=3, ISRLU=10, LINEAR=11, LEAKY_RELU=14, RELU=16, SELU=17, SOFTMAX=22)
+NORM = dict(NONE=0, BN=1, BRN=2)
+DROP = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3)
+STATE = dict(INFERENCE=0, TRAINING=1, UPDATE_BATCH_NORM=2)
+
+
+def build_oracle():
+    subprocess.run(["make", "-C", _HERE], check=True, stdout=subprocess.DEVNULL)
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(vp)
+
+
+class _Leaves:
+    """Shared leaf-level wrappers.  ``self._f(name)`` resolves a C symbol,
+    ``self.dtype`` is the numpy element type the library works in."""
+
+    dtype = np.float32
+
+    def _a(self, x, copy=False):
+        if x is None:
+            return None
+        a = np.ascontiguousarray(x, dtype=self.dtype)
+        return a.copy() if copy and a is x else a
+
+    def _real(self, v):
+        return c_f(v) if self.dtype == np.float32 else c_d(v)
+
+    def fc_fwd(self, X, W, nthreads=0):
+        X, W = self._a(X), self._a(W)
+        B, K = X.shape
+        H = W.shape[0]
+        Z = np.empty((B, H), self.dtype)
+        self._f("fc_fwd")(c_int(nthreads), c_sz(B), c_sz(K), c_sz(H), _ptr(X), _ptr(W), _ptr(Z))
+        return Z
+
+    def bias_fwd(self, Z, bias, nthreads=0):
+        Z = np.array(Z, dtype=self.dtype, order="C", copy=True)
+        bias = self._a(bias)
+        B, H = Z.shape
+        self._f("bias_fwd")(c_int(nthreads), c_sz(B), c_sz(H), _ptr(bias), _ptr(Z))
+        return Z
+
+    def norm_fwd_train(self, x, gamma, beta, mov_mean, mov_std, momentum, eps,
+                       r_max=1.0, d_max=0.0, renorm=True, nthreads=0):
+        """Returns dict(mean, std, mov_mean, mov_std, r, d, xhat, out)."""
+        x, gamma, beta = self._a(x), self._a(gamma), self._a(beta)
+        B, H = x.shape
+        mm = np.array(mov_mean, dtype=self.dtype, copy=True)
+        ms = np.array(mov_std, dtype=self.dtype, copy=True)
+        mean = np.empty(H, self.dtype)
+        std = np.empty(H, self.dtype)
+        r = np.ones(H, self.dtype)
+        d = np.zeros(H, self.dtype)
+        xhat = np.empty((B, H), self.dtype)
+        out = np.empty((B, H), self.dtype)
+        self._f("norm_fwd_train")(
+            c_int(nthreads), c_int(1 if renorm else 0), c_sz(B), c_sz(H),
+            self._real(momentum), self._real(eps), self._real(r_max), self._real(d_max),
+            _ptr(x), _ptr(gamma), _ptr(beta), _ptr(mean), _ptr(std), _ptr(mm), _ptr(ms),
+            _ptr(r), _ptr(d), _ptr(xhat), _ptr(out))
+        return dict(mean=mean, std=std, mov_mean=mm, mov_std=ms, r=r, d=d, xhat=xhat, out=out)
+
+    def norm_fwd_infer(self, x, gamma, beta, mov_mean, mov_std, nthreads=0):
+        x = self._a(x)
+        B, H = x.shape
+        out = np.empty((B, H), self.dtype)
+        self._f("norm_fwd_infer")(c_int(nthreads), c_sz(B), c_sz(H), _ptr(x), _ptr(self._a(gamma)),
+                                  _ptr(self._a(beta)), _ptr(self._a(mov_mean)), _ptr(self._a(mov_std)),
+                                  _ptr(out))
+        return out
+
+    def act_fwd(self, act, x, nthreads=0):
+        x = self._a(x)
+        B, H = x.shape
+        y = np.empty((B, H), self.dtype)
+        self._f("act_fwd")(c_int(nthreads), c_int(act), c_sz(B), c_sz(H), _ptr(x), _ptr(y))
+        return y
+
+    def softmax_fwd(self, x, nthreads=0):
+        x = self._a(x)
+        B, H = x.shape
+        y = np.empty((B, H), self.dtype)
+        self._f("softmax_fwd")(c_int(nthreads), c_sz(B), c_sz(H), _ptr(x), _ptr(y))
+        return y
+
+    def identity_add(self, a, b, nthreads=0):
+        a, b = self._a(a), self._a(b)
+        B, H = a.shape
+        out = np.empty((B, H), self.dtype)
+        self._f("identity_add")(c_int(nthreads), c_sz(B), c_sz(H), _ptr(a), _ptr(b), _ptr(out))
+        return out
+
+    def fc_bwd_dx(self, dZn, Wn, dY_init=None, nthreads=0):
+        dZn, Wn = self._a(dZn), self._a(Wn)
+        B, Hn = dZn.shape
+        H = Wn.shape[1]
+        dY = (np.zeros((B, H), self.dtype) if dY_init is None
+              else np.array(dY_init, dtype=self.dtype, order="C", copy=True))
+        self._f("fc_bwd_dx")(c_int(nthreads), c_sz(B), c_sz(Hn), c_sz(H), _ptr(dZn), _ptr(Wn), _ptr(dY))
+        return dY
+
+    def act_bwd(self, act, pre, post, dY, nthreads=0):
+        pre, post, dY = self._a(pre), self._a(post), self._a(dY)
+        B, H = pre.shape
+        dN = np.empty((B, H), self.dtype)
+        self._f("act_bwd")(c_int(nthreads), c_int(act), c_sz(B), c_sz(H), _ptr(pre), _ptr(post),
+                           _ptr(dY), _ptr(dN))
+        return dN
+
+    def norm_bwd(self, mean, std, gamma, r, x, xhat, dN, dgamma_init=None, dbeta_init=None,
+                 renorm=True, nthreads=0):
+        """Returns dict(dgamma, dbeta, dmean, dstd, dx)."""
+        x, xhat, dN = self._a(x), self._a(xhat), self._a(dN)
+        B, H = x.shape
+        dg = (np.zeros(H, self.dtype) if dgamma_init is None
+              else np.array(dgamma_init, dtype=self.dtype, copy=True))
+        db = (np.zeros(H, self.dtype) if dbeta_init is None
+              else np.array(dbeta_init, dtype=self.dtype, copy=True))
+        dmean = np.empty(H, self.dtype)
+        dstd = np.empty(H, self.dtype)
+        dx = np.empty((B, H), self.dtype)
+        r = np.ones(H, self.dtype) if r is None else self._a(r)
+        self._f("norm_bwd")(c_int(nthreads), c_int(1 if renorm else 0), c_sz(B), c_sz(H),
+                            _ptr(self._a(mean)), _ptr(self._a(std)), _ptr(self._a(gamma)), _ptr(r),
+                            _ptr(x), _ptr(xhat), _ptr(dN), _ptr(dg), _ptr(db), _ptr(dmean),
+                            _ptr(dstd), _ptr(dx))
+        return dict(dgamma=dg, dbeta=db, dmean=dmean, dstd=dstd, dx=dx)
+
+    def fc_bwd_dw(self, Xin, dZ, dW_init=None, db_init=None, with_bias=True, nthreads=0):
+        Xin, dZ = self._a(Xin), self._a(dZ)
+        B, K = Xin.shape
+        H = dZ.shape[1]
+        dW = (np.zeros((H, K), self.dtype) if dW_init is None
+              else np.array(dW_init, dtype=self.dtype, order="C", copy=True))
+        db = None
+        if with_bias:
+            db = (np.zeros(H, self.dtype) if db_init is None
+                  else np.array(db_init, dtype=self.dtype, copy=True))
+        self._f("fc_bwd_dw")(c_int(nthreads), c_sz(B), c_sz(K), c_sz(H), _ptr(Xin), _ptr(dZ),
+                             _ptr(dW), _ptr(db))
+        return dW, db
+
+
+class Oracle(_Leaves):
+    """The restatement; ``Oracle(np.float64)`` selects the double arbiter."""
+
+    def __init__(self, dtype=np.float32):
+        if not os.path.exists(ORACLE_SO):
+            build_oracle()
+        self.lib = ctypes.CDLL(ORACLE_SO)
+        self.dtype = np.dtype(dtype).type
+        self.suffix = "_f32" if self.dtype == np.float32 else "_f64"
+        self.lib.dlo_max_threads.restype = c_int
+        self.lib.dlo_mlp_create.restype = vp
+        for n in ("parameters", "dparameters", "moving_mean", "moving_std"):
+            getattr(self.lib, "dlo_mlp_" + n).restype = ctypes.POINTER(c_f)
+        self.lib.dlo_mlp_layer_buffer.restype = ctypes.POINTER(c_f)
+        self.lib.dlo_mlp_layer_vector.restype = ctypes.POINTER(c_f)
+        self.lib.dlo_mlp_total_parameters.restype = c_sz
+        self.lib.dlo_mlp_total_units.restype = c_sz
+        self.lib.dlo_mlp_loss_sum.restype = c_d
+        self.lib.dlo_mlp_n_correct.restype = c_d
+
+    name = "oracle"
+
+    def max_threads(self):
+        return self.lib.dlo_max_threads()
+
+    def _f(self, leaf):
+        fn = getattr(self.lib, "dlo_" + leaf + self.suffix)
+        fn.restype = None
+        return fn
+
+    def dropout_fwd(self, kind, v, mask, scale_or_keep, nthreads=0):
+        """kind 0 inverted, 1 plain, 2 inference.  mask [H] (reference semantics,
+        one value per unit) or [B,H] (per element) uint8."""
+        v = np.array(v, dtype=self.dtype, order="C", copy=True)
+        B, H = v.shape
+        per_element = 0
+        m = None
+        if mask is not None:
+            m = np.ascontiguousarray(mask, dtype=np.uint8)
+            per_element = 1 if m.ndim == 2 else 0
+        self._f("dropout_fwd")(c_int(nthreads), c_int(kind), c_int(per_element), c_sz(B), c_sz(H),
+                               _ptr(m), self._real(scale_or_keep), _ptr(v))
+        return v
+
+    def softmax_ce_seed(self, q, y, nthreads=0):
+        """Returns (dZ, loss_sum, n_correct)."""
+        q, y = self._a(q), self._a(y)
+        B, H = q.shape
+        dZ = np.empty((B, H), self.dtype)
+        loss = c_d(0.0)
+        corr = c_d(0.0)
+        self._f("softmax_ce_seed")(c_int(nthreads), c_sz(B), c_sz(H), _ptr(q), _ptr(y), _ptr(dZ),
+                                   ctypes.byref(loss), ctypes.byref(corr))
+        return dZ, loss.value, corr.value
+
+    def mlp(self, widths):
+        return OracleMLP(self, widths)
+
+
+class OracleMLP:
+    """Whole-model restatement (float only): dispatcher order + packed
+    parameter layout of the reference."""
+
+    def __init__(self, oracle, widths):
+        self.o = oracle
+        self.lib = oracle.lib
+        self.widths = [int(w) for w in widths]
+        arr = (c_sz * len(widths))(*self.widths)
+        self.h = vp(self.lib.dlo_mlp_create(c_sz(len(widths)), arr))
+        self.P = self.lib.dlo_mlp_total_parameters(self.h)
+        self.n_units = self.lib.dlo_mlp_total_units(self.h)
+        self.max_batch = 0
+
+    def __del__(self):
+        try:
+            self.lib.dlo_mlp_destroy(self.h)
+        except Exception:
+            pass
+
+    def set_layer(self, l, act, norm=0, drop=0, keep=1.0, mask=None):
+        m = None if mask is None else np.ascontiguousarray(mask, dtype=np.uint8)
+        self.lib.dlo_mlp_set_layer(self.h, c_sz(l), c_int(act), c_int(norm), c_int(drop), c_f(keep), _ptr(m))
+
+    def set_norm_hyper(self, momentum, eps, r_max, d_max):
+        self.lib.dlo_mlp_set_norm_hyper(self.h, c_f(momentum), c_f(eps), c_f(r_max), c_f(d_max))
+
+    def layer_offsets(self, l):
+        out = (c_sz * 6)()
+        self.lib.dlo_mlp_layer_offsets(self.h, c_sz(l), out)
+        return list(out)
+
+    def prepare(self, max_batch, nthreads=0):
+        self.max_batch = max_batch
+        self.nthreads = nthreads
+        self.lib.dlo_mlp_prepare(self.h, c_sz(max_batch))
+
+    def _view(self, fn, n):
+        return np.ctypeslib.as_array(fn(self.h), shape=(n,))
+
+    @property
+    def parameters(self):
+        return self._view(self.lib.dlo_mlp_parameters, self.P)
+
+    @property
+    def dparameters(self):
+        return self._view(self.lib.dlo_mlp_dparameters, self.P)
+
+    @property
+    def moving_mean(self):
+        return self._view(self.lib.dlo_mlp_moving_mean, self.n_units)
+
+    @property
+    def moving_std(self):
+        return self._view(self.lib.dlo_mlp_moving_std, self.n_units)
+
+    def step(self, state, X, Y=None, backward=True):
+        X = np.ascontiguousarray(X, np.float32)
+        B = X.shape[0]
+        self.B = B
+        self.lib.dlo_mlp_forward(self.h, c_int(self.nthreads), c_int(state), c_sz(B), _ptr(X))
+        if backward:
+            Y = np.ascontiguousarray(Y, np.float32)
+            self.lib.dlo_mlp_backward(self.h, c_int(self.nthreads), c_sz(B), _ptr(Y))
+
+    def layer_buffer(self, l, which):
+        p = self.lib.dlo_mlp_layer_buffer(self.h, c_sz(l), c_int(which))
+        return np.ctypeslib.as_array(p, shape=(self.max_batch, self.widths[l]))[: self.B].copy()
+
+    def layer_vector(self, l, which):
+        p = self.lib.dlo_mlp_layer_vector(self.h, c_sz(l), c_int(which))
+        return np.ctypeslib.as_array(p, shape=(self.widths[l],)).copy()
+
+    def get_dparams(self):
+        return self.dparameters.copy()
+
+    def get_moving(self):
+        return self.moving_mean.copy(), self.moving_std.copy()
+
+
+def reference_available():
+    return os.path.exists(REF_SO)
+
+
+class Reference(_Leaves):
+    """The real reference sources, compiled.  The shared object leaves the
+    reference's console / file-IO symbols undefined (their translation units
+    need Boost / systemd and are not on this path), so it must be opened with
+    lazy binding; ctypes.CDLL alone forces RTLD_NOW."""
+
+    name = "reference"
+
+    def __init__(self):
+        if not reference_available():
+            raise FileNotFoundError(REF_SO)
+        dl = ctypes.CDLL(None)
+        dl.dlopen.restype = vp
+        dl.dlopen.argtypes = [ctypes.c_char_p, c_int]
+        handle = dl.dlopen(REF_SO.encode(), os.RTLD_LAZY | os.RTLD_LOCAL)
+        if not handle:
+            raise OSError("dlopen failed for " + REF_SO)
+        self.lib = ctypes.CDLL(REF_SO, handle=handle)
+        self.lib.dlref_init()
+        self.lib.dlref_max_threads.restype = c_int
+        self.lib.dlref_model_create.restype = vp
+        for n in ("number_threads", "total_parameters", "total_norm_units"):
+            getattr(self.lib, "dlref_model_" + n).restype = c_sz
+
+    def max_threads(self):
+        return self.lib.dlref_max_threads()
+
+    def _f(self, leaf):
+        fn = getattr(self.lib, "dlref_" + leaf)
+        fn.restype = None
+        return fn
+
+    def dropout_fwd(self, kind, v, mask, scale_or_keep, nthreads=0):
+        v = np.array(v, dtype=np.float32, order="C", copy=True)
+        B, H = v.shape
+        m = None if mask is None else np.ascontiguousarray(mask, dtype=np.uint8)
+        assert m is None or m.ndim == 1, "the reference's mask is per unit"
+        self._f("dropout_fwd")(c_int(nthreads), c_int(kind), c_sz(B), c_sz(H), _ptr(m),
+                               c_f(scale_or_keep), _ptr(v))
+        return v
+
+    def mlp(self, widths, allowable_bytes=1 << 32):
+        return ReferenceMLP(self, widths, allowable_bytes)
+
+
+class ReferenceMLP:
+    """A real DL::v1::Model built through compile() and the public setters."""
+
+    def __init__(self, ref, widths, allowable_bytes):
+        self.lib = ref.lib
+        self.widths = [int(w) for w in widths]
+        arr = (c_sz * len(widths))(*self.widths)
+        h = self.lib.dlref_model_create(c_sz(len(widths)), arr, c_sz(allowable_bytes))
+        if not h:
+            raise RuntimeError("reference Model::compile failed")
+        self.h = vp(h)
+        self.P = self.lib.dlref_model_total_parameters(self.h)
+        self.n_units = self.lib.dlref_model_total_norm_units(self.h)
+        self._hyper = None
+
+    def __del__(self):
+        try:
+            self.lib.dlref_model_destroy(self.h)
+        except Exception:
+            pass
+
+    def set_layer(self, l, act, norm=0, drop=0, keep=1.0, mask=None):
+        ok = self.lib.dlref_model_set_activation(self.h, c_sz(l), c_int(act))
+        assert ok, "set_layer_activation_function refused"
+        if norm:
+            ok = self.lib.dlref_model_set_normalization(self.h, c_sz(l), c_int(norm))
+            assert ok, "Set__Layer_Normalization refused"
+        if drop:
+            ok = self.lib.dlref_model_set_dropout(self.h, c_sz(l), c_int(drop), c_f(keep))
+            assert ok, "set_dropout refused"
+        self._masks = getattr(self, "_masks", {})
+        if mask is not None:
+            self._masks[l] = np.ascontiguousarray(mask, dtype=np.uint8)
+
+    def set_norm_hyper(self, momentum, eps, r_max, d_max):
+        ok = self.lib.dlref_model_set_norm_hyper(self.h, c_f(momentum), c_f(eps), c_f(r_max), c_f(d_max))
+        assert ok
+
+    def layer_offsets(self, l):
+        out = (c_sz * 6)()
+        self.lib.dlref_model_layer_offsets(self.h, c_sz(l), out)
+        return list(out)
+
+    def prepare(self, max_batch, nthreads=0):
+        self.max_batch = max_batch
+        ok = self.lib.dlref_model_prepare(self.h, c_sz(max_batch), c_int(nthreads))
+        assert ok, "reference prepare failed"
+        for l, m in getattr(self, "_masks", {}).items():
+            ok = self.lib.dlref_model_set_dropout_mask(self.h, c_sz(l), c_sz(self.widths[l]), _ptr(m))
+            assert ok
+        self.lib.dlref_model_zero_dparams(self.h)
+        # the normalization parameters are only allocated once a layer asks for them
+        self.P = self.lib.dlref_model_total_parameters(self.h)
+        self.n_units = self.lib.dlref_model_total_norm_units(self.h)
+
+    def number_threads(self):
+        return self.lib.dlref_model_number_threads(self.h)
+
+    def set_parameters(self, p):
+        p = np.ascontiguousarray(p, np.float32)
+        assert p.size == self.P
+        self.lib.dlref_model_set_parameters(self.h, _ptr(p), c_sz(self.P))
+
+    def get_parameters(self):
+        p = np.empty(self.P, np.float32)
+        self.lib.dlref_model_get_parameters(self.h, _ptr(p), c_sz(self.P))
+        return p
+
+    def set_moving(self, mean, std):
+        mean = np.ascontiguousarray(mean, np.float32)
+        std = np.ascontiguousarray(std, np.float32)
+        self.lib.dlref_model_set_moving(self.h, _ptr(mean), _ptr(std), c_sz(self.n_units))
+
+    def get_moving(self):
+        mean = np.empty(self.n_units, np.float32)
+        std = np.empty(self.n_units, np.float32)
+        self.lib.dlref_model_get_moving(self.h, _ptr(mean), _ptr(std), c_sz(self.n_units))
+        return mean, std
+
+    def step(self, state, X, Y=None, backward=True):
+        X = np.ascontiguousarray(X, np.float32)
+        B, K0 = X.shape
+        self.B = B
+        Yp, Hout = None, self.widths[-1]
+        if backward:
+            Y = np.ascontiguousarray(Y, np.float32)
+            Yp = _ptr(Y)
+        self.lib.dlref_model_step(self.h, c_int(state), c_sz(B), _ptr(X), c_sz(K0), Yp, c_sz(Hout),
+                                  c_int(1 if backward else 0))
+
+    def layer_buffer(self, l, which):
+        out = np.empty((self.max_batch, self.widths[l]), np.float32)
+        ok = self.lib.dlref_model_get_layer_buffer(self.h, c_sz(l), c_int(which), c_sz(self.max_batch),
+                                                   _ptr(out))
+        assert ok
+        return out[: self.B].copy()
+
+    def layer_vector(self, l, which):
+        out = np.empty(self.widths[l], np.float32)
+        ok = self.lib.dlref_model_get_layer_vector(self.h, c_sz(l), c_int(which), _ptr(out))
+        assert ok
+        return out
+
+    def get_dparams(self):
+        p = np.empty(self.P, np.float32)
+        self.lib.dlref_model_get_dparams(self.h, _ptr(p), c_sz(self.P))
+        return p

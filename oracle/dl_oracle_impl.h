@@ -1,0 +1,468 @@
+/* TEST INFRASTRUCTURE — not part of the product.  Included twice by
+ * dl_oracle.c, once with REAL=float (the reference's Release `real`) and once
+ * with REAL=double (the arbiter for tolerance disputes).
+ *
+ * Every function restates one leaf of the reference's CPU path with the same
+ * loop order, the same accumulators and the same per-thread partial buffers.
+ * `nthreads == 0` follows the `*__Loop` (single-thread) leaf, `nthreads >= 1`
+ * the `*__OpenMP` leaf run by `nthreads` threads.  All file:line citations are
+ * relative to /root/reference/lib/deep-learning/.
+ *
+ * Layout everywhere: row-major [B, H], element (b, j) at b*H + j
+ * (v1/learner/fwp_st.cpp:4538-4542).
+ */
+
+/* ---- activations: v1/ops/activations/functions.hpp:82-108, 124-220 -------- */
+static inline REAL FN(af_fire)(int type, REAL x) {
+  switch (type) {
+    case DLO_ACT_ISRLU: /* functions.hpp:86-87, slope 1 (:196) */
+      return x < (REAL)0 ? x * ((REAL)1 / SQRT((REAL)1 + (REAL)1 * x * x)) : x;
+    case DLO_ACT_ELU: /* functions.hpp:91, slope 1 (:199) */
+      return x < (REAL)0 ? (REAL)1 * (EXP(x) - (REAL)1) : x;
+    case DLO_ACT_SELU: /* functions.hpp:95-98 */
+      return SELU_SCALE * (x <= (REAL)0 ? SELU_ALPHA * EXP(x) - SELU_ALPHA : x);
+    case DLO_ACT_RELU: /* functions.hpp:102 */
+      return x < (REAL)0 ? (REAL)0 : x;
+    case DLO_ACT_LEAKY_RELU: /* functions.hpp:106-108, slope 0.01 */
+      return x < (REAL)0 ? LRELU_ALPHA * x : x;
+    case DLO_ACT_LINEAR: /* functions.hpp AF_LINEAR_real: identity */
+      return x;
+    default:
+      return x;
+  }
+}
+
+/* v1/learner/model.cpp:2594-2651 with the macros of functions.hpp:88,92,99,
+ * 103,107: x = pre-activation, q = stored post-activation value. */
+static inline REAL FN(af_derive)(int type, REAL x, REAL q) {
+  switch (type) {
+    case DLO_ACT_ISRLU:
+      return x < (REAL)0 ? POW(q / x, (REAL)3) : (REAL)1;
+    case DLO_ACT_ELU:
+      return x < (REAL)0 ? (REAL)1 * q : (REAL)1;
+    case DLO_ACT_SELU:
+      return SELU_SCALE * (x <= (REAL)0 ? (q + SELU_ALPHA) : (REAL)1);
+    case DLO_ACT_RELU:
+      return x < (REAL)0 ? (REAL)0 : (REAL)1;
+    case DLO_ACT_LEAKY_RELU:
+      return x < (REAL)0 ? LRELU_ALPHA : (REAL)1;
+    case DLO_ACT_LINEAR:
+      return (REAL)1;
+    default:
+      return q;
+  }
+}
+
+/* ops/math.hpp:56-59 */
+static inline REAL FN(clip)(REAL v, REAL lo, REAL hi) {
+  return v < lo ? lo : (v > hi ? hi : v);
+}
+
+static inline int FN(nthr)(int nthreads, size_t B) {
+  /* v1/learner/update_size.cpp:76 — threads never exceed the batch size. */
+  if (nthreads <= 0) return 0;
+  return (size_t)nthreads > B ? (int)B : nthreads;
+}
+
+/* ---- a7  FC forward: fwp_st.cpp:4518-4555, fwp_mp.cpp:4419-4459 ----------- */
+void FN(dlo_fc_fwd)(int nthreads, size_t B, size_t K, size_t H, REAL const *X,
+                    REAL const *W, REAL *Z) {
+  int const N = FN(nthr)(nthreads, B);
+  int const Bi = (int)B;
+  int b;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (b = 0; b < Bi; ++b) {
+    REAL const *x = X + (size_t)b * K;
+    REAL const *w = W;
+    REAL *z = Z + (size_t)b * H;
+    for (size_t h = 0; h != H; ++h, w += K) {
+      REAL s = (REAL)0;
+      for (size_t k = 0; k != K; ++k) s += x[k] * w[k];
+      z[h] = s;
+    }
+  }
+}
+
+/* ---- a8  bias: fwp_st.cpp:4498-4516, fwp_mp.cpp:4396-4417 ----------------- */
+void FN(dlo_bias_fwd)(int nthreads, size_t B, size_t H, REAL const *bias,
+                      REAL *Z) {
+  int const N = FN(nthr)(nthreads, B);
+  int const Bi = (int)B;
+  int b;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (b = 0; b < Bi; ++b) {
+    REAL *z = Z + (size_t)b * H;
+    for (size_t h = 0; h != H; ++h) z[h] += bias[h];
+  }
+}
+
+/* ---- a9/a10  batch (re)normalization, training ----------------------------
+ * fwp_st.cpp:4586-4663 (BN), :4665-4766 (BRN); fwp_mp.cpp:4493-4603, 4605-4739.
+ * The "variance" arrays hold the standard deviation; the moving averages are
+ * updated BEFORE r and d are formed from them.  BN is BRN with r=1, d=0 and
+ * the shorter x_hat expression. */
+void FN(dlo_norm_fwd_train)(int nthreads, int renorm, size_t B, size_t H,
+                            REAL momentum, REAL eps, REAL r_max, REAL d_max,
+                            REAL const *x, REAL const *gamma, REAL const *beta,
+                            REAL *mean, REAL *stdv, REAL *mov_mean,
+                            REAL *mov_std, REAL *r, REAL *d, REAL *xhat,
+                            REAL *out) {
+  int const N = FN(nthr)(nthreads, B);
+  int const NT = N > 0 ? N : 1;
+  int const Bi = (int)B, Hi = (int)H;
+  REAL const batch_scale = (REAL)1 / (REAL)B;
+  REAL *means = (REAL *)calloc((size_t)NT * H, sizeof(REAL));
+  REAL *vars = (REAL *)calloc((size_t)NT * H, sizeof(REAL));
+
+#pragma omp parallel num_threads(NT) if (N > 0)
+  {
+    int b, j;
+    /* Summation (per-thread slices: fwp_mp.cpp:4651-4662). */
+#pragma omp for schedule(static)
+    for (b = 0; b < Bi; ++b) {
+      size_t const row = (size_t)b * H;
+      size_t const slice = (size_t)(N > 0 ? omp_get_thread_num() : 0) * H;
+      for (size_t i = 0; i != H; ++i) {
+        REAL const s = x[row + i];
+        means[slice + i] += s;
+        vars[slice + i] += s * s;
+      }
+    }
+    /* Average (fwp_mp.cpp:4666-4718; fwp_st.cpp:4709-4746). */
+#pragma omp for schedule(static)
+    for (j = 0; j < Hi; ++j) {
+      REAL rm = (REAL)0, rv = (REAL)0;
+      for (int t = 1; t < NT; ++t) {
+        rm += means[(size_t)t * H + j];
+        rv += vars[(size_t)t * H + j];
+      }
+      if (NT > 1) {
+        means[j] += rm;
+        vars[j] += rv;
+      }
+      means[j] *= batch_scale;
+      mov_mean[j] += momentum * (means[j] - mov_mean[j]);
+      vars[j] = SQRT(vars[j] * batch_scale - means[j] * means[j] + eps);
+      mov_std[j] += momentum * (vars[j] - mov_std[j]);
+      if (renorm) {
+        REAL const g = vars[j] / mov_std[j];
+        REAL const lo = (REAL)1 / r_max;
+        r[j] = FN(clip)(g, lo, r_max);
+        REAL const dd = (means[j] - mov_mean[j]) / mov_std[j];
+        d[j] = FN(clip)(dd, -d_max, d_max);
+      }
+    }
+    /* Normalize, scale and shift. */
+#pragma omp for schedule(static)
+    for (b = 0; b < Bi; ++b) {
+      size_t const row = (size_t)b * H;
+      for (size_t i = 0; i != H; ++i) {
+        REAL s = x[row + i];
+        if (renorm)
+          s = (s - means[i]) / vars[i] * r[i] + d[i];
+        else
+          s = (s - means[i]) / vars[i];
+        xhat[row + i] = s;
+        out[row + i] = gamma[i] * s + beta[i];
+      }
+    }
+  }
+  memcpy(mean, means, H * sizeof(REAL));
+  memcpy(stdv, vars, H * sizeof(REAL));
+  free(means);
+  free(vars);
+}
+
+/* ---- a11  inference: fwp_st.cpp:4557-4584, fwp_mp.cpp:4461-4491 ----------- *
+ * Divides by the moving standard deviation, no epsilon.                       */
+void FN(dlo_norm_fwd_infer)(int nthreads, size_t B, size_t H, REAL const *x,
+                            REAL const *gamma, REAL const *beta,
+                            REAL const *mov_mean, REAL const *mov_std,
+                            REAL *out) {
+  int const N = FN(nthr)(nthreads, B);
+  int const Bi = (int)B;
+  int b;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (b = 0; b < Bi; ++b) {
+    size_t const row = (size_t)b * H;
+    for (size_t i = 0; i != H; ++i)
+      out[row + i] = gamma[i] * ((x[row + i] - mov_mean[i]) / mov_std[i]) + beta[i];
+  }
+}
+
+/* ---- a12  activation forward: fwp_st.cpp:4768-4794, fwp_mp.cpp:4741-4770 -- */
+void FN(dlo_act_fwd)(int nthreads, int type, size_t B, size_t H, REAL const *x,
+                     REAL *y) {
+  int const N = FN(nthr)(nthreads, B);
+  int const Bi = (int)B;
+  int b;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (b = 0; b < Bi; ++b) {
+    size_t const row = (size_t)b * H;
+    for (size_t i = 0; i != H; ++i) y[row + i] = FN(af_fire)(type, x[row + i]);
+  }
+}
+
+/* ---- a13  softmax: fwp_st.cpp:4796-4828 ----------------------------------- */
+void FN(dlo_softmax_fwd)(int nthreads, size_t B, size_t H, REAL const *x,
+                         REAL *y) {
+  int const N = FN(nthr)(nthreads, B);
+  int const Bi = (int)B;
+  int b;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (b = 0; b < Bi; ++b) {
+    REAL const *xi = x + (size_t)b * H;
+    REAL *yi = y + (size_t)b * H;
+    REAL mx = -REAL_MAX, s = (REAL)0;
+    for (size_t i = 0; i != H; ++i) mx = mx > xi[i] ? mx : xi[i];
+    for (size_t i = 0; i != H; ++i) s += yi[i] = EXP(xi[i] - mx);
+    s = (REAL)1 / s;
+    for (size_t i = 0; i != H; ++i) yi[i] *= s;
+  }
+}
+
+/* ---- a14  dropout: fwp_st.cpp:4830-4904 -----------------------------------
+ * kind 0: Bernoulli inverted (mask ? v*scale : 0), 1: Bernoulli (mask ? v : 0),
+ * 2: Bernoulli inference (v *= keep).  The reference's mask is one bool per
+ * unit, shared by the batch (per_element == 0).  per_element != 0 is this
+ * build's generalisation to a [B, H] mask; it reduces to the reference when
+ * every row of the mask is the same. */
+void FN(dlo_dropout_fwd)(int nthreads, int kind, int per_element, size_t B,
+                         size_t H, uint8_t const *mask, REAL scale_or_keep,
+                         REAL *v) {
+  int const N = FN(nthr)(nthreads, B);
+  int const Bi = (int)B;
+  int b;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (b = 0; b < Bi; ++b) {
+    REAL *vi = v + (size_t)b * H;
+    uint8_t const *m = mask ? (per_element ? mask + (size_t)b * H : mask) : NULL;
+    for (size_t i = 0; i != H; ++i) {
+      if (kind == 0) {
+        if (m[i]) vi[i] *= scale_or_keep; else vi[i] = (REAL)0;
+      } else if (kind == 1) {
+        if (!m[i]) vi[i] = (REAL)0;
+      } else {
+        vi[i] *= scale_or_keep;
+      }
+    }
+  }
+}
+
+/* ---- a15  identity add, equal widths: fwp_st.cpp:5051-5112 ---------------- */
+void FN(dlo_identity_add)(int nthreads, size_t B, size_t H, REAL const *a,
+                          REAL const *bb, REAL *out) {
+  int const N = FN(nthr)(nthreads, B);
+  int const Bi = (int)B;
+  int b;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (b = 0; b < Bi; ++b) {
+    size_t const row = (size_t)b * H;
+    for (size_t i = 0; i != H; ++i) out[row + i] = a[row + i] + bb[row + i];
+  }
+}
+
+/* ---- a18  dY += dZn * Wn: bwp_st.cpp:1009-1045, bwp_mp.cpp:968-1007 ------- */
+void FN(dlo_fc_bwd_dx)(int nthreads, size_t B, size_t Hn, size_t H,
+                       REAL const *dZn, REAL const *Wn, REAL *dY) {
+  int const N = FN(nthr)(nthreads, B);
+  int const Bi = (int)B;
+  int b;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (b = 0; b < Bi; ++b) {
+    REAL const *dz = dZn + (size_t)b * Hn;
+    REAL const *w = Wn;
+    REAL *dy = dY + (size_t)b * H;
+    for (size_t i = 0; i != Hn; ++i, w += H) {
+      REAL const e = dz[i];
+      for (size_t c = 0; c != H; ++c) dy[c] += e * w[c];
+    }
+  }
+}
+
+/* ---- a19  dN = dY * f'(pre, post): bwp_st.cpp:1177-1209 ------------------- */
+void FN(dlo_act_bwd)(int nthreads, int type, size_t B, size_t H,
+                     REAL const *pre, REAL const *post, REAL const *dY,
+                     REAL *dN) {
+  int const N = FN(nthr)(nthreads, B);
+  int const Bi = (int)B;
+  int b;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (b = 0; b < Bi; ++b) {
+    size_t const row = (size_t)b * H;
+    for (size_t i = 0; i != H; ++i)
+      dN[row + i] = dY[row + i] * FN(af_derive)(type, pre[row + i], post[row + i]);
+  }
+}
+
+/* ---- a20/a21  batch (re)normalization backward ----------------------------
+ * bwp_st.cpp:1284-1366 (BN), :1447-1532 (BRN); bwp_mp.cpp:1265-1385, 1504-1627.
+ * dgamma / dbeta accumulate (+=).  MP: per-thread copies of dgamma/dbeta are
+ * merged like merge.cpp:76-100 (thread 1..N-1 added to thread 0 in order). */
+void FN(dlo_norm_bwd)(int nthreads, int renorm, size_t B, size_t H,
+                      REAL const *mean, REAL const *stdv, REAL const *gamma,
+                      REAL const *r, REAL const *x, REAL const *xhat,
+                      REAL const *dN, REAL *dgamma, REAL *dbeta, REAL *dmean,
+                      REAL *dstd, REAL *dx) {
+  int const N = FN(nthr)(nthreads, B);
+  int const NT = N > 0 ? N : 1;
+  int const Bi = (int)B, Hi = (int)H;
+  REAL const batch_scale = (REAL)1 / (REAL)B;
+  REAL *dg = (REAL *)calloc((size_t)NT * H, sizeof(REAL));
+  REAL *db = (REAL *)calloc((size_t)NT * H, sizeof(REAL));
+  REAL *dm = (REAL *)calloc((size_t)NT * H, sizeof(REAL));
+  REAL *dv = (REAL *)calloc((size_t)NT * H, sizeof(REAL));
+  memcpy(dg, dgamma, H * sizeof(REAL));
+  memcpy(db, dbeta, H * sizeof(REAL));
+
+#pragma omp parallel num_threads(NT) if (N > 0)
+  {
+    int b, j;
+#pragma omp for schedule(static)
+    for (b = 0; b < Bi; ++b) {
+      size_t const row = (size_t)b * H;
+      size_t const slice = (size_t)(N > 0 ? omp_get_thread_num() : 0) * H;
+      for (size_t i = 0; i != H; ++i) {
+        REAL e = dN[row + i];
+        REAL const sd = stdv[i];
+        REAL const neg_r = renorm ? -r[i] : (REAL)-1;
+        dg[slice + i] += e * xhat[row + i];
+        db[slice + i] += e;
+        e *= gamma[i];
+        dm[slice + i] += e * (neg_r / sd);
+        dv[slice + i] += e * (x[row + i] - mean[i]) * (neg_r / (sd * sd));
+        dx[row + i] = e;
+      }
+    }
+#pragma omp for schedule(static)
+    for (j = 0; j < Hi; ++j) {
+      REAL rm = (REAL)0, rv = (REAL)0;
+      for (int t = 1; t < NT; ++t) {
+        rm += dm[(size_t)t * H + j];
+        rv += dv[(size_t)t * H + j];
+      }
+      if (NT > 1) {
+        dm[j] += rm;
+        dv[j] += rv;
+      }
+    }
+#pragma omp for schedule(static)
+    for (b = 0; b < Bi; ++b) {
+      size_t const row = (size_t)b * H;
+      for (size_t i = 0; i != H; ++i) {
+        REAL e = dx[row + i];
+        REAL const sd = stdv[i];
+        if (renorm)
+          e *= r[i] / sd;
+        else
+          e *= (REAL)1 / sd;
+        e += dv[i] * ((x[row + i] - mean[i]) / ((REAL)B * sd));
+        e += dm[i] * batch_scale;
+        dx[row + i] = e;
+      }
+    }
+  }
+  /* merge.cpp:76-100 */
+  for (int t = 1; t < NT; ++t)
+    for (size_t i = 0; i != H; ++i) {
+      dg[i] += dg[(size_t)t * H + i];
+      db[i] += db[(size_t)t * H + i];
+    }
+  memcpy(dgamma, dg, H * sizeof(REAL));
+  memcpy(dbeta, db, H * sizeof(REAL));
+  memcpy(dmean, dm, H * sizeof(REAL));
+  memcpy(dstd, dv, H * sizeof(REAL));
+  free(dg); free(db); free(dm); free(dv);
+}
+
+/* ---- a23  dW += dZ^T Xin, db += sum_b dZ -----------------------------------
+ * update_derivative_fwp_st.cpp:246-302, update_derivative_fwp_mp.cpp:175-240,
+ * merge.cpp:76-100.  db may be NULL (normalized layers have no bias). */
+void FN(dlo_fc_bwd_dw)(int nthreads, size_t B, size_t K, size_t H,
+                       REAL const *Xin, REAL const *dZ, REAL *dW, REAL *db) {
+  int const N = FN(nthr)(nthreads, B);
+  int const NT = N > 0 ? N : 1;
+  int const Bi = (int)B;
+  size_t const P = H * K + H;
+  REAL *dpar = (REAL *)calloc((size_t)NT * P, sizeof(REAL));
+  memcpy(dpar, dW, H * K * sizeof(REAL));
+  if (db) memcpy(dpar + H * K, db, H * sizeof(REAL));
+
+#pragma omp parallel num_threads(NT) if (N > 0)
+  {
+    int b;
+#pragma omp for schedule(static)
+    for (b = 0; b < Bi; ++b) {
+      REAL const *xi = Xin + (size_t)b * K;
+      REAL const *dz = dZ + (size_t)b * H;
+      REAL *dw = dpar + (size_t)(N > 0 ? omp_get_thread_num() : 0) * P;
+      for (size_t h = 0; h != H; ++h, dw += K) {
+        REAL const e = dz[h];
+        for (size_t k = 0; k != K; ++k) dw[k] += e * xi[k];
+      }
+    }
+    if (db) {
+#pragma omp for schedule(static)
+      for (b = 0; b < Bi; ++b) {
+        REAL const *dz = dZ + (size_t)b * H;
+        REAL *dbt = dpar + (size_t)(N > 0 ? omp_get_thread_num() : 0) * P + H * K;
+        for (size_t h = 0; h != H; ++h) dbt[h] += dz[h];
+      }
+    }
+  }
+  for (int t = 1; t < NT; ++t) {
+    REAL const *src = dpar + (size_t)t * P;
+    int i;
+    int const Pi = (int)P;
+#pragma omp parallel for schedule(static) num_threads(NT) if (N > 0)
+    for (i = 0; i < Pi; ++i) dpar[i] += src[i];
+  }
+  memcpy(dW, dpar, H * K * sizeof(REAL));
+  if (db) memcpy(db, dpar + H * K, H * sizeof(REAL));
+  free(dpar);
+}
+
+/* ---- a16  softmax + cross-entropy seed gradient ---------------------------
+ * compute_error_st.cpp:26-131, compute_loss.cpp:101-138 (CROSS_ENTROPY),
+ * loss: compute_loss.cpp:88-95, accuracy: compute_error_st.cpp:55-79.
+ * q [B,H] = softmax output, y [B,H] = targets (one-hot), dZ [B,H] out.
+ * loss_sum / n_correct (doubles) accumulate; either may be NULL. */
+void FN(dlo_softmax_ce_seed)(int nthreads, size_t B, size_t H, REAL const *q,
+                             REAL const *y, REAL *dZ, double *loss_sum,
+                             double *n_correct) {
+  int const N = FN(nthr)(nthreads, B);
+  int const Bi = (int)B;
+  double loss = 0.0, correct = 0.0;
+  int b;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0) \
+    reduction(+ : loss, correct)
+  for (b = 0; b < Bi; ++b) {
+    REAL const *qi = q + (size_t)b * H;
+    REAL const *yi = y + (size_t)b * H;
+    REAL *dz = dZ + (size_t)b * H;
+    size_t k_target = H, k_predict = 0;
+    REAL q_max = -REAL_MAX;
+    for (size_t k = 0; k != H; ++k) {
+      if (qi[k] >= q_max) { k_predict = k; q_max = qi[k]; }
+      if (yi[k] == (REAL)1) k_target = k;
+    }
+    correct += (double)(k_target == k_predict);
+    for (size_t i = 0; i != H; ++i) {
+      REAL const qv = qi[i];
+      /* loss_fn CROSS_ENTROPY */
+      REAL l = FN(clip)(qv, DLO_EPSILON, (REAL)1 - DLO_EPSILON);
+      l = yi[i] == (REAL)1 ? -(yi[i] * LOG(l)) : (REAL)0;
+      loss += (double)l;
+      REAL acc = (REAL)0;
+      for (size_t k = 0; k != H; ++k) {
+        REAL dl = FN(clip)(qi[k], DLO_EPSILON, (REAL)1 - DLO_EPSILON);
+        dl = yi[k] == (REAL)1 ? (REAL)-1 / dl : (REAL)0;
+        dl /= (REAL)B;
+        acc += (qv * (REAL)(i == k) - qi[k] * qv) * dl;
+      }
+      dz[i] = acc;
+    }
+  }
+  if (loss_sum) *loss_sum += loss;
+  if (n_correct) *n_correct += correct;
+}

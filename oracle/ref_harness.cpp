@@ -1,0 +1,574 @@
+// TEST INFRASTRUCTURE — not part of the product.
+//
+// C-ABI driver around the *real* reference sources (compiled in place from
+// /root/reference/lib by oracle/Makefile.ref into oracle/_ref/libdlref.so).
+// It owns no arithmetic of its own: every number it returns is produced by a
+// reference member function of DL::v1::Model.  Used to
+//   * validate the CPU restatement in oracle/dl_oracle.c,
+//   * write the golden vectors under tests/golden/,
+//   * optionally serve as the timed CPU baseline ("reference" kind).
+//
+// `nthreads == 0` selects the reference's single-thread `*__Loop` leaves;
+// `nthreads >= 1` selects the `*__OpenMP` leaves, called by every thread of one
+// enclosing `omp parallel` region exactly as drivers/driver.cpp:241-257 does.
+#include <omp.h>
+
+#include <cstdint>
+#include <cstring>
+#include <vector>
+
+#include "deep-learning/io/logger.hpp"
+#include "deep-learning/v1/learner/model.hpp"
+
+using namespace DL;
+using namespace DL::v1;
+
+namespace {
+Logger *g_logger = nullptr;
+
+// A Model that never went through compile(): only the scalar members the leaf
+// functions read are set.  Leaves take every array as an argument.
+struct LeafModel {
+  Model m;
+  LeafModel(size_t B, int nthreads, size_t P = 0) {
+    m.batch_size = B;
+    m.seq_w = 1;
+    m.number_threads = nthreads > 0 ? static_cast<size_t>(nthreads) : 1;
+    m.total_parameters_allocated = P;
+    m.total_parameters = P;
+  }
+};
+
+inline int clampThreads(int nthreads, size_t B) {
+  // update_size.cpp:76 — never more threads than examples.
+  if (nthreads <= 0) return 0;
+  return static_cast<int>(std::min<size_t>(static_cast<size_t>(nthreads), B));
+}
+}  // namespace
+
+extern "C" {
+
+int dlref_init(void) {
+  if (g_logger == nullptr) g_logger = new Logger(LOGLEVEL::INFO);
+  omp_set_dynamic(0);
+  return 0;
+}
+
+int dlref_max_threads(void) { return omp_get_num_procs(); }
+
+// ---- a7: Z = X * W^T -------------------------------------------------------
+void dlref_fc_fwd(int nthreads, size_t B, size_t K, size_t H, float const *X,
+                  float const *W, float *Z) {
+  nthreads = clampThreads(nthreads, B);
+  LeafModel lm(B, nthreads);
+  if (nthreads == 0) {
+    lm.m.Forward_Pass__FC__Loop(0, B, K, H, X, W, Z);
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    lm.m.Forward_Pass__FC__OpenMP(0, B, K, H, X, W, Z);
+  }
+}
+
+// ---- a8: Z += bias ---------------------------------------------------------
+void dlref_bias_fwd(int nthreads, size_t B, size_t H, float const *bias,
+                    float *Z) {
+  nthreads = clampThreads(nthreads, B);
+  LeafModel lm(B, nthreads);
+  if (nthreads == 0) {
+    lm.m.Forward_Pass__Bias__Loop(0, B, H, bias, Z);
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    lm.m.Forward_Pass__Bias__OpenMP(0, B, H, bias, Z);
+  }
+}
+
+// ---- a9 / a10: batch (re)normalization, training ---------------------------
+// renorm != 0 → Batch_Renormalization, else Batch_Normalization.
+// mean/std out: [H]; mov_mean/mov_std: [H] in/out; r/d: [H] out (renorm only).
+void dlref_norm_fwd_train(int nthreads, int renorm, size_t B, size_t H,
+                          float momentum, float eps, float r_max, float d_max,
+                          float const *x, float const *gamma, float const *beta,
+                          float *mean, float *stdv, float *mov_mean,
+                          float *mov_std, float *r, float *d, float *xhat,
+                          float *out) {
+  nthreads = clampThreads(nthreads, B);
+  LeafModel lm(B, nthreads);
+  lm.m.normalization_momentum_average = momentum;
+  lm.m.normalization_epsilon = eps;
+  lm.m.batch_renormalization_r_correction_maximum = r_max;
+  lm.m.batch_renormalization_d_correction_maximum = d_max;
+  size_t const N = lm.m.number_threads;
+  std::vector<float> means(N * H, 0.0f), vars(N * H, 0.0f);
+  if (nthreads == 0) {
+    if (renorm)
+      lm.m.Forward_Pass__Batch_Renormalization__Training__Loop(
+          0, B, H, x, gamma, beta, means.data(), vars.data(), mov_mean, mov_std,
+          r, d, xhat, out);
+    else
+      lm.m.Forward_Pass__Batch_Normalization__Training__Loop(
+          0, B, H, x, gamma, beta, means.data(), vars.data(), mov_mean, mov_std,
+          xhat, out);
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    {
+      if (renorm)
+        lm.m.Forward_Pass__Batch_Renormalization__Training__OpenMP(
+            0, B, H, x, gamma, beta, means.data(), vars.data(), mov_mean,
+            mov_std, r, d, xhat, out);
+      else
+        lm.m.Forward_Pass__Batch_Normalization__Training__OpenMP(
+            0, B, H, x, gamma, beta, means.data(), vars.data(), mov_mean,
+            mov_std, xhat, out);
+    }
+  }
+  std::memcpy(mean, means.data(), H * sizeof(float));
+  std::memcpy(stdv, vars.data(), H * sizeof(float));
+}
+
+// ---- a11: normalization, inference -----------------------------------------
+void dlref_norm_fwd_infer(int nthreads, size_t B, size_t H, float const *x,
+                          float const *gamma, float const *beta,
+                          float const *mov_mean, float const *mov_std,
+                          float *out) {
+  nthreads = clampThreads(nthreads, B);
+  LeafModel lm(B, nthreads);
+  if (nthreads == 0) {
+    lm.m.Forward_Pass__Batch_Normalization__Inference__Loop(
+        0, B, H, x, gamma, beta, mov_mean, mov_std, out);
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    lm.m.Forward_Pass__Batch_Normalization__Inference__OpenMP(
+        0, B, H, x, gamma, beta, mov_mean, mov_std, out);
+  }
+}
+
+// ---- a12: activation forward (one type for the whole layer) ----------------
+void dlref_act_fwd(int nthreads, int type, size_t B, size_t H, float const *x,
+                   float *y) {
+  nthreads = clampThreads(nthreads, B);
+  LeafModel lm(B, nthreads);
+  std::vector<ACTIVATION::TYPE> types(H, static_cast<ACTIVATION::TYPE>(type));
+  if (nthreads == 0) {
+    lm.m.Forward_Pass__FC_AF__Loop(0, B, H, x, y, types.data());
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    lm.m.Forward_Pass__FC_AF__OpenMP(0, B, H, x, y, types.data());
+  }
+}
+
+// ---- a13: softmax ----------------------------------------------------------
+void dlref_softmax_fwd(int nthreads, size_t B, size_t H, float const *x,
+                       float *y) {
+  nthreads = clampThreads(nthreads, B);
+  LeafModel lm(B, nthreads);
+  if (nthreads == 0) {
+    lm.m.Forward_Pass__FC_AF__Softmax__Loop(0, B, H, x, y);
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    lm.m.Forward_Pass__FC_AF__Softmax__OpenMP(0, B, H, x, y);
+  }
+}
+
+// ---- a14: dropout ----------------------------------------------------------
+// kind 0: Bernoulli inverted (training), 1: Bernoulli (training),
+// kind 2: Bernoulli inference (v *= keep).  mask is per unit [H].
+void dlref_dropout_fwd(int nthreads, int kind, size_t B, size_t H,
+                       uint8_t const *mask, float scale_or_keep, float *v) {
+  nthreads = clampThreads(nthreads, B);
+  LeafModel lm(B, nthreads);
+  std::vector<char> maskb(H ? H : 1);
+  bool *mb = reinterpret_cast<bool *>(maskb.data());
+  if (mask)
+    for (size_t j = 0; j < H; ++j) mb[j] = mask[j] != 0;
+  if (nthreads == 0) {
+    if (kind == 0)
+      lm.m.Forward_Pass__Dropout__Bernoulli__Inverted__Loop(mb, 0, B, H,
+                                                           scale_or_keep, v);
+    else if (kind == 1)
+      lm.m.Forward_Pass__Dropout__Bernoulli__Training__Loop(mb, 0, B, H, v);
+    else
+      lm.m.Forward_Pass__Dropout__Bernoulli__Inference__Loop(0, B, H,
+                                                            scale_or_keep, v);
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    {
+      if (kind == 0)
+        lm.m.Forward_Pass__Dropout__Bernoulli__Inverted__OpenMP(
+            mb, 0, B, H, scale_or_keep, v);
+      else if (kind == 1)
+        lm.m.Forward_Pass__Dropout__Bernoulli__Training__OpenMP(mb, 0, B, H, v);
+      else
+        lm.m.Forward_Pass__Dropout__Bernoulli__Inference__OpenMP(
+            0, B, H, scale_or_keep, v);
+    }
+  }
+}
+
+// ---- a15: identity add (equal widths, no padding): out = a + b -------------
+void dlref_identity_add(int nthreads, size_t B, size_t H, float const *a,
+                        float const *b, float *out) {
+  nthreads = clampThreads(nthreads, B);
+  LeafModel lm(B, nthreads);
+  if (nthreads == 0) {
+    lm.m.Forward_Pass__Zero_Padded_Identity__Loop(0, B, H, H, 0, a, b, out);
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    lm.m.Forward_Pass__Zero_Padded_Identity__OpenMP(0, B, H, H, 0, a, b, out);
+  }
+}
+
+// ---- a18: dY += dZn * Wn  (dY is NOT cleared here) -------------------------
+void dlref_fc_bwd_dx(int nthreads, size_t B, size_t Hn, size_t H,
+                     float const *dZn, float const *Wn, float *dY) {
+  nthreads = clampThreads(nthreads, B);
+  LeafModel lm(B, nthreads);
+  if (nthreads == 0) {
+    lm.m.Backward_Pass__FC__Loop(0, B, Hn, H, dZn, Wn, dY);
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    lm.m.Backward_Pass__FC__OpenMP(0, B, Hn, H, dZn, Wn, dY);
+  }
+}
+
+// ---- a19: dN = dY * f'(pre, post) ------------------------------------------
+void dlref_act_bwd(int nthreads, int type, size_t B, size_t H,
+                   float const *pre, float const *post, float const *dY,
+                   float *dN) {
+  nthreads = clampThreads(nthreads, B);
+  LeafModel lm(B, nthreads);
+  std::vector<ACTIVATION::TYPE> types(H, static_cast<ACTIVATION::TYPE>(type));
+  if (nthreads == 0) {
+    lm.m.Backward_Pass__FC__DF__Loop(0, B, H, types.data(), pre, post, dY, dN);
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    lm.m.Backward_Pass__FC__DF__OpenMP(0, B, H, types.data(), pre, post, dY,
+                                       dN);
+  }
+}
+
+// ---- a20 / a21: batch (re)normalization backward (with shift) --------------
+// dgamma/dbeta [H] accumulate (+=) like the reference; dmean/dstd [H] out.
+void dlref_norm_bwd(int nthreads, int renorm, size_t B, size_t H,
+                    float const *mean, float const *stdv, float const *gamma,
+                    float const *r, float const *x, float const *xhat,
+                    float const *dN, float *dgamma, float *dbeta, float *dmean,
+                    float *dstd, float *dx) {
+  nthreads = clampThreads(nthreads, B);
+  size_t const P = 2 * H;  // [dgamma | dbeta] per thread copy
+  LeafModel lm(B, nthreads, P);
+  size_t const N = lm.m.number_threads;
+  std::vector<float> dpar(N * P, 0.0f), dmeans(N * H, 0.0f), dvars(N * H, 0.0f);
+  std::memcpy(dpar.data(), dgamma, H * sizeof(float));
+  std::memcpy(dpar.data() + H, dbeta, H * sizeof(float));
+  if (nthreads == 0) {
+    if (renorm)
+      lm.m.Backward_Pass__Batch_Renormalization__Loop(
+          0, B, H, mean, stdv, gamma, r, x, xhat, dN, dpar.data(),
+          dpar.data() + H, dmeans.data(), dvars.data(), dx);
+    else
+      lm.m.Backward_Pass__Batch_Normalization__Loop(
+          0, B, H, mean, stdv, gamma, x, xhat, dN, dpar.data(), dpar.data() + H,
+          dmeans.data(), dvars.data(), dx);
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    {
+      if (renorm)
+        lm.m.Backward_Pass__Batch_Renormalization__OpenMP(
+            0, B, H, mean, stdv, gamma, r, x, xhat, dN, dpar.data(),
+            dpar.data() + H, dmeans.data(), dvars.data(), dx);
+      else
+        lm.m.Backward_Pass__Batch_Normalization__OpenMP(
+            0, B, H, mean, stdv, gamma, x, xhat, dN, dpar.data(),
+            dpar.data() + H, dmeans.data(), dvars.data(), dx);
+    }
+    lm.m.use_mp = true;
+    lm.m.is_mp_initialized = true;
+    lm.m.ptr_array_derivatives_parameters = dpar.data();
+    lm.m.merge_mp_derivatives(0, P);
+    lm.m.ptr_array_derivatives_parameters = nullptr;
+    lm.m.use_mp = false;
+    lm.m.is_mp_initialized = false;
+  }
+  std::memcpy(dgamma, dpar.data(), H * sizeof(float));
+  std::memcpy(dbeta, dpar.data() + H, H * sizeof(float));
+  std::memcpy(dmean, dmeans.data(), H * sizeof(float));
+  std::memcpy(dstd, dvars.data(), H * sizeof(float));
+}
+
+// ---- a23: dW += dZ^T * Xin ; db += sum_b dZ --------------------------------
+// dW [H,K] and db [H] accumulate.  db may be null.
+void dlref_fc_bwd_dw(int nthreads, size_t B, size_t K, size_t H,
+                     float const *Xin, float const *dZ, float *dW, float *db) {
+  nthreads = clampThreads(nthreads, B);
+  size_t const P = H * K + H;
+  LeafModel lm(B, nthreads, P);
+  size_t const N = lm.m.number_threads;
+  std::vector<float> dpar(N * P, 0.0f);
+  std::memcpy(dpar.data(), dW, H * K * sizeof(float));
+  if (db) std::memcpy(dpar.data() + H * K, db, H * sizeof(float));
+  if (nthreads == 0) {
+    lm.m.Update_Derivative_Weight__FC__Loop(0, B, K, H, Xin, dZ, dpar.data());
+    if (db)
+      lm.m.Update_Derivative_Weight__Bias__Loop(0, B, H, dZ,
+                                                dpar.data() + H * K);
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    {
+      lm.m.Update_Derivative_Weight__FC__OpenMP(0, B, K, H, Xin, dZ,
+                                                dpar.data());
+      if (db)
+        lm.m.Update_Derivative_Weight__Bias__OpenMP(0, B, H, dZ,
+                                                    dpar.data() + H * K);
+    }
+    lm.m.use_mp = true;
+    lm.m.is_mp_initialized = true;
+    lm.m.ptr_array_derivatives_parameters = dpar.data();
+    lm.m.merge_mp_derivatives(0, P);
+    lm.m.ptr_array_derivatives_parameters = nullptr;
+    lm.m.use_mp = false;
+    lm.m.is_mp_initialized = false;
+  }
+  std::memcpy(dW, dpar.data(), H * K * sizeof(float));
+  if (db) std::memcpy(db, dpar.data() + H * K, H * sizeof(float));
+}
+
+// ===========================================================================
+// Whole-model path (a1-a6, a16, a17, a22, a24): a real Model built with
+// compile() and the public setters, as run/deep-learning/mnist.cpp:43-80 and
+// run/deep-learning/v1/custom.cpp:983-1036 do.
+// ===========================================================================
+struct RefModel {
+  Model model;
+  size_t n_layers = 0;
+  int nthreads = 0;
+};
+
+// widths[n_layers] (entry 0 = input width). Returns nullptr on failure.
+void *dlref_model_create(size_t n_layers, size_t const *widths,
+                         size_t allowable_bytes) {
+  dlref_init();
+  RefModel *rm = new RefModel;
+  rm->n_layers = n_layers;
+  std::vector<Layer_Parameters> lp(n_layers);
+  for (size_t i = 0; i < n_layers; ++i) {
+    lp[i].type_layer = LAYER::FULLY_CONNECTED;
+    lp[i].unit_parameters[0] = widths[i];
+  }
+  if (!rm->model.compile(n_layers, 1, MODEL::FEEDFORWARD, lp.data(),
+                         allowable_bytes)) {
+    delete rm;
+    return nullptr;
+  }
+  rm->model.set_loss_fn(LOSS_FN::CROSS_ENTROPY);
+  rm->model.set_accu_fn(ACCU_FN::CROSS_ENTROPY);
+  return rm;
+}
+
+void dlref_model_destroy(void *h) { delete static_cast<RefModel *>(h); }
+
+int dlref_model_set_activation(void *h, size_t layer, int type) {
+  return static_cast<RefModel *>(h)->model.set_layer_activation_function(
+      layer, static_cast<ACTIVATION::TYPE>(type));
+}
+
+int dlref_model_set_normalization(void *h, size_t layer, int type) {
+  return static_cast<RefModel *>(h)->model.Set__Layer_Normalization(
+      layer, static_cast<LAYER_NORM::TYPE>(type));
+}
+
+int dlref_model_set_norm_hyper(void *h, float momentum, float eps, float r_max,
+                               float d_max) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  bool ok = m.Set__Normalization_Momentum_Average(momentum);
+  ok = m.Set__Normalization_Epsilon(eps) && ok;
+  ok = m.Set__Batch_Renormalization_r_Correction_Maximum(r_max) && ok;
+  ok = m.Set__Batch_Renormalization_d_Correction_Maximum(d_max) && ok;
+  return ok;
+}
+
+// dropout type per LAYER_DROPOUT; keep = retention probability.
+int dlref_model_set_dropout(void *h, size_t layer, int type, float keep) {
+  real values[3] = {keep, 0, 0};
+  return static_cast<RefModel *>(h)->model.set_dropout(
+      layer, static_cast<LAYER_DROPOUT::TYPE>(type), values);
+}
+
+// Overwrite the per-unit Bernoulli mask of a layer (the reference samples it
+// from a clock-seeded generator, allocate.cpp:93).
+int dlref_model_set_dropout_mask(void *h, size_t layer, size_t H,
+                                 uint8_t const *mask) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  Layer &l = m.ptr_array_layers[layer];
+  if (l.ptr_array__mask__dropout__bernoulli == nullptr) return 0;
+  for (size_t j = 0; j < H; ++j)
+    l.ptr_array__mask__dropout__bernoulli[j] = mask[j] != 0;
+  return 1;
+}
+
+int dlref_model_prepare(void *h, size_t max_batch, int nthreads) {
+  RefModel *rm = static_cast<RefModel *>(h);
+  Model &m = rm->model;
+  if (!m.set_max_batch_size(max_batch)) return 0;
+  if (!m.update_mem_batch_size(max_batch)) return 0;
+  rm->nthreads = clampThreads(nthreads, max_batch);
+  if (rm->nthreads > 0) {
+    if (!m.set_mp(true)) return 0;
+    m.pct_threads =
+        100.0 * static_cast<double>(rm->nthreads) /
+        static_cast<double>(omp_get_num_procs());
+    if (!m.update_mem_thread_size(max_batch)) return 0;
+    rm->nthreads = static_cast<int>(m.number_threads);
+  }
+  m.clear_training_arrays();
+  return 1;
+}
+
+size_t dlref_model_number_threads(void *h) {
+  return static_cast<RefModel *>(h)->model.number_threads;
+}
+size_t dlref_model_total_parameters(void *h) {
+  return static_cast<RefModel *>(h)->model.total_parameters;
+}
+size_t dlref_model_total_norm_units(void *h) {
+  return static_cast<RefModel *>(h)->model.total_normalized_units;
+}
+
+// Layout probes (a2): offsets into the parameter array for one layer.
+// out[0]=first weight index, out[1]=first bias index, out[2]=gamma offset,
+// out[3]=beta offset, out[4]=offset of the layer's slot in the moving-stat
+// arrays, out[5]=use_bias.
+void dlref_model_layer_offsets(void *h, size_t layer, size_t *out) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  Layer &l = m.ptr_array_layers[layer];
+  out[0] = l.ptr_array_neuron_units
+               ? *l.ptr_array_neuron_units->ptr_first_connection_index
+               : 0;
+  out[1] = l.first_bias_connection_index;
+  auto &nu = l.ptr_array_normalized_units->normalized_batch_units;
+  out[2] = static_cast<size_t>(nu.ptr_scale - m.ptr_array_parameters);
+  out[3] = static_cast<size_t>(nu.ptr_shift - m.ptr_array_parameters);
+  out[4] = static_cast<size_t>(
+      nu.ptr_mean_average - m.ptr_array_normalized_batch_units_means_averages);
+  out[5] = l.Use__Bias();
+}
+
+void dlref_model_set_parameters(void *h, float const *p, size_t n) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  std::memcpy(m.ptr_array_parameters, p, n * sizeof(float));
+}
+void dlref_model_get_parameters(void *h, float *p, size_t n) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  std::memcpy(p, m.ptr_array_parameters, n * sizeof(float));
+}
+void dlref_model_set_moving(void *h, float const *mean, float const *stdv,
+                            size_t n) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  std::memcpy(m.ptr_array_normalized_batch_units_means_averages, mean,
+              n * sizeof(float));
+  std::memcpy(m.ptr_array_normalized_batch_units_variances_averages, stdv,
+              n * sizeof(float));
+}
+void dlref_model_get_moving(void *h, float *mean, float *stdv, size_t n) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  std::memcpy(mean, m.ptr_array_normalized_batch_units_means_averages,
+              n * sizeof(float));
+  std::memcpy(stdv, m.ptr_array_normalized_batch_units_variances_averages,
+              n * sizeof(float));
+}
+void dlref_model_zero_dparams(void *h) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  std::memset(m.ptr_array_derivatives_parameters, 0,
+              m.number_threads * m.total_parameters_allocated * sizeof(float));
+}
+void dlref_model_get_dparams(void *h, float *p, size_t n) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  std::memcpy(p, m.ptr_array_derivatives_parameters, n * sizeof(float));
+}
+
+// One step. X [B,K0] and Y [B,Hout] are dense row-major; the row-pointer
+// arrays the reference's API wants are built here.  state per PROPAGATION.
+// do_backward: also compute_error + backward_pass + update_derivatives
+// (+ merge_mp_derivatives), the region drivers/driver.cpp:241-259 covers.
+void dlref_model_step(void *h, int state, size_t B, float const *X, size_t K0,
+                      float const *Y, size_t Hout, int do_backward) {
+  RefModel *rm = static_cast<RefModel *>(h);
+  Model &m = rm->model;
+  m.type_state_propagation = static_cast<PROPAGATION::TYPE>(state);
+  std::vector<float const *> Xm(B), Ym(B);
+  for (size_t i = 0; i < B; ++i) {
+    Xm[i] = X + i * K0;
+    Ym[i] = Y ? Y + i * Hout : nullptr;
+  }
+  if (rm->nthreads > 0) {
+    omp_set_num_threads(static_cast<int>(m.number_threads));
+#pragma omp parallel
+    {
+      m.forward_pass(B, Xm.data());
+      if (do_backward) {
+        m.compute_error(B, Ym.data());
+        m.backward_pass(B);
+        m.update_derivatives(B, m.ptr_array_layers + 1, m.ptr_last_layer);
+      }
+    }
+    if (do_backward) m.merge_mp_derivatives(0, m.total_parameters);
+  } else {
+    m.forward_pass(B, Xm.data());
+    if (do_backward) {
+      m.compute_error(B, Ym.data());
+      m.backward_pass(B);
+      m.update_derivatives(B, m.ptr_array_layers + 1, m.ptr_last_layer);
+    }
+  }
+}
+
+// Per-layer buffers, [B,H] each. which: 0 summations (Z), 1 values_hats,
+// 2 values_normalizes, 3 AF values (post-dropout), 4 neuron errors (dZ),
+// 5 derivative_outputs (aliases the AF units' errors, ordering.cpp:165: holds
+// dY * f' once the backward pass has run), 6 layer outputs (ptr_array_outputs).
+int dlref_model_get_layer_buffer(void *h, size_t layer, int which, size_t B,
+                                 float *out) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  Layer &l = m.ptr_array_layers[layer];
+  size_t const H = *l.ptr_number_outputs;
+  float const *src = nullptr;
+  switch (which) {
+    case 0: src = l.ptr_array_neuron_units->ptr_array_summations; break;
+    case 1:
+      src = l.ptr_array_normalized_units->normalized_batch_units
+                .ptr_array_values_hats;
+      break;
+    case 2:
+      src = l.ptr_array_normalized_units->normalized_batch_units
+                .ptr_array_values_normalizes;
+      break;
+    case 3: src = l.ptr_array_AF_units->ptr_array_values; break;
+    case 4: src = l.ptr_array_neuron_units->ptr_array_errors; break;
+    case 5: src = l.ptr_array_derivative_outputs; break;
+    case 6: src = l.ptr_array_outputs; break;
+    default: return 0;
+  }
+  if (src == nullptr) return 0;
+  std::memcpy(out, src, B * H * sizeof(float));
+  return 1;
+}
+
+// Per-layer [H] vectors. which: 0 batch mean, 1 batch std, 2 r, 3 d.
+int dlref_model_get_layer_vector(void *h, size_t layer, int which, float *out) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  Layer &l = m.ptr_array_layers[layer];
+  size_t const H = *l.ptr_number_outputs;
+  auto &nu = l.ptr_array_normalized_units->normalized_batch_units;
+  float const *src = nullptr;
+  switch (which) {
+    case 0: src = nu.ptr_array_means; break;
+    case 1: src = nu.ptr_array_variances; break;
+    case 2: src = nu.ptr_r_correction; break;
+    case 3: src = nu.ptr_d_correction; break;
+    default: return 0;
+  }
+  if (src == nullptr) return 0;
+  std::memcpy(out, src, H * sizeof(float));
+  return 1;
+}
+
+}  // extern "C"

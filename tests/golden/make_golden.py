@@ -1,0 +1,193 @@
+"""Writes the golden vectors under tests/golden/ by running the REAL reference
+sources (compiled by oracle/Makefile.ref into oracle/_ref/libdlref.so) on
+seeded inputs.  Run from the repository root, in a container that holds
+/root/reference:
+
+    make -f oracle/Makefile.ref -j8 && python tests/golden/make_golden.py
+
+The fixtures are data only: inputs and the reference's outputs (npz, float32 /
+uint8 arrays, loaded with allow_pickle=False).  Every value in an "exp_*" array
+was produced by a member function of the reference's DL::v1::Model.
+"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from oracle.binding import ACT, DROP, NORM, STATE, Reference  # noqa: E402
+
+OUT = os.path.dirname(os.path.abspath(__file__))
+ACTS = ["ELU", "ISRLU", "LEAKY_RELU", "RELU", "SELU", "LINEAR"]
+LEAF_SHAPES = [(4, 5, 3), (7, 130, 5), (33, 24, 66)]  # (B, K, H)
+THREADS = [0, 3]  # 0 = single-thread leaves, 3 = OpenMP leaves on 3 threads
+
+
+def f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def leaves(R):
+    rng = np.random.default_rng(20240607)
+    d = {}
+    for ci, (B, K, H) in enumerate(LEAF_SHAPES):
+        p = f"c{ci}_"
+        X = f32(rng.standard_normal((B, K)))
+        W = f32(rng.uniform(-1, 1, (H, K)) * np.sqrt(6.0 / (K + H)))
+        bias = f32(rng.uniform(-0.5, 0.5, H))
+        x = f32(rng.standard_normal((B, H)) * rng.uniform(0.5, 2, H) + rng.uniform(-1, 1, H))
+        gamma = f32(rng.uniform(0.8, 1.2, H))
+        beta = f32(rng.uniform(-0.1, 0.1, H))
+        mov_mean = f32(rng.uniform(-1, 1, H))
+        mov_std = f32(rng.uniform(0.5, 2, H))
+        dN = f32(rng.standard_normal((B, H)))
+        dZ = f32(rng.standard_normal((B, H)))
+        dW0 = f32(rng.standard_normal((H, K)))
+        db0 = f32(rng.standard_normal(H))
+        mask = (rng.uniform(size=H) < 0.7).astype(np.uint8)
+        d.update({p + "shape": np.array([B, K, H]), p + "X": X, p + "W": W, p + "bias": bias, p + "x": x,
+                  p + "gamma": gamma, p + "beta": beta, p + "mov_mean": mov_mean, p + "mov_std": mov_std,
+                  p + "dN": dN, p + "dZ": dZ, p + "dW0": dW0, p + "db0": db0, p + "mask": mask})
+        for nt in THREADS:
+            q = f"{p}t{nt}_"
+            Z = R.fc_fwd(X, W, nt)
+            d[q + "fc_fwd"] = Z
+            d[q + "bias_fwd"] = R.bias_fwd(Z, bias, nt)
+            # three normalization settings: (a) fresh moving stats, clips do not
+            # bind; (b) warm moving stats + tight clips, both bind; (c) plain BN
+            settings = dict(
+                brn_loose=dict(mm=np.zeros(H), ms=np.ones(H), mom=0.99, rmax=3.0, dmax=5.0, renorm=True),
+                brn_tight=dict(mm=mov_mean, ms=mov_std, mom=0.05, rmax=1.1, dmax=0.05, renorm=True),
+                bn=dict(mm=mov_mean, ms=mov_std, mom=0.3, rmax=1.0, dmax=0.0, renorm=False))
+            for sname, s in settings.items():
+                fw = R.norm_fwd_train(x, gamma, beta, s["mm"], s["ms"], s["mom"], 1e-5, s["rmax"],
+                                      s["dmax"], s["renorm"], nt)
+                for k, v in fw.items():
+                    d[f"{q}{sname}_fwd_{k}"] = v
+                bw = R.norm_bwd(fw["mean"], fw["std"], gamma, fw["r"], x, fw["xhat"], dN,
+                                dgamma_init=gamma * 0.5, dbeta_init=beta * 2, renorm=s["renorm"], nthreads=nt)
+                for k, v in bw.items():
+                    d[f"{q}{sname}_bwd_{k}"] = v
+            d[q + "norm_infer"] = R.norm_fwd_infer(x, gamma, beta, mov_mean, mov_std, nt)
+            for a in ACTS:
+                y = R.act_fwd(ACT[a], x, nt)
+                d[f"{q}act_fwd_{a}"] = y
+                d[f"{q}act_bwd_{a}"] = R.act_bwd(ACT[a], x, y, dN, nt)
+            d[q + "softmax"] = R.softmax_fwd(x, nt)
+            d[q + "drop_inverted"] = R.dropout_fwd(0, x, mask, np.float32(1.0) / np.float32(0.7), nt)
+            d[q + "drop_plain"] = R.dropout_fwd(1, x, mask, 0.0, nt)
+            d[q + "drop_infer"] = R.dropout_fwd(2, x, None, 0.7, nt)
+            d[q + "identity_add"] = R.identity_add(x, dN, nt)
+            d[q + "fc_bwd_dx"] = R.fc_bwd_dx(dZ, W, nthreads=nt)
+            d[q + "fc_bwd_dx_acc"] = R.fc_bwd_dx(dZ, W, dY_init=f32(np.ones((B, K))), nthreads=nt)
+            dW, db = R.fc_bwd_dw(X, dZ, dW_init=dW0, db_init=db0, nthreads=nt)
+            d[q + "fc_bwd_dw"] = dW
+            d[q + "fc_bwd_db"] = db
+    # activation special points (one row): signed zeros, tiny, large, around the knees
+    pts = f32([[-0.0, 0.0, -1e-30, 1e-30, -1e-6, 1e-6, -0.5, 0.5, -1.0, 1.0, -5.0, 5.0, -20.0, 20.0,
+                -88.0, 88.0, -1e4, 1e4]])
+    d["pts"] = pts
+    ones = np.ones_like(pts)
+    for a in ACTS:
+        y = R.act_fwd(ACT[a], pts, 0)
+        d[f"pts_fwd_{a}"] = y
+        d[f"pts_bwd_{a}"] = R.act_bwd(ACT[a], pts, y, ones, 0)
+    np.savez_compressed(os.path.join(OUT, "leaves.npz"), **d)
+    return len(d)
+
+
+MLP_CASES = {
+    # name: (widths, B, per-layer (act, norm, drop, keep), hyper(m, eps, rmax, dmax))
+    "mlp_relu_brn": ([8, 6, 6, 3], 5, [("RELU", "BRN", "NONE", 1.0), ("RELU", "BRN", "NONE", 1.0)],
+                     (0.99, 1e-5, 3.0, 5.0)),
+    "mlp_c1_small": ([20, 16, 16, 10], 12, [("RELU", "BRN", "NONE", 1.0), ("RELU", "BRN", "NONE", 1.0)],
+                     (0.99, 1e-5, 3.0, 5.0)),
+    "mlp_mixed": ([9, 7, 12, 5, 4], 11,
+                  [("SELU", "BRN", "BERNOULLI_INVERTED", 0.8), ("ELU", "NONE", "NONE", 1.0),
+                   ("ISRLU", "BRN", "BERNOULLI", 0.6)], (0.3, 1e-3, 1.2, 0.1)),
+    # the reference refuses BN and BRN layers in one model (the first BN layer
+    # re-allocates arrays the BRN layers already own, normalization.cpp:351), so
+    # plain batch normalization gets a model of its own
+    "mlp_bn": ([7, 9, 8, 3], 10, [("ISRLU", "BN", "NONE", 1.0), ("SELU", "BN", "BERNOULLI_INVERTED", 0.75)],
+               (0.2, 1e-5, 1.0, 0.0)),
+    "mlp_lrelu_plain": ([6, 10, 10, 4], 9, [("LEAKY_RELU", "NONE", "NONE", 1.0), ("LEAKY_RELU", "BRN", "NONE", 1.0)],
+                        (0.5, 1e-5, 2.0, 1.0)),
+}
+
+
+def glorot(rng, H, K):
+    lim = np.sqrt(6.0 / (K + H))
+    return f32(rng.uniform(-lim, lim, (H, K)))
+
+
+def mlps(R):
+    d = {}
+    for name, (widths, B, hidden, hyper) in MLP_CASES.items():
+        rng = np.random.default_rng(sum(map(ord, name)))
+        L = len(widths)
+        X = f32(rng.uniform(0, 1, (B, widths[0])))
+        labels = rng.integers(0, widths[-1], B)
+        Y = f32(np.eye(widths[-1])[labels])
+        masks = {l: (rng.uniform(size=widths[l]) < hidden[l - 1][3]).astype(np.uint8) for l in range(1, L - 1)}
+        d[name + "_widths"] = np.array(widths)
+        d[name + "_X"] = X
+        d[name + "_Y"] = Y
+        d[name + "_hyper"] = f32(hyper)
+        for l, mk in masks.items():
+            d[f"{name}_mask{l}"] = mk
+        params = None
+        for nt in THREADS:
+            M = R.mlp(widths)
+            for l in range(1, L - 1):
+                a, n, dr, keep = hidden[l - 1]
+                M.set_layer(l, ACT[a], NORM[n], DROP[dr], keep, masks[l] if dr != "NONE" else None)
+            M.set_layer(L - 1, ACT["SOFTMAX"])
+            M.set_norm_hyper(*hyper)
+            M.prepare(B, nt)
+            if params is None:
+                # harness-generated parameters in the reference's packed layout
+                params = M.get_parameters()  # gamma=1, beta=0 from the reference's allocator
+                offs = [M.layer_offsets(l) for l in range(L)]
+                d[name + "_offsets"] = np.array(offs)
+                for l in range(1, L):
+                    K, H = widths[l - 1], widths[l]
+                    params[offs[l][0]:offs[l][0] + H * K] = glorot(rng, H, K).ravel()
+                    params[offs[l][1]:offs[l][1] + H] = f32(rng.uniform(-0.2, 0.2, H))
+                    params[offs[l][2]:offs[l][2] + H] = f32(rng.uniform(0.8, 1.2, H))
+                    params[offs[l][3]:offs[l][3] + H] = f32(rng.uniform(-0.1, 0.1, H))
+                d[name + "_params"] = params.copy()
+                d[name + "_P"] = np.array([M.P, M.n_units])
+            M.set_parameters(params)
+            q = f"{name}_t{nt}_"
+            M.step(STATE["TRAINING"], X, Y, backward=True)
+            for l in range(1, L):
+                for which, wn in ((0, "Z"), (3, "out"), (4, "dZ")):
+                    d[f"{q}L{l}_{wn}"] = M.layer_buffer(l, which)
+                if l < L - 1:
+                    # derivative_outputs aliases the AF units' error array
+                    # (ordering.cpp:165), so after the backward pass it holds
+                    # dY * f'(pre, post), not dY
+                    d[f"{q}L{l}_dAF"] = M.layer_buffer(l, 5)
+                    if hidden[l - 1][1] != "NONE":
+                        d[f"{q}L{l}_xhat"] = M.layer_buffer(l, 1)
+                        d[f"{q}L{l}_nrm"] = M.layer_buffer(l, 2)
+                        vecs = ((0, "mean"), (1, "std"), (2, "r"), (3, "d"))
+                        for which, wn in vecs if hidden[l - 1][1] == "BRN" else vecs[:2]:
+                            d[f"{q}L{l}_{wn}"] = M.layer_vector(l, which)
+            d[q + "dparams"] = M.get_dparams()
+            mm, ms = M.get_moving()
+            d[q + "mov_mean"] = mm
+            d[q + "mov_std"] = ms
+            # inference forward with the moving statistics just updated
+            M.step(STATE["INFERENCE"], X, None, backward=False)
+            for l in range(1, L):
+                d[f"{q}infer_L{l}_out"] = M.layer_buffer(l, 3)
+    np.savez_compressed(os.path.join(OUT, "mlp.npz"), **d)
+    return len(d)
+
+
+if __name__ == "__main__":
+    R = Reference()
+    print("leaves:", leaves(R), "arrays")
+    print("mlp:", mlps(R), "arrays")
