@@ -19,17 +19,19 @@ def rms(a):
     return float(np.sqrt(np.mean(a * a))) if a.size else 0.0
 
 
-def max_rel_err(got, exp):
-    """max |got-exp| / max(|exp|, rms(exp)) (0 for empty tensors)."""
+def max_rel_err(got, exp, floor=0.0):
+    """max |got-exp| / max(|exp|, rms(exp), floor) (0 for empty tensors).
+    `floor` names the natural scale of a quantity whose expected value may be
+    identically zero (a shift in units of sigma, a gradient that cancels)."""
     got = np.asarray(got, np.float64)
     exp = np.asarray(exp, np.float64)
     if exp.size == 0:
         return 0.0
-    den = np.maximum(np.abs(exp), max(rms(exp), 1e-30))
+    den = np.maximum(np.abs(exp), max(rms(exp), floor, 1e-30))
     return float(np.max(np.abs(got - exp) / den))
 
 
-def assert_close(got, exp, rtol, what=""):
+def assert_close(got, exp, rtol, what="", floor=0.0):
     got = np.asarray(got)
     exp = np.asarray(exp)
     assert got.shape == exp.shape, f"{what}: shape {got.shape} != {exp.shape}"
@@ -37,6 +39,6 @@ def assert_close(got, exp, rtol, what=""):
     fin = np.isfinite(exp)
     # infinities / NaNs must match in kind
     assert np.array_equal(got[~fin].astype(str), exp[~fin].astype(str)), f"{what}: inf/nan differ"
-    err = max_rel_err(got[fin], exp[fin])
+    err = max_rel_err(got[fin], exp[fin], floor)
     assert err <= rtol, f"{what}: max rel err {err:.3e} > {rtol:.1e}"
     return err
