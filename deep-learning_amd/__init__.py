@@ -1,0 +1,276 @@
+"""deep-learning_amd — MI355X (gfx950) implementation of the fully-connected /
+batch-(re)normalization / activation hot path of SebastienKeroack/deep-learning.
+
+The product is ``lib/libdlmi.so`` (hand-written HIP kernels behind the C ABI of
+``include/dlmi.h`` plus the C++ ``Model`` facade of ``include/dlmi_model.h``).
+This module is only the thin Python binding the tests and the benchmark use:
+PyTorch supplies device memory and the stream, every computation goes through
+the C ABI.  There is no CPU or PyTorch fallback: if the library is not built, or
+no gfx950 device is present, construction raises.
+
+The directory name carries a hyphen, so import it by path::
+
+    spec = importlib.util.spec_from_file_location(
+        "deep_learning_amd", ".../deep-learning_amd/__init__.py",
+        submodule_search_locations=[".../deep-learning_amd"])
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libdlmi.so")
+
+c_sz = ctypes.c_size_t
+c_int = ctypes.c_int
+c_f = ctypes.c_float
+vp = ctypes.c_void_p
+
+# enum values shared with the reference (include/dlmi.h)
+ACT = dict(ELU=3, ISRLU=10, LINEAR=11, LEAKY_RELU=14, RELU=16, SELU=17, SOFTMAX=22)
+NORM = dict(NONE=0, BN=1, BRN=2)
+DROP = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3)
+DROP_BWD = dict(REFERENCE=0, MASKED=1)
+STATE = dict(INFERENCE=0, TRAINING=1, UPDATE_BATCH_NORM=2)
+
+# every symbol include/dlmi.h declares
+C_ABI_SYMBOLS = [
+    "dlmi_ctx_create", "dlmi_ctx_destroy", "dlmi_ctx_set_stream", "dlmi_ctx_synchronize", "dlmi_last_error",
+    "dlmi_ctx_compute_units", "dlmi_fc_fwd", "dlmi_fc_bwd_dx", "dlmi_fc_bwd_dw", "dlmi_bias_fwd",
+    "dlmi_norm_fwd_train", "dlmi_norm_fwd_infer", "dlmi_norm_bwd", "dlmi_act_fwd", "dlmi_act_bwd",
+    "dlmi_softmax_fwd", "dlmi_dropout_fwd", "dlmi_identity_add", "dlmi_softmax_ce_seed",
+    "dlmi_fused_norm_act_fwd", "dlmi_fused_norm_act_bwd", "dlmi_fused_norm_act_infer",
+]
+
+
+class FusedDesc(ctypes.Structure):
+    """dlmi_fused_desc of include/dlmi.h."""
+    _fields_ = [("norm", c_int), ("act", c_int), ("dropout", c_int), ("mask_per_element", c_int),
+                ("dropout_bwd", c_int), ("momentum", c_f), ("eps", c_f), ("r_max", c_f), ("d_max", c_f),
+                ("drop_scale", c_f)]
+
+
+class DlmiError(RuntimeError):
+    pass
+
+
+def load_library():
+    if not os.path.exists(LIB_PATH):
+        raise DlmiError("%s is missing: build it with `python deep-learning_amd/build.py` "
+                        "(there is no fallback path)" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.dlmi_last_error.restype = ctypes.c_char_p
+    lib.dlmi_last_error.argtypes = [vp]
+    return lib
+
+
+def _p(t):
+    return vp(0) if t is None else vp(t.data_ptr())
+
+
+class Dlmi:
+    """One dlmi context bound to a torch CUDA(HIP) device and its current stream."""
+
+    def __init__(self, device=0):
+        import torch
+        self.torch = torch
+        self.lib = load_library()
+        if not torch.cuda.is_available():
+            raise DlmiError("no GPU visible: dlmi has no CPU path")
+        self.device = torch.device("cuda", device)
+        ctx = vp()
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        rc = self.lib.dlmi_ctx_create(ctypes.byref(ctx), c_int(device), vp(stream))
+        if rc != 0:
+            raise DlmiError("dlmi_ctx_create failed with %d" % rc)
+        self.ctx = ctx
+
+    def close(self):
+        if getattr(self, "ctx", None):
+            self.lib.dlmi_ctx_destroy(self.ctx)
+            self.ctx = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # ------------------------------------------------------------ helpers
+    def _ck(self, rc):
+        if rc != 0:
+            raise DlmiError("dlmi call failed (%d): %s" % (rc, self.lib.dlmi_last_error(self.ctx).decode()))
+
+    def _chk(self, *tensors):
+        for t in tensors:
+            if t is None:
+                continue
+            assert t.is_cuda and t.is_contiguous(), "dlmi takes contiguous device tensors"
+
+    def empty(self, *shape, dtype=None):
+        return self.torch.empty(*shape, dtype=dtype or self.torch.float32, device=self.device)
+
+    def zeros(self, *shape, dtype=None):
+        return self.torch.zeros(*shape, dtype=dtype or self.torch.float32, device=self.device)
+
+    def set_stream(self, stream):
+        self._ck(self.lib.dlmi_ctx_set_stream(self.ctx, vp(stream.cuda_stream)))
+
+    def synchronize(self):
+        self._ck(self.lib.dlmi_ctx_synchronize(self.ctx))
+
+    def compute_units(self):
+        return self.lib.dlmi_ctx_compute_units(self.ctx)
+
+    # ------------------------------------------------------------ GEMMs
+    def fc_fwd(self, X, W, bias=None, out=None):
+        self._chk(X, W, bias, out)
+        B, K = X.shape
+        H = W.shape[0]
+        assert W.shape[1] == K
+        Z = out if out is not None else self.empty(B, H)
+        self._ck(self.lib.dlmi_fc_fwd(self.ctx, c_sz(B), c_sz(K), c_sz(H), _p(X), _p(W), _p(bias), _p(Z)))
+        return Z
+
+    def fc_bwd_dx(self, dZn, Wn, out=None, accumulate=False):
+        self._chk(dZn, Wn, out)
+        B, Hn = dZn.shape
+        H = Wn.shape[1]
+        assert Wn.shape[0] == Hn
+        dY = out if out is not None else self.empty(B, H)
+        assert out is not None or not accumulate
+        self._ck(self.lib.dlmi_fc_bwd_dx(self.ctx, c_sz(B), c_sz(Hn), c_sz(H), _p(dZn), _p(Wn), _p(dY),
+                                         c_int(1 if accumulate else 0)))
+        return dY
+
+    def fc_bwd_dw(self, Xin, dZ, dW=None, db=None, with_bias=False, accumulate=False):
+        self._chk(Xin, dZ, dW, db)
+        B, K = Xin.shape
+        H = dZ.shape[1]
+        assert dZ.shape[0] == B
+        if dW is None:
+            assert not accumulate
+            dW = self.empty(H, K)
+        if db is None and with_bias:
+            db = self.empty(H)
+        self._ck(self.lib.dlmi_fc_bwd_dw(self.ctx, c_sz(B), c_sz(K), c_sz(H), _p(Xin), _p(dZ), _p(dW), _p(db),
+                                         c_int(1 if accumulate else 0)))
+        return dW, db
+
+    def bias_fwd(self, Z, bias):
+        self._chk(Z, bias)
+        B, H = Z.shape
+        self._ck(self.lib.dlmi_bias_fwd(self.ctx, c_sz(B), c_sz(H), _p(bias), _p(Z)))
+        return Z
+
+    # ------------------------------------------------------------ normalization (un-fused leaves)
+    def norm_fwd_train(self, x, gamma, beta, mov_mean, mov_std, momentum, eps, r_max=1.0, d_max=0.0,
+                       renorm=True, want_xhat=True, want_out=True):
+        """mov_mean / mov_std are updated in place.  Returns dict(mean,std,r,d,xhat,out)."""
+        self._chk(x, gamma, beta, mov_mean, mov_std)
+        B, H = x.shape
+        o = dict(mean=self.empty(H), std=self.empty(H), r=self.empty(H), d=self.empty(H),
+                 xhat=self.empty(B, H) if want_xhat else None, out=self.empty(B, H) if want_out else None)
+        self._ck(self.lib.dlmi_norm_fwd_train(
+            self.ctx, c_int(NORM["BRN"] if renorm else NORM["BN"]), c_sz(B), c_sz(H), c_f(momentum), c_f(eps),
+            c_f(r_max), c_f(d_max), _p(x), _p(gamma), _p(beta), _p(o["mean"]), _p(o["std"]), _p(mov_mean),
+            _p(mov_std), _p(o["r"]), _p(o["d"]), _p(o["xhat"]), _p(o["out"])))
+        return o
+
+    def norm_fwd_infer(self, x, gamma, beta, mov_mean, mov_std):
+        self._chk(x, gamma, beta, mov_mean, mov_std)
+        B, H = x.shape
+        out = self.empty(B, H)
+        self._ck(self.lib.dlmi_norm_fwd_infer(self.ctx, c_sz(B), c_sz(H), _p(x), _p(gamma), _p(beta), _p(mov_mean),
+                                              _p(mov_std), _p(out)))
+        return out
+
+    def norm_bwd(self, mean, std, gamma, r, x, xhat, dN, dgamma, dbeta, renorm=True):
+        """dgamma / dbeta accumulate in place.  Returns dict(dmean,dstd,dx)."""
+        self._chk(mean, std, gamma, r, x, xhat, dN, dgamma, dbeta)
+        B, H = x.shape
+        o = dict(dmean=self.empty(H), dstd=self.empty(H), dx=self.empty(B, H))
+        self._ck(self.lib.dlmi_norm_bwd(self.ctx, c_int(NORM["BRN"] if renorm else NORM["BN"]), c_sz(B), c_sz(H),
+                                        _p(mean), _p(std), _p(gamma), _p(r), _p(x), _p(xhat), _p(dN), _p(dgamma),
+                                        _p(dbeta), _p(o["dmean"]), _p(o["dstd"]), _p(o["dx"])))
+        return o
+
+    # ------------------------------------------------------------ element-wise leaves
+    def act_fwd(self, act, x, out=None):
+        self._chk(x, out)
+        B, H = x.shape
+        y = out if out is not None else self.empty(B, H)
+        self._ck(self.lib.dlmi_act_fwd(self.ctx, c_int(act), c_sz(B), c_sz(H), _p(x), _p(y)))
+        return y
+
+    def act_bwd(self, act, pre, post, dY, out=None):
+        self._chk(pre, post, dY, out)
+        B, H = pre.shape
+        dN = out if out is not None else self.empty(B, H)
+        self._ck(self.lib.dlmi_act_bwd(self.ctx, c_int(act), c_sz(B), c_sz(H), _p(pre), _p(post), _p(dY), _p(dN)))
+        return dN
+
+    def softmax_fwd(self, x):
+        self._chk(x)
+        B, H = x.shape
+        y = self.empty(B, H)
+        self._ck(self.lib.dlmi_softmax_fwd(self.ctx, c_sz(B), c_sz(H), _p(x), _p(y)))
+        return y
+
+    def dropout_fwd(self, kind, v, mask, scale, training=True):
+        """In place on v.  mask [H] or [B,H] uint8."""
+        self._chk(v, mask)
+        B, H = v.shape
+        per_element = 1 if (mask is not None and mask.dim() == 2) else 0
+        self._ck(self.lib.dlmi_dropout_fwd(self.ctx, c_int(kind), c_int(1 if training else 0), c_int(per_element),
+                                           c_sz(B), c_sz(H), _p(mask), c_f(scale), _p(v)))
+        return v
+
+    def identity_add(self, a, b, out=None):
+        self._chk(a, b, out)
+        o = out if out is not None else self.torch.empty_like(a)
+        self._ck(self.lib.dlmi_identity_add(self.ctx, c_sz(a.numel()), _p(a), _p(b), _p(o)))
+        return o
+
+    def softmax_ce_seed(self, q, y, stats=None):
+        """stats: optional device tensor of 2 float64 accumulators."""
+        self._chk(q, y, stats)
+        B, H = q.shape
+        dZ = self.empty(B, H)
+        self._ck(self.lib.dlmi_softmax_ce_seed(self.ctx, c_sz(B), c_sz(H), _p(q), _p(y), _p(dZ), _p(stats)))
+        return dZ
+
+    # ------------------------------------------------------------ fused hot path
+    @staticmethod
+    def desc(act, renorm=True, dropout=0, mask_per_element=False, dropout_bwd=0, momentum=0.99, eps=1e-5,
+             r_max=3.0, d_max=5.0, drop_scale=1.0):
+        return FusedDesc(NORM["BRN"] if renorm else NORM["BN"], act, dropout, 1 if mask_per_element else 0,
+                         dropout_bwd, momentum, eps, r_max, d_max, drop_scale)
+
+    def fused_fwd(self, desc, x, gamma, beta, mov_mean, mov_std, mask=None, out=None, stats=None):
+        """Returns (y, stats) with stats = dict(mean,std,r,d) kept for the backward."""
+        self._chk(x, gamma, beta, mov_mean, mov_std, mask, out)
+        B, H = x.shape
+        y = out if out is not None else self.empty(B, H)
+        s = stats or dict(mean=self.empty(H), std=self.empty(H), r=self.empty(H), d=self.empty(H))
+        self._ck(self.lib.dlmi_fused_norm_act_fwd(self.ctx, ctypes.byref(desc), c_sz(B), c_sz(H), _p(x), _p(gamma),
+                                                  _p(beta), _p(mask), _p(s["mean"]), _p(s["std"]), _p(mov_mean),
+                                                  _p(mov_std), _p(s["r"]), _p(s["d"]), _p(y)))
+        return y, s
+
+    def fused_bwd(self, desc, x, gamma, beta, stats, dY, dgamma, dbeta, mask=None, out=None):
+        self._chk(x, gamma, beta, dY, dgamma, dbeta, mask, out)
+        B, H = x.shape
+        dX = out if out is not None else self.empty(B, H)
+        self._ck(self.lib.dlmi_fused_norm_act_bwd(self.ctx, ctypes.byref(desc), c_sz(B), c_sz(H), _p(x), _p(gamma),
+                                                  _p(beta), _p(mask), _p(stats["mean"]), _p(stats["std"]),
+                                                  _p(stats["r"]), _p(stats["d"]), _p(dY), _p(dgamma), _p(dbeta),
+                                                  _p(dX)))
+        return dX
+
+    def fused_infer(self, desc, x, gamma, beta, mov_mean, mov_std, out=None):
+        self._chk(x, gamma, beta, mov_mean, mov_std, out)
+        B, H = x.shape
+        y = out if out is not None else self.empty(B, H)
+        self._ck(self.lib.dlmi_fused_norm_act_infer(self.ctx, ctypes.byref(desc), c_sz(B), c_sz(H), _p(x), _p(gamma),
+                                                    _p(beta), _p(mov_mean), _p(mov_std), _p(y)))
+        return y

@@ -1,0 +1,78 @@
+// Device-side activation functions and the derivative forms the reference's
+// backward pass uses (a function of the pre-activation x AND the stored output
+// q).  Citations: /root/reference/lib/deep-learning/v1/ops/activations/functions.hpp.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "../../include/dlmi.h"
+
+namespace dlmi {
+
+// functions.hpp:95-96, 108 — the reference's `_r` literals are floats in Release
+constexpr float kSeluAlpha = 1.6732632423543772848170429916717f;
+constexpr float kSeluScale = 1.0507009873554804934193349852946f;
+constexpr float kLreluAlpha = 0.01f;
+
+template <int ACT>
+__device__ __forceinline__ float act_fire(float x) {
+  if constexpr (ACT == DLMI_ACT_ISRLU) {  // functions.hpp:86-87, slope 1
+    return x < 0.0f ? x * (1.0f / sqrtf(1.0f + x * x)) : x;
+  } else if constexpr (ACT == DLMI_ACT_ELU) {  // functions.hpp:91, slope 1: exp(x) - 1, not expm1
+    return x < 0.0f ? (expf(x) - 1.0f) : x;
+  } else if constexpr (ACT == DLMI_ACT_SELU) {  // functions.hpp:97-98
+    return kSeluScale * (x <= 0.0f ? kSeluAlpha * expf(x) - kSeluAlpha : x);
+  } else if constexpr (ACT == DLMI_ACT_RELU) {  // functions.hpp:102
+    return x < 0.0f ? 0.0f : x;
+  } else if constexpr (ACT == DLMI_ACT_LEAKY_RELU) {  // functions.hpp:106
+    return x < 0.0f ? kLreluAlpha * x : x;
+  } else {  // LINEAR
+    return x;
+  }
+}
+
+// functions.hpp:88 (ISRLU), :92 (ELU), :99 (SELU), :103 (ReLU), :107 (leaky)
+template <int ACT>
+__device__ __forceinline__ float act_derive(float x, float q) {
+  if constexpr (ACT == DLMI_ACT_ISRLU) {
+    float const t = q / x;  // std::pow(q / x, 3)
+    return x < 0.0f ? t * t * t : 1.0f;
+  } else if constexpr (ACT == DLMI_ACT_ELU) {
+    return x < 0.0f ? q : 1.0f;
+  } else if constexpr (ACT == DLMI_ACT_SELU) {
+    return kSeluScale * (x <= 0.0f ? (q + kSeluAlpha) : 1.0f);
+  } else if constexpr (ACT == DLMI_ACT_RELU) {
+    return x < 0.0f ? 0.0f : 1.0f;
+  } else if constexpr (ACT == DLMI_ACT_LEAKY_RELU) {
+    return x < 0.0f ? kLreluAlpha : 1.0f;
+  } else {
+    return 1.0f;
+  }
+}
+
+inline bool act_supported(int act) {
+  switch (act) {
+    case DLMI_ACT_ISRLU:
+    case DLMI_ACT_ELU:
+    case DLMI_ACT_SELU:
+    case DLMI_ACT_RELU:
+    case DLMI_ACT_LEAKY_RELU:
+    case DLMI_ACT_LINEAR:
+      return true;
+    default:
+      return false;
+  }
+}
+
+// Calls f.template operator()<ACT>() for the runtime activation code.
+#define DLMI_DISPATCH_ACT(act, ...)                                        \
+  switch (act) {                                                           \
+    case DLMI_ACT_ISRLU: { constexpr int ACT = DLMI_ACT_ISRLU; __VA_ARGS__; } break;           \
+    case DLMI_ACT_ELU: { constexpr int ACT = DLMI_ACT_ELU; __VA_ARGS__; } break;               \
+    case DLMI_ACT_SELU: { constexpr int ACT = DLMI_ACT_SELU; __VA_ARGS__; } break;             \
+    case DLMI_ACT_RELU: { constexpr int ACT = DLMI_ACT_RELU; __VA_ARGS__; } break;             \
+    case DLMI_ACT_LEAKY_RELU: { constexpr int ACT = DLMI_ACT_LEAKY_RELU; __VA_ARGS__; } break; \
+    default: { constexpr int ACT = DLMI_ACT_LINEAR; __VA_ARGS__; } break;                      \
+  }
+
+}  // namespace dlmi

@@ -1,0 +1,60 @@
+// Shared host-side plumbing of the dlmi library: the context object, error
+// capture and launch-geometry helpers.  HIP only, gfx950 only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/dlmi.h"
+
+struct dlmi_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  int num_cu = 256;
+  // Device scratch for reduction partials and per-unit constants.  Grown on
+  // demand (never inside a launch sequence that already holds pointers to it).
+  char *scratch = nullptr;
+  size_t scratch_bytes = 0;
+  char err[512] = {0};
+};
+
+inline int dlmi_fail(dlmi_ctx *ctx, int code, char const *fmt, ...) {
+  if (ctx != nullptr) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(ctx->err, sizeof(ctx->err), fmt, ap);
+    va_end(ap);
+  }
+  return code;
+}
+
+#define DLMI_HIP(ctx, call)                                                              \
+  do {                                                                                   \
+    hipError_t e_ = (call);                                                              \
+    if (e_ != hipSuccess)                                                                \
+      return dlmi_fail((ctx), DLMI_E_HIP, "%s failed: %s (%s:%d)", #call,                \
+                       hipGetErrorString(e_), __FILE__, __LINE__);                       \
+  } while (0)
+
+// After a kernel launch: surfaces launch-configuration errors without syncing.
+#define DLMI_LAUNCH_CHECK(ctx, what)                                                     \
+  do {                                                                                   \
+    hipError_t e_ = hipGetLastError();                                                   \
+    if (e_ != hipSuccess)                                                                \
+      return dlmi_fail((ctx), DLMI_E_HIP, "launch of %s failed: %s", (what),             \
+                       hipGetErrorString(e_));                                           \
+  } while (0)
+
+#define DLMI_REQUIRE(ctx, cond, msg)                                                     \
+  do {                                                                                   \
+    if (!(cond)) return dlmi_fail((ctx), DLMI_E_INVALID, "%s: %s", __func__, (msg));      \
+  } while (0)
+
+// Makes sure the context's scratch holds at least `bytes`.
+int dlmi_scratch_reserve(dlmi_ctx *ctx, size_t bytes);
+
+inline bool dlmi_aligned16(void const *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline size_t dlmi_ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }

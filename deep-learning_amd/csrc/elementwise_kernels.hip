@@ -1,0 +1,346 @@
+// Element-wise leaves of the fully-connected path for gfx950: bias add,
+// activation forward / derivative, dropout, identity add, inference-mode
+// normalization (optionally fused with the activation), row softmax and the
+// softmax + cross-entropy seed gradient.  One coalesced pass each; float4
+// accesses whenever the row length and the pointers allow it.
+//
+// Citations: /root/reference/lib/deep-learning/v1/learner/.
+#include <initializer_list>
+
+#include "activations.hpp"
+#include "dlmi_common.hpp"
+
+namespace dlmi {
+
+constexpr int kEwBlock = 256;
+
+static unsigned ew_grid(dlmi_ctx const *ctx, size_t work_items) {
+  size_t const blocks = dlmi_ceil_div(work_items, kEwBlock);
+  size_t const cap = static_cast<size_t>(ctx->num_cu) * 16;
+  return static_cast<unsigned>(blocks < cap ? (blocks ? blocks : 1) : cap);
+}
+
+static bool all_aligned16(std::initializer_list<void const *> ptrs) {
+  for (void const *p : ptrs)
+    if (p != nullptr && !dlmi_aligned16(p)) return false;
+  return true;
+}
+
+// ---- activation forward / backward (fwp_st.cpp:4768-4794, bwp_st.cpp:1177-1209)
+template <int ACT>
+__global__ __launch_bounds__(kEwBlock) void k_act_fwd(float const *__restrict__ x, float *__restrict__ y, size_t n4,
+                                                       size_t n) {
+  size_t const stride = static_cast<size_t>(gridDim.x) * kEwBlock;
+  size_t i = static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x;
+  for (; i < n4; i += stride) {
+    float4 v = reinterpret_cast<float4 const *>(x)[i];
+    v.x = act_fire<ACT>(v.x); v.y = act_fire<ACT>(v.y); v.z = act_fire<ACT>(v.z); v.w = act_fire<ACT>(v.w);
+    reinterpret_cast<float4 *>(y)[i] = v;
+  }
+  for (i = n4 * 4 + static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x; i < n; i += stride)
+    y[i] = act_fire<ACT>(x[i]);
+}
+
+template <int ACT>
+__global__ __launch_bounds__(kEwBlock) void k_act_bwd(float const *__restrict__ pre, float const *__restrict__ post,
+                                                       float const *__restrict__ dY, float *__restrict__ dN,
+                                                       size_t n4, size_t n) {
+  size_t const stride = static_cast<size_t>(gridDim.x) * kEwBlock;
+  size_t i = static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x;
+  for (; i < n4; i += stride) {
+    float4 const a = reinterpret_cast<float4 const *>(pre)[i];
+    float4 const q = reinterpret_cast<float4 const *>(post)[i];
+    float4 g = reinterpret_cast<float4 const *>(dY)[i];
+    g.x *= act_derive<ACT>(a.x, q.x); g.y *= act_derive<ACT>(a.y, q.y);
+    g.z *= act_derive<ACT>(a.z, q.z); g.w *= act_derive<ACT>(a.w, q.w);
+    reinterpret_cast<float4 *>(dN)[i] = g;
+  }
+  for (i = n4 * 4 + static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x; i < n; i += stride)
+    dN[i] = dY[i] * act_derive<ACT>(pre[i], post[i]);
+}
+
+// ---- out = a + b (fwp_st.cpp:5051-5112 with equal widths)
+__global__ __launch_bounds__(kEwBlock) void k_add(float const *__restrict__ a, float const *__restrict__ b,
+                                                   float *__restrict__ out, size_t n4, size_t n) {
+  size_t const stride = static_cast<size_t>(gridDim.x) * kEwBlock;
+  size_t i = static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x;
+  for (; i < n4; i += stride) {
+    float4 const u = reinterpret_cast<float4 const *>(a)[i];
+    float4 const v = reinterpret_cast<float4 const *>(b)[i];
+    reinterpret_cast<float4 *>(out)[i] = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
+  }
+  for (i = n4 * 4 + static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x; i < n; i += stride) out[i] = a[i] + b[i];
+}
+
+// ---- per-unit row kernels: element e = b*H + j, unit j = e % H ----------------
+// mode 0: Z += bias                                     (fwp_st.cpp:4498-4516)
+// mode 1: dropout, kind/per_element/scale in the args   (fwp_st.cpp:4830-4904)
+// mode 2: y = f(gamma*((x-mov_mean)/mov_std)+beta) [* keep]  (fwp_st.cpp:4557-4584)
+struct RowArgs {
+  float const *x;
+  float *y;
+  float const *p0, *p1, *p2, *p3;  // per-unit vectors
+  uint8_t const *mask;
+  size_t B, H;
+  int drop_kind, per_element;
+  float scale;
+};
+
+template <int MODE, int ACT>
+__device__ __forceinline__ float row_op(RowArgs const &a, float v, size_t e, size_t j) {
+  if constexpr (MODE == 0) {
+    return v + a.p0[j];
+  } else if constexpr (MODE == 1) {
+    if (a.drop_kind == 3) return v * a.scale;  // inference rescale
+    uint8_t const m = a.per_element ? a.mask[e] : a.mask[j];
+    return a.drop_kind == 1 ? (m ? v : 0.0f) : (m ? v * a.scale : 0.0f);
+  } else {
+    float const nn = a.p0[j] * ((v - a.p2[j]) / a.p3[j]) + a.p1[j];
+    return act_fire<ACT>(nn) * a.scale;
+  }
+}
+
+template <int MODE, int ACT, int VEC>
+__global__ __launch_bounds__(kEwBlock) void k_row(RowArgs a) {
+  size_t const n = a.B * a.H;
+  size_t const stride = static_cast<size_t>(gridDim.x) * kEwBlock * VEC;
+  for (size_t e = (static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x) * VEC; e < n; e += stride) {
+    size_t const j = e % a.H;
+    if constexpr (VEC == 4) {
+      float4 v = *reinterpret_cast<float4 const *>(a.x + e);
+      v.x = row_op<MODE, ACT>(a, v.x, e, j);
+      v.y = row_op<MODE, ACT>(a, v.y, e + 1, j + 1);
+      v.z = row_op<MODE, ACT>(a, v.z, e + 2, j + 2);
+      v.w = row_op<MODE, ACT>(a, v.w, e + 3, j + 3);
+      *reinterpret_cast<float4 *>(a.y + e) = v;
+    } else {
+      a.y[e] = row_op<MODE, ACT>(a, a.x[e], e, j);
+    }
+  }
+}
+
+template <int MODE, int ACT>
+static int launch_row(dlmi_ctx *ctx, RowArgs const &a, char const *what) {
+  bool const vec4 = a.H % 4 == 0 && all_aligned16({a.x, a.y});
+  size_t const n = a.B * a.H;
+  if (vec4)
+    hipLaunchKernelGGL((k_row<MODE, ACT, 4>), dim3(ew_grid(ctx, n / 4)), dim3(kEwBlock), 0, ctx->stream, a);
+  else
+    hipLaunchKernelGGL((k_row<MODE, ACT, 1>), dim3(ew_grid(ctx, n)), dim3(kEwBlock), 0, ctx->stream, a);
+  DLMI_LAUNCH_CHECK(ctx, what);
+  return DLMI_OK;
+}
+
+// ---- softmax: one wavefront per row (fwp_st.cpp:4796-4828) -------------------
+__global__ __launch_bounds__(kEwBlock) void k_softmax(float const *__restrict__ x, float *__restrict__ y, size_t B,
+                                                       size_t H) {
+  int const lane = threadIdx.x & 63;
+  size_t const row = static_cast<size_t>(blockIdx.x) * (kEwBlock / 64) + threadIdx.x / 64;
+  if (row >= B) return;
+  float const *xi = x + row * H;
+  float *yi = y + row * H;
+  float mx = -3.402823466e+38f;
+  for (size_t i = lane; i < H; i += 64) mx = fmaxf(mx, xi[i]);
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+  float s = 0.0f;
+  for (size_t i = lane; i < H; i += 64) {
+    float const e = expf(xi[i] - mx);
+    yi[i] = e;
+    s += e;
+  }
+  for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+  s = 1.0f / s;
+  for (size_t i = lane; i < H; i += 64) yi[i] *= s;
+}
+
+// ---- softmax + cross-entropy seed gradient (compute_error_st.cpp:26-131,
+// compute_loss.cpp:88-95, 101-138).  One wavefront per row; the double
+// accumulators are combined with one atomic per block (they are reported
+// metrics, not part of the gradient).
+__global__ __launch_bounds__(kEwBlock) void k_softmax_ce_seed(float const *__restrict__ q, float const *__restrict__ y,
+                                                               float *__restrict__ dZ, size_t B, size_t H,
+                                                               double *__restrict__ stats) {
+  constexpr float kEps = 0.0000001f;  // data/dtypes.hpp:113
+  int const lane = threadIdx.x & 63;
+  size_t const row = static_cast<size_t>(blockIdx.x) * (kEwBlock / 64) + threadIdx.x / 64;
+  double loss = 0.0, correct = 0.0;
+  if (row < B) {
+    float const *qi = q + row * H;
+    float const *yi = y + row * H;
+    float const inv_b = static_cast<float>(B);
+    // S = sum_k q_k * dL_k  (dL_k != 0 only where y_k == 1)
+    float s = 0.0f, lsum = 0.0f;
+    float best = -3.402823466e+38f;
+    long long best_k = -1, target_k = static_cast<long long>(H);
+    for (size_t k = lane; k < H; k += 64) {
+      float const qk = qi[k];
+      float const c = qk < kEps ? kEps : (qk > 1.0f - kEps ? 1.0f - kEps : qk);
+      if (yi[k] == 1.0f) {
+        s += qk * ((-1.0f / c) / inv_b);
+        lsum += -(yi[k] * logf(c));
+        target_k = static_cast<long long>(k);  // last k with y == 1 wins below
+      }
+      if (qk >= best) { best = qk; best_k = static_cast<long long>(k); }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+      s += __shfl_xor(s, off, 64);
+      lsum += __shfl_xor(lsum, off, 64);
+      float const ob = __shfl_xor(best, off, 64);
+      long long const ok = __shfl_xor(best_k, off, 64);
+      // ">=" scan keeps the LAST maximal index (compute_error_st.cpp:62-68)
+      if (ob > best || (ob == best && ok > best_k)) { best = ob; best_k = ok; }
+      long long const ot = __shfl_xor(target_k, off, 64);
+      // the sequential scan keeps the last k with y_k == 1; H means "none"
+      long long const a = target_k == static_cast<long long>(H) ? -1 : target_k;
+      long long const b = ot == static_cast<long long>(H) ? -1 : ot;
+      long long const m = a > b ? a : b;
+      target_k = m < 0 ? static_cast<long long>(H) : m;
+    }
+    for (size_t i = lane; i < H; i += 64) {
+      float const qv = qi[i];
+      float const c = qv < kEps ? kEps : (qv > 1.0f - kEps ? 1.0f - kEps : qv);
+      float const dl = yi[i] == 1.0f ? (-1.0f / c) / inv_b : 0.0f;
+      // sum_k (q_i [i==k] - q_k q_i) dL_k = q_i dL_i - q_i S
+      dZ[row * H + i] = qv * dl - qv * s;
+    }
+    if (lane == 0) {
+      loss = static_cast<double>(lsum);
+      correct = (target_k == best_k) ? 1.0 : 0.0;
+    }
+  }
+  if (stats != nullptr) {
+    __shared__ double sh[2][kEwBlock / 64];
+    if (lane == 0) {
+      sh[0][threadIdx.x / 64] = loss;
+      sh[1][threadIdx.x / 64] = correct;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      double l = 0.0, c = 0.0;
+      for (int w = 0; w < kEwBlock / 64; ++w) { l += sh[0][w]; c += sh[1][w]; }
+      atomicAdd(&stats[0], l);
+      atomicAdd(&stats[1], c);
+    }
+  }
+}
+
+}  // namespace dlmi
+
+using namespace dlmi;
+
+extern "C" {
+
+int dlmi_act_fwd(dlmi_ctx *ctx, dlmi_activation act, size_t B, size_t H, float const *x, float *y) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, act_supported(act), "unsupported activation");
+  DLMI_REQUIRE(ctx, x && y, "null pointer");
+  size_t const n = B * H;
+  if (n == 0) return DLMI_OK;
+  size_t const n4 = all_aligned16({x, y}) ? n / 4 : 0;
+  unsigned const grid = ew_grid(ctx, n4 ? n4 : n);
+  DLMI_DISPATCH_ACT(act, hipLaunchKernelGGL((k_act_fwd<ACT>), dim3(grid), dim3(kEwBlock), 0, ctx->stream, x, y, n4, n));
+  DLMI_LAUNCH_CHECK(ctx, "k_act_fwd");
+  return DLMI_OK;
+}
+
+int dlmi_act_bwd(dlmi_ctx *ctx, dlmi_activation act, size_t B, size_t H, float const *pre, float const *post,
+                 float const *dY, float *dN) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, act_supported(act), "unsupported activation");
+  DLMI_REQUIRE(ctx, pre && post && dY && dN, "null pointer");
+  size_t const n = B * H;
+  if (n == 0) return DLMI_OK;
+  size_t const n4 = all_aligned16({pre, post, dY, dN}) ? n / 4 : 0;
+  unsigned const grid = ew_grid(ctx, n4 ? n4 : n);
+  DLMI_DISPATCH_ACT(act, hipLaunchKernelGGL((k_act_bwd<ACT>), dim3(grid), dim3(kEwBlock), 0, ctx->stream, pre, post,
+                                            dY, dN, n4, n));
+  DLMI_LAUNCH_CHECK(ctx, "k_act_bwd");
+  return DLMI_OK;
+}
+
+int dlmi_identity_add(dlmi_ctx *ctx, size_t n, float const *a, float const *b, float *out) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, a && b && out, "null pointer");
+  if (n == 0) return DLMI_OK;
+  size_t const n4 = all_aligned16({a, b, out}) ? n / 4 : 0;
+  hipLaunchKernelGGL(k_add, dim3(ew_grid(ctx, n4 ? n4 : n)), dim3(kEwBlock), 0, ctx->stream, a, b, out, n4, n);
+  DLMI_LAUNCH_CHECK(ctx, "k_add");
+  return DLMI_OK;
+}
+
+int dlmi_bias_fwd(dlmi_ctx *ctx, size_t B, size_t H, float const *bias, float *Z) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, bias && Z, "null pointer");
+  if (B * H == 0) return DLMI_OK;
+  RowArgs a{};
+  a.x = Z; a.y = Z; a.p0 = bias; a.B = B; a.H = H; a.scale = 1.0f;
+  return launch_row<0, DLMI_ACT_LINEAR>(ctx, a, "k_row<bias>");
+}
+
+int dlmi_dropout_fwd(dlmi_ctx *ctx, dlmi_dropout kind, int training, int per_element, size_t B, size_t H,
+                     uint8_t const *mask, float scale, float *v) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, v != nullptr, "null pointer");
+  DLMI_REQUIRE(ctx, kind == DLMI_DROP_NONE || kind == DLMI_DROP_BERNOULLI || kind == DLMI_DROP_BERNOULLI_INVERTED,
+               "unsupported dropout");
+  if (B * H == 0 || kind == DLMI_DROP_NONE) return DLMI_OK;
+  RowArgs a{};
+  a.x = v; a.y = v; a.mask = mask; a.B = B; a.H = H; a.per_element = per_element; a.scale = scale;
+  if (training) {
+    DLMI_REQUIRE(ctx, mask != nullptr, "training-mode dropout needs a mask");
+    a.drop_kind = kind == DLMI_DROP_BERNOULLI ? 1 : 2;
+  } else {
+    if (kind != DLMI_DROP_BERNOULLI) return DLMI_OK;  // inverted dropout is the identity at inference
+    a.drop_kind = 3;
+  }
+  return launch_row<1, DLMI_ACT_LINEAR>(ctx, a, "k_row<dropout>");
+}
+
+int dlmi_norm_fwd_infer(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float const *gamma, float const *beta,
+                        float const *mov_mean, float const *mov_std, float *out) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, x && gamma && beta && mov_mean && mov_std && out, "null pointer");
+  if (B * H == 0) return DLMI_OK;
+  RowArgs a{};
+  a.x = x; a.y = out; a.p0 = gamma; a.p1 = beta; a.p2 = mov_mean; a.p3 = mov_std; a.B = B; a.H = H; a.scale = 1.0f;
+  return launch_row<2, DLMI_ACT_LINEAR>(ctx, a, "k_row<norm_infer>");
+}
+
+int dlmi_fused_norm_act_infer(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
+                              float const *gamma, float const *beta, float const *mov_mean, float const *mov_std,
+                              float *y) {
+  if (ctx == nullptr || desc == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, act_supported(desc->act), "unsupported activation");
+  DLMI_REQUIRE(ctx, x && gamma && beta && mov_mean && mov_std && y, "null pointer");
+  if (B * H == 0) return DLMI_OK;
+  RowArgs a{};
+  a.x = x; a.y = y; a.p0 = gamma; a.p1 = beta; a.p2 = mov_mean; a.p3 = mov_std; a.B = B; a.H = H;
+  // plain Bernoulli rescales by the keep probability at inference (fwp_st.cpp:705-716)
+  a.scale = desc->dropout == DLMI_DROP_BERNOULLI ? desc->drop_scale : 1.0f;
+  int rc = DLMI_OK;
+  DLMI_DISPATCH_ACT(desc->act, rc = (launch_row<2, ACT>(ctx, a, "k_row<norm_act_infer>")));
+  return rc;
+}
+
+int dlmi_softmax_fwd(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *y) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, x && y, "null pointer");
+  if (B * H == 0) return DLMI_OK;
+  hipLaunchKernelGGL(k_softmax, dim3(static_cast<unsigned>(dlmi_ceil_div(B, kEwBlock / 64))), dim3(kEwBlock), 0,
+                     ctx->stream, x, y, B, H);
+  DLMI_LAUNCH_CHECK(ctx, "k_softmax");
+  return DLMI_OK;
+}
+
+int dlmi_softmax_ce_seed(dlmi_ctx *ctx, size_t B, size_t H, float const *q, float const *y, float *dZ,
+                         double *stats) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, q && y && dZ, "null pointer");
+  if (B * H == 0) return DLMI_OK;
+  hipLaunchKernelGGL(k_softmax_ce_seed, dim3(static_cast<unsigned>(dlmi_ceil_div(B, kEwBlock / 64))), dim3(kEwBlock),
+                     0, ctx->stream, q, y, dZ, B, H, stats);
+  DLMI_LAUNCH_CHECK(ctx, "k_softmax_ce_seed");
+  return DLMI_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,387 @@
+// FP32 matrix-core (MFMA) contractions of the fully-connected layer for gfx950:
+//
+//   forward  Z  = X   * W^T   M=B, N=H,  K=K    A k-contiguous, B k-contiguous
+//   dX       dY = dZn * Wn    M=B, N=H,  K=Hn   A k-contiguous, B n-contiguous
+//   dW       dW = dZ^T * Xin  M=H, N=K,  K=B    A m-contiguous, B n-contiguous
+//
+// (reference leaves: v1/learner/fwp_st.cpp:4518-4555, bwp_st.cpp:1009-1045,
+//  update_derivative_fwp_st.cpp:246-281 under /root/reference/lib/deep-learning.)
+//
+// One kernel template covers the three operand layouts.  A 256-thread
+// workgroup (4 wavefronts, 2 x 2) owns a BM x BN tile of C; each wavefront
+// owns (BM/2) x (BN/2) as a grid of 32x32 v_mfma_f32_32x32x2_f32 blocks whose
+// accumulators stay in registers for the whole K loop.  Operand tiles are
+// staged through LDS (double buffered, one barrier per K tile) while the next
+// tile's global loads are already in flight in registers.
+//
+// The MFMA consumes two k per instruction: lanes 0-31 supply k_lo, lanes 32-63
+// k_hi.  Because the sum over k is order-free inside a tile, the kernel feeds
+// k = {s, s+4} (s = 0..3) of every group of 8 instead of {2s, 2s+1}: a lane
+// then needs 4 CONSECUTIVE k of one row, i.e. one ds_read_b128 per 4 MFMAs for
+// k-contiguous operands.  Rows are padded by 4 floats so those 16-byte reads
+// hit distinct banks.
+//
+// Workgroup ids are remapped so that (a) the ids that land on one XCD (id % 8)
+// cover a compact block of tiles and (b) tiles are walked in groups of 8 rows
+// of tiles, which keeps the A and B panels of concurrently running workgroups
+// resident in that XCD's L2.
+#include <initializer_list>
+
+#include "dlmi_common.hpp"
+
+namespace dlmi {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kGemmThreads = 256;
+constexpr int kXcds = 8;
+constexpr int kGroupM = 8;
+
+struct GemmArgs {
+  float const *A;
+  float const *B;
+  float *C;
+  float const *bias;  // per-n, may be null
+  size_t M, N, K;
+  size_t lda, ldb, ldc;
+  size_t k_per_split;  // K range of one blockIdx.z slice (multiple of BK)
+  float *split_out;    // when gridDim.z > 1: [splits][M][N] partial products
+  int accumulate;      // C += result (only when gridDim.z == 1)
+  unsigned tiles_m, tiles_n;
+};
+
+// LDS tile of an operand whose k index is contiguous in memory: [ROWS][BK+4].
+// LDS tile of an operand whose row (m or n) index is contiguous:  [BK][ROWS+PAD].
+template <int ROWS, int BK, bool KCONTIG>
+struct TileShape {
+  static constexpr int kStride = KCONTIG ? BK + 4 : ROWS + 8;
+  static constexpr int kFloats = KCONTIG ? ROWS * (BK + 4) : BK * (ROWS + 8);
+  static constexpr int kVec4 = ROWS * BK / 4;             // float4 per tile
+  static constexpr int kPerThread = kVec4 / kGemmThreads;  // float4 per thread
+  static_assert(kVec4 % kGemmThreads == 0, "tile must divide evenly over the workgroup");
+};
+
+// Global -> registers for one operand tile.  `row0` is the tile's first row
+// (m or n), `k0` its first k.  FAST: whole tile in bounds, 16-byte aligned.
+template <int ROWS, int BK, bool KCONTIG, bool FAST>
+__device__ __forceinline__ void tile_load(float const *__restrict__ P, size_t ld, size_t row0, size_t k0,
+                                          size_t rows_total, size_t k_end,
+                                          float4 (&regs)[TileShape<ROWS, BK, KCONTIG>::kPerThread]) {
+  using T = TileShape<ROWS, BK, KCONTIG>;
+#pragma unroll
+  for (int i = 0; i < T::kPerThread; ++i) {
+    int const f = threadIdx.x + i * kGemmThreads;
+    size_t row, k;
+    if constexpr (KCONTIG) {
+      row = row0 + f / (BK / 4);
+      k = k0 + (f % (BK / 4)) * 4;
+    } else {
+      k = k0 + f / (ROWS / 4);
+      row = row0 + (f % (ROWS / 4)) * 4;
+    }
+    if constexpr (FAST) {
+      float const *src = KCONTIG ? P + row * ld + k : P + k * ld + row;
+      regs[i] = *reinterpret_cast<float4 const *>(src);
+    } else {
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        size_t const rr = KCONTIG ? row : row + e;
+        size_t const kk = KCONTIG ? k + e : k;
+        v[e] = (rr < rows_total && kk < k_end) ? (KCONTIG ? P[rr * ld + kk] : P[kk * ld + rr]) : 0.0f;
+      }
+      regs[i] = make_float4(v[0], v[1], v[2], v[3]);
+    }
+  }
+}
+
+template <int ROWS, int BK, bool KCONTIG>
+__device__ __forceinline__ void tile_store(float *__restrict__ lds,
+                                           float4 const (&regs)[TileShape<ROWS, BK, KCONTIG>::kPerThread]) {
+  using T = TileShape<ROWS, BK, KCONTIG>;
+#pragma unroll
+  for (int i = 0; i < T::kPerThread; ++i) {
+    int const f = threadIdx.x + i * kGemmThreads;
+    int off;
+    if constexpr (KCONTIG) {
+      off = (f / (BK / 4)) * T::kStride + (f % (BK / 4)) * 4;
+    } else {
+      off = (f / (ROWS / 4)) * T::kStride + (f % (ROWS / 4)) * 4;
+    }
+    *reinterpret_cast<float4 *>(lds + off) = regs[i];
+  }
+}
+
+// Fragment for 4 consecutive MFMA steps of one 32-row block: element s feeds
+// step s.  `r` = row inside the tile (block base + lane % 32), `kk` = first k
+// of this lane's 4 (group base + (lane / 32) * 4).
+template <int ROWS, int BK, bool KCONTIG>
+__device__ __forceinline__ float4 frag_load(float const *__restrict__ lds, int r, int kk) {
+  using T = TileShape<ROWS, BK, KCONTIG>;
+  if constexpr (KCONTIG) {
+    return *reinterpret_cast<float4 const *>(lds + r * T::kStride + kk);
+  } else {
+    return make_float4(lds[(kk + 0) * T::kStride + r], lds[(kk + 1) * T::kStride + r],
+                       lds[(kk + 2) * T::kStride + r], lds[(kk + 3) * T::kStride + r]);
+  }
+}
+
+__device__ __forceinline__ float f4_get(float4 const &v, int s) {
+  return s == 0 ? v.x : (s == 1 ? v.y : (s == 2 ? v.z : v.w));
+}
+
+template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, bool FAST>
+__global__ __launch_bounds__(kGemmThreads) void k_gemm_f32(GemmArgs g) {
+  using TA = TileShape<BM, BK, A_KCONTIG>;
+  using TB = TileShape<BN, BK, B_KCONTIG>;
+  constexpr int WM = BM / 2, WN = BN / 2;  // wavefront tile
+  constexpr int TM = WM / 32, TN = WN / 32;
+  static_assert(BK % 8 == 0, "K tile is consumed in groups of 8");
+  __shared__ __attribute__((aligned(16))) float lds[2 * (TA::kFloats + TB::kFloats)];
+
+  // ---- which tile: XCD-aware remap, then grouped ordering -------------------
+  unsigned const ntiles = g.tiles_m * g.tiles_n;
+  unsigned lid = blockIdx.x;
+  if (ntiles % kXcds == 0) lid = (blockIdx.x % kXcds) * (ntiles / kXcds) + blockIdx.x / kXcds;
+  unsigned const per_group = kGroupM * g.tiles_n;
+  unsigned const first_m = (lid / per_group) * kGroupM;
+  unsigned const gsize = (g.tiles_m - first_m) < kGroupM ? (g.tiles_m - first_m) : kGroupM;
+  unsigned const tile_m = first_m + (lid % per_group) % gsize;
+  unsigned const tile_n = (lid % per_group) / gsize;
+  size_t const m0 = static_cast<size_t>(tile_m) * BM;
+  size_t const n0 = static_cast<size_t>(tile_n) * BN;
+
+  size_t const k_begin = blockIdx.z * g.k_per_split;
+  size_t const k_end = (k_begin + g.k_per_split < g.K) ? k_begin + g.k_per_split : g.K;
+  int const ktiles = static_cast<int>((k_end - k_begin + BK - 1) / BK);
+
+  int const lane = threadIdx.x & 63;
+  int const wave = threadIdx.x >> 6;
+  int const wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
+  int const lr = lane & 31;         // row inside a 32-block (A: m, B: n)
+  int const lk = (lane >> 5) * 4;   // this lane's k offset inside a group of 8
+
+  v16f acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  float4 ra[TA::kPerThread], rb[TB::kPerThread];
+  constexpr int kStage = TA::kFloats + TB::kFloats;  // stage s: A at s*kStage, B right after it
+
+  if (ktiles > 0) {
+    tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, k_begin, g.M, k_end, ra);
+    tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, k_begin, g.N, k_end, rb);
+    tile_store<BM, BK, A_KCONTIG>(lds, ra);
+    tile_store<BN, BK, B_KCONTIG>(lds + TA::kFloats, rb);
+  }
+  __syncthreads();
+
+  for (int kt = 0; kt < ktiles; ++kt) {
+    int const cur = kt & 1;
+    bool const more = kt + 1 < ktiles;
+    if (more) {  // next tile's global loads fly while this tile is multiplied
+      size_t const kn = k_begin + static_cast<size_t>(kt + 1) * BK;
+      tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, kn, g.M, k_end, ra);
+      tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, kn, g.N, k_end, rb);
+    }
+    float const *const sa = lds + cur * kStage;
+    float const *const sb = sa + TA::kFloats;
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 8) {
+      float4 fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[i] = frag_load<BM, BK, A_KCONTIG>(sa, wm0 + i * 32 + lr, kk + lk);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fb[j] = frag_load<BN, BK, B_KCONTIG>(sb, wn0 + j * 32 + lr, kk + lk);
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(f4_get(fa[i], s), f4_get(fb[j], s), acc[i][j], 0, 0, 0);
+    }
+    if (more) {
+      tile_store<BM, BK, A_KCONTIG>(lds + (cur ^ 1) * kStage, ra);
+      tile_store<BN, BK, B_KCONTIG>(lds + (cur ^ 1) * kStage + TA::kFloats, rb);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: accumulator register e of lane l holds
+  //      row (e/4)*8 + (l/32)*4 + e%4, column l%32 of its 32x32 block
+  bool const split = gridDim.z > 1;
+  float *const out = split ? g.split_out + static_cast<size_t>(blockIdx.z) * g.M * g.N : g.C;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      size_t const col = n0 + wn0 + j * 32 + lr;
+      float const bv = (!split && g.bias != nullptr && (FAST || col < g.N)) ? g.bias[col] : 0.0f;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        size_t const row = m0 + wm0 + i * 32 + (e / 4) * 8 + (lane >> 5) * 4 + (e % 4);
+        if (FAST || (row < g.M && col < g.N)) {
+          float *p = out + row * g.ldc + col;
+          float v = acc[i][j][e] + bv;
+          if (!split && g.accumulate) v += *p;
+          *p = v;
+        }
+      }
+    }
+}
+
+// Fixed-order sum of the split-K partial products (+ bias, + previous C).
+__global__ __launch_bounds__(256) void k_splitk_reduce(float const *__restrict__ part, unsigned splits, size_t mn,
+                                                        size_t N, float const *__restrict__ bias,
+                                                        float *__restrict__ C, int accumulate) {
+  size_t const stride = static_cast<size_t>(gridDim.x) * 256;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < mn; i += stride) {
+    float s = 0.0f;
+    for (unsigned z = 0; z < splits; ++z) s += part[z * mn + i];
+    if (bias != nullptr) s += bias[i % N];
+    if (accumulate) s += C[i];
+    C[i] = s;
+  }
+}
+
+// db[h] (+)= sum_b dZ[b,h]: column sums over the batch in a fixed order
+// (update_derivative_fwp_st.cpp:283-302).  Thread per column group, blocks
+// over batch chunks, partials combined by k_colsum_finish.
+__global__ __launch_bounds__(256) void k_colsum_partial(float const *__restrict__ x, size_t B, size_t H,
+                                                         size_t rows_per_chunk, float *__restrict__ partial) {
+  size_t const j = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (j >= H) return;
+  size_t const b0 = blockIdx.y * rows_per_chunk;
+  size_t const b1 = (b0 + rows_per_chunk < B) ? b0 + rows_per_chunk : B;
+  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+  size_t b = b0;
+  for (; b + 3 < b1; b += 4) {
+    s0 += x[(b + 0) * H + j];
+    s1 += x[(b + 1) * H + j];
+    s2 += x[(b + 2) * H + j];
+    s3 += x[(b + 3) * H + j];
+  }
+  for (; b < b1; ++b) s0 += x[b * H + j];
+  partial[static_cast<size_t>(blockIdx.y) * H + j] = (s0 + s1) + (s2 + s3);
+}
+
+__global__ __launch_bounds__(256) void k_colsum_finish(float const *__restrict__ partial, unsigned nchunks, size_t H,
+                                                        float *__restrict__ out, int accumulate) {
+  size_t const j = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (j >= H) return;
+  float s = 0.0f;
+  for (unsigned c = 0; c < nchunks; ++c) s += partial[static_cast<size_t>(c) * H + j];
+  out[j] = accumulate ? out[j] + s : s;
+}
+
+// ---------------------------------------------------------------- host side
+template <int BM, int BN, int BK, bool AK, bool BKC>
+static int launch_gemm(dlmi_ctx *ctx, GemmArgs g, unsigned splits, bool fast) {
+  g.tiles_m = static_cast<unsigned>(dlmi_ceil_div(g.M, BM));
+  g.tiles_n = static_cast<unsigned>(dlmi_ceil_div(g.N, BN));
+  dim3 const grid(g.tiles_m * g.tiles_n, 1, splits);
+  if (fast)
+    hipLaunchKernelGGL((k_gemm_f32<BM, BN, BK, AK, BKC, true>), grid, dim3(kGemmThreads), 0, ctx->stream, g);
+  else
+    hipLaunchKernelGGL((k_gemm_f32<BM, BN, BK, AK, BKC, false>), grid, dim3(kGemmThreads), 0, ctx->stream, g);
+  DLMI_LAUNCH_CHECK(ctx, "k_gemm_f32");
+  return DLMI_OK;
+}
+
+constexpr int kBM = 128, kBN = 128, kBK = 16;
+
+// C[M,N] (+)= A . B with the operand layouts given by the two flags.
+template <bool AK, bool BKC>
+static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, size_t lda, float const *B, size_t ldb,
+                float *C, float const *bias, int accumulate) {
+  GemmArgs g;
+  g.A = A; g.B = B; g.C = C; g.bias = bias; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldc = N;
+  g.accumulate = accumulate; g.split_out = nullptr;
+  bool const fast = M % kBM == 0 && N % kBN == 0 && K % kBK == 0 && lda % 4 == 0 && ldb % 4 == 0 &&
+                    dlmi_aligned16(A) && dlmi_aligned16(B);
+  // Split K when the output alone cannot fill the machine (few tiles, long K):
+  // each slice writes its partial product, a second kernel adds them in order.
+  size_t const tiles = dlmi_ceil_div(M, kBM) * dlmi_ceil_div(N, kBN);
+  size_t const ktiles = dlmi_ceil_div(K, kBK);
+  unsigned splits = 1;
+  size_t const target = static_cast<size_t>(ctx->num_cu) * 2;
+  if (tiles < target / 2 && ktiles >= 16) {
+    size_t s = dlmi_ceil_div(target, tiles);
+    size_t const max_s = ktiles / 8;  // at least 8 K tiles per slice
+    if (s > max_s) s = max_s;
+    if (s > 1) {
+      int rc = dlmi_scratch_reserve(ctx, s * M * N * sizeof(float));
+      if (rc != DLMI_OK) return rc;
+      splits = static_cast<unsigned>(s);
+    }
+  }
+  size_t const kt_per_split = dlmi_ceil_div(ktiles, splits);
+  g.k_per_split = kt_per_split * kBK;
+  splits = static_cast<unsigned>(dlmi_ceil_div(ktiles, kt_per_split));
+  if (splits > 1) g.split_out = reinterpret_cast<float *>(ctx->scratch);
+  int rc = launch_gemm<kBM, kBN, kBK, AK, BKC>(ctx, g, splits, fast);
+  if (rc != DLMI_OK) return rc;
+  if (splits > 1) {
+    size_t const mn = M * N;
+    size_t blocks = dlmi_ceil_div(mn, 256);
+    size_t const cap = static_cast<size_t>(ctx->num_cu) * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(k_splitk_reduce, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, ctx->stream,
+                       g.split_out, splits, mn, N, bias, C, accumulate);
+    DLMI_LAUNCH_CHECK(ctx, "k_splitk_reduce");
+  }
+  return DLMI_OK;
+}
+
+}  // namespace dlmi
+
+using namespace dlmi;
+
+extern "C" {
+
+int dlmi_fc_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, float const *W, float const *bias,
+                float *Z) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, X && W && Z, "null pointer");
+  DLMI_REQUIRE(ctx, B > 0 && K > 0 && H > 0, "empty operand");
+  return gemm<true, true>(ctx, B, H, K, X, K, W, K, Z, bias, 0);
+}
+
+int dlmi_fc_bwd_dx(dlmi_ctx *ctx, size_t B, size_t Hn, size_t H, float const *dZn, float const *Wn, float *dY,
+                   int accumulate) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, dZn && Wn && dY, "null pointer");
+  DLMI_REQUIRE(ctx, B > 0 && Hn > 0 && H > 0, "empty operand");
+  return gemm<true, false>(ctx, B, H, Hn, dZn, Hn, Wn, H, dY, nullptr, accumulate);
+}
+
+int dlmi_fc_bwd_dw(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float *dW,
+                   float *db, int accumulate) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, Xin && dZ && dW, "null pointer");
+  DLMI_REQUIRE(ctx, B > 0 && K > 0 && H > 0, "empty operand");
+  int rc = gemm<false, false>(ctx, H, K, B, dZ, H, Xin, K, dW, nullptr, accumulate);
+  if (rc != DLMI_OK || db == nullptr) return rc;
+  size_t chunks = dlmi_ceil_div(static_cast<size_t>(ctx->num_cu) * 4, dlmi_ceil_div(H, 256));
+  if (chunks > dlmi_ceil_div(B, 32)) chunks = dlmi_ceil_div(B, 32);
+  if (chunks < 1) chunks = 1;
+  size_t const rows = dlmi_ceil_div(B, chunks);
+  chunks = dlmi_ceil_div(B, rows);
+  rc = dlmi_scratch_reserve(ctx, chunks * H * sizeof(float));
+  if (rc != DLMI_OK) return rc;
+  float *partial = reinterpret_cast<float *>(ctx->scratch);
+  hipLaunchKernelGGL(k_colsum_partial, dim3(static_cast<unsigned>(dlmi_ceil_div(H, 256)), static_cast<unsigned>(chunks)),
+                     dim3(256), 0, ctx->stream, dZ, B, H, rows, partial);
+  DLMI_LAUNCH_CHECK(ctx, "k_colsum_partial");
+  hipLaunchKernelGGL(k_colsum_finish, dim3(static_cast<unsigned>(dlmi_ceil_div(H, 256))), dim3(256), 0, ctx->stream,
+                     partial, static_cast<unsigned>(chunks), H, db, accumulate);
+  DLMI_LAUNCH_CHECK(ctx, "k_colsum_finish");
+  return DLMI_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,222 @@
+/* dlmi — MI355X (gfx950) implementation of the fully-connected / batch
+ * (re)normalization / activation hot path of SebastienKeroack/deep-learning.
+ *
+ * C ABI.  Every pointer argument marked "device" is a HIP device pointer to
+ * fp32 (or uint8 for masks); sizes are element counts.  All tensors are
+ * row-major [B, H]: element (b, j) lives at b*H + j, the layout of the
+ * reference's activations (lib/deep-learning/v1/learner/fwp_st.cpp:4538-4542).
+ * Weights are [H][K] row-major, one output unit's fan-in contiguous
+ * (v1/learner/connections_prepare.cpp:25-45), so the forward product is
+ * Z = X * W^T.
+ *
+ * Every call is asynchronous on the context's HIP stream and returns
+ * DLMI_OK (0) or a negative DLMI_E_* code; dlmi_last_error() gives the text.
+ * Nothing here falls back to the CPU: without a GPU, dlmi_ctx_create fails.
+ *
+ * File:line citations are relative to /root/reference/lib/deep-learning/.
+ */
+#ifndef DLMI_H
+#define DLMI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DLMI_OK 0
+#define DLMI_E_INVALID (-1) /* bad argument (null pointer, unknown enum, size 0 where not allowed) */
+#define DLMI_E_HIP (-2)     /* a HIP runtime call failed */
+#define DLMI_E_NOMEM (-3)   /* scratch allocation failed */
+#define DLMI_E_UNSUPPORTED (-4)
+
+/* Values identical to the reference's enums so callers can pass them through:
+ * v1/data/enum/activation.hpp:24-53 */
+typedef enum {
+  DLMI_ACT_ELU = 3,
+  DLMI_ACT_ISRLU = 10,
+  DLMI_ACT_LINEAR = 11,
+  DLMI_ACT_LEAKY_RELU = 14,
+  DLMI_ACT_RELU = 16,
+  DLMI_ACT_SELU = 17,
+  DLMI_ACT_SOFTMAX = 22
+} dlmi_activation;
+
+/* v1/data/enum/layer_norm.hpp:24-26 */
+typedef enum { DLMI_NORM_NONE = 0, DLMI_NORM_BATCH = 1, DLMI_NORM_BATCH_RENORM = 2 } dlmi_norm;
+
+/* v1/data/enum/layer_dropout.hpp:24-28 */
+typedef enum { DLMI_DROP_NONE = 0, DLMI_DROP_BERNOULLI = 2, DLMI_DROP_BERNOULLI_INVERTED = 3 } dlmi_dropout;
+
+/* How the fused backward treats dropout.
+ * REFERENCE: what the reference's CPU backward does — the gradient is NOT
+ *   masked or rescaled; the activation derivative merely sees the post-dropout
+ *   output q (bwp_st.cpp:1177-1209 reads AF_unit::ptr_array_values, which
+ *   fwp_st.cpp:657-732 has overwritten in place).
+ * MASKED: the mathematically matching backward, dY * mask * scale * f'(n, q)
+ *   with q the pre-dropout activation. */
+typedef enum { DLMI_DROP_BWD_REFERENCE = 0, DLMI_DROP_BWD_MASKED = 1 } dlmi_dropout_bwd;
+
+typedef struct dlmi_ctx dlmi_ctx;
+
+/* ---- context ------------------------------------------------------------- */
+/* device: HIP device ordinal.  stream: a hipStream_t (NULL = default stream).
+ * The context owns a device scratch buffer for reduction partials. */
+int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream);
+int dlmi_ctx_destroy(dlmi_ctx *ctx);
+int dlmi_ctx_set_stream(dlmi_ctx *ctx, void *stream);
+int dlmi_ctx_synchronize(dlmi_ctx *ctx);
+const char *dlmi_last_error(dlmi_ctx const *ctx);
+/* Compute units of the context's device (for callers sizing their own work). */
+int dlmi_ctx_compute_units(dlmi_ctx const *ctx);
+
+/* ---- fully-connected contractions (fp32 MFMA) ----------------------------- */
+/* Z[b,h] = sum_k X[b,k] * W[h,k] (+ bias[h] if bias != NULL); overwrites Z.
+ * Replaces Model::Forward_Pass__FC__{Loop,OpenMP} (v1/learner/fwp_st.cpp:4518-4555,
+ * fwp_mp.cpp:4419-4459) and, when bias is given, Forward_Pass__Bias__*
+ * (fwp_st.cpp:4498-4516).  X [B,K], W [H,K], bias [H], Z [B,H]: device. */
+int dlmi_fc_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, float const *W,
+                float const *bias, float *Z);
+
+/* dY[b,c] (+)= sum_i dZn[b,i] * Wn[i,c].  accumulate != 0 adds into dY like the
+ * reference (which clears the buffer first, bwp_st.cpp:115); 0 overwrites.
+ * Replaces Model::Backward_Pass__FC__{Loop,OpenMP} (bwp_st.cpp:1009-1045,
+ * bwp_mp.cpp:968-1007).  dZn [B,Hn], Wn [Hn,H], dY [B,H]: device. */
+int dlmi_fc_bwd_dx(dlmi_ctx *ctx, size_t B, size_t Hn, size_t H, float const *dZn, float const *Wn,
+                   float *dY, int accumulate);
+
+/* dW[h,k] (+)= sum_b dZ[b,h] * Xin[b,k];  db[h] (+)= sum_b dZ[b,h] (db may be
+ * NULL: normalized layers have no bias, v1/learner/model.hpp:708).
+ * Replaces Model::Update_Derivative_Weight__FC__* and …__Bias__*
+ * (update_derivative_fwp_st.cpp:246-302, update_derivative_fwp_mp.cpp:175-240)
+ * together with the thread merge of merge.cpp:76-100.
+ * Xin [B,K], dZ [B,H], dW [H,K], db [H]: device. */
+int dlmi_fc_bwd_dw(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ,
+                   float *dW, float *db, int accumulate);
+
+/* Z[b,h] += bias[h]  (Forward_Pass__Bias__*, fwp_st.cpp:4498-4516). */
+int dlmi_bias_fwd(dlmi_ctx *ctx, size_t B, size_t H, float const *bias, float *Z);
+
+/* ---- batch (re)normalization, un-fused (materialises x_hat and out) -------- */
+/* Training-mode forward.  norm = DLMI_NORM_BATCH or DLMI_NORM_BATCH_RENORM.
+ * Per unit j, in this order (fwp_st.cpp:4709-4746):
+ *   mean = S1/B; mov_mean += m*(mean-mov_mean); std = sqrt(S2/B - mean^2 + eps);
+ *   mov_std += m*(std-mov_std); r = clip(std/mov_std, 1/r_max, r_max);
+ *   d = clip((mean-mov_mean)/mov_std, -d_max, d_max)   (r, d only for renorm)
+ * then x_hat = (x-mean)/std*r + d, out = gamma*x_hat + beta.
+ * The "std" outputs are standard deviations, as in the reference's "variance"
+ * arrays.  x [B,H]; gamma, beta, mean, std, mov_mean, mov_std, r, d [H]; xhat,
+ * out [B,H] (either may be NULL to skip that store): device.
+ * Replaces Forward_Pass__Batch_{Normalization,Renormalization}__Training__*
+ * (fwp_st.cpp:4586-4766, fwp_mp.cpp:4493-4739). */
+int dlmi_norm_fwd_train(dlmi_ctx *ctx, dlmi_norm norm, size_t B, size_t H, float momentum, float eps,
+                        float r_max, float d_max, float const *x, float const *gamma,
+                        float const *beta, float *mean, float *std, float *mov_mean, float *mov_std,
+                        float *r, float *d, float *xhat, float *out);
+
+/* out = gamma * ((x - mov_mean) / mov_std) + beta — divides by the moving
+ * standard deviation, no epsilon.  Replaces
+ * Forward_Pass__Batch_Normalization__Inference__* (fwp_st.cpp:4557-4584). */
+int dlmi_norm_fwd_infer(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float const *gamma,
+                        float const *beta, float const *mov_mean, float const *mov_std, float *out);
+
+/* Backward of the above (r, d are constants).  dgamma, dbeta accumulate (+=)
+ * like the reference; dmean, dstd are outputs (may be NULL); dx may alias dN.
+ * Replaces Backward_Pass__Batch_{Normalization,Renormalization}__*
+ * (bwp_st.cpp:1284-1366, 1447-1532; bwp_mp.cpp:1265-1385, 1504-1627). */
+int dlmi_norm_bwd(dlmi_ctx *ctx, dlmi_norm norm, size_t B, size_t H, float const *mean,
+                  float const *std, float const *gamma, float const *r, float const *x,
+                  float const *xhat, float const *dN, float *dgamma, float *dbeta, float *dmean,
+                  float *dstd, float *dx);
+
+/* ---- activations, dropout, add, softmax ------------------------------------ */
+/* y = f(x) for one activation type per layer (the reference sets a layer's
+ * units all at once, v1/learner/train.cpp:285-472).  Replaces
+ * Forward_Pass__FC_AF__* (fwp_st.cpp:4768-4794) + AF_FIRE
+ * (v1/ops/activations/functions.hpp:124-220).  y may alias x. */
+int dlmi_act_fwd(dlmi_ctx *ctx, dlmi_activation act, size_t B, size_t H, float const *x, float *y);
+
+/* dN = dY * f'(pre, post), with the reference's derivative forms
+ * (functions.hpp:88,92,99,103,107; v1/learner/model.cpp:2594-2651):
+ * ELU' = post (x<0), SELU' = scale*(post+alpha) (x<=0), ISRLU' = (post/pre)^3 (x<0).
+ * Replaces Backward_Pass__FC__DF__* (bwp_st.cpp:1177-1209).  dN may alias dY. */
+int dlmi_act_bwd(dlmi_ctx *ctx, dlmi_activation act, size_t B, size_t H, float const *pre,
+                 float const *post, float const *dY, float *dN);
+
+/* Row-wise softmax (Forward_Pass__FC_AF__Softmax__*, fwp_st.cpp:4796-4828). */
+int dlmi_softmax_fwd(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *y);
+
+/* In place on v [B,H].  kind = DLMI_DROP_BERNOULLI_INVERTED: mask ? v*scale : 0;
+ * DLMI_DROP_BERNOULLI: mask ? v : 0; training != 0.  With training == 0 only
+ * DLMI_DROP_BERNOULLI acts: v *= scale (scale = keep probability).
+ * mask is uint8 (0/1): [H] shared by all rows when per_element == 0 (the
+ * reference's bool mask per unit, fwp_st.cpp:4846-4856) or [B,H] when
+ * per_element != 0.  Replaces Forward_Pass__Dropout__Bernoulli__*
+ * (fwp_st.cpp:4830-4904). */
+int dlmi_dropout_fwd(dlmi_ctx *ctx, dlmi_dropout kind, int training, int per_element, size_t B,
+                     size_t H, uint8_t const *mask, float scale, float *v);
+
+/* out = a + b (Forward_Pass__Zero_Padded_Identity__* with equal widths and no
+ * padding, fwp_st.cpp:5051-5112; also the gradient fan-out of
+ * Backward_Pass__Residual__*, bwp_st.cpp:1112-1175).  out may alias a or b. */
+int dlmi_identity_add(dlmi_ctx *ctx, size_t n, float const *a, float const *b, float *out);
+
+/* Softmax + cross-entropy seed gradient of the output layer:
+ * dZ_i = sum_k (q_i [i==k] - q_k q_i) * dL_k,  dL_k = (y_k==1 ? -1/clip(q_k,1e-7,1-1e-7) : 0)/B.
+ * stats (device, 2 doubles, may be NULL) accumulates { sum of CE losses, number
+ * of rows whose arg-max matches the target } like the reference's accumulators.
+ * Replaces compute_error_fwp_{st,mp} (v1/learner/compute_error_st.cpp:26-131) with
+ * loss_fn_derivative (compute_loss.cpp:101-138). */
+int dlmi_softmax_ce_seed(dlmi_ctx *ctx, size_t B, size_t H, float const *q, float const *y,
+                         float *dZ, double *stats);
+
+/* ---- the fused hot path ----------------------------------------------------
+ * One training-mode layer tail: x (= Z) -> batch (re)norm -> activation ->
+ * optional dropout, without materialising x_hat or the pre-activation.
+ *
+ * Forward (3 launches): column statistics (wavefront shuffles + LDS tree over
+ * batch chunks), per-unit finalize, one coalesced pass reading x and writing y.
+ * Algorithmic HBM traffic 12 B/element (+1 with a per-element mask).
+ * Backward (3 launches): reduction pass reading dY and x (recomputing x_hat,
+ * the pre-activation and the activation), per-unit finalize, one pass reading
+ * dY and x and writing dX: 20 B/element (+2 with a per-element mask).
+ */
+typedef struct {
+  dlmi_norm norm;          /* DLMI_NORM_BATCH or DLMI_NORM_BATCH_RENORM */
+  dlmi_activation act;     /* any but SOFTMAX */
+  dlmi_dropout dropout;    /* NONE, BERNOULLI or BERNOULLI_INVERTED */
+  int mask_per_element;    /* 0: mask [H] (reference semantics), 1: mask [B,H] */
+  dlmi_dropout_bwd dropout_bwd;
+  float momentum, eps, r_max, d_max;
+  float drop_scale;        /* 1/keep for BERNOULLI_INVERTED (0 if keep == 0) */
+} dlmi_fused_desc;
+
+/* y [B,H] out; mean, std, r, d [H] out (kept for the backward); mov_mean,
+ * mov_std [H] in/out.  Composition of the reference's leaves a9/a10 -> a12 ->
+ * a14 in the order of Forward_Pass__FC__Loop (fwp_st.cpp:340-470, 657-700). */
+int dlmi_fused_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H,
+                            float const *x, float const *gamma, float const *beta,
+                            uint8_t const *mask, float *mean, float *std, float *mov_mean,
+                            float *mov_std, float *r, float *d, float *y);
+
+/* dX [B,H] out (may alias dY); dgamma, dbeta [H] accumulate (+=).  Composition
+ * of a19 -> a20/a21 in the order of Backward_Pass__Gradient__FC__Loop
+ * (bwp_st.cpp:543-701).  mean/std/r/d are the forward's outputs. */
+int dlmi_fused_norm_act_bwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H,
+                            float const *x, float const *gamma, float const *beta,
+                            uint8_t const *mask, float const *mean, float const *std,
+                            float const *r, float const *d, float const *dY, float *dgamma,
+                            float *dbeta, float *dX);
+
+/* Inference-mode tail: y = f(gamma*((x-mov_mean)/mov_std)+beta), then the
+ * inference branch of dropout (plain Bernoulli rescales by keep = drop_scale;
+ * inverted does nothing, fwp_st.cpp:705-716).  One pass, 8 B/element. */
+int dlmi_fused_norm_act_infer(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H,
+                              float const *x, float const *gamma, float const *beta,
+                              float const *mov_mean, float const *mov_std, float *y);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DLMI_H */

@@ -45,3 +45,32 @@ def golden_leaves():
 def golden_mlp():
     import numpy as np
     return np.load(os.path.join(ROOT, "tests", "golden", "mlp.npz"), allow_pickle=False)
+
+
+def load_package():
+    """Imports deep-learning_amd/ (hyphenated directory) as `deep_learning_amd`."""
+    import importlib.util
+    if "deep_learning_amd" in sys.modules:
+        return sys.modules["deep_learning_amd"]
+    pkg_dir = os.path.join(ROOT, "deep-learning_amd")
+    spec = importlib.util.spec_from_file_location("deep_learning_amd", os.path.join(pkg_dir, "__init__.py"),
+                                                  submodule_search_locations=[pkg_dir])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules["deep_learning_amd"] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+@pytest.fixture(scope="session")
+def pkg():
+    return load_package()
+
+
+@pytest.fixture(scope="session")
+def dl(pkg):
+    """A dlmi context on cuda:0.  GPU tests only; never falls back."""
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    d = pkg.Dlmi(0)
+    yield d
+    d.close()

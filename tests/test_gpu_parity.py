@@ -1,0 +1,338 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against
+(a) the golden vectors written by the real reference sources,
+(b) the CPU oracle on seeded random inputs (sizes it finishes in seconds),
+(c) size-independent properties at the full configuration sizes.
+
+Tolerances (fp32): 1e-5 relative for element-wise results, 1e-4 after
+reductions and GEMMs, relative to max(|expected|, rms(expected)) — see
+tests/helpers.py for why the tensor scale enters.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import RTOL_ELEMENTWISE as TE
+from helpers import RTOL_REDUCED as TR
+from helpers import assert_close
+from oracle.binding import ACT, DROP
+
+pytestmark = pytest.mark.gpu
+
+ACTS = ["ELU", "ISRLU", "LEAKY_RELU", "RELU", "SELU", "LINEAR"]
+
+
+def dev(a, dtype=torch.float32):
+    return torch.as_tensor(np.ascontiguousarray(a)).to("cuda", dtype=dtype).contiguous()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+# ------------------------------------------------------------------ golden vectors
+SETTINGS = dict(
+    brn_loose=dict(fresh=True, mom=0.99, rmax=3.0, dmax=5.0, renorm=True),
+    brn_tight=dict(fresh=False, mom=0.05, rmax=1.1, dmax=0.05, renorm=True),
+    bn=dict(fresh=False, mom=0.3, rmax=1.0, dmax=0.0, renorm=False))
+
+
+@pytest.mark.parametrize("case", [0, 1, 2])
+def test_leaves_against_reference_golden(dl, golden_leaves, case):
+    g = golden_leaves
+    p, q = f"c{case}_", f"c{case}_t0_"
+    B, K, H = (int(v) for v in g[p + "shape"])
+    X, W, x = dev(g[p + "X"]), dev(g[p + "W"]), dev(g[p + "x"])
+    gamma, beta = dev(g[p + "gamma"]), dev(g[p + "beta"])
+    dN, dZ = dev(g[p + "dN"]), dev(g[p + "dZ"])
+    mask = dev(g[p + "mask"], torch.uint8)
+    assert_close(host(dl.fc_fwd(X, W)), g[q + "fc_fwd"], TR, "fc_fwd")
+    assert_close(host(dl.fc_fwd(X, W, dev(g[p + "bias"]))), g[q + "bias_fwd"], TR, "fc_fwd + bias")
+    assert_close(host(dl.bias_fwd(dev(g[q + "fc_fwd"]), dev(g[p + "bias"]))), g[q + "bias_fwd"], TE, "bias_fwd")
+    for sname, s in SETTINGS.items():
+        mm = dev(np.zeros(H, np.float32) if s["fresh"] else g[p + "mov_mean"])
+        ms = dev(np.ones(H, np.float32) if s["fresh"] else g[p + "mov_std"])
+        fw = dl.norm_fwd_train(x, gamma, beta, mm, ms, s["mom"], 1e-5, s["rmax"], s["dmax"], s["renorm"])
+        fw["mov_mean"], fw["mov_std"] = mm, ms
+        for k, v in fw.items():
+            assert_close(host(v), g[f"{q}{sname}_fwd_{k}"], TR, f"{sname} fwd {k}", floor=1.0 if k == "d" else 0.0)
+        e = {k: dev(g[f"{q}{sname}_fwd_{k}"]) for k in ("mean", "std", "r", "xhat")}
+        dg, db = dev(g[p + "gamma"] * 0.5), dev(g[p + "beta"] * 2)
+        bw = dl.norm_bwd(e["mean"], e["std"], gamma, e["r"], x, e["xhat"], dN, dg, db, renorm=s["renorm"])
+        bw["dgamma"], bw["dbeta"] = dg, db
+        for k, v in bw.items():
+            assert_close(host(v), g[f"{q}{sname}_bwd_{k}"], TR, f"{sname} bwd {k}")
+    assert_close(host(dl.norm_fwd_infer(x, gamma, beta, dev(g[p + "mov_mean"]), dev(g[p + "mov_std"]))),
+                 g[q + "norm_infer"], TE, "norm_infer")
+    for a in ACTS:
+        assert_close(host(dl.act_fwd(ACT[a], x)), g[f"{q}act_fwd_{a}"], TE, "act_fwd " + a)
+        assert_close(host(dl.act_bwd(ACT[a], x, dev(g[f"{q}act_fwd_{a}"]), dN)), g[f"{q}act_bwd_{a}"], TE,
+                     "act_bwd " + a)
+    assert_close(host(dl.softmax_fwd(x)), g[q + "softmax"], TE, "softmax")
+    inv = float(np.float32(1.0) / np.float32(0.7))
+    assert np.array_equal(host(dl.dropout_fwd(DROP["BERNOULLI_INVERTED"], x.clone(), mask, inv)), g[q + "drop_inverted"])
+    assert np.array_equal(host(dl.dropout_fwd(DROP["BERNOULLI"], x.clone(), mask, 0.0)), g[q + "drop_plain"])
+    assert np.array_equal(host(dl.dropout_fwd(DROP["BERNOULLI"], x.clone(), None, 0.7, training=False)),
+                          g[q + "drop_infer"])
+    assert np.array_equal(host(dl.dropout_fwd(DROP["BERNOULLI_INVERTED"], x.clone(), None, 0.7, training=False)),
+                          g[p + "x"])
+    assert np.array_equal(host(dl.identity_add(x, dN)), g[q + "identity_add"])
+    assert_close(host(dl.fc_bwd_dx(dZ, W)), g[q + "fc_bwd_dx"], TR, "fc_bwd_dx")
+    acc = torch.ones(B, K, device="cuda")
+    assert_close(host(dl.fc_bwd_dx(dZ, W, out=acc, accumulate=True)), g[q + "fc_bwd_dx_acc"], TR, "fc_bwd_dx +=")
+    dW, db = dev(g[p + "dW0"]), dev(g[p + "db0"])
+    dl.fc_bwd_dw(X, dZ, dW=dW, db=db, accumulate=True)
+    assert_close(host(dW), g[q + "fc_bwd_dw"], TR, "fc_bwd_dw")
+    assert_close(host(db), g[q + "fc_bwd_db"], TR, "fc_bwd_db")
+
+
+@pytest.mark.parametrize("a", ACTS)
+def test_activation_special_points(dl, golden_leaves, a):
+    g = golden_leaves
+    pts = dev(g["pts"])
+    y = host(dl.act_fwd(ACT[a], pts))
+    assert_close(y, g[f"pts_fwd_{a}"], TE, "fwd " + a)
+    assert np.array_equal(np.signbit(y), np.signbit(g[f"pts_fwd_{a}"]))
+    d = host(dl.act_bwd(ACT[a], pts, dev(g[f"pts_fwd_{a}"]), torch.ones_like(pts)))
+    assert_close(d, g[f"pts_bwd_{a}"], TE, "bwd " + a)
+
+
+# ------------------------------------------------------------------ GEMMs against the oracle
+GEMM_SHAPES = [  # (B, K, H): tile-aligned (fast path) and ragged (guarded path)
+    (128, 128, 128), (256, 64, 384), (384, 256, 128), (1, 1, 1), (7, 13, 5), (130, 70, 129), (128, 784, 512),
+    (128, 512, 10), (33, 1000, 17), (512, 16, 256)]
+
+
+@pytest.mark.parametrize("B,K,H", GEMM_SHAPES)
+def test_gemms_against_oracle(dl, oracle, B, K, H):
+    rng = np.random.default_rng(B * 7 + K * 3 + H)
+    X = rng.standard_normal((B, K)).astype(np.float32)
+    W = (rng.uniform(-1, 1, (H, K)) * np.sqrt(6.0 / (K + H))).astype(np.float32)
+    bias = rng.uniform(-.5, .5, H).astype(np.float32)
+    dZ = rng.standard_normal((B, H)).astype(np.float32)
+    nt = oracle.max_threads()
+    Zo = oracle.fc_fwd(X, W, nt)
+    assert_close(host(dl.fc_fwd(dev(X), dev(W))), Zo, TR, "Z = X W^T")
+    assert_close(host(dl.fc_fwd(dev(X), dev(W), dev(bias))), oracle.bias_fwd(Zo, bias), TR, "Z + b")
+    assert_close(host(dl.fc_bwd_dx(dev(dZ), dev(W))), oracle.fc_bwd_dx(dZ, W, nthreads=nt), TR, "dX")
+    dWo, dbo = oracle.fc_bwd_dw(X, dZ, nthreads=nt)
+    dW, db = dl.fc_bwd_dw(dev(X), dev(dZ), with_bias=True)
+    assert_close(host(dW), dWo, TR, "dW")
+    assert_close(host(db), dbo, TR, "db")
+
+
+def test_gemm_split_k_tall_skinny(dl, oracle):
+    """dW of a tall batch and a narrow layer: few output tiles, long reduction
+    (the shape class of the 65536 x 256 x 256 configuration, scaled so the CPU
+    oracle finishes in seconds)."""
+    rng = np.random.default_rng(5)
+    B, K, H = 8192, 256, 256
+    X = rng.standard_normal((B, K)).astype(np.float32)
+    dZ = rng.standard_normal((B, H)).astype(np.float32)
+    dWo, dbo = oracle.fc_bwd_dw(X, dZ, nthreads=oracle.max_threads())
+    dW0 = rng.standard_normal((H, K)).astype(np.float32)
+    dW = dev(dW0)
+    db = torch.zeros(H, device="cuda")
+    dl.fc_bwd_dw(dev(X), dev(dZ), dW=dW, db=db, accumulate=True)
+    assert_close(host(dW), dWo + dW0, TR, "dW split-K, accumulate")
+    assert_close(host(db), dbo, TR, "db")
+
+
+def test_gemm_full_size_adjoint_and_library(dl):
+    """[8192 x 4096 x 4096]: <dZ, X W^T> = <dZ W, X> = <dZ^T X, W>, and each
+    product against the library GEMM in float64 on a slab of rows/columns."""
+    torch.manual_seed(3)
+    B, K, H = 8192, 4096, 4096
+    X = torch.randn(B, K, device="cuda")
+    W = (torch.rand(H, K, device="cuda") * 2 - 1) * float(np.sqrt(6.0 / (K + H)))
+    dZ = torch.randn(B, H, device="cuda")
+    Z = dl.fc_fwd(X, W)
+    dX = dl.fc_bwd_dx(dZ, W)
+    dW, _ = dl.fc_bwd_dw(X, dZ)
+    a = float((dZ.double() * Z.double()).sum()); b = float((dX.double() * X.double()).sum())
+    c = float((dW.double() * W.double()).sum())
+    scale = float(np.sqrt(B * H) * Z.double().pow(2).mean().sqrt())
+    assert abs(a - b) <= 1e-4 * scale and abs(a - c) <= 1e-4 * scale, (a, b, c)
+    rows = torch.arange(0, B, 61, device="cuda")
+    assert_close(host(Z[rows]), host(X[rows].double() @ W.double().T), TR, "Z slab")
+    assert_close(host(dX[rows]), host(dZ[rows].double() @ W.double()), TR, "dX slab")
+    hs = torch.arange(0, H, 37, device="cuda")
+    assert_close(host(dW[hs]), host(dZ[:, hs].double().T @ X.double()), TR, "dW slab")
+
+
+# ------------------------------------------------------------------ fused BRN + activation + dropout
+def oracle_fused(oracle, act, x, gamma, beta, mm, ms, hyper, renorm, drop, mask, scale, bwd_masked, dY,
+                 dg0, db0, nt=0):
+    """Composition of the oracle's leaves in the reference's order."""
+    fw = oracle.norm_fwd_train(x, gamma, beta, mm, ms, *hyper, renorm, nt)
+    qv = oracle.act_fwd(act, fw["out"], nt)
+    kind = {DROP["NONE"]: None, DROP["BERNOULLI"]: 1, DROP["BERNOULLI_INVERTED"]: 0}[drop]
+    y = qv if kind is None else oracle.dropout_fwd(kind, qv, mask, scale, nt)
+    if kind is not None and bwd_masked:
+        dN = oracle.act_bwd(act, fw["out"], qv, oracle.dropout_fwd(kind, dY, mask, scale, nt), nt)
+    else:
+        dN = oracle.act_bwd(act, fw["out"], y, dY, nt)  # derivative sees the post-dropout output
+    bw = oracle.norm_bwd(fw["mean"], fw["std"], gamma, fw["r"], x, fw["xhat"], dN, dgamma_init=dg0,
+                         dbeta_init=db0, renorm=renorm, nthreads=nt)
+    return fw, y, bw
+
+
+FUSED_SHAPES = [(64, 256), (100, 132), (257, 64), (33, 5), (512, 1024), (2048, 16), (9, 4096)]
+
+
+@pytest.mark.parametrize("B,H", FUSED_SHAPES)
+@pytest.mark.parametrize("act", ["SELU", "ELU", "ISRLU", "RELU", "LEAKY_RELU"])
+def test_fused_norm_act_against_oracle(dl, oracle, pkg, B, H, act):
+    rng = np.random.default_rng(B * 31 + H)
+    x = (rng.standard_normal((B, H)) * rng.uniform(.5, 2, H) + rng.uniform(-1, 1, H)).astype(np.float32)
+    gamma = rng.uniform(.8, 1.2, H).astype(np.float32); beta = rng.uniform(-.1, .1, H).astype(np.float32)
+    dY = rng.standard_normal((B, H)).astype(np.float32)
+    dg0 = rng.standard_normal(H).astype(np.float32); db0 = rng.standard_normal(H).astype(np.float32)
+    hyper = (0.99, 1e-5, 3.0, 5.0)
+    mm, ms = np.zeros(H, np.float32), np.ones(H, np.float32)
+    fw, y, bw = oracle_fused(oracle, ACT[act], x, gamma, beta, mm, ms, hyper, True, DROP["NONE"], None, 1.0, False,
+                             dY, dg0, db0, nt=4)
+    desc = pkg.Dlmi.desc(ACT[act], renorm=True, momentum=hyper[0], eps=hyper[1], r_max=hyper[2], d_max=hyper[3])
+    dmm, dms = dev(mm), dev(ms)
+    yg, st = dl.fused_fwd(desc, dev(x), dev(gamma), dev(beta), dmm, dms)
+    assert_close(host(yg), y, TR, "y")
+    for k in ("mean", "std", "r", "d"):
+        assert_close(host(st[k]), fw[k], TR, k, floor=1.0 if k == "d" else 0.0)
+    assert_close(host(dmm), fw["mov_mean"], TR, "moving mean")
+    assert_close(host(dms), fw["mov_std"], TR, "moving std")
+    dg, db = dev(dg0), dev(db0)
+    dX = dl.fused_bwd(desc, dev(x), dev(gamma), dev(beta), st, dev(dY), dg, db)
+    assert_close(host(dX), bw["dx"], TR, "dX")
+    assert_close(host(dg), bw["dgamma"], TR, "dgamma")
+    assert_close(host(db), bw["dbeta"], TR, "dbeta")
+
+
+@pytest.mark.parametrize("B,H", [(64, 256), (37, 11)])
+@pytest.mark.parametrize("drop", ["BERNOULLI", "BERNOULLI_INVERTED"])
+@pytest.mark.parametrize("per_element", [False, True])
+@pytest.mark.parametrize("bwd_masked", [False, True])
+@pytest.mark.parametrize("renorm", [True, False])
+def test_fused_dropout_modes_against_oracle(dl, oracle, pkg, B, H, drop, per_element, bwd_masked, renorm):
+    rng = np.random.default_rng(B + H + per_element * 2 + bwd_masked)
+    x = (rng.standard_normal((B, H)) * 1.5 + 0.2).astype(np.float32)
+    gamma = rng.uniform(.8, 1.2, H).astype(np.float32); beta = rng.uniform(-.1, .1, H).astype(np.float32)
+    mm = rng.uniform(-1, 1, H).astype(np.float32); ms = rng.uniform(.5, 2, H).astype(np.float32)
+    dY = rng.standard_normal((B, H)).astype(np.float32)
+    keep = 0.8
+    mask = (rng.uniform(size=(B, H) if per_element else H) < keep).astype(np.uint8)
+    scale = float(np.float32(1.0) / np.float32(keep)) if drop == "BERNOULLI_INVERTED" else 1.0
+    hyper = (0.1, 1e-5, 1.2, 0.1)  # clips bind
+    zero = np.zeros(H, np.float32)
+    for act in ("ISRLU", "SELU"):
+        fw, y, bw = oracle_fused(oracle, ACT[act], x, gamma, beta, mm, ms, hyper, renorm, DROP[drop], mask, scale,
+                                 bwd_masked, dY, zero, zero)
+        desc = pkg.Dlmi.desc(ACT[act], renorm=renorm, dropout=DROP[drop], mask_per_element=per_element,
+                             dropout_bwd=1 if bwd_masked else 0, momentum=hyper[0], eps=hyper[1], r_max=hyper[2],
+                             d_max=hyper[3], drop_scale=scale)
+        dmm, dms = dev(mm), dev(ms)
+        dmask = dev(mask, torch.uint8)
+        yg, st = dl.fused_fwd(desc, dev(x), dev(gamma), dev(beta), dmm, dms, mask=dmask)
+        assert_close(host(yg), y, TR, "y")
+        dg, db = dev(zero), dev(zero)
+        dX = dl.fused_bwd(desc, dev(x), dev(gamma), dev(beta), st, dev(dY), dg, db, mask=dmask)
+        assert_close(host(dX), bw["dx"], TR, "dX")
+        assert_close(host(dg), bw["dgamma"], TR, "dgamma")
+        assert_close(host(db), bw["dbeta"], TR, "dbeta")
+        # inference tail with the updated moving statistics
+        yo = oracle.act_fwd(ACT[act], oracle.norm_fwd_infer(x, gamma, beta, fw["mov_mean"], fw["mov_std"]))
+        if drop == "BERNOULLI":
+            yo = oracle.dropout_fwd(2, yo, None, keep)
+            desc.drop_scale = keep
+        assert_close(host(dl.fused_infer(desc, dev(x), dev(gamma), dev(beta), dmm, dms)), yo, TE, "inference")
+
+
+def test_tall_skinny_with_outliers(dl, oracle, oracle64, pkg):
+    """[65536 x 256]-class input (scaled to 16384 rows for the CPU): N(0,1) with
+    1% outliers x50, BRN + leaky ReLU forward/backward and the inference
+    forward.  Both implementations are also measured against float64."""
+    rng = np.random.default_rng(65536)
+    B, H = 16384, 256
+    x = rng.standard_normal((B, H)).astype(np.float32)
+    x[rng.uniform(size=(B, H)) < 0.01] *= 50
+    gamma = rng.uniform(.8, 1.2, H).astype(np.float32); beta = rng.uniform(-.1, .1, H).astype(np.float32)
+    dY = rng.standard_normal((B, H)).astype(np.float32)
+    zero, one = np.zeros(H, np.float32), np.ones(H, np.float32)
+    hyper = (0.99, 1e-5, 3.0, 5.0)
+    a = ACT["LEAKY_RELU"]
+    nt = oracle.max_threads()
+    fw, y, bw = oracle_fused(oracle, a, x, gamma, beta, zero, one, hyper, True, DROP["NONE"], None, 1.0, False, dY,
+                             zero, zero, nt=nt)
+    fw64, y64, bw64 = oracle_fused(oracle64, a, x, gamma, beta, zero, one, hyper, True, DROP["NONE"], None, 1.0,
+                                   False, dY, zero, zero, nt=nt)
+    desc = pkg.Dlmi.desc(a, momentum=hyper[0], eps=hyper[1], r_max=hyper[2], d_max=hyper[3])
+    dmm, dms = dev(zero), dev(one)
+    yg, st = dl.fused_fwd(desc, dev(x), dev(gamma), dev(beta), dmm, dms)
+    dg, db = dev(zero), dev(zero)
+    dX = dl.fused_bwd(desc, dev(x), dev(gamma), dev(beta), st, dev(dY), dg, db)
+    assert_close(host(yg), y, TR, "y vs oracle")
+    assert_close(host(dX), bw["dx"], TR, "dX vs oracle")
+    assert_close(host(dg), bw["dgamma"], TR, "dgamma vs oracle")
+    # the GPU's tree sums should be at least as close to float64 as the CPU's sequential sums
+    from helpers import max_rel_err
+    assert max_rel_err(host(st["mean"]), fw64["mean"], floor=1.0) <= 2 * max_rel_err(fw["mean"], fw64["mean"], floor=1.0) + 1e-6
+    assert_close(host(st["std"]), fw64["std"], TR, "std vs float64")
+    mvm = rng.uniform(-1, 1, H).astype(np.float32); mvs = rng.uniform(.5, 2, H).astype(np.float32)
+    yo = oracle.act_fwd(a, oracle.norm_fwd_infer(x, gamma, beta, mvm, mvs, nt), nt)
+    assert_close(host(dl.fused_infer(desc, dev(x), dev(gamma), dev(beta), dev(mvm), dev(mvs))), yo, TE, "inference")
+
+
+def test_fused_full_size_properties(dl, pkg):
+    """[4096 x 4096] BRN + SELU at full size: checked against a float64
+    evaluation of the same formulas with torch on the GPU, plus the invariants
+    sum_b dX = 0 and dbeta = sum_b dN."""
+    torch.manual_seed(2)
+    B = H = 4096
+    s = torch.rand(H, device="cuda") * 1.5 + 0.5
+    m = torch.rand(H, device="cuda") * 2 - 1
+    x = torch.randn(B, H, device="cuda") * s + m
+    gamma = torch.rand(H, device="cuda") * 0.4 + 0.8
+    beta = torch.rand(H, device="cuda") * 0.2 - 0.1
+    dY = torch.randn(B, H, device="cuda")
+    mm, ms = torch.zeros(H, device="cuda"), torch.ones(H, device="cuda")
+    desc = pkg.Dlmi.desc(ACT["SELU"], momentum=0.99, eps=1e-5, r_max=3.0, d_max=5.0)
+    y, st = dl.fused_fwd(desc, x, gamma, beta, mm, ms)
+    dg, db = torch.zeros(H, device="cuda"), torch.zeros(H, device="cuda")
+    dX = dl.fused_bwd(desc, x, gamma, beta, st, dY, dg, db)
+    xd = x.double()
+    mu = xd.mean(0); sd = ((xd * xd).mean(0) - mu * mu + 1e-5).sqrt()
+    mm2 = 0.99 * mu; ms2 = 1 + 0.99 * (sd - 1)
+    r = (sd / ms2).clamp(1 / 3.0, 3.0); d = ((mu - mm2) / ms2).clamp(-5.0, 5.0)
+    xh = (xd - mu) / sd * r + d
+    n = gamma.double() * xh + beta.double()
+    al, sc = 1.6732632423543772, 1.0507009873554805
+    q = sc * torch.where(n <= 0, al * n.exp() - al, n)
+    assert_close(host(st["mean"]), host(mu), TR, "mean", floor=1.0)
+    assert_close(host(st["std"]), host(sd), TR, "std")
+    assert_close(host(mm), host(mm2), TR, "moving mean", floor=1.0)
+    assert_close(host(ms), host(ms2), TR, "moving std")
+    assert_close(host(y), host(q), TR, "y")
+    dn = dY.double() * sc * torch.where(n <= 0, q + al, torch.ones_like(q))
+    e = dn * gamma.double()
+    dmu = (e * (-r / sd)).sum(0); dsd = (e * (xd - mu) * (-r / (sd * sd))).sum(0)
+    dx = e * (r / sd) + dsd * ((xd - mu) / (B * sd)) + dmu / B
+    assert_close(host(dX), host(dx), TR, "dX")
+    assert_close(host(dg), host((dn * xh).sum(0)), TR, "dgamma")
+    assert_close(host(db), host(dn.sum(0)), TR, "dbeta")
+    assert float(dX.double().sum(0).abs().max()) < 1e-3 * float(dX.double().abs().sum(0).max())
+
+
+# ------------------------------------------------------------------ softmax + cross-entropy seed
+@pytest.mark.parametrize("B,H", [(128, 10), (5, 3), (70, 130)])
+def test_softmax_ce_seed(dl, oracle, B, H):
+    rng = np.random.default_rng(B + H)
+    z = (rng.standard_normal((B, H)) * 3).astype(np.float32)
+    labels = rng.integers(0, H, B)
+    y = np.eye(H, dtype=np.float32)[labels]
+    q = oracle.softmax_fwd(z)
+    qg = dl.softmax_fwd(dev(z))
+    assert_close(host(qg), q, TE, "softmax")
+    dZo, loss, correct = oracle.softmax_ce_seed(q, y)
+    stats = torch.zeros(2, dtype=torch.float64, device="cuda")
+    dZ = dl.softmax_ce_seed(dev(q), dev(y), stats)
+    assert_close(host(dZ), dZo, TE, "seed gradient")
+    st = host(stats)
+    assert abs(st[0] - loss) <= 1e-5 * max(1.0, abs(loss)) and st[1] == correct
