@@ -189,6 +189,9 @@ def test_fused_norm_act_against_oracle(dl, oracle, pkg, B, H, act):
     dg0 = rng.standard_normal(H).astype(np.float32); db0 = rng.standard_normal(H).astype(np.float32)
     hyper = (0.99, 1e-5, 3.0, 5.0)
     mm, ms = np.zeros(H, np.float32), np.ones(H, np.float32)
+    # the derivatives jump at a pre-activation of 0: no gradient through elements within rounding of it
+    pre = oracle.norm_fwd_train(x, gamma, beta, mm, ms, *hyper, True, 4)["out"]
+    dY[np.abs(pre) < 1e-5] = 0
     fw, y, bw = oracle_fused(oracle, ACT[act], x, gamma, beta, mm, ms, hyper, True, DROP["NONE"], None, 1.0, False,
                              dY, dg0, db0, nt=4)
     desc = pkg.Dlmi.desc(ACT[act], renorm=True, momentum=hyper[0], eps=hyper[1], r_max=hyper[2], d_max=hyper[3])
@@ -295,8 +298,6 @@ def test_fused_full_size_properties(dl, pkg):
     mm, ms = torch.zeros(H, device="cuda"), torch.ones(H, device="cuda")
     desc = pkg.Dlmi.desc(ACT["SELU"], momentum=0.99, eps=1e-5, r_max=3.0, d_max=5.0)
     y, st = dl.fused_fwd(desc, x, gamma, beta, mm, ms)
-    dg, db = torch.zeros(H, device="cuda"), torch.zeros(H, device="cuda")
-    dX = dl.fused_bwd(desc, x, gamma, beta, st, dY, dg, db)
     xd = x.double()
     mu = xd.mean(0); sd = ((xd * xd).mean(0) - mu * mu + 1e-5).sqrt()
     mm2 = 0.99 * mu; ms2 = 1 + 0.99 * (sd - 1)
@@ -310,6 +311,11 @@ def test_fused_full_size_properties(dl, pkg):
     assert_close(host(mm), host(mm2), TR, "moving mean", floor=1.0)
     assert_close(host(ms), host(ms2), TR, "moving std")
     assert_close(host(y), host(q), TR, "y")
+    # The reference's SELU derivative jumps at n = 0 (scale*(q+alpha) -> scale); an element whose
+    # pre-activation is within rounding of 0 may take either branch, so it carries no gradient here.
+    dY = torch.where(n.abs() < 1e-4, torch.zeros_like(dY), dY)
+    dg, db = torch.zeros(H, device="cuda"), torch.zeros(H, device="cuda")
+    dX = dl.fused_bwd(desc, x, gamma, beta, st, dY, dg, db)
     dn = dY.double() * sc * torch.where(n <= 0, q + al, torch.ones_like(q))
     e = dn * gamma.double()
     dmu = (e * (-r / sd)).sum(0); dsd = (e * (xd - mu) * (-r / (sd * sd))).sum(0)
