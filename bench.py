@@ -1,0 +1,250 @@
+"""Benchmark of the fully-connected + batch-renorm + activation hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c5]
+
+A "step" is one forward + backward pass of the layer over one synthetic batch
+resident in HBM:  Z = X W^T (+bias) -> batch renorm -> activation, then
+dZ = d(activation, batch renorm), dX = dZ W, dW = dZ^T X, db, dgamma, dbeta.
+Prints ONE JSON line: samples/s of the whole step, the roofline of the dominant
+kernel (fp32 MFMA GEMM for c3/c5, the fused normalization kernels for c2), the
+HBM roofline of the fused normalization + activation kernels, and the CPU
+baseline measured on the host cores on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0         # MI355X HBM3E
+MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix
+
+WORKLOADS = {
+    # name: (B, K, H, activation, description)
+    "c3": (8192, 4096, 4096, "ELU", "FC 4096->4096 on batch 8192 + batch renorm + ELU, fwd+bwd (dX,dW,db,dgamma,dbeta)"),
+    "c2": (4096, 0, 4096, "SELU", "batch renorm + SELU fwd+bwd on [4096 x 4096] (no FC)"),
+    "c5": (65536, 256, 256, "LEAKY_RELU", "FC 256->256 on batch 65536 + batch renorm + leaky ReLU, fwd+bwd"),
+}
+HYPER = dict(momentum=0.99, eps=1e-5, r_max=3.0, d_max=5.0)
+
+
+def make_inputs(torch, name):
+    B, K, H, act, _ = WORKLOADS[name]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1234)
+    t = {}
+    if K:
+        t["X"] = torch.randn(B, K, device="cuda", generator=g)
+        if name == "c5":  # 1% outliers x50
+            t["X"] = torch.where(torch.rand(B, K, device="cuda", generator=g) < 0.01, t["X"] * 50, t["X"])
+        lim = (6.0 / (K + H)) ** 0.5
+        t["W"] = (torch.rand(H, K, device="cuda", generator=g) * 2 - 1) * lim
+        t["bias"] = torch.zeros(H, device="cuda")
+        t["gamma"] = torch.ones(H, device="cuda")
+        t["beta"] = torch.zeros(H, device="cuda")
+        t["Z"] = torch.empty(B, H, device="cuda")
+        t["dX"] = torch.empty(B, K, device="cuda")
+        t["dW"] = torch.empty(H, K, device="cuda")
+        t["db"] = torch.empty(H, device="cuda")
+    else:
+        s = torch.rand(H, device="cuda", generator=g) * 1.5 + 0.5
+        m = torch.rand(H, device="cuda", generator=g) * 2 - 1
+        t["Z"] = torch.randn(B, H, device="cuda", generator=g) * s + m
+        t["gamma"] = torch.rand(H, device="cuda", generator=g) * 0.4 + 0.8
+        t["beta"] = torch.rand(H, device="cuda", generator=g) * 0.2 - 0.1
+    t["dY"] = torch.randn(B, H, device="cuda", generator=g)
+    t["y"] = torch.empty(B, H, device="cuda")
+    t["dZ"] = torch.empty(B, H, device="cuda")
+    t["mov_mean"] = torch.zeros(H, device="cuda")
+    t["mov_std"] = torch.ones(H, device="cuda")
+    t["dgamma"] = torch.zeros(H, device="cuda")
+    t["dbeta"] = torch.zeros(H, device="cuda")
+    t["stats"] = {k: torch.empty(H, device="cuda") for k in ("mean", "std", "r", "d")}
+    return t
+
+
+class Step:
+    """The pieces of one step, callable separately so each can be timed."""
+
+    def __init__(self, dl, pkg, name, t):
+        self.dl, self.t = dl, t
+        self.B, self.K, self.H, act, _ = WORKLOADS[name]
+        self.desc = pkg.Dlmi.desc(pkg.ACT[act], renorm=True, **HYPER)
+
+    def gemm_fwd(self):
+        t = self.t
+        self.dl.fc_fwd(t["X"], t["W"], t["bias"], out=t["Z"])
+
+    def norm_fwd(self):
+        t = self.t
+        self.dl.fused_fwd(self.desc, t["Z"], t["gamma"], t["beta"], t["mov_mean"], t["mov_std"], out=t["y"],
+                          stats=t["stats"])
+
+    def norm_bwd(self):
+        t = self.t
+        self.dl.fused_bwd(self.desc, t["Z"], t["gamma"], t["beta"], t["stats"], t["dY"], t["dgamma"], t["dbeta"],
+                          out=t["dZ"])
+
+    def gemm_dx(self):
+        t = self.t
+        self.dl.fc_bwd_dx(t["dZ"], t["W"], out=t["dX"])
+
+    def gemm_dw(self):
+        t = self.t
+        self.dl.fc_bwd_dw(t["X"], t["dZ"], dW=t["dW"], db=t["db"])
+
+    def parts(self):
+        if self.K:
+            return [self.gemm_fwd, self.norm_fwd, self.norm_bwd, self.gemm_dx, self.gemm_dw]
+        return [self.norm_fwd, self.norm_bwd]
+
+    def __call__(self):
+        for p in self.parts():
+            p()
+
+
+def time_events(torch, fn, reps, warmup=2):
+    """Average duration (ms) of fn() over `reps` back-to-back calls, measured
+    with HIP events recorded on the stream the kernels are launched on."""
+    for _ in range(warmup):
+        fn()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    s.record()
+    for _ in range(reps):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / reps
+
+
+def cpu_baseline(name, budget_rows):
+    """The reference's OpenMP CPU path (the real reference compiled, if
+    oracle/_ref is present; else this repository's restatement of it) on the
+    first `budget_rows` rows of the same workload shape, host cores only."""
+    import numpy as np
+    from oracle.binding import ACT, Oracle, Reference, reference_available
+    B, K, H, act, _ = WORKLOADS[name]
+    Bs = min(B, budget_rows)
+    kind = "reference" if reference_available() else "port"
+    cpu = Reference() if kind == "reference" else Oracle()
+    nt = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+    nt = max(1, min(nt, os.cpu_count() or 1, 64))
+    rng = np.random.default_rng(1234)
+    zero, one = np.zeros(H, np.float32), np.ones(H, np.float32)
+    dY = rng.standard_normal((Bs, H), dtype=np.float32)
+    if K:
+        X = rng.standard_normal((Bs, K), dtype=np.float32)
+        W = ((rng.random((H, K), dtype=np.float32) * 2 - 1) * np.float32((6.0 / (K + H)) ** 0.5))
+    else:
+        Z = rng.standard_normal((Bs, H), dtype=np.float32)
+    t0 = time.perf_counter()
+    if K:
+        Z = cpu.fc_fwd(X, W, nt)
+    fw = cpu.norm_fwd_train(Z, one, zero, zero, one, HYPER["momentum"], HYPER["eps"], HYPER["r_max"],
+                            HYPER["d_max"], True, nt)
+    y = cpu.act_fwd(ACT[act], fw["out"], nt)
+    dN = cpu.act_bwd(ACT[act], fw["out"], y, dY, nt)
+    bw = cpu.norm_bwd(fw["mean"], fw["std"], one, fw["r"], Z, fw["xhat"], dN, renorm=True, nthreads=nt)
+    if K:
+        cpu.fc_bwd_dx(bw["dx"], W, nthreads=nt)
+        cpu.fc_bwd_dw(X, bw["dx"], with_bias=False, nthreads=nt)
+    dt = time.perf_counter() - t0
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next(l.split(":", 1)[1].strip() for l in f if l.startswith("model name"))
+    except Exception:
+        pass
+    return {"value": Bs / dt, "unit": "samples/s", "cores": nt, "kind": kind,
+            "sample": "first %d of %d rows of the same layer shape, one fwd+bwd pass, %.1f s, OpenMP leaves on %d threads (%s)"
+                      % (Bs, B, dt, nt, model)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-rows", type=int, default=-1, help="rows of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--only", default="", help="profiling aid: run just this part (gemm_fwd, gemm_dx, gemm_dw, "
+                                               "norm_fwd, norm_bwd) --steps times and exit without a JSON line")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from __graft_entry__ import load_package
+    pkg = load_package()
+    dl = pkg.Dlmi(0)  # raises if the HIP library or the GPU is missing: no fallback
+    name = args.workload
+    B, K, H, act, descr = WORKLOADS[name]
+    t = make_inputs(torch, name)
+    step = Step(dl, pkg, name, t)
+
+    if args.only:
+        step()  # every buffer a part reads has been produced once
+        part = getattr(step, args.only)
+        ms = time_events(torch, part, args.steps, warmup=args.warmup)
+        print("%s: %.4f ms per call over %d calls" % (args.only, ms, args.steps), file=sys.stderr)
+        dl.close()
+        return
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+
+    # per-kernel-group timings with HIP events on the launch stream
+    E = B * H
+    t_nf = time_events(torch, step.norm_fwd, 20)
+    t_nb = time_events(torch, step.norm_bwd, 20)
+    hbm_bytes = 32.0 * E  # fwd 12 B/element + bwd 20 B/element
+    hbm = {"bound": "hbm", "achieved": hbm_bytes / ((t_nf + t_nb) * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+           "traffic": None, "kernels": "k_col_stats+k_fwd_finalize+k_fwd_apply / k_bwd_reduce+k_bwd_finalize+k_bwd_apply",
+           "ms_fwd": t_nf, "ms_bwd": t_nb, "bytes_fwd": 12.0 * E, "bytes_bwd": 20.0 * E}
+    hbm["frac"] = hbm["achieved"] / hbm["peak"]
+    detail = {"ms_norm_fwd": t_nf, "ms_norm_bwd": t_nb}
+    if K:
+        t_gf = time_events(torch, step.gemm_fwd, 10)
+        t_gx = time_events(torch, step.gemm_dx, 10)
+        t_gw = time_events(torch, lambda: dl.fc_bwd_dw(t["X"], t["dZ"], dW=t["dW"]), 10)
+        flops = 2.0 * B * K * H
+        avg = (t_gf + t_gx + t_gw) / 3.0
+        roof = {"bound": "mfma", "achieved": flops / (avg * 1e-3) / 1e12, "peak": MFMA_FP32_PEAK_TFLOPS,
+                "unit": "TFLOP/s", "traffic": None, "kernel": "k_gemm_f32 (avg of fwd NT, dX NN, dW TN launches)",
+                "tflops_fwd": flops / (t_gf * 1e-3) / 1e12, "tflops_dx": flops / (t_gx * 1e-3) / 1e12,
+                "tflops_dw": flops / (t_gw * 1e-3) / 1e12}
+        roof["frac"] = roof["achieved"] / roof["peak"]
+        detail.update({"ms_gemm_fwd": t_gf, "ms_gemm_dx": t_gx, "ms_gemm_dw": t_gw})
+    else:
+        roof = dict(hbm)
+
+    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 1024, "c2": 4096, "c5": 65536}[name]
+    cpu = cpu_baseline(name, cpu_rows) if cpu_rows else None
+
+    out = {
+        "metric": "FC+BRN+act fwd+bwd samples/sec; % HBM peak (norm/act), % FP32 MFMA peak (GEMM)",
+        "value": B / (ms_per_step * 1e-3), "unit": "samples/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": name + ": " + descr, "batch": B, "fan_in": K, "units": H, "activation": act,
+                   "norm": "batch renorm rmax=3 dmax=5 momentum=0.99 eps=1e-5", "inputs": "resident in HBM"},
+        "roofline": roof, "roofline_norm_act": hbm, "cpu_baseline": cpu, "detail": detail,
+    }
+    print(json.dumps(out))
+    dl.close()
+
+
+if __name__ == "__main__":
+    main()

@@ -25,12 +25,13 @@
 // cover a compact block of tiles and (b) tiles are walked in groups of 8 rows
 // of tiles, which keeps the A and B panels of concurrently running workgroups
 // resident in that XCD's L2.
-#include <initializer_list>
+#include <cstdlib>
 
 #include "dlmi_common.hpp"
 
 namespace dlmi {
 
+typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kGemmThreads = 256;
@@ -51,23 +52,28 @@ struct GemmArgs {
 };
 
 // LDS tile of an operand whose k index is contiguous in memory: [ROWS][BK+4].
-// LDS tile of an operand whose row (m or n) index is contiguous:  [BK][ROWS+PAD].
+// LDS tile of an operand whose row (m or n) index is contiguous:  [BK][ROWS+8].
 template <int ROWS, int BK, bool KCONTIG>
 struct TileShape {
   static constexpr int kStride = KCONTIG ? BK + 4 : ROWS + 8;
   static constexpr int kFloats = KCONTIG ? ROWS * (BK + 4) : BK * (ROWS + 8);
-  static constexpr int kVec4 = ROWS * BK / 4;             // float4 per tile
-  static constexpr int kPerThread = kVec4 / kGemmThreads;  // float4 per thread
+  static constexpr int kVec4 = ROWS * BK / 4;             // 16-byte pieces per tile
+  static constexpr int kPerThread = kVec4 / kGemmThreads;  // pieces per thread
   static_assert(kVec4 % kGemmThreads == 0, "tile must divide evenly over the workgroup");
+  // the prefetch registers of one thread as ONE vector value (a first-class
+  // SSA value: it can neither be spilled to scratch nor be promoted to LDS the
+  // way a local array can)
+  typedef float Regs __attribute__((ext_vector_type(4 * kPerThread)));
 };
 
 // Global -> registers for one operand tile.  `row0` is the tile's first row
 // (m or n), `k0` its first k.  FAST: whole tile in bounds, 16-byte aligned.
 template <int ROWS, int BK, bool KCONTIG, bool FAST>
-__device__ __forceinline__ void tile_load(float const *__restrict__ P, size_t ld, size_t row0, size_t k0,
-                                          size_t rows_total, size_t k_end,
-                                          float4 (&regs)[TileShape<ROWS, BK, KCONTIG>::kPerThread]) {
+__device__ __forceinline__ typename TileShape<ROWS, BK, KCONTIG>::Regs tile_load(float const *__restrict__ P,
+                                                                               size_t ld, size_t row0, size_t k0,
+                                                                               size_t rows_total, size_t k_end) {
   using T = TileShape<ROWS, BK, KCONTIG>;
+  typename T::Regs regs;
 #pragma unroll
   for (int i = 0; i < T::kPerThread; ++i) {
     int const f = threadIdx.x + i * kGemmThreads;
@@ -79,25 +85,27 @@ __device__ __forceinline__ void tile_load(float const *__restrict__ P, size_t ld
       k = k0 + f / (ROWS / 4);
       row = row0 + (f % (ROWS / 4)) * 4;
     }
+    v4f t;
     if constexpr (FAST) {
       float const *src = KCONTIG ? P + row * ld + k : P + k * ld + row;
-      regs[i] = *reinterpret_cast<float4 const *>(src);
+      t = *reinterpret_cast<v4f const *>(src);
     } else {
-      float v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         size_t const rr = KCONTIG ? row : row + e;
         size_t const kk = KCONTIG ? k + e : k;
-        v[e] = (rr < rows_total && kk < k_end) ? (KCONTIG ? P[rr * ld + kk] : P[kk * ld + rr]) : 0.0f;
+        t[e] = (rr < rows_total && kk < k_end) ? (KCONTIG ? P[rr * ld + kk] : P[kk * ld + rr]) : 0.0f;
       }
-      regs[i] = make_float4(v[0], v[1], v[2], v[3]);
     }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) regs[4 * i + e] = t[e];
   }
+  return regs;
 }
 
 template <int ROWS, int BK, bool KCONTIG>
 __device__ __forceinline__ void tile_store(float *__restrict__ lds,
-                                           float4 const (&regs)[TileShape<ROWS, BK, KCONTIG>::kPerThread]) {
+                                           typename TileShape<ROWS, BK, KCONTIG>::Regs const &regs) {
   using T = TileShape<ROWS, BK, KCONTIG>;
 #pragma unroll
   for (int i = 0; i < T::kPerThread; ++i) {
@@ -108,7 +116,10 @@ __device__ __forceinline__ void tile_store(float *__restrict__ lds,
     } else {
       off = (f / (ROWS / 4)) * T::kStride + (f % (ROWS / 4)) * 4;
     }
-    *reinterpret_cast<float4 *>(lds + off) = regs[i];
+    v4f t;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) t[e] = regs[4 * i + e];
+    *reinterpret_cast<v4f *>(lds + off) = t;
   }
 }
 
@@ -116,28 +127,28 @@ __device__ __forceinline__ void tile_store(float *__restrict__ lds,
 // step s.  `r` = row inside the tile (block base + lane % 32), `kk` = first k
 // of this lane's 4 (group base + (lane / 32) * 4).
 template <int ROWS, int BK, bool KCONTIG>
-__device__ __forceinline__ float4 frag_load(float const *__restrict__ lds, int r, int kk) {
+__device__ __forceinline__ v4f frag_load(float const *__restrict__ lds, int r, int kk) {
   using T = TileShape<ROWS, BK, KCONTIG>;
   if constexpr (KCONTIG) {
-    return *reinterpret_cast<float4 const *>(lds + r * T::kStride + kk);
+    return *reinterpret_cast<v4f const *>(lds + r * T::kStride + kk);
   } else {
-    return make_float4(lds[(kk + 0) * T::kStride + r], lds[(kk + 1) * T::kStride + r],
-                       lds[(kk + 2) * T::kStride + r], lds[(kk + 3) * T::kStride + r]);
+    v4f t;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) t[s] = lds[(kk + s) * T::kStride + r];
+    return t;
   }
 }
 
-__device__ __forceinline__ float f4_get(float4 const &v, int s) {
-  return s == 0 ? v.x : (s == 1 ? v.y : (s == 2 ? v.z : v.w));
-}
-
-template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, bool FAST>
-__global__ __launch_bounds__(kGemmThreads) void k_gemm_f32(GemmArgs g) {
+template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, bool FAST, int WAVES_PER_EU>
+__global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
+void k_gemm_f32(GemmArgs g) {
   using TA = TileShape<BM, BK, A_KCONTIG>;
   using TB = TileShape<BN, BK, B_KCONTIG>;
   constexpr int WM = BM / 2, WN = BN / 2;  // wavefront tile
   constexpr int TM = WM / 32, TN = WN / 32;
   static_assert(BK % 8 == 0, "K tile is consumed in groups of 8");
-  __shared__ __attribute__((aligned(16))) float lds[2 * (TA::kFloats + TB::kFloats)];
+  extern __shared__ __attribute__((aligned(16))) float lds[];  // 2 stages of (A tile, B tile)
+  constexpr int kStage = TA::kFloats + TB::kFloats;
 
   // ---- which tile: XCD-aware remap, then grouped ordering -------------------
   unsigned const ntiles = g.tiles_m * g.tiles_n;
@@ -158,8 +169,8 @@ __global__ __launch_bounds__(kGemmThreads) void k_gemm_f32(GemmArgs g) {
   int const lane = threadIdx.x & 63;
   int const wave = threadIdx.x >> 6;
   int const wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
-  int const lr = lane & 31;         // row inside a 32-block (A: m, B: n)
-  int const lk = (lane >> 5) * 4;   // this lane's k offset inside a group of 8
+  int const lr = lane & 31;        // row inside a 32-block (A: m, B: n)
+  int const lk = (lane >> 5) * 4;  // this lane's k offset inside a group of 8
 
   v16f acc[TM][TN];
 #pragma unroll
@@ -169,30 +180,11 @@ __global__ __launch_bounds__(kGemmThreads) void k_gemm_f32(GemmArgs g) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  float4 ra[TA::kPerThread], rb[TB::kPerThread];
-  constexpr int kStage = TA::kFloats + TB::kFloats;  // stage s: A at s*kStage, B right after it
-
-  if (ktiles > 0) {
-    tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, k_begin, g.M, k_end, ra);
-    tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, k_begin, g.N, k_end, rb);
-    tile_store<BM, BK, A_KCONTIG>(lds, ra);
-    tile_store<BN, BK, B_KCONTIG>(lds + TA::kFloats, rb);
-  }
-  __syncthreads();
-
-  for (int kt = 0; kt < ktiles; ++kt) {
-    int const cur = kt & 1;
-    bool const more = kt + 1 < ktiles;
-    if (more) {  // next tile's global loads fly while this tile is multiplied
-      size_t const kn = k_begin + static_cast<size_t>(kt + 1) * BK;
-      tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, kn, g.M, k_end, ra);
-      tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, kn, g.N, k_end, rb);
-    }
-    float const *const sa = lds + cur * kStage;
-    float const *const sb = sa + TA::kFloats;
+  // All MFMAs of one K tile staged at `sa` / `sb`.
+  auto mma_tile = [&](float const *__restrict__ sa, float const *__restrict__ sb) {
 #pragma unroll
     for (int kk = 0; kk < BK; kk += 8) {
-      float4 fa[TM], fb[TN];
+      v4f fa[TM], fb[TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i) fa[i] = frag_load<BM, BK, A_KCONTIG>(sa, wm0 + i * 32 + lr, kk + lk);
 #pragma unroll
@@ -203,13 +195,34 @@ __global__ __launch_bounds__(kGemmThreads) void k_gemm_f32(GemmArgs g) {
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(f4_get(fa[i], s), f4_get(fb[j], s), acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
     }
-    if (more) {
+  };
+
+  if (ktiles > 0) {
+    typename TA::Regs ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, k_begin, g.M, k_end);
+    typename TB::Regs rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, k_begin, g.N, k_end);
+    tile_store<BM, BK, A_KCONTIG>(lds, ra);
+    tile_store<BN, BK, B_KCONTIG>(lds + TA::kFloats, rb);
+    __syncthreads();
+    // Steady state.  The next tile's global loads are issued first and stay in
+    // flight underneath this tile's MFMAs; the scheduling barriers stop the
+    // compiler from sinking them to the end of the tile (where it would then
+    // wait on them at once) to save registers.
+    for (int kt = 0; kt + 1 < ktiles; ++kt) {
+      int const cur = kt & 1;
+      size_t const kn = k_begin + static_cast<size_t>(kt + 1) * BK;
+      ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, kn, g.M, k_end);
+      rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, kn, g.N, k_end);
+      __builtin_amdgcn_sched_barrier(0);
+      mma_tile(lds + cur * kStage, lds + cur * kStage + TA::kFloats);
+      __builtin_amdgcn_sched_barrier(0);
       tile_store<BM, BK, A_KCONTIG>(lds + (cur ^ 1) * kStage, ra);
       tile_store<BN, BK, B_KCONTIG>(lds + (cur ^ 1) * kStage + TA::kFloats, rb);
+      __syncthreads();
     }
-    __syncthreads();
+    int const last = (ktiles - 1) & 1;
+    mma_tile(lds + last * kStage, lds + last * kStage + TA::kFloats);
   }
 
   // ---- epilogue: accumulator register e of lane l holds
@@ -250,8 +263,8 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(float const *__restrict__
 }
 
 // db[h] (+)= sum_b dZ[b,h]: column sums over the batch in a fixed order
-// (update_derivative_fwp_st.cpp:283-302).  Thread per column group, blocks
-// over batch chunks, partials combined by k_colsum_finish.
+// (update_derivative_fwp_st.cpp:283-302).  Thread per column, blocks over batch
+// chunks, partials combined by k_colsum_finish.
 __global__ __launch_bounds__(256) void k_colsum_partial(float const *__restrict__ x, size_t B, size_t H,
                                                          size_t rows_per_chunk, float *__restrict__ partial) {
   size_t const j = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
@@ -280,34 +293,70 @@ __global__ __launch_bounds__(256) void k_colsum_finish(float const *__restrict__
 }
 
 // ---------------------------------------------------------------- host side
-template <int BM, int BN, int BK, bool AK, bool BKC>
+template <int BM, int BN, int BK, bool AK, bool BKC, int WPE>
 static int launch_gemm(dlmi_ctx *ctx, GemmArgs g, unsigned splits, bool fast) {
+  using TA = TileShape<BM, BK, AK>;
+  using TB = TileShape<BN, BK, BKC>;
+  constexpr size_t lds_bytes = 2 * (TA::kFloats + TB::kFloats) * sizeof(float);
   g.tiles_m = static_cast<unsigned>(dlmi_ceil_div(g.M, BM));
   g.tiles_n = static_cast<unsigned>(dlmi_ceil_div(g.N, BN));
   dim3 const grid(g.tiles_m * g.tiles_n, 1, splits);
+  auto const kfast = k_gemm_f32<BM, BN, BK, AK, BKC, true, WPE>;
+  auto const kslow = k_gemm_f32<BM, BN, BK, AK, BKC, false, WPE>;
+  static bool attr_set = false;  // more than 64 KB of LDS has to be asked for once per kernel
+  if (!attr_set) {
+    DLMI_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<void const *>(kfast),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+    DLMI_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<void const *>(kslow),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+    attr_set = true;
+  }
   if (fast)
-    hipLaunchKernelGGL((k_gemm_f32<BM, BN, BK, AK, BKC, true>), grid, dim3(kGemmThreads), 0, ctx->stream, g);
+    hipLaunchKernelGGL(kfast, grid, dim3(kGemmThreads), lds_bytes, ctx->stream, g);
   else
-    hipLaunchKernelGGL((k_gemm_f32<BM, BN, BK, AK, BKC, false>), grid, dim3(kGemmThreads), 0, ctx->stream, g);
+    hipLaunchKernelGGL(kslow, grid, dim3(kGemmThreads), lds_bytes, ctx->stream, g);
   DLMI_LAUNCH_CHECK(ctx, "k_gemm_f32");
   return DLMI_OK;
 }
 
-constexpr int kBM = 128, kBN = 128, kBK = 16;
+struct TileCfg {
+  int bm, bn, bk;
+};
+
+// Tuning aid: DLMI_GEMM_TILE=<index> picks another compiled tile shape.
+static int tile_choice() {
+  static int const c = [] {
+    char const *e = std::getenv("DLMI_GEMM_TILE");
+    return e != nullptr ? std::atoi(e) : -1;  // -1: choose by shape
+  }();
+  return c;
+}
 
 // C[M,N] (+)= A . B with the operand layouts given by the two flags.
 template <bool AK, bool BKC>
 static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, size_t lda, float const *B, size_t ldb,
                 float *C, float const *bias, int accumulate) {
+  static TileCfg const cfgs[] = {{128, 128, 16}, {128, 128, 32}, {256, 128, 16}, {256, 128, 32}, {256, 256, 16}};
+  int choice = tile_choice();
+  if (choice < 0 || choice >= static_cast<int>(sizeof(cfgs) / sizeof(cfgs[0]))) {
+    // default: 256 x 256 tiles (one wavefront per SIMD, 16 MFMA blocks each) when
+    // the output splits evenly into at least two of them per CU, else 128 x 128
+    choice = (M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 2 * static_cast<size_t>(ctx->num_cu)) ? 4 : 0;
+  }
+  // a big tile only pays when the output has enough of them to fill the GPU
+  if (dlmi_ceil_div(M, cfgs[choice].bm) * dlmi_ceil_div(N, cfgs[choice].bn) < static_cast<size_t>(ctx->num_cu))
+    choice = 0;
+  int const bm = cfgs[choice].bm, bn = cfgs[choice].bn, bk = cfgs[choice].bk;
+
   GemmArgs g;
   g.A = A; g.B = B; g.C = C; g.bias = bias; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldc = N;
   g.accumulate = accumulate; g.split_out = nullptr;
-  bool const fast = M % kBM == 0 && N % kBN == 0 && K % kBK == 0 && lda % 4 == 0 && ldb % 4 == 0 &&
+  bool const fast = M % bm == 0 && N % bn == 0 && K % bk == 0 && lda % 4 == 0 && ldb % 4 == 0 &&
                     dlmi_aligned16(A) && dlmi_aligned16(B);
   // Split K when the output alone cannot fill the machine (few tiles, long K):
   // each slice writes its partial product, a second kernel adds them in order.
-  size_t const tiles = dlmi_ceil_div(M, kBM) * dlmi_ceil_div(N, kBN);
-  size_t const ktiles = dlmi_ceil_div(K, kBK);
+  size_t const tiles = dlmi_ceil_div(M, bm) * dlmi_ceil_div(N, bn);
+  size_t const ktiles = dlmi_ceil_div(K, bk);
   unsigned splits = 1;
   size_t const target = static_cast<size_t>(ctx->num_cu) * 2;
   if (tiles < target / 2 && ktiles >= 16) {
@@ -321,10 +370,17 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
     }
   }
   size_t const kt_per_split = dlmi_ceil_div(ktiles, splits);
-  g.k_per_split = kt_per_split * kBK;
+  g.k_per_split = kt_per_split * bk;
   splits = static_cast<unsigned>(dlmi_ceil_div(ktiles, kt_per_split));
   if (splits > 1) g.split_out = reinterpret_cast<float *>(ctx->scratch);
-  int rc = launch_gemm<kBM, kBN, kBK, AK, BKC>(ctx, g, splits, fast);
+  int rc;
+  switch (choice) {
+    case 1: rc = launch_gemm<128, 128, 32, AK, BKC, 2>(ctx, g, splits, fast); break;
+    case 2: rc = launch_gemm<256, 128, 16, AK, BKC, 2>(ctx, g, splits, fast); break;
+    case 3: rc = launch_gemm<256, 128, 32, AK, BKC, 2>(ctx, g, splits, fast); break;
+    case 4: rc = launch_gemm<256, 256, 16, AK, BKC, 1>(ctx, g, splits, fast); break;
+    default: rc = launch_gemm<128, 128, 16, AK, BKC, 2>(ctx, g, splits, fast); break;
+  }
   if (rc != DLMI_OK) return rc;
   if (splits > 1) {
     size_t const mn = M * N;

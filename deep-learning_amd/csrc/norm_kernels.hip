@@ -183,8 +183,39 @@ __global__ __launch_bounds__(kBlock) void k_col_stats(float const *__restrict__ 
   }
 }
 
+// Sums NA partial-sum planes over the batch chunks for 64 adjacent units per
+// block: wavefront w adds chunks w, w+4, w+8, ... (coalesced 256-byte rows, four
+// independent accumulation chains per unit), then the four wavefront totals
+// are combined through LDS in a fixed order.  On return the threads of
+// wavefront 0 hold the totals of unit blockIdx.x*64 + lane.
+constexpr int kFinCols = 64;
+template <int NA>
+__device__ __forceinline__ void chunk_totals(float const *__restrict__ partial, unsigned nchunks, size_t H,
+                                             float (&tot)[NA], float *lds) {
+  int const lane = threadIdx.x & (kWave - 1);
+  int const wave = threadIdx.x / kWave;
+  size_t const j = static_cast<size_t>(blockIdx.x) * kFinCols + lane;
+#pragma unroll
+  for (int a = 0; a < NA; ++a) tot[a] = 0.0f;
+  if (j < H) {
+    for (unsigned c = wave; c < nchunks; c += kBlock / kWave) {
+#pragma unroll
+      for (int a = 0; a < NA; ++a) tot[a] += partial[(a * static_cast<size_t>(nchunks) + c) * H + j];
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < NA; ++a) lds[(wave * kWave + lane) * NA + a] = tot[a];
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+      tot[a] = (lds[(0 * kWave + lane) * NA + a] + lds[(1 * kWave + lane) * NA + a]) +
+               (lds[(2 * kWave + lane) * NA + a] + lds[(3 * kWave + lane) * NA + a]);
+  }
+}
+
 // Phase 2 of fwp_st.cpp:4709-4746: batch mean, moving mean, batch std, moving
-// std, then r and d from the UPDATED moving statistics.  One thread per unit.
+// std, then r and d from the UPDATED moving statistics.  64 units per block.
 __global__ __launch_bounds__(kBlock) void k_fwd_finalize(float const *__restrict__ partial, unsigned nchunks,
                                                           size_t B, size_t H, int renorm, float momentum,
                                                           float eps, float r_max, float d_max,
@@ -192,13 +223,12 @@ __global__ __launch_bounds__(kBlock) void k_fwd_finalize(float const *__restrict
                                                           float *__restrict__ mov_mean,
                                                           float *__restrict__ mov_std, float *__restrict__ r,
                                                           float *__restrict__ d) {
-  size_t const j = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
-  if (j >= H) return;
-  float s1 = 0.0f, s2 = 0.0f;
-  for (unsigned c = 0; c < nchunks; ++c) {
-    s1 += partial[(0 * static_cast<size_t>(nchunks) + c) * H + j];
-    s2 += partial[(1 * static_cast<size_t>(nchunks) + c) * H + j];
-  }
+  __shared__ float lds[kBlock * 2];
+  float tot[2];
+  chunk_totals<2>(partial, nchunks, H, tot, lds);
+  size_t const j = static_cast<size_t>(blockIdx.x) * kFinCols + threadIdx.x;
+  if (threadIdx.x >= kWave || j >= H) return;
+  float const s1 = tot[0], s2 = tot[1];
   float const batch_scale = 1.0f / static_cast<float>(B);
   float const mu = s1 * batch_scale;
   float mm = mov_mean[j];
@@ -464,14 +494,12 @@ __global__ __launch_bounds__(kBlock) void k_bwd_finalize(float const *__restrict
                                                           float *__restrict__ dgamma, float *__restrict__ dbeta,
                                                           float *__restrict__ dmean, float *__restrict__ dstd,
                                                           float *__restrict__ coef) {
-  size_t const j = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
-  if (j >= H) return;
-  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f;
-  for (unsigned c = 0; c < nchunks; ++c) {
-    s0 += partial[(0 * static_cast<size_t>(nchunks) + c) * H + j];
-    s1 += partial[(1 * static_cast<size_t>(nchunks) + c) * H + j];
-    s2 += partial[(2 * static_cast<size_t>(nchunks) + c) * H + j];
-  }
+  __shared__ float lds[kBlock * 3];
+  float tot[3];
+  chunk_totals<3>(partial, nchunks, H, tot, lds);
+  size_t const j = static_cast<size_t>(blockIdx.x) * kFinCols + threadIdx.x;
+  if (threadIdx.x >= kWave || j >= H) return;
+  float const s0 = tot[0], s1 = tot[1], s2 = tot[2];
   float const sd = stdv[j];
   float const rr = r != nullptr ? r[j] : 1.0f;
   float const ga = gamma[j];
@@ -595,7 +623,7 @@ static int run_fwd_train(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &
   else
     hipLaunchKernelGGL(k_col_stats<1>, grid, block, 0, ctx->stream, c.x, B, H, g.tx_log2, g.rows_per_chunk, partial);
   DLMI_LAUNCH_CHECK(ctx, "k_col_stats");
-  hipLaunchKernelGGL(k_fwd_finalize, dim3(static_cast<unsigned>(dlmi_ceil_div(H, kBlock))), block, 0, ctx->stream,
+  hipLaunchKernelGGL(k_fwd_finalize, dim3(static_cast<unsigned>(dlmi_ceil_div(H, kFinCols))), block, 0, ctx->stream,
                      partial, g.nchunks, B, H, c.norm == DLMI_NORM_BATCH_RENORM ? 1 : 0, c.momentum, c.eps,
                      c.r_max, c.d_max, c.mean, c.stdv, c.mov_mean, c.mov_std, c.r, c.d);
   DLMI_LAUNCH_CHECK(ctx, "k_fwd_finalize");
@@ -652,7 +680,7 @@ static int run_bwd(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c) {
     });
   }
   DLMI_LAUNCH_CHECK(ctx, "k_bwd_reduce");
-  hipLaunchKernelGGL(k_bwd_finalize, dim3(static_cast<unsigned>(dlmi_ceil_div(H, kBlock))), block, 0, ctx->stream,
+  hipLaunchKernelGGL(k_bwd_finalize, dim3(static_cast<unsigned>(dlmi_ceil_div(H, kFinCols))), block, 0, ctx->stream,
                      partial, g.nchunks, B, H, c.gamma, c.stdv, c.r, c.dgamma, c.dbeta, c.dmean, c.dstd, coef);
   DLMI_LAUNCH_CHECK(ctx, "k_bwd_finalize");
   if (c.xhat_given) {
