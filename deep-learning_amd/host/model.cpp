@@ -1,0 +1,532 @@
+// Implementation of the host-side Model facade (include/dlmi_model.hpp): the
+// reference's dispatcher order for a stack of fully-connected layers, with every
+// computation done by the HIP kernels behind the C ABI of include/dlmi.h.
+//
+// Dispatcher order followed (paths under /root/reference/lib/deep-learning/):
+//   forward   v1/learner/fwp_st.cpp:118-185 (batch loop), :298-733 (layer)
+//   error     v1/learner/compute_error_st.cpp:26-131
+//   backward  v1/learner/bwp_st.cpp:80-185 (batch loop), :543-701 (layer)
+//   dW / db   v1/learner/update_derivative_fwp_st.cpp:189-244
+// Parameter array layout: v1/learner/connections_prepare.cpp:25-45, 225-234 and
+// allocate.cpp:1150-1177:  [ W_1 .. W_{L-1} | b_1 .. b_{L-1} | gamma(all layers,
+// input included) | beta(all layers) ],  W_l row-major [H_l][K_l].
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "../../include/dlmi_model.hpp"
+
+namespace dlmi {
+namespace v1 {
+
+struct Model::Impl {
+  dlmi_ctx *ctx = nullptr;
+  hipStream_t stream = nullptr;
+  float *d_params = nullptr;   // [P]
+  float *d_dparams = nullptr;  // [P]
+  float *d_mov_mean = nullptr, *d_mov_std = nullptr;  // [units]
+  float *d_input = nullptr;    // [batch, n_in]
+  float *d_targets = nullptr;  // [batch, n_out]
+  double *d_stats = nullptr;   // { loss sum, correct count }
+  float *h_stage = nullptr;    // pinned staging for the row-pointer gather
+  size_t h_stage_floats = 0;
+  mutable std::vector<float> out_host;  // get_out() cache
+  mutable bool out_valid = false;
+  size_t out_batch = 0;
+  size_t allocated_batch = 0;
+  mutable std::string err;
+};
+
+namespace {
+bool hip_ok(hipError_t e, std::string &err, char const *what) {
+  if (e == hipSuccess) return true;
+  err = std::string(what) + ": " + hipGetErrorString(e);
+  std::fprintf(stderr, "dlmi::Model: %s\n", err.c_str());
+  return false;
+}
+template <typename T>
+bool dev_alloc(T **p, size_t n, std::string &err) {
+  void *q = nullptr;
+  if (!hip_ok(hipMalloc(&q, (n ? n : 1) * sizeof(T)), err, "hipMalloc")) return false;
+  *p = static_cast<T *>(q);
+  return true;
+}
+template <typename T>
+void dev_free(T *&p) {
+  if (p != nullptr) (void)hipFree(p);
+  p = nullptr;
+}
+bool act_on_path(ACTIVATION::TYPE t) {
+  switch (t) {
+    case ACTIVATION::ELU: case ACTIVATION::ISRLU: case ACTIVATION::LINEAR: case ACTIVATION::LEAKY_RELU:
+    case ACTIVATION::RELU: case ACTIVATION::SELU:
+      return true;
+    default:
+      return false;
+  }
+}
+}  // namespace
+
+Model::Model(void) : impl_(new Impl) { real_gen.seed(5489u); }
+
+Model::~Model(void) {
+  if (impl_->ctx != nullptr) (void)dlmi_ctx_synchronize(impl_->ctx);
+  free_batch();
+  dev_free(impl_->d_params);
+  dev_free(impl_->d_dparams);
+  dev_free(impl_->d_mov_mean);
+  dev_free(impl_->d_mov_std);
+  dev_free(impl_->d_stats);
+  if (ptr_array_layers != nullptr)
+    for (Layer *l = ptr_array_layers; l != ptr_last_layer; ++l) {
+      dev_free(l->d_mean); dev_free(l->d_std); dev_free(l->d_r); dev_free(l->d_d); dev_free(l->d_mask);
+    }
+  if (impl_->h_stage != nullptr) (void)hipHostFree(impl_->h_stage);
+  if (impl_->ctx != nullptr) (void)dlmi_ctx_destroy(impl_->ctx);
+  delete[] ptr_array_layers;
+  delete[] ptr_array_parameters;
+  delete[] ptr_array_derivatives_parameters;
+  delete[] ptr_array_normalized_batch_units_means_averages;
+  delete[] ptr_array_normalized_batch_units_variances_averages;
+  delete impl_;
+}
+
+bool Model::fail(char const *what) const {
+  impl_->err = what;
+  if (impl_->ctx != nullptr && dlmi_last_error(impl_->ctx)[0] != '\0')
+    impl_->err += std::string(" (") + dlmi_last_error(impl_->ctx) + ")";
+  std::fprintf(stderr, "dlmi::Model: %s\n", impl_->err.c_str());  // the reference logs and carries on
+  return false;
+}
+
+char const *Model::last_error(void) const { return impl_->err.c_str(); }
+
+bool Model::synchronize(void) const {
+  return impl_->ctx != nullptr && dlmi_ctx_synchronize(impl_->ctx) == DLMI_OK;
+}
+
+// ---------------------------------------------------------------- construction
+bool Model::compile(size_t const n_layers, size_t const number_recurrent_depth_received,
+                    MODEL::TYPE const type_network_received, Layer_Parameters const *const lp,
+                    size_t const /*allowable_memory: HBM is not budgeted the way host RAM is*/) {
+  if (ptr_array_layers != nullptr) return fail("compile: the model is already compiled");
+  if (n_layers < 2 || lp == nullptr) return fail("compile: need an input layer and an output layer");
+  if (number_recurrent_depth_received != 1) return fail("compile: only seq_w = 1 (no recurrence) is on this path");
+  if (type_network_received != MODEL::FEEDFORWARD) return fail("compile: only MODEL::FEEDFORWARD is on this path");
+  for (size_t i = 0; i < n_layers; ++i) {
+    if (lp[i].type_layer != LAYER::FULLY_CONNECTED) return fail("compile: only LAYER::FULLY_CONNECTED is on this path");
+    if (lp[i].unit_parameters[0] == 0) return fail("compile: a layer has no units");
+  }
+  if (dlmi_ctx_create(&impl_->ctx, 0, nullptr) != DLMI_OK)
+    return fail("compile: no gfx950 device / context (there is no CPU path)");
+  type = type_network_received;
+  seq_w = 1;
+  total_layers = n_layers;
+  ptr_array_layers = new Layer[n_layers];
+  ptr_last_layer = ptr_array_layers + n_layers;
+  size_t nw = 0, nb = 0, nu = 0;
+  for (size_t i = 0; i < n_layers; ++i) {
+    Layer &l = ptr_array_layers[i];
+    l.type_layer = LAYER::FULLY_CONNECTED;
+    l.n_out = lp[i].unit_parameters[0];
+    l.unit_index = nu;
+    nu += l.n_out;
+    if (i > 0) {
+      l.first_connection_index = nw;
+      nw += l.n_out * ptr_array_layers[i - 1].n_out;
+    }
+  }
+  for (size_t i = 1; i < n_layers; ++i) {
+    ptr_array_layers[i].first_bias_connection_index = nw + nb;
+    nb += ptr_array_layers[i].n_out;
+  }
+  for (size_t i = 0; i < n_layers; ++i) {
+    ptr_array_layers[i].scale_index = nw + nb + ptr_array_layers[i].unit_index;
+    ptr_array_layers[i].shift_index = nw + nb + nu + ptr_array_layers[i].unit_index;
+  }
+  total_weights = nw;
+  total_bias = nb;
+  total_normalized_units = nu;
+  total_parameters = nw + nb + 2 * nu;
+  ptr_array_parameters = new var[total_parameters]();
+  ptr_array_derivatives_parameters = new real[total_parameters]();
+  ptr_array_normalized_batch_units_means_averages = new var[nu]();
+  ptr_array_normalized_batch_units_variances_averages = new var[nu];
+  for (size_t i = 0; i < nu; ++i) {  // allocate.cpp:1167-1170, 1274-1284
+    ptr_array_parameters[nw + nb + i] = 1.0f;
+    ptr_array_normalized_batch_units_variances_averages[i] = 1.0f;
+  }
+  std::string &err = impl_->err;
+  if (!dev_alloc(&impl_->d_params, total_parameters, err) || !dev_alloc(&impl_->d_dparams, total_parameters, err) ||
+      !dev_alloc(&impl_->d_mov_mean, nu, err) || !dev_alloc(&impl_->d_mov_std, nu, err) ||
+      !dev_alloc(&impl_->d_stats, 2, err))
+    return false;
+  for (size_t i = 1; i < n_layers; ++i) {
+    Layer &l = ptr_array_layers[i];
+    if (!dev_alloc(&l.d_mean, l.n_out, err) || !dev_alloc(&l.d_std, l.n_out, err) ||
+        !dev_alloc(&l.d_r, l.n_out, err) || !dev_alloc(&l.d_d, l.n_out, err) || !dev_alloc(&l.d_mask, l.n_out, err))
+      return false;
+    l.mask_dropout_bernoulli.assign(l.n_out, 1);
+  }
+  if (!hip_ok(hipMemsetAsync(impl_->d_dparams, 0, total_parameters * sizeof(float), impl_->stream), err, "memset") ||
+      !hip_ok(hipMemsetAsync(impl_->d_stats, 0, 2 * sizeof(double), impl_->stream), err, "memset"))
+    return false;
+  return upload_parameters() && upload_moving_statistics() && set_max_batch_size(1) && update_mem_batch_size(1);
+}
+
+bool Model::set_layer_activation_function(size_t const i, ACTIVATION::TYPE const t) {
+  if (ptr_array_layers == nullptr || i == 0 || i >= total_layers) return fail("set_layer_activation_function: bad layer index");
+  if (t == ACTIVATION::SOFTMAX) {
+    if (i + 1 != total_layers) return fail("softmax is only available on the output layer");  // train.cpp:400-406
+  } else if (!act_on_path(t)) {
+    return fail("set_layer_activation_function: activation not implemented on this path");
+  }
+  ptr_array_layers[i].type_activation_function = t;
+  return true;
+}
+
+bool Model::Set__Layer_Normalization(size_t const i, LAYER_NORM::TYPE const t, bool const, bool const) {
+  if (ptr_array_layers == nullptr || i >= total_layers) return fail("Set__Layer_Normalization: bad layer index");
+  // normalization.cpp:206-215: refused on the input and on the output layer
+  if (i == 0) return fail("Layer received as argument is the input layer.");
+  if (i + 1 == total_layers) return fail("Layer received as argument is the output layer.");
+  if (t != LAYER_NORM::NONE && t != LAYER_NORM::BATCH_NORMALIZATION && t != LAYER_NORM::BATCH_RENORMALIZATION)
+    return fail("Set__Layer_Normalization: normalization type not implemented on this path");
+  ptr_array_layers[i].type_normalization = t;
+  return true;
+}
+
+bool Model::Set__Normalization_Momentum_Average(real const v) {
+  normalization_momentum_average = v;
+  return true;
+}
+bool Model::Set__Normalization_Epsilon(real const v) {
+  normalization_epsilon = v;
+  return true;
+}
+bool Model::Set__Batch_Renormalization_r_Correction_Maximum(real const v) {
+  batch_renormalization_r_correction_maximum = v;
+  return true;
+}
+bool Model::Set__Batch_Renormalization_d_Correction_Maximum(real const v) {
+  batch_renormalization_d_correction_maximum = v;
+  return true;
+}
+
+bool Model::set_dropout(size_t const i, LAYER_DROPOUT::TYPE const t, real const values[], bool const) {
+  if (ptr_array_layers == nullptr || i == 0 || i >= total_layers) return fail("set_dropout: bad layer index");
+  if (t != LAYER_DROPOUT::NONE && t != LAYER_DROPOUT::BERNOULLI && t != LAYER_DROPOUT::BERNOULLI_INVERTED)
+    return fail("set_dropout: dropout type not implemented on this path");
+  Layer &l = ptr_array_layers[i];
+  if (t != LAYER_DROPOUT::NONE) {
+    if (values == nullptr || values[0] < 0.0f || values[0] > 1.0f) return fail("set_dropout: keep probability out of [0, 1]");
+    l.dropout_values[0] = values[0];
+  }
+  l.type_dropout = t;
+  return true;
+}
+
+bool Model::set_dropout_mask(size_t const i, uint8_t const *mask) {
+  if (ptr_array_layers == nullptr || i == 0 || i >= total_layers || mask == nullptr) return fail("set_dropout_mask: bad argument");
+  Layer &l = ptr_array_layers[i];
+  l.mask_dropout_bernoulli.assign(mask, mask + l.n_out);
+  return hip_ok(hipMemcpy(l.d_mask, l.mask_dropout_bernoulli.data(), l.n_out, hipMemcpyHostToDevice), impl_->err, "mask upload");
+}
+
+void Model::Dropout_Bernoulli(void) {
+  for (size_t i = 1; i < total_layers; ++i) {
+    Layer &l = ptr_array_layers[i];
+    if (!l.Use__Dropout()) continue;
+    real const keep = l.dropout_values[0];
+    std::bernoulli_distribution dist(keep);
+    for (size_t j = 0; j < l.n_out; ++j) l.mask_dropout_bernoulli[j] = keep != 0.0f ? (dist(real_gen) ? 1 : 0) : 0;
+    (void)hipMemcpy(l.d_mask, l.mask_dropout_bernoulli.data(), l.n_out, hipMemcpyHostToDevice);
+  }
+}
+
+bool Model::set_max_batch_size(size_t const n) {
+  if (n == 0) return fail("Maximum batch size can not be equal to zero.");  // model.cpp:2652
+  maximum_batch_size = n;
+  return true;
+}
+
+void Model::free_batch(void) {
+  if (ptr_array_layers != nullptr)
+    for (Layer *l = ptr_array_layers; l != ptr_last_layer; ++l) {
+      dev_free(l->d_summations); dev_free(l->d_outputs); dev_free(l->d_errors);
+    }
+  dev_free(impl_->d_input);
+  dev_free(impl_->d_targets);
+  impl_->allocated_batch = 0;
+}
+
+bool Model::allocate_batch(size_t const n) {
+  if (impl_->ctx != nullptr) (void)dlmi_ctx_synchronize(impl_->ctx);
+  free_batch();
+  std::string &err = impl_->err;
+  for (size_t i = 1; i < total_layers; ++i) {
+    Layer &l = ptr_array_layers[i];
+    if (!dev_alloc(&l.d_summations, n * l.n_out, err) || !dev_alloc(&l.d_outputs, n * l.n_out, err) ||
+        !dev_alloc(&l.d_errors, n * l.n_out, err))
+      return false;
+  }
+  size_t const n_in = ptr_array_layers[0].n_out, n_o = ptr_array_layers[total_layers - 1].n_out;
+  if (!dev_alloc(&impl_->d_input, n * n_in, err) || !dev_alloc(&impl_->d_targets, n * n_o, err)) return false;
+  size_t const stage = n * (n_in > n_o ? n_in : n_o);
+  if (stage > impl_->h_stage_floats) {
+    if (impl_->h_stage != nullptr) (void)hipHostFree(impl_->h_stage);
+    impl_->h_stage = nullptr;
+    void *p = nullptr;
+    if (!hip_ok(hipHostMalloc(&p, stage * sizeof(float), hipHostMallocDefault), err, "hipHostMalloc")) return false;
+    impl_->h_stage = static_cast<float *>(p);
+    impl_->h_stage_floats = stage;
+  }
+  impl_->allocated_batch = n;
+  return true;
+}
+
+bool Model::update_mem_batch_size(size_t const desired, bool const force) {
+  if (ptr_array_layers == nullptr) return fail("update_mem_batch_size: the model is not compiled");
+  size_t const n = desired < maximum_batch_size ? desired : maximum_batch_size;  // update_size.cpp:26-116
+  if (n == 0) return fail("update_mem_batch_size: batch size 0");
+  if (n == impl_->allocated_batch && !force) {
+    batch_size = n;
+    return true;
+  }
+  if (!allocate_batch(n)) return false;
+  batch_size = n;
+  return true;
+}
+
+void Model::clear_training_arrays(void) {
+  if (impl_->d_dparams == nullptr) return;
+  (void)hipMemsetAsync(impl_->d_dparams, 0, total_parameters * sizeof(float), impl_->stream);
+  (void)hipMemsetAsync(impl_->d_stats, 0, 2 * sizeof(double), impl_->stream);
+  std::memset(ptr_array_derivatives_parameters, 0, total_parameters * sizeof(real));
+}
+
+// ---------------------------------------------------------------- buffer movement
+bool Model::upload_parameters(void) {
+  return hip_ok(hipMemcpy(impl_->d_params, ptr_array_parameters, total_parameters * sizeof(float), hipMemcpyHostToDevice),
+                impl_->err, "parameter upload");
+}
+bool Model::download_parameters(void) {
+  return hip_ok(hipMemcpy(ptr_array_parameters, impl_->d_params, total_parameters * sizeof(float), hipMemcpyDeviceToHost),
+                impl_->err, "parameter download");
+}
+bool Model::download_derivatives(void) {
+  return hip_ok(hipMemcpy(ptr_array_derivatives_parameters, impl_->d_dparams, total_parameters * sizeof(float),
+                          hipMemcpyDeviceToHost), impl_->err, "gradient download");
+}
+bool Model::upload_moving_statistics(void) {
+  size_t const n = total_normalized_units * sizeof(float);
+  return hip_ok(hipMemcpy(impl_->d_mov_mean, ptr_array_normalized_batch_units_means_averages, n, hipMemcpyHostToDevice),
+                impl_->err, "moving mean upload") &&
+         hip_ok(hipMemcpy(impl_->d_mov_std, ptr_array_normalized_batch_units_variances_averages, n, hipMemcpyHostToDevice),
+                impl_->err, "moving std upload");
+}
+bool Model::download_moving_statistics(void) {
+  size_t const n = total_normalized_units * sizeof(float);
+  return hip_ok(hipMemcpy(ptr_array_normalized_batch_units_means_averages, impl_->d_mov_mean, n, hipMemcpyDeviceToHost),
+                impl_->err, "moving mean download") &&
+         hip_ok(hipMemcpy(ptr_array_normalized_batch_units_variances_averages, impl_->d_mov_std, n, hipMemcpyDeviceToHost),
+                impl_->err, "moving std download");
+}
+
+bool Model::download_layer(size_t const i, int which, size_t batch, float *out) const {
+  if (ptr_array_layers == nullptr || i == 0 || i >= total_layers || out == nullptr) return fail("download_layer: bad argument");
+  Layer const &l = ptr_array_layers[i];
+  float const *src = nullptr;
+  size_t n = batch * l.n_out;
+  switch (which) {
+    case 0: src = l.d_summations; break;
+    case 3: src = l.d_outputs; break;
+    case 4: src = l.d_errors; break;
+    case 10: src = l.d_mean; n = l.n_out; break;
+    case 11: src = l.d_std; n = l.n_out; break;
+    case 12: src = l.d_r; n = l.n_out; break;
+    case 13: src = l.d_d; n = l.n_out; break;
+    default: return fail("download_layer: unknown buffer");
+  }
+  if (batch > impl_->allocated_batch) return fail("download_layer: batch larger than the allocation");
+  return hip_ok(hipMemcpy(out, src, n * sizeof(float), hipMemcpyDeviceToHost), impl_->err, "layer download");
+}
+
+double Model::get_loss_sum(void) const {
+  double s[2] = {0, 0};
+  (void)hipMemcpy(s, impl_->d_stats, sizeof(s), hipMemcpyDeviceToHost);
+  return s[0];
+}
+double Model::get_accuracy_sum(void) const {
+  double s[2] = {0, 0};
+  (void)hipMemcpy(s, impl_->d_stats, sizeof(s), hipMemcpyDeviceToHost);
+  return s[1];
+}
+
+// ---------------------------------------------------------------- the hot path
+static dlmi_fused_desc make_desc(Model const &m, Layer const &l) {
+  dlmi_fused_desc d;
+  d.norm = l.type_normalization == LAYER_NORM::BATCH_RENORMALIZATION ? DLMI_NORM_BATCH_RENORM : DLMI_NORM_BATCH;
+  d.act = static_cast<dlmi_activation>(l.type_activation_function);
+  d.dropout = static_cast<dlmi_dropout>(l.type_dropout);
+  d.mask_per_element = 0;
+  d.dropout_bwd = m.dropout_backward_mode;
+  d.momentum = m.normalization_momentum_average;
+  d.eps = m.normalization_epsilon;
+  d.r_max = m.batch_renormalization_r_correction_maximum;
+  d.d_max = m.batch_renormalization_d_correction_maximum;
+  // fwp_st.cpp:674: 1/keep, 0 when keep == 0; plain Bernoulli does not rescale in training
+  d.drop_scale = l.type_dropout == LAYER_DROPOUT::BERNOULLI_INVERTED
+                     ? (l.dropout_values[0] == 0.0f ? 0.0f : 1.0f / l.dropout_values[0])
+                     : 1.0f;
+  return d;
+}
+
+void Model::forward_pass(size_t const B, real const *const *const Xm, long long int in_idx, long long int out_idx) {
+  if (ptr_array_layers == nullptr || Xm == nullptr) { fail("forward_pass: model not compiled or null input"); return; }
+  if (in_idx == -1ll) in_idx = 0;
+  if (out_idx == -1ll) out_idx = static_cast<long long>(total_layers);
+  if (in_idx != 0 || out_idx != static_cast<long long>(total_layers)) { fail("forward_pass: only whole-network passes are on this path"); return; }
+  if (B == 0 || B > impl_->allocated_batch) { fail("forward_pass: batch size exceeds update_mem_batch_size()"); return; }
+  dlmi_ctx *ctx = impl_->ctx;
+  size_t const n_in = ptr_array_layers[0].n_out;
+  // assign_inputs.cpp:22-40: gather the row pointers into a dense [B, K] block
+  // (pinned staging buffer: the previous step's copy out of it has completed
+  // once the stream is idle)
+  (void)hipStreamSynchronize(impl_->stream);
+  for (size_t i = 0; i < B; ++i) std::memcpy(impl_->h_stage + i * n_in, Xm[i], n_in * sizeof(float));
+  if (!hip_ok(hipMemcpyAsync(impl_->d_input, impl_->h_stage, B * n_in * sizeof(float), hipMemcpyHostToDevice, impl_->stream),
+              impl_->err, "input upload"))
+    return;
+  bool const training = type_state_propagation >= PROPAGATION::TRAINING;
+  float const *in = impl_->d_input;
+  size_t K = n_in;
+  for (size_t li = 1; li < total_layers; ++li) {
+    Layer &l = ptr_array_layers[li];
+    size_t const H = l.n_out;
+    float const *W = impl_->d_params + l.first_connection_index;
+    float const *bias = l.Use__Bias() ? impl_->d_params + l.first_bias_connection_index : nullptr;
+    if (dlmi_fc_fwd(ctx, B, K, H, in, W, bias, l.d_summations) != DLMI_OK) { fail("forward_pass: dlmi_fc_fwd"); return; }
+    bool const softmax = l.type_activation_function == ACTIVATION::SOFTMAX;
+    if (!softmax && !act_on_path(l.type_activation_function)) { fail("forward_pass: layer activation not set to one on this path"); return; }
+    int rc = DLMI_OK;
+    if (l.Use__Normalization()) {
+      dlmi_fused_desc d = make_desc(*this, l);
+      float const *gamma = impl_->d_params + l.scale_index, *beta = impl_->d_params + l.shift_index;
+      float *mm = impl_->d_mov_mean + l.unit_index, *ms = impl_->d_mov_std + l.unit_index;
+      if (training) {
+        // dropout acts only in PROPAGATION::TRAINING, not in UPDATE_BATCH_NORM (fwp_st.cpp:657)
+        if (type_state_propagation != PROPAGATION::TRAINING) d.dropout = DLMI_DROP_NONE;
+        rc = dlmi_fused_norm_act_fwd(ctx, &d, B, H, l.d_summations, gamma, beta, l.d_mask, l.d_mean, l.d_std, mm, ms,
+                                     l.d_r, l.d_d, l.d_outputs);
+        if (rc == DLMI_OK && type_state_propagation != PROPAGATION::TRAINING && l.Use__Dropout())
+          rc = dlmi_dropout_fwd(ctx, static_cast<dlmi_dropout>(l.type_dropout), 0, 0, B, H, nullptr, l.dropout_values[0],
+                                l.d_outputs);
+      } else {
+        d.drop_scale = l.dropout_values[0];  // plain Bernoulli rescales by keep at inference (fwp_st.cpp:705-716)
+        rc = dlmi_fused_norm_act_infer(ctx, &d, B, H, l.d_summations, gamma, beta, mm, ms, l.d_outputs);
+      }
+    } else {
+      rc = softmax ? dlmi_softmax_fwd(ctx, B, H, l.d_summations, l.d_outputs)
+                   : dlmi_act_fwd(ctx, static_cast<dlmi_activation>(l.type_activation_function), B, H, l.d_summations,
+                                  l.d_outputs);
+      if (rc == DLMI_OK && l.Use__Dropout()) {
+        if (type_state_propagation == PROPAGATION::TRAINING)
+          rc = dlmi_dropout_fwd(ctx, static_cast<dlmi_dropout>(l.type_dropout), 1, 0, B, H, l.d_mask,
+                                l.dropout_values[0] == 0.0f ? 0.0f : 1.0f / l.dropout_values[0], l.d_outputs);
+        else  // every other state: plain Bernoulli rescales by keep (fwp_st.cpp:705-716)
+          rc = dlmi_dropout_fwd(ctx, static_cast<dlmi_dropout>(l.type_dropout), 0, 0, B, H, nullptr, l.dropout_values[0],
+                                l.d_outputs);
+      }
+    }
+    if (rc != DLMI_OK) { fail("forward_pass: layer tail"); return; }
+    in = l.d_outputs;
+    K = H;
+  }
+  impl_->out_valid = false;
+  impl_->out_batch = B;
+}
+
+var const *Model::get_out(size_t const data_index, size_t const) const {
+  if (ptr_array_layers == nullptr || data_index >= impl_->out_batch) { fail("get_out: no such row"); return nullptr; }
+  Layer const &o = ptr_array_layers[total_layers - 1];
+  if (!impl_->out_valid) {
+    impl_->out_host.resize(impl_->out_batch * o.n_out);
+    if (!hip_ok(hipMemcpy(impl_->out_host.data(), o.d_outputs, impl_->out_host.size() * sizeof(float),
+                          hipMemcpyDeviceToHost), impl_->err, "output download"))
+      return nullptr;
+    impl_->out_valid = true;
+  }
+  return impl_->out_host.data() + data_index * o.n_out;
+}
+
+void Model::compute_error(size_t const B, real const *const *const Ym) {
+  if (ptr_array_layers == nullptr || Ym == nullptr || B == 0 || B > impl_->allocated_batch) { fail("compute_error: bad argument"); return; }
+  Layer &o = ptr_array_layers[total_layers - 1];
+  if (o.type_activation_function != ACTIVATION::SOFTMAX || type_loss_function != LOSS_FN::CROSS_ENTROPY) {
+    fail("compute_error: only softmax + cross-entropy is on this path");
+    return;
+  }
+  size_t const H = o.n_out;
+  (void)hipStreamSynchronize(impl_->stream);
+  for (size_t i = 0; i < B; ++i) std::memcpy(impl_->h_stage + i * H, Ym[i], H * sizeof(float));
+  if (!hip_ok(hipMemcpyAsync(impl_->d_targets, impl_->h_stage, B * H * sizeof(float), hipMemcpyHostToDevice, impl_->stream),
+              impl_->err, "target upload"))
+    return;
+  if (dlmi_softmax_ce_seed(impl_->ctx, B, H, o.d_outputs, impl_->d_targets, o.d_errors, impl_->d_stats) != DLMI_OK)
+    fail("compute_error: dlmi_softmax_ce_seed");
+}
+
+void Model::backward_pass(size_t const B) {
+  if (ptr_array_layers == nullptr || B == 0 || B > impl_->allocated_batch) { fail("backward_pass: bad argument"); return; }
+  dlmi_ctx *ctx = impl_->ctx;
+  // bwp_st.cpp:106-183: from the layer below the output down to layer 1; the
+  // gradient with respect to the network input is never formed.
+  for (size_t li = total_layers - 2; li >= 1; --li) {
+    Layer &l = ptr_array_layers[li];
+    Layer const &nx = ptr_array_layers[li + 1];
+    size_t const H = l.n_out;
+    // dY = dZ_next . W_next, written straight over the (would-be zeroed) buffer
+    if (dlmi_fc_bwd_dx(ctx, B, nx.n_out, H, nx.d_errors, impl_->d_params + nx.first_connection_index, l.d_errors, 0) != DLMI_OK) {
+      fail("backward_pass: dlmi_fc_bwd_dx");
+      return;
+    }
+    int rc;
+    if (l.Use__Normalization()) {
+      dlmi_fused_desc d = make_desc(*this, l);
+      if (type_state_propagation != PROPAGATION::TRAINING) d.dropout = DLMI_DROP_NONE;
+      rc = dlmi_fused_norm_act_bwd(ctx, &d, B, H, l.d_summations, impl_->d_params + l.scale_index,
+                                   impl_->d_params + l.shift_index, l.d_mask, l.d_mean, l.d_std, l.d_r, l.d_d, l.d_errors,
+                                   impl_->d_dparams + l.scale_index, impl_->d_dparams + l.shift_index, l.d_errors);
+    } else {
+      // dN = dY * f'(Z, post-dropout output), in place (bwp_st.cpp:1177-1209)
+      rc = dlmi_act_bwd(ctx, static_cast<dlmi_activation>(l.type_activation_function), B, H, l.d_summations, l.d_outputs,
+                        l.d_errors, l.d_errors);
+    }
+    if (rc != DLMI_OK) { fail("backward_pass: layer gradient"); return; }
+    if (li == 1) break;
+  }
+}
+
+void Model::update_derivatives(size_t const B, Layer *const first, Layer const *const last) {
+  if (ptr_array_layers == nullptr || first == nullptr || last == nullptr || B == 0 || B > impl_->allocated_batch) {
+    fail("update_derivatives: bad argument");
+    return;
+  }
+  for (Layer *l = first; l != last; ++l) {
+    size_t const li = static_cast<size_t>(l - ptr_array_layers);
+    if (li == 0 || li >= total_layers) continue;
+    float const *in = li == 1 ? impl_->d_input : ptr_array_layers[li - 1].d_outputs;
+    size_t const K = ptr_array_layers[li - 1].n_out;
+    float *db = l->Use__Bias() ? impl_->d_dparams + l->first_bias_connection_index : nullptr;
+    if (dlmi_fc_bwd_dw(impl_->ctx, B, K, l->n_out, in, l->d_errors, impl_->d_dparams + l->first_connection_index, db, 1) != DLMI_OK) {
+      fail("update_derivatives: dlmi_fc_bwd_dw");
+      return;
+    }
+  }
+}
+
+}  // namespace v1
+}  // namespace dlmi

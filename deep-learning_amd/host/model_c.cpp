@@ -1,0 +1,137 @@
+// C binding of the Model facade (include/dlmi_model.h).
+#include <cstring>
+#include <vector>
+
+#include "../../include/dlmi_model.h"
+#include "../../include/dlmi_model.hpp"
+
+using namespace dlmi::v1;
+
+struct dlmi_model {
+  Model m;
+};
+
+extern "C" {
+
+dlmi_model *dlmi_model_create(size_t n_layers, size_t const *widths) {
+  if (widths == nullptr) return nullptr;
+  dlmi_model *h = new dlmi_model;
+  std::vector<Layer_Parameters> lp(n_layers);
+  for (size_t i = 0; i < n_layers; ++i) {
+    lp[i].type_layer = LAYER::FULLY_CONNECTED;
+    lp[i].unit_parameters[0] = widths[i];
+  }
+  if (!h->m.compile(n_layers, 1, MODEL::FEEDFORWARD, lp.data())) {
+    delete h;
+    return nullptr;
+  }
+  return h;
+}
+
+void dlmi_model_destroy(dlmi_model *h) { delete h; }
+char const *dlmi_model_last_error(dlmi_model const *h) { return h ? h->m.last_error() : "null model"; }
+
+int dlmi_model_set_layer_activation_function(dlmi_model *h, size_t layer, int a) {
+  return h->m.set_layer_activation_function(layer, static_cast<ACTIVATION::TYPE>(a));
+}
+int dlmi_model_set_layer_normalization(dlmi_model *h, size_t layer, int n) {
+  return h->m.Set__Layer_Normalization(layer, static_cast<LAYER_NORM::TYPE>(n));
+}
+int dlmi_model_set_norm_hyper(dlmi_model *h, float momentum, float eps, float r_max, float d_max) {
+  bool ok = h->m.Set__Normalization_Momentum_Average(momentum);
+  ok = h->m.Set__Normalization_Epsilon(eps) && ok;
+  ok = h->m.Set__Batch_Renormalization_r_Correction_Maximum(r_max) && ok;
+  ok = h->m.Set__Batch_Renormalization_d_Correction_Maximum(d_max) && ok;
+  return ok;
+}
+int dlmi_model_set_dropout(dlmi_model *h, size_t layer, int d, float keep) {
+  real values[3] = {keep, 0, 0};
+  return h->m.set_dropout(layer, static_cast<LAYER_DROPOUT::TYPE>(d), values);
+}
+int dlmi_model_set_dropout_mask(dlmi_model *h, size_t layer, uint8_t const *mask) {
+  return h->m.set_dropout_mask(layer, mask);
+}
+int dlmi_model_set_dropout_backward_mode(dlmi_model *h, int mode) {
+  h->m.dropout_backward_mode = mode ? DLMI_DROP_BWD_MASKED : DLMI_DROP_BWD_REFERENCE;
+  return 1;
+}
+int dlmi_model_prepare(dlmi_model *h, size_t max_batch) {
+  h->m.set_loss_fn(LOSS_FN::CROSS_ENTROPY);
+  h->m.set_accu_fn(ACCU_FN::CROSS_ENTROPY);
+  if (!h->m.set_max_batch_size(max_batch) || !h->m.update_mem_batch_size(max_batch)) return 0;
+  h->m.set_mp(true);
+  h->m.update_mem_thread_size(max_batch);
+  h->m.clear_training_arrays();
+  return 1;
+}
+size_t dlmi_model_total_parameters(dlmi_model const *h) { return h->m.total_parameters; }
+size_t dlmi_model_total_normalized_units(dlmi_model const *h) { return h->m.total_normalized_units; }
+void dlmi_model_layer_offsets(dlmi_model const *h, size_t layer, size_t *out) {
+  Layer const &l = h->m.ptr_array_layers[layer];
+  out[0] = l.first_connection_index;
+  out[1] = l.first_bias_connection_index;
+  out[2] = l.scale_index;
+  out[3] = l.shift_index;
+  out[4] = l.unit_index;
+  out[5] = l.Use__Bias();
+}
+int dlmi_model_set_parameters(dlmi_model *h, float const *p, size_t n) {
+  if (n != h->m.total_parameters) return 0;
+  std::memcpy(h->m.ptr_array_parameters, p, n * sizeof(float));
+  return h->m.upload_parameters();
+}
+int dlmi_model_get_parameters(dlmi_model *h, float *p, size_t n) {
+  if (n != h->m.total_parameters || !h->m.download_parameters()) return 0;
+  std::memcpy(p, h->m.ptr_array_parameters, n * sizeof(float));
+  return 1;
+}
+int dlmi_model_set_moving(dlmi_model *h, float const *mean, float const *stdv, size_t n) {
+  if (n != h->m.total_normalized_units) return 0;
+  std::memcpy(h->m.ptr_array_normalized_batch_units_means_averages, mean, n * sizeof(float));
+  std::memcpy(h->m.ptr_array_normalized_batch_units_variances_averages, stdv, n * sizeof(float));
+  return h->m.upload_moving_statistics();
+}
+int dlmi_model_get_moving(dlmi_model *h, float *mean, float *stdv, size_t n) {
+  if (n != h->m.total_normalized_units || !h->m.download_moving_statistics()) return 0;
+  std::memcpy(mean, h->m.ptr_array_normalized_batch_units_means_averages, n * sizeof(float));
+  std::memcpy(stdv, h->m.ptr_array_normalized_batch_units_variances_averages, n * sizeof(float));
+  return 1;
+}
+int dlmi_model_get_derivatives(dlmi_model *h, float *p, size_t n) {
+  if (n != h->m.total_parameters || !h->m.download_derivatives()) return 0;
+  std::memcpy(p, h->m.ptr_array_derivatives_parameters, n * sizeof(float));
+  return 1;
+}
+void dlmi_model_clear_training_arrays(dlmi_model *h) { h->m.clear_training_arrays(); }
+
+int dlmi_model_step(dlmi_model *h, int state, size_t B, float const *X, float const *Y, int do_backward) {
+  Model &m = h->m;
+  m.type_state_propagation = static_cast<PROPAGATION::TYPE>(state);
+  size_t const K0 = m.ptr_array_layers[0].n_out, Ho = m.Get__Output_Layer()->n_out;
+  std::vector<float const *> Xm(B), Ym(B);
+  for (size_t i = 0; i < B; ++i) {
+    Xm[i] = X + i * K0;
+    Ym[i] = Y ? Y + i * Ho : nullptr;
+  }
+  m.forward_pass(B, Xm.data());
+  if (do_backward) {
+    m.compute_error(B, Ym.data());
+    m.backward_pass(B);
+    m.update_derivatives(B, m.ptr_array_layers + 1, m.ptr_last_layer);
+    m.merge_mp_derivatives(0, m.total_parameters);
+  }
+  return m.synchronize() && m.last_error()[0] == '\0';
+}
+int dlmi_model_download_layer(dlmi_model const *h, size_t layer, int which, size_t batch, float *out) {
+  return h->m.download_layer(layer, which, batch, out);
+}
+int dlmi_model_get_out(dlmi_model const *h, size_t row, float *out) {
+  var const *p = h->m.get_out(row);
+  if (p == nullptr) return 0;
+  std::memcpy(out, p, h->m.Get__Output_Layer()->n_out * sizeof(float));
+  return 1;
+}
+double dlmi_model_loss_sum(dlmi_model const *h) { return h->m.get_loss_sum(); }
+double dlmi_model_accuracy_sum(dlmi_model const *h) { return h->m.get_accuracy_sum(); }
+
+}  // extern "C"

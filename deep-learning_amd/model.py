@@ -1,0 +1,151 @@
+"""ctypes binding of the C++ Model facade (include/dlmi_model.h): the
+reference's Model API for a stack of fully-connected layers, running on the GPU.
+Host numpy arrays go in and out here because that is the boundary the reference
+has (`forward_pass(batch, rows of X)`); the copies to HBM happen inside the
+facade."""
+import ctypes
+
+import numpy as np
+
+c_sz = ctypes.c_size_t
+c_int = ctypes.c_int
+c_f = ctypes.c_float
+vp = ctypes.c_void_p
+
+MODEL_C_ABI_SYMBOLS = [
+    "dlmi_model_create", "dlmi_model_destroy", "dlmi_model_last_error", "dlmi_model_set_layer_activation_function",
+    "dlmi_model_set_layer_normalization", "dlmi_model_set_norm_hyper", "dlmi_model_set_dropout",
+    "dlmi_model_set_dropout_mask", "dlmi_model_set_dropout_backward_mode", "dlmi_model_prepare",
+    "dlmi_model_total_parameters", "dlmi_model_total_normalized_units", "dlmi_model_layer_offsets",
+    "dlmi_model_set_parameters", "dlmi_model_get_parameters", "dlmi_model_set_moving", "dlmi_model_get_moving",
+    "dlmi_model_get_derivatives", "dlmi_model_clear_training_arrays", "dlmi_model_step", "dlmi_model_download_layer",
+    "dlmi_model_get_out", "dlmi_model_loss_sum", "dlmi_model_accuracy_sum",
+]
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(vp)
+
+
+class Model:
+    """Same driving interface as the oracle's and the reference's whole-model
+    wrappers in oracle/binding.py, so one test body can run all three."""
+
+    def __init__(self, lib, widths):
+        self.lib = lib
+        lib.dlmi_model_create.restype = vp
+        lib.dlmi_model_last_error.restype = ctypes.c_char_p
+        lib.dlmi_model_last_error.argtypes = [vp]
+        lib.dlmi_model_total_parameters.restype = c_sz
+        lib.dlmi_model_total_normalized_units.restype = c_sz
+        lib.dlmi_model_loss_sum.restype = ctypes.c_double
+        lib.dlmi_model_accuracy_sum.restype = ctypes.c_double
+        self.widths = [int(w) for w in widths]
+        arr = (c_sz * len(widths))(*self.widths)
+        h = lib.dlmi_model_create(c_sz(len(widths)), arr)
+        if not h:
+            raise RuntimeError("dlmi_model_create failed (no GPU, or the library is not built for it)")
+        self.h = vp(h)
+        self.P = lib.dlmi_model_total_parameters(self.h)
+        self.n_units = lib.dlmi_model_total_normalized_units(self.h)
+        self.max_batch = 0
+
+    def close(self):
+        if getattr(self, "h", None):
+            self.lib.dlmi_model_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _ok(self, rc, what):
+        if not rc:
+            raise RuntimeError("%s failed: %s" % (what, self.lib.dlmi_model_last_error(self.h).decode()))
+
+    def set_layer(self, l, act, norm=0, drop=0, keep=1.0, mask=None):
+        self._ok(self.lib.dlmi_model_set_layer_activation_function(self.h, c_sz(l), c_int(act)), "activation")
+        if norm:
+            self._ok(self.lib.dlmi_model_set_layer_normalization(self.h, c_sz(l), c_int(norm)), "normalization")
+        if drop:
+            self._ok(self.lib.dlmi_model_set_dropout(self.h, c_sz(l), c_int(drop), c_f(keep)), "dropout")
+        if mask is not None:
+            m = np.ascontiguousarray(mask, dtype=np.uint8)
+            self._ok(self.lib.dlmi_model_set_dropout_mask(self.h, c_sz(l), _ptr(m)), "dropout mask")
+
+    def set_norm_hyper(self, momentum, eps, r_max, d_max):
+        self._ok(self.lib.dlmi_model_set_norm_hyper(self.h, c_f(momentum), c_f(eps), c_f(r_max), c_f(d_max)), "hyper")
+
+    def set_dropout_backward_mode(self, masked):
+        self.lib.dlmi_model_set_dropout_backward_mode(self.h, c_int(1 if masked else 0))
+
+    def layer_offsets(self, l):
+        out = (c_sz * 6)()
+        self.lib.dlmi_model_layer_offsets(self.h, c_sz(l), out)
+        return list(out)
+
+    def prepare(self, max_batch, nthreads=0):
+        self.max_batch = max_batch
+        self._ok(self.lib.dlmi_model_prepare(self.h, c_sz(max_batch)), "prepare")
+
+    def set_parameters(self, p):
+        p = np.ascontiguousarray(p, np.float32)
+        self._ok(self.lib.dlmi_model_set_parameters(self.h, _ptr(p), c_sz(p.size)), "set_parameters")
+
+    def get_parameters(self):
+        p = np.empty(self.P, np.float32)
+        self._ok(self.lib.dlmi_model_get_parameters(self.h, _ptr(p), c_sz(self.P)), "get_parameters")
+        return p
+
+    def set_moving(self, mean, std):
+        mean = np.ascontiguousarray(mean, np.float32)
+        std = np.ascontiguousarray(std, np.float32)
+        self._ok(self.lib.dlmi_model_set_moving(self.h, _ptr(mean), _ptr(std), c_sz(self.n_units)), "set_moving")
+
+    def get_moving(self):
+        mean = np.empty(self.n_units, np.float32)
+        std = np.empty(self.n_units, np.float32)
+        self._ok(self.lib.dlmi_model_get_moving(self.h, _ptr(mean), _ptr(std), c_sz(self.n_units)), "get_moving")
+        return mean, std
+
+    def clear_training_arrays(self):
+        self.lib.dlmi_model_clear_training_arrays(self.h)
+
+    def step(self, state, X, Y=None, backward=True):
+        X = np.ascontiguousarray(X, np.float32)
+        self.B = X.shape[0]
+        Yp = None
+        if backward:
+            Y = np.ascontiguousarray(Y, np.float32)
+            Yp = _ptr(Y)
+        self._ok(self.lib.dlmi_model_step(self.h, c_int(state), c_sz(self.B), _ptr(X), Yp, c_int(1 if backward else 0)),
+                 "step")
+
+    def layer_buffer(self, l, which):
+        out = np.empty((self.B, self.widths[l]), np.float32)
+        self._ok(self.lib.dlmi_model_download_layer(self.h, c_sz(l), c_int(which), c_sz(self.B), _ptr(out)), "download")
+        return out
+
+    def layer_vector(self, l, which):
+        out = np.empty(self.widths[l], np.float32)
+        self._ok(self.lib.dlmi_model_download_layer(self.h, c_sz(l), c_int(10 + which), c_sz(1), _ptr(out)), "download")
+        return out
+
+    def get_out(self):
+        out = np.empty((self.B, self.widths[-1]), np.float32)
+        for i in range(self.B):
+            self._ok(self.lib.dlmi_model_get_out(self.h, c_sz(i), _ptr(out[i])), "get_out")
+        return out
+
+    def get_dparams(self):
+        p = np.empty(self.P, np.float32)
+        self._ok(self.lib.dlmi_model_get_derivatives(self.h, _ptr(p), c_sz(self.P)), "get_derivatives")
+        return p
+
+    def loss_sum(self):
+        return self.lib.dlmi_model_loss_sum(self.h)
+
+    def accuracy_sum(self):
+        return self.lib.dlmi_model_accuracy_sum(self.h)

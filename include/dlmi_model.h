@@ -1,0 +1,53 @@
+/* C binding of the C++ Model facade (dlmi_model.hpp) for callers that cannot
+ * include C++ headers (the Python tests drive it through ctypes).  Each call
+ * forwards to the member function of the same name, which in turn mirrors the
+ * reference's DL::v1::Model member (lib/deep-learning/v1/learner/model.hpp:752).
+ * Functions returning int give 1 for success and 0 for failure, like the
+ * reference's bool setters. */
+#ifndef DLMI_MODEL_H
+#define DLMI_MODEL_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct dlmi_model dlmi_model;
+
+/* new Model + compile(n_layers, 1, MODEL::FEEDFORWARD, {FULLY_CONNECTED, widths[i]}) */
+dlmi_model *dlmi_model_create(size_t n_layers, size_t const *widths);
+void dlmi_model_destroy(dlmi_model *m);
+char const *dlmi_model_last_error(dlmi_model const *m);
+int dlmi_model_set_layer_activation_function(dlmi_model *m, size_t layer, int activation);
+int dlmi_model_set_layer_normalization(dlmi_model *m, size_t layer, int norm);
+int dlmi_model_set_norm_hyper(dlmi_model *m, float momentum, float eps, float r_max, float d_max);
+int dlmi_model_set_dropout(dlmi_model *m, size_t layer, int dropout, float keep);
+int dlmi_model_set_dropout_mask(dlmi_model *m, size_t layer, uint8_t const *mask_per_unit);
+int dlmi_model_set_dropout_backward_mode(dlmi_model *m, int mode);
+/* set_loss_fn(CROSS_ENTROPY), set_accu_fn(CROSS_ENTROPY), set_max_batch_size, update_mem_batch_size,
+ * clear_training_arrays */
+int dlmi_model_prepare(dlmi_model *m, size_t max_batch);
+size_t dlmi_model_total_parameters(dlmi_model const *m);
+size_t dlmi_model_total_normalized_units(dlmi_model const *m);
+/* out[0..5] = first weight index, first bias index, gamma index, beta index, moving-stat index, Use__Bias() */
+void dlmi_model_layer_offsets(dlmi_model const *m, size_t layer, size_t *out);
+int dlmi_model_set_parameters(dlmi_model *m, float const *p, size_t n);       /* host mirror + upload */
+int dlmi_model_get_parameters(dlmi_model *m, float *p, size_t n);
+int dlmi_model_set_moving(dlmi_model *m, float const *mean, float const *stdv, size_t n);
+int dlmi_model_get_moving(dlmi_model *m, float *mean, float *stdv, size_t n);
+int dlmi_model_get_derivatives(dlmi_model *m, float *p, size_t n);            /* download + copy */
+void dlmi_model_clear_training_arrays(dlmi_model *m);
+/* type_state_propagation = state; forward_pass(B, rows of X); if do_backward: compute_error(B, rows of Y),
+ * backward_pass(B), update_derivatives(B, layers + 1, last_layer).  X [B,K0], Y [B,Hout] dense host arrays. */
+int dlmi_model_step(dlmi_model *m, int state, size_t B, float const *X, float const *Y, int do_backward);
+int dlmi_model_download_layer(dlmi_model const *m, size_t layer, int which, size_t batch, float *out);
+int dlmi_model_get_out(dlmi_model const *m, size_t row, float *out);          /* get_out(row) copied */
+double dlmi_model_loss_sum(dlmi_model const *m);
+double dlmi_model_accuracy_sum(dlmi_model const *m);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DLMI_MODEL_H */

@@ -1,0 +1,200 @@
+// Host-side C++ facade that keeps the reference's Model / Layer API for the
+// fully-connected path (layer construction, forward pass, error seed, backward
+// pass, parameter-gradient accumulation, parameter buffers) and runs it on one
+// MI355X through the C ABI of dlmi.h.
+//
+// Names, argument order and return conventions follow
+// /root/reference/lib/deep-learning/v1/learner/model.hpp (class Model :752,
+// struct Layer :558, struct Layer_Parameters :70) and the enums under
+// v1/data/enum/.  What differs, by design:
+//   * every activation / parameter buffer lives in HBM; the public
+//     `ptr_array_parameters` / `ptr_array_derivatives_parameters` members are
+//     host mirrors that the caller moves with upload_parameters() /
+//     download_derivatives() (the reference's members are the storage itself);
+//   * OpenMP knobs (set_mp, update_mem_thread_size, merge_mp_derivatives) are
+//     accepted and do nothing: there are no per-thread gradient copies to merge;
+//   * only LAYER::FULLY_CONNECTED layers, the activations ReLU / leaky ReLU /
+//     ELU / SELU / ISRLU / linear (+ softmax on the output layer), batch
+//     normalization / renormalization before the activation, Bernoulli and
+//     inverted-Bernoulli dropout and the cross-entropy loss are implemented;
+//     anything else makes the setter return false, as the reference does for
+//     settings it refuses.
+//
+// To compile reference-side code against this header unchanged, define
+// DLMI_ALIAS_DL_NAMESPACE before including it: `DL::v1::Model` then names this
+// class.
+#ifndef DLMI_MODEL_HPP
+#define DLMI_MODEL_HPP
+
+#include <cstddef>
+#include <cstdint>
+#include <random>
+#include <vector>
+
+#include "dlmi.h"
+
+namespace dlmi {
+namespace v1 {
+
+typedef float real;  // lib/framework.hpp:31-37 with NDEBUG
+typedef float var;   // data/dtypes.hpp:68-102 without Adept
+
+// v1/data/enum/*.hpp — values identical to the reference
+struct LAYER { typedef enum : int { NONE = 0, AVERAGE_POOLING = 1, CONVOLUTION = 2, FULLY_CONNECTED = 3,
+  FULLY_CONNECTED_INDEPENDENTLY_RECURRENT = 4, FULLY_CONNECTED_RECURRENT = 5, GRU = 6, LSTM = 7, MAX_POOLING = 8,
+  RESIDUAL = 9, SHORTCUT = 10, LENGTH = 11 } TYPE; };
+struct ACTIVATION { typedef enum : int { NONE = 0, COSINE = 1, COSINE_SYMMETRIC = 2, ELU = 3, ELLIOT = 4,
+  ELLIOT_SYMMETRIC = 5, GAUSSIAN = 6, GAUSSIAN_STEPWISE = 7, GAUSSIAN_SYMMETRIC = 8, ISRU = 9, ISRLU = 10,
+  LINEAR = 11, LINEAR_PIECE = 12, LINEAR_PIECE_SYMMETRIC = 13, LEAKY_RELU = 14, PARAMETRIC_RELU = 15, RELU = 16,
+  SELU = 17, SIGMOID = 18, SINE = 19, SIGMOID_STEPWISE = 20, SINE_SYMMETRIC = 21, SOFTMAX = 22, TANH = 23,
+  TANH_STEPWISE = 24, THRESHOLD = 25, THRESHOLD_SYMMETRIC = 26, LENGTH = 27 } TYPE; };
+struct LAYER_NORM { typedef enum : int { NONE = 0, BATCH_NORMALIZATION = 1, BATCH_RENORMALIZATION = 2,
+  GHOST_BATCH_NORMALIZATION = 3, STREAMING_NORMALIZATION = 4, LENGTH = 5 } TYPE; };
+struct LAYER_DROPOUT { typedef enum : int { NONE = 0, ALPHA = 1, BERNOULLI = 2, BERNOULLI_INVERTED = 3,
+  GAUSSIAN = 4, SHAKEDROP = 5, UOUT = 6, ZONEOUT = 7, LENGTH = 8 } TYPE; };
+struct PROPAGATION { typedef enum : int { INFERENCE = 0, TRAINING = 1, UPDATE_BATCH_NORM = 2, LENGTH = 3 } TYPE; };
+struct MODEL { typedef enum : int { NONE = 0, AUTOENCODER = 1, CONVOLUTIONAL = 2, FEEDFORWARD = 3, RECURRENT = 4,
+  LENGTH = 5 } TYPE; };
+struct LOSS_FN { typedef enum : int { NONE = 0, BIT = 1, CROSS_ENTROPY = 2, L1 = 3, L2 = 4, MAE = 5, MAPE = 6,
+  MASE_NON_SEASONAL = 7, MASE_SEASONAL = 8, ME = 9, MSE = 10, RMSE = 11, SMAPE = 12, LENGTH = 13 } TYPE; };
+struct ACCU_FN { typedef enum : int { NONE = 0, CROSS_ENTROPY = 1, DIRECTIONAL = 2, DISTANCE = 3, R = 4, SIGN = 5,
+  LENGTH = 6 } TYPE; };
+
+// v1/learner/model.hpp:70-93
+struct Layer_Parameters {
+  bool use_bidirectional = false;
+  LAYER::TYPE type_layer = LAYER::NONE;
+  size_t unit_parameters[5] = {0};  // [0]: number of units of a fully-connected layer
+};
+
+// The subset of v1/learner/model.hpp:558-744 this path uses.  Device pointers
+// are row-major [batch_size, n_out].
+struct Layer {
+  LAYER::TYPE type_layer = LAYER::NONE;
+  ACTIVATION::TYPE type_activation_function = ACTIVATION::SIGMOID;  // compile.cpp:627-628 default
+  LAYER_NORM::TYPE type_normalization = LAYER_NORM::NONE;
+  LAYER_DROPOUT::TYPE type_dropout = LAYER_DROPOUT::NONE;
+  bool use_layer_normalization_before_activation = true;
+  real dropout_values[3] = {0};  // [0]: keep probability
+  size_t n_out = 0;
+  size_t first_connection_index = 0;       // offset of W [n_out][n_in] in the parameter array
+  size_t first_bias_connection_index = 0;  // offset of the bias slot [n_out]
+  size_t scale_index = 0, shift_index = 0; // offsets of gamma / beta [n_out]
+  size_t unit_index = 0;                   // offset in the moving-statistic arrays
+  std::vector<uint8_t> mask_dropout_bernoulli;  // host copy of the per-unit mask [n_out]
+
+  float *d_summations = nullptr;          // Z (Neuron_unit::ptr_array_summations)
+  float *d_outputs = nullptr;             // layer output after activation and dropout (ptr_array_outputs)
+  float *d_errors = nullptr;              // dZ (Neuron_unit::ptr_array_errors); holds dY in between
+  float *d_mean = nullptr, *d_std = nullptr, *d_r = nullptr, *d_d = nullptr;  // batch statistics [n_out]
+  uint8_t *d_mask = nullptr;              // device copy of the dropout mask [n_out]
+
+  size_t get_n_out(void) const { return n_out; }
+  bool Use__Normalization(void) const { return type_normalization != LAYER_NORM::NONE; }
+  bool Use__Bias(void) const { return !Use__Normalization(); }  // model.hpp:708
+  bool Use__Dropout(void) const { return type_dropout != LAYER_DROPOUT::NONE; }
+};
+
+class Model {
+ public:
+  Model(void);
+  ~Model(void);
+  Model(Model const &) = delete;
+  Model &operator=(Model const &) = delete;
+
+  // ---- construction (model.hpp:2528; compile.cpp:532-812) -------------------
+  bool compile(size_t const n_layers, size_t const number_recurrent_depth_received,
+               MODEL::TYPE const type_network_received, Layer_Parameters const *const ptr_array_layers_received,
+               size_t const allowable_memory = 32u * 1024u * 1024u);
+  bool set_layer_activation_function(size_t const index_layer_received, ACTIVATION::TYPE const type);
+  bool Set__Layer_Normalization(size_t const index_layer_received, LAYER_NORM::TYPE const type,
+                                bool const reallocate_dimension_parameters_received = true,
+                                bool const organize_pointers_received = true);
+  bool Set__Normalization_Momentum_Average(real const momentum_average_received);
+  bool Set__Normalization_Epsilon(real const epsilon_received);
+  bool Set__Batch_Renormalization_r_Correction_Maximum(real const r_correction_maximum_received);
+  bool Set__Batch_Renormalization_d_Correction_Maximum(real const d_correction_maximum_received);
+  bool set_dropout(size_t const index_layer_received, LAYER_DROPOUT::TYPE const type, real const values[],
+                   bool const scale_weights = true);
+  void set_loss_fn(LOSS_FN::TYPE const type) { type_loss_function = type; }
+  void set_accu_fn(ACCU_FN::TYPE const type) { type_accuracy_function = type; }
+  bool set_max_batch_size(size_t const max_batch_size);
+  bool update_mem_batch_size(size_t const desired_batch_size_received, bool const force_update_received = false);
+  bool set_mp(bool const) { return true; }
+  bool update_mem_thread_size(size_t const) { return true; }
+  void merge_mp_derivatives(size_t const, size_t const) {}
+  void clear_training_arrays(void);  // train.cpp:110-141: zeroes the gradient array
+  void Dropout_Bernoulli(void);      // bernoulli_st.cpp:69-100: resample every per-unit mask
+
+  // ---- the hot path (model.hpp:2980, 1054, 1687, 2156) ----------------------
+  void forward_pass(size_t const batch_size, real const *const *const ptr_array_inputs_received,
+                    long long int input_layer_index_received = -1ll,
+                    long long int output_layer_index_received = -1ll);
+  void compute_error(size_t const batch_size, real const *const *const Ym);
+  void backward_pass(size_t const batch_size);
+  void update_derivatives(size_t const batch_size, Layer *const layer_it, Layer const *const last_layer);
+  // Row `data_index` of the output layer (host pointer, valid until the next call).
+  var const *get_out(size_t const data_index_received, size_t const time_step_index_received = 0) const;
+
+  // ---- buffers moved explicitly between host mirrors and HBM ----------------
+  bool upload_parameters(void);     // ptr_array_parameters -> device
+  bool download_parameters(void);   // device -> ptr_array_parameters
+  bool download_derivatives(void);  // device gradient array -> ptr_array_derivatives_parameters
+  bool upload_moving_statistics(void);
+  bool download_moving_statistics(void);
+  bool set_dropout_mask(size_t const index_layer_received, uint8_t const *mask_per_unit);
+  // Copies a per-layer device buffer [batch, n_out] to `out`.  which: 0 Z,
+  // 3 output, 4 dZ; per-unit vectors [n_out]: 10 mean, 11 std, 12 r, 13 d.
+  bool download_layer(size_t const index_layer_received, int which, size_t batch, float *out) const;
+  double get_loss_sum(void) const;     // sum of cross-entropy losses since clear_training_arrays()
+  double get_accuracy_sum(void) const; // number of correct arg-max predictions since then
+  char const *last_error(void) const;
+  bool synchronize(void) const;
+
+  // ---- public state, as in the reference ------------------------------------
+  size_t total_layers = 0, total_parameters = 0, total_weights = 0, total_bias = 0;
+  size_t total_normalized_units = 0;  // one slot per unit of EVERY layer, input included
+  size_t batch_size = 1, maximum_batch_size = 1, seq_w = 1;
+  size_t number_threads = 1;
+  Layer *ptr_array_layers = nullptr;
+  Layer *ptr_last_layer = nullptr;  // one past the output layer
+  var *ptr_array_parameters = nullptr;               // host mirror [P]: W.. | b.. | gamma.. | beta..
+  real *ptr_array_derivatives_parameters = nullptr;  // host mirror [P]
+  var *ptr_array_normalized_batch_units_means_averages = nullptr;      // host mirror [units]
+  var *ptr_array_normalized_batch_units_variances_averages = nullptr;  // host mirror [units] (std-devs)
+  real normalization_momentum_average = 0.999f;  // model.hpp:3045-3048
+  real normalization_epsilon = 1e-5f;
+  real batch_renormalization_r_correction_maximum = 1.0f;
+  real batch_renormalization_d_correction_maximum = 0.0f;
+  MODEL::TYPE type = MODEL::NONE;
+  LOSS_FN::TYPE type_loss_function = LOSS_FN::NONE;
+  ACCU_FN::TYPE type_accuracy_function = ACCU_FN::NONE;
+  PROPAGATION::TYPE type_state_propagation = PROPAGATION::INFERENCE;
+  // How the backward treats dropout (see dlmi_dropout_bwd).  The reference's CPU
+  // path is DLMI_DROP_BWD_REFERENCE.
+  dlmi_dropout_bwd dropout_backward_mode = DLMI_DROP_BWD_REFERENCE;
+  std::mt19937 real_gen;  // mask sampling (the reference seeds its generators from the clock)
+
+  Layer *Get__Input_Layer(void) const { return ptr_array_layers; }
+  Layer *Get__Output_Layer(void) const { return ptr_last_layer - 1; }
+
+ private:
+  struct Impl;
+  Impl *impl_;
+  bool allocate_batch(size_t batch);
+  void free_batch(void);
+  bool fail(char const *what) const;
+};
+
+}  // namespace v1
+}  // namespace dlmi
+
+#ifdef DLMI_ALIAS_DL_NAMESPACE
+namespace DL {
+namespace v1 {
+using namespace ::dlmi::v1;
+}
+}  // namespace DL
+#endif
+
+#endif  // DLMI_MODEL_HPP
