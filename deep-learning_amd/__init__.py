@@ -38,7 +38,7 @@ C_ABI_SYMBOLS = [
     "dlmi_ctx_compute_units", "dlmi_fc_fwd", "dlmi_fc_bwd_dx", "dlmi_fc_bwd_dw", "dlmi_bias_fwd",
     "dlmi_norm_fwd_train", "dlmi_norm_fwd_infer", "dlmi_norm_bwd", "dlmi_act_fwd", "dlmi_act_bwd",
     "dlmi_softmax_fwd", "dlmi_dropout_fwd", "dlmi_identity_add", "dlmi_softmax_ce_seed",
-    "dlmi_fused_norm_act_fwd", "dlmi_fused_norm_act_bwd", "dlmi_fused_norm_act_infer",
+    "dlmi_fused_norm_act_fwd", "dlmi_fused_norm_act_bwd", "dlmi_fused_norm_act_infer", "dlmi_fc_norm_act_fwd",
 ]
 
 
@@ -256,6 +256,20 @@ class Dlmi:
                                                   _p(beta), _p(mask), _p(s["mean"]), _p(s["std"]), _p(mov_mean),
                                                   _p(mov_std), _p(s["r"]), _p(s["d"]), _p(y)))
         return y, s
+
+    def fc_norm_act_fwd(self, desc, X, W, gamma, beta, mov_mean, mov_std, mask=None, Z=None, out=None, stats=None):
+        """Z = X W^T with the batch statistics taken in the GEMM epilogue, then
+        normalization + activation (+ dropout).  Returns (Z, y, stats)."""
+        self._chk(X, W, gamma, beta, mov_mean, mov_std, mask, Z, out)
+        B, K = X.shape
+        H = W.shape[0]
+        Z = Z if Z is not None else self.empty(B, H)
+        y = out if out is not None else self.empty(B, H)
+        s = stats or dict(mean=self.empty(H), std=self.empty(H), r=self.empty(H), d=self.empty(H))
+        self._ck(self.lib.dlmi_fc_norm_act_fwd(self.ctx, ctypes.byref(desc), c_sz(B), c_sz(K), c_sz(H), _p(X), _p(W),
+                                               _p(gamma), _p(beta), _p(mask), _p(Z), _p(s["mean"]), _p(s["std"]),
+                                               _p(mov_mean), _p(mov_std), _p(s["r"]), _p(s["d"]), _p(y)))
+        return Z, y, s
 
     def fused_bwd(self, desc, x, gamma, beta, stats, dY, dgamma, dbeta, mask=None, out=None):
         self._chk(x, gamma, beta, dY, dgamma, dbeta, mask, out)

@@ -56,5 +56,14 @@ inline int dlmi_fail(dlmi_ctx *ctx, int code, char const *fmt, ...) {
 // Makes sure the context's scratch holds at least `bytes`.
 int dlmi_scratch_reserve(dlmi_ctx *ctx, size_t bytes);
 
+namespace dlmi {
+// Batch-(re)norm forward tail (finalize + apply) from column-sum partials
+// [2][nchunks][H] that a producer (the GEMM epilogue) already wrote.
+int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
+                            float const *gamma, float const *beta, uint8_t const *mask, float *mean, float *stdv,
+                            float *mov_mean, float *mov_std, float *r, float *d, float *y, float const *partial,
+                            unsigned nchunks);
+}  // namespace dlmi
+
 inline bool dlmi_aligned16(void const *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline size_t dlmi_ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }

@@ -47,6 +47,7 @@ struct GemmArgs {
   size_t lda, ldb, ldc;
   size_t k_per_split;  // K range of one blockIdx.z slice (multiple of BK)
   float *split_out;    // when gridDim.z > 1: [splits][M][N] partial products
+  float *stats_out;    // optional [2][tiles_m][N]: per tile-row column sums of C and C^2 (gridDim.z == 1)
   int accumulate;      // C += result (only when gridDim.z == 1)
   unsigned tiles_m, tiles_n;
 };
@@ -246,6 +247,44 @@ void k_gemm_f32(GemmArgs g) {
         }
       }
     }
+
+  // ---- optional fused epilogue: column sums of this tile's outputs and of
+  // their squares, the batch-chunk partials the batch-(re)norm finalize kernel
+  // consumes (chunk = tile row).  Fixed order: rows of a lane, the two lane
+  // halves, the two wavefronts stacked along M.
+  if (g.stats_out != nullptr) {
+    __syncthreads();  // every wavefront is done reading the operand tiles: reuse that LDS
+    float *const sl = lds;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      size_t const col = n0 + wn0 + j * 32 + lr;
+      float const bv = (g.bias != nullptr && (FAST || col < g.N)) ? g.bias[col] : 0.0f;
+      float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          size_t const row = m0 + wm0 + i * 32 + (e / 4) * 8 + (lane >> 5) * 4 + (e % 4);
+          float const v = (FAST || row < g.M) ? acc[i][j][e] + bv : 0.0f;
+          s1 += v;
+          s2 += v * v;
+        }
+      s1 += __shfl_xor(s1, 32, 64);
+      s2 += __shfl_xor(s2, 32, 64);
+      if (lane < 32) {
+        sl[((wave >> 1) * BN + wn0 + j * 32 + lr) * 2 + 0] = s1;
+        sl[((wave >> 1) * BN + wn0 + j * 32 + lr) * 2 + 1] = s2;
+      }
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < BN; c += kGemmThreads) {
+      size_t const col = n0 + c;
+      if (FAST || col < g.N) {
+        g.stats_out[(0 * static_cast<size_t>(g.tiles_m) + tile_m) * g.N + col] = sl[(0 * BN + c) * 2 + 0] + sl[(1 * BN + c) * 2 + 0];
+        g.stats_out[(1 * static_cast<size_t>(g.tiles_m) + tile_m) * g.N + col] = sl[(0 * BN + c) * 2 + 1] + sl[(1 * BN + c) * 2 + 1];
+      }
+    }
+  }
 }
 
 // Fixed-order sum of the split-K partial products (+ bias, + previous C).
@@ -333,9 +372,11 @@ static int tile_choice() {
 }
 
 // C[M,N] (+)= A . B with the operand layouts given by the two flags.
+// stats_chunks != nullptr: also write the column-sum partials [2][*stats_chunks][N]
+// of C into the first half of the context's scratch (no split-K then).
 template <bool AK, bool BKC>
 static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, size_t lda, float const *B, size_t ldb,
-                float *C, float const *bias, int accumulate) {
+                float *C, float const *bias, int accumulate, unsigned *stats_chunks = nullptr) {
   static TileCfg const cfgs[] = {{128, 128, 16}, {128, 128, 32}, {256, 128, 16}, {256, 128, 32}, {256, 256, 16}};
   int choice = tile_choice();
   if (choice < 0 || choice >= static_cast<int>(sizeof(cfgs) / sizeof(cfgs[0]))) {
@@ -350,7 +391,13 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
 
   GemmArgs g;
   g.A = A; g.B = B; g.C = C; g.bias = bias; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldc = N;
-  g.accumulate = accumulate; g.split_out = nullptr;
+  g.accumulate = accumulate; g.split_out = nullptr; g.stats_out = nullptr;
+  if (stats_chunks != nullptr) {
+    *stats_chunks = static_cast<unsigned>(dlmi_ceil_div(M, bm));
+    int rc = dlmi_scratch_reserve(ctx, 2 * 2 * static_cast<size_t>(*stats_chunks) * N * sizeof(float));
+    if (rc != DLMI_OK) return rc;
+    g.stats_out = reinterpret_cast<float *>(ctx->scratch);
+  }
   bool const fast = M % bm == 0 && N % bn == 0 && K % bk == 0 && lda % 4 == 0 && ldb % 4 == 0 &&
                     dlmi_aligned16(A) && dlmi_aligned16(B);
   // Split K when the output alone cannot fill the machine (few tiles, long K):
@@ -359,7 +406,7 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   size_t const ktiles = dlmi_ceil_div(K, bk);
   unsigned splits = 1;
   size_t const target = static_cast<size_t>(ctx->num_cu) * 2;
-  if (tiles < target / 2 && ktiles >= 16) {
+  if (tiles < target / 2 && ktiles >= 16 && stats_chunks == nullptr) {
     size_t s = dlmi_ceil_div(target, tiles);
     size_t const max_s = ktiles / 8;  // at least 8 K tiles per slice
     if (s > max_s) s = max_s;
@@ -406,6 +453,19 @@ int dlmi_fc_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, flo
   DLMI_REQUIRE(ctx, X && W && Z, "null pointer");
   DLMI_REQUIRE(ctx, B > 0 && K > 0 && H > 0, "empty operand");
   return gemm<true, true>(ctx, B, H, K, X, K, W, K, Z, bias, 0);
+}
+
+int dlmi_fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t K, size_t H, float const *X,
+                         float const *W, float const *gamma, float const *beta, uint8_t const *mask, float *Z,
+                         float *mean, float *stdv, float *mov_mean, float *mov_std, float *r, float *d, float *y) {
+  if (ctx == nullptr || desc == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, X && W && Z, "null pointer");
+  DLMI_REQUIRE(ctx, B > 0 && K > 0 && H > 0, "empty operand");
+  unsigned chunks = 0;
+  int rc = gemm<true, true>(ctx, B, H, K, X, K, W, K, Z, nullptr, 0, &chunks);
+  if (rc != DLMI_OK) return rc;
+  return fused_fwd_from_partials(ctx, desc, B, H, Z, gamma, beta, mask, mean, stdv, mov_mean, mov_std, r, d, y,
+                                 reinterpret_cast<float const *>(ctx->scratch), chunks);
 }
 
 int dlmi_fc_bwd_dx(dlmi_ctx *ctx, size_t B, size_t Hn, size_t H, float const *dZn, float const *Wn, float *dY,

@@ -3,7 +3,8 @@
 //
 // All of them are bound by HBM bandwidth, so the design goal is the minimum
 // number of passes over the [B, H] tensors with fully coalesced 16-byte
-// accesses and enough independent loads in flight per CU:
+// accesses, enough independent loads in flight per CU and few enough ALU
+// instructions per element that the vector units never become the limit:
 //
 //   forward : stats (read x)            -> finalize [H] -> apply (read x, write y)
 //   backward: reduce (read dY, x)       -> finalize [H] -> apply (read dY, x, write dX)
@@ -13,13 +14,21 @@
 //
 // Thread geometry of the column passes: a 256-thread block is TX x TY; a
 // thread owns VEC (=4, one float4) adjacent units and walks the rows of its
-// block's batch chunk with stride TY.  TX <= 64, so when H is small a
-// wavefront spans several rows: those are combined with wavefront shuffles,
-// the four wavefronts of the block with a small LDS tree, and the chunks of the
-// batch by the finalize kernel in a fixed order (no float atomics: results are
-// reproducible run to run).
+// block's batch chunk with stride TY.  In the reduction kernels TX <= 64, so
+// when H is small a wavefront spans several rows: those are combined with
+// wavefront shuffles, the four wavefronts of the block with a small LDS tree,
+// and the chunks of the batch by the finalize kernel in a fixed order (no float
+// atomics: results are reproducible run to run).  The apply kernels have
+// nothing to reduce and use TX = 256 when H allows, so that every load / store
+// instruction of a block covers 4 KiB of one row.
+//
+// Everything that is uniform over a launch and would put a branch between two
+// loads (dropout mode, materialising x_hat) is a template parameter: a branch
+// there makes the compiler wait for each load before issuing the next.
 //
 // Citations: /root/reference/lib/deep-learning/v1/learner/.
+#include <initializer_list>
+
 #include "activations.hpp"
 #include "dlmi_common.hpp"
 
@@ -28,32 +37,38 @@ namespace dlmi {
 constexpr int kBlock = 256;
 constexpr int kWave = 64;
 
+// dropout as a template mode
+constexpr int kDropNone = 0, kDropUnit = 1, kDropElem = 2;
+
 struct ColGeom {
-  int vec;        // 4 (float4 path) or 1 (any H, any alignment)
-  int tx, tx_log2, ty;
+  int vec;  // 4 (float4 path) or 1 (any H, any alignment)
+  int tx_log2;
   unsigned grid_x;
   unsigned nchunks;
   size_t rows_per_chunk;
 };
 
-static ColGeom col_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, int nacc) {
+// Geometry of a reduction pass (TX <= 64).
+static ColGeom reduce_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, int nacc) {
   ColGeom g;
   g.vec = vec4 ? 4 : 1;
   size_t const groups = dlmi_ceil_div(H, g.vec);
-  g.tx = 64;
+  int tx = 64;
   g.tx_log2 = 6;
-  while (g.tx > 1 && static_cast<size_t>(g.tx / 2) >= groups) {
-    g.tx /= 2;
+  while (tx > 1 && static_cast<size_t>(tx / 2) >= groups) {
+    tx /= 2;
     --g.tx_log2;
   }
-  g.ty = kBlock / g.tx;
-  g.grid_x = static_cast<unsigned>(dlmi_ceil_div(groups, g.tx));
-  // enough blocks to cover every CU a few times over, but each thread should
-  // still stream >= 8 rows so the partials stay a small fraction of the traffic
+  int const ty = kBlock / tx;
+  g.grid_x = static_cast<unsigned>(dlmi_ceil_div(groups, tx));
+  // enough blocks to cover every CU several times over, but each thread still
+  // streams >= 16 rows: the partial sums stay a small fraction of the traffic
+  // and the fixed cost of a block is amortised (measured optimum on 4096-wide
+  // tensors: 64 rows per chunk)
   size_t want = dlmi_ceil_div(static_cast<size_t>(ctx->num_cu) * 8, g.grid_x);
-  size_t const max_by_rows = B / (static_cast<size_t>(g.ty) * 8);
+  size_t const max_by_rows = B / (static_cast<size_t>(ty) * 16);
   if (want > max_by_rows) want = max_by_rows;
-  // partial sums must fit the scratch block: nacc * nchunks * H floats (half of it)
+  // partial sums must fit half of the scratch block: nacc * nchunks * H floats
   size_t const max_by_scratch = (ctx->scratch_bytes / 2) / (static_cast<size_t>(nacc) * H * sizeof(float));
   if (want > max_by_scratch) want = max_by_scratch;
   if (want < 1) want = 1;
@@ -63,18 +78,30 @@ static ColGeom col_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, 
   return g;
 }
 
-template <int VEC>
-struct Vec;
-template <>
-struct Vec<4> {
-  using f = float4;
-  using u = uchar4;
-};
-template <>
-struct Vec<1> {
-  using f = float;
-  using u = unsigned char;
-};
+// Geometry of an apply pass: as wide as the row allows (TX up to 256), 8 rows
+// per thread.
+static ColGeom apply_geometry(size_t B, size_t H, bool vec4) {
+  ColGeom g;
+  g.vec = vec4 ? 4 : 1;
+  size_t const groups = dlmi_ceil_div(H, g.vec);
+  int tx = 256;
+  g.tx_log2 = 8;
+  while (tx > 1 && static_cast<size_t>(tx / 2) >= groups) {
+    tx /= 2;
+    --g.tx_log2;
+  }
+  int const ty = kBlock / tx;
+  g.grid_x = static_cast<unsigned>(dlmi_ceil_div(groups, tx));
+  g.rows_per_chunk = static_cast<size_t>(ty) * 8;
+  size_t chunks = dlmi_ceil_div(B, g.rows_per_chunk);
+  if (chunks > 65535) {
+    chunks = 65535;
+    g.rows_per_chunk = dlmi_ceil_div(B, chunks);
+    chunks = dlmi_ceil_div(B, g.rows_per_chunk);
+  }
+  g.nchunks = static_cast<unsigned>(chunks);
+  return g;
+}
 
 template <int VEC>
 __device__ __forceinline__ void load_f(float const *p, float (&v)[VEC]) {
@@ -103,8 +130,9 @@ __device__ __forceinline__ void load_u8(uint8_t const *p, uint8_t (&v)[VEC]) {
   }
 }
 
-// Sum NV per-thread values over the TY rows of the block.  On return the
-// threads with threadIdx.x < TX hold the block totals for their column group.
+// Sum NV per-thread values over the TY rows of the block (TX <= 64).  On
+// return the threads with threadIdx.x < TX hold the block totals for their
+// column group.
 template <int NV>
 __device__ __forceinline__ void block_rows_reduce(float (&v)[NV], int tx, float *lds) {
   int const lane = threadIdx.x & (kWave - 1);
@@ -114,14 +142,13 @@ __device__ __forceinline__ void block_rows_reduce(float (&v)[NV], int tx, float 
 #pragma unroll
     for (int i = 0; i < NV; ++i) v[i] += __shfl_xor(v[i], off, kWave);
   }
-  int const cols_in_wave = tx < kWave ? tx : kWave;
-  if (lane < cols_in_wave) {
+  if (lane < tx) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) lds[(wave * kWave + lane) * NV + i] = v[i];
   }
   __syncthreads();
   // LDS tree over the four wavefronts: (0+1) + (2+3), fixed order
-  if (threadIdx.x < cols_in_wave) {
+  if (threadIdx.x < tx) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       float const a = lds[(0 * kWave + lane) * NV + i] + lds[(1 * kWave + lane) * NV + i];
@@ -149,13 +176,14 @@ __global__ __launch_bounds__(kBlock) void k_col_stats(float const *__restrict__ 
 #pragma unroll
   for (int i = 0; i < 2 * VEC; ++i) acc[i] = 0.0f;
   if (live) {
+    constexpr int U = 8;
     size_t b = b0 + ty;
-    for (; b + 3 * static_cast<size_t>(TY) < b1; b += 4 * static_cast<size_t>(TY)) {
-      float v[4][VEC];
+    for (; b + (U - 1) * static_cast<size_t>(TY) < b1; b += U * static_cast<size_t>(TY)) {
+      float v[U][VEC];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) load_f<VEC>(x + (b + u * static_cast<size_t>(TY)) * H + col, v[u]);
+      for (int u = 0; u < U; ++u) load_f<VEC>(x + (b + u * static_cast<size_t>(TY)) * H + col, v[u]);
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
           acc[i] += v[u][i];
@@ -183,39 +211,44 @@ __global__ __launch_bounds__(kBlock) void k_col_stats(float const *__restrict__ 
   }
 }
 
-// Sums NA partial-sum planes over the batch chunks for 64 adjacent units per
-// block: wavefront w adds chunks w, w+4, w+8, ... (coalesced 256-byte rows, four
-// independent accumulation chains per unit), then the four wavefront totals
-// are combined through LDS in a fixed order.  On return the threads of
-// wavefront 0 hold the totals of unit blockIdx.x*64 + lane.
-constexpr int kFinCols = 64;
+// Sums NA partial-sum planes over the batch chunks for 16 adjacent units per
+// block: thread (lane c of 16, unit j of 16) adds chunks c, c+16, c+32, ... with
+// independent loads, then the 16 lane totals of a unit are combined through
+// LDS in a fixed order.  On return thread t < 16 holds the totals of unit
+// blockIdx.x*16 + t.
+constexpr int kFinCols = 16;
+constexpr int kFinLanes = kBlock / kFinCols;
 template <int NA>
 __device__ __forceinline__ void chunk_totals(float const *__restrict__ partial, unsigned nchunks, size_t H,
                                              float (&tot)[NA], float *lds) {
-  int const lane = threadIdx.x & (kWave - 1);
-  int const wave = threadIdx.x / kWave;
-  size_t const j = static_cast<size_t>(blockIdx.x) * kFinCols + lane;
+  int const cj = threadIdx.x % kFinCols;
+  int const cl = threadIdx.x / kFinCols;
+  size_t const j = static_cast<size_t>(blockIdx.x) * kFinCols + cj;
 #pragma unroll
   for (int a = 0; a < NA; ++a) tot[a] = 0.0f;
   if (j < H) {
-    for (unsigned c = wave; c < nchunks; c += kBlock / kWave) {
+#pragma unroll 4
+    for (unsigned c = cl; c < nchunks; c += kFinLanes) {
 #pragma unroll
       for (int a = 0; a < NA; ++a) tot[a] += partial[(a * static_cast<size_t>(nchunks) + c) * H + j];
     }
   }
 #pragma unroll
-  for (int a = 0; a < NA; ++a) lds[(wave * kWave + lane) * NA + a] = tot[a];
+  for (int a = 0; a < NA; ++a) lds[(cl * kFinCols + cj) * NA + a] = tot[a];
   __syncthreads();
-  if (wave == 0) {
+  if (threadIdx.x < kFinCols) {
 #pragma unroll
-    for (int a = 0; a < NA; ++a)
-      tot[a] = (lds[(0 * kWave + lane) * NA + a] + lds[(1 * kWave + lane) * NA + a]) +
-               (lds[(2 * kWave + lane) * NA + a] + lds[(3 * kWave + lane) * NA + a]);
+    for (int a = 0; a < NA; ++a) {
+      float s = 0.0f;
+#pragma unroll
+      for (int l = 0; l < kFinLanes; ++l) s += lds[(l * kFinCols + threadIdx.x) * NA + a];
+      tot[a] = s;
+    }
   }
 }
 
 // Phase 2 of fwp_st.cpp:4709-4746: batch mean, moving mean, batch std, moving
-// std, then r and d from the UPDATED moving statistics.  64 units per block.
+// std, then r and d from the UPDATED moving statistics.
 __global__ __launch_bounds__(kBlock) void k_fwd_finalize(float const *__restrict__ partial, unsigned nchunks,
                                                           size_t B, size_t H, int renorm, float momentum,
                                                           float eps, float r_max, float d_max,
@@ -227,7 +260,7 @@ __global__ __launch_bounds__(kBlock) void k_fwd_finalize(float const *__restrict
   float tot[2];
   chunk_totals<2>(partial, nchunks, H, tot, lds);
   size_t const j = static_cast<size_t>(blockIdx.x) * kFinCols + threadIdx.x;
-  if (threadIdx.x >= kWave || j >= H) return;
+  if (threadIdx.x >= kFinCols || j >= H) return;
   float const s1 = tot[0], s2 = tot[1];
   float const batch_scale = 1.0f / static_cast<float>(B);
   float const mu = s1 * batch_scale;
@@ -252,28 +285,28 @@ __global__ __launch_bounds__(kBlock) void k_fwd_finalize(float const *__restrict
   }
 }
 
-// Dropout as the forward applies it (fwp_st.cpp:4830-4883): kind 0 none,
-// 1 plain Bernoulli (mask ? v : 0), 2 inverted (mask ? v*scale : 0).
-__device__ __forceinline__ float drop_apply(int kind, uint8_t m, float scale, float v) {
-  if (kind == 0) return v;
-  if (kind == 1) return m ? v : 0.0f;
-  return m ? v * scale : 0.0f;
-}
+// Dropout as the forward applies it (fwp_st.cpp:4830-4883): mask ? v*scale : 0
+// with scale = 1 for plain Bernoulli, 1/keep for inverted Bernoulli.
+__device__ __forceinline__ float drop_apply(uint8_t m, float scale, float v) { return m ? v * scale : 0.0f; }
 
 struct FwdApplyArgs {
   float const *x, *gamma, *beta, *mean, *stdv, *r, *d;
   uint8_t const *mask;
-  float *y;     // activation output after dropout (may be null)
-  float *xhat;  // optional materialised x_hat
-  float *nrm;   // optional materialised gamma*x_hat + beta
+  float *y;     // activation output after dropout
+  float *xhat;  // optional materialised x_hat            (MAT only)
+  float *nrm;   // optional materialised gamma*x_hat+beta (MAT only)
   size_t B, H, rows_per_chunk;
-  int tx_log2, drop_kind, mask_per_element;
+  int tx_log2;
   float drop_scale;
 };
 
 // Phase 3 of fwp_st.cpp:4748-4765, then AF_FIRE (fwp_st.cpp:4768-4794), then the
 // dropout leaf, in one pass.
-template <int VEC, int ACT>
+// MAT: materialise x_hat / the pre-activation (the un-fused leaf) with the
+// reference's expression order.  Otherwise the per-unit constants are folded so
+// that an element costs one subtraction and one fused multiply-add before the
+// activation:  n = (x - mean) * (gamma*r/std) + (gamma*d + beta).
+template <int VEC, int ACT, int DROPM, bool MAT>
 __global__ __launch_bounds__(kBlock) void k_fwd_apply(FwdApplyArgs a) {
   int const TX = 1 << a.tx_log2, TY = kBlock >> a.tx_log2;
   int const tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> a.tx_log2;
@@ -291,52 +324,66 @@ __global__ __launch_bounds__(kBlock) void k_fwd_apply(FwdApplyArgs a) {
   load_f<VEC>(a.beta + col, be);
 #pragma unroll
   for (int i = 0; i < VEC; ++i) {
-    inv[i] = 1.0f / inv[i];
+    inv[i] = fast_rcp(inv[i]);
     mk[i] = 1;
+    if constexpr (!MAT) {
+      rr[i] = ga[i] * (rr[i] * inv[i]);  // gamma * r / std
+      dd[i] = ga[i] * dd[i] + be[i];     // gamma * d + beta
+    }
   }
-  if (a.drop_kind != 0 && !a.mask_per_element) load_u8<VEC>(a.mask + col, mk);
+  if constexpr (DROPM == kDropUnit) load_u8<VEC>(a.mask + col, mk);
   constexpr int U = 4;
-  size_t b = b0 + ty;
-  auto body = [&](size_t row, float const (&xv)[VEC], uint8_t const (&mv)[VEC]) {
+  auto body = [&](size_t off, float const (&xv)[VEC], uint8_t const (&mv)[VEC]) {
     float xh[VEC], nn[VEC], q[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
-      xh[i] = (xv[i] - mu[i]) * inv[i] * rr[i] + dd[i];
-      nn[i] = ga[i] * xh[i] + be[i];
-      q[i] = drop_apply(a.drop_kind, mv[i], a.drop_scale, act_fire<ACT>(nn[i]));
+      if constexpr (MAT) {
+        xh[i] = (xv[i] - mu[i]) * inv[i] * rr[i] + dd[i];
+        nn[i] = ga[i] * xh[i] + be[i];
+      } else {
+        nn[i] = (xv[i] - mu[i]) * rr[i] + dd[i];
+      }
+      q[i] = act_fire<ACT>(nn[i]);
+      if constexpr (DROPM != kDropNone) q[i] = drop_apply(mv[i], a.drop_scale, q[i]);
     }
-    if (a.xhat != nullptr) store_f<VEC>(a.xhat + row * a.H + col, xh);
-    if (a.nrm != nullptr) store_f<VEC>(a.nrm + row * a.H + col, nn);
-    if (a.y != nullptr) store_f<VEC>(a.y + row * a.H + col, q);
+    if constexpr (MAT) {
+      if (a.xhat != nullptr) store_f<VEC>(a.xhat + off, xh);
+      if (a.nrm != nullptr) store_f<VEC>(a.nrm + off, nn);
+      if (a.y != nullptr) store_f<VEC>(a.y + off, q);
+    } else {
+      store_f<VEC>(a.y + off, q);
+    }
   };
+  size_t b = b0 + ty;
   for (; b + (U - 1) * static_cast<size_t>(TY) < b1; b += U * static_cast<size_t>(TY)) {
     float xv[U][VEC];
     uint8_t mv[U][VEC];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      size_t const row = b + u * static_cast<size_t>(TY);
-      load_f<VEC>(a.x + row * a.H + col, xv[u]);
-      if (a.drop_kind != 0 && a.mask_per_element) {
-        load_u8<VEC>(a.mask + row * a.H + col, mv[u]);
+      size_t const off = (b + u * static_cast<size_t>(TY)) * a.H + col;
+      load_f<VEC>(a.x + off, xv[u]);
+      if constexpr (DROPM == kDropElem) {
+        load_u8<VEC>(a.mask + off, mv[u]);
       } else {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) mv[u][i] = mk[i];
       }
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u) body(b + u * static_cast<size_t>(TY), xv[u], mv[u]);
+    for (int u = 0; u < U; ++u) body((b + u * static_cast<size_t>(TY)) * a.H + col, xv[u], mv[u]);
   }
   for (; b < b1; b += TY) {
     float xv[VEC];
     uint8_t mv[VEC];
-    load_f<VEC>(a.x + b * a.H + col, xv);
-    if (a.drop_kind != 0 && a.mask_per_element) {
-      load_u8<VEC>(a.mask + b * a.H + col, mv);
+    size_t const off = b * a.H + col;
+    load_f<VEC>(a.x + off, xv);
+    if constexpr (DROPM == kDropElem) {
+      load_u8<VEC>(a.mask + off, mv);
     } else {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) mv[i] = mk[i];
     }
-    body(b, xv, mv);
+    body(off, xv, mv);
   }
 }
 
@@ -350,31 +397,57 @@ struct BwdArgs {
   float const *coef;  // apply: [3][H]  c1 = gamma*r/std, c2 = dstd/(B*std), c3 = dmean/B
   float *dX;
   size_t B, H, rows_per_chunk;
-  int tx_log2, drop_kind, mask_per_element, drop_bwd_masked;
+  int tx_log2, drop_bwd_masked;
   float drop_scale;
 };
+
+// Per-unit constants of the backward recompute, loaded once per thread.
+template <int VEC>
+struct UnitConsts {
+  float mu[VEC], rs[VEC], dd[VEC], ga[VEC], be[VEC];  // rs = r / std
+  uint8_t mk[VEC];
+};
+
+template <int VEC, int DROPM, bool XHAT_GIVEN>
+__device__ __forceinline__ void load_unit_consts(BwdArgs const &a, size_t col, UnitConsts<VEC> &u) {
+  load_f<VEC>(a.mean + col, u.mu);
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    u.rs[i] = 1.0f; u.dd[i] = 0.0f; u.ga[i] = 1.0f; u.be[i] = 0.0f; u.mk[i] = 1;
+  }
+  if constexpr (!XHAT_GIVEN) {
+    float sd[VEC], rr[VEC];
+    load_f<VEC>(a.stdv + col, sd);
+    load_f<VEC>(a.r + col, rr);
+    load_f<VEC>(a.d + col, u.dd);
+    load_f<VEC>(a.gamma + col, u.ga);
+    load_f<VEC>(a.beta + col, u.be);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) u.rs[i] = rr[i] * fast_rcp(sd[i]);
+    if constexpr (DROPM == kDropUnit) load_u8<VEC>(a.mask + col, u.mk);
+  }
+}
 
 // dn = dY * f'(n, q) for one element, recomputing x_hat, n and q from x.
 // REFERENCE dropout mode: q is the post-dropout output and dY is untouched
 // (bwp_st.cpp:1177-1209 reads the array the dropout leaf overwrote in place);
 // MASKED mode: q is the pre-dropout activation and dY is masked and rescaled.
-template <int ACT, bool XHAT_GIVEN>
-__device__ __forceinline__ float bwd_dn(BwdArgs const &a, float xv, float dy, uint8_t m, float mu, float inv,
-                                        float rr, float dd, float ga, float be, float &xh) {
+template <int ACT, int DROPM, bool XHAT_GIVEN>
+__device__ __forceinline__ float bwd_dn(BwdArgs const &a, float xv, float dy, uint8_t m, float mu, float rs,
+                                        float dd, float ga, float be, float &xh) {
   if constexpr (XHAT_GIVEN) {
-    (void)xv; (void)m; (void)mu; (void)inv; (void)rr; (void)dd; (void)ga; (void)be;
+    (void)a; (void)xv; (void)m; (void)mu; (void)rs; (void)dd; (void)ga; (void)be;
     return dy;
   } else {
-    xh = (xv - mu) * inv * rr + dd;
+    xh = (xv - mu) * rs + dd;
     float const nn = ga * xh + be;
     float q = act_fire<ACT>(nn);
     float g = dy;
-    if (a.drop_kind != 0) {
-      if (a.drop_bwd_masked) {
-        g = drop_apply(a.drop_kind, m, a.drop_scale, dy);
-      } else {
-        q = drop_apply(a.drop_kind, m, a.drop_scale, q);
-      }
+    if constexpr (DROPM != kDropNone) {
+      float const gm = drop_apply(m, a.drop_scale, dy);
+      float const qm = drop_apply(m, a.drop_scale, q);
+      g = a.drop_bwd_masked ? gm : dy;
+      q = a.drop_bwd_masked ? q : qm;
     }
     return g * act_derive<ACT>(nn, q);
   }
@@ -383,7 +456,7 @@ __device__ __forceinline__ float bwd_dn(BwdArgs const &a, float xv, float dy, ui
 // Pass 1 of bwp_st.cpp:1478-1506: column sums of dn*x_hat, dn and dn*(x-mean).
 // (dmean and dstd follow from the last two in the finalize kernel:
 //  sum e*(-r/std) = -(r/std)*gamma*sum dn, sum e*(x-mean)*(-r/std^2) likewise.)
-template <int VEC, int ACT, bool XHAT_GIVEN>
+template <int VEC, int ACT, int DROPM, bool XHAT_GIVEN>
 __global__ __launch_bounds__(kBlock) void k_bwd_reduce(BwdArgs a) {
   __shared__ float lds[4 * kWave * 3 * VEC];
   int const TX = 1 << a.tx_log2, TY = kBlock >> a.tx_log2;
@@ -396,34 +469,19 @@ __global__ __launch_bounds__(kBlock) void k_bwd_reduce(BwdArgs a) {
 #pragma unroll
   for (int i = 0; i < 3 * VEC; ++i) acc[i] = 0.0f;
   if (live) {
-    float mu[VEC], inv[VEC], rr[VEC], dd[VEC], ga[VEC], be[VEC];
-    uint8_t mk[VEC];
-    load_f<VEC>(a.mean + col, mu);
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      inv[i] = 1.0f; rr[i] = 1.0f; dd[i] = 0.0f; ga[i] = 1.0f; be[i] = 0.0f; mk[i] = 1;
-    }
-    if constexpr (!XHAT_GIVEN) {
-      load_f<VEC>(a.stdv + col, inv);
-      load_f<VEC>(a.r + col, rr);
-      load_f<VEC>(a.d + col, dd);
-      load_f<VEC>(a.gamma + col, ga);
-      load_f<VEC>(a.beta + col, be);
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) inv[i] = 1.0f / inv[i];
-      if (a.drop_kind != 0 && !a.mask_per_element) load_u8<VEC>(a.mask + col, mk);
-    }
-    constexpr int U = 2;
+    UnitConsts<VEC> uc;
+    load_unit_consts<VEC, DROPM, XHAT_GIVEN>(a, col, uc);
+    constexpr int U = 4;
     auto body = [&](float const (&xv)[VEC], float const (&dy)[VEC], float const (&xg)[VEC],
                     uint8_t const (&mv)[VEC]) {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
         float xh = xg[i];
-        float const dn = bwd_dn<ACT, XHAT_GIVEN>(a, xv[i], dy[i], mv[i], mu[i], inv[i], rr[i], dd[i], ga[i],
-                                                 be[i], xh);
+        float const dn = bwd_dn<ACT, DROPM, XHAT_GIVEN>(a, xv[i], dy[i], mv[i], uc.mu[i], uc.rs[i], uc.dd[i],
+                                                        uc.ga[i], uc.be[i], xh);
         acc[i] += dn * xh;
         acc[VEC + i] += dn;
-        acc[2 * VEC + i] += dn * (xv[i] - mu[i]);
+        acc[2 * VEC + i] += dn * (xv[i] - uc.mu[i]);
       }
     };
     size_t b = b0 + ty;
@@ -441,11 +499,11 @@ __global__ __launch_bounds__(kBlock) void k_bwd_reduce(BwdArgs a) {
 #pragma unroll
           for (int i = 0; i < VEC; ++i) xg[u][i] = 0.0f;
         }
-        if (!XHAT_GIVEN && a.drop_kind != 0 && a.mask_per_element) {
+        if constexpr (DROPM == kDropElem) {
           load_u8<VEC>(a.mask + off, mv[u]);
         } else {
 #pragma unroll
-          for (int i = 0; i < VEC; ++i) mv[u][i] = mk[i];
+          for (int i = 0; i < VEC; ++i) mv[u][i] = uc.mk[i];
         }
       }
 #pragma unroll
@@ -463,11 +521,11 @@ __global__ __launch_bounds__(kBlock) void k_bwd_reduce(BwdArgs a) {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) xg[i] = 0.0f;
       }
-      if (!XHAT_GIVEN && a.drop_kind != 0 && a.mask_per_element) {
+      if constexpr (DROPM == kDropElem) {
         load_u8<VEC>(a.mask + off, mv);
       } else {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) mv[i] = mk[i];
+        for (int i = 0; i < VEC; ++i) mv[i] = uc.mk[i];
       }
       body(xv, dy, xg, mv);
     }
@@ -498,7 +556,7 @@ __global__ __launch_bounds__(kBlock) void k_bwd_finalize(float const *__restrict
   float tot[3];
   chunk_totals<3>(partial, nchunks, H, tot, lds);
   size_t const j = static_cast<size_t>(blockIdx.x) * kFinCols + threadIdx.x;
-  if (threadIdx.x >= kWave || j >= H) return;
+  if (threadIdx.x >= kFinCols || j >= H) return;
   float const s0 = tot[0], s1 = tot[1], s2 = tot[2];
   float const sd = stdv[j];
   float const rr = r != nullptr ? r[j] : 1.0f;
@@ -515,7 +573,7 @@ __global__ __launch_bounds__(kBlock) void k_bwd_finalize(float const *__restrict
   coef[2 * H + j] = dm * batch_scale;
 }
 
-template <int VEC, int ACT, bool XHAT_GIVEN>
+template <int VEC, int ACT, int DROPM, bool XHAT_GIVEN>
 __global__ __launch_bounds__(kBlock) void k_bwd_apply(BwdArgs a) {
   int const TX = 1 << a.tx_log2, TY = kBlock >> a.tx_log2;
   int const tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> a.tx_log2;
@@ -523,35 +581,21 @@ __global__ __launch_bounds__(kBlock) void k_bwd_apply(BwdArgs a) {
   if (col >= a.H) return;
   size_t const b0 = blockIdx.y * a.rows_per_chunk;
   size_t const b1 = (b0 + a.rows_per_chunk < a.B) ? b0 + a.rows_per_chunk : a.B;
-  float mu[VEC], inv[VEC], rr[VEC], dd[VEC], ga[VEC], be[VEC], c1[VEC], c2[VEC], c3[VEC];
-  uint8_t mk[VEC];
-  load_f<VEC>(a.mean + col, mu);
+  UnitConsts<VEC> uc;
+  load_unit_consts<VEC, DROPM, XHAT_GIVEN>(a, col, uc);
+  float c1[VEC], c2[VEC], c3[VEC];
   load_f<VEC>(a.coef + 0 * a.H + col, c1);
   load_f<VEC>(a.coef + 1 * a.H + col, c2);
   load_f<VEC>(a.coef + 2 * a.H + col, c3);
-#pragma unroll
-  for (int i = 0; i < VEC; ++i) {
-    inv[i] = 1.0f; rr[i] = 1.0f; dd[i] = 0.0f; ga[i] = 1.0f; be[i] = 0.0f; mk[i] = 1;
-  }
-  if constexpr (!XHAT_GIVEN) {
-    load_f<VEC>(a.stdv + col, inv);
-    load_f<VEC>(a.r + col, rr);
-    load_f<VEC>(a.d + col, dd);
-    load_f<VEC>(a.gamma + col, ga);
-    load_f<VEC>(a.beta + col, be);
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) inv[i] = 1.0f / inv[i];
-    if (a.drop_kind != 0 && !a.mask_per_element) load_u8<VEC>(a.mask + col, mk);
-  }
-  constexpr int U = 2;
+  constexpr int U = 4;
   auto body = [&](size_t off, float const (&xv)[VEC], float const (&dy)[VEC], uint8_t const (&mv)[VEC]) {
     float dx[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
       float xh = 0.0f;
-      float const dn = bwd_dn<ACT, XHAT_GIVEN>(a, xv[i], dy[i], mv[i], mu[i], inv[i], rr[i], dd[i], ga[i],
-                                               be[i], xh);
-      dx[i] = dn * c1[i] + (xv[i] - mu[i]) * c2[i] + c3[i];
+      float const dn = bwd_dn<ACT, DROPM, XHAT_GIVEN>(a, xv[i], dy[i], mv[i], uc.mu[i], uc.rs[i], uc.dd[i], uc.ga[i],
+                                                      uc.be[i], xh);
+      dx[i] = dn * c1[i] + (xv[i] - uc.mu[i]) * c2[i] + c3[i];
     }
     store_f<VEC>(a.dX + off, dx);
   };
@@ -564,11 +608,11 @@ __global__ __launch_bounds__(kBlock) void k_bwd_apply(BwdArgs a) {
       size_t const off = (b + u * static_cast<size_t>(TY)) * a.H + col;
       load_f<VEC>(a.x + off, xv[u]);
       load_f<VEC>(a.dY + off, dy[u]);
-      if (!XHAT_GIVEN && a.drop_kind != 0 && a.mask_per_element) {
+      if constexpr (DROPM == kDropElem) {
         load_u8<VEC>(a.mask + off, mv[u]);
       } else {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) mv[u][i] = mk[i];
+        for (int i = 0; i < VEC; ++i) mv[u][i] = uc.mk[i];
       }
     }
 #pragma unroll
@@ -580,21 +624,17 @@ __global__ __launch_bounds__(kBlock) void k_bwd_apply(BwdArgs a) {
     size_t const off = b * a.H + col;
     load_f<VEC>(a.x + off, xv);
     load_f<VEC>(a.dY + off, dy);
-    if (!XHAT_GIVEN && a.drop_kind != 0 && a.mask_per_element) {
+    if constexpr (DROPM == kDropElem) {
       load_u8<VEC>(a.mask + off, mv);
     } else {
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) mv[i] = mk[i];
+      for (int i = 0; i < VEC; ++i) mv[i] = uc.mk[i];
     }
     body(off, xv, dy, mv);
   }
 }
 
 // ---------------------------------------------------------------- host drivers
-static int drop_kind_of(dlmi_dropout d) {
-  return d == DLMI_DROP_BERNOULLI ? 1 : (d == DLMI_DROP_BERNOULLI_INVERTED ? 2 : 0);
-}
-
 static bool use_vec4(size_t H, std::initializer_list<void const *> ptrs) {
   if (H % 4 != 0) return false;
   for (void const *p : ptrs)
@@ -602,42 +642,69 @@ static bool use_vec4(size_t H, std::initializer_list<void const *> ptrs) {
   return true;
 }
 
+// Runs f.template operator()<DROPM>() for the runtime dropout mode.
+#define DLMI_DISPATCH_DROP(mode, ...)                                         \
+  switch (mode) {                                                             \
+    case kDropUnit: { constexpr int DROPM = kDropUnit; __VA_ARGS__; } break;  \
+    case kDropElem: { constexpr int DROPM = kDropElem; __VA_ARGS__; } break;  \
+    default: { constexpr int DROPM = kDropNone; __VA_ARGS__; } break;         \
+  }
+
 struct FwdTrainCall {
   dlmi_norm norm;
   int act;
-  int drop_kind, mask_per_element;
+  int drop_mode;  // kDropNone / kDropUnit / kDropElem
   float momentum, eps, r_max, d_max, drop_scale;
   float const *x, *gamma, *beta;
   uint8_t const *mask;
   float *mean, *stdv, *mov_mean, *mov_std, *r, *d, *y, *xhat, *nrm;
+  float const *partial_in = nullptr;  // column-sum partials already produced elsewhere ...
+  unsigned partial_chunks = 0;        // ... [2][partial_chunks][H]; skips the statistics pass
 };
 
 static int run_fwd_train(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c) {
+  int rc = dlmi_scratch_reserve(ctx, 2 * 16 * 2 * H * sizeof(float));
+  if (rc != DLMI_OK) return rc;
   bool const vec4 = use_vec4(H, {c.x, c.gamma, c.beta, c.mean, c.stdv, c.r, c.d, c.y, c.xhat, c.nrm}) &&
-                    (c.drop_kind == 0 || (reinterpret_cast<uintptr_t>(c.mask) & 3u) == 0);
-  ColGeom const g = col_geometry(ctx, B, H, vec4, 2);
-  float *partial = reinterpret_cast<float *>(ctx->scratch);
-  dim3 const grid(g.grid_x, g.nchunks), block(kBlock);
-  if (vec4)
-    hipLaunchKernelGGL(k_col_stats<4>, grid, block, 0, ctx->stream, c.x, B, H, g.tx_log2, g.rows_per_chunk, partial);
-  else
-    hipLaunchKernelGGL(k_col_stats<1>, grid, block, 0, ctx->stream, c.x, B, H, g.tx_log2, g.rows_per_chunk, partial);
-  DLMI_LAUNCH_CHECK(ctx, "k_col_stats");
+                    (c.drop_mode == kDropNone || (reinterpret_cast<uintptr_t>(c.mask) & 3u) == 0);
+  dim3 const block(kBlock);
+  float const *partial = c.partial_in;
+  unsigned nchunks = c.partial_chunks;
+  if (partial == nullptr) {
+    ColGeom const g = reduce_geometry(ctx, B, H, vec4, 2);
+    float *pw = reinterpret_cast<float *>(ctx->scratch);
+    dim3 const grid(g.grid_x, g.nchunks);
+    if (vec4)
+      hipLaunchKernelGGL(k_col_stats<4>, grid, block, 0, ctx->stream, c.x, B, H, g.tx_log2, g.rows_per_chunk, pw);
+    else
+      hipLaunchKernelGGL(k_col_stats<1>, grid, block, 0, ctx->stream, c.x, B, H, g.tx_log2, g.rows_per_chunk, pw);
+    DLMI_LAUNCH_CHECK(ctx, "k_col_stats");
+    partial = pw;
+    nchunks = g.nchunks;
+  }
   hipLaunchKernelGGL(k_fwd_finalize, dim3(static_cast<unsigned>(dlmi_ceil_div(H, kFinCols))), block, 0, ctx->stream,
-                     partial, g.nchunks, B, H, c.norm == DLMI_NORM_BATCH_RENORM ? 1 : 0, c.momentum, c.eps,
+                     partial, nchunks, B, H, c.norm == DLMI_NORM_BATCH_RENORM ? 1 : 0, c.momentum, c.eps,
                      c.r_max, c.d_max, c.mean, c.stdv, c.mov_mean, c.mov_std, c.r, c.d);
   DLMI_LAUNCH_CHECK(ctx, "k_fwd_finalize");
+  ColGeom const ga = apply_geometry(B, H, vec4);
   FwdApplyArgs a;
   a.x = c.x; a.gamma = c.gamma; a.beta = c.beta; a.mean = c.mean; a.stdv = c.stdv; a.r = c.r; a.d = c.d;
   a.mask = c.mask; a.y = c.y; a.xhat = c.xhat; a.nrm = c.nrm;
-  a.B = B; a.H = H; a.rows_per_chunk = g.rows_per_chunk; a.tx_log2 = g.tx_log2;
-  a.drop_kind = c.drop_kind; a.mask_per_element = c.mask_per_element; a.drop_scale = c.drop_scale;
-  DLMI_DISPATCH_ACT(c.act, {
+  a.B = B; a.H = H; a.rows_per_chunk = ga.rows_per_chunk; a.tx_log2 = ga.tx_log2; a.drop_scale = c.drop_scale;
+  dim3 const agrid(ga.grid_x, ga.nchunks);
+  if (c.xhat != nullptr || c.nrm != nullptr) {  // un-fused leaf: LINEAR, no dropout by construction
     if (vec4)
-      hipLaunchKernelGGL((k_fwd_apply<4, ACT>), grid, block, 0, ctx->stream, a);
+      hipLaunchKernelGGL((k_fwd_apply<4, DLMI_ACT_LINEAR, kDropNone, true>), agrid, block, 0, ctx->stream, a);
     else
-      hipLaunchKernelGGL((k_fwd_apply<1, ACT>), grid, block, 0, ctx->stream, a);
-  });
+      hipLaunchKernelGGL((k_fwd_apply<1, DLMI_ACT_LINEAR, kDropNone, true>), agrid, block, 0, ctx->stream, a);
+  } else if (c.y != nullptr) {
+    DLMI_DISPATCH_ACT(c.act, DLMI_DISPATCH_DROP(c.drop_mode, {
+      if (vec4)
+        hipLaunchKernelGGL((k_fwd_apply<4, ACT, DROPM, false>), agrid, block, 0, ctx->stream, a);
+      else
+        hipLaunchKernelGGL((k_fwd_apply<1, ACT, DROPM, false>), agrid, block, 0, ctx->stream, a);
+    }));
+  }
   DLMI_LAUNCH_CHECK(ctx, "k_fwd_apply");
   return DLMI_OK;
 }
@@ -645,7 +712,7 @@ static int run_fwd_train(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &
 struct BwdCall {
   int act;
   bool xhat_given;
-  int drop_kind, mask_per_element, drop_bwd_masked;
+  int drop_mode, drop_bwd_masked;
   float drop_scale;
   float const *x, *gamma, *beta, *mean, *stdv, *r, *d, *xhat, *dY;
   uint8_t const *mask;
@@ -653,9 +720,11 @@ struct BwdCall {
 };
 
 static int run_bwd(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c) {
+  int rc = dlmi_scratch_reserve(ctx, 2 * 16 * 3 * H * sizeof(float));
+  if (rc != DLMI_OK) return rc;
   bool const vec4 = use_vec4(H, {c.x, c.gamma, c.beta, c.mean, c.stdv, c.r, c.d, c.xhat, c.dY, c.dX}) &&
-                    (c.drop_kind == 0 || (reinterpret_cast<uintptr_t>(c.mask) & 3u) == 0);
-  ColGeom const g = col_geometry(ctx, B, H, vec4, 3);
+                    (c.drop_mode == kDropNone || (reinterpret_cast<uintptr_t>(c.mask) & 3u) == 0);
+  ColGeom const g = reduce_geometry(ctx, B, H, vec4, 3);
   // scratch: first half partials [3][nchunks][H], second half coefficients [3][H]
   float *partial = reinterpret_cast<float *>(ctx->scratch);
   float *coef = reinterpret_cast<float *>(ctx->scratch + ctx->scratch_bytes / 2);
@@ -663,38 +732,41 @@ static int run_bwd(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c) {
   a.x = c.x; a.gamma = c.gamma; a.beta = c.beta; a.mean = c.mean; a.stdv = c.stdv; a.r = c.r; a.d = c.d;
   a.xhat = c.xhat; a.mask = c.mask; a.dY = c.dY; a.partial = partial; a.coef = coef; a.dX = c.dX;
   a.B = B; a.H = H; a.rows_per_chunk = g.rows_per_chunk; a.tx_log2 = g.tx_log2;
-  a.drop_kind = c.drop_kind; a.mask_per_element = c.mask_per_element; a.drop_bwd_masked = c.drop_bwd_masked;
-  a.drop_scale = c.drop_scale;
+  a.drop_bwd_masked = c.drop_bwd_masked; a.drop_scale = c.drop_scale;
   dim3 const grid(g.grid_x, g.nchunks), block(kBlock);
   if (c.xhat_given) {
     if (vec4)
-      hipLaunchKernelGGL((k_bwd_reduce<4, DLMI_ACT_LINEAR, true>), grid, block, 0, ctx->stream, a);
+      hipLaunchKernelGGL((k_bwd_reduce<4, DLMI_ACT_LINEAR, kDropNone, true>), grid, block, 0, ctx->stream, a);
     else
-      hipLaunchKernelGGL((k_bwd_reduce<1, DLMI_ACT_LINEAR, true>), grid, block, 0, ctx->stream, a);
+      hipLaunchKernelGGL((k_bwd_reduce<1, DLMI_ACT_LINEAR, kDropNone, true>), grid, block, 0, ctx->stream, a);
   } else {
-    DLMI_DISPATCH_ACT(c.act, {
+    DLMI_DISPATCH_ACT(c.act, DLMI_DISPATCH_DROP(c.drop_mode, {
       if (vec4)
-        hipLaunchKernelGGL((k_bwd_reduce<4, ACT, false>), grid, block, 0, ctx->stream, a);
+        hipLaunchKernelGGL((k_bwd_reduce<4, ACT, DROPM, false>), grid, block, 0, ctx->stream, a);
       else
-        hipLaunchKernelGGL((k_bwd_reduce<1, ACT, false>), grid, block, 0, ctx->stream, a);
-    });
+        hipLaunchKernelGGL((k_bwd_reduce<1, ACT, DROPM, false>), grid, block, 0, ctx->stream, a);
+    }));
   }
   DLMI_LAUNCH_CHECK(ctx, "k_bwd_reduce");
   hipLaunchKernelGGL(k_bwd_finalize, dim3(static_cast<unsigned>(dlmi_ceil_div(H, kFinCols))), block, 0, ctx->stream,
                      partial, g.nchunks, B, H, c.gamma, c.stdv, c.r, c.dgamma, c.dbeta, c.dmean, c.dstd, coef);
   DLMI_LAUNCH_CHECK(ctx, "k_bwd_finalize");
+  ColGeom const ga = apply_geometry(B, H, vec4);
+  a.rows_per_chunk = ga.rows_per_chunk;
+  a.tx_log2 = ga.tx_log2;
+  dim3 const agrid(ga.grid_x, ga.nchunks);
   if (c.xhat_given) {
     if (vec4)
-      hipLaunchKernelGGL((k_bwd_apply<4, DLMI_ACT_LINEAR, true>), grid, block, 0, ctx->stream, a);
+      hipLaunchKernelGGL((k_bwd_apply<4, DLMI_ACT_LINEAR, kDropNone, true>), agrid, block, 0, ctx->stream, a);
     else
-      hipLaunchKernelGGL((k_bwd_apply<1, DLMI_ACT_LINEAR, true>), grid, block, 0, ctx->stream, a);
+      hipLaunchKernelGGL((k_bwd_apply<1, DLMI_ACT_LINEAR, kDropNone, true>), agrid, block, 0, ctx->stream, a);
   } else {
-    DLMI_DISPATCH_ACT(c.act, {
+    DLMI_DISPATCH_ACT(c.act, DLMI_DISPATCH_DROP(c.drop_mode, {
       if (vec4)
-        hipLaunchKernelGGL((k_bwd_apply<4, ACT, false>), grid, block, 0, ctx->stream, a);
+        hipLaunchKernelGGL((k_bwd_apply<4, ACT, DROPM, false>), agrid, block, 0, ctx->stream, a);
       else
-        hipLaunchKernelGGL((k_bwd_apply<1, ACT, false>), grid, block, 0, ctx->stream, a);
-    });
+        hipLaunchKernelGGL((k_bwd_apply<1, ACT, DROPM, false>), agrid, block, 0, ctx->stream, a);
+    }));
   }
   DLMI_LAUNCH_CHECK(ctx, "k_bwd_apply");
   return DLMI_OK;
@@ -712,6 +784,33 @@ static int check_desc(dlmi_ctx *ctx, dlmi_fused_desc const *desc, uint8_t const 
   return DLMI_OK;
 }
 
+static int drop_mode_of(dlmi_fused_desc const *desc) {
+  if (desc->dropout == DLMI_DROP_NONE) return kDropNone;
+  return desc->mask_per_element ? kDropElem : kDropUnit;
+}
+// plain Bernoulli keeps the value as it is (scale 1); inverted rescales by 1/keep
+static float drop_scale_of(dlmi_fused_desc const *desc) {
+  return desc->dropout == DLMI_DROP_BERNOULLI_INVERTED ? desc->drop_scale : 1.0f;
+}
+
+int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
+                            float const *gamma, float const *beta, uint8_t const *mask, float *mean, float *stdv,
+                            float *mov_mean, float *mov_std, float *r, float *d, float *y, float const *partial,
+                            unsigned nchunks) {
+  int rc = check_desc(ctx, desc, mask);
+  if (rc != DLMI_OK) return rc;
+  DLMI_REQUIRE(ctx, x && gamma && beta && mean && stdv && mov_mean && mov_std && r && d && y, "null pointer");
+  FwdTrainCall c;
+  c.norm = desc->norm; c.act = desc->act; c.drop_mode = drop_mode_of(desc);
+  c.momentum = desc->momentum; c.eps = desc->eps; c.r_max = desc->r_max; c.d_max = desc->d_max;
+  c.drop_scale = drop_scale_of(desc);
+  c.x = x; c.gamma = gamma; c.beta = beta; c.mask = mask;
+  c.mean = mean; c.stdv = stdv; c.mov_mean = mov_mean; c.mov_std = mov_std; c.r = r; c.d = d;
+  c.y = y; c.xhat = nullptr; c.nrm = nullptr;
+  c.partial_in = partial; c.partial_chunks = nchunks;
+  return run_fwd_train(ctx, B, H, c);
+}
+
 }  // namespace dlmi
 
 using namespace dlmi;
@@ -727,7 +826,7 @@ int dlmi_norm_fwd_train(dlmi_ctx *ctx, dlmi_norm norm, size_t B, size_t H, float
   DLMI_REQUIRE(ctx, B > 0 && H > 0, "empty tensor");
   DLMI_REQUIRE(ctx, x && gamma && beta && mean && stdv && mov_mean && mov_std && r && d, "null pointer");
   FwdTrainCall c;
-  c.norm = norm; c.act = DLMI_ACT_LINEAR; c.drop_kind = 0; c.mask_per_element = 0;
+  c.norm = norm; c.act = DLMI_ACT_LINEAR; c.drop_mode = kDropNone;
   c.momentum = momentum; c.eps = eps; c.r_max = r_max; c.d_max = d_max; c.drop_scale = 1.0f;
   c.x = x; c.gamma = gamma; c.beta = beta; c.mask = nullptr;
   c.mean = mean; c.stdv = stdv; c.mov_mean = mov_mean; c.mov_std = mov_std; c.r = r; c.d = d;
@@ -744,10 +843,9 @@ int dlmi_fused_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
   DLMI_REQUIRE(ctx, B > 0 && H > 0, "empty tensor");
   DLMI_REQUIRE(ctx, x && gamma && beta && mean && stdv && mov_mean && mov_std && r && d && y, "null pointer");
   FwdTrainCall c;
-  c.norm = desc->norm; c.act = desc->act; c.drop_kind = drop_kind_of(desc->dropout);
-  c.mask_per_element = desc->mask_per_element;
+  c.norm = desc->norm; c.act = desc->act; c.drop_mode = drop_mode_of(desc);
   c.momentum = desc->momentum; c.eps = desc->eps; c.r_max = desc->r_max; c.d_max = desc->d_max;
-  c.drop_scale = desc->drop_scale;
+  c.drop_scale = drop_scale_of(desc);
   c.x = x; c.gamma = gamma; c.beta = beta; c.mask = mask;
   c.mean = mean; c.stdv = stdv; c.mov_mean = mov_mean; c.mov_std = mov_std; c.r = r; c.d = d;
   c.y = y; c.xhat = nullptr; c.nrm = nullptr;
@@ -763,7 +861,7 @@ int dlmi_norm_bwd(dlmi_ctx *ctx, dlmi_norm norm, size_t B, size_t H, float const
   DLMI_REQUIRE(ctx, mean && stdv && gamma && x && xhat && dN && dgamma && dbeta && dx, "null pointer");
   DLMI_REQUIRE(ctx, norm == DLMI_NORM_BATCH || r != nullptr, "renormalization needs r");
   BwdCall c;
-  c.act = DLMI_ACT_LINEAR; c.xhat_given = true; c.drop_kind = 0; c.mask_per_element = 0; c.drop_bwd_masked = 0;
+  c.act = DLMI_ACT_LINEAR; c.xhat_given = true; c.drop_mode = kDropNone; c.drop_bwd_masked = 0;
   c.drop_scale = 1.0f;
   c.x = x; c.gamma = gamma; c.beta = nullptr; c.mean = mean; c.stdv = stdv;
   c.r = norm == DLMI_NORM_BATCH_RENORM ? r : nullptr; c.d = nullptr; c.xhat = xhat; c.dY = dN; c.mask = nullptr;
@@ -781,10 +879,9 @@ int dlmi_fused_norm_act_bwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
   DLMI_REQUIRE(ctx, B > 0 && H > 0, "empty tensor");
   DLMI_REQUIRE(ctx, x && gamma && beta && mean && stdv && r && d && dY && dgamma && dbeta && dX, "null pointer");
   BwdCall c;
-  c.act = desc->act; c.xhat_given = false; c.drop_kind = drop_kind_of(desc->dropout);
-  c.mask_per_element = desc->mask_per_element;
+  c.act = desc->act; c.xhat_given = false; c.drop_mode = drop_mode_of(desc);
   c.drop_bwd_masked = desc->dropout_bwd == DLMI_DROP_BWD_MASKED ? 1 : 0;
-  c.drop_scale = desc->drop_scale;
+  c.drop_scale = drop_scale_of(desc);
   c.x = x; c.gamma = gamma; c.beta = beta; c.mean = mean; c.stdv = stdv; c.r = r; c.d = d; c.xhat = nullptr;
   c.dY = dY; c.mask = mask;
   c.dgamma = dgamma; c.dbeta = dbeta; c.dmean = nullptr; c.dstd = nullptr; c.dX = dX;

@@ -200,6 +200,18 @@ int dlmi_fused_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
                             uint8_t const *mask, float *mean, float *std, float *mov_mean,
                             float *mov_std, float *r, float *d, float *y);
 
+/* The whole forward of one normalized layer: Z = X W^T with the column sums of Z
+ * and Z^2 accumulated in the GEMM epilogue (per 128- or 256-row tile, combined
+ * in a fixed order), then the finalize and apply passes of
+ * dlmi_fused_norm_act_fwd.  The statistics pass over Z disappears: the
+ * normalization reads Z once (8 B/element instead of 12).  Normalized layers
+ * have no bias (v1/learner/model.hpp:708).  Z [B,H] is kept for the backward.
+ * Composition of Forward_Pass__FC__Loop (fwp_st.cpp:298-470) for such a layer. */
+int dlmi_fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t K, size_t H,
+                         float const *X, float const *W, float const *gamma, float const *beta,
+                         uint8_t const *mask, float *Z, float *mean, float *std, float *mov_mean,
+                         float *mov_std, float *r, float *d, float *y);
+
 /* dX [B,H] out (may alias dY); dgamma, dbeta [H] accumulate (+=).  Composition
  * of a19 -> a20/a21 in the order of Backward_Pass__Gradient__FC__Loop
  * (bwp_st.cpp:543-701).  mean/std/r/d are the forward's outputs. */
