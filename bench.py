@@ -30,6 +30,15 @@ WORKLOADS = {
 }
 HYPER = dict(momentum=0.99, eps=1e-5, r_max=3.0, d_max=5.0)
 
+# HBM-side bytes per launch (sequence) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# file's --only parts, calibrated against the plain copy of --only copy
+# (profiles/c3_c2_hbm_traffic_pmc.md).  They cannot be measured from inside this process.
+MIB = 1024.0 * 1024.0
+MEASURED_TRAFFIC_BYTES = {
+    "c3": {"gemm": (897.1 + 896.8 + 1579.5) / 3.0 * MIB, "norm_act": 1055.9 * MIB},
+    "c2": {"norm_act": (66.1 + 128.3 + 131.2 + 192.6) * MIB},
+}
+
 
 def make_inputs(torch, name):
     B, K, H, act, _ = WORKLOADS[name]
@@ -102,6 +111,11 @@ class Step:
         t = self.t
         self.dl.fc_norm_act_fwd(self.desc, t["X"], t["W"], t["gamma"], t["beta"], t["mov_mean"], t["mov_std"],
                                 Z=t["Z"], out=t["y"], stats=t["stats"])
+
+    def copy(self):
+        """A plain device copy of one [B, H] tensor (known size): calibrates the
+        FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run."""
+        self.t["y"].copy_(self.t["dY"])
 
     def parts(self):
         if self.K:
@@ -218,7 +232,7 @@ def main():
     t_nb = time_events(torch, step.norm_bwd, 20)
     hbm_bytes = 32.0 * E  # fwd 12 B/element + bwd 20 B/element
     hbm = {"bound": "hbm", "achieved": hbm_bytes / ((t_nf + t_nb) * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-           "traffic": None, "kernels": "k_col_stats+k_fwd_finalize+k_fwd_apply / k_bwd_reduce+k_bwd_finalize+k_bwd_apply",
+           "traffic": MEASURED_TRAFFIC_BYTES.get(name, {}).get("norm_act"), "kernels": "k_col_stats+k_fwd_finalize+k_fwd_apply / k_bwd_reduce+k_bwd_finalize+k_bwd_apply",
            "ms_fwd": t_nf, "ms_bwd": t_nb, "bytes_fwd": 12.0 * E, "bytes_bwd": 20.0 * E}
     hbm["frac"] = hbm["achieved"] / hbm["peak"]
     detail = {"ms_norm_fwd": t_nf, "ms_norm_bwd": t_nb}
@@ -229,7 +243,7 @@ def main():
         flops = 2.0 * B * K * H
         avg = (t_gf + t_gx + t_gw) / 3.0
         roof = {"bound": "mfma", "achieved": flops / (avg * 1e-3) / 1e12, "peak": MFMA_FP32_PEAK_TFLOPS,
-                "unit": "TFLOP/s", "traffic": None, "kernel": "k_gemm_f32 (avg of fwd NT, dX NN, dW TN launches)",
+                "unit": "TFLOP/s", "traffic": MEASURED_TRAFFIC_BYTES.get(name, {}).get("gemm"), "kernel": "k_gemm_f32 (avg of fwd NT, dX NN, dW TN launches)",
                 "tflops_fwd": flops / (t_gf * 1e-3) / 1e12, "tflops_dx": flops / (t_gx * 1e-3) / 1e12,
                 "tflops_dw": flops / (t_gw * 1e-3) / 1e12}
         roof["frac"] = roof["achieved"] / roof["peak"]

@@ -408,9 +408,10 @@ void Model::forward_pass(size_t const B, real const *const *const Xm, long long 
     size_t const H = l.n_out;
     float const *W = impl_->d_params + l.first_connection_index;
     float const *bias = l.Use__Bias() ? impl_->d_params + l.first_bias_connection_index : nullptr;
-    if (dlmi_fc_fwd(ctx, B, K, H, in, W, bias, l.d_summations) != DLMI_OK) { fail("forward_pass: dlmi_fc_fwd"); return; }
     bool const softmax = l.type_activation_function == ACTIVATION::SOFTMAX;
     if (!softmax && !act_on_path(l.type_activation_function)) { fail("forward_pass: layer activation not set to one on this path"); return; }
+    bool const fused_fc_norm = l.Use__Normalization() && training;  // the GEMM epilogue takes the batch statistics
+    if (!fused_fc_norm && dlmi_fc_fwd(ctx, B, K, H, in, W, bias, l.d_summations) != DLMI_OK) { fail("forward_pass: dlmi_fc_fwd"); return; }
     int rc = DLMI_OK;
     if (l.Use__Normalization()) {
       dlmi_fused_desc d = make_desc(*this, l);
@@ -419,8 +420,8 @@ void Model::forward_pass(size_t const B, real const *const *const Xm, long long 
       if (training) {
         // dropout acts only in PROPAGATION::TRAINING, not in UPDATE_BATCH_NORM (fwp_st.cpp:657)
         if (type_state_propagation != PROPAGATION::TRAINING) d.dropout = DLMI_DROP_NONE;
-        rc = dlmi_fused_norm_act_fwd(ctx, &d, B, H, l.d_summations, gamma, beta, l.d_mask, l.d_mean, l.d_std, mm, ms,
-                                     l.d_r, l.d_d, l.d_outputs);
+        rc = dlmi_fc_norm_act_fwd(ctx, &d, B, K, H, in, W, gamma, beta, l.d_mask, l.d_summations, l.d_mean, l.d_std, mm,
+                                  ms, l.d_r, l.d_d, l.d_outputs);
         if (rc == DLMI_OK && type_state_propagation != PROPAGATION::TRAINING && l.Use__Dropout())
           rc = dlmi_dropout_fwd(ctx, static_cast<dlmi_dropout>(l.type_dropout), 0, 0, B, H, nullptr, l.dropout_values[0],
                                 l.d_outputs);
