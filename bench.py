@@ -256,7 +256,7 @@ def main():
     else:
         roof = dict(hbm)
 
-    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 1024, "c2": 4096, "c5": 65536}[name]
+    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 8192, "c2": 4096, "c5": 65536}[name]  # c3: ~10 s on 16 cores
     cpu = cpu_baseline(name, cpu_rows) if cpu_rows else None
 
     out = {
