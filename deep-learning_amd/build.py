@@ -20,6 +20,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops is switched off: the compiler must not form v_pk_*_f32.
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+FLAGS += os.environ.get("DLMI_HIPCC_EXTRA", "").split()  # e.g. -DDLMI_BWD_REDUCE_U=8 while tuning
 
 
 def sources():

@@ -27,6 +27,7 @@
 // there makes the compiler wait for each load before issuing the next.
 //
 // Citations: /root/reference/lib/deep-learning/v1/learner/.
+#include <cstdlib>
 #include <initializer_list>
 
 #include "activations.hpp"
@@ -36,6 +37,14 @@ namespace dlmi {
 
 constexpr int kBlock = 256;
 constexpr int kWave = 64;
+
+// rows in flight per thread in the reduction passes
+#ifndef DLMI_STATS_U
+#define DLMI_STATS_U 8
+#endif
+#ifndef DLMI_BWD_REDUCE_U
+#define DLMI_BWD_REDUCE_U 4
+#endif
 
 // dropout as a template mode
 constexpr int kDropNone = 0, kDropUnit = 1, kDropElem = 2;
@@ -48,13 +57,28 @@ struct ColGeom {
   size_t rows_per_chunk;
 };
 
-// Geometry of a reduction pass (TX <= 64).
+// Tuning aids: DLMI_NORM_{STATS,BWD}_TX (64, 128 or 256), .._ROWS_PER_THREAD and
+// .._BLOCKS_PER_CU override the geometry of the two reduction passes,
+// DLMI_NORM_APPLY_ROWS_PER_THREAD that of the apply passes.
+static int env_int(char const *name, int dflt) {
+  char const *e = getenv(name);
+  if (e == nullptr || *e == 0) return dflt;
+  int const v = atoi(e);
+  return v > 0 ? v : dflt;
+}
+
+// Geometry of a reduction pass.
 static ColGeom reduce_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, int nacc) {
+  static int const tx_caps[2] = {env_int("DLMI_NORM_STATS_TX", 64), env_int("DLMI_NORM_BWD_TX", 256)};
+  static int const rpts[2] = {env_int("DLMI_NORM_STATS_ROWS_PER_THREAD", 16), env_int("DLMI_NORM_BWD_ROWS_PER_THREAD", 16)};
+  static int const bpcs[2] = {env_int("DLMI_NORM_STATS_BLOCKS_PER_CU", 8), env_int("DLMI_NORM_BWD_BLOCKS_PER_CU", 1)};
+  int const which = nacc == 2 ? 0 : 1;
+  int const tx_cap = tx_caps[which], rows_per_thread = rpts[which], blocks_per_cu = bpcs[which];
   ColGeom g;
   g.vec = vec4 ? 4 : 1;
   size_t const groups = dlmi_ceil_div(H, g.vec);
-  int tx = 64;
-  g.tx_log2 = 6;
+  int tx = tx_cap >= 256 ? 256 : (tx_cap >= 128 ? 128 : 64);
+  g.tx_log2 = tx == 256 ? 8 : (tx == 128 ? 7 : 6);
   while (tx > 1 && static_cast<size_t>(tx / 2) >= groups) {
     tx /= 2;
     --g.tx_log2;
@@ -63,10 +87,9 @@ static ColGeom reduce_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec
   g.grid_x = static_cast<unsigned>(dlmi_ceil_div(groups, tx));
   // enough blocks to cover every CU several times over, but each thread still
   // streams >= 16 rows: the partial sums stay a small fraction of the traffic
-  // and the fixed cost of a block is amortised (measured optimum on 4096-wide
-  // tensors: 64 rows per chunk)
-  size_t want = dlmi_ceil_div(static_cast<size_t>(ctx->num_cu) * 8, g.grid_x);
-  size_t const max_by_rows = B / (static_cast<size_t>(ty) * 16);
+  // and the fixed cost of a block is amortised
+  size_t want = dlmi_ceil_div(static_cast<size_t>(ctx->num_cu) * blocks_per_cu, g.grid_x);
+  size_t const max_by_rows = B / (static_cast<size_t>(ty) * rows_per_thread);
   if (want > max_by_rows) want = max_by_rows;
   // partial sums must fit half of the scratch block: nacc * nchunks * H floats
   size_t const max_by_scratch = (ctx->scratch_bytes / 2) / (static_cast<size_t>(nacc) * H * sizeof(float));
@@ -92,7 +115,8 @@ static ColGeom apply_geometry(size_t B, size_t H, bool vec4) {
   }
   int const ty = kBlock / tx;
   g.grid_x = static_cast<unsigned>(dlmi_ceil_div(groups, tx));
-  g.rows_per_chunk = static_cast<size_t>(ty) * 8;
+  static int const rows_per_thread = env_int("DLMI_NORM_APPLY_ROWS_PER_THREAD", 8);
+  g.rows_per_chunk = static_cast<size_t>(ty) * rows_per_thread;
   size_t chunks = dlmi_ceil_div(B, g.rows_per_chunk);
   if (chunks > 65535) {
     chunks = 65535;
@@ -130,9 +154,10 @@ __device__ __forceinline__ void load_u8(uint8_t const *p, uint8_t (&v)[VEC]) {
   }
 }
 
-// Sum NV per-thread values over the TY rows of the block (TX <= 64).  On
-// return the threads with threadIdx.x < TX hold the block totals for their
-// column group.
+// Sum NV per-thread values over the TY rows of the block.  On return the
+// threads with threadIdx.x < TX hold the block totals for their column group.
+// TX < 64: rows that share a wavefront are combined with shuffles first, then
+// the four wavefronts through LDS; TX >= 64: the 256/TX rows through LDS.
 template <int NV>
 __device__ __forceinline__ void block_rows_reduce(float (&v)[NV], int tx, float *lds) {
   int const lane = threadIdx.x & (kWave - 1);
@@ -142,18 +167,22 @@ __device__ __forceinline__ void block_rows_reduce(float (&v)[NV], int tx, float 
 #pragma unroll
     for (int i = 0; i < NV; ++i) v[i] += __shfl_xor(v[i], off, kWave);
   }
-  if (lane < tx) {
+  int const nrows = tx < kWave ? kBlock / kWave : kBlock / tx;
+  if (nrows == 1) return;
+  int const row = tx < kWave ? wave : static_cast<int>(threadIdx.x) / tx;
+  int const cg = tx < kWave ? lane : static_cast<int>(threadIdx.x) & (tx - 1);
+  if (tx >= kWave || lane < tx) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) lds[(wave * kWave + lane) * NV + i] = v[i];
+    for (int i = 0; i < NV; ++i) lds[(row * tx + cg) * NV + i] = v[i];
   }
   __syncthreads();
-  // LDS tree over the four wavefronts: (0+1) + (2+3), fixed order
-  if (threadIdx.x < tx) {
+  // fixed order: (0+1) + (2+3) for four rows, 0+1 for two
+  if (static_cast<int>(threadIdx.x) < tx) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      float const a = lds[(0 * kWave + lane) * NV + i] + lds[(1 * kWave + lane) * NV + i];
-      float const b = lds[(2 * kWave + lane) * NV + i] + lds[(3 * kWave + lane) * NV + i];
-      v[i] = a + b;
+      float s = lds[(0 * tx + cg) * NV + i] + lds[(1 * tx + cg) * NV + i];
+      if (nrows == 4) s += lds[(2 * tx + cg) * NV + i] + lds[(3 * tx + cg) * NV + i];
+      v[i] = s;
     }
   }
 }
@@ -176,7 +205,7 @@ __global__ __launch_bounds__(kBlock) void k_col_stats(float const *__restrict__ 
 #pragma unroll
   for (int i = 0; i < 2 * VEC; ++i) acc[i] = 0.0f;
   if (live) {
-    constexpr int U = 8;
+    constexpr int U = DLMI_STATS_U;
     size_t b = b0 + ty;
     for (; b + (U - 1) * static_cast<size_t>(TY) < b1; b += U * static_cast<size_t>(TY)) {
       float v[U][VEC];
@@ -471,7 +500,7 @@ __global__ __launch_bounds__(kBlock) void k_bwd_reduce(BwdArgs a) {
   if (live) {
     UnitConsts<VEC> uc;
     load_unit_consts<VEC, DROPM, XHAT_GIVEN>(a, col, uc);
-    constexpr int U = 4;
+    constexpr int U = DLMI_BWD_REDUCE_U;
     auto body = [&](float const (&xv)[VEC], float const (&dy)[VEC], float const (&xg)[VEC],
                     uint8_t const (&mv)[VEC]) {
 #pragma unroll

@@ -176,7 +176,8 @@ def oracle_fused(oracle, act, x, gamma, beta, mm, ms, hyper, renorm, drop, mask,
     return fw, y, bw
 
 
-FUSED_SHAPES = [(64, 256), (100, 132), (257, 64), (33, 5), (512, 1024), (2048, 16), (9, 4096)]
+FUSED_SHAPES = [(64, 256), (100, 132), (257, 64), (33, 5), (512, 1024), (2048, 16), (9, 4096),
+                (300, 1023), (64, 1536), (1030, 700)]
 
 
 @pytest.mark.parametrize("B,H", FUSED_SHAPES)
