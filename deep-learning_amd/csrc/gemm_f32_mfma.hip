@@ -11,21 +11,25 @@
 // workgroup (4 wavefronts, 2 x 2) owns a BM x BN tile of C; each wavefront
 // owns (BM/2) x (BN/2) as a grid of 32x32 v_mfma_f32_32x32x2_f32 blocks whose
 // accumulators stay in registers for the whole K loop.  Operand tiles are
-// staged through LDS (double buffered, one barrier per K tile) while the next
-// tile's global loads are already in flight in registers.
+// staged through LDS (two stages, one barrier per K tile) behind a register
+// stage: the global loads run two tiles ahead of the MFMAs, and the LDS writes,
+// the global loads and the fragment reads of a tile are spread between the
+// MFMAs of the previous one with scheduling-group hints.
 //
 // The MFMA consumes two k per instruction: lanes 0-31 supply k_lo, lanes 32-63
 // k_hi.  Because the sum over k is order-free inside a tile, the kernel feeds
 // k = {s, s+4} (s = 0..3) of every group of 8 instead of {2s, 2s+1}: a lane
 // then needs 4 CONSECUTIVE k of one row, i.e. one ds_read_b128 per 4 MFMAs for
-// k-contiguous operands.  Rows are padded by 4 floats so those 16-byte reads
-// hit distinct banks.
+// either operand (one whose row index is contiguous in memory is transposed on
+// its way into LDS).  Rows are padded by 4 floats so those 16-byte reads hit
+// distinct banks.
 //
 // Workgroup ids are remapped so that (a) the ids that land on one XCD (id % 8)
 // cover a compact block of tiles and (b) tiles are walked in groups of 8 rows
 // of tiles, which keeps the A and B panels of concurrently running workgroups
 // resident in that XCD's L2.
 #include <cstdlib>
+#include <type_traits>
 
 #include "dlmi_common.hpp"
 
@@ -52,19 +56,40 @@ struct GemmArgs {
   unsigned tiles_m, tiles_n;
 };
 
-// LDS tile of an operand whose k index is contiguous in memory: [ROWS][BK+4].
-// LDS tile of an operand whose row (m or n) index is contiguous:  [BK][ROWS+8].
+// LDS tile of either operand: [ROWS][BK+4], k contiguous, so that the MFMA
+// fragments of both operands are 16-byte LDS reads whatever the layout in
+// memory.  An operand whose row (m or n) index is contiguous in memory is
+// transposed on its way into LDS.
 template <int ROWS, int BK, bool KCONTIG>
 struct TileShape {
-  static constexpr int kStride = KCONTIG ? BK + 4 : ROWS + 8;
-  static constexpr int kFloats = KCONTIG ? ROWS * (BK + 4) : BK * (ROWS + 8);
+  static constexpr int kStride = BK + 4;
+  static constexpr int kFloats = ROWS * (BK + 4);
   static constexpr int kVec4 = ROWS * BK / 4;             // 16-byte pieces per tile
   static constexpr int kPerThread = kVec4 / kGemmThreads;  // pieces per thread
   static_assert(kVec4 % kGemmThreads == 0, "tile must divide evenly over the workgroup");
+  static_assert(ROWS % 32 == 0 && BK % 8 == 0, "tile shape");
   // the prefetch registers of one thread as ONE vector value (a first-class
   // SSA value: it can neither be spilled to scratch nor be promoted to LDS the
   // way a local array can)
   typedef float Regs __attribute__((ext_vector_type(4 * kPerThread)));
+
+  // Which 16-byte piece thread-slot f (0 .. kVec4-1) moves: `row` and `k` are
+  // relative to the tile; the piece covers 4 consecutive k (KCONTIG) or 4
+  // consecutive rows (!KCONTIG).
+  // !KCONTIG: a wavefront covers 8 k x 8 row groups, i.e. 8 segments of 128
+  // contiguous bytes in memory; its transposed 4-byte LDS stores then fall
+  // into 32 distinct banks (stride 20: row groups 4 apart share a bank).
+  __device__ static __forceinline__ void piece(int f, int &row, int &k) {
+    if constexpr (KCONTIG) {
+      row = f / (BK / 4);
+      k = (f % (BK / 4)) * 4;
+    } else {
+      int const kl = f & 7, rl = (f >> 3) & 7, rest = f >> 6;
+      int const rh = rest % (ROWS / 32), kh = rest / (ROWS / 32);
+      k = kh * 8 + kl;
+      row = (rh * 8 + rl) * 4;
+    }
+  }
 };
 
 // Global -> registers for one operand tile.  `row0` is the tile's first row
@@ -77,15 +102,9 @@ __device__ __forceinline__ typename TileShape<ROWS, BK, KCONTIG>::Regs tile_load
   typename T::Regs regs;
 #pragma unroll
   for (int i = 0; i < T::kPerThread; ++i) {
-    int const f = threadIdx.x + i * kGemmThreads;
-    size_t row, k;
-    if constexpr (KCONTIG) {
-      row = row0 + f / (BK / 4);
-      k = k0 + (f % (BK / 4)) * 4;
-    } else {
-      k = k0 + f / (ROWS / 4);
-      row = row0 + (f % (ROWS / 4)) * 4;
-    }
+    int tr, tk;
+    T::piece(threadIdx.x + i * kGemmThreads, tr, tk);
+    size_t const row = row0 + tr, k = k0 + tk;
     v4f t;
     if constexpr (FAST) {
       float const *src = KCONTIG ? P + row * ld + k : P + k * ld + row;
@@ -110,17 +129,17 @@ __device__ __forceinline__ void tile_store(float *__restrict__ lds,
   using T = TileShape<ROWS, BK, KCONTIG>;
 #pragma unroll
   for (int i = 0; i < T::kPerThread; ++i) {
-    int const f = threadIdx.x + i * kGemmThreads;
-    int off;
+    int tr, tk;
+    T::piece(threadIdx.x + i * kGemmThreads, tr, tk);
     if constexpr (KCONTIG) {
-      off = (f / (BK / 4)) * T::kStride + (f % (BK / 4)) * 4;
-    } else {
-      off = (f / (ROWS / 4)) * T::kStride + (f % (ROWS / 4)) * 4;
-    }
-    v4f t;
+      v4f t;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) t[e] = regs[4 * i + e];
-    *reinterpret_cast<v4f *>(lds + off) = t;
+      for (int e = 0; e < 4; ++e) t[e] = regs[4 * i + e];
+      *reinterpret_cast<v4f *>(lds + tr * T::kStride + tk) = t;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) lds[(tr + e) * T::kStride + tk] = regs[4 * i + e];
+    }
   }
 }
 
@@ -130,13 +149,22 @@ __device__ __forceinline__ void tile_store(float *__restrict__ lds,
 template <int ROWS, int BK, bool KCONTIG>
 __device__ __forceinline__ v4f frag_load(float const *__restrict__ lds, int r, int kk) {
   using T = TileShape<ROWS, BK, KCONTIG>;
-  if constexpr (KCONTIG) {
-    return *reinterpret_cast<v4f const *>(lds + r * T::kStride + kk);
-  } else {
-    v4f t;
-#pragma unroll
-    for (int s = 0; s < 4; ++s) t[s] = lds[(kk + s) * T::kStride + r];
-    return t;
+  return *reinterpret_cast<v4f const *>(lds + r * T::kStride + kk);
+}
+
+// Instruction-order hints for the software pipeline (scheduling group masks:
+// 0x008 MFMA, 0x020 vector-memory read, 0x100 LDS read, 0x200 LDS write).
+template <int MASK, int N>
+__device__ __forceinline__ void sched_group() {
+  if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, 0);
+}
+// CNT instructions of kind MASK spread evenly behind NMF consecutive MFMAs.
+template <int NMF, int MASK, int CNT, int M = 0>
+__device__ __forceinline__ void sched_spread() {
+  if constexpr (M < NMF) {
+    sched_group<0x008, 1>();
+    sched_group<MASK, ((M + 1) * CNT) / NMF - (M * CNT) / NMF>();
+    sched_spread<NMF, MASK, CNT, M + 1>();
   }
 }
 
@@ -181,49 +209,94 @@ void k_gemm_f32(GemmArgs g) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  // All MFMAs of one K tile staged at `sa` / `sb`.
-  auto mma_tile = [&](float const *__restrict__ sa, float const *__restrict__ sb) {
+  // Fragments of K group `kk` (8 consecutive k) of the tile staged at sa / sb.
+  auto frags = [&](float const *__restrict__ sa, float const *__restrict__ sb, int kk, v4f (&fa)[TM], v4f (&fb)[TN]) {
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 8) {
-      v4f fa[TM], fb[TN];
+    for (int i = 0; i < TM; ++i) fa[i] = frag_load<BM, BK, A_KCONTIG>(sa, wm0 + i * 32 + lr, kk + lk);
 #pragma unroll
-      for (int i = 0; i < TM; ++i) fa[i] = frag_load<BM, BK, A_KCONTIG>(sa, wm0 + i * 32 + lr, kk + lk);
+    for (int j = 0; j < TN; ++j) fb[j] = frag_load<BN, BK, B_KCONTIG>(sb, wn0 + j * 32 + lr, kk + lk);
+  };
+  // MFMA steps s0 .. s1-1 (of 4) of one K group for every block of the wavefront.
+  auto steps = [&](v4f const (&fa)[TM], v4f const (&fb)[TN], int s0, int s1) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j) fb[j] = frag_load<BN, BK, B_KCONTIG>(sb, wn0 + j * 32 + lr, kk + lk);
+    for (int s = s0; s < s1; ++s)
 #pragma unroll
-      for (int s = 0; s < 4; ++s)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
-    }
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
   };
 
+  static_assert(BK == 16, "the pipeline below is written for two K groups per tile");
+  constexpr int NM = TM * TN * (BK / 2);                                     // MFMAs per K tile
+  constexpr int NFR = TM + TN;                                               // LDS reads per K group
+  constexpr int NWR = (A_KCONTIG ? 1 : 4) * TA::kPerThread + (B_KCONTIG ? 1 : 4) * TB::kPerThread;  // LDS writes
+  constexpr int NLD = TA::kPerThread + TB::kPerThread;                       // global loads
+
   if (ktiles > 0) {
+    // Software pipeline over the K tiles: two LDS stages, one register stage.
+    // During tile kt (LDS stage kt&1): tile kt+1, fetched from memory during
+    // tile kt-1, moves from registers into the other stage, the global loads of
+    // tile kt+2 are issued, and after the barrier - placed three quarters into
+    // the tile's MFMAs, when every wavefront is done with both the reads of this
+    // stage and the writes of the next - the first fragments of tile kt+1 are
+    // read.  LDS and memory traffic is spread between the MFMAs, so the matrix
+    // pipe only waits at the barrier itself.
     typename TA::Regs ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, k_begin, g.M, k_end);
     typename TB::Regs rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, k_begin, g.N, k_end);
     tile_store<BM, BK, A_KCONTIG>(lds, ra);
     tile_store<BN, BK, B_KCONTIG>(lds + TA::kFloats, rb);
-    __syncthreads();
-    // Steady state.  The next tile's global loads are issued first and stay in
-    // flight underneath this tile's MFMAs; the scheduling barriers stop the
-    // compiler from sinking them to the end of the tile (where it would then
-    // wait on them at once) to save registers.
-    for (int kt = 0; kt + 1 < ktiles; ++kt) {
-      int const cur = kt & 1;
-      size_t const kn = k_begin + static_cast<size_t>(kt + 1) * BK;
-      ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, kn, g.M, k_end);
-      rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, kn, g.N, k_end);
-      __builtin_amdgcn_sched_barrier(0);
-      mma_tile(lds + cur * kStage, lds + cur * kStage + TA::kFloats);
-      __builtin_amdgcn_sched_barrier(0);
-      tile_store<BM, BK, A_KCONTIG>(lds + (cur ^ 1) * kStage, ra);
-      tile_store<BN, BK, B_KCONTIG>(lds + (cur ^ 1) * kStage + TA::kFloats, rb);
-      __syncthreads();
+    if (ktiles > 1) {
+      ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, k_begin + BK, g.M, k_end);
+      rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, k_begin + BK, g.N, k_end);
     }
-    int const last = (ktiles - 1) & 1;
-    mma_tile(lds + last * kStage, lds + last * kStage + TA::kFloats);
+    __syncthreads();
+    v4f f0a[TM], f0b[TN];
+    frags(lds, lds + TA::kFloats, 0, f0a, f0b);
+
+    // one K tile; STORE: a next tile exists (in registers), LOAD: one after that exists
+    auto tile_step = [&](int kt, auto store_c, auto load_c) {
+      constexpr bool STORE = decltype(store_c)::value, LOAD = decltype(load_c)::value;
+      float const *const sa = lds + (kt & 1) * kStage;
+      float *const na = lds + ((kt & 1) ^ 1) * kStage;
+      v4f f1a[TM], f1b[TN];
+      frags(sa, sa + TA::kFloats, 8, f1a, f1b);
+      steps(f0a, f0b, 0, 4);
+      if constexpr (STORE) {
+        tile_store<BM, BK, A_KCONTIG>(na, ra);
+        tile_store<BN, BK, B_KCONTIG>(na + TA::kFloats, rb);
+      }
+      if constexpr (LOAD) {
+        size_t const kn = k_begin + static_cast<size_t>(kt + 2) * BK;
+        ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, kn, g.M, k_end);
+        rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, kn, g.N, k_end);
+      }
+      steps(f1a, f1b, 0, 2);
+      if constexpr (FAST) {
+        sched_spread<NM / 8, 0x100, NFR>();
+        sched_spread<NM / 4, 0x200, STORE ? NWR : 0>();
+        sched_spread<NM / 4, 0x020, LOAD ? NLD : 0>();
+        sched_group<0x008, NM / 8>();
+      }
+      if constexpr (STORE) {
+        __syncthreads();
+        frags(na, na + TA::kFloats, 0, f0a, f0b);
+      }
+      steps(f1a, f1b, 2, 4);
+      if constexpr (FAST && STORE) {
+        sched_group<0x100, NFR>();
+        sched_group<0x008, NM / 4>();
+      }
+    };
+    using std::false_type;
+    using std::true_type;
+    int kt = 0;
+    for (; kt + 2 < ktiles; ++kt) tile_step(kt, true_type{}, true_type{});
+    if (kt + 1 < ktiles) {
+      tile_step(kt, true_type{}, false_type{});
+      ++kt;
+    }
+    tile_step(kt, false_type{}, false_type{});
   }
 
   // ---- epilogue: accumulator register e of lane l holds
@@ -362,7 +435,7 @@ struct TileCfg {
   int bm, bn, bk;
 };
 
-// Tuning aid: DLMI_GEMM_TILE=<index> picks another compiled tile shape.
+// Tuning aid: DLMI_GEMM_TILE=<index> forces a tile shape (0: 128x128, 1: 256x128, 2: 256x256).
 static int tile_choice() {
   static int const c = [] {
     char const *e = std::getenv("DLMI_GEMM_TILE");
@@ -377,16 +450,25 @@ static int tile_choice() {
 template <bool AK, bool BKC>
 static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, size_t lda, float const *B, size_t ldb,
                 float *C, float const *bias, int accumulate, unsigned *stats_chunks = nullptr) {
-  static TileCfg const cfgs[] = {{128, 128, 16}, {128, 128, 32}, {256, 128, 16}, {256, 128, 32}, {256, 256, 16}};
+  static TileCfg const cfgs[] = {{128, 128, 16}, {256, 128, 16}, {256, 256, 16}};
   int choice = tile_choice();
   if (choice < 0 || choice >= static_cast<int>(sizeof(cfgs) / sizeof(cfgs[0]))) {
-    // default: 256 x 256 tiles (one wavefront per SIMD, 16 MFMA blocks each) when
-    // the output splits evenly into at least two of them per CU, else 128 x 128
-    choice = (M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= 2 * static_cast<size_t>(ctx->num_cu)) ? 4 : 0;
+    // default: the shape with the smallest estimated time = rounds of workgroups
+    // over the CUs x work per round / measured relative efficiency of the shape
+    // (256 x 256 runs one workgroup per CU, the smaller shapes two)
+    static int const per_cu[] = {2, 2, 1};
+    static double const eff[] = {0.95, 0.97, 1.0};
+    double best = 0.0;
+    for (int c = 0; c < static_cast<int>(sizeof(cfgs) / sizeof(cfgs[0])); ++c) {
+      size_t const tiles = dlmi_ceil_div(M, cfgs[c].bm) * dlmi_ceil_div(N, cfgs[c].bn);
+      size_t const rounds = dlmi_ceil_div(tiles, static_cast<size_t>(ctx->num_cu) * per_cu[c]);
+      double const t = static_cast<double>(rounds) * cfgs[c].bm * cfgs[c].bn * per_cu[c] / eff[c];
+      if (c == 0 || t < best) {
+        best = t;
+        choice = c;
+      }
+    }
   }
-  // a big tile only pays when the output has enough of them to fill the GPU
-  if (dlmi_ceil_div(M, cfgs[choice].bm) * dlmi_ceil_div(N, cfgs[choice].bn) < static_cast<size_t>(ctx->num_cu))
-    choice = 0;
   int const bm = cfgs[choice].bm, bn = cfgs[choice].bn, bk = cfgs[choice].bk;
 
   GemmArgs g;
@@ -422,10 +504,8 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   if (splits > 1) g.split_out = reinterpret_cast<float *>(ctx->scratch);
   int rc;
   switch (choice) {
-    case 1: rc = launch_gemm<128, 128, 32, AK, BKC, 2>(ctx, g, splits, fast); break;
-    case 2: rc = launch_gemm<256, 128, 16, AK, BKC, 2>(ctx, g, splits, fast); break;
-    case 3: rc = launch_gemm<256, 128, 32, AK, BKC, 2>(ctx, g, splits, fast); break;
-    case 4: rc = launch_gemm<256, 256, 16, AK, BKC, 1>(ctx, g, splits, fast); break;
+    case 1: rc = launch_gemm<256, 128, 16, AK, BKC, 2>(ctx, g, splits, fast); break;
+    case 2: rc = launch_gemm<256, 256, 16, AK, BKC, 1>(ctx, g, splits, fast); break;
     default: rc = launch_gemm<128, 128, 16, AK, BKC, 2>(ctx, g, splits, fast); break;
   }
   if (rc != DLMI_OK) return rc;
