@@ -35,8 +35,8 @@ HYPER = dict(momentum=0.99, eps=1e-5, r_max=3.0, d_max=5.0)
 # (profiles/c3_c2_hbm_traffic_pmc.md).  They cannot be measured from inside this process.
 MIB = 1024.0 * 1024.0
 MEASURED_TRAFFIC_BYTES = {
-    "c3": {"gemm": (897.1 + 896.8 + 1579.5) / 3.0 * MIB, "norm_act": 1055.9 * MIB},
-    "c2": {"norm_act": (66.1 + 128.3 + 131.2 + 192.6) * MIB},
+    "c3": {"gemm": (897.9 + 897.3 + 832.8) / 3.0 * MIB, "norm_act": 1047.0 * MIB},
+    "c2": {"norm_act": 528.8 * MIB},
 }
 
 
