@@ -39,6 +39,7 @@ C_ABI_SYMBOLS = [
     "dlmi_norm_fwd_train", "dlmi_norm_fwd_infer", "dlmi_norm_bwd", "dlmi_act_fwd", "dlmi_act_bwd",
     "dlmi_softmax_fwd", "dlmi_dropout_fwd", "dlmi_identity_add", "dlmi_softmax_ce_seed",
     "dlmi_fused_norm_act_fwd", "dlmi_fused_norm_act_bwd", "dlmi_fused_norm_act_infer", "dlmi_fc_norm_act_fwd",
+    "dlmi_opt_gd", "dlmi_opt_gd_momentum", "dlmi_opt_adam",
 ]
 
 
@@ -230,6 +231,21 @@ class Dlmi:
         o = out if out is not None else self.torch.empty_like(a)
         self._ck(self.lib.dlmi_identity_add(self.ctx, c_sz(a.numel()), _p(a), _p(b), _p(o)))
         return o
+
+    # optimizer steps: every tensor argument is updated in place, grads end up zero
+    def opt_gd(self, p, g, mask, lr, wd, nthreads=0):
+        self._chk(p, g, mask)
+        self._ck(self.lib.dlmi_opt_gd(self.ctx, c_sz(p.numel()), _p(p), _p(g), _p(mask), c_f(lr), c_f(wd)))
+
+    def opt_gd_momentum(self, p, g, delta_prev, mask, lr, mom, wd, nesterov, nthreads=0):
+        self._chk(p, g, delta_prev, mask)
+        self._ck(self.lib.dlmi_opt_gd_momentum(self.ctx, c_sz(p.numel()), _p(p), _p(g), _p(delta_prev), _p(mask),
+                                               c_f(lr), c_f(mom), c_f(wd), c_int(1 if nesterov else 0)))
+
+    def opt_adam(self, p, g, m1, m2, vhat, mask, lr_t, beta1, beta2, eps, wd, nthreads=0):
+        self._chk(p, g, m1, m2, vhat, mask)
+        self._ck(self.lib.dlmi_opt_adam(self.ctx, c_sz(p.numel()), _p(p), _p(g), _p(m1), _p(m2), _p(vhat), _p(mask),
+                                        c_f(lr_t), c_f(beta1), c_f(beta2), c_f(eps), c_f(wd)))
 
     def softmax_ce_seed(self, q, y, stats=None):
         """stats: optional device tensor of 2 float64 accumulators."""

@@ -228,6 +228,36 @@ int dlmi_fused_norm_act_infer(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t
                               float const *x, float const *gamma, float const *beta,
                               float const *mov_mean, float const *mov_std, float *y);
 
+/* ---- optimizer steps over n packed parameters (the caller-side neighbour of
+ * the path: Model::Update_Parameter, v1/learner/model.cpp:4703-4866) ----------
+ * All arrays are device memory of n floats and are updated in place; every
+ * call zeroes `grads` like the reference's loops do.  `mask` is the
+ * regularization mask (1 for weights, 0 for biases and normalization
+ * parameters: allocate.cpp:1178-1196, indexing.cpp:59-85); it is read only
+ * when wd != 0 and may be NULL otherwise.  The host-side scalars (time step,
+ * bias-corrected step size, normalized weight decay) are the caller's. */
+
+/* p -= lr*g + mask*wd*p.  Replaces Update_Parameter__Gradient_Descent__{Loop,OpenMP}
+ * (v1/optimizers/gradient_descent.cpp:57-131). */
+int dlmi_opt_gd(dlmi_ctx *ctx, size_t n, float *params, float *grads, float const *mask, float lr,
+                float wd);
+
+/* delta = lr*g + momentum*delta_prev; delta_prev = delta;
+ * nesterov == 0: p -= delta + mask*wd*p          (gradient_descent_momentum.cpp:23-107)
+ * nesterov != 0: p -= momentum*delta - lr*g + mask*wd*p, the reference's sign
+ *                (nesterov_accelerated_gradient.cpp:23-107). */
+int dlmi_opt_gd_momentum(dlmi_ctx *ctx, size_t n, float *params, float *grads, float *delta_prev,
+                         float const *mask, float lr, float momentum, float wd, int nesterov);
+
+/* m1 = beta1*m1 + (1-beta1)*g; m2 = beta2*m2 + (1-beta2)*g*g;
+ * p -= lr_t*m1/(sqrt(m2)+eps) + mask*wd*p, with lr_t the step size after the
+ * optional bias correction lr*sqrt(1-beta2^t)/(1-beta1^t) (adam.cpp:33-166).
+ * m2_hat != NULL selects AMSGrad: m2_hat = max(m2_hat, m2) replaces m2 in the
+ * denominator (amsgrad.cpp:34-192). */
+int dlmi_opt_adam(dlmi_ctx *ctx, size_t n, float *params, float *grads, float *m1, float *m2,
+                  float *m2_hat, float const *mask, float lr_t, float beta1, float beta2, float eps,
+                  float wd);
+
 #ifdef __cplusplus
 }
 #endif

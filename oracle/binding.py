@@ -33,6 +33,8 @@ ACT = dict(ELU=3, ISRLU=10, LINEAR=11, LEAKY_RELU=14, RELU=16, SELU=17, SOFTMAX=
 NORM = dict(NONE=0, BN=1, BRN=2)
 DROP = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3)
 STATE = dict(INFERENCE=0, TRAINING=1, UPDATE_BATCH_NORM=2)
+# v1/data/enum/optimizer.hpp:24-42
+OPT = dict(NONE=0, ADAM=2, AMSGRAD=5, GD=6)
 
 
 def build_oracle():
@@ -41,6 +43,54 @@ def build_oracle():
 
 def _ptr(a):
     return None if a is None else a.ctypes.data_as(vp)
+
+
+class OptimizerHost:
+    """The host arithmetic around an optimizer leaf, in float like the reference:
+    time step, bias-corrected step size (adam.cpp:50-54), normalized weight decay
+    (train.cpp:278-283; GD scales wd by lr_scale = 1 without warm restarts,
+    gradient_descent.cpp:72-75).  `leaves` is anything with opt_gd /
+    opt_gd_momentum / opt_adam updating float32 arrays in place."""
+
+    def __init__(self, leaves, n, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9,
+                 beta2=0.999, eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True, mask=None):
+        f = np.float32
+        self.leaves, self.n, self.kind = leaves, n, kind
+        self.lr, self.momentum, self.nesterov = f(lr), f(momentum), bool(nesterov)
+        self.adam_lr, self.beta1, self.beta2, self.eps = f(adam_lr), f(beta1), f(beta2), f(eps)
+        self.bias_correction, self.weight_decay, self.normalized_wd = bool(bias_correction), f(weight_decay), bool(normalized_wd)
+        self.mask = None if mask is None else np.ascontiguousarray(mask, np.float32)
+        self.t = f(0)
+        self.epoch_time_step = f(1)
+        self.delta = np.zeros(n, np.float32) if kind == OPT["GD"] and self.momentum != 0 else None
+        self.m1 = np.zeros(n, np.float32) if kind in (OPT["ADAM"], OPT["AMSGRAD"]) else None
+        self.m2 = np.zeros(n, np.float32) if kind in (OPT["ADAM"], OPT["AMSGRAD"]) else None
+        self.vhat = np.zeros(n, np.float32) if kind == OPT["AMSGRAD"] else None
+
+    def wd(self, batch, training_size):
+        f = np.float32
+        if self.normalized_wd:
+            return f(self.weight_decay * np.sqrt(f(f(batch) / f(f(training_size) * self.epoch_time_step))))
+        return self.weight_decay
+
+    def lr_t(self):
+        f = np.float32
+        if not self.bias_correction:
+            return self.adam_lr
+        return f(f(self.adam_lr * np.sqrt(f(f(1) - np.power(self.beta2, self.t)))) / f(f(1) - np.power(self.beta1, self.t)))
+
+    def update(self, p, g, batch, training_size, nthreads=0):
+        self.t = np.float32(self.t + np.float32(1))
+        wd = self.wd(batch, training_size)
+        if self.kind == OPT["GD"]:
+            if self.momentum != 0:
+                self.leaves.opt_gd_momentum(p, g, self.delta, self.mask, self.lr, self.momentum, wd, self.nesterov,
+                                            nthreads)
+            else:
+                self.leaves.opt_gd(p, g, self.mask, self.lr, wd, nthreads)
+        else:
+            self.leaves.opt_adam(p, g, self.m1, self.m2, self.vhat, self.mask, self.lr_t(), self.beta1, self.beta2,
+                                 self.eps, wd, nthreads)
 
 
 class _Leaves:
@@ -203,6 +253,20 @@ class Oracle(_Leaves):
         fn = getattr(self.lib, "dlo_" + leaf + self.suffix)
         fn.restype = None
         return fn
+
+    # ---- optimizer leaves: all update their array arguments IN PLACE ----------
+    def opt_gd(self, p, g, mask, lr, wd, nthreads=0):
+        self._f("opt_gd")(c_int(nthreads), c_sz(p.size), _ptr(p), _ptr(g), _ptr(mask), self._real(lr),
+                          self._real(wd))
+
+    def opt_gd_momentum(self, p, g, delta_prev, mask, lr, mom, wd, nesterov, nthreads=0):
+        self._f("opt_gd_momentum")(c_int(nthreads), c_sz(p.size), _ptr(p), _ptr(g), _ptr(delta_prev), _ptr(mask),
+                                   self._real(lr), self._real(mom), self._real(wd), c_int(1 if nesterov else 0))
+
+    def opt_adam(self, p, g, m1, m2, vhat, mask, lr_t, beta1, beta2, eps, wd, nthreads=0):
+        self._f("opt_adam")(c_int(nthreads), c_sz(p.size), _ptr(p), _ptr(g), _ptr(m1), _ptr(m2), _ptr(vhat),
+                            _ptr(mask), self._real(lr_t), self._real(beta1), self._real(beta2), self._real(eps),
+                            self._real(wd))
 
     def dropout_fwd(self, kind, v, mask, scale_or_keep, nthreads=0):
         """kind 0 inverted, 1 plain, 2 inference.  mask [H] (reference semantics,
@@ -469,3 +533,30 @@ class ReferenceMLP:
         p = np.empty(self.P, np.float32)
         self.lib.dlref_model_get_dparams(self.h, _ptr(p), c_sz(self.P))
         return p
+
+    # ---- optimizer (Model::Update_Parameter) ---------------------------------
+    def set_optimizer(self, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9, beta2=0.999,
+                      eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True):
+        ok = self.lib.dlref_model_set_optimizer(self.h, c_int(kind), c_f(lr), c_f(momentum), c_int(int(nesterov)),
+                                                c_f(adam_lr), c_f(beta1), c_f(beta2), c_f(eps),
+                                                c_int(int(bias_correction)), c_f(weight_decay),
+                                                c_int(int(normalized_wd)))
+        assert ok, "reference refused the optimizer settings"
+
+    def set_epoch_time_step(self, v):
+        self.lib.dlref_model_set_epoch_time_step(self.h, c_f(v))
+
+    def set_dparams(self, g):
+        g = np.ascontiguousarray(g, np.float32)
+        assert g.size == self.P
+        self.lib.dlref_model_set_dparams(self.h, _ptr(g), c_sz(self.P))
+
+    def update_parameter(self, batch, training_size):
+        self.lib.dlref_model_update_parameter(self.h, c_sz(batch), c_sz(training_size))
+
+    def opt_state(self, which):
+        """which: 0 previous delta, 1 first moment, 2 second moment, 3 second moment hat, 4 regularization mask;
+        None when the reference has not allocated it."""
+        out = np.empty(self.P, np.float32)
+        ok = self.lib.dlref_model_get_opt_state(self.h, c_int(which), _ptr(out), c_sz(self.P))
+        return out if ok else None

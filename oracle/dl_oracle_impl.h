@@ -262,6 +262,69 @@ void FN(dlo_identity_add)(int nthreads, size_t B, size_t H, REAL const *a,
   }
 }
 
+/* ---- optimizer steps over parameters [str, end) of the packed arrays ---------
+ * mask: the regularization mask (1 weights, 0 biases / gamma / beta:
+ * allocate.cpp:1178-1196, indexing.cpp:59-85), read only when wd != 0.
+ * Every variant zeroes the gradient it consumed.  The OpenMP variants of the
+ * reference are the same loops under `omp parallel for schedule(static)`. */
+
+/* plain gradient descent: gradient_descent.cpp:57-92 (wd already scaled by the caller) */
+void FN(dlo_opt_gd)(int nthreads, size_t n, REAL *p, REAL *g, REAL const *mask, REAL lr, REAL wd) {
+  int const N = nthreads, ni = (int)n;
+  int i;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (i = 0; i < ni; ++i) {
+    if (wd != (REAL)0) p[i] -= lr * g[i] + mask[i] * wd * p[i];
+    else p[i] -= lr * g[i];
+    g[i] = (REAL)0;
+  }
+}
+
+/* momentum: gradient_descent_momentum.cpp:23-63; Nesterov:
+ * nesterov_accelerated_gradient.cpp:23-63 (note its sign: the parameter moves by
+ * -(mom*delta - lr*g)) */
+void FN(dlo_opt_gd_momentum)(int nthreads, size_t n, REAL *p, REAL *g, REAL *delta_prev, REAL const *mask, REAL lr,
+                             REAL mom, REAL wd, int nesterov) {
+  int const N = nthreads, ni = (int)n;
+  int i;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (i = 0; i < ni; ++i) {
+    REAL const delta = lr * g[i] + mom * delta_prev[i];
+    delta_prev[i] = delta;
+    if (nesterov) {
+      if (wd != (REAL)0) p[i] -= mom * delta - lr * g[i] + mask[i] * wd * p[i];
+      else p[i] -= mom * delta - lr * g[i];
+    } else {
+      if (wd != (REAL)0) p[i] -= delta + mask[i] * wd * p[i];
+      else p[i] -= delta;
+    }
+    g[i] = (REAL)0;
+  }
+}
+
+/* Adam: adam.cpp:33-97; AMSGrad (vhat != NULL): amsgrad.cpp:34-117.  lr_t is the
+ * bias-corrected step size the reference computes once per call (adam.cpp:50-54). */
+void FN(dlo_opt_adam)(int nthreads, size_t n, REAL *p, REAL *g, REAL *m1, REAL *m2, REAL *vhat, REAL const *mask,
+                      REAL lr_t, REAL beta1, REAL beta2, REAL eps, REAL wd) {
+  int const N = nthreads, ni = (int)n;
+  int i;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (i = 0; i < ni; ++i) {
+    REAL const d = g[i];
+    REAL const a = beta1 * m1[i] + ((REAL)1 - beta1) * d;
+    REAL v = beta2 * m2[i] + ((REAL)1 - beta2) * d * d;
+    m1[i] = a;
+    m2[i] = v;
+    if (vhat != NULL) {
+      v = vhat[i] > v ? vhat[i] : v;
+      vhat[i] = v;
+    }
+    if (wd != (REAL)0) p[i] -= lr_t * a / (SQRT(v) + eps) + mask[i] * wd * p[i];
+    else p[i] -= lr_t * a / (SQRT(v) + eps);
+    g[i] = (REAL)0;
+  }
+}
+
 /* ---- a18  dY += dZn * Wn: bwp_st.cpp:1009-1045, bwp_mp.cpp:968-1007 ------- */
 void FN(dlo_fc_bwd_dx)(int nthreads, size_t B, size_t Hn, size_t H,
                        REAL const *dZn, REAL const *Wn, REAL *dY) {

@@ -571,4 +571,56 @@ int dlref_model_get_layer_vector(void *h, size_t layer, int which, float *out) {
   return 1;
 }
 
+// ---- optimizer step (drivers/driver.cpp:265 -> Model::Update_Parameter,
+// model.cpp:4703-4866).  All hyper-parameters are public members; they are set
+// before set_optimizer so that the state arrays get allocated (allocate.cpp:1052-1146).
+int dlref_model_set_optimizer(void *h, int type, float lr, float momentum, int nesterov, float adam_lr,
+                              float beta1, float beta2, float eps, int bias_correction, float weight_decay,
+                              int normalized_wd) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  m.learning_rate = lr;
+  m.learning_momentum = momentum;
+  m.use_nesterov = nesterov != 0;
+  m.adam_learning_rate = adam_lr;
+  m.adam_beta1 = beta1;
+  m.adam_beta2 = beta2;
+  m.adam_epsilon = eps;
+  m.use_adam_bias_correction = bias_correction != 0;
+  m.use_normalized_weight_decay = normalized_wd != 0;
+  m.use_warm_restarts = false;
+  m.optimizer_time_step = 0.0f;
+  m.epoch_time_step = 1.0f;
+  m.set_optimizer(static_cast<OPTIMIZER::TYPE>(type));
+  if (!m.set_weight_decay(weight_decay)) return 0;
+  return 1;
+}
+void dlref_model_set_epoch_time_step(void *h, float v) { static_cast<RefModel *>(h)->model.epoch_time_step = v; }
+float dlref_model_opt_time_step(void *h) { return static_cast<RefModel *>(h)->model.optimizer_time_step; }
+void dlref_model_set_dparams(void *h, float const *p, size_t n) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  std::memcpy(m.ptr_array_derivatives_parameters, p, n * sizeof(float));
+}
+void dlref_model_update_parameter(void *h, size_t batch, size_t training_size) {
+  RefModel *rm = static_cast<RefModel *>(h);
+  if (rm->nthreads > 0) omp_set_num_threads(static_cast<int>(rm->model.number_threads));
+  rm->model.Update_Parameter(batch, training_size);
+}
+// which: 0 previous delta (momentum), 1 first moment, 2 second moment,
+// 3 second moment hat (AMSGrad), 4 regularization mask
+int dlref_model_get_opt_state(void *h, int which, float *out, size_t n) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  float const *src = nullptr;
+  switch (which) {
+    case 0: src = m.ptr_array_previous_delta_parameters; break;
+    case 1: src = m.ptr_array_previous_biased_first_moment; break;
+    case 2: src = m.ptr_array_previous_biased_second_moment; break;
+    case 3: src = m.ptr_array_previous_biased_second_moment_hat; break;
+    case 4: src = m.ptr_array_mask_regularized_parameters; break;
+    default: return 0;
+  }
+  if (src == nullptr) return 0;
+  std::memcpy(out, src, n * sizeof(float));
+  return 1;
+}
+
 }  // extern "C"

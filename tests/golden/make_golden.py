@@ -9,6 +9,7 @@ The fixtures are data only: inputs and the reference's outputs (npz, float32 /
 uint8 arrays, loaded with allow_pickle=False).  Every value in an "exp_*" array
 was produced by a member function of the reference's DL::v1::Model.
 """
+import json
 import os
 import sys
 
@@ -16,7 +17,7 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 sys.path.insert(0, ROOT)
-from oracle.binding import ACT, DROP, NORM, STATE, Reference  # noqa: E402
+from oracle.binding import ACT, DROP, NORM, OPT, STATE, Reference  # noqa: E402
 
 OUT = os.path.dirname(os.path.abspath(__file__))
 ACTS = ["ELU", "ISRLU", "LEAKY_RELU", "RELU", "SELU", "LINEAR"]
@@ -187,7 +188,102 @@ def mlps(R):
     return len(d)
 
 
+OPT_CASES = {
+    # name: (optimizer, keyword settings of ReferenceMLP.set_optimizer)
+    "gd_plain": ("GD", dict(lr=0.05, momentum=0.0)),
+    "gd_wd": ("GD", dict(lr=0.05, momentum=0.0, weight_decay=0.02, normalized_wd=False)),
+    "gd_momentum": ("GD", dict(lr=0.02, momentum=0.9)),
+    "gd_momentum_wd_norm": ("GD", dict(lr=0.02, momentum=0.8, weight_decay=0.05, normalized_wd=True)),
+    "gd_nesterov": ("GD", dict(lr=0.02, momentum=0.9, nesterov=True)),
+    "adam": ("ADAM", dict(adam_lr=0.001)),
+    "adam_nobias_wd": ("ADAM", dict(adam_lr=0.01, beta1=0.8, beta2=0.99, eps=1e-6, bias_correction=False,
+                                    weight_decay=0.03, normalized_wd=True)),
+    "amsgrad": ("AMSGRAD", dict(adam_lr=0.005, beta1=0.7, beta2=0.9)),
+    "amsgrad_wd": ("AMSGRAD", dict(adam_lr=0.005, weight_decay=0.01, normalized_wd=False)),
+}
+OPT_STEPS = 4
+OPT_BATCH, OPT_TRAINING_SIZE = 5, 60
+
+
+def small_brn_model(R, widths, B, nt):
+    M = R.mlp(widths)
+    for l in range(1, len(widths) - 1):
+        M.set_layer(l, ACT["RELU"], NORM["BRN"])
+    M.set_layer(len(widths) - 1, ACT["SOFTMAX"])
+    M.set_norm_hyper(0.99, 1e-5, 3.0, 5.0)
+    M.prepare(B, nt)
+    return M
+
+
+def optimizers(R):
+    """(a) Model::Update_Parameter on given gradients, OPT_STEPS times in a row;
+    (b) whole training steps (forward, error, backward, derivatives, update) on
+    one batch with Adam and with momentum + weight decay."""
+    d = {}
+    widths = [8, 6, 6, 3]
+    rng = np.random.default_rng(77)
+    M0 = small_brn_model(R, widths, OPT_BATCH, 0)
+    P = M0.P
+    p0 = f32(rng.standard_normal(P))
+    grads = f32(rng.standard_normal((OPT_STEPS, P)))
+    grads[1, ::7] = 0  # zero gradients: second moments stay where they are
+    d["opt_p0"], d["opt_grads"] = p0, grads
+    d["opt_sizes"] = np.array([OPT_BATCH, OPT_TRAINING_SIZE])
+    # the settings travel with the vectors (JSON text as bytes)
+    traj = {"traj_adam": ("ADAM", dict(adam_lr=0.01)),
+            "traj_momentum_wd": ("GD", dict(lr=0.1, momentum=0.9, weight_decay=0.01, normalized_wd=True))}
+    d["opt_cases_json"] = np.frombuffer(json.dumps({"leaf": OPT_CASES, "traj": traj}).encode(), dtype=np.uint8)
+    for name, (kind, kw) in OPT_CASES.items():
+        for nt in THREADS:
+            M = small_brn_model(R, widths, OPT_BATCH, nt)
+            M.set_parameters(p0)
+            M.set_optimizer(OPT[kind], **kw)
+            if nt == 0:
+                mask = M.opt_state(4)
+                d[f"opt_{name}_mask"] = mask if mask is not None else np.zeros(0, np.float32)
+            for t in range(OPT_STEPS):
+                M.set_dparams(grads[t])
+                M.update_parameter(OPT_BATCH, OPT_TRAINING_SIZE)
+                q = f"opt_{name}_t{nt}_s{t}_"
+                d[q + "params"] = M.get_parameters()
+                assert not M.get_dparams().any(), "the reference zeroes the consumed gradient"
+                for which, wn in ((0, "delta"), (1, "m1"), (2, "m2"), (3, "vhat")):
+                    st = M.opt_state(which)
+                    if st is not None and t == OPT_STEPS - 1:
+                        d[q + wn] = st
+    # (b) training trajectories
+    for name, (kind, kw) in traj.items():
+        widths, B = [20, 16, 16, 10], 12
+        rng = np.random.default_rng(sum(map(ord, name)))
+        X = f32(rng.uniform(0, 1, (B, widths[0])))
+        Y = f32(np.eye(widths[-1])[rng.integers(0, widths[-1], B)])
+        d[name + "_X"], d[name + "_Y"], d[name + "_widths"] = X, Y, np.array(widths)
+        params = None
+        for nt in THREADS:
+            M = small_brn_model(R, widths, B, nt)
+            if params is None:
+                params = M.get_parameters()
+                for l in range(1, len(widths)):
+                    o = M.layer_offsets(l)
+                    K, H = widths[l - 1], widths[l]
+                    params[o[0]:o[0] + H * K] = glorot(rng, H, K).ravel()
+                d[name + "_params"] = params.copy()
+            M.set_parameters(params)
+            M.set_optimizer(OPT[kind], **kw)
+            for t in range(3):
+                M.step(STATE["TRAINING"], X, Y, backward=True)
+                if t == 0:
+                    d[f"{name}_t{nt}_s0_dparams"] = M.get_dparams()
+                M.update_parameter(B, 5 * B)
+                d[f"{name}_t{nt}_s{t}_params"] = M.get_parameters()
+            mm, ms = M.get_moving()
+            d[f"{name}_t{nt}_mov_mean"], d[f"{name}_t{nt}_mov_std"] = mm, ms
+    np.savez_compressed(os.path.join(OUT, "optim.npz"), **d)
+    return len(d)
+
+
 if __name__ == "__main__":
     R = Reference()
     print("leaves:", leaves(R), "arrays")
     print("mlp:", mlps(R), "arrays")
+    print("optim:", optimizers(R), "arrays")

@@ -1,0 +1,110 @@
+"""dlmi_opt_* through the C ABI: against the golden vectors of the compiled
+reference (tests/golden/optim.npz), and against the oracle on larger, ragged
+and unaligned arrays."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import RTOL_ELEMENTWISE as TE
+from helpers import assert_close
+from oracle.binding import OPT, OptimizerHost
+from test_oracle_optimizers import leaf_case_names, run_leaf_case
+
+pytestmark = pytest.mark.gpu
+
+
+class GpuLeaves:
+    """opt_gd / opt_gd_momentum / opt_adam on numpy arrays, in place, computed on
+    the GPU: every array goes to the device, through the C ABI and back."""
+
+    def __init__(self, dl):
+        self.dl = dl
+
+    def _run(self, fn, arrays, *scalars):
+        dev = [None if a is None else torch.from_numpy(a).cuda() for a in arrays]
+        fn(*dev, *scalars)
+        torch.cuda.synchronize()
+        for a, d in zip(arrays, dev):
+            if a is not None:
+                a[...] = d.cpu().numpy()
+
+    def opt_gd(self, p, g, mask, lr, wd, nthreads=0):
+        self._run(self.dl.opt_gd, [p, g, mask], float(lr), float(wd))
+
+    def opt_gd_momentum(self, p, g, delta, mask, lr, mom, wd, nesterov, nthreads=0):
+        self._run(self.dl.opt_gd_momentum, [p, g, delta, mask], float(lr), float(mom), float(wd), nesterov)
+
+    def opt_adam(self, p, g, m1, m2, vhat, mask, lr_t, b1, b2, eps, wd, nthreads=0):
+        self._run(self.dl.opt_adam, [p, g, m1, m2, vhat, mask], float(lr_t), float(b1), float(b2), float(eps),
+                  float(wd))
+
+
+@pytest.fixture(scope="module")
+def golden_optim():
+    import os
+    from conftest import ROOT
+    return np.load(os.path.join(ROOT, "tests", "golden", "optim.npz"), allow_pickle=False)
+
+
+@pytest.mark.parametrize("name", leaf_case_names())
+def test_gpu_optimizer_against_golden(dl, golden_optim, name):
+    g = golden_optim
+    for t, p, host in run_leaf_case(GpuLeaves(dl), g, name, 0):
+        assert_close(p, g[f"opt_{name}_t0_s{t}_params"], TE, f"{name} parameters after step {t}")
+    q = f"opt_{name}_t0_s{len(g['opt_grads']) - 1}_"
+    for key, arr in (("delta", host.delta), ("m1", host.m1), ("m2", host.m2), ("vhat", host.vhat)):
+        if q + key in g.files:
+            assert_close(arr, g[q + key], TE, f"{name} {key}")
+
+
+@pytest.mark.parametrize("n", [1, 3, 4, 1000, 4099, 1 << 20])
+@pytest.mark.parametrize("kind,kw", [
+    ("GD", dict(lr=0.05, momentum=0.0, weight_decay=0.1, normalized_wd=False)),
+    ("GD", dict(lr=0.05, momentum=0.9)),
+    ("GD", dict(lr=0.05, momentum=0.9, nesterov=True, weight_decay=0.1, normalized_wd=True)),
+    ("ADAM", dict(adam_lr=0.01, weight_decay=0.05)),
+    ("AMSGRAD", dict(adam_lr=0.01, beta2=0.9)),
+])
+def test_gpu_optimizer_against_oracle(dl, oracle, n, kind, kw):
+    rng = np.random.default_rng(n + len(kind))
+    p0 = rng.standard_normal(n).astype(np.float32)
+    mask = (rng.uniform(size=n) < 0.7).astype(np.float32)
+    ho = OptimizerHost(oracle, n, OPT[kind], mask=mask, **kw)
+    hg = OptimizerHost(GpuLeaves(dl), n, OPT[kind], mask=mask, **kw)
+    po, pg = p0.copy(), p0.copy()
+    for _ in range(3):
+        g = rng.standard_normal(n).astype(np.float32)
+        go, gg = g.copy(), g.copy()
+        ho.update(po, go, 32, 4096)
+        hg.update(pg, gg, 32, 4096)
+        assert not gg.any(), "gradient zeroed"
+        assert_close(pg, po, TE, "parameters")
+    for a, b, what in ((hg.delta, ho.delta, "delta"), (hg.m1, ho.m1, "m1"), (hg.m2, ho.m2, "m2"),
+                       (hg.vhat, ho.vhat, "vhat")):
+        if b is not None:
+            assert_close(a, b, TE, what)
+
+
+def test_gpu_optimizer_on_unaligned_views(dl, oracle):
+    """A parameter range that does not start on a 16-byte boundary (str/end of the
+    reference's Update_Parameters__*(…, str, end)) takes the scalar path."""
+    n = 1001
+    rng = np.random.default_rng(9)
+    base = [torch.from_numpy(rng.standard_normal(n + 1).astype(np.float32)).cuda() for _ in range(4)]
+    first = [float(b[0]) for b in base]
+    p, g, m1, m2 = (b[1:] for b in base)
+    po, go, m1o, m2o = (t.cpu().numpy().copy() for t in (p, g, m1, m2))
+    m1o, m2o = np.abs(m1o), np.abs(m2o)
+    m1.copy_(torch.from_numpy(m1o)); m2.copy_(torch.from_numpy(m2o))
+    dl.opt_adam(p, g, m1, m2, None, None, 0.01, 0.9, 0.999, 1e-8, 0.0)
+    oracle.opt_adam(po, go, m1o, m2o, None, None, 0.01, 0.9, 0.999, 1e-8, 0.0)
+    assert_close(p.cpu().numpy(), po, TE, "parameters")
+    assert_close(m2.cpu().numpy(), m2o, TE, "m2")
+    assert not g.cpu().numpy().any()
+    assert first == [float(b[0]) for b in base], "the element before the range is untouched"
+
+
+def test_weight_decay_without_mask_is_refused(dl):
+    p = torch.zeros(8, device="cuda")
+    with pytest.raises(RuntimeError):
+        dl.opt_gd(p, p.clone(), None, 0.1, 0.5)

@@ -1,0 +1,196 @@
+"""Optimizer steps of the oracle: against the golden vectors the compiled
+reference wrote (tests/golden/optim.npz), against closed forms and torch's
+library optimizers, and against the compiled reference on fresh random cases."""
+import json
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import RTOL_RESTATEMENT, assert_close
+from oracle.binding import ACT, NORM, OPT, OptimizerHost
+
+T = 4 * RTOL_RESTATEMENT
+
+
+@pytest.fixture(scope="session")
+def golden_optim():
+    import os
+    from conftest import ROOT
+    return np.load(os.path.join(ROOT, "tests", "golden", "optim.npz"), allow_pickle=False)
+
+
+def cases(g, which):
+    return json.loads(bytes(g["opt_cases_json"]))[which]
+
+
+def leaf_case_names():
+    import os
+    from conftest import ROOT
+    g = np.load(os.path.join(ROOT, "tests", "golden", "optim.npz"), allow_pickle=False)
+    return list(json.loads(bytes(g["opt_cases_json"]))["leaf"])
+
+
+def run_leaf_case(leaves, g, name, nt):
+    """Replays one golden optimizer case on `leaves`; yields (step, params, host)."""
+    kind, kw = cases(g, "leaf")[name]
+    mask = g[f"opt_{name}_mask"]
+    p = g["opt_p0"].copy()
+    host = OptimizerHost(leaves, p.size, OPT[kind], mask=mask if mask.size else None, **kw)
+    B, N = (int(v) for v in g["opt_sizes"])
+    for t, grad in enumerate(g["opt_grads"]):
+        gg = grad.copy()
+        host.update(p, gg, B, N, nt)
+        assert not gg.any(), "the step zeroes the gradient it consumed"
+        yield t, p, host
+
+
+@pytest.mark.parametrize("nt", [0, 3])
+@pytest.mark.parametrize("name", leaf_case_names())
+def test_oracle_optimizer_against_golden(oracle, golden_optim, name, nt):
+    g = golden_optim
+    for t, p, host in run_leaf_case(oracle, g, name, nt):
+        assert_close(p, g[f"opt_{name}_t{nt}_s{t}_params"], T, f"{name} parameters after step {t}")
+    q = f"opt_{name}_t{nt}_s{len(g['opt_grads']) - 1}_"
+    for key, arr in (("delta", host.delta), ("m1", host.m1), ("m2", host.m2), ("vhat", host.vhat)):
+        if q + key in g.files:
+            assert arr is not None, key
+            assert_close(arr, g[q + key], T, f"{name} {key}")
+        else:
+            assert arr is None, f"the reference allocates no {key} for {name}"
+
+
+def test_regularization_mask_covers_exactly_the_weights(golden_optim):
+    """8-6-6-3 network: 102 weights first, then biases and gamma / beta."""
+    m = golden_optim["opt_gd_wd_mask"]
+    assert m.size == 163 and m[:102].all() and not m[102:].any()
+    assert golden_optim["opt_gd_plain_mask"].size == 0  # no weight decay: the reference allocates none
+
+
+# ---- what the mathematics fixes ------------------------------------------------
+def test_gd_closed_form(oracle64):
+    rng = np.random.default_rng(1)
+    p0, g = rng.standard_normal(50), rng.standard_normal(50)
+    mask = (np.arange(50) < 30).astype(np.float64)
+    p, gg = p0.copy(), g.copy()
+    oracle64.opt_gd(p, gg, mask, 0.1, 0.0)
+    np.testing.assert_allclose(p, p0 - 0.1 * g, rtol=1e-14)
+    assert not gg.any()
+    p, gg = p0.copy(), g.copy()
+    oracle64.opt_gd(p, gg, mask, 0.1, 0.25)
+    np.testing.assert_allclose(p, p0 - (0.1 * g + mask * 0.25 * p0), rtol=1e-14)
+    np.testing.assert_allclose(p[30:], (p0 - 0.1 * g)[30:], rtol=1e-14)  # unmasked entries do not decay
+
+
+def test_momentum_matches_torch_sgd(oracle64):
+    """lr*g + mom*delta with constant lr is torch.optim.SGD's momentum buffer times lr."""
+    rng = np.random.default_rng(2)
+    p0 = rng.standard_normal(40)
+    grads = rng.standard_normal((5, 40))
+    tp = torch.tensor(p0.copy(), requires_grad=True)
+    opt = torch.optim.SGD([tp], lr=0.05, momentum=0.9)
+    p, delta = p0.copy(), np.zeros(40)
+    for gr in grads:
+        tp.grad = torch.tensor(gr.copy())
+        opt.step()
+        gg = gr.copy()
+        oracle64.opt_gd_momentum(p, gg, delta, None, 0.05, 0.9, 0.0, False)
+        np.testing.assert_allclose(p, tp.detach().numpy(), rtol=1e-12, atol=1e-14)
+
+
+def test_nesterov_variant_closed_form(oracle64):
+    """The reference moves the parameter by -(mom*delta - lr*g): two steps by hand."""
+    p0, lr, mom = np.array([1.0, -2.0]), 0.1, 0.5
+    g1, g2 = np.array([0.3, -0.7]), np.array([-1.1, 0.4])
+    p, delta = p0.copy(), np.zeros(2)
+    oracle64.opt_gd_momentum(p, g1.copy(), delta, None, lr, mom, 0.0, True)
+    d1 = lr * g1
+    e1 = p0 - (mom * d1 - lr * g1)
+    np.testing.assert_allclose(p, e1, rtol=1e-14)
+    oracle64.opt_gd_momentum(p, g2.copy(), delta, None, lr, mom, 0.0, True)
+    d2 = lr * g2 + mom * d1
+    np.testing.assert_allclose(delta, d2, rtol=1e-14)
+    np.testing.assert_allclose(p, e1 - (mom * d2 - lr * g2), rtol=1e-14)
+
+
+def test_adam_first_step_is_sign_of_gradient(oracle64):
+    """With bias correction the first step is lr * g / (|g| + eps/sqrt(1-beta2)) ~ lr * sign(g)."""
+    rng = np.random.default_rng(3)
+    g = rng.standard_normal(64)
+    p = np.zeros(64)
+    host = OptimizerHost(oracle64, 64, OPT["ADAM"], adam_lr=0.01, eps=1e-8)
+    host.m1, host.m2 = np.zeros(64), np.zeros(64)
+    oracle64.opt_adam(p, g.copy(), host.m1, host.m2, None, None, 0.01 * np.sqrt(1 - 0.999) / (1 - 0.9), 0.9, 0.999,
+                      1e-8, 0.0)
+    np.testing.assert_allclose(p, -0.01 * g / (np.abs(g) + 1e-8 / np.sqrt(1 - 0.999)), rtol=1e-10)
+    big = np.abs(g) > 0.1
+    np.testing.assert_allclose(p[big], -0.01 * np.sign(g[big]), rtol=1e-5)
+    np.testing.assert_allclose(host.m1, 0.1 * g, rtol=1e-12)
+    np.testing.assert_allclose(host.m2, 0.001 * g * g, rtol=1e-12)
+
+
+def test_adam_matches_torch_adam_when_eps_vanishes(oracle64):
+    """torch puts eps next to sqrt(v_hat), the reference next to sqrt(v): identical as eps -> 0."""
+    rng = np.random.default_rng(4)
+    p0 = rng.standard_normal(30)
+    grads = rng.standard_normal((6, 30)) + 0.1
+    tp = torch.tensor(p0.copy(), requires_grad=True)
+    opt = torch.optim.Adam([tp], lr=0.003, betas=(0.8, 0.95), eps=1e-30)
+    p, m1, m2 = p0.copy(), np.zeros(30), np.zeros(30)
+    for t, gr in enumerate(grads, 1):
+        tp.grad = torch.tensor(gr.copy())
+        opt.step()
+        lr_t = 0.003 * np.sqrt(1 - 0.95 ** t) / (1 - 0.8 ** t)
+        oracle64.opt_adam(p, gr.copy(), m1, m2, None, None, lr_t, 0.8, 0.95, 1e-30, 0.0)
+        np.testing.assert_allclose(p, tp.detach().numpy(), rtol=1e-10)
+
+
+def test_amsgrad_denominator_never_shrinks(oracle64):
+    rng = np.random.default_rng(5)
+    n = 20
+    p, m1, m2, vh = np.zeros(n), np.zeros(n), np.zeros(n), np.zeros(n)
+    prev = vh.copy()
+    for scale in (3.0, 0.1, 2.0, 0.01):
+        oracle64.opt_adam(p, scale * rng.standard_normal(n), m1, m2, vh, None, 0.01, 0.9, 0.5, 1e-8, 0.0)
+        assert (vh >= prev).all() and (vh >= m2).all()
+        prev = vh.copy()
+    assert (vh > m2).any()  # after the small gradients the running maximum is what counts
+
+
+def test_host_scalars(oracle):
+    """Normalized weight decay wd*sqrt(B/(N*epochs)) (train.cpp:278-283) and the
+    bias-corrected step size (adam.cpp:50-54), in float."""
+    h = OptimizerHost(oracle, 4, OPT["ADAM"], adam_lr=0.001, weight_decay=0.04, normalized_wd=True)
+    assert abs(float(h.wd(25, 100)) / (0.04 * 0.5) - 1) < 1e-6
+    h.epoch_time_step = np.float32(4)
+    assert abs(float(h.wd(25, 100)) / (0.04 * 0.25) - 1) < 1e-6
+    h.t = np.float32(1)
+    assert abs(float(h.lr_t()) / (0.001 * np.sqrt(1 - 0.999) / (1 - 0.9)) - 1) < 1e-5
+
+
+# ---- against the compiled reference, fresh cases ----------------------------------
+@pytest.mark.parametrize("seed", range(4))
+def test_oracle_optimizer_against_reference(oracle, reference, seed):
+    rng = np.random.default_rng(300 + seed)
+    widths = [int(rng.integers(3, 12)) for _ in range(4)]
+    nt = int(rng.integers(0, 4))
+    kind = ["GD", "GD", "ADAM", "AMSGRAD"][seed]
+    kw = [dict(lr=0.03, momentum=0.0, weight_decay=0.1, normalized_wd=True),
+          dict(lr=0.03, momentum=0.7, nesterov=bool(seed % 2), weight_decay=0.02, normalized_wd=False),
+          dict(adam_lr=0.02, beta1=0.85, beta2=0.97, eps=1e-7, weight_decay=0.05),
+          dict(adam_lr=0.02, bias_correction=False)][seed]
+    M = reference.mlp(widths)
+    for l in (1, 2):
+        M.set_layer(l, ACT["ELU"], NORM["BRN"])
+    M.set_layer(3, ACT["SOFTMAX"])
+    M.prepare(6, nt)
+    p = rng.standard_normal(M.P).astype(np.float32)
+    M.set_parameters(p)
+    M.set_optimizer(OPT[kind], **kw)
+    host = OptimizerHost(oracle, M.P, OPT[kind], mask=M.opt_state(4), **kw)
+    for _ in range(5):
+        g = rng.standard_normal(M.P).astype(np.float32)
+        M.set_dparams(g)
+        M.update_parameter(6, 48)
+        host.update(p, g.copy(), 6, 48, nt)
+        assert_close(p, M.get_parameters(), T, "parameters")
