@@ -112,6 +112,15 @@ class Step:
         self.dl.fc_norm_act_fwd(self.desc, t["X"], t["W"], t["gamma"], t["beta"], t["mov_mean"], t["mov_std"],
                                 Z=t["Z"], out=t["y"], stats=t["stats"])
 
+    def adam(self):
+        """Adam step over the layer's weights (not part of the timed step: the
+        metric is forward + backward; reported under detail)."""
+        t = self.t
+        if "m1" not in t:
+            import torch
+            t["m1"], t["m2"] = torch.zeros_like(t["W"]), torch.zeros_like(t["W"])
+        self.dl.opt_adam(t["W"], t["dW"], t["m1"], t["m2"], None, None, 1e-6, 0.9, 0.999, 1e-8, 0.0)
+
     def copy(self):
         """A plain device copy of one [B, H] tensor (known size): calibrates the
         FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run."""
@@ -193,7 +202,8 @@ def main():
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-rows", type=int, default=-1, help="rows of the CPU baseline sample (0 = skip)")
     ap.add_argument("--only", default="", help="profiling aid: run just this part (gemm_fwd, gemm_dx, gemm_dw, "
-                                               "norm_fwd, norm_bwd) --steps times and exit without a JSON line")
+                                               "norm_fwd, norm_bwd, fc_norm_fwd, adam, copy) --steps times and exit "
+                                               "without a JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -253,6 +263,11 @@ def main():
                        # forward costs what the fused call takes beyond the plain GEMM and moves 8 B/element
                        "epilogue_fused_norm_fwd": {"ms": t_ff - t_gf, "bytes": 8.0 * E,
                                                    "GBps": 8.0 * E / max(t_ff - t_gf, 1e-6) / 1e6}})
+        # the optimizer step that follows a training step (Adam over the H x K weights: reads and writes
+        # parameter, gradient and both moments = 32 B/parameter), timed last because it consumes dW
+        t_ad = time_events(torch, step.adam, 10)
+        detail["adam_step"] = {"ms": t_ad, "bytes": 32.0 * H * K, "GBps": 32.0 * H * K / t_ad / 1e6,
+                               "frac_hbm_peak": 32.0 * H * K / t_ad / 1e6 / HBM_PEAK_GBS}
     else:
         roof = dict(hbm)
 

@@ -12,9 +12,11 @@
 // input included) | beta(all layers) ],  W_l row-major [H_l][K_l].
 #include <hip/hip_runtime.h>
 
+#include <cmath>
 #include <cstdio>
 #include <cstring>
 #include <string>
+#include <vector>
 
 #include "../../include/dlmi_model.hpp"
 
@@ -30,6 +32,9 @@ struct Model::Impl {
   float *d_input = nullptr;    // [batch, n_in]
   float *d_targets = nullptr;  // [batch, n_out]
   double *d_stats = nullptr;   // { loss sum, correct count }
+  // optimizer state [P] each: 0 previous delta, 1 first moment, 2 second moment,
+  // 3 second moment hat, 4 regularization mask; allocated (zeroed) on first use
+  float *d_opt[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
   float *h_stage = nullptr;    // pinned staging for the row-pointer gather
   size_t h_stage_floats = 0;
   mutable std::vector<float> out_host;  // get_out() cache
@@ -79,6 +84,7 @@ Model::~Model(void) {
   dev_free(impl_->d_mov_mean);
   dev_free(impl_->d_mov_std);
   dev_free(impl_->d_stats);
+  for (float *&s : impl_->d_opt) dev_free(s);
   if (ptr_array_layers != nullptr)
     for (Layer *l = ptr_array_layers; l != ptr_last_layer; ++l) {
       dev_free(l->d_mean); dev_free(l->d_std); dev_free(l->d_r); dev_free(l->d_d); dev_free(l->d_mask);
@@ -320,6 +326,10 @@ bool Model::download_derivatives(void) {
   return hip_ok(hipMemcpy(ptr_array_derivatives_parameters, impl_->d_dparams, total_parameters * sizeof(float),
                           hipMemcpyDeviceToHost), impl_->err, "gradient download");
 }
+bool Model::upload_derivatives(void) {
+  return hip_ok(hipMemcpy(impl_->d_dparams, ptr_array_derivatives_parameters, total_parameters * sizeof(float),
+                          hipMemcpyHostToDevice), impl_->err, "gradient upload");
+}
 bool Model::upload_moving_statistics(void) {
   size_t const n = total_normalized_units * sizeof(float);
   return hip_ok(hipMemcpy(impl_->d_mov_mean, ptr_array_normalized_batch_units_means_averages, n, hipMemcpyHostToDevice),
@@ -527,6 +537,103 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
       return;
     }
   }
+}
+
+// ---------------------------------------------------------------- optimizer step
+namespace {
+// A zero-filled device array of n floats in *p, allocated on first use.
+bool opt_array(float **p, size_t n, hipStream_t stream, std::string &err) {
+  if (*p != nullptr) return true;
+  if (!dev_alloc(p, n, err)) return false;
+  return hip_ok(hipMemsetAsync(*p, 0, (n ? n : 1) * sizeof(float), stream), err, "optimizer state clear");
+}
+}  // namespace
+
+// train.cpp:77-104: drop the previous optimizer's arrays, allocate the new
+// one's (allocate.cpp:1052-1146), clear the training arrays.
+void Model::set_optimizer(OPTIMIZER::TYPE const type_received) {
+  if (type_optimizer_function == type_received) return;
+  switch (type_received) {
+    case OPTIMIZER::NONE: case OPTIMIZER::GD: case OPTIMIZER::ADAM: case OPTIMIZER::AMSGRAD: break;
+    default: fail("set_optimizer: only GD, ADAM and AMSGRAD run on the device"); return;
+  }
+  if (impl_->ctx != nullptr) (void)dlmi_ctx_synchronize(impl_->ctx);
+  for (int i = 0; i < 4; ++i) dev_free(impl_->d_opt[i]);
+  type_optimizer_function = type_received;
+  clear_training_arrays();
+}
+
+// ops/regularizers/weight_decay.cpp:26-62.  The mask is 1 on the weights and 0 on
+// biases, scales and shifts (allocate.cpp:1178-1196, indexing.cpp:59-85).
+bool Model::set_weight_decay(real const val) {
+  if (val < 0.0f) return fail("set_weight_decay: less than zero");
+  if (val > 1.0f) return fail("set_weight_decay: bigger than one");
+  weight_decay = val;
+  if (val != 0.0f && impl_->d_opt[4] == nullptr && total_parameters != 0) {
+    std::vector<float> mask(total_parameters, 0.0f);
+    for (size_t i = 0; i < total_weights; ++i) mask[i] = 1.0f;
+    if (!dev_alloc(&impl_->d_opt[4], total_parameters, impl_->err)) return false;
+    if (!hip_ok(hipMemcpy(impl_->d_opt[4], mask.data(), total_parameters * sizeof(float), hipMemcpyHostToDevice),
+                impl_->err, "regularization mask upload"))
+      return false;
+  }
+  return true;
+}
+
+// train.cpp:278-283
+real Model::normalized_wd(size_t const batch, size_t const training_size) {
+  return weight_decay * std::sqrt(static_cast<real>(batch) / (static_cast<real>(training_size) * epoch_time_step));
+}
+
+// model.cpp:4703-4866 for the optimizers on this path; the host-side scalars
+// follow gradient_descent.cpp:64-75, gradient_descent_momentum.cpp:29-39 and
+// adam.cpp:38-54 in float.
+void Model::Update_Parameter(size_t const batch, size_t const training_size) {
+  if (impl_->d_params == nullptr) { fail("Update_Parameter: model not compiled"); return; }
+  if (use_warm_restarts) { fail("Update_Parameter: warm restarts are not implemented"); return; }
+  size_t const P = total_parameters;
+  Impl &m = *impl_;
+  real const wd = use_normalized_weight_decay ? normalized_wd(batch, training_size) : weight_decay;
+  if (wd != 0.0f && m.d_opt[4] == nullptr && !set_weight_decay(weight_decay)) return;
+  int rc = DLMI_OK;
+  switch (type_optimizer_function) {
+    case OPTIMIZER::GD: {
+      optimizer_time_step += 1.0f;
+      if (learning_momentum != 0.0f) {
+        if (!opt_array(&m.d_opt[0], P, m.stream, m.err)) return;
+        rc = dlmi_opt_gd_momentum(m.ctx, P, m.d_params, m.d_dparams, m.d_opt[0], m.d_opt[4], learning_rate,
+                                  learning_momentum, wd, use_nesterov ? 1 : 0);
+      } else {
+        rc = dlmi_opt_gd(m.ctx, P, m.d_params, m.d_dparams, m.d_opt[4], learning_rate, wd);
+      }
+      break;
+    }
+    case OPTIMIZER::ADAM:
+    case OPTIMIZER::AMSGRAD: {
+      optimizer_time_step += 1.0f;
+      bool const ams = type_optimizer_function == OPTIMIZER::AMSGRAD;
+      if (!opt_array(&m.d_opt[1], P, m.stream, m.err) || !opt_array(&m.d_opt[2], P, m.stream, m.err)) return;
+      if (ams && !opt_array(&m.d_opt[3], P, m.stream, m.err)) return;
+      real const lr = adam_learning_rate;
+      real const lr_t = use_adam_bias_correction
+                            ? lr * std::sqrt(1.0f - std::pow(adam_beta2, optimizer_time_step)) /
+                                  (1.0f - std::pow(adam_beta1, optimizer_time_step))
+                            : lr;
+      rc = dlmi_opt_adam(m.ctx, P, m.d_params, m.d_dparams, m.d_opt[1], m.d_opt[2], ams ? m.d_opt[3] : nullptr,
+                         m.d_opt[4], lr_t, adam_beta1, adam_beta2, adam_epsilon, wd);
+      break;
+    }
+    default:
+      fail("Update_Parameter: optimizer type is not managed");
+      return;
+  }
+  if (rc != DLMI_OK) fail("Update_Parameter: optimizer kernel");
+}
+
+bool Model::download_optimizer_state(int which, float *out) const {
+  if (which < 0 || which > 4 || impl_->d_opt[which] == nullptr || out == nullptr) return false;
+  return hip_ok(hipMemcpy(out, impl_->d_opt[which], total_parameters * sizeof(float), hipMemcpyDeviceToHost),
+                impl_->err, "optimizer state download");
 }
 
 }  // namespace v1

@@ -134,4 +134,36 @@ int dlmi_model_get_out(dlmi_model const *h, size_t row, float *out) {
 double dlmi_model_loss_sum(dlmi_model const *h) { return h->m.get_loss_sum(); }
 double dlmi_model_accuracy_sum(dlmi_model const *h) { return h->m.get_accuracy_sum(); }
 
+int dlmi_model_set_optimizer(dlmi_model *h, int type, float lr, float momentum, int nesterov, float adam_lr,
+                             float beta1, float beta2, float eps, int bias_correction, float weight_decay,
+                             int normalized_wd) {
+  Model &m = h->m;
+  m.learning_rate = lr;
+  m.learning_momentum = momentum;
+  m.use_nesterov = nesterov != 0;
+  m.adam_learning_rate = adam_lr;
+  m.adam_beta1 = beta1;
+  m.adam_beta2 = beta2;
+  m.adam_epsilon = eps;
+  m.use_adam_bias_correction = bias_correction != 0;
+  m.use_normalized_weight_decay = normalized_wd != 0;
+  m.optimizer_time_step = 0.0f;
+  m.epoch_time_step = 1.0f;
+  m.set_optimizer(static_cast<OPTIMIZER::TYPE>(type));
+  if (m.type_optimizer_function != static_cast<OPTIMIZER::TYPE>(type)) return 0;
+  return m.set_weight_decay(weight_decay) ? 1 : 0;
+}
+void dlmi_model_set_epoch_time_step(dlmi_model *h, float v) { h->m.epoch_time_step = v; }
+int dlmi_model_set_derivatives(dlmi_model *h, float const *g, size_t n) {
+  if (n != h->m.total_parameters) return 0;
+  std::memcpy(h->m.ptr_array_derivatives_parameters, g, n * sizeof(float));
+  return h->m.upload_derivatives() ? 1 : 0;
+}
+void dlmi_model_update_parameter(dlmi_model *h, size_t batch, size_t training_size) {
+  h->m.Update_Parameter(batch, training_size);
+}
+int dlmi_model_get_optimizer_state(dlmi_model const *h, int which, float *out) {
+  return h->m.download_optimizer_state(which, out) ? 1 : 0;
+}
+
 }  // extern "C"

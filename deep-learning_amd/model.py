@@ -19,7 +19,9 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_model_total_parameters", "dlmi_model_total_normalized_units", "dlmi_model_layer_offsets",
     "dlmi_model_set_parameters", "dlmi_model_get_parameters", "dlmi_model_set_moving", "dlmi_model_get_moving",
     "dlmi_model_get_derivatives", "dlmi_model_clear_training_arrays", "dlmi_model_step", "dlmi_model_download_layer",
-    "dlmi_model_get_out", "dlmi_model_loss_sum", "dlmi_model_accuracy_sum",
+    "dlmi_model_get_out", "dlmi_model_loss_sum", "dlmi_model_accuracy_sum", "dlmi_model_set_optimizer",
+    "dlmi_model_set_epoch_time_step", "dlmi_model_set_derivatives", "dlmi_model_update_parameter",
+    "dlmi_model_get_optimizer_state",
 ]
 
 
@@ -149,3 +151,26 @@ class Model:
 
     def accuracy_sum(self):
         return self.lib.dlmi_model_accuracy_sum(self.h)
+
+    # ---- optimizer (Model::set_optimizer / set_weight_decay / Update_Parameter) ----
+    def set_optimizer(self, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9, beta2=0.999,
+                      eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True):
+        self._ok(self.lib.dlmi_model_set_optimizer(self.h, c_int(kind), c_f(lr), c_f(momentum), c_int(int(nesterov)),
+                                                   c_f(adam_lr), c_f(beta1), c_f(beta2), c_f(eps),
+                                                   c_int(int(bias_correction)), c_f(weight_decay),
+                                                   c_int(int(normalized_wd))), "set_optimizer")
+
+    def set_epoch_time_step(self, v):
+        self.lib.dlmi_model_set_epoch_time_step(self.h, c_f(v))
+
+    def set_dparams(self, g):
+        g = np.ascontiguousarray(g, np.float32)
+        self._ok(self.lib.dlmi_model_set_derivatives(self.h, _ptr(g), c_sz(g.size)), "set_derivatives")
+
+    def update_parameter(self, batch, training_size):
+        self.lib.dlmi_model_update_parameter(self.h, c_sz(batch), c_sz(training_size))
+
+    def opt_state(self, which):
+        out = np.empty(self.P, np.float32)
+        ok = self.lib.dlmi_model_get_optimizer_state(self.h, c_int(which), _ptr(out))
+        return out if ok else None

@@ -46,6 +46,15 @@ int dlmi_model_download_layer(dlmi_model const *m, size_t layer, int which, size
 int dlmi_model_get_out(dlmi_model const *m, size_t row, float *out);          /* get_out(row) copied */
 double dlmi_model_loss_sum(dlmi_model const *m);
 double dlmi_model_accuracy_sum(dlmi_model const *m);
+/* The optimizer members (learning_rate, learning_momentum, use_nesterov, adam_*, use_adam_bias_correction,
+ * use_normalized_weight_decay) are assigned, then set_optimizer(type) and set_weight_decay(weight_decay). */
+int dlmi_model_set_optimizer(dlmi_model *m, int type, float lr, float momentum, int nesterov, float adam_lr,
+                             float beta1, float beta2, float eps, int bias_correction, float weight_decay,
+                             int normalized_wd);
+void dlmi_model_set_epoch_time_step(dlmi_model *m, float v);
+int dlmi_model_set_derivatives(dlmi_model *m, float const *g, size_t n);      /* host array -> device gradient array */
+void dlmi_model_update_parameter(dlmi_model *m, size_t batch, size_t training_size);  /* Update_Parameter */
+int dlmi_model_get_optimizer_state(dlmi_model const *m, int which, float *out);
 
 #ifdef __cplusplus
 }

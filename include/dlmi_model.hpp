@@ -59,6 +59,8 @@ struct LOSS_FN { typedef enum : int { NONE = 0, BIT = 1, CROSS_ENTROPY = 2, L1 =
   MASE_NON_SEASONAL = 7, MASE_SEASONAL = 8, ME = 9, MSE = 10, RMSE = 11, SMAPE = 12, LENGTH = 13 } TYPE; };
 struct ACCU_FN { typedef enum : int { NONE = 0, CROSS_ENTROPY = 1, DIRECTIONAL = 2, DISTANCE = 3, R = 4, SIGN = 5,
   LENGTH = 6 } TYPE; };
+struct OPTIMIZER { typedef enum : int { NONE = 0, ADABOUND = 1, ADAM = 2, ADAMAX = 3, AMSBOUND = 4, AMSGRAD = 5,
+  GD = 6, IRPROP_MINUS = 7, IRPROP_PLUS = 8, NOSADAM = 9, QUICKPROP = 10, SARPROP = 11, LENGTH = 12 } TYPE; };
 
 // v1/learner/model.hpp:70-93
 struct Layer_Parameters {
@@ -136,10 +138,24 @@ class Model {
   // Row `data_index` of the output layer (host pointer, valid until the next call).
   var const *get_out(size_t const data_index_received, size_t const time_step_index_received = 0) const;
 
+  // ---- optimizer step (model.hpp:848, 2965; train.cpp:77-104, 278-283;
+  //      ops/regularizers/weight_decay.cpp:26-62; model.cpp:4703-4866) ----------
+  // GD (plain, momentum, Nesterov), ADAM and AMSGRAD run on the device; the
+  // others are refused.  set_optimizer also clears the training arrays, like the
+  // reference.  Update_Parameter consumes and zeroes the device gradient array.
+  void set_optimizer(OPTIMIZER::TYPE const type);
+  bool set_weight_decay(real const val);
+  real normalized_wd(size_t const batch_size, size_t const training_size);
+  void Update_Parameter(size_t const batch_size, size_t const training_size);
+  // which: 0 previous delta, 1 first moment, 2 second moment, 3 second moment hat,
+  // 4 regularization mask; false when that array does not exist.
+  bool download_optimizer_state(int which, float *out) const;
+
   // ---- buffers moved explicitly between host mirrors and HBM ----------------
   bool upload_parameters(void);     // ptr_array_parameters -> device
   bool download_parameters(void);   // device -> ptr_array_parameters
   bool download_derivatives(void);  // device gradient array -> ptr_array_derivatives_parameters
+  bool upload_derivatives(void);    // ptr_array_derivatives_parameters -> device gradient array
   bool upload_moving_statistics(void);
   bool download_moving_statistics(void);
   bool set_dropout_mask(size_t const index_layer_received, uint8_t const *mask_per_unit);
@@ -166,6 +182,21 @@ class Model {
   real normalization_epsilon = 1e-5f;
   real batch_renormalization_r_correction_maximum = 1.0f;
   real batch_renormalization_d_correction_maximum = 0.0f;
+  // optimizer hyper-parameters, defaults of model.hpp:2839-2841, 3020-3036
+  OPTIMIZER::TYPE type_optimizer_function = OPTIMIZER::NONE;
+  bool use_nesterov = false;
+  bool use_normalized_weight_decay = true;
+  bool use_adam_bias_correction = true;
+  bool use_warm_restarts = false;  // warm restarts are not implemented: Update_Parameter refuses them
+  real learning_rate = 0.01f;
+  real learning_momentum = 0.9f;
+  real weight_decay = 0.0f;
+  real adam_learning_rate = 0.001f;
+  real adam_beta1 = 0.9f;
+  real adam_beta2 = 0.999f;
+  real adam_epsilon = 1e-8f;
+  real optimizer_time_step = 0.0f;
+  real epoch_time_step = 1.0f;
   MODEL::TYPE type = MODEL::NONE;
   LOSS_FN::TYPE type_loss_function = LOSS_FN::NONE;
   ACCU_FN::TYPE type_accuracy_function = ACCU_FN::NONE;
