@@ -1,0 +1,138 @@
+// Epoch driver over the GPU Model facade (include/dlmi_driver.hpp).  Control
+// flow of /root/reference/lib/deep-learning/drivers/driver.cpp: evalt :60-108,
+// train :110-193, evalt_st :244-257, train_st :294-340.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "../../include/dlmi_driver.hpp"
+
+namespace dlmi {
+
+using namespace v1;
+
+Driver::Driver(Dataset &dataset_received, ENV::TYPE const &env_type_received, Model &model_received,
+               size_t const minibatch_size_received)
+    : minibatch_size(minibatch_size_received), dataset(dataset_received), env_type(env_type_received),
+      model(model_received) {}
+
+Driver::~Driver(void) {
+  if (d_X_ != nullptr || d_Y_ != nullptr) (void)model.synchronize();
+  if (d_X_ != nullptr) (void)hipFree(d_X_);
+  if (d_Y_ != nullptr) (void)hipFree(d_Y_);
+}
+
+// One dense copy of the data set in HBM.  Returns false (and leaves the driver
+// on the staged path) when it is switched off or the memory is not there.
+bool Driver::make_resident(void) {
+  if (d_X_ != nullptr) return true;
+  if (resident_tried_ || !keep_dataset_on_device) return false;
+  resident_tried_ = true;
+  size_t const n = dataset.n_data, ni = dataset.n_inp, no = dataset.n_out;
+  if (n == 0 || dataset.Xm == nullptr || dataset.Ym == nullptr) return false;
+  void *px = nullptr, *py = nullptr;
+  if (hipMalloc(&px, n * ni * sizeof(float)) != hipSuccess) { (void)hipGetLastError(); return false; }
+  if (hipMalloc(&py, n * no * sizeof(float)) != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipFree(px);
+    return false;
+  }
+  // gather the row pointers into dense blocks, 64 Mi floats at a time
+  size_t const chunk_rows_x = ni ? ((size_t(1) << 26) / ni ? (size_t(1) << 26) / ni : 1) : n;
+  std::vector<float> stage;
+  bool ok = true;
+  for (size_t r0 = 0; r0 < n && ok; r0 += chunk_rows_x) {
+    size_t const rows = r0 + chunk_rows_x < n ? chunk_rows_x : n - r0;
+    stage.resize(rows * (ni > no ? ni : no));
+    for (size_t i = 0; i < rows; ++i) std::memcpy(stage.data() + i * ni, dataset.Xm[r0 + i], ni * sizeof(float));
+    ok = hipMemcpy(static_cast<float *>(px) + r0 * ni, stage.data(), rows * ni * sizeof(float), hipMemcpyHostToDevice) == hipSuccess;
+    for (size_t i = 0; i < rows; ++i) std::memcpy(stage.data() + i * no, dataset.Ym[r0 + i], no * sizeof(float));
+    ok = ok && hipMemcpy(static_cast<float *>(py) + r0 * no, stage.data(), rows * no * sizeof(float), hipMemcpyHostToDevice) == hipSuccess;
+  }
+  if (!ok) {
+    (void)hipGetLastError();
+    (void)hipFree(px);
+    (void)hipFree(py);
+    return false;
+  }
+  d_X_ = static_cast<float *>(px);
+  d_Y_ = static_cast<float *>(py);
+  return true;
+}
+
+double Driver::evalt(void) {
+  model.reset_loss();
+  model.type_state_propagation = PROPAGATION::INFERENCE;
+  if (!model.update_mem_batch_size(dataset.n_data)) {
+    std::fprintf(stderr, "dlmi::Driver: update_mem_batch_size(%zu) failed\n", dataset.n_data);
+    return HUGE_VAL;
+  }
+  evalt_st();
+  model.n_acc_trial = dataset.n_data * (dataset.seq_w - model.n_time_delay) *
+                      (ACCU_FN::CROSS_ENTROPY == model.type_accuracy_function ? size_t(1) : dataset.n_out);
+  double const loss = model.get_loss(ENV::NONE);
+  model.set_loss(env_type, loss);
+  model.set_accu(env_type, model.get_accu(ENV::NONE));
+  return loss;
+}
+
+double Driver::train(void) {
+  if (model.ptr_array_derivatives_parameters == nullptr) model.clear_training_arrays();
+  model.type_state_propagation = PROPAGATION::TRAINING;
+  if (!model.update_mem_batch_size(dataset.n_data)) {
+    std::fprintf(stderr, "dlmi::Driver: update_mem_batch_size(%zu) failed\n", dataset.n_data);
+    return HUGE_VAL;
+  }
+  if (resample_dropout_masks && (model.Use__Dropout__Bernoulli() || model.Use__Dropout__Bernoulli__Inverted()))
+    model.Dropout_Bernoulli();
+  model.reset_loss();
+  train_st();
+  model.type_state_propagation = PROPAGATION::INFERENCE;
+  model.epoch_time_step += 1.0f;
+  model.n_acc_trial = dataset.n_data * (dataset.seq_w - model.n_time_delay) *
+                      (ACCU_FN::CROSS_ENTROPY == model.type_accuracy_function ? size_t(1) : dataset.n_out);
+  double const loss = model.get_loss(ENV::NONE);
+  model.set_loss(env_type, loss);
+  model.set_accu(env_type, model.get_accu(ENV::NONE));
+  return loss;
+}
+
+void Driver::evalt_st(void) {
+  size_t const n_data = dataset.n_data, batch_size_max = model.batch_size;
+  size_t const n_batch = static_cast<size_t>(std::ceil(static_cast<double>(n_data) / static_cast<double>(batch_size_max)));
+  bool const resident = make_resident();
+  for (size_t i = 0; i != n_batch; ++i) {
+    size_t const batch_size = i + 1 != n_batch ? batch_size_max : n_data - i * batch_size_max;
+    if (resident) {
+      model.forward_pass_device(batch_size, d_X_ + i * batch_size_max * dataset.n_inp);
+      model.compute_loss_device(batch_size, d_Y_ + i * batch_size_max * dataset.n_out);
+    } else {
+      model.forward_pass(batch_size, dataset.Xm + i * batch_size_max);
+      model.compute_loss(batch_size, dataset.Ym + i * batch_size_max);
+    }
+  }
+}
+
+void Driver::train_st(void) {
+  size_t const n_data = dataset.n_data, batch_size_max = model.batch_size;
+  size_t const n_batch = static_cast<size_t>(std::ceil(static_cast<double>(n_data) / static_cast<double>(batch_size_max)));
+  bool const resident = make_resident();
+  for (size_t i = 0; i != n_batch; ++i) {
+    size_t const batch_size = i + 1 != n_batch ? batch_size_max : n_data - i * batch_size_max;
+    if (resident) {
+      model.forward_pass_device(batch_size, d_X_ + i * batch_size_max * dataset.n_inp);
+      model.compute_error_device(batch_size, d_Y_ + i * batch_size_max * dataset.n_out);
+    } else {
+      model.forward_pass(batch_size, dataset.Xm + i * batch_size_max);
+      model.compute_error(batch_size, dataset.Ym + i * batch_size_max);
+    }
+    model.backward_pass(batch_size);
+    model.update_derivatives(batch_size, model.ptr_array_layers + 1, model.ptr_last_layer);
+  }
+  model.Update_Parameter(n_data, n_data);
+}
+
+}  // namespace dlmi

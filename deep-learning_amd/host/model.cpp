@@ -35,6 +35,8 @@ struct Model::Impl {
   // optimizer state [P] each: 0 previous delta, 1 first moment, 2 second moment,
   // 3 second moment hat, 4 regularization mask; allocated (zeroed) on first use
   float *d_opt[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+  float const *cur_input = nullptr;  // [batch, n_in] of the pass in flight: d_input or a caller's device rows
+  size_t n_loss_examples = 0;        // examples whose loss has been accumulated since reset_loss()
   float *h_stage = nullptr;    // pinned staging for the row-pointer gather
   size_t h_stage_floats = 0;
   mutable std::vector<float> out_host;  // get_out() cache
@@ -310,6 +312,7 @@ void Model::clear_training_arrays(void) {
   if (impl_->d_dparams == nullptr) return;
   (void)hipMemsetAsync(impl_->d_dparams, 0, total_parameters * sizeof(float), impl_->stream);
   (void)hipMemsetAsync(impl_->d_stats, 0, 2 * sizeof(double), impl_->stream);
+  impl_->n_loss_examples = 0;
   std::memset(ptr_array_derivatives_parameters, 0, total_parameters * sizeof(real));
 }
 
@@ -400,7 +403,6 @@ void Model::forward_pass(size_t const B, real const *const *const Xm, long long 
   if (out_idx == -1ll) out_idx = static_cast<long long>(total_layers);
   if (in_idx != 0 || out_idx != static_cast<long long>(total_layers)) { fail("forward_pass: only whole-network passes are on this path"); return; }
   if (B == 0 || B > impl_->allocated_batch) { fail("forward_pass: batch size exceeds update_mem_batch_size()"); return; }
-  dlmi_ctx *ctx = impl_->ctx;
   size_t const n_in = ptr_array_layers[0].n_out;
   // assign_inputs.cpp:22-40: gather the row pointers into a dense [B, K] block
   // (pinned staging buffer: the previous step's copy out of it has completed
@@ -410,9 +412,23 @@ void Model::forward_pass(size_t const B, real const *const *const Xm, long long 
   if (!hip_ok(hipMemcpyAsync(impl_->d_input, impl_->h_stage, B * n_in * sizeof(float), hipMemcpyHostToDevice, impl_->stream),
               impl_->err, "input upload"))
     return;
+  impl_->cur_input = impl_->d_input;
+  forward_layers(B);
+}
+
+void Model::forward_pass_device(size_t const B, float const *d_inputs) {
+  if (ptr_array_layers == nullptr || d_inputs == nullptr) { fail("forward_pass_device: model not compiled or null input"); return; }
+  if (B == 0 || B > impl_->allocated_batch) { fail("forward_pass_device: batch size exceeds update_mem_batch_size()"); return; }
+  impl_->cur_input = d_inputs;
+  forward_layers(B);
+}
+
+// Layer loop of FF__Forward_Pass_Batch__Loop (fwp_st.cpp:118-185, 298-733) on impl_->cur_input.
+void Model::forward_layers(size_t const B) {
+  dlmi_ctx *ctx = impl_->ctx;
   bool const training = type_state_propagation >= PROPAGATION::TRAINING;
-  float const *in = impl_->d_input;
-  size_t K = n_in;
+  float const *in = impl_->cur_input;
+  size_t K = ptr_array_layers[0].n_out;
   for (size_t li = 1; li < total_layers; ++li) {
     Layer &l = ptr_array_layers[li];
     size_t const H = l.n_out;
@@ -475,19 +491,91 @@ var const *Model::get_out(size_t const data_index, size_t const) const {
 
 void Model::compute_error(size_t const B, real const *const *const Ym) {
   if (ptr_array_layers == nullptr || Ym == nullptr || B == 0 || B > impl_->allocated_batch) { fail("compute_error: bad argument"); return; }
-  Layer &o = ptr_array_layers[total_layers - 1];
-  if (o.type_activation_function != ACTIVATION::SOFTMAX || type_loss_function != LOSS_FN::CROSS_ENTROPY) {
-    fail("compute_error: only softmax + cross-entropy is on this path");
-    return;
-  }
-  size_t const H = o.n_out;
+  size_t const H = ptr_array_layers[total_layers - 1].n_out;
   (void)hipStreamSynchronize(impl_->stream);
   for (size_t i = 0; i < B; ++i) std::memcpy(impl_->h_stage + i * H, Ym[i], H * sizeof(float));
   if (!hip_ok(hipMemcpyAsync(impl_->d_targets, impl_->h_stage, B * H * sizeof(float), hipMemcpyHostToDevice, impl_->stream),
               impl_->err, "target upload"))
     return;
-  if (dlmi_softmax_ce_seed(impl_->ctx, B, H, o.d_outputs, impl_->d_targets, o.d_errors, impl_->d_stats) != DLMI_OK)
+  seed_error(B, impl_->d_targets);
+}
+
+void Model::compute_error_device(size_t const B, float const *d_targets) {
+  if (ptr_array_layers == nullptr || d_targets == nullptr || B == 0 || B > impl_->allocated_batch) { fail("compute_error_device: bad argument"); return; }
+  seed_error(B, d_targets);
+}
+
+// Loss and accuracy are accumulated by the same kernel that forms the seed
+// gradient; without a backward pass behind it the gradient is simply unused.
+void Model::compute_loss(size_t const B, real const *const *const Ym) { compute_error(B, Ym); }
+void Model::compute_loss_device(size_t const B, float const *d_targets) { compute_error_device(B, d_targets); }
+
+void Model::seed_error(size_t const B, float const *d_targets) {
+  Layer &o = ptr_array_layers[total_layers - 1];
+  if (o.type_activation_function != ACTIVATION::SOFTMAX || type_loss_function != LOSS_FN::CROSS_ENTROPY) {
+    fail("compute_error: only softmax + cross-entropy is on this path");
+    return;
+  }
+  if (dlmi_softmax_ce_seed(impl_->ctx, B, o.n_out, o.d_outputs, d_targets, o.d_errors, impl_->d_stats) != DLMI_OK) {
     fail("compute_error: dlmi_softmax_ce_seed");
+    return;
+  }
+  impl_->n_loss_examples += B;
+}
+
+// ---------------------------------------------------------------- loss / accuracy bookkeeping
+void Model::reset_loss(void) {
+  n_acc_trial = 0;
+  impl_->n_loss_examples = 0;
+  if (impl_->d_stats != nullptr) (void)hipMemsetAsync(impl_->d_stats, 0, 2 * sizeof(double), impl_->stream);
+}
+// get_ace (loss.cpp:212-221): summed cross-entropy / number of examples
+double Model::get_loss(ENV::TYPE const env) const {
+  switch (env) {
+    case ENV::TRAIN: return loss_train;
+    case ENV::VALID: return loss_valid;
+    case ENV::TESTG: return loss_testg;
+    case ENV::NONE:
+      if (type_loss_function != LOSS_FN::CROSS_ENTROPY) return 1.0;
+      return impl_->n_loss_examples != 0 ? get_loss_sum() / static_cast<double>(impl_->n_loss_examples) : HUGE_VAL;
+    default: return 1.0;
+  }
+}
+// metrics.cpp:89-114
+double Model::get_accu(ENV::TYPE const env) const {
+  switch (env) {
+    case ENV::TRAIN: return acc_train;
+    case ENV::VALID: return acc_valid;
+    case ENV::TESTG: return acc_testg;
+    case ENV::NONE: return n_acc_trial == 0 ? 0.0 : get_accuracy_sum() / static_cast<double>(n_acc_trial) * 100.0;
+    default: return 0.0;
+  }
+}
+void Model::set_loss(ENV::TYPE const env, double const loss) {
+  switch (env) {
+    case ENV::TRAIN: loss_train = loss; break;
+    case ENV::VALID: loss_valid = loss; break;
+    case ENV::TESTG: loss_testg = loss; break;
+    default: fail("set_loss: loss type is not managed"); break;
+  }
+}
+void Model::set_accu(ENV::TYPE const env, double const accu) {
+  switch (env) {
+    case ENV::TRAIN: acc_train = accu; break;
+    case ENV::VALID: acc_valid = accu; break;
+    case ENV::TESTG: acc_testg = accu; break;
+    default: fail("set_accu: accuracy type is not managed"); break;
+  }
+}
+bool Model::Use__Dropout__Bernoulli(void) const {
+  for (Layer const *l = ptr_array_layers; l != ptr_last_layer; ++l)
+    if (l->type_dropout == LAYER_DROPOUT::BERNOULLI) return true;
+  return false;
+}
+bool Model::Use__Dropout__Bernoulli__Inverted(void) const {
+  for (Layer const *l = ptr_array_layers; l != ptr_last_layer; ++l)
+    if (l->type_dropout == LAYER_DROPOUT::BERNOULLI_INVERTED) return true;
+  return false;
 }
 
 void Model::backward_pass(size_t const B) {
@@ -529,7 +617,7 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
   for (Layer *l = first; l != last; ++l) {
     size_t const li = static_cast<size_t>(l - ptr_array_layers);
     if (li == 0 || li >= total_layers) continue;
-    float const *in = li == 1 ? impl_->d_input : ptr_array_layers[li - 1].d_outputs;
+    float const *in = li == 1 ? impl_->cur_input : ptr_array_layers[li - 1].d_outputs;
     size_t const K = ptr_array_layers[li - 1].n_out;
     float *db = l->Use__Bias() ? impl_->d_dparams + l->first_bias_connection_index : nullptr;
     if (dlmi_fc_bwd_dw(impl_->ctx, B, K, l->n_out, in, l->d_errors, impl_->d_dparams + l->first_connection_index, db, 1) != DLMI_OK) {

@@ -2,6 +2,7 @@
 #include <cstring>
 #include <vector>
 
+#include "../../include/dlmi_driver.hpp"
 #include "../../include/dlmi_model.h"
 #include "../../include/dlmi_model.hpp"
 
@@ -9,6 +10,16 @@ using namespace dlmi::v1;
 
 struct dlmi_model {
   Model m;
+};
+
+// The driver with the data it was created on: dense copies and the row-pointer
+// arrays the reference's Dataset exposes.
+struct dlmi_driver {
+  std::vector<float> X, Y;
+  std::vector<float const *> Xm, Ym;
+  dlmi::Dataset ds;
+  dlmi::Driver *drv = nullptr;
+  ~dlmi_driver() { delete drv; }
 };
 
 extern "C" {
@@ -164,6 +175,40 @@ void dlmi_model_update_parameter(dlmi_model *h, size_t batch, size_t training_si
 }
 int dlmi_model_get_optimizer_state(dlmi_model const *h, int which, float *out) {
   return h->m.download_optimizer_state(which, out) ? 1 : 0;
+}
+
+dlmi_driver *dlmi_driver_create(dlmi_model *h, size_t n_data, float const *X, float const *Y, int env, int on_device) {
+  if (h == nullptr || X == nullptr || Y == nullptr || n_data == 0 || h->m.ptr_array_layers == nullptr) return nullptr;
+  dlmi_driver *d = new dlmi_driver;
+  size_t const ni = h->m.ptr_array_layers[0].n_out, no = h->m.Get__Output_Layer()->n_out;
+  d->X.assign(X, X + n_data * ni);
+  d->Y.assign(Y, Y + n_data * no);
+  d->Xm.resize(n_data);
+  d->Ym.resize(n_data);
+  for (size_t i = 0; i < n_data; ++i) {
+    d->Xm[i] = d->X.data() + i * ni;
+    d->Ym[i] = d->Y.data() + i * no;
+  }
+  d->ds.n_data = n_data; d->ds.n_inp = ni; d->ds.n_out = no; d->ds.seq_w = 1;
+  d->ds.Xm = d->Xm.data();
+  d->ds.Ym = d->Ym.data();
+  d->drv = new dlmi::Driver(d->ds, static_cast<ENV::TYPE>(env), h->m);
+  d->drv->keep_dataset_on_device = on_device != 0;
+  return d;
+}
+void dlmi_driver_destroy(dlmi_driver *d) { delete d; }
+int dlmi_driver_train(dlmi_driver *d, int resample_dropout_masks, double *out) {
+  if (d == nullptr || out == nullptr) return 0;
+  d->drv->resample_dropout_masks = resample_dropout_masks != 0;
+  out[0] = d->drv->train();
+  out[1] = d->drv->model.get_accu(d->drv->env_type);
+  return d->drv->model.last_error()[0] == '\0' ? 1 : 0;
+}
+int dlmi_driver_evalt(dlmi_driver *d, double *out) {
+  if (d == nullptr || out == nullptr) return 0;
+  out[0] = d->drv->evalt();
+  out[1] = d->drv->model.get_accu(d->drv->env_type);
+  return d->drv->model.last_error()[0] == '\0' ? 1 : 0;
 }
 
 }  // extern "C"

@@ -21,7 +21,8 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_model_get_derivatives", "dlmi_model_clear_training_arrays", "dlmi_model_step", "dlmi_model_download_layer",
     "dlmi_model_get_out", "dlmi_model_loss_sum", "dlmi_model_accuracy_sum", "dlmi_model_set_optimizer",
     "dlmi_model_set_epoch_time_step", "dlmi_model_set_derivatives", "dlmi_model_update_parameter",
-    "dlmi_model_get_optimizer_state",
+    "dlmi_model_get_optimizer_state", "dlmi_driver_create", "dlmi_driver_destroy", "dlmi_driver_train",
+    "dlmi_driver_evalt",
 ]
 
 
@@ -53,6 +54,8 @@ class Model:
         self.max_batch = 0
 
     def close(self):
+        for d, _, _ in self.__dict__.pop("_drivers", {}).values():
+            self.lib.dlmi_driver_destroy(d)
         if getattr(self, "h", None):
             self.lib.dlmi_model_destroy(self.h)
             self.h = None
@@ -174,3 +177,28 @@ class Model:
         out = np.empty(self.P, np.float32)
         ok = self.lib.dlmi_model_get_optimizer_state(self.h, c_int(which), _ptr(out))
         return out if ok else None
+
+    # ---- epoch driver (Driver::train / Driver::evalt) -------------------------------
+    def _driver(self, X, Y, on_device=True):
+        """One driver per data set (identified by the arrays' contents' identity)."""
+        X, Y = np.ascontiguousarray(X, np.float32), np.ascontiguousarray(Y, np.float32)
+        key = (X.ctypes.data, Y.ctypes.data, X.shape, on_device)
+        drivers = self.__dict__.setdefault("_drivers", {})
+        if key not in drivers:
+            self.lib.dlmi_driver_create.restype = vp
+            d = self.lib.dlmi_driver_create(self.h, c_sz(X.shape[0]), _ptr(X), _ptr(Y), c_int(1), c_int(int(on_device)))
+            if not d:
+                raise RuntimeError("dlmi_driver_create failed")
+            drivers[key] = (vp(d), X, Y)  # the arrays stay alive with the key
+        return drivers[key][0]
+
+    def train_epoch(self, X, Y, resample_masks=False, on_device=True):
+        out = (ctypes.c_double * 2)()
+        self._ok(self.lib.dlmi_driver_train(self._driver(X, Y, on_device), c_int(int(resample_masks)), out),
+                 "Driver::train")
+        return out[0], out[1]
+
+    def evalt(self, X, Y, on_device=True):
+        out = (ctypes.c_double * 2)()
+        self._ok(self.lib.dlmi_driver_evalt(self._driver(X, Y, on_device), out), "Driver::evalt")
+        return out[0], out[1]

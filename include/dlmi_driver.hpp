@@ -1,0 +1,78 @@
+// Epoch driver with the reference's interface (lib/deep-learning/drivers/
+// driver.hpp:24-45, driver.cpp:52-340) over the GPU Model facade.
+//
+//   Driver::train()  one pass over the data set in sub-batches of
+//                    model.batch_size rows: forward, error, backward and
+//                    parameter-gradient accumulation per sub-batch, then ONE
+//                    optimizer step with batch = training size = n_data
+//                    (driver.cpp:110-193, 259-340)
+//   Driver::evalt()  forward + loss/accuracy per sub-batch (driver.cpp:60-108,
+//                    195-257)
+//
+// What differs, by design: on first use the driver copies the data set to HBM
+// once (dense [n_data, n_inp] and [n_data, n_out]); the sub-batches of every
+// later epoch are then slices of those device arrays and no input crosses PCIe
+// again.  If the data set does not fit, the rows are staged per sub-batch as
+// Model::forward_pass(batch, rows) does.  The *_mp variants are the *_st ones:
+// there are no host threads to split the batch over.
+#ifndef DLMI_DRIVER_HPP
+#define DLMI_DRIVER_HPP
+
+#include <cstddef>
+
+#include "dlmi_model.hpp"
+
+namespace dlmi {
+
+// The public data members of the reference's Dataset (data/dataset.hpp:24-51)
+// that the driver reads.  The caller owns the rows.
+struct Dataset {
+  size_t n_data = 0, n_inp = 0, n_out = 0, seq_w = 1;
+  v1::real const **Xm = nullptr;  // n_data row pointers, n_inp floats each
+  v1::real const **Ym = nullptr;  // n_data row pointers, n_out floats each
+};
+
+class Driver {
+ public:
+  Driver(Dataset &dataset, v1::ENV::TYPE const &env_type, v1::Model &model, size_t const minibatch_size = 0);
+  ~Driver(void);
+  Driver(Driver const &) = delete;
+  Driver &operator=(Driver const &) = delete;
+
+  double evalt(void);
+  double train(void);
+
+  size_t minibatch_size = 0;  // unused, as in the reference (driver.hpp:33-34)
+
+  void evalt_mp(void) { evalt_st(); }
+  void evalt_st(void);
+  void train_mp(void) { train_st(); }
+  void train_st(void);
+
+  // false: Driver::train leaves the dropout masks as they are instead of calling
+  // Model::Dropout_Bernoulli() (for runs that install their own masks)
+  bool resample_dropout_masks = true;
+  // false: never keep the data set in HBM
+  bool keep_dataset_on_device = true;
+
+  Dataset &dataset;
+  v1::ENV::TYPE env_type;
+  v1::Model &model;
+
+ private:
+  bool make_resident(void);
+  float *d_X_ = nullptr, *d_Y_ = nullptr;
+  bool resident_tried_ = false;
+};
+
+}  // namespace dlmi
+
+#ifdef DLMI_ALIAS_DL_NAMESPACE
+namespace DL {
+using ::dlmi::Dataset;
+using ::dlmi::Driver;
+using ENV = ::dlmi::v1::ENV;  // DL::ENV::TYPE, DL::ENV::TRAIN ... (data/enum/env.hpp)
+}  // namespace DL
+#endif
+
+#endif  // DLMI_DRIVER_HPP

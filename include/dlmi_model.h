@@ -56,6 +56,16 @@ int dlmi_model_set_derivatives(dlmi_model *m, float const *g, size_t n);      /*
 void dlmi_model_update_parameter(dlmi_model *m, size_t batch, size_t training_size);  /* Update_Parameter */
 int dlmi_model_get_optimizer_state(dlmi_model const *m, int which, float *out);
 
+/* Epoch driver (dlmi_driver.hpp; the reference's Driver, drivers/driver.hpp:24-45).  X [n_data, n_inp] and
+ * Y [n_data, n_out] are dense host arrays; the driver keeps its own copy of them.  env: ENV::TYPE (1 TRAIN,
+ * 2 VALID, 3 TESTG).  on_device != 0 keeps the data set in HBM after the first pass. */
+typedef struct dlmi_driver dlmi_driver;
+dlmi_driver *dlmi_driver_create(dlmi_model *m, size_t n_data, float const *X, float const *Y, int env, int on_device);
+void dlmi_driver_destroy(dlmi_driver *d);
+/* Driver::train() / Driver::evalt(); out[0] = loss, out[1] = accuracy in percent (get_loss / get_accu of env). */
+int dlmi_driver_train(dlmi_driver *d, int resample_dropout_masks, double *out);
+int dlmi_driver_evalt(dlmi_driver *d, double *out);
+
 #ifdef __cplusplus
 }
 #endif

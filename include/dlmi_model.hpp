@@ -59,6 +59,7 @@ struct LOSS_FN { typedef enum : int { NONE = 0, BIT = 1, CROSS_ENTROPY = 2, L1 =
   MASE_NON_SEASONAL = 7, MASE_SEASONAL = 8, ME = 9, MSE = 10, RMSE = 11, SMAPE = 12, LENGTH = 13 } TYPE; };
 struct ACCU_FN { typedef enum : int { NONE = 0, CROSS_ENTROPY = 1, DIRECTIONAL = 2, DISTANCE = 3, R = 4, SIGN = 5,
   LENGTH = 6 } TYPE; };
+struct ENV { typedef enum : int { NONE = 0, TRAIN = 1, VALID = 2, TESTG = 3, LENGTH = 4 } TYPE; };  // data/enum/env.hpp
 struct OPTIMIZER { typedef enum : int { NONE = 0, ADABOUND = 1, ADAM = 2, ADAMAX = 3, AMSBOUND = 4, AMSGRAD = 5,
   GD = 6, IRPROP_MINUS = 7, IRPROP_PLUS = 8, NOSADAM = 9, QUICKPROP = 10, SARPROP = 11, LENGTH = 12 } TYPE; };
 
@@ -135,6 +136,22 @@ class Model {
   void compute_error(size_t const batch_size, real const *const *const Ym);
   void backward_pass(size_t const batch_size);
   void update_derivatives(size_t const batch_size, Layer *const layer_it, Layer const *const last_layer);
+  // compute_loss.cpp: the loss / accuracy accumulation of compute_error without the seed gradient
+  void compute_loss(size_t const batch_size, real const *const *const Ym);
+  // The same three calls on rows that already sit in HBM (dense row-major device
+  // arrays [batch_size, n_inp] / [batch_size, n_out]): what the epoch driver uses
+  // once the data set is resident.  No reference counterpart.
+  void forward_pass_device(size_t const batch_size, float const *d_inputs);
+  void compute_error_device(size_t const batch_size, float const *d_targets);
+  void compute_loss_device(size_t const batch_size, float const *d_targets);
+  // loss.cpp:35-75, 103-134, 212-221; metrics.cpp:75-114 (cross-entropy loss and accuracy only)
+  void reset_loss(void);
+  double get_loss(ENV::TYPE const env) const;
+  double get_accu(ENV::TYPE const env) const;
+  void set_loss(ENV::TYPE const env, double const loss);
+  void set_accu(ENV::TYPE const env, double const accu);
+  bool Use__Dropout__Bernoulli(void) const;
+  bool Use__Dropout__Bernoulli__Inverted(void) const;
   // Row `data_index` of the output layer (host pointer, valid until the next call).
   var const *get_out(size_t const data_index_received, size_t const time_step_index_received = 0) const;
 
@@ -172,6 +189,9 @@ class Model {
   size_t total_normalized_units = 0;  // one slot per unit of EVERY layer, input included
   size_t batch_size = 1, maximum_batch_size = 1, seq_w = 1;
   size_t number_threads = 1;
+  size_t n_acc_trial = 0, n_time_delay = 0;
+  double loss_train = 3.40282e38, loss_valid = 3.40282e38, loss_testg = 3.40282e38;  // model.hpp: FLT_MAX defaults
+  double acc_train = 0.0, acc_valid = 0.0, acc_testg = 0.0;
   Layer *ptr_array_layers = nullptr;
   Layer *ptr_last_layer = nullptr;  // one past the output layer
   var *ptr_array_parameters = nullptr;               // host mirror [P]: W.. | b.. | gamma.. | beta..
@@ -213,6 +233,8 @@ class Model {
   struct Impl;
   Impl *impl_;
   bool allocate_batch(size_t batch);
+  void forward_layers(size_t batch);
+  void seed_error(size_t batch, float const *d_targets);
   void free_batch(void);
   bool fail(char const *what) const;
 };

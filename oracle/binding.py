@@ -373,6 +373,48 @@ class OracleMLP:
     def get_dparams(self):
         return self.dparameters.copy()
 
+    # ---- optimizer and epoch driver (drivers/driver.cpp:60-340) --------------------
+    def set_optimizer(self, kind, **kw):
+        wd = kw.get("weight_decay", 0.0)
+        mask = None
+        if wd != 0.0:  # 1 on the weights, 0 on biases / gamma / beta (indexing.cpp:59-85)
+            nw = sum(self.widths[l] * self.widths[l - 1] for l in range(1, len(self.widths)))
+            mask = np.zeros(self.P, np.float32)
+            mask[:nw] = 1
+        self.opt = OptimizerHost(self.o, self.P, kind, mask=mask, **kw)
+
+    def update_parameter(self, batch, training_size):
+        self.opt.update(self.parameters, self.dparameters, batch, training_size, self.nthreads)
+
+    def _batches(self, n):
+        bs = min(self.max_batch, n)
+        return [(i, min(bs, n - i)) for i in range(0, n, bs)]
+
+    def _loss_accu(self, n):
+        loss = self.lib.dlo_mlp_loss_sum(self.h) / n if n else float("inf")  # get_ace, loss.cpp:212-221
+        return loss, self.lib.dlo_mlp_n_correct(self.h) / n * 100.0           # get_accu, metrics.cpp:89-114
+
+    def train_epoch(self, X, Y):
+        """Driver::train: gradients accumulate over the sub-batches, ONE parameter
+        update with batch = training size = n_data, then epoch_time_step += 1."""
+        X, Y = np.ascontiguousarray(X, np.float32), np.ascontiguousarray(Y, np.float32)
+        n = X.shape[0]
+        self.lib.dlo_mlp_reset_loss(self.h)
+        for i, b in self._batches(n):
+            self.step(STATE["TRAINING"], X[i:i + b], Y[i:i + b], backward=True)
+        self.update_parameter(n, n)
+        self.opt.epoch_time_step = np.float32(self.opt.epoch_time_step + np.float32(1))
+        return self._loss_accu(n)
+
+    def evalt(self, X, Y):
+        X, Y = np.ascontiguousarray(X, np.float32), np.ascontiguousarray(Y, np.float32)
+        n = X.shape[0]
+        self.lib.dlo_mlp_reset_loss(self.h)
+        for i, b in self._batches(n):
+            self.step(STATE["INFERENCE"], X[i:i + b], None, backward=False)
+            self.lib.dlo_mlp_compute_loss(self.h, c_int(self.nthreads), c_sz(b), _ptr(Y[i:i + b]))
+        return self._loss_accu(n)
+
     def get_moving(self):
         return self.moving_mean.copy(), self.moving_std.copy()
 
@@ -560,3 +602,18 @@ class ReferenceMLP:
         out = np.empty(self.P, np.float32)
         ok = self.lib.dlref_model_get_opt_state(self.h, c_int(which), _ptr(out), c_sz(self.P))
         return out if ok else None
+
+    # ---- epoch driver (Driver::train / Driver::evalt over dense arrays) ---------------
+    def train_epoch(self, X, Y, resample_masks=False):
+        X, Y = np.ascontiguousarray(X, np.float32), np.ascontiguousarray(Y, np.float32)
+        out = (c_d * 2)()
+        self.lib.dlref_model_train_epoch(self.h, c_sz(X.shape[0]), _ptr(X), c_sz(X.shape[1]), _ptr(Y),
+                                         c_sz(Y.shape[1]), c_int(int(resample_masks)), out)
+        return out[0], out[1]
+
+    def evalt(self, X, Y):
+        X, Y = np.ascontiguousarray(X, np.float32), np.ascontiguousarray(Y, np.float32)
+        out = (c_d * 2)()
+        self.lib.dlref_model_evalt(self.h, c_sz(X.shape[0]), _ptr(X), c_sz(X.shape[1]), _ptr(Y), c_sz(Y.shape[1]),
+                                   out)
+        return out[0], out[1]

@@ -14,6 +14,7 @@
 #include <omp.h>
 
 #include <cstdint>
+#include <cmath>
 #include <cstring>
 #include <vector>
 
@@ -622,5 +623,101 @@ int dlref_model_get_opt_state(void *h, int which, float *out, size_t n) {
   std::memcpy(out, src, n * sizeof(float));
   return 1;
 }
+
+// ---- epoch driver.  Driver (drivers/driver.cpp) cannot be compiled here: its
+// Dataset base class (data/dataset/dataset.cpp) needs the fmt library, which
+// this image does not ship.  The functions below are driver.cpp:110-193
+// (Driver::train), :60-108 (Driver::evalt), :195-257 (evalt_mp / evalt_st) and
+// :259-340 (train_mp / train_st) with the dataset passed as dense arrays; every
+// call inside them is the reference's own Model member.
+// resample_masks == 0 skips Model::Dropout_Bernoulli() (its generator is seeded
+// from the clock, allocate.cpp:93) so that installed masks stay in place.
+// out[0] = loss (get_loss(ENV::NONE)), out[1] = accuracy (get_accu(ENV::NONE)).
+void dlref_model_train_epoch(void *h, size_t n_data, float const *X, size_t K0, float const *Y, size_t Hout,
+                             int resample_masks, double *out) {
+  RefModel *rm = static_cast<RefModel *>(h);
+  Model &m = rm->model;
+  std::vector<float const *> Xm(n_data), Ym(n_data);
+  for (size_t i = 0; i < n_data; ++i) {
+    Xm[i] = X + i * K0;
+    Ym[i] = Y + i * Hout;
+  }
+  if (m.ptr_array_derivatives_parameters == nullptr) m.clear_training_arrays();
+  m.type_state_propagation = PROPAGATION::TRAINING;
+  m.update_mem_batch_size(n_data);
+  if (resample_masks && (m.Use__Dropout__Bernoulli() || m.Use__Dropout__Bernoulli__Inverted())) m.Dropout_Bernoulli();
+  m.reset_loss();
+  size_t const batch_size_max = m.batch_size;
+  int const n_batch = static_cast<int>(std::ceil(static_cast<double>(n_data) / static_cast<double>(batch_size_max)));
+  if (m.use_mp && m.is_mp_initialized) {
+    m.update_mem_thread_size(n_data);
+    omp_set_num_threads(static_cast<int>(m.number_threads));
+    int i = 0;
+    size_t batch_size = 0;
+#pragma omp parallel private(i, batch_size)
+    for (i = 0; i < n_batch; ++i) {
+      batch_size = i + 1 != n_batch ? batch_size_max : n_data - static_cast<size_t>(i) * batch_size_max;
+      m.forward_pass(batch_size, Xm.data() + static_cast<size_t>(i) * batch_size_max);
+      m.compute_error(batch_size, Ym.data() + static_cast<size_t>(i) * batch_size_max);
+      m.backward_pass(batch_size);
+      m.update_derivatives(batch_size, m.ptr_array_layers + 1, m.ptr_last_layer);
+    }
+    m.merge_mp_derivatives(0, m.total_parameters);
+    m.merge_mp_accu_loss();
+    m.update_weights_mp(n_data, n_data);
+  } else {
+    for (int i = 0; i < n_batch; ++i) {
+      size_t const batch_size = i + 1 != n_batch ? batch_size_max : n_data - static_cast<size_t>(i) * batch_size_max;
+      m.forward_pass(batch_size, Xm.data() + static_cast<size_t>(i) * batch_size_max);
+      m.compute_error(batch_size, Ym.data() + static_cast<size_t>(i) * batch_size_max);
+      m.backward_pass(batch_size);
+      m.update_derivatives(batch_size, m.ptr_array_layers + 1, m.ptr_last_layer);
+    }
+    m.update_weights_st(n_data, n_data);
+  }
+  m.type_state_propagation = PROPAGATION::INFERENCE;
+  m.epoch_time_step += 1.0f;
+  m.n_acc_trial = n_data * (1 - m.n_time_delay) * (ACCU_FN::CROSS_ENTROPY == m.type_accuracy_function ? 1 : Hout);
+  out[0] = m.get_loss(DL::ENV::NONE);
+  out[1] = m.get_accu(DL::ENV::NONE);
+}
+
+void dlref_model_evalt(void *h, size_t n_data, float const *X, size_t K0, float const *Y, size_t Hout, double *out) {
+  RefModel *rm = static_cast<RefModel *>(h);
+  Model &m = rm->model;
+  std::vector<float const *> Xm(n_data), Ym(n_data);
+  for (size_t i = 0; i < n_data; ++i) {
+    Xm[i] = X + i * K0;
+    Ym[i] = Y + i * Hout;
+  }
+  m.reset_loss();
+  m.type_state_propagation = PROPAGATION::INFERENCE;
+  m.update_mem_batch_size(n_data);
+  size_t const batch_size_max = m.batch_size;
+  int const n_batch = static_cast<int>(std::ceil(static_cast<double>(n_data) / static_cast<double>(batch_size_max)));
+  if (m.use_mp && m.is_mp_initialized) {
+    m.update_mem_thread_size(n_data);
+    omp_set_num_threads(static_cast<int>(m.number_threads));
+    int i = 0;
+    size_t batch_size = 0;
+#pragma omp parallel private(i, batch_size)
+    for (i = 0; i < n_batch; ++i) {
+      batch_size = i + 1 != n_batch ? batch_size_max : n_data - static_cast<size_t>(i) * batch_size_max;
+      m.forward_pass(batch_size, Xm.data() + static_cast<size_t>(i) * batch_size_max);
+      m.compute_loss(batch_size, Ym.data() + static_cast<size_t>(i) * batch_size_max);
+    }
+    m.merge_mp_accu_loss();
+  } else {
+    for (int i = 0; i < n_batch; ++i) {
+      size_t const batch_size = i + 1 != n_batch ? batch_size_max : n_data - static_cast<size_t>(i) * batch_size_max;
+      m.forward_pass(batch_size, Xm.data() + static_cast<size_t>(i) * batch_size_max);
+      m.compute_loss(batch_size, Ym.data() + static_cast<size_t>(i) * batch_size_max);
+    }
+  }
+  m.n_acc_trial = n_data * (1 - m.n_time_delay) * (ACCU_FN::CROSS_ENTROPY == m.type_accuracy_function ? 1 : Hout);
+  out[0] = m.get_loss(DL::ENV::NONE);
+  out[1] = m.get_accu(DL::ENV::NONE);
+}
+size_t dlref_model_batch_size(void *h) { return static_cast<RefModel *>(h)->model.batch_size; }
 
 }  // extern "C"

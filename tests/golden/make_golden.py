@@ -282,8 +282,66 @@ def optimizers(R):
     return len(d)
 
 
+EPOCH_CASES = {
+    # name: (widths, n_data, sub-batch, hidden (act, norm, drop, keep), optimizer, settings)
+    "epoch_adam_brn": ([20, 16, 16, 10], 50, 16, [("RELU", "BRN", "NONE", 1.0)] * 2, "ADAM",
+                       dict(adam_lr=0.01, weight_decay=0.01)),
+    "epoch_nesterov_dropout": ([12, 24, 9, 5], 37, 37, [("ELU", "BRN", "BERNOULLI_INVERTED", 0.8),
+                                                         ("LEAKY_RELU", "NONE", "NONE", 1.0)], "GD",
+                               dict(lr=0.05, momentum=0.9, nesterov=True)),
+    "epoch_gd_even_batches": ([10, 8, 8, 4], 48, 12, [("SELU", "BN", "NONE", 1.0), ("ISRLU", "BN", "NONE", 1.0)], "GD",
+                              dict(lr=0.1, momentum=0.0, weight_decay=0.02, normalized_wd=False)),
+}
+EPOCHS = 3
+
+
+def epochs(R):
+    """Driver::train three times, then Driver::evalt, on one small data set:
+    loss, accuracy, parameters and moving statistics after every epoch."""
+    d = {"epoch_cases_json": np.frombuffer(json.dumps(EPOCH_CASES).encode(), dtype=np.uint8)}
+    for name, (widths, n, sub, hidden, kind, kw) in EPOCH_CASES.items():
+        rng = np.random.default_rng(sum(map(ord, name)))
+        L = len(widths)
+        X = f32(rng.uniform(0, 1, (n, widths[0])))
+        Y = f32(np.eye(widths[-1])[rng.integers(0, widths[-1], n)])
+        masks = {l: (rng.uniform(size=widths[l]) < hidden[l - 1][3]).astype(np.uint8) for l in range(1, L - 1)}
+        d[name + "_X"], d[name + "_Y"] = X, Y
+        for l, mk in masks.items():
+            d[f"{name}_mask{l}"] = mk
+        params = None
+        for nt in THREADS:
+            M = R.mlp(widths)
+            for l in range(1, L - 1):
+                a, nm, dr, keep = hidden[l - 1]
+                M.set_layer(l, ACT[a], NORM[nm], DROP[dr], keep, masks[l] if dr != "NONE" else None)
+            M.set_layer(L - 1, ACT["SOFTMAX"])
+            M.set_norm_hyper(0.9, 1e-5, 3.0, 5.0)
+            M.prepare(sub, nt)
+            if params is None:
+                params = M.get_parameters()
+                for l in range(1, L):
+                    o = M.layer_offsets(l)
+                    K, H = widths[l - 1], widths[l]
+                    params[o[0]:o[0] + H * K] = glorot(rng, H, K).ravel()
+                d[name + "_params"] = params.copy()
+            M.set_parameters(params)
+            M.set_optimizer(OPT[kind], **kw)
+            q = f"{name}_t{nt}_"
+            la = []
+            for e in range(EPOCHS):
+                la.append(M.train_epoch(X, Y, resample_masks=False))
+                d[f"{q}e{e}_params"] = M.get_parameters()
+            la.append(M.evalt(X, Y))
+            d[q + "loss_accu"] = np.array(la, dtype=np.float64)  # rows: epochs 0..2 (training), evaluation
+            mm, ms = M.get_moving()
+            d[q + "mov_mean"], d[q + "mov_std"] = mm, ms
+    np.savez_compressed(os.path.join(OUT, "epoch.npz"), **d)
+    return len(d)
+
+
 if __name__ == "__main__":
     R = Reference()
     print("leaves:", leaves(R), "arrays")
     print("mlp:", mlps(R), "arrays")
     print("optim:", optimizers(R), "arrays")
+    print("epoch:", epochs(R), "arrays")
