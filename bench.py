@@ -1,6 +1,6 @@
 """Benchmark of the fully-connected + batch-renorm + activation hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c5|c1]
 
 A "step" is one forward + backward pass of the layer over one synthetic batch
 resident in HBM:  Z = X W^T (+bias) -> batch renorm -> activation, then
@@ -194,12 +194,90 @@ def cpu_baseline(name, budget_rows):
                       % (Bs, B, dt, nt, model)}
 
 
+def bench_c1(args):
+    """Workload c1: MLP 784-512-512-10, batch 128, batch renorm + ReLU hidden layers, softmax +
+    cross-entropy output, through the Model / Driver facade.  A step is one forward + error +
+    backward + parameter-gradient pass over one batch of 128 rows (data set resident in HBM); every
+    64 steps Driver::train ends in one Adam update.  Launch- and latency-bound: about 25 kernel
+    launches of a few microseconds each per step."""
+    import numpy as np
+    from __graft_entry__ import load_package
+    from oracle.binding import ACT, NORM, OPT
+    pkg = load_package()
+    from deep_learning_amd.model import Model
+    widths, B, per_epoch = [784, 512, 512, 10], 128, 64
+    n = B * per_epoch
+    rng = np.random.default_rng(1234)
+    X = rng.random((n, widths[0]), dtype=np.float32)
+    Y = np.eye(widths[-1], dtype=np.float32)[rng.integers(0, widths[-1], n)]
+
+    def build(make):
+        M = make(widths)
+        for l in (1, 2):
+            M.set_layer(l, ACT["RELU"], NORM["BRN"])
+        M.set_layer(3, ACT["SOFTMAX"])
+        M.set_norm_hyper(HYPER["momentum"], HYPER["eps"], HYPER["r_max"], HYPER["d_max"])
+        return M
+
+    M = build(lambda w: Model(pkg.load_library(), w))  # raises without the HIP library or a GPU
+    M.prepare(B)
+    p = M.get_parameters()
+    for l in range(1, 4):
+        o = M.layer_offsets(l)
+        K, H = widths[l - 1], widths[l]
+        p[o[0]:o[0] + H * K] = ((rng.random(H * K, dtype=np.float32) * 2 - 1) * np.float32((6.0 / (K + H)) ** 0.5))
+    M.set_parameters(p)
+    M.set_optimizer(OPT["ADAM"], adam_lr=1e-3)
+    epochs = max(1, args.steps // per_epoch)
+    for _ in range(max(1, args.warmup // per_epoch)):
+        M.train_epoch(X, Y)
+    t0 = time.perf_counter()
+    for _ in range(epochs):
+        loss, accu = M.train_epoch(X, Y)  # returns after the loss has been read back: the stream is idle
+    dt = time.perf_counter() - t0
+    steps = epochs * per_epoch
+    ms = dt / steps * 1e3
+    flops = 2.0 * B * (784 * 512 + 512 * 512 + 512 * 10) * 2 + 2.0 * B * (512 * 512 + 512 * 10)  # fwd + dW, dX of layers 2, 3
+    roof = {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "traffic": None, "kernel": "whole step (launch-bound: the GEMMs are 128 x 512 x 784 and smaller)"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    cpu = None
+    if args.cpu_rows != 0:
+        from oracle.binding import Oracle, OracleMLP, Reference, reference_available
+        kind = "reference" if reference_available() else "port"
+        nt = max(1, min(int(os.environ.get("OMP_NUM_THREADS", "0")) or 16, os.cpu_count() or 1, 64))
+        R = build((lambda w: Reference().mlp(w)) if kind == "reference" else (lambda w: OracleMLP(Oracle(), w)))
+        R.prepare(B, nt)
+        if kind == "reference":
+            R.set_parameters(p)
+        else:
+            R.parameters[:] = p
+        R.set_optimizer(OPT["ADAM"], adam_lr=1e-3)
+        R.train_epoch(X[:B * 4], Y[:B * 4])
+        t1 = time.perf_counter()
+        R.train_epoch(X, Y)
+        dtc = time.perf_counter() - t1
+        cpu = {"value": n / dtc, "unit": "samples/s", "cores": nt, "kind": kind,
+               "sample": "one Driver::train epoch over the same %d rows in batches of %d, %.1f s, %d OpenMP threads"
+                         % (n, B, dtc, nt)}
+    out = {"metric": "FC+BRN+act fwd+bwd samples/sec; % HBM peak (norm/act), % FP32 MFMA peak (GEMM)",
+           "value": B / (ms * 1e-3), "unit": "samples/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+           "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+           "data": "synthetic",
+           "config": {"workload": "c1: MLP 784-512-512-10, batch 128, batch renorm + ReLU, softmax cross-entropy, "
+                                  "fwd+bwd per batch, Adam update every 64 batches (Driver::train)",
+                      "batch": B, "inputs": "resident in HBM"},
+           "roofline": roof, "cpu_baseline": cpu, "detail": {"final_loss": loss, "final_accuracy": accu}}
+    print(json.dumps(out))
+    M.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c1"])
     ap.add_argument("--cpu-rows", type=int, default=-1, help="rows of the CPU baseline sample (0 = skip)")
     ap.add_argument("--only", default="", help="profiling aid: run just this part (gemm_fwd, gemm_dx, gemm_dw, "
                                                "norm_fwd, norm_bwd, fc_norm_fwd, adam, copy) --steps times and exit "
@@ -208,6 +286,12 @@ def main():
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
+
+    if args.workload == "c1":
+        if args.steps == 20:
+            args.steps = 640  # ten epochs of 64 batches unless told otherwise
+        bench_c1(args)
+        return
 
     import torch
     from __graft_entry__ import load_package

@@ -53,6 +53,7 @@ struct GemmArgs {
   float *split_out;    // when gridDim.z > 1: [splits][M][N] partial products
   float *stats_out;    // optional [2][tiles_m][N]: per tile-row column sums of C and C^2 (gridDim.z == 1)
   int accumulate;      // C += result (only when gridDim.z == 1)
+  int a_vec, b_vec;    // operand base and leading dimension allow 16-byte loads (ragged variant)
   unsigned tiles_m, tiles_n;
 };
 
@@ -97,7 +98,8 @@ struct TileShape {
 template <int ROWS, int BK, bool KCONTIG, bool FAST>
 __device__ __forceinline__ typename TileShape<ROWS, BK, KCONTIG>::Regs tile_load(float const *__restrict__ P,
                                                                                size_t ld, size_t row0, size_t k0,
-                                                                               size_t rows_total, size_t k_end) {
+                                                                               size_t rows_total, size_t k_end,
+                                                                               bool vec_ok) {
   using T = TileShape<ROWS, BK, KCONTIG>;
   typename T::Regs regs;
 #pragma unroll
@@ -105,16 +107,25 @@ __device__ __forceinline__ typename TileShape<ROWS, BK, KCONTIG>::Regs tile_load
     int tr, tk;
     T::piece(threadIdx.x + i * kGemmThreads, tr, tk);
     size_t const row = row0 + tr, k = k0 + tk;
+    float const *src = KCONTIG ? P + row * ld + k : P + k * ld + row;
     v4f t;
     if constexpr (FAST) {
-      float const *src = KCONTIG ? P + row * ld + k : P + k * ld + row;
+      (void)vec_ok;
       t = *reinterpret_cast<v4f const *>(src);
     } else {
+      // ragged shape: a piece that lies wholly inside the operand still moves as
+      // one 16-byte load when the operand's alignment allows (vec_ok); only the
+      // pieces on the edge go element by element, zero-filled outside
+      bool const whole = KCONTIG ? (row < rows_total && k + 3 < k_end) : (row + 3 < rows_total && k < k_end);
+      if (vec_ok && whole) {
+        t = *reinterpret_cast<v4f const *>(src);
+      } else {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        size_t const rr = KCONTIG ? row : row + e;
-        size_t const kk = KCONTIG ? k + e : k;
-        t[e] = (rr < rows_total && kk < k_end) ? (KCONTIG ? P[rr * ld + kk] : P[kk * ld + rr]) : 0.0f;
+        for (int e = 0; e < 4; ++e) {
+          size_t const rr = KCONTIG ? row : row + e;
+          size_t const kk = KCONTIG ? k + e : k;
+          t[e] = (rr < rows_total && kk < k_end) ? (KCONTIG ? P[rr * ld + kk] : P[kk * ld + rr]) : 0.0f;
+        }
       }
     }
 #pragma unroll
@@ -242,13 +253,13 @@ void k_gemm_f32(GemmArgs g) {
     // stage and the writes of the next - the first fragments of tile kt+1 are
     // read.  LDS and memory traffic is spread between the MFMAs, so the matrix
     // pipe only waits at the barrier itself.
-    typename TA::Regs ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, k_begin, g.M, k_end);
-    typename TB::Regs rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, k_begin, g.N, k_end);
+    typename TA::Regs ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, k_begin, g.M, k_end, g.a_vec != 0);
+    typename TB::Regs rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, k_begin, g.N, k_end, g.b_vec != 0);
     tile_store<BM, BK, A_KCONTIG>(lds, ra);
     tile_store<BN, BK, B_KCONTIG>(lds + TA::kFloats, rb);
     if (ktiles > 1) {
-      ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, k_begin + BK, g.M, k_end);
-      rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, k_begin + BK, g.N, k_end);
+      ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, k_begin + BK, g.M, k_end, g.a_vec != 0);
+      rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, k_begin + BK, g.N, k_end, g.b_vec != 0);
     }
     __syncthreads();
     v4f f0a[TM], f0b[TN];
@@ -268,8 +279,8 @@ void k_gemm_f32(GemmArgs g) {
       }
       if constexpr (LOAD) {
         size_t const kn = k_begin + static_cast<size_t>(kt + 2) * BK;
-        ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, kn, g.M, k_end);
-        rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, kn, g.N, k_end);
+        ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, kn, g.M, k_end, g.a_vec != 0);
+        rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, kn, g.N, k_end, g.b_vec != 0);
       }
       steps(f1a, f1b, 0, 2);
       if constexpr (FAST) {
@@ -435,7 +446,7 @@ struct TileCfg {
   int bm, bn, bk;
 };
 
-// Tuning aid: DLMI_GEMM_TILE=<index> forces a tile shape (0: 128x128, 1: 256x128, 2: 256x256).
+// Tuning aid: DLMI_GEMM_TILE=<index> forces a tile shape (0: 128x128, 1: 256x128, 2: 256x256, 3: 64x64).
 static int tile_choice() {
   static int const c = [] {
     char const *e = std::getenv("DLMI_GEMM_TILE");
@@ -450,19 +461,23 @@ static int tile_choice() {
 template <bool AK, bool BKC>
 static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, size_t lda, float const *B, size_t ldb,
                 float *C, float const *bias, int accumulate, unsigned *stats_chunks = nullptr) {
-  static TileCfg const cfgs[] = {{128, 128, 16}, {256, 128, 16}, {256, 256, 16}};
+  static TileCfg const cfgs[] = {{128, 128, 16}, {256, 128, 16}, {256, 256, 16}, {64, 64, 16}};
   int choice = tile_choice();
   if (choice < 0 || choice >= static_cast<int>(sizeof(cfgs) / sizeof(cfgs[0]))) {
     // default: the shape with the smallest estimated time = rounds of workgroups
-    // over the CUs x work per round / measured relative efficiency of the shape
-    // (256 x 256 runs one workgroup per CU, the smaller shapes two)
-    static int const per_cu[] = {2, 2, 1};
-    static double const eff[] = {0.95, 0.97, 1.0};
+    // over the CUs x work of one workgroup x workgroups sharing a CU / measured
+    // relative efficiency of the shape (256 x 256 runs one workgroup per CU,
+    // 128-wide shapes two, 64 x 64 four).  A small output picks small tiles: a
+    // workgroup's time is its own MFMA count as long as it has a CU to itself.
+    static int const per_cu[] = {2, 2, 1, 4};
+    static double const eff[] = {0.95, 0.97, 1.0, 0.8};
     double best = 0.0;
     for (int c = 0; c < static_cast<int>(sizeof(cfgs) / sizeof(cfgs[0])); ++c) {
       size_t const tiles = dlmi_ceil_div(M, cfgs[c].bm) * dlmi_ceil_div(N, cfgs[c].bn);
-      size_t const rounds = dlmi_ceil_div(tiles, static_cast<size_t>(ctx->num_cu) * per_cu[c]);
-      double const t = static_cast<double>(rounds) * cfgs[c].bm * cfgs[c].bn * per_cu[c] / eff[c];
+      size_t const slots = static_cast<size_t>(ctx->num_cu) * per_cu[c];
+      size_t const rounds = dlmi_ceil_div(tiles, slots);
+      size_t const sharing = dlmi_ceil_div(tiles < slots ? tiles : slots, static_cast<size_t>(ctx->num_cu));
+      double const t = static_cast<double>(rounds) * cfgs[c].bm * cfgs[c].bn * sharing / eff[c];
       if (c == 0 || t < best) {
         best = t;
         choice = c;
@@ -474,21 +489,16 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   GemmArgs g;
   g.A = A; g.B = B; g.C = C; g.bias = bias; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldc = N;
   g.accumulate = accumulate; g.split_out = nullptr; g.stats_out = nullptr;
-  if (stats_chunks != nullptr) {
-    *stats_chunks = static_cast<unsigned>(dlmi_ceil_div(M, bm));
-    int rc = dlmi_scratch_reserve(ctx, 2 * 2 * static_cast<size_t>(*stats_chunks) * N * sizeof(float));
-    if (rc != DLMI_OK) return rc;
-    g.stats_out = reinterpret_cast<float *>(ctx->scratch);
-  }
-  bool const fast = M % bm == 0 && N % bn == 0 && K % bk == 0 && lda % 4 == 0 && ldb % 4 == 0 &&
-                    dlmi_aligned16(A) && dlmi_aligned16(B);
+  g.a_vec = (lda % 4 == 0 && dlmi_aligned16(A)) ? 1 : 0;
+  g.b_vec = (ldb % 4 == 0 && dlmi_aligned16(B)) ? 1 : 0;
+  bool const fast = M % bm == 0 && N % bn == 0 && K % bk == 0 && g.a_vec && g.b_vec;
   // Split K when the output alone cannot fill the machine (few tiles, long K):
   // each slice writes its partial product, a second kernel adds them in order.
   size_t const tiles = dlmi_ceil_div(M, bm) * dlmi_ceil_div(N, bn);
   size_t const ktiles = dlmi_ceil_div(K, bk);
   unsigned splits = 1;
   size_t const target = static_cast<size_t>(ctx->num_cu) * 2;
-  if (tiles < target / 2 && ktiles >= 16 && stats_chunks == nullptr) {
+  if (tiles < target / 2 && ktiles >= 16) {
     size_t s = dlmi_ceil_div(target, tiles);
     size_t const max_s = ktiles / 8;  // at least 8 K tiles per slice
     if (s > max_s) s = max_s;
@@ -496,6 +506,16 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
       int rc = dlmi_scratch_reserve(ctx, s * M * N * sizeof(float));
       if (rc != DLMI_OK) return rc;
       splits = static_cast<unsigned>(s);
+    }
+  }
+  if (stats_chunks != nullptr) {
+    if (splits > 1) {
+      *stats_chunks = 0;  // the slices hold partial products: the caller takes the statistics from C itself
+    } else {
+      *stats_chunks = static_cast<unsigned>(dlmi_ceil_div(M, bm));
+      int rc = dlmi_scratch_reserve(ctx, 2 * 2 * static_cast<size_t>(*stats_chunks) * N * sizeof(float));
+      if (rc != DLMI_OK) return rc;
+      g.stats_out = reinterpret_cast<float *>(ctx->scratch);
     }
   }
   size_t const kt_per_split = dlmi_ceil_div(ktiles, splits);
@@ -506,6 +526,7 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   switch (choice) {
     case 1: rc = launch_gemm<256, 128, 16, AK, BKC, 2>(ctx, g, splits, fast); break;
     case 2: rc = launch_gemm<256, 256, 16, AK, BKC, 1>(ctx, g, splits, fast); break;
+    case 3: rc = launch_gemm<64, 64, 16, AK, BKC, 4>(ctx, g, splits, fast); break;
     default: rc = launch_gemm<128, 128, 16, AK, BKC, 2>(ctx, g, splits, fast); break;
   }
   if (rc != DLMI_OK) return rc;
@@ -544,8 +565,10 @@ int dlmi_fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, s
   unsigned chunks = 0;
   int rc = gemm<true, true>(ctx, B, H, K, X, K, W, K, Z, nullptr, 0, &chunks);
   if (rc != DLMI_OK) return rc;
+  // a small output runs split over K, where no slice sees whole sums: the
+  // statistics then come from a pass over Z (nullptr / 0)
   return fused_fwd_from_partials(ctx, desc, B, H, Z, gamma, beta, mask, mean, stdv, mov_mean, mov_std, r, d, y,
-                                 reinterpret_cast<float const *>(ctx->scratch), chunks);
+                                 chunks != 0 ? reinterpret_cast<float const *>(ctx->scratch) : nullptr, chunks);
 }
 
 int dlmi_fc_bwd_dx(dlmi_ctx *ctx, size_t B, size_t Hn, size_t H, float const *dZn, float const *Wn, float *dY,
