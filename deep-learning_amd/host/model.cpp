@@ -263,7 +263,7 @@ bool Model::set_max_batch_size(size_t const n) {
 void Model::free_batch(void) {
   if (ptr_array_layers != nullptr)
     for (Layer *l = ptr_array_layers; l != ptr_last_layer; ++l) {
-      dev_free(l->d_summations); dev_free(l->d_outputs); dev_free(l->d_errors);
+      dev_free(l->d_summations); dev_free(l->d_outputs); dev_free(l->d_errors); dev_free(l->d_af_values);
     }
   dev_free(impl_->d_input);
   dev_free(impl_->d_targets);
@@ -278,6 +278,10 @@ bool Model::allocate_batch(size_t const n) {
     Layer &l = ptr_array_layers[i];
     if (!dev_alloc(&l.d_summations, n * l.n_out, err) || !dev_alloc(&l.d_outputs, n * l.n_out, err) ||
         !dev_alloc(&l.d_errors, n * l.n_out, err))
+      return false;
+    // normalization after the activation keeps the activation values as well
+    if (l.Use__Normalization() && !l.use_layer_normalization_before_activation &&
+        !dev_alloc(&l.d_af_values, n * l.n_out, err))
       return false;
   }
   size_t const n_in = ptr_array_layers[0].n_out, n_o = ptr_array_layers[total_layers - 1].n_out;
@@ -436,10 +440,36 @@ void Model::forward_layers(size_t const B) {
     float const *bias = l.Use__Bias() ? impl_->d_params + l.first_bias_connection_index : nullptr;
     bool const softmax = l.type_activation_function == ACTIVATION::SOFTMAX;
     if (!softmax && !act_on_path(l.type_activation_function)) { fail("forward_pass: layer activation not set to one on this path"); return; }
-    bool const fused_fc_norm = l.Use__Normalization() && training;  // the GEMM epilogue takes the batch statistics
+    bool const norm_after = l.Use__Normalization() && !l.use_layer_normalization_before_activation;
+    // the GEMM epilogue takes the batch statistics when the normalization follows the GEMM directly
+    bool const fused_fc_norm = l.Use__Normalization() && training && !norm_after;
     if (!fused_fc_norm && dlmi_fc_fwd(ctx, B, K, H, in, W, bias, l.d_summations) != DLMI_OK) { fail("forward_pass: dlmi_fc_fwd"); return; }
     int rc = DLMI_OK;
-    if (l.Use__Normalization()) {
+    if (norm_after) {
+      // fwp_st.cpp:405-511 / 596-655: activation, then the normalization of the
+      // activation values; dropout then acts on the normalized values
+      // (fwp_st.cpp:657-732), which are the layer's output
+      if (softmax) { fail("forward_pass: softmax layers are not normalized"); return; }
+      if (l.d_af_values == nullptr) { fail("forward_pass: call update_mem_batch_size() after changing the normalization order"); return; }
+      dlmi_fused_desc d = make_desc(*this, l);
+      d.act = DLMI_ACT_LINEAR;
+      float const *gamma = impl_->d_params + l.scale_index, *beta = impl_->d_params + l.shift_index;
+      float *mm = impl_->d_mov_mean + l.unit_index, *ms = impl_->d_mov_std + l.unit_index;
+      rc = dlmi_act_fwd(ctx, static_cast<dlmi_activation>(l.type_activation_function), B, H, l.d_summations, l.d_af_values);
+      if (rc == DLMI_OK) {
+        if (training) {
+          if (type_state_propagation != PROPAGATION::TRAINING) d.dropout = DLMI_DROP_NONE;
+          rc = dlmi_fused_norm_act_fwd(ctx, &d, B, H, l.d_af_values, gamma, beta, l.d_mask, l.d_mean, l.d_std, mm, ms,
+                                       l.d_r, l.d_d, l.d_outputs);
+          if (rc == DLMI_OK && type_state_propagation != PROPAGATION::TRAINING && l.Use__Dropout())
+            rc = dlmi_dropout_fwd(ctx, static_cast<dlmi_dropout>(l.type_dropout), 0, 0, B, H, nullptr,
+                                  l.dropout_values[0], l.d_outputs);
+        } else {
+          d.drop_scale = l.dropout_values[0];
+          rc = dlmi_fused_norm_act_infer(ctx, &d, B, H, l.d_af_values, gamma, beta, mm, ms, l.d_outputs);
+        }
+      }
+    } else if (l.Use__Normalization()) {
       dlmi_fused_desc d = make_desc(*this, l);
       float const *gamma = impl_->d_params + l.scale_index, *beta = impl_->d_params + l.shift_index;
       float *mm = impl_->d_mov_mean + l.unit_index, *ms = impl_->d_mov_std + l.unit_index;
@@ -593,7 +623,20 @@ void Model::backward_pass(size_t const B) {
       return;
     }
     int rc;
-    if (l.Use__Normalization()) {
+    if (l.Use__Normalization() && !l.use_layer_normalization_before_activation) {
+      // bwp_st.cpp:559-606, 619-632: normalization backward on the activation
+      // values (in REFERENCE dropout mode the gradient passes unmasked), then the
+      // activation derivative with the summations and the activation values
+      dlmi_fused_desc d = make_desc(*this, l);
+      d.act = DLMI_ACT_LINEAR;
+      if (type_state_propagation != PROPAGATION::TRAINING) d.dropout = DLMI_DROP_NONE;
+      rc = dlmi_fused_norm_act_bwd(ctx, &d, B, H, l.d_af_values, impl_->d_params + l.scale_index,
+                                   impl_->d_params + l.shift_index, l.d_mask, l.d_mean, l.d_std, l.d_r, l.d_d, l.d_errors,
+                                   impl_->d_dparams + l.scale_index, impl_->d_dparams + l.shift_index, l.d_errors);
+      if (rc == DLMI_OK)
+        rc = dlmi_act_bwd(ctx, static_cast<dlmi_activation>(l.type_activation_function), B, H, l.d_summations,
+                          l.d_af_values, l.d_errors, l.d_errors);
+    } else if (l.Use__Normalization()) {
       dlmi_fused_desc d = make_desc(*this, l);
       if (type_state_propagation != PROPAGATION::TRAINING) d.dropout = DLMI_DROP_NONE;
       rc = dlmi_fused_norm_act_bwd(ctx, &d, B, H, l.d_summations, impl_->d_params + l.scale_index,

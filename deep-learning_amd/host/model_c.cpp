@@ -48,6 +48,11 @@ int dlmi_model_set_layer_activation_function(dlmi_model *h, size_t layer, int a)
 int dlmi_model_set_layer_normalization(dlmi_model *h, size_t layer, int n) {
   return h->m.Set__Layer_Normalization(layer, static_cast<LAYER_NORM::TYPE>(n));
 }
+int dlmi_model_set_layer_normalization_order(dlmi_model *h, size_t layer, int before_activation) {
+  if (h->m.ptr_array_layers == nullptr || layer >= h->m.total_layers) return 0;
+  h->m.ptr_array_layers[layer].use_layer_normalization_before_activation = before_activation != 0;
+  return 1;
+}
 int dlmi_model_set_norm_hyper(dlmi_model *h, float momentum, float eps, float r_max, float d_max) {
   bool ok = h->m.Set__Normalization_Momentum_Average(momentum);
   ok = h->m.Set__Normalization_Epsilon(eps) && ok;

@@ -14,7 +14,7 @@ vp = ctypes.c_void_p
 
 MODEL_C_ABI_SYMBOLS = [
     "dlmi_model_create", "dlmi_model_destroy", "dlmi_model_last_error", "dlmi_model_set_layer_activation_function",
-    "dlmi_model_set_layer_normalization", "dlmi_model_set_norm_hyper", "dlmi_model_set_dropout",
+    "dlmi_model_set_layer_normalization", "dlmi_model_set_layer_normalization_order", "dlmi_model_set_norm_hyper", "dlmi_model_set_dropout",
     "dlmi_model_set_dropout_mask", "dlmi_model_set_dropout_backward_mode", "dlmi_model_prepare",
     "dlmi_model_total_parameters", "dlmi_model_total_normalized_units", "dlmi_model_layer_offsets",
     "dlmi_model_set_parameters", "dlmi_model_get_parameters", "dlmi_model_set_moving", "dlmi_model_get_moving",
@@ -70,9 +70,11 @@ class Model:
         if not rc:
             raise RuntimeError("%s failed: %s" % (what, self.lib.dlmi_model_last_error(self.h).decode()))
 
-    def set_layer(self, l, act, norm=0, drop=0, keep=1.0, mask=None):
+    def set_layer(self, l, act, norm=0, drop=0, keep=1.0, mask=None, norm_before=True):
         self._ok(self.lib.dlmi_model_set_layer_activation_function(self.h, c_sz(l), c_int(act)), "activation")
         if norm:
+            self._ok(self.lib.dlmi_model_set_layer_normalization_order(self.h, c_sz(l), c_int(int(norm_before))),
+                     "normalization order")
             self._ok(self.lib.dlmi_model_set_layer_normalization(self.h, c_sz(l), c_int(norm)), "normalization")
         if drop:
             self._ok(self.lib.dlmi_model_set_dropout(self.h, c_sz(l), c_int(drop), c_f(keep)), "dropout")

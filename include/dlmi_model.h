@@ -22,6 +22,8 @@ void dlmi_model_destroy(dlmi_model *m);
 char const *dlmi_model_last_error(dlmi_model const *m);
 int dlmi_model_set_layer_activation_function(dlmi_model *m, size_t layer, int activation);
 int dlmi_model_set_layer_normalization(dlmi_model *m, size_t layer, int norm);
+/* Layer::use_layer_normalization_before_activation (model.hpp:573), assigned as user_controls.cpp:1974 does */
+int dlmi_model_set_layer_normalization_order(dlmi_model *m, size_t layer, int before_activation);
 int dlmi_model_set_norm_hyper(dlmi_model *m, float momentum, float eps, float r_max, float d_max);
 int dlmi_model_set_dropout(dlmi_model *m, size_t layer, int dropout, float keep);
 int dlmi_model_set_dropout_mask(dlmi_model *m, size_t layer, uint8_t const *mask_per_unit);

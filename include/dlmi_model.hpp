@@ -89,6 +89,8 @@ struct Layer {
   float *d_summations = nullptr;          // Z (Neuron_unit::ptr_array_summations)
   float *d_outputs = nullptr;             // layer output after activation and dropout (ptr_array_outputs)
   float *d_errors = nullptr;              // dZ (Neuron_unit::ptr_array_errors); holds dY in between
+  float *d_af_values = nullptr;           // activation values (AF_unit::ptr_array_values), kept only when the
+                                          // normalization comes after the activation
   float *d_mean = nullptr, *d_std = nullptr, *d_r = nullptr, *d_d = nullptr;  // batch statistics [n_out]
   uint8_t *d_mask = nullptr;              // device copy of the dropout mask [n_out]
 

@@ -317,9 +317,10 @@ class OracleMLP:
         except Exception:
             pass
 
-    def set_layer(self, l, act, norm=0, drop=0, keep=1.0, mask=None):
+    def set_layer(self, l, act, norm=0, drop=0, keep=1.0, mask=None, norm_before=True):
         m = None if mask is None else np.ascontiguousarray(mask, dtype=np.uint8)
         self.lib.dlo_mlp_set_layer(self.h, c_sz(l), c_int(act), c_int(norm), c_int(drop), c_f(keep), _ptr(m))
+        self.lib.dlo_mlp_set_norm_order(self.h, c_sz(l), c_int(int(norm_before)))
 
     def set_norm_hyper(self, momentum, eps, r_max, d_max):
         self.lib.dlo_mlp_set_norm_hyper(self.h, c_f(momentum), c_f(eps), c_f(r_max), c_f(d_max))
@@ -489,10 +490,11 @@ class ReferenceMLP:
         except Exception:
             pass
 
-    def set_layer(self, l, act, norm=0, drop=0, keep=1.0, mask=None):
+    def set_layer(self, l, act, norm=0, drop=0, keep=1.0, mask=None, norm_before=True):
         ok = self.lib.dlref_model_set_activation(self.h, c_sz(l), c_int(act))
         assert ok, "set_layer_activation_function refused"
         if norm:
+            self.lib.dlref_model_set_norm_order(self.h, c_sz(l), c_int(int(norm_before)))
             ok = self.lib.dlref_model_set_normalization(self.h, c_sz(l), c_int(norm))
             assert ok, "Set__Layer_Normalization refused"
         if drop:

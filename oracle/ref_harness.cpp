@@ -377,6 +377,14 @@ int dlref_model_set_normalization(void *h, size_t layer, int type) {
       layer, static_cast<LAYER_NORM::TYPE>(type));
 }
 
+// Layer::use_layer_normalization_before_activation (model.hpp:573), assigned like
+// user_controls.cpp:1974 does.  Call BEFORE dlref_model_set_normalization: that
+// call wires the layer's buffers according to the flag (ordering.cpp:150-175).
+void dlref_model_set_norm_order(void *h, size_t layer, int before_activation) {
+  static_cast<RefModel *>(h)->model.ptr_array_layers[layer].use_layer_normalization_before_activation =
+      before_activation != 0;
+}
+
 int dlref_model_set_norm_hyper(void *h, float momentum, float eps, float r_max,
                                float d_max) {
   Model &m = static_cast<RefModel *>(h)->model;

@@ -29,6 +29,17 @@ def f32(a):
     return np.ascontiguousarray(a, dtype=np.float32)
 
 
+def save(name, d):
+    """Writes tests/golden/<name> unless the file already holds exactly these
+    arrays (an npz is a zip: rewriting it would change its bytes for nothing)."""
+    path = os.path.join(OUT, name)
+    if os.path.exists(path):
+        old = np.load(path, allow_pickle=False)
+        if set(old.files) == set(d) and all(np.array_equal(old[k], np.asarray(d[k])) for k in d):
+            return
+    np.savez_compressed(path, **d)
+
+
 def leaves(R):
     rng = np.random.default_rng(20240607)
     d = {}
@@ -94,7 +105,7 @@ def leaves(R):
         y = R.act_fwd(ACT[a], pts, 0)
         d[f"pts_fwd_{a}"] = y
         d[f"pts_bwd_{a}"] = R.act_bwd(ACT[a], pts, y, ones, 0)
-    np.savez_compressed(os.path.join(OUT, "leaves.npz"), **d)
+    save("leaves.npz", d)
     return len(d)
 
 
@@ -184,7 +195,7 @@ def mlps(R):
             M.step(STATE["INFERENCE"], X, None, backward=False)
             for l in range(1, L):
                 d[f"{q}infer_L{l}_out"] = M.layer_buffer(l, 3)
-    np.savez_compressed(os.path.join(OUT, "mlp.npz"), **d)
+    save("mlp.npz", d)
     return len(d)
 
 
@@ -278,7 +289,7 @@ def optimizers(R):
                 d[f"{name}_t{nt}_s{t}_params"] = M.get_parameters()
             mm, ms = M.get_moving()
             d[f"{name}_t{nt}_mov_mean"], d[f"{name}_t{nt}_mov_std"] = mm, ms
-    np.savez_compressed(os.path.join(OUT, "optim.npz"), **d)
+    save("optim.npz", d)
     return len(d)
 
 
@@ -335,7 +346,71 @@ def epochs(R):
             d[q + "loss_accu"] = np.array(la, dtype=np.float64)  # rows: epochs 0..2 (training), evaluation
             mm, ms = M.get_moving()
             d[q + "mov_mean"], d[q + "mov_std"] = mm, ms
-    np.savez_compressed(os.path.join(OUT, "epoch.npz"), **d)
+    save("epoch.npz", d)
+    return len(d)
+
+
+VARIANT_CASES = {
+    # name: (widths, B, hidden (act, norm, drop, keep, normalization before the activation), hyper)
+    "var_norm_after": ([9, 7, 12, 5, 4], 11, [("SELU", "BRN", "BERNOULLI_INVERTED", 0.8, False),
+                                              ("ELU", "BRN", "NONE", 1.0, True),
+                                              ("ISRLU", "BRN", "BERNOULLI", 0.6, False)], (0.3, 1e-3, 1.2, 0.1)),
+    "var_norm_after_bn": ([6, 10, 8, 3], 13, [("LEAKY_RELU", "BN", "NONE", 1.0, False),
+                                              ("RELU", "BN", "BERNOULLI_INVERTED", 0.7, False)], (0.1, 1e-5, 1.0, 0.0)),
+    "var_before_dropout": ([8, 6, 6, 3], 9, [("ELU", "BRN", "BERNOULLI", 0.5, True),
+                                             ("SELU", "NONE", "BERNOULLI_INVERTED", 0.5, True)], (0.9, 1e-5, 3.0, 5.0)),
+}
+
+
+def variants(R):
+    """Layer orderings and propagation states beyond mlp.npz: normalization after
+    the activation (fwp_st.cpp:466-511, bwp_st.cpp:559-606) and the
+    PROPAGATION::UPDATE_BATCH_NORM forward (batch statistics, no dropout mask)."""
+    d = {"variant_cases_json": np.frombuffer(json.dumps(VARIANT_CASES).encode(), dtype=np.uint8)}
+    for name, (widths, B, hidden, hyper) in VARIANT_CASES.items():
+        rng = np.random.default_rng(sum(map(ord, name)))
+        L = len(widths)
+        X = f32(rng.uniform(0, 1, (B, widths[0])))
+        Y = f32(np.eye(widths[-1])[rng.integers(0, widths[-1], B)])
+        masks = {l: (rng.uniform(size=widths[l]) < hidden[l - 1][3]).astype(np.uint8) for l in range(1, L - 1)}
+        d[name + "_X"], d[name + "_Y"] = X, Y
+        for l, mk in masks.items():
+            d[f"{name}_mask{l}"] = mk
+        params = None
+        for nt in THREADS:
+            M = R.mlp(widths)
+            for l in range(1, L - 1):
+                a, nm, dr, keep, before = hidden[l - 1]
+                M.set_layer(l, ACT[a], NORM[nm], DROP[dr], keep, masks[l] if dr != "NONE" else None, norm_before=before)
+            M.set_layer(L - 1, ACT["SOFTMAX"])
+            M.set_norm_hyper(*hyper)
+            M.prepare(B, nt)
+            if params is None:
+                params = M.get_parameters()
+                for l in range(1, L):
+                    o = M.layer_offsets(l)
+                    K, H = widths[l - 1], widths[l]
+                    params[o[0]:o[0] + H * K] = glorot(rng, H, K).ravel()
+                    params[o[1]:o[1] + H] = f32(rng.uniform(-0.2, 0.2, H))
+                    params[o[2]:o[2] + H] = f32(rng.uniform(0.8, 1.2, H))
+                    params[o[3]:o[3] + H] = f32(rng.uniform(-0.1, 0.1, H))
+                d[name + "_params"] = params.copy()
+            M.set_parameters(params)
+            q = f"{name}_t{nt}_"
+            M.step(STATE["TRAINING"], X, Y, backward=True)
+            for l in range(1, L):
+                d[f"{q}train_L{l}_out"] = M.layer_buffer(l, 6)
+                d[f"{q}train_L{l}_dZ"] = M.layer_buffer(l, 4)
+            d[q + "dparams"] = M.get_dparams()
+            d[q + "train_mov_mean"], d[q + "train_mov_std"] = M.get_moving()
+            M.step(STATE["UPDATE_BATCH_NORM"], X, None, backward=False)
+            for l in range(1, L):
+                d[f"{q}ubn_L{l}_out"] = M.layer_buffer(l, 6)
+            d[q + "ubn_mov_mean"], d[q + "ubn_mov_std"] = M.get_moving()
+            M.step(STATE["INFERENCE"], X, None, backward=False)
+            for l in range(1, L):
+                d[f"{q}infer_L{l}_out"] = M.layer_buffer(l, 6)
+    save("variants.npz", d)
     return len(d)
 
 
@@ -345,3 +420,4 @@ if __name__ == "__main__":
     print("mlp:", mlps(R), "arrays")
     print("optim:", optimizers(R), "arrays")
     print("epoch:", epochs(R), "arrays")
+    print("variants:", variants(R), "arrays")
