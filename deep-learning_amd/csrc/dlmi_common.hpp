@@ -63,6 +63,9 @@ int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
                             float const *gamma, float const *beta, uint8_t const *mask, float *mean, float *stdv,
                             float *mov_mean, float *mov_std, float *r, float *d, float *y, float const *partial,
                             unsigned nchunks);
+// out[j] (+)= sum over the B rows of x[b, j], in a fixed order (the statistics
+// pass of the normalization kernels with its second plane unused).
+int column_sums(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *out, int accumulate);
 }  // namespace dlmi
 
 inline bool dlmi_aligned16(void const *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -385,36 +385,6 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(float const *__restrict__
   }
 }
 
-// db[h] (+)= sum_b dZ[b,h]: column sums over the batch in a fixed order
-// (update_derivative_fwp_st.cpp:283-302).  Thread per column, blocks over batch
-// chunks, partials combined by k_colsum_finish.
-__global__ __launch_bounds__(256) void k_colsum_partial(float const *__restrict__ x, size_t B, size_t H,
-                                                         size_t rows_per_chunk, float *__restrict__ partial) {
-  size_t const j = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (j >= H) return;
-  size_t const b0 = blockIdx.y * rows_per_chunk;
-  size_t const b1 = (b0 + rows_per_chunk < B) ? b0 + rows_per_chunk : B;
-  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
-  size_t b = b0;
-  for (; b + 3 < b1; b += 4) {
-    s0 += x[(b + 0) * H + j];
-    s1 += x[(b + 1) * H + j];
-    s2 += x[(b + 2) * H + j];
-    s3 += x[(b + 3) * H + j];
-  }
-  for (; b < b1; ++b) s0 += x[b * H + j];
-  partial[static_cast<size_t>(blockIdx.y) * H + j] = (s0 + s1) + (s2 + s3);
-}
-
-__global__ __launch_bounds__(256) void k_colsum_finish(float const *__restrict__ partial, unsigned nchunks, size_t H,
-                                                        float *__restrict__ out, int accumulate) {
-  size_t const j = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (j >= H) return;
-  float s = 0.0f;
-  for (unsigned c = 0; c < nchunks; ++c) s += partial[static_cast<size_t>(c) * H + j];
-  out[j] = accumulate ? out[j] + s : s;
-}
-
 // ---------------------------------------------------------------- host side
 template <int BM, int BN, int BK, bool AK, bool BKC, int WPE>
 static int launch_gemm(dlmi_ctx *ctx, GemmArgs g, unsigned splits, bool fast) {
@@ -586,21 +556,8 @@ int dlmi_fc_bwd_dw(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin
   DLMI_REQUIRE(ctx, B > 0 && K > 0 && H > 0, "empty operand");
   int rc = gemm<false, false>(ctx, H, K, B, dZ, H, Xin, K, dW, nullptr, accumulate);
   if (rc != DLMI_OK || db == nullptr) return rc;
-  size_t chunks = dlmi_ceil_div(static_cast<size_t>(ctx->num_cu) * 4, dlmi_ceil_div(H, 256));
-  if (chunks > dlmi_ceil_div(B, 32)) chunks = dlmi_ceil_div(B, 32);
-  if (chunks < 1) chunks = 1;
-  size_t const rows = dlmi_ceil_div(B, chunks);
-  chunks = dlmi_ceil_div(B, rows);
-  rc = dlmi_scratch_reserve(ctx, chunks * H * sizeof(float));
-  if (rc != DLMI_OK) return rc;
-  float *partial = reinterpret_cast<float *>(ctx->scratch);
-  hipLaunchKernelGGL(k_colsum_partial, dim3(static_cast<unsigned>(dlmi_ceil_div(H, 256)), static_cast<unsigned>(chunks)),
-                     dim3(256), 0, ctx->stream, dZ, B, H, rows, partial);
-  DLMI_LAUNCH_CHECK(ctx, "k_colsum_partial");
-  hipLaunchKernelGGL(k_colsum_finish, dim3(static_cast<unsigned>(dlmi_ceil_div(H, 256))), dim3(256), 0, ctx->stream,
-                     partial, static_cast<unsigned>(chunks), H, db, accumulate);
-  DLMI_LAUNCH_CHECK(ctx, "k_colsum_finish");
-  return DLMI_OK;
+  // db[h] (+)= sum_b dZ[b,h] (update_derivative_fwp_st.cpp:283-302)
+  return column_sums(ctx, B, H, dZ, db, accumulate);
 }
 
 }  // extern "C"

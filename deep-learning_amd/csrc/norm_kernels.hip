@@ -840,6 +840,35 @@ int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
   return run_fwd_train(ctx, B, H, c);
 }
 
+// out[j] (+)= column sum, from the first plane of the statistics partials.
+__global__ __launch_bounds__(kBlock) void k_colsum_finalize(float const *__restrict__ partial, unsigned nchunks,
+                                                             size_t H, float *__restrict__ out, int accumulate) {
+  __shared__ float lds[kBlock];
+  float tot[1];
+  chunk_totals<1>(partial, nchunks, H, tot, lds);
+  size_t const j = static_cast<size_t>(blockIdx.x) * kFinCols + threadIdx.x;
+  if (threadIdx.x >= kFinCols || j >= H) return;
+  out[j] = accumulate ? out[j] + tot[0] : tot[0];
+}
+
+int column_sums(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *out, int accumulate) {
+  int rc = dlmi_scratch_reserve(ctx, 2 * 16 * 2 * H * sizeof(float));
+  if (rc != DLMI_OK) return rc;
+  bool const vec4 = use_vec4(H, {x});
+  ColGeom const g = reduce_geometry(ctx, B, H, vec4, 2);
+  float *pw = reinterpret_cast<float *>(ctx->scratch);
+  dim3 const grid(g.grid_x, g.nchunks), block(kBlock);
+  if (vec4)
+    hipLaunchKernelGGL(k_col_stats<4>, grid, block, 0, ctx->stream, x, B, H, g.tx_log2, g.rows_per_chunk, pw);
+  else
+    hipLaunchKernelGGL(k_col_stats<1>, grid, block, 0, ctx->stream, x, B, H, g.tx_log2, g.rows_per_chunk, pw);
+  DLMI_LAUNCH_CHECK(ctx, "k_col_stats");
+  hipLaunchKernelGGL(k_colsum_finalize, dim3(static_cast<unsigned>(dlmi_ceil_div(H, kFinCols))), block, 0, ctx->stream,
+                     pw, g.nchunks, H, out, accumulate);
+  DLMI_LAUNCH_CHECK(ctx, "k_colsum_finalize");
+  return DLMI_OK;
+}
+
 }  // namespace dlmi
 
 using namespace dlmi;
