@@ -39,7 +39,7 @@ C_ABI_SYMBOLS = [
     "dlmi_norm_fwd_train", "dlmi_norm_fwd_infer", "dlmi_norm_bwd", "dlmi_act_fwd", "dlmi_act_bwd",
     "dlmi_softmax_fwd", "dlmi_dropout_fwd", "dlmi_identity_add", "dlmi_softmax_ce_seed",
     "dlmi_fused_norm_act_fwd", "dlmi_fused_norm_act_bwd", "dlmi_fused_norm_act_infer", "dlmi_fc_norm_act_fwd",
-    "dlmi_opt_gd", "dlmi_opt_gd_momentum", "dlmi_opt_adam",
+    "dlmi_opt_gd", "dlmi_opt_gd_momentum", "dlmi_opt_adam", "dlmi_zero_padded_identity_fwd", "dlmi_residual_bwd",
 ]
 
 
@@ -231,6 +231,22 @@ class Dlmi:
         o = out if out is not None else self.torch.empty_like(a)
         self._ck(self.lib.dlmi_identity_add(self.ctx, c_sz(a.numel()), _p(a), _p(b), _p(o)))
         return o
+
+    def zero_padded_identity_fwd(self, a, b, padding, out=None):
+        self._chk(a, b, out)
+        B, HA = a.shape
+        HB = b.shape[1]
+        o = out if out is not None else self.empty(B, max(HA, HB))
+        self._ck(self.lib.dlmi_zero_padded_identity_fwd(self.ctx, c_sz(B), c_sz(HA), c_sz(HB), c_sz(padding), _p(a),
+                                                        _p(b), _p(o)))
+        return o
+
+    def residual_bwd(self, d_inputs, derivatives, padding):
+        """derivatives += the routed columns of d_inputs, in place."""
+        self._chk(d_inputs, derivatives)
+        self._ck(self.lib.dlmi_residual_bwd(self.ctx, c_sz(d_inputs.shape[0]), c_sz(d_inputs.shape[1]),
+                                            c_sz(derivatives.shape[1]), c_sz(padding), _p(d_inputs), _p(derivatives)))
+        return derivatives
 
     # optimizer steps: every tensor argument is updated in place, grads end up zero
     def opt_gd(self, p, g, mask, lr, wd, nthreads=0):

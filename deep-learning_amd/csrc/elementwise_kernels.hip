@@ -72,6 +72,32 @@ __global__ __launch_bounds__(kEwBlock) void k_add(float const *__restrict__ a, f
   for (i = n4 * 4 + static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x; i < n; i += stride) out[i] = a[i] + b[i];
 }
 
+// ---- zero-padded identity shortcut (fwp_st.cpp:5051-5112, padding != 0):
+// out [B, Hw] = wide [B, Hw], plus narrow [B, Hn] at column offset `pad`
+__global__ __launch_bounds__(kEwBlock) void k_padded_add(float const *__restrict__ wide,
+                                                          float const *__restrict__ narrow, float *__restrict__ out,
+                                                          size_t B, size_t Hw, size_t Hn, size_t pad) {
+  size_t const n = B * Hw, stride = static_cast<size_t>(gridDim.x) * kEwBlock;
+  for (size_t e = static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x; e < n; e += stride) {
+    size_t const b = e / Hw, j = e - b * Hw;
+    float v = wide[e];
+    if (j >= pad && j - pad < Hn) v += narrow[b * Hn + (j - pad)];
+    out[e] = v;
+  }
+}
+
+// ---- shortcut gradient routing (bwp_st.cpp:1112-1175): over the Hc = min(Hi, Hd)
+// shared columns, dd[b, j + od] += di[b, j + oi]
+__global__ __launch_bounds__(kEwBlock) void k_residual_bwd(float const *__restrict__ di, float *__restrict__ dd,
+                                                            size_t B, size_t Hi, size_t Hd, size_t Hc, size_t oi,
+                                                            size_t od) {
+  size_t const n = B * Hc, stride = static_cast<size_t>(gridDim.x) * kEwBlock;
+  for (size_t e = static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x; e < n; e += stride) {
+    size_t const b = e / Hc, j = e - b * Hc;
+    dd[b * Hd + j + od] += di[b * Hi + j + oi];
+  }
+}
+
 // ---- per-unit row kernels: element e = b*H + j, unit j = e % H ----------------
 // mode 0: Z += bias                                     (fwp_st.cpp:4498-4516)
 // mode 1: dropout, kind/per_element/scale in the args   (fwp_st.cpp:4830-4904)
@@ -265,6 +291,41 @@ int dlmi_identity_add(dlmi_ctx *ctx, size_t n, float const *a, float const *b, f
   size_t const n4 = all_aligned16({a, b, out}) ? n / 4 : 0;
   hipLaunchKernelGGL(k_add, dim3(ew_grid(ctx, n4 ? n4 : n)), dim3(kEwBlock), 0, ctx->stream, a, b, out, n4, n);
   DLMI_LAUNCH_CHECK(ctx, "k_add");
+  return DLMI_OK;
+}
+
+int dlmi_zero_padded_identity_fwd(dlmi_ctx *ctx, size_t B, size_t HA, size_t HB, size_t padding, float const *a,
+                                  float const *b, float *out) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, a && b && out, "null pointer");
+  if (padding == 0) {
+    DLMI_REQUIRE(ctx, HA == HB, "no padding needs equal widths");
+    return dlmi_identity_add(ctx, B * HA, a, b, out);
+  }
+  DLMI_REQUIRE(ctx, HA != HB, "padding needs operands of different widths");
+  bool const a_wide = HA > HB;
+  size_t const Hw = a_wide ? HA : HB, Hn = a_wide ? HB : HA;
+  DLMI_REQUIRE(ctx, padding + Hn <= Hw, "the padded operand does not fit the wider one");
+  if (B * Hw == 0) return DLMI_OK;
+  hipLaunchKernelGGL(k_padded_add, dim3(ew_grid(ctx, B * Hw)), dim3(kEwBlock), 0, ctx->stream, a_wide ? a : b,
+                     a_wide ? b : a, out, B, Hw, Hn, padding);
+  DLMI_LAUNCH_CHECK(ctx, "k_padded_add");
+  return DLMI_OK;
+}
+
+int dlmi_residual_bwd(dlmi_ctx *ctx, size_t B, size_t input_size, size_t derivative_size, size_t padding,
+                      float const *d_inputs, float *derivatives) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, d_inputs && derivatives, "null pointer");
+  size_t const Hc = input_size < derivative_size ? input_size : derivative_size;
+  size_t const Hwide = input_size < derivative_size ? derivative_size : input_size;
+  size_t const pad = input_size == derivative_size ? 0 : padding;
+  DLMI_REQUIRE(ctx, pad + Hc <= Hwide, "the padded operand does not fit the wider one");
+  if (B * Hc == 0) return DLMI_OK;
+  hipLaunchKernelGGL(k_residual_bwd, dim3(ew_grid(ctx, B * Hc)), dim3(kEwBlock), 0, ctx->stream, d_inputs, derivatives,
+                     B, input_size, derivative_size, Hc, input_size > derivative_size ? pad : 0,
+                     input_size < derivative_size ? pad : 0);
+  DLMI_LAUNCH_CHECK(ctx, "k_residual_bwd");
   return DLMI_OK;
 }
 

@@ -162,6 +162,21 @@ int dlmi_dropout_fwd(dlmi_ctx *ctx, dlmi_dropout kind, int training, int per_ele
  * Backward_Pass__Residual__*, bwp_st.cpp:1112-1175).  out may alias a or b. */
 int dlmi_identity_add(dlmi_ctx *ctx, size_t n, float const *a, float const *b, float *out);
 
+/* Zero-padded identity shortcut of a residual block: out [B, max(HA, HB)] = the
+ * wider operand, plus the narrower one at column offset `padding`; padding == 0
+ * is the plain sum and needs HA == HB.  out must not alias the narrower operand.
+ * Replaces Forward_Pass__Zero_Padded_Identity__{Loop,OpenMP} (fwp_st.cpp:5051-5112). */
+int dlmi_zero_padded_identity_fwd(dlmi_ctx *ctx, size_t B, size_t HA, size_t HB, size_t padding,
+                                  float const *a, float const *b, float *out);
+
+/* Gradient routing of that shortcut: derivatives [B, derivative_size] += the
+ * matching columns of d_inputs [B, input_size] (equal sizes: all of them; the
+ * wider side is read / written at column offset `padding`).  Replaces
+ * Backward_Pass__Residual__{Loop,OpenMP} (bwp_st.cpp:1112-1175) and
+ * Backward_Pass__Identity__{Loop,OpenMP} (bwp_st.cpp:1047-1068). */
+int dlmi_residual_bwd(dlmi_ctx *ctx, size_t B, size_t input_size, size_t derivative_size, size_t padding,
+                      float const *d_inputs, float *derivatives);
+
 /* Softmax + cross-entropy seed gradient of the output layer:
  * dZ_i = sum_k (q_i [i==k] - q_k q_i) * dL_k,  dL_k = (y_k==1 ? -1/clip(q_k,1e-7,1-1e-7) : 0)/B.
  * stats (device, 2 doubles, may be NULL) accumulates { sum of CE losses, number

@@ -173,6 +173,23 @@ class _Leaves:
         self._f("identity_add")(c_int(nthreads), c_sz(B), c_sz(H), _ptr(a), _ptr(b), _ptr(out))
         return out
 
+    def zero_padded_identity_fwd(self, a, b, padding, nthreads=0):
+        a, b = self._a(a), self._a(b)
+        B, HA = a.shape
+        HB = b.shape[1]
+        out = np.empty((B, max(HA, HB)), self.dtype)
+        self._f("zero_padded_identity_fwd")(c_int(nthreads), c_sz(B), c_sz(HA), c_sz(HB), c_sz(padding), _ptr(a),
+                                            _ptr(b), _ptr(out))
+        return out
+
+    def residual_bwd(self, d_inputs, derivatives, padding, nthreads=0):
+        """Returns derivatives + the routed columns of d_inputs."""
+        di = self._a(d_inputs)
+        dd = np.array(derivatives, dtype=self.dtype, order="C", copy=True)
+        self._f("residual_bwd")(c_int(nthreads), c_sz(di.shape[0]), c_sz(di.shape[1]), c_sz(dd.shape[1]),
+                                c_sz(padding), _ptr(di), _ptr(dd))
+        return dd
+
     def fc_bwd_dx(self, dZn, Wn, dY_init=None, nthreads=0):
         dZn, Wn = self._a(dZn), self._a(Wn)
         B, Hn = dZn.shape

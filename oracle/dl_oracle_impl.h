@@ -262,6 +262,53 @@ void FN(dlo_identity_add)(int nthreads, size_t B, size_t H, REAL const *a,
   }
 }
 
+/* ---- a15 with padding: zero-padded identity shortcut, fwp_st.cpp:5051-5112 ----
+ * out [B, max(HA, HB)]: the wider operand copied, the narrower one added at
+ * column offset `padding`; padding == 0 is the plain sum and needs HA == HB. */
+void FN(dlo_zero_padded_identity_fwd)(int nthreads, size_t B, size_t HA, size_t HB, size_t padding, REAL const *a,
+                                      REAL const *bb, REAL *out) {
+  int const N = FN(nthr)(nthreads, B);
+  int const Bi = (int)B;
+  int b;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (b = 0; b < Bi; ++b) {
+    REAL const *ra = a + (size_t)b * HA, *rb = bb + (size_t)b * HB;
+    if (padding == 0) {
+      REAL *ro = out + (size_t)b * HA;
+      for (size_t i = 0; i != HA; ++i) ro[i] = ra[i] + rb[i];
+    } else if (HA > HB) {
+      REAL *ro = out + (size_t)b * HA;
+      for (size_t i = 0; i != HA; ++i) ro[i] = ra[i];
+      for (size_t i = 0; i != HB; ++i) ro[i + padding] += rb[i];
+    } else {
+      REAL *ro = out + (size_t)b * HB;
+      for (size_t i = 0; i != HB; ++i) ro[i] = rb[i];
+      for (size_t i = 0; i != HA; ++i) ro[i + padding] += ra[i];
+    }
+  }
+}
+
+/* ---- a22: shortcut gradient routing, bwp_st.cpp:1112-1175 (and :1047-1068 when
+ * the widths are equal).  derivatives [B, Hd] accumulate. */
+void FN(dlo_residual_bwd)(int nthreads, size_t B, size_t Hi, size_t Hd, size_t padding, REAL const *d_inputs,
+                          REAL *derivatives) {
+  int const N = FN(nthr)(nthreads, B);
+  int const Bi = (int)B;
+  int b;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (b = 0; b < Bi; ++b) {
+    REAL const *di = d_inputs + (size_t)b * Hi;
+    REAL *dd = derivatives + (size_t)b * Hd;
+    if (Hi == Hd) {
+      for (size_t i = 0; i != Hi; ++i) dd[i] += di[i];
+    } else if (Hi > Hd) {
+      for (size_t i = 0; i != Hd; ++i) dd[i] += di[i + padding];
+    } else {
+      for (size_t i = 0; i != Hi; ++i) dd[i + padding] += di[i];
+    }
+  }
+}
+
 /* ---- optimizer steps over parameters [str, end) of the packed arrays ---------
  * mask: the regularization mask (1 weights, 0 biases / gamma / beta:
  * allocate.cpp:1178-1196, indexing.cpp:59-85), read only when wd != 0.

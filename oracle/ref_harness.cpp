@@ -218,6 +218,35 @@ void dlref_identity_add(int nthreads, size_t B, size_t H, float const *a,
   }
 }
 
+// ---- a15 with padding: out [B, max(HA, HB)] = the wider operand, plus the
+// narrower one at column offset `padding` (padding == 0 needs HA == HB) --------
+void dlref_zero_padded_identity_fwd(int nthreads, size_t B, size_t HA, size_t HB, size_t padding, float const *a,
+                                    float const *b, float *out) {
+  nthreads = clampThreads(nthreads, B);
+  LeafModel lm(B, nthreads);
+  if (nthreads == 0) {
+    lm.m.Forward_Pass__Zero_Padded_Identity__Loop(0, B, HA, HB, padding, a, b, out);
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    lm.m.Forward_Pass__Zero_Padded_Identity__OpenMP(0, B, HA, HB, padding, a, b, out);
+  }
+}
+
+// ---- a22: gradient routing of the shortcut, derivatives [B, Hd] += the matching
+// columns of d_inputs [B, Hi] (bwp_st.cpp:1112-1175); Hi == Hd is also
+// Backward_Pass__Identity__Loop (bwp_st.cpp:1047-1068) ---------------------------
+void dlref_residual_bwd(int nthreads, size_t B, size_t Hi, size_t Hd, size_t padding, float const *d_inputs,
+                        float *derivatives) {
+  nthreads = clampThreads(nthreads, B);
+  LeafModel lm(B, nthreads);
+  if (nthreads == 0) {
+    lm.m.Backward_Pass__Residual__Loop(0, B, Hi, Hd, padding, d_inputs, derivatives);
+  } else {
+#pragma omp parallel num_threads(nthreads)
+    lm.m.Backward_Pass__Residual__OpenMP(0, B, Hi, Hd, padding, d_inputs, derivatives);
+  }
+}
+
 // ---- a18: dY += dZn * Wn  (dY is NOT cleared here) -------------------------
 void dlref_fc_bwd_dx(int nthreads, size_t B, size_t Hn, size_t H,
                      float const *dZn, float const *Wn, float *dY) {

@@ -414,6 +414,27 @@ def variants(R):
     return len(d)
 
 
+SHORTCUT_CASES = [(9, 6, 6, 0), (9, 10, 6, 2), (9, 6, 10, 3), (5, 8, 4, 4), (33, 130, 66, 17), (1, 3, 3, 0)]  # B, HA, HB, padding (0 only with equal widths)
+
+
+def shortcuts(R):
+    """Zero-padded identity shortcut of a residual block and the routing of its
+    gradient (fwp_st.cpp:5051-5112, bwp_st.cpp:1047-1068, 1112-1175)."""
+    rng = np.random.default_rng(5051)
+    d = {"shortcut_cases": np.array(SHORTCUT_CASES)}
+    for ci, (B, HA, HB, pad) in enumerate(SHORTCUT_CASES):
+        a, b = f32(rng.standard_normal((B, HA))), f32(rng.standard_normal((B, HB)))
+        g = f32(rng.standard_normal((B, max(HA, HB))))       # gradient of the block's output
+        da0, db0 = f32(rng.standard_normal((B, HA))), f32(rng.standard_normal((B, HB)))
+        d[f"sc{ci}_a"], d[f"sc{ci}_b"], d[f"sc{ci}_g"], d[f"sc{ci}_da0"], d[f"sc{ci}_db0"] = a, b, g, da0, db0
+        for nt in THREADS:
+            d[f"sc{ci}_t{nt}_out"] = R.zero_padded_identity_fwd(a, b, pad, nt)
+            d[f"sc{ci}_t{nt}_da"] = R.residual_bwd(g, da0, pad, nt)
+            d[f"sc{ci}_t{nt}_db"] = R.residual_bwd(g, db0, pad, nt)
+    save("shortcut.npz", d)
+    return len(d)
+
+
 if __name__ == "__main__":
     R = Reference()
     print("leaves:", leaves(R), "arrays")
@@ -421,3 +442,4 @@ if __name__ == "__main__":
     print("optim:", optimizers(R), "arrays")
     print("epoch:", epochs(R), "arrays")
     print("variants:", variants(R), "arrays")
+    print("shortcut:", shortcuts(R), "arrays")
