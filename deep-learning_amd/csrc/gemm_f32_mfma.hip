@@ -483,7 +483,10 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
       *stats_chunks = 0;  // the slices hold partial products: the caller takes the statistics from C itself
     } else {
       *stats_chunks = static_cast<unsigned>(dlmi_ceil_div(M, bm));
-      int rc = dlmi_scratch_reserve(ctx, 2 * 2 * static_cast<size_t>(*stats_chunks) * N * sizeof(float));
+      // also what the normalization tail reserves itself: it must not have to grow
+      // (and thereby free) the block while these partials sit in it
+      size_t const chunks_reserved = *stats_chunks > 32 ? *stats_chunks : 32;
+      int rc = dlmi_scratch_reserve(ctx, 2 * 2 * static_cast<size_t>(chunks_reserved) * N * sizeof(float));
       if (rc != DLMI_OK) return rc;
       g.stats_out = reinterpret_cast<float *>(ctx->scratch);
     }

@@ -62,7 +62,10 @@ typedef struct dlmi_ctx dlmi_ctx;
 
 /* ---- context ------------------------------------------------------------- */
 /* device: HIP device ordinal.  stream: a hipStream_t (NULL = default stream).
- * The context owns a device scratch buffer for reduction partials. */
+ * The context owns a device scratch buffer for reduction partials.  Calls on a
+ * context come from one thread at a time, with the context's device current
+ * (dlmi_ctx_create makes it so); the scratch buffer is shared by consecutive
+ * calls, which the stream orders. */
 int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream);
 int dlmi_ctx_destroy(dlmi_ctx *ctx);
 int dlmi_ctx_set_stream(dlmi_ctx *ctx, void *stream);

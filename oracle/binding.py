@@ -636,3 +636,149 @@ class ReferenceMLP:
         self.lib.dlref_model_evalt(self.h, c_sz(X.shape[0]), _ptr(X), c_sz(X.shape[1]), _ptr(Y), c_sz(Y.shape[1]),
                                    out)
         return out[0], out[1]
+
+
+# ---- layer lists with residual blocks ---------------------------------------------
+LAYER = dict(FULLY_CONNECTED=3, RESIDUAL=9)  # v1/data/enum/layer.hpp
+
+
+class _NetBase:
+    """Driving interface shared by OracleNet and ReferenceNet.  `layers` is a list
+    of ("FC", units) and ("RES", depth, padding) entries, entry 0 the input width."""
+
+    def _spec(self, layers):
+        self.layers = list(layers)
+        n = len(layers)
+        types = [LAYER["FULLY_CONNECTED"] if e[0] == "FC" else LAYER["RESIDUAL"] for e in layers]
+        units = [int(e[1]) for e in layers]
+        pads = [int(e[2]) if len(e) > 2 else 0 for e in layers]
+        return n, (c_int * n)(*types), (c_sz * n)(*units), (c_sz * n)(*pads)
+
+    def info(self, l):
+        """dict(type, n_out, w0, w1, bias, use_bias, n_unit, gamma, unit, n_af, depth, padding)"""
+        out = (c_sz * 12)()
+        self._info(l, out)
+        keys = ("type", "n_out", "w0", "w1", "bias", "use_bias", "n_unit", "gamma", "unit", "n_af", "depth", "padding")
+        return dict(zip(keys, (int(v) for v in out)))
+
+    def fc_layers(self):
+        return [l for l, e in enumerate(self.layers) if l > 0 and e[0] == "FC"]
+
+
+class OracleNet(_NetBase):
+    def __init__(self, oracle, layers):
+        self.o, self.lib = oracle, oracle.lib
+        n, t, u, p = self._spec(layers)
+        self.lib.dlo_net_create.restype = vp
+        for f in ("parameters", "dparameters", "moving_mean", "moving_std", "layer_output", "layer_error"):
+            getattr(self.lib, "dlo_net_" + f).restype = ctypes.POINTER(c_f)
+        self.lib.dlo_net_total_parameters.restype = c_sz
+        self.lib.dlo_net_total_units.restype = c_sz
+        self.lib.dlo_net_loss_sum.restype = c_d
+        self.lib.dlo_net_n_correct.restype = c_d
+        self.h = vp(self.lib.dlo_net_create(c_sz(n), t, u, p))
+        self.P = self.lib.dlo_net_total_parameters(self.h)
+        self.n_units = self.lib.dlo_net_total_units(self.h)
+
+    def __del__(self):
+        try:
+            self.lib.dlo_net_destroy(self.h)
+        except Exception:
+            pass
+
+    def _info(self, l, out):
+        self.lib.dlo_net_layer_info(self.h, c_sz(l), out)
+
+    def set_layer(self, l, act, norm=0, drop=0, keep=1.0, mask=None):
+        m = None if mask is None else np.ascontiguousarray(mask, dtype=np.uint8)
+        self.lib.dlo_net_set_layer(self.h, c_sz(l), c_int(act), c_int(norm), c_int(drop), c_f(keep), _ptr(m))
+
+    def set_norm_hyper(self, momentum, eps, r_max, d_max):
+        self.lib.dlo_net_set_norm_hyper(self.h, c_f(momentum), c_f(eps), c_f(r_max), c_f(d_max))
+
+    def prepare(self, max_batch, nthreads=0):
+        self.max_batch, self.nthreads = max_batch, nthreads
+        self.lib.dlo_net_prepare(self.h, c_sz(max_batch))
+
+    def _view(self, fn, n):
+        return np.ctypeslib.as_array(fn(self.h), shape=(n,))
+
+    def set_parameters(self, p):
+        self._view(self.lib.dlo_net_parameters, self.P)[:] = p
+
+    def get_parameters(self):
+        return self._view(self.lib.dlo_net_parameters, self.P).copy()
+
+    def get_dparams(self):
+        return self._view(self.lib.dlo_net_dparameters, self.P).copy()
+
+    def get_moving(self):
+        return (self._view(self.lib.dlo_net_moving_mean, self.n_units).copy(),
+                self._view(self.lib.dlo_net_moving_std, self.n_units).copy())
+
+    def step(self, state, X, Y=None, backward=True):
+        X = np.ascontiguousarray(X, np.float32)
+        self.B = X.shape[0]
+        self.lib.dlo_net_forward(self.h, c_int(self.nthreads), c_int(state), c_sz(self.B), _ptr(X))
+        if backward:
+            Y = np.ascontiguousarray(Y, np.float32)
+            self.lib.dlo_net_backward(self.h, c_int(self.nthreads), c_sz(self.B), _ptr(Y))
+
+    def layer_output(self, l):
+        w = self.info(l)["n_out"]
+        return np.ctypeslib.as_array(self.lib.dlo_net_layer_output(self.h, c_sz(l)), shape=(self.max_batch, w))[: self.B].copy()
+
+    def layer_error(self, l):
+        w = self.info(l)["n_out"]
+        return np.ctypeslib.as_array(self.lib.dlo_net_layer_error(self.h, c_sz(l)), shape=(self.max_batch, w))[: self.B].copy()
+
+
+class ReferenceNet(_NetBase, ReferenceMLP):
+    """A real DL::v1::Model compiled from a typed layer list."""
+
+    def __init__(self, ref, layers, allowable_bytes=1 << 32):
+        self.lib = ref.lib
+        n, t, u, p = self._spec(layers)
+        self.lib.dlref_model_create_typed.restype = vp
+        h = self.lib.dlref_model_create_typed(c_sz(n), t, u, p, c_sz(allowable_bytes))
+        if not h:
+            raise RuntimeError("reference Model::compile failed")
+        self.h = vp(h)
+        self.P = self.lib.dlref_model_total_parameters(self.h)
+        self.n_units = self.lib.dlref_model_total_norm_units(self.h)
+        self.widths = [0] * n  # filled by prepare(): outputs per entry
+
+    def _info(self, l, out):
+        self.lib.dlref_model_layer_info(self.h, c_sz(l), out)
+
+    def set_layer(self, l, act, norm=0, drop=0, keep=1.0, mask=None):
+        if self.layers[l][0] == "FC":
+            ok = self.lib.dlref_model_set_activation(self.h, c_sz(l), c_int(act))
+            assert ok, "set_layer_activation_function refused"
+        if norm:
+            ok = self.lib.dlref_model_set_normalization(self.h, c_sz(l), c_int(norm))
+            assert ok, "Set__Layer_Normalization refused"
+        if drop:
+            ok = self.lib.dlref_model_set_dropout(self.h, c_sz(l), c_int(drop), c_f(keep))
+            assert ok, "set_dropout refused"
+        self._masks = getattr(self, "_masks", {})
+        if mask is not None:
+            self._masks[l] = np.ascontiguousarray(mask, dtype=np.uint8)
+
+    def prepare(self, max_batch, nthreads=0):
+        self.max_batch = max_batch
+        ok = self.lib.dlref_model_prepare(self.h, c_sz(max_batch), c_int(nthreads))
+        assert ok, "reference prepare failed"
+        for l, m in getattr(self, "_masks", {}).items():
+            ok = self.lib.dlref_model_set_dropout_mask(self.h, c_sz(l), c_sz(m.size), _ptr(m))
+            assert ok
+        self.lib.dlref_model_zero_dparams(self.h)
+        self.P = self.lib.dlref_model_total_parameters(self.h)
+        self.n_units = self.lib.dlref_model_total_norm_units(self.h)
+        self.widths = [self.info(l)["n_out"] for l in range(len(self.layers))]
+
+    def layer_output(self, l):
+        return self.layer_buffer(l, 6)
+
+    def layer_error(self, l):
+        return self.layer_buffer(l, 4)

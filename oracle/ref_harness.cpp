@@ -394,6 +394,57 @@ void *dlref_model_create(size_t n_layers, size_t const *widths,
   return rm;
 }
 
+// The same with a layer type per entry (LAYER::TYPE; 9 = RESIDUAL, whose units[i]
+// is the block depth and whose padding[i] the zero-padding of its shortcut,
+// compile.cpp:127-170, run/deep-learning/v1/custom.cpp:449-470).
+void *dlref_model_create_typed(size_t n_layers, int const *types, size_t const *units, size_t const *padding,
+                               size_t allowable_bytes) {
+  dlref_init();
+  RefModel *rm = new RefModel;
+  rm->n_layers = n_layers;
+  std::vector<Layer_Parameters> lp(n_layers);
+  for (size_t i = 0; i < n_layers; ++i) {
+    lp[i].type_layer = static_cast<LAYER::TYPE>(types[i]);
+    lp[i].unit_parameters[0] = units[i];
+    if (padding != nullptr) lp[i].unit_parameters[2] = padding[i];
+  }
+  if (!rm->model.compile(n_layers, 1, MODEL::FEEDFORWARD, lp.data(), allowable_bytes)) {
+    delete rm;
+    return nullptr;
+  }
+  rm->model.set_loss_fn(LOSS_FN::CROSS_ENTROPY);
+  rm->model.set_accu_fn(ACCU_FN::CROSS_ENTROPY);
+  return rm;
+}
+
+// Structure of one layer, for layouts the dense-MLP accessors do not cover.
+// out[0] type, [1] number of outputs, [2] first connection index (or 0),
+// [3] last connection index, [4] first bias index, [5] Use__Bias, [6] number of
+// normalized units, [7] gamma offset, [8] moving-statistic offset, [9] number of
+// AF units, [10] block depth, [11] shortcut padding
+void dlref_model_layer_info(void *h, size_t layer, size_t *out) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  Layer &l = m.ptr_array_layers[layer];
+  out[0] = static_cast<size_t>(l.type_layer);
+  out[1] = l.ptr_number_outputs ? *l.ptr_number_outputs : 0;
+  bool const has_neurons = l.ptr_array_neuron_units != nullptr && l.ptr_last_neuron_unit != l.ptr_array_neuron_units;
+  out[2] = has_neurons ? *l.ptr_array_neuron_units->ptr_first_connection_index : 0;
+  out[3] = has_neurons ? *(l.ptr_last_neuron_unit - 1)->ptr_last_connection_index : 0;
+  out[4] = l.first_bias_connection_index;
+  out[5] = l.Use__Bias();
+  out[6] = static_cast<size_t>(l.ptr_last_normalized_unit - l.ptr_array_normalized_units);
+  out[7] = out[6] && l.ptr_array_normalized_units->normalized_batch_units.ptr_scale
+               ? static_cast<size_t>(l.ptr_array_normalized_units->normalized_batch_units.ptr_scale - m.ptr_array_parameters)
+               : 0;
+  out[8] = out[6] && l.ptr_array_normalized_units->normalized_batch_units.ptr_mean_average
+               ? static_cast<size_t>(l.ptr_array_normalized_units->normalized_batch_units.ptr_mean_average -
+                                     m.ptr_array_normalized_batch_units_means_averages)
+               : 0;
+  out[9] = static_cast<size_t>(l.ptr_last_AF_unit - l.ptr_array_AF_units);
+  out[10] = l.block_depth;
+  out[11] = l.pooling_values[2];
+}
+
 void dlref_model_destroy(void *h) { delete static_cast<RefModel *>(h); }
 
 int dlref_model_set_activation(void *h, size_t layer, int type) {
