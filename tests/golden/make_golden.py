@@ -17,7 +17,7 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 sys.path.insert(0, ROOT)
-from oracle.binding import ACT, DROP, NORM, OPT, STATE, Reference  # noqa: E402
+from oracle.binding import ACT, DROP, NORM, OPT, STATE, Reference, ReferenceNet  # noqa: E402
 
 OUT = os.path.dirname(os.path.abspath(__file__))
 ACTS = ["ELU", "ISRLU", "LEAKY_RELU", "RELU", "SELU", "LINEAR"]
@@ -435,6 +435,75 @@ def shortcuts(R):
     return len(d)
 
 
+RESNET_CASES = {
+    # name: (layer list, batch, {entry: (activation or None, norm, dropout, keep)}, hyper)
+    "res_two_blocks": ([("FC", 8), ("FC", 6), ("RES", 2), ("FC", 6), ("FC", 6), ("RES", 2), ("FC", 5), ("FC", 6), ("FC", 3)], 7,
+                       {1: ("RELU", "BRN", "NONE", 1.0), 2: (None, "BRN", "NONE", 1.0), 3: ("ELU", "BRN", "NONE", 1.0),
+                        4: ("ELU", "BRN", "NONE", 1.0), 5: (None, "NONE", "NONE", 1.0), 6: ("SELU", "BRN", "NONE", 1.0),
+                        7: ("SELU", "NONE", "NONE", 1.0)}, (0.5, 1e-5, 2.0, 1.0)),
+    "res_padded_narrow_block": ([("FC", 8), ("FC", 6), ("RES", 2), ("FC", 7), ("FC", 4), ("FC", 3)], 9,
+                                {1: ("RELU", "BRN", "NONE", 1.0), 2: (None, "BRN", "NONE", 1.0),
+                                 3: ("ISRLU", "BRN", "NONE", 1.0), 4: ("LEAKY_RELU", "BRN", "NONE", 1.0)},
+                                (0.9, 1e-5, 3.0, 5.0)),
+    "res_dropout_wide_block": ([("FC", 8), ("FC", 6), ("RES", 3), ("FC", 7), ("FC", 5), ("FC", 9), ("RES", 2), ("FC", 9),
+                                ("FC", 4), ("FC", 3)], 11,
+                               {1: ("RELU", "BN", "BERNOULLI_INVERTED", 0.7), 2: (None, "BN", "NONE", 1.0),
+                                3: ("ISRLU", "BN", "NONE", 1.0), 4: ("LEAKY_RELU", "NONE", "BERNOULLI", 0.6),
+                                5: ("ELU", "BN", "BERNOULLI_INVERTED", 0.8), 7: ("SELU", "BN", "NONE", 1.0),
+                                8: ("RELU", "BN", "BERNOULLI_INVERTED", 0.5)}, (0.3, 1e-4, 1.0, 0.0)),
+}
+
+
+def resnets(R):
+    """Layer lists with the reference's residual blocks (fwp_st.cpp:3876-4442,
+    bwp_st.cpp:80-185, 345-541): outputs of every entry in the three propagation
+    states, the error of every FC layer, parameter gradients, moving statistics."""
+    d = {"resnet_cases_json": np.frombuffer(json.dumps({k: [v[0], v[1], {str(a): b for a, b in v[2].items()}, v[3]]
+                                                        for k, v in RESNET_CASES.items()}).encode(), dtype=np.uint8)}
+    for name, (layers, B, cfg, hyper) in RESNET_CASES.items():
+        rng = np.random.default_rng(sum(map(ord, name)))
+        n = len(layers)
+        X = f32(rng.uniform(0, 1, (B, layers[0][1])))
+        Y = f32(np.eye(layers[-1][1])[rng.integers(0, layers[-1][1], B)])
+        d[name + "_X"], d[name + "_Y"] = X, Y
+        unit_masks = {l: (rng.uniform(size=64) < c[3]).astype(np.uint8) for l, c in cfg.items() if c[2] != "NONE"}
+        params = None
+        for nt in THREADS:
+            M = ReferenceNet(R, layers)
+            for l, (a, nm, dr, keep) in cfg.items():
+                M.set_layer(l, ACT[a] if a else 0, NORM[nm], DROP[dr], keep)
+            M.set_layer(n - 1, ACT["SOFTMAX"])
+            M.set_norm_hyper(*hyper)
+            # dropout units of a block layer are as many as its inputs: known once the normalization is set up
+            for l, mk in unit_masks.items():
+                nu = M.info(l)["n_unit"]
+                M._masks[l] = mk[:nu].copy()
+                d[f"{name}_mask{l}"] = mk[:nu].copy()
+            M.prepare(B, nt)
+            if params is None:
+                d[name + "_info"] = np.array([list(M.info(l).values()) for l in range(n)])
+                d[name + "_P"] = np.array([M.P, M.n_units])
+                params = M.get_parameters()  # gamma 1, beta 0 from the reference's allocator
+                nwb = M.info(0)["gamma"]     # weights and biases come first
+                params[:nwb] = f32(rng.uniform(-0.5, 0.5, nwb))
+                params[nwb:nwb + M.n_units] = f32(rng.uniform(0.8, 1.2, M.n_units))
+                params[nwb + M.n_units:] = f32(rng.uniform(-0.1, 0.1, M.n_units))
+                d[name + "_params"] = params.copy()
+            M.set_parameters(params)
+            q = f"{name}_t{nt}_"
+            for st in ("TRAINING", "UPDATE_BATCH_NORM", "INFERENCE"):
+                M.step(STATE[st], X, Y, backward=(st == "TRAINING"))
+                for l in range(1, n):
+                    d[f"{q}{st}_L{l}_out"] = M.layer_output(l)
+                if st == "TRAINING":
+                    for l in M.fc_layers():
+                        d[f"{q}L{l}_dZ"] = M.layer_error(l)
+                    d[q + "dparams"] = M.get_dparams()
+                    d[q + "mov_mean"], d[q + "mov_std"] = M.get_moving()
+    save("resnet.npz", d)
+    return len(d)
+
+
 if __name__ == "__main__":
     R = Reference()
     print("leaves:", leaves(R), "arrays")
@@ -443,3 +512,4 @@ if __name__ == "__main__":
     print("epoch:", epochs(R), "arrays")
     print("variants:", variants(R), "arrays")
     print("shortcut:", shortcuts(R), "arrays")
+    print("resnet:", resnets(R), "arrays")
