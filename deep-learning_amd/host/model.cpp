@@ -30,6 +30,7 @@ struct Model::Impl {
   float *d_dparams = nullptr;  // [P]
   float *d_mov_mean = nullptr, *d_mov_std = nullptr;  // [units]
   float *d_input = nullptr;    // [batch, n_in]
+  float *d_input_grad = nullptr;  // [batch, n_in], only when a residual block reads the network input
   float *d_targets = nullptr;  // [batch, n_out]
   double *d_stats = nullptr;   // { loss sum, correct count }
   // optimizer state [P] each: 0 previous delta, 1 first moment, 2 second moment,
@@ -124,8 +125,21 @@ bool Model::compile(size_t const n_layers, size_t const number_recurrent_depth_r
   if (number_recurrent_depth_received != 1) return fail("compile: only seq_w = 1 (no recurrence) is on this path");
   if (type_network_received != MODEL::FEEDFORWARD) return fail("compile: only MODEL::FEEDFORWARD is on this path");
   for (size_t i = 0; i < n_layers; ++i) {
-    if (lp[i].type_layer != LAYER::FULLY_CONNECTED) return fail("compile: only LAYER::FULLY_CONNECTED is on this path");
-    if (lp[i].unit_parameters[0] == 0) return fail("compile: a layer has no units");
+    if (lp[i].type_layer != LAYER::FULLY_CONNECTED && lp[i].type_layer != LAYER::RESIDUAL)
+      return fail("compile: only LAYER::FULLY_CONNECTED and LAYER::RESIDUAL are on this path");
+    if (lp[i].unit_parameters[0] == 0) return fail("compile: a layer has no units, or a residual block no layers");
+  }
+  // a {RESIDUAL, depth} entry is followed by the `depth` fully-connected layers of
+  // its block (compile.cpp:127-170); the input and the output layer stand outside
+  if (lp[0].type_layer != LAYER::FULLY_CONNECTED || lp[n_layers - 1].type_layer != LAYER::FULLY_CONNECTED)
+    return fail("compile: the input and the output layer are fully-connected entries");
+  for (size_t i = 1; i < n_layers; ++i) {
+    if (lp[i].type_layer != LAYER::RESIDUAL) continue;
+    size_t const depth = lp[i].unit_parameters[0];
+    if (i + depth + 1 >= n_layers) return fail("compile: a residual block runs past the layer below the output layer");
+    for (size_t j = 1; j <= depth; ++j)
+      if (lp[i + j].type_layer != LAYER::FULLY_CONNECTED) return fail("compile: a residual block holds fully-connected layers only");
+    i += depth;
   }
   if (dlmi_ctx_create(&impl_->ctx, 0, nullptr) != DLMI_OK)
     return fail("compile: no gfx950 device / context (there is no CPU path)");
@@ -134,19 +148,55 @@ bool Model::compile(size_t const n_layers, size_t const number_recurrent_depth_r
   total_layers = n_layers;
   ptr_array_layers = new Layer[n_layers];
   ptr_last_layer = ptr_array_layers + n_layers;
+  // widths and the entry each entry reads (compile.cpp:283-520)
+  ptr_array_layers[0].type_layer = LAYER::FULLY_CONNECTED;
+  ptr_array_layers[0].n_out = ptr_array_layers[0].n_units = lp[0].unit_parameters[0];
+  size_t feeding = 0;  // the entry whose outputs the next entry reads
+  for (size_t i = 1; i < n_layers;) {
+    Layer &l = ptr_array_layers[i];
+    l.type_layer = lp[i].type_layer;
+    l.feed_index = feeding;
+    if (l.type_layer == LAYER::RESIDUAL) {
+      size_t const depth = lp[i].unit_parameters[0];
+      l.block_depth = depth;
+      size_t cur = feeding;
+      for (size_t j = 1; j <= depth; ++j) {
+        Layer &b = ptr_array_layers[i + j];
+        b.type_layer = LAYER::FULLY_CONNECTED;
+        b.in_block = true;
+        b.block_first = j == 1;
+        b.block_index = i;
+        b.feed_index = cur;
+        b.n_inp = b.n_units = ptr_array_layers[cur].n_out;
+        b.n_out = lp[i + j].unit_parameters[0];
+        cur = i + j;
+      }
+      size_t const shortcut = ptr_array_layers[feeding].n_out, block = ptr_array_layers[i + depth].n_out;
+      l.n_units = block;
+      l.n_out = shortcut > block ? shortcut : block;
+      // compile.cpp:495-510: the narrower of the two is centred in the wider one
+      l.pooling_values[2] = ((shortcut > block ? shortcut - block : block - shortcut) + 1) / 2;
+      feeding = i;
+      i += depth + 1;
+    } else {
+      l.n_inp = ptr_array_layers[feeding].n_out;
+      l.n_out = l.n_units = lp[i].unit_parameters[0];
+      feeding = i;
+      ++i;
+    }
+  }
   size_t nw = 0, nb = 0, nu = 0;
   for (size_t i = 0; i < n_layers; ++i) {
     Layer &l = ptr_array_layers[i];
-    l.type_layer = LAYER::FULLY_CONNECTED;
-    l.n_out = lp[i].unit_parameters[0];
     l.unit_index = nu;
-    nu += l.n_out;
-    if (i > 0) {
+    nu += l.n_units;
+    if (i > 0 && l.type_layer == LAYER::FULLY_CONNECTED) {
       l.first_connection_index = nw;
-      nw += l.n_out * ptr_array_layers[i - 1].n_out;
+      nw += l.n_out * l.n_inp;
     }
   }
   for (size_t i = 1; i < n_layers; ++i) {
+    if (ptr_array_layers[i].type_layer != LAYER::FULLY_CONNECTED) continue;
     ptr_array_layers[i].first_bias_connection_index = nw + nb;
     nb += ptr_array_layers[i].n_out;
   }
@@ -173,10 +223,11 @@ bool Model::compile(size_t const n_layers, size_t const number_recurrent_depth_r
     return false;
   for (size_t i = 1; i < n_layers; ++i) {
     Layer &l = ptr_array_layers[i];
-    if (!dev_alloc(&l.d_mean, l.n_out, err) || !dev_alloc(&l.d_std, l.n_out, err) ||
-        !dev_alloc(&l.d_r, l.n_out, err) || !dev_alloc(&l.d_d, l.n_out, err) || !dev_alloc(&l.d_mask, l.n_out, err))
+    if (!dev_alloc(&l.d_mean, l.n_units, err) || !dev_alloc(&l.d_std, l.n_units, err) ||
+        !dev_alloc(&l.d_r, l.n_units, err) || !dev_alloc(&l.d_d, l.n_units, err) || !dev_alloc(&l.d_mask, l.n_units, err))
       return false;
-    l.mask_dropout_bernoulli.assign(l.n_out, 1);
+    l.mask_dropout_bernoulli.assign(l.n_units, 1);
+    if (!hip_ok(hipMemset(l.d_mask, 1, l.n_units ? l.n_units : 1), err, "mask fill")) return false;
   }
   if (!hip_ok(hipMemsetAsync(impl_->d_dparams, 0, total_parameters * sizeof(float), impl_->stream), err, "memset") ||
       !hip_ok(hipMemsetAsync(impl_->d_stats, 0, 2 * sizeof(double), impl_->stream), err, "memset"))
@@ -191,6 +242,7 @@ bool Model::set_layer_activation_function(size_t const i, ACTIVATION::TYPE const
   } else if (!act_on_path(t)) {
     return fail("set_layer_activation_function: activation not implemented on this path");
   }
+  if (ptr_array_layers[i].type_layer == LAYER::RESIDUAL) return fail("set_layer_activation_function: a residual entry has no activation of its own");
   ptr_array_layers[i].type_activation_function = t;
   return true;
 }
@@ -228,6 +280,11 @@ bool Model::set_dropout(size_t const i, LAYER_DROPOUT::TYPE const t, real const 
   if (t != LAYER_DROPOUT::NONE && t != LAYER_DROPOUT::BERNOULLI && t != LAYER_DROPOUT::BERNOULLI_INVERTED)
     return fail("set_dropout: dropout type not implemented on this path");
   Layer &l = ptr_array_layers[i];
+  // A block's first layer feeds its weights the (normalized) block input as it
+  // is, without activation or dropout (fwp_st.cpp:4049-4442), and a RESIDUAL
+  // entry has no dropout units.
+  if (t != LAYER_DROPOUT::NONE && (l.type_layer == LAYER::RESIDUAL || l.block_first))
+    return fail("set_dropout: no dropout on a residual entry or on the first layer of its block");
   if (t != LAYER_DROPOUT::NONE) {
     if (values == nullptr || values[0] < 0.0f || values[0] > 1.0f) return fail("set_dropout: keep probability out of [0, 1]");
     l.dropout_values[0] = values[0];
@@ -239,8 +296,8 @@ bool Model::set_dropout(size_t const i, LAYER_DROPOUT::TYPE const t, real const 
 bool Model::set_dropout_mask(size_t const i, uint8_t const *mask) {
   if (ptr_array_layers == nullptr || i == 0 || i >= total_layers || mask == nullptr) return fail("set_dropout_mask: bad argument");
   Layer &l = ptr_array_layers[i];
-  l.mask_dropout_bernoulli.assign(mask, mask + l.n_out);
-  return hip_ok(hipMemcpy(l.d_mask, l.mask_dropout_bernoulli.data(), l.n_out, hipMemcpyHostToDevice), impl_->err, "mask upload");
+  l.mask_dropout_bernoulli.assign(mask, mask + l.n_units);
+  return hip_ok(hipMemcpy(l.d_mask, l.mask_dropout_bernoulli.data(), l.n_units, hipMemcpyHostToDevice), impl_->err, "mask upload");
 }
 
 void Model::Dropout_Bernoulli(void) {
@@ -249,8 +306,8 @@ void Model::Dropout_Bernoulli(void) {
     if (!l.Use__Dropout()) continue;
     real const keep = l.dropout_values[0];
     std::bernoulli_distribution dist(keep);
-    for (size_t j = 0; j < l.n_out; ++j) l.mask_dropout_bernoulli[j] = keep != 0.0f ? (dist(real_gen) ? 1 : 0) : 0;
-    (void)hipMemcpy(l.d_mask, l.mask_dropout_bernoulli.data(), l.n_out, hipMemcpyHostToDevice);
+    for (size_t j = 0; j < l.n_units; ++j) l.mask_dropout_bernoulli[j] = keep != 0.0f ? (dist(real_gen) ? 1 : 0) : 0;
+    (void)hipMemcpy(l.d_mask, l.mask_dropout_bernoulli.data(), l.n_units, hipMemcpyHostToDevice);
   }
 }
 
@@ -263,8 +320,11 @@ bool Model::set_max_batch_size(size_t const n) {
 void Model::free_batch(void) {
   if (ptr_array_layers != nullptr)
     for (Layer *l = ptr_array_layers; l != ptr_last_layer; ++l) {
+      if (l->d_summations == l->d_outputs) l->d_summations = nullptr;  // one buffer for a layer inside a block
       dev_free(l->d_summations); dev_free(l->d_outputs); dev_free(l->d_errors); dev_free(l->d_af_values);
+      dev_free(l->d_block_values);
     }
+  dev_free(impl_->d_input_grad);
   dev_free(impl_->d_input);
   dev_free(impl_->d_targets);
   impl_->allocated_batch = 0;
@@ -276,6 +336,17 @@ bool Model::allocate_batch(size_t const n) {
   std::string &err = impl_->err;
   for (size_t i = 1; i < total_layers; ++i) {
     Layer &l = ptr_array_layers[i];
+    if (l.type_layer == LAYER::RESIDUAL) {
+      if (!dev_alloc(&l.d_outputs, n * l.n_out, err) || !dev_alloc(&l.d_errors, n * l.n_out, err)) return false;
+      if (l.Use__Normalization() && !dev_alloc(&l.d_block_values, n * l.n_units, err)) return false;
+      continue;
+    }
+    if (l.in_block) {
+      if (!dev_alloc(&l.d_outputs, n * l.n_out, err) || !dev_alloc(&l.d_errors, n * l.n_out, err)) return false;
+      l.d_summations = l.d_outputs;
+      if ((l.Use__Normalization() || !l.block_first) && !dev_alloc(&l.d_block_values, n * l.n_inp, err)) return false;
+      continue;
+    }
     if (!dev_alloc(&l.d_summations, n * l.n_out, err) || !dev_alloc(&l.d_outputs, n * l.n_out, err) ||
         !dev_alloc(&l.d_errors, n * l.n_out, err))
       return false;
@@ -286,6 +357,10 @@ bool Model::allocate_batch(size_t const n) {
   }
   size_t const n_in = ptr_array_layers[0].n_out, n_o = ptr_array_layers[total_layers - 1].n_out;
   if (!dev_alloc(&impl_->d_input, n * n_in, err) || !dev_alloc(&impl_->d_targets, n * n_o, err)) return false;
+  // a block that reads the network input still sends a gradient through its first
+  // layer's normalization (for that layer's scale and shift)
+  if (total_layers > 1 && ptr_array_layers[1].type_layer == LAYER::RESIDUAL && !dev_alloc(&impl_->d_input_grad, n * n_in, err))
+    return false;
   size_t const stage = n * (n_in > n_o ? n_in : n_o);
   if (stage > impl_->h_stage_floats) {
     if (impl_->h_stage != nullptr) (void)hipHostFree(impl_->h_stage);
@@ -361,12 +436,14 @@ bool Model::download_layer(size_t const i, int which, size_t batch, float *out) 
     case 0: src = l.d_summations; break;
     case 3: src = l.d_outputs; break;
     case 4: src = l.d_errors; break;
-    case 10: src = l.d_mean; n = l.n_out; break;
-    case 11: src = l.d_std; n = l.n_out; break;
-    case 12: src = l.d_r; n = l.n_out; break;
-    case 13: src = l.d_d; n = l.n_out; break;
+    case 5: src = l.d_block_values; n = batch * (l.type_layer == LAYER::RESIDUAL ? l.n_units : l.n_inp); break;
+    case 10: src = l.d_mean; n = l.n_units; break;
+    case 11: src = l.d_std; n = l.n_units; break;
+    case 12: src = l.d_r; n = l.n_units; break;
+    case 13: src = l.d_d; n = l.n_units; break;
     default: return fail("download_layer: unknown buffer");
   }
+  if (src == nullptr) return fail("download_layer: this entry has no such buffer");
   if (batch > impl_->allocated_batch) return fail("download_layer: batch larger than the allocation");
   return hip_ok(hipMemcpy(out, src, n * sizeof(float), hipMemcpyDeviceToHost), impl_->err, "layer download");
 }
@@ -431,10 +508,15 @@ void Model::forward_pass_device(size_t const B, float const *d_inputs) {
 void Model::forward_layers(size_t const B) {
   dlmi_ctx *ctx = impl_->ctx;
   bool const training = type_state_propagation >= PROPAGATION::TRAINING;
-  float const *in = impl_->cur_input;
-  size_t K = ptr_array_layers[0].n_out;
   for (size_t li = 1; li < total_layers; ++li) {
     Layer &l = ptr_array_layers[li];
+    if (l.type_layer == LAYER::RESIDUAL) continue;  // finished together with the last layer of its block
+    if (l.in_block) {
+      if (!forward_block_layer(B, li)) return;
+      continue;
+    }
+    float const *in = outputs_of(l.feed_index);
+    size_t const K = l.n_inp;
     size_t const H = l.n_out;
     float const *W = impl_->d_params + l.first_connection_index;
     float const *bias = l.Use__Bias() ? impl_->d_params + l.first_bias_connection_index : nullptr;
@@ -499,11 +581,94 @@ void Model::forward_layers(size_t const B) {
       }
     }
     if (rc != DLMI_OK) { fail("forward_pass: layer tail"); return; }
-    in = l.d_outputs;
-    K = H;
   }
   impl_->out_valid = false;
   impl_->out_batch = B;
+}
+
+float const *Model::outputs_of(size_t const li) const {
+  return li == 0 ? impl_->cur_input : ptr_array_layers[li].d_outputs;
+}
+
+// Batch (re)normalization of x [B, layer.n_units] with the layer's scale, shift
+// and statistics, then desc's activation and dropout, in the current propagation
+// state (fwp_st.cpp:596-732): dropout masks only in TRAINING; in every other
+// state plain Bernoulli rescales by the keep probability.
+int Model::norm_act_tail(Layer &l, dlmi_fused_desc d, size_t const B, float const *x, float *y) {
+  dlmi_ctx *ctx = impl_->ctx;
+  size_t const U = l.n_units;
+  float const *gamma = impl_->d_params + l.scale_index, *beta = impl_->d_params + l.shift_index;
+  float *mm = impl_->d_mov_mean + l.unit_index, *ms = impl_->d_mov_std + l.unit_index;
+  if (type_state_propagation >= PROPAGATION::TRAINING) {
+    dlmi_dropout const drop = d.dropout;
+    if (type_state_propagation != PROPAGATION::TRAINING) d.dropout = DLMI_DROP_NONE;
+    int rc = dlmi_fused_norm_act_fwd(ctx, &d, B, U, x, gamma, beta, l.d_mask, l.d_mean, l.d_std, mm, ms, l.d_r, l.d_d, y);
+    if (rc == DLMI_OK && type_state_propagation != PROPAGATION::TRAINING && drop != DLMI_DROP_NONE)
+      rc = dlmi_dropout_fwd(ctx, drop, 0, 0, B, U, nullptr, l.dropout_values[0], y);
+    return rc;
+  }
+  d.drop_scale = l.dropout_values[0];
+  return dlmi_fused_norm_act_infer(ctx, &d, B, U, x, gamma, beta, mm, ms, y);
+}
+
+// Dropout of values [B, units] with the layer's settings when no normalization
+// kernel carries it (fwp_st.cpp:657-732).
+int Model::dropout_tail(Layer const &l, size_t const B, size_t const U, float *v) {
+  if (!l.Use__Dropout()) return DLMI_OK;
+  if (type_state_propagation == PROPAGATION::TRAINING)
+    return dlmi_dropout_fwd(impl_->ctx, static_cast<dlmi_dropout>(l.type_dropout), 1, 0, B, U, l.d_mask,
+                            l.dropout_values[0] == 0.0f ? 0.0f : 1.0f / l.dropout_values[0], v);
+  return dlmi_dropout_fwd(impl_->ctx, static_cast<dlmi_dropout>(l.type_dropout), 0, 0, B, U, nullptr, l.dropout_values[0], v);
+}
+
+// One layer inside a residual block, K inputs -> H outputs
+// (Forward_Pass__Residual__FC__Loop, fwp_st.cpp:4049-4442): normalization of the
+// INPUT, then activation and dropout of that (not for the block's first layer),
+// then the weights (+ bias when the layer is not normalized); the summation is
+// the layer's output.  After the block's last layer: the block-level
+// normalization and the zero-padded identity shortcut with what fed the block
+// (Forward_Pass__Residual__Loop, fwp_st.cpp:3876-4010, 5051-5112).
+bool Model::forward_block_layer(size_t const B, size_t const li) {
+  dlmi_ctx *ctx = impl_->ctx;
+  Layer &l = ptr_array_layers[li];
+  size_t const K = l.n_inp, H = l.n_out;
+  float const *t = outputs_of(l.feed_index);
+  if (!l.block_first && !act_on_path(l.type_activation_function)) return fail("forward_pass: layer activation not set to one on this path");
+  if ((l.Use__Normalization() || !l.block_first) && l.d_block_values == nullptr)
+    return fail("forward_pass: call update_mem_batch_size() after changing a layer's normalization");
+  int rc = DLMI_OK;
+  if (l.Use__Normalization()) {
+    dlmi_fused_desc d = make_desc(*this, l);
+    if (l.block_first) {
+      d.act = DLMI_ACT_LINEAR;
+      d.dropout = DLMI_DROP_NONE;
+    }
+    rc = norm_act_tail(l, d, B, t, l.d_block_values);
+    t = l.d_block_values;
+  } else if (!l.block_first) {
+    rc = dlmi_act_fwd(ctx, static_cast<dlmi_activation>(l.type_activation_function), B, K, t, l.d_block_values);
+    if (rc == DLMI_OK) rc = dropout_tail(l, B, K, l.d_block_values);
+    t = l.d_block_values;
+  }
+  if (rc != DLMI_OK) return fail("forward_pass: block layer input");
+  float const *bias = l.Use__Bias() ? impl_->d_params + l.first_bias_connection_index : nullptr;
+  if (dlmi_fc_fwd(ctx, B, K, H, t, impl_->d_params + l.first_connection_index, bias, l.d_outputs) != DLMI_OK)
+    return fail("forward_pass: dlmi_fc_fwd");
+  Layer &r = ptr_array_layers[l.block_index];
+  if (li != l.block_index + r.block_depth) return true;
+  float const *block = l.d_outputs;
+  if (r.Use__Normalization()) {
+    if (r.d_block_values == nullptr) return fail("forward_pass: call update_mem_batch_size() after changing a layer's normalization");
+    dlmi_fused_desc d = make_desc(*this, r);
+    d.act = DLMI_ACT_LINEAR;
+    d.dropout = DLMI_DROP_NONE;
+    if (norm_act_tail(r, d, B, block, r.d_block_values) != DLMI_OK) return fail("forward_pass: block normalization");
+    block = r.d_block_values;
+  }
+  if (dlmi_zero_padded_identity_fwd(ctx, B, ptr_array_layers[r.feed_index].n_out, H, r.pooling_values[2],
+                                    outputs_of(r.feed_index), block, r.d_outputs) != DLMI_OK)
+    return fail("forward_pass: dlmi_zero_padded_identity_fwd");
+  return true;
 }
 
 var const *Model::get_out(size_t const data_index, size_t const) const {
@@ -611,19 +776,24 @@ bool Model::Use__Dropout__Bernoulli__Inverted(void) const {
 void Model::backward_pass(size_t const B) {
   if (ptr_array_layers == nullptr || B == 0 || B > impl_->allocated_batch) { fail("backward_pass: bad argument"); return; }
   dlmi_ctx *ctx = impl_->ctx;
-  // bwp_st.cpp:106-183: from the layer below the output down to layer 1; the
-  // gradient with respect to the network input is never formed.
-  for (size_t li = total_layers - 2; li >= 1; --li) {
+  // bwp_st.cpp:106-183: from the output layer down to layer 1.  Each plain layer
+  // turns the gradient with respect to its outputs (left in its error buffer by
+  // the entry above) into dZ in place, then hands dZ . W to the entry it reads;
+  // a residual block is unwound as a whole.  The gradient with respect to the
+  // network input is never formed.
+  for (size_t li = total_layers - 1; li >= 1; --li) {
     Layer &l = ptr_array_layers[li];
-    Layer const &nx = ptr_array_layers[li + 1];
-    size_t const H = l.n_out;
-    // dY = dZ_next . W_next, written straight over the (would-be zeroed) buffer
-    if (dlmi_fc_bwd_dx(ctx, B, nx.n_out, H, nx.d_errors, impl_->d_params + nx.first_connection_index, l.d_errors, 0) != DLMI_OK) {
-      fail("backward_pass: dlmi_fc_bwd_dx");
-      return;
+    if (l.in_block) {
+      if (!backward_block(B, l.block_index)) return;
+      li = l.block_index;
+      if (li == 1) break;
+      continue;
     }
-    int rc;
-    if (l.Use__Normalization() && !l.use_layer_normalization_before_activation) {
+    size_t const H = l.n_out;
+    int rc = DLMI_OK;
+    if (li + 1 == total_layers) {
+      // the output layer's dZ is the seed gradient of compute_error()
+    } else if (l.Use__Normalization() && !l.use_layer_normalization_before_activation) {
       // bwp_st.cpp:559-606, 619-632: normalization backward on the activation
       // values (in REFERENCE dropout mode the gradient passes unmasked), then the
       // activation derivative with the summations and the activation values
@@ -648,8 +818,70 @@ void Model::backward_pass(size_t const B) {
                         l.d_errors, l.d_errors);
     }
     if (rc != DLMI_OK) { fail("backward_pass: layer gradient"); return; }
+    // dY = dZ . W, written straight over the (would-be zeroed) buffer of the entry this layer reads
+    if (l.feed_index != 0 &&
+        dlmi_fc_bwd_dx(ctx, B, H, l.n_inp, l.d_errors, impl_->d_params + l.first_connection_index,
+                       ptr_array_layers[l.feed_index].d_errors, 0) != DLMI_OK) {
+      fail("backward_pass: dlmi_fc_bwd_dx");
+      return;
+    }
     if (li == 1) break;
   }
+}
+
+// Backward of the residual block whose RESIDUAL entry is `ri`, given the gradient
+// with respect to the block's output in that entry's error buffer
+// (bwp_st.cpp:345-541, 1112-1175): the block's share through the block-level
+// normalization and the layers from last to first, each layer's dZ left in its
+// error buffer; then both shares into the entry that fed the block.  As in the
+// plain layers, activation derivatives see post-dropout values and the gradient
+// itself is not masked unless dropout_backward_mode says so.
+bool Model::backward_block(size_t const B, size_t const ri) {
+  dlmi_ctx *ctx = impl_->ctx;
+  Layer &r = ptr_array_layers[ri];
+  size_t const D = r.block_depth, f = r.feed_index, pad = r.pooling_values[2];
+  Layer &last = ptr_array_layers[ri + D];
+  size_t const HD = last.n_out;
+  float *g = last.d_errors;
+  if (!hip_ok(hipMemsetAsync(g, 0, B * HD * sizeof(float), impl_->stream), impl_->err, "memset")) return false;
+  if (dlmi_residual_bwd(ctx, B, r.n_out, HD, pad, r.d_errors, g) != DLMI_OK) return fail("backward_pass: dlmi_residual_bwd");
+  if (r.Use__Normalization()) {
+    dlmi_fused_desc d = make_desc(*this, r);
+    d.act = DLMI_ACT_LINEAR;
+    d.dropout = DLMI_DROP_NONE;
+    if (dlmi_fused_norm_act_bwd(ctx, &d, B, HD, last.d_outputs, impl_->d_params + r.scale_index, impl_->d_params + r.shift_index,
+                                r.d_mask, r.d_mean, r.d_std, r.d_r, r.d_d, g, impl_->d_dparams + r.scale_index,
+                                impl_->d_dparams + r.shift_index, g) != DLMI_OK)
+      return fail("backward_pass: block normalization");
+  }
+  for (size_t i = ri + D; i > ri; --i) {
+    Layer &l = ptr_array_layers[i];
+    size_t const K = l.n_inp;
+    // the gradient with respect to what layer i reads goes where that entry keeps its own
+    float *dst = l.feed_index == 0 ? impl_->d_input_grad : ptr_array_layers[l.feed_index].d_errors;
+    if (l.feed_index == 0 && !l.Use__Normalization()) break;  // nothing below needs it
+    if (dlmi_fc_bwd_dx(ctx, B, l.n_out, K, l.d_errors, impl_->d_params + l.first_connection_index, dst, 0) != DLMI_OK)
+      return fail("backward_pass: dlmi_fc_bwd_dx");
+    float const *x = outputs_of(l.feed_index);
+    int rc = DLMI_OK;
+    if (l.Use__Normalization()) {
+      dlmi_fused_desc d = make_desc(*this, l);
+      if (l.block_first) {
+        d.act = DLMI_ACT_LINEAR;
+        d.dropout = DLMI_DROP_NONE;
+      }
+      if (type_state_propagation != PROPAGATION::TRAINING) d.dropout = DLMI_DROP_NONE;
+      rc = dlmi_fused_norm_act_bwd(ctx, &d, B, K, x, impl_->d_params + l.scale_index, impl_->d_params + l.shift_index, l.d_mask,
+                                   l.d_mean, l.d_std, l.d_r, l.d_d, dst, impl_->d_dparams + l.scale_index,
+                                   impl_->d_dparams + l.shift_index, dst);
+    } else if (!l.block_first) {
+      rc = dlmi_act_bwd(ctx, static_cast<dlmi_activation>(l.type_activation_function), B, K, x, l.d_block_values, dst, dst);
+    }
+    if (rc != DLMI_OK) return fail("backward_pass: block layer gradient");
+  }
+  if (f != 0 && dlmi_residual_bwd(ctx, B, r.n_out, ptr_array_layers[f].n_out, pad, r.d_errors, ptr_array_layers[f].d_errors) != DLMI_OK)
+    return fail("backward_pass: dlmi_residual_bwd");
+  return true;
 }
 
 void Model::update_derivatives(size_t const B, Layer *const first, Layer const *const last) {
@@ -659,9 +891,11 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
   }
   for (Layer *l = first; l != last; ++l) {
     size_t const li = static_cast<size_t>(l - ptr_array_layers);
-    if (li == 0 || li >= total_layers) continue;
-    float const *in = li == 1 ? impl_->cur_input : ptr_array_layers[li - 1].d_outputs;
-    size_t const K = ptr_array_layers[li - 1].n_out;
+    if (li == 0 || li >= total_layers || l->type_layer != LAYER::FULLY_CONNECTED) continue;
+    // what the weights saw: the feeding entry's outputs, or a block layer's own
+    // normalized / activated copy of them
+    float const *in = l->in_block && (l->Use__Normalization() || !l->block_first) ? l->d_block_values : outputs_of(l->feed_index);
+    size_t const K = l->n_inp;
     float *db = l->Use__Bias() ? impl_->d_dparams + l->first_bias_connection_index : nullptr;
     if (dlmi_fc_bwd_dw(impl_->ctx, B, K, l->n_out, in, l->d_errors, impl_->d_dparams + l->first_connection_index, db, 1) != DLMI_OK) {
       fail("update_derivatives: dlmi_fc_bwd_dw");

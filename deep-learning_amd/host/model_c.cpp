@@ -39,6 +39,38 @@ dlmi_model *dlmi_model_create(size_t n_layers, size_t const *widths) {
   return h;
 }
 
+dlmi_model *dlmi_model_create_typed(size_t n_layers, int const *types, size_t const *units) {
+  if (types == nullptr || units == nullptr) return nullptr;
+  dlmi_model *h = new dlmi_model;
+  std::vector<Layer_Parameters> lp(n_layers);
+  for (size_t i = 0; i < n_layers; ++i) {
+    lp[i].type_layer = static_cast<LAYER::TYPE>(types[i]);
+    lp[i].unit_parameters[0] = units[i];
+  }
+  if (!h->m.compile(n_layers, 1, MODEL::FEEDFORWARD, lp.data())) {
+    delete h;
+    return nullptr;
+  }
+  return h;
+}
+
+void dlmi_model_layer_info(dlmi_model const *h, size_t layer, size_t *out) {
+  Layer const &l = h->m.ptr_array_layers[layer];
+  bool const fc = layer > 0 && l.type_layer == LAYER::FULLY_CONNECTED;
+  out[0] = static_cast<size_t>(l.type_layer);
+  out[1] = l.n_out;
+  out[2] = fc ? l.first_connection_index : 0;
+  out[3] = fc ? l.first_connection_index + l.n_out * l.n_inp : 0;
+  out[4] = fc ? l.first_bias_connection_index : 0;
+  out[5] = l.Use__Bias();
+  out[6] = l.n_units;
+  out[7] = l.scale_index;
+  out[8] = l.unit_index;
+  out[9] = l.type_layer == LAYER::RESIDUAL ? 0 : (l.in_block ? (l.block_first ? 0 : l.n_units) : l.n_out);
+  out[10] = l.block_depth;
+  out[11] = l.pooling_values[2];
+}
+
 void dlmi_model_destroy(dlmi_model *h) { delete h; }
 char const *dlmi_model_last_error(dlmi_model const *h) { return h ? h->m.last_error() : "null model"; }
 

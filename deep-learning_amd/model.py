@@ -22,8 +22,10 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_model_get_out", "dlmi_model_loss_sum", "dlmi_model_accuracy_sum", "dlmi_model_set_optimizer",
     "dlmi_model_set_epoch_time_step", "dlmi_model_set_derivatives", "dlmi_model_update_parameter",
     "dlmi_model_get_optimizer_state", "dlmi_driver_create", "dlmi_driver_destroy", "dlmi_driver_train",
-    "dlmi_driver_evalt",
+    "dlmi_driver_evalt", "dlmi_model_create_typed", "dlmi_model_layer_info",
 ]
+
+LAYER_FULLY_CONNECTED, LAYER_RESIDUAL = 3, 9  # v1/data/enum/layer.hpp
 
 
 def _ptr(a):
@@ -35,22 +37,30 @@ class Model:
     wrappers in oracle/binding.py, so one test body can run all three."""
 
     def __init__(self, lib, widths):
+        self._bind(lib)
+        self.widths = [int(w) for w in widths]
+        arr = (c_sz * len(widths))(*self.widths)
+        h = lib.dlmi_model_create(c_sz(len(widths)), arr)
+        self._created(h)
+
+    def _bind(self, lib):
         self.lib = lib
         lib.dlmi_model_create.restype = vp
+        lib.dlmi_model_create_typed.restype = vp
         lib.dlmi_model_last_error.restype = ctypes.c_char_p
         lib.dlmi_model_last_error.argtypes = [vp]
         lib.dlmi_model_total_parameters.restype = c_sz
         lib.dlmi_model_total_normalized_units.restype = c_sz
         lib.dlmi_model_loss_sum.restype = ctypes.c_double
         lib.dlmi_model_accuracy_sum.restype = ctypes.c_double
-        self.widths = [int(w) for w in widths]
-        arr = (c_sz * len(widths))(*self.widths)
-        h = lib.dlmi_model_create(c_sz(len(widths)), arr)
+
+    def _created(self, h):
         if not h:
-            raise RuntimeError("dlmi_model_create failed (no GPU, or the library is not built for it)")
+            raise RuntimeError("dlmi_model_create failed (no GPU, the library is not built for it, or a layer list "
+                               "the path does not take)")
         self.h = vp(h)
-        self.P = lib.dlmi_model_total_parameters(self.h)
-        self.n_units = lib.dlmi_model_total_normalized_units(self.h)
+        self.P = self.lib.dlmi_model_total_parameters(self.h)
+        self.n_units = self.lib.dlmi_model_total_normalized_units(self.h)
         self.max_batch = 0
 
     def close(self):
@@ -204,3 +214,47 @@ class Model:
         out = (ctypes.c_double * 2)()
         self._ok(self.lib.dlmi_driver_evalt(self._driver(X, Y, on_device), out), "Driver::evalt")
         return out[0], out[1]
+
+
+class Net(Model):
+    """A Model compiled from a typed layer list: ("FC", units) entries and
+    ("RES", depth) entries, each of the latter followed by the `depth` layers of its
+    residual block.  Entry 0 is the input width.  Same driving interface as
+    OracleNet / ReferenceNet in oracle/binding.py."""
+
+    INFO_KEYS = ("type", "n_out", "w0", "w1", "bias", "use_bias", "n_unit", "gamma", "unit", "n_af", "depth", "padding")
+
+    def __init__(self, lib, layers):
+        self._bind(lib)
+        self.layers = list(layers)
+        n = len(self.layers)
+        types = (c_int * n)(*[LAYER_FULLY_CONNECTED if e[0] == "FC" else LAYER_RESIDUAL for e in self.layers])
+        units = (c_sz * n)(*[int(e[1]) for e in self.layers])
+        self._created(lib.dlmi_model_create_typed(c_sz(n), types, units))
+        self.widths = [self.info(l)["n_out"] for l in range(n)]
+
+    def info(self, l):
+        out = (c_sz * 12)()
+        self.lib.dlmi_model_layer_info(self.h, c_sz(l), out)
+        return dict(zip(self.INFO_KEYS, (int(v) for v in out)))
+
+    def fc_layers(self):
+        return [l for l, e in enumerate(self.layers) if l > 0 and e[0] == "FC"]
+
+    def set_layer(self, l, act, norm=0, drop=0, keep=1.0, mask=None, norm_before=True):
+        if self.layers[l][0] == "FC":
+            self._ok(self.lib.dlmi_model_set_layer_activation_function(self.h, c_sz(l), c_int(act)), "activation")
+        if norm:
+            self._ok(self.lib.dlmi_model_set_layer_normalization(self.h, c_sz(l), c_int(norm)), "normalization")
+        if drop:
+            self._ok(self.lib.dlmi_model_set_dropout(self.h, c_sz(l), c_int(drop), c_f(keep)), "dropout")
+        if mask is not None:
+            m = np.ascontiguousarray(mask, dtype=np.uint8)
+            assert m.size == self.info(l)["n_unit"], "one mask entry per dropout unit of the entry"
+            self._ok(self.lib.dlmi_model_set_dropout_mask(self.h, c_sz(l), _ptr(m)), "dropout mask")
+
+    def layer_output(self, l):
+        return self.layer_buffer(l, 3)
+
+    def layer_error(self, l):
+        return self.layer_buffer(l, 4)

@@ -18,6 +18,14 @@ typedef struct dlmi_model dlmi_model;
 
 /* new Model + compile(n_layers, 1, MODEL::FEEDFORWARD, {FULLY_CONNECTED, widths[i]}) */
 dlmi_model *dlmi_model_create(size_t n_layers, size_t const *widths);
+/* The same with typed entries: types[i] is LAYER::FULLY_CONNECTED (3) with units[i]
+ * units, or LAYER::RESIDUAL (9) with units[i] = the depth of the block, followed by
+ * that many fully-connected entries (compile.cpp:127-170, 283-520). */
+dlmi_model *dlmi_model_create_typed(size_t n_layers, int const *types, size_t const *units);
+/* out[0..11] = type, outputs, first weight index, one past the last weight, bias
+ * index, Use__Bias(), normalization units, gamma index, moving-statistic index,
+ * activation units, block depth, zero padding of the shortcut */
+void dlmi_model_layer_info(dlmi_model const *m, size_t layer, size_t *out);
 void dlmi_model_destroy(dlmi_model *m);
 char const *dlmi_model_last_error(dlmi_model const *m);
 int dlmi_model_set_layer_activation_function(dlmi_model *m, size_t layer, int activation);

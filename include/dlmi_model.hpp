@@ -13,9 +13,10 @@
 //     download_derivatives() (the reference's members are the storage itself);
 //   * OpenMP knobs (set_mp, update_mem_thread_size, merge_mp_derivatives) are
 //     accepted and do nothing: there are no per-thread gradient copies to merge;
-//   * only LAYER::FULLY_CONNECTED layers, the activations ReLU / leaky ReLU /
-//     ELU / SELU / ISRLU / linear (+ softmax on the output layer), batch
-//     normalization / renormalization before the activation, Bernoulli and
+//   * only LAYER::FULLY_CONNECTED layers and LAYER::RESIDUAL blocks of them
+//     (a {RESIDUAL, depth} entry followed by the `depth` layers of its block),
+//     the activations ReLU / leaky ReLU / ELU / SELU / ISRLU / linear (+ softmax
+//     on the output layer), batch normalization / renormalization, Bernoulli and
 //     inverted-Bernoulli dropout and the cross-entropy loss are implemented;
 //     anything else makes the setter return false, as the reference does for
 //     settings it refuses.
@@ -80,19 +81,34 @@ struct Layer {
   bool use_layer_normalization_before_activation = true;
   real dropout_values[3] = {0};  // [0]: keep probability
   size_t n_out = 0;
-  size_t first_connection_index = 0;       // offset of W [n_out][n_in] in the parameter array
+  size_t n_inp = 0;                        // inputs of a fully-connected entry
+  // Normalization, activation and dropout units (compile.cpp:283-520): n_out for a
+  // plain layer; as many as the INPUTS for a layer inside a residual block (which
+  // normalizes and activates what it reads, not what it writes); the width of the
+  // block's last layer for a RESIDUAL entry.
+  size_t n_units = 0;
+  size_t feed_index = 0;                   // the entry whose outputs this entry reads
+  size_t block_depth = 0;                  // RESIDUAL: layers in its block (model.hpp Layer::block_depth)
+  size_t block_index = 0;                  // layer inside a block: index of its RESIDUAL entry
+  size_t pooling_values[5] = {0};          // RESIDUAL: [2] zero padding of the shortcut (compile.cpp:495-510)
+  bool in_block = false, block_first = false;
+  size_t first_connection_index = 0;       // offset of W [n_out][n_inp] in the parameter array
   size_t first_bias_connection_index = 0;  // offset of the bias slot [n_out]
-  size_t scale_index = 0, shift_index = 0; // offsets of gamma / beta [n_out]
+  size_t scale_index = 0, shift_index = 0; // offsets of gamma / beta [n_units]
   size_t unit_index = 0;                   // offset in the moving-statistic arrays
-  std::vector<uint8_t> mask_dropout_bernoulli;  // host copy of the per-unit mask [n_out]
+  std::vector<uint8_t> mask_dropout_bernoulli;  // host copy of the per-unit mask [n_units]
 
-  float *d_summations = nullptr;          // Z (Neuron_unit::ptr_array_summations)
+  float *d_summations = nullptr;          // Z (Neuron_unit::ptr_array_summations); a block layer's output is its Z
   float *d_outputs = nullptr;             // layer output after activation and dropout (ptr_array_outputs)
-  float *d_errors = nullptr;              // dZ (Neuron_unit::ptr_array_errors); holds dY in between
+  float *d_errors = nullptr;              // dZ (Neuron_unit::ptr_array_errors); holds dY in between.  RESIDUAL:
+                                          // the gradient with respect to the block's output
   float *d_af_values = nullptr;           // activation values (AF_unit::ptr_array_values), kept only when the
                                           // normalization comes after the activation
-  float *d_mean = nullptr, *d_std = nullptr, *d_r = nullptr, *d_d = nullptr;  // batch statistics [n_out]
-  uint8_t *d_mask = nullptr;              // device copy of the dropout mask [n_out]
+  float *d_block_values = nullptr;        // layer inside a block: what its weights see [batch, n_inp] (the
+                                          // normalized, activated, dropped-out input); RESIDUAL: the normalized
+                                          // output of the block [batch, n_units]
+  float *d_mean = nullptr, *d_std = nullptr, *d_r = nullptr, *d_d = nullptr;  // batch statistics [n_units]
+  uint8_t *d_mask = nullptr;              // device copy of the dropout mask [n_units]
 
   size_t get_n_out(void) const { return n_out; }
   bool Use__Normalization(void) const { return type_normalization != LAYER_NORM::NONE; }
@@ -236,6 +252,11 @@ class Model {
   Impl *impl_;
   bool allocate_batch(size_t batch);
   void forward_layers(size_t batch);
+  bool forward_block_layer(size_t batch, size_t index_layer);
+  bool backward_block(size_t batch, size_t index_residual);
+  int norm_act_tail(Layer &layer, dlmi_fused_desc desc, size_t batch, float const *x, float *y);
+  int dropout_tail(Layer const &layer, size_t batch, size_t units, float *values);
+  float const *outputs_of(size_t index_layer) const;
   void seed_error(size_t batch, float const *d_targets);
   void free_batch(void);
   bool fail(char const *what) const;
