@@ -1,5 +1,6 @@
 // C binding of the Model facade (include/dlmi_model.h).
 #include <cstring>
+#include <string>
 #include <vector>
 
 #include "../../include/dlmi_driver.hpp"
@@ -20,6 +21,11 @@ struct dlmi_driver {
   dlmi::Dataset ds;
   dlmi::Driver *drv = nullptr;
   ~dlmi_driver() { delete drv; }
+};
+
+struct dlmi_mnist {
+  explicit dlmi_mnist(char const *workdir) : ds(std::string(workdir)) {}
+  dlmi::MNIST ds;
 };
 
 extern "C" {
@@ -233,6 +239,27 @@ dlmi_driver *dlmi_driver_create(dlmi_model *h, size_t n_data, float const *X, fl
   d->drv->keep_dataset_on_device = on_device != 0;
   return d;
 }
+dlmi_mnist *dlmi_mnist_create(char const *workdir) {
+  if (workdir == nullptr) return nullptr;
+  return new dlmi_mnist(workdir);
+}
+void dlmi_mnist_destroy(dlmi_mnist *h) { delete h; }
+int dlmi_mnist_load(dlmi_mnist *h, int env, size_t *shape) {
+  if (h == nullptr || shape == nullptr) return 0;
+  bool const ok = h->ds.load(static_cast<ENV::TYPE>(env));
+  shape[0] = h->ds.n_data;
+  shape[1] = h->ds.n_inp;
+  shape[2] = h->ds.n_out;
+  return ok ? 1 : 0;
+}
+char const *dlmi_mnist_last_error(dlmi_mnist const *h) { return h ? h->ds.last_error() : "null data set"; }
+int dlmi_mnist_copy(dlmi_mnist const *h, float *X, float *Y) {
+  if (h == nullptr || h->ds.n_data == 0) return 0;
+  if (X != nullptr) std::memcpy(X, h->ds.X, h->ds.n_data * h->ds.n_inp * sizeof(float));
+  if (Y != nullptr) std::memcpy(Y, h->ds.Y, h->ds.n_data * h->ds.n_out * sizeof(float));
+  return 1;
+}
+
 void dlmi_driver_destroy(dlmi_driver *d) { delete d; }
 int dlmi_driver_train(dlmi_driver *d, int resample_dropout_masks, double *out) {
   if (d == nullptr || out == nullptr) return 0;

@@ -22,7 +22,8 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_model_get_out", "dlmi_model_loss_sum", "dlmi_model_accuracy_sum", "dlmi_model_set_optimizer",
     "dlmi_model_set_epoch_time_step", "dlmi_model_set_derivatives", "dlmi_model_update_parameter",
     "dlmi_model_get_optimizer_state", "dlmi_driver_create", "dlmi_driver_destroy", "dlmi_driver_train",
-    "dlmi_driver_evalt", "dlmi_model_create_typed", "dlmi_model_layer_info",
+    "dlmi_driver_evalt", "dlmi_model_create_typed", "dlmi_model_layer_info", "dlmi_mnist_create",
+    "dlmi_mnist_destroy", "dlmi_mnist_load", "dlmi_mnist_last_error", "dlmi_mnist_copy",
 ]
 
 LAYER_FULLY_CONNECTED, LAYER_RESIDUAL = 3, 9  # v1/data/enum/layer.hpp
@@ -214,6 +215,26 @@ class Model:
         out = (ctypes.c_double * 2)()
         self._ok(self.lib.dlmi_driver_evalt(self._driver(X, Y, on_device), out), "Driver::evalt")
         return out[0], out[1]
+
+
+def load_mnist(lib, workdir, train=True):
+    """dlmi::MNIST(workdir).load(ENV::TRAIN or ENV::TESTG): (X [n, rows*cols] in [0, 1],
+    Y [n, 10] one-hot) from the IDX files in `workdir`.  Host code only (no GPU needed)."""
+    lib.dlmi_mnist_create.restype = vp
+    lib.dlmi_mnist_last_error.restype = ctypes.c_char_p
+    lib.dlmi_mnist_last_error.argtypes = [vp]
+    h = vp(lib.dlmi_mnist_create(str(workdir).encode()))
+    try:
+        shape = (c_sz * 3)()
+        if not lib.dlmi_mnist_load(h, c_int(1 if train else 3), shape):
+            raise RuntimeError("MNIST::load failed: " + lib.dlmi_mnist_last_error(h).decode())
+        X = np.empty((shape[0], shape[1]), np.float32)
+        Y = np.empty((shape[0], shape[2]), np.float32)
+        if not lib.dlmi_mnist_copy(h, _ptr(X), _ptr(Y)):
+            raise RuntimeError("dlmi_mnist_copy failed")
+        return X, Y
+    finally:
+        lib.dlmi_mnist_destroy(h)
 
 
 class Net(Model):

@@ -19,6 +19,7 @@
 #define DLMI_DRIVER_HPP
 
 #include <cstddef>
+#include <string>
 
 #include "dlmi_model.hpp"
 
@@ -30,6 +31,37 @@ struct Dataset {
   size_t n_data = 0, n_inp = 0, n_out = 0, seq_w = 1;
   v1::real const **Xm = nullptr;  // n_data row pointers, n_inp floats each
   v1::real const **Ym = nullptr;  // n_data row pointers, n_out floats each
+};
+
+// The MNIST reader of the reference (data/dataset/mnist.hpp:27-45,
+// mnist.cpp:56-227): `load(ENV::TRAIN)` reads train-images-idx3-ubyte and
+// train-labels-idx1-ubyte from the working directory, any other environment the
+// t10k pair.  Images: big-endian header {2051, count, rows, cols}, then one
+// unsigned byte per pixel, stored as byte / 255; labels: header {2049, count},
+// one byte per example, stored one-hot over 10 classes.  The object owns the
+// rows.  Unlike the reference it never downloads: missing files make load()
+// return false.
+class MNIST : public Dataset {
+ public:
+  explicit MNIST(std::wstring const &workdir);
+  explicit MNIST(std::string const &workdir);
+  ~MNIST(void);
+  MNIST(MNIST const &) = delete;
+  MNIST &operator=(MNIST const &) = delete;
+
+  bool load(v1::ENV::TYPE const &env_type);
+  char const *last_error(void) const { return err_.c_str(); }
+
+  v1::real *X = nullptr;  // [n_data, n_inp], rows * cols pixels per example
+  v1::real *Y = nullptr;  // [n_data, 10]
+  std::string workdir;
+
+ private:
+  bool load_images(std::string const &path_name, size_t shape[2]);
+  bool load_labels(std::string const &path_name, size_t shape[2]);
+  void release(void);
+  int n_rows_ = 0, n_cols_ = 0;
+  std::string err_;
 };
 
 class Driver {
@@ -71,6 +103,7 @@ class Driver {
 namespace DL {
 using ::dlmi::Dataset;
 using ::dlmi::Driver;
+using ::dlmi::MNIST;
 using ENV = ::dlmi::v1::ENV;  // DL::ENV::TYPE, DL::ENV::TRAIN ... (data/enum/env.hpp)
 }  // namespace DL
 #endif

@@ -76,6 +76,16 @@ void dlmi_driver_destroy(dlmi_driver *d);
 int dlmi_driver_train(dlmi_driver *d, int resample_dropout_masks, double *out);
 int dlmi_driver_evalt(dlmi_driver *d, double *out);
 
+/* ---- MNIST reader (data/dataset/mnist.cpp:56-227): IDX files of `workdir`, pixels / 255,
+ * one-hot labels over 10 classes.  env = ENV::TRAIN (1) reads the train pair, any other
+ * value the t10k pair.  Never downloads.  shape = {n_data, n_inp, n_out}. */
+typedef struct dlmi_mnist dlmi_mnist;
+dlmi_mnist *dlmi_mnist_create(char const *workdir);
+void dlmi_mnist_destroy(dlmi_mnist *d);
+int dlmi_mnist_load(dlmi_mnist *d, int env, size_t *shape);
+char const *dlmi_mnist_last_error(dlmi_mnist const *d);
+int dlmi_mnist_copy(dlmi_mnist const *d, float *X, float *Y); /* dense [n_data, n_inp] and [n_data, n_out] */
+
 #ifdef __cplusplus
 }
 #endif
