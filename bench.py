@@ -438,6 +438,14 @@ def main():
         t_ad = time_events(torch, step.adam, 10)
         detail["adam_step"] = {"ms": t_ad, "bytes": 32.0 * H * K, "GBps": 32.0 * H * K / t_ad / 1e6,
                                "frac_hbm_peak": 32.0 * H * K / t_ad / 1e6 / HBM_PEAK_GBS}
+        # What a caller pays who hands over host rows every step, as the facade's forward_pass(batch, rows)
+        # does: the [B, K] input block from pinned host memory over PCIe, on top of the step.  Not `value`.
+        pinned = torch.empty((B, K), dtype=torch.float32, pin_memory=True)
+        pinned.copy_(t["X"])
+        staging = torch.empty_like(t["X"])
+        t_up = time_events(torch, lambda: staging.copy_(pinned, non_blocking=True), 5, warmup=1)
+        detail["host_rows_upload"] = {"ms": t_up, "GBps": 4.0 * B * K / t_up / 1e6,
+                                      "samples_per_s_with_upload": B / ((ms_per_step + t_up) * 1e-3)}
     else:
         roof = dict(hbm)
 
