@@ -15,6 +15,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <limits>
 #include <string>
 #include <vector>
 
@@ -38,6 +39,7 @@ struct Model::Impl {
   float *d_opt[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
   float const *cur_input = nullptr;  // [batch, n_in] of the pass in flight: d_input or a caller's device rows
   size_t n_loss_examples = 0;        // examples whose loss has been accumulated since reset_loss()
+  size_t all_units = 0;              // normalization units of all entries: the slots a normalized model has
   float *h_stage = nullptr;    // pinned staging for the row-pointer gather
   size_t h_stage_floats = 0;
   mutable std::vector<float> out_host;  // get_out() cache
@@ -206,21 +208,11 @@ bool Model::compile(size_t const n_layers, size_t const number_recurrent_depth_r
   }
   total_weights = nw;
   total_bias = nb;
-  total_normalized_units = nu;
-  total_parameters = nw + nb + 2 * nu;
-  ptr_array_parameters = new var[total_parameters]();
-  ptr_array_derivatives_parameters = new real[total_parameters]();
-  ptr_array_normalized_batch_units_means_averages = new var[nu]();
-  ptr_array_normalized_batch_units_variances_averages = new var[nu];
-  for (size_t i = 0; i < nu; ++i) {  // allocate.cpp:1167-1170, 1274-1284
-    ptr_array_parameters[nw + nb + i] = 1.0f;
-    ptr_array_normalized_batch_units_variances_averages[i] = 1.0f;
-  }
+  impl_->all_units = nu;
   std::string &err = impl_->err;
-  if (!dev_alloc(&impl_->d_params, total_parameters, err) || !dev_alloc(&impl_->d_dparams, total_parameters, err) ||
-      !dev_alloc(&impl_->d_mov_mean, nu, err) || !dev_alloc(&impl_->d_mov_std, nu, err) ||
-      !dev_alloc(&impl_->d_stats, 2, err))
-    return false;
+  // the scale / shift slots and the moving statistics come with the first
+  // normalized layer (normalization.cpp:296-352), not before
+  if (!resize_normalization_slots(false) || !dev_alloc(&impl_->d_stats, 2, err)) return false;
   for (size_t i = 1; i < n_layers; ++i) {
     Layer &l = ptr_array_layers[i];
     if (!dev_alloc(&l.d_mean, l.n_units, err) || !dev_alloc(&l.d_std, l.n_units, err) ||
@@ -229,10 +221,51 @@ bool Model::compile(size_t const n_layers, size_t const number_recurrent_depth_r
     l.mask_dropout_bernoulli.assign(l.n_units, 1);
     if (!hip_ok(hipMemset(l.d_mask, 1, l.n_units ? l.n_units : 1), err, "mask fill")) return false;
   }
-  if (!hip_ok(hipMemsetAsync(impl_->d_dparams, 0, total_parameters * sizeof(float), impl_->stream), err, "memset") ||
-      !hip_ok(hipMemsetAsync(impl_->d_stats, 0, 2 * sizeof(double), impl_->stream), err, "memset"))
+  if (!hip_ok(hipMemsetAsync(impl_->d_stats, 0, 2 * sizeof(double), impl_->stream), err, "memset")) return false;
+  return set_max_batch_size(1) && update_mem_batch_size(1);
+}
+
+// The packed parameter array is [weights | biases] until a layer asks for
+// normalization; then it grows by one scale and one shift slot per unit of
+// EVERY entry, and the moving statistics appear (Allocate__Parameter__Normalization
+// and Allocate__Normalized_Unit, allocate.cpp:1150-1330, on the first normalized
+// layer, normalization.cpp:296-352); when the last normalized layer goes back to
+// NONE they are dropped again (normalization.cpp:356-368).  Weights and biases
+// keep their values; scales start at 1, shifts at 0, moving means at 0, moving
+// std-devs at 1; the gradient array and the optimizer's arrays start over.
+bool Model::resize_normalization_slots(bool const present) {
+  Impl &m = *impl_;
+  std::string &err = m.err;
+  size_t const nwb = total_weights + total_bias, nu = present ? m.all_units : 0, P = nwb + 2 * nu;
+  if (m.ctx != nullptr) (void)dlmi_ctx_synchronize(m.ctx);
+  var *params = new var[P ? P : 1]();
+  if (ptr_array_parameters != nullptr) {
+    if (m.d_params != nullptr && !download_parameters()) { delete[] params; return false; }
+    std::memcpy(params, ptr_array_parameters, nwb * sizeof(var));
+  }
+  for (size_t i = 0; i < nu; ++i) params[nwb + i] = 1.0f;  // allocate.cpp:1167-1170
+  delete[] ptr_array_parameters;
+  delete[] ptr_array_derivatives_parameters;
+  delete[] ptr_array_normalized_batch_units_means_averages;
+  delete[] ptr_array_normalized_batch_units_variances_averages;
+  ptr_array_parameters = params;
+  ptr_array_derivatives_parameters = new real[P ? P : 1]();
+  ptr_array_normalized_batch_units_means_averages = new var[nu ? nu : 1]();
+  ptr_array_normalized_batch_units_variances_averages = new var[nu ? nu : 1];
+  for (size_t i = 0; i < (nu ? nu : 1); ++i) ptr_array_normalized_batch_units_variances_averages[i] = 1.0f;  // allocate.cpp:1274-1284
+  total_parameters = P;
+  total_normalized_units = nu;
+  dev_free(m.d_params);
+  dev_free(m.d_dparams);
+  dev_free(m.d_mov_mean);
+  dev_free(m.d_mov_std);
+  for (float *&s : m.d_opt) dev_free(s);
+  if (!dev_alloc(&m.d_params, P, err) || !dev_alloc(&m.d_dparams, P, err) || !dev_alloc(&m.d_mov_mean, nu, err) ||
+      !dev_alloc(&m.d_mov_std, nu, err))
     return false;
-  return upload_parameters() && upload_moving_statistics() && set_max_batch_size(1) && update_mem_batch_size(1);
+  if (!hip_ok(hipMemsetAsync(m.d_dparams, 0, (P ? P : 1) * sizeof(float), m.stream), err, "memset")) return false;
+  if (!upload_parameters() || !upload_moving_statistics()) return false;
+  return weight_decay == 0.0f || set_weight_decay(weight_decay);  // the regularization mask has the array's length
 }
 
 bool Model::set_layer_activation_function(size_t const i, ACTIVATION::TYPE const t) {
@@ -242,7 +275,7 @@ bool Model::set_layer_activation_function(size_t const i, ACTIVATION::TYPE const
   } else if (!act_on_path(t)) {
     return fail("set_layer_activation_function: activation not implemented on this path");
   }
-  if (ptr_array_layers[i].type_layer == LAYER::RESIDUAL) return fail("set_layer_activation_function: a residual entry has no activation of its own");
+  if (ptr_array_layers[i].type_layer == LAYER::RESIDUAL) return true;  // useless there, accepted with a warning (train.cpp:380-387)
   ptr_array_layers[i].type_activation_function = t;
   return true;
 }
@@ -254,7 +287,18 @@ bool Model::Set__Layer_Normalization(size_t const i, LAYER_NORM::TYPE const t, b
   if (i + 1 == total_layers) return fail("Layer received as argument is the output layer.");
   if (t != LAYER_NORM::NONE && t != LAYER_NORM::BATCH_NORMALIZATION && t != LAYER_NORM::BATCH_RENORMALIZATION)
     return fail("Set__Layer_Normalization: normalization type not implemented on this path");
+  auto any_normalized = [this]() {
+    for (Layer const *l = ptr_array_layers; l != ptr_last_layer; ++l)
+      if (l->Use__Normalization()) return true;
+    return false;
+  };
+  bool const had = any_normalized();
+  LAYER_NORM::TYPE const before = ptr_array_layers[i].type_normalization;
   ptr_array_layers[i].type_normalization = t;
+  if (any_normalized() != had && !resize_normalization_slots(!had)) {
+    ptr_array_layers[i].type_normalization = before;
+    return false;
+  }
   return true;
 }
 
@@ -387,12 +431,114 @@ bool Model::update_mem_batch_size(size_t const desired, bool const force) {
   return true;
 }
 
+// ---------------------------------------------------------------- weight initializers
+namespace {
+// Initialization__Gain__Scale (glorot.cpp:27-66)
+real gain_scale(ACTIVATION::TYPE const t) {
+  switch (t) {
+    case ACTIVATION::LEAKY_RELU: return std::sqrt(2.0f / (1.0f + std::pow(0.01f, 2.0f)));
+    case ACTIVATION::PARAMETRIC_RELU: return std::sqrt(2.0f / (1.0f + std::pow(0.25f, 2.0f)));
+    case ACTIVATION::RELU: return std::sqrt(2.0f);
+    case ACTIVATION::TANH: case ACTIVATION::TANH_STEPWISE: return 5.0f / 3.0f;
+    default: return 1.0f;
+  }
+}
+// Initialization__Uniform__Variance (glorot.cpp:91-111) on the activation classes
+// of Activation_Function__To__Class_Activation_Function (train.cpp:312-363):
+// rectifiers and SELU use the fan-in alone.
+real uniform_variance(size_t const n_inp, size_t const n_out, ACTIVATION::TYPE const t) {
+  switch (t) {
+    case ACTIVATION::LEAKY_RELU: case ACTIVATION::PARAMETRIC_RELU: case ACTIVATION::RELU: case ACTIVATION::SELU:
+      return std::sqrt(6.0f / static_cast<real>(n_inp));
+    default:
+      return std::sqrt(6.0f / static_cast<real>(n_inp + n_out));
+  }
+}
+// One draw of std::uniform_real_distribution<real>(lo, hi) over std::mt19937, the
+// reference's Dist::Real (ops/distributions/real.cpp): libstdc++ returns
+// u * (hi - lo) + lo with u = generate_canonical.  The reference's builds (GCC on
+// a target with FMA, which its -march=native release configuration gives on
+// any current host) contract that expression into one fused multiply-add, so it
+// is written as one here: bit-identical weights whatever this file is compiled for.
+real uniform_draw(std::mt19937 &gen, real const lo, real const hi) {
+  real const u = std::generate_canonical<real, std::numeric_limits<real>::digits>(gen);
+  return std::fma(u, hi - lo, lo);
+}
+}  // namespace
+
+// The tail both initializers share: scales 1, shifts 0, moving mean 0, moving
+// std 1 (Clear__Parameter__Normalized_Unit, model.cpp:3959-4025), gradient and
+// optimizer arrays cleared (clear_training_arrays), host mirrors uploaded.
+static void finish_initialization(Model &m) {
+  size_t const first_scale = m.total_weights + m.total_bias, nu = m.total_normalized_units;
+  for (size_t i = 0; i < nu; ++i) {
+    m.ptr_array_parameters[first_scale + i] = 1.0f;
+    m.ptr_array_parameters[first_scale + nu + i] = 0.0f;
+    m.ptr_array_normalized_batch_units_means_averages[i] = 0.0f;
+    m.ptr_array_normalized_batch_units_variances_averages[i] = 1.0f;
+  }
+  m.clear_training_arrays();
+  (void)m.upload_parameters();
+  (void)m.upload_moving_statistics();
+}
+
+void Model::initialize_weights_with_glorot_uniform(real const bias) {
+  if (ptr_array_layers == nullptr) { fail("initialize_weights_with_glorot_uniform: model not compiled"); return; }
+  for (size_t li = 1; li < total_layers; ++li) {
+    Layer const &l = ptr_array_layers[li];
+    if (l.type_layer != LAYER::FULLY_CONNECTED) continue;
+    size_t const n_inp = l.n_inp;
+    // fan-out as glorot.cpp:253-268 finds it through next_connected_layers: the
+    // next layer's width; for the last layer of a block the width of its RESIDUAL
+    // entry; for a layer followed by a block the mean of the RESIDUAL entry's
+    // width and the block's first layer's; for the output layer the fan-in.
+    size_t n_out = n_inp;
+    if (li + 1 != total_layers) {
+      Layer const &nx = ptr_array_layers[li + 1];
+      if (l.in_block && li == l.block_index + ptr_array_layers[l.block_index].block_depth)
+        n_out = ptr_array_layers[l.block_index].n_out;
+      else if (nx.type_layer == LAYER::RESIDUAL)
+        n_out = (nx.n_out + ptr_array_layers[li + 2].n_out) / 2;
+      else
+        n_out = nx.n_out;
+    }
+    // The gain is read from the layer's first activation unit (glorot.cpp:273).  A
+    // block's first layer has none, and the read lands on the first unit of the
+    // next layer that has some: that layer's activation sets the gain.
+    size_t ga = li;
+    while (ga + 1 < total_layers && (ptr_array_layers[ga].type_layer != LAYER::FULLY_CONNECTED || ptr_array_layers[ga].block_first)) ++ga;
+    real const v = gain_scale(ptr_array_layers[ga].type_activation_function) * uniform_variance(n_inp, n_out, l.type_activation_function);
+    var *w = ptr_array_parameters + l.first_connection_index;
+    for (size_t i = 0, n = l.n_out * n_inp; i < n; ++i) w[i] = uniform_draw(real_gen, -v, v);  // model.cpp:5087-5096
+    for (size_t i = 0; i < l.n_out; ++i) ptr_array_parameters[l.first_bias_connection_index + i] = bias;  // model.cpp:5031-5042
+  }
+  finish_initialization(*this);
+}
+
+void Model::Initialization__Uniform(real const bias, real const lower_bound, real const upper_bound) {
+  if (ptr_array_layers == nullptr) { fail("Initialization__Uniform: model not compiled"); return; }
+  if (!(lower_bound < upper_bound)) { fail("Initialization__Uniform: the lower bound is not below the upper bound"); return; }
+  for (size_t li = 1; li < total_layers; ++li) {
+    Layer const &l = ptr_array_layers[li];
+    if (l.type_layer != LAYER::FULLY_CONNECTED) continue;
+    var *w = ptr_array_parameters + l.first_connection_index;
+    for (size_t i = 0, n = l.n_out * l.n_inp; i < n; ++i) w[i] = uniform_draw(real_gen, lower_bound, upper_bound);
+    for (size_t i = 0; i < l.n_out; ++i) ptr_array_parameters[l.first_bias_connection_index + i] = bias;
+  }
+  finish_initialization(*this);
+}
+
 void Model::clear_training_arrays(void) {
   if (impl_->d_dparams == nullptr) return;
   (void)hipMemsetAsync(impl_->d_dparams, 0, total_parameters * sizeof(float), impl_->stream);
   (void)hipMemsetAsync(impl_->d_stats, 0, 2 * sizeof(double), impl_->stream);
   impl_->n_loss_examples = 0;
   std::memset(ptr_array_derivatives_parameters, 0, total_parameters * sizeof(real));
+  // Clear_Optimizer (train.cpp:136-248): the optimizer's own arrays and its clocks
+  for (int i = 0; i < 4; ++i)
+    if (impl_->d_opt[i] != nullptr) (void)hipMemsetAsync(impl_->d_opt[i], 0, total_parameters * sizeof(float), impl_->stream);
+  optimizer_time_step = 0.0f;
+  epoch_time_step = 1.0f;
 }
 
 // ---------------------------------------------------------------- buffer movement

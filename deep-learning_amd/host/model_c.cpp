@@ -77,6 +77,15 @@ void dlmi_model_layer_info(dlmi_model const *h, size_t layer, size_t *out) {
   out[11] = l.pooling_values[2];
 }
 
+void dlmi_model_glorot_uniform(dlmi_model *h, unsigned seed, float bias) {
+  h->m.real_gen.seed(seed);
+  h->m.initialize_weights_with_glorot_uniform(bias);
+}
+void dlmi_model_init_uniform(dlmi_model *h, unsigned seed, float bias, float lower, float upper) {
+  h->m.real_gen.seed(seed);
+  h->m.Initialization__Uniform(bias, lower, upper);
+}
+
 void dlmi_model_destroy(dlmi_model *h) { delete h; }
 char const *dlmi_model_last_error(dlmi_model const *h) { return h ? h->m.last_error() : "null model"; }
 

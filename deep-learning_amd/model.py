@@ -24,6 +24,7 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_model_get_optimizer_state", "dlmi_driver_create", "dlmi_driver_destroy", "dlmi_driver_train",
     "dlmi_driver_evalt", "dlmi_model_create_typed", "dlmi_model_layer_info", "dlmi_mnist_create",
     "dlmi_mnist_destroy", "dlmi_mnist_load", "dlmi_mnist_last_error", "dlmi_mnist_copy",
+    "dlmi_model_glorot_uniform", "dlmi_model_init_uniform",
 ]
 
 LAYER_FULLY_CONNECTED, LAYER_RESIDUAL = 3, 9  # v1/data/enum/layer.hpp
@@ -92,6 +93,7 @@ class Model:
         if mask is not None:
             m = np.ascontiguousarray(mask, dtype=np.uint8)
             self._ok(self.lib.dlmi_model_set_dropout_mask(self.h, c_sz(l), _ptr(m)), "dropout mask")
+        self._sizes()
 
     def set_norm_hyper(self, momentum, eps, r_max, d_max):
         self._ok(self.lib.dlmi_model_set_norm_hyper(self.h, c_f(momentum), c_f(eps), c_f(r_max), c_f(d_max)), "hyper")
@@ -107,6 +109,12 @@ class Model:
     def prepare(self, max_batch, nthreads=0):
         self.max_batch = max_batch
         self._ok(self.lib.dlmi_model_prepare(self.h, c_sz(max_batch)), "prepare")
+        self._sizes()
+
+    def _sizes(self):
+        """The scale / shift slots exist only once a layer is normalized: re-read the lengths."""
+        self.P = self.lib.dlmi_model_total_parameters(self.h)
+        self.n_units = self.lib.dlmi_model_total_normalized_units(self.h)
 
     def set_parameters(self, p):
         p = np.ascontiguousarray(p, np.float32)
@@ -130,6 +138,14 @@ class Model:
 
     def clear_training_arrays(self):
         self.lib.dlmi_model_clear_training_arrays(self.h)
+
+    def glorot_uniform(self, seed, bias=0.0):
+        """real_gen.seed(seed); initialize_weights_with_glorot_uniform(bias)"""
+        self.lib.dlmi_model_glorot_uniform(self.h, ctypes.c_uint(seed), c_f(bias))
+
+    def init_uniform(self, seed, bias=0.0, lower=-1.0, upper=1.0):
+        """real_gen.seed(seed); Initialization__Uniform(bias, lower, upper)"""
+        self.lib.dlmi_model_init_uniform(self.h, ctypes.c_uint(seed), c_f(bias), c_f(lower), c_f(upper))
 
     def step(self, state, X, Y=None, backward=True):
         X = np.ascontiguousarray(X, np.float32)
@@ -273,6 +289,7 @@ class Net(Model):
             m = np.ascontiguousarray(mask, dtype=np.uint8)
             assert m.size == self.info(l)["n_unit"], "one mask entry per dropout unit of the entry"
             self._ok(self.lib.dlmi_model_set_dropout_mask(self.h, c_sz(l), _ptr(m)), "dropout mask")
+        self._sizes()
 
     def layer_output(self, l):
         return self.layer_buffer(l, 3)

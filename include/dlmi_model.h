@@ -26,6 +26,10 @@ dlmi_model *dlmi_model_create_typed(size_t n_layers, int const *types, size_t co
  * index, Use__Bias(), normalization units, gamma index, moving-statistic index,
  * activation units, block depth, zero padding of the shortcut */
 void dlmi_model_layer_info(dlmi_model const *m, size_t layer, size_t *out);
+/* real_gen.seed(seed), then initialize_weights_with_glorot_uniform(bias) (glorot.cpp:225-359) or
+ * Initialization__Uniform(bias, lower, upper) (uniform.cpp:26-90) */
+void dlmi_model_glorot_uniform(dlmi_model *m, unsigned seed, float bias);
+void dlmi_model_init_uniform(dlmi_model *m, unsigned seed, float bias, float lower, float upper);
 void dlmi_model_destroy(dlmi_model *m);
 char const *dlmi_model_last_error(dlmi_model const *m);
 int dlmi_model_set_layer_activation_function(dlmi_model *m, size_t layer, int activation);

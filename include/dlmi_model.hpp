@@ -144,6 +144,17 @@ class Model {
   bool set_mp(bool const) { return true; }
   bool update_mem_thread_size(size_t const) { return true; }
   void merge_mp_derivatives(size_t const, size_t const) {}
+  // Weight initializers (v1/ops/initializers/glorot.cpp:225-359, uniform.cpp:26-90;
+  // model.cpp:5031-5096, 3959-4025).  Weights are drawn in parameter order from
+  // std::uniform_real_distribution<real> over `real_gen` (seed it for a
+  // reproducible start: the reference seeds from the clock), every bias slot is
+  // set to `bias`, scales / shifts / moving statistics go back to 1 / 0 / 0 / 1,
+  // the training arrays are cleared, and everything is uploaded.  Glorot bound of
+  // a layer: gain(activation) * sqrt(6 / fan_in) for rectifier and SELU layers,
+  // gain * sqrt(6 / (fan_in + fan_out)) otherwise, with the reference's fan_out
+  // (see the definition for the residual cases).
+  void initialize_weights_with_glorot_uniform(real const bias = 0.0f);
+  void Initialization__Uniform(real const bias = 0.0f, real const lower_bound = -1.0f, real const upper_bound = 1.0f);
   void clear_training_arrays(void);  // train.cpp:110-141: zeroes the gradient array
   void Dropout_Bernoulli(void);      // bernoulli_st.cpp:69-100: resample every per-unit mask
 
@@ -204,7 +215,7 @@ class Model {
 
   // ---- public state, as in the reference ------------------------------------
   size_t total_layers = 0, total_parameters = 0, total_weights = 0, total_bias = 0;
-  size_t total_normalized_units = 0;  // one slot per unit of EVERY layer, input included
+  size_t total_normalized_units = 0;  // 0 until a layer is normalized; then one slot per unit of EVERY entry, input included
   size_t batch_size = 1, maximum_batch_size = 1, seq_w = 1;
   size_t number_threads = 1;
   size_t n_acc_trial = 0, n_time_delay = 0;
@@ -212,7 +223,7 @@ class Model {
   double acc_train = 0.0, acc_valid = 0.0, acc_testg = 0.0;
   Layer *ptr_array_layers = nullptr;
   Layer *ptr_last_layer = nullptr;  // one past the output layer
-  var *ptr_array_parameters = nullptr;               // host mirror [P]: W.. | b.. | gamma.. | beta..
+  var *ptr_array_parameters = nullptr;               // host mirror [P]: W.. | b.. [| gamma.. | beta.. once a layer is normalized]
   real *ptr_array_derivatives_parameters = nullptr;  // host mirror [P]
   var *ptr_array_normalized_batch_units_means_averages = nullptr;      // host mirror [units]
   var *ptr_array_normalized_batch_units_variances_averages = nullptr;  // host mirror [units] (std-devs)
@@ -251,6 +262,7 @@ class Model {
   struct Impl;
   Impl *impl_;
   bool allocate_batch(size_t batch);
+  bool resize_normalization_slots(bool present);
   void forward_layers(size_t batch);
   bool forward_block_layer(size_t batch, size_t index_layer);
   bool backward_block(size_t batch, size_t index_residual);

@@ -555,6 +555,14 @@ class ReferenceMLP:
         self.lib.dlref_model_get_parameters(self.h, _ptr(p), c_sz(self.P))
         return p
 
+    def glorot_uniform(self, seed, bias=0.0):
+        """real_gen.seed(seed); initialize_weights_with_glorot_uniform(bias)"""
+        self.lib.dlref_model_glorot_uniform(self.h, ctypes.c_uint(seed), c_f(bias))
+
+    def init_uniform(self, seed, bias=0.0, lower=-1.0, upper=1.0):
+        """real_gen.seed(seed); Initialization__Uniform(bias, lower, upper)"""
+        self.lib.dlref_model_init_uniform(self.h, ctypes.c_uint(seed), c_f(bias), c_f(lower), c_f(upper))
+
     def set_moving(self, mean, std):
         mean = np.ascontiguousarray(mean, np.float32)
         std = np.ascontiguousarray(std, np.float32)

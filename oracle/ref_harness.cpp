@@ -445,6 +445,19 @@ void dlref_model_layer_info(void *h, size_t layer, size_t *out) {
   out[11] = l.pooling_values[2];
 }
 
+// Weight initializers with the model's generator seeded first (it is clock-seeded
+// otherwise, allocate.cpp:65-176): glorot.cpp:225-359 and uniform.cpp:26-90.
+void dlref_model_glorot_uniform(void *h, unsigned seed, float bias) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  m.real_gen.seed(seed);
+  m.initialize_weights_with_glorot_uniform(bias);
+}
+void dlref_model_init_uniform(void *h, unsigned seed, float bias, float lower, float upper) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  m.real_gen.seed(seed);
+  m.Initialization__Uniform(bias, lower, upper);
+}
+
 void dlref_model_destroy(void *h) { delete static_cast<RefModel *>(h); }
 
 int dlref_model_set_activation(void *h, size_t layer, int type) {

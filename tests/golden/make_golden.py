@@ -504,6 +504,52 @@ def resnets(R):
     return len(d)
 
 
+INIT_CASES = {
+    # name: (layer list, {entry: activation}, {entry: norm}, seed, bias, None for Glorot or (lower, upper))
+    "glorot_plain": ([("FC", 8), ("FC", 20), ("FC", 30), ("FC", 12), ("FC", 5)],
+                     {1: "RELU", 2: "ELU", 3: "LEAKY_RELU", 4: "SOFTMAX"}, {2: "BRN"}, 123, 0.0, None),
+    "glorot_selu_default": ([("FC", 7), ("FC", 16), ("FC", 9), ("FC", 11), ("FC", 3)],
+                            {1: "SELU", 3: "ISRLU", 4: "SOFTMAX"}, {}, 5489, 0.25, None),  # entry 2 keeps the sigmoid default
+    "glorot_two_blocks": ([("FC", 6), ("FC", 10), ("RES", 2), ("FC", 14), ("FC", 18), ("RES", 3), ("FC", 22), ("FC", 26),
+                           ("FC", 30), ("FC", 34), ("FC", 4)],
+                          {1: "ELU", 3: "ELU", 4: "ELU", 6: "ELU", 7: "ELU", 8: "ELU", 9: "ELU", 10: "SOFTMAX"},
+                          {1: "BN", 2: "BN", 4: "BN"}, 77, 0.5, None),
+    "glorot_block_gains": ([("FC", 6), ("FC", 10), ("RES", 1), ("FC", 14), ("FC", 9), ("RES", 2), ("FC", 5), ("FC", 12),
+                            ("FC", 4)],
+                           {1: "LINEAR", 3: "RELU", 4: "SELU", 6: "SELU", 7: "RELU", 8: "SOFTMAX"}, {3: "BRN"}, 1, 0.0, None),
+    "uniform_plain": ([("FC", 8), ("FC", 20), ("FC", 5)], {1: "RELU", 2: "SOFTMAX"}, {1: "BN"}, 9, 0.1, (-0.3, 0.7)),
+    "uniform_block": ([("FC", 6), ("FC", 10), ("RES", 2), ("FC", 14), ("FC", 8), ("FC", 4)],
+                      {1: "ELU", 3: "ELU", 4: "RELU", 5: "SOFTMAX"}, {2: "BRN", 3: "BRN"}, 31337, -0.2, (-1.0, 1.0)),
+}
+
+
+def inits(R):
+    """Uniform weight initializers (glorot.cpp:225-359, uniform.cpp:26-90) with the
+    model's generator seeded: the parameter vector and the moving statistics after
+    the call, from a model whose parameters and statistics held other values."""
+    d = {"init_cases_json": np.frombuffer(json.dumps({k: [v[0], {str(a): b for a, b in v[1].items()},
+                                                         {str(a): b for a, b in v[2].items()}, v[3], v[4], v[5]]
+                                                     for k, v in INIT_CASES.items()}).encode(), dtype=np.uint8)}
+    for name, (layers, acts, norms, seed, bias, rng_bounds) in INIT_CASES.items():
+        M = ReferenceNet(R, layers)
+        for l in sorted(set(acts) | set(norms)):
+            M.set_layer(l, ACT[acts[l]] if l in acts else 0, NORM[norms.get(l, "NONE")])
+        M.prepare(4)
+        rng = np.random.default_rng(seed)
+        M.set_parameters(f32(rng.uniform(-2, 2, M.P)))
+        M.set_moving(f32(rng.uniform(-2, 2, M.n_units)), f32(rng.uniform(1, 3, M.n_units)))
+        if rng_bounds is None:
+            M.glorot_uniform(seed, bias)
+        else:
+            M.init_uniform(seed, bias, *rng_bounds)
+        d[name + "_info"] = np.array([list(M.info(l).values()) for l in range(len(layers))])
+        d[name + "_P"] = np.array([M.P, M.n_units])
+        d[name + "_params"] = M.get_parameters()
+        d[name + "_mov_mean"], d[name + "_mov_std"] = M.get_moving()
+    save("init.npz", d)
+    return len(d)
+
+
 if __name__ == "__main__":
     R = Reference()
     print("leaves:", leaves(R), "arrays")
@@ -513,3 +559,4 @@ if __name__ == "__main__":
     print("variants:", variants(R), "arrays")
     print("shortcut:", shortcuts(R), "arrays")
     print("resnet:", resnets(R), "arrays")
+    print("init:", inits(R), "arrays")
