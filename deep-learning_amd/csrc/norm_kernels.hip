@@ -70,7 +70,7 @@ static int env_int(char const *name, int dflt) {
 // Geometry of a reduction pass.
 static ColGeom reduce_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, int nacc) {
   static int const tx_caps[2] = {env_int("DLMI_NORM_STATS_TX", 64), env_int("DLMI_NORM_BWD_TX", 256)};
-  static int const rpts[2] = {env_int("DLMI_NORM_STATS_ROWS_PER_THREAD", 16), env_int("DLMI_NORM_BWD_ROWS_PER_THREAD", 16)};
+  static int const rpts[2] = {env_int("DLMI_NORM_STATS_ROWS_PER_THREAD", 16), env_int("DLMI_NORM_BWD_ROWS_PER_THREAD", 8)};
   static int const bpcs[2] = {env_int("DLMI_NORM_STATS_BLOCKS_PER_CU", 8), env_int("DLMI_NORM_BWD_BLOCKS_PER_CU", 1)};
   int const which = nacc == 2 ? 0 : 1;
   int const tx_cap = tx_caps[which], rows_per_thread = rpts[which], blocks_per_cu = bpcs[which];
@@ -86,8 +86,10 @@ static ColGeom reduce_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec
   int const ty = kBlock / tx;
   g.grid_x = static_cast<unsigned>(dlmi_ceil_div(groups, tx));
   // enough blocks to cover every CU several times over, but each thread still
-  // streams >= 16 rows: the partial sums stay a small fraction of the traffic
-  // and the fixed cost of a block is amortised
+  // streams rows_per_thread rows (16 in the statistics pass, 8 in the backward
+  // reduction, where a batch of 1024 rows otherwise leaves half the CUs idle):
+  // the partial sums stay a small fraction of the traffic and the fixed cost of
+  // a block is amortised
   size_t want = dlmi_ceil_div(static_cast<size_t>(ctx->num_cu) * blocks_per_cu, g.grid_x);
   size_t const max_by_rows = B / (static_cast<size_t>(ty) * rows_per_thread);
   if (want > max_by_rows) want = max_by_rows;

@@ -299,6 +299,8 @@ bool Model::Set__Layer_Normalization(size_t const i, LAYER_NORM::TYPE const t, b
     ptr_array_layers[i].type_normalization = before;
     return false;
   }
+  // which per-batch buffers a layer keeps depends on its normalization
+  if (before != t && impl_->allocated_batch != 0) return allocate_batch(impl_->allocated_batch);
   return true;
 }
 
@@ -678,7 +680,9 @@ void Model::forward_layers(size_t const B) {
       // activation values; dropout then acts on the normalized values
       // (fwp_st.cpp:657-732), which are the layer's output
       if (softmax) { fail("forward_pass: softmax layers are not normalized"); return; }
-      if (l.d_af_values == nullptr) { fail("forward_pass: call update_mem_batch_size() after changing the normalization order"); return; }
+      // the order is a public member assigned directly (user_controls.cpp:1974): the extra buffer
+      // comes with the first pass that needs it
+      if (l.d_af_values == nullptr && !dev_alloc(&l.d_af_values, impl_->allocated_batch * H, impl_->err)) return;
       dlmi_fused_desc d = make_desc(*this, l);
       d.act = DLMI_ACT_LINEAR;
       float const *gamma = impl_->d_params + l.scale_index, *beta = impl_->d_params + l.shift_index;
