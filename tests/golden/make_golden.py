@@ -454,6 +454,9 @@ RESNET_CASES = {
 }
 
 
+RESNET_EPOCH_CASE = "res_dropout_wide_block"
+
+
 def resnets(R):
     """Layer lists with the reference's residual blocks (fwp_st.cpp:3876-4442,
     bwp_st.cpp:80-185, 345-541): outputs of every entry in the three propagation
@@ -500,6 +503,38 @@ def resnets(R):
                         d[f"{q}L{l}_dZ"] = M.layer_error(l)
                     d[q + "dparams"] = M.get_dparams()
                     d[q + "mov_mean"], d[q + "mov_std"] = M.get_moving()
+    # The whole caller-side chain on the network with dropout inside its blocks: Glorot
+    # initialization from a seeded generator, two Driver::train epochs over 30 rows in
+    # sub-batches of 11 (one Nesterov-momentum step each), then Driver::evalt.
+    name = RESNET_EPOCH_CASE
+    layers, B, cfg, hyper = RESNET_CASES[name]
+    rng = np.random.default_rng(99)
+    X = f32(rng.uniform(0, 1, (30, layers[0][1])))
+    Y = f32(np.eye(layers[-1][1])[rng.integers(0, layers[-1][1], 30)])
+    d["epoch_X"], d["epoch_Y"] = X, Y
+    for nt in THREADS:
+        M = ReferenceNet(R, layers)
+        for l, (a, nm, dr, keep) in cfg.items():
+            M.set_layer(l, ACT[a] if a else 0, NORM[nm], DROP[dr], keep)
+        M.set_layer(len(layers) - 1, ACT["SOFTMAX"])
+        M.set_norm_hyper(*hyper)
+        for l in cfg:
+            if f"{name}_mask{l}" in d:
+                M._masks[l] = d[f"{name}_mask{l}"]
+        M.prepare(B, nt)
+        M.glorot_uniform(2024, 0.0)
+        d[f"epoch_t{nt}_init"] = M.get_parameters()
+        # momentum rather than Adam: the bias of an un-normalized layer that feeds a batch
+        # normalization has an analytically zero gradient, and Adam turns the rounding noise
+        # computed in its place into full-size steps of random sign
+        M.set_optimizer(OPT["GD"], lr=0.01, momentum=0.9, nesterov=True, weight_decay=0.01)
+        la = []
+        for e in range(2):
+            la.append(M.train_epoch(X, Y, resample_masks=False))
+            d[f"epoch_t{nt}_e{e}_params"] = M.get_parameters()
+        la.append(M.evalt(X, Y))
+        d[f"epoch_t{nt}_loss_accu"] = np.array(la, dtype=np.float64)
+        d[f"epoch_t{nt}_mov_mean"], d[f"epoch_t{nt}_mov_std"] = M.get_moving()
     save("resnet.npz", d)
     return len(d)
 

@@ -35,6 +35,34 @@ def test_gpu_resnet_against_golden(net_factory, name):
     check_resnet(M, g, name, 0, TR)
 
 
+def test_gpu_resnet_initialize_train_evaluate_against_golden(net_factory):
+    """The caller-side chain in one piece, on the network with dropout inside its
+    blocks: Glorot initialization from a seeded generator (bit-identical), two
+    Driver::train epochs of 30 rows in sub-batches of 11 with one Nesterov-momentum
+    step each, then Driver::evalt — parameters after every epoch, losses,
+    accuracies and moving statistics as the compiled reference has them."""
+    from oracle.binding import OPT
+    g = load_resnet_golden()
+    name = "res_dropout_wide_block"
+    M = build_resnet(net_factory, g, name, 0)
+    M.glorot_uniform(2024, 0.0)
+    assert np.array_equal(M.get_parameters(), g["epoch_t0_init"])
+    M.set_optimizer(OPT["GD"], lr=0.01, momentum=0.9, nesterov=True, weight_decay=0.01)
+    X, Y = g["epoch_X"], g["epoch_Y"]
+    from helpers import assert_close
+    exp = g["epoch_t0_loss_accu"]
+    for e in range(2):
+        loss, accu = M.train_epoch(X, Y, resample_masks=False)
+        assert abs(loss - exp[e, 0]) <= TR * max(1.0, abs(exp[e, 0])), (e, loss, exp[e, 0])
+        assert accu == pytest.approx(exp[e, 1], abs=1e-9), (e, accu, exp[e, 1])
+        assert_close(M.get_parameters(), g[f"epoch_t0_e{e}_params"], TR, f"parameters after epoch {e}")
+    loss, accu = M.evalt(X, Y)
+    assert abs(loss - exp[2, 0]) <= TR * max(1.0, abs(exp[2, 0])) and accu == pytest.approx(exp[2, 1], abs=1e-9)
+    mm, ms = M.get_moving()
+    assert_close(mm, g["epoch_t0_mov_mean"], TR, "moving mean", floor=1.0)
+    assert_close(ms, g["epoch_t0_mov_std"], TR, "moving std")
+
+
 def test_gpu_resnet_wide_against_oracle(net_factory, oracle):
     """Widths and a batch at which the GEMM tiles, the split reductions and the
     16-byte paths are all in play: two blocks (one widening, one narrowing the
