@@ -26,7 +26,9 @@ c_sz = ctypes.c_size_t
 vp = ctypes.c_void_p
 
 
-@pytest.mark.parametrize("B,H", [(2, 1), (2, 7), (3, 1), (5000, 1), (40000, 3), (2, 4100)])
+@pytest.mark.parametrize("B,H", [(2, 1), (2, 7), (3, 1), (5000, 1), (40000, 3), (2, 4100),
+                                 # a million units (odd: the scalar path; partial sums beyond the first scratch block)
+                                 (16, 1_000_003), (24, 600_000)])
 @pytest.mark.parametrize("renorm", [True, False])
 def test_fused_degenerate_shapes(dl, oracle, pkg, B, H, renorm):
     rng = np.random.default_rng(B * 13 + H)
@@ -56,6 +58,37 @@ def test_fused_degenerate_shapes(dl, oracle, pkg, B, H, renorm):
     assert_close(host(db), bw["dbeta"], TR, "dbeta", floor=1.0)
     yi = dl.fused_infer(desc, dev(x), dev(gamma), dev(beta), dev(mm), dev(ms))
     assert_close(host(yi), oracle.act_fwd(ACT["ELU"], oracle.norm_fwd_infer(x, gamma, beta, mm, ms)), TR, "inference")
+
+
+def test_three_million_rows_against_float64(dl, oracle, oracle64, pkg):
+    """[3 000 000 x 8]: the batch is cut into the largest number of chunks the grid takes.  At this
+    length the reference's single fp32 accumulator per thread is itself off by more than the
+    tolerance (about 7e-4 on the outputs), so float64 arbitrates: the GPU's chunked sums must
+    meet the tolerance against it, and be nearer to it than the fp32 restatement is."""
+    from helpers import max_rel_err
+    B, H = 3_000_000, 8
+    rng = np.random.default_rng(3)
+    x = (rng.standard_normal((B, H)) * rng.uniform(.5, 2, H) + rng.uniform(-1, 1, H)).astype(np.float32)
+    gamma, beta = rng.uniform(.8, 1.2, H).astype(np.float32), rng.uniform(-.1, .1, H).astype(np.float32)
+    dY = rng.standard_normal((B, H)).astype(np.float32)
+    zero, one = np.zeros(H, np.float32), np.ones(H, np.float32)
+    hyper = (0.9, 1e-5, 3.0, 5.0)
+    a = ACT["LEAKY_RELU"]
+    args = (a, x, gamma, beta, zero, one, hyper, True, DROP["NONE"], None, 1.0, False, dY, zero, zero)
+    fw32, y32, bw32 = oracle_fused(oracle, *args, nt=oracle.max_threads())
+    fw64, y64, bw64 = oracle_fused(oracle64, *args, nt=oracle.max_threads())
+    desc = pkg.Dlmi.desc(a, momentum=hyper[0], eps=hyper[1], r_max=hyper[2], d_max=hyper[3])
+    dmm, dms = dev(zero), dev(one)
+    yg, st = dl.fused_fwd(desc, dev(x), dev(gamma), dev(beta), dmm, dms)
+    dg, db = dev(zero), dev(zero)
+    dX = dl.fused_bwd(desc, dev(x), dev(gamma), dev(beta), st, dev(dY), dg, db)
+    assert_close(host(st["mean"]), fw64["mean"], TR, "mean vs float64", floor=1.0)
+    assert_close(host(st["std"]), fw64["std"], TR, "std vs float64")
+    assert_close(host(yg), y64, TR, "y vs float64")
+    assert_close(host(dX), bw64["dx"], TR, "dX vs float64", floor=1e-3)
+    assert_close(host(dg), bw64["dgamma"], TR, "dgamma vs float64", floor=1.0)
+    assert_close(host(db), bw64["dbeta"], TR, "dbeta vs float64", floor=1.0)
+    assert max_rel_err(host(yg), y64, 0.0) <= max_rel_err(y32, y64, 0.0)
 
 
 @pytest.mark.parametrize("B,K,H", [(1, 4096, 1), (1, 1, 300), (4097, 1, 1), (2, 3, 4099), (3, 5000, 2)])
