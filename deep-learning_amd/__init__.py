@@ -40,6 +40,7 @@ C_ABI_SYMBOLS = [
     "dlmi_softmax_fwd", "dlmi_dropout_fwd", "dlmi_identity_add", "dlmi_softmax_ce_seed",
     "dlmi_fused_norm_act_fwd", "dlmi_fused_norm_act_bwd", "dlmi_fused_norm_act_infer", "dlmi_fc_norm_act_fwd",
     "dlmi_opt_gd", "dlmi_opt_gd_momentum", "dlmi_opt_adam", "dlmi_zero_padded_identity_fwd", "dlmi_residual_bwd",
+    "dlmi_opt_adabound",
 ]
 
 
@@ -262,6 +263,12 @@ class Dlmi:
         self._chk(p, g, m1, m2, vhat, mask)
         self._ck(self.lib.dlmi_opt_adam(self.ctx, c_sz(p.numel()), _p(p), _p(g), _p(m1), _p(m2), _p(vhat), _p(mask),
                                         c_f(lr_t), c_f(beta1), c_f(beta2), c_f(eps), c_f(wd)))
+
+    def opt_adabound(self, p, g, m1, m2, vhat, mask, lr_t, beta1, beta2, eps, wd, rate_lower, rate_upper, nthreads=0):
+        self._chk(p, g, m1, m2, vhat, mask)
+        self._ck(self.lib.dlmi_opt_adabound(self.ctx, c_sz(p.numel()), _p(p), _p(g), _p(m1), _p(m2), _p(vhat), _p(mask),
+                                            c_f(lr_t), c_f(beta1), c_f(beta2), c_f(eps), c_f(wd), c_f(rate_lower),
+                                            c_f(rate_upper)))
 
     def softmax_ce_seed(self, q, y, stats=None):
         """stats: optional device tensor of 2 float64 accumulators."""

@@ -1,5 +1,5 @@
 // Optimizer steps over the packed parameter array for gfx950: plain gradient
-// descent, momentum, the reference's Nesterov variant, Adam and AMSGrad, each
+// descent, momentum, the reference's Nesterov variant, Adam, AMSGrad, AdaBound and AMSBound, each
 // with the optional masked weight decay, each zeroing the gradient it consumed.
 //
 // One pass, one thread per 4 parameters (float4), every array read once and
@@ -15,7 +15,8 @@
 namespace dlmi {
 
 constexpr int kOptBlock = 256;
-constexpr int kOptGd = 0, kOptMomentum = 1, kOptNesterov = 2, kOptAdam = 3, kOptAmsgrad = 4;
+constexpr int kOptGd = 0, kOptMomentum = 1, kOptNesterov = 2, kOptAdam = 3, kOptAmsgrad = 4, kOptAdabound = 5,
+              kOptAmsbound = 6;
 
 struct OptArgs {
   float *p, *g;
@@ -26,10 +27,12 @@ struct OptArgs {
   size_t n;
   float lr;           // GD family: learning rate; Adam family: bias-corrected step size
   float mom, beta1, beta2, eps, wd;
+  float rate_lo, rate_hi;  // AdaBound / AMSBound: the band the per-parameter step size is clipped into
 };
 
 // One parameter.  gradient_descent.cpp:79-92, gradient_descent_momentum.cpp:44-63,
-// nesterov_accelerated_gradient.cpp:44-63, adam.cpp:65-97, amsgrad.cpp:75-117.
+// nesterov_accelerated_gradient.cpp:44-63, adam.cpp:65-97, amsgrad.cpp:75-117, adabound.cpp:72-112,
+// amsbound.cpp:80-124.
 template <int KIND, bool WD>
 __device__ __forceinline__ void opt_one(OptArgs const &a, float &p, float g, float &s0, float &s1, float &s2,
                                         float mask) {
@@ -46,11 +49,19 @@ __device__ __forceinline__ void opt_one(OptArgs const &a, float &p, float g, flo
     s0 = a.beta1 * s0 + (1.0f - a.beta1) * g;
     s1 = a.beta2 * s1 + (1.0f - a.beta2) * g * g;
     float v = s1;
-    if constexpr (KIND == kOptAmsgrad) {
+    if constexpr (KIND == kOptAmsgrad || KIND == kOptAmsbound) {
       v = s2 > v ? s2 : v;
       s2 = v;
     }
-    step = a.lr * s0 / (sqrtf(v) + a.eps);
+    if constexpr (KIND == kOptAdabound || KIND == kOptAmsbound) {
+      // the per-parameter step size, clipped into the band that closes on the final
+      // learning rate (adabound.cpp:83-87, amsbound.cpp:94-99)
+      float rate = a.lr / (sqrtf(v) + a.eps);
+      rate = rate < a.rate_lo ? a.rate_lo : (rate > a.rate_hi ? a.rate_hi : rate);
+      step = rate * s0;
+    } else {
+      step = a.lr * s0 / (sqrtf(v) + a.eps);
+    }
   }
   if constexpr (WD) step += mask * a.wd * p;
   p -= step;
@@ -58,7 +69,7 @@ __device__ __forceinline__ void opt_one(OptArgs const &a, float &p, float g, flo
 
 template <int KIND, bool WD>
 __global__ __launch_bounds__(kOptBlock) void k_opt(OptArgs a, size_t n4) {
-  constexpr bool kS0 = KIND != kOptGd, kS1 = KIND >= kOptAdam, kS2 = KIND == kOptAmsgrad;
+  constexpr bool kS0 = KIND != kOptGd, kS1 = KIND >= kOptAdam, kS2 = KIND == kOptAmsgrad || KIND == kOptAmsbound;
   size_t const stride = static_cast<size_t>(gridDim.x) * kOptBlock;
   size_t i = static_cast<size_t>(blockIdx.x) * kOptBlock + threadIdx.x;
   for (; i < n4; i += stride) {
@@ -152,6 +163,20 @@ int dlmi_opt_adam(dlmi_ctx *ctx, size_t n, float *params, float *grads, float *m
   a.lr = lr_t; a.beta1 = beta1; a.beta2 = beta2; a.eps = eps; a.wd = wd;
   return m2_hat != nullptr ? launch_opt<kOptAmsgrad>(ctx, a, "k_opt<amsgrad>")
                            : launch_opt<kOptAdam>(ctx, a, "k_opt<adam>");
+}
+
+int dlmi_opt_adabound(dlmi_ctx *ctx, size_t n, float *params, float *grads, float *m1, float *m2, float *m2_hat,
+                      float const *mask, float lr_t, float beta1, float beta2, float eps, float wd, float rate_lower,
+                      float rate_upper) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, n == 0 || (params && grads && m1 && m2), "null pointer");
+  DLMI_REQUIRE(ctx, wd == 0.0f || mask != nullptr, "weight decay needs the regularization mask");
+  DLMI_REQUIRE(ctx, rate_lower <= rate_upper, "the lower bound of the step size exceeds the upper one");
+  OptArgs a{};
+  a.p = params; a.g = grads; a.s0 = m1; a.s1 = m2; a.s2 = m2_hat; a.mask = mask; a.n = n;
+  a.lr = lr_t; a.beta1 = beta1; a.beta2 = beta2; a.eps = eps; a.wd = wd; a.rate_lo = rate_lower; a.rate_hi = rate_upper;
+  return m2_hat != nullptr ? launch_opt<kOptAmsbound>(ctx, a, "k_opt<amsbound>")
+                           : launch_opt<kOptAdabound>(ctx, a, "k_opt<adabound>");
 }
 
 }  // extern "C"

@@ -541,6 +541,7 @@ void Model::clear_training_arrays(void) {
     if (impl_->d_opt[i] != nullptr) (void)hipMemsetAsync(impl_->d_opt[i], 0, total_parameters * sizeof(float), impl_->stream);
   optimizer_time_step = 0.0f;
   epoch_time_step = 1.0f;
+  adam_previous_beta2 = 0.0f;
 }
 
 // ---------------------------------------------------------------- buffer movement
@@ -1069,8 +1070,9 @@ bool opt_array(float **p, size_t n, hipStream_t stream, std::string &err) {
 void Model::set_optimizer(OPTIMIZER::TYPE const type_received) {
   if (type_optimizer_function == type_received) return;
   switch (type_received) {
-    case OPTIMIZER::NONE: case OPTIMIZER::GD: case OPTIMIZER::ADAM: case OPTIMIZER::AMSGRAD: break;
-    default: fail("set_optimizer: only GD, ADAM and AMSGRAD run on the device"); return;
+    case OPTIMIZER::NONE: case OPTIMIZER::GD: case OPTIMIZER::ADAM: case OPTIMIZER::AMSGRAD: case OPTIMIZER::ADABOUND:
+    case OPTIMIZER::AMSBOUND: case OPTIMIZER::NOSADAM: break;
+    default: fail("set_optimizer: only GD, ADAM, AMSGRAD, ADABOUND, AMSBOUND and NOSADAM run on the device"); return;
   }
   if (impl_->ctx != nullptr) (void)dlmi_ctx_synchronize(impl_->ctx);
   for (int i = 0; i < 4; ++i) dev_free(impl_->d_opt[i]);
@@ -1136,6 +1138,42 @@ void Model::Update_Parameter(size_t const batch, size_t const training_size) {
                             : lr;
       rc = dlmi_opt_adam(m.ctx, P, m.d_params, m.d_dparams, m.d_opt[1], m.d_opt[2], ams ? m.d_opt[3] : nullptr,
                          m.d_opt[4], lr_t, adam_beta1, adam_beta2, adam_epsilon, wd);
+      break;
+    }
+    case OPTIMIZER::ADABOUND:
+    case OPTIMIZER::AMSBOUND: {
+      // adabound.cpp:37-112, amsbound.cpp:38-124: Adam whose per-parameter step size is clipped into a
+      // band around learning_rate_final that narrows with the time step
+      optimizer_time_step += 1.0f;
+      bool const ams = type_optimizer_function == OPTIMIZER::AMSBOUND;
+      if (!opt_array(&m.d_opt[1], P, m.stream, m.err) || !opt_array(&m.d_opt[2], P, m.stream, m.err)) return;
+      if (ams && !opt_array(&m.d_opt[3], P, m.stream, m.err)) return;
+      real const lr = adam_learning_rate;
+      real const lower = learning_rate_final * (1.0f - 1.0f / (learning_gamma * optimizer_time_step + 1.0f));
+      real const upper = learning_rate_final * (1.0f + 1.0f / (learning_gamma * optimizer_time_step));
+      real const lr_t = use_adam_bias_correction
+                            ? lr * std::sqrt(1.0f - std::pow(adam_beta2, optimizer_time_step)) /
+                                  (1.0f - std::pow(adam_beta1, optimizer_time_step))
+                            : lr;
+      rc = dlmi_opt_adabound(m.ctx, P, m.d_params, m.d_dparams, m.d_opt[1], m.d_opt[2], ams ? m.d_opt[3] : nullptr,
+                             m.d_opt[4], lr_t, adam_beta1, adam_beta2, adam_epsilon, wd, lower, upper);
+      break;
+    }
+    case OPTIMIZER::NOSADAM: {
+      // nosadam.cpp:37-100: Adam whose second-moment decay at step t is B_{t-1} / B_t with
+      // B_t = sum_{k<=t} k^-adam_gamma; the bias correction keeps the fixed adam_beta2
+      optimizer_time_step += 1.0f;
+      if (!opt_array(&m.d_opt[1], P, m.stream, m.err) || !opt_array(&m.d_opt[2], P, m.stream, m.err)) return;
+      real const lr = adam_learning_rate;
+      real const beta2_at_power_gamma = std::pow(optimizer_time_step, -adam_gamma);
+      real const beta2_at_time_t = adam_previous_beta2 / (adam_previous_beta2 + beta2_at_power_gamma);
+      real const lr_t = use_adam_bias_correction
+                            ? lr * std::sqrt(1.0f - std::pow(adam_beta2, optimizer_time_step)) /
+                                  (1.0f - std::pow(adam_beta1, optimizer_time_step))
+                            : lr;
+      adam_previous_beta2 += beta2_at_power_gamma;
+      rc = dlmi_opt_adam(m.ctx, P, m.d_params, m.d_dparams, m.d_opt[1], m.d_opt[2], nullptr, m.d_opt[4], lr_t, adam_beta1,
+                         beta2_at_time_t, adam_epsilon, wd);
       break;
     }
     default:

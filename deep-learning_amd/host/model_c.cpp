@@ -216,6 +216,11 @@ int dlmi_model_set_optimizer(dlmi_model *h, int type, float lr, float momentum, 
   if (m.type_optimizer_function != static_cast<OPTIMIZER::TYPE>(type)) return 0;
   return m.set_weight_decay(weight_decay) ? 1 : 0;
 }
+void dlmi_model_set_bound_hyper(dlmi_model *h, float lr_final, float gamma, float adam_gamma) {
+  h->m.learning_rate_final = lr_final;
+  h->m.learning_gamma = gamma;
+  h->m.adam_gamma = adam_gamma;
+}
 void dlmi_model_set_epoch_time_step(dlmi_model *h, float v) { h->m.epoch_time_step = v; }
 int dlmi_model_set_derivatives(dlmi_model *h, float const *g, size_t n) {
   if (n != h->m.total_parameters) return 0;

@@ -276,6 +276,16 @@ int dlmi_opt_adam(dlmi_ctx *ctx, size_t n, float *params, float *grads, float *m
                   float *m2_hat, float const *mask, float lr_t, float beta1, float beta2, float eps,
                   float wd);
 
+/* AdaBound: the moments of dlmi_opt_adam, then
+ * p -= clip(lr_t/(sqrt(m2)+eps), rate_lower, rate_upper)*m1 + mask*wd*p, the band
+ * [rate_lower, rate_upper] being what the caller computes per step from
+ * learning_rate_final and learning_gamma (adabound.cpp:37-190).  m2_hat != NULL
+ * selects AMSBound (amsbound.cpp:38-214).  NosAdam (nosadam.cpp:37-170) is
+ * dlmi_opt_adam with the step's own beta2. */
+int dlmi_opt_adabound(dlmi_ctx *ctx, size_t n, float *params, float *grads, float *m1, float *m2,
+                      float *m2_hat, float const *mask, float lr_t, float beta1, float beta2,
+                      float eps, float wd, float rate_lower, float rate_upper);
+
 #ifdef __cplusplus
 }
 #endif

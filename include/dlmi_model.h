@@ -65,6 +65,9 @@ double dlmi_model_accuracy_sum(dlmi_model const *m);
 int dlmi_model_set_optimizer(dlmi_model *m, int type, float lr, float momentum, int nesterov, float adam_lr,
                              float beta1, float beta2, float eps, int bias_correction, float weight_decay,
                              int normalized_wd);
+/* learning_rate_final, learning_gamma (AdaBound / AMSBound) and adam_gamma (NosAdam): call before
+ * dlmi_model_set_optimizer */
+void dlmi_model_set_bound_hyper(dlmi_model *m, float lr_final, float gamma, float adam_gamma);
 void dlmi_model_set_epoch_time_step(dlmi_model *m, float v);
 int dlmi_model_set_derivatives(dlmi_model *m, float const *g, size_t n);      /* host array -> device gradient array */
 void dlmi_model_update_parameter(dlmi_model *m, size_t batch, size_t training_size);  /* Update_Parameter */

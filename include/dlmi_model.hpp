@@ -186,8 +186,9 @@ class Model {
 
   // ---- optimizer step (model.hpp:848, 2965; train.cpp:77-104, 278-283;
   //      ops/regularizers/weight_decay.cpp:26-62; model.cpp:4703-4866) ----------
-  // GD (plain, momentum, Nesterov), ADAM and AMSGRAD run on the device; the
-  // others are refused.  set_optimizer also clears the training arrays, like the
+  // GD (plain, momentum, Nesterov), ADAM, AMSGRAD, ADABOUND, AMSBOUND and NOSADAM
+  // (adabound.cpp, amsbound.cpp, nosadam.cpp) run on the device; the others are
+  // refused.  set_optimizer also clears the training arrays, like the
   // reference.  Update_Parameter consumes and zeroes the device gradient array.
   void set_optimizer(OPTIMIZER::TYPE const type);
   bool set_weight_decay(real const val);
@@ -244,6 +245,10 @@ class Model {
   real adam_beta1 = 0.9f;
   real adam_beta2 = 0.999f;
   real adam_epsilon = 1e-8f;
+  real learning_rate_final = 0.1f;  // AdaBound / AMSBound: the rate the band closes on (model.hpp:3021)
+  real learning_gamma = 1e-3f;      // AdaBound / AMSBound: how fast it closes (model.hpp:3023)
+  real adam_previous_beta2 = 0.0f;  // NosAdam: B_{t-1} (model.hpp:3032)
+  real adam_gamma = 0.1f;           // NosAdam: exponent of the hyper-harmonic weights (model.hpp:3034)
   real optimizer_time_step = 0.0f;
   real epoch_time_step = 1.0f;
   MODEL::TYPE type = MODEL::NONE;

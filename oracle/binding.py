@@ -34,7 +34,8 @@ NORM = dict(NONE=0, BN=1, BRN=2)
 DROP = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3)
 STATE = dict(INFERENCE=0, TRAINING=1, UPDATE_BATCH_NORM=2)
 # v1/data/enum/optimizer.hpp:24-42
-OPT = dict(NONE=0, ADAM=2, AMSGRAD=5, GD=6)
+OPT = dict(NONE=0, ADABOUND=1, ADAM=2, AMSBOUND=4, AMSGRAD=5, GD=6, NOSADAM=9)
+_ADAM_FAMILY = (1, 2, 4, 5, 9)
 
 
 def build_oracle():
@@ -53,19 +54,22 @@ class OptimizerHost:
     opt_gd_momentum / opt_adam updating float32 arrays in place."""
 
     def __init__(self, leaves, n, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9,
-                 beta2=0.999, eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True, mask=None):
+                 beta2=0.999, eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True, mask=None,
+                 lr_final=0.1, gamma=1e-3, adam_gamma=0.1):
         f = np.float32
         self.leaves, self.n, self.kind = leaves, n, kind
         self.lr, self.momentum, self.nesterov = f(lr), f(momentum), bool(nesterov)
         self.adam_lr, self.beta1, self.beta2, self.eps = f(adam_lr), f(beta1), f(beta2), f(eps)
         self.bias_correction, self.weight_decay, self.normalized_wd = bool(bias_correction), f(weight_decay), bool(normalized_wd)
+        # AdaBound / AMSBound: learning_rate_final, learning_gamma; NosAdam: adam_gamma (model.hpp:3021-3034)
+        self.lr_final, self.gamma, self.adam_gamma, self.previous_beta2 = f(lr_final), f(gamma), f(adam_gamma), f(0)
         self.mask = None if mask is None else np.ascontiguousarray(mask, np.float32)
         self.t = f(0)
         self.epoch_time_step = f(1)
         self.delta = np.zeros(n, np.float32) if kind == OPT["GD"] and self.momentum != 0 else None
-        self.m1 = np.zeros(n, np.float32) if kind in (OPT["ADAM"], OPT["AMSGRAD"]) else None
-        self.m2 = np.zeros(n, np.float32) if kind in (OPT["ADAM"], OPT["AMSGRAD"]) else None
-        self.vhat = np.zeros(n, np.float32) if kind == OPT["AMSGRAD"] else None
+        self.m1 = np.zeros(n, np.float32) if kind in _ADAM_FAMILY else None
+        self.m2 = np.zeros(n, np.float32) if kind in _ADAM_FAMILY else None
+        self.vhat = np.zeros(n, np.float32) if kind in (OPT["AMSGRAD"], OPT["AMSBOUND"]) else None
 
     def wd(self, batch, training_size):
         f = np.float32
@@ -88,6 +92,22 @@ class OptimizerHost:
                                             nthreads)
             else:
                 self.leaves.opt_gd(p, g, self.mask, self.lr, wd, nthreads)
+        elif self.kind in (OPT["ADABOUND"], OPT["AMSBOUND"]):
+            # adabound.cpp:49-55: the band closes on learning_rate_final as the time step grows
+            f, one = np.float32, np.float32(1)
+            lower = f(self.lr_final * f(one - f(one / f(f(self.gamma * self.t) + one))))
+            upper = f(self.lr_final * f(one + f(one / f(self.gamma * self.t))))
+            self.leaves.opt_adabound(p, g, self.m1, self.m2, self.vhat, self.mask, self.lr_t(), self.beta1, self.beta2,
+                                     self.eps, wd, lower, upper, nthreads)
+        elif self.kind == OPT["NOSADAM"]:
+            # nosadam.cpp:49-52, 68: the second-moment decay of step t is B_{t-1} / B_t with
+            # B_t = sum_{k<=t} k^-gamma; the bias correction still uses the fixed beta2
+            f = np.float32
+            term = f(np.power(self.t, f(-self.adam_gamma)))
+            beta2_t = f(self.previous_beta2 / f(self.previous_beta2 + term))
+            self.previous_beta2 = f(self.previous_beta2 + term)
+            self.leaves.opt_adam(p, g, self.m1, self.m2, None, self.mask, self.lr_t(), self.beta1, beta2_t, self.eps, wd,
+                                 nthreads)
         else:
             self.leaves.opt_adam(p, g, self.m1, self.m2, self.vhat, self.mask, self.lr_t(), self.beta1, self.beta2,
                                  self.eps, wd, nthreads)
@@ -284,6 +304,11 @@ class Oracle(_Leaves):
         self._f("opt_adam")(c_int(nthreads), c_sz(p.size), _ptr(p), _ptr(g), _ptr(m1), _ptr(m2), _ptr(vhat),
                             _ptr(mask), self._real(lr_t), self._real(beta1), self._real(beta2), self._real(eps),
                             self._real(wd))
+
+    def opt_adabound(self, p, g, m1, m2, vhat, mask, lr_t, beta1, beta2, eps, wd, rate_lower, rate_upper, nthreads=0):
+        self._f("opt_adabound")(c_int(nthreads), c_sz(p.size), _ptr(p), _ptr(g), _ptr(m1), _ptr(m2), _ptr(vhat),
+                                _ptr(mask), self._real(lr_t), self._real(beta1), self._real(beta2), self._real(eps),
+                                self._real(wd), self._real(rate_lower), self._real(rate_upper))
 
     def dropout_fwd(self, kind, v, mask, scale_or_keep, nthreads=0):
         """kind 0 inverted, 1 plain, 2 inference.  mask [H] (reference semantics,
@@ -605,7 +630,9 @@ class ReferenceMLP:
 
     # ---- optimizer (Model::Update_Parameter) ---------------------------------
     def set_optimizer(self, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9, beta2=0.999,
-                      eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True):
+                      eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True, lr_final=0.1, gamma=1e-3,
+                      adam_gamma=0.1):
+        self.lib.dlref_model_set_bound_hyper(self.h, c_f(lr_final), c_f(gamma), c_f(adam_gamma))
         ok = self.lib.dlref_model_set_optimizer(self.h, c_int(kind), c_f(lr), c_f(momentum), c_int(int(nesterov)),
                                                 c_f(adam_lr), c_f(beta1), c_f(beta2), c_f(eps),
                                                 c_int(int(bias_correction)), c_f(weight_decay),

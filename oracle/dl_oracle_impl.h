@@ -372,6 +372,34 @@ void FN(dlo_opt_adam)(int nthreads, size_t n, REAL *p, REAL *g, REAL *m1, REAL *
   }
 }
 
+/* AdaBound: adabound.cpp:37-112; AMSBound (vhat != NULL): amsbound.cpp:38-124.  The
+ * per-parameter step size lr_t / (sqrt(v) + eps) is clipped into [rate_lower,
+ * rate_upper], the band the reference computes once per call from
+ * learning_rate_final and learning_gamma (adabound.cpp:49-55); clip as ops/math.hpp:56-59. */
+void FN(dlo_opt_adabound)(int nthreads, size_t n, REAL *p, REAL *g, REAL *m1, REAL *m2, REAL *vhat, REAL const *mask,
+                          REAL lr_t, REAL beta1, REAL beta2, REAL eps, REAL wd, REAL rate_lower, REAL rate_upper) {
+  int const N = nthreads, ni = (int)n;
+  int i;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (i = 0; i < ni; ++i) {
+    REAL const d = g[i];
+    REAL const a = beta1 * m1[i] + ((REAL)1 - beta1) * d;
+    REAL v = beta2 * m2[i] + ((REAL)1 - beta2) * d * d;
+    REAL rate;
+    m1[i] = a;
+    m2[i] = v;
+    if (vhat != NULL) {
+      v = vhat[i] > v ? vhat[i] : v;
+      vhat[i] = v;
+    }
+    rate = lr_t / (SQRT(v) + eps);
+    rate = rate < rate_lower ? rate_lower : (rate > rate_upper ? rate_upper : rate);
+    if (wd != (REAL)0) p[i] -= rate * a + mask[i] * wd * p[i];
+    else p[i] -= rate * a;
+    g[i] = (REAL)0;
+  }
+}
+
 /* ---- a18  dY += dZn * Wn: bwp_st.cpp:1009-1045, bwp_mp.cpp:968-1007 ------- */
 void FN(dlo_fc_bwd_dx)(int nthreads, size_t B, size_t Hn, size_t H,
                        REAL const *dZn, REAL const *Wn, REAL *dY) {

@@ -696,6 +696,13 @@ int dlref_model_set_optimizer(void *h, int type, float lr, float momentum, int n
   if (!m.set_weight_decay(weight_decay)) return 0;
   return 1;
 }
+// AdaBound / AMSBound: learning_rate_final, learning_gamma; NosAdam: adam_gamma (model.hpp:3021-3034)
+void dlref_model_set_bound_hyper(void *h, float lr_final, float gamma, float adam_gamma) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  m.learning_rate_final = lr_final;
+  m.learning_gamma = gamma;
+  m.adam_gamma = adam_gamma;
+}
 void dlref_model_set_epoch_time_step(void *h, float v) { static_cast<RefModel *>(h)->model.epoch_time_step = v; }
 float dlref_model_opt_time_step(void *h) { return static_cast<RefModel *>(h)->model.optimizer_time_step; }
 void dlref_model_set_dparams(void *h, float const *p, size_t n) {

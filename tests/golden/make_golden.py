@@ -211,6 +211,14 @@ OPT_CASES = {
                                     weight_decay=0.03, normalized_wd=True)),
     "amsgrad": ("AMSGRAD", dict(adam_lr=0.005, beta1=0.7, beta2=0.9)),
     "amsgrad_wd": ("AMSGRAD", dict(adam_lr=0.005, weight_decay=0.01, normalized_wd=False)),
+    # a fast-closing band (gamma large), so that both clips bind within the four steps
+    "adabound": ("ADABOUND", dict(adam_lr=0.01, lr_final=0.05, gamma=0.5)),
+    "adabound_wd_norm": ("ADABOUND", dict(adam_lr=0.01, beta1=0.8, beta2=0.99, lr_final=0.1, gamma=1e-3,
+                                          weight_decay=0.03, normalized_wd=True)),
+    "amsbound": ("AMSBOUND", dict(adam_lr=0.005, beta1=0.7, beta2=0.9, lr_final=0.02, gamma=0.3)),
+    "nosadam": ("NOSADAM", dict(adam_lr=0.002, adam_gamma=0.1)),
+    "nosadam_wd": ("NOSADAM", dict(adam_lr=0.002, adam_gamma=0.05, bias_correction=False, weight_decay=0.02,
+                                   normalized_wd=False)),
 }
 OPT_STEPS = 4
 OPT_BATCH, OPT_TRAINING_SIZE = 5, 60

@@ -38,6 +38,10 @@ class GpuLeaves:
         self._run(self.dl.opt_adam, [p, g, m1, m2, vhat, mask], float(lr_t), float(b1), float(b2), float(eps),
                   float(wd))
 
+    def opt_adabound(self, p, g, m1, m2, vhat, mask, lr_t, b1, b2, eps, wd, lower, upper, nthreads=0):
+        self._run(self.dl.opt_adabound, [p, g, m1, m2, vhat, mask], float(lr_t), float(b1), float(b2), float(eps),
+                  float(wd), float(lower), float(upper))
+
 
 @pytest.fixture(scope="module")
 def golden_optim():
@@ -64,6 +68,9 @@ def test_gpu_optimizer_against_golden(dl, golden_optim, name):
     ("GD", dict(lr=0.05, momentum=0.9, nesterov=True, weight_decay=0.1, normalized_wd=True)),
     ("ADAM", dict(adam_lr=0.01, weight_decay=0.05)),
     ("AMSGRAD", dict(adam_lr=0.01, beta2=0.9)),
+    ("ADABOUND", dict(adam_lr=0.01, lr_final=0.05, gamma=0.5, weight_decay=0.05)),
+    ("AMSBOUND", dict(adam_lr=0.01, beta2=0.9, lr_final=0.02, gamma=0.3)),
+    ("NOSADAM", dict(adam_lr=0.01, adam_gamma=0.1, weight_decay=0.02, normalized_wd=False)),
 ])
 def test_gpu_optimizer_against_oracle(dl, oracle, n, kind, kw):
     rng = np.random.default_rng(n + len(kind))

@@ -157,6 +157,49 @@ def test_amsgrad_denominator_never_shrinks(oracle64):
     assert (vh > m2).any()  # after the small gradients the running maximum is what counts
 
 
+def test_adabound_reduces_to_adam_and_to_sgd_on_the_first_moment(oracle64):
+    """With a band wide enough never to bind, AdaBound is Adam; with a band of zero
+    width at eta it is p -= eta * m1 (plain descent on the first moment), whatever the
+    second moment says.  In between, the step size of each parameter is the clipped one."""
+    rng = np.random.default_rng(6)
+    n = 40
+    p0, g = rng.standard_normal(n), rng.standard_normal(n) * np.exp(rng.uniform(-6, 2, n))
+    pa, m1a, m2a = p0.copy(), np.zeros(n), np.zeros(n)
+    oracle64.opt_adam(pa, g.copy(), m1a, m2a, None, None, 0.01, 0.9, 0.999, 1e-8, 0.0)
+    pb, m1b, m2b = p0.copy(), np.zeros(n), np.zeros(n)
+    oracle64.opt_adabound(pb, g.copy(), m1b, m2b, None, None, 0.01, 0.9, 0.999, 1e-8, 0.0, 0.0, 1e30)
+    np.testing.assert_allclose(pb, pa, rtol=1e-14)
+    pc, m1c, m2c = p0.copy(), np.zeros(n), np.zeros(n)
+    oracle64.opt_adabound(pc, g.copy(), m1c, m2c, None, None, 0.01, 0.9, 0.999, 1e-8, 0.0, 0.07, 0.07)
+    np.testing.assert_allclose(pc, p0 - 0.07 * 0.1 * g, rtol=1e-13)
+    pd, m1d, m2d = p0.copy(), np.zeros(n), np.zeros(n)
+    oracle64.opt_adabound(pd, g.copy(), m1d, m2d, None, None, 0.01, 0.9, 0.999, 1e-8, 0.0, 0.1, 2.0)
+    rate = np.clip(0.01 / (np.sqrt(0.001 * g * g) + 1e-8), 0.1, 2.0)
+    assert (rate == 0.1).any() and (rate == 2.0).any() and ((rate > 0.1) & (rate < 2.0)).any()
+    np.testing.assert_allclose(pd, p0 - rate * 0.1 * g, rtol=1e-13)
+    # AMSBound: the running maximum replaces the second moment
+    vh = np.full(n, 4.0)
+    pe, m1e, m2e = p0.copy(), np.zeros(n), np.zeros(n)
+    oracle64.opt_adabound(pe, g.copy(), m1e, m2e, vh, None, 0.01, 0.9, 0.999, 1e-8, 0.0, 0.0, 1e30)
+    assert (vh >= 4.0).all()
+    np.testing.assert_allclose(pe, p0 - 0.01 / (np.sqrt(vh) + 1e-8) * 0.1 * g, rtol=1e-13)
+
+
+def test_nosadam_weights_the_past_by_a_hyper_harmonic_series(oracle64):
+    """NosAdam's second moment after t steps is sum_k k^-gamma g_k^2 / sum_k k^-gamma
+    (Huang et al. 2019, eq. 5): the decay B_{t-1}/B_t telescopes to that."""
+    rng = np.random.default_rng(8)
+    n, steps, gamma = 12, 6, 0.1
+    host = OptimizerHost(oracle64, n, OPT["NOSADAM"], adam_lr=0.001, adam_gamma=gamma)
+    host.m1, host.m2 = np.zeros(n), np.zeros(n)
+    p = np.zeros(n)
+    gs = rng.standard_normal((steps, n))
+    for gk in gs:
+        host.update(p, gk.copy(), 1, 1)
+    w = np.arange(1, steps + 1, dtype=np.float64) ** -gamma
+    np.testing.assert_allclose(host.m2, (w[:, None] * gs * gs).sum(0) / w.sum(), rtol=1e-5)  # host scalars are float
+
+
 def test_host_scalars(oracle):
     """Normalized weight decay wd*sqrt(B/(N*epochs)) (train.cpp:278-283) and the
     bias-corrected step size (adam.cpp:50-54), in float."""
@@ -169,16 +212,19 @@ def test_host_scalars(oracle):
 
 
 # ---- against the compiled reference, fresh cases ----------------------------------
-@pytest.mark.parametrize("seed", range(4))
+@pytest.mark.parametrize("seed", range(7))
 def test_oracle_optimizer_against_reference(oracle, reference, seed):
     rng = np.random.default_rng(300 + seed)
     widths = [int(rng.integers(3, 12)) for _ in range(4)]
     nt = int(rng.integers(0, 4))
-    kind = ["GD", "GD", "ADAM", "AMSGRAD"][seed]
+    kind = ["GD", "GD", "ADAM", "AMSGRAD", "ADABOUND", "AMSBOUND", "NOSADAM"][seed]
     kw = [dict(lr=0.03, momentum=0.0, weight_decay=0.1, normalized_wd=True),
           dict(lr=0.03, momentum=0.7, nesterov=bool(seed % 2), weight_decay=0.02, normalized_wd=False),
           dict(adam_lr=0.02, beta1=0.85, beta2=0.97, eps=1e-7, weight_decay=0.05),
-          dict(adam_lr=0.02, bias_correction=False)][seed]
+          dict(adam_lr=0.02, bias_correction=False),
+          dict(adam_lr=0.02, lr_final=0.04, gamma=0.4, weight_decay=0.05),
+          dict(adam_lr=0.02, beta2=0.95, lr_final=0.03, gamma=0.2),
+          dict(adam_lr=0.02, adam_gamma=0.05, weight_decay=0.01, normalized_wd=False)][seed]
     M = reference.mlp(widths)
     for l in (1, 2):
         M.set_layer(l, ACT["ELU"], NORM["BRN"])
