@@ -40,7 +40,7 @@ C_ABI_SYMBOLS = [
     "dlmi_softmax_fwd", "dlmi_dropout_fwd", "dlmi_identity_add", "dlmi_softmax_ce_seed",
     "dlmi_fused_norm_act_fwd", "dlmi_fused_norm_act_bwd", "dlmi_fused_norm_act_infer", "dlmi_fc_norm_act_fwd",
     "dlmi_opt_gd", "dlmi_opt_gd_momentum", "dlmi_opt_adam", "dlmi_zero_padded_identity_fwd", "dlmi_residual_bwd",
-    "dlmi_opt_adabound",
+    "dlmi_opt_adabound", "dlmi_clip_gradient", "dlmi_max_norm_rows",
 ]
 
 
@@ -269,6 +269,17 @@ class Dlmi:
         self._ck(self.lib.dlmi_opt_adabound(self.ctx, c_sz(p.numel()), _p(p), _p(g), _p(m1), _p(m2), _p(vhat), _p(mask),
                                             c_f(lr_t), c_f(beta1), c_f(beta2), c_f(eps), c_f(wd), c_f(rate_lower),
                                             c_f(rate_upper)))
+
+    def clip_gradient(self, g, max_norm):
+        """In place: g *= max_norm / ||g|| when ||g|| >= max_norm."""
+        self._chk(g)
+        self._ck(self.lib.dlmi_clip_gradient(self.ctx, c_sz(g.numel()), _p(g), c_f(max_norm)))
+
+    def max_norm_rows(self, W, max_norm):
+        """In place, per row of W [rows, cols]."""
+        self._chk(W)
+        rows, cols = W.shape
+        self._ck(self.lib.dlmi_max_norm_rows(self.ctx, c_sz(rows), c_sz(cols), _p(W), c_f(max_norm)))
 
     def softmax_ce_seed(self, q, y, stats=None):
         """stats: optional device tensor of 2 float64 accumulators."""

@@ -1113,6 +1113,13 @@ void Model::Update_Parameter(size_t const batch, size_t const training_size) {
   real const wd = use_normalized_weight_decay ? normalized_wd(batch, training_size) : weight_decay;
   if (wd != 0.0f && m.d_opt[4] == nullptr && !set_weight_decay(weight_decay)) return;
   int rc = DLMI_OK;
+  // update_weights_{st,mp} (model.cpp:4711-4866) clip the gradient first.  (The L1 / L2 terms those
+  // functions would add before that never act in the reference: their call passes (batch_size, 0,
+  // total_weights) to a (start, end, batch_size) signature, an empty range, so there is nothing to match.)
+  if (use_clip_gradient && dlmi_clip_gradient(m.ctx, P, m.d_dparams, clip_gradient) != DLMI_OK) {
+    fail("Update_Parameter: dlmi_clip_gradient");
+    return;
+  }
   switch (type_optimizer_function) {
     case OPTIMIZER::GD: {
       optimizer_time_step += 1.0f;
@@ -1180,7 +1187,29 @@ void Model::Update_Parameter(size_t const batch, size_t const training_size) {
       fail("Update_Parameter: optimizer type is not managed");
       return;
   }
-  if (rc != DLMI_OK) fail("Update_Parameter: optimizer kernel");
+  if (rc != DLMI_OK) { fail("Update_Parameter: optimizer kernel"); return; }
+  // max_norm.cpp:61-78: every unit's incoming weights, the output layer's included
+  if (regularization__max_norm_constraints != 0.0f)
+    for (size_t li = 1; li < total_layers; ++li) {
+      Layer const &l = ptr_array_layers[li];
+      if (l.type_layer != LAYER::FULLY_CONNECTED) continue;
+      if (dlmi_max_norm_rows(m.ctx, l.n_out, l.n_inp, m.d_params + l.first_connection_index,
+                             regularization__max_norm_constraints) != DLMI_OK) {
+        fail("Update_Parameter: dlmi_max_norm_rows");
+        return;
+      }
+    }
+}
+
+bool Model::set_clip_gradient(real const clip_gradient_received) {
+  clip_gradient = clip_gradient_received;
+  return true;
+}
+
+bool Model::Set__Regularization__Max_Norm_Constraints(real const v) {
+  if (v < 0.0f) return fail("Max-norm constraints less than zero.");  // max_norm.cpp:33-38
+  regularization__max_norm_constraints = v;
+  return true;
 }
 
 bool Model::download_optimizer_state(int which, float *out) const {

@@ -221,6 +221,11 @@ void dlmi_model_set_bound_hyper(dlmi_model *h, float lr_final, float gamma, floa
   h->m.learning_gamma = gamma;
   h->m.adam_gamma = adam_gamma;
 }
+int dlmi_model_set_constraints(dlmi_model *h, int use_clip, float clip, float max_norm) {
+  h->m.set_clip_gradient(use_clip != 0);
+  if (!h->m.set_clip_gradient(clip)) return 0;
+  return h->m.Set__Regularization__Max_Norm_Constraints(max_norm) ? 1 : 0;
+}
 void dlmi_model_set_epoch_time_step(dlmi_model *h, float v) { h->m.epoch_time_step = v; }
 int dlmi_model_set_derivatives(dlmi_model *h, float const *g, size_t n) {
   if (n != h->m.total_parameters) return 0;

@@ -24,7 +24,7 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_model_get_optimizer_state", "dlmi_driver_create", "dlmi_driver_destroy", "dlmi_driver_train",
     "dlmi_driver_evalt", "dlmi_model_create_typed", "dlmi_model_layer_info", "dlmi_mnist_create",
     "dlmi_mnist_destroy", "dlmi_mnist_load", "dlmi_mnist_last_error", "dlmi_mnist_copy",
-    "dlmi_model_glorot_uniform", "dlmi_model_init_uniform", "dlmi_model_set_bound_hyper",
+    "dlmi_model_glorot_uniform", "dlmi_model_init_uniform", "dlmi_model_set_bound_hyper", "dlmi_model_set_constraints",
 ]
 
 LAYER_FULLY_CONNECTED, LAYER_RESIDUAL = 3, 9  # v1/data/enum/layer.hpp
@@ -187,8 +187,10 @@ class Model:
     # ---- optimizer (Model::set_optimizer / set_weight_decay / Update_Parameter) ----
     def set_optimizer(self, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9, beta2=0.999,
                       eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True, lr_final=0.1, gamma=1e-3,
-                      adam_gamma=0.1):
+                      adam_gamma=0.1, clip=None, max_norm=0.0):
         self.lib.dlmi_model_set_bound_hyper(self.h, c_f(lr_final), c_f(gamma), c_f(adam_gamma))
+        self._ok(self.lib.dlmi_model_set_constraints(self.h, c_int(int(clip is not None)),
+                                                     c_f(1.0 if clip is None else clip), c_f(max_norm)), "constraints")
         self._ok(self.lib.dlmi_model_set_optimizer(self.h, c_int(kind), c_f(lr), c_f(momentum), c_int(int(nesterov)),
                                                    c_f(adam_lr), c_f(beta1), c_f(beta2), c_f(eps),
                                                    c_int(int(bias_correction)), c_f(weight_decay),

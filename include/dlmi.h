@@ -286,6 +286,17 @@ int dlmi_opt_adabound(dlmi_ctx *ctx, size_t n, float *params, float *grads, floa
                       float *m2_hat, float const *mask, float lr_t, float beta1, float beta2,
                       float eps, float wd, float rate_lower, float rate_upper);
 
+/* ---- Euclidean-norm constraints either side of the optimizer step -----------
+ * (euclidean_norm_{st,mp}, v1/ops/constraints/euclidean.cpp:24-62: when the norm
+ * is >= max_norm, every element is multiplied by max_norm / norm) */
+/* Over the whole gradient array, before the step (Clip_Gradient__{Loop,OpenMP},
+ * v1/ops/constraints/clip_gradient.cpp:75-83). */
+int dlmi_clip_gradient(dlmi_ctx *ctx, size_t n, float *grads, float max_norm);
+/* Over each row of W [rows][cols] = each unit's fan-in, after the step
+ * (Update_Weight_Regularization__Max_Norm_Constraints__Neurons__*,
+ * v1/ops/constraints/max_norm.cpp:61-78, 278-300). */
+int dlmi_max_norm_rows(dlmi_ctx *ctx, size_t rows, size_t cols, float *W, float max_norm);
+
 #ifdef __cplusplus
 }
 #endif

@@ -68,6 +68,8 @@ int dlmi_model_set_optimizer(dlmi_model *m, int type, float lr, float momentum, 
 /* learning_rate_final, learning_gamma (AdaBound / AMSBound) and adam_gamma (NosAdam): call before
  * dlmi_model_set_optimizer */
 void dlmi_model_set_bound_hyper(dlmi_model *m, float lr_final, float gamma, float adam_gamma);
+/* set_clip_gradient(use_clip != 0), set_clip_gradient(clip), Set__Regularization__Max_Norm_Constraints(max_norm) */
+int dlmi_model_set_constraints(dlmi_model *m, int use_clip, float clip, float max_norm);
 void dlmi_model_set_epoch_time_step(dlmi_model *m, float v);
 int dlmi_model_set_derivatives(dlmi_model *m, float const *g, size_t n);      /* host array -> device gradient array */
 void dlmi_model_update_parameter(dlmi_model *m, size_t batch, size_t training_size);  /* Update_Parameter */

@@ -194,6 +194,15 @@ class Model {
   bool set_weight_decay(real const val);
   real normalized_wd(size_t const batch_size, size_t const training_size);
   void Update_Parameter(size_t const batch_size, size_t const training_size);
+  // The Euclidean-norm constraints Update_Parameter applies around the step
+  // (model.cpp:4797-4866): the whole gradient array is scaled onto the ball of
+  // radius clip_gradient before it (v1/ops/constraints/clip_gradient.cpp:30-83),
+  // each unit's incoming weights onto the ball of radius
+  // regularization__max_norm_constraints after it (max_norm.cpp:28-78); 0 = off.
+  void set_clip_gradient(bool const use_clip_gradient_received) { use_clip_gradient = use_clip_gradient_received; }
+  bool set_clip_gradient(real const clip_gradient_received);
+  bool Use__Clip_Gradient(void) const { return use_clip_gradient; }
+  bool Set__Regularization__Max_Norm_Constraints(real const regularization__max_norm_constraints_received);
   // which: 0 previous delta, 1 first moment, 2 second moment, 3 second moment hat,
   // 4 regularization mask; false when that array does not exist.
   bool download_optimizer_state(int which, float *out) const;
@@ -245,6 +254,9 @@ class Model {
   real adam_beta1 = 0.9f;
   real adam_beta2 = 0.999f;
   real adam_epsilon = 1e-8f;
+  bool use_clip_gradient = false;                     // model.hpp:2843
+  real clip_gradient = 1.0f;                          // model.hpp:3044
+  real regularization__max_norm_constraints = 0.0f;   // model.hpp:3024
   real learning_rate_final = 0.1f;  // AdaBound / AMSBound: the rate the band closes on (model.hpp:3021)
   real learning_gamma = 1e-3f;      // AdaBound / AMSBound: how fast it closes (model.hpp:3023)
   real adam_previous_beta2 = 0.0f;  // NosAdam: B_{t-1} (model.hpp:3032)

@@ -55,8 +55,11 @@ class OptimizerHost:
 
     def __init__(self, leaves, n, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9,
                  beta2=0.999, eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True, mask=None,
-                 lr_final=0.1, gamma=1e-3, adam_gamma=0.1):
+                 lr_final=0.1, gamma=1e-3, adam_gamma=0.1, clip=None, max_norm=0.0, weight_rows=()):
         f = np.float32
+        # Update_Parameter (model.cpp:4797-4866): [gradient clip] -> optimizer -> [max-norm per unit].
+        # weight_rows: (first weight index, units, fan-in) of every fully-connected layer.
+        self.clip, self.max_norm, self.weight_rows = clip, f(max_norm), tuple(weight_rows)
         self.leaves, self.n, self.kind = leaves, n, kind
         self.lr, self.momentum, self.nesterov = f(lr), f(momentum), bool(nesterov)
         self.adam_lr, self.beta1, self.beta2, self.eps = f(adam_lr), f(beta1), f(beta2), f(eps)
@@ -84,6 +87,14 @@ class OptimizerHost:
         return f(f(self.adam_lr * np.sqrt(f(f(1) - np.power(self.beta2, self.t)))) / f(f(1) - np.power(self.beta1, self.t)))
 
     def update(self, p, g, batch, training_size, nthreads=0):
+        if self.clip is not None:
+            self.leaves.clip_gradient(g, np.float32(self.clip), nthreads)
+        self._step(p, g, batch, training_size, nthreads)
+        if self.max_norm != 0:
+            for w0, rows, cols in self.weight_rows:
+                self.leaves.max_norm_rows(p[w0:w0 + rows * cols].reshape(rows, cols), self.max_norm, nthreads)
+
+    def _step(self, p, g, batch, training_size, nthreads):
         self.t = np.float32(self.t + np.float32(1))
         wd = self.wd(batch, training_size)
         if self.kind == OPT["GD"]:
@@ -305,6 +316,14 @@ class Oracle(_Leaves):
                             _ptr(mask), self._real(lr_t), self._real(beta1), self._real(beta2), self._real(eps),
                             self._real(wd))
 
+    def clip_gradient(self, g, max_norm, nthreads=0):
+        """euclidean_norm on the whole array, in place."""
+        self._f("euclidean_norm")(c_int(nthreads), c_sz(g.size), self._real(max_norm), _ptr(g))
+
+    def max_norm_rows(self, W, max_norm, nthreads=0):
+        """euclidean_norm on every row of W [rows, cols], in place."""
+        self._f("max_norm_rows")(c_int(nthreads), c_sz(W.shape[0]), c_sz(W.shape[1]), self._real(max_norm), _ptr(W))
+
     def opt_adabound(self, p, g, m1, m2, vhat, mask, lr_t, beta1, beta2, eps, wd, rate_lower, rate_upper, nthreads=0):
         self._f("opt_adabound")(c_int(nthreads), c_sz(p.size), _ptr(p), _ptr(g), _ptr(m1), _ptr(m2), _ptr(vhat),
                                 _ptr(mask), self._real(lr_t), self._real(beta1), self._real(beta2), self._real(eps),
@@ -424,7 +443,8 @@ class OracleMLP:
             nw = sum(self.widths[l] * self.widths[l - 1] for l in range(1, len(self.widths)))
             mask = np.zeros(self.P, np.float32)
             mask[:nw] = 1
-        self.opt = OptimizerHost(self.o, self.P, kind, mask=mask, **kw)
+        rows = [(self.layer_offsets(l)[0], self.widths[l], self.widths[l - 1]) for l in range(1, len(self.widths))]
+        self.opt = OptimizerHost(self.o, self.P, kind, mask=mask, weight_rows=rows, **kw)
 
     def update_parameter(self, batch, training_size):
         self.opt.update(self.parameters, self.dparameters, batch, training_size, self.nthreads)
@@ -506,6 +526,15 @@ class Reference(_Leaves):
         self._f("dropout_fwd")(c_int(nthreads), c_int(kind), c_sz(B), c_sz(H), _ptr(m),
                                c_f(scale_or_keep), _ptr(v))
         return v
+
+    def clip_gradient(self, g, max_norm, nthreads=0):
+        """euclidean_norm_st (nthreads 0) / euclidean_norm_mp on a float32 array, in place."""
+        self._f("euclidean_norm")(c_int(nthreads), c_sz(g.size), c_f(max_norm), _ptr(g))
+
+    def max_norm_rows(self, W, max_norm, nthreads=0):
+        # max_norm.cpp:61-78 walks the units and calls euclidean_norm_st on each one's weights
+        for r in range(W.shape[0]):
+            self._f("euclidean_norm")(c_int(0), c_sz(W.shape[1]), c_f(max_norm), _ptr(W[r]))
 
     def mlp(self, widths, allowable_bytes=1 << 32):
         return ReferenceMLP(self, widths, allowable_bytes)
@@ -631,8 +660,11 @@ class ReferenceMLP:
     # ---- optimizer (Model::Update_Parameter) ---------------------------------
     def set_optimizer(self, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9, beta2=0.999,
                       eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True, lr_final=0.1, gamma=1e-3,
-                      adam_gamma=0.1):
+                      adam_gamma=0.1, clip=None, max_norm=0.0):
         self.lib.dlref_model_set_bound_hyper(self.h, c_f(lr_final), c_f(gamma), c_f(adam_gamma))
+        ok = self.lib.dlref_model_set_constraints(self.h, c_int(int(clip is not None)), c_f(1.0 if clip is None else clip),
+                                                  c_f(max_norm))
+        assert ok, "reference refused the constraint settings"
         ok = self.lib.dlref_model_set_optimizer(self.h, c_int(kind), c_f(lr), c_f(momentum), c_int(int(nesterov)),
                                                 c_f(adam_lr), c_f(beta1), c_f(beta2), c_f(eps),
                                                 c_int(int(bias_correction)), c_f(weight_decay),

@@ -400,6 +400,30 @@ void FN(dlo_opt_adabound)(int nthreads, size_t n, REAL *p, REAL *g, REAL *m1, RE
   }
 }
 
+/* euclidean_norm_{st,mp}: v1/ops/constraints/euclidean.cpp:24-62.  Used on the whole
+ * gradient array before the optimizer step (clip_gradient.cpp:75-83) and on each
+ * unit's fan-in after it (max_norm.cpp:61-78, 278-300). */
+void FN(dlo_euclidean_norm)(int nthreads, size_t n, REAL max_norm, REAL *v) {
+  int const N = nthreads, ni = (int)n;
+  int i;
+  REAL norm = (REAL)0;
+#pragma omp parallel for reduction(+ : norm) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (i = 0; i < ni; ++i) norm += v[i] * v[i];
+  norm = SQRT(norm);
+  if (norm >= max_norm) {
+    REAL const desired = max_norm / norm;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+    for (i = 0; i < ni; ++i) v[i] *= desired;
+  }
+}
+/* every row of W [rows][cols] (one unit's incoming weights) */
+void FN(dlo_max_norm_rows)(int nthreads, size_t rows, size_t cols, REAL max_norm, REAL *W) {
+  int const N = nthreads, nr = (int)rows;
+  int r;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (r = 0; r < nr; ++r) FN(dlo_euclidean_norm)(0, cols, max_norm, W + (size_t)r * cols);
+}
+
 /* ---- a18  dY += dZn * Wn: bwp_st.cpp:1009-1045, bwp_mp.cpp:968-1007 ------- */
 void FN(dlo_fc_bwd_dx)(int nthreads, size_t B, size_t Hn, size_t H,
                        REAL const *dZn, REAL const *Wn, REAL *dY) {

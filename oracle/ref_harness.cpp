@@ -703,6 +703,22 @@ void dlref_model_set_bound_hyper(void *h, float lr_final, float gamma, float ada
   m.learning_gamma = gamma;
   m.adam_gamma = adam_gamma;
 }
+// Gradient clipping (clip_gradient.cpp:30-83) and the max-norm constraint (max_norm.cpp:28-51) of Update_Parameter
+int dlref_model_set_constraints(void *h, int use_clip, float clip, float max_norm) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  m.set_clip_gradient(use_clip != 0);
+  if (!m.set_clip_gradient(clip)) return 0;
+  return m.Set__Regularization__Max_Norm_Constraints(max_norm) ? 1 : 0;
+}
+// euclidean_norm_{st,mp} (euclidean.cpp:24-62) on a caller's array, in place
+void dlref_euclidean_norm(int nthreads, size_t n, float max_norm, float *v) {
+  if (nthreads > 0) {
+    omp_set_num_threads(nthreads);
+    euclidean_norm_mp<real>(0, n, max_norm, v);
+  } else {
+    euclidean_norm_st<real>(0, n, max_norm, v);
+  }
+}
 void dlref_model_set_epoch_time_step(void *h, float v) { static_cast<RefModel *>(h)->model.epoch_time_step = v; }
 float dlref_model_opt_time_step(void *h) { return static_cast<RefModel *>(h)->model.optimizer_time_step; }
 void dlref_model_set_dparams(void *h, float const *p, size_t n) {

@@ -219,6 +219,12 @@ OPT_CASES = {
     "nosadam": ("NOSADAM", dict(adam_lr=0.002, adam_gamma=0.1)),
     "nosadam_wd": ("NOSADAM", dict(adam_lr=0.002, adam_gamma=0.05, bias_correction=False, weight_decay=0.02,
                                    normalized_wd=False)),
+    # the Euclidean-norm constraints around the step.  The gradients have norm ~ sqrt(163) ~ 12.8, the
+    # parameter rows ~ sqrt(fan-in): thresholds well away from both, binding and not binding
+    "gd_clip_binding": ("GD", dict(lr=0.05, momentum=0.0, clip=4.0)),
+    "gd_clip_loose": ("GD", dict(lr=0.05, momentum=0.9, clip=40.0)),
+    "adam_maxnorm": ("ADAM", dict(adam_lr=0.05, max_norm=2.0)),
+    "gd_clip_maxnorm_wd": ("GD", dict(lr=0.1, momentum=0.5, weight_decay=0.02, clip=6.0, max_norm=2.5)),
 }
 OPT_STEPS = 4
 OPT_BATCH, OPT_TRAINING_SIZE = 5, 60
@@ -248,6 +254,8 @@ def optimizers(R):
     grads[1, ::7] = 0  # zero gradients: second moments stay where they are
     d["opt_p0"], d["opt_grads"] = p0, grads
     d["opt_sizes"] = np.array([OPT_BATCH, OPT_TRAINING_SIZE])
+    # (first weight index, units, fan-in) of every layer: what the max-norm constraint walks
+    d["opt_weight_rows"] = np.array([[M0.layer_offsets(l)[0], widths[l], widths[l - 1]] for l in range(1, len(widths))])
     # the settings travel with the vectors (JSON text as bytes)
     traj = {"traj_adam": ("ADAM", dict(adam_lr=0.01)),
             "traj_momentum_wd": ("GD", dict(lr=0.1, momentum=0.9, weight_decay=0.01, normalized_wd=True))}

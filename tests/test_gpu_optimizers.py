@@ -38,6 +38,12 @@ class GpuLeaves:
         self._run(self.dl.opt_adam, [p, g, m1, m2, vhat, mask], float(lr_t), float(b1), float(b2), float(eps),
                   float(wd))
 
+    def clip_gradient(self, g, max_norm, nthreads=0):
+        self._run(self.dl.clip_gradient, [g], float(max_norm))
+
+    def max_norm_rows(self, W, max_norm, nthreads=0):
+        self._run(self.dl.max_norm_rows, [W], float(max_norm))
+
     def opt_adabound(self, p, g, m1, m2, vhat, mask, lr_t, b1, b2, eps, wd, lower, upper, nthreads=0):
         self._run(self.dl.opt_adabound, [p, g, m1, m2, vhat, mask], float(lr_t), float(b1), float(b2), float(eps),
                   float(wd), float(lower), float(upper))
@@ -90,6 +96,45 @@ def test_gpu_optimizer_against_oracle(dl, oracle, n, kind, kw):
                        (hg.vhat, ho.vhat, "vhat")):
         if b is not None:
             assert_close(a, b, TE, what)
+
+
+@pytest.mark.parametrize("n", [1, 5, 4099, 1 << 22])
+def test_gpu_clip_gradient_against_oracle(dl, oracle64, n):
+    """float64 arbitrates: over four million terms the oracle's own float sum drifts."""
+    rng = np.random.default_rng(n)
+    g = rng.standard_normal(n).astype(np.float32)
+    norm = float(np.linalg.norm(g.astype(np.float64)))
+    for c in (0.5 * norm, 2.0 * norm):
+        exp = g.astype(np.float64)
+        oracle64.clip_gradient(exp, c)
+        t = torch.from_numpy(g.copy()).cuda()
+        dl.clip_gradient(t, c)
+        assert_close(t.cpu().numpy(), exp, TE, f"clip at {c:.3g}")
+        if c > norm:
+            assert np.array_equal(t.cpu().numpy(), g), "below the threshold nothing is rewritten"
+    # a range that does not start on a 16-byte boundary
+    if n > 1:
+        t = torch.from_numpy(g.copy()).cuda()
+        exp = g[1:].astype(np.float64)
+        oracle64.clip_gradient(exp, 0.25 * norm)
+        dl.clip_gradient(t[1:], 0.25 * norm)
+        assert_close(t[1:].cpu().numpy(), exp, TE, "unaligned view")
+        assert float(t[0]) == float(g[0])
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (7, 50), (512, 784), (10, 4097), (3000, 33)])
+def test_gpu_max_norm_rows_against_oracle(dl, oracle64, rows, cols):
+    rng = np.random.default_rng(rows * 31 + cols)
+    W = (rng.standard_normal((rows, cols)) * rng.uniform(0.05, 2, (rows, 1))).astype(np.float32)
+    c = float(np.median(np.linalg.norm(W.astype(np.float64), axis=1))) * 1.001
+    exp = W.astype(np.float64)
+    oracle64.max_norm_rows(exp, c)
+    t = torch.from_numpy(W.copy()).cuda()
+    dl.max_norm_rows(t, c)
+    got = t.cpu().numpy()
+    assert_close(got, exp, TE, "rows")
+    untouched = np.linalg.norm(W.astype(np.float64), axis=1) < c * 0.999
+    assert np.array_equal(got[untouched], W[untouched])
 
 
 def test_gpu_optimizer_on_unaligned_views(dl, oracle):

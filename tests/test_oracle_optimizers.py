@@ -36,7 +36,8 @@ def run_leaf_case(leaves, g, name, nt):
     kind, kw = cases(g, "leaf")[name]
     mask = g[f"opt_{name}_mask"]
     p = g["opt_p0"].copy()
-    host = OptimizerHost(leaves, p.size, OPT[kind], mask=mask if mask.size else None, **kw)
+    rows = [tuple(int(v) for v in r) for r in g["opt_weight_rows"]]
+    host = OptimizerHost(leaves, p.size, OPT[kind], mask=mask if mask.size else None, weight_rows=rows, **kw)
     B, N = (int(v) for v in g["opt_sizes"])
     for t, grad in enumerate(g["opt_grads"]):
         gg = grad.copy()
@@ -198,6 +199,35 @@ def test_nosadam_weights_the_past_by_a_hyper_harmonic_series(oracle64):
         host.update(p, gk.copy(), 1, 1)
     w = np.arange(1, steps + 1, dtype=np.float64) ** -gamma
     np.testing.assert_allclose(host.m2, (w[:, None] * gs * gs).sum(0) / w.sum(), rtol=1e-5)  # host scalars are float
+
+
+def test_euclidean_norm_constraint_closed_form(oracle64, reference):
+    """Above the threshold the array lands on the sphere of that radius, direction
+    unchanged; below it nothing moves; row by row for the max-norm constraint.  The
+    compiled reference's own helper agrees on the same arrays."""
+    rng = np.random.default_rng(11)
+    v = rng.standard_normal(1000)
+    a = v.copy()
+    oracle64.clip_gradient(a, 3.0)
+    np.testing.assert_allclose(np.linalg.norm(a), 3.0, rtol=1e-12)
+    np.testing.assert_allclose(a / np.linalg.norm(a), v / np.linalg.norm(v), rtol=1e-12)
+    b = v.copy()
+    oracle64.clip_gradient(b, 1e6)
+    assert np.array_equal(b, v)
+    W = rng.standard_normal((7, 50)) * rng.uniform(0.05, 2, (7, 1))
+    Wc = W.copy()
+    oracle64.max_norm_rows(Wc, 4.0)
+    n0, n1 = np.linalg.norm(W, axis=1), np.linalg.norm(Wc, axis=1)
+    assert (n0 > 4).any() and (n0 < 4).any()
+    np.testing.assert_allclose(n1, np.minimum(n0, 4.0), rtol=1e-12)
+    assert np.array_equal(Wc[n0 < 4], W[n0 < 4])
+    for nt in (0, 3):
+        r32 = v.astype(np.float32)
+        reference.clip_gradient(r32, 3.0, nt)
+        np.testing.assert_allclose(r32, a, rtol=2e-6)
+        R = W.astype(np.float32)
+        reference.max_norm_rows(R, 4.0, nt)
+        np.testing.assert_allclose(R, Wc, rtol=2e-6)
 
 
 def test_host_scalars(oracle):
