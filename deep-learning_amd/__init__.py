@@ -40,7 +40,7 @@ C_ABI_SYMBOLS = [
     "dlmi_softmax_fwd", "dlmi_dropout_fwd", "dlmi_identity_add", "dlmi_softmax_ce_seed",
     "dlmi_fused_norm_act_fwd", "dlmi_fused_norm_act_bwd", "dlmi_fused_norm_act_infer", "dlmi_fc_norm_act_fwd",
     "dlmi_opt_gd", "dlmi_opt_gd_momentum", "dlmi_opt_adam", "dlmi_zero_padded_identity_fwd", "dlmi_residual_bwd",
-    "dlmi_opt_adabound", "dlmi_clip_gradient", "dlmi_max_norm_rows",
+    "dlmi_opt_adabound", "dlmi_clip_gradient", "dlmi_max_norm_rows", "dlmi_opt_irprop_plus",
 ]
 
 
@@ -269,6 +269,12 @@ class Dlmi:
         self._ck(self.lib.dlmi_opt_adabound(self.ctx, c_sz(p.numel()), _p(p), _p(g), _p(m1), _p(m2), _p(vhat), _p(mask),
                                             c_f(lr_t), c_f(beta1), c_f(beta2), c_f(eps), c_f(wd), c_f(rate_lower),
                                             c_f(rate_upper)))
+
+    def opt_irprop_plus(self, p, g, prev_g, prev_move, steps, incr, decr, step_min, step_max, worse, nthreads=0):
+        self._chk(p, g, prev_g, prev_move, steps)
+        self._ck(self.lib.dlmi_opt_irprop_plus(self.ctx, c_sz(p.numel()), _p(p), _p(g), _p(prev_g), _p(prev_move),
+                                               _p(steps), c_f(incr), c_f(decr), c_f(step_min), c_f(step_max),
+                                               c_int(1 if worse else 0)))
 
     def clip_gradient(self, g, max_norm):
         """In place: g *= max_norm / ||g|| when ||g|| >= max_norm."""

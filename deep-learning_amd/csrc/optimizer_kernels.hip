@@ -1,6 +1,6 @@
 // Optimizer steps over the packed parameter array for gfx950: plain gradient
 // descent, momentum, the reference's Nesterov variant, Adam, AMSGrad, AdaBound and AMSBound, each
-// with the optional masked weight decay, each zeroing the gradient it consumed.
+// with the optional masked weight decay, and iRPROP+; each zeroing the gradient it consumed.
 //
 // One pass, one thread per 4 parameters (float4), every array read once and
 // written once: bound by HBM bandwidth (Adam: 32 bytes per parameter).  The
@@ -16,7 +16,7 @@ namespace dlmi {
 
 constexpr int kOptBlock = 256;
 constexpr int kOptGd = 0, kOptMomentum = 1, kOptNesterov = 2, kOptAdam = 3, kOptAmsgrad = 4, kOptAdabound = 5,
-              kOptAmsbound = 6;
+              kOptAmsbound = 6, kOptIrpropPlus = 7;
 
 struct OptArgs {
   float *p, *g;
@@ -28,6 +28,10 @@ struct OptArgs {
   float lr;           // GD family: learning rate; Adam family: bias-corrected step size
   float mom, beta1, beta2, eps, wd;
   float rate_lo, rate_hi;  // AdaBound / AMSBound: the band the per-parameter step size is clipped into
+  // iRPROP+: s0 previous gradient, s1 previous parameter move, s2 step size; factors and limits of the
+  // step size; whether the loss got worse since the previous call
+  float incr, decr, step_min, step_max;
+  int loss_got_worse;
 };
 
 // One parameter.  gradient_descent.cpp:79-92, gradient_descent_momentum.cpp:44-63,
@@ -36,6 +40,32 @@ struct OptArgs {
 template <int KIND, bool WD>
 __device__ __forceinline__ void opt_one(OptArgs const &a, float &p, float g, float &s0, float &s1, float &s2,
                                         float mask) {
+  if constexpr (KIND == kOptIrpropPlus) {
+    // irprop_plus.cpp:53-77: the step size of a parameter grows while its gradient keeps its sign and
+    // shrinks when the sign flips; after a flip the last move is taken back if the loss got worse, and
+    // the stored gradient is cleared so that the next call takes the plain-step branch.  Only signs and
+    // one product per branch: bit-identical to the reference.
+    float const prod = s0 * g;
+    float const sgn = static_cast<float>((0.0f < g) - (g < 0.0f));  // ops/math.hpp:67-70
+    if (prod > 0.0f) {
+      float dt = s2 * a.incr;
+      dt = a.step_max < dt ? a.step_max : dt;
+      s2 = dt;
+      s1 = -sgn * dt;
+      p += s1;
+      s0 = g;
+    } else if (prod < 0.0f) {
+      float const dt = s2 * a.decr;
+      s2 = dt < a.step_min ? a.step_min : dt;
+      if (a.loss_got_worse) p -= s1;
+      s0 = 0.0f;
+    } else {
+      s1 = -sgn * s2;
+      p += s1;
+      s0 = g;
+    }
+    return;
+  }
   float step;
   if constexpr (KIND == kOptGd) {
     step = a.lr * g;
@@ -69,7 +99,7 @@ __device__ __forceinline__ void opt_one(OptArgs const &a, float &p, float g, flo
 
 template <int KIND, bool WD>
 __global__ __launch_bounds__(kOptBlock) void k_opt(OptArgs a, size_t n4) {
-  constexpr bool kS0 = KIND != kOptGd, kS1 = KIND >= kOptAdam, kS2 = KIND == kOptAmsgrad || KIND == kOptAmsbound;
+  constexpr bool kS0 = KIND != kOptGd, kS1 = KIND >= kOptAdam, kS2 = KIND == kOptAmsgrad || KIND == kOptAmsbound || KIND == kOptIrpropPlus;
   size_t const stride = static_cast<size_t>(gridDim.x) * kOptBlock;
   size_t i = static_cast<size_t>(blockIdx.x) * kOptBlock + threadIdx.x;
   for (; i < n4; i += stride) {
@@ -163,6 +193,18 @@ int dlmi_opt_adam(dlmi_ctx *ctx, size_t n, float *params, float *grads, float *m
   a.lr = lr_t; a.beta1 = beta1; a.beta2 = beta2; a.eps = eps; a.wd = wd;
   return m2_hat != nullptr ? launch_opt<kOptAmsgrad>(ctx, a, "k_opt<amsgrad>")
                            : launch_opt<kOptAdam>(ctx, a, "k_opt<adam>");
+}
+
+int dlmi_opt_irprop_plus(dlmi_ctx *ctx, size_t n, float *params, float *grads, float *prev_grads, float *prev_moves,
+                         float *step_sizes, float increase, float decrease, float step_min, float step_max,
+                         int loss_got_worse) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, n == 0 || (params && grads && prev_grads && prev_moves && step_sizes), "null pointer");
+  OptArgs a{};
+  a.p = params; a.g = grads; a.s0 = prev_grads; a.s1 = prev_moves; a.s2 = step_sizes; a.n = n;
+  a.incr = increase; a.decr = decrease; a.step_min = step_min; a.step_max = step_max;
+  a.loss_got_worse = loss_got_worse != 0 ? 1 : 0;
+  return launch_opt<kOptIrpropPlus>(ctx, a, "k_opt<irprop+>");
 }
 
 int dlmi_opt_adabound(dlmi_ctx *ctx, size_t n, float *params, float *grads, float *m1, float *m2, float *m2_hat,

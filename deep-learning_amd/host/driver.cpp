@@ -120,6 +120,10 @@ void Driver::train_st(void) {
   size_t const n_data = dataset.n_data, batch_size_max = model.batch_size;
   size_t const n_batch = static_cast<size_t>(std::ceil(static_cast<double>(n_data) / static_cast<double>(batch_size_max)));
   bool const resident = make_resident();
+  // iRPROP compares the loss of this epoch with that of the previous one (driver.cpp:269-273, 337)
+  bool const irprop = v1::OPTIMIZER::IRPROP_MINUS == model.type_optimizer_function ||
+                      v1::OPTIMIZER::IRPROP_PLUS == model.type_optimizer_function;
+  if (irprop) model.loss_rprop_tm1 = model.loss_rprop;
   for (size_t i = 0; i != n_batch; ++i) {
     size_t const batch_size = i + 1 != n_batch ? batch_size_max : n_data - i * batch_size_max;
     if (resident) {
@@ -132,6 +136,7 @@ void Driver::train_st(void) {
     model.backward_pass(batch_size);
     model.update_derivatives(batch_size, model.ptr_array_layers + 1, model.ptr_last_layer);
   }
+  if (irprop) model.loss_rprop = std::fabs(model.get_loss(v1::ENV::NONE));  // one device-to-host read of the loss sum
   model.Update_Parameter(n_data, n_data);
 }
 

@@ -35,8 +35,9 @@ struct Model::Impl {
   float *d_targets = nullptr;  // [batch, n_out]
   double *d_stats = nullptr;   // { loss sum, correct count }
   // optimizer state [P] each: 0 previous delta, 1 first moment, 2 second moment,
-  // 3 second moment hat, 4 regularization mask; allocated (zeroed) on first use
-  float *d_opt[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+  // 3 second moment hat, 4 regularization mask, 5 previous gradient, 6 step sizes (iRPROP+);
+  // allocated (zeroed; the step sizes filled with rprop_delta_zero) on first use
+  float *d_opt[7] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
   float const *cur_input = nullptr;  // [batch, n_in] of the pass in flight: d_input or a caller's device rows
   size_t n_loss_examples = 0;        // examples whose loss has been accumulated since reset_loss()
   size_t all_units = 0;              // normalization units of all entries: the slots a normalized model has
@@ -537,11 +538,13 @@ void Model::clear_training_arrays(void) {
   impl_->n_loss_examples = 0;
   std::memset(ptr_array_derivatives_parameters, 0, total_parameters * sizeof(real));
   // Clear_Optimizer (train.cpp:136-248): the optimizer's own arrays and its clocks
-  for (int i = 0; i < 4; ++i)
+  for (int i : {0, 1, 2, 3, 5})
     if (impl_->d_opt[i] != nullptr) (void)hipMemsetAsync(impl_->d_opt[i], 0, total_parameters * sizeof(float), impl_->stream);
+  dev_free(impl_->d_opt[6]);  // the step sizes start from rprop_delta_zero again: refilled on the next use
   optimizer_time_step = 0.0f;
   epoch_time_step = 1.0f;
   adam_previous_beta2 = 0.0f;
+  loss_rprop = loss_rprop_tm1 = static_cast<double>(std::numeric_limits<real>::max());  // train.cpp:167-168
 }
 
 // ---------------------------------------------------------------- buffer movement
@@ -1071,11 +1074,13 @@ void Model::set_optimizer(OPTIMIZER::TYPE const type_received) {
   if (type_optimizer_function == type_received) return;
   switch (type_received) {
     case OPTIMIZER::NONE: case OPTIMIZER::GD: case OPTIMIZER::ADAM: case OPTIMIZER::AMSGRAD: case OPTIMIZER::ADABOUND:
-    case OPTIMIZER::AMSBOUND: case OPTIMIZER::NOSADAM: break;
-    default: fail("set_optimizer: only GD, ADAM, AMSGRAD, ADABOUND, AMSBOUND and NOSADAM run on the device"); return;
+    case OPTIMIZER::AMSBOUND: case OPTIMIZER::NOSADAM: case OPTIMIZER::IRPROP_PLUS: break;
+    default:
+      fail("set_optimizer: only GD, ADAM, AMSGRAD, ADABOUND, AMSBOUND, NOSADAM and IRPROP_PLUS run on the device");
+      return;
   }
   if (impl_->ctx != nullptr) (void)dlmi_ctx_synchronize(impl_->ctx);
-  for (int i = 0; i < 4; ++i) dev_free(impl_->d_opt[i]);
+  for (int i : {0, 1, 2, 3, 5, 6}) dev_free(impl_->d_opt[i]);
   type_optimizer_function = type_received;
   clear_training_arrays();
 }
@@ -1166,6 +1171,22 @@ void Model::Update_Parameter(size_t const batch, size_t const training_size) {
                              m.d_opt[4], lr_t, adam_beta1, adam_beta2, adam_epsilon, wd, lower, upper);
       break;
     }
+    case OPTIMIZER::IRPROP_PLUS: {
+      // irprop_plus.cpp:33-77.  loss_rprop / loss_rprop_tm1 are kept by the epoch driver
+      // (drivers/driver.cpp:232, 263); no learning rate, no weight decay, no time step.
+      if (!opt_array(&m.d_opt[0], P, m.stream, m.err) || !opt_array(&m.d_opt[5], P, m.stream, m.err)) return;
+      if (m.d_opt[6] == nullptr) {
+        std::vector<float> const steps(P ? P : 1, rprop_delta_zero);  // allocate.cpp / train.cpp:177-182
+        if (!dev_alloc(&m.d_opt[6], P, m.err)) return;
+        if (!hip_ok(hipMemcpy(m.d_opt[6], steps.data(), (P ? P : 1) * sizeof(float), hipMemcpyHostToDevice), m.err,
+                    "step size fill"))
+          return;
+      }
+      rc = dlmi_opt_irprop_plus(m.ctx, P, m.d_params, m.d_dparams, m.d_opt[5], m.d_opt[0], m.d_opt[6],
+                                rprop_increase_factor, rprop_decrease_factor, rprop_delta_min, rprop_delta_max,
+                                loss_rprop > loss_rprop_tm1 ? 1 : 0);
+      break;
+    }
     case OPTIMIZER::NOSADAM: {
       // nosadam.cpp:37-100: Adam whose second-moment decay at step t is B_{t-1} / B_t with
       // B_t = sum_{k<=t} k^-adam_gamma; the bias correction keeps the fixed adam_beta2
@@ -1213,7 +1234,7 @@ bool Model::Set__Regularization__Max_Norm_Constraints(real const v) {
 }
 
 bool Model::download_optimizer_state(int which, float *out) const {
-  if (which < 0 || which > 4 || impl_->d_opt[which] == nullptr || out == nullptr) return false;
+  if (which < 0 || which > 6 || impl_->d_opt[which] == nullptr || out == nullptr) return false;
   return hip_ok(hipMemcpy(out, impl_->d_opt[which], total_parameters * sizeof(float), hipMemcpyDeviceToHost),
                 impl_->err, "optimizer state download");
 }

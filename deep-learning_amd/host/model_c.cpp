@@ -221,6 +221,17 @@ void dlmi_model_set_bound_hyper(dlmi_model *h, float lr_final, float gamma, floa
   h->m.learning_gamma = gamma;
   h->m.adam_gamma = adam_gamma;
 }
+void dlmi_model_set_rprop(dlmi_model *h, float incr, float decr, float delta_min, float delta_max, float delta_zero) {
+  h->m.rprop_increase_factor = incr;
+  h->m.rprop_decrease_factor = decr;
+  h->m.rprop_delta_min = delta_min;
+  h->m.rprop_delta_max = delta_max;
+  h->m.rprop_delta_zero = delta_zero;
+}
+void dlmi_model_set_rprop_loss(dlmi_model *h, double loss, double loss_tm1) {
+  h->m.loss_rprop = loss;
+  h->m.loss_rprop_tm1 = loss_tm1;
+}
 int dlmi_model_set_constraints(dlmi_model *h, int use_clip, float clip, float max_norm) {
   h->m.set_clip_gradient(use_clip != 0);
   if (!h->m.set_clip_gradient(clip)) return 0;

@@ -25,6 +25,7 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_driver_evalt", "dlmi_model_create_typed", "dlmi_model_layer_info", "dlmi_mnist_create",
     "dlmi_mnist_destroy", "dlmi_mnist_load", "dlmi_mnist_last_error", "dlmi_mnist_copy",
     "dlmi_model_glorot_uniform", "dlmi_model_init_uniform", "dlmi_model_set_bound_hyper", "dlmi_model_set_constraints",
+    "dlmi_model_set_rprop", "dlmi_model_set_rprop_loss",
 ]
 
 LAYER_FULLY_CONNECTED, LAYER_RESIDUAL = 3, 9  # v1/data/enum/layer.hpp
@@ -187,8 +188,13 @@ class Model:
     # ---- optimizer (Model::set_optimizer / set_weight_decay / Update_Parameter) ----
     def set_optimizer(self, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9, beta2=0.999,
                       eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True, lr_final=0.1, gamma=1e-3,
-                      adam_gamma=0.1, clip=None, max_norm=0.0):
+                      adam_gamma=0.1, clip=None, max_norm=0.0, rprop=(1.2, 0.5, 1e-6, 50.0, 0.1), rprop_losses=None):
+        """rprop: iRPROP+ (increase, decrease, delta_min, delta_max, delta_zero).  rprop_losses: a recorded
+        sequence of [loss_rprop, loss_rprop_tm1] to install before each update_parameter() call, for callers
+        that drive the updates themselves (train_epoch keeps the two losses on its own)."""
         self.lib.dlmi_model_set_bound_hyper(self.h, c_f(lr_final), c_f(gamma), c_f(adam_gamma))
+        self.lib.dlmi_model_set_rprop(self.h, *(c_f(v) for v in rprop))
+        self._rprop_losses, self._n_updates = rprop_losses, 0
         self._ok(self.lib.dlmi_model_set_constraints(self.h, c_int(int(clip is not None)),
                                                      c_f(1.0 if clip is None else clip), c_f(max_norm)), "constraints")
         self._ok(self.lib.dlmi_model_set_optimizer(self.h, c_int(kind), c_f(lr), c_f(momentum), c_int(int(nesterov)),
@@ -204,6 +210,10 @@ class Model:
         self._ok(self.lib.dlmi_model_set_derivatives(self.h, _ptr(g), c_sz(g.size)), "set_derivatives")
 
     def update_parameter(self, batch, training_size):
+        if getattr(self, "_rprop_losses", None) is not None:
+            loss, loss_tm1 = self._rprop_losses[self._n_updates]
+            self.lib.dlmi_model_set_rprop_loss(self.h, ctypes.c_double(loss), ctypes.c_double(loss_tm1))
+        self._n_updates = getattr(self, "_n_updates", 0) + 1
         self.lib.dlmi_model_update_parameter(self.h, c_sz(batch), c_sz(training_size))
 
     def opt_state(self, which):

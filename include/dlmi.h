@@ -286,6 +286,17 @@ int dlmi_opt_adabound(dlmi_ctx *ctx, size_t n, float *params, float *grads, floa
                       float *m2_hat, float const *mask, float lr_t, float beta1, float beta2,
                       float eps, float wd, float rate_lower, float rate_upper);
 
+/* iRPROP+ (irprop_plus.cpp:33-122): per parameter, with d the gradient, d' the stored
+ * previous one, s the step size and m the previous move:
+ *   d'*d > 0:  s = min(s*increase, step_max); m = -sign(d)*s; p += m; d' = d
+ *   d'*d < 0:  s = max(s*decrease, step_min); if loss_got_worse: p -= m; d' = 0
+ *   else:      m = -sign(d)*s; p += m; d' = d
+ * and the gradient is zeroed.  loss_got_worse is the caller's loss_rprop >
+ * loss_rprop_tm1 (drivers/driver.cpp:232, 263). */
+int dlmi_opt_irprop_plus(dlmi_ctx *ctx, size_t n, float *params, float *grads, float *prev_grads,
+                         float *prev_moves, float *step_sizes, float increase, float decrease,
+                         float step_min, float step_max, int loss_got_worse);
+
 /* ---- Euclidean-norm constraints either side of the optimizer step -----------
  * (euclidean_norm_{st,mp}, v1/ops/constraints/euclidean.cpp:24-62: when the norm
  * is >= max_norm, every element is multiplied by max_norm / norm) */

@@ -68,6 +68,11 @@ int dlmi_model_set_optimizer(dlmi_model *m, int type, float lr, float momentum, 
 /* learning_rate_final, learning_gamma (AdaBound / AMSBound) and adam_gamma (NosAdam): call before
  * dlmi_model_set_optimizer */
 void dlmi_model_set_bound_hyper(dlmi_model *m, float lr_final, float gamma, float adam_gamma);
+/* iRPROP+: rprop_increase_factor, rprop_decrease_factor, rprop_delta_min, rprop_delta_max, rprop_delta_zero
+ * (assign before dlmi_model_set_optimizer); loss_rprop / loss_rprop_tm1 for callers that drive
+ * Update_Parameter themselves (the epoch driver keeps them on its own) */
+void dlmi_model_set_rprop(dlmi_model *m, float incr, float decr, float delta_min, float delta_max, float delta_zero);
+void dlmi_model_set_rprop_loss(dlmi_model *m, double loss, double loss_tm1);
 /* set_clip_gradient(use_clip != 0), set_clip_gradient(clip), Set__Regularization__Max_Norm_Constraints(max_norm) */
 int dlmi_model_set_constraints(dlmi_model *m, int use_clip, float clip, float max_norm);
 void dlmi_model_set_epoch_time_step(dlmi_model *m, float v);

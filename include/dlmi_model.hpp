@@ -27,6 +27,7 @@
 #ifndef DLMI_MODEL_HPP
 #define DLMI_MODEL_HPP
 
+#include <cmath>
 #include <cstddef>
 #include <cstdint>
 #include <random>
@@ -186,9 +187,9 @@ class Model {
 
   // ---- optimizer step (model.hpp:848, 2965; train.cpp:77-104, 278-283;
   //      ops/regularizers/weight_decay.cpp:26-62; model.cpp:4703-4866) ----------
-  // GD (plain, momentum, Nesterov), ADAM, AMSGRAD, ADABOUND, AMSBOUND and NOSADAM
-  // (adabound.cpp, amsbound.cpp, nosadam.cpp) run on the device; the others are
-  // refused.  set_optimizer also clears the training arrays, like the
+  // GD (plain, momentum, Nesterov), ADAM, AMSGRAD, ADABOUND, AMSBOUND, NOSADAM and
+  // IRPROP_PLUS run on the device: every type the reference's update_weights_*
+  // dispatches (model.cpp:4745-4790).  The others are refused, there as here.  set_optimizer also clears the training arrays, like the
   // reference.  Update_Parameter consumes and zeroes the device gradient array.
   void set_optimizer(OPTIMIZER::TYPE const type);
   bool set_weight_decay(real const val);
@@ -254,6 +255,15 @@ class Model {
   real adam_beta1 = 0.9f;
   real adam_beta2 = 0.999f;
   real adam_epsilon = 1e-8f;
+  // iRPROP+ (model.hpp:3331-3335, 2957-2958): factors and limits of the per-parameter step size, its
+  // start value, and the losses of this and of the previous epoch, which the epoch driver keeps
+  real rprop_increase_factor = 1.2f;
+  real rprop_decrease_factor = 0.5f;
+  real rprop_delta_min = 1e-6f;
+  real rprop_delta_max = 50.0f;
+  real rprop_delta_zero = 0.1f;
+  double loss_rprop = HUGE_VAL;
+  double loss_rprop_tm1 = HUGE_VAL;
   bool use_clip_gradient = false;                     // model.hpp:2843
   real clip_gradient = 1.0f;                          // model.hpp:3044
   real regularization__max_norm_constraints = 0.0f;   // model.hpp:3024

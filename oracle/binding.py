@@ -34,7 +34,7 @@ NORM = dict(NONE=0, BN=1, BRN=2)
 DROP = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3)
 STATE = dict(INFERENCE=0, TRAINING=1, UPDATE_BATCH_NORM=2)
 # v1/data/enum/optimizer.hpp:24-42
-OPT = dict(NONE=0, ADABOUND=1, ADAM=2, AMSBOUND=4, AMSGRAD=5, GD=6, NOSADAM=9)
+OPT = dict(NONE=0, ADABOUND=1, ADAM=2, AMSBOUND=4, AMSGRAD=5, GD=6, IRPROP_PLUS=8, NOSADAM=9)
 _ADAM_FAMILY = (1, 2, 4, 5, 9)
 
 
@@ -55,8 +55,20 @@ class OptimizerHost:
 
     def __init__(self, leaves, n, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9,
                  beta2=0.999, eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True, mask=None,
-                 lr_final=0.1, gamma=1e-3, adam_gamma=0.1, clip=None, max_norm=0.0, weight_rows=()):
+                 lr_final=0.1, gamma=1e-3, adam_gamma=0.1, clip=None, max_norm=0.0, weight_rows=(),
+                 rprop=(1.2, 0.5, 1e-6, 50.0, 0.1), rprop_losses=None):
         f = np.float32
+        # iRPROP+: (increase, decrease, delta_min, delta_max, delta_zero), model.hpp:3331-3335.  loss_rprop /
+        # loss_rprop_tm1 are the caller's (drivers/driver.cpp:232, 263); rprop_losses, if given, is the
+        # [loss, loss_tm1] pair to install before each update (for replaying a recorded sequence).
+        self.rprop = tuple(f(v) for v in rprop)
+        self.loss_rprop = self.loss_rprop_tm1 = float(np.finfo(np.float32).max)  # train.cpp:167-168
+        self.rprop_losses, self.n_updates = rprop_losses, 0
+        if kind == OPT["IRPROP_PLUS"]:
+            self.prev_g, self.prev_move = np.zeros(n, np.float32), np.zeros(n, np.float32)
+            self.steps = np.full(n, self.rprop[4], np.float32)
+        else:
+            self.prev_g = self.prev_move = self.steps = None
         # Update_Parameter (model.cpp:4797-4866): [gradient clip] -> optimizer -> [max-norm per unit].
         # weight_rows: (first weight index, units, fan-in) of every fully-connected layer.
         self.clip, self.max_norm, self.weight_rows = clip, f(max_norm), tuple(weight_rows)
@@ -70,6 +82,8 @@ class OptimizerHost:
         self.t = f(0)
         self.epoch_time_step = f(1)
         self.delta = np.zeros(n, np.float32) if kind == OPT["GD"] and self.momentum != 0 else None
+        if kind == OPT["IRPROP_PLUS"]:
+            self.delta = self.prev_move  # the reference keeps it in the same array (previous delta parameters)
         self.m1 = np.zeros(n, np.float32) if kind in _ADAM_FAMILY else None
         self.m2 = np.zeros(n, np.float32) if kind in _ADAM_FAMILY else None
         self.vhat = np.zeros(n, np.float32) if kind in (OPT["AMSGRAD"], OPT["AMSBOUND"]) else None
@@ -95,6 +109,14 @@ class OptimizerHost:
                 self.leaves.max_norm_rows(p[w0:w0 + rows * cols].reshape(rows, cols), self.max_norm, nthreads)
 
     def _step(self, p, g, batch, training_size, nthreads):
+        if self.kind == OPT["IRPROP_PLUS"]:
+            if self.rprop_losses is not None:
+                self.loss_rprop, self.loss_rprop_tm1 = (float(v) for v in self.rprop_losses[self.n_updates])
+            self.n_updates += 1
+            incr, decr, dmin, dmax, _ = self.rprop
+            self.leaves.opt_irprop_plus(p, g, self.prev_g, self.prev_move, self.steps, incr, decr, dmin, dmax,
+                                        self.loss_rprop > self.loss_rprop_tm1, nthreads)
+            return
         self.t = np.float32(self.t + np.float32(1))
         wd = self.wd(batch, training_size)
         if self.kind == OPT["GD"]:
@@ -316,6 +338,11 @@ class Oracle(_Leaves):
                             _ptr(mask), self._real(lr_t), self._real(beta1), self._real(beta2), self._real(eps),
                             self._real(wd))
 
+    def opt_irprop_plus(self, p, g, prev_g, prev_move, steps, incr, decr, step_min, step_max, worse, nthreads=0):
+        self._f("opt_irprop_plus")(c_int(nthreads), c_sz(p.size), _ptr(p), _ptr(g), _ptr(prev_g), _ptr(prev_move),
+                                   _ptr(steps), self._real(incr), self._real(decr), self._real(step_min),
+                                   self._real(step_max), c_int(1 if worse else 0))
+
     def clip_gradient(self, g, max_norm, nthreads=0):
         """euclidean_norm on the whole array, in place."""
         self._f("euclidean_norm")(c_int(nthreads), c_sz(g.size), self._real(max_norm), _ptr(g))
@@ -463,8 +490,13 @@ class OracleMLP:
         X, Y = np.ascontiguousarray(X, np.float32), np.ascontiguousarray(Y, np.float32)
         n = X.shape[0]
         self.lib.dlo_mlp_reset_loss(self.h)
+        irprop = self.opt.kind == OPT["IRPROP_PLUS"]  # drivers/driver.cpp:228-232, 263
+        if irprop:
+            self.opt.loss_rprop_tm1 = self.opt.loss_rprop
         for i, b in self._batches(n):
             self.step(STATE["TRAINING"], X[i:i + b], Y[i:i + b], backward=True)
+        if irprop:
+            self.opt.loss_rprop = abs(self._loss_accu(n)[0])
         self.update_parameter(n, n)
         self.opt.epoch_time_step = np.float32(self.opt.epoch_time_step + np.float32(1))
         return self._loss_accu(n)
@@ -660,8 +692,10 @@ class ReferenceMLP:
     # ---- optimizer (Model::Update_Parameter) ---------------------------------
     def set_optimizer(self, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9, beta2=0.999,
                       eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True, lr_final=0.1, gamma=1e-3,
-                      adam_gamma=0.1, clip=None, max_norm=0.0):
+                      adam_gamma=0.1, clip=None, max_norm=0.0, rprop=(1.2, 0.5, 1e-6, 50.0, 0.1), rprop_losses=None):
         self.lib.dlref_model_set_bound_hyper(self.h, c_f(lr_final), c_f(gamma), c_f(adam_gamma))
+        self.lib.dlref_model_set_rprop(self.h, *(c_f(v) for v in rprop))
+        self._rprop_losses, self._n_updates = rprop_losses, 0
         ok = self.lib.dlref_model_set_constraints(self.h, c_int(int(clip is not None)), c_f(1.0 if clip is None else clip),
                                                   c_f(max_norm))
         assert ok, "reference refused the constraint settings"
@@ -680,11 +714,15 @@ class ReferenceMLP:
         self.lib.dlref_model_set_dparams(self.h, _ptr(g), c_sz(self.P))
 
     def update_parameter(self, batch, training_size):
+        if getattr(self, "_rprop_losses", None) is not None:  # replay of a recorded loss sequence (iRPROP+)
+            loss, loss_tm1 = self._rprop_losses[self._n_updates]
+            self.lib.dlref_model_set_rprop_loss(self.h, c_d(loss), c_d(loss_tm1))
+        self._n_updates = getattr(self, "_n_updates", 0) + 1
         self.lib.dlref_model_update_parameter(self.h, c_sz(batch), c_sz(training_size))
 
     def opt_state(self, which):
-        """which: 0 previous delta, 1 first moment, 2 second moment, 3 second moment hat, 4 regularization mask;
-        None when the reference has not allocated it."""
+        """which: 0 previous delta, 1 first moment, 2 second moment, 3 second moment hat, 4 regularization mask,
+        5 previous gradient, 6 step sizes (iRPROP+); None when the reference has not allocated it."""
         out = np.empty(self.P, np.float32)
         ok = self.lib.dlref_model_get_opt_state(self.h, c_int(which), _ptr(out), c_sz(self.P))
         return out if ok else None

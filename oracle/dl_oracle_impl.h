@@ -400,6 +400,38 @@ void FN(dlo_opt_adabound)(int nthreads, size_t n, REAL *p, REAL *g, REAL *m1, RE
   }
 }
 
+/* iRPROP+: irprop_plus.cpp:33-122.  prev_g the stored previous gradient, prev_move the
+ * previous parameter move, steps the per-parameter step size; worse = loss_rprop >
+ * loss_rprop_tm1 of the caller.  sign as ops/math.hpp:67-70. */
+void FN(dlo_opt_irprop_plus)(int nthreads, size_t n, REAL *p, REAL *g, REAL *prev_g, REAL *prev_move, REAL *steps,
+                             REAL incr, REAL decr, REAL step_min, REAL step_max, int worse) {
+  int const N = nthreads, ni = (int)n;
+  int i;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0)
+  for (i = 0; i < ni; ++i) {
+    REAL const d = g[i];
+    REAL const sgn = (REAL)(((REAL)0 < d) - (d < (REAL)0));
+    if (prev_g[i] * d > (REAL)0) {
+      REAL dt = steps[i] * incr;
+      dt = step_max < dt ? step_max : dt;
+      steps[i] = dt;
+      prev_move[i] = -sgn * dt;
+      p[i] += prev_move[i];
+      prev_g[i] = d;
+    } else if (prev_g[i] * d < (REAL)0) {
+      REAL const dt = steps[i] * decr;
+      steps[i] = dt < step_min ? step_min : dt;
+      if (worse) p[i] -= prev_move[i];
+      prev_g[i] = (REAL)0;
+    } else {
+      prev_move[i] = -sgn * steps[i];
+      p[i] += prev_move[i];
+      prev_g[i] = d;
+    }
+    g[i] = (REAL)0;
+  }
+}
+
 /* euclidean_norm_{st,mp}: v1/ops/constraints/euclidean.cpp:24-62.  Used on the whole
  * gradient array before the optimizer step (clip_gradient.cpp:75-83) and on each
  * unit's fan-in after it (max_norm.cpp:61-78, 278-300). */

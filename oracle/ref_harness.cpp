@@ -741,11 +741,28 @@ int dlref_model_get_opt_state(void *h, int which, float *out, size_t n) {
     case 2: src = m.ptr_array_previous_biased_second_moment; break;
     case 3: src = m.ptr_array_previous_biased_second_moment_hat; break;
     case 4: src = m.ptr_array_mask_regularized_parameters; break;
+    case 5: src = m.ptr_array_previous_derivatives_parameters; break;
+    case 6: src = m.ptr_array_previous_steps; break;
     default: return 0;
   }
   if (src == nullptr) return 0;
   std::memcpy(out, src, n * sizeof(float));
   return 1;
+}
+// iRPROP+: the step-size factors and limits (model.hpp:3331-3335; assign before set_optimizer, which fills
+// the step sizes with rprop_delta_zero) and the two losses Update_Parameter__iRPROP_plus compares
+void dlref_model_set_rprop(void *h, float incr, float decr, float delta_min, float delta_max, float delta_zero) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  m.rprop_increase_factor = incr;
+  m.rprop_decrease_factor = decr;
+  m.rprop_delta_min = delta_min;
+  m.rprop_delta_max = delta_max;
+  m.rprop_delta_zero = delta_zero;
+}
+void dlref_model_set_rprop_loss(void *h, double loss, double loss_tm1) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  m.loss_rprop = loss;
+  m.loss_rprop_tm1 = loss_tm1;
 }
 
 // ---- epoch driver.  Driver (drivers/driver.cpp) cannot be compiled here: its
@@ -771,6 +788,9 @@ void dlref_model_train_epoch(void *h, size_t n_data, float const *X, size_t K0, 
   m.update_mem_batch_size(n_data);
   if (resample_masks && (m.Use__Dropout__Bernoulli() || m.Use__Dropout__Bernoulli__Inverted())) m.Dropout_Bernoulli();
   m.reset_loss();
+  // driver.cpp:228-232, 263 / 269-273, 337: iRPROP compares this epoch's loss with the previous one's
+  bool const irprop = OPTIMIZER::IRPROP_MINUS == m.type_optimizer_function || OPTIMIZER::IRPROP_PLUS == m.type_optimizer_function;
+  if (irprop) m.loss_rprop_tm1 = m.loss_rprop;
   size_t const batch_size_max = m.batch_size;
   int const n_batch = static_cast<int>(std::ceil(static_cast<double>(n_data) / static_cast<double>(batch_size_max)));
   if (m.use_mp && m.is_mp_initialized) {
@@ -788,6 +808,7 @@ void dlref_model_train_epoch(void *h, size_t n_data, float const *X, size_t K0, 
     }
     m.merge_mp_derivatives(0, m.total_parameters);
     m.merge_mp_accu_loss();
+    if (irprop) m.loss_rprop = std::abs(m.get_loss(DL::ENV::NONE));
     m.update_weights_mp(n_data, n_data);
   } else {
     for (int i = 0; i < n_batch; ++i) {
@@ -797,6 +818,7 @@ void dlref_model_train_epoch(void *h, size_t n_data, float const *X, size_t K0, 
       m.backward_pass(batch_size);
       m.update_derivatives(batch_size, m.ptr_array_layers + 1, m.ptr_last_layer);
     }
+    if (irprop) m.loss_rprop = std::abs(m.get_loss(DL::ENV::NONE));
     m.update_weights_st(n_data, n_data);
   }
   m.type_state_propagation = PROPAGATION::INFERENCE;

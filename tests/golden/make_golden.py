@@ -225,6 +225,11 @@ OPT_CASES = {
     "gd_clip_loose": ("GD", dict(lr=0.05, momentum=0.9, clip=40.0)),
     "adam_maxnorm": ("ADAM", dict(adam_lr=0.05, max_norm=2.0)),
     "gd_clip_maxnorm_wd": ("GD", dict(lr=0.1, momentum=0.5, weight_decay=0.02, clip=6.0, max_norm=2.5)),
+    # iRPROP+: [loss, previous loss] installed before each of the four updates (worse on the third);
+    # the second case makes both limits of the step size bind and the loss always worse
+    "irprop_plus": ("IRPROP_PLUS", dict(rprop_losses=[[3e38, 3e38], [0.9, 1.0], [1.1, 0.9], [1.0, 1.1]])),
+    "irprop_plus_limits": ("IRPROP_PLUS", dict(rprop=[3.0, 0.01, 0.02, 0.25, 0.1],
+                                               rprop_losses=[[2.0, 1.0], [3.0, 2.0], [4.0, 3.0], [5.0, 4.0]])),
 }
 OPT_STEPS = 4
 OPT_BATCH, OPT_TRAINING_SIZE = 5, 60
@@ -274,7 +279,7 @@ def optimizers(R):
                 q = f"opt_{name}_t{nt}_s{t}_"
                 d[q + "params"] = M.get_parameters()
                 assert not M.get_dparams().any(), "the reference zeroes the consumed gradient"
-                for which, wn in ((0, "delta"), (1, "m1"), (2, "m2"), (3, "vhat")):
+                for which, wn in ((0, "delta"), (1, "m1"), (2, "m2"), (3, "vhat"), (5, "prev_g"), (6, "steps")):
                     st = M.opt_state(which)
                     if st is not None and t == OPT_STEPS - 1:
                         d[q + wn] = st
@@ -318,6 +323,9 @@ EPOCH_CASES = {
                                dict(lr=0.05, momentum=0.9, nesterov=True)),
     "epoch_gd_even_batches": ([10, 8, 8, 4], 48, 12, [("SELU", "BN", "NONE", 1.0), ("ISRLU", "BN", "NONE", 1.0)], "GD",
                               dict(lr=0.1, momentum=0.0, weight_decay=0.02, normalized_wd=False)),
+    # iRPROP+ with the epoch driver keeping the two losses; a start step large enough for the loss to get worse
+    "epoch_irprop_plus": ([10, 8, 8, 4], 40, 16, [("ELU", "BRN", "NONE", 1.0), ("RELU", "NONE", "NONE", 1.0)], "IRPROP_PLUS",
+                          dict(rprop=[1.2, 0.5, 1e-6, 50.0, 0.3])),
 }
 EPOCHS = 3
 

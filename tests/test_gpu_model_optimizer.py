@@ -63,7 +63,7 @@ def test_update_parameter_against_golden(model_factory, golden_optim, name):
         assert_close(M.get_parameters(), g[f"opt_{name}_t0_s{t}_params"], TE, f"{name} parameters after step {t}")
         assert not M.get_dparams().any(), "Update_Parameter zeroes the gradient array"
     q = f"opt_{name}_t0_s{steps - 1}_"
-    for which, key in ((0, "delta"), (1, "m1"), (2, "m2"), (3, "vhat")):
+    for which, key in ((0, "delta"), (1, "m1"), (2, "m2"), (3, "vhat"), (5, "prev_g"), (6, "steps")):
         if q + key in g.files:
             assert_close(M.opt_state(which), g[q + key], TE, f"{name} {key}")
 
@@ -93,4 +93,4 @@ def test_training_trajectory_against_golden(model_factory, golden_optim, name):
 def test_unsupported_optimizer_is_refused(model_factory):
     M = model_factory([8, 6, 6, 3], 4)
     with pytest.raises(Exception):
-        M.set_optimizer(8)  # iRPROP+
+        M.set_optimizer(7)  # iRPROP-: the reference's Update_Parameter does not dispatch it either

@@ -38,6 +38,10 @@ class GpuLeaves:
         self._run(self.dl.opt_adam, [p, g, m1, m2, vhat, mask], float(lr_t), float(b1), float(b2), float(eps),
                   float(wd))
 
+    def opt_irprop_plus(self, p, g, prev_g, prev_move, steps, incr, decr, step_min, step_max, worse, nthreads=0):
+        self._run(self.dl.opt_irprop_plus, [p, g, prev_g, prev_move, steps], float(incr), float(decr), float(step_min),
+                  float(step_max), bool(worse))
+
     def clip_gradient(self, g, max_norm, nthreads=0):
         self._run(self.dl.clip_gradient, [g], float(max_norm))
 
@@ -62,7 +66,8 @@ def test_gpu_optimizer_against_golden(dl, golden_optim, name):
     for t, p, host in run_leaf_case(GpuLeaves(dl), g, name, 0):
         assert_close(p, g[f"opt_{name}_t0_s{t}_params"], TE, f"{name} parameters after step {t}")
     q = f"opt_{name}_t0_s{len(g['opt_grads']) - 1}_"
-    for key, arr in (("delta", host.delta), ("m1", host.m1), ("m2", host.m2), ("vhat", host.vhat)):
+    for key, arr in (("delta", host.delta), ("m1", host.m1), ("m2", host.m2), ("vhat", host.vhat),
+                     ("prev_g", host.prev_g), ("steps", host.steps)):
         if q + key in g.files:
             assert_close(arr, g[q + key], TE, f"{name} {key}")
 
@@ -77,6 +82,7 @@ def test_gpu_optimizer_against_golden(dl, golden_optim, name):
     ("ADABOUND", dict(adam_lr=0.01, lr_final=0.05, gamma=0.5, weight_decay=0.05)),
     ("AMSBOUND", dict(adam_lr=0.01, beta2=0.9, lr_final=0.02, gamma=0.3)),
     ("NOSADAM", dict(adam_lr=0.01, adam_gamma=0.1, weight_decay=0.02, normalized_wd=False)),
+    ("IRPROP_PLUS", dict(rprop=[1.5, 0.4, 0.01, 0.3, 0.1], rprop_losses=[[2.0, 1.0], [1.0, 2.0], [3.0, 1.0]])),
 ])
 def test_gpu_optimizer_against_oracle(dl, oracle, n, kind, kw):
     rng = np.random.default_rng(n + len(kind))

@@ -53,7 +53,8 @@ def test_oracle_optimizer_against_golden(oracle, golden_optim, name, nt):
     for t, p, host in run_leaf_case(oracle, g, name, nt):
         assert_close(p, g[f"opt_{name}_t{nt}_s{t}_params"], T, f"{name} parameters after step {t}")
     q = f"opt_{name}_t{nt}_s{len(g['opt_grads']) - 1}_"
-    for key, arr in (("delta", host.delta), ("m1", host.m1), ("m2", host.m2), ("vhat", host.vhat)):
+    for key, arr in (("delta", host.delta), ("m1", host.m1), ("m2", host.m2), ("vhat", host.vhat),
+                     ("prev_g", host.prev_g), ("steps", host.steps)):
         if q + key in g.files:
             assert arr is not None, key
             assert_close(arr, g[q + key], T, f"{name} {key}")
@@ -199,6 +200,39 @@ def test_nosadam_weights_the_past_by_a_hyper_harmonic_series(oracle64):
         host.update(p, gk.copy(), 1, 1)
     w = np.arange(1, steps + 1, dtype=np.float64) ** -gamma
     np.testing.assert_allclose(host.m2, (w[:, None] * gs * gs).sum(0) / w.sum(), rtol=1e-5)  # host scalars are float
+
+
+def test_irprop_plus_by_hand(oracle64):
+    """Four parameters through three calls, every branch, worked by hand (Igel & Hüsken 2000,
+    iRPROP+): increase 1.2, decrease 0.5, step in [0.01, 0.13], start 0.1."""
+    p = np.array([1.0, 1.0, 1.0, 1.0])
+    prev_g, move, steps = np.zeros(4), np.zeros(4), np.full(4, 0.1)
+    args = (1.2, 0.5, 0.01, 0.13)
+    # call 1: no history -> plain step of the start size against the sign; zero gradient -> no move
+    g = np.array([2.0, -3.0, 0.0, 5.0])
+    oracle64.opt_irprop_plus(p, g, prev_g, move, steps, *args, False)
+    np.testing.assert_allclose(p, [0.9, 1.1, 1.0, 0.9], rtol=1e-15)
+    np.testing.assert_allclose(prev_g, [2.0, -3.0, 0.0, 5.0])
+    assert not g.any()
+    # call 2: same sign -> step 0.12; flipped sign with a worse loss -> last move taken back, step halved,
+    # stored gradient cleared; zero history -> plain step; flipped sign again
+    g = np.array([1.0, 4.0, -1.0, -2.0])
+    oracle64.opt_irprop_plus(p, g, prev_g, move, steps, *args, True)
+    np.testing.assert_allclose(p, [0.9 - 0.12, 1.0, 1.1, 1.0], rtol=1e-15)
+    np.testing.assert_allclose(steps, [0.12, 0.05, 0.1, 0.05], rtol=1e-15)
+    np.testing.assert_allclose(prev_g, [1.0, 0.0, -1.0, 0.0])
+    # call 3: same sign -> 0.144 capped at 0.13; cleared history -> plain step of 0.05; same sign -> 0.12;
+    # cleared history and a loss that did not get worse
+    g = np.array([0.5, 4.0, -7.0, -2.0])
+    oracle64.opt_irprop_plus(p, g, prev_g, move, steps, *args, False)
+    np.testing.assert_allclose(p, [0.78 - 0.13, 1.0 - 0.05, 1.1 + 0.12, 1.0 + 0.05], rtol=1e-15)
+    np.testing.assert_allclose(steps, [0.13, 0.05, 0.12, 0.05], rtol=1e-15)
+    # a flip without a worse loss leaves the parameter where it is, and the lower limit binds
+    steps[:] = 0.015
+    prev_g[:] = 1.0
+    before = p.copy()
+    oracle64.opt_irprop_plus(p, np.full(4, -1.0), prev_g, move, steps, *args, False)
+    assert np.array_equal(p, before) and np.allclose(steps, 0.01) and not prev_g.any()
 
 
 def test_euclidean_norm_constraint_closed_form(oracle64, reference):
