@@ -12,6 +12,7 @@
 // input included) | beta(all layers) ],  W_l row-major [H_l][K_l].
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -537,7 +538,13 @@ void Model::clear_training_arrays(void) {
   (void)hipMemsetAsync(impl_->d_stats, 0, 2 * sizeof(double), impl_->stream);
   impl_->n_loss_examples = 0;
   std::memset(ptr_array_derivatives_parameters, 0, total_parameters * sizeof(real));
-  // Clear_Optimizer (train.cpp:136-248): the optimizer's own arrays and its clocks
+  Clear_Optimizer();
+  warm_restarts_maximum_learning_rate = warm_restarts_initial_maximum_learning_rate;  // train.cpp:130-132
+  warm_restarts_T_i = warm_restarts_initial_T_i;
+}
+
+// train.cpp:136-248: the optimizer's own arrays and its clocks
+void Model::Clear_Optimizer(void) {
   for (int i : {0, 1, 2, 3, 5})
     if (impl_->d_opt[i] != nullptr) (void)hipMemsetAsync(impl_->d_opt[i], 0, total_parameters * sizeof(float), impl_->stream);
   dev_free(impl_->d_opt[6]);  // the step sizes start from rprop_delta_zero again: refilled on the next use
@@ -545,6 +552,24 @@ void Model::clear_training_arrays(void) {
   epoch_time_step = 1.0f;
   adam_previous_beta2 = 0.0f;
   loss_rprop = loss_rprop_tm1 = static_cast<double>(std::numeric_limits<real>::max());  // train.cpp:167-168
+}
+
+// Cosine annealing with warm restarts (train.cpp:250-275; Loshchilov & Hutter, SGDR): the learning rate
+// of the step about to be taken.  When the period is over the optimizer starts afresh, the period is
+// stretched by warm_restarts_multiplier and the peak rate decays (never below the minimum).
+real Model::warm_restarts_decay(void) {
+  real const pi = 3.14159265358979323846f;
+  real const lr_decayed =
+      warm_restarts_minimum_learning_rate +
+      0.5f * (warm_restarts_maximum_learning_rate - warm_restarts_minimum_learning_rate) *
+          (1.0f + std::cos(optimizer_time_step / warm_restarts_T_i * pi));
+  if (optimizer_time_step >= warm_restarts_T_i) {
+    Clear_Optimizer();
+    warm_restarts_T_i *= warm_restarts_multiplier;
+    warm_restarts_maximum_learning_rate *= warm_restarts_decay_learning_rate;
+    warm_restarts_maximum_learning_rate = std::max(warm_restarts_maximum_learning_rate, warm_restarts_minimum_learning_rate);
+  }
+  return lr_decayed;
 }
 
 // ---------------------------------------------------------------- buffer movement
@@ -1112,10 +1137,16 @@ real Model::normalized_wd(size_t const batch, size_t const training_size) {
 // adam.cpp:38-54 in float.
 void Model::Update_Parameter(size_t const batch, size_t const training_size) {
   if (impl_->d_params == nullptr) { fail("Update_Parameter: model not compiled"); return; }
-  if (use_warm_restarts) { fail("Update_Parameter: warm restarts are not implemented"); return; }
   size_t const P = total_parameters;
   Impl &m = *impl_;
-  real const wd = use_normalized_weight_decay ? normalized_wd(batch, training_size) : weight_decay;
+  // Every optimizer but iRPROP+ starts by asking the warm-restart schedule for its rate (which may
+  // restart the optimizer, clocks included), then reads the weight decay; gradient descent scales the
+  // decay by the same factor, the Adam family does not (gradient_descent.cpp:66-75, adam.cpp:38-49).
+  bool const gd = type_optimizer_function == OPTIMIZER::GD;
+  bool const scheduled = use_warm_restarts && type_optimizer_function != OPTIMIZER::IRPROP_PLUS &&
+                         type_optimizer_function != OPTIMIZER::NONE;
+  real const lr_scale = scheduled ? warm_restarts_decay() / (gd ? learning_rate : adam_learning_rate) : 1.0f;
+  real const wd = (gd ? lr_scale : 1.0f) * (use_normalized_weight_decay ? normalized_wd(batch, training_size) : weight_decay);
   if (wd != 0.0f && m.d_opt[4] == nullptr && !set_weight_decay(weight_decay)) return;
   int rc = DLMI_OK;
   // update_weights_{st,mp} (model.cpp:4711-4866) clip the gradient first.  (The L1 / L2 terms those
@@ -1128,12 +1159,13 @@ void Model::Update_Parameter(size_t const batch, size_t const training_size) {
   switch (type_optimizer_function) {
     case OPTIMIZER::GD: {
       optimizer_time_step += 1.0f;
+      real const lr = lr_scale * learning_rate;
       if (learning_momentum != 0.0f) {
         if (!opt_array(&m.d_opt[0], P, m.stream, m.err)) return;
-        rc = dlmi_opt_gd_momentum(m.ctx, P, m.d_params, m.d_dparams, m.d_opt[0], m.d_opt[4], learning_rate,
-                                  learning_momentum, wd, use_nesterov ? 1 : 0);
+        rc = dlmi_opt_gd_momentum(m.ctx, P, m.d_params, m.d_dparams, m.d_opt[0], m.d_opt[4], lr, learning_momentum, wd,
+                                  use_nesterov ? 1 : 0);
       } else {
-        rc = dlmi_opt_gd(m.ctx, P, m.d_params, m.d_dparams, m.d_opt[4], learning_rate, wd);
+        rc = dlmi_opt_gd(m.ctx, P, m.d_params, m.d_dparams, m.d_opt[4], lr, wd);
       }
       break;
     }
@@ -1143,7 +1175,7 @@ void Model::Update_Parameter(size_t const batch, size_t const training_size) {
       bool const ams = type_optimizer_function == OPTIMIZER::AMSGRAD;
       if (!opt_array(&m.d_opt[1], P, m.stream, m.err) || !opt_array(&m.d_opt[2], P, m.stream, m.err)) return;
       if (ams && !opt_array(&m.d_opt[3], P, m.stream, m.err)) return;
-      real const lr = adam_learning_rate;
+      real const lr = lr_scale * adam_learning_rate;
       real const lr_t = use_adam_bias_correction
                             ? lr * std::sqrt(1.0f - std::pow(adam_beta2, optimizer_time_step)) /
                                   (1.0f - std::pow(adam_beta1, optimizer_time_step))
@@ -1160,9 +1192,9 @@ void Model::Update_Parameter(size_t const batch, size_t const training_size) {
       bool const ams = type_optimizer_function == OPTIMIZER::AMSBOUND;
       if (!opt_array(&m.d_opt[1], P, m.stream, m.err) || !opt_array(&m.d_opt[2], P, m.stream, m.err)) return;
       if (ams && !opt_array(&m.d_opt[3], P, m.stream, m.err)) return;
-      real const lr = adam_learning_rate;
-      real const lower = learning_rate_final * (1.0f - 1.0f / (learning_gamma * optimizer_time_step + 1.0f));
-      real const upper = learning_rate_final * (1.0f + 1.0f / (learning_gamma * optimizer_time_step));
+      real const lr = lr_scale * adam_learning_rate;
+      real const lower = lr_scale * learning_rate_final * (1.0f - 1.0f / (learning_gamma * optimizer_time_step + 1.0f));
+      real const upper = lr_scale * learning_rate_final * (1.0f + 1.0f / (learning_gamma * optimizer_time_step));
       real const lr_t = use_adam_bias_correction
                             ? lr * std::sqrt(1.0f - std::pow(adam_beta2, optimizer_time_step)) /
                                   (1.0f - std::pow(adam_beta1, optimizer_time_step))
@@ -1192,7 +1224,7 @@ void Model::Update_Parameter(size_t const batch, size_t const training_size) {
       // B_t = sum_{k<=t} k^-adam_gamma; the bias correction keeps the fixed adam_beta2
       optimizer_time_step += 1.0f;
       if (!opt_array(&m.d_opt[1], P, m.stream, m.err) || !opt_array(&m.d_opt[2], P, m.stream, m.err)) return;
-      real const lr = adam_learning_rate;
+      real const lr = lr_scale * adam_learning_rate;
       real const beta2_at_power_gamma = std::pow(optimizer_time_step, -adam_gamma);
       real const beta2_at_time_t = adam_previous_beta2 / (adam_previous_beta2 + beta2_at_power_gamma);
       real const lr_t = use_adam_bias_correction

@@ -221,6 +221,16 @@ void dlmi_model_set_bound_hyper(dlmi_model *h, float lr_final, float gamma, floa
   h->m.learning_gamma = gamma;
   h->m.adam_gamma = adam_gamma;
 }
+void dlmi_model_set_warm_restarts(dlmi_model *h, int use, float decay_lr, float max_lr, float min_lr, float t_i,
+                                  float multiplier) {
+  Model &m = h->m;
+  m.use_warm_restarts = use != 0;
+  m.warm_restarts_decay_learning_rate = decay_lr;
+  m.warm_restarts_initial_maximum_learning_rate = m.warm_restarts_maximum_learning_rate = max_lr;
+  m.warm_restarts_minimum_learning_rate = min_lr;
+  m.warm_restarts_initial_T_i = m.warm_restarts_T_i = t_i;
+  m.warm_restarts_multiplier = multiplier;
+}
 void dlmi_model_set_rprop(dlmi_model *h, float incr, float decr, float delta_min, float delta_max, float delta_zero) {
   h->m.rprop_increase_factor = incr;
   h->m.rprop_decrease_factor = decr;

@@ -25,7 +25,7 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_driver_evalt", "dlmi_model_create_typed", "dlmi_model_layer_info", "dlmi_mnist_create",
     "dlmi_mnist_destroy", "dlmi_mnist_load", "dlmi_mnist_last_error", "dlmi_mnist_copy",
     "dlmi_model_glorot_uniform", "dlmi_model_init_uniform", "dlmi_model_set_bound_hyper", "dlmi_model_set_constraints",
-    "dlmi_model_set_rprop", "dlmi_model_set_rprop_loss",
+    "dlmi_model_set_rprop", "dlmi_model_set_rprop_loss", "dlmi_model_set_warm_restarts",
 ]
 
 LAYER_FULLY_CONNECTED, LAYER_RESIDUAL = 3, 9  # v1/data/enum/layer.hpp
@@ -188,10 +188,14 @@ class Model:
     # ---- optimizer (Model::set_optimizer / set_weight_decay / Update_Parameter) ----
     def set_optimizer(self, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9, beta2=0.999,
                       eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True, lr_final=0.1, gamma=1e-3,
-                      adam_gamma=0.1, clip=None, max_norm=0.0, rprop=(1.2, 0.5, 1e-6, 50.0, 0.1), rprop_losses=None):
+                      adam_gamma=0.1, clip=None, max_norm=0.0, rprop=(1.2, 0.5, 1e-6, 50.0, 0.1), rprop_losses=None,
+                      warm_restarts=None):
         """rprop: iRPROP+ (increase, decrease, delta_min, delta_max, delta_zero).  rprop_losses: a recorded
         sequence of [loss_rprop, loss_rprop_tm1] to install before each update_parameter() call, for callers
-        that drive the updates themselves (train_epoch keeps the two losses on its own)."""
+        that drive the updates themselves (train_epoch keeps the two losses on its own).  warm_restarts: None
+        or (decay of the peak rate, peak rate, floor, first period in steps, period multiplier)."""
+        wr = warm_restarts or (1.0, 1.0, 1e-7, 1.0, 2.0)
+        self.lib.dlmi_model_set_warm_restarts(self.h, c_int(int(warm_restarts is not None)), *(c_f(v) for v in wr))
         self.lib.dlmi_model_set_bound_hyper(self.h, c_f(lr_final), c_f(gamma), c_f(adam_gamma))
         self.lib.dlmi_model_set_rprop(self.h, *(c_f(v) for v in rprop))
         self._rprop_losses, self._n_updates = rprop_losses, 0

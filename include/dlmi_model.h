@@ -68,6 +68,11 @@ int dlmi_model_set_optimizer(dlmi_model *m, int type, float lr, float momentum, 
 /* learning_rate_final, learning_gamma (AdaBound / AMSBound) and adam_gamma (NosAdam): call before
  * dlmi_model_set_optimizer */
 void dlmi_model_set_bound_hyper(dlmi_model *m, float lr_final, float gamma, float adam_gamma);
+/* use_warm_restarts and the warm_restarts_* members (cosine annealing with warm restarts, train.cpp:250-275):
+ * decay of the peak rate per period, peak and floor of the rate, first period in optimizer steps, stretch of
+ * the period.  Call before dlmi_model_set_optimizer. */
+void dlmi_model_set_warm_restarts(dlmi_model *m, int use, float decay_lr, float max_lr, float min_lr, float t_i,
+                                  float multiplier);
 /* iRPROP+: rprop_increase_factor, rprop_decrease_factor, rprop_delta_min, rprop_delta_max, rprop_delta_zero
  * (assign before dlmi_model_set_optimizer); loss_rprop / loss_rprop_tm1 for callers that drive
  * Update_Parameter themselves (the epoch driver keeps them on its own) */

@@ -195,6 +195,8 @@ class Model {
   bool set_weight_decay(real const val);
   real normalized_wd(size_t const batch_size, size_t const training_size);
   void Update_Parameter(size_t const batch_size, size_t const training_size);
+  void Clear_Optimizer(void);      // train.cpp:136-248
+  real warm_restarts_decay(void);  // train.cpp:250-275
   // The Euclidean-norm constraints Update_Parameter applies around the step
   // (model.cpp:4797-4866): the whole gradient array is scaled onto the ball of
   // radius clip_gradient before it (v1/ops/constraints/clip_gradient.cpp:30-83),
@@ -247,7 +249,15 @@ class Model {
   bool use_nesterov = false;
   bool use_normalized_weight_decay = true;
   bool use_adam_bias_correction = true;
-  bool use_warm_restarts = false;  // warm restarts are not implemented: Update_Parameter refuses them
+  // cosine annealing with warm restarts (model.hpp:2838, 3037-3043; train.cpp:250-275)
+  bool use_warm_restarts = false;
+  real warm_restarts_decay_learning_rate = 1.0f;
+  real warm_restarts_initial_maximum_learning_rate = 1.0f;
+  real warm_restarts_maximum_learning_rate = 1.0f;
+  real warm_restarts_minimum_learning_rate = 1e-7f;
+  real warm_restarts_initial_T_i = 1.0f;
+  real warm_restarts_T_i = 1.0f;
+  real warm_restarts_multiplier = 2.0f;
   real learning_rate = 0.01f;
   real learning_momentum = 0.9f;
   real weight_decay = 0.0f;

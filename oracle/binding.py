@@ -56,8 +56,11 @@ class OptimizerHost:
     def __init__(self, leaves, n, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9,
                  beta2=0.999, eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True, mask=None,
                  lr_final=0.1, gamma=1e-3, adam_gamma=0.1, clip=None, max_norm=0.0, weight_rows=(),
-                 rprop=(1.2, 0.5, 1e-6, 50.0, 0.1), rprop_losses=None):
+                 rprop=(1.2, 0.5, 1e-6, 50.0, 0.1), rprop_losses=None, warm_restarts=None):
         f = np.float32
+        # warm_restarts: None or (decay of the peak rate, peak rate, floor, first period, period multiplier)
+        self.wr = None if warm_restarts is None else dict(zip(("decay", "max", "min", "T", "mult"),
+                                                              (f(v) for v in warm_restarts)))
         # iRPROP+: (increase, decrease, delta_min, delta_max, delta_zero), model.hpp:3331-3335.  loss_rprop /
         # loss_rprop_tm1 are the caller's (drivers/driver.cpp:232, 263); rprop_losses, if given, is the
         # [loss, loss_tm1] pair to install before each update (for replaying a recorded sequence).
@@ -94,11 +97,34 @@ class OptimizerHost:
             return f(self.weight_decay * np.sqrt(f(f(batch) / f(f(training_size) * self.epoch_time_step))))
         return self.weight_decay
 
-    def lr_t(self):
+    def lr_t(self, lr_scale=np.float32(1)):
         f = np.float32
+        lr = f(lr_scale * self.adam_lr)
         if not self.bias_correction:
-            return self.adam_lr
-        return f(f(self.adam_lr * np.sqrt(f(f(1) - np.power(self.beta2, self.t)))) / f(f(1) - np.power(self.beta1, self.t)))
+            return lr
+        return f(f(lr * np.sqrt(f(f(1) - np.power(self.beta2, self.t)))) / f(f(1) - np.power(self.beta1, self.t)))
+
+    def clear(self):
+        """Clear_Optimizer, train.cpp:136-248."""
+        f = np.float32
+        for a in (self.delta, self.m1, self.m2, self.vhat, self.prev_g):
+            if a is not None:
+                a[...] = 0
+        if self.steps is not None:
+            self.steps[...] = self.rprop[4]
+        self.t, self.epoch_time_step, self.previous_beta2 = f(0), f(1), f(0)
+
+    def warm_restarts_decay(self):
+        """train.cpp:250-275: cosine annealing of the rate over a period of T_i steps; at the end of the
+        period the optimizer restarts, the period stretches and the peak rate decays."""
+        f = np.float32
+        w = self.wr
+        lr = f(w["min"] + f(f(f(0.5) * f(w["max"] - w["min"])) * f(f(1) + np.cos(f(f(self.t / w["T"]) * f(np.pi))))))
+        if self.t >= w["T"]:
+            self.clear()
+            w["T"] = f(w["T"] * w["mult"])
+            w["max"] = max(f(w["max"] * w["decay"]), w["min"])
+        return lr
 
     def update(self, p, g, batch, training_size, nthreads=0):
         if self.clip is not None:
@@ -117,20 +143,26 @@ class OptimizerHost:
             self.leaves.opt_irprop_plus(p, g, self.prev_g, self.prev_move, self.steps, incr, decr, dmin, dmax,
                                         self.loss_rprop > self.loss_rprop_tm1, nthreads)
             return
+        # every one of these asks the warm-restart schedule first (it may restart the optimizer, clocks
+        # included), then advances the time step and reads the weight decay; gradient descent scales the decay
+        # by the same factor, the Adam family does not (gradient_descent.cpp:66-75, adam.cpp:38-49)
+        f = np.float32
+        gd = self.kind == OPT["GD"]
+        scale = f(self.warm_restarts_decay() / (self.lr if gd else self.adam_lr)) if self.wr is not None else f(1)
         self.t = np.float32(self.t + np.float32(1))
         wd = self.wd(batch, training_size)
-        if self.kind == OPT["GD"]:
+        if gd:
+            lr, wd = f(scale * self.lr), f(scale * wd)
             if self.momentum != 0:
-                self.leaves.opt_gd_momentum(p, g, self.delta, self.mask, self.lr, self.momentum, wd, self.nesterov,
-                                            nthreads)
+                self.leaves.opt_gd_momentum(p, g, self.delta, self.mask, lr, self.momentum, wd, self.nesterov, nthreads)
             else:
-                self.leaves.opt_gd(p, g, self.mask, self.lr, wd, nthreads)
+                self.leaves.opt_gd(p, g, self.mask, lr, wd, nthreads)
         elif self.kind in (OPT["ADABOUND"], OPT["AMSBOUND"]):
             # adabound.cpp:49-55: the band closes on learning_rate_final as the time step grows
             f, one = np.float32, np.float32(1)
-            lower = f(self.lr_final * f(one - f(one / f(f(self.gamma * self.t) + one))))
-            upper = f(self.lr_final * f(one + f(one / f(self.gamma * self.t))))
-            self.leaves.opt_adabound(p, g, self.m1, self.m2, self.vhat, self.mask, self.lr_t(), self.beta1, self.beta2,
+            lower = f(f(scale * self.lr_final) * f(one - f(one / f(f(self.gamma * self.t) + one))))
+            upper = f(f(scale * self.lr_final) * f(one + f(one / f(self.gamma * self.t))))
+            self.leaves.opt_adabound(p, g, self.m1, self.m2, self.vhat, self.mask, self.lr_t(scale), self.beta1, self.beta2,
                                      self.eps, wd, lower, upper, nthreads)
         elif self.kind == OPT["NOSADAM"]:
             # nosadam.cpp:49-52, 68: the second-moment decay of step t is B_{t-1} / B_t with
@@ -139,10 +171,10 @@ class OptimizerHost:
             term = f(np.power(self.t, f(-self.adam_gamma)))
             beta2_t = f(self.previous_beta2 / f(self.previous_beta2 + term))
             self.previous_beta2 = f(self.previous_beta2 + term)
-            self.leaves.opt_adam(p, g, self.m1, self.m2, None, self.mask, self.lr_t(), self.beta1, beta2_t, self.eps, wd,
+            self.leaves.opt_adam(p, g, self.m1, self.m2, None, self.mask, self.lr_t(scale), self.beta1, beta2_t, self.eps, wd,
                                  nthreads)
         else:
-            self.leaves.opt_adam(p, g, self.m1, self.m2, self.vhat, self.mask, self.lr_t(), self.beta1, self.beta2,
+            self.leaves.opt_adam(p, g, self.m1, self.m2, self.vhat, self.mask, self.lr_t(scale), self.beta1, self.beta2,
                                  self.eps, wd, nthreads)
 
 
@@ -692,7 +724,11 @@ class ReferenceMLP:
     # ---- optimizer (Model::Update_Parameter) ---------------------------------
     def set_optimizer(self, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9, beta2=0.999,
                       eps=1e-8, bias_correction=True, weight_decay=0.0, normalized_wd=True, lr_final=0.1, gamma=1e-3,
-                      adam_gamma=0.1, clip=None, max_norm=0.0, rprop=(1.2, 0.5, 1e-6, 50.0, 0.1), rprop_losses=None):
+                      adam_gamma=0.1, clip=None, max_norm=0.0, rprop=(1.2, 0.5, 1e-6, 50.0, 0.1), rprop_losses=None,
+                      warm_restarts=None):
+        """warm_restarts: None or (decay of the peak rate, peak rate, floor, first period, period multiplier)."""
+        wr = warm_restarts or (1.0, 1.0, 1e-7, 1.0, 2.0)
+        self.lib.dlref_model_set_warm_restarts(self.h, c_int(int(warm_restarts is not None)), *(c_f(v) for v in wr))
         self.lib.dlref_model_set_bound_hyper(self.h, c_f(lr_final), c_f(gamma), c_f(adam_gamma))
         self.lib.dlref_model_set_rprop(self.h, *(c_f(v) for v in rprop))
         self._rprop_losses, self._n_updates = rprop_losses, 0

@@ -689,7 +689,6 @@ int dlref_model_set_optimizer(void *h, int type, float lr, float momentum, int n
   m.adam_epsilon = eps;
   m.use_adam_bias_correction = bias_correction != 0;
   m.use_normalized_weight_decay = normalized_wd != 0;
-  m.use_warm_restarts = false;
   m.optimizer_time_step = 0.0f;
   m.epoch_time_step = 1.0f;
   m.set_optimizer(static_cast<OPTIMIZER::TYPE>(type));
@@ -758,6 +757,17 @@ void dlref_model_set_rprop(void *h, float incr, float decr, float delta_min, flo
   m.rprop_delta_min = delta_min;
   m.rprop_delta_max = delta_max;
   m.rprop_delta_zero = delta_zero;
+}
+// cosine annealing with warm restarts: use_warm_restarts and the warm_restarts_* members (model.hpp:3037-3043)
+void dlref_model_set_warm_restarts(void *h, int use, float decay_lr, float max_lr, float min_lr, float t_i,
+                                   float multiplier) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  m.use_warm_restarts = use != 0;
+  m.warm_restarts_decay_learning_rate = decay_lr;
+  m.warm_restarts_initial_maximum_learning_rate = m.warm_restarts_maximum_learning_rate = max_lr;
+  m.warm_restarts_minimum_learning_rate = min_lr;
+  m.warm_restarts_initial_T_i = m.warm_restarts_T_i = t_i;
+  m.warm_restarts_multiplier = multiplier;
 }
 void dlref_model_set_rprop_loss(void *h, double loss, double loss_tm1) {
   Model &m = static_cast<RefModel *>(h)->model;

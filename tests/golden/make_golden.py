@@ -225,6 +225,13 @@ OPT_CASES = {
     "gd_clip_loose": ("GD", dict(lr=0.05, momentum=0.9, clip=40.0)),
     "adam_maxnorm": ("ADAM", dict(adam_lr=0.05, max_norm=2.0)),
     "gd_clip_maxnorm_wd": ("GD", dict(lr=0.1, momentum=0.5, weight_decay=0.02, clip=6.0, max_norm=2.5)),
+    # cosine annealing with warm restarts, (decay of the peak, peak, floor, first period, multiplier): a period
+    # of two steps, so the four updates see the peak, the middle, the floor + restart, and the stretched period
+    "gd_warm_restarts": ("GD", dict(lr=0.05, momentum=0.9, weight_decay=0.02, normalized_wd=False,
+                                    warm_restarts=[0.5, 0.08, 0.001, 2.0, 2.0])),
+    "adam_warm_restarts": ("ADAM", dict(adam_lr=0.01, weight_decay=0.01, warm_restarts=[0.7, 0.02, 1e-4, 2.0, 1.5])),
+    "amsbound_warm_restarts": ("AMSBOUND", dict(adam_lr=0.005, beta2=0.9, lr_final=0.02, gamma=0.3,
+                                                warm_restarts=[1.0, 0.01, 1e-3, 3.0, 2.0])),
     # iRPROP+: [loss, previous loss] installed before each of the four updates (worse on the third);
     # the second case makes both limits of the step size bind and the loss always worse
     "irprop_plus": ("IRPROP_PLUS", dict(rprop_losses=[[3e38, 3e38], [0.9, 1.0], [1.1, 0.9], [1.0, 1.1]])),

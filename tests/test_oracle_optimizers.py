@@ -202,6 +202,33 @@ def test_nosadam_weights_the_past_by_a_hyper_harmonic_series(oracle64):
     np.testing.assert_allclose(host.m2, (w[:, None] * gs * gs).sum(0) / w.sum(), rtol=1e-5)  # host scalars are float
 
 
+def test_warm_restart_schedule_is_sgdr():
+    """The rates handed to the leaf over 14 steps with a first period of 2 steps, multiplier 2 and a peak
+    decaying by 0.5: eta_min + (eta_max - eta_min)(1 + cos(pi t / T)) / 2 (Loshchilov & Hutter 2017, eq. 5),
+    the step that finds t == T taking the floor and restarting the clock, which the same call then advances
+    to 1: the first period takes t = 0..2, the later ones t = 1..T (their peak itself is never visited)."""
+    class Recorder:
+        def __init__(self):
+            self.rates = []
+
+        def opt_gd(self, p, g, mask, lr, wd, nthreads=0):
+            self.rates.append(float(lr))
+
+    rec = Recorder()
+    host = OptimizerHost(rec, 1, OPT["GD"], lr=0.05, momentum=0.0, warm_restarts=(0.5, 0.08, 0.001, 2.0, 2.0))
+    p, g = np.zeros(1, np.float32), np.zeros(1, np.float32)
+    for _ in range(14):
+        host.update(p, g, 1, 1)
+    expect, peak, period, first = [], 0.08, 2.0, 0
+    while len(expect) < 14:
+        for t in range(first, int(period) + 1):
+            expect.append(0.001 + 0.5 * (peak - 0.001) * (1 + np.cos(np.pi * t / period)))
+        peak, period, first = max(peak * 0.5, 0.001), period * 2, 1
+    np.testing.assert_allclose(rec.rates, expect[:14], rtol=2e-6, atol=1e-9)
+    assert rec.rates[0] == pytest.approx(0.08) and rec.rates[2] == pytest.approx(0.001)
+    assert rec.rates[6] == pytest.approx(0.001) and rec.rates[7] == pytest.approx(0.001 + 0.5 * 0.019 * (1 + np.cos(np.pi / 8)))
+
+
 def test_irprop_plus_by_hand(oracle64):
     """Four parameters through three calls, every branch, worked by hand (Igel & Hüsken 2000,
     iRPROP+): increase 1.2, decrease 0.5, step in [0.01, 0.13], start 0.1."""
