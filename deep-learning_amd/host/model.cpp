@@ -81,7 +81,10 @@ bool act_on_path(ACTIVATION::TYPE t) {
 }
 }  // namespace
 
-Model::Model(void) : impl_(new Impl) { real_gen.seed(5489u); }
+Model::Model(void) : impl_(new Impl) {
+  real_gen.seed(5489u);
+  bernoulli = new Dist::Bernoulli[1];
+}
 
 Model::~Model(void) {
   if (impl_->ctx != nullptr) (void)dlmi_ctx_synchronize(impl_->ctx);
@@ -98,6 +101,7 @@ Model::~Model(void) {
     }
   if (impl_->h_stage != nullptr) (void)hipHostFree(impl_->h_stage);
   if (impl_->ctx != nullptr) (void)dlmi_ctx_destroy(impl_->ctx);
+  delete[] bernoulli;
   delete[] ptr_array_layers;
   delete[] ptr_array_parameters;
   delete[] ptr_array_derivatives_parameters;
@@ -348,13 +352,20 @@ bool Model::set_dropout_mask(size_t const i, uint8_t const *mask) {
   return hip_ok(hipMemcpy(l.d_mask, l.mask_dropout_bernoulli.data(), l.n_units, hipMemcpyHostToDevice), impl_->err, "mask upload");
 }
 
+// Dropout_Bernoulli__Loop / __Layer__Loop (bernoulli_st.cpp:39-100): only layers whose type is exactly
+// LAYER_DROPOUT::BERNOULLI are resampled (the inverted kind is not: its masks keep their values), in layer
+// order, one draw of the shared generator per unit; a keep probability of 0 clears the mask without drawing.
 void Model::Dropout_Bernoulli(void) {
   for (size_t i = 1; i < total_layers; ++i) {
     Layer &l = ptr_array_layers[i];
-    if (!l.Use__Dropout()) continue;
+    if (l.type_dropout != LAYER_DROPOUT::BERNOULLI) continue;
     real const keep = l.dropout_values[0];
-    std::bernoulli_distribution dist(keep);
-    for (size_t j = 0; j < l.n_units; ++j) l.mask_dropout_bernoulli[j] = keep != 0.0f ? (dist(real_gen) ? 1 : 0) : 0;
+    if (keep != 0.0f) {
+      bernoulli->probability(keep);
+      for (size_t j = 0; j < l.n_units; ++j) l.mask_dropout_bernoulli[j] = (*bernoulli)() ? 1 : 0;
+    } else {
+      std::fill(l.mask_dropout_bernoulli.begin(), l.mask_dropout_bernoulli.end(), uint8_t(0));
+    }
     (void)hipMemcpy(l.d_mask, l.mask_dropout_bernoulli.data(), l.n_units, hipMemcpyHostToDevice);
   }
 }

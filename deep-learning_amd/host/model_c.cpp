@@ -114,6 +114,18 @@ int dlmi_model_set_dropout(dlmi_model *h, size_t layer, int d, float keep) {
 int dlmi_model_set_dropout_mask(dlmi_model *h, size_t layer, uint8_t const *mask) {
   return h->m.set_dropout_mask(layer, mask);
 }
+int dlmi_model_dropout_bernoulli(dlmi_model *h, unsigned seed, int reseed) {
+  if (h->m.ptr_array_layers == nullptr) return 0;
+  if (reseed) h->m.bernoulli[0].seed(seed);
+  h->m.Dropout_Bernoulli();
+  return 1;
+}
+int dlmi_model_get_dropout_mask(dlmi_model const *h, size_t layer, uint8_t *mask) {
+  if (h->m.ptr_array_layers == nullptr || layer == 0 || layer >= h->m.total_layers || mask == nullptr) return 0;
+  Layer const &l = h->m.ptr_array_layers[layer];
+  std::memcpy(mask, l.mask_dropout_bernoulli.data(), l.mask_dropout_bernoulli.size());
+  return 1;
+}
 int dlmi_model_set_dropout_backward_mode(dlmi_model *h, int mode) {
   h->m.dropout_backward_mode = mode ? DLMI_DROP_BWD_MASKED : DLMI_DROP_BWD_REFERENCE;
   return 1;

@@ -26,6 +26,7 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_mnist_destroy", "dlmi_mnist_load", "dlmi_mnist_last_error", "dlmi_mnist_copy",
     "dlmi_model_glorot_uniform", "dlmi_model_init_uniform", "dlmi_model_set_bound_hyper", "dlmi_model_set_constraints",
     "dlmi_model_set_rprop", "dlmi_model_set_rprop_loss", "dlmi_model_set_warm_restarts",
+    "dlmi_model_dropout_bernoulli", "dlmi_model_get_dropout_mask",
 ]
 
 LAYER_FULLY_CONNECTED, LAYER_RESIDUAL = 3, 9  # v1/data/enum/layer.hpp
@@ -98,6 +99,16 @@ class Model:
 
     def set_norm_hyper(self, momentum, eps, r_max, d_max):
         self._ok(self.lib.dlmi_model_set_norm_hyper(self.h, c_f(momentum), c_f(eps), c_f(r_max), c_f(d_max)), "hyper")
+
+    def dropout_bernoulli(self, seed=None):
+        """[bernoulli[0].seed(seed);] Model::Dropout_Bernoulli()"""
+        self._ok(self.lib.dlmi_model_dropout_bernoulli(self.h, ctypes.c_uint(seed or 0), c_int(int(seed is not None))),
+                 "Dropout_Bernoulli")
+
+    def dropout_mask(self, l, n):
+        out = np.zeros(n, np.uint8)
+        self._ok(self.lib.dlmi_model_get_dropout_mask(self.h, c_sz(l), _ptr(out)), "dropout mask")
+        return out
 
     def set_dropout_backward_mode(self, masked):
         self.lib.dlmi_model_set_dropout_backward_mode(self.h, c_int(1 if masked else 0))

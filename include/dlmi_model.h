@@ -39,6 +39,10 @@ int dlmi_model_set_layer_normalization_order(dlmi_model *m, size_t layer, int be
 int dlmi_model_set_norm_hyper(dlmi_model *m, float momentum, float eps, float r_max, float d_max);
 int dlmi_model_set_dropout(dlmi_model *m, size_t layer, int dropout, float keep);
 int dlmi_model_set_dropout_mask(dlmi_model *m, size_t layer, uint8_t const *mask_per_unit);
+/* [bernoulli[0].seed(seed) when reseed != 0;] Dropout_Bernoulli() (bernoulli_st.cpp:27-100); the host copy of a
+ * layer's per-unit mask (Layer::n_units bytes) */
+int dlmi_model_dropout_bernoulli(dlmi_model *m, unsigned seed, int reseed);
+int dlmi_model_get_dropout_mask(dlmi_model const *m, size_t layer, uint8_t *mask);
 int dlmi_model_set_dropout_backward_mode(dlmi_model *m, int mode);
 /* set_loss_fn(CROSS_ENTROPY), set_accu_fn(CROSS_ENTROPY), set_max_batch_size, update_mem_batch_size,
  * clear_training_arrays */

@@ -65,6 +65,26 @@ struct ENV { typedef enum : int { NONE = 0, TRAIN = 1, VALID = 2, TESTG = 3, LEN
 struct OPTIMIZER { typedef enum : int { NONE = 0, ADABOUND = 1, ADAM = 2, ADAMAX = 3, AMSBOUND = 4, AMSGRAD = 5,
   GD = 6, IRPROP_MINUS = 7, IRPROP_PLUS = 8, NOSADAM = 9, QUICKPROP = 10, SARPROP = 11, LENGTH = 12 } TYPE; };
 
+// The reference's mask generator (ops/distributions/bernoulli.hpp, distribution.hpp:23-47):
+// std::bernoulli_distribution over a std::mt19937 of its own, default seed 5489.
+namespace Dist {
+class Bernoulli {
+ public:
+  void seed(unsigned int const seed_received) { gen_.seed(seed_received); }
+  void probability(real const probability_received) {
+    if (probability_ == probability_received) return;
+    probability_ = probability_received;
+    dist_.param(std::bernoulli_distribution::param_type(probability_received));
+  }
+  bool operator()(void) { return dist_(gen_); }
+
+ private:
+  std::mt19937 gen_{5489u};
+  std::bernoulli_distribution dist_;
+  real probability_ = 0.0f;
+};
+}  // namespace Dist
+
 // v1/learner/model.hpp:70-93
 struct Layer_Parameters {
   bool use_bidirectional = false;
@@ -157,7 +177,10 @@ class Model {
   void initialize_weights_with_glorot_uniform(real const bias = 0.0f);
   void Initialization__Uniform(real const bias = 0.0f, real const lower_bound = -1.0f, real const upper_bound = 1.0f);
   void clear_training_arrays(void);  // train.cpp:110-141: zeroes the gradient array
-  void Dropout_Bernoulli(void);      // bernoulli_st.cpp:69-100: resample every per-unit mask
+  // bernoulli_st.cpp:27-100: resample the per-unit masks of the LAYER_DROPOUT::BERNOULLI layers, in layer
+  // order, from bernoulli[0].  As in the reference, the masks of BERNOULLI_INVERTED layers are NOT touched by
+  // it: they keep what they were allocated with (all ones) or what set_dropout_mask() installed.
+  void Dropout_Bernoulli(void);
 
   // ---- the hot path (model.hpp:2980, 1054, 1687, 2156) ----------------------
   void forward_pass(size_t const batch_size, real const *const *const ptr_array_inputs_received,
@@ -290,7 +313,10 @@ class Model {
   // How the backward treats dropout (see dlmi_dropout_bwd).  The reference's CPU
   // path is DLMI_DROP_BWD_REFERENCE.
   dlmi_dropout_bwd dropout_backward_mode = DLMI_DROP_BWD_REFERENCE;
-  std::mt19937 real_gen;  // mask sampling (the reference seeds its generators from the clock)
+  std::mt19937 real_gen;  // weight initializers (the engine inside the reference's Dist::Real real_gen)
+  // Dropout mask generator: `bernoulli[0]`, the one the reference's single-thread Dropout_Bernoulli draws
+  // from (model.hpp:3159, allocate.cpp:86-100; clock-seeded there, seed 5489 here until the caller seeds it).
+  Dist::Bernoulli *bernoulli = nullptr;
 
   Layer *Get__Input_Layer(void) const { return ptr_array_layers; }
   Layer *Get__Output_Layer(void) const { return ptr_last_layer - 1; }

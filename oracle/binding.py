@@ -681,6 +681,15 @@ class ReferenceMLP:
         """real_gen.seed(seed); Initialization__Uniform(bias, lower, upper)"""
         self.lib.dlref_model_init_uniform(self.h, ctypes.c_uint(seed), c_f(bias), c_f(lower), c_f(upper))
 
+    def dropout_bernoulli(self, seed=None):
+        """[bernoulli[0].seed(seed);] Model::Dropout_Bernoulli() on a single-thread model."""
+        ok = self.lib.dlref_model_dropout_bernoulli(self.h, ctypes.c_uint(seed or 0), c_int(int(seed is not None)))
+        assert ok, "the reference has no mask generator (no dropout layer set)"
+
+    def dropout_mask(self, l, n):
+        out = np.zeros(n, np.uint8)
+        return out if self.lib.dlref_model_get_dropout_mask(self.h, c_sz(l), c_sz(n), _ptr(out)) else None
+
     def set_moving(self, mean, std):
         mean = np.ascontiguousarray(mean, np.float32)
         std = np.ascontiguousarray(std, np.float32)

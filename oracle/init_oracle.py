@@ -151,3 +151,31 @@ def initialize(layers, acts, seed, bias, info, P, n_units, lower=None, upper=Non
     p[g0:g0 + n_units] = 1
     p[g0 + n_units:g0 + 2 * n_units] = 0
     return p
+
+
+# ---- dropout masks: Model::Dropout_Bernoulli, v1/learner/bernoulli_st.cpp:27-100 ------------------
+class BernoulliStream:
+    """Dist::Bernoulli (ops/distributions/bernoulli.cpp): std::bernoulli_distribution over a std::mt19937
+    of its own.  libstdc++ draws u = generate_canonical<double, 53>: two 32-bit words, (w0 + w1 * 2^32) / 2^64
+    in double, and keeps the unit when u < p (p the float probability widened to double)."""
+
+    def __init__(self, seed):
+        self.rs = np.random.RandomState(seed)
+
+    def draw(self, n, p):
+        w = self.rs.randint(0, 2 ** 32, size=2 * n, dtype=np.uint64).astype(np.float64)
+        u = (w[0::2] + w[1::2] * 2.0 ** 32) / 2.0 ** 64
+        u[u >= 1.0] = np.nextafter(1.0, 0.0)
+        return (u < np.float64(f32(p))).astype(np.uint8)
+
+
+def dropout_bernoulli(stream, units, dropout, masks):
+    """One call of Dropout_Bernoulli: `dropout` maps a layer to (kind, keep), `units` to its number of units,
+    `masks` holds the current masks and is updated in place.  Only the plain Bernoulli layers are resampled,
+    in layer order; a keep probability of 0 clears the mask without drawing (bernoulli_st.cpp:39-100)."""
+    for l in sorted(dropout):
+        kind, keep = dropout[l]
+        if kind != "BERNOULLI":
+            continue
+        masks[l] = stream.draw(units[l], keep) if f32(keep) != 0 else np.zeros(units[l], np.uint8)
+    return masks

@@ -507,6 +507,24 @@ int dlref_model_set_dropout_mask(void *h, size_t layer, size_t H,
   return 1;
 }
 
+// Mask resampling as Driver::train asks for it (drivers/driver.cpp:126-130): the first generator seeded
+// (allocate.cpp:86-100 seeds it from the clock), then Model::Dropout_Bernoulli() (bernoulli_st.cpp:27-100).
+// Single-thread models only: the OpenMP variant splits the units over per-thread generators.
+int dlref_model_dropout_bernoulli(void *h, unsigned seed, int reseed) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  if (m.bernoulli == nullptr) return 0;
+  if (reseed) m.bernoulli[0].seed(seed);
+  m.Dropout_Bernoulli();
+  return 1;
+}
+int dlref_model_get_dropout_mask(void *h, size_t layer, size_t H, uint8_t *mask) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  Layer &l = m.ptr_array_layers[layer];
+  if (l.ptr_array__mask__dropout__bernoulli == nullptr) return 0;
+  for (size_t j = 0; j < H; ++j) mask[j] = l.ptr_array__mask__dropout__bernoulli[j] ? 1 : 0;
+  return 1;
+}
+
 int dlref_model_prepare(void *h, size_t max_batch, int nthreads) {
   RefModel *rm = static_cast<RefModel *>(h);
   Model &m = rm->model;

@@ -616,6 +616,32 @@ def inits(R):
     return len(d)
 
 
+MASK_CASE = dict(widths=[8, 40, 30, 20, 25, 5], seed=42,
+                 dropout={1: ("BERNOULLI", 0.6), 2: ("BERNOULLI_INVERTED", 0.7), 3: ("BERNOULLI", 0.0), 4: ("BERNOULLI", 0.3)})
+
+
+def dropout_masks(R):
+    """Model::Dropout_Bernoulli (bernoulli_st.cpp:27-100) twice in a row on a single-thread model
+    whose first generator was seeded: the per-unit masks of every layer after each call."""
+    c = MASK_CASE
+    d = {"mask_case_json": np.frombuffer(json.dumps({"widths": c["widths"], "seed": c["seed"],
+                                                     "dropout": {str(k): v for k, v in c["dropout"].items()}}).encode(),
+                                         dtype=np.uint8)}
+    M = R.mlp(c["widths"])
+    for l, (kind, keep) in c["dropout"].items():
+        M.set_layer(l, ACT["RELU"], NORM["NONE"], DROP[kind], keep)
+    M.set_layer(len(c["widths"]) - 1, ACT["SOFTMAX"])
+    M.prepare(4, 0)
+    for l in c["dropout"]:
+        d[f"mask_initial_L{l}"] = M.dropout_mask(l, c["widths"][l])
+    for call in range(2):
+        M.dropout_bernoulli(c["seed"] if call == 0 else None)
+        for l in c["dropout"]:
+            d[f"mask_call{call}_L{l}"] = M.dropout_mask(l, c["widths"][l])
+    save("masks.npz", d)
+    return len(d)
+
+
 if __name__ == "__main__":
     R = Reference()
     print("leaves:", leaves(R), "arrays")
@@ -626,3 +652,4 @@ if __name__ == "__main__":
     print("shortcut:", shortcuts(R), "arrays")
     print("resnet:", resnets(R), "arrays")
     print("init:", inits(R), "arrays")
+    print("masks:", dropout_masks(R), "arrays")
