@@ -40,7 +40,7 @@ struct Model::Impl {
   // allocated (zeroed; the step sizes filled with rprop_delta_zero) on first use
   float *d_opt[7] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
   float const *cur_input = nullptr;  // [batch, n_in] of the pass in flight: d_input or a caller's device rows
-  size_t n_loss_examples = 0;        // examples whose loss has been accumulated since reset_loss()
+  size_t n_loss_values = 0;          // outputs whose loss term has been accumulated since reset_loss()
   size_t all_units = 0;              // normalization units of all entries: the slots a normalized model has
   float *h_stage = nullptr;    // pinned staging for the row-pointer gather
   size_t h_stage_floats = 0;
@@ -547,7 +547,7 @@ void Model::clear_training_arrays(void) {
   if (impl_->d_dparams == nullptr) return;
   (void)hipMemsetAsync(impl_->d_dparams, 0, total_parameters * sizeof(float), impl_->stream);
   (void)hipMemsetAsync(impl_->d_stats, 0, 2 * sizeof(double), impl_->stream);
-  impl_->n_loss_examples = 0;
+  impl_->n_loss_values = 0;
   std::memset(ptr_array_derivatives_parameters, 0, total_parameters * sizeof(real));
   Clear_Optimizer();
   warm_restarts_maximum_learning_rate = warm_restarts_initial_maximum_learning_rate;  // train.cpp:130-132
@@ -897,34 +897,60 @@ void Model::compute_loss_device(size_t const B, float const *d_targets) { comput
 
 void Model::seed_error(size_t const B, float const *d_targets) {
   Layer &o = ptr_array_layers[total_layers - 1];
-  if (o.type_activation_function != ACTIVATION::SOFTMAX || type_loss_function != LOSS_FN::CROSS_ENTROPY) {
-    fail("compute_error: only softmax + cross-entropy is on this path");
-    return;
+  if (o.type_activation_function == ACTIVATION::SOFTMAX) {
+    if (type_loss_function != LOSS_FN::CROSS_ENTROPY || type_accuracy_function != ACCU_FN::CROSS_ENTROPY) {
+      fail("compute_error: a softmax output layer takes the cross-entropy loss and accuracy on this path");
+      return;
+    }
+    if (dlmi_softmax_ce_seed(impl_->ctx, B, o.n_out, o.d_outputs, d_targets, o.d_errors, impl_->d_stats) != DLMI_OK) {
+      fail("compute_error: dlmi_softmax_ce_seed");
+      return;
+    }
+  } else {
+    // element-wise output activation: f'(x, q) * loss_fn_derivative(q, y) (compute_error_st.cpp:118-123)
+    if (dlmi_loss_seed(impl_->ctx, static_cast<dlmi_loss>(type_loss_function), static_cast<dlmi_accuracy>(type_accuracy_function),
+                       acc_var, static_cast<dlmi_activation>(o.type_activation_function), B, o.n_out, o.d_summations,
+                       o.d_outputs, d_targets, o.d_errors, impl_->d_stats) != DLMI_OK) {
+      fail((std::string("compute_error: ") + dlmi_last_error(impl_->ctx)).c_str());
+      return;
+    }
   }
-  if (dlmi_softmax_ce_seed(impl_->ctx, B, o.n_out, o.d_outputs, d_targets, o.d_errors, impl_->d_stats) != DLMI_OK) {
-    fail("compute_error: dlmi_softmax_ce_seed");
-    return;
-  }
-  impl_->n_loss_examples += B;
+  impl_->n_loss_values += B * o.n_out;  // update_loss counts every output (compute_loss.cpp:50-52)
 }
 
 // ---------------------------------------------------------------- loss / accuracy bookkeeping
 void Model::reset_loss(void) {
   n_acc_trial = 0;
-  impl_->n_loss_examples = 0;
+  impl_->n_loss_values = 0;
   if (impl_->d_stats != nullptr) (void)hipMemsetAsync(impl_->d_stats, 0, 2 * sizeof(double), impl_->stream);
 }
-// get_ace (loss.cpp:212-221): summed cross-entropy / number of examples
+// loss.cpp:98-221: the accumulated terms over their number (ME, MAE, MSE), as they are (L1, L2), the root
+// of their mean (RMSE), or over the number of examples (cross-entropy, get_ace)
 double Model::get_loss(ENV::TYPE const env) const {
   switch (env) {
     case ENV::TRAIN: return loss_train;
     case ENV::VALID: return loss_valid;
     case ENV::TESTG: return loss_testg;
-    case ENV::NONE:
-      if (type_loss_function != LOSS_FN::CROSS_ENTROPY) return 1.0;
-      return impl_->n_loss_examples != 0 ? get_loss_sum() / static_cast<double>(impl_->n_loss_examples) : HUGE_VAL;
+    case ENV::NONE: {
+      size_t const n = impl_->n_loss_values;
+      switch (type_loss_function) {
+        case LOSS_FN::ME: case LOSS_FN::MAE: return n != 0 ? get_loss_sum() / static_cast<double>(n) : 1.0;
+        case LOSS_FN::MSE: return n != 0 ? 1.0 / static_cast<double>(n) * get_loss_sum() : 1.0;
+        case LOSS_FN::RMSE: return n != 0 ? std::sqrt(1.0 / static_cast<double>(n) * get_loss_sum()) : 1.0;
+        case LOSS_FN::L1: case LOSS_FN::L2: return get_loss_sum();
+        case LOSS_FN::CROSS_ENTROPY: return n != 0 ? get_loss_sum() / static_cast<double>(n / ptr_array_layers[total_layers - 1].n_out) : HUGE_VAL;
+        default: return 1.0;
+      }
+    }
     default: return 1.0;
   }
+}
+bool Model::Set__Accurancy_Variance(real const v) {
+  if (acc_var == v) return true;
+  if (v < 0.0f) return fail("Accuracy variance less than zero.");
+  if (v > 1.0f) return fail("Accuracy variance bigger than one.");
+  acc_var = v;
+  return true;
 }
 // metrics.cpp:89-114
 double Model::get_accu(ENV::TYPE const env) const {

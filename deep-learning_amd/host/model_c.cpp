@@ -139,6 +139,17 @@ int dlmi_model_prepare(dlmi_model *h, size_t max_batch) {
   h->m.clear_training_arrays();
   return 1;
 }
+int dlmi_model_set_loss(dlmi_model *h, int loss, int accu, float accu_variance) {
+  h->m.set_loss_fn(static_cast<LOSS_FN::TYPE>(loss));
+  h->m.set_accu_fn(static_cast<ACCU_FN::TYPE>(accu));
+  return h->m.Set__Accurancy_Variance(accu_variance) ? 1 : 0;
+}
+void dlmi_model_reset_loss(dlmi_model *h) { h->m.reset_loss(); }
+void dlmi_model_loss_accu(dlmi_model *h, size_t n_data, double *out) {
+  h->m.n_acc_trial = n_data * (ACCU_FN::CROSS_ENTROPY == h->m.type_accuracy_function ? size_t(1) : h->m.ptr_array_layers[h->m.total_layers - 1].n_out);
+  out[0] = h->m.get_loss(ENV::NONE);
+  out[1] = h->m.get_accu(ENV::NONE);
+}
 size_t dlmi_model_total_parameters(dlmi_model const *h) { return h->m.total_parameters; }
 size_t dlmi_model_total_normalized_units(dlmi_model const *h) { return h->m.total_normalized_units; }
 void dlmi_model_layer_offsets(dlmi_model const *h, size_t layer, size_t *out) {

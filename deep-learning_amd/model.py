@@ -26,7 +26,8 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_mnist_destroy", "dlmi_mnist_load", "dlmi_mnist_last_error", "dlmi_mnist_copy",
     "dlmi_model_glorot_uniform", "dlmi_model_init_uniform", "dlmi_model_set_bound_hyper", "dlmi_model_set_constraints",
     "dlmi_model_set_rprop", "dlmi_model_set_rprop_loss", "dlmi_model_set_warm_restarts",
-    "dlmi_model_dropout_bernoulli", "dlmi_model_get_dropout_mask",
+    "dlmi_model_dropout_bernoulli", "dlmi_model_get_dropout_mask", "dlmi_model_set_loss", "dlmi_model_reset_loss",
+    "dlmi_model_loss_accu",
 ]
 
 LAYER_FULLY_CONNECTED, LAYER_RESIDUAL = 3, 9  # v1/data/enum/layer.hpp
@@ -189,6 +190,19 @@ class Model:
         p = np.empty(self.P, np.float32)
         self._ok(self.lib.dlmi_model_get_derivatives(self.h, _ptr(p), c_sz(self.P)), "get_derivatives")
         return p
+
+    def set_loss(self, loss, accu, acc_var=0.49):
+        """set_loss_fn / set_accu_fn / Set__Accurancy_Variance (after prepare, which selects cross-entropy)."""
+        self._ok(self.lib.dlmi_model_set_loss(self.h, c_int(loss), c_int(accu), c_f(acc_var)), "set_loss")
+
+    def reset_loss(self):
+        self.lib.dlmi_model_reset_loss(self.h)
+
+    def loss_accu(self, n_data):
+        """(get_loss(NONE), get_accu(NONE)) as the epoch driver reports them after n_data examples."""
+        out = (ctypes.c_double * 2)()
+        self.lib.dlmi_model_loss_accu(self.h, c_sz(n_data), out)
+        return out[0], out[1]
 
     def loss_sum(self):
         return self.lib.dlmi_model_loss_sum(self.h)

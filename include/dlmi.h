@@ -189,6 +189,25 @@ int dlmi_residual_bwd(dlmi_ctx *ctx, size_t B, size_t input_size, size_t derivat
 int dlmi_softmax_ce_seed(dlmi_ctx *ctx, size_t B, size_t H, float const *q, float const *y,
                          float *dZ, double *stats);
 
+/* v1/data/enum/loss_fn.hpp:22-71: the loss functions that have a derivative, and the accuracy functions */
+typedef enum {
+  DLMI_LOSS_CROSS_ENTROPY = 2, DLMI_LOSS_L1 = 3, DLMI_LOSS_L2 = 4, DLMI_LOSS_MAE = 5, DLMI_LOSS_ME = 9,
+  DLMI_LOSS_MSE = 10, DLMI_LOSS_RMSE = 11
+} dlmi_loss;
+typedef enum { DLMI_ACCU_CROSS_ENTROPY = 1, DLMI_ACCU_DIRECTIONAL = 2, DLMI_ACCU_DISTANCE = 3, DLMI_ACCU_SIGN = 5 } dlmi_accuracy;
+
+/* Seed gradient of an output layer with an element-wise activation f (any but softmax):
+ *   dZ = f'(z, q) * dl(q, y),  dl = -1 (ME, L1) | sign(q - y) (MAE) | 2 (q - y) (L2, MSE, RMSE), over B*H;
+ *                                   (y == 1 ? -1 / clip(q, 1e-7, 1 - 1e-7) : 0) over B (cross-entropy).
+ * stats (device, 2 doubles, may be NULL) accumulates { sum of the loss terms q - y | |q - y| | (q - y)^2 |
+ * -log(clip(q)) where y == 1, number of accurate outputs }: |q - y| <= accu_threshold (DISTANCE), every output
+ * (DIRECTIONAL), sign(y) == sign(q) or y == 0 and |q| <= 1e-7 (SIGN), rows whose arg-max is the target
+ * (CROSS_ENTROPY).  dZ may be NULL (loss and accuracy only; z is then unused).
+ * Replaces the element-wise branch of compute_error_fwp_{st,mp} (v1/learner/compute_error_st.cpp:26-131) with
+ * loss_fn, loss_fn_derivative and update_loss (compute_loss.cpp:25-138). */
+int dlmi_loss_seed(dlmi_ctx *ctx, dlmi_loss loss, dlmi_accuracy accu, float accu_threshold, dlmi_activation act,
+                   size_t B, size_t H, float const *z, float const *q, float const *y, float *dZ, double *stats);
+
 /* ---- the fused hot path ----------------------------------------------------
  * One training-mode layer tail: x (= Z) -> batch (re)norm -> activation ->
  * optional dropout, without materialising x_hat or the pre-activation.

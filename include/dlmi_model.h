@@ -47,6 +47,13 @@ int dlmi_model_set_dropout_backward_mode(dlmi_model *m, int mode);
 /* set_loss_fn(CROSS_ENTROPY), set_accu_fn(CROSS_ENTROPY), set_max_batch_size, update_mem_batch_size,
  * clear_training_arrays */
 int dlmi_model_prepare(dlmi_model *m, size_t max_batch);
+/* set_loss_fn(loss), set_accu_fn(accu), Set__Accurancy_Variance(accu_variance): after dlmi_model_prepare,
+ * which selects cross-entropy */
+int dlmi_model_set_loss(dlmi_model *m, int loss, int accu, float accu_variance);
+/* reset_loss(); out[0] = get_loss(ENV::NONE), out[1] = get_accu(ENV::NONE) with n_acc_trial = n_data outputs'
+ * worth of trials (driver.cpp:95-99) */
+void dlmi_model_reset_loss(dlmi_model *m);
+void dlmi_model_loss_accu(dlmi_model *m, size_t n_data, double *out);
 size_t dlmi_model_total_parameters(dlmi_model const *m);
 size_t dlmi_model_total_normalized_units(dlmi_model const *m);
 /* out[0..5] = first weight index, first bias index, gamma index, beta index, moving-stat index, Use__Bias() */

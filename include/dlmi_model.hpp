@@ -160,6 +160,7 @@ class Model {
                    bool const scale_weights = true);
   void set_loss_fn(LOSS_FN::TYPE const type) { type_loss_function = type; }
   void set_accu_fn(ACCU_FN::TYPE const type) { type_accuracy_function = type; }
+  bool Set__Accurancy_Variance(real const accurancy_variance_received);  // metrics.cpp:27-52: within [0, 1]
   bool set_max_batch_size(size_t const max_batch_size);
   bool update_mem_batch_size(size_t const desired_batch_size_received, bool const force_update_received = false);
   bool set_mp(bool const) { return true; }
@@ -297,6 +298,7 @@ class Model {
   real rprop_delta_zero = 0.1f;
   double loss_rprop = HUGE_VAL;
   double loss_rprop_tm1 = HUGE_VAL;
+  real acc_var = 0.49f;                               // model.hpp:3019, the reach of ACCU_FN::DISTANCE
   bool use_clip_gradient = false;                     // model.hpp:2843
   real clip_gradient = 1.0f;                          // model.hpp:3044
   real regularization__max_norm_constraints = 0.0f;   // model.hpp:3024

@@ -34,6 +34,9 @@ NORM = dict(NONE=0, BN=1, BRN=2)
 DROP = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3)
 STATE = dict(INFERENCE=0, TRAINING=1, UPDATE_BATCH_NORM=2)
 # v1/data/enum/optimizer.hpp:24-42
+# v1/data/enum/loss_fn.hpp:22-71
+LOSS = dict(CROSS_ENTROPY=2, L1=3, L2=4, MAE=5, MAPE=6, ME=9, MSE=10, RMSE=11, SMAPE=12)
+ACCU = dict(CROSS_ENTROPY=1, DIRECTIONAL=2, DISTANCE=3, R=4, SIGN=5)
 OPT = dict(NONE=0, ADABOUND=1, ADAM=2, AMSBOUND=4, AMSGRAD=5, GD=6, IRPROP_PLUS=8, NOSADAM=9)
 _ADAM_FAMILY = (1, 2, 4, 5, 9)
 
@@ -413,6 +416,21 @@ class Oracle(_Leaves):
                                    ctypes.byref(loss), ctypes.byref(corr))
         return dZ, loss.value, corr.value
 
+    def loss_seed(self, loss, accu, acc_var, act, z, q, y, nthreads=0, want_dz=True):
+        """Returns (dZ or None, loss_sum, n_accurate) of an element-wise output layer."""
+        z, q, y = self._a(z), self._a(q), self._a(y)
+        B, H = q.shape
+        dZ = np.empty((B, H), self.dtype) if want_dz else None
+        loss_sum = c_d(0.0)
+        acc = c_d(0.0)
+        f = self._f("loss_seed")
+        f.restype = c_int
+        rc = f(c_int(nthreads), c_int(loss), c_int(accu), self._real(acc_var), c_int(act), c_sz(B), c_sz(H), _ptr(z),
+               _ptr(q), _ptr(y), _ptr(dZ) if want_dz else None, ctypes.byref(loss_sum), ctypes.byref(acc))
+        if rc != 0:
+            raise ValueError("loss / accuracy function not managed")
+        return dZ, loss_sum.value, acc.value
+
     def mlp(self, widths):
         return OracleMLP(self, widths)
 
@@ -512,9 +530,31 @@ class OracleMLP:
         bs = min(self.max_batch, n)
         return [(i, min(bs, n - i)) for i in range(0, n, bs)]
 
+    def set_loss(self, loss, accu, acc_var=0.49):
+        """set_loss_fn / set_accu_fn / acc_var for an output layer with an element-wise activation."""
+        self.loss_fn, self.accu_fn = LOSS[loss] if isinstance(loss, str) else loss, ACCU[accu] if isinstance(accu, str) else accu
+        self.lib.dlo_mlp_set_loss(self.h, c_int(self.loss_fn), c_int(self.accu_fn), c_f(acc_var))
+
+    def reset_loss(self):
+        self.lib.dlo_mlp_reset_loss(self.h)
+
+    def loss_accu(self, n_data):
+        return self._loss_accu(n_data)
+
     def _loss_accu(self, n):
-        loss = self.lib.dlo_mlp_loss_sum(self.h) / n if n else float("inf")  # get_ace, loss.cpp:212-221
-        return loss, self.lib.dlo_mlp_n_correct(self.h) / n * 100.0           # get_accu, metrics.cpp:89-114
+        total, hout = self.lib.dlo_mlp_loss_sum(self.h), self.widths[-1]
+        loss_fn, accu_fn = getattr(self, "loss_fn", LOSS["CROSS_ENTROPY"]), getattr(self, "accu_fn", ACCU["CROSS_ENTROPY"])
+        terms = n * hout  # update_loss counts every output (compute_loss.cpp:50-52)
+        if loss_fn == LOSS["CROSS_ENTROPY"]:
+            loss = total / n if n else float("inf")                            # get_ace, loss.cpp:212-221
+        elif loss_fn in (LOSS["L1"], LOSS["L2"]):
+            loss = total                                                       # loss.cpp:146, 158
+        elif loss_fn == LOSS["RMSE"]:
+            loss = float(np.sqrt(total / terms)) if terms else 1.0             # loss.cpp:170-178
+        else:
+            loss = total / terms if terms else 1.0                             # get_me / get_mae / get_mse
+        trials = n * (1 if accu_fn == ACCU["CROSS_ENTROPY"] else hout)         # drivers/driver.cpp:95-99
+        return loss, self.lib.dlo_mlp_n_correct(self.h) / trials * 100.0       # get_accu, metrics.cpp:89-114
 
     def train_epoch(self, X, Y):
         """Driver::train: gradients accumulate over the sub-batches, ONE parameter
@@ -729,6 +769,20 @@ class ReferenceMLP:
         p = np.empty(self.P, np.float32)
         self.lib.dlref_model_get_dparams(self.h, _ptr(p), c_sz(self.P))
         return p
+
+    # ---- loss / accuracy function (set_loss_fn, set_accu_fn, acc_var) -----------
+    def set_loss(self, loss, accu, acc_var=0.49):
+        self.lib.dlref_model_set_loss(self.h, c_int(LOSS[loss] if isinstance(loss, str) else loss),
+                                      c_int(ACCU[accu] if isinstance(accu, str) else accu), c_f(acc_var))
+
+    def reset_loss(self):
+        self.lib.dlref_model_reset_loss(self.h)
+
+    def loss_accu(self, n_data):
+        """(get_loss(NONE), get_accu(NONE)) as Driver reports them after n_data examples."""
+        out = (c_d * 2)()
+        self.lib.dlref_model_loss_accu(self.h, c_sz(n_data), out)
+        return out[0], out[1]
 
     # ---- optimizer (Model::Update_Parameter) ---------------------------------
     def set_optimizer(self, kind, lr=0.01, momentum=0.9, nesterov=False, adam_lr=0.001, beta1=0.9, beta2=0.999,

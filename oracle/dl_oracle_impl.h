@@ -660,3 +660,70 @@ void FN(dlo_softmax_ce_seed)(int nthreads, size_t B, size_t H, REAL const *q,
   if (loss_sum) *loss_sum += loss;
   if (n_correct) *n_correct += correct;
 }
+
+/* ---- a16, element-wise output layer: compute_error_st.cpp:26-131 (the branch for
+ * an activation other than softmax), compute_error_mp.cpp the same per thread.
+ *   loss term      loss_fn           compute_loss.cpp:52-99
+ *   accuracy       by accu           compute_error_st.cpp:50-104
+ *   dZ = f'(x, q) * loss_fn_derivative(q, y, B, H)   compute_loss.cpp:101-138
+ * loss: LOSS_FN::TYPE (2 CE, 3 L1, 4 L2, 5 MAE, 9 ME, 10 MSE, 11 RMSE), accu:
+ * ACCU_FN::TYPE (1 CE, 2 DIRECTIONAL, 3 DISTANCE, 5 SIGN).  x = pre-activation,
+ * q = activation value.  dZ may be NULL (compute_loss).  Returns 0, or -1 for a
+ * loss / accuracy function the reference's switch reports as not managed. */
+static inline REAL FN(sign)(REAL v) { return (REAL)(((REAL)0 < v) - (v < (REAL)0)); }
+int FN(dlo_loss_seed)(int nthreads, int loss_fn, int accu_fn, REAL acc_var, int act, size_t B, size_t H,
+                      REAL const *x, REAL const *q, REAL const *y, REAL *dZ, double *loss_sum,
+                      double *n_accurate) {
+  int const N = FN(nthr)(nthreads, B);
+  int const Bi = (int)B;
+  double loss = 0.0, accurate = 0.0;
+  int b;
+  if (!(loss_fn == 2 || loss_fn == 3 || loss_fn == 4 || loss_fn == 5 || loss_fn == 9 || loss_fn == 10 || loss_fn == 11)) return -1;
+  if (!(accu_fn == 1 || accu_fn == 2 || accu_fn == 3 || accu_fn == 5)) return -1;
+#pragma omp parallel for schedule(static) num_threads(N > 0 ? N : 1) if (N > 0) \
+    reduction(+ : loss, accurate)
+  for (b = 0; b < Bi; ++b) {
+    REAL const *qi = q + (size_t)b * H;
+    REAL const *yi = y + (size_t)b * H;
+    if (accu_fn == 1) {
+      size_t k_target = H, k_predict = 0;
+      REAL q_max = -REAL_MAX;
+      for (size_t k = 0; k != H; ++k) {
+        if (qi[k] >= q_max) { k_predict = k; q_max = qi[k]; }
+        if (yi[k] == (REAL)1) k_target = k;
+      }
+      accurate += (double)(k_target == k_predict);
+    }
+    for (size_t k = 0; k != H; ++k) {
+      REAL const qv = qi[k], yv = yi[k];
+      REAL l, dl;
+      switch (loss_fn) {
+        case 9: case 3: l = qv - yv; dl = (REAL)-1; break;
+        case 5: l = FABS(qv - yv); dl = qv > yv ? (REAL)1 : (qv < yv ? (REAL)-1 : (REAL)0); break;
+        case 2:
+          l = FN(clip)(qv, DLO_EPSILON, (REAL)1 - DLO_EPSILON);
+          dl = yv == (REAL)1 ? (REAL)-1 / l : (REAL)0;
+          l = yv == (REAL)1 ? -(yv * LOG(l)) : (REAL)0;
+          break;
+        default: l = (qv - yv) * (qv - yv); dl = (REAL)2 * (qv - yv); break;
+      }
+      loss += (double)l;
+      switch (accu_fn) {
+        case 3: if (FABS(qv - yv) <= acc_var) accurate += 1.0; break;
+        case 2: accurate += 1.0; break;
+        case 5:
+          if (FN(sign)(yv) == FN(sign)(qv) || (FN(sign)(yv) == (REAL)0 && qv >= -DLO_EPSILON && qv <= DLO_EPSILON))
+            accurate += 1.0;
+          break;
+        default: break;
+      }
+      if (dZ) {
+        if (loss_fn == 2) dl /= (REAL)B; else dl /= (REAL)(B * H);
+        dZ[(size_t)b * H + k] = FN(af_derive)(act, x[(size_t)b * H + k], qv) * dl;
+      }
+    }
+  }
+  if (loss_sum) *loss_sum += loss;
+  if (n_accurate) *n_accurate += accurate;
+  return 0;
+}

@@ -641,6 +641,26 @@ void dlref_model_step(void *h, int state, size_t B, float const *X, size_t K0,
   }
 }
 
+// Loss and accuracy function of the output layer (set_loss_fn / set_accu_fn, acc_var of ACCU_FN::DISTANCE),
+// reset of their accumulators, and what Driver reports after n_data examples (drivers/driver.cpp:93-105:
+// n_acc_trial, then get_loss / get_accu of ENV::NONE).  In an OpenMP model the per-thread accumulators are
+// merged first, as Driver::train_mp does.
+void dlref_model_set_loss(void *h, int loss, int accu, float acc_var) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  m.set_loss_fn(static_cast<LOSS_FN::TYPE>(loss));
+  m.set_accu_fn(static_cast<ACCU_FN::TYPE>(accu));
+  m.acc_var = acc_var;
+}
+void dlref_model_reset_loss(void *h) { static_cast<RefModel *>(h)->model.reset_loss(); }
+void dlref_model_loss_accu(void *h, size_t n_data, double *out) {
+  RefModel *rm = static_cast<RefModel *>(h);
+  Model &m = rm->model;
+  if (rm->nthreads > 0) m.merge_mp_accu_loss();
+  m.n_acc_trial = n_data * (1 - m.n_time_delay) * (ACCU_FN::CROSS_ENTROPY == m.type_accuracy_function ? 1 : m.get_n_out());
+  out[0] = m.get_loss(DL::ENV::NONE);
+  out[1] = m.get_accu(DL::ENV::NONE);
+}
+
 // Per-layer buffers, [B,H] each. which: 0 summations (Z), 1 values_hats,
 // 2 values_normalizes, 3 AF values (post-dropout), 4 neuron errors (dZ),
 // 5 derivative_outputs (aliases the AF units' errors, ordering.cpp:165: holds

@@ -17,7 +17,7 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 sys.path.insert(0, ROOT)
-from oracle.binding import ACT, DROP, NORM, OPT, STATE, Reference, ReferenceNet  # noqa: E402
+from oracle.binding import ACCU, ACT, DROP, LOSS, NORM, OPT, STATE, Reference, ReferenceNet  # noqa: E402
 
 OUT = os.path.dirname(os.path.abspath(__file__))
 ACTS = ["ELU", "ISRLU", "LEAKY_RELU", "RELU", "SELU", "LINEAR"]
@@ -642,14 +642,85 @@ def dropout_masks(R):
     return len(d)
 
 
+# name: (widths, B, output activation, loss, accuracy, acc_var, kind of targets)
+REGRESS_CASES = {
+    "linear_mse_distance": ([7, 12, 5], 19, "LINEAR", "MSE", "DISTANCE", 0.3, "real"),
+    "elu_mae_sign": ([6, 9, 4], 13, "ELU", "MAE", "SIGN", 0.49, "signed"),
+    "isrlu_l2_directional": ([5, 8, 3], 11, "ISRLU", "L2", "DIRECTIONAL", 0.49, "real"),
+    "selu_rmse_distance": ([9, 14, 6], 23, "SELU", "RMSE", "DISTANCE", 0.49, "real"),
+    "lrelu_me_sign": ([4, 10, 7], 16, "LEAKY_RELU", "ME", "SIGN", 0.49, "signed"),
+    "relu_l1_distance": ([8, 11, 2], 9, "RELU", "L1", "DISTANCE", 0.1, "real"),
+    "linear_ce_ce": ([6, 10, 4], 15, "LINEAR", "CROSS_ENTROPY", "CROSS_ENTROPY", 0.49, "onehot"),
+    "linear_mse_wide": ([20, 40, 130], 37, "LINEAR", "MSE", "DISTANCE", 0.49, "real"),
+}
+
+
+def regressions(R):
+    """Output layers with an element-wise activation and the regression losses
+    (compute_error_st.cpp:80-123, compute_loss.cpp:25-138, loss.cpp:98-221): one
+    training step with its seed gradient, loss and accuracy, then three epochs of
+    Nesterov momentum through the epoch driver with the loss it reports."""
+    d = {"regress_cases_json": np.frombuffer(json.dumps(REGRESS_CASES).encode(), dtype=np.uint8)}
+    for name, (widths, B, out_act, loss, accu, acc_var, targets) in REGRESS_CASES.items():
+        rng = np.random.default_rng(sum(map(ord, name)))
+        L = len(widths)
+        X = f32(rng.uniform(-1, 1, (B, widths[0])))
+        if targets == "onehot":
+            Y = f32(np.eye(widths[-1])[rng.integers(0, widths[-1], B)])
+        else:
+            Y = f32(rng.uniform(-1, 1, (B, widths[-1])))
+            if targets == "signed":
+                Y[rng.uniform(size=Y.shape) < 0.2] = 0.0
+        d[name + "_X"], d[name + "_Y"] = X, Y
+        params = None
+        for nt in THREADS:
+            M = R.mlp(widths)
+            for l in range(1, L - 1):
+                M.set_layer(l, ACT["ELU"], NORM["BRN"])
+            M.set_layer(L - 1, ACT[out_act])
+            M.prepare(B, nt)
+            M.set_loss(loss, accu, acc_var)
+            if params is None:
+                M.glorot_uniform(sum(map(ord, name)))
+                params = M.get_parameters()
+                d[name + "_params"] = params.copy()
+            M.set_parameters(params)
+            q = f"{name}_t{nt}_"
+            M.reset_loss()
+            M.step(STATE["TRAINING"], X, Y, backward=True)
+            for l in range(1, L):
+                d[f"{q}L{l}_Z"] = M.layer_buffer(l, 0)
+                d[f"{q}L{l}_out"] = M.layer_buffer(l, 6)
+                d[f"{q}L{l}_dZ"] = M.layer_buffer(l, 4)
+            d[q + "dparams"] = M.get_dparams()
+            d[q + "loss_accu"] = np.array(M.loss_accu(B))
+            if targets == "onehot":  # clipped probabilities give gradients of 1e7: one step is enough
+                continue
+            # the epoch driver on the same data: sub-batches of 7, one update per epoch
+            M2 = R.mlp(widths)
+            for l in range(1, L - 1):
+                M2.set_layer(l, ACT["ELU"], NORM["BRN"])
+            M2.set_layer(L - 1, ACT[out_act])
+            M2.set_norm_hyper(0.5, 1e-5, 3.0, 5.0)
+            M2.prepare(7, nt)
+            M2.set_loss(loss, accu, acc_var)
+            M2.set_parameters(params)
+            M2.set_optimizer(OPT["GD"], lr=0.01, momentum=0.9, nesterov=True)
+            rep = []
+            for _ in range(3):
+                rep.append(M2.train_epoch(X, Y))
+            rep.append(M2.evalt(X, Y))
+            d[q + "epoch_reports"] = np.array(rep)
+            d[q + "epoch_params"] = M2.get_parameters()
+    save("regress.npz", d)
+    return len(d)
+
+
 if __name__ == "__main__":
     R = Reference()
-    print("leaves:", leaves(R), "arrays")
-    print("mlp:", mlps(R), "arrays")
-    print("optim:", optimizers(R), "arrays")
-    print("epoch:", epochs(R), "arrays")
-    print("variants:", variants(R), "arrays")
-    print("shortcut:", shortcuts(R), "arrays")
-    print("resnet:", resnets(R), "arrays")
-    print("init:", inits(R), "arrays")
-    print("masks:", dropout_masks(R), "arrays")
+    only = sys.argv[1:]  # names of the fixtures to write; all of them without arguments
+    for label, fn in [("leaves", leaves), ("mlp", mlps), ("optim", optimizers), ("epoch", epochs), ("variants", variants),
+                      ("shortcut", shortcuts), ("resnet", resnets), ("init", inits), ("masks", dropout_masks),
+                      ("regress", regressions)]:
+        if not only or label in only:
+            print(label + ":", fn(R), "arrays")

@@ -1,0 +1,134 @@
+"""The HIP path on output layers with an element-wise activation and the
+regression losses, through the C ABI: the seed kernel against the compiled
+reference's output-layer buffers (tests/golden/regress.npz) and against the CPU
+restatement on larger seeded inputs, then the model facade and its epoch driver
+against the same fixture.
+
+Tolerances (fp32): 1e-5 relative for the element-wise seed, 1e-4 behind the
+GEMMs and column reductions of the whole model."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import RTOL_ELEMENTWISE as TE
+from helpers import RTOL_REDUCED as TR
+from helpers import assert_close
+from oracle.binding import ACCU, ACT, LOSS
+from test_oracle_regress import (build_regress_model, check_regress_epochs, check_regress_step, load_regress_golden,
+                                 regress_cases)
+
+pytestmark = pytest.mark.gpu
+
+LOSSES = ["ME", "L1", "MAE", "MSE", "L2", "RMSE", "CROSS_ENTROPY"]
+ACCUS = ["DISTANCE", "DIRECTIONAL", "SIGN", "CROSS_ENTROPY"]
+
+
+def dev(a, dtype=torch.float32):
+    return torch.as_tensor(np.ascontiguousarray(a)).to("cuda", dtype=dtype).contiguous()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+@pytest.fixture(scope="module")
+def model_factory(pkg):
+    from deep_learning_amd.model import Model
+    lib = pkg.load_library()
+    made = []
+
+    def make(widths):
+        m = Model(lib, widths)
+        made.append(m)
+        return m
+
+    yield make
+    for m in made:
+        m.close()
+
+
+@pytest.mark.parametrize("name", list(regress_cases()))
+def test_seed_kernel_against_golden_output_layer(dl, name):
+    g = load_regress_golden()
+    widths, B, out_act, loss, accu, acc_var, _ = regress_cases()[name]
+    o, q = len(widths) - 1, f"{name}_t0_"
+    stats = torch.zeros(2, dtype=torch.float64, device="cuda")
+    dZ = dl.loss_seed(LOSS[loss], ACCU[accu], acc_var, ACT[out_act], dev(g[f"{q}L{o}_Z"]), dev(g[f"{q}L{o}_out"]),
+                      dev(g[name + "_Y"]), stats)
+    assert_close(host(dZ), g[f"{q}L{o}_dZ"], TE, "seed gradient")
+    total, acc = host(stats)
+    n = B * widths[-1]
+    rep = {"L1": total, "L2": total, "RMSE": np.sqrt(total / n), "CROSS_ENTROPY": total / B}.get(loss, total / n)
+    assert rep == pytest.approx(g[q + "loss_accu"][0], rel=1e-5)
+    trials = B * (1 if accu == "CROSS_ENTROPY" else widths[-1])
+    assert acc / trials * 100.0 == pytest.approx(g[q + "loss_accu"][1], abs=1e-9)
+
+
+@pytest.mark.parametrize("B,H", [(1, 1), (3, 64), (257, 10), (70, 130), (4099, 7)])
+@pytest.mark.parametrize("act", ["LINEAR", "ELU", "ISRLU", "LEAKY_RELU", "RELU", "SELU"])
+def test_seed_kernel_against_oracle(dl, oracle, B, H, act):
+    rng = np.random.default_rng(B * 131 + H + ACT[act])
+    z = (rng.standard_normal((B, H)) * 1.5).astype(np.float32)
+    q = oracle.act_fwd(ACT[act], z)
+    y = rng.uniform(-1, 1, (B, H)).astype(np.float32)
+    y[rng.uniform(size=y.shape) < 0.2] = 0.0
+    y[np.arange(B), rng.integers(0, H, B)] = 1.0  # a target of exactly one somewhere in each row
+    zd, qd, yd = dev(z), dev(q), dev(y)
+    for loss in LOSSES:
+        for accu in ACCUS:
+            dZo, total, acc = oracle.loss_seed(LOSS[loss], ACCU[accu], 0.37, ACT[act], z, q, y)
+            stats = torch.zeros(2, dtype=torch.float64, device="cuda")
+            dZ = dl.loss_seed(LOSS[loss], ACCU[accu], 0.37, ACT[act], zd, qd, yd, stats)
+            assert_close(host(dZ), dZo, TE, f"{loss}/{accu} seed gradient")
+            st = host(stats)
+            assert abs(st[0] - total) <= 1e-5 * max(1.0, abs(total)), f"{loss}/{accu} loss sum"
+            assert st[1] == acc, f"{loss}/{accu} accuracy count"
+
+
+def test_seed_kernel_loss_only_and_accumulation(dl, oracle):
+    rng = np.random.default_rng(77)
+    q = rng.standard_normal((33, 12)).astype(np.float32)
+    y = rng.standard_normal((33, 12)).astype(np.float32)
+    _, total, acc = oracle.loss_seed(LOSS["MSE"], ACCU["DISTANCE"], 0.49, ACT["LINEAR"], q, q, y, want_dz=False)
+    stats = torch.zeros(2, dtype=torch.float64, device="cuda")
+    for _ in range(3):  # the sums accumulate until the caller clears them, like the reference's
+        assert dl.loss_seed(LOSS["MSE"], ACCU["DISTANCE"], 0.49, ACT["LINEAR"], None, dev(q), dev(y), stats,
+                            want_dz=False) is None
+    st = host(stats)
+    assert st[0] == pytest.approx(3 * total, rel=1e-6) and st[1] == 3 * acc
+
+
+def test_seed_kernel_empty_and_refused(dl):
+    e = torch.empty((0, 5), device="cuda")
+    assert dl.loss_seed(LOSS["MSE"], ACCU["DISTANCE"], 0.49, ACT["LINEAR"], e, e, e).shape == (0, 5)
+    t = torch.zeros((2, 3), device="cuda")
+    for loss, accu, act in [(LOSS["MAPE"], ACCU["DISTANCE"], ACT["LINEAR"]), (LOSS["SMAPE"], ACCU["SIGN"], ACT["ELU"]),
+                            (1, ACCU["DISTANCE"], ACT["LINEAR"]), (LOSS["MSE"], ACCU["R"], ACT["LINEAR"]),
+                            (LOSS["MSE"], ACCU["DISTANCE"], ACT["SOFTMAX"]), (LOSS["MSE"], ACCU["DISTANCE"], 18)]:
+        with pytest.raises(RuntimeError):
+            dl.loss_seed(loss, accu, 0.49, act, t, t, t)
+
+
+@pytest.mark.parametrize("name", list(regress_cases()))
+def test_gpu_model_step_against_golden(model_factory, name):
+    g = load_regress_golden()
+    M = build_regress_model(model_factory, g, name, 0)
+    check_regress_step(M, g, name, 0, TR)
+
+
+@pytest.mark.parametrize("name", [n for n, c in regress_cases().items() if c[6] != "onehot"])
+def test_gpu_model_epochs_against_golden(model_factory, name):
+    g = load_regress_golden()
+    M = build_regress_model(model_factory, g, name, 0, max_batch=7, hyper=(0.5, 1e-5, 3.0, 5.0))
+    check_regress_epochs(M, g, name, 0, 4 * TR)
+
+
+def test_gpu_model_refuses_unmanaged_losses(model_factory):
+    g = load_regress_golden()
+    name = "linear_mse_distance"
+    M = build_regress_model(model_factory, g, name, 0)
+    M.set_loss(LOSS["MAPE"], ACCU["DISTANCE"], 0.49)
+    with pytest.raises(RuntimeError):
+        M.step(1, g[name + "_X"], g[name + "_Y"], backward=True)
+    with pytest.raises(RuntimeError):
+        M.set_loss(LOSS["MSE"], ACCU["DISTANCE"], 1.5)  # Set__Accurancy_Variance: within [0, 1]
