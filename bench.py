@@ -198,8 +198,8 @@ def bench_c1(args):
     """Workload c1: MLP 784-512-512-10, batch 128, batch renorm + ReLU hidden layers, softmax +
     cross-entropy output, through the Model / Driver facade.  A step is one forward + error +
     backward + parameter-gradient pass over one batch of 128 rows (data set resident in HBM); every
-    64 steps Driver::train ends in one Adam update.  Launch- and latency-bound: about 25 kernel
-    launches of a few microseconds each per step."""
+    64 steps Driver::train ends in one Adam update.  Latency-bound: about 25 kernels of a few
+    microseconds each per step, replayed as one recorded HIP graph per batch."""
     import numpy as np
     from __graft_entry__ import load_package
     from oracle.binding import ACT, NORM, OPT
@@ -229,7 +229,10 @@ def bench_c1(args):
     M.set_parameters(p)
     M.set_optimizer(OPT["ADAM"], adam_lr=1e-3)
     epochs = max(1, args.steps // per_epoch)
-    for _ in range(max(1, args.warmup // per_epoch)):
+    # the driver launches the first epoch kernel by kernel, records the second into one HIP graph per
+    # batch and replays from the third on: at least those two stay outside the timed region
+    args.warmup = max(args.warmup, 2 * per_epoch)
+    for _ in range(args.warmup // per_epoch):
         M.train_epoch(X, Y)
     t0 = time.perf_counter()
     for _ in range(epochs):
@@ -239,7 +242,7 @@ def bench_c1(args):
     ms = dt / steps * 1e3
     flops = 2.0 * B * (784 * 512 + 512 * 512 + 512 * 10) * 2 + 2.0 * B * (512 * 512 + 512 * 10)  # fwd + dW, dX of layers 2, 3
     roof = {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "traffic": None, "kernel": "whole step (launch-bound: the GEMMs are 128 x 512 x 784 and smaller)"}
+            "traffic": None, "kernel": "whole step (latency-bound: the GEMMs are 128 x 512 x 784 and smaller; each batch is one HIP graph replay)"}
     roof["frac"] = roof["achieved"] / roof["peak"]
     cpu = None
     if args.cpu_rows != 0:

@@ -101,6 +101,7 @@ Model::~Model(void) {
     }
   if (impl_->h_stage != nullptr) (void)hipHostFree(impl_->h_stage);
   if (impl_->ctx != nullptr) (void)dlmi_ctx_destroy(impl_->ctx);
+  if (impl_->stream != nullptr) (void)hipStreamDestroy(impl_->stream);
   delete[] bernoulli;
   delete[] ptr_array_layers;
   delete[] ptr_array_parameters;
@@ -149,7 +150,15 @@ bool Model::compile(size_t const n_layers, size_t const number_recurrent_depth_r
       if (lp[i + j].type_layer != LAYER::FULLY_CONNECTED) return fail("compile: a residual block holds fully-connected layers only");
     i += depth;
   }
-  if (dlmi_ctx_create(&impl_->ctx, 0, nullptr) != DLMI_OK)
+  // A stream of the model's own (default priority; a blocking one, so the synchronous copies of the
+  // accessors stay ordered with it): the launches of a mini-batch can be recorded on it, which the
+  // null stream does not allow.
+  if (impl_->stream == nullptr && hipStreamCreate(&impl_->stream) != hipSuccess) {
+    (void)hipGetLastError();
+    impl_->stream = nullptr;
+    return fail("compile: no gfx950 device / stream (there is no CPU path)");
+  }
+  if (dlmi_ctx_create(&impl_->ctx, 0, impl_->stream) != DLMI_OK)
     return fail("compile: no gfx950 device / context (there is no CPU path)");
   type = type_network_received;
   seq_w = 1;
@@ -916,6 +925,46 @@ void Model::seed_error(size_t const B, float const *d_targets) {
     }
   }
   impl_->n_loss_values += B * o.n_out;  // update_loss counts every output (compute_loss.cpp:50-52)
+}
+
+// ---------------------------------------------------------------- what a recorded batch depends on
+void *Model::native_stream(void) const { return static_cast<void *>(impl_->stream); }
+
+void Model::account_replayed_batch(size_t const batch_size, float const *d_inputs) {
+  if (ptr_array_layers == nullptr) return;
+  impl_->n_loss_values += batch_size * ptr_array_layers[total_layers - 1].n_out;
+  impl_->cur_input = d_inputs;
+  impl_->out_valid = false;
+  impl_->out_batch = batch_size;
+}
+
+uint64_t Model::launch_signature(void) const {
+  if (ptr_array_layers == nullptr) return 0;
+  uint64_t h = 1469598103934665603ull;  // FNV-1a over the raw bytes of every value below
+  auto mix = [&h](void const *p, size_t n) {
+    unsigned char const *b = static_cast<unsigned char const *>(p);
+    for (size_t i = 0; i != n; ++i) { h ^= b[i]; h *= 1099511628211ull; }
+  };
+#define DLMI_MIX(v) mix(&(v), sizeof(v))
+  DLMI_MIX(total_layers); DLMI_MIX(total_parameters); DLMI_MIX(impl_->allocated_batch);
+  DLMI_MIX(impl_->d_params); DLMI_MIX(impl_->d_dparams); DLMI_MIX(impl_->d_mov_mean); DLMI_MIX(impl_->d_mov_std);
+  DLMI_MIX(impl_->d_stats); DLMI_MIX(impl_->d_input); DLMI_MIX(impl_->d_input_grad);
+  DLMI_MIX(type_loss_function); DLMI_MIX(type_accuracy_function); DLMI_MIX(acc_var);
+  DLMI_MIX(normalization_momentum_average); DLMI_MIX(normalization_epsilon);
+  DLMI_MIX(batch_renormalization_r_correction_maximum); DLMI_MIX(batch_renormalization_d_correction_maximum);
+  DLMI_MIX(dropout_backward_mode); DLMI_MIX(type_state_propagation);
+  for (size_t i = 0; i != total_layers; ++i) {
+    Layer const &l = ptr_array_layers[i];
+    if (l.type_layer == LAYER::RESIDUAL) return 0;  // its backward clears a buffer with a memset: not recorded
+    DLMI_MIX(l.type_layer); DLMI_MIX(l.n_out); DLMI_MIX(l.n_inp); DLMI_MIX(l.type_activation_function);
+    DLMI_MIX(l.type_normalization); DLMI_MIX(l.use_layer_normalization_before_activation); DLMI_MIX(l.type_dropout);
+    DLMI_MIX(l.dropout_values[0]); DLMI_MIX(l.first_connection_index); DLMI_MIX(l.first_bias_connection_index);
+    DLMI_MIX(l.scale_index); DLMI_MIX(l.shift_index); DLMI_MIX(l.unit_index);
+    DLMI_MIX(l.d_summations); DLMI_MIX(l.d_outputs); DLMI_MIX(l.d_errors); DLMI_MIX(l.d_af_values);
+    DLMI_MIX(l.d_block_values); DLMI_MIX(l.d_mean); DLMI_MIX(l.d_std); DLMI_MIX(l.d_r); DLMI_MIX(l.d_d); DLMI_MIX(l.d_mask);
+  }
+#undef DLMI_MIX
+  return h != 0 ? h : 1;
 }
 
 // ---------------------------------------------------------------- loss / accuracy bookkeeping

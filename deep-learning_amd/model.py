@@ -27,7 +27,7 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_model_glorot_uniform", "dlmi_model_init_uniform", "dlmi_model_set_bound_hyper", "dlmi_model_set_constraints",
     "dlmi_model_set_rprop", "dlmi_model_set_rprop_loss", "dlmi_model_set_warm_restarts",
     "dlmi_model_dropout_bernoulli", "dlmi_model_get_dropout_mask", "dlmi_model_set_loss", "dlmi_model_reset_loss",
-    "dlmi_model_loss_accu",
+    "dlmi_model_loss_accu", "dlmi_driver_set_record_batches", "dlmi_driver_recorded_batches",
 ]
 
 LAYER_FULLY_CONNECTED, LAYER_RESIDUAL = 3, 9  # v1/data/enum/layer.hpp
@@ -264,11 +264,19 @@ class Model:
             drivers[key] = (vp(d), X, Y)  # the arrays stay alive with the key
         return drivers[key][0]
 
-    def train_epoch(self, X, Y, resample_masks=False, on_device=True):
+    def train_epoch(self, X, Y, resample_masks=False, on_device=True, record_batches=None):
+        """record_batches: None leaves Driver::record_batches as it is (on, unless DLMI_RECORD_BATCHES=0)."""
         out = (ctypes.c_double * 2)()
-        self._ok(self.lib.dlmi_driver_train(self._driver(X, Y, on_device), c_int(int(resample_masks)), out),
-                 "Driver::train")
+        d = self._driver(X, Y, on_device)
+        if record_batches is not None:
+            self.lib.dlmi_driver_set_record_batches(d, c_int(int(record_batches)))
+        self._ok(self.lib.dlmi_driver_train(d, c_int(int(resample_masks)), out), "Driver::train")
         return out[0], out[1]
+
+    def recorded_batches(self, X, Y, on_device=True):
+        """Mini-batches of this data set's driver that are held as HIP graphs."""
+        self.lib.dlmi_driver_recorded_batches.restype = c_sz
+        return int(self.lib.dlmi_driver_recorded_batches(self._driver(X, Y, on_device)))
 
     def evalt(self, X, Y, on_device=True):
         out = (ctypes.c_double * 2)()

@@ -19,6 +19,7 @@
 #define DLMI_DRIVER_HPP
 
 #include <cstddef>
+#include <vector>
 #include <string>
 
 #include "dlmi_model.hpp"
@@ -86,6 +87,14 @@ class Driver {
   bool resample_dropout_masks = true;
   // false: never keep the data set in HBM
   bool keep_dataset_on_device = true;
+  // true: once an epoch has run kernel by kernel (so every buffer exists), train_st records the
+  // launches of each mini-batch (forward, seed, backward, weight gradients) into a HIP graph per
+  // mini-batch and replays those in later epochs: a small network's epoch is bound by launch
+  // latency, not by its kernels.  The graphs are dropped and recorded again whenever
+  // Model::launch_signature() or the data set changes.  Needs the data set resident in HBM.
+  // DLMI_RECORD_BATCHES=0 in the environment makes false the default.
+  bool record_batches = true;
+  size_t recorded_batches(void) const { return graphs_.size(); }
 
   Dataset &dataset;
   v1::ENV::TYPE env_type;
@@ -93,8 +102,13 @@ class Driver {
 
  private:
   bool make_resident(void);
+  void train_batch(size_t i, size_t batch_size, size_t batch_size_max, bool resident);
+  void drop_graphs(void);
   float *d_X_ = nullptr, *d_Y_ = nullptr;
   bool resident_tried_ = false;
+  std::vector<void *> graphs_;   // hipGraphExec_t per mini-batch, empty until recorded
+  uint64_t graphs_signature_ = 0;
+  bool warmed_up_ = false, recording_failed_ = false;
 };
 
 }  // namespace dlmi

@@ -105,6 +105,10 @@ void dlmi_driver_destroy(dlmi_driver *d);
 /* Driver::train() / Driver::evalt(); out[0] = loss, out[1] = accuracy in percent (get_loss / get_accu of env). */
 int dlmi_driver_train(dlmi_driver *d, int resample_dropout_masks, double *out);
 int dlmi_driver_evalt(dlmi_driver *d, double *out);
+/* Driver::record_batches (replay of each mini-batch's launches as a HIP graph from the third epoch of a
+ * configuration on; on by default) and the number of mini-batches currently held as graphs */
+void dlmi_driver_set_record_batches(dlmi_driver *d, int on);
+size_t dlmi_driver_recorded_batches(dlmi_driver const *d);
 
 /* ---- MNIST reader (data/dataset/mnist.cpp:56-227): IDX files of `workdir`, pixels / 255,
  * one-hot labels over 10 classes.  env = ENV::TRAIN (1) reads the train pair, any other

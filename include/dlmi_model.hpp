@@ -249,6 +249,17 @@ class Model {
   double get_accuracy_sum(void) const; // number of correct arg-max predictions since then
   char const *last_error(void) const;
   bool synchronize(void) const;
+  // The stream every kernel of this model is launched on (a hipStream_t), and a hash of
+  // everything the kernels of one batch take by value or by address (layer settings,
+  // hyper-parameters, propagation state, buffer addresses): two batches of the same size
+  // over the same data addresses launch identical kernels while it stays the same.  0: the
+  // model holds a layer whose batch cannot be recorded into a HIP graph (a residual block).
+  void *native_stream(void) const;
+  uint64_t launch_signature(void) const;
+  // Host-side bookkeeping of compute_error() for a mini-batch whose launches were replayed from a
+  // recording instead of being issued through it (the number of loss terms behind get_loss(), which
+  // batch get_out() reads).
+  void account_replayed_batch(size_t const batch_size, float const *d_inputs);
 
   // ---- public state, as in the reference ------------------------------------
   size_t total_layers = 0, total_parameters = 0, total_weights = 0, total_bias = 0;
