@@ -40,7 +40,7 @@ C_ABI_SYMBOLS = [
     "dlmi_softmax_fwd", "dlmi_dropout_fwd", "dlmi_identity_add", "dlmi_softmax_ce_seed",
     "dlmi_fused_norm_act_fwd", "dlmi_fused_norm_act_bwd", "dlmi_fused_norm_act_infer", "dlmi_fc_norm_act_fwd",
     "dlmi_opt_gd", "dlmi_opt_gd_momentum", "dlmi_opt_adam", "dlmi_zero_padded_identity_fwd", "dlmi_residual_bwd",
-    "dlmi_opt_adabound", "dlmi_clip_gradient", "dlmi_max_norm_rows", "dlmi_opt_irprop_plus", "dlmi_loss_seed",
+    "dlmi_opt_adabound", "dlmi_clip_gradient", "dlmi_max_norm_rows", "dlmi_opt_irprop_plus", "dlmi_loss_seed", "dlmi_zero",
 ]
 
 
@@ -294,6 +294,11 @@ class Dlmi:
         dZ = self.empty(B, H)
         self._ck(self.lib.dlmi_softmax_ce_seed(self.ctx, c_sz(B), c_sz(H), _p(q), _p(y), _p(dZ), _p(stats)))
         return dZ
+
+    def zero(self, t):
+        self._chk(t)
+        self._ck(self.lib.dlmi_zero(self.ctx, c_sz(t.numel()), _p(t)))
+        return t
 
     def loss_seed(self, loss, accu, accu_threshold, act, z, q, y, stats=None, want_dz=True):
         """Seed gradient of an element-wise output layer; stats: optional device tensor of 2 float64 accumulators."""

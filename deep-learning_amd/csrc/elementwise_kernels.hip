@@ -98,6 +98,13 @@ __global__ __launch_bounds__(kEwBlock) void k_residual_bwd(float const *__restri
   }
 }
 
+// ---- clearing a buffer with a kernel (the reference's memset of the error arrays,
+// bwp_st.cpp:115): unlike a memset node, this can be recorded into a HIP graph
+__global__ __launch_bounds__(kEwBlock) void k_zero(float *__restrict__ p, size_t n) {
+  size_t const stride = static_cast<size_t>(gridDim.x) * kEwBlock;
+  for (size_t e = static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x; e < n; e += stride) p[e] = 0.0f;
+}
+
 // ---- per-unit row kernels: element e = b*H + j, unit j = e % H ----------------
 // mode 0: Z += bias                                     (fwp_st.cpp:4498-4516)
 // mode 1: dropout, kind/per_element/scale in the args   (fwp_st.cpp:4830-4904)
@@ -326,6 +333,15 @@ int dlmi_residual_bwd(dlmi_ctx *ctx, size_t B, size_t input_size, size_t derivat
                      B, input_size, derivative_size, Hc, input_size > derivative_size ? pad : 0,
                      input_size < derivative_size ? pad : 0);
   DLMI_LAUNCH_CHECK(ctx, "k_residual_bwd");
+  return DLMI_OK;
+}
+
+int dlmi_zero(dlmi_ctx *ctx, size_t n, float *p) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  if (n == 0) return DLMI_OK;
+  DLMI_REQUIRE(ctx, p != nullptr, "null pointer");
+  hipLaunchKernelGGL(k_zero, dim3(ew_grid(ctx, n)), dim3(kEwBlock), 0, ctx->stream, p, n);
+  DLMI_LAUNCH_CHECK(ctx, "k_zero");
   return DLMI_OK;
 }
 

@@ -955,8 +955,8 @@ uint64_t Model::launch_signature(void) const {
   DLMI_MIX(dropout_backward_mode); DLMI_MIX(type_state_propagation);
   for (size_t i = 0; i != total_layers; ++i) {
     Layer const &l = ptr_array_layers[i];
-    if (l.type_layer == LAYER::RESIDUAL) return 0;  // its backward clears a buffer with a memset: not recorded
-    DLMI_MIX(l.type_layer); DLMI_MIX(l.n_out); DLMI_MIX(l.n_inp); DLMI_MIX(l.type_activation_function);
+    DLMI_MIX(l.type_layer); DLMI_MIX(l.n_out); DLMI_MIX(l.n_inp); DLMI_MIX(l.n_units); DLMI_MIX(l.feed_index);
+    DLMI_MIX(l.block_depth); DLMI_MIX(l.pooling_values[2]); DLMI_MIX(l.type_activation_function);
     DLMI_MIX(l.type_normalization); DLMI_MIX(l.use_layer_normalization_before_activation); DLMI_MIX(l.type_dropout);
     DLMI_MIX(l.dropout_values[0]); DLMI_MIX(l.first_connection_index); DLMI_MIX(l.first_bias_connection_index);
     DLMI_MIX(l.scale_index); DLMI_MIX(l.shift_index); DLMI_MIX(l.unit_index);
@@ -1108,7 +1108,7 @@ bool Model::backward_block(size_t const B, size_t const ri) {
   Layer &last = ptr_array_layers[ri + D];
   size_t const HD = last.n_out;
   float *g = last.d_errors;
-  if (!hip_ok(hipMemsetAsync(g, 0, B * HD * sizeof(float), impl_->stream), impl_->err, "memset")) return false;
+  if (dlmi_zero(ctx, B * HD, g) != DLMI_OK) return fail("backward_pass: dlmi_zero");
   if (dlmi_residual_bwd(ctx, B, r.n_out, HD, pad, r.d_errors, g) != DLMI_OK) return fail("backward_pass: dlmi_residual_bwd");
   if (r.Use__Normalization()) {
     dlmi_fused_desc d = make_desc(*this, r);

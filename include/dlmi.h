@@ -180,6 +180,10 @@ int dlmi_zero_padded_identity_fwd(dlmi_ctx *ctx, size_t B, size_t HA, size_t HB,
 int dlmi_residual_bwd(dlmi_ctx *ctx, size_t B, size_t input_size, size_t derivative_size, size_t padding,
                       float const *d_inputs, float *derivatives);
 
+/* p[0..n) = 0 by a kernel on the context's stream: the clearing of an error array before gradients are
+ * accumulated into it (the memset of bwp_st.cpp:115), in a form that a HIP graph can record. */
+int dlmi_zero(dlmi_ctx *ctx, size_t n, float *p);
+
 /* Softmax + cross-entropy seed gradient of the output layer:
  * dZ_i = sum_k (q_i [i==k] - q_k q_i) * dL_k,  dL_k = (y_k==1 ? -1/clip(q_k,1e-7,1-1e-7) : 0)/B.
  * stats (device, 2 doubles, may be NULL) accumulates { sum of CE losses, number

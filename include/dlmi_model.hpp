@@ -253,7 +253,7 @@ class Model {
   // everything the kernels of one batch take by value or by address (layer settings,
   // hyper-parameters, propagation state, buffer addresses): two batches of the same size
   // over the same data addresses launch identical kernels while it stays the same.  0: the
-  // model holds a layer whose batch cannot be recorded into a HIP graph (a residual block).
+  // model is not compiled.
   void *native_stream(void) const;
   uint64_t launch_signature(void) const;
   // Host-side bookkeeping of compute_error() for a mini-batch whose launches were replayed from a

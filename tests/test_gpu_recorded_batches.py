@@ -84,19 +84,25 @@ def test_regression_output_layer_is_recorded_too(lib):
         b.close()
 
 
-def test_residual_blocks_are_never_recorded(lib):
+def test_residual_blocks_are_recorded_too(lib):
     from deep_learning_amd.model import Net
-    net = Net(lib, [("FC", 10), ("RES", 2), ("FC", 10), ("FC", 10), ("FC", 4)])
-    try:
-        for l in (2, 3):
-            net.set_layer(l, ACT["ELU"])
-        net.set_layer(4, ACT["SOFTMAX"])
+
+    def make():
+        net = Net(lib, [("FC", 10), ("RES", 2), ("FC", 14), ("FC", 10), ("RES", 2), ("FC", 10), ("FC", 6), ("FC", 4)])
+        for l in (2, 3, 5, 6):
+            net.set_layer(l, ACT["ELU"], NORM["BRN"])
+        net.set_layer(1, 0, NORM["BRN"])
+        net.set_layer(7, ACT["SOFTMAX"])
+        net.set_norm_hyper(0.9, 1e-5, 3.0, 5.0)
         net.prepare(8)
         net.glorot_uniform(5)
-        net.set_optimizer(OPT["GD"], lr=0.01)
+        net.set_optimizer(OPT["GD"], lr=0.01, momentum=0.9, nesterov=True)
+        return net
+
+    a, b = make(), make()
+    try:
         X, Y = data(20, 10, 4)
-        for _ in range(3):
-            net.train_epoch(X, Y)
-        assert net.recorded_batches(X, Y) == 0
+        run_pair(a, b, X, Y, 5, [0, 3, 3, 3, 3])
     finally:
-        net.close()
+        a.close()
+        b.close()
