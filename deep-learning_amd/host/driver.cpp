@@ -27,8 +27,10 @@ Driver::Driver(Dataset &dataset_received, ENV::TYPE const &env_type_received, Mo
 }
 
 Driver::~Driver(void) {
-  if (d_X_ != nullptr || d_Y_ != nullptr || !graphs_.empty()) (void)model.synchronize();
-  drop_graphs();
+  if (d_X_ != nullptr || d_Y_ != nullptr || !train_rec_.graphs.empty() || !evalt_rec_.graphs.empty())
+    (void)model.synchronize();
+  drop_graphs(train_rec_);
+  drop_graphs(evalt_rec_);
   if (d_X_ != nullptr) (void)hipFree(d_X_);
   if (d_Y_ != nullptr) (void)hipFree(d_Y_);
 }
@@ -108,49 +110,38 @@ double Driver::train(void) {
   return loss;
 }
 
-void Driver::evalt_st(void) {
-  size_t const n_data = dataset.n_data, batch_size_max = model.batch_size;
-  size_t const n_batch = static_cast<size_t>(std::ceil(static_cast<double>(n_data) / static_cast<double>(batch_size_max)));
-  bool const resident = make_resident();
-  for (size_t i = 0; i != n_batch; ++i) {
-    size_t const batch_size = i + 1 != n_batch ? batch_size_max : n_data - i * batch_size_max;
-    if (resident) {
-      model.forward_pass_device(batch_size, d_X_ + i * batch_size_max * dataset.n_inp);
-      model.compute_loss_device(batch_size, d_Y_ + i * batch_size_max * dataset.n_out);
-    } else {
-      model.forward_pass(batch_size, dataset.Xm + i * batch_size_max);
-      model.compute_loss(batch_size, dataset.Ym + i * batch_size_max);
-    }
-  }
-}
+void Driver::evalt_st(void) { run_batches(evalt_rec_, false); }
 
-void Driver::train_batch(size_t const i, size_t const batch_size, size_t const batch_size_max, bool const resident) {
+// One mini-batch: forward and loss (evaluation), or forward, seed gradient, backward and
+// parameter gradients (training).
+void Driver::one_batch(size_t const i, size_t const batch_size, size_t const batch_size_max, bool const resident,
+                       bool const training) {
   if (resident) {
-    model.forward_pass_device(batch_size, d_X_ + i * batch_size_max * dataset.n_inp);
-    model.compute_error_device(batch_size, d_Y_ + i * batch_size_max * dataset.n_out);
+    float const *const x = d_X_ + i * batch_size_max * dataset.n_inp, *const y = d_Y_ + i * batch_size_max * dataset.n_out;
+    model.forward_pass_device(batch_size, x);
+    if (training) model.compute_error_device(batch_size, y); else model.compute_loss_device(batch_size, y);
   } else {
     model.forward_pass(batch_size, dataset.Xm + i * batch_size_max);
-    model.compute_error(batch_size, dataset.Ym + i * batch_size_max);
+    if (training) model.compute_error(batch_size, dataset.Ym + i * batch_size_max);
+    else model.compute_loss(batch_size, dataset.Ym + i * batch_size_max);
   }
+  if (!training) return;
   model.backward_pass(batch_size);
   model.update_derivatives(batch_size, model.ptr_array_layers + 1, model.ptr_last_layer);
 }
 
-void Driver::drop_graphs(void) {
-  for (void *g : graphs_) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(g));
-  graphs_.clear();
+void Driver::drop_graphs(Recorded &rec) {
+  for (void *g : rec.graphs) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(g));
+  rec.graphs.clear();
 }
 
-void Driver::train_st(void) {
+// The mini-batch loop of evalt_st / train_st (driver.cpp:244-257, 294-336).  Recorded mini-batches:
+// the first pass of a configuration runs kernel by kernel (buffers and scratch memory reach their
+// final size), the second is recorded into one HIP graph per mini-batch, later ones replay.
+void Driver::run_batches(Recorded &rec, bool const training) {
   size_t const n_data = dataset.n_data, batch_size_max = model.batch_size;
   size_t const n_batch = static_cast<size_t>(std::ceil(static_cast<double>(n_data) / static_cast<double>(batch_size_max)));
   bool const resident = make_resident();
-  // iRPROP compares the loss of this epoch with that of the previous one (driver.cpp:269-273, 337)
-  bool const irprop = v1::OPTIMIZER::IRPROP_MINUS == model.type_optimizer_function ||
-                      v1::OPTIMIZER::IRPROP_PLUS == model.type_optimizer_function;
-  if (irprop) model.loss_rprop_tm1 = model.loss_rprop;
-  // Recorded mini-batches: the first epoch of a configuration runs kernel by kernel (buffers and
-  // scratch memory reach their final size), the second is recorded, later ones replay.
   hipStream_t const stream = static_cast<hipStream_t>(model.native_stream());
   uint64_t sig = resident && record_batches && !recording_failed_ ? model.launch_signature() : 0;
   if (sig != 0) {
@@ -158,50 +149,58 @@ void Driver::train_st(void) {
     for (uint64_t v : extra) sig = (sig ^ v) * 1099511628211ull;
     if (sig == 0) sig = 1;
   }
-  if (sig != graphs_signature_) {
-    drop_graphs();
-    graphs_signature_ = sig;
-    warmed_up_ = false;
+  if (sig != rec.signature) {
+    drop_graphs(rec);
+    rec.signature = sig;
+    rec.warmed_up = false;
   }
-  bool const replay = sig != 0 && graphs_.size() == n_batch;
-  bool const record = sig != 0 && !replay && warmed_up_ && model.last_error()[0] == '\0';
+  bool const replay = sig != 0 && rec.graphs.size() == n_batch;
+  bool const record = sig != 0 && !replay && rec.warmed_up && model.last_error()[0] == '\0';
   for (size_t i = 0; i != n_batch; ++i) {
     size_t const batch_size = i + 1 != n_batch ? batch_size_max : n_data - i * batch_size_max;
     if (replay) {
-      if (hipGraphLaunch(static_cast<hipGraphExec_t>(graphs_[i]), stream) != hipSuccess) {
+      if (hipGraphLaunch(static_cast<hipGraphExec_t>(rec.graphs[i]), stream) != hipSuccess) {
         (void)hipGetLastError();
-        recording_failed_ = true;  // this epoch goes on kernel by kernel, and so do all later ones
+        recording_failed_ = true;  // this pass goes on kernel by kernel, and so do all later ones
         for (size_t j = i; j != n_batch; ++j)
-          train_batch(j, j + 1 != n_batch ? batch_size_max : n_data - j * batch_size_max, batch_size_max, resident);
+          one_batch(j, j + 1 != n_batch ? batch_size_max : n_data - j * batch_size_max, batch_size_max, resident, training);
         break;
       }
       model.account_replayed_batch(batch_size, d_X_ + i * batch_size_max * dataset.n_inp);
       continue;
     }
-    if (record && graphs_.size() == i) {
+    if (record && rec.graphs.size() == i) {
       hipGraph_t graph = nullptr;
       hipGraphExec_t exec = nullptr;
       bool ok = hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed) == hipSuccess;
       if (ok) {
-        train_batch(i, batch_size, batch_size_max, resident);
+        one_batch(i, batch_size, batch_size_max, resident, training);
         ok = hipStreamEndCapture(stream, &graph) == hipSuccess && graph != nullptr && model.last_error()[0] == '\0';
       }
       ok = ok && hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) == hipSuccess;
       if (graph != nullptr) (void)hipGraphDestroy(graph);
       if (ok && hipGraphLaunch(exec, stream) == hipSuccess) {
-        graphs_.push_back(static_cast<void *>(exec));
+        rec.graphs.push_back(static_cast<void *>(exec));
         continue;
       }
       (void)hipGetLastError();
       if (exec != nullptr) (void)hipGraphExecDestroy(exec);
       recording_failed_ = true;  // nothing of this batch has run yet: fall through to the plain launches
     }
-    train_batch(i, batch_size, batch_size_max, resident);
+    one_batch(i, batch_size, batch_size_max, resident, training);
   }
-  if (graphs_.size() != n_batch && !graphs_.empty()) drop_graphs();  // a partial recording is of no use
-  warmed_up_ = true;
+  if (rec.graphs.size() != n_batch && !rec.graphs.empty()) drop_graphs(rec);  // a partial recording is of no use
+  rec.warmed_up = true;
+}
+
+void Driver::train_st(void) {
+  // iRPROP compares the loss of this epoch with that of the previous one (driver.cpp:269-273, 337)
+  bool const irprop = v1::OPTIMIZER::IRPROP_MINUS == model.type_optimizer_function ||
+                      v1::OPTIMIZER::IRPROP_PLUS == model.type_optimizer_function;
+  if (irprop) model.loss_rprop_tm1 = model.loss_rprop;
+  run_batches(train_rec_, true);
   if (irprop) model.loss_rprop = std::fabs(model.get_loss(v1::ENV::NONE));  // one device-to-host read of the loss sum
-  model.Update_Parameter(n_data, n_data);
+  model.Update_Parameter(dataset.n_data, dataset.n_data);
 }
 
 }  // namespace dlmi

@@ -327,7 +327,9 @@ void dlmi_driver_destroy(dlmi_driver *d) { delete d; }
 void dlmi_driver_set_record_batches(dlmi_driver *d, int on) {
   if (d != nullptr) d->drv->record_batches = on != 0;
 }
-size_t dlmi_driver_recorded_batches(dlmi_driver const *d) { return d != nullptr ? d->drv->recorded_batches() : 0; }
+size_t dlmi_driver_recorded_batches(dlmi_driver const *d) {
+  return d != nullptr ? d->drv->recorded_batches() + d->drv->recorded_evalt_batches() : 0;
+}
 int dlmi_driver_train(dlmi_driver *d, int resample_dropout_masks, double *out) {
   if (d == nullptr || out == nullptr) return 0;
   d->drv->resample_dropout_masks = resample_dropout_masks != 0;

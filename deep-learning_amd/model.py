@@ -273,8 +273,11 @@ class Model:
         self._ok(self.lib.dlmi_driver_train(d, c_int(int(resample_masks)), out), "Driver::train")
         return out[0], out[1]
 
+    def set_record_batches(self, X, Y, on, on_device=True):
+        self.lib.dlmi_driver_set_record_batches(self._driver(X, Y, on_device), c_int(int(on)))
+
     def recorded_batches(self, X, Y, on_device=True):
-        """Mini-batches of this data set's driver that are held as HIP graphs."""
+        """Mini-batches of this data set's driver that are held as HIP graphs (training plus evaluation passes)."""
         self.lib.dlmi_driver_recorded_batches.restype = c_sz
         return int(self.lib.dlmi_driver_recorded_batches(self._driver(X, Y, on_device)))
 

@@ -87,14 +87,15 @@ class Driver {
   bool resample_dropout_masks = true;
   // false: never keep the data set in HBM
   bool keep_dataset_on_device = true;
-  // true: once an epoch has run kernel by kernel (so every buffer exists), train_st records the
-  // launches of each mini-batch (forward, seed, backward, weight gradients) into a HIP graph per
-  // mini-batch and replays those in later epochs: a small network's epoch is bound by launch
+  // true: once a pass has run kernel by kernel (so every buffer exists), train_st and evalt_st
+  // record the launches of each mini-batch (forward, seed or loss, backward, weight gradients) into
+  // a HIP graph per mini-batch and replay those in later passes: a small network's epoch is bound by launch
   // latency, not by its kernels.  The graphs are dropped and recorded again whenever
   // Model::launch_signature() or the data set changes.  Needs the data set resident in HBM.
   // DLMI_RECORD_BATCHES=0 in the environment makes false the default.
   bool record_batches = true;
-  size_t recorded_batches(void) const { return graphs_.size(); }
+  size_t recorded_batches(void) const { return train_rec_.graphs.size(); }        // of train_st
+  size_t recorded_evalt_batches(void) const { return evalt_rec_.graphs.size(); }  // of evalt_st
 
   Dataset &dataset;
   v1::ENV::TYPE env_type;
@@ -102,13 +103,17 @@ class Driver {
 
  private:
   bool make_resident(void);
-  void train_batch(size_t i, size_t batch_size, size_t batch_size_max, bool resident);
-  void drop_graphs(void);
+  struct Recorded {
+    std::vector<void *> graphs;  // hipGraphExec_t per mini-batch, empty until recorded
+    uint64_t signature = 0;      // what the graphs were recorded for
+    bool warmed_up = false;      // a plain pass has run for that signature
+  };
+  void one_batch(size_t i, size_t batch_size, size_t batch_size_max, bool resident, bool training);
+  void run_batches(Recorded &rec, bool training);
+  void drop_graphs(Recorded &rec);
   float *d_X_ = nullptr, *d_Y_ = nullptr;
-  bool resident_tried_ = false;
-  std::vector<void *> graphs_;   // hipGraphExec_t per mini-batch, empty until recorded
-  uint64_t graphs_signature_ = 0;
-  bool warmed_up_ = false, recording_failed_ = false;
+  bool resident_tried_ = false, recording_failed_ = false;
+  Recorded train_rec_, evalt_rec_;
 };
 
 }  // namespace dlmi

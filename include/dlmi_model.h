@@ -106,7 +106,7 @@ void dlmi_driver_destroy(dlmi_driver *d);
 int dlmi_driver_train(dlmi_driver *d, int resample_dropout_masks, double *out);
 int dlmi_driver_evalt(dlmi_driver *d, double *out);
 /* Driver::record_batches (replay of each mini-batch's launches as a HIP graph from the third epoch of a
- * configuration on; on by default) and the number of mini-batches currently held as graphs */
+ * configuration on; on by default) and the number of mini-batches currently held as graphs (training plus evaluation passes) */
 void dlmi_driver_set_record_batches(dlmi_driver *d, int on);
 size_t dlmi_driver_recorded_batches(dlmi_driver const *d);
 

@@ -39,6 +39,8 @@ def data(n, k, h, onehot=True, seed=3):
 
 
 def run_pair(a, b, X, Y, epochs, expect_recorded):
+    """expect_recorded[e]: mini-batches of the TRAINING pass held as graphs after epoch e; the evaluation pass
+    that follows each epoch is recorded on the same schedule (plain, recorded, replayed ...)."""
     for e in range(epochs):
         ra = a.train_epoch(X, Y, resample_masks=True, record_batches=False)
         rb = b.train_epoch(X, Y, resample_masks=True, record_batches=True)
@@ -47,9 +49,10 @@ def run_pair(a, b, X, Y, epochs, expect_recorded):
         ma, mb = a.get_moving(), b.get_moving()
         assert np.array_equal(ma[0], mb[0]) and np.array_equal(ma[1], mb[1]), f"epoch {e}: moving statistics differ"
         assert a.recorded_batches(X, Y) == 0
-        assert b.recorded_batches(X, Y) == expect_recorded[e], f"epoch {e}"
-        ea, eb = a.evalt(X, Y), b.evalt(X, Y)  # unrecorded work between the replays
-        assert eb[0] == pytest.approx(ea[0], rel=1e-9) and eb[1] == ea[1]
+        ea, eb = a.evalt(X, Y), b.evalt(X, Y)
+        assert eb[0] == pytest.approx(ea[0], rel=1e-9) and eb[1] == ea[1], f"epoch {e}: evaluation {ea} / {eb}"
+        assert b.recorded_batches(X, Y) == 2 * expect_recorded[e], f"epoch {e}, after its evaluation pass"
+        assert a.recorded_batches(X, Y) == 0
 
 
 def test_replays_match_plain_launches_epoch_by_epoch(lib):
