@@ -128,7 +128,7 @@ bool Model::synchronize(void) const {
 // ---------------------------------------------------------------- construction
 bool Model::compile(size_t const n_layers, size_t const number_recurrent_depth_received,
                     MODEL::TYPE const type_network_received, Layer_Parameters const *const lp,
-                    size_t const /*allowable_memory: HBM is not budgeted the way host RAM is*/) {
+                    size_t const allowable_memory) {
   if (ptr_array_layers != nullptr) return fail("compile: the model is already compiled");
   if (n_layers < 2 || lp == nullptr) return fail("compile: need an input layer and an output layer");
   if (number_recurrent_depth_received != 1) return fail("compile: only seq_w = 1 (no recurrence) is on this path");
@@ -161,6 +161,14 @@ bool Model::compile(size_t const n_layers, size_t const number_recurrent_depth_r
   if (dlmi_ctx_create(&impl_->ctx, 0, impl_->stream) != DLMI_OK)
     return fail("compile: no gfx950 device / context (there is no CPU path)");
   type = type_network_received;
+  // the reference budgets host memory (model.hpp:2528); here the same number budgets device memory.
+  // 0: all of the device's memory.
+  maximum_allowable_memory_bytes = allowable_memory;
+  if (allowable_memory == 0) {
+    size_t free_bytes = 0, total_bytes = 0;
+    if (hipMemGetInfo(&free_bytes, &total_bytes) != hipSuccess) { (void)hipGetLastError(); total_bytes = ~size_t(0); }
+    maximum_allowable_memory_bytes = total_bytes;
+  }
   seq_w = 1;
   total_layers = n_layers;
   ptr_array_layers = new Layer[n_layers];
@@ -442,9 +450,63 @@ bool Model::allocate_batch(size_t const n) {
   return true;
 }
 
+// Device bytes that grow with the batch, for `batch` examples (the reference's Get__Batch_Sizeof, for the
+// buffers this layout keeps: allocate_batch() above)
+size_t Model::Get__Batch_Sizeof(size_t const batch) const {
+  if (ptr_array_layers == nullptr) return 0;
+  size_t floats = ptr_array_layers[0].n_out + ptr_array_layers[total_layers - 1].n_out;  // input rows and targets
+  if (total_layers > 1 && ptr_array_layers[1].type_layer == LAYER::RESIDUAL) floats += ptr_array_layers[0].n_out;
+  for (size_t i = 1; i < total_layers; ++i) {
+    Layer const &l = ptr_array_layers[i];
+    if (l.type_layer == LAYER::RESIDUAL) floats += 2 * l.n_out + (l.Use__Normalization() ? l.n_units : 0);
+    else if (l.in_block) floats += 2 * l.n_out + ((l.Use__Normalization() || !l.block_first) ? l.n_inp : 0);
+    else floats += 3 * l.n_out + ((l.Use__Normalization() && !l.use_layer_normalization_before_activation) ? l.n_out : 0);
+  }
+  return floats * sizeof(float) * batch;
+}
+
+// Device bytes of the model with `batch` examples: parameters, gradients, the optimizer's arrays, moving and
+// batch statistics, masks, and the batch buffers (the reference's Get__Sizeof; there are no per-thread copies)
+size_t Model::Get__Sizeof(size_t const /*number_threads*/, size_t const batch) const {
+  if (ptr_array_layers == nullptr) return 0;
+  size_t arrays = 2;  // parameters and their gradients
+  for (float const *s : impl_->d_opt) arrays += s != nullptr ? 1 : 0;
+  size_t bytes = arrays * total_parameters * sizeof(float) + 2 * total_normalized_units * sizeof(float) + 2 * sizeof(double);
+  for (size_t i = 1; i < total_layers; ++i) bytes += ptr_array_layers[i].n_units * (4 * sizeof(float) + 1);
+  return bytes + Get__Batch_Sizeof(batch);
+}
+
+// update_size.cpp:26-116 without its thread dimension: the largest batch, up to the desired one and
+// maximum_batch_size, whose buffers fit maximum_allowable_memory_bytes beside the model itself.
+bool Model::Allouable__Batch_Size(size_t const desired, size_t &batch_allouable, size_t &threads_allouable) const {
+  batch_allouable = threads_allouable = 0;
+  size_t const size_batch = Get__Batch_Sizeof(1), size_network = Get__Sizeof(1, 0);
+  if (maximum_allowable_memory_bytes < size_network) {
+    std::fprintf(stderr, "dlmi: Maximum allowable memory (%zu) is less than the memory allocate (%zu).\n",
+                 maximum_allowable_memory_bytes, size_network + size_batch);
+    return false;
+  }
+  size_t const available = maximum_allowable_memory_bytes - size_network;
+  if (available < size_batch) {
+    std::fprintf(stderr, "dlmi: No enought available memory (%zu) for allocating %zu bytes.\n", available, size_batch);
+    return false;
+  }
+  size_t const fits = available / size_batch;
+  size_t n = desired < maximum_batch_size ? desired : maximum_batch_size;
+  if (n > fits) {
+    std::fprintf(stderr, "dlmi: Can not allocate the optimal batch size (%zu). The batch size allocated will be reduced to %zu.\n",
+                 n, fits);
+    n = fits;
+  }
+  batch_allouable = n;
+  threads_allouable = 1;
+  return true;
+}
+
 bool Model::update_mem_batch_size(size_t const desired, bool const force) {
   if (ptr_array_layers == nullptr) return fail("update_mem_batch_size: the model is not compiled");
-  size_t const n = desired < maximum_batch_size ? desired : maximum_batch_size;  // update_size.cpp:26-116
+  size_t n = 0, threads = 0;
+  if (!Allouable__Batch_Size(desired, n, threads)) return fail("update_mem_batch_size: the memory budget given to compile() does not hold the model with one example");
   if (n == 0) return fail("update_mem_batch_size: batch size 0");
   if (n == impl_->allocated_batch && !force) {
     batch_size = n;

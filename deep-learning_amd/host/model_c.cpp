@@ -38,7 +38,7 @@ dlmi_model *dlmi_model_create(size_t n_layers, size_t const *widths) {
     lp[i].type_layer = LAYER::FULLY_CONNECTED;
     lp[i].unit_parameters[0] = widths[i];
   }
-  if (!h->m.compile(n_layers, 1, MODEL::FEEDFORWARD, lp.data())) {
+  if (!h->m.compile(n_layers, 1, MODEL::FEEDFORWARD, lp.data(), 0)) {
     delete h;
     return nullptr;
   }
@@ -53,7 +53,7 @@ dlmi_model *dlmi_model_create_typed(size_t n_layers, int const *types, size_t co
     lp[i].type_layer = static_cast<LAYER::TYPE>(types[i]);
     lp[i].unit_parameters[0] = units[i];
   }
-  if (!h->m.compile(n_layers, 1, MODEL::FEEDFORWARD, lp.data())) {
+  if (!h->m.compile(n_layers, 1, MODEL::FEEDFORWARD, lp.data(), 0)) {
     delete h;
     return nullptr;
   }
@@ -138,6 +138,13 @@ int dlmi_model_prepare(dlmi_model *h, size_t max_batch) {
   h->m.update_mem_thread_size(max_batch);
   h->m.clear_training_arrays();
   return 1;
+}
+void dlmi_model_set_allowable_memory(dlmi_model *h, size_t bytes) { h->m.maximum_allowable_memory_bytes = bytes; }
+void dlmi_model_memory(dlmi_model const *h, size_t *out) {
+  out[0] = h->m.maximum_allowable_memory_bytes;
+  out[1] = h->m.Get__Sizeof(1, 0);
+  out[2] = h->m.Get__Batch_Sizeof(1);
+  out[3] = h->m.batch_size;
 }
 int dlmi_model_set_loss(dlmi_model *h, int loss, int accu, float accu_variance) {
   h->m.set_loss_fn(static_cast<LOSS_FN::TYPE>(loss));

@@ -28,6 +28,7 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_model_set_rprop", "dlmi_model_set_rprop_loss", "dlmi_model_set_warm_restarts",
     "dlmi_model_dropout_bernoulli", "dlmi_model_get_dropout_mask", "dlmi_model_set_loss", "dlmi_model_reset_loss",
     "dlmi_model_loss_accu", "dlmi_driver_set_record_batches", "dlmi_driver_recorded_batches",
+    "dlmi_model_set_allowable_memory", "dlmi_model_memory",
 ]
 
 LAYER_FULLY_CONNECTED, LAYER_RESIDUAL = 3, 9  # v1/data/enum/layer.hpp
@@ -190,6 +191,15 @@ class Model:
         p = np.empty(self.P, np.float32)
         self._ok(self.lib.dlmi_model_get_derivatives(self.h, _ptr(p), c_sz(self.P)), "get_derivatives")
         return p
+
+    def set_allowable_memory(self, nbytes):
+        """maximum_allowable_memory_bytes: the device-memory budget update_mem_batch_size() sizes the batch for."""
+        self.lib.dlmi_model_set_allowable_memory(self.h, c_sz(nbytes))
+
+    def memory(self):
+        out = (c_sz * 4)()
+        self.lib.dlmi_model_memory(self.h, out)
+        return dict(zip(("budget", "model_bytes", "bytes_per_example", "batch_size"), (int(v) for v in out)))
 
     def set_loss(self, loss, accu, acc_var=0.49):
         """set_loss_fn / set_accu_fn / Set__Accurancy_Variance (after prepare, which selects cross-entropy)."""

@@ -54,6 +54,10 @@ int dlmi_model_set_loss(dlmi_model *m, int loss, int accu, float accu_variance);
  * worth of trials (driver.cpp:95-99) */
 void dlmi_model_reset_loss(dlmi_model *m);
 void dlmi_model_loss_accu(dlmi_model *m, size_t n_data, double *out);
+/* maximum_allowable_memory_bytes (device memory; dlmi_model_create passes 0 = all of the device to compile()),
+ * assigned before dlmi_model_prepare; out[0..3] = that budget, Get__Sizeof(1, 0), Get__Batch_Sizeof(1), batch_size */
+void dlmi_model_set_allowable_memory(dlmi_model *m, size_t bytes);
+void dlmi_model_memory(dlmi_model const *m, size_t *out);
 size_t dlmi_model_total_parameters(dlmi_model const *m);
 size_t dlmi_model_total_normalized_units(dlmi_model const *m);
 /* out[0..5] = first weight index, first bias index, gamma index, beta index, moving-stat index, Use__Bias() */

@@ -163,6 +163,12 @@ class Model {
   bool Set__Accurancy_Variance(real const accurancy_variance_received);  // metrics.cpp:27-52: within [0, 1]
   bool set_max_batch_size(size_t const max_batch_size);
   bool update_mem_batch_size(size_t const desired_batch_size_received, bool const force_update_received = false);
+  // update_size.cpp:26-116, model.hpp:2938-2941: the batch that fits maximum_allowable_memory_bytes (DEVICE memory
+  // here) beside the model, and the sizes it is worked out from.  There is one "thread".
+  bool Allouable__Batch_Size(size_t const desired_batch_size_received, size_t &ref_batch_size_allouable_received,
+                             size_t &ref_number_threads_allouable_received) const;
+  size_t Get__Batch_Sizeof(size_t const batch_size = 1) const;
+  size_t Get__Sizeof(size_t const number_threads = 1, size_t const batch_size = 0) const;
   bool set_mp(bool const) { return true; }
   bool update_mem_thread_size(size_t const) { return true; }
   void merge_mp_derivatives(size_t const, size_t const) {}
@@ -265,6 +271,7 @@ class Model {
   size_t total_layers = 0, total_parameters = 0, total_weights = 0, total_bias = 0;
   size_t total_normalized_units = 0;  // 0 until a layer is normalized; then one slot per unit of EVERY entry, input included
   size_t batch_size = 1, maximum_batch_size = 1, seq_w = 1;
+  size_t maximum_allowable_memory_bytes = 0;  // compile()'s allowable_memory; 0 there = all of the device
   size_t number_threads = 1;
   size_t n_acc_trial = 0, n_time_delay = 0;
   double loss_train = 3.40282e38, loss_valid = 3.40282e38, loss_testg = 3.40282e38;  // model.hpp: FLT_MAX defaults
