@@ -20,7 +20,8 @@ constexpr float kLreluAlpha = 0.01f;
 // the ~40 of the branchy library routine, which made the fused normalization
 // kernels VALU-bound instead of HBM-bound.  Max error ~2 ulp for x <= 0 (the
 // only range whose result is used); overflow to +inf for large x is harmless
-// because the positive branch of every activation discards it.
+// because the positive branch of the rectifier family discards it and the
+// sigmoid and tanh only take its reciprocal.
 __device__ __forceinline__ float fast_exp(float x) {
   constexpr float kLog2eHi = 1.44269502162933349609375f;   // float(log2 e)
   constexpr float kLog2eLo = 1.925963033500011e-8f;        // log2 e - kLog2eHi
@@ -46,12 +47,16 @@ __device__ __forceinline__ float act_fire(float x) {
     return x < 0.0f ? 0.0f : x;
   } else if constexpr (ACT == DLMI_ACT_LEAKY_RELU) {  // functions.hpp:106
     return x < 0.0f ? kLreluAlpha * x : x;
+  } else if constexpr (ACT == DLMI_ACT_SIGMOID) {  // functions.hpp:40
+    return fast_rcp(1.0f + fast_exp(-x));
+  } else if constexpr (ACT == DLMI_ACT_TANH) {  // functions.hpp:44
+    return 2.0f * fast_rcp(1.0f + fast_exp(-2.0f * x)) - 1.0f;
   } else {  // LINEAR
     return x;
   }
 }
 
-// functions.hpp:88 (ISRLU), :92 (ELU), :99 (SELU), :103 (ReLU), :107 (leaky)
+// functions.hpp:88 (ISRLU), :92 (ELU), :99 (SELU), :103 (ReLU), :107 (leaky), :41 (sigmoid), :45 (tanh)
 template <int ACT>
 __device__ __forceinline__ float act_derive(float x, float q) {
   if constexpr (ACT == DLMI_ACT_ISRLU) {
@@ -65,6 +70,10 @@ __device__ __forceinline__ float act_derive(float x, float q) {
     return x < 0.0f ? 0.0f : 1.0f;
   } else if constexpr (ACT == DLMI_ACT_LEAKY_RELU) {
     return x < 0.0f ? kLreluAlpha : 1.0f;
+  } else if constexpr (ACT == DLMI_ACT_SIGMOID) {  // functions.hpp:41
+    return q * (1.0f - q);
+  } else if constexpr (ACT == DLMI_ACT_TANH) {  // functions.hpp:45
+    return 1.0f - q * q;
   } else {
     return 1.0f;
   }
@@ -78,6 +87,8 @@ inline bool act_supported(int act) {
     case DLMI_ACT_RELU:
     case DLMI_ACT_LEAKY_RELU:
     case DLMI_ACT_LINEAR:
+    case DLMI_ACT_SIGMOID:
+    case DLMI_ACT_TANH:
       return true;
     default:
       return false;
@@ -92,6 +103,8 @@ inline bool act_supported(int act) {
     case DLMI_ACT_SELU: { constexpr int ACT = DLMI_ACT_SELU; __VA_ARGS__; } break;             \
     case DLMI_ACT_RELU: { constexpr int ACT = DLMI_ACT_RELU; __VA_ARGS__; } break;             \
     case DLMI_ACT_LEAKY_RELU: { constexpr int ACT = DLMI_ACT_LEAKY_RELU; __VA_ARGS__; } break; \
+    case DLMI_ACT_SIGMOID: { constexpr int ACT = DLMI_ACT_SIGMOID; __VA_ARGS__; } break;       \
+    case DLMI_ACT_TANH: { constexpr int ACT = DLMI_ACT_TANH; __VA_ARGS__; } break;             \
     default: { constexpr int ACT = DLMI_ACT_LINEAR; __VA_ARGS__; } break;                      \
   }
 

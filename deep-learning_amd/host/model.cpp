@@ -73,7 +73,7 @@ void dev_free(T *&p) {
 bool act_on_path(ACTIVATION::TYPE t) {
   switch (t) {
     case ACTIVATION::ELU: case ACTIVATION::ISRLU: case ACTIVATION::LINEAR: case ACTIVATION::LEAKY_RELU:
-    case ACTIVATION::RELU: case ACTIVATION::SELU:
+    case ACTIVATION::RELU: case ACTIVATION::SELU: case ACTIVATION::SIGMOID: case ACTIVATION::TANH:
       return true;
     default:
       return false;

@@ -40,7 +40,9 @@ typedef enum {
   DLMI_ACT_LEAKY_RELU = 14,
   DLMI_ACT_RELU = 16,
   DLMI_ACT_SELU = 17,
-  DLMI_ACT_SOFTMAX = 22
+  DLMI_ACT_SIGMOID = 18,
+  DLMI_ACT_SOFTMAX = 22,
+  DLMI_ACT_TANH = 23
 } dlmi_activation;
 
 /* v1/data/enum/layer_norm.hpp:24-26 */

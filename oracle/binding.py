@@ -29,7 +29,7 @@ vp = ctypes.c_void_p
 # ACTIVATION / LAYER_NORM / LAYER_DROPOUT / PROPAGATION values of the reference
 # (v1/data/enum/activation.hpp:24-53, layer_norm.hpp:24-26,
 #  layer_dropout.hpp:24-28, propagation.hpp)
-ACT = dict(ELU=3, ISRLU=10, LINEAR=11, LEAKY_RELU=14, RELU=16, SELU=17, SOFTMAX=22)
+ACT = dict(ELU=3, ISRLU=10, LINEAR=11, LEAKY_RELU=14, RELU=16, SELU=17, SIGMOID=18, SOFTMAX=22, TANH=23)
 NORM = dict(NONE=0, BN=1, BRN=2)
 DROP = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3)
 STATE = dict(INFERENCE=0, TRAINING=1, UPDATE_BATCH_NORM=2)

@@ -27,6 +27,10 @@ static inline REAL FN(af_fire)(int type, REAL x) {
       return x < (REAL)0 ? LRELU_ALPHA * x : x;
     case DLO_ACT_LINEAR: /* functions.hpp AF_LINEAR_real: identity */
       return x;
+    case DLO_ACT_SIGMOID: /* functions.hpp:40 */
+      return (REAL)1 / ((REAL)1 + EXP(-x));
+    case DLO_ACT_TANH: /* functions.hpp:44 */
+      return (REAL)2 / ((REAL)1 + EXP((REAL)-2 * x)) - (REAL)1;
     default:
       return x;
   }
@@ -46,6 +50,10 @@ static inline REAL FN(af_derive)(int type, REAL x, REAL q) {
       return x < (REAL)0 ? (REAL)0 : (REAL)1;
     case DLO_ACT_LEAKY_RELU:
       return x < (REAL)0 ? LRELU_ALPHA : (REAL)1;
+    case DLO_ACT_SIGMOID: /* functions.hpp:41 */
+      return q * ((REAL)1 - q);
+    case DLO_ACT_TANH: /* functions.hpp:45 */
+      return (REAL)1 - q * q;
     case DLO_ACT_LINEAR:
       return (REAL)1;
     default:

@@ -652,7 +652,12 @@ REGRESS_CASES = {
     "relu_l1_distance": ([8, 11, 2], 9, "RELU", "L1", "DISTANCE", 0.1, "real"),
     "linear_ce_ce": ([6, 10, 4], 15, "LINEAR", "CROSS_ENTROPY", "CROSS_ENTROPY", 0.49, "onehot"),
     "linear_mse_wide": ([20, 40, 130], 37, "LINEAR", "MSE", "DISTANCE", 0.49, "real"),
+    "sigmoid_net_mse_distance": ([8, 13, 9, 5], 21, "SIGMOID", "MSE", "DISTANCE", 0.25, "unit"),
+    "tanh_net_mae_sign": ([7, 11, 6], 17, "TANH", "MAE", "SIGN", 0.49, "signed"),
+    "sigmoid_ce_ce": ([6, 10, 4], 15, "SIGMOID", "CROSS_ENTROPY", "CROSS_ENTROPY", 0.49, "onehot"),
 }
+# activation of the hidden layers where it is not ELU
+REGRESS_HIDDEN = {"sigmoid_net_mse_distance": "SIGMOID", "tanh_net_mae_sign": "TANH"}
 
 
 def regressions(R):
@@ -660,13 +665,17 @@ def regressions(R):
     (compute_error_st.cpp:80-123, compute_loss.cpp:25-138, loss.cpp:98-221): one
     training step with its seed gradient, loss and accuracy, then three epochs of
     Nesterov momentum through the epoch driver with the loss it reports."""
-    d = {"regress_cases_json": np.frombuffer(json.dumps(REGRESS_CASES).encode(), dtype=np.uint8)}
+    d = {"regress_cases_json": np.frombuffer(json.dumps(REGRESS_CASES).encode(), dtype=np.uint8),
+         "regress_hidden_json": np.frombuffer(json.dumps(REGRESS_HIDDEN).encode(), dtype=np.uint8)}
     for name, (widths, B, out_act, loss, accu, acc_var, targets) in REGRESS_CASES.items():
         rng = np.random.default_rng(sum(map(ord, name)))
         L = len(widths)
         X = f32(rng.uniform(-1, 1, (B, widths[0])))
+        hidden = ACT[REGRESS_HIDDEN.get(name, "ELU")]
         if targets == "onehot":
             Y = f32(np.eye(widths[-1])[rng.integers(0, widths[-1], B)])
+        elif targets == "unit":
+            Y = f32(rng.uniform(0, 1, (B, widths[-1])))
         else:
             Y = f32(rng.uniform(-1, 1, (B, widths[-1])))
             if targets == "signed":
@@ -676,7 +685,7 @@ def regressions(R):
         for nt in THREADS:
             M = R.mlp(widths)
             for l in range(1, L - 1):
-                M.set_layer(l, ACT["ELU"], NORM["BRN"])
+                M.set_layer(l, hidden, NORM["BRN"])
             M.set_layer(L - 1, ACT[out_act])
             M.prepare(B, nt)
             M.set_loss(loss, accu, acc_var)
@@ -699,7 +708,7 @@ def regressions(R):
             # the epoch driver on the same data: sub-batches of 7, one update per epoch
             M2 = R.mlp(widths)
             for l in range(1, L - 1):
-                M2.set_layer(l, ACT["ELU"], NORM["BRN"])
+                M2.set_layer(l, hidden, NORM["BRN"])
             M2.set_layer(L - 1, ACT[out_act])
             M2.set_norm_hyper(0.5, 1e-5, 3.0, 5.0)
             M2.prepare(7, nt)

@@ -112,8 +112,8 @@ def test_refused_arguments_leave_the_context_usable(dl, pkg):
     v = torch.ones(4, device="cuda")
     p = lambda t: vp(t.data_ptr())
     desc = pkg.Dlmi.desc(ACT["RELU"])
-    SIGMOID = 18  # ACTIVATION::SIGMOID, the reference's default and not one of the path's activations
-    bad_act = pkg.Dlmi.desc(SIGMOID)
+    OFF_PATH = 19  # ACTIVATION::SINE: not one of the path's activations
+    bad_act = pkg.Dlmi.desc(OFF_PATH)
     INVALID, UNSUPPORTED = -1, -4
     calls = {
         "fc_fwd, no rows": lambda: lib.dlmi_fc_fwd(ctx, c_sz(0), c_sz(4), c_sz(4), p(a), p(a), None, p(a)),
@@ -129,7 +129,7 @@ def test_refused_arguments_leave_the_context_usable(dl, pkg):
                                                                           p(v), p(v), p(v), p(v), p(v), p(v), p(a)),
         "fused fwd, activation off the path": lambda: lib.dlmi_fused_norm_act_fwd(
             ctx, ctypes.byref(bad_act), c_sz(4), c_sz(4), p(a), p(v), p(v), None, p(v), p(v), p(v), p(v), p(v), p(v), p(a)),
-        "act_fwd, activation off the path": lambda: lib.dlmi_act_fwd(ctx, SIGMOID, c_sz(4), c_sz(4), p(a), p(a)),
+        "act_fwd, activation off the path": lambda: lib.dlmi_act_fwd(ctx, OFF_PATH, c_sz(4), c_sz(4), p(a), p(a)),
         "zero-padded identity, padding past the wider operand": lambda: lib.dlmi_zero_padded_identity_fwd(
             ctx, c_sz(4), c_sz(4), c_sz(2), c_sz(3), p(a), p(a), p(a)),
     }

@@ -72,7 +72,7 @@ def test_setters_refuse_what_the_reference_refuses(model_factory):
     assert lib.dlmi_model_set_layer_activation_function(h, c_sz(1), c_int(ACT["SOFTMAX"])) == 0
     assert lib.dlmi_model_set_layer_activation_function(h, c_sz(3), c_int(ACT["SOFTMAX"])) == 1
     # activations outside the path
-    assert lib.dlmi_model_set_layer_activation_function(h, c_sz(1), c_int(23)) == 0  # TANH
+    assert lib.dlmi_model_set_layer_activation_function(h, c_sz(1), c_int(19)) == 0  # SINE
     # batch size 0 (model.cpp:2652)
     assert lib.dlmi_model_prepare(h, c_sz(0)) == 0
 

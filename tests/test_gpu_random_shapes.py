@@ -49,7 +49,7 @@ def test_products_on_random_shapes(dl, oracle, B, K, H):
 @pytest.mark.parametrize("B,H", [s for s in draw_shapes(7, 40, 2, 3_000_000) if s[0] >= 2])
 def test_fused_norm_on_random_shapes(dl, oracle, pkg, B, H):
     rng = np.random.default_rng(B * 1013 + H)
-    act = ["SELU", "ELU", "ISRLU", "RELU", "LEAKY_RELU"][(B + H) % 5]
+    act = ["SELU", "ELU", "ISRLU", "RELU", "LEAKY_RELU", "SIGMOID", "TANH"][(B + H) % 7]
     drop = ["NONE", "BERNOULLI", "BERNOULLI_INVERTED"][(B * 7 + H) % 3]
     renorm = bool((B + 3 * H) % 2)
     x = (rng.standard_normal((B, H)) * rng.uniform(.5, 2, H) + rng.uniform(-1, 1, H)).astype(np.float32)

@@ -65,7 +65,7 @@ def test_seed_kernel_against_golden_output_layer(dl, name):
 
 
 @pytest.mark.parametrize("B,H", [(1, 1), (3, 64), (257, 10), (70, 130), (4099, 7)])
-@pytest.mark.parametrize("act", ["LINEAR", "ELU", "ISRLU", "LEAKY_RELU", "RELU", "SELU"])
+@pytest.mark.parametrize("act", ["LINEAR", "ELU", "ISRLU", "LEAKY_RELU", "RELU", "SELU", "SIGMOID", "TANH"])
 def test_seed_kernel_against_oracle(dl, oracle, B, H, act):
     rng = np.random.default_rng(B * 131 + H + ACT[act])
     z = (rng.standard_normal((B, H)) * 1.5).astype(np.float32)
@@ -83,6 +83,18 @@ def test_seed_kernel_against_oracle(dl, oracle, B, H, act):
             st = host(stats)
             assert abs(st[0] - total) <= 1e-5 * max(1.0, abs(total)), f"{loss}/{accu} loss sum"
             assert st[1] == acc, f"{loss}/{accu} accuracy count"
+
+
+@pytest.mark.parametrize("act", ["SIGMOID", "TANH"])
+@pytest.mark.parametrize("B,H", [(5, 3), (130, 70), (1024, 2048)])
+def test_sigmoid_and_tanh_leaves_against_oracle(dl, oracle, act, B, H):
+    rng = np.random.default_rng(B + H + ACT[act])
+    x = (rng.standard_normal((B, H)) * 4).astype(np.float32)
+    x.flat[:6] = [0.0, -0.0, 30.0, -30.0, 100.0, -100.0][: min(6, x.size)]  # saturation on both sides
+    dY = rng.standard_normal((B, H)).astype(np.float32)
+    q = oracle.act_fwd(ACT[act], x)
+    assert_close(host(dl.act_fwd(ACT[act], dev(x))), q, TE, act + " forward")
+    assert_close(host(dl.act_bwd(ACT[act], dev(x), dev(q), dev(dY))), oracle.act_bwd(ACT[act], x, q, dY), TE, act + " backward")
 
 
 def test_seed_kernel_loss_only_and_accumulation(dl, oracle):
@@ -104,7 +116,7 @@ def test_seed_kernel_empty_and_refused(dl):
     t = torch.zeros((2, 3), device="cuda")
     for loss, accu, act in [(LOSS["MAPE"], ACCU["DISTANCE"], ACT["LINEAR"]), (LOSS["SMAPE"], ACCU["SIGN"], ACT["ELU"]),
                             (1, ACCU["DISTANCE"], ACT["LINEAR"]), (LOSS["MSE"], ACCU["R"], ACT["LINEAR"]),
-                            (LOSS["MSE"], ACCU["DISTANCE"], ACT["SOFTMAX"]), (LOSS["MSE"], ACCU["DISTANCE"], 18)]:
+                            (LOSS["MSE"], ACCU["DISTANCE"], ACT["SOFTMAX"]), (LOSS["MSE"], ACCU["DISTANCE"], 19)]:
         with pytest.raises(RuntimeError):
             dl.loss_seed(loss, accu, 0.49, act, t, t, t)
 

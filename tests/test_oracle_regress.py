@@ -30,10 +30,11 @@ def regress_cases():
 
 def build_regress_model(make, g, name, nt, max_batch=None, hyper=None):
     widths, B, out_act, loss, accu, acc_var, _ = regress_cases()[name]
+    hidden = ACT[json.loads(bytes(g["regress_hidden_json"])).get(name, "ELU")]
     L = len(widths)
     M = make(widths)
     for l in range(1, L - 1):
-        M.set_layer(l, ACT["ELU"], NORM["BRN"])
+        M.set_layer(l, hidden, NORM["BRN"])
     M.set_layer(L - 1, ACT[out_act])
     if hyper is not None:
         M.set_norm_hyper(*hyper)
@@ -136,6 +137,19 @@ def test_leaf_refuses_what_the_reference_does_not_manage(oracle, loss, accu):
     # accuracy needs a second pass the training path never makes
     with pytest.raises(ValueError):
         oracle.loss_seed(loss, accu, 0.49, ACT["LINEAR"], Q, Q, Y)
+
+
+def test_sigmoid_and_tanh_against_the_library_functions(oracle, oracle64):
+    x = np.linspace(-12, 12, 481).astype(np.float32)[None, :]
+    for o, dt, tol in ((oracle, np.float32, 3e-7), (oracle64, np.float64, 1e-15)):
+        xs = x.astype(dt)
+        s = o.act_fwd(ACT["SIGMOID"], xs)
+        t = o.act_fwd(ACT["TANH"], xs)
+        np.testing.assert_allclose(s, 1.0 / (1.0 + np.exp(-xs.astype(np.float64))), rtol=tol, atol=tol)
+        np.testing.assert_allclose(t, np.tanh(xs.astype(np.float64)), rtol=0, atol=4 * tol)
+        one = np.ones_like(xs)
+        np.testing.assert_allclose(o.act_bwd(ACT["SIGMOID"], xs, s, one), s * (1 - s), rtol=4 * tol, atol=tol)  # functions.hpp:41
+        np.testing.assert_allclose(o.act_bwd(ACT["TANH"], xs, t, one), 1 - t * t, rtol=4 * tol, atol=4 * tol)  # functions.hpp:45
 
 
 # ---- against the compiled reference ---------------------------------------------------------------
