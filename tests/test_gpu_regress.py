@@ -144,3 +144,24 @@ def test_gpu_model_refuses_unmanaged_losses(model_factory):
         M.step(1, g[name + "_X"], g[name + "_Y"], backward=True)
     with pytest.raises(RuntimeError):
         M.set_loss(LOSS["MSE"], ACCU["DISTANCE"], 1.5)  # Set__Accurancy_Variance: within [0, 1]
+
+
+def test_a_model_without_activation_setters_runs_on_sigmoids_like_the_reference(model_factory):
+    """compile.cpp:627-628: every layer starts as a sigmoid layer."""
+    from oracle.binding import STATE
+    rng = np.random.default_rng(8)
+    X = rng.uniform(-1, 1, (9, 6)).astype(np.float32)
+    Y = rng.uniform(0, 1, (9, 3)).astype(np.float32)
+    outs = []
+    for explicit in (False, True):
+        M = model_factory([6, 7, 3])
+        if explicit:
+            M.set_layer(1, ACT["SIGMOID"])
+            M.set_layer(2, ACT["SIGMOID"])
+        M.prepare(9)
+        M.set_loss(LOSS["MSE"], ACCU["DISTANCE"], 0.3)
+        M.glorot_uniform(11)
+        M.step(STATE["TRAINING"], X, Y, backward=True)
+        outs.append((M.layer_buffer(2, 3), M.get_dparams()))
+    assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+    assert np.all((outs[0][0] > 0) & (outs[0][0] < 1)) and np.abs(outs[0][1]).max() > 0
