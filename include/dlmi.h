@@ -143,8 +143,9 @@ int dlmi_norm_bwd(dlmi_ctx *ctx, dlmi_norm norm, size_t B, size_t H, float const
 int dlmi_act_fwd(dlmi_ctx *ctx, dlmi_activation act, size_t B, size_t H, float const *x, float *y);
 
 /* dN = dY * f'(pre, post), with the reference's derivative forms
- * (functions.hpp:88,92,99,103,107; v1/learner/model.cpp:2594-2651):
- * ELU' = post (x<0), SELU' = scale*(post+alpha) (x<=0), ISRLU' = (post/pre)^3 (x<0).
+ * (functions.hpp:41,45,88,92,99,103,107; v1/learner/model.cpp:2594-2651):
+ * ELU' = post (x<0), SELU' = scale*(post+alpha) (x<=0), ISRLU' = (post/pre)^3 (x<0),
+ * sigmoid' = post*(1-post), tanh' = 1-post^2.
  * Replaces Backward_Pass__FC__DF__* (bwp_st.cpp:1177-1209).  dN may alias dY. */
 int dlmi_act_bwd(dlmi_ctx *ctx, dlmi_activation act, size_t B, size_t H, float const *pre,
                  float const *post, float const *dY, float *dN);

@@ -15,9 +15,10 @@
 //     accepted and do nothing: there are no per-thread gradient copies to merge;
 //   * only LAYER::FULLY_CONNECTED layers and LAYER::RESIDUAL blocks of them
 //     (a {RESIDUAL, depth} entry followed by the `depth` layers of its block),
-//     the activations ReLU / leaky ReLU / ELU / SELU / ISRLU / linear (+ softmax
-//     on the output layer), batch normalization / renormalization, Bernoulli and
-//     inverted-Bernoulli dropout and the cross-entropy loss are implemented;
+//     the activations ReLU / leaky ReLU / ELU / SELU / ISRLU / linear / sigmoid /
+//     tanh (+ softmax on the output layer), batch normalization / renormalization,
+//     Bernoulli and inverted-Bernoulli dropout, and the losses with a derivative
+//     (cross-entropy, ME, L1, MAE, L2, MSE, RMSE) are implemented;
 //     anything else makes the setter return false, as the reference does for
 //     settings it refuses.
 //
