@@ -18,10 +18,12 @@ constexpr float kLreluAlpha = 0.01f;
 // product x*log2(e) is formed in two pieces so that its rounding error (which
 // would otherwise grow with |x|) is folded back in.  ~6 instructions instead of
 // the ~40 of the branchy library routine, which made the fused normalization
-// kernels VALU-bound instead of HBM-bound.  Max error ~2 ulp for x <= 0 (the
-// only range whose result is used); overflow to +inf for large x is harmless
-// because the positive branch of the rectifier family discards it and the
-// sigmoid and tanh only take its reciprocal.
+// kernels VALU-bound instead of HBM-bound.  Max error ~2 ulp.
+// Valid for x < 88.7 only: once 2^t overflows, the correction r*(e*ln 2) is
+// +-inf and r + correction is NaN for about a third of the arguments.  The
+// rectifier family calls it with x <= 0 (the positive side is discarded by a
+// select, which does not propagate the NaN); anything that can see a large
+// positive argument uses fast_exp_sat.
 __device__ __forceinline__ float fast_exp(float x) {
   constexpr float kLog2eHi = 1.44269502162933349609375f;   // float(log2 e)
   constexpr float kLog2eLo = 1.925963033500011e-8f;        // log2 e - kLog2eHi
@@ -30,6 +32,17 @@ __device__ __forceinline__ float fast_exp(float x) {
   float const e = __builtin_fmaf(x, kLog2eHi, -t) + x * kLog2eLo;
   float const r = __builtin_amdgcn_exp2f(t);
   return __builtin_fmaf(r, e * kLn2, r);
+}
+// The same, saturating to +inf like std::exp when the result overflows (the
+// sigmoid and tanh take its reciprocal: 1/(1+inf) = 0, as in the reference).
+__device__ __forceinline__ float fast_exp_sat(float x) {
+  constexpr float kLog2eHi = 1.44269502162933349609375f;
+  constexpr float kLog2eLo = 1.925963033500011e-8f;
+  constexpr float kLn2 = 0.693147182464599609375f;
+  float const t = x * kLog2eHi;
+  float const e = __builtin_fmaf(x, kLog2eHi, -t) + x * kLog2eLo;
+  float const r = __builtin_amdgcn_exp2f(t);
+  return r == __builtin_inff() ? r : __builtin_fmaf(r, e * kLn2, r);
 }
 // 1/sqrt(v) and 1/v at hardware rate (1 ulp each).
 __device__ __forceinline__ float fast_rsqrt(float v) { return __builtin_amdgcn_rsqf(v); }
@@ -48,9 +61,9 @@ __device__ __forceinline__ float act_fire(float x) {
   } else if constexpr (ACT == DLMI_ACT_LEAKY_RELU) {  // functions.hpp:106
     return x < 0.0f ? kLreluAlpha * x : x;
   } else if constexpr (ACT == DLMI_ACT_SIGMOID) {  // functions.hpp:40
-    return fast_rcp(1.0f + fast_exp(-x));
+    return fast_rcp(1.0f + fast_exp_sat(-x));
   } else if constexpr (ACT == DLMI_ACT_TANH) {  // functions.hpp:44
-    return 2.0f * fast_rcp(1.0f + fast_exp(-2.0f * x)) - 1.0f;
+    return 2.0f * fast_rcp(1.0f + fast_exp_sat(-2.0f * x)) - 1.0f;
   } else {  // LINEAR
     return x;
   }

@@ -97,6 +97,25 @@ def test_sigmoid_and_tanh_leaves_against_oracle(dl, oracle, act, B, H):
     assert_close(host(dl.act_bwd(ACT[act], dev(x), dev(q), dev(dY))), oracle.act_bwd(ACT[act], x, q, dY), TE, act + " backward")
 
 
+@pytest.mark.parametrize("act", ["SIGMOID", "TANH"])
+def test_sigmoid_and_tanh_saturate_without_nan(dl, oracle, act):
+    """Beyond the overflow of exp (x <= -88.8 for the sigmoid, x <= -44.4 for tanh) the reference
+    returns exactly 0 / -1; a device exponential that is not saturated returns NaN for about a third
+    of such arguments (not for x = -100: the sign of its correction term happens to be right there)."""
+    lo, hi = (-200.0, -89.0) if act == "SIGMOID" else (-150.0, -44.5)
+    x = np.concatenate([np.linspace(lo, hi, 4093), [-95.0, -101.0, -47.5, -300.0, 300.0, 95.0, 47.5]]).astype(np.float32)
+    x = x.reshape(-1, 100)
+    q = host(dl.act_fwd(ACT[act], dev(x)))
+    assert not np.isnan(q).any(), act + " produced NaN in saturation"
+    qo = oracle.act_fwd(ACT[act], x)
+    assert np.array_equal(q[x <= hi], qo[x <= hi]), act + " saturated values differ from the reference's"
+    assert np.all(q[x <= hi] == (0.0 if act == "SIGMOID" else -1.0))
+    assert_close(q, qo, TE, act + " forward, saturated")
+    # the derivative q(1-q) / 1-q^2 of a saturated output is finite as well
+    dY = np.ones_like(x)
+    assert not np.isnan(host(dl.act_bwd(ACT[act], dev(x), dev(q), dev(dY)))).any()
+
+
 def test_seed_kernel_loss_only_and_accumulation(dl, oracle):
     rng = np.random.default_rng(77)
     q = rng.standard_normal((33, 12)).astype(np.float32)
