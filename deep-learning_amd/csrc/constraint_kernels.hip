@@ -105,7 +105,7 @@ int dlmi_clip_gradient(dlmi_ctx *ctx, size_t n, float *grads, float max_norm) {
   if (blocks > cap) blocks = cap;
   int rc = dlmi_scratch_reserve(ctx, (blocks + 1) * sizeof(float));
   if (rc != DLMI_OK) return rc;
-  float *const partial = reinterpret_cast<float *>(ctx->scratch);
+  float *const partial = reinterpret_cast<float *>(dlmi_scratch_data(ctx));
   float *const factor = partial + blocks;
   hipLaunchKernelGGL(k_sumsq_partial, dim3(static_cast<unsigned>(blocks)), dim3(kCBlock), 0, ctx->stream, grads, n, n4,
                      partial);

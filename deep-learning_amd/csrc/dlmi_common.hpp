@@ -10,16 +10,36 @@
 
 #include "../../include/dlmi.h"
 
+// Launch-geometry knobs of the normalization kernels, read once per context
+// from the environment (DLMI_NORM_*; tuning aids, the defaults are the measured
+// best on MI355X).
+struct dlmi_tuning {
+  int reduce_tx_cap = 128;        // widest column span of a reduction block, in column groups
+  int reduce_blocks_per_cu = 1;   // reduction blocks per compute unit
+  int reduce_min_rows = 4;        // fewest rows a thread of a reduction block walks
+  int apply_blocks_per_cu = 2;    // blocks per compute unit in the apply passes
+  int apply_min_rows = 4;
+  int reduce_interleave = 0;      // 1: blocks take every n-th group of rows instead of a contiguous chunk
+  int apply_interleave = 0;
+};
+
 struct dlmi_ctx {
   int device = 0;
   hipStream_t stream = nullptr;
   int num_cu = 256;
-  // Device scratch for reduction partials and per-unit constants.  Grown on
-  // demand (never inside a launch sequence that already holds pointers to it).
+  // Device scratch for reduction partials and per-unit constants, grown on
+  // demand.  A block that has been handed to kernels is never freed before the
+  // context is destroyed (recorded HIP graphs keep its address): growing
+  // retires it and allocates a larger one.
   char *scratch = nullptr;
   size_t scratch_bytes = 0;
+  char *retired[32] = {nullptr};
+  int n_retired = 0;
+  dlmi_tuning tune;
   char err[512] = {0};
 };
+
+inline char *dlmi_scratch_data(dlmi_ctx const *ctx) { return ctx->scratch; }
 
 inline int dlmi_fail(dlmi_ctx *ctx, int code, char const *fmt, ...) {
   if (ctx != nullptr) {
@@ -54,15 +74,19 @@ inline int dlmi_fail(dlmi_ctx *ctx, int code, char const *fmt, ...) {
   } while (0)
 
 // Makes sure the context's scratch holds at least `bytes`.
+// Growing allocates (and synchronizes the stream): it is refused while the
+// stream is being captured into a HIP graph.
 int dlmi_scratch_reserve(dlmi_ctx *ctx, size_t bytes);
 
 namespace dlmi {
 // Batch-(re)norm forward tail (finalize + apply) from column-sum partials
 // [2][nchunks][H] that a producer (the GEMM epilogue) already wrote.
+// partial == nullptr: the statistics come from a pass over x.  residual != nullptr:
+// y = residual + (activation output after dropout), the identity shortcut of a block.
 int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
-                            float const *gamma, float const *beta, uint8_t const *mask, float *mean, float *stdv,
-                            float *mov_mean, float *mov_std, float *r, float *d, float *y, float const *partial,
-                            unsigned nchunks);
+                            float const *gamma, float const *beta, uint8_t const *mask, float const *residual,
+                            float *mean, float *stdv, float *mov_mean, float *mov_std, float *r, float *d, float *y,
+                            float const *partial, unsigned nchunks);
 // out[j] (+)= sum over the B rows of x[b, j], in a fixed order (the statistics
 // pass of the normalization kernels with its second plane unused).
 int column_sums(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *out, int accumulate);

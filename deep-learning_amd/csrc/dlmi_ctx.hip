@@ -1,22 +1,44 @@
 // Context management of the dlmi C ABI.
+#include <cstdlib>
+
 #include "dlmi_common.hpp"
 
 int dlmi_scratch_reserve(dlmi_ctx *ctx, size_t bytes) {
-  if (bytes <= ctx->scratch_bytes) return DLMI_OK;
-  // Work already queued on the stream may still read the old block.
-  DLMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
-  if (ctx->scratch != nullptr) DLMI_HIP(ctx, hipFree(ctx->scratch));
-  ctx->scratch = nullptr;
-  ctx->scratch_bytes = 0;
-  size_t const want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+  if (ctx->scratch != nullptr && bytes <= ctx->scratch_bytes) return DLMI_OK;
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(ctx->stream, &cap) != hipSuccess) (void)hipGetLastError();
+  if (cap != hipStreamCaptureStatusNone)
+    return dlmi_fail(ctx, DLMI_E_INVALID,
+                     "scratch would have to grow to %zu bytes while the stream is being captured: run the "
+                     "same calls once outside the capture first", bytes);
+  if (ctx->scratch != nullptr && ctx->n_retired >= static_cast<int>(sizeof(ctx->retired) / sizeof(ctx->retired[0])))
+    return dlmi_fail(ctx, DLMI_E_NOMEM, "scratch grew too many times");
+  // at least double, so that a context retires only a handful of blocks in its life
+  size_t want = bytes > 2 * ctx->scratch_bytes ? bytes : 2 * ctx->scratch_bytes;
+  want = (want + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
   void *p = nullptr;
   if (hipMalloc(&p, want) != hipSuccess) {
     (void)hipGetLastError();
     return dlmi_fail(ctx, DLMI_E_NOMEM, "scratch allocation of %zu bytes failed", want);
   }
+  // Work already queued (or recorded into a graph) may still use the old block:
+  // it stays allocated until the context goes.
+  if (ctx->scratch != nullptr) ctx->retired[ctx->n_retired++] = ctx->scratch;
   ctx->scratch = static_cast<char *>(p);
   ctx->scratch_bytes = want;
   return DLMI_OK;
+}
+
+static int env_knob(char const *name, int dflt) {
+  char const *e = getenv(name);
+  if (e == nullptr || *e == 0) return dflt;
+  int const v = atoi(e);
+  return v > 0 ? v : dflt;
+}
+
+static int env_flag(char const *name, int dflt) {
+  char const *e = getenv(name);
+  return (e == nullptr || *e == 0) ? dflt : (atoi(e) != 0 ? 1 : 0);
 }
 
 extern "C" {
@@ -41,6 +63,14 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
   ctx->device = device;
   ctx->stream = static_cast<hipStream_t>(stream);
   ctx->num_cu = prop.multiProcessorCount;
+  dlmi_tuning &t = ctx->tune;
+  t.reduce_tx_cap = env_knob("DLMI_NORM_REDUCE_TX", t.reduce_tx_cap);
+  t.reduce_blocks_per_cu = env_knob("DLMI_NORM_REDUCE_BLOCKS_PER_CU", t.reduce_blocks_per_cu);
+  t.reduce_min_rows = env_knob("DLMI_NORM_REDUCE_MIN_ROWS", t.reduce_min_rows);
+  t.apply_blocks_per_cu = env_knob("DLMI_NORM_APPLY_BLOCKS_PER_CU", t.apply_blocks_per_cu);
+  t.apply_min_rows = env_knob("DLMI_NORM_APPLY_MIN_ROWS", t.apply_min_rows);
+  t.reduce_interleave = env_flag("DLMI_NORM_REDUCE_INTERLEAVE", t.reduce_interleave);
+  t.apply_interleave = env_flag("DLMI_NORM_APPLY_INTERLEAVE", t.apply_interleave);
   int rc = dlmi_scratch_reserve(ctx, size_t(16) << 20);
   if (rc != DLMI_OK) {
     delete ctx;
@@ -54,6 +84,7 @@ int dlmi_ctx_destroy(dlmi_ctx *ctx) {
   if (ctx == nullptr) return DLMI_OK;
   (void)hipStreamSynchronize(ctx->stream);
   if (ctx->scratch != nullptr) (void)hipFree(ctx->scratch);
+  for (int i = 0; i < ctx->n_retired; ++i) (void)hipFree(ctx->retired[i]);
   delete ctx;
   return DLMI_OK;
 }

@@ -488,13 +488,13 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
       size_t const chunks_reserved = *stats_chunks > 32 ? *stats_chunks : 32;
       int rc = dlmi_scratch_reserve(ctx, 2 * 2 * static_cast<size_t>(chunks_reserved) * N * sizeof(float));
       if (rc != DLMI_OK) return rc;
-      g.stats_out = reinterpret_cast<float *>(ctx->scratch);
+      g.stats_out = reinterpret_cast<float *>(dlmi_scratch_data(ctx));
     }
   }
   size_t const kt_per_split = dlmi_ceil_div(ktiles, splits);
   g.k_per_split = kt_per_split * bk;
   splits = static_cast<unsigned>(dlmi_ceil_div(ktiles, kt_per_split));
-  if (splits > 1) g.split_out = reinterpret_cast<float *>(ctx->scratch);
+  if (splits > 1) g.split_out = reinterpret_cast<float *>(dlmi_scratch_data(ctx));
   int rc;
   switch (choice) {
     case 1: rc = launch_gemm<256, 128, 16, AK, BKC, 2>(ctx, g, splits, fast); break;
@@ -540,8 +540,8 @@ int dlmi_fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, s
   if (rc != DLMI_OK) return rc;
   // a small output runs split over K, where no slice sees whole sums: the
   // statistics then come from a pass over Z (nullptr / 0)
-  return fused_fwd_from_partials(ctx, desc, B, H, Z, gamma, beta, mask, mean, stdv, mov_mean, mov_std, r, d, y,
-                                 chunks != 0 ? reinterpret_cast<float const *>(ctx->scratch) : nullptr, chunks);
+  return fused_fwd_from_partials(ctx, desc, B, H, Z, gamma, beta, mask, nullptr, mean, stdv, mov_mean, mov_std, r, d, y,
+                                 chunks != 0 ? reinterpret_cast<float const *>(dlmi_scratch_data(ctx)) : nullptr, chunks);
 }
 
 int dlmi_fc_bwd_dx(dlmi_ctx *ctx, size_t B, size_t Hn, size_t H, float const *dZn, float const *Wn, float *dY,

@@ -6,8 +6,8 @@
 // accesses, enough independent loads in flight per CU and few enough ALU
 // instructions per element that the vector units never become the limit:
 //
-//   forward : stats (read x)            -> finalize [H] -> apply (read x, write y)
-//   backward: reduce (read dY, x)       -> finalize [H] -> apply (read dY, x, write dX)
+//   forward : statistics (read x)      -> finalize [H] -> apply (read x, write y)
+//   backward: reduce (read dY, x)      -> finalize [H] -> apply (read dY, x, write dX)
 //
 // x_hat, the pre-activation n = gamma*x_hat + beta and the activation output
 // are recomputed in registers instead of being stored and re-read.
@@ -17,10 +17,14 @@
 // block's batch chunk with stride TY.  In the reduction kernels TX <= 64, so
 // when H is small a wavefront spans several rows: those are combined with
 // wavefront shuffles, the four wavefronts of the block with a small LDS tree,
-// and the chunks of the batch by the finalize kernel in a fixed order (no float
-// atomics: results are reproducible run to run).  The apply kernels have
-// nothing to reduce and use TX = 256 when H allows, so that every load / store
-// instruction of a block covers 4 KiB of one row.
+// and the chunks of the batch by the finalize kernel in chunk order.  No float
+// atomics, a fixed summation order: results are reproducible run to run.
+// (Folding the finalize into the reduction - the block that draws the last of a
+// column group's tickets combines the chunks - was built and measured: its tail
+// of device-scope round trips costs 10 us at [4096 x 4096], twice the separate
+// launch.)
+// The apply kernels have nothing to reduce and use TX = 256 when H allows, so
+// that every load / store instruction of a block covers 4 KiB of one row.
 //
 // Everything that is uniform over a launch and would put a branch between two
 // loads (dropout mode, materialising x_hat) is a template parameter: a branch
@@ -38,14 +42,6 @@ namespace dlmi {
 constexpr int kBlock = 256;
 constexpr int kWave = 64;
 
-// rows in flight per thread in the reduction passes
-#ifndef DLMI_STATS_U
-#define DLMI_STATS_U 8
-#endif
-#ifndef DLMI_BWD_REDUCE_U
-#define DLMI_BWD_REDUCE_U 4
-#endif
-
 // dropout as a template mode
 constexpr int kDropNone = 0, kDropUnit = 1, kDropElem = 2;
 
@@ -57,44 +53,39 @@ struct ColGeom {
   size_t rows_per_chunk;
 };
 
-// Tuning aids: DLMI_NORM_{STATS,BWD}_TX (64, 128 or 256), .._ROWS_PER_THREAD and
-// .._BLOCKS_PER_CU override the geometry of the two reduction passes,
-// DLMI_NORM_APPLY_ROWS_PER_THREAD that of the apply passes.
-static int env_int(char const *name, int dflt) {
-  char const *e = getenv(name);
-  if (e == nullptr || *e == 0) return dflt;
-  int const v = atoi(e);
-  return v > 0 ? v : dflt;
-}
+// A region of device memory the reduction kernels may use for partial sums and
+// the backward coefficients.
+struct ScratchView {
+  char *data;
+  size_t data_bytes;
+};
 
-// Geometry of a reduction pass.
-static ColGeom reduce_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, int nacc) {
-  static int const tx_caps[2] = {env_int("DLMI_NORM_STATS_TX", 64), env_int("DLMI_NORM_BWD_TX", 256)};
-  static int const rpts[2] = {env_int("DLMI_NORM_STATS_ROWS_PER_THREAD", 16), env_int("DLMI_NORM_BWD_ROWS_PER_THREAD", 8)};
-  static int const bpcs[2] = {env_int("DLMI_NORM_STATS_BLOCKS_PER_CU", 8), env_int("DLMI_NORM_BWD_BLOCKS_PER_CU", 1)};
-  int const which = nacc == 2 ? 0 : 1;
-  int const tx_cap = tx_caps[which], rows_per_thread = rpts[which], blocks_per_cu = bpcs[which];
+static size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Geometry of a reduction pass over [B, H] with `nplanes` sums per unit: blocks
+// as wide as the cap allows (TX column groups, up to 256: every load of a block
+// then covers 4 KiB of one row), a few blocks per compute unit, each thread
+// walking at least reduce_min_rows rows.
+static ColGeom reduce_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, int nplanes, size_t data_bytes) {
+  dlmi_tuning const &t = ctx->tune;
   ColGeom g;
   g.vec = vec4 ? 4 : 1;
   size_t const groups = dlmi_ceil_div(H, g.vec);
-  int tx = tx_cap >= 256 ? 256 : (tx_cap >= 128 ? 128 : 64);
-  g.tx_log2 = tx == 256 ? 8 : (tx == 128 ? 7 : 6);
-  while (tx > 1 && static_cast<size_t>(tx / 2) >= groups) {
+  int tx = 256;
+  g.tx_log2 = 8;
+  while (tx > 1 && (tx > t.reduce_tx_cap || static_cast<size_t>(tx / 2) >= groups)) {
     tx /= 2;
     --g.tx_log2;
   }
   int const ty = kBlock / tx;
   g.grid_x = static_cast<unsigned>(dlmi_ceil_div(groups, tx));
-  // enough blocks to cover every CU several times over, but each thread still
-  // streams rows_per_thread rows (16 in the statistics pass, 8 in the backward
-  // reduction, where a batch of 1024 rows otherwise leaves half the CUs idle):
-  // the partial sums stay a small fraction of the traffic and the fixed cost of
-  // a block is amortised
-  size_t want = dlmi_ceil_div(static_cast<size_t>(ctx->num_cu) * blocks_per_cu, g.grid_x);
-  size_t const max_by_rows = B / (static_cast<size_t>(ty) * rows_per_thread);
+  size_t want = dlmi_ceil_div(static_cast<size_t>(ctx->num_cu) * t.reduce_blocks_per_cu, g.grid_x);
+  size_t const max_by_rows = B / (static_cast<size_t>(ty) * t.reduce_min_rows);
   if (want > max_by_rows) want = max_by_rows;
-  // partial sums must fit half of the scratch block: nacc * nchunks * H floats
-  size_t const max_by_scratch = (ctx->scratch_bytes / 2) / (static_cast<size_t>(nacc) * H * sizeof(float));
+  // partial sums [nplanes][nchunks][H] must fit the data region (beside 3*H coefficients)
+  size_t const fixed = round_up(3 * H * sizeof(float), 256);
+  size_t const max_by_scratch =
+      data_bytes > fixed ? (data_bytes - fixed) / (static_cast<size_t>(nplanes) * H * sizeof(float)) : 0;
   if (want > max_by_scratch) want = max_by_scratch;
   if (want < 1) want = 1;
   if (want > 65535) want = 65535;
@@ -103,9 +94,10 @@ static ColGeom reduce_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec
   return g;
 }
 
-// Geometry of an apply pass: as wide as the row allows (TX up to 256), 8 rows
-// per thread.
-static ColGeom apply_geometry(size_t B, size_t H, bool vec4) {
+// Geometry of an apply pass: as wide as the row allows (TX up to 256), a few
+// blocks per compute unit, each walking its share of the rows.
+static ColGeom apply_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4) {
+  dlmi_tuning const &t = ctx->tune;
   ColGeom g;
   g.vec = vec4 ? 4 : 1;
   size_t const groups = dlmi_ceil_div(H, g.vec);
@@ -117,15 +109,13 @@ static ColGeom apply_geometry(size_t B, size_t H, bool vec4) {
   }
   int const ty = kBlock / tx;
   g.grid_x = static_cast<unsigned>(dlmi_ceil_div(groups, tx));
-  static int const rows_per_thread = env_int("DLMI_NORM_APPLY_ROWS_PER_THREAD", 8);
-  g.rows_per_chunk = static_cast<size_t>(ty) * rows_per_thread;
-  size_t chunks = dlmi_ceil_div(B, g.rows_per_chunk);
-  if (chunks > 65535) {
-    chunks = 65535;
-    g.rows_per_chunk = dlmi_ceil_div(B, chunks);
-    chunks = dlmi_ceil_div(B, g.rows_per_chunk);
-  }
-  g.nchunks = static_cast<unsigned>(chunks);
+  size_t want = dlmi_ceil_div(static_cast<size_t>(ctx->num_cu) * t.apply_blocks_per_cu, g.grid_x);
+  size_t const max_by_rows = B / (static_cast<size_t>(ty) * t.apply_min_rows);
+  if (want > max_by_rows) want = max_by_rows;
+  if (want < 1) want = 1;
+  if (want > 65535) want = 65535;
+  g.rows_per_chunk = dlmi_ceil_div(B, want);
+  g.nchunks = static_cast<unsigned>(dlmi_ceil_div(B, g.rows_per_chunk));
   return g;
 }
 
@@ -155,6 +145,39 @@ __device__ __forceinline__ void load_u8(uint8_t const *p, uint8_t (&v)[VEC]) {
     v[0] = *p;
   }
 }
+
+// The rows of one thread: first, first + step, ... (count of them).  A block
+// either owns a contiguous chunk of rows_per_chunk rows (walked with stride TY)
+// or, with rows_per_chunk == 0, every gridDim.y-th group of TY rows: all blocks
+// of the launch then sweep through memory together as one moving window.
+// (B < 2^32 rows; 32-bit arithmetic and shifts: a 64-bit division here costs
+// every thread a hundred instructions before its first load.)
+struct RowWalk {
+  size_t first, step;
+  unsigned count;
+};
+__device__ __forceinline__ RowWalk row_walk(size_t B, size_t rows_per_chunk, int tx_log2, int ty) {
+  int const ty_log2 = 8 - tx_log2;
+  RowWalk w;
+  if (rows_per_chunk == 0) {
+    unsigned const first = (blockIdx.y << ty_log2) + ty;
+    unsigned const step = gridDim.y << ty_log2;
+    w.first = first;
+    w.step = step;
+    w.count = first < B ? (static_cast<unsigned>(B) - first + step - 1) / step : 0u;
+  } else {
+    size_t const b0 = blockIdx.y * rows_per_chunk;
+    size_t const b1 = (b0 + rows_per_chunk < B) ? b0 + rows_per_chunk : B;
+    w.first = b0 + ty;
+    w.step = size_t(1) << ty_log2;
+    w.count = w.first < b1 ? static_cast<unsigned>((b1 - w.first + w.step - 1) >> ty_log2) : 0u;
+  }
+  return w;
+}
+
+// Keeps the instruction scheduler from moving anything across this point: the
+// loads of a batch of rows stay ahead of the arithmetic on them.
+__device__ __forceinline__ void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
 
 // Sum NV per-thread values over the TY rows of the block.  On return the
 // threads with threadIdx.x < TX hold the block totals for their column group.
@@ -189,130 +212,174 @@ __device__ __forceinline__ void block_rows_reduce(float (&v)[NV], int tx, float 
   }
 }
 
-// ---------------------------------------------------------------- forward: statistics
-// partial[(a * nchunks + chunk) * H + j], a = 0: sum x, 1: sum x^2
-// (phase 1 of fwp_st.cpp:4692-4707 / fwp_mp.cpp:4640-4662)
-template <int VEC>
-__global__ __launch_bounds__(kBlock) void k_col_stats(float const *__restrict__ x, size_t B, size_t H,
-                                                       int tx_log2, size_t rows_per_chunk,
-                                                       float *__restrict__ partial) {
-  __shared__ float lds[4 * kWave * 2 * VEC];
+// Column totals of NP planes of partial sums [NP][nchunks][H] for the block's
+// TX column groups: thread (tx, ty) adds chunks ty, ty+TY, ... with independent
+// loads, then the TY lanes of a column group are combined in a fixed order.  On
+// return threads < TX hold the totals (plane a in tot[a*VEC..]).
+template <int VEC, int NP>
+__device__ __forceinline__ void chunk_totals(float const *partial, unsigned nchunks, size_t H, int tx_log2,
+                                             size_t col, bool live, float (&tot)[NP * VEC], float *lds) {
   int const TX = 1 << tx_log2, TY = kBlock >> tx_log2;
-  int const tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> tx_log2;
-  size_t const col = (static_cast<size_t>(blockIdx.x) * TX + tx) * VEC;
-  bool const live = col < H;
-  size_t const b0 = blockIdx.y * rows_per_chunk;
-  size_t const b1 = (b0 + rows_per_chunk < B) ? b0 + rows_per_chunk : B;
-  float acc[2 * VEC];
+  int const ty = threadIdx.x >> tx_log2;
 #pragma unroll
-  for (int i = 0; i < 2 * VEC; ++i) acc[i] = 0.0f;
+  for (int i = 0; i < NP * VEC; ++i) tot[i] = 0.0f;
   if (live) {
-    constexpr int U = DLMI_STATS_U;
-    size_t b = b0 + ty;
-    for (; b + (U - 1) * static_cast<size_t>(TY) < b1; b += U * static_cast<size_t>(TY)) {
+#pragma unroll 8
+    for (unsigned c = ty; c < nchunks; c += TY) {
+#pragma unroll
+      for (int a = 0; a < NP; ++a) {
+        float v[VEC];
+        load_f<VEC>(partial + (a * static_cast<size_t>(nchunks) + c) * H + col, v);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) tot[a * VEC + i] += v[i];
+      }
+    }
+  }
+  block_rows_reduce<NP * VEC>(tot, TX, lds);
+}
+
+// ---------------------------------------------------------------- forward
+// Phase 2 of fwp_st.cpp:4709-4746 for one unit: batch mean, moving mean, batch
+// std, moving std, then r and d from the UPDATED moving statistics.
+struct FwdFinalize {
+  float *mean, *stdv, *mov_mean, *mov_std, *r, *d;
+  float batch_scale;  // 1 / B as a float, multiplied like the reference's tmp_batch_scale
+  float momentum, eps, r_max, d_max;
+  int renorm;
+};
+
+// mm, ms: the unit's moving mean and moving std as loaded before the sums were
+// formed (so that their latency overlaps the partial-sum loads).
+__device__ __forceinline__ void fwd_finalize_unit(FwdFinalize const &f, size_t j, float s1, float s2, float mm,
+                                                  float ms) {
+  float const mu = s1 * f.batch_scale;
+  mm += f.momentum * (mu - mm);
+  float const sd = sqrtf(s2 * f.batch_scale - mu * mu + f.eps);
+  ms += f.momentum * (sd - ms);
+  f.mean[j] = mu;
+  f.stdv[j] = sd;
+  f.mov_mean[j] = mm;
+  f.mov_std[j] = ms;
+  if (f.renorm) {
+    float const g = sd / ms;
+    float const lo = 1.0f / f.r_max;
+    f.r[j] = g < lo ? lo : (g > f.r_max ? f.r_max : g);
+    float const dd = (mu - mm) / ms;
+    f.d[j] = dd < -f.d_max ? -f.d_max : (dd > f.d_max ? f.d_max : dd);
+  } else {
+    if (f.r != nullptr) f.r[j] = 1.0f;
+    if (f.d != nullptr) f.d[j] = 0.0f;
+  }
+}
+
+struct StatsArgs {
+  float const *x;
+  size_t B, H, rows_per_chunk;
+  int tx_log2;
+  float *partial;  // [NP][nchunks][H]: sum x (and sum x^2) per batch chunk
+};
+
+// Phase 1 of fwp_st.cpp:4692-4707 / fwp_mp.cpp:4640-4662: column sums of x and
+// (NP == 2) x^2 per batch chunk.
+template <int VEC, int NP>
+__global__ __launch_bounds__(kBlock) void k_col_stats(StatsArgs a) {
+  __shared__ float lds[4 * kWave * NP * VEC];
+  int const TX = 1 << a.tx_log2;
+  int const tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> a.tx_log2;
+  size_t const col = (static_cast<size_t>(blockIdx.x) * TX + tx) * VEC;
+  bool const live = col < a.H;
+  RowWalk const w = row_walk(a.B, a.rows_per_chunk, a.tx_log2, ty);
+  float acc[NP * VEC];
+#pragma unroll
+  for (int i = 0; i < NP * VEC; ++i) acc[i] = 0.0f;
+  if (live && w.count > 0) {
+    constexpr int U = 8;
+    size_t const stride = w.step * a.H;
+    float const *p = a.x + w.first * a.H + col;
+    unsigned n = w.count;
+    for (; n >= U; n -= U, p += U * stride) {
       float v[U][VEC];
 #pragma unroll
-      for (int u = 0; u < U; ++u) load_f<VEC>(x + (b + u * static_cast<size_t>(TY)) * H + col, v[u]);
+      for (int u = 0; u < U; ++u) load_f<VEC>(p + u * stride, v[u]);
+      sched_fence();
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
           acc[i] += v[u][i];
-          acc[VEC + i] += v[u][i] * v[u][i];
+          if constexpr (NP == 2) acc[VEC + i] += v[u][i] * v[u][i];
         }
     }
-    for (; b < b1; b += TY) {
+    for (; n > 0; --n, p += stride) {
       float v[VEC];
-      load_f<VEC>(x + b * H + col, v);
+      load_f<VEC>(p, v);
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
         acc[i] += v[i];
-        acc[VEC + i] += v[i] * v[i];
+        if constexpr (NP == 2) acc[VEC + i] += v[i] * v[i];
       }
     }
   }
-  block_rows_reduce<2 * VEC>(acc, TX, lds);
+  block_rows_reduce<NP * VEC>(acc, TX, lds);
+  unsigned const nch = gridDim.y;
   if (threadIdx.x < TX && live) {
-    size_t const nch = gridDim.y;
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      partial[(0 * nch + blockIdx.y) * H + col + i] = acc[i];
-      partial[(1 * nch + blockIdx.y) * H + col + i] = acc[VEC + i];
+    for (int a_ = 0; a_ < NP; ++a_) {
+      float v[VEC];
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[i] = acc[a_ * VEC + i];
+      store_f<VEC>(a.partial + (a_ * static_cast<size_t>(nch) + blockIdx.y) * a.H + col, v);
     }
   }
 }
 
-// Sums NA partial-sum planes over the batch chunks for 16 adjacent units per
-// block: thread (lane c of 16, unit j of 16) adds chunks c, c+16, c+32, ... with
-// independent loads, then the 16 lane totals of a unit are combined through
-// LDS in a fixed order.  On return thread t < 16 holds the totals of unit
-// blockIdx.x*16 + t.
-constexpr int kFinCols = 16;
-constexpr int kFinLanes = kBlock / kFinCols;
-template <int NA>
-__device__ __forceinline__ void chunk_totals(float const *__restrict__ partial, unsigned nchunks, size_t H,
-                                             float (&tot)[NA], float *lds) {
-  int const cj = threadIdx.x % kFinCols;
-  int const cl = threadIdx.x / kFinCols;
-  size_t const j = static_cast<size_t>(blockIdx.x) * kFinCols + cj;
-#pragma unroll
-  for (int a = 0; a < NA; ++a) tot[a] = 0.0f;
-  if (j < H) {
-#pragma unroll 4
-    for (unsigned c = cl; c < nchunks; c += kFinLanes) {
-#pragma unroll
-      for (int a = 0; a < NA; ++a) tot[a] += partial[(a * static_cast<size_t>(nchunks) + c) * H + j];
-    }
+// Geometry of the finalize kernels: a 256-thread block is TX column groups x
+// TY lanes over the chunks, TY the power of two nearest the chunk count (2..64).
+static int finalize_tx_log2(unsigned nchunks) {
+  int ty_log2 = 1;
+  while (ty_log2 < 6 && (1u << ty_log2) < nchunks) ++ty_log2;
+  return 8 - ty_log2;
+}
+
+// Forward finalize from partial sums [2][nchunks][H] (the statistics kernel's,
+// or the GEMM epilogue's with one chunk per tile row).
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void k_fwd_finalize(float const *__restrict__ partial, unsigned nchunks, size_t H,
+                                                          int tx_log2, FwdFinalize fin) {
+  __shared__ float lds[4 * kWave * 2 * VEC];
+  int const TX = 1 << tx_log2;
+  int const tx = threadIdx.x & (TX - 1);
+  size_t const col = (static_cast<size_t>(blockIdx.x) * TX + tx) * VEC;
+  bool const live = col < H;
+  bool const owner = static_cast<int>(threadIdx.x) < TX && live;
+  float mm[VEC], ms[VEC];
+  if (owner) {
+    load_f<VEC>(fin.mov_mean + col, mm);
+    load_f<VEC>(fin.mov_std + col, ms);
   }
+  float tot[2 * VEC];
+  chunk_totals<VEC, 2>(partial, nchunks, H, tx_log2, col, live, tot, lds);
+  if (owner) {
 #pragma unroll
-  for (int a = 0; a < NA; ++a) lds[(cl * kFinCols + cj) * NA + a] = tot[a];
-  __syncthreads();
-  if (threadIdx.x < kFinCols) {
-#pragma unroll
-    for (int a = 0; a < NA; ++a) {
-      float s = 0.0f;
-#pragma unroll
-      for (int l = 0; l < kFinLanes; ++l) s += lds[(l * kFinCols + threadIdx.x) * NA + a];
-      tot[a] = s;
-    }
+    for (int i = 0; i < VEC; ++i) fwd_finalize_unit(fin, col + i, tot[i], tot[VEC + i], mm[i], ms[i]);
   }
 }
 
-// Phase 2 of fwp_st.cpp:4709-4746: batch mean, moving mean, batch std, moving
-// std, then r and d from the UPDATED moving statistics.
-__global__ __launch_bounds__(kBlock) void k_fwd_finalize(float const *__restrict__ partial, unsigned nchunks,
-                                                          size_t B, size_t H, int renorm, float momentum,
-                                                          float eps, float r_max, float d_max,
-                                                          float *__restrict__ mean, float *__restrict__ stdv,
-                                                          float *__restrict__ mov_mean,
-                                                          float *__restrict__ mov_std, float *__restrict__ r,
-                                                          float *__restrict__ d) {
-  __shared__ float lds[kBlock * 2];
-  float tot[2];
-  chunk_totals<2>(partial, nchunks, H, tot, lds);
-  size_t const j = static_cast<size_t>(blockIdx.x) * kFinCols + threadIdx.x;
-  if (threadIdx.x >= kFinCols || j >= H) return;
-  float const s1 = tot[0], s2 = tot[1];
-  float const batch_scale = 1.0f / static_cast<float>(B);
-  float const mu = s1 * batch_scale;
-  float mm = mov_mean[j];
-  mm += momentum * (mu - mm);
-  float const sd = sqrtf(s2 * batch_scale - mu * mu + eps);
-  float ms = mov_std[j];
-  ms += momentum * (sd - ms);
-  mean[j] = mu;
-  stdv[j] = sd;
-  mov_mean[j] = mm;
-  mov_std[j] = ms;
-  if (renorm) {
-    float const g = sd / ms;
-    float const lo = 1.0f / r_max;
-    r[j] = g < lo ? lo : (g > r_max ? r_max : g);
-    float const dd = (mu - mm) / ms;
-    d[j] = dd < -d_max ? -d_max : (dd > d_max ? d_max : dd);
-  } else {
-    if (r != nullptr) r[j] = 1.0f;
-    if (d != nullptr) d[j] = 0.0f;
+// out[j] (+)= column sum, from one plane of statistics partials.
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void k_colsum_finalize(float const *__restrict__ partial, unsigned nchunks,
+                                                             size_t H, int tx_log2, float *__restrict__ out,
+                                                             int accumulate) {
+  __shared__ float lds[4 * kWave * VEC];
+  int const TX = 1 << tx_log2;
+  int const tx = threadIdx.x & (TX - 1);
+  size_t const col = (static_cast<size_t>(blockIdx.x) * TX + tx) * VEC;
+  bool const live = col < H;
+  float tot[VEC];
+  chunk_totals<VEC, 1>(partial, nchunks, H, tx_log2, col, live, tot, lds);
+  if (static_cast<int>(threadIdx.x) < TX && live) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) out[col + i] = accumulate ? out[col + i] + tot[i] : tot[i];
   }
 }
 
@@ -323,6 +390,7 @@ __device__ __forceinline__ float drop_apply(uint8_t m, float scale, float v) { r
 struct FwdApplyArgs {
   float const *x, *gamma, *beta, *mean, *stdv, *r, *d;
   uint8_t const *mask;
+  float const *residual;  // optional [B,H]: y = residual + (activation output after dropout)
   float *y;     // activation output after dropout
   float *xhat;  // optional materialised x_hat            (MAT only)
   float *nrm;   // optional materialised gamma*x_hat+beta (MAT only)
@@ -332,19 +400,19 @@ struct FwdApplyArgs {
 };
 
 // Phase 3 of fwp_st.cpp:4748-4765, then AF_FIRE (fwp_st.cpp:4768-4794), then the
-// dropout leaf, in one pass.
+// dropout leaf (and, with RES, the identity shortcut of fwp_st.cpp:5051-5112),
+// in one pass.
 // MAT: materialise x_hat / the pre-activation (the un-fused leaf) with the
 // reference's expression order.  Otherwise the per-unit constants are folded so
 // that an element costs one subtraction and one fused multiply-add before the
 // activation:  n = (x - mean) * (gamma*r/std) + (gamma*d + beta).
-template <int VEC, int ACT, int DROPM, bool MAT>
+template <int VEC, int ACT, int DROPM, bool MAT, bool RES>
 __global__ __launch_bounds__(kBlock) void k_fwd_apply(FwdApplyArgs a) {
-  int const TX = 1 << a.tx_log2, TY = kBlock >> a.tx_log2;
+  int const TX = 1 << a.tx_log2;
   int const tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> a.tx_log2;
   size_t const col = (static_cast<size_t>(blockIdx.x) * TX + tx) * VEC;
-  if (col >= a.H) return;
-  size_t const b0 = blockIdx.y * a.rows_per_chunk;
-  size_t const b1 = (b0 + a.rows_per_chunk < a.B) ? b0 + a.rows_per_chunk : a.B;
+  RowWalk const w = row_walk(a.B, a.rows_per_chunk, a.tx_log2, ty);
+  if (col >= a.H || w.count == 0) return;
   float mu[VEC], inv[VEC], rr[VEC], dd[VEC], ga[VEC], be[VEC];
   uint8_t mk[VEC];
   load_f<VEC>(a.mean + col, mu);
@@ -364,7 +432,7 @@ __global__ __launch_bounds__(kBlock) void k_fwd_apply(FwdApplyArgs a) {
   }
   if constexpr (DROPM == kDropUnit) load_u8<VEC>(a.mask + col, mk);
   constexpr int U = 4;
-  auto body = [&](size_t off, float const (&xv)[VEC], uint8_t const (&mv)[VEC]) {
+  auto body = [&](size_t off, float const (&xv)[VEC], uint8_t const (&mv)[VEC], float const (&rv)[VEC]) {
     float xh[VEC], nn[VEC], q[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
@@ -376,6 +444,7 @@ __global__ __launch_bounds__(kBlock) void k_fwd_apply(FwdApplyArgs a) {
       }
       q[i] = act_fire<ACT>(nn[i]);
       if constexpr (DROPM != kDropNone) q[i] = drop_apply(mv[i], a.drop_scale, q[i]);
+      if constexpr (RES) q[i] = rv[i] + q[i];
     }
     if constexpr (MAT) {
       if (a.xhat != nullptr) store_f<VEC>(a.xhat + off, xh);
@@ -385,47 +454,85 @@ __global__ __launch_bounds__(kBlock) void k_fwd_apply(FwdApplyArgs a) {
       store_f<VEC>(a.y + off, q);
     }
   };
-  size_t b = b0 + ty;
-  for (; b + (U - 1) * static_cast<size_t>(TY) < b1; b += U * static_cast<size_t>(TY)) {
-    float xv[U][VEC];
+  size_t const stride = w.step * a.H;
+  size_t off = w.first * a.H + col;
+  unsigned n = w.count;
+  for (; n >= U; n -= U, off += U * stride) {
+    float xv[U][VEC], rv[U][VEC];
     uint8_t mv[U][VEC];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      size_t const off = (b + u * static_cast<size_t>(TY)) * a.H + col;
-      load_f<VEC>(a.x + off, xv[u]);
+      load_f<VEC>(a.x + off + u * stride, xv[u]);
+      if constexpr (RES) {
+        load_f<VEC>(a.residual + off + u * stride, rv[u]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) rv[u][i] = 0.0f;
+      }
       if constexpr (DROPM == kDropElem) {
-        load_u8<VEC>(a.mask + off, mv[u]);
+        load_u8<VEC>(a.mask + off + u * stride, mv[u]);
       } else {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) mv[u][i] = mk[i];
       }
     }
+    sched_fence();
 #pragma unroll
-    for (int u = 0; u < U; ++u) body((b + u * static_cast<size_t>(TY)) * a.H + col, xv[u], mv[u]);
+    for (int u = 0; u < U; ++u) body(off + u * stride, xv[u], mv[u], rv[u]);
   }
-  for (; b < b1; b += TY) {
-    float xv[VEC];
+  for (; n > 0; --n, off += stride) {
+    float xv[VEC], rv[VEC];
     uint8_t mv[VEC];
-    size_t const off = b * a.H + col;
     load_f<VEC>(a.x + off, xv);
+    if constexpr (RES) {
+      load_f<VEC>(a.residual + off, rv);
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) rv[i] = 0.0f;
+    }
     if constexpr (DROPM == kDropElem) {
       load_u8<VEC>(a.mask + off, mv);
     } else {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) mv[i] = mk[i];
     }
-    body(off, xv, mv);
+    body(off, xv, mv, rv);
   }
 }
 
 // ---------------------------------------------------------------- backward
+// dgamma += S0, dbeta += S1 (accumulating like the reference's derivative
+// array), dmean, dstd, and the three per-unit coefficients of pass 2
+// (bwp_st.cpp:1508-1531):  dx = e*(r/std) + dstd*((x-mean)/(B*std)) + dmean*(1/B).
+struct BwdFinalize {
+  float const *gamma, *stdv, *r;
+  float *dgamma, *dbeta, *dmean, *dstd;
+  float *coef;  // [3][H]  c1 = gamma*r/std, c2 = dstd/(B*std), c3 = dmean/B
+  float batch_f, batch_scale;  // B and 1/B as floats
+};
+
+// sd, rr, ga, dg, db: the unit's std, r, gamma and running dgamma, dbeta as loaded
+// before the sums were formed.
+__device__ __forceinline__ void bwd_finalize_unit(BwdFinalize const &f, size_t H, size_t j, float s0, float s1,
+                                                  float s2, float sd, float rr, float ga, float dg, float db) {
+  f.dgamma[j] = dg + s0;
+  f.dbeta[j] = db + s1;
+  float const dm = (ga * s1) * (-rr / sd);
+  float const ds = (ga * s2) * (-rr / (sd * sd));
+  if (f.dmean != nullptr) f.dmean[j] = dm;
+  if (f.dstd != nullptr) f.dstd[j] = ds;
+  f.coef[0 * H + j] = ga * (rr / sd);
+  f.coef[1 * H + j] = ds / (f.batch_f * sd);
+  f.coef[2 * H + j] = dm * f.batch_scale;
+}
+
 struct BwdArgs {
   float const *x, *gamma, *beta, *mean, *stdv, *r, *d;
   float const *xhat;  // only when XHAT_GIVEN (un-fused leaf: dn = dY, x_hat stored)
   uint8_t const *mask;
   float const *dY;
   float *partial;     // reduce: [3][nchunks][H]
-  float const *coef;  // apply: [3][H]  c1 = gamma*r/std, c2 = dstd/(B*std), c3 = dmean/B
+  float const *coef;  // apply: [3][H]
   float *dX;
   size_t B, H, rows_per_chunk;
   int tx_log2, drop_bwd_masked;
@@ -484,25 +591,24 @@ __device__ __forceinline__ float bwd_dn(BwdArgs const &a, float xv, float dy, ui
   }
 }
 
-// Pass 1 of bwp_st.cpp:1478-1506: column sums of dn*x_hat, dn and dn*(x-mean).
-// (dmean and dstd follow from the last two in the finalize kernel:
-//  sum e*(-r/std) = -(r/std)*gamma*sum dn, sum e*(x-mean)*(-r/std^2) likewise.)
+// Pass 1 of bwp_st.cpp:1478-1506: column sums of dn*x_hat, dn and dn*(x-mean)
+// per batch chunk (dmean and dstd follow from the last two in the finalize
+// kernel: sum e*(-r/std) = -(r/std)*gamma*sum dn, sum e*(x-mean)*(-r/std^2) likewise).
 template <int VEC, int ACT, int DROPM, bool XHAT_GIVEN>
 __global__ __launch_bounds__(kBlock) void k_bwd_reduce(BwdArgs a) {
   __shared__ float lds[4 * kWave * 3 * VEC];
-  int const TX = 1 << a.tx_log2, TY = kBlock >> a.tx_log2;
+  int const TX = 1 << a.tx_log2;
   int const tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> a.tx_log2;
   size_t const col = (static_cast<size_t>(blockIdx.x) * TX + tx) * VEC;
   bool const live = col < a.H;
-  size_t const b0 = blockIdx.y * a.rows_per_chunk;
-  size_t const b1 = (b0 + a.rows_per_chunk < a.B) ? b0 + a.rows_per_chunk : a.B;
+  RowWalk const w = row_walk(a.B, a.rows_per_chunk, a.tx_log2, ty);
   float acc[3 * VEC];
 #pragma unroll
   for (int i = 0; i < 3 * VEC; ++i) acc[i] = 0.0f;
-  if (live) {
+  if (live && w.count > 0) {
     UnitConsts<VEC> uc;
     load_unit_consts<VEC, DROPM, XHAT_GIVEN>(a, col, uc);
-    constexpr int U = DLMI_BWD_REDUCE_U;
+    constexpr int U = 4;
     auto body = [&](float const (&xv)[VEC], float const (&dy)[VEC], float const (&xg)[VEC],
                     uint8_t const (&mv)[VEC]) {
 #pragma unroll
@@ -515,35 +621,36 @@ __global__ __launch_bounds__(kBlock) void k_bwd_reduce(BwdArgs a) {
         acc[2 * VEC + i] += dn * (xv[i] - uc.mu[i]);
       }
     };
-    size_t b = b0 + ty;
-    for (; b + (U - 1) * static_cast<size_t>(TY) < b1; b += U * static_cast<size_t>(TY)) {
+    size_t const stride = w.step * a.H;
+    size_t off = w.first * a.H + col;
+    unsigned n = w.count;
+    for (; n >= U; n -= U, off += U * stride) {
       float xv[U][VEC], dy[U][VEC], xg[U][VEC];
       uint8_t mv[U][VEC];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        size_t const off = (b + u * static_cast<size_t>(TY)) * a.H + col;
-        load_f<VEC>(a.x + off, xv[u]);
-        load_f<VEC>(a.dY + off, dy[u]);
+        load_f<VEC>(a.x + off + u * stride, xv[u]);
+        load_f<VEC>(a.dY + off + u * stride, dy[u]);
         if constexpr (XHAT_GIVEN) {
-          load_f<VEC>(a.xhat + off, xg[u]);
+          load_f<VEC>(a.xhat + off + u * stride, xg[u]);
         } else {
 #pragma unroll
           for (int i = 0; i < VEC; ++i) xg[u][i] = 0.0f;
         }
         if constexpr (DROPM == kDropElem) {
-          load_u8<VEC>(a.mask + off, mv[u]);
+          load_u8<VEC>(a.mask + off + u * stride, mv[u]);
         } else {
 #pragma unroll
           for (int i = 0; i < VEC; ++i) mv[u][i] = uc.mk[i];
         }
       }
+      sched_fence();
 #pragma unroll
       for (int u = 0; u < U; ++u) body(xv[u], dy[u], xg[u], mv[u]);
     }
-    for (; b < b1; b += TY) {
+    for (; n > 0; --n, off += stride) {
       float xv[VEC], dy[VEC], xg[VEC];
       uint8_t mv[VEC];
-      size_t const off = b * a.H + col;
       load_f<VEC>(a.x + off, xv);
       load_f<VEC>(a.dY + off, dy);
       if constexpr (XHAT_GIVEN) {
@@ -562,56 +669,60 @@ __global__ __launch_bounds__(kBlock) void k_bwd_reduce(BwdArgs a) {
     }
   }
   block_rows_reduce<3 * VEC>(acc, TX, lds);
+  unsigned const nch = gridDim.y;
   if (threadIdx.x < TX && live) {
-    size_t const nch = gridDim.y;
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      a.partial[(0 * nch + blockIdx.y) * a.H + col + i] = acc[i];
-      a.partial[(1 * nch + blockIdx.y) * a.H + col + i] = acc[VEC + i];
-      a.partial[(2 * nch + blockIdx.y) * a.H + col + i] = acc[2 * VEC + i];
+    for (int a_ = 0; a_ < 3; ++a_) {
+      float v[VEC];
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[i] = acc[a_ * VEC + i];
+      store_f<VEC>(a.partial + (a_ * static_cast<size_t>(nch) + blockIdx.y) * a.H + col, v);
     }
   }
 }
 
-// dgamma += S0, dbeta += S1 (accumulating like the reference's derivative
-// array), dmean, dstd, and the three per-unit coefficients of pass 2
-// (bwp_st.cpp:1508-1531):  dx = e*(r/std) + dstd*((x-mean)/(B*std)) + dmean*(1/B).
-__global__ __launch_bounds__(kBlock) void k_bwd_finalize(float const *__restrict__ partial, unsigned nchunks,
-                                                          size_t B, size_t H, float const *__restrict__ gamma,
-                                                          float const *__restrict__ stdv,
-                                                          float const *__restrict__ r,
-                                                          float *__restrict__ dgamma, float *__restrict__ dbeta,
-                                                          float *__restrict__ dmean, float *__restrict__ dstd,
-                                                          float *__restrict__ coef) {
-  __shared__ float lds[kBlock * 3];
-  float tot[3];
-  chunk_totals<3>(partial, nchunks, H, tot, lds);
-  size_t const j = static_cast<size_t>(blockIdx.x) * kFinCols + threadIdx.x;
-  if (threadIdx.x >= kFinCols || j >= H) return;
-  float const s0 = tot[0], s1 = tot[1], s2 = tot[2];
-  float const sd = stdv[j];
-  float const rr = r != nullptr ? r[j] : 1.0f;
-  float const ga = gamma[j];
-  dgamma[j] += s0;
-  dbeta[j] += s1;
-  float const dm = (ga * s1) * (-rr / sd);
-  float const ds = (ga * s2) * (-rr / (sd * sd));
-  if (dmean != nullptr) dmean[j] = dm;
-  if (dstd != nullptr) dstd[j] = ds;
-  float const batch_scale = 1.0f / static_cast<float>(B);
-  coef[0 * H + j] = ga * (rr / sd);
-  coef[1 * H + j] = ds / (static_cast<float>(B) * sd);
-  coef[2 * H + j] = dm * batch_scale;
+// Backward finalize from the partial sums [3][nchunks][H].
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void k_bwd_finalize(float const *__restrict__ partial, unsigned nchunks, size_t H,
+                                                          int tx_log2, BwdFinalize fin) {
+  __shared__ float lds[4 * kWave * 3 * VEC];
+  int const TX = 1 << tx_log2;
+  int const tx = threadIdx.x & (TX - 1);
+  size_t const col = (static_cast<size_t>(blockIdx.x) * TX + tx) * VEC;
+  bool const live = col < H;
+  bool const owner = static_cast<int>(threadIdx.x) < TX && live;
+  float sd[VEC], rr[VEC], ga[VEC], dg[VEC], db[VEC];
+  if (owner) {
+    load_f<VEC>(fin.stdv + col, sd);
+    load_f<VEC>(fin.gamma + col, ga);
+    load_f<VEC>(fin.dgamma + col, dg);
+    load_f<VEC>(fin.dbeta + col, db);
+    if (fin.r != nullptr) {
+      load_f<VEC>(fin.r + col, rr);
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) rr[i] = 1.0f;
+    }
+  }
+  float tot[3 * VEC];
+  chunk_totals<VEC, 3>(partial, nchunks, H, tx_log2, col, live, tot, lds);
+  if (owner) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i)
+      bwd_finalize_unit(fin, H, col + i, tot[i], tot[VEC + i], tot[2 * VEC + i], sd[i], rr[i], ga[i], dg[i], db[i]);
+  }
 }
 
-template <int VEC, int ACT, int DROPM, bool XHAT_GIVEN>
+// Pass 2 of bwp_st.cpp:1508-1531 with the activation derivative recomputed.
+// ACC: dX += instead of dX = (the error array of a layer that also receives a
+// shortcut's gradient, bwp_st.cpp:1112-1175).
+template <int VEC, int ACT, int DROPM, bool XHAT_GIVEN, bool ACC>
 __global__ __launch_bounds__(kBlock) void k_bwd_apply(BwdArgs a) {
-  int const TX = 1 << a.tx_log2, TY = kBlock >> a.tx_log2;
+  int const TX = 1 << a.tx_log2;
   int const tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> a.tx_log2;
   size_t const col = (static_cast<size_t>(blockIdx.x) * TX + tx) * VEC;
-  if (col >= a.H) return;
-  size_t const b0 = blockIdx.y * a.rows_per_chunk;
-  size_t const b1 = (b0 + a.rows_per_chunk < a.B) ? b0 + a.rows_per_chunk : a.B;
+  RowWalk const w = row_walk(a.B, a.rows_per_chunk, a.tx_log2, ty);
+  if (col >= a.H || w.count == 0) return;
   UnitConsts<VEC> uc;
   load_unit_consts<VEC, DROPM, XHAT_GIVEN>(a, col, uc);
   float c1[VEC], c2[VEC], c3[VEC];
@@ -619,7 +730,8 @@ __global__ __launch_bounds__(kBlock) void k_bwd_apply(BwdArgs a) {
   load_f<VEC>(a.coef + 1 * a.H + col, c2);
   load_f<VEC>(a.coef + 2 * a.H + col, c3);
   constexpr int U = 4;
-  auto body = [&](size_t off, float const (&xv)[VEC], float const (&dy)[VEC], uint8_t const (&mv)[VEC]) {
+  auto body = [&](size_t off, float const (&xv)[VEC], float const (&dy)[VEC], uint8_t const (&mv)[VEC],
+                  float const (&old)[VEC]) {
     float dx[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
@@ -627,41 +739,55 @@ __global__ __launch_bounds__(kBlock) void k_bwd_apply(BwdArgs a) {
       float const dn = bwd_dn<ACT, DROPM, XHAT_GIVEN>(a, xv[i], dy[i], mv[i], uc.mu[i], uc.rs[i], uc.dd[i], uc.ga[i],
                                                       uc.be[i], xh);
       dx[i] = dn * c1[i] + (xv[i] - uc.mu[i]) * c2[i] + c3[i];
+      if constexpr (ACC) dx[i] += old[i];
     }
     store_f<VEC>(a.dX + off, dx);
   };
-  size_t b = b0 + ty;
-  for (; b + (U - 1) * static_cast<size_t>(TY) < b1; b += U * static_cast<size_t>(TY)) {
-    float xv[U][VEC], dy[U][VEC];
+  size_t const stride = w.step * a.H;
+  size_t off = w.first * a.H + col;
+  unsigned n = w.count;
+  for (; n >= U; n -= U, off += U * stride) {
+    float xv[U][VEC], dy[U][VEC], old[U][VEC];
     uint8_t mv[U][VEC];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      size_t const off = (b + u * static_cast<size_t>(TY)) * a.H + col;
-      load_f<VEC>(a.x + off, xv[u]);
-      load_f<VEC>(a.dY + off, dy[u]);
+      load_f<VEC>(a.x + off + u * stride, xv[u]);
+      load_f<VEC>(a.dY + off + u * stride, dy[u]);
+      if constexpr (ACC) {
+        load_f<VEC>(a.dX + off + u * stride, old[u]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) old[u][i] = 0.0f;
+      }
       if constexpr (DROPM == kDropElem) {
-        load_u8<VEC>(a.mask + off, mv[u]);
+        load_u8<VEC>(a.mask + off + u * stride, mv[u]);
       } else {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) mv[u][i] = uc.mk[i];
       }
     }
+    sched_fence();
 #pragma unroll
-    for (int u = 0; u < U; ++u) body((b + u * static_cast<size_t>(TY)) * a.H + col, xv[u], dy[u], mv[u]);
+    for (int u = 0; u < U; ++u) body(off + u * stride, xv[u], dy[u], mv[u], old[u]);
   }
-  for (; b < b1; b += TY) {
-    float xv[VEC], dy[VEC];
+  for (; n > 0; --n, off += stride) {
+    float xv[VEC], dy[VEC], old[VEC];
     uint8_t mv[VEC];
-    size_t const off = b * a.H + col;
     load_f<VEC>(a.x + off, xv);
     load_f<VEC>(a.dY + off, dy);
+    if constexpr (ACC) {
+      load_f<VEC>(a.dX + off, old);
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) old[i] = 0.0f;
+    }
     if constexpr (DROPM == kDropElem) {
       load_u8<VEC>(a.mask + off, mv);
     } else {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) mv[i] = uc.mk[i];
     }
-    body(off, xv, dy, mv);
+    body(off, xv, dy, mv, old);
   }
 }
 
@@ -673,13 +799,26 @@ static bool use_vec4(size_t H, std::initializer_list<void const *> ptrs) {
   return true;
 }
 
-// Runs f.template operator()<DROPM>() for the runtime dropout mode.
+// Runs the statement with DROPM bound to the runtime dropout mode.
 #define DLMI_DISPATCH_DROP(mode, ...)                                         \
   switch (mode) {                                                             \
     case kDropUnit: { constexpr int DROPM = kDropUnit; __VA_ARGS__; } break;  \
     case kDropElem: { constexpr int DROPM = kDropElem; __VA_ARGS__; } break;  \
     default: { constexpr int DROPM = kDropNone; __VA_ARGS__; } break;         \
   }
+
+// The context's own scratch, grown to what a reduction over [*, H] can use:
+// 3 planes of partial sums [chunks][H] with chunks * H <= blocks * (widest
+// block: 256 column groups of 4 units) + H, and the 3*H backward coefficients.
+static int ctx_scratch(dlmi_ctx *ctx, size_t H, ScratchView *v) {
+  size_t const blocks = static_cast<size_t>(ctx->num_cu) * ctx->tune.reduce_blocks_per_cu;
+  size_t const need = 3 * sizeof(float) * (blocks * 1024 + 2 * H) + round_up(3 * H * sizeof(float), 256) + 4096;
+  int rc = dlmi_scratch_reserve(ctx, need);
+  if (rc != DLMI_OK) return rc;
+  v->data = dlmi_scratch_data(ctx);
+  v->data_bytes = ctx->scratch_bytes;
+  return DLMI_OK;
+}
 
 struct FwdTrainCall {
   dlmi_norm norm;
@@ -688,53 +827,81 @@ struct FwdTrainCall {
   float momentum, eps, r_max, d_max, drop_scale;
   float const *x, *gamma, *beta;
   uint8_t const *mask;
+  float const *residual = nullptr;
   float *mean, *stdv, *mov_mean, *mov_std, *r, *d, *y, *xhat, *nrm;
   float const *partial_in = nullptr;  // column-sum partials already produced elsewhere ...
   unsigned partial_chunks = 0;        // ... [2][partial_chunks][H]; skips the statistics pass
 };
 
-static int run_fwd_train(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c) {
-  int rc = dlmi_scratch_reserve(ctx, 2 * 16 * 2 * H * sizeof(float));
-  if (rc != DLMI_OK) return rc;
-  bool const vec4 = use_vec4(H, {c.x, c.gamma, c.beta, c.mean, c.stdv, c.r, c.d, c.y, c.xhat, c.nrm}) &&
+static int run_fwd_train(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, FwdTrainCall const &c) {
+  bool const vec4 = use_vec4(H, {c.x, c.gamma, c.beta, c.mean, c.stdv, c.mov_mean, c.mov_std, c.r, c.d, c.y, c.xhat, c.nrm,
+                                 c.residual}) &&
                     (c.drop_mode == kDropNone || (reinterpret_cast<uintptr_t>(c.mask) & 3u) == 0);
   dim3 const block(kBlock);
+  FwdFinalize fin;
+  fin.mean = c.mean; fin.stdv = c.stdv; fin.mov_mean = c.mov_mean; fin.mov_std = c.mov_std; fin.r = c.r; fin.d = c.d;
+  fin.batch_scale = 1.0f / static_cast<float>(B);
+  fin.momentum = c.momentum; fin.eps = c.eps; fin.r_max = c.r_max; fin.d_max = c.d_max;
+  fin.renorm = c.norm == DLMI_NORM_BATCH_RENORM ? 1 : 0;
   float const *partial = c.partial_in;
   unsigned nchunks = c.partial_chunks;
   if (partial == nullptr) {
-    ColGeom const g = reduce_geometry(ctx, B, H, vec4, 2);
-    float *pw = reinterpret_cast<float *>(ctx->scratch);
+    ColGeom const g = reduce_geometry(ctx, B, H, vec4, 2, sv.data_bytes);
+    if (static_cast<size_t>(2) * g.nchunks * H * sizeof(float) > sv.data_bytes)
+      return dlmi_fail(ctx, DLMI_E_UNSUPPORTED, "%zu units need more scratch than the %zu bytes at hand", H,
+                       sv.data_bytes);
+    StatsArgs s{};
+    s.x = c.x; s.B = B; s.H = H;
+    s.rows_per_chunk = ctx->tune.reduce_interleave ? 0 : g.rows_per_chunk; s.tx_log2 = g.tx_log2;
+    s.partial = reinterpret_cast<float *>(sv.data);
     dim3 const grid(g.grid_x, g.nchunks);
     if (vec4)
-      hipLaunchKernelGGL(k_col_stats<4>, grid, block, 0, ctx->stream, c.x, B, H, g.tx_log2, g.rows_per_chunk, pw);
+      hipLaunchKernelGGL((k_col_stats<4, 2>), grid, block, 0, ctx->stream, s);
     else
-      hipLaunchKernelGGL(k_col_stats<1>, grid, block, 0, ctx->stream, c.x, B, H, g.tx_log2, g.rows_per_chunk, pw);
+      hipLaunchKernelGGL((k_col_stats<1, 2>), grid, block, 0, ctx->stream, s);
     DLMI_LAUNCH_CHECK(ctx, "k_col_stats");
-    partial = pw;
+    partial = s.partial;
     nchunks = g.nchunks;
   }
-  hipLaunchKernelGGL(k_fwd_finalize, dim3(static_cast<unsigned>(dlmi_ceil_div(H, kFinCols))), block, 0, ctx->stream,
-                     partial, nchunks, B, H, c.norm == DLMI_NORM_BATCH_RENORM ? 1 : 0, c.momentum, c.eps,
-                     c.r_max, c.d_max, c.mean, c.stdv, c.mov_mean, c.mov_std, c.r, c.d);
-  DLMI_LAUNCH_CHECK(ctx, "k_fwd_finalize");
-  ColGeom const ga = apply_geometry(B, H, vec4);
+  {
+    bool const pvec4 = vec4 && dlmi_aligned16(partial);
+    size_t const groups = dlmi_ceil_div(H, pvec4 ? 4 : 1);
+    int const ftx = finalize_tx_log2(nchunks);
+    dim3 const grid(static_cast<unsigned>(dlmi_ceil_div(groups, size_t(1) << ftx)));
+    if (pvec4)
+      hipLaunchKernelGGL(k_fwd_finalize<4>, grid, block, 0, ctx->stream, partial, nchunks, H, ftx, fin);
+    else
+      hipLaunchKernelGGL(k_fwd_finalize<1>, grid, block, 0, ctx->stream, partial, nchunks, H, ftx, fin);
+    DLMI_LAUNCH_CHECK(ctx, "k_fwd_finalize");
+  }
+  ColGeom const ga = apply_geometry(ctx, B, H, vec4);
   FwdApplyArgs a;
   a.x = c.x; a.gamma = c.gamma; a.beta = c.beta; a.mean = c.mean; a.stdv = c.stdv; a.r = c.r; a.d = c.d;
-  a.mask = c.mask; a.y = c.y; a.xhat = c.xhat; a.nrm = c.nrm;
-  a.B = B; a.H = H; a.rows_per_chunk = ga.rows_per_chunk; a.tx_log2 = ga.tx_log2; a.drop_scale = c.drop_scale;
+  a.mask = c.mask; a.residual = c.residual; a.y = c.y; a.xhat = c.xhat; a.nrm = c.nrm;
+  a.B = B; a.H = H; a.rows_per_chunk = ctx->tune.apply_interleave ? 0 : ga.rows_per_chunk; a.tx_log2 = ga.tx_log2;
+  a.drop_scale = c.drop_scale;
   dim3 const agrid(ga.grid_x, ga.nchunks);
   if (c.xhat != nullptr || c.nrm != nullptr) {  // un-fused leaf: LINEAR, no dropout by construction
     if (vec4)
-      hipLaunchKernelGGL((k_fwd_apply<4, DLMI_ACT_LINEAR, kDropNone, true>), agrid, block, 0, ctx->stream, a);
+      hipLaunchKernelGGL((k_fwd_apply<4, DLMI_ACT_LINEAR, kDropNone, true, false>), agrid, block, 0, ctx->stream, a);
     else
-      hipLaunchKernelGGL((k_fwd_apply<1, DLMI_ACT_LINEAR, kDropNone, true>), agrid, block, 0, ctx->stream, a);
+      hipLaunchKernelGGL((k_fwd_apply<1, DLMI_ACT_LINEAR, kDropNone, true, false>), agrid, block, 0, ctx->stream, a);
   } else if (c.y != nullptr) {
-    DLMI_DISPATCH_ACT(c.act, DLMI_DISPATCH_DROP(c.drop_mode, {
-      if (vec4)
-        hipLaunchKernelGGL((k_fwd_apply<4, ACT, DROPM, false>), agrid, block, 0, ctx->stream, a);
-      else
-        hipLaunchKernelGGL((k_fwd_apply<1, ACT, DROPM, false>), agrid, block, 0, ctx->stream, a);
-    }));
+    if (c.residual != nullptr) {
+      DLMI_DISPATCH_ACT(c.act, DLMI_DISPATCH_DROP(c.drop_mode, {
+        if (vec4)
+          hipLaunchKernelGGL((k_fwd_apply<4, ACT, DROPM, false, true>), agrid, block, 0, ctx->stream, a);
+        else
+          hipLaunchKernelGGL((k_fwd_apply<1, ACT, DROPM, false, true>), agrid, block, 0, ctx->stream, a);
+      }));
+    } else {
+      DLMI_DISPATCH_ACT(c.act, DLMI_DISPATCH_DROP(c.drop_mode, {
+        if (vec4)
+          hipLaunchKernelGGL((k_fwd_apply<4, ACT, DROPM, false, false>), agrid, block, 0, ctx->stream, a);
+        else
+          hipLaunchKernelGGL((k_fwd_apply<1, ACT, DROPM, false, false>), agrid, block, 0, ctx->stream, a);
+      }));
+    }
   }
   DLMI_LAUNCH_CHECK(ctx, "k_fwd_apply");
   return DLMI_OK;
@@ -748,21 +915,29 @@ struct BwdCall {
   float const *x, *gamma, *beta, *mean, *stdv, *r, *d, *xhat, *dY;
   uint8_t const *mask;
   float *dgamma, *dbeta, *dmean, *dstd, *dX;
+  bool accumulate = false;  // dX += instead of dX =
 };
 
-static int run_bwd(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c) {
-  int rc = dlmi_scratch_reserve(ctx, 2 * 16 * 3 * H * sizeof(float));
-  if (rc != DLMI_OK) return rc;
-  bool const vec4 = use_vec4(H, {c.x, c.gamma, c.beta, c.mean, c.stdv, c.r, c.d, c.xhat, c.dY, c.dX}) &&
+static int run_bwd(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, BwdCall const &c) {
+  bool const vec4 = use_vec4(H, {c.x, c.gamma, c.beta, c.mean, c.stdv, c.r, c.d, c.xhat, c.dY, c.dX, c.dgamma, c.dbeta}) &&
                     (c.drop_mode == kDropNone || (reinterpret_cast<uintptr_t>(c.mask) & 3u) == 0);
-  ColGeom const g = reduce_geometry(ctx, B, H, vec4, 3);
-  // scratch: first half partials [3][nchunks][H], second half coefficients [3][H]
-  float *partial = reinterpret_cast<float *>(ctx->scratch);
-  float *coef = reinterpret_cast<float *>(ctx->scratch + ctx->scratch_bytes / 2);
-  BwdArgs a;
+  ColGeom const g = reduce_geometry(ctx, B, H, vec4, 3, sv.data_bytes);
+  // data region: coefficients [3][H] first, then the partial sums [3][nchunks][H]
+  size_t const coef_bytes = round_up(3 * H * sizeof(float), 256);
+  if (coef_bytes + static_cast<size_t>(3) * g.nchunks * H * sizeof(float) > sv.data_bytes)
+    return dlmi_fail(ctx, DLMI_E_UNSUPPORTED, "%zu units need more scratch than the %zu bytes at hand", H,
+                     sv.data_bytes);
+  float *coef = reinterpret_cast<float *>(sv.data);
+  float *partial = reinterpret_cast<float *>(sv.data + coef_bytes);
+  BwdArgs a{};
   a.x = c.x; a.gamma = c.gamma; a.beta = c.beta; a.mean = c.mean; a.stdv = c.stdv; a.r = c.r; a.d = c.d;
-  a.xhat = c.xhat; a.mask = c.mask; a.dY = c.dY; a.partial = partial; a.coef = coef; a.dX = c.dX;
-  a.B = B; a.H = H; a.rows_per_chunk = g.rows_per_chunk; a.tx_log2 = g.tx_log2;
+  a.xhat = c.xhat; a.mask = c.mask; a.dY = c.dY; a.partial = partial; a.coef = coef;
+  a.dX = c.dX;
+  BwdFinalize fin;
+  fin.gamma = c.gamma; fin.stdv = c.stdv; fin.r = c.r; fin.dgamma = c.dgamma; fin.dbeta = c.dbeta;
+  fin.dmean = c.dmean; fin.dstd = c.dstd; fin.coef = coef;
+  fin.batch_f = static_cast<float>(B); fin.batch_scale = 1.0f / static_cast<float>(B);
+  a.B = B; a.H = H; a.rows_per_chunk = ctx->tune.reduce_interleave ? 0 : g.rows_per_chunk; a.tx_log2 = g.tx_log2;
   a.drop_bwd_masked = c.drop_bwd_masked; a.drop_scale = c.drop_scale;
   dim3 const grid(g.grid_x, g.nchunks), block(kBlock);
   if (c.xhat_given) {
@@ -779,24 +954,38 @@ static int run_bwd(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c) {
     }));
   }
   DLMI_LAUNCH_CHECK(ctx, "k_bwd_reduce");
-  hipLaunchKernelGGL(k_bwd_finalize, dim3(static_cast<unsigned>(dlmi_ceil_div(H, kFinCols))), block, 0, ctx->stream,
-                     partial, g.nchunks, B, H, c.gamma, c.stdv, c.r, c.dgamma, c.dbeta, c.dmean, c.dstd, coef);
-  DLMI_LAUNCH_CHECK(ctx, "k_bwd_finalize");
-  ColGeom const ga = apply_geometry(B, H, vec4);
-  a.rows_per_chunk = ga.rows_per_chunk;
+  {
+    size_t const groups = dlmi_ceil_div(H, vec4 ? 4 : 1);
+    int const ftx = finalize_tx_log2(g.nchunks);
+    dim3 const fgrid(static_cast<unsigned>(dlmi_ceil_div(groups, size_t(1) << ftx)));
+    if (vec4)
+      hipLaunchKernelGGL(k_bwd_finalize<4>, fgrid, block, 0, ctx->stream, partial, g.nchunks, H, ftx, fin);
+    else
+      hipLaunchKernelGGL(k_bwd_finalize<1>, fgrid, block, 0, ctx->stream, partial, g.nchunks, H, ftx, fin);
+    DLMI_LAUNCH_CHECK(ctx, "k_bwd_finalize");
+  }
+  ColGeom const ga = apply_geometry(ctx, B, H, vec4);
+  a.rows_per_chunk = ctx->tune.apply_interleave ? 0 : ga.rows_per_chunk;
   a.tx_log2 = ga.tx_log2;
   dim3 const agrid(ga.grid_x, ga.nchunks);
   if (c.xhat_given) {
     if (vec4)
-      hipLaunchKernelGGL((k_bwd_apply<4, DLMI_ACT_LINEAR, kDropNone, true>), agrid, block, 0, ctx->stream, a);
+      hipLaunchKernelGGL((k_bwd_apply<4, DLMI_ACT_LINEAR, kDropNone, true, false>), agrid, block, 0, ctx->stream, a);
     else
-      hipLaunchKernelGGL((k_bwd_apply<1, DLMI_ACT_LINEAR, kDropNone, true>), agrid, block, 0, ctx->stream, a);
+      hipLaunchKernelGGL((k_bwd_apply<1, DLMI_ACT_LINEAR, kDropNone, true, false>), agrid, block, 0, ctx->stream, a);
+  } else if (c.accumulate) {
+    DLMI_DISPATCH_ACT(c.act, DLMI_DISPATCH_DROP(c.drop_mode, {
+      if (vec4)
+        hipLaunchKernelGGL((k_bwd_apply<4, ACT, DROPM, false, true>), agrid, block, 0, ctx->stream, a);
+      else
+        hipLaunchKernelGGL((k_bwd_apply<1, ACT, DROPM, false, true>), agrid, block, 0, ctx->stream, a);
+    }));
   } else {
     DLMI_DISPATCH_ACT(c.act, DLMI_DISPATCH_DROP(c.drop_mode, {
       if (vec4)
-        hipLaunchKernelGGL((k_bwd_apply<4, ACT, DROPM, false>), agrid, block, 0, ctx->stream, a);
+        hipLaunchKernelGGL((k_bwd_apply<4, ACT, DROPM, false, false>), agrid, block, 0, ctx->stream, a);
       else
-        hipLaunchKernelGGL((k_bwd_apply<1, ACT, DROPM, false>), agrid, block, 0, ctx->stream, a);
+        hipLaunchKernelGGL((k_bwd_apply<1, ACT, DROPM, false, false>), agrid, block, 0, ctx->stream, a);
     }));
   }
   DLMI_LAUNCH_CHECK(ctx, "k_bwd_apply");
@@ -824,13 +1013,9 @@ static float drop_scale_of(dlmi_fused_desc const *desc) {
   return desc->dropout == DLMI_DROP_BERNOULLI_INVERTED ? desc->drop_scale : 1.0f;
 }
 
-int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
-                            float const *gamma, float const *beta, uint8_t const *mask, float *mean, float *stdv,
-                            float *mov_mean, float *mov_std, float *r, float *d, float *y, float const *partial,
-                            unsigned nchunks) {
-  int rc = check_desc(ctx, desc, mask);
-  if (rc != DLMI_OK) return rc;
-  DLMI_REQUIRE(ctx, x && gamma && beta && mean && stdv && mov_mean && mov_std && r && d && y, "null pointer");
+static FwdTrainCall fused_fwd_call(dlmi_fused_desc const *desc, float const *x, float const *gamma, float const *beta,
+                                   uint8_t const *mask, float *mean, float *stdv, float *mov_mean, float *mov_std,
+                                   float *r, float *d, float *y) {
   FwdTrainCall c;
   c.norm = desc->norm; c.act = desc->act; c.drop_mode = drop_mode_of(desc);
   c.momentum = desc->momentum; c.eps = desc->eps; c.r_max = desc->r_max; c.d_max = desc->d_max;
@@ -838,35 +1023,49 @@ int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
   c.x = x; c.gamma = gamma; c.beta = beta; c.mask = mask;
   c.mean = mean; c.stdv = stdv; c.mov_mean = mov_mean; c.mov_std = mov_std; c.r = r; c.d = d;
   c.y = y; c.xhat = nullptr; c.nrm = nullptr;
-  c.partial_in = partial; c.partial_chunks = nchunks;
-  return run_fwd_train(ctx, B, H, c);
+  return c;
 }
 
-// out[j] (+)= column sum, from the first plane of the statistics partials.
-__global__ __launch_bounds__(kBlock) void k_colsum_finalize(float const *__restrict__ partial, unsigned nchunks,
-                                                             size_t H, float *__restrict__ out, int accumulate) {
-  __shared__ float lds[kBlock];
-  float tot[1];
-  chunk_totals<1>(partial, nchunks, H, tot, lds);
-  size_t const j = static_cast<size_t>(blockIdx.x) * kFinCols + threadIdx.x;
-  if (threadIdx.x >= kFinCols || j >= H) return;
-  out[j] = accumulate ? out[j] + tot[0] : tot[0];
+int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
+                            float const *gamma, float const *beta, uint8_t const *mask, float const *residual,
+                            float *mean, float *stdv, float *mov_mean, float *mov_std, float *r, float *d, float *y,
+                            float const *partial, unsigned nchunks) {
+  int rc = check_desc(ctx, desc, mask);
+  if (rc != DLMI_OK) return rc;
+  DLMI_REQUIRE(ctx, x && gamma && beta && mean && stdv && mov_mean && mov_std && r && d && y, "null pointer");
+  FwdTrainCall c = fused_fwd_call(desc, x, gamma, beta, mask, mean, stdv, mov_mean, mov_std, r, d, y);
+  c.residual = residual;
+  c.partial_in = partial; c.partial_chunks = nchunks;
+  ScratchView sv{};
+  if (partial == nullptr) {
+    rc = ctx_scratch(ctx, H, &sv);
+    if (rc != DLMI_OK) return rc;
+  }
+  return run_fwd_train(ctx, sv, B, H, c);
 }
 
 int column_sums(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *out, int accumulate) {
-  int rc = dlmi_scratch_reserve(ctx, 2 * 16 * 2 * H * sizeof(float));
+  ScratchView sv{};
+  int rc = ctx_scratch(ctx, H, &sv);
   if (rc != DLMI_OK) return rc;
-  bool const vec4 = use_vec4(H, {x});
-  ColGeom const g = reduce_geometry(ctx, B, H, vec4, 2);
-  float *pw = reinterpret_cast<float *>(ctx->scratch);
+  bool const vec4 = use_vec4(H, {x, out});
+  ColGeom const g = reduce_geometry(ctx, B, H, vec4, 1, sv.data_bytes);
+  StatsArgs s{};
+  s.x = x; s.B = B; s.H = H; s.rows_per_chunk = ctx->tune.reduce_interleave ? 0 : g.rows_per_chunk; s.tx_log2 = g.tx_log2;
+  s.partial = reinterpret_cast<float *>(sv.data);
   dim3 const grid(g.grid_x, g.nchunks), block(kBlock);
   if (vec4)
-    hipLaunchKernelGGL(k_col_stats<4>, grid, block, 0, ctx->stream, x, B, H, g.tx_log2, g.rows_per_chunk, pw);
+    hipLaunchKernelGGL((k_col_stats<4, 1>), grid, block, 0, ctx->stream, s);
   else
-    hipLaunchKernelGGL(k_col_stats<1>, grid, block, 0, ctx->stream, x, B, H, g.tx_log2, g.rows_per_chunk, pw);
+    hipLaunchKernelGGL((k_col_stats<1, 1>), grid, block, 0, ctx->stream, s);
   DLMI_LAUNCH_CHECK(ctx, "k_col_stats");
-  hipLaunchKernelGGL(k_colsum_finalize, dim3(static_cast<unsigned>(dlmi_ceil_div(H, kFinCols))), block, 0, ctx->stream,
-                     pw, g.nchunks, H, out, accumulate);
+  size_t const groups = dlmi_ceil_div(H, vec4 ? 4 : 1);
+  int const ftx = finalize_tx_log2(g.nchunks);
+  dim3 const fgrid(static_cast<unsigned>(dlmi_ceil_div(groups, size_t(1) << ftx)));
+  if (vec4)
+    hipLaunchKernelGGL(k_colsum_finalize<4>, fgrid, block, 0, ctx->stream, s.partial, g.nchunks, H, ftx, out, accumulate);
+  else
+    hipLaunchKernelGGL(k_colsum_finalize<1>, fgrid, block, 0, ctx->stream, s.partial, g.nchunks, H, ftx, out, accumulate);
   DLMI_LAUNCH_CHECK(ctx, "k_colsum_finalize");
   return DLMI_OK;
 }
@@ -891,7 +1090,10 @@ int dlmi_norm_fwd_train(dlmi_ctx *ctx, dlmi_norm norm, size_t B, size_t H, float
   c.x = x; c.gamma = gamma; c.beta = beta; c.mask = nullptr;
   c.mean = mean; c.stdv = stdv; c.mov_mean = mov_mean; c.mov_std = mov_std; c.r = r; c.d = d;
   c.y = nullptr; c.xhat = xhat; c.nrm = out;
-  return run_fwd_train(ctx, B, H, c);
+  ScratchView sv{};
+  int rc = ctx_scratch(ctx, H, &sv);
+  if (rc != DLMI_OK) return rc;
+  return run_fwd_train(ctx, sv, B, H, c);
 }
 
 int dlmi_fused_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
@@ -902,14 +1104,11 @@ int dlmi_fused_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
   if (rc != DLMI_OK) return rc;
   DLMI_REQUIRE(ctx, B > 0 && H > 0, "empty tensor");
   DLMI_REQUIRE(ctx, x && gamma && beta && mean && stdv && mov_mean && mov_std && r && d && y, "null pointer");
-  FwdTrainCall c;
-  c.norm = desc->norm; c.act = desc->act; c.drop_mode = drop_mode_of(desc);
-  c.momentum = desc->momentum; c.eps = desc->eps; c.r_max = desc->r_max; c.d_max = desc->d_max;
-  c.drop_scale = drop_scale_of(desc);
-  c.x = x; c.gamma = gamma; c.beta = beta; c.mask = mask;
-  c.mean = mean; c.stdv = stdv; c.mov_mean = mov_mean; c.mov_std = mov_std; c.r = r; c.d = d;
-  c.y = y; c.xhat = nullptr; c.nrm = nullptr;
-  return run_fwd_train(ctx, B, H, c);
+  FwdTrainCall const c = fused_fwd_call(desc, x, gamma, beta, mask, mean, stdv, mov_mean, mov_std, r, d, y);
+  ScratchView sv{};
+  rc = ctx_scratch(ctx, H, &sv);
+  if (rc != DLMI_OK) return rc;
+  return run_fwd_train(ctx, sv, B, H, c);
 }
 
 int dlmi_norm_bwd(dlmi_ctx *ctx, dlmi_norm norm, size_t B, size_t H, float const *mean, float const *stdv,
@@ -926,7 +1125,10 @@ int dlmi_norm_bwd(dlmi_ctx *ctx, dlmi_norm norm, size_t B, size_t H, float const
   c.x = x; c.gamma = gamma; c.beta = nullptr; c.mean = mean; c.stdv = stdv;
   c.r = norm == DLMI_NORM_BATCH_RENORM ? r : nullptr; c.d = nullptr; c.xhat = xhat; c.dY = dN; c.mask = nullptr;
   c.dgamma = dgamma; c.dbeta = dbeta; c.dmean = dmean; c.dstd = dstd; c.dX = dx;
-  return run_bwd(ctx, B, H, c);
+  ScratchView sv{};
+  int rc = ctx_scratch(ctx, H, &sv);
+  if (rc != DLMI_OK) return rc;
+  return run_bwd(ctx, sv, B, H, c);
 }
 
 int dlmi_fused_norm_act_bwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
@@ -945,7 +1147,10 @@ int dlmi_fused_norm_act_bwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
   c.x = x; c.gamma = gamma; c.beta = beta; c.mean = mean; c.stdv = stdv; c.r = r; c.d = d; c.xhat = nullptr;
   c.dY = dY; c.mask = mask;
   c.dgamma = dgamma; c.dbeta = dbeta; c.dmean = nullptr; c.dstd = nullptr; c.dX = dX;
-  return run_bwd(ctx, B, H, c);
+  ScratchView sv{};
+  rc = ctx_scratch(ctx, H, &sv);
+  if (rc != DLMI_OK) return rc;
+  return run_bwd(ctx, sv, B, H, c);
 }
 
 }  // extern "C"

@@ -46,16 +46,22 @@ def test_fused_degenerate_shapes(dl, oracle, pkg, B, H, renorm):
     desc = pkg.Dlmi.desc(ACT["ELU"], renorm=renorm, momentum=hyper[0], eps=hyper[1], r_max=hyper[2], d_max=hyper[3])
     dmm, dms = dev(mm), dev(ms)
     yg, st = dl.fused_fwd(desc, dev(x), dev(gamma), dev(beta), dmm, dms)
-    assert_close(host(yg), y, TR, "y")
+    # E[x^2] - mean^2 in fp32 loses log2(E[x^2] / variance) bits: with two or three rows whose values
+    # nearly agree the variance is as small as eps, and every order of evaluation (the reference's own
+    # OpenMP path included) lands within a few roundings of E[x^2], not of the variance
+    x64 = x.astype(np.float64)
+    cond = float(np.max(((x64 * x64).mean(0) + hyper[1]) / (x64.var(0) + hyper[1])))
+    TRC = max(TR, 4 * 2.0 ** -24 * cond)
+    assert_close(host(yg), y, TRC, "y")
     for k in ("mean", "std", "r", "d"):
-        assert_close(host(st[k]), fw[k], TR, k, floor=1.0)
+        assert_close(host(st[k]), fw[k], TRC, k, floor=1.0)
     assert_close(host(dmm), fw["mov_mean"], TR, "moving mean", floor=1.0)
-    assert_close(host(dms), fw["mov_std"], TR, "moving std")
+    assert_close(host(dms), fw["mov_std"], TRC, "moving std")
     dg, db = dev(dg0), dev(db0)
     dX = dl.fused_bwd(desc, dev(x), dev(gamma), dev(beta), st, dev(dY), dg, db)
-    assert_close(host(dX), bw["dx"], TR, "dX", floor=1e-3)
-    assert_close(host(dg), bw["dgamma"], TR, "dgamma", floor=1.0)
-    assert_close(host(db), bw["dbeta"], TR, "dbeta", floor=1.0)
+    assert_close(host(dX), bw["dx"], TRC, "dX", floor=1e-3)
+    assert_close(host(dg), bw["dgamma"], TRC, "dgamma", floor=1.0)
+    assert_close(host(db), bw["dbeta"], TRC, "dbeta", floor=1.0)
     yi = dl.fused_infer(desc, dev(x), dev(gamma), dev(beta), dev(mm), dev(ms))
     assert_close(host(yi), oracle.act_fwd(ACT["ELU"], oracle.norm_fwd_infer(x, gamma, beta, mm, ms)), TR, "inference")
 
