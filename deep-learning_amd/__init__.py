@@ -41,6 +41,7 @@ C_ABI_SYMBOLS = [
     "dlmi_fused_norm_act_fwd", "dlmi_fused_norm_act_bwd", "dlmi_fused_norm_act_infer", "dlmi_fc_norm_act_fwd",
     "dlmi_opt_gd", "dlmi_opt_gd_momentum", "dlmi_opt_adam", "dlmi_zero_padded_identity_fwd", "dlmi_residual_bwd",
     "dlmi_opt_adabound", "dlmi_clip_gradient", "dlmi_max_norm_rows", "dlmi_opt_irprop_plus", "dlmi_loss_seed", "dlmi_zero",
+    "dlmi_fused_norm_act_fwd_noalloc",
 ]
 
 
@@ -316,13 +317,16 @@ class Dlmi:
         return FusedDesc(NORM["BRN"] if renorm else NORM["BN"], act, dropout, 1 if mask_per_element else 0,
                          dropout_bwd, momentum, eps, r_max, d_max, drop_scale)
 
-    def fused_fwd(self, desc, x, gamma, beta, mov_mean, mov_std, mask=None, out=None, stats=None):
-        """Returns (y, stats) with stats = dict(mean,std,r,d) kept for the backward."""
+    def fused_fwd(self, desc, x, gamma, beta, mov_mean, mov_std, mask=None, out=None, stats=None, noalloc=False):
+        """Returns (y, stats) with stats = dict(mean,std,r,d) kept for the backward.
+        noalloc: go through dlmi_fused_norm_act_fwd_noalloc (the library's fixed scratch array; the
+        caller then passes `out` and `stats` so that nothing is allocated on the way)."""
         self._chk(x, gamma, beta, mov_mean, mov_std, mask, out)
         B, H = x.shape
         y = out if out is not None else self.empty(B, H)
         s = stats or dict(mean=self.empty(H), std=self.empty(H), r=self.empty(H), d=self.empty(H))
-        self._ck(self.lib.dlmi_fused_norm_act_fwd(self.ctx, ctypes.byref(desc), c_sz(B), c_sz(H), _p(x), _p(gamma),
+        fn = self.lib.dlmi_fused_norm_act_fwd_noalloc if noalloc else self.lib.dlmi_fused_norm_act_fwd
+        self._ck(fn(self.ctx, ctypes.byref(desc), c_sz(B), c_sz(H), _p(x), _p(gamma),
                                                   _p(beta), _p(mask), _p(s["mean"]), _p(s["std"]), _p(mov_mean),
                                                   _p(mov_std), _p(s["r"]), _p(s["d"]), _p(y)))
         return y, s

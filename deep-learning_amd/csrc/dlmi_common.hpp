@@ -35,6 +35,9 @@ struct dlmi_ctx {
   size_t scratch_bytes = 0;
   char *retired[32] = {nullptr};
   int n_retired = 0;
+  // this device's copy of the fixed scratch array of the entry point that allocates nothing
+  char *static_scratch = nullptr;
+  size_t static_scratch_bytes = 0;
   dlmi_tuning tune;
   char err[512] = {0};
 };
@@ -79,6 +82,8 @@ inline int dlmi_fail(dlmi_ctx *ctx, int code, char const *fmt, ...) {
 int dlmi_scratch_reserve(dlmi_ctx *ctx, size_t bytes);
 
 namespace dlmi {
+// Finds the device address of the library's fixed scratch array for the context's device (current).
+int static_scratch_init(dlmi_ctx *ctx);
 // Batch-(re)norm forward tail (finalize + apply) from column-sum partials
 // [2][nchunks][H] that a producer (the GEMM epilogue) already wrote.
 // partial == nullptr: the statistics come from a pass over x.  residual != nullptr:

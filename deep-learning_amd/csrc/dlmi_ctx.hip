@@ -72,7 +72,10 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
   t.reduce_interleave = env_flag("DLMI_NORM_REDUCE_INTERLEAVE", t.reduce_interleave);
   t.apply_interleave = env_flag("DLMI_NORM_APPLY_INTERLEAVE", t.apply_interleave);
   int rc = dlmi_scratch_reserve(ctx, size_t(16) << 20);
+  if (rc == DLMI_OK) rc = dlmi::static_scratch_init(ctx);
   if (rc != DLMI_OK) {
+    fprintf(stderr, "dlmi: %s\n", ctx->err);
+    if (ctx->scratch != nullptr) (void)hipFree(ctx->scratch);
     delete ctx;
     return rc;
   }

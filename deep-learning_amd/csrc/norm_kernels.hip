@@ -33,11 +33,44 @@
 // Citations: /root/reference/lib/deep-learning/v1/learner/.
 #include <cstdlib>
 #include <initializer_list>
+#include <mutex>
 
 #include "activations.hpp"
 #include "dlmi_common.hpp"
 
+// Reduction scratch of the entry point that allocates nothing
+// (dlmi_fused_norm_act_fwd_noalloc): part of the code object, so every GPU the
+// library runs on holds its own copy from module load until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress; the
+// device address it yields (per device) is what kernels and copies are given.
+constexpr size_t kStaticScratchBytes = size_t(2) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace dlmi {
+
+constexpr int kMaxDevices = 64;
+static void *g_static_scratch[kMaxDevices] = {nullptr};
+static std::mutex g_static_scratch_mutex;
+
+// Called by dlmi_ctx_create with the context's device current: looks up, once
+// per device, where that device keeps its copy of the static scratch array.
+int static_scratch_init(dlmi_ctx *ctx) {
+  if (ctx->device < 0 || ctx->device >= kMaxDevices)
+    return dlmi_fail(ctx, DLMI_E_UNSUPPORTED, "device ordinal %d beyond %d", ctx->device, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  if (g_static_scratch[ctx->device] == nullptr) {
+    void *p = nullptr;
+    hipError_t const e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      return dlmi_fail(ctx, DLMI_E_HIP, "hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
+    }
+    g_static_scratch[ctx->device] = p;
+  }
+  ctx->static_scratch = static_cast<char *>(g_static_scratch[ctx->device]);
+  ctx->static_scratch_bytes = kStaticScratchBytes;
+  return DLMI_OK;
+}
 
 constexpr int kBlock = 256;
 constexpr int kWave = 64;
@@ -1108,6 +1141,28 @@ int dlmi_fused_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
   ScratchView sv{};
   rc = ctx_scratch(ctx, H, &sv);
   if (rc != DLMI_OK) return rc;
+  return run_fwd_train(ctx, sv, B, H, c);
+}
+
+int dlmi_fused_norm_act_fwd_noalloc(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
+                                    float const *gamma, float const *beta, uint8_t const *mask, float *mean,
+                                    float *stdv, float *mov_mean, float *mov_std, float *r, float *d, float *y) {
+  if (ctx == nullptr || desc == nullptr) return DLMI_E_INVALID;
+  int rc = check_desc(ctx, desc, mask);
+  if (rc != DLMI_OK) return rc;
+  DLMI_REQUIRE(ctx, B > 0 && H > 0, "empty tensor");
+  DLMI_REQUIRE(ctx, x && gamma && beta && mean && stdv && mov_mean && mov_std && r && d && y, "null pointer");
+  if (H > DLMI_NOALLOC_MAX_UNITS)
+    return dlmi_fail(ctx, DLMI_E_UNSUPPORTED,
+                     "dlmi_fused_norm_act_fwd_noalloc: %zu units exceed the %d its fixed scratch of %zu bytes is sized for "
+                     "(use dlmi_fused_norm_act_fwd)", H, DLMI_NOALLOC_MAX_UNITS, kStaticScratchBytes);
+  if (ctx->static_scratch == nullptr) return dlmi_fail(ctx, DLMI_E_HIP, "the static scratch of device %d was not found", ctx->device);
+  FwdTrainCall const c = fused_fwd_call(desc, x, gamma, beta, mask, mean, stdv, mov_mean, mov_std, r, d, y);
+  // the device's own copy of the file-scope array, by its device address: no hipMalloc, no hipFree, no
+  // memset (every partial sum the finalize kernel reads is written by the statistics kernel first)
+  ScratchView sv{};
+  sv.data = ctx->static_scratch;
+  sv.data_bytes = ctx->static_scratch_bytes;
   return run_fwd_train(ctx, sv, B, H, c);
 }
 

@@ -244,6 +244,23 @@ int dlmi_fused_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
                             uint8_t const *mask, float *mean, float *std, float *mov_mean,
                             float *mov_std, float *r, float *d, float *y);
 
+/* dlmi_fused_norm_act_fwd for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): same arguments, same kernels and results, but the reduction
+ * partials live in a fixed array of 2 MiB inside the library's code object
+ * (held by every GPU the library is loaded on until the process ends) instead
+ * of the context's growable scratch, so the call reaches no hipMalloc, hipFree
+ * or memset.  It has no counterpart in the reference.  H is limited to
+ * DLMI_NOALLOC_MAX_UNITS units (B is not limited); beyond it the call returns
+ * DLMI_E_UNSUPPORTED.  All calls on one GPU share that GPU's array: calls that
+ * overlap in time on one GPU (two streams, two contexts) race; calls on one
+ * stream are ordered by it. */
+#define DLMI_NOALLOC_MAX_UNITS 65536
+int dlmi_fused_norm_act_fwd_noalloc(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H,
+                                    float const *x, float const *gamma, float const *beta,
+                                    uint8_t const *mask, float *mean, float *std, float *mov_mean,
+                                    float *mov_std, float *r, float *d, float *y);
+
 /* The whole forward of one normalized layer: Z = X W^T with the column sums of Z
  * and Z^2 accumulated in the GEMM epilogue (per 128- or 256-row tile, combined
  * in a fixed order), then the finalize and apply passes of
