@@ -19,8 +19,9 @@ struct dlmi_tuning {
   int reduce_min_rows = 4;        // fewest rows a thread of a reduction block walks
   int apply_blocks_per_cu = 2;    // blocks per compute unit in the apply passes
   int apply_min_rows = 4;
-  int reduce_interleave = 0;      // 1: blocks take every n-th group of rows instead of a contiguous chunk
+  int reduce_interleave = 1;      // 1: blocks take every n-th group of rows instead of a contiguous chunk
   int apply_interleave = 0;
+  int fold_finalize = 1;          // 0: always run the finalize kernels (never fold them into the apply passes)
 };
 
 struct dlmi_ctx {

@@ -71,6 +71,7 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
   t.apply_min_rows = env_knob("DLMI_NORM_APPLY_MIN_ROWS", t.apply_min_rows);
   t.reduce_interleave = env_flag("DLMI_NORM_REDUCE_INTERLEAVE", t.reduce_interleave);
   t.apply_interleave = env_flag("DLMI_NORM_APPLY_INTERLEAVE", t.apply_interleave);
+  t.fold_finalize = env_flag("DLMI_NORM_FOLD_FINALIZE", t.fold_finalize);
   int rc = dlmi_scratch_reserve(ctx, size_t(16) << 20);
   if (rc == DLMI_OK) rc = dlmi::static_scratch_init(ctx);
   if (rc != DLMI_OK) {

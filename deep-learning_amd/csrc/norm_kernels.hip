@@ -6,23 +6,38 @@
 // accesses, enough independent loads in flight per CU and few enough ALU
 // instructions per element that the vector units never become the limit:
 //
-//   forward : statistics (read x)      -> finalize [H] -> apply (read x, write y)
-//   backward: reduce (read dY, x)      -> finalize [H] -> apply (read dY, x, write dX)
+//   forward : statistics (read x)      -> [finalize H] -> apply (read x, write y)
+//   backward: reduce (read dY, x)      -> [finalize H] -> apply (read dY, x, write dX)
 //
 // x_hat, the pre-activation n = gamma*x_hat + beta and the activation output
 // are recomputed in registers instead of being stored and re-read.
 //
 // Thread geometry of the column passes: a 256-thread block is TX x TY; a
-// thread owns VEC (=4, one float4) adjacent units and walks the rows of its
-// block's batch chunk with stride TY.  In the reduction kernels TX <= 64, so
-// when H is small a wavefront spans several rows: those are combined with
-// wavefront shuffles, the four wavefronts of the block with a small LDS tree,
-// and the chunks of the batch by the finalize kernel in chunk order.  No float
-// atomics, a fixed summation order: results are reproducible run to run.
-// (Folding the finalize into the reduction - the block that draws the last of a
-// column group's tickets combines the chunks - was built and measured: its tail
-// of device-scope round trips costs 10 us at [4096 x 4096], twice the separate
-// launch.)
+// thread owns VEC (=4, one float4) adjacent units and walks rows with stride
+// TY.  Rows that share a wavefront are combined with wavefront shuffles, the
+// four wavefronts of the block with a small LDS tree, the chunks of the batch
+// in chunk order.  No float atomics, a fixed summation order: results are
+// reproducible run to run.
+//
+// Who combines the chunks.  Where the shape allows at most 16 chunks per unit
+// and still a block on most compute units (any layer a few thousand units
+// wide), there is NO finalize launch: every block of the apply pass adds the
+// 16 partial sums of its own units in its prologue (they sit in L2) and does
+// the per-unit arithmetic itself; the blocks of one chunk store the per-unit
+// results, and the statistics pass leaves a snapshot of the moving statistics
+// so that every block sees them as they were before the step.  Tall, narrow
+// tensors need many chunks to fill the machine: there a small finalize kernel
+// combines them (TY lanes per unit, then an LDS tree) between the two passes.
+// Both alternatives to this were built and measured on MI355X and rejected:
+// (a) the reduction's last block of a column group (found with a device-scope
+//     ticket) doing the finalize: its chain of device-scope round trips, about
+//     2 us each across XCDs, made the statistics pass 22.8 us at [4096 x 4096]
+//     against 12.7 + 4.4 us for two launches;
+// (b) one launch per direction with a grid-wide barrier and the block's share
+//     of x kept in registers (8 instead of 12 B/element forward): forward 36 us
+//     against 38, backward 73 us against 58 at [4096 x 4096] - the barrier's
+//     round trips and the low occupancy of 1024-thread register-heavy blocks
+//     cost more than the saved re-read.
 // The apply kernels have nothing to reduce and use TX = 256 when H allows, so
 // that every load / store instruction of a block covers 4 KiB of one row.
 //
@@ -99,14 +114,16 @@ static size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // as wide as the cap allows (TX column groups, up to 256: every load of a block
 // then covers 4 KiB of one row), a few blocks per compute unit, each thread
 // walking at least reduce_min_rows rows.
-static ColGeom reduce_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, int nplanes, size_t data_bytes) {
+static ColGeom reduce_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, int nplanes, size_t data_bytes,
+                               int tx_cap = 0, size_t max_chunks = 65535) {
   dlmi_tuning const &t = ctx->tune;
+  if (tx_cap == 0) tx_cap = t.reduce_tx_cap;
   ColGeom g;
   g.vec = vec4 ? 4 : 1;
   size_t const groups = dlmi_ceil_div(H, g.vec);
   int tx = 256;
   g.tx_log2 = 8;
-  while (tx > 1 && (tx > t.reduce_tx_cap || static_cast<size_t>(tx / 2) >= groups)) {
+  while (tx > 1 && (tx > tx_cap || static_cast<size_t>(tx / 2) >= groups)) {
     tx /= 2;
     --g.tx_log2;
   }
@@ -120,11 +137,31 @@ static ColGeom reduce_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec
   size_t const max_by_scratch =
       data_bytes > fixed ? (data_bytes - fixed) / (static_cast<size_t>(nplanes) * H * sizeof(float)) : 0;
   if (want > max_by_scratch) want = max_by_scratch;
+  if (want > max_chunks) want = max_chunks;
   if (want < 1) want = 1;
   if (want > 65535) want = 65535;
   g.rows_per_chunk = dlmi_ceil_div(B, want);
   g.nchunks = static_cast<unsigned>(dlmi_ceil_div(B, g.rows_per_chunk));
   return g;
+}
+
+// Reduction geometry for the two-launch scheme (the apply pass does the per-unit arithmetic from the
+// partial sums): at most kFoldChunks chunks, blocks as narrow as it takes (64, 32 or 16 column groups)
+// to still put a block on most compute units.  False when the shape cannot give both (few units, many
+// rows): the finalize kernel then combines as many chunks as the reduction wants.
+constexpr size_t kFoldChunks = 16;
+static bool fold_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, int nplanes, size_t data_bytes,
+                          ColGeom *g) {
+  if (ctx->tune.fold_finalize == 0) return false;
+  for (int tx = 64; tx >= 16; tx /= 2) {
+    *g = reduce_geometry(ctx, B, H, vec4, nplanes, data_bytes, tx, kFoldChunks);
+    size_t const blocks = static_cast<size_t>(g->grid_x) * g->nchunks;
+    if (blocks * 4 >= static_cast<size_t>(ctx->num_cu) * 3) return true;
+    // small batches never need more chunks than this: few blocks are then all there is to have
+    size_t const ty = kBlock >> g->tx_log2;
+    if (B / (ty * ctx->tune.reduce_min_rows) <= kFoldChunks) return true;
+  }
+  return false;
 }
 
 // Geometry of an apply pass: as wide as the row allows (TX up to 256), a few
@@ -189,17 +226,20 @@ struct RowWalk {
   size_t first, step;
   unsigned count;
 };
-__device__ __forceinline__ RowWalk row_walk(size_t B, size_t rows_per_chunk, int tx_log2, int ty) {
+// `reverse`: block y takes the chunk gridDim.y-1-y.  The apply passes walk the batch from its end: what
+// the reduction pass before them read LAST is what the memory-side cache still holds.
+__device__ __forceinline__ RowWalk row_walk(size_t B, size_t rows_per_chunk, int tx_log2, int ty, bool reverse = false) {
   int const ty_log2 = 8 - tx_log2;
+  unsigned const by = reverse ? gridDim.y - 1u - blockIdx.y : blockIdx.y;
   RowWalk w;
   if (rows_per_chunk == 0) {
-    unsigned const first = (blockIdx.y << ty_log2) + ty;
+    unsigned const first = (by << ty_log2) + ty;
     unsigned const step = gridDim.y << ty_log2;
     w.first = first;
     w.step = step;
     w.count = first < B ? (static_cast<unsigned>(B) - first + step - 1) / step : 0u;
   } else {
-    size_t const b0 = blockIdx.y * rows_per_chunk;
+    size_t const b0 = by * rows_per_chunk;
     size_t const b1 = (b0 + rows_per_chunk < B) ? b0 + rows_per_chunk : B;
     w.first = b0 + ty;
     w.step = size_t(1) << ty_log2;
@@ -281,28 +321,43 @@ struct FwdFinalize {
   int renorm;
 };
 
+// The six per-unit results of the forward step from the two column sums and the
+// unit's moving mean / std as they were before the step.
+struct UnitStats {
+  float mean, stdv, mov_mean, mov_std, r, d;
+};
+__device__ __forceinline__ UnitStats fwd_unit_stats(FwdFinalize const &f, float s1, float s2, float mm, float ms) {
+  UnitStats u;
+  u.mean = s1 * f.batch_scale;
+  mm += f.momentum * (u.mean - mm);
+  u.stdv = sqrtf(s2 * f.batch_scale - u.mean * u.mean + f.eps);
+  ms += f.momentum * (u.stdv - ms);
+  u.mov_mean = mm;
+  u.mov_std = ms;
+  u.r = 1.0f;
+  u.d = 0.0f;
+  if (f.renorm) {
+    float const g = u.stdv / ms;
+    float const lo = 1.0f / f.r_max;
+    u.r = g < lo ? lo : (g > f.r_max ? f.r_max : g);
+    float const dd = (u.mean - mm) / ms;
+    u.d = dd < -f.d_max ? -f.d_max : (dd > f.d_max ? f.d_max : dd);
+  }
+  return u;
+}
+__device__ __forceinline__ void store_unit_stats(FwdFinalize const &f, size_t j, UnitStats const &u) {
+  f.mean[j] = u.mean;
+  f.stdv[j] = u.stdv;
+  f.mov_mean[j] = u.mov_mean;
+  f.mov_std[j] = u.mov_std;
+  if (f.r != nullptr) f.r[j] = u.r;
+  if (f.d != nullptr) f.d[j] = u.d;
+}
 // mm, ms: the unit's moving mean and moving std as loaded before the sums were
 // formed (so that their latency overlaps the partial-sum loads).
 __device__ __forceinline__ void fwd_finalize_unit(FwdFinalize const &f, size_t j, float s1, float s2, float mm,
                                                   float ms) {
-  float const mu = s1 * f.batch_scale;
-  mm += f.momentum * (mu - mm);
-  float const sd = sqrtf(s2 * f.batch_scale - mu * mu + f.eps);
-  ms += f.momentum * (sd - ms);
-  f.mean[j] = mu;
-  f.stdv[j] = sd;
-  f.mov_mean[j] = mm;
-  f.mov_std[j] = ms;
-  if (f.renorm) {
-    float const g = sd / ms;
-    float const lo = 1.0f / f.r_max;
-    f.r[j] = g < lo ? lo : (g > f.r_max ? f.r_max : g);
-    float const dd = (mu - mm) / ms;
-    f.d[j] = dd < -f.d_max ? -f.d_max : (dd > f.d_max ? f.d_max : dd);
-  } else {
-    if (f.r != nullptr) f.r[j] = 1.0f;
-    if (f.d != nullptr) f.d[j] = 0.0f;
-  }
+  store_unit_stats(f, j, fwd_unit_stats(f, s1, s2, mm, ms));
 }
 
 struct StatsArgs {
@@ -310,6 +365,10 @@ struct StatsArgs {
   size_t B, H, rows_per_chunk;
   int tx_log2;
   float *partial;  // [NP][nchunks][H]: sum x (and sum x^2) per batch chunk
+  // optional: the moving statistics are copied to snap [2][H] (by the blocks of chunk 0) for an apply
+  // pass that does the per-unit arithmetic itself and must see them as they were before the step
+  float const *mov_mean, *mov_std;
+  float *snap;
 };
 
 // Phase 1 of fwp_st.cpp:4692-4707 / fwp_mp.cpp:4640-4662: column sums of x and
@@ -362,6 +421,15 @@ __global__ __launch_bounds__(kBlock) void k_col_stats(StatsArgs a) {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) v[i] = acc[a_ * VEC + i];
       store_f<VEC>(a.partial + (a_ * static_cast<size_t>(nch) + blockIdx.y) * a.H + col, v);
+    }
+    if constexpr (NP == 2) {
+      if (a.snap != nullptr && blockIdx.y == 0) {
+        float v[VEC];
+        load_f<VEC>(a.mov_mean + col, v);
+        store_f<VEC>(a.snap + col, v);
+        load_f<VEC>(a.mov_std + col, v);
+        store_f<VEC>(a.snap + a.H + col, v);
+      }
     }
   }
 }
@@ -430,6 +498,12 @@ struct FwdApplyArgs {
   size_t B, H, rows_per_chunk;
   int tx_log2;
   float drop_scale;
+  // fin_partial != nullptr: no finalize kernel ran.  Every block forms the statistics of its own units
+  // from the partial sums [2][fin_chunks][H] (few chunks, summed in chunk order) and the snapshot of the
+  // moving statistics; the blocks of one chunk store the per-unit results.
+  float const *fin_partial, *mov_mean_in, *mov_std_in;
+  unsigned fin_chunks;
+  FwdFinalize fin;
 };
 
 // Phase 3 of fwp_st.cpp:4748-4765, then AF_FIRE (fwp_st.cpp:4768-4794), then the
@@ -444,16 +518,44 @@ __global__ __launch_bounds__(kBlock) void k_fwd_apply(FwdApplyArgs a) {
   int const TX = 1 << a.tx_log2;
   int const tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> a.tx_log2;
   size_t const col = (static_cast<size_t>(blockIdx.x) * TX + tx) * VEC;
-  RowWalk const w = row_walk(a.B, a.rows_per_chunk, a.tx_log2, ty);
+  RowWalk const w = row_walk(a.B, a.rows_per_chunk, a.tx_log2, ty, true);
   if (col >= a.H || w.count == 0) return;
   float mu[VEC], inv[VEC], rr[VEC], dd[VEC], ga[VEC], be[VEC];
   uint8_t mk[VEC];
-  load_f<VEC>(a.mean + col, mu);
-  load_f<VEC>(a.stdv + col, inv);
-  load_f<VEC>(a.r + col, rr);
-  load_f<VEC>(a.d + col, dd);
   load_f<VEC>(a.gamma + col, ga);
   load_f<VEC>(a.beta + col, be);
+  if (!MAT && a.fin_partial != nullptr) {
+    float mm[VEC], ms[VEC], s1[VEC], s2[VEC];
+    load_f<VEC>(a.mov_mean_in + col, mm);
+    load_f<VEC>(a.mov_std_in + col, ms);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) s1[i] = s2[i] = 0.0f;
+    float const *p1 = a.fin_partial + col;
+    float const *p2 = p1 + static_cast<size_t>(a.fin_chunks) * a.H;
+#pragma unroll 8
+    for (unsigned c = 0; c < a.fin_chunks; ++c) {
+      float v1[VEC], v2[VEC];
+      load_f<VEC>(p1 + c * a.H, v1);
+      load_f<VEC>(p2 + c * a.H, v2);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        s1[i] += v1[i];
+        s2[i] += v2[i];
+      }
+    }
+    bool const writer = blockIdx.y == 0 && ty == 0;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      UnitStats const u = fwd_unit_stats(a.fin, s1[i], s2[i], mm[i], ms[i]);
+      if (writer) store_unit_stats(a.fin, col + i, u);
+      mu[i] = u.mean; inv[i] = u.stdv; rr[i] = u.r; dd[i] = u.d;
+    }
+  } else {
+    load_f<VEC>(a.mean + col, mu);
+    load_f<VEC>(a.stdv + col, inv);
+    load_f<VEC>(a.r + col, rr);
+    load_f<VEC>(a.d + col, dd);
+  }
 #pragma unroll
   for (int i = 0; i < VEC; ++i) {
     inv[i] = fast_rcp(inv[i]);
@@ -566,6 +668,12 @@ struct BwdArgs {
   float const *dY;
   float *partial;     // reduce: [3][nchunks][H]
   float const *coef;  // apply: [3][H]
+  // apply, fin_partial != nullptr: no finalize kernel ran; every block forms the coefficients of its
+  // own units from the partial sums [3][fin_chunks][H], the blocks of one chunk accumulate dgamma / dbeta
+  float const *fin_partial;
+  unsigned fin_chunks;
+  float *dgamma, *dbeta;
+  float batch_f, batch_scale;
   float *dX;
   size_t B, H, rows_per_chunk;
   int tx_log2, drop_bwd_masked;
@@ -604,10 +712,10 @@ __device__ __forceinline__ void load_unit_consts(BwdArgs const &a, size_t col, U
 // (bwp_st.cpp:1177-1209 reads the array the dropout leaf overwrote in place);
 // MASKED mode: q is the pre-dropout activation and dY is masked and rescaled.
 template <int ACT, int DROPM, bool XHAT_GIVEN>
-__device__ __forceinline__ float bwd_dn(BwdArgs const &a, float xv, float dy, uint8_t m, float mu, float rs,
-                                        float dd, float ga, float be, float &xh) {
+__device__ __forceinline__ float bwd_dn(float drop_scale, int drop_bwd_masked, float xv, float dy, uint8_t m,
+                                        float mu, float rs, float dd, float ga, float be, float &xh) {
   if constexpr (XHAT_GIVEN) {
-    (void)a; (void)xv; (void)m; (void)mu; (void)rs; (void)dd; (void)ga; (void)be;
+    (void)drop_scale; (void)drop_bwd_masked; (void)xv; (void)m; (void)mu; (void)rs; (void)dd; (void)ga; (void)be;
     return dy;
   } else {
     xh = (xv - mu) * rs + dd;
@@ -615,10 +723,10 @@ __device__ __forceinline__ float bwd_dn(BwdArgs const &a, float xv, float dy, ui
     float q = act_fire<ACT>(nn);
     float g = dy;
     if constexpr (DROPM != kDropNone) {
-      float const gm = drop_apply(m, a.drop_scale, dy);
-      float const qm = drop_apply(m, a.drop_scale, q);
-      g = a.drop_bwd_masked ? gm : dy;
-      q = a.drop_bwd_masked ? q : qm;
+      float const gm = drop_apply(m, drop_scale, dy);
+      float const qm = drop_apply(m, drop_scale, q);
+      g = drop_bwd_masked ? gm : dy;
+      q = drop_bwd_masked ? q : qm;
     }
     return g * act_derive<ACT>(nn, q);
   }
@@ -647,7 +755,7 @@ __global__ __launch_bounds__(kBlock) void k_bwd_reduce(BwdArgs a) {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
         float xh = xg[i];
-        float const dn = bwd_dn<ACT, DROPM, XHAT_GIVEN>(a, xv[i], dy[i], mv[i], uc.mu[i], uc.rs[i], uc.dd[i],
+        float const dn = bwd_dn<ACT, DROPM, XHAT_GIVEN>(a.drop_scale, a.drop_bwd_masked, xv[i], dy[i], mv[i], uc.mu[i], uc.rs[i], uc.dd[i],
                                                         uc.ga[i], uc.be[i], xh);
         acc[i] += dn * xh;
         acc[VEC + i] += dn;
@@ -754,14 +862,57 @@ __global__ __launch_bounds__(kBlock) void k_bwd_apply(BwdArgs a) {
   int const TX = 1 << a.tx_log2;
   int const tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> a.tx_log2;
   size_t const col = (static_cast<size_t>(blockIdx.x) * TX + tx) * VEC;
-  RowWalk const w = row_walk(a.B, a.rows_per_chunk, a.tx_log2, ty);
+  RowWalk const w = row_walk(a.B, a.rows_per_chunk, a.tx_log2, ty, true);
   if (col >= a.H || w.count == 0) return;
   UnitConsts<VEC> uc;
   load_unit_consts<VEC, DROPM, XHAT_GIVEN>(a, col, uc);
   float c1[VEC], c2[VEC], c3[VEC];
-  load_f<VEC>(a.coef + 0 * a.H + col, c1);
-  load_f<VEC>(a.coef + 1 * a.H + col, c2);
-  load_f<VEC>(a.coef + 2 * a.H + col, c3);
+  if (!XHAT_GIVEN && a.fin_partial != nullptr) {
+    float sd[VEC], rr[VEC], s0[VEC], s1[VEC], s2[VEC];
+    load_f<VEC>(a.stdv + col, sd);
+    load_f<VEC>(a.r + col, rr);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) s0[i] = s1[i] = s2[i] = 0.0f;
+    size_t const plane = static_cast<size_t>(a.fin_chunks) * a.H;
+    float const *p0 = a.fin_partial + col;
+#pragma unroll 4
+    for (unsigned c = 0; c < a.fin_chunks; ++c) {
+      float v0[VEC], v1[VEC], v2[VEC];
+      load_f<VEC>(p0 + c * a.H, v0);
+      load_f<VEC>(p0 + plane + c * a.H, v1);
+      load_f<VEC>(p0 + 2 * plane + c * a.H, v2);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        s0[i] += v0[i];
+        s1[i] += v1[i];
+        s2[i] += v2[i];
+      }
+    }
+    if (blockIdx.y == 0 && ty == 0) {
+      float dg[VEC], db[VEC];
+      load_f<VEC>(a.dgamma + col, dg);
+      load_f<VEC>(a.dbeta + col, db);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        dg[i] += s0[i];
+        db[i] += s1[i];
+      }
+      store_f<VEC>(a.dgamma + col, dg);
+      store_f<VEC>(a.dbeta + col, db);
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {  // as bwd_finalize_unit
+      float const dm = (uc.ga[i] * s1[i]) * (-rr[i] / sd[i]);
+      float const ds = (uc.ga[i] * s2[i]) * (-rr[i] / (sd[i] * sd[i]));
+      c1[i] = uc.ga[i] * (rr[i] / sd[i]);
+      c2[i] = ds / (a.batch_f * sd[i]);
+      c3[i] = dm * a.batch_scale;
+    }
+  } else {
+    load_f<VEC>(a.coef + 0 * a.H + col, c1);
+    load_f<VEC>(a.coef + 1 * a.H + col, c2);
+    load_f<VEC>(a.coef + 2 * a.H + col, c3);
+  }
   constexpr int U = 4;
   auto body = [&](size_t off, float const (&xv)[VEC], float const (&dy)[VEC], uint8_t const (&mv)[VEC],
                   float const (&old)[VEC]) {
@@ -769,7 +920,7 @@ __global__ __launch_bounds__(kBlock) void k_bwd_apply(BwdArgs a) {
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
       float xh = 0.0f;
-      float const dn = bwd_dn<ACT, DROPM, XHAT_GIVEN>(a, xv[i], dy[i], mv[i], uc.mu[i], uc.rs[i], uc.dd[i], uc.ga[i],
+      float const dn = bwd_dn<ACT, DROPM, XHAT_GIVEN>(a.drop_scale, a.drop_bwd_masked, xv[i], dy[i], mv[i], uc.mu[i], uc.rs[i], uc.dd[i], uc.ga[i],
                                                       uc.be[i], xh);
       dx[i] = dn * c1[i] + (xv[i] - uc.mu[i]) * c2[i] + c3[i];
       if constexpr (ACC) dx[i] += old[i];
@@ -878,15 +1029,24 @@ static int run_fwd_train(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t 
   fin.renorm = c.norm == DLMI_NORM_BATCH_RENORM ? 1 : 0;
   float const *partial = c.partial_in;
   unsigned nchunks = c.partial_chunks;
+  // data region: [2][H] snapshot of the moving statistics (two-launch scheme), then the partial sums
+  size_t const fixed = round_up(3 * H * sizeof(float), 256);
+  float *const snap = reinterpret_cast<float *>(sv.data);
+  bool fold = false;
   if (partial == nullptr) {
-    ColGeom const g = reduce_geometry(ctx, B, H, vec4, 2, sv.data_bytes);
-    if (static_cast<size_t>(2) * g.nchunks * H * sizeof(float) > sv.data_bytes)
+    ColGeom g;
+    fold = c.xhat == nullptr && c.nrm == nullptr && c.y != nullptr && fold_geometry(ctx, B, H, vec4, 2, sv.data_bytes, &g);
+    if (!fold) g = reduce_geometry(ctx, B, H, vec4, 2, sv.data_bytes);
+    if (fixed + static_cast<size_t>(2) * g.nchunks * H * sizeof(float) > sv.data_bytes)
       return dlmi_fail(ctx, DLMI_E_UNSUPPORTED, "%zu units need more scratch than the %zu bytes at hand", H,
                        sv.data_bytes);
     StatsArgs s{};
     s.x = c.x; s.B = B; s.H = H;
     s.rows_per_chunk = ctx->tune.reduce_interleave ? 0 : g.rows_per_chunk; s.tx_log2 = g.tx_log2;
-    s.partial = reinterpret_cast<float *>(sv.data);
+    s.partial = reinterpret_cast<float *>(sv.data + fixed);
+    if (fold) {
+      s.mov_mean = c.mov_mean; s.mov_std = c.mov_std; s.snap = snap;
+    }
     dim3 const grid(g.grid_x, g.nchunks);
     if (vec4)
       hipLaunchKernelGGL((k_col_stats<4, 2>), grid, block, 0, ctx->stream, s);
@@ -896,7 +1056,7 @@ static int run_fwd_train(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t 
     partial = s.partial;
     nchunks = g.nchunks;
   }
-  {
+  if (!fold) {
     bool const pvec4 = vec4 && dlmi_aligned16(partial);
     size_t const groups = dlmi_ceil_div(H, pvec4 ? 4 : 1);
     int const ftx = finalize_tx_log2(nchunks);
@@ -913,6 +1073,8 @@ static int run_fwd_train(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t 
   a.mask = c.mask; a.residual = c.residual; a.y = c.y; a.xhat = c.xhat; a.nrm = c.nrm;
   a.B = B; a.H = H; a.rows_per_chunk = ctx->tune.apply_interleave ? 0 : ga.rows_per_chunk; a.tx_log2 = ga.tx_log2;
   a.drop_scale = c.drop_scale;
+  a.fin_partial = fold ? partial : nullptr; a.mov_mean_in = snap; a.mov_std_in = snap + H; a.fin_chunks = nchunks;
+  a.fin = fin;
   dim3 const agrid(ga.grid_x, ga.nchunks);
   if (c.xhat != nullptr || c.nrm != nullptr) {  // un-fused leaf: LINEAR, no dropout by construction
     if (vec4)
@@ -954,7 +1116,10 @@ struct BwdCall {
 static int run_bwd(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, BwdCall const &c) {
   bool const vec4 = use_vec4(H, {c.x, c.gamma, c.beta, c.mean, c.stdv, c.r, c.d, c.xhat, c.dY, c.dX, c.dgamma, c.dbeta}) &&
                     (c.drop_mode == kDropNone || (reinterpret_cast<uintptr_t>(c.mask) & 3u) == 0);
-  ColGeom const g = reduce_geometry(ctx, B, H, vec4, 3, sv.data_bytes);
+  ColGeom g;
+  bool const fold = !c.xhat_given && c.dmean == nullptr && c.dstd == nullptr &&
+                    fold_geometry(ctx, B, H, vec4, 3, sv.data_bytes, &g);
+  if (!fold) g = reduce_geometry(ctx, B, H, vec4, 3, sv.data_bytes);
   // data region: coefficients [3][H] first, then the partial sums [3][nchunks][H]
   size_t const coef_bytes = round_up(3 * H * sizeof(float), 256);
   if (coef_bytes + static_cast<size_t>(3) * g.nchunks * H * sizeof(float) > sv.data_bytes)
@@ -966,6 +1131,8 @@ static int run_bwd(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, Bwd
   a.x = c.x; a.gamma = c.gamma; a.beta = c.beta; a.mean = c.mean; a.stdv = c.stdv; a.r = c.r; a.d = c.d;
   a.xhat = c.xhat; a.mask = c.mask; a.dY = c.dY; a.partial = partial; a.coef = coef;
   a.dX = c.dX;
+  a.fin_partial = fold ? partial : nullptr; a.fin_chunks = g.nchunks; a.dgamma = c.dgamma; a.dbeta = c.dbeta;
+  a.batch_f = static_cast<float>(B); a.batch_scale = 1.0f / static_cast<float>(B);
   BwdFinalize fin;
   fin.gamma = c.gamma; fin.stdv = c.stdv; fin.r = c.r; fin.dgamma = c.dgamma; fin.dbeta = c.dbeta;
   fin.dmean = c.dmean; fin.dstd = c.dstd; fin.coef = coef;
@@ -987,7 +1154,7 @@ static int run_bwd(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, Bwd
     }));
   }
   DLMI_LAUNCH_CHECK(ctx, "k_bwd_reduce");
-  {
+  if (!fold) {
     size_t const groups = dlmi_ceil_div(H, vec4 ? 4 : 1);
     int const ftx = finalize_tx_log2(g.nchunks);
     dim3 const fgrid(static_cast<unsigned>(dlmi_ceil_div(groups, size_t(1) << ftx)));

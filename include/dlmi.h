@@ -219,12 +219,14 @@ int dlmi_loss_seed(dlmi_ctx *ctx, dlmi_loss loss, dlmi_accuracy accu, float accu
  * One training-mode layer tail: x (= Z) -> batch (re)norm -> activation ->
  * optional dropout, without materialising x_hat or the pre-activation.
  *
- * Forward (3 launches): column statistics (wavefront shuffles + LDS tree over
- * batch chunks), per-unit finalize, one coalesced pass reading x and writing y.
+ * Forward: column statistics (wavefront shuffles + LDS tree over batch chunks),
+ * then one coalesced pass reading x and writing y whose blocks do the per-unit
+ * arithmetic in their prologue (a small finalize kernel runs in between only
+ * for tall, narrow tensors that need more than 16 batch chunks).
  * Algorithmic HBM traffic 12 B/element (+1 with a per-element mask).
- * Backward (3 launches): reduction pass reading dY and x (recomputing x_hat,
- * the pre-activation and the activation), per-unit finalize, one pass reading
- * dY and x and writing dX: 20 B/element (+2 with a per-element mask).
+ * Backward: reduction pass reading dY and x (recomputing x_hat, the
+ * pre-activation and the activation), then one pass reading dY and x and
+ * writing dX: 20 B/element (+2 with a per-element mask).
  */
 typedef struct {
   dlmi_norm norm;          /* DLMI_NORM_BATCH or DLMI_NORM_BATCH_RENORM */

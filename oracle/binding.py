@@ -41,6 +41,42 @@ OPT = dict(NONE=0, ADABOUND=1, ADAM=2, AMSBOUND=4, AMSGRAD=5, GD=6, IRPROP_PLUS=
 _ADAM_FAMILY = (1, 2, 4, 5, 9)
 
 
+class HarnessRng:
+    """The benchmark harness's input generator (oracle/harness_rng.c): one mt19937_64 stream per
+    tensor, seed = base + tensor id; both sides of bench.py are fed the arrays it returns."""
+
+    def __init__(self, base_seed=1234):
+        if not os.path.exists(ORACLE_SO):
+            build_oracle()
+        self.lib = ctypes.CDLL(ORACLE_SO)
+        self.base = int(base_seed)
+
+    def raw(self, tensor_id, n):
+        out = np.empty(n, np.uint64)
+        self.lib.dlo_rng_raw(ctypes.c_uint64(self.base + tensor_id), c_sz(n), _ptr(out))
+        return out
+
+    def uniform(self, tensor_id, shape, lo=0.0, hi=1.0):
+        out = np.empty(shape, np.float32)
+        self.lib.dlo_rng_uniform(ctypes.c_uint64(self.base + tensor_id), c_sz(out.size), c_f(lo), c_f(hi), _ptr(out))
+        return out
+
+    def normal(self, tensor_id, shape):
+        out = np.empty(shape, np.float32)
+        self.lib.dlo_rng_normal(ctypes.c_uint64(self.base + tensor_id), c_sz(out.size), _ptr(out))
+        return out
+
+    def bernoulli_u8(self, tensor_id, shape, keep):
+        out = np.empty(shape, np.uint8)
+        self.lib.dlo_rng_bernoulli_u8(ctypes.c_uint64(self.base + tensor_id), c_sz(out.size), c_f(keep), _ptr(out))
+        return out
+
+    def index(self, tensor_id, n, k):
+        out = np.empty(n, np.uint32)
+        self.lib.dlo_rng_index(ctypes.c_uint64(self.base + tensor_id), c_sz(n), ctypes.c_uint32(k), _ptr(out))
+        return out
+
+
 def build_oracle():
     subprocess.run(["make", "-C", _HERE], check=True, stdout=subprocess.DEVNULL)
 

@@ -31,6 +31,22 @@ def max_rel_err(got, exp, floor=0.0):
     return float(np.max(np.abs(got - exp) / den))
 
 
+def max_rel_err_strict(got, exp):
+    """The element-wise metric of the measurement contract: max |got-exp| / max(|exp|, 1e-6 * max|exp|).
+    Every element is judged against ITSELF; only elements a million times below the largest one share a
+    floor.  Holds at 1e-5 for element-wise leaves outside their cancellation zones (exp(x)-1 and
+    2/(1+exp(-2x))-1 near x = 0, where the reference's own float evaluation is no better); it cannot hold
+    at 1e-4 for every element of a reduction or a GEMM output (an element that happens to cancel to
+    1e-3 of the typical magnitude carries the absolute error of its terms), which is why the assertions
+    behind reductions use max_rel_err above and this one is reported beside it."""
+    got = np.asarray(got, np.float64)
+    exp = np.asarray(exp, np.float64)
+    if exp.size == 0:
+        return 0.0
+    den = np.maximum(np.abs(exp), max(1e-6 * float(np.max(np.abs(exp))), 1e-300))
+    return float(np.max(np.abs(got - exp) / den))
+
+
 def assert_close(got, exp, rtol, what="", floor=0.0):
     got = np.asarray(got)
     exp = np.asarray(exp)

