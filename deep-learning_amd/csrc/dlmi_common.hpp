@@ -17,11 +17,17 @@ struct dlmi_tuning {
   int reduce_tx_cap = 128;        // widest column span of a reduction block, in column groups
   int reduce_blocks_per_cu = 1;   // reduction blocks per compute unit
   int reduce_min_rows = 4;        // fewest rows a thread of a reduction block walks
-  int apply_blocks_per_cu = 2;    // blocks per compute unit in the apply passes
+  int apply_fwd_blocks_per_cu = 16;  // blocks per compute unit in the forward apply pass (one read, one write stream)
+  int apply_bwd_blocks_per_cu = 2;   // ... in the backward apply pass (two read streams, one write stream)
   int apply_min_rows = 4;
   int reduce_interleave = 1;      // 1: blocks take every n-th group of rows instead of a contiguous chunk
   int apply_interleave = 0;
-  int fold_finalize = 1;          // 0: always run the finalize kernels (never fold them into the apply passes)
+  // Folding the finalize into the apply pass's prologue (two launches instead of three).  Backward: a gain
+  // at every size measured.  Forward: its apply pass wants many small blocks, each of which would repeat the
+  // prologue, so it pays only for small, launch-bound tensors.  0 never, 1 up to fold_fwd_max_elements, 2 always.
+  int fold_fwd = 1;
+  int fold_bwd = 2;
+  size_t fold_fwd_max_elements = size_t(1) << 20;
 };
 
 struct dlmi_ctx {

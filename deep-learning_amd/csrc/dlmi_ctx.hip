@@ -36,6 +36,10 @@ static int env_knob(char const *name, int dflt) {
   return v > 0 ? v : dflt;
 }
 
+static int env_level(char const *name, int dflt) {
+  char const *e = getenv(name);
+  return (e == nullptr || *e == 0) ? dflt : atoi(e);
+}
 static int env_flag(char const *name, int dflt) {
   char const *e = getenv(name);
   return (e == nullptr || *e == 0) ? dflt : (atoi(e) != 0 ? 1 : 0);
@@ -67,11 +71,13 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
   t.reduce_tx_cap = env_knob("DLMI_NORM_REDUCE_TX", t.reduce_tx_cap);
   t.reduce_blocks_per_cu = env_knob("DLMI_NORM_REDUCE_BLOCKS_PER_CU", t.reduce_blocks_per_cu);
   t.reduce_min_rows = env_knob("DLMI_NORM_REDUCE_MIN_ROWS", t.reduce_min_rows);
-  t.apply_blocks_per_cu = env_knob("DLMI_NORM_APPLY_BLOCKS_PER_CU", t.apply_blocks_per_cu);
+  t.apply_fwd_blocks_per_cu = env_knob("DLMI_NORM_APPLY_FWD_BLOCKS_PER_CU", t.apply_fwd_blocks_per_cu);
+  t.apply_bwd_blocks_per_cu = env_knob("DLMI_NORM_APPLY_BWD_BLOCKS_PER_CU", t.apply_bwd_blocks_per_cu);
   t.apply_min_rows = env_knob("DLMI_NORM_APPLY_MIN_ROWS", t.apply_min_rows);
   t.reduce_interleave = env_flag("DLMI_NORM_REDUCE_INTERLEAVE", t.reduce_interleave);
   t.apply_interleave = env_flag("DLMI_NORM_APPLY_INTERLEAVE", t.apply_interleave);
-  t.fold_finalize = env_flag("DLMI_NORM_FOLD_FINALIZE", t.fold_finalize);
+  t.fold_fwd = env_level("DLMI_NORM_FOLD_FWD", t.fold_fwd);
+  t.fold_bwd = env_level("DLMI_NORM_FOLD_BWD", t.fold_bwd);
   int rc = dlmi_scratch_reserve(ctx, size_t(16) << 20);
   if (rc == DLMI_OK) rc = dlmi::static_scratch_init(ctx);
   if (rc != DLMI_OK) {

@@ -152,7 +152,8 @@ static ColGeom reduce_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec
 constexpr size_t kFoldChunks = 16;
 static bool fold_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, int nplanes, size_t data_bytes,
                           ColGeom *g) {
-  if (ctx->tune.fold_finalize == 0) return false;
+  int const level = nplanes == 3 ? ctx->tune.fold_bwd : ctx->tune.fold_fwd;
+  if (level <= 0 || (level == 1 && B * H > ctx->tune.fold_fwd_max_elements)) return false;
   for (int tx = 64; tx >= 16; tx /= 2) {
     *g = reduce_geometry(ctx, B, H, vec4, nplanes, data_bytes, tx, kFoldChunks);
     size_t const blocks = static_cast<size_t>(g->grid_x) * g->nchunks;
@@ -166,7 +167,7 @@ static bool fold_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, in
 
 // Geometry of an apply pass: as wide as the row allows (TX up to 256), a few
 // blocks per compute unit, each walking its share of the rows.
-static ColGeom apply_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4) {
+static ColGeom apply_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, int blocks_per_cu) {
   dlmi_tuning const &t = ctx->tune;
   ColGeom g;
   g.vec = vec4 ? 4 : 1;
@@ -179,7 +180,7 @@ static ColGeom apply_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4
   }
   int const ty = kBlock / tx;
   g.grid_x = static_cast<unsigned>(dlmi_ceil_div(groups, tx));
-  size_t want = dlmi_ceil_div(static_cast<size_t>(ctx->num_cu) * t.apply_blocks_per_cu, g.grid_x);
+  size_t want = dlmi_ceil_div(static_cast<size_t>(ctx->num_cu) * blocks_per_cu, g.grid_x);
   size_t const max_by_rows = B / (static_cast<size_t>(ty) * t.apply_min_rows);
   if (want > max_by_rows) want = max_by_rows;
   if (want < 1) want = 1;
@@ -1067,7 +1068,7 @@ static int run_fwd_train(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t 
       hipLaunchKernelGGL(k_fwd_finalize<1>, grid, block, 0, ctx->stream, partial, nchunks, H, ftx, fin);
     DLMI_LAUNCH_CHECK(ctx, "k_fwd_finalize");
   }
-  ColGeom const ga = apply_geometry(ctx, B, H, vec4);
+  ColGeom const ga = apply_geometry(ctx, B, H, vec4, ctx->tune.apply_fwd_blocks_per_cu);
   FwdApplyArgs a;
   a.x = c.x; a.gamma = c.gamma; a.beta = c.beta; a.mean = c.mean; a.stdv = c.stdv; a.r = c.r; a.d = c.d;
   a.mask = c.mask; a.residual = c.residual; a.y = c.y; a.xhat = c.xhat; a.nrm = c.nrm;
@@ -1164,7 +1165,7 @@ static int run_bwd(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, Bwd
       hipLaunchKernelGGL(k_bwd_finalize<1>, fgrid, block, 0, ctx->stream, partial, g.nchunks, H, ftx, fin);
     DLMI_LAUNCH_CHECK(ctx, "k_bwd_finalize");
   }
-  ColGeom const ga = apply_geometry(ctx, B, H, vec4);
+  ColGeom const ga = apply_geometry(ctx, B, H, vec4, ctx->tune.apply_bwd_blocks_per_cu);
   a.rows_per_chunk = ctx->tune.apply_interleave ? 0 : ga.rows_per_chunk;
   a.tx_log2 = ga.tx_log2;
   dim3 const agrid(ga.grid_x, ga.nchunks);
