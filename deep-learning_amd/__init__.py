@@ -41,7 +41,7 @@ C_ABI_SYMBOLS = [
     "dlmi_fused_norm_act_fwd", "dlmi_fused_norm_act_bwd", "dlmi_fused_norm_act_infer", "dlmi_fc_norm_act_fwd",
     "dlmi_opt_gd", "dlmi_opt_gd_momentum", "dlmi_opt_adam", "dlmi_zero_padded_identity_fwd", "dlmi_residual_bwd",
     "dlmi_opt_adabound", "dlmi_clip_gradient", "dlmi_max_norm_rows", "dlmi_opt_irprop_plus", "dlmi_loss_seed", "dlmi_zero",
-    "dlmi_fused_norm_act_fwd_noalloc",
+    "dlmi_fused_norm_act_fwd_noalloc", "dlmi_fused_norm_act_residual_fwd", "dlmi_fc_norm_act_residual_fwd",
 ]
 
 
@@ -317,29 +317,44 @@ class Dlmi:
         return FusedDesc(NORM["BRN"] if renorm else NORM["BN"], act, dropout, 1 if mask_per_element else 0,
                          dropout_bwd, momentum, eps, r_max, d_max, drop_scale)
 
-    def fused_fwd(self, desc, x, gamma, beta, mov_mean, mov_std, mask=None, out=None, stats=None, noalloc=False):
+    def fused_fwd(self, desc, x, gamma, beta, mov_mean, mov_std, mask=None, out=None, stats=None, noalloc=False,
+                  shortcut=None):
         """Returns (y, stats) with stats = dict(mean,std,r,d) kept for the backward.
         noalloc: go through dlmi_fused_norm_act_fwd_noalloc (the library's fixed scratch array; the
-        caller then passes `out` and `stats` so that nothing is allocated on the way)."""
-        self._chk(x, gamma, beta, mov_mean, mov_std, mask, out)
+        caller then passes `out` and `stats` so that nothing is allocated on the way).
+        shortcut: y = shortcut + (activation output after dropout), dlmi_fused_norm_act_residual_fwd."""
+        self._chk(x, gamma, beta, mov_mean, mov_std, mask, out, shortcut)
         B, H = x.shape
         y = out if out is not None else self.empty(B, H)
         s = stats or dict(mean=self.empty(H), std=self.empty(H), r=self.empty(H), d=self.empty(H))
+        if shortcut is not None:
+            assert not noalloc and shortcut.shape == x.shape
+            self._ck(self.lib.dlmi_fused_norm_act_residual_fwd(
+                self.ctx, ctypes.byref(desc), c_sz(B), c_sz(H), _p(x), _p(gamma), _p(beta), _p(mask), _p(shortcut),
+                _p(s["mean"]), _p(s["std"]), _p(mov_mean), _p(mov_std), _p(s["r"]), _p(s["d"]), _p(y)))
+            return y, s
         fn = self.lib.dlmi_fused_norm_act_fwd_noalloc if noalloc else self.lib.dlmi_fused_norm_act_fwd
         self._ck(fn(self.ctx, ctypes.byref(desc), c_sz(B), c_sz(H), _p(x), _p(gamma),
                                                   _p(beta), _p(mask), _p(s["mean"]), _p(s["std"]), _p(mov_mean),
                                                   _p(mov_std), _p(s["r"]), _p(s["d"]), _p(y)))
         return y, s
 
-    def fc_norm_act_fwd(self, desc, X, W, gamma, beta, mov_mean, mov_std, mask=None, Z=None, out=None, stats=None):
+    def fc_norm_act_fwd(self, desc, X, W, gamma, beta, mov_mean, mov_std, mask=None, Z=None, out=None, stats=None,
+                        shortcut=None):
         """Z = X W^T with the batch statistics taken in the GEMM epilogue, then
-        normalization + activation (+ dropout).  Returns (Z, y, stats)."""
-        self._chk(X, W, gamma, beta, mov_mean, mov_std, mask, Z, out)
+        normalization + activation (+ dropout) (+ shortcut).  Returns (Z, y, stats)."""
+        self._chk(X, W, gamma, beta, mov_mean, mov_std, mask, Z, out, shortcut)
         B, K = X.shape
         H = W.shape[0]
         Z = Z if Z is not None else self.empty(B, H)
         y = out if out is not None else self.empty(B, H)
         s = stats or dict(mean=self.empty(H), std=self.empty(H), r=self.empty(H), d=self.empty(H))
+        if shortcut is not None:
+            self._ck(self.lib.dlmi_fc_norm_act_residual_fwd(
+                self.ctx, ctypes.byref(desc), c_sz(B), c_sz(K), c_sz(H), _p(X), _p(W), _p(gamma), _p(beta), _p(mask),
+                _p(shortcut), _p(Z), _p(s["mean"]), _p(s["std"]), _p(mov_mean), _p(mov_std), _p(s["r"]), _p(s["d"]),
+                _p(y)))
+            return Z, y, s
         self._ck(self.lib.dlmi_fc_norm_act_fwd(self.ctx, ctypes.byref(desc), c_sz(B), c_sz(K), c_sz(H), _p(X), _p(W),
                                                _p(gamma), _p(beta), _p(mask), _p(Z), _p(s["mean"]), _p(s["std"]),
                                                _p(mov_mean), _p(mov_std), _p(s["r"]), _p(s["d"]), _p(y)))

@@ -529,19 +529,36 @@ int dlmi_fc_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, flo
   return gemm<true, true>(ctx, B, H, K, X, K, W, K, Z, bias, 0);
 }
 
+static int fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t K, size_t H, float const *X,
+                           float const *W, float const *gamma, float const *beta, uint8_t const *mask,
+                           float const *shortcut, float *Z, float *mean, float *stdv, float *mov_mean, float *mov_std,
+                           float *r, float *d, float *y) {
+  unsigned chunks = 0;
+  int rc = gemm<true, true>(ctx, B, H, K, X, K, W, K, Z, nullptr, 0, &chunks);
+  if (rc != DLMI_OK) return rc;
+  // a small output runs split over K, where no slice sees whole sums: the
+  // statistics then come from a pass over Z (nullptr / 0)
+  return fused_fwd_from_partials(ctx, desc, B, H, Z, gamma, beta, mask, shortcut, mean, stdv, mov_mean, mov_std, r, d, y,
+                                 chunks != 0 ? reinterpret_cast<float const *>(dlmi_scratch_data(ctx)) : nullptr, chunks);
+}
+
 int dlmi_fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t K, size_t H, float const *X,
                          float const *W, float const *gamma, float const *beta, uint8_t const *mask, float *Z,
                          float *mean, float *stdv, float *mov_mean, float *mov_std, float *r, float *d, float *y) {
   if (ctx == nullptr || desc == nullptr) return DLMI_E_INVALID;
   DLMI_REQUIRE(ctx, X && W && Z, "null pointer");
   DLMI_REQUIRE(ctx, B > 0 && K > 0 && H > 0, "empty operand");
-  unsigned chunks = 0;
-  int rc = gemm<true, true>(ctx, B, H, K, X, K, W, K, Z, nullptr, 0, &chunks);
-  if (rc != DLMI_OK) return rc;
-  // a small output runs split over K, where no slice sees whole sums: the
-  // statistics then come from a pass over Z (nullptr / 0)
-  return fused_fwd_from_partials(ctx, desc, B, H, Z, gamma, beta, mask, nullptr, mean, stdv, mov_mean, mov_std, r, d, y,
-                                 chunks != 0 ? reinterpret_cast<float const *>(dlmi_scratch_data(ctx)) : nullptr, chunks);
+  return fc_norm_act_fwd(ctx, desc, B, K, H, X, W, gamma, beta, mask, nullptr, Z, mean, stdv, mov_mean, mov_std, r, d, y);
+}
+
+int dlmi_fc_norm_act_residual_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t K, size_t H,
+                                  float const *X, float const *W, float const *gamma, float const *beta,
+                                  uint8_t const *mask, float const *shortcut, float *Z, float *mean, float *stdv,
+                                  float *mov_mean, float *mov_std, float *r, float *d, float *y) {
+  if (ctx == nullptr || desc == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, X && W && Z && shortcut, "null pointer");
+  DLMI_REQUIRE(ctx, B > 0 && K > 0 && H > 0, "empty operand");
+  return fc_norm_act_fwd(ctx, desc, B, K, H, X, W, gamma, beta, mask, shortcut, Z, mean, stdv, mov_mean, mov_std, r, d, y);
 }
 
 int dlmi_fc_bwd_dx(dlmi_ctx *ctx, size_t B, size_t Hn, size_t H, float const *dZn, float const *Wn, float *dY,

@@ -580,7 +580,12 @@ __global__ __launch_bounds__(kBlock) void k_fwd_apply(FwdApplyArgs a) {
       }
       q[i] = act_fire<ACT>(nn[i]);
       if constexpr (DROPM != kDropNone) q[i] = drop_apply(mv[i], a.drop_scale, q[i]);
-      if constexpr (RES) q[i] = rv[i] + q[i];
+      if constexpr (RES) {
+        // a separate rounding, as the reference's own add of two stored arrays: the empty statement makes q a
+        // value of its own, so that the add cannot be fused into the activation's last multiply
+        asm volatile("" : "+v"(q[i]));
+        q[i] = rv[i] + q[i];
+      }
     }
     if constexpr (MAT) {
       if (a.xhat != nullptr) store_f<VEC>(a.xhat + off, xh);
@@ -1310,6 +1315,17 @@ int dlmi_fused_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
   rc = ctx_scratch(ctx, H, &sv);
   if (rc != DLMI_OK) return rc;
   return run_fwd_train(ctx, sv, B, H, c);
+}
+
+int dlmi_fused_norm_act_residual_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
+                                     float const *gamma, float const *beta, uint8_t const *mask,
+                                     float const *shortcut, float *mean, float *stdv, float *mov_mean, float *mov_std,
+                                     float *r, float *d, float *y) {
+  if (ctx == nullptr || desc == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, B > 0 && H > 0, "empty tensor");
+  DLMI_REQUIRE(ctx, shortcut != nullptr, "null pointer");
+  return fused_fwd_from_partials(ctx, desc, B, H, x, gamma, beta, mask, shortcut, mean, stdv, mov_mean, mov_std, r, d, y,
+                                 nullptr, 0);
 }
 
 int dlmi_fused_norm_act_fwd_noalloc(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,

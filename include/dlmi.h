@@ -275,6 +275,21 @@ int dlmi_fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, s
                          uint8_t const *mask, float *Z, float *mean, float *std, float *mov_mean,
                          float *mov_std, float *r, float *d, float *y);
 
+/* The two forwards above with the identity shortcut of a residual block in the
+ * same pass: y = shortcut + (activation output after dropout), shortcut [B,H]
+ * (y may alias it).  Saves the separate add and its 12 B/element.  The sum is
+ * formed as Forward_Pass__Zero_Padded_Identity__{Loop,OpenMP} forms it
+ * (fwp_st.cpp:5051-5112, equal widths, no padding), so the result is
+ * bit-identical to dlmi_identity_add after the un-fused call. */
+int dlmi_fused_norm_act_residual_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H,
+                                     float const *x, float const *gamma, float const *beta,
+                                     uint8_t const *mask, float const *shortcut, float *mean, float *std,
+                                     float *mov_mean, float *mov_std, float *r, float *d, float *y);
+int dlmi_fc_norm_act_residual_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t K, size_t H,
+                                  float const *X, float const *W, float const *gamma, float const *beta,
+                                  uint8_t const *mask, float const *shortcut, float *Z, float *mean,
+                                  float *std, float *mov_mean, float *mov_std, float *r, float *d, float *y);
+
 /* dX [B,H] out (may alias dY); dgamma, dbeta [H] accumulate (+=).  Composition
  * of a19 -> a20/a21 in the order of Backward_Pass__Gradient__FC__Loop
  * (bwp_st.cpp:543-701).  mean/std/r/d are the forward's outputs. */
