@@ -102,6 +102,8 @@ int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
 // out[j] (+)= sum over the B rows of x[b, j], in a fixed order (the statistics
 // pass of the normalization kernels with its second plane unused).
 int column_sums(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *out, int accumulate);
+// acc[0] += sum_b pairs[2b], acc[1] += sum_b pairs[2b+1] over nblocks per-block pairs, in a fixed order.
+int sum_block_pairs(dlmi_ctx *ctx, double const *pairs, unsigned nblocks, double *acc);
 }  // namespace dlmi
 
 inline bool dlmi_aligned16(void const *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -251,10 +251,38 @@ __global__ __launch_bounds__(kEwBlock) void k_softmax_ce_seed(float const *__res
     if (threadIdx.x == 0) {
       double l = 0.0, c = 0.0;
       for (int w = 0; w < kEwBlock / 64; ++w) { l += sh[0][w]; c += sh[1][w]; }
-      atomicAdd(&stats[0], l);
-      atomicAdd(&stats[1], c);
+      // one pair per block, added in block order by sum_block_pairs
+      stats[2 * blockIdx.x] = l;
+      stats[2 * blockIdx.x + 1] = c;
     }
   }
+}
+
+// acc[0] += sum of pairs[2b], acc[1] += sum of pairs[2b+1] over the blocks b of a seed kernel, in a fixed
+// order: thread t adds blocks t, t+256, ..., then the 256 lane totals are added in lane order.
+__global__ __launch_bounds__(kEwBlock) void k_sum_block_pairs(double const *__restrict__ pairs, unsigned nblocks,
+                                                               double *__restrict__ acc) {
+  __shared__ double sh[2][kEwBlock];
+  double l = 0.0, c = 0.0;
+  for (unsigned b = threadIdx.x; b < nblocks; b += kEwBlock) {
+    l += pairs[2 * b];
+    c += pairs[2 * b + 1];
+  }
+  sh[0][threadIdx.x] = l;
+  sh[1][threadIdx.x] = c;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double tl = 0.0, tc = 0.0;
+    for (int i = 0; i < kEwBlock; ++i) { tl += sh[0][i]; tc += sh[1][i]; }
+    acc[0] += tl;
+    acc[1] += tc;
+  }
+}
+
+int sum_block_pairs(dlmi_ctx *ctx, double const *pairs, unsigned nblocks, double *acc) {
+  hipLaunchKernelGGL(k_sum_block_pairs, dim3(1), dim3(kEwBlock), 0, ctx->stream, pairs, nblocks, acc);
+  DLMI_LAUNCH_CHECK(ctx, "k_sum_block_pairs");
+  return DLMI_OK;
 }
 
 }  // namespace dlmi
@@ -414,10 +442,16 @@ int dlmi_softmax_ce_seed(dlmi_ctx *ctx, size_t B, size_t H, float const *q, floa
   if (ctx == nullptr) return DLMI_E_INVALID;
   DLMI_REQUIRE(ctx, q && y && dZ, "null pointer");
   if (B * H == 0) return DLMI_OK;
-  hipLaunchKernelGGL(k_softmax_ce_seed, dim3(static_cast<unsigned>(dlmi_ceil_div(B, kEwBlock / 64))), dim3(kEwBlock),
-                     0, ctx->stream, q, y, dZ, B, H, stats);
+  unsigned const nblocks = static_cast<unsigned>(dlmi_ceil_div(B, kEwBlock / 64));
+  double *pairs = nullptr;
+  if (stats != nullptr) {
+    int rc = dlmi_scratch_reserve(ctx, static_cast<size_t>(nblocks) * 2 * sizeof(double));
+    if (rc != DLMI_OK) return rc;
+    pairs = reinterpret_cast<double *>(dlmi_scratch_data(ctx));
+  }
+  hipLaunchKernelGGL(k_softmax_ce_seed, dim3(nblocks), dim3(kEwBlock), 0, ctx->stream, q, y, dZ, B, H, pairs);
   DLMI_LAUNCH_CHECK(ctx, "k_softmax_ce_seed");
-  return DLMI_OK;
+  return stats != nullptr ? sum_block_pairs(ctx, pairs, nblocks, stats) : DLMI_OK;
 }
 
 }  // extern "C"

@@ -416,6 +416,15 @@ struct TileCfg {
   int bm, bn, bk;
 };
 
+// Tuning aid: DLMI_GEMM_SPLIT=<n> forces the number of K slices (1 = none).
+static int split_choice() {
+  static int const c = [] {
+    char const *e = std::getenv("DLMI_GEMM_SPLIT");
+    return e != nullptr ? std::atoi(e) : 0;  // 0: choose by shape
+  }();
+  return c;
+}
+
 // Tuning aid: DLMI_GEMM_TILE=<index> forces a tile shape (0: 128x128, 1: 256x128, 2: 256x256, 3: 64x64).
 static int tile_choice() {
   static int const c = [] {
@@ -468,10 +477,11 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   size_t const ktiles = dlmi_ceil_div(K, bk);
   unsigned splits = 1;
   size_t const target = static_cast<size_t>(ctx->num_cu) * 2;
-  if (tiles < target / 2 && ktiles >= 16) {
+  if ((tiles < target / 2 && ktiles >= 16) || split_choice() > 1) {
     size_t s = dlmi_ceil_div(target, tiles);
     size_t const max_s = ktiles / 8;  // at least 8 K tiles per slice
     if (s > max_s) s = max_s;
+    if (split_choice() > 0) s = static_cast<size_t>(split_choice());
     if (s > 1) {
       int rc = dlmi_scratch_reserve(ctx, s * M * N * sizeof(float));
       if (rc != DLMI_OK) return rc;

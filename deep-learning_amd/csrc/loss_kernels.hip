@@ -88,8 +88,10 @@ __global__ __launch_bounds__(kLossBlock) void k_loss_seed(int loss, int accu, fl
     if (threadIdx.x == 0) {
       double l = 0.0, c = 0.0;
       for (int w = 0; w < kLossBlock / 64; ++w) { l += sh[0][w]; c += sh[1][w]; }
-      atomicAdd(&stats[0], l);
-      atomicAdd(&stats[1], c);
+      // one pair per block; sum_block_pairs adds them in block order (no atomics: the sums, which iRPROP+
+      // branches on, are the same from run to run)
+      stats[2 * blockIdx.x] = l;
+      stats[2 * blockIdx.x + 1] = c;
     }
   }
 }
@@ -117,10 +119,16 @@ int dlmi_loss_seed(dlmi_ctx *ctx, dlmi_loss loss, dlmi_accuracy accu, float accu
   DLMI_REQUIRE(ctx, q && y && (dZ == nullptr || z != nullptr), "null pointer");
   dim3 const grid(static_cast<unsigned>(dlmi_ceil_div(B, kLossBlock / 64))), block(kLossBlock);
   float const *zz = z != nullptr ? z : q;  // unused without dZ
+  double *pairs = nullptr;
+  if (stats != nullptr) {
+    int rc = dlmi_scratch_reserve(ctx, static_cast<size_t>(grid.x) * 2 * sizeof(double));
+    if (rc != DLMI_OK) return rc;
+    pairs = reinterpret_cast<double *>(dlmi_scratch_data(ctx));
+  }
   DLMI_DISPATCH_ACT(act, hipLaunchKernelGGL((k_loss_seed<ACT>), grid, block, 0, ctx->stream, static_cast<int>(loss),
-                                            static_cast<int>(accu), accu_threshold, zz, q, y, dZ, B, H, stats));
+                                            static_cast<int>(accu), accu_threshold, zz, q, y, dZ, B, H, pairs));
   DLMI_LAUNCH_CHECK(ctx, "k_loss_seed");
-  return DLMI_OK;
+  return stats != nullptr ? sum_block_pairs(ctx, pairs, grid.x, stats) : DLMI_OK;
 }
 
 }  // extern "C"

@@ -327,6 +327,69 @@ def test_fused_full_size_properties(dl, pkg):
     assert float(dX.double().sum(0).abs().max()) < 1e-3 * float(dX.double().abs().sum(0).max())
 
 
+def test_config3_timed_sequence_full_size(dl, pkg):
+    """Configuration 3 at full size, the very sequence bench.py times: dlmi_fc_norm_act_fwd (ELU; the batch
+    statistics come from the GEMM epilogue, one partial per 256-row tile, 32 of them) ->
+    dlmi_fused_norm_act_bwd -> dX, dW, db at [8192 x 4096 x 4096], against a float64 evaluation with torch
+    of fwp_st.cpp:4709-4765 and bwp_st.cpp:1478-1531: the per-unit vectors in full, the [B, H] tensors on
+    row and column slabs, the GEMM outputs on slabs, plus the invariants sum_b dZ = 0 and dbeta = sum_b dN."""
+    torch.manual_seed(3)
+    B, K, H = 8192, 4096, 4096
+    X = torch.randn(B, K, device="cuda")
+    W = (torch.rand(H, K, device="cuda") * 2 - 1) * (6.0 / (K + H)) ** 0.5
+    gamma, beta = torch.ones(H, device="cuda"), torch.zeros(H, device="cuda")
+    dY = torch.randn(B, H, device="cuda")
+    mm, ms = torch.zeros(H, device="cuda"), torch.ones(H, device="cuda")
+    desc = pkg.Dlmi.desc(ACT["ELU"], momentum=0.99, eps=1e-5, r_max=3.0, d_max=5.0)
+    Z, y, st = dl.fc_norm_act_fwd(desc, X, W, gamma, beta, mm, ms)
+    rows = torch.cat([torch.arange(0, 64), torch.arange(4000, 4064), torch.arange(B - 64, B)]).cuda()
+    cols = torch.cat([torch.arange(0, 32), torch.arange(2047, 2079), torch.arange(H - 32, H)]).cuda()
+    Xd, Wd = X.double(), W.double()
+    assert_close(host(Z[rows]), host(Xd[rows] @ Wd.T), TR, "Z rows")
+    assert_close(host(Z[:, cols]), host(Xd @ Wd[cols].T), TR, "Z columns")
+    # statistics and forward from the GPU's own Z, in float64
+    zd = Z.double()
+    mu = zd.mean(0); sd = ((zd * zd).mean(0) - mu * mu + 1e-5).sqrt()
+    mm2 = 0.99 * mu; ms2 = 1 + 0.99 * (sd - 1)
+    r = (sd / ms2).clamp(1 / 3.0, 3.0); d = ((mu - mm2) / ms2).clamp(-5.0, 5.0)
+    assert_close(host(st["mean"]), host(mu), TR, "mean", floor=1.0)
+    assert_close(host(st["std"]), host(sd), TR, "std")
+    assert_close(host(st["r"]), host(r), TR, "r")
+    assert_close(host(st["d"]), host(d), TR, "d", floor=1.0)
+    assert_close(host(mm), host(mm2), TR, "moving mean", floor=1.0)
+    assert_close(host(ms), host(ms2), TR, "moving std")
+    xh = (zd - mu) / sd * r + d
+    n = gamma.double() * xh + beta.double()
+    q = torch.where(n < 0, n.exp() - 1, n)  # functions.hpp:91, slope 1
+    assert_close(host(y[rows]), host(q[rows]), TR, "y rows")
+    assert_close(host(y[:, cols]), host(q[:, cols]), TR, "y columns")
+    # ELU' = q below zero, 1 otherwise (functions.hpp:92): it jumps at n = 0, so an element within rounding of
+    # it carries no upstream gradient here
+    dY = torch.where(n.abs() < 1e-4, torch.zeros_like(dY), dY)
+    dg, db = torch.zeros(H, device="cuda"), torch.zeros(H, device="cuda")
+    dZ = dl.fused_bwd(desc, Z, gamma, beta, st, dY, dg, db)
+    dn = dY.double() * torch.where(n < 0, q, torch.ones_like(q))
+    e = dn * gamma.double()
+    dmu = (e * (-r / sd)).sum(0); dsd = (e * (zd - mu) * (-r / (sd * sd))).sum(0)
+    dz = e * (r / sd) + dsd * ((zd - mu) / (B * sd)) + dmu / B
+    assert_close(host(dZ[rows]), host(dz[rows]), TR, "dZ rows")
+    assert_close(host(dZ[:, cols]), host(dz[:, cols]), TR, "dZ columns")
+    assert_close(host(dg), host((dn * xh).sum(0)), TR, "dgamma")
+    assert_close(host(db), host(dn.sum(0)), TR, "dbeta", floor=1.0)
+    assert float(dZ.double().sum(0).abs().max()) < 1e-3 * float(dZ.double().abs().sum(0).max())
+    del xh, n, q, dn, e, dz, zd
+    # the two backward contractions and the bias gradient from the GPU's own dZ
+    dX = dl.fc_bwd_dx(dZ, W)
+    dW, dbias = dl.fc_bwd_dw(X, dZ, with_bias=True)
+    dZd = dZ.double()
+    assert_close(host(dX[rows]), host(dZd[rows] @ Wd), TR, "dX rows")
+    assert_close(host(dX[:, cols]), host(dZd @ Wd[:, cols]), TR, "dX columns")
+    assert_close(host(dW[cols]), host(dZd[:, cols].T @ Xd), TR, "dW rows")
+    assert_close(host(dW[:, cols]), host(dZd.T @ Xd[:, cols]), TR, "dW columns")
+    # the bias gradient of a normalized layer cancels analytically (sum_b dZ = 0): judged against the size of its terms
+    assert_close(host(dbias), host(dZd.sum(0)), TR, "db", floor=float(dZd.abs().sum(0).max()))
+
+
 # ------------------------------------------------------------------ softmax + cross-entropy seed
 @pytest.mark.parametrize("B,H", [(128, 10), (5, 3), (70, 130)])
 def test_softmax_ce_seed(dl, oracle, B, H):

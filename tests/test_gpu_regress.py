@@ -184,3 +184,27 @@ def test_a_model_without_activation_setters_runs_on_sigmoids_like_the_reference(
         outs.append((M.layer_buffer(2, 3), M.get_dparams()))
     assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
     assert np.all((outs[0][0] > 0) & (outs[0][0] < 1)) and np.abs(outs[0][1]).max() > 0
+
+
+def test_loss_and_accuracy_sums_do_not_depend_on_the_run(dl, oracle):
+    """The per-block loss / accuracy pairs are added in block order (no atomics): repeated runs give
+    bit-identical sums, for the softmax seed and for the element-wise one, over a thousand blocks."""
+    rng = np.random.default_rng(5)
+    B, H = 4099, 37
+    z = (rng.standard_normal((B, H)) * 2).astype(np.float32)
+    y = np.eye(H, dtype=np.float32)[rng.integers(0, H, B)]
+    q = dev(oracle.softmax_fwd(z))
+    qe = dev(oracle.act_fwd(ACT["TANH"], z))
+    yd, zd = dev(y), dev(z)
+    seen_ce, seen_mse = set(), set()
+    for _ in range(6):
+        st = torch.zeros(2, dtype=torch.float64, device="cuda")
+        dl.softmax_ce_seed(q, yd, st)
+        seen_ce.add(tuple(host(st).tobytes()))
+        st = torch.zeros(2, dtype=torch.float64, device="cuda")
+        dl.loss_seed(LOSS["MSE"], ACCU["DISTANCE"], 0.3, ACT["TANH"], zd, qe, yd, st)
+        seen_mse.add(tuple(host(st).tobytes()))
+    assert len(seen_ce) == 1 and len(seen_mse) == 1
+    _, total, acc = oracle.loss_seed(LOSS["MSE"], ACCU["DISTANCE"], 0.3, ACT["TANH"], z, host(qe), y)
+    st = np.frombuffer(bytes(next(iter(seen_mse))), np.float64)
+    assert abs(st[0] - total) <= 1e-6 * abs(total) and st[1] == acc
