@@ -42,6 +42,7 @@ C_ABI_SYMBOLS = [
     "dlmi_opt_gd", "dlmi_opt_gd_momentum", "dlmi_opt_adam", "dlmi_zero_padded_identity_fwd", "dlmi_residual_bwd",
     "dlmi_opt_adabound", "dlmi_clip_gradient", "dlmi_max_norm_rows", "dlmi_opt_irprop_plus", "dlmi_loss_seed", "dlmi_zero",
     "dlmi_fused_norm_act_fwd_noalloc", "dlmi_fused_norm_act_residual_fwd", "dlmi_fc_norm_act_residual_fwd",
+    "dlmi_ctx_reserve_layer", "dlmi_ctx_scratch_generation",
 ]
 
 

@@ -102,6 +102,9 @@ int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
 // out[j] (+)= sum over the B rows of x[b, j], in a fixed order (the statistics
 // pass of the normalization kernels with its second plane unused).
 int column_sums(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *out, int accumulate);
+// Scratch bytes the calls of this library may ask for on a layer [B, K] -> [B, H] / on [*, H] normalized units.
+size_t fc_scratch_bytes(dlmi_ctx const *ctx, size_t B, size_t K, size_t H);
+size_t norm_scratch_bytes(dlmi_ctx const *ctx, size_t H);
 // acc[0] += sum_b pairs[2b], acc[1] += sum_b pairs[2b+1] over nblocks per-block pairs, in a fixed order.
 int sum_block_pairs(dlmi_ctx *ctx, double const *pairs, unsigned nblocks, double *acc);
 }  // namespace dlmi

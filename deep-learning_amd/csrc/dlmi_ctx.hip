@@ -111,6 +111,24 @@ int dlmi_ctx_synchronize(dlmi_ctx *ctx) {
   return DLMI_OK;
 }
 
+int dlmi_ctx_reserve_layer(dlmi_ctx *ctx, size_t B, size_t K, size_t H) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  size_t need = dlmi::norm_scratch_bytes(ctx, H);
+  if (K != 0) {
+    size_t const fc = dlmi::fc_scratch_bytes(ctx, B, K, H);
+    if (fc > need) need = fc;
+    size_t const nk = dlmi::norm_scratch_bytes(ctx, K);  // a block layer normalizes its input
+    if (nk > need) need = nk;
+  }
+  size_t const pairs = (B / 4 + 2) * 2 * sizeof(double);  // loss / accuracy pairs of a seed kernel
+  if (pairs > need) need = pairs;
+  return dlmi_scratch_reserve(ctx, need);
+}
+
+unsigned long long dlmi_ctx_scratch_generation(dlmi_ctx const *ctx) {
+  return ctx != nullptr ? static_cast<unsigned long long>(ctx->n_retired) + 1ull : 0ull;
+}
+
 char const *dlmi_last_error(dlmi_ctx const *ctx) { return ctx != nullptr ? ctx->err : "null context"; }
 
 int dlmi_ctx_compute_units(dlmi_ctx const *ctx) { return ctx != nullptr ? ctx->num_cu : 0; }

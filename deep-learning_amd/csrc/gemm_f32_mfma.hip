@@ -434,12 +434,13 @@ static int tile_choice() {
   return c;
 }
 
-// C[M,N] (+)= A . B with the operand layouts given by the two flags.
-// stats_chunks != nullptr: also write the column-sum partials [2][*stats_chunks][N]
-// of C into the first half of the context's scratch (no split-K then).
-template <bool AK, bool BKC>
-static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, size_t lda, float const *B, size_t ldb,
-                float *C, float const *bias, int accumulate, unsigned *stats_chunks = nullptr) {
+// Tile shape and K split of a product, from its shape alone.
+struct GemmPlan {
+  int choice, bm, bn, bk;
+  unsigned splits;       // K slices (1: none)
+  size_t scratch_bytes;  // partial products of the slices
+};
+static GemmPlan plan_gemm(dlmi_ctx const *ctx, size_t M, size_t N, size_t K) {
   static TileCfg const cfgs[] = {{128, 128, 16}, {256, 128, 16}, {256, 256, 16}, {64, 64, 16}};
   int choice = tile_choice();
   if (choice < 0 || choice >= static_cast<int>(sizeof(cfgs) / sizeof(cfgs[0]))) {
@@ -463,19 +464,14 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
       }
     }
   }
-  int const bm = cfgs[choice].bm, bn = cfgs[choice].bn, bk = cfgs[choice].bk;
-
-  GemmArgs g;
-  g.A = A; g.B = B; g.C = C; g.bias = bias; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldc = N;
-  g.accumulate = accumulate; g.split_out = nullptr; g.stats_out = nullptr;
-  g.a_vec = (lda % 4 == 0 && dlmi_aligned16(A)) ? 1 : 0;
-  g.b_vec = (ldb % 4 == 0 && dlmi_aligned16(B)) ? 1 : 0;
-  bool const fast = M % bm == 0 && N % bn == 0 && K % bk == 0 && g.a_vec && g.b_vec;
+  GemmPlan p;
+  p.choice = choice; p.bm = cfgs[choice].bm; p.bn = cfgs[choice].bn; p.bk = cfgs[choice].bk;
+  p.splits = 1;
+  p.scratch_bytes = 0;
   // Split K when the output alone cannot fill the machine (few tiles, long K):
   // each slice writes its partial product, a second kernel adds them in order.
-  size_t const tiles = dlmi_ceil_div(M, bm) * dlmi_ceil_div(N, bn);
-  size_t const ktiles = dlmi_ceil_div(K, bk);
-  unsigned splits = 1;
+  size_t const tiles = dlmi_ceil_div(M, p.bm) * dlmi_ceil_div(N, p.bn);
+  size_t const ktiles = dlmi_ceil_div(K, p.bk);
   size_t const target = static_cast<size_t>(ctx->num_cu) * 2;
   if ((tiles < target / 2 && ktiles >= 16) || split_choice() > 1) {
     size_t s = dlmi_ceil_div(target, tiles);
@@ -483,10 +479,47 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
     if (s > max_s) s = max_s;
     if (split_choice() > 0) s = static_cast<size_t>(split_choice());
     if (s > 1) {
-      int rc = dlmi_scratch_reserve(ctx, s * M * N * sizeof(float));
-      if (rc != DLMI_OK) return rc;
-      splits = static_cast<unsigned>(s);
+      p.splits = static_cast<unsigned>(s);
+      p.scratch_bytes = s * M * N * sizeof(float);
     }
+  }
+  return p;
+}
+
+// Scratch the three products of a layer [B, K] -> [B, H] may ask for (K splits, epilogue statistics).
+size_t fc_scratch_bytes(dlmi_ctx const *ctx, size_t B, size_t K, size_t H) {
+  size_t need = 2 * 2 * 64 * H * sizeof(float);  // epilogue statistics: at most B / 64 ... 64 tile rows reserved
+  size_t const rows = dlmi_ceil_div(B, 64);
+  if (2 * 2 * rows * H * sizeof(float) > need) need = 2 * 2 * rows * H * sizeof(float);
+  size_t const shapes[3][3] = {{B, H, K}, {B, K, H}, {H, K, B}};
+  for (auto const &sh : shapes) {
+    size_t const b = plan_gemm(ctx, sh[0], sh[1], sh[2]).scratch_bytes;
+    if (b > need) need = b;
+  }
+  return need;
+}
+
+// C[M,N] (+)= A . B with the operand layouts given by the two flags.
+// stats_chunks != nullptr: also write the column-sum partials [2][*stats_chunks][N]
+// of C into the first half of the context's scratch (no split-K then).
+template <bool AK, bool BKC>
+static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, size_t lda, float const *B, size_t ldb,
+                float *C, float const *bias, int accumulate, unsigned *stats_chunks = nullptr) {
+  GemmPlan const plan = plan_gemm(ctx, M, N, K);
+  int const choice = plan.choice;
+  int const bm = plan.bm, bn = plan.bn, bk = plan.bk;
+
+  GemmArgs g;
+  g.A = A; g.B = B; g.C = C; g.bias = bias; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldc = N;
+  g.accumulate = accumulate; g.split_out = nullptr; g.stats_out = nullptr;
+  g.a_vec = (lda % 4 == 0 && dlmi_aligned16(A)) ? 1 : 0;
+  g.b_vec = (ldb % 4 == 0 && dlmi_aligned16(B)) ? 1 : 0;
+  bool const fast = M % bm == 0 && N % bn == 0 && K % bk == 0 && g.a_vec && g.b_vec;
+  size_t const ktiles = dlmi_ceil_div(K, bk);
+  unsigned splits = plan.splits;
+  if (splits > 1) {
+    int rc = dlmi_scratch_reserve(ctx, plan.scratch_bytes);
+    if (rc != DLMI_OK) return rc;
   }
   if (stats_chunks != nullptr) {
     if (splits > 1) {

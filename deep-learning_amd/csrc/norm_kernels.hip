@@ -1000,10 +1000,12 @@ static bool use_vec4(size_t H, std::initializer_list<void const *> ptrs) {
 // The context's own scratch, grown to what a reduction over [*, H] can use:
 // 3 planes of partial sums [chunks][H] with chunks * H <= blocks * (widest
 // block: 256 column groups of 4 units) + H, and the 3*H backward coefficients.
-static int ctx_scratch(dlmi_ctx *ctx, size_t H, ScratchView *v) {
+size_t norm_scratch_bytes(dlmi_ctx const *ctx, size_t H) {
   size_t const blocks = static_cast<size_t>(ctx->num_cu) * ctx->tune.reduce_blocks_per_cu;
-  size_t const need = 3 * sizeof(float) * (blocks * 1024 + 2 * H) + round_up(3 * H * sizeof(float), 256) + 4096;
-  int rc = dlmi_scratch_reserve(ctx, need);
+  return 3 * sizeof(float) * (blocks * 1024 + 2 * H) + round_up(3 * H * sizeof(float), 256) + 4096;
+}
+static int ctx_scratch(dlmi_ctx *ctx, size_t H, ScratchView *v) {
+  int rc = dlmi_scratch_reserve(ctx, norm_scratch_bytes(ctx, H));
   if (rc != DLMI_OK) return rc;
   v->data = dlmi_scratch_data(ctx);
   v->data_bytes = ctx->scratch_bytes;

@@ -143,6 +143,9 @@ void Driver::run_batches(Recorded &rec, bool const training) {
   size_t const n_batch = static_cast<size_t>(std::ceil(static_cast<double>(n_data) / static_cast<double>(batch_size_max)));
   bool const resident = make_resident();
   hipStream_t const stream = static_cast<hipStream_t>(model.native_stream());
+  // nothing may allocate inside a capture: the scratch of every layer shape and the lazily allocated buffers
+  // come first (this can change the scratch generation, which the signature below includes)
+  if (resident && record_batches && !recording_failed_ && !model.reserve_for(batch_size_max)) recording_failed_ = true;
   uint64_t sig = resident && record_batches && !recording_failed_ ? model.launch_signature() : 0;
   if (sig != 0) {
     uint64_t const extra[4] = {n_data, batch_size_max, reinterpret_cast<uintptr_t>(d_X_), reinterpret_cast<uintptr_t>(d_Y_)};
@@ -155,7 +158,9 @@ void Driver::run_batches(Recorded &rec, bool const training) {
     rec.warmed_up = false;
   }
   bool const replay = sig != 0 && rec.graphs.size() == n_batch;
-  bool const record = sig != 0 && !replay && rec.warmed_up && model.last_error()[0] == '\0';
+  // (an error text left by an earlier refused setter does not stand in the way: only errors of the captured
+  // pass itself do, see below)
+  bool const record = sig != 0 && !replay && rec.warmed_up;
   for (size_t i = 0; i != n_batch; ++i) {
     size_t const batch_size = i + 1 != n_batch ? batch_size_max : n_data - i * batch_size_max;
     if (replay) {
@@ -172,10 +177,14 @@ void Driver::run_batches(Recorded &rec, bool const training) {
     if (record && rec.graphs.size() == i) {
       hipGraph_t graph = nullptr;
       hipGraphExec_t exec = nullptr;
+      // the pass also counts loss terms and moves get_out()'s batch on the host: if the capture fails, the
+      // batch is issued again below and must not be counted twice
+      Model::PassState const before = model.pass_state();
       bool ok = hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed) == hipSuccess;
       if (ok) {
         one_batch(i, batch_size, batch_size_max, resident, training);
-        ok = hipStreamEndCapture(stream, &graph) == hipSuccess && graph != nullptr && model.last_error()[0] == '\0';
+        bool const pass_ok = model.error_count() == before.n_errors;
+        ok = hipStreamEndCapture(stream, &graph) == hipSuccess && graph != nullptr && pass_ok;
       }
       ok = ok && hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) == hipSuccess;
       if (graph != nullptr) (void)hipGraphDestroy(graph);
@@ -185,6 +194,7 @@ void Driver::run_batches(Recorded &rec, bool const training) {
       }
       (void)hipGetLastError();
       if (exec != nullptr) (void)hipGraphExecDestroy(exec);
+      model.restore_pass_state(before);
       recording_failed_ = true;  // nothing of this batch has run yet: fall through to the plain launches
     }
     one_batch(i, batch_size, batch_size_max, resident, training);

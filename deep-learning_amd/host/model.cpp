@@ -40,6 +40,7 @@ struct Model::Impl {
   // allocated (zeroed; the step sizes filled with rprop_delta_zero) on first use
   float *d_opt[7] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
   float const *cur_input = nullptr;  // [batch, n_in] of the pass in flight: d_input or a caller's device rows
+  size_t n_errors = 0;               // failed calls so far
   size_t n_loss_values = 0;          // outputs whose loss term has been accumulated since reset_loss()
   size_t all_units = 0;              // normalization units of all entries: the slots a normalized model has
   float *h_stage = nullptr;    // pinned staging for the row-pointer gather
@@ -113,6 +114,7 @@ Model::~Model(void) {
 
 bool Model::fail(char const *what) const {
   impl_->err = what;
+  ++impl_->n_errors;
   if (impl_->ctx != nullptr && dlmi_last_error(impl_->ctx)[0] != '\0')
     impl_->err += std::string(" (") + dlmi_last_error(impl_->ctx) + ")";
   std::fprintf(stderr, "dlmi::Model: %s\n", impl_->err.c_str());  // the reference logs and carries on
@@ -120,6 +122,32 @@ bool Model::fail(char const *what) const {
 }
 
 char const *Model::last_error(void) const { return impl_->err.c_str(); }
+
+bool Model::reserve_for(size_t const batch) {
+  if (ptr_array_layers == nullptr || impl_->ctx == nullptr) return false;
+  for (size_t i = 1; i < total_layers; ++i) {
+    Layer &l = ptr_array_layers[i];
+    size_t const K = l.type_layer == LAYER::RESIDUAL ? 0 : (l.in_block ? l.n_inp : ptr_array_layers[i - 1].n_out);
+    if (dlmi_ctx_reserve_layer(impl_->ctx, batch, K, l.n_out) != DLMI_OK) return fail("reserve_for: dlmi_ctx_reserve_layer");
+    // normalization after the activation keeps the activation values: the order is a public member that
+    // may have been flipped since allocate_batch()
+    if (l.type_layer != LAYER::RESIDUAL && !l.in_block && l.Use__Normalization() &&
+        !l.use_layer_normalization_before_activation && l.d_af_values == nullptr &&
+        !dev_alloc(&l.d_af_values, impl_->allocated_batch * l.n_out, impl_->err))
+      return false;
+  }
+  return true;
+}
+
+Model::PassState Model::pass_state(void) const {
+  return PassState{impl_->n_loss_values, impl_->out_batch, impl_->cur_input, impl_->n_errors};
+}
+void Model::restore_pass_state(PassState const &s) {
+  impl_->n_loss_values = s.n_loss_values;
+  impl_->out_batch = s.out_batch;
+  impl_->cur_input = s.cur_input;
+}
+size_t Model::error_count(void) const { return impl_->n_errors; }
 
 bool Model::synchronize(void) const {
   return impl_->ctx != nullptr && dlmi_ctx_synchronize(impl_->ctx) == DLMI_OK;
@@ -991,6 +1019,7 @@ void Model::seed_error(size_t const B, float const *d_targets) {
 
 // ---------------------------------------------------------------- what a recorded batch depends on
 void *Model::native_stream(void) const { return static_cast<void *>(impl_->stream); }
+void *Model::native_context(void) const { return static_cast<void *>(impl_->ctx); }
 
 void Model::account_replayed_batch(size_t const batch_size, float const *d_inputs) {
   if (ptr_array_layers == nullptr) return;
@@ -1011,6 +1040,10 @@ uint64_t Model::launch_signature(void) const {
   DLMI_MIX(total_layers); DLMI_MIX(total_parameters); DLMI_MIX(impl_->allocated_batch);
   DLMI_MIX(impl_->d_params); DLMI_MIX(impl_->d_dparams); DLMI_MIX(impl_->d_mov_mean); DLMI_MIX(impl_->d_mov_std);
   DLMI_MIX(impl_->d_stats); DLMI_MIX(impl_->d_input); DLMI_MIX(impl_->d_input_grad);
+  // the context's scratch block, whose address the kernels of a batch are given: a recording made before it grew
+  // keeps working (a retired block stays allocated) but is made again, so that every launch uses the same block
+  unsigned long long const scratch_generation = dlmi_ctx_scratch_generation(impl_->ctx);
+  DLMI_MIX(scratch_generation);
   DLMI_MIX(type_loss_function); DLMI_MIX(type_accuracy_function); DLMI_MIX(acc_var);
   DLMI_MIX(normalization_momentum_average); DLMI_MIX(normalization_epsilon);
   DLMI_MIX(batch_renormalization_r_correction_maximum); DLMI_MIX(batch_renormalization_d_correction_maximum);

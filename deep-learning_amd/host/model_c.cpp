@@ -87,6 +87,7 @@ void dlmi_model_init_uniform(dlmi_model *h, unsigned seed, float bias, float low
 }
 
 void dlmi_model_destroy(dlmi_model *h) { delete h; }
+void *dlmi_model_context(dlmi_model const *h) { return h ? h->m.native_context() : nullptr; }
 char const *dlmi_model_last_error(dlmi_model const *h) { return h ? h->m.last_error() : "null model"; }
 
 int dlmi_model_set_layer_activation_function(dlmi_model *h, size_t layer, int a) {

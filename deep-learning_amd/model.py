@@ -13,7 +13,7 @@ c_f = ctypes.c_float
 vp = ctypes.c_void_p
 
 MODEL_C_ABI_SYMBOLS = [
-    "dlmi_model_create", "dlmi_model_destroy", "dlmi_model_last_error", "dlmi_model_set_layer_activation_function",
+    "dlmi_model_create", "dlmi_model_destroy", "dlmi_model_context", "dlmi_model_last_error", "dlmi_model_set_layer_activation_function",
     "dlmi_model_set_layer_normalization", "dlmi_model_set_layer_normalization_order", "dlmi_model_set_norm_hyper", "dlmi_model_set_dropout",
     "dlmi_model_set_dropout_mask", "dlmi_model_set_dropout_backward_mode", "dlmi_model_prepare",
     "dlmi_model_total_parameters", "dlmi_model_total_normalized_units", "dlmi_model_layer_offsets",
@@ -290,6 +290,11 @@ class Model:
         """Mini-batches of this data set's driver that are held as HIP graphs (training plus evaluation passes)."""
         self.lib.dlmi_driver_recorded_batches.restype = c_sz
         return int(self.lib.dlmi_driver_recorded_batches(self._driver(X, Y, on_device)))
+
+    def context(self):
+        """The dlmi_ctx handle the model's kernels run on (owned by the model)."""
+        self.lib.dlmi_model_context.restype = vp
+        return vp(self.lib.dlmi_model_context(self.h))
 
     def evalt(self, X, Y, on_device=True):
         out = (ctypes.c_double * 2)()

@@ -73,6 +73,16 @@ int dlmi_ctx_destroy(dlmi_ctx *ctx);
 int dlmi_ctx_set_stream(dlmi_ctx *ctx, void *stream);
 int dlmi_ctx_synchronize(dlmi_ctx *ctx);
 const char *dlmi_last_error(dlmi_ctx const *ctx);
+/* Grows the context's scratch to what any call of this library can ask for on a
+ * layer [B, K] -> [B, H] (K = 0: a normalization / activation tail on [B, H]
+ * alone), so that those calls allocate nothing afterwards.  A caller that
+ * captures its launches into a HIP graph does this for every layer shape first:
+ * growing is refused while the stream is being captured.  A scratch block that
+ * kernels were given is never freed before dlmi_ctx_destroy (recorded graphs keep
+ * its address); growing retires it.  dlmi_ctx_scratch_generation changes
+ * whenever the scratch block has changed. */
+int dlmi_ctx_reserve_layer(dlmi_ctx *ctx, size_t B, size_t K, size_t H);
+unsigned long long dlmi_ctx_scratch_generation(dlmi_ctx const *ctx);
 /* Compute units of the context's device (for callers sizing their own work). */
 int dlmi_ctx_compute_units(dlmi_ctx const *ctx);
 

@@ -31,6 +31,8 @@ void dlmi_model_layer_info(dlmi_model const *m, size_t layer, size_t *out);
 void dlmi_model_glorot_uniform(dlmi_model *m, unsigned seed, float bias);
 void dlmi_model_init_uniform(dlmi_model *m, unsigned seed, float bias, float lower, float upper);
 void dlmi_model_destroy(dlmi_model *m);
+/* the dlmi_ctx (dlmi.h) the model's kernels run on; owned by the model (no counterpart in the reference) */
+void *dlmi_model_context(dlmi_model const *m);
 char const *dlmi_model_last_error(dlmi_model const *m);
 int dlmi_model_set_layer_activation_function(dlmi_model *m, size_t layer, int activation);
 int dlmi_model_set_layer_normalization(dlmi_model *m, size_t layer, int norm);

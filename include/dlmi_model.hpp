@@ -262,11 +262,27 @@ class Model {
   // over the same data addresses launch identical kernels while it stays the same.  0: the
   // model is not compiled.
   void *native_stream(void) const;
+  void *native_context(void) const;  // the dlmi_ctx the model's kernels run on (owned by the model)
   uint64_t launch_signature(void) const;
   // Host-side bookkeeping of compute_error() for a mini-batch whose launches were replayed from a
   // recording instead of being issued through it (the number of loss terms behind get_loss(), which
   // batch get_out() reads).
   void account_replayed_batch(size_t const batch_size, float const *d_inputs);
+  // Before a mini-batch is recorded into a HIP graph: everything a pass over `batch` rows could still
+  // allocate (the context's scratch for every layer shape, buffers that come with the first pass that
+  // needs them) is allocated now, outside the capture.
+  bool reserve_for(size_t const batch);
+  // Host-side state a pass changes (loss-term count, which batch get_out() reads, the error text): saved
+  // before a capture attempt and put back when the attempt fails and the batch is issued again.
+  // error_count(): how many calls have failed so far (a pass was clean if it did not change).
+  struct PassState {
+    size_t n_loss_values, out_batch;
+    float const *cur_input;
+    size_t n_errors;  // calls of this model that have failed so far
+  };
+  PassState pass_state(void) const;
+  size_t error_count(void) const;
+  void restore_pass_state(PassState const &s);
 
   // ---- public state, as in the reference ------------------------------------
   size_t total_layers = 0, total_parameters = 0, total_weights = 0, total_bias = 0;

@@ -109,3 +109,26 @@ def test_residual_blocks_are_recorded_too(lib):
     finally:
         a.close()
         b.close()
+
+
+def test_scratch_that_moves_between_replays_drops_the_recording(lib):
+    """The recorded kernels hold addresses inside the context's scratch block.  When another call on the same
+    context makes the block grow (and move), the recording is stale: the next epoch must notice, launch plainly
+    and record again, and every epoch must still equal the twin that never records."""
+    import ctypes
+    widths = [20, 32, 24, 5]
+    X, Y = data(50, 20, 5)
+    a, b = build(lib, widths), build(lib, widths)
+    try:
+        run_pair(a, b, X, Y, 3, [0, 4, 4])
+        lib.dlmi_ctx_scratch_generation.restype = ctypes.c_ulonglong
+        lib.dlmi_ctx_scratch_generation.argtypes = [ctypes.c_void_p]
+        lib.dlmi_ctx_reserve_layer.argtypes = [ctypes.c_void_p] + [ctypes.c_size_t] * 3
+        gen = lib.dlmi_ctx_scratch_generation(b.context())
+        # a very tall layer's loss pairs need more than the block holds: it grows
+        assert lib.dlmi_ctx_reserve_layer(b.context(), 1 << 24, 0, 8) == 0
+        assert lib.dlmi_ctx_scratch_generation(b.context()) == gen + 1
+        run_pair(a, b, X, Y, 4, [0, 4, 4, 4])
+    finally:
+        a.close()
+        b.close()
