@@ -87,7 +87,8 @@ Model::Model(void) : impl_(new Impl) {
   bernoulli = new Dist::Bernoulli[1];
 }
 
-Model::~Model(void) {
+// Everything compile() / load() built goes; the settings go back to their defaults, the stream stays.
+void Model::clear(void) {
   if (impl_->ctx != nullptr) (void)dlmi_ctx_synchronize(impl_->ctx);
   free_batch();
   dev_free(impl_->d_params);
@@ -102,13 +103,27 @@ Model::~Model(void) {
     }
   if (impl_->h_stage != nullptr) (void)hipHostFree(impl_->h_stage);
   if (impl_->ctx != nullptr) (void)dlmi_ctx_destroy(impl_->ctx);
-  if (impl_->stream != nullptr) (void)hipStreamDestroy(impl_->stream);
-  delete[] bernoulli;
+  hipStream_t const stream = impl_->stream;
+  size_t const n_errors = impl_->n_errors;
+  Dist::Bernoulli *const masks = bernoulli;
   delete[] ptr_array_layers;
   delete[] ptr_array_parameters;
   delete[] ptr_array_derivatives_parameters;
   delete[] ptr_array_normalized_batch_units_means_averages;
   delete[] ptr_array_normalized_batch_units_variances_averages;
+  Impl *const impl = impl_;
+  *impl = Impl();
+  impl->stream = stream;
+  impl->n_errors = n_errors;
+  static_cast<Model_State &>(*this) = Model_State();  // every public member takes its default again
+  real_gen.seed(5489u);
+  bernoulli = masks;
+}
+
+Model::~Model(void) {
+  clear();
+  if (impl_->stream != nullptr) (void)hipStreamDestroy(impl_->stream);
+  delete[] bernoulli;
   delete impl_;
 }
 

@@ -86,6 +86,40 @@ void dlmi_model_init_uniform(dlmi_model *h, unsigned seed, float bias, float low
   h->m.Initialization__Uniform(bias, lower, upper);
 }
 
+// An uncompiled model: what dlmi_model_load() fills.
+dlmi_model *dlmi_model_create_empty(void) { return new dlmi_model; }
+
+namespace {
+std::wstring widen(char const *s) {
+  std::wstring w;
+  for (; s != nullptr && *s != '\0'; ++s) w += static_cast<wchar_t>(static_cast<unsigned char>(*s));
+  return w;
+}
+}  // namespace
+
+int dlmi_model_save_params(dlmi_model *h, char const *path) { return h->m.save_params(widen(path)); }
+int dlmi_model_save_spec_params(dlmi_model *h, char const *path) { return h->m.save_spec_params(widen(path)); }
+int dlmi_model_load_spec_params(dlmi_model *h, char const *path) { return h->m.load_spec_params(widen(path)); }
+int dlmi_model_load(dlmi_model *h, char const *path_params, char const *path_spec_params, size_t allowable_memory) {
+  return h->m.load(widen(path_params), widen(path_spec_params), allowable_memory);
+}
+size_t dlmi_model_total_layers(dlmi_model const *h) { return h->m.total_layers; }
+
+struct dlmi_checkpointer {
+  dlmi_checkpointer(char const *dir, dlmi_model *m, int keep) : step(0), c(widen(dir), &m->m, keep, step) {}
+  int step;
+  dlmi::Checkpointer c;
+};
+dlmi_checkpointer *dlmi_checkpointer_create(char const *dir, dlmi_model *h, int max_to_keep) {
+  return dir != nullptr && h != nullptr ? new dlmi_checkpointer(dir, h, max_to_keep) : nullptr;
+}
+void dlmi_checkpointer_destroy(dlmi_checkpointer *c) { delete c; }
+int dlmi_checkpointer_save(dlmi_checkpointer *c, int step) {
+  c->step = step;
+  return c->c.save();
+}
+int dlmi_checkpointer_load(dlmi_checkpointer *c) { return c->c.load(); }
+
 void dlmi_model_destroy(dlmi_model *h) { delete h; }
 void *dlmi_model_context(dlmi_model const *h) { return h ? h->m.native_context() : nullptr; }
 char const *dlmi_model_last_error(dlmi_model const *h) { return h ? h->m.last_error() : "null model"; }

@@ -28,7 +28,9 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_model_set_rprop", "dlmi_model_set_rprop_loss", "dlmi_model_set_warm_restarts",
     "dlmi_model_dropout_bernoulli", "dlmi_model_get_dropout_mask", "dlmi_model_set_loss", "dlmi_model_reset_loss",
     "dlmi_model_loss_accu", "dlmi_driver_set_record_batches", "dlmi_driver_recorded_batches",
-    "dlmi_model_set_allowable_memory", "dlmi_model_memory",
+    "dlmi_model_set_allowable_memory", "dlmi_model_memory", "dlmi_model_create_empty", "dlmi_model_save_params",
+    "dlmi_model_save_spec_params", "dlmi_model_load_spec_params", "dlmi_model_load", "dlmi_model_total_layers",
+    "dlmi_checkpointer_create", "dlmi_checkpointer_destroy", "dlmi_checkpointer_save", "dlmi_checkpointer_load",
 ]
 
 LAYER_FULLY_CONNECTED, LAYER_RESIDUAL = 3, 9  # v1/data/enum/layer.hpp
@@ -291,6 +293,52 @@ class Model:
         self.lib.dlmi_driver_recorded_batches.restype = c_sz
         return int(self.lib.dlmi_driver_recorded_batches(self._driver(X, Y, on_device)))
 
+    # ---- text files of the reference (Model::save_params / save_spec_params / load) ----
+    def save_params(self, path):
+        """`model.net`: dimensions, per-layer settings, weights, biases, scales / shifts, moving statistics."""
+        self._ok(self.lib.dlmi_model_save_params(self.h, str(path).encode()), "save_params")
+
+    def save_spec_params(self, path):
+        """`model.nn`: the hyper-parameter sections."""
+        self._ok(self.lib.dlmi_model_save_spec_params(self.h, str(path).encode()), "save_spec_params")
+
+    def load_spec_params(self, path):
+        self._ok(self.lib.dlmi_model_load_spec_params(self.h, str(path).encode()), "load_spec_params")
+
+    def load_files(self, path_params, path_spec_params, allowable_memory=0):
+        """Model::load into THIS model (cleared first); False with last_error() set when the files are refused."""
+        ok = bool(self.lib.dlmi_model_load(self.h, str(path_params).encode(), str(path_spec_params).encode(),
+                                           c_sz(allowable_memory)))
+        if ok:
+            self.P = self.lib.dlmi_model_total_parameters(self.h)
+            self.n_units = self.lib.dlmi_model_total_normalized_units(self.h)
+            self.lib.dlmi_model_total_layers.restype = c_sz
+            n = int(self.lib.dlmi_model_total_layers(self.h))
+            info = (c_sz * 12)()
+            self.widths = []
+            for l in range(n):
+                self.lib.dlmi_model_layer_info(self.h, c_sz(l), info)
+                self.widths.append(int(info[1]))
+        return ok
+
+    @classmethod
+    def load(cls, lib, path_params, path_spec_params, allowable_memory=0):
+        """A new model read from the two files."""
+        self = cls.__new__(cls)
+        self._bind(lib)
+        lib.dlmi_model_create_empty.restype = vp
+        self.h = vp(lib.dlmi_model_create_empty())
+        self.P = self.n_units = self.max_batch = 0
+        self.widths = []
+        if not self.load_files(path_params, path_spec_params, allowable_memory):
+            err = self.last_error()
+            self.close()
+            raise RuntimeError("Model::load failed: " + err)
+        return self
+
+    def last_error(self):
+        return self.lib.dlmi_model_last_error(self.h).decode()
+
     def context(self):
         """The dlmi_ctx handle the model's kernels run on (owned by the model)."""
         self.lib.dlmi_model_context.restype = vp
@@ -365,3 +413,30 @@ class Net(Model):
 
     def layer_error(self, l):
         return self.layer_buffer(l, 4)
+
+
+class Checkpointer:
+    """nn/checkpointer.cpp: `<dir>/ckpt-<step>/{model.net, model.nn}` plus the `<dir>/checkpoint` pointer file,
+    the `max_to_keep` newest directories kept."""
+
+    def __init__(self, model, directory, max_to_keep=5):
+        self.model, self.lib = model, model.lib
+        self.lib.dlmi_checkpointer_create.restype = vp
+        self.h = vp(self.lib.dlmi_checkpointer_create(str(directory).encode(), model.h, c_int(max_to_keep)))
+        if not self.h:
+            raise RuntimeError("dlmi_checkpointer_create failed")
+
+    def save(self, step):
+        return bool(self.lib.dlmi_checkpointer_save(self.h, c_int(int(step))))
+
+    def load(self):
+        ok = bool(self.lib.dlmi_checkpointer_load(self.h))
+        if ok:
+            self.model.P = self.lib.dlmi_model_total_parameters(self.model.h)
+            self.model.n_units = self.lib.dlmi_model_total_normalized_units(self.model.h)
+        return ok
+
+    def close(self):
+        if getattr(self, "h", None):
+            self.lib.dlmi_checkpointer_destroy(self.h)
+            self.h = None

@@ -30,6 +30,22 @@ void dlmi_model_layer_info(dlmi_model const *m, size_t layer, size_t *out);
  * Initialization__Uniform(bias, lower, upper) (uniform.cpp:26-90) */
 void dlmi_model_glorot_uniform(dlmi_model *m, unsigned seed, float bias);
 void dlmi_model_init_uniform(dlmi_model *m, unsigned seed, float bias, float lower, float upper);
+/* Text files of the reference: Model::save_params (`model.net`, v1/learner/save.cpp:190-520), save_spec_params
+ * (`model.nn`, :35-188), load_spec_params / load (load.cpp:36, :1243; `load` clears the model first, so it also
+ * fills a model from dlmi_model_create_empty()).  Paths are UTF-8.  1 = done, 0 = refused (dlmi_model_last_error). */
+dlmi_model *dlmi_model_create_empty(void);
+int dlmi_model_save_params(dlmi_model *m, char const *path);
+int dlmi_model_save_spec_params(dlmi_model *m, char const *path);
+int dlmi_model_load_spec_params(dlmi_model *m, char const *path);
+int dlmi_model_load(dlmi_model *m, char const *path_params, char const *path_spec_params, size_t allowable_memory);
+size_t dlmi_model_total_layers(dlmi_model const *m);
+/* nn/checkpointer.cpp:40-218: save writes <dir>/ckpt-<step>/{model.net, model.nn}, points <dir>/checkpoint at it and
+ * keeps the max_to_keep newest ckpt-* directories; load reads the pointer file and loads that checkpoint. */
+typedef struct dlmi_checkpointer dlmi_checkpointer;
+dlmi_checkpointer *dlmi_checkpointer_create(char const *dir, dlmi_model *m, int max_to_keep);
+void dlmi_checkpointer_destroy(dlmi_checkpointer *c);
+int dlmi_checkpointer_save(dlmi_checkpointer *c, int step);
+int dlmi_checkpointer_load(dlmi_checkpointer *c);
 void dlmi_model_destroy(dlmi_model *m);
 /* the dlmi_ctx (dlmi.h) the model's kernels run on; owned by the model (no counterpart in the reference) */
 void *dlmi_model_context(dlmi_model const *m);

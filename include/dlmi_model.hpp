@@ -32,6 +32,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <random>
+#include <string>
 #include <vector>
 
 #include "dlmi.h"
@@ -138,7 +139,95 @@ struct Layer {
   bool Use__Dropout(void) const { return type_dropout != LAYER_DROPOUT::NONE; }
 };
 
-class Model {
+// The public data members of the reference's Model that this path keeps (names and defaults as in
+// model.hpp): a base of their own, so that Model::clear() can put every one back to its default at once.
+struct Model_State {
+  size_t total_layers = 0, total_parameters = 0, total_weights = 0, total_bias = 0;
+  size_t total_normalized_units = 0;  // 0 until a layer is normalized; then one slot per unit of EVERY entry, input included
+  size_t batch_size = 1, maximum_batch_size = 1, seq_w = 1;
+  size_t maximum_allowable_memory_bytes = 0;  // compile()'s allowable_memory; 0 there = all of the device
+  size_t number_threads = 1;
+  size_t n_acc_trial = 0, n_time_delay = 0;
+  double loss_train = 3.40282e38, loss_valid = 3.40282e38, loss_testg = 3.40282e38;  // model.hpp: FLT_MAX defaults
+  double acc_train = 0.0, acc_valid = 0.0, acc_testg = 0.0;
+  Layer *ptr_array_layers = nullptr;
+  Layer *ptr_last_layer = nullptr;  // one past the output layer
+  var *ptr_array_parameters = nullptr;               // host mirror [P]: W.. | b.. [| gamma.. | beta.. once a layer is normalized]
+  real *ptr_array_derivatives_parameters = nullptr;  // host mirror [P]
+  var *ptr_array_normalized_batch_units_means_averages = nullptr;      // host mirror [units]
+  var *ptr_array_normalized_batch_units_variances_averages = nullptr;  // host mirror [units] (std-devs)
+  real normalization_momentum_average = 0.999f;  // model.hpp:3045-3048
+  real normalization_epsilon = 1e-5f;
+  real batch_renormalization_r_correction_maximum = 1.0f;
+  real batch_renormalization_d_correction_maximum = 0.0f;
+  // optimizer hyper-parameters, defaults of model.hpp:2839-2841, 3020-3036
+  OPTIMIZER::TYPE type_optimizer_function = OPTIMIZER::NONE;
+  bool use_nesterov = false;
+  bool use_normalized_weight_decay = true;
+  bool use_adam_bias_correction = true;
+  // cosine annealing with warm restarts (model.hpp:2838, 3037-3043; train.cpp:250-275)
+  bool use_warm_restarts = false;
+  real warm_restarts_decay_learning_rate = 1.0f;
+  real warm_restarts_initial_maximum_learning_rate = 1.0f;
+  real warm_restarts_maximum_learning_rate = 1.0f;
+  real warm_restarts_minimum_learning_rate = 1e-7f;
+  real warm_restarts_initial_T_i = 1.0f;
+  real warm_restarts_T_i = 1.0f;
+  real warm_restarts_multiplier = 2.0f;
+  real learning_rate = 0.01f;
+  real learning_momentum = 0.9f;
+  real weight_decay = 0.0f;
+  real adam_learning_rate = 0.001f;
+  real adam_beta1 = 0.9f;
+  real adam_beta2 = 0.999f;
+  real adam_epsilon = 1e-8f;
+  // iRPROP+ (model.hpp:3331-3335, 2957-2958): factors and limits of the per-parameter step size, its
+  // start value, and the losses of this and of the previous epoch, which the epoch driver keeps
+  real rprop_increase_factor = 1.2f;
+  real rprop_decrease_factor = 0.5f;
+  real rprop_delta_min = 1e-6f;
+  real rprop_delta_max = 50.0f;
+  real rprop_delta_zero = 0.1f;
+  double loss_rprop = HUGE_VAL;
+  double loss_rprop_tm1 = HUGE_VAL;
+  real acc_var = 0.49f;                               // model.hpp:3019, the reach of ACCU_FN::DISTANCE
+  bool use_clip_gradient = false;                     // model.hpp:2843
+  real clip_gradient = 1.0f;                          // model.hpp:3044
+  real regularization__max_norm_constraints = 0.0f;   // model.hpp:3024
+  real learning_rate_final = 0.1f;  // AdaBound / AMSBound: the rate the band closes on (model.hpp:3021)
+  real learning_gamma = 1e-3f;      // AdaBound / AMSBound: how fast it closes (model.hpp:3023)
+  real adam_previous_beta2 = 0.0f;  // NosAdam: B_{t-1} (model.hpp:3032)
+  real adam_gamma = 0.1f;           // NosAdam: exponent of the hyper-harmonic weights (model.hpp:3034)
+  real optimizer_time_step = 0.0f;
+  real epoch_time_step = 1.0f;
+  // Settings of the reference's model file that nothing on this path reads: kept so that a file written here
+  // holds every field, and a file read here is written back unchanged (model.hpp:2836-2857, 2906, 2950, 2962,
+  // 3025-3027, 3228, 3328-3341).
+  real quickprop_decay = -0.0001f, quickprop_mu = 1.75f;
+  real sarprop_weight_decay_shift = -6.644f, sarprop_step_error_threshold_factor = 0.1f;
+  real sarprop_step_error_shift = 1.385f, sarprop_temperature = 0.015f;
+  size_t sarprop_epoch = 0;
+  double bit_fail_limit = 0.35;
+  size_t pre_training_level = 0;
+  real regularization__l1 = 0.0f, regularization__l2 = 0.0f, regularization__srip = 0.0f;
+  bool use_cu = false, use_mp = false;
+  double pct_threads = 100.0;
+  bool use_first_layer_as_input = true, use_last_layer_as_output = true;
+  MODEL::TYPE type = MODEL::NONE;
+  LOSS_FN::TYPE type_loss_function = LOSS_FN::NONE;
+  ACCU_FN::TYPE type_accuracy_function = ACCU_FN::NONE;
+  PROPAGATION::TYPE type_state_propagation = PROPAGATION::INFERENCE;
+  // How the backward treats dropout (see dlmi_dropout_bwd).  The reference's CPU
+  // path is DLMI_DROP_BWD_REFERENCE.
+  dlmi_dropout_bwd dropout_backward_mode = DLMI_DROP_BWD_REFERENCE;
+  std::mt19937 real_gen;  // weight initializers (the engine inside the reference's Dist::Real real_gen)
+  // Dropout mask generator: `bernoulli[0]`, the one the reference's single-thread Dropout_Bernoulli draws
+  // from (model.hpp:3159, allocate.cpp:86-100; clock-seeded there, seed 5489 here until the caller seeds it).
+  Dist::Bernoulli *bernoulli = nullptr;
+
+};
+
+class Model : public Model_State {
  public:
   Model(void);
   ~Model(void);
@@ -284,76 +373,23 @@ class Model {
   size_t error_count(void) const;
   void restore_pass_state(PassState const &s);
 
-  // ---- public state, as in the reference ------------------------------------
-  size_t total_layers = 0, total_parameters = 0, total_weights = 0, total_bias = 0;
-  size_t total_normalized_units = 0;  // 0 until a layer is normalized; then one slot per unit of EVERY entry, input included
-  size_t batch_size = 1, maximum_batch_size = 1, seq_w = 1;
-  size_t maximum_allowable_memory_bytes = 0;  // compile()'s allowable_memory; 0 there = all of the device
-  size_t number_threads = 1;
-  size_t n_acc_trial = 0, n_time_delay = 0;
-  double loss_train = 3.40282e38, loss_valid = 3.40282e38, loss_testg = 3.40282e38;  // model.hpp: FLT_MAX defaults
-  double acc_train = 0.0, acc_valid = 0.0, acc_testg = 0.0;
-  Layer *ptr_array_layers = nullptr;
-  Layer *ptr_last_layer = nullptr;  // one past the output layer
-  var *ptr_array_parameters = nullptr;               // host mirror [P]: W.. | b.. [| gamma.. | beta.. once a layer is normalized]
-  real *ptr_array_derivatives_parameters = nullptr;  // host mirror [P]
-  var *ptr_array_normalized_batch_units_means_averages = nullptr;      // host mirror [units]
-  var *ptr_array_normalized_batch_units_variances_averages = nullptr;  // host mirror [units] (std-devs)
-  real normalization_momentum_average = 0.999f;  // model.hpp:3045-3048
-  real normalization_epsilon = 1e-5f;
-  real batch_renormalization_r_correction_maximum = 1.0f;
-  real batch_renormalization_d_correction_maximum = 0.0f;
-  // optimizer hyper-parameters, defaults of model.hpp:2839-2841, 3020-3036
-  OPTIMIZER::TYPE type_optimizer_function = OPTIMIZER::NONE;
-  bool use_nesterov = false;
-  bool use_normalized_weight_decay = true;
-  bool use_adam_bias_correction = true;
-  // cosine annealing with warm restarts (model.hpp:2838, 3037-3043; train.cpp:250-275)
-  bool use_warm_restarts = false;
-  real warm_restarts_decay_learning_rate = 1.0f;
-  real warm_restarts_initial_maximum_learning_rate = 1.0f;
-  real warm_restarts_maximum_learning_rate = 1.0f;
-  real warm_restarts_minimum_learning_rate = 1e-7f;
-  real warm_restarts_initial_T_i = 1.0f;
-  real warm_restarts_T_i = 1.0f;
-  real warm_restarts_multiplier = 2.0f;
-  real learning_rate = 0.01f;
-  real learning_momentum = 0.9f;
-  real weight_decay = 0.0f;
-  real adam_learning_rate = 0.001f;
-  real adam_beta1 = 0.9f;
-  real adam_beta2 = 0.999f;
-  real adam_epsilon = 1e-8f;
-  // iRPROP+ (model.hpp:3331-3335, 2957-2958): factors and limits of the per-parameter step size, its
-  // start value, and the losses of this and of the previous epoch, which the epoch driver keeps
-  real rprop_increase_factor = 1.2f;
-  real rprop_decrease_factor = 0.5f;
-  real rprop_delta_min = 1e-6f;
-  real rprop_delta_max = 50.0f;
-  real rprop_delta_zero = 0.1f;
-  double loss_rprop = HUGE_VAL;
-  double loss_rprop_tm1 = HUGE_VAL;
-  real acc_var = 0.49f;                               // model.hpp:3019, the reach of ACCU_FN::DISTANCE
-  bool use_clip_gradient = false;                     // model.hpp:2843
-  real clip_gradient = 1.0f;                          // model.hpp:3044
-  real regularization__max_norm_constraints = 0.0f;   // model.hpp:3024
-  real learning_rate_final = 0.1f;  // AdaBound / AMSBound: the rate the band closes on (model.hpp:3021)
-  real learning_gamma = 1e-3f;      // AdaBound / AMSBound: how fast it closes (model.hpp:3023)
-  real adam_previous_beta2 = 0.0f;  // NosAdam: B_{t-1} (model.hpp:3032)
-  real adam_gamma = 0.1f;           // NosAdam: exponent of the hyper-harmonic weights (model.hpp:3034)
-  real optimizer_time_step = 0.0f;
-  real epoch_time_step = 1.0f;
-  MODEL::TYPE type = MODEL::NONE;
-  LOSS_FN::TYPE type_loss_function = LOSS_FN::NONE;
-  ACCU_FN::TYPE type_accuracy_function = ACCU_FN::NONE;
-  PROPAGATION::TYPE type_state_propagation = PROPAGATION::INFERENCE;
-  // How the backward treats dropout (see dlmi_dropout_bwd).  The reference's CPU
-  // path is DLMI_DROP_BWD_REFERENCE.
-  dlmi_dropout_bwd dropout_backward_mode = DLMI_DROP_BWD_REFERENCE;
-  std::mt19937 real_gen;  // weight initializers (the engine inside the reference's Dist::Real real_gen)
-  // Dropout mask generator: `bernoulli[0]`, the one the reference's single-thread Dropout_Bernoulli draws
-  // from (model.hpp:3159, allocate.cpp:86-100; clock-seeded there, seed 5489 here until the caller seeds it).
-  Dist::Bernoulli *bernoulli = nullptr;
+  // ---- text (de)serialisation (v1/learner/save.cpp:35-520, 523-935; load.cpp:36-1241, 1243-4052) ----------
+  // save_params writes the `model.net` text (the DIMENSION section: totals, then every layer with its settings,
+  // normalized units, connections and weights, biases), save_spec_params the `model.nn` text (the twelve
+  // hyper-parameter sections); field names, order, indentation, CRLF line ends and number format
+  // (16 significant digits, %g style) follow the reference's writer.  Both first bring parameters and moving
+  // statistics back from the device, and keep the previous file as `<path>.tmp` until the new one is complete
+  // (io/file/file.cpp:63-112, 336-361).  load() reads the two files back into an EMPTY or cleared model:
+  // it compiles the layer list, applies every setting through the setters above, checks that the parameter
+  // indices in the file are this model's layout, and uploads.  Settings the file can hold but this path does
+  // not run (other layer types, tied weights, k-sparsity, coded dropout, L1 / L2 / SRIP, pre-training,
+  // recurrence) make it return false.  clear() releases everything and returns the model to its state after
+  // construction (model.hpp `clear`), so that load() or compile() can be called again.
+  bool save_spec_params(std::wstring const &path_name);
+  bool save_params(std::wstring const &path_name);
+  bool load_spec_params(std::wstring const &path_name);
+  bool load(std::wstring const &path_params, std::wstring const &path_spec_params, size_t const allowable_memory = 0);
+  void clear(void);
 
   Layer *Get__Input_Layer(void) const { return ptr_array_layers; }
   Layer *Get__Output_Layer(void) const { return ptr_last_layer - 1; }
@@ -375,6 +411,26 @@ class Model {
 };
 
 }  // namespace v1
+
+// nn/checkpointer.cpp:40-218: a directory of checkpoints.  save() writes `<dir>/ckpt-<step>/model.net`
+// (Model::save_params) and `model.nn` (Model::save_spec_params), points `<dir>/checkpoint` at it with the line
+// `model_checkpoint_path: ckpt-<step>`, and keeps the `max_to_keep` most recently written `ckpt-*`
+// directories.  load() reads the pointer file and loads that checkpoint into the model.
+class Checkpointer {
+ public:
+  Checkpointer(std::wstring const &ckpt_dir, v1::Model *model, int const max_to_keep, int const &step_train);
+  bool load(void);
+  bool save(void);
+  std::wstring read_model_checkpoint_path(void);
+
+ private:
+  bool save_model_checkpoint_path(void);
+  void rotate(void);
+  v1::Model *model;
+  int max_to_keep;
+  int const &step_train;
+  std::wstring ckpt_dir, ckpt_file;
+};
 }  // namespace dlmi
 
 #ifdef DLMI_ALIAS_DL_NAMESPACE
