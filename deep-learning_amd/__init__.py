@@ -35,7 +35,7 @@ STATE = dict(INFERENCE=0, TRAINING=1, UPDATE_BATCH_NORM=2)
 # every symbol include/dlmi.h declares
 C_ABI_SYMBOLS = [
     "dlmi_ctx_create", "dlmi_ctx_destroy", "dlmi_ctx_set_stream", "dlmi_ctx_synchronize", "dlmi_last_error",
-    "dlmi_ctx_compute_units", "dlmi_fc_fwd", "dlmi_fc_bwd_dx", "dlmi_fc_bwd_dw", "dlmi_bias_fwd",
+    "dlmi_ctx_compute_units", "dlmi_layer_variance", "dlmi_scale", "dlmi_fc_fwd", "dlmi_fc_bwd_dx", "dlmi_fc_bwd_dw", "dlmi_bias_fwd",
     "dlmi_norm_fwd_train", "dlmi_norm_fwd_infer", "dlmi_norm_bwd", "dlmi_act_fwd", "dlmi_act_bwd",
     "dlmi_softmax_fwd", "dlmi_dropout_fwd", "dlmi_identity_add", "dlmi_softmax_ce_seed",
     "dlmi_fused_norm_act_fwd", "dlmi_fused_norm_act_bwd", "dlmi_fused_norm_act_infer", "dlmi_fc_norm_act_fwd",
@@ -61,6 +61,13 @@ def load_library():
     if not os.path.exists(LIB_PATH):
         raise DlmiError("%s is missing: build it with `python deep-learning_amd/build.py` "
                         "(there is no fallback path)" % LIB_PATH)
+    # A process that also uses torch on the GPU must have torch's HIP runtime loaded before this library's:
+    # with the order reversed, torch.cuda.is_available() turns False later on.  Without torch installed the
+    # library stands alone (the Model facade needs no torch).
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = ctypes.CDLL(LIB_PATH)
     lib.dlmi_last_error.restype = ctypes.c_char_p
     lib.dlmi_last_error.argtypes = [vp]
@@ -296,6 +303,20 @@ class Dlmi:
         dZ = self.empty(B, H)
         self._ck(self.lib.dlmi_softmax_ce_seed(self.ctx, c_sz(B), c_sz(H), _p(q), _p(y), _p(dZ), _p(stats)))
         return dZ
+
+    def layer_variance(self, y):
+        """Model::get_layer_variance: population variance of all values of y [B, H] (a float, on the host)."""
+        self._chk(y)
+        out = ctypes.c_float(0)
+        B, H = (y.shape[0], y.numel() // y.shape[0]) if y.dim() > 1 else (1, y.numel())
+        self._ck(self.lib.dlmi_layer_variance(self.ctx, c_sz(B), c_sz(H), _p(y), ctypes.byref(out)))
+        return out.value
+
+    def scale(self, t, factor, n=None):
+        """t[0:n] *= factor (scale_parameters_st)."""
+        self._chk(t)
+        self._ck(self.lib.dlmi_scale(self.ctx, c_sz(t.numel() if n is None else n), _p(t), ctypes.c_float(factor)))
+        return t
 
     def zero(self, t):
         self._chk(t)

@@ -279,6 +279,64 @@ __global__ __launch_bounds__(kEwBlock) void k_sum_block_pairs(double const *__re
   }
 }
 
+// ---- variance over a whole buffer (get_layer_variance, model.cpp:2824-2858) and a scaled range
+// (scale_parameters_st, lsuv.cpp:101-104): what the LSUV loop needs between two forward passes.
+// Block b owns elements [b * kMomentSpan, (b + 1) * kMomentSpan): the split, and with it the order of the
+// double additions, depends on the buffer's length only, not on the device.
+constexpr size_t kMomentSpan = size_t(kEwBlock) * 16;
+__global__ __launch_bounds__(kEwBlock) void k_moment_pairs(float const *__restrict__ x, size_t n,
+                                                            double *__restrict__ pairs) {
+  __shared__ double sh[2][kEwBlock];
+  size_t const first = static_cast<size_t>(blockIdx.x) * kMomentSpan;
+  size_t const last = first + kMomentSpan < n ? first + kMomentSpan : n;
+  double s = 0.0, q = 0.0;
+  for (size_t e = first + threadIdx.x; e < last; e += kEwBlock) {
+    double const v = static_cast<double>(x[e]);
+    s += v;
+    q += v * v;
+  }
+  sh[0][threadIdx.x] = s;
+  sh[1][threadIdx.x] = q;
+  __syncthreads();
+  for (int half = kEwBlock / 2; half > 0; half >>= 1) {  // fixed pairing: lane i takes lane i + half
+    if (static_cast<int>(threadIdx.x) < half) {
+      sh[0][threadIdx.x] += sh[0][threadIdx.x + half];
+      sh[1][threadIdx.x] += sh[1][threadIdx.x + half];
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    pairs[2 * blockIdx.x] = sh[0][0];
+    pairs[2 * blockIdx.x + 1] = sh[1][0];
+  }
+}
+
+// variance = sum(x^2) / n - (sum(x) / n)^2 from the block pairs, added in block order by one thread per
+// 256-block stride and then in lane order; written as one float
+__global__ __launch_bounds__(kEwBlock) void k_variance_from_pairs(double const *__restrict__ pairs, unsigned nblocks,
+                                                                   double inv_n, float *__restrict__ out) {
+  __shared__ double sh[2][kEwBlock];
+  double s = 0.0, q = 0.0;
+  for (unsigned b = threadIdx.x; b < nblocks; b += kEwBlock) {
+    s += pairs[2 * b];
+    q += pairs[2 * b + 1];
+  }
+  sh[0][threadIdx.x] = s;
+  sh[1][threadIdx.x] = q;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double ts = 0.0, tq = 0.0;
+    for (int i = 0; i < kEwBlock; ++i) { ts += sh[0][i]; tq += sh[1][i]; }
+    double const mean = ts * inv_n;
+    out[0] = static_cast<float>(tq * inv_n - mean * mean);
+  }
+}
+
+__global__ __launch_bounds__(kEwBlock) void k_scale(float *__restrict__ p, size_t n, float factor) {
+  size_t const stride = static_cast<size_t>(gridDim.x) * kEwBlock;
+  for (size_t e = static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x; e < n; e += stride) p[e] *= factor;
+}
+
 int sum_block_pairs(dlmi_ctx *ctx, double const *pairs, unsigned nblocks, double *acc) {
   hipLaunchKernelGGL(k_sum_block_pairs, dim3(1), dim3(kEwBlock), 0, ctx->stream, pairs, nblocks, acc);
   DLMI_LAUNCH_CHECK(ctx, "k_sum_block_pairs");
@@ -370,6 +428,37 @@ int dlmi_zero(dlmi_ctx *ctx, size_t n, float *p) {
   DLMI_REQUIRE(ctx, p != nullptr, "null pointer");
   hipLaunchKernelGGL(k_zero, dim3(ew_grid(ctx, n)), dim3(kEwBlock), 0, ctx->stream, p, n);
   DLMI_LAUNCH_CHECK(ctx, "k_zero");
+  return DLMI_OK;
+}
+
+int dlmi_layer_variance(dlmi_ctx *ctx, size_t B, size_t H, float const *y, float *variance) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, y != nullptr && variance != nullptr, "null pointer");
+  size_t const n = B * H;
+  DLMI_REQUIRE(ctx, n != 0, "dlmi_layer_variance: empty buffer");
+  size_t const nblocks = dlmi_ceil_div(n, kMomentSpan);
+  DLMI_REQUIRE(ctx, nblocks <= 0x7fffffffu, "dlmi_layer_variance: buffer too long");
+  int rc = dlmi_scratch_reserve(ctx, nblocks * 2 * sizeof(double) + 256);
+  if (rc != DLMI_OK) return rc;
+  // the result sits in front of the pairs (256 bytes keep the doubles aligned)
+  float *d_out = reinterpret_cast<float *>(dlmi_scratch_data(ctx));
+  double *pairs = reinterpret_cast<double *>(reinterpret_cast<unsigned char *>(dlmi_scratch_data(ctx)) + 256);
+  hipLaunchKernelGGL(k_moment_pairs, dim3(static_cast<unsigned>(nblocks)), dim3(kEwBlock), 0, ctx->stream, y, n, pairs);
+  DLMI_LAUNCH_CHECK(ctx, "k_moment_pairs");
+  hipLaunchKernelGGL(k_variance_from_pairs, dim3(1), dim3(kEwBlock), 0, ctx->stream, pairs,
+                     static_cast<unsigned>(nblocks), 1.0 / static_cast<double>(n), d_out);
+  DLMI_LAUNCH_CHECK(ctx, "k_variance_from_pairs");
+  hipError_t const e = hipMemcpyAsync(variance, d_out, sizeof(float), hipMemcpyDeviceToHost, ctx->stream);
+  if (e != hipSuccess) return dlmi_fail(ctx, DLMI_E_HIP, "dlmi_layer_variance: copy: %s", hipGetErrorString(e));
+  return dlmi_ctx_synchronize(ctx);
+}
+
+int dlmi_scale(dlmi_ctx *ctx, size_t n, float *p, float factor) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  if (n == 0) return DLMI_OK;
+  DLMI_REQUIRE(ctx, p != nullptr, "null pointer");
+  hipLaunchKernelGGL(k_scale, dim3(ew_grid(ctx, n)), dim3(kEwBlock), 0, ctx->stream, p, n, factor);
+  DLMI_LAUNCH_CHECK(ctx, "k_scale");
   return DLMI_OK;
 }
 

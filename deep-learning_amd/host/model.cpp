@@ -49,6 +49,8 @@ struct Model::Impl {
   mutable bool out_valid = false;
   size_t out_batch = 0;
   size_t allocated_batch = 0;
+  Model::LSUV_Parameters lsuv;
+  std::vector<size_t> lsuv_trials;  // per layer: scalings done by the last Initialization__LSUV
   mutable std::string err;
 };
 
@@ -657,6 +659,84 @@ void Model::Initialization__Uniform(real const bias, real const lower_bound, rea
   finish_initialization(*this);
 }
 
+// ---------------------------------------------------------------- LSUV
+bool Model::Initialize__LSUV(size_t const max_n_trials, size_t const max_batch_size, real const bias,
+                             real const var_target, real const var_tolerance) {
+  if (max_batch_size == 0) return fail("Maximum batch size can not be equal to zero.");  // lsuv.cpp:30-39
+  if (var_target < 0.0f) return fail("Variance target can not be less than zero.");
+  if (var_tolerance < 0.0f) return fail("Variance tolerance can not be less than zero.");
+  impl_->lsuv.maximum_number_trials = max_n_trials;
+  impl_->lsuv.maximum_batch_size = max_batch_size;
+  impl_->lsuv.initial_bias = bias;
+  impl_->lsuv.variance_target = var_target;
+  impl_->lsuv.variance_tolerance = var_tolerance;
+  return true;
+}
+
+real Model::get_layer_variance(size_t const li, size_t const max_batch_size) const {
+  if (max_batch_size == 0) { fail("Maximum batch size can not be equal to zero."); return 0.0f; }  // model.cpp:2826-2829
+  if (ptr_array_layers == nullptr || li == 0 || li >= total_layers || max_batch_size > impl_->allocated_batch) {
+    fail("get_layer_variance: bad layer index or batch size");
+    return 0.0f;
+  }
+  float v = 0.0f;
+  if (dlmi_layer_variance(impl_->ctx, max_batch_size, ptr_array_layers[li].n_out, outputs_of(li), &v) != DLMI_OK) {
+    fail("get_layer_variance: dlmi_layer_variance");
+    return 0.0f;
+  }
+  return v;
+}
+
+size_t Model::Get__LSUV_Trials(size_t const li) const { return li < impl_->lsuv_trials.size() ? impl_->lsuv_trials[li] : 0; }
+
+// Initialization__LSUV / Initialization__LSUV__Loop (lsuv.cpp:53-177)
+bool Model::Initialization__LSUV(size_t const n_data_set, real const *const *const inputs) {
+  if (ptr_array_layers == nullptr || inputs == nullptr || n_data_set == 0) return fail("Initialization__LSUV: model not compiled or no data");
+  LSUV_Parameters const &p = impl_->lsuv;
+  // the bias slots, as the pre-initialization would leave them (orthogonal.cpp:62)
+  if (!download_parameters()) return false;
+  for (size_t li = 1; li < total_layers; ++li) {
+    Layer const &l = ptr_array_layers[li];
+    if (l.type_layer != LAYER::FULLY_CONNECTED) continue;
+    for (size_t i = 0; i < l.n_out; ++i) ptr_array_parameters[l.first_bias_connection_index + i] = p.initial_bias;
+  }
+  if (!upload_parameters()) return false;
+  size_t const n_data = std::min(p.maximum_batch_size, n_data_set);
+  if (!update_mem_batch_size(n_data)) return false;
+  size_t const batch_size_max = std::min(batch_size, n_data);
+  size_t const n_batch = (n_data + batch_size_max - 1) / batch_size_max;
+  real const epsilon = p.epsilon, var_target = std::max(p.variance_target, epsilon), var_tolerance = p.variance_tolerance;
+  size_t const errors_before = error_count();
+  impl_->lsuv_trials.assign(total_layers, 0);
+  for (size_t li = 1; li < total_layers; ++li) {
+    Layer const &l = ptr_array_layers[li];
+    if (l.type_layer != LAYER::FULLY_CONNECTED) continue;
+    auto compute_variance = [&]() -> real {
+      real variance = 0.0f;
+      for (size_t i = 0; i < n_batch; ++i) {
+        size_t const rows = i + 1 != n_batch ? batch_size_max : n_data - i * batch_size_max;
+        forward_pass(rows, inputs + i * batch_size_max, 0ll, static_cast<long long>(li) + 1ll);
+        variance += get_layer_variance(li, rows);  // summed over the mini-batches, not averaged (lsuv.cpp:137)
+      }
+      return variance <= 0.0f ? epsilon : variance;
+    };
+    size_t trial = 0;
+    real variance = compute_variance();
+    while (error_count() == errors_before && std::abs(variance - var_target) >= var_tolerance) {
+      real const scale = 1.0f / (std::sqrt(variance) / std::sqrt(var_target));
+      if (dlmi_scale(impl_->ctx, l.n_out * l.n_inp, impl_->d_params + l.first_connection_index, scale) != DLMI_OK)
+        return fail("Initialization__LSUV: dlmi_scale");
+      if (++trial < p.maximum_number_trials) variance = compute_variance();
+      else break;
+    }
+    impl_->lsuv_trials[li] = trial;
+    if (error_count() != errors_before) return false;
+  }
+  if (!download_parameters()) return false;
+  finish_initialization(*this);  // clear_training_arrays + Clear__Parameter__Normalized_Unit (lsuv.cpp:90-93)
+  return true;
+}
+
 void Model::clear_training_arrays(void) {
   if (impl_->d_dparams == nullptr) return;
   (void)hipMemsetAsync(impl_->d_dparams, 0, total_parameters * sizeof(float), impl_->stream);
@@ -784,7 +864,9 @@ void Model::forward_pass(size_t const B, real const *const *const Xm, long long 
   if (ptr_array_layers == nullptr || Xm == nullptr) { fail("forward_pass: model not compiled or null input"); return; }
   if (in_idx == -1ll) in_idx = 0;
   if (out_idx == -1ll) out_idx = static_cast<long long>(total_layers);
-  if (in_idx != 0 || out_idx != static_cast<long long>(total_layers)) { fail("forward_pass: only whole-network passes are on this path"); return; }
+  // a pass may stop early: layers [1, out_idx) run (fwp_st.cpp:118-185 with its output_layer_index); it always
+  // starts at the inputs
+  if (in_idx != 0 || out_idx < 2 || out_idx > static_cast<long long>(total_layers)) { fail("forward_pass: a pass starts at the input layer and ends at one of the layers"); return; }
   if (B == 0 || B > impl_->allocated_batch) { fail("forward_pass: batch size exceeds update_mem_batch_size()"); return; }
   size_t const n_in = ptr_array_layers[0].n_out;
   // assign_inputs.cpp:22-40: gather the row pointers into a dense [B, K] block
@@ -796,21 +878,21 @@ void Model::forward_pass(size_t const B, real const *const *const Xm, long long 
               impl_->err, "input upload"))
     return;
   impl_->cur_input = impl_->d_input;
-  forward_layers(B);
+  forward_layers(B, static_cast<size_t>(out_idx));
 }
 
 void Model::forward_pass_device(size_t const B, float const *d_inputs) {
   if (ptr_array_layers == nullptr || d_inputs == nullptr) { fail("forward_pass_device: model not compiled or null input"); return; }
   if (B == 0 || B > impl_->allocated_batch) { fail("forward_pass_device: batch size exceeds update_mem_batch_size()"); return; }
   impl_->cur_input = d_inputs;
-  forward_layers(B);
+  forward_layers(B, total_layers);
 }
 
 // Layer loop of FF__Forward_Pass_Batch__Loop (fwp_st.cpp:118-185, 298-733) on impl_->cur_input.
-void Model::forward_layers(size_t const B) {
+void Model::forward_layers(size_t const B, size_t const end_layer) {
   dlmi_ctx *ctx = impl_->ctx;
   bool const training = type_state_propagation >= PROPAGATION::TRAINING;
-  for (size_t li = 1; li < total_layers; ++li) {
+  for (size_t li = 1; li < end_layer; ++li) {
     Layer &l = ptr_array_layers[li];
     if (l.type_layer == LAYER::RESIDUAL) continue;  // finished together with the last layer of its block
     if (l.in_block) {

@@ -234,6 +234,7 @@ void dlmi_model_clear_training_arrays(dlmi_model *h) { h->m.clear_training_array
 
 int dlmi_model_step(dlmi_model *h, int state, size_t B, float const *X, float const *Y, int do_backward) {
   Model &m = h->m;
+  size_t const errors_before = m.error_count();  // an earlier, reported failure does not fail this call
   m.type_state_propagation = static_cast<PROPAGATION::TYPE>(state);
   size_t const K0 = m.ptr_array_layers[0].n_out, Ho = m.Get__Output_Layer()->n_out;
   std::vector<float const *> Xm(B), Ym(B);
@@ -248,8 +249,31 @@ int dlmi_model_step(dlmi_model *h, int state, size_t B, float const *X, float co
     m.update_derivatives(B, m.ptr_array_layers + 1, m.ptr_last_layer);
     m.merge_mp_derivatives(0, m.total_parameters);
   }
-  return m.synchronize() && m.last_error()[0] == '\0';
+  return m.synchronize() && m.error_count() == errors_before;
 }
+// forward_pass(B, rows of X, 0, end_layer): the layers [1, end_layer) only
+int dlmi_model_forward_to(dlmi_model *h, int state, size_t B, float const *X, size_t end_layer) {
+  Model &m = h->m;
+  size_t const errors_before = m.error_count();
+  m.type_state_propagation = static_cast<PROPAGATION::TYPE>(state);
+  size_t const K0 = m.ptr_array_layers[0].n_out;
+  std::vector<float const *> Xm(B);
+  for (size_t i = 0; i < B; ++i) Xm[i] = X + i * K0;
+  m.forward_pass(B, Xm.data(), 0ll, static_cast<long long>(end_layer));
+  return m.synchronize() && m.error_count() == errors_before;
+}
+// Initialize__LSUV(...) then Initialization__LSUV(data set of n_data dense rows)
+int dlmi_model_lsuv(dlmi_model *h, size_t max_n_trials, size_t max_batch_size, float bias, float var_target,
+                    float var_tolerance, size_t n_data, float const *X) {
+  Model &m = h->m;
+  if (!m.Initialize__LSUV(max_n_trials, max_batch_size, bias, var_target, var_tolerance)) return 0;
+  size_t const K0 = m.ptr_array_layers != nullptr ? m.ptr_array_layers[0].n_out : 0;
+  std::vector<float const *> Xm(n_data);
+  for (size_t i = 0; i < n_data; ++i) Xm[i] = X + i * K0;
+  return m.Initialization__LSUV(n_data, Xm.data());
+}
+size_t dlmi_model_lsuv_trials(dlmi_model const *h, size_t layer) { return h->m.Get__LSUV_Trials(layer); }
+float dlmi_model_layer_variance(dlmi_model const *h, size_t layer, size_t batch) { return h->m.get_layer_variance(layer, batch); }
 int dlmi_model_download_layer(dlmi_model const *h, size_t layer, int which, size_t batch, float *out) {
   return h->m.download_layer(layer, which, batch, out);
 }
@@ -375,15 +399,17 @@ size_t dlmi_driver_recorded_batches(dlmi_driver const *d) {
 int dlmi_driver_train(dlmi_driver *d, int resample_dropout_masks, double *out) {
   if (d == nullptr || out == nullptr) return 0;
   d->drv->resample_dropout_masks = resample_dropout_masks != 0;
+  size_t const errors_before = d->drv->model.error_count();
   out[0] = d->drv->train();
   out[1] = d->drv->model.get_accu(d->drv->env_type);
-  return d->drv->model.last_error()[0] == '\0' ? 1 : 0;
+  return d->drv->model.error_count() == errors_before ? 1 : 0;
 }
 int dlmi_driver_evalt(dlmi_driver *d, double *out) {
   if (d == nullptr || out == nullptr) return 0;
+  size_t const errors_before = d->drv->model.error_count();
   out[0] = d->drv->evalt();
   out[1] = d->drv->model.get_accu(d->drv->env_type);
-  return d->drv->model.last_error()[0] == '\0' ? 1 : 0;
+  return d->drv->model.error_count() == errors_before ? 1 : 0;
 }
 
 }  // extern "C"

@@ -31,6 +31,7 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_model_set_allowable_memory", "dlmi_model_memory", "dlmi_model_create_empty", "dlmi_model_save_params",
     "dlmi_model_save_spec_params", "dlmi_model_load_spec_params", "dlmi_model_load", "dlmi_model_total_layers",
     "dlmi_checkpointer_create", "dlmi_checkpointer_destroy", "dlmi_checkpointer_save", "dlmi_checkpointer_load",
+    "dlmi_model_forward_to", "dlmi_model_lsuv", "dlmi_model_lsuv_trials", "dlmi_model_layer_variance",
 ]
 
 LAYER_FULLY_CONNECTED, LAYER_RESIDUAL = 3, 9  # v1/data/enum/layer.hpp
@@ -172,6 +173,24 @@ class Model:
             Yp = _ptr(Y)
         self._ok(self.lib.dlmi_model_step(self.h, c_int(state), c_sz(self.B), _ptr(X), Yp, c_int(1 if backward else 0)),
                  "step")
+
+    def forward_to(self, state, X, end_layer):
+        """forward_pass(B, X, 0, end_layer): layers [1, end_layer) only."""
+        X = np.ascontiguousarray(X, np.float32)
+        self.B = X.shape[0]
+        self._ok(self.lib.dlmi_model_forward_to(self.h, c_int(state), c_sz(self.B), _ptr(X), c_sz(end_layer)), "forward_to")
+
+    def lsuv(self, X, max_n_trials=10, max_batch_size=32, bias=0.0, var_target=1.0, var_tolerance=0.01):
+        """Initialize__LSUV + Initialization__LSUV on the rows of X; returns the scalings applied per layer."""
+        X = np.ascontiguousarray(X, np.float32)
+        self._ok(self.lib.dlmi_model_lsuv(self.h, c_sz(max_n_trials), c_sz(max_batch_size), c_f(bias), c_f(var_target),
+                                          c_f(var_tolerance), c_sz(X.shape[0]), _ptr(X)), "Initialization__LSUV")
+        self.lib.dlmi_model_lsuv_trials.restype = c_sz
+        return [int(self.lib.dlmi_model_lsuv_trials(self.h, c_sz(l))) for l in range(len(self.widths))]
+
+    def layer_variance(self, l, batch):
+        self.lib.dlmi_model_layer_variance.restype = c_f
+        return float(self.lib.dlmi_model_layer_variance(self.h, c_sz(l), c_sz(batch)))
 
     def layer_buffer(self, l, which):
         out = np.empty((self.B, self.widths[l]), np.float32)

@@ -193,6 +193,15 @@ int dlmi_zero_padded_identity_fwd(dlmi_ctx *ctx, size_t B, size_t HA, size_t HB,
 int dlmi_residual_bwd(dlmi_ctx *ctx, size_t B, size_t input_size, size_t derivative_size, size_t padding,
                       float const *d_inputs, float *derivatives);
 
+/* Model::get_layer_variance (v1/learner/model.cpp:2824-2858): the variance of ALL B*H values of a layer's
+ * output taken as one population, sum(y^2)/n - (sum(y)/n)^2, which the LSUV initializer steers
+ * (v1/ops/initializers/lsuv.cpp:108-177).  The sums are taken in double, in an order that depends on B*H only
+ * (the reference adds sequentially in float).  *variance is HOST memory; the call returns after the stream
+ * has finished. */
+int dlmi_layer_variance(dlmi_ctx *ctx, size_t B, size_t H, float const *y, float *variance);
+/* scale_parameters_st (lsuv.cpp:101-104): p[0..n) *= factor */
+int dlmi_scale(dlmi_ctx *ctx, size_t n, float *p, float factor);
+
 /* p[0..n) = 0 by a kernel on the context's stream: the clearing of an error array before gradients are
  * accumulated into it (the memset of bwp_st.cpp:115), in a form that a HIP graph can record. */
 int dlmi_zero(dlmi_ctx *ctx, size_t n, float *p);

@@ -89,6 +89,17 @@ void dlmi_model_clear_training_arrays(dlmi_model *m);
 /* type_state_propagation = state; forward_pass(B, rows of X); if do_backward: compute_error(B, rows of Y),
  * backward_pass(B), update_derivatives(B, layers + 1, last_layer).  X [B,K0], Y [B,Hout] dense host arrays. */
 int dlmi_model_step(dlmi_model *m, int state, size_t B, float const *X, float const *Y, int do_backward);
+/* forward_pass(batch, rows of X, 0, end_layer): only the layers [1, end_layer) run (the partial pass the LSUV
+ * initializer uses, lsuv.cpp:131-135) */
+int dlmi_model_forward_to(dlmi_model *m, int state, size_t batch, float const *X, size_t end_layer);
+/* Initialize__LSUV + Initialization__LSUV (v1/ops/initializers/lsuv.cpp:27-177) on a data set of n_data dense rows;
+ * the weights are scaled from what they hold (the reference's orthogonal start is not part of this).
+ * dlmi_model_lsuv_trials: scalings the last run applied to a layer; dlmi_model_layer_variance:
+ * Model::get_layer_variance (model.cpp:2813-2858) after the last forward pass. */
+int dlmi_model_lsuv(dlmi_model *m, size_t max_n_trials, size_t max_batch_size, float bias, float var_target,
+                    float var_tolerance, size_t n_data, float const *X);
+size_t dlmi_model_lsuv_trials(dlmi_model const *m, size_t layer);
+float dlmi_model_layer_variance(dlmi_model const *m, size_t layer, size_t batch);
 int dlmi_model_download_layer(dlmi_model const *m, size_t layer, int which, size_t batch, float *out);
 int dlmi_model_get_out(dlmi_model const *m, size_t row, float *out);          /* get_out(row) copied */
 double dlmi_model_loss_sum(dlmi_model const *m);

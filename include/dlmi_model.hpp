@@ -273,6 +273,35 @@ class Model : public Model_State {
   // (see the definition for the residual cases).
   void initialize_weights_with_glorot_uniform(real const bias = 0.0f);
   void Initialization__Uniform(real const bias = 0.0f, real const lower_bound = -1.0f, real const upper_bound = 1.0f);
+  // LSUV, "all you need is a good init" (v1/ops/initializers/lsuv.cpp:27-177; model.cpp:2813-2858).
+  // Initialize__LSUV keeps the settings; Initialization__LSUV then, layer by layer from the first hidden one,
+  // forwards up to `maximum_batch_size` rows of the data set through the layers up to that one, measures the
+  // variance of ALL values the layer puts out (one population), and multiplies the layer's weights by
+  // sqrt(variance_target / variance) until |variance - target| < tolerance or `maximum_number_trials`
+  // scalings are done; the variance of a data set that takes several mini-batches is the SUM of the
+  // mini-batch variances, as in the reference.  Forward passes, variance sums (in double) and scalings run on
+  // the device; the host reads one float per trial.  The reference starts from its orthogonal initializer
+  // (orthogonal.cpp:39-172, an Eigen QR that is not available here): here the weights are what the caller
+  // initialized before (a Glorot or uniform start, a loaded file) and only the bias slots are set to
+  // `initial_bias`, as that initializer would.  Afterwards: training arrays cleared, scales / shifts /
+  // moving statistics back to 1 / 0 / 0 / 1.  The dataset argument of the reference (get_n_data(),
+  // Get__Input_Array()) is passed as its two parts.
+  struct LSUV_Parameters {  // model.hpp:224-235
+    real initial_bias = 0.0f;
+    real epsilon = 1e-7f;
+    real variance_target = 1.0f;
+    real variance_tolerance = 0.01f;
+    size_t maximum_number_trials = 10;
+    size_t maximum_batch_size = 32;
+  };
+  bool Initialize__LSUV(size_t const max_n_trials = 10, size_t const max_batch_size = 32, real const bias = 0.0f,
+                        real const var_target = 1.0f, real const var_tolerance = 0.01f);
+  bool Initialization__LSUV(size_t const n_data, real const *const *const ptr_array_inputs);
+  // Variance of all `max_batch_size * n_out` values of a layer's output after the last forward pass.
+  real get_layer_variance(size_t const layer_index_received, size_t const max_batch_size) const;
+  // How many times Initialization__LSUV scaled the weights of a layer (no reference counterpart: for tests
+  // and logs).
+  size_t Get__LSUV_Trials(size_t const layer_index_received) const;
   void clear_training_arrays(void);  // train.cpp:110-141: zeroes the gradient array
   // bernoulli_st.cpp:27-100: resample the per-unit masks of the LAYER_DROPOUT::BERNOULLI layers, in layer
   // order, from bernoulli[0].  As in the reference, the masks of BERNOULLI_INVERTED layers are NOT touched by
@@ -399,7 +428,7 @@ class Model : public Model_State {
   Impl *impl_;
   bool allocate_batch(size_t batch);
   bool resize_normalization_slots(bool present);
-  void forward_layers(size_t batch);
+  void forward_layers(size_t batch, size_t end_layer);
   bool forward_block_layer(size_t batch, size_t index_layer);
   bool backward_block(size_t batch, size_t index_residual);
   int norm_act_tail(Layer &layer, dlmi_fused_desc desc, size_t batch, float const *x, float *y);

@@ -621,6 +621,58 @@ class OracleMLP:
     def get_moving(self):
         return self.moving_mean.copy(), self.moving_std.copy()
 
+    # ---- LSUV (v1/ops/initializers/lsuv.cpp:53-177) on weights the caller initialized ----------------
+    def layer_variance(self, l, batch):
+        """get_layer_variance(layer, batch) after the last forward pass (model.cpp:2824-2858)."""
+        self.lib.dlo_layer_variance.restype = c_f
+        out = np.ascontiguousarray(self.layer_buffer(l, 3)[:batch])
+        return float(self.lib.dlo_layer_variance(c_sz(batch), c_sz(self.widths[l]), _ptr(out)))
+
+    def lsuv(self, X, max_n_trials=10, max_batch_size=32, bias=0.0, var_target=1.0, var_tolerance=0.01, state=0):
+        """Initialization__LSUV without the orthogonal pre-initialization: constant biases, then layer by layer
+        scale the weights until the variance of the layer's output meets the target (Initialization__LSUV__Loop,
+        lsuv.cpp:108-177; a multi-batch data set SUMS the mini-batch variances, lsuv.cpp:137), then the
+        normalization parameters back to their start values.  Returns the scalings applied per layer.  A pass
+        here runs the whole network; the layers behind the one being measured do not change its output."""
+        X = np.ascontiguousarray(X, np.float32)
+        f32 = np.float32
+        eps = f32(1e-7)
+        target, tol = max(f32(var_target), eps), f32(var_tolerance)
+        n = min(int(max_batch_size), X.shape[0])
+        self.prepare(n, self.nthreads)  # update_mem_batch_size(n_data): one mini-batch holds the whole sample
+        L = len(self.widths)
+        for l in range(1, L):
+            b0 = self.layer_offsets(l)[1]
+            self.parameters[b0:b0 + self.widths[l]] = f32(bias)
+        trials = [0] * L
+
+        def variance(l):
+            self.step(state, X[:n], None, backward=False)
+            v = f32(self.layer_variance(l, n))
+            return eps if v <= 0 else v
+
+        for l in range(1, L):
+            w0 = self.layer_offsets(l)[0]
+            w1 = w0 + self.widths[l] * self.widths[l - 1]
+            v = variance(l)
+            while abs(f32(v - target)) >= tol:
+                w = np.ascontiguousarray(self.parameters[w0:w1])
+                self.lib.dlo_lsuv_scale(_ptr(w), c_sz(w.size), c_f(v), c_f(target))
+                self.parameters[w0:w1] = w
+                trials[l] += 1
+                if trials[l] < max_n_trials:
+                    v = variance(l)
+                else:
+                    break
+        self.dparameters[:] = 0
+        if self.n_units:  # Clear__Parameter__Normalized_Unit: scales 1, shifts 0, moving mean 0, moving std 1
+            g0 = self.P - 2 * self.n_units
+            self.parameters[g0:g0 + self.n_units] = 1
+            self.parameters[g0 + self.n_units:] = 0
+            self.moving_mean[:] = 0
+            self.moving_std[:] = 1
+        return trials
+
 
 def reference_available():
     return os.path.exists(REF_SO)
@@ -776,6 +828,19 @@ class ReferenceMLP:
         std = np.empty(self.n_units, np.float32)
         self.lib.dlref_model_get_moving(self.h, _ptr(mean), _ptr(std), c_sz(self.n_units))
         return mean, std
+
+    def lsuv(self, X, max_n_trials=10, max_batch_size=32, bias=0.0, var_target=1.0, var_tolerance=0.01):
+        """The reference's Initialize__LSUV + Initialization__LSUV__Loop on weights already initialized (its
+        orthogonal pre-initialization needs Eigen and is not built)."""
+        X = np.ascontiguousarray(X, np.float32)
+        ok = self.lib.dlref_model_lsuv(self.h, c_sz(max_n_trials), c_sz(max_batch_size), c_f(bias), c_f(var_target),
+                                       c_f(var_tolerance), c_sz(X.shape[0]), _ptr(X), c_sz(X.shape[1]))
+        if not ok:
+            raise RuntimeError("reference LSUV failed")
+
+    def layer_variance(self, l, batch):
+        self.lib.dlref_model_layer_variance.restype = c_f
+        return float(self.lib.dlref_model_layer_variance(self.h, c_sz(l), c_sz(batch)))
 
     def step(self, state, X, Y=None, backward=True):
         X = np.ascontiguousarray(X, np.float32)

@@ -19,6 +19,7 @@
 #include <vector>
 
 #include "deep-learning/io/logger.hpp"
+#include "deep-learning/v1/data/datasets.hpp"
 #include "deep-learning/v1/learner/model.hpp"
 
 using namespace DL;
@@ -639,6 +640,44 @@ void dlref_model_step(void *h, int state, size_t B, float const *X, size_t K0,
       m.update_derivatives(B, m.ptr_array_layers + 1, m.ptr_last_layer);
     }
   }
+}
+
+// The reference's LSUV scaling loop on weights the caller has initialized: Initialize__LSUV (lsuv.cpp:27-51)
+// keeps the settings, then what Initialization__LSUV does around the loop (lsuv.cpp:57-93) WITHOUT its first
+// line, the orthogonal pre-initialization (orthogonal.cpp needs Eigen, which this build does not have):
+// constant biases, update_mem_batch_size(min(max_batch, n_data)), Initialization__LSUV__Loop on a DatasetV1
+// that points at the caller's rows, clear_training_arrays, Clear__Parameter__Normalized_Unit.
+namespace {
+struct RowsDataset : DL::v1::DatasetV1 {
+  RowsDataset(size_t n, float const **rows) {
+    this->p_n_data = n;
+    this->Xm = rows;
+  }
+  ~RowsDataset(void) override {
+    this->p_n_data = 0;
+    this->Xm = nullptr;  // the rows belong to the caller: nothing for Deallocate() to free
+  }
+};
+}  // namespace
+
+int dlref_model_lsuv(void *h, size_t max_n_trials, size_t max_batch_size, float bias, float var_target,
+                     float var_tolerance, size_t n_data, float const *X, size_t K0) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  if (!m.Initialize__LSUV(max_n_trials, max_batch_size, bias, var_target, var_tolerance)) return 0;
+  for (Layer *l = m.ptr_array_layers + 1; l != m.ptr_last_layer; ++l)
+    if (l->type_layer == LAYER::FULLY_CONNECTED) m.layer_initialize_const_bias(bias, l);
+  std::vector<float const *> rows(n_data);
+  for (size_t i = 0; i < n_data; ++i) rows[i] = X + i * K0;
+  RowsDataset ds(n_data, rows.data());
+  if (!m.update_mem_batch_size(std::min(max_batch_size, n_data))) return 0;
+  if (!m.Initialization__LSUV__Loop(&ds)) return 0;
+  if (m.ptr_array_derivatives_parameters != nullptr) m.clear_training_arrays();
+  if (m.Use__Normalization()) m.Clear__Parameter__Normalized_Unit();
+  return 1;
+}
+// Model::get_layer_variance (model.cpp:2813-2858) after the last forward pass
+float dlref_model_layer_variance(void *h, size_t layer, size_t batch) {
+  return static_cast<RefModel *>(h)->model.get_layer_variance(layer, batch);
 }
 
 // Loss and accuracy function of the output layer (set_loss_fn / set_accu_fn, acc_var of ACCU_FN::DISTANCE),
