@@ -46,6 +46,12 @@ struct dlmi_ctx {
   char *static_scratch = nullptr;
   size_t static_scratch_bytes = 0;
   dlmi_tuning tune;
+  // single-launch (column panel) normalization kernels: barrier words in device memory, whether this
+  // device qualifies (256 CUs, 32 workgroups of a 256-workgroup launch on each of 8 XCDs), and whether
+  // one has been launched since the words were last inspected
+  unsigned *panel_state = nullptr;
+  int panel_ok = 0;
+  int panel_used = 0;
   char err[512] = {0};
 };
 
@@ -105,6 +111,11 @@ int column_sums(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *out, i
 // Scratch bytes the calls of this library may ask for on a layer [B, K] -> [B, H] / on [*, H] normalized units.
 size_t fc_scratch_bytes(dlmi_ctx const *ctx, size_t B, size_t K, size_t H);
 size_t norm_scratch_bytes(dlmi_ctx const *ctx, size_t H);
+// Column panel kernels (norm_panel_*.hip): set-up at context creation, inspection after a synchronize,
+// scratch they need for [*, H].
+int panel_init(dlmi_ctx *ctx);
+int panel_check(dlmi_ctx *ctx);
+size_t panel_scratch_bytes(size_t H);
 // acc[0] += sum_b pairs[2b], acc[1] += sum_b pairs[2b+1] over nblocks per-block pairs, in a fixed order.
 int sum_block_pairs(dlmi_ctx *ctx, double const *pairs, unsigned nblocks, double *acc);
 }  // namespace dlmi

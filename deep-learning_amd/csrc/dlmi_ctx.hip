@@ -80,9 +80,11 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
   t.fold_bwd = env_level("DLMI_NORM_FOLD_BWD", t.fold_bwd);
   int rc = dlmi_scratch_reserve(ctx, size_t(16) << 20);
   if (rc == DLMI_OK) rc = dlmi::static_scratch_init(ctx);
+  if (rc == DLMI_OK) rc = dlmi::panel_init(ctx);
   if (rc != DLMI_OK) {
     fprintf(stderr, "dlmi: %s\n", ctx->err);
     if (ctx->scratch != nullptr) (void)hipFree(ctx->scratch);
+    if (ctx->panel_state != nullptr) (void)hipFree(ctx->panel_state);
     delete ctx;
     return rc;
   }
@@ -95,6 +97,7 @@ int dlmi_ctx_destroy(dlmi_ctx *ctx) {
   (void)hipStreamSynchronize(ctx->stream);
   if (ctx->scratch != nullptr) (void)hipFree(ctx->scratch);
   for (int i = 0; i < ctx->n_retired; ++i) (void)hipFree(ctx->retired[i]);
+  if (ctx->panel_state != nullptr) (void)hipFree(ctx->panel_state);
   delete ctx;
   return DLMI_OK;
 }
@@ -108,7 +111,7 @@ int dlmi_ctx_set_stream(dlmi_ctx *ctx, void *stream) {
 int dlmi_ctx_synchronize(dlmi_ctx *ctx) {
   if (ctx == nullptr) return DLMI_E_INVALID;
   DLMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
-  return DLMI_OK;
+  return dlmi::panel_check(ctx);
 }
 
 int dlmi_ctx_reserve_layer(dlmi_ctx *ctx, size_t B, size_t K, size_t H) {

@@ -396,7 +396,9 @@ static int launch_gemm(dlmi_ctx *ctx, GemmArgs g, unsigned splits, bool fast) {
   dim3 const grid(g.tiles_m * g.tiles_n, 1, splits);
   auto const kfast = k_gemm_f32<BM, BN, BK, AK, BKC, true, WPE>;
   auto const kslow = k_gemm_f32<BM, BN, BK, AK, BKC, false, WPE>;
-  static bool attr_set = false;  // more than 64 KB of LDS has to be asked for once per kernel
+  // more than 64 KB of LDS has to be asked for once per kernel and device
+  static bool attr_set_on[64] = {false};
+  bool &attr_set = attr_set_on[ctx->device >= 0 && ctx->device < 64 ? ctx->device : 0];
   if (!attr_set) {
     DLMI_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<void const *>(kfast),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
@@ -452,7 +454,7 @@ static GemmPlan plan_gemm(dlmi_ctx const *ctx, size_t M, size_t N, size_t K) {
     static int const per_cu[] = {2, 2, 1, 4};
     static double const eff[] = {0.95, 0.97, 1.0, 0.8};
     double best = 0.0;
-    for (int c = 0; c < static_cast<int>(sizeof(cfgs) / sizeof(cfgs[0])); ++c) {
+    for (int c = 0; c < 4; ++c) {
       size_t const tiles = dlmi_ceil_div(M, cfgs[c].bm) * dlmi_ceil_div(N, cfgs[c].bn);
       size_t const slots = static_cast<size_t>(ctx->num_cu) * per_cu[c];
       size_t const rounds = dlmi_ceil_div(tiles, slots);
@@ -464,10 +466,26 @@ static GemmPlan plan_gemm(dlmi_ctx const *ctx, size_t M, size_t N, size_t K) {
       }
     }
   }
+  // A small output behind a very long reduction (the weight gradient of a narrow layer on a tall batch) is
+  // split over K anyway; its slices then run best as 128 x 128 tiles, one workgroup per CU (measured on
+  // 256 x 256 x 65536: 92 us against 98 us with 64 x 64 tiles and 32 slices).
+  size_t const tiles_128 = dlmi_ceil_div(M, 128) * dlmi_ceil_div(N, 128);
+  bool const long_k = tile_choice() < 0 && split_choice() <= 0 && K >= 8192 && tiles_128 * 8 <= static_cast<size_t>(ctx->num_cu);
+  if (long_k) choice = 0;
   GemmPlan p;
   p.choice = choice; p.bm = cfgs[choice].bm; p.bn = cfgs[choice].bn; p.bk = cfgs[choice].bk;
   p.splits = 1;
   p.scratch_bytes = 0;
+  if (long_k) {
+    size_t s = static_cast<size_t>(ctx->num_cu) / tiles_128;
+    size_t const max_s = dlmi_ceil_div(K, p.bk) / 8;
+    if (s > max_s) s = max_s;
+    if (s > 1) {
+      p.splits = static_cast<unsigned>(s);
+      p.scratch_bytes = s * M * N * sizeof(float);
+    }
+    return p;
+  }
   // Split K when the output alone cannot fill the machine (few tiles, long K):
   // each slice writes its partial product, a second kernel adds them in order.
   size_t const tiles = dlmi_ceil_div(M, p.bm) * dlmi_ceil_div(N, p.bn);

@@ -52,6 +52,7 @@
 
 #include "activations.hpp"
 #include "dlmi_common.hpp"
+#include "norm_shared.hpp"
 
 // Reduction scratch of the entry point that allocates nothing
 // (dlmi_fused_norm_act_fwd_noalloc): part of the code object, so every GPU the
@@ -89,9 +90,6 @@ int static_scratch_init(dlmi_ctx *ctx) {
 
 constexpr int kBlock = 256;
 constexpr int kWave = 64;
-
-// dropout as a template mode
-constexpr int kDropNone = 0, kDropUnit = 1, kDropElem = 2;
 
 struct ColGeom {
   int vec;  // 4 (float4 path) or 1 (any H, any alignment)
@@ -315,52 +313,6 @@ __device__ __forceinline__ void chunk_totals(float const *partial, unsigned nchu
 // ---------------------------------------------------------------- forward
 // Phase 2 of fwp_st.cpp:4709-4746 for one unit: batch mean, moving mean, batch
 // std, moving std, then r and d from the UPDATED moving statistics.
-struct FwdFinalize {
-  float *mean, *stdv, *mov_mean, *mov_std, *r, *d;
-  float batch_scale;  // 1 / B as a float, multiplied like the reference's tmp_batch_scale
-  float momentum, eps, r_max, d_max;
-  int renorm;
-};
-
-// The six per-unit results of the forward step from the two column sums and the
-// unit's moving mean / std as they were before the step.
-struct UnitStats {
-  float mean, stdv, mov_mean, mov_std, r, d;
-};
-__device__ __forceinline__ UnitStats fwd_unit_stats(FwdFinalize const &f, float s1, float s2, float mm, float ms) {
-  UnitStats u;
-  u.mean = s1 * f.batch_scale;
-  mm += f.momentum * (u.mean - mm);
-  u.stdv = sqrtf(s2 * f.batch_scale - u.mean * u.mean + f.eps);
-  ms += f.momentum * (u.stdv - ms);
-  u.mov_mean = mm;
-  u.mov_std = ms;
-  u.r = 1.0f;
-  u.d = 0.0f;
-  if (f.renorm) {
-    float const g = u.stdv / ms;
-    float const lo = 1.0f / f.r_max;
-    u.r = g < lo ? lo : (g > f.r_max ? f.r_max : g);
-    float const dd = (u.mean - mm) / ms;
-    u.d = dd < -f.d_max ? -f.d_max : (dd > f.d_max ? f.d_max : dd);
-  }
-  return u;
-}
-__device__ __forceinline__ void store_unit_stats(FwdFinalize const &f, size_t j, UnitStats const &u) {
-  f.mean[j] = u.mean;
-  f.stdv[j] = u.stdv;
-  f.mov_mean[j] = u.mov_mean;
-  f.mov_std[j] = u.mov_std;
-  if (f.r != nullptr) f.r[j] = u.r;
-  if (f.d != nullptr) f.d[j] = u.d;
-}
-// mm, ms: the unit's moving mean and moving std as loaded before the sums were
-// formed (so that their latency overlaps the partial-sum loads).
-__device__ __forceinline__ void fwd_finalize_unit(FwdFinalize const &f, size_t j, float s1, float s2, float mm,
-                                                  float ms) {
-  store_unit_stats(f, j, fwd_unit_stats(f, s1, s2, mm, ms));
-}
-
 struct StatsArgs {
   float const *x;
   size_t B, H, rows_per_chunk;
@@ -487,8 +439,6 @@ __global__ __launch_bounds__(kBlock) void k_colsum_finalize(float const *__restr
 
 // Dropout as the forward applies it (fwp_st.cpp:4830-4883): mask ? v*scale : 0
 // with scale = 1 for plain Bernoulli, 1/keep for inverted Bernoulli.
-__device__ __forceinline__ float drop_apply(uint8_t m, float scale, float v) { return m ? v * scale : 0.0f; }
-
 struct FwdApplyArgs {
   float const *x, *gamma, *beta, *mean, *stdv, *r, *d;
   uint8_t const *mask;
@@ -710,31 +660,6 @@ __device__ __forceinline__ void load_unit_consts(BwdArgs const &a, size_t col, U
 #pragma unroll
     for (int i = 0; i < VEC; ++i) u.rs[i] = rr[i] * fast_rcp(sd[i]);
     if constexpr (DROPM == kDropUnit) load_u8<VEC>(a.mask + col, u.mk);
-  }
-}
-
-// dn = dY * f'(n, q) for one element, recomputing x_hat, n and q from x.
-// REFERENCE dropout mode: q is the post-dropout output and dY is untouched
-// (bwp_st.cpp:1177-1209 reads the array the dropout leaf overwrote in place);
-// MASKED mode: q is the pre-dropout activation and dY is masked and rescaled.
-template <int ACT, int DROPM, bool XHAT_GIVEN>
-__device__ __forceinline__ float bwd_dn(float drop_scale, int drop_bwd_masked, float xv, float dy, uint8_t m,
-                                        float mu, float rs, float dd, float ga, float be, float &xh) {
-  if constexpr (XHAT_GIVEN) {
-    (void)drop_scale; (void)drop_bwd_masked; (void)xv; (void)m; (void)mu; (void)rs; (void)dd; (void)ga; (void)be;
-    return dy;
-  } else {
-    xh = (xv - mu) * rs + dd;
-    float const nn = ga * xh + be;
-    float q = act_fire<ACT>(nn);
-    float g = dy;
-    if constexpr (DROPM != kDropNone) {
-      float const gm = drop_apply(m, drop_scale, dy);
-      float const qm = drop_apply(m, drop_scale, q);
-      g = drop_bwd_masked ? gm : dy;
-      q = drop_bwd_masked ? q : qm;
-    }
-    return g * act_derive<ACT>(nn, q);
   }
 }
 
@@ -1002,7 +927,9 @@ static bool use_vec4(size_t H, std::initializer_list<void const *> ptrs) {
 // block: 256 column groups of 4 units) + H, and the 3*H backward coefficients.
 size_t norm_scratch_bytes(dlmi_ctx const *ctx, size_t H) {
   size_t const blocks = static_cast<size_t>(ctx->num_cu) * ctx->tune.reduce_blocks_per_cu;
-  return 3 * sizeof(float) * (blocks * 1024 + 2 * H) + round_up(3 * H * sizeof(float), 256) + 4096;
+  size_t const multi = 3 * sizeof(float) * (blocks * 1024 + 2 * H) + round_up(3 * H * sizeof(float), 256) + 4096;
+  size_t const panel = panel_scratch_bytes(H);
+  return multi > panel ? multi : panel;
 }
 static int ctx_scratch(dlmi_ctx *ctx, size_t H, ScratchView *v) {
   int rc = dlmi_scratch_reserve(ctx, norm_scratch_bytes(ctx, H));
@@ -1012,23 +939,12 @@ static int ctx_scratch(dlmi_ctx *ctx, size_t H, ScratchView *v) {
   return DLMI_OK;
 }
 
-struct FwdTrainCall {
-  dlmi_norm norm;
-  int act;
-  int drop_mode;  // kDropNone / kDropUnit / kDropElem
-  float momentum, eps, r_max, d_max, drop_scale;
-  float const *x, *gamma, *beta;
-  uint8_t const *mask;
-  float const *residual = nullptr;
-  float *mean, *stdv, *mov_mean, *mov_std, *r, *d, *y, *xhat, *nrm;
-  float const *partial_in = nullptr;  // column-sum partials already produced elsewhere ...
-  unsigned partial_chunks = 0;        // ... [2][partial_chunks][H]; skips the statistics pass
-};
-
 static int run_fwd_train(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, FwdTrainCall const &c) {
   bool const vec4 = use_vec4(H, {c.x, c.gamma, c.beta, c.mean, c.stdv, c.mov_mean, c.mov_std, c.r, c.d, c.y, c.xhat, c.nrm,
                                  c.residual}) &&
                     (c.drop_mode == kDropNone || (reinterpret_cast<uintptr_t>(c.mask) & 3u) == 0);
+  // a few thousand rows, H a multiple of 1024: one launch that reads x once
+  if (int const took = panel_fwd_try(ctx, B, H, c, vec4); took != 0) return took < 0 ? took : DLMI_OK;
   dim3 const block(kBlock);
   FwdFinalize fin;
   fin.mean = c.mean; fin.stdv = c.stdv; fin.mov_mean = c.mov_mean; fin.mov_std = c.mov_std; fin.r = c.r; fin.d = c.d;
@@ -1109,17 +1025,6 @@ static int run_fwd_train(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t 
   DLMI_LAUNCH_CHECK(ctx, "k_fwd_apply");
   return DLMI_OK;
 }
-
-struct BwdCall {
-  int act;
-  bool xhat_given;
-  int drop_mode, drop_bwd_masked;
-  float drop_scale;
-  float const *x, *gamma, *beta, *mean, *stdv, *r, *d, *xhat, *dY;
-  uint8_t const *mask;
-  float *dgamma, *dbeta, *dmean, *dstd, *dX;
-  bool accumulate = false;  // dX += instead of dX =
-};
 
 static int run_bwd(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, BwdCall const &c) {
   bool const vec4 = use_vec4(H, {c.x, c.gamma, c.beta, c.mean, c.stdv, c.r, c.d, c.xhat, c.dY, c.dX, c.dgamma, c.dbeta}) &&

@@ -1,0 +1,114 @@
+// Single-launch batch-(re)normalization for tensors of a few thousand rows: the column panel scheme.
+//
+// MI355X has 8 XCDs of 32 CUs, each XCD with an L2 of its own; whatever misses an L2 crosses the fabric to
+// the memory side at about 6.5 TB/s in total, so a kernel pair that reads a tensor twice (statistics, then
+// apply) cannot move its 12 B/element (forward) faster than that.  Here the tensor is read ONCE: the
+// launch has one workgroup per CU; the 32 workgroups that run on one XCD own H/8 columns together and walk
+// them in panels of P columns.  Per panel every workgroup loads its own B/32 rows of the panel into
+// registers, forms the column sums of those rows, publishes them as one chunk partial, waits until the
+// other 31 workgroups of the XCD have published theirs, adds the 32 partials in rank order (the same
+// fixed-order, atomic-free sum as the multi-launch path), and applies the result to the rows it still
+// holds in registers.  Three panels are in flight per workgroup (loading p+2, published p+1, applying p), so
+// the wait for the other workgroups overlaps the memory stream.
+//
+// The exchange among the 32 workgroups never leaves their XCD: the partials are written with ordinary
+// stores (write-through to the L2), completed with s_waitcnt before the workgroup's arrival is counted, and
+// both the arrival counter and its polling are read-modify-write atomics, which execute in the L2 itself
+// (a plain or workgroup-scope atomic LOAD may be served by the CU's own L1 and never see the other CUs'
+// arrivals).  Which XCD a workgroup runs on is read from the XCC_ID hardware register, its rank among the
+// workgroups of that XCD from a ticket counter in the same L2; nothing is assumed about the dispatch order
+// except that every XCD receives 32 of the 256 workgroups, which dlmi_ctx_create checks with a probe
+// launch.  Every wait is bounded: a workgroup that does not see its XCD complete within kPanelSpinLimit
+// polls raises the abort word and leaves, the others follow, the host reports the failure at the next
+// dlmi_ctx_synchronize and the context stays on the multi-launch path from then on.  That cannot happen
+// while one panel kernel runs at a time (256 workgroups always fit 256 CUs): launches on different streams
+// of one process are ordered with an event for that reason.
+#ifndef DLMI_NORM_PANEL_COMMON_HPP
+#define DLMI_NORM_PANEL_COMMON_HPP
+
+#include "norm_shared.hpp"
+
+namespace dlmi {
+
+constexpr int kPanelRanks = 32;   // workgroups per XCD
+constexpr int kPanelXcds = 8;
+constexpr int kPanelThreads = 512;
+constexpr int kPanelSpinLimit = 1 << 20;
+// words of the barrier state: [xcd][16] = { rank ticket, arrivals, departures, abort }.  Every word is only
+// ever touched by the workgroups of its own XCD (the L2s of different XCDs are not coherent inside a kernel).
+constexpr int kPanelStateStride = 16;
+constexpr int kPanelStateWords = kPanelXcds * kPanelStateStride;
+
+typedef float pv4f __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ unsigned panel_xcc_id() {
+  unsigned x;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(x));
+  return x & 0xfu;
+}
+// the counter's value as the L2 holds it
+__device__ __forceinline__ unsigned panel_poll(unsigned *p) {
+  unsigned r, zero = 0;
+  asm volatile("global_atomic_add %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)" : "=v"(r) : "v"(p), "v"(zero) : "memory");
+  return r;
+}
+__device__ __forceinline__ unsigned panel_ticket(unsigned *p) {
+  unsigned r, one = 1;
+  asm volatile("global_atomic_add %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)" : "=v"(r) : "v"(p), "v"(one) : "memory");
+  return r;
+}
+__device__ __forceinline__ void panel_count(unsigned *p) {
+  unsigned one = 1;
+  asm volatile("global_atomic_add %0, %1, off" ::"v"(p), "v"(one) : "memory");
+}
+
+// Entry of a panel kernel: the workgroup's XCD and its rank there.  false: more than 32 workgroups on this
+// XCD (abort word set).
+struct PanelWho {
+  unsigned xcd, rank;
+  unsigned *st;
+};
+__device__ __forceinline__ bool panel_enter(unsigned *state, PanelWho &w, unsigned *s_rank) {
+  w.xcd = panel_xcc_id();
+  if (w.xcd >= static_cast<unsigned>(kPanelXcds)) w.xcd = 0;  // the probe at context creation rules this out
+  w.st = state + w.xcd * kPanelStateStride;
+  if (threadIdx.x == 0) *s_rank = panel_ticket(w.st + 0);
+  __syncthreads();
+  w.rank = *s_rank;
+  if (w.rank >= static_cast<unsigned>(kPanelRanks)) {
+    if (threadIdx.x == 0) w.st[3] = 1;
+    return false;
+  }
+  return true;
+}
+// Thread 0 waits until `target` arrivals have been counted on this XCD.  Returns false after the spin limit.
+__device__ __forceinline__ bool panel_wait(PanelWho const &w, unsigned target) {
+  int spins = 0;
+  while (panel_poll(w.st + 1) < target) {
+    if (++spins > kPanelSpinLimit || (spins % 1024 == 0 && panel_poll(w.st + 3) != 0)) {
+      panel_count(w.st + 3);
+      return false;
+    }
+  }
+  return true;
+}
+// Exit: the last workgroup of an XCD to leave puts the three words back to zero for the next launch.
+__device__ __forceinline__ void panel_leave(PanelWho const &w) {
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned const d = panel_ticket(w.st + 2);
+    if (d == static_cast<unsigned>(kPanelRanks) - 1) {
+      w.st[0] = 0;
+      w.st[1] = 0;
+      w.st[2] = 0;
+    }
+  }
+}
+
+// host side (norm_panel_fwd.hip; panel_init / panel_check / panel_scratch_bytes are declared in dlmi_common.hpp)
+int panel_order_launch(dlmi_ctx *ctx);         // before a panel launch: orders it behind the last one of another stream
+void panel_launched(dlmi_ctx *ctx);            // after it
+
+}  // namespace dlmi
+
+#endif  // DLMI_NORM_PANEL_COMMON_HPP

@@ -1,0 +1,129 @@
+"""The single-launch (column panel) normalization kernels against the multi-launch path of the same library
+and against the oracle: same per-unit arithmetic, the batch summed in 32 chunks instead of <= 16, so the two
+paths agree to rounding of the column sums (1e-6 relative on the statistics), not bit for bit.  A context
+created with DLMI_NORM_PANEL=0 never takes the panel path; that is the twin here."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_close
+from oracle.binding import ACT, DROP
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def twins(pkg):
+    os.environ["DLMI_NORM_PANEL"] = "0"
+    try:
+        plain = pkg.Dlmi(0)
+    finally:
+        del os.environ["DLMI_NORM_PANEL"]
+    panel = pkg.Dlmi(0)
+    yield panel, plain
+    panel.close()
+    plain.close()
+
+
+def dev(a, dtype=torch.float32):
+    return torch.as_tensor(np.ascontiguousarray(a), dtype=dtype, device="cuda")
+
+
+def make(B, H, seed):
+    rng = np.random.default_rng(seed)
+    s = rng.uniform(0.5, 2.0, H).astype(np.float32)
+    m = rng.uniform(-1, 1, H).astype(np.float32)
+    x = (rng.standard_normal((B, H)).astype(np.float32) * s + m).astype(np.float32)
+    return dict(x=x, gamma=rng.uniform(.8, 1.2, H).astype(np.float32), beta=rng.uniform(-.1, .1, H).astype(np.float32),
+                mm=rng.uniform(-.2, .2, H).astype(np.float32), ms=rng.uniform(.6, 1.6, H).astype(np.float32),
+                dy=rng.standard_normal((B, H)).astype(np.float32), short=rng.standard_normal((B, H)).astype(np.float32),
+                emask=(rng.uniform(size=(B, H)) < 0.9).astype(np.uint8), umask=(rng.uniform(size=H) < 0.8).astype(np.uint8))
+
+
+def run_fwd(dl, pkg, d, act, drop, per_element, shortcut, renorm=True):
+    desc = pkg.Dlmi.desc(ACT[act], renorm=renorm, dropout=DROP[drop], mask_per_element=per_element, momentum=0.9, eps=1e-5,
+                         r_max=3.0, d_max=5.0, drop_scale=float(np.float32(1) / np.float32(0.9)))
+    mask = None if drop == "NONE" else dev(d["emask"] if per_element else d["umask"], torch.uint8)
+    mm, ms = dev(d["mm"]), dev(d["ms"])
+    y, st = dl.fused_fwd(desc, dev(d["x"]), dev(d["gamma"]), dev(d["beta"]), mm, ms, mask=mask,
+                         shortcut=dev(d["short"]) if shortcut else None)
+    dl.synchronize()
+    out = {k: v.cpu().numpy() for k, v in st.items()}
+    out.update(y=y.cpu().numpy(), mov_mean=mm.cpu().numpy(), mov_std=ms.cpu().numpy())
+    return out, desc, mask, st
+
+
+CASES = [  # B, H, act, dropout, per element, shortcut
+    (1024, 1024, "RELU", "NONE", False, False),
+    (1024, 2048, "ISRLU", "BERNOULLI_INVERTED", True, True),    # a block of workload c4
+    (2048, 1024, "ELU", "BERNOULLI", False, False),              # per-unit mask
+    (2048, 3072, "TANH", "NONE", False, True),
+    (4096, 1024, "SELU", "NONE", False, False),
+    (4096, 2048, "LEAKY_RELU", "BERNOULLI_INVERTED", True, False),
+    (8192, 1024, "ELU", "NONE", False, False),
+    (8192, 2048, "SIGMOID", "BERNOULLI", False, False),
+]
+
+
+@pytest.mark.parametrize("B,H,act,drop,per_element,shortcut", CASES)
+def test_forward_panel_equals_multi_launch_to_rounding(twins, pkg, B, H, act, drop, per_element, shortcut):
+    panel, plain = twins
+    d = make(B, H, B + H)
+    a, *_ = run_fwd(panel, pkg, d, act, drop, per_element, shortcut)
+    b, *_ = run_fwd(plain, pkg, d, act, drop, per_element, shortcut)
+    for k in ("mean", "std", "mov_mean", "mov_std", "r", "d"):
+        assert_close(a[k], b[k], 2e-6, f"{k} [{B}x{H}]")
+    assert_close(a["y"], b["y"], 1e-5, f"y [{B}x{H}]", floor=1.0)
+
+
+def test_forward_panel_against_float64(twins, pkg):
+    """4096 x 1024, batch renormalization + SELU: the closed form in float64."""
+    panel, _ = twins
+    B, H = 4096, 1024
+    d = make(B, H, 5)
+    a, *_ = run_fwd(panel, pkg, d, "SELU", "NONE", False, False)
+    x = d["x"].astype(np.float64)
+    mean = x.mean(0)
+    std = np.sqrt((x * x).mean(0) - mean * mean + 1e-5)
+    mm = d["mm"] + 0.9 * (mean - d["mm"])
+    ms = d["ms"] + 0.9 * (std - d["ms"])
+    r = np.clip(std / ms, 1 / 3.0, 3.0)
+    dd = np.clip((mean - mm) / ms, -5.0, 5.0)
+    n = d["gamma"] * ((x - mean) / std * r + dd) + d["beta"]
+    al, sc = 1.6732632423543772, 1.0507009873554805
+    y = sc * np.where(n > 0, n, al * np.expm1(n))
+    assert_close(a["mean"], mean, 2e-6, "mean")
+    assert_close(a["std"], std, 2e-6, "std")
+    assert_close(a["mov_mean"], mm, 2e-6, "moving mean")
+    assert_close(a["mov_std"], ms, 2e-6, "moving std")
+    assert_close(a["r"], r, 2e-6, "r")
+    assert_close(a["d"], dd, 1e-5, "d", floor=1.0)
+    assert_close(a["y"], y, 1e-5, "y", floor=1.0)
+
+
+def test_forward_panel_is_reproducible_and_leaves_no_state(twins, pkg):
+    """Same bits on every call (fixed summation order), also after a call of another shape in between: the
+    barrier words are back at zero when a launch ends."""
+    panel, _ = twins
+    d = make(2048, 1024, 9)
+    first, *_ = run_fwd(panel, pkg, d, "ELU", "NONE", False, False)
+    other = make(1024, 2048, 10)
+    run_fwd(panel, pkg, other, "RELU", "NONE", False, False)
+    for _ in range(3):
+        again, *_ = run_fwd(panel, pkg, d, "ELU", "NONE", False, False)
+        for k in first:
+            assert np.array_equal(first[k], again[k]), k
+
+
+def test_shapes_outside_the_panel_geometry_take_the_multi_launch_path(twins, pkg):
+    """Batches that are not 1024 / 2048 / 4096 / 8192 rows or widths that are not multiples of 1024: bit-identical
+    results from both contexts, because both run the same kernels."""
+    panel, plain = twins
+    for B, H in [(1536, 1024), (1024, 1536), (512, 1024), (4096, 1000)]:
+        d = make(B, H, B * 3 + H)
+        a, *_ = run_fwd(panel, pkg, d, "ELU", "NONE", False, False)
+        b, *_ = run_fwd(plain, pkg, d, "ELU", "NONE", False, False)
+        for k in a:
+            assert np.array_equal(a[k], b[k]), (B, H, k)
