@@ -1,4 +1,5 @@
-"""The single-launch (column panel) normalization kernels against the multi-launch path of the same library
+"""The single-launch (column panel) normalization kernels (forward: 1024 - 8192 rows, backward: 1024 - 4096 rows; the
+8192-row backward cases below run the multi-launch kernels in both contexts) against the multi-launch path of the same library
 and against the oracle: same per-unit arithmetic, the batch summed in 32 chunks instead of <= 16, so the two
 paths agree to rounding of the column sums (1e-6 relative on the statistics), not bit for bit.  A context
 created with DLMI_NORM_PANEL=0 never takes the panel path; that is the twin here."""
@@ -127,3 +128,54 @@ def test_shapes_outside_the_panel_geometry_take_the_multi_launch_path(twins, pkg
         b, *_ = run_fwd(plain, pkg, d, "ELU", "NONE", False, False)
         for k in a:
             assert np.array_equal(a[k], b[k]), (B, H, k)
+
+
+def run_bwd(dl, pkg, d, desc, mask, st):
+    B, H = d["x"].shape
+    dg, db = torch.full((H,), 0.25, device="cuda"), torch.full((H,), -0.5, device="cuda")  # they accumulate
+    dx = dl.fused_bwd(desc, dev(d["x"]), dev(d["gamma"]), dev(d["beta"]), st, dev(d["dy"]), dg, db, mask=mask)
+    dl.synchronize()
+    return dict(dx=dx.cpu().numpy(), dgamma=dg.cpu().numpy(), dbeta=db.cpu().numpy())
+
+
+@pytest.mark.parametrize("B,H,act,drop,per_element,shortcut", CASES)
+def test_backward_panel_equals_multi_launch_to_rounding(twins, pkg, B, H, act, drop, per_element, shortcut):
+    panel, plain = twins
+    d = make(B, H, B + H + 1)
+    # both backward passes start from the SAME forward results (the multi-launch context's)
+    _, desc, mask, st = run_fwd(plain, pkg, d, act, drop, per_element, False)
+    a = run_bwd(panel, pkg, d, desc, mask, st)
+    b = run_bwd(plain, pkg, d, desc, mask, st)
+    assert_close(a["dx"], b["dx"], 1e-4, f"dX [{B}x{H}]", floor=1.0)
+    assert_close(a["dgamma"], b["dgamma"], 1e-4, "dgamma", floor=1.0)
+    assert_close(a["dbeta"], b["dbeta"], 1e-4, "dbeta", floor=1.0)
+
+
+def test_backward_panel_against_float64(twins, pkg):
+    """4096 x 1024, batch renormalization + ELU: dX, dgamma, dbeta from the closed form in float64, and the
+    invariant that r-corrected batch normalization removes the column mean of dX."""
+    panel, _ = twins
+    B, H = 4096, 1024
+    d = make(B, H, 6)
+    a, desc, mask, st = run_fwd(panel, pkg, d, "ELU", "NONE", False, False)
+    g = run_bwd(panel, pkg, d, desc, mask, st)
+    x, dy = d["x"].astype(np.float64), d["dy"].astype(np.float64)
+    mean, std, r, dd = (a[k].astype(np.float64) for k in ("mean", "std", "r", "d"))
+    xh = (x - mean) / std * r + dd
+    n = d["gamma"] * xh + d["beta"]
+    keep = np.abs(n) > 1e-4  # the derivative of ELU jumps at 0: leave the few elements within rounding of it out
+    # the reference's ELU derivative for n < 0 is the activation value itself, alpha * (exp(n) - 1), not
+    # alpha * exp(n) (v1/ops/activations/functions.hpp:92): the kernels keep that
+    dn = dy * np.where(n > 0, 1.0, np.expm1(n)) * keep
+    # the GPU sees the same zeros
+    dyk = (dy * keep).astype(np.float32)
+    d2 = dict(d, dy=dyk)
+    g = run_bwd(panel, pkg, d2, desc, mask, st)
+    e = dn * d["gamma"]
+    dmean = (e * (-r / std)).sum(0)
+    dstd = (e * (x - mean) * (-r / std ** 2)).sum(0)
+    dx = e * (r / std) + dstd * (x - mean) / (B * std) + dmean / B
+    assert_close(g["dx"], dx, 1e-4, "dX", floor=1.0)
+    assert_close(g["dgamma"], 0.25 + (dn * xh).sum(0), 1e-4, "dgamma", floor=1.0)
+    assert_close(g["dbeta"], -0.5 + dn.sum(0), 1e-4, "dbeta", floor=1.0)
+    assert np.max(np.abs(g["dx"].astype(np.float64).sum(0))) < 1e-2  # sum_b dX = 0 up to rounding of 4096 terms
