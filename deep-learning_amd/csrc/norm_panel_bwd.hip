@@ -5,7 +5,7 @@
 //
 // Geometry: 512 threads = P/4 column groups of 4 units x 2048/P rows; a workgroup owns B/32 = RPT * 2048/P rows
 // and walks panels of P columns: P = 64 (256 B per row) while four panels of x and dn fit the registers, P = 32
-// for 4096 rows with a per-element mask.  B in {1024, 2048, 4096}, H a multiple of 512.  (Wider panels stream
+// for 4096 rows with a per-element mask.  B in {2048, 4096}, H a multiple of 512.  (Wider panels stream
 // faster - the forward kernel's 128 columns reach 5.1 TB/s of actual traffic, 64 columns 3.7 TB/s - but the
 // backward pass holds two values per element; the kernel still beats the multi-launch pair because it moves
 // 12 instead of 20 bytes per element.)
@@ -263,7 +263,9 @@ int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4
   if (H % 512 != 0) return 0;
   // 8192 rows: four panels of x and dn only fit the registers at 32 columns per panel, and rows cut into
   // 128-byte pieces stream slower than the multi-launch kernels (measured 113 us against 108 us at 8192 x 4096)
-  if (B != 1024 && B != 2048 && B != 4096) return 0;
+  // 1024 rows: no faster than the multi-launch pair in isolation (15 us both) and slower inside a step, where a
+  // launch that needs every CU at once cannot start into the tail of the kernel before it
+  if (B != 2048 && B != 4096) return 0;
   bool const extra = c.accumulate || c.drop_mode == kDropElem;
   if (c.drop_mode == kDropElem && (reinterpret_cast<uintptr_t>(c.mask) & 3u) != 0) return 0;
   int rc = dlmi_scratch_reserve(ctx, panel_scratch_bytes(H));
@@ -282,13 +284,11 @@ int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4
   DLMI_DISPATCH_ACT(c.act, {
     if (extra) {
       switch (B) {
-        case 1024: launch_bwd<ACT, 64, 1, true>(ctx, a); break;
         case 2048: launch_bwd<ACT, 64, 2, true>(ctx, a); break;
         default: launch_bwd<ACT, 32, 2, true>(ctx, a); break;  // 4096 rows
       }
     } else {
       switch (B) {
-        case 1024: launch_bwd<ACT, 64, 1, false>(ctx, a); break;
         case 2048: launch_bwd<ACT, 64, 2, false>(ctx, a); break;
         default: launch_bwd<ACT, 64, 4, false>(ctx, a); break;  // 4096 rows
       }
