@@ -46,8 +46,8 @@ LAYER_WORKLOADS = {
 MIB = 1024.0 * 1024.0
 TRAFFIC_PROFILE = "profiles/c3_c2_hbm_traffic_pmc.md"
 MEASURED_TRAFFIC_BYTES = {
-    "c3": {"gemm": (897.9 + 897.3 + 832.8) / 3.0 * MIB, "norm_act": 1047.0 * MIB},
-    "c2": {"norm_act": 528.8 * MIB},
+    "c3": {"gemm": (897.8 + 897.3 + 832.8) / 3.0 * MIB, "norm_act": 901.8 * MIB},
+    "c2": {"norm_act": 326.4 * MIB},
 }
 
 
@@ -350,7 +350,11 @@ def run_layer(args, torch, pkg, dl, name, full):
     hbm = {"bound": "hbm", "achieved": 32.0 * E / ((t_nf + t_nb) * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
            "traffic": MEASURED_TRAFFIC_BYTES.get(name, {}).get("norm_act"),
            "traffic_source": TRAFFIC_PROFILE if name in MEASURED_TRAFFIC_BYTES else None,
-           "kernels": "k_col_stats+k_fwd_finalize+k_fwd_apply / k_bwd_reduce+k_bwd_apply (algorithmic 12 + 20 B/element)",
+           "kernels": "dlmi_fused_norm_act_fwd + dlmi_fused_norm_act_bwd; `achieved` counts the two-pass accounting "
+                      "of 12 + 20 B/element.  Batches of 1024-8192 rows (forward) / 2048-4096 rows (backward) with a "
+                      "width that is a multiple of 1024 run the single-launch panel kernels, which read every tensor "
+                      "once (8 + 12 B/element of actual traffic, see `traffic`); other shapes run k_col_stats -> "
+                      "k_fwd_apply / k_bwd_reduce -> k_bwd_apply",
            "ms_fwd": t_nf, "ms_bwd": t_nb, "bytes_fwd": 12.0 * E, "bytes_bwd": 20.0 * E}
     hbm["frac"] = hbm["achieved"] / hbm["peak"]
     detail = {"ms_norm_fwd": t_nf, "ms_norm_bwd": t_nb}

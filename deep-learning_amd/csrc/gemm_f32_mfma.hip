@@ -371,14 +371,24 @@ void k_gemm_f32(GemmArgs g) {
   }
 }
 
-// Fixed-order sum of the split-K partial products (+ bias, + previous C).
+// Fixed-order sum of the split-K partial products (+ bias, + previous C): slice 0, 1, 2, ... as before, with
+// the loads of eight slices in flight at a time (one thread per element would otherwise walk the slices one
+// memory latency after the other: 17 us for 64 slices of a 256 x 256 product).
 __global__ __launch_bounds__(256) void k_splitk_reduce(float const *__restrict__ part, unsigned splits, size_t mn,
                                                         size_t N, float const *__restrict__ bias,
                                                         float *__restrict__ C, int accumulate) {
   size_t const stride = static_cast<size_t>(gridDim.x) * 256;
   for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < mn; i += stride) {
     float s = 0.0f;
-    for (unsigned z = 0; z < splits; ++z) s += part[z * mn + i];
+    unsigned z = 0;
+    for (; z + 8 <= splits; z += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = part[(z + u) * mn + i];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    for (; z < splits; ++z) s += part[z * mn + i];
     if (bias != nullptr) s += bias[i % N];
     if (accumulate) s += C[i];
     C[i] = s;
