@@ -944,7 +944,7 @@ static int run_fwd_train(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t 
                                  c.residual}) &&
                     (c.drop_mode == kDropNone || (reinterpret_cast<uintptr_t>(c.mask) & 3u) == 0);
   // a few thousand rows, H a multiple of 1024: one launch that reads x once
-  if (int const took = panel_fwd_try(ctx, B, H, c, vec4); took != 0) return took < 0 ? took : DLMI_OK;
+  if (int const took = panel_fwd_try(ctx, B, H, c, vec4, sv.data, sv.data_bytes); took != 0) return took < 0 ? took : DLMI_OK;
   dim3 const block(kBlock);
   FwdFinalize fin;
   fin.mean = c.mean; fin.stdv = c.stdv; fin.mov_mean = c.mov_mean; fin.mov_std = c.mov_std; fin.r = c.r; fin.d = c.d;
@@ -1030,7 +1030,7 @@ static int run_bwd(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, Bwd
   bool const vec4 = use_vec4(H, {c.x, c.gamma, c.beta, c.mean, c.stdv, c.r, c.d, c.xhat, c.dY, c.dX, c.dgamma, c.dbeta}) &&
                     (c.drop_mode == kDropNone || (reinterpret_cast<uintptr_t>(c.mask) & 3u) == 0);
   // a few thousand rows, H a multiple of 512: one launch that reads dY and x once
-  if (int const took = panel_bwd_try(ctx, B, H, c, vec4); took != 0) return took < 0 ? took : DLMI_OK;
+  if (int const took = panel_bwd_try(ctx, B, H, c, vec4, sv.data, sv.data_bytes); took != 0) return took < 0 ? took : DLMI_OK;
   ColGeom g;
   bool const fold = !c.xhat_given && c.dmean == nullptr && c.dstd == nullptr &&
                     fold_geometry(ctx, B, H, vec4, 3, sv.data_bytes, &g);

@@ -258,7 +258,7 @@ void launch_bwd(dlmi_ctx *ctx, PanelBwdArgs const &a) {
 
 }  // namespace
 
-int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4) {
+int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4, void *scratch, size_t scratch_bytes) {
   if (!ctx->panel_ok || !vec4 || c.xhat_given || c.dmean != nullptr || c.dstd != nullptr) return 0;
   if (H % 512 != 0) return 0;
   // 8192 rows: four panels of x and dn only fit the registers at 32 columns per panel, and rows cut into
@@ -268,8 +268,10 @@ int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4
   if (B != 2048 && B != 4096) return 0;
   bool const extra = c.accumulate || c.drop_mode == kDropElem;
   if (c.drop_mode == kDropElem && (reinterpret_cast<uintptr_t>(c.mask) & 3u) != 0) return 0;
-  int rc = dlmi_scratch_reserve(ctx, panel_scratch_bytes(H));
-  if (rc != DLMI_OK) return rc;
+  // the caller's scratch (the context's block, already reserved, or the fixed array of the entry point that
+  // allocates nothing): too small for the chunk partials means the multi-launch kernels
+  if (scratch == nullptr || scratch_bytes < panel_scratch_bytes(H)) return 0;
+  int rc;
   PanelBwdArgs a;
   a.x = c.x; a.dY = c.dY; a.gamma = c.gamma; a.beta = c.beta; a.mean = c.mean; a.stdv = c.stdv; a.r = c.r; a.d = c.d;
   a.mask = c.mask; a.dX = c.dX; a.dgamma = c.dgamma; a.dbeta = c.dbeta;
@@ -277,7 +279,7 @@ int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4
   a.batch_f = static_cast<float>(B); a.batch_scale = 1.0f / static_cast<float>(B); a.drop_scale = c.drop_scale;
   a.drop_mode = c.drop_mode; a.drop_bwd_masked = c.drop_bwd_masked; a.accumulate = c.accumulate ? 1 : 0;
   a.state = ctx->panel_state;
-  a.part = reinterpret_cast<float *>(dlmi_scratch_data(ctx));
+  a.part = static_cast<float *>(scratch);
   rc = panel_order_launch(ctx);
   if (rc != DLMI_OK) return rc;
   // rows per workgroup = B / 32 = RPT * 2048 / P

@@ -291,7 +291,7 @@ int panel_check(dlmi_ctx *ctx) {
 
 size_t panel_scratch_bytes(size_t H) { return static_cast<size_t>(kPanelRanks) * 3 * H * sizeof(float) + 4096; }
 
-int panel_fwd_try(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c, bool vec4) {
+int panel_fwd_try(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c, bool vec4, void *scratch, size_t scratch_bytes) {
   if (!ctx->panel_ok || !vec4 || c.partial_in != nullptr || c.xhat != nullptr || c.nrm != nullptr || c.y == nullptr) return 0;
   if (H % (static_cast<size_t>(kPanelXcds) * kP) != 0 || B % (static_cast<size_t>(kPanelRanks) * kTY) != 0) return 0;
   size_t const rpt = B / (static_cast<size_t>(kPanelRanks) * kTY);
@@ -299,8 +299,10 @@ int panel_fwd_try(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c, bool
   bool const extra = c.residual != nullptr || c.drop_mode == kDropElem;
   if (extra && rpt == 16) return 0;  // the three panels in flight plus the extra streams do not fit the registers
   if (c.drop_mode == kDropElem && (reinterpret_cast<uintptr_t>(c.mask) & 3u) != 0) return 0;
-  int rc = dlmi_scratch_reserve(ctx, panel_scratch_bytes(H));
-  if (rc != DLMI_OK) return rc;
+  // the caller's scratch (the context's block, already reserved, or the fixed array of the entry point that
+  // allocates nothing): too small for the chunk partials means the multi-launch kernels
+  if (scratch == nullptr || scratch_bytes < panel_scratch_bytes(H)) return 0;
+  int rc;
   PanelFwdArgs a;
   a.x = c.x; a.gamma = c.gamma; a.beta = c.beta; a.residual = c.residual; a.mask = c.mask; a.y = c.y;
   a.B = B; a.H = H;
@@ -310,7 +312,7 @@ int panel_fwd_try(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c, bool
   a.fin.renorm = c.norm == DLMI_NORM_BATCH_RENORM ? 1 : 0;
   a.drop_mode = c.drop_mode; a.drop_scale = c.drop_scale;
   a.state = ctx->panel_state;
-  a.part = reinterpret_cast<float *>(dlmi_scratch_data(ctx));
+  a.part = static_cast<float *>(scratch);
   rc = panel_order_launch(ctx);
   if (rc != DLMI_OK) return rc;
   DLMI_DISPATCH_ACT(c.act, {

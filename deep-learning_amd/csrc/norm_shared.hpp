@@ -117,8 +117,8 @@ struct BwdCall {
 // The single-launch panel kernels (norm_panel_fwd.hip, norm_panel_bwd.hip).  Return 1 when the call was
 // launched that way, 0 when the shape or the context does not qualify (the caller goes on with the
 // multi-launch path), a negative DLMI_E_* code on failure.
-int panel_fwd_try(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c, bool vec4);
-int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4);
+int panel_fwd_try(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c, bool vec4, void *scratch, size_t scratch_bytes);
+int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4, void *scratch, size_t scratch_bytes);
 
 }  // namespace dlmi
 

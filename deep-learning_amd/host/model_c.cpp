@@ -28,6 +28,14 @@ struct dlmi_mnist {
   dlmi::MNIST ds;
 };
 
+namespace {
+std::wstring widen(char const *s) {
+  std::wstring w;
+  for (; s != nullptr && *s != '\0'; ++s) w += static_cast<wchar_t>(static_cast<unsigned char>(*s));
+  return w;
+}
+}  // namespace
+
 extern "C" {
 
 dlmi_model *dlmi_model_create(size_t n_layers, size_t const *widths) {
@@ -88,14 +96,6 @@ void dlmi_model_init_uniform(dlmi_model *h, unsigned seed, float bias, float low
 
 // An uncompiled model: what dlmi_model_load() fills.
 dlmi_model *dlmi_model_create_empty(void) { return new dlmi_model; }
-
-namespace {
-std::wstring widen(char const *s) {
-  std::wstring w;
-  for (; s != nullptr && *s != '\0'; ++s) w += static_cast<wchar_t>(static_cast<unsigned char>(*s));
-  return w;
-}
-}  // namespace
 
 int dlmi_model_save_params(dlmi_model *h, char const *path) { return h->m.save_params(widen(path)); }
 int dlmi_model_save_spec_params(dlmi_model *h, char const *path) { return h->m.save_spec_params(widen(path)); }

@@ -61,6 +61,45 @@ def test_noalloc_entry_matches_the_allocating_one_twice_in_a_row(dl, pkg, act):
             assert np.array_equal(o["noalloc"][k], v), f"[{B}x{H}] {k}: same kernels, same geometry, yet not identical"
 
 
+def test_noalloc_entry_on_single_launch_shapes(dl, pkg):
+    """A few thousand rows: the allocating entry point runs the single-launch panel kernel, whose chunk
+    partials need 384 bytes per unit.  The entry point that allocates nothing runs the same kernel while
+    they fit its fixed array (bit-identical then) and the multi-launch kernels beyond (same tolerance as
+    any two summation orders)."""
+    o = run_both(dl, pkg, 2048, 1024, "ELU", 5, True)
+    for k, v in o["alloc"].items():
+        assert np.array_equal(o["noalloc"][k], v), k
+    o = run_both(dl, pkg, 1024, 8192, "ELU", 6, False)   # 3 MiB of panel partials: more than the array
+    for k, v in o["alloc"].items():
+        assert np.all(np.isfinite(v)), k
+        assert_close(o["noalloc"][k], v, 1e-5 if k == "y" else TR, f"[1024x8192] {k}", floor=1.0)
+
+
+def test_noalloc_entry_never_touches_the_context_scratch(pkg):
+    """On a context of its own, whose scratch block nothing has grown yet: the block's generation and the
+    device's free memory stay what they were across calls of every kernel family."""
+    import ctypes
+    d = pkg.Dlmi(0)
+    try:
+        d.lib.dlmi_ctx_scratch_generation.restype = ctypes.c_ulonglong
+        gen0 = d.lib.dlmi_ctx_scratch_generation(d.ctx)
+        desc = pkg.Dlmi.desc(pkg.ACT["RELU"], renorm=True)
+        for B, H in ((4096, 4096), (64, 65536), (8192, 1024), (100, 36)):
+            x = torch.randn((B, H), device="cuda")
+            v = lambda: torch.ones(H, device="cuda")
+            args = (desc, x, v(), v() * 0, v() * 0, v())
+            kw = dict(out=torch.empty_like(x), stats={k: v() for k in ("mean", "std", "r", "d")}, noalloc=True)
+            torch.cuda.synchronize()
+            free0 = torch.cuda.mem_get_info()[0]
+            d.fused_fwd(*args, **kw)
+            torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info()[0] == free0, (B, H)
+            assert d.lib.dlmi_ctx_scratch_generation(d.ctx) == gen0, (B, H)
+            assert torch.isfinite(kw["out"]).all()
+    finally:
+        d.close()
+
+
 def test_noalloc_entry_refuses_more_units_than_its_array_holds(dl, pkg):
     H = 65536 + 4
     desc = pkg.Dlmi.desc(pkg.ACT["RELU"])
