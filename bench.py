@@ -155,7 +155,7 @@ def layer_inputs(name):
     import numpy as np
     from oracle.binding import HarnessRng
     B, K, H, act, _ = LAYER_WORKLOADS[name]
-    rng = HarnessRng(1234 + {"c2": 200, "c3": 300, "c5": 500}[name])
+    rng = HarnessRng(1234 + {"c2": 200, "c3": 300, "c5": 500}.get(name, 900))
     t = {}
     if K:
         t["X"] = rng.normal(1, (B, K))
@@ -657,7 +657,14 @@ def main():
     ap.add_argument("--only", default="", help="profiling aid (layer workloads): run just this part (gemm_fwd, gemm_dx, "
                                                "gemm_dw, norm_fwd, norm_bwd, fc_norm_fwd, infer_fwd, adam, copy) "
                                                "--steps times and exit without a JSON line")
+    ap.add_argument("--shape", default="", help="profiling aid, with --only: B,K,H of the layer to run the part on instead "
+                                                "of a workload's (e.g. 1024,2048,2048: one block of c4)")
     args = ap.parse_args()
+    if args.shape:
+        if not args.only:
+            ap.error("--shape needs --only")
+        LAYER_WORKLOADS["shape"] = tuple(int(v) for v in args.shape.split(",")) + ("ELU", "profiling shape " + args.shape)
+        args.workload = "shape"
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
