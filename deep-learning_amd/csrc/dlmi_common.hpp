@@ -28,6 +28,7 @@ struct dlmi_tuning {
   int fold_fwd = 1;
   int fold_bwd = 2;
   size_t fold_fwd_max_elements = size_t(1) << 20;
+  int norm_small = 1;             // mini-batches (at most 256 rows, 2^20 elements) run the one-launch small-batch kernels
 };
 
 struct dlmi_ctx {
@@ -104,7 +105,12 @@ int static_scratch_init(dlmi_ctx *ctx);
 int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
                             float const *gamma, float const *beta, uint8_t const *mask, float const *residual,
                             float *mean, float *stdv, float *mov_mean, float *mov_std, float *r, float *d, float *y,
-                            float const *partial, unsigned nchunks);
+                            float const *partial, unsigned nchunks, float const *slices = nullptr,
+                            unsigned nslices = 0);
+// Whether a [B, H] tensor runs the small-batch normalization kernels.  Those also accept x as `nslices`
+// partial products [nslices][B][H] still to be added (the slices of a split-K product, passed to
+// fused_fwd_from_partials with x = where the sum is to be stored): a producer may skip its own reduction then.
+bool small_norm_eligible(dlmi_ctx const *ctx, size_t B, size_t H);
 // out[j] (+)= sum over the B rows of x[b, j], in a fixed order (the statistics
 // pass of the normalization kernels with its second plane unused).
 int column_sums(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *out, int accumulate);

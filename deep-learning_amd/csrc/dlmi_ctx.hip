@@ -78,6 +78,7 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
   t.apply_interleave = env_flag("DLMI_NORM_APPLY_INTERLEAVE", t.apply_interleave);
   t.fold_fwd = env_level("DLMI_NORM_FOLD_FWD", t.fold_fwd);
   t.fold_bwd = env_level("DLMI_NORM_FOLD_BWD", t.fold_bwd);
+  t.norm_small = env_flag("DLMI_NORM_SMALL", t.norm_small);
   int rc = dlmi_scratch_reserve(ctx, size_t(16) << 20);
   if (rc == DLMI_OK) rc = dlmi::static_scratch_init(ctx);
   if (rc == DLMI_OK) rc = dlmi::panel_init(ctx);

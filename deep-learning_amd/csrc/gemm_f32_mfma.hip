@@ -532,7 +532,8 @@ size_t fc_scratch_bytes(dlmi_ctx const *ctx, size_t B, size_t K, size_t H) {
 // of C into the first half of the context's scratch (no split-K then).
 template <bool AK, bool BKC>
 static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, size_t lda, float const *B, size_t ldb,
-                float *C, float const *bias, int accumulate, unsigned *stats_chunks = nullptr) {
+                float *C, float const *bias, int accumulate, unsigned *stats_chunks = nullptr,
+                unsigned *defer_slices = nullptr) {
   GemmPlan const plan = plan_gemm(ctx, M, N, K);
   int const choice = plan.choice;
   int const bm = plan.bm, bn = plan.bn, bk = plan.bk;
@@ -574,6 +575,11 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
     default: rc = launch_gemm<128, 128, 16, AK, BKC, 2>(ctx, g, splits, fast); break;
   }
   if (rc != DLMI_OK) return rc;
+  if (defer_slices != nullptr) {
+    // the caller adds the slices itself ([splits][M][N] at the start of the scratch block, slice order)
+    *defer_slices = splits > 1 ? splits : 0;
+    if (splits > 1) return DLMI_OK;
+  }
   if (splits > 1) {
     size_t const mn = M * N;
     size_t blocks = dlmi_ceil_div(mn, 256);
@@ -604,13 +610,19 @@ static int fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B,
                            float const *W, float const *gamma, float const *beta, uint8_t const *mask,
                            float const *shortcut, float *Z, float *mean, float *stdv, float *mov_mean, float *mov_std,
                            float *r, float *d, float *y) {
-  unsigned chunks = 0;
-  int rc = gemm<true, true>(ctx, B, H, K, X, K, W, K, Z, nullptr, 0, &chunks);
+  unsigned chunks = 0, slices = 0;
+  // a mini-batch: the normalization kernel that follows owns whole columns and adds the K slices itself
+  bool const defer = small_norm_eligible(ctx, B, H);
+  int rc = gemm<true, true>(ctx, B, H, K, X, K, W, K, Z, nullptr, 0, &chunks, defer ? &slices : nullptr);
   if (rc != DLMI_OK) return rc;
+  float const *const scratch = reinterpret_cast<float const *>(dlmi_scratch_data(ctx));
+  if (slices != 0)
+    return fused_fwd_from_partials(ctx, desc, B, H, Z, gamma, beta, mask, shortcut, mean, stdv, mov_mean, mov_std, r, d, y,
+                                   nullptr, 0, scratch, slices);
   // a small output runs split over K, where no slice sees whole sums: the
   // statistics then come from a pass over Z (nullptr / 0)
   return fused_fwd_from_partials(ctx, desc, B, H, Z, gamma, beta, mask, shortcut, mean, stdv, mov_mean, mov_std, r, d, y,
-                                 chunks != 0 ? reinterpret_cast<float const *>(dlmi_scratch_data(ctx)) : nullptr, chunks);
+                                 chunks != 0 ? scratch : nullptr, chunks);
 }
 
 int dlmi_fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t K, size_t H, float const *X,

@@ -943,6 +943,8 @@ static int run_fwd_train(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t 
   bool const vec4 = use_vec4(H, {c.x, c.gamma, c.beta, c.mean, c.stdv, c.mov_mean, c.mov_std, c.r, c.d, c.y, c.xhat, c.nrm,
                                  c.residual}) &&
                     (c.drop_mode == kDropNone || (reinterpret_cast<uintptr_t>(c.mask) & 3u) == 0);
+  // a mini-batch of a few hundred rows: one launch, a workgroup per 8 columns
+  if (int const took = small_fwd_try(ctx, B, H, c); took != 0) return took < 0 ? took : DLMI_OK;
   // a few thousand rows, H a multiple of 1024: one launch that reads x once
   if (int const took = panel_fwd_try(ctx, B, H, c, vec4, sv.data, sv.data_bytes); took != 0) return took < 0 ? took : DLMI_OK;
   dim3 const block(kBlock);
@@ -1029,6 +1031,7 @@ static int run_fwd_train(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t 
 static int run_bwd(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, BwdCall const &c) {
   bool const vec4 = use_vec4(H, {c.x, c.gamma, c.beta, c.mean, c.stdv, c.r, c.d, c.xhat, c.dY, c.dX, c.dgamma, c.dbeta}) &&
                     (c.drop_mode == kDropNone || (reinterpret_cast<uintptr_t>(c.mask) & 3u) == 0);
+  if (int const took = small_bwd_try(ctx, B, H, c); took != 0) return took < 0 ? took : DLMI_OK;
   // a few thousand rows, H a multiple of 512: one launch that reads dY and x once
   if (int const took = panel_bwd_try(ctx, B, H, c, vec4, sv.data, sv.data_bytes); took != 0) return took < 0 ? took : DLMI_OK;
   ColGeom g;
@@ -1144,15 +1147,18 @@ static FwdTrainCall fused_fwd_call(dlmi_fused_desc const *desc, float const *x, 
 int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
                             float const *gamma, float const *beta, uint8_t const *mask, float const *residual,
                             float *mean, float *stdv, float *mov_mean, float *mov_std, float *r, float *d, float *y,
-                            float const *partial, unsigned nchunks) {
+                            float const *partial, unsigned nchunks, float const *slices, unsigned nslices) {
   int rc = check_desc(ctx, desc, mask);
   if (rc != DLMI_OK) return rc;
   DLMI_REQUIRE(ctx, x && gamma && beta && mean && stdv && mov_mean && mov_std && r && d && y, "null pointer");
   FwdTrainCall c = fused_fwd_call(desc, x, gamma, beta, mask, mean, stdv, mov_mean, mov_std, r, d, y);
   c.residual = residual;
   c.partial_in = partial; c.partial_chunks = nchunks;
+  if (nslices > 0) {
+    c.slices = slices; c.nslices = nslices; c.z_out = const_cast<float *>(x);
+  }
   ScratchView sv{};
-  if (partial == nullptr) {
+  if (partial == nullptr && nslices == 0) {
     rc = ctx_scratch(ctx, H, &sv);
     if (rc != DLMI_OK) return rc;
   }
@@ -1160,6 +1166,7 @@ int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
 }
 
 int column_sums(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *out, int accumulate) {
+  if (int const took = small_colsum_try(ctx, B, H, x, out, accumulate); took != 0) return took < 0 ? took : DLMI_OK;
   ScratchView sv{};
   int rc = ctx_scratch(ctx, H, &sv);
   if (rc != DLMI_OK) return rc;

@@ -101,6 +101,11 @@ struct FwdTrainCall {
   float *mean, *stdv, *mov_mean, *mov_std, *r, *d, *y, *xhat, *nrm;
   float const *partial_in = nullptr;  // column-sum partials already produced elsewhere ...
   unsigned partial_chunks = 0;        // ... [2][partial_chunks][H]; skips the statistics pass
+  // x itself not formed yet: it is the sum of `nslices` partial products [nslices][B][H] (split-K slices), to
+  // be added in slice order and stored to z_out (== x) by the small-batch kernel, the only one that takes them
+  float const *slices = nullptr;
+  unsigned nslices = 0;
+  float *z_out = nullptr;
 };
 
 struct BwdCall {
@@ -119,6 +124,13 @@ struct BwdCall {
 // multi-launch path), a negative DLMI_E_* code on failure.
 int panel_fwd_try(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c, bool vec4, void *scratch, size_t scratch_bytes);
 int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4, void *scratch, size_t scratch_bytes);
+
+
+// The small-batch kernels (norm_small.hip): one launch per direction for at most 256 rows and 2^20 elements.
+// Same return convention (small_norm_eligible, the shape test alone, is declared in dlmi_common.hpp).
+int small_fwd_try(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c);
+int small_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c);
+int small_colsum_try(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *out, int accumulate);
 
 }  // namespace dlmi
 
