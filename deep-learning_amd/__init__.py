@@ -42,6 +42,7 @@ C_ABI_SYMBOLS = [
     "dlmi_opt_gd", "dlmi_opt_gd_momentum", "dlmi_opt_adam", "dlmi_zero_padded_identity_fwd", "dlmi_residual_bwd",
     "dlmi_opt_adabound", "dlmi_clip_gradient", "dlmi_max_norm_rows", "dlmi_opt_irprop_plus", "dlmi_loss_seed", "dlmi_zero",
     "dlmi_fused_norm_act_fwd_noalloc", "dlmi_fused_norm_act_residual_fwd", "dlmi_fc_norm_act_residual_fwd",
+    "dlmi_fc_softmax_fwd", "dlmi_fc_bwd_dx_norm_act_bwd",
     "dlmi_ctx_reserve_layer", "dlmi_ctx_scratch_generation",
 ]
 
@@ -390,6 +391,27 @@ class Dlmi:
                                                   _p(beta), _p(mask), _p(stats["mean"]), _p(stats["std"]),
                                                   _p(stats["r"]), _p(stats["d"]), _p(dY), _p(dgamma), _p(dbeta),
                                                   _p(dX)))
+        return dX
+
+    def fc_softmax_fwd(self, X, W, bias=None):
+        """Z = X W^T + bias, Q = softmax(Z).  Returns (Z, Q)."""
+        self._chk(X, W, bias)
+        B, K = X.shape
+        H = W.shape[0]
+        Z, Q = self.empty(B, H), self.empty(B, H)
+        self._ck(self.lib.dlmi_fc_softmax_fwd(self.ctx, c_sz(B), c_sz(K), c_sz(H), _p(X), _p(W), _p(bias), _p(Z), _p(Q)))
+        return Z, Q
+
+    def fc_bwd_dx_fused_bwd(self, desc, dZn, Wn, x, gamma, beta, stats, dgamma, dbeta, mask=None):
+        """dY = dZn Wn, then the fused normalization backward on dY.  Returns dX."""
+        self._chk(dZn, Wn, x, gamma, beta, dgamma, dbeta, mask)
+        B, Hn = dZn.shape
+        H = Wn.shape[1]
+        assert Wn.shape[0] == Hn and tuple(x.shape) == (B, H)
+        dX = self.empty(B, H)
+        self._ck(self.lib.dlmi_fc_bwd_dx_norm_act_bwd(
+            self.ctx, ctypes.byref(desc), c_sz(B), c_sz(Hn), c_sz(H), _p(dZn), _p(Wn), _p(x), _p(gamma), _p(beta),
+            _p(mask), _p(stats["mean"]), _p(stats["std"]), _p(stats["r"]), _p(stats["d"]), _p(dgamma), _p(dbeta), _p(dX)))
         return dX
 
     def fused_infer(self, desc, x, gamma, beta, mov_mean, mov_std, out=None):

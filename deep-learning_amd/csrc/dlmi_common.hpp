@@ -28,6 +28,7 @@ struct dlmi_tuning {
   int fold_fwd = 1;
   int fold_bwd = 2;
   size_t fold_fwd_max_elements = size_t(1) << 20;
+  int fc_narrow = 1;              // layers of at most 16 units on a mini-batch run the narrow-layer kernels (fc_small.hip)
   int norm_small = 1;             // mini-batches (at most 256 rows, 2^20 elements) run the one-launch small-batch kernels
 };
 
@@ -122,6 +123,20 @@ size_t norm_scratch_bytes(dlmi_ctx const *ctx, size_t H);
 int panel_init(dlmi_ctx *ctx);
 int panel_check(dlmi_ctx *ctx);
 size_t panel_scratch_bytes(size_t H);
+// Narrow layers on a mini-batch (fc_small.hip).  narrow_fc_fwd: Z = X W^T + bias and, with Q != nullptr,
+// Q = softmax(Z), one launch; call only when narrow_fc_fwd_eligible.  narrow_dw_try: dW and db in one launch;
+// returns 1 when launched, 0 when the shape does not qualify, < 0 on failure.
+bool narrow_fc_fwd_eligible(dlmi_ctx const *ctx, size_t B, size_t H);
+int narrow_fc_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, float const *W, float const *bias, float *Z,
+                  float *Q);
+int narrow_dw_try(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float *dW, float *db,
+                  int accumulate);
+// The fused backward of dlmi_fused_norm_act_bwd whose upstream gradient dY is still `nslices` partial products
+// [nslices][B][H] (split-K slices of the dX product above it); small-batch shapes only.
+int fused_bwd_from_slices(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
+                          float const *gamma, float const *beta, uint8_t const *mask, float const *mean,
+                          float const *stdv, float const *r, float const *d, float const *slices, unsigned nslices,
+                          float *dgamma, float *dbeta, float *dX);
 // acc[0] += sum_b pairs[2b], acc[1] += sum_b pairs[2b+1] over nblocks per-block pairs, in a fixed order.
 int sum_block_pairs(dlmi_ctx *ctx, double const *pairs, unsigned nblocks, double *acc);
 }  // namespace dlmi

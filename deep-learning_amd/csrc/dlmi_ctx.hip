@@ -79,6 +79,7 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
   t.fold_fwd = env_level("DLMI_NORM_FOLD_FWD", t.fold_fwd);
   t.fold_bwd = env_level("DLMI_NORM_FOLD_BWD", t.fold_bwd);
   t.norm_small = env_flag("DLMI_NORM_SMALL", t.norm_small);
+  t.fc_narrow = env_flag("DLMI_FC_NARROW", t.fc_narrow);
   int rc = dlmi_scratch_reserve(ctx, size_t(16) << 20);
   if (rc == DLMI_OK) rc = dlmi::static_scratch_init(ctx);
   if (rc == DLMI_OK) rc = dlmi::panel_init(ctx);

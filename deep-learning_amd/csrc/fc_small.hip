@@ -1,0 +1,185 @@
+// Fully-connected products of a NARROW layer on a mini-batch (at most 16 units: the 10-way output layer of
+// the reference's own example network).  A 128 x 10 output is one sixth of one MFMA tile; the tiled GEMM
+// needs a K split, a slice reduction and then separate softmax / bias-gradient launches around it, each
+// of which costs more in launch latency than in work.  Here:
+//   k_narrow_fc_fwd  Z = X W^T + b, optionally Q = softmax(Z), one wavefront per row
+//                    (fwp_st.cpp:4498-4555, 4796-4828);
+//   k_narrow_dw      dW (+)= dZ^T X and db (+)= column sums of dZ in one launch, a workgroup per 8 columns
+//                    of X for all rows (update_derivative_fwp_st.cpp:246-302).
+// Sums run in a fixed order (no float atomics).  Citations: /root/reference/lib/deep-learning/v1/learner/.
+#include <hip/hip_runtime.h>
+
+#include "dlmi_common.hpp"
+
+namespace dlmi {
+namespace {
+
+constexpr int kNarrowMaxUnits = 16;
+constexpr size_t kNarrowMaxRowsFwd = 1024;
+constexpr size_t kNarrowMaxRowsDw = 256;
+constexpr int kNarrowThreads = 256;
+constexpr int kNarrowFwdThreads = 64;  // one row per workgroup: a mini-batch spreads over as many CUs as it has rows
+
+typedef float nv4f __attribute__((ext_vector_type(4)));
+
+// One wavefront per row.  Lane l takes k = 4l .. 4l+3, then + 256, ... (16-byte loads, coalesced over X's row
+// and over each row of W; VEC = 1: k = l, l + 64, ... for rows that are not 16-byte aligned); all loads of a
+// step are independent, so they are in flight together.  The 64 partial sums of an output are combined with the
+// xor-shuffle tree; lane o then holds output o.  H is a template parameter so that the loops over the outputs
+// unroll without predicates.
+template <int H, int VEC, bool SOFTMAX>
+__global__ __launch_bounds__(kNarrowFwdThreads) void k_narrow_fc_fwd(float const *__restrict__ X, float const *__restrict__ W,
+                                                                   float const *__restrict__ bias, float *__restrict__ Z,
+                                                                   float *__restrict__ Q, size_t B, size_t K) {
+  int const lane = threadIdx.x & 63;
+  size_t const row = static_cast<size_t>(blockIdx.x) * (kNarrowFwdThreads / 64) + threadIdx.x / 64;
+  if (row >= B) return;
+  float acc[H];
+#pragma unroll
+  for (int o = 0; o < H; ++o) acc[o] = 0.0f;
+  float const *xr = X + row * K;
+  if constexpr (VEC == 4) {
+#pragma unroll 2
+    for (size_t k = static_cast<size_t>(lane) * 4; k < K; k += 256) {
+      nv4f const xv = *reinterpret_cast<nv4f const *>(xr + k);
+      nv4f w[H];
+#pragma unroll
+      for (int o = 0; o < H; ++o) w[o] = *reinterpret_cast<nv4f const *>(W + static_cast<size_t>(o) * K + k);
+#pragma unroll
+      for (int o = 0; o < H; ++o) {
+        acc[o] += xv[0] * w[o][0];
+        acc[o] += xv[1] * w[o][1];
+        acc[o] += xv[2] * w[o][2];
+        acc[o] += xv[3] * w[o][3];
+      }
+    }
+  } else {
+#pragma unroll 4
+    for (size_t k = lane; k < K; k += 64) {
+      float const xv = xr[k];
+      float w[H];
+#pragma unroll
+      for (int o = 0; o < H; ++o) w[o] = W[static_cast<size_t>(o) * K + k];
+#pragma unroll
+      for (int o = 0; o < H; ++o) acc[o] += xv * w[o];
+    }
+  }
+  float z = 0.0f;
+#pragma unroll
+  for (int o = 0; o < H; ++o) {
+    float s = acc[o];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if (lane == o) z = s;
+  }
+  bool const mine = lane < H;
+  if (mine) {
+    if (bias != nullptr) z += bias[lane];
+    Z[row * H + lane] = z;
+  }
+  if constexpr (SOFTMAX) {
+    // the arithmetic of the stand-alone softmax leaf: max, exp(x - max), sum over the same tree, times 1 / sum
+    float mx = mine ? z : -3.402823466e+38f;
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float const e = mine ? expf(z - mx) : 0.0f;
+    float s = e;
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    s = 1.0f / s;
+    if (mine) Q[row * H + lane] = e * s;
+  }
+}
+
+constexpr int kDwCols = 8, kDwGroups = 32;
+
+// dW[o][j] (+)= sum_b dZ[b][o] X[b][j], db[o] (+)= sum_b dZ[b][o].  B <= 256, H <= 16.
+__global__ __launch_bounds__(kNarrowThreads) void k_narrow_dw(float const *__restrict__ X, float const *__restrict__ dZ,
+                                                               float *__restrict__ dW, float *__restrict__ db, size_t B,
+                                                               size_t K, int H, int accumulate) {
+  constexpr int kStride = kNarrowMaxUnits + 1;
+  __shared__ float dz[kNarrowMaxRowsDw * kStride];
+  __shared__ float red[kDwGroups][kNarrowMaxUnits][kDwCols];
+  for (size_t i = threadIdx.x; i < B * static_cast<size_t>(H); i += kNarrowThreads)
+    dz[(i / H) * kStride + (i % H)] = dZ[i];
+  __syncthreads();
+  int const c = threadIdx.x % kDwCols, rg = threadIdx.x / kDwCols;
+  size_t const col = static_cast<size_t>(blockIdx.x) * kDwCols + c;
+  float acc[kNarrowMaxUnits];
+#pragma unroll
+  for (int o = 0; o < kNarrowMaxUnits; ++o) acc[o] = 0.0f;
+  if (col < K) {
+    for (size_t b = rg; b < B; b += kDwGroups) {
+      float const xv = X[b * K + col];
+#pragma unroll
+      for (int o = 0; o < kNarrowMaxUnits; ++o)
+        if (o < H) acc[o] += dz[b * kStride + o] * xv;
+    }
+  }
+#pragma unroll
+  for (int o = 0; o < kNarrowMaxUnits; ++o) red[rg][o][c] = acc[o];
+  __syncthreads();
+  if (static_cast<int>(threadIdx.x) < H * kDwCols) {
+    int const o = threadIdx.x / kDwCols, cc = threadIdx.x % kDwCols;
+    size_t const j = static_cast<size_t>(blockIdx.x) * kDwCols + cc;
+    if (j < K) {
+      float t = 0.0f;
+#pragma unroll
+      for (int g = 0; g < kDwGroups; ++g) t += red[g][o][cc];
+      float *dst = dW + static_cast<size_t>(o) * K + j;
+      *dst = accumulate ? *dst + t : t;
+    }
+  }
+  if (db != nullptr && blockIdx.x == 0 && static_cast<int>(threadIdx.x) >= kNarrowThreads - H) {
+    int const o = kNarrowThreads - 1 - static_cast<int>(threadIdx.x);
+    float t = 0.0f;
+    for (size_t b = 0; b < B; ++b) t += dz[b * kStride + o];
+    db[o] = accumulate ? db[o] + t : t;
+  }
+}
+
+}  // namespace
+
+bool narrow_fc_fwd_eligible(dlmi_ctx const *ctx, size_t B, size_t H) {
+  return ctx->tune.fc_narrow != 0 && H <= static_cast<size_t>(kNarrowMaxUnits) && B <= kNarrowMaxRowsFwd;
+}
+
+template <int H>
+static void launch_narrow_fwd(dlmi_ctx *ctx, dim3 grid, bool vec, float const *X, float const *W, float const *bias, float *Z,
+                              float *Q, size_t B, size_t K) {
+  dim3 const block(kNarrowFwdThreads);
+  if (Q != nullptr) {
+    if (vec) hipLaunchKernelGGL((k_narrow_fc_fwd<H, 4, true>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K);
+    else hipLaunchKernelGGL((k_narrow_fc_fwd<H, 1, true>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K);
+  } else {
+    if (vec) hipLaunchKernelGGL((k_narrow_fc_fwd<H, 4, false>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K);
+    else hipLaunchKernelGGL((k_narrow_fc_fwd<H, 1, false>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K);
+  }
+}
+
+int narrow_fc_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, float const *W, float const *bias, float *Z,
+                  float *Q) {
+  dim3 const grid(static_cast<unsigned>(dlmi_ceil_div(B, static_cast<size_t>(kNarrowFwdThreads / 64))));
+  bool const vec = K % 4 == 0 && dlmi_aligned16(X) && dlmi_aligned16(W);
+  switch (H) {
+#define DLMI_NARROW_CASE(n) case n: launch_narrow_fwd<n>(ctx, grid, vec, X, W, bias, Z, Q, B, K); break;
+    DLMI_NARROW_CASE(1) DLMI_NARROW_CASE(2) DLMI_NARROW_CASE(3) DLMI_NARROW_CASE(4) DLMI_NARROW_CASE(5)
+    DLMI_NARROW_CASE(6) DLMI_NARROW_CASE(7) DLMI_NARROW_CASE(8) DLMI_NARROW_CASE(9) DLMI_NARROW_CASE(10)
+    DLMI_NARROW_CASE(11) DLMI_NARROW_CASE(12) DLMI_NARROW_CASE(13) DLMI_NARROW_CASE(14) DLMI_NARROW_CASE(15)
+    DLMI_NARROW_CASE(16)
+#undef DLMI_NARROW_CASE
+    default: return dlmi_fail(ctx, DLMI_E_INVALID, "narrow_fc_fwd: %zu units", H);
+  }
+  DLMI_LAUNCH_CHECK(ctx, "k_narrow_fc_fwd");
+  return DLMI_OK;
+}
+
+int narrow_dw_try(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float *dW, float *db,
+                  int accumulate) {
+  if (ctx->tune.fc_narrow == 0 || H > static_cast<size_t>(kNarrowMaxUnits) || B > kNarrowMaxRowsDw) return 0;
+  dim3 const grid(static_cast<unsigned>(dlmi_ceil_div(K, static_cast<size_t>(kDwCols))));
+  hipLaunchKernelGGL(k_narrow_dw, grid, dim3(kNarrowThreads), 0, ctx->stream, Xin, dZ, dW, db, B, K, static_cast<int>(H),
+                     accumulate);
+  DLMI_LAUNCH_CHECK(ctx, "k_narrow_dw");
+  return 1;
+}
+
+}  // namespace dlmi

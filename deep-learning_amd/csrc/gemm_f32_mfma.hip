@@ -603,7 +603,18 @@ int dlmi_fc_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, flo
   if (ctx == nullptr) return DLMI_E_INVALID;
   DLMI_REQUIRE(ctx, X && W && Z, "null pointer");
   DLMI_REQUIRE(ctx, B > 0 && K > 0 && H > 0, "empty operand");
+  if (narrow_fc_fwd_eligible(ctx, B, H)) return narrow_fc_fwd(ctx, B, K, H, X, W, bias, Z, nullptr);
   return gemm<true, true>(ctx, B, H, K, X, K, W, K, Z, bias, 0);
+}
+
+int dlmi_fc_softmax_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, float const *W, float const *bias,
+                        float *Z, float *Q) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, X && W && Z && Q, "null pointer");
+  DLMI_REQUIRE(ctx, B > 0 && K > 0 && H > 0, "empty operand");
+  if (narrow_fc_fwd_eligible(ctx, B, H)) return narrow_fc_fwd(ctx, B, K, H, X, W, bias, Z, Q);
+  int const rc = gemm<true, true>(ctx, B, H, K, X, K, W, K, Z, bias, 0);
+  return rc != DLMI_OK ? rc : dlmi_softmax_fwd(ctx, B, H, Z, Q);
 }
 
 static int fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t K, size_t H, float const *X,
@@ -652,11 +663,31 @@ int dlmi_fc_bwd_dx(dlmi_ctx *ctx, size_t B, size_t Hn, size_t H, float const *dZ
   return gemm<true, false>(ctx, B, H, Hn, dZn, Hn, Wn, H, dY, nullptr, accumulate);
 }
 
+int dlmi_fc_bwd_dx_norm_act_bwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t Hn, size_t H,
+                                float const *dZn, float const *Wn, float const *x, float const *gamma, float const *beta,
+                                uint8_t const *mask, float const *mean, float const *stdv, float const *r, float const *d,
+                                float *dgamma, float *dbeta, float *dX) {
+  if (ctx == nullptr || desc == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, dZn && Wn && dX, "null pointer");
+  DLMI_REQUIRE(ctx, B > 0 && Hn > 0 && H > 0, "empty operand");
+  // a mini-batch: the normalization kernel owns whole columns and adds the K slices of dY = dZn . Wn itself
+  unsigned slices = 0;
+  bool const defer = small_norm_eligible(ctx, B, H);
+  int rc = gemm<true, false>(ctx, B, H, Hn, dZn, Hn, Wn, H, dX, nullptr, 0, nullptr, defer ? &slices : nullptr);
+  if (rc != DLMI_OK) return rc;
+  if (slices != 0)
+    return fused_bwd_from_slices(ctx, desc, B, H, x, gamma, beta, mask, mean, stdv, r, d,
+                                 reinterpret_cast<float const *>(dlmi_scratch_data(ctx)), slices, dgamma, dbeta, dX);
+  return dlmi_fused_norm_act_bwd(ctx, desc, B, H, x, gamma, beta, mask, mean, stdv, r, d, dX, dgamma, dbeta, dX);
+}
+
 int dlmi_fc_bwd_dw(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float *dW,
                    float *db, int accumulate) {
   if (ctx == nullptr) return DLMI_E_INVALID;
   DLMI_REQUIRE(ctx, Xin && dZ && dW, "null pointer");
   DLMI_REQUIRE(ctx, B > 0 && K > 0 && H > 0, "empty operand");
+  // a narrow layer on a mini-batch: dW and db in one launch
+  if (int const took = narrow_dw_try(ctx, B, K, H, Xin, dZ, dW, db, accumulate); took != 0) return took < 0 ? took : DLMI_OK;
   int rc = gemm<false, false>(ctx, H, K, B, dZ, H, Xin, K, dW, nullptr, accumulate);
   if (rc != DLMI_OK || db == nullptr) return rc;
   // db[h] (+)= sum_b dZ[b,h] (update_derivative_fwp_st.cpp:283-302)

@@ -1165,6 +1165,26 @@ int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
   return run_fwd_train(ctx, sv, B, H, c);
 }
 
+int fused_bwd_from_slices(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
+                          float const *gamma, float const *beta, uint8_t const *mask, float const *mean,
+                          float const *stdv, float const *r, float const *d, float const *slices, unsigned nslices,
+                          float *dgamma, float *dbeta, float *dX) {
+  int rc = check_desc(ctx, desc, mask);
+  if (rc != DLMI_OK) return rc;
+  DLMI_REQUIRE(ctx, x && gamma && beta && mean && stdv && r && d && slices && nslices > 0 && dgamma && dbeta && dX,
+               "null pointer");
+  BwdCall c;
+  c.act = desc->act; c.xhat_given = false; c.drop_mode = drop_mode_of(desc);
+  c.drop_bwd_masked = desc->dropout_bwd == DLMI_DROP_BWD_MASKED ? 1 : 0;
+  c.drop_scale = drop_scale_of(desc);
+  c.x = x; c.gamma = gamma; c.beta = beta; c.mean = mean; c.stdv = stdv; c.r = r; c.d = d; c.xhat = nullptr;
+  c.dY = nullptr; c.mask = mask; c.dy_slices = slices; c.nslices = nslices;
+  c.dgamma = dgamma; c.dbeta = dbeta; c.dmean = nullptr; c.dstd = nullptr; c.dX = dX;
+  int const took = small_bwd_try(ctx, B, H, c);
+  if (took == 0) return dlmi_fail(ctx, DLMI_E_INVALID, "fused_bwd_from_slices: not a small-batch shape");
+  return took < 0 ? took : DLMI_OK;
+}
+
 int column_sums(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *out, int accumulate) {
   if (int const took = small_colsum_try(ctx, B, H, x, out, accumulate); took != 0) return took < 0 ? took : DLMI_OK;
   ScratchView sv{};

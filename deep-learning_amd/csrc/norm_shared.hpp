@@ -117,6 +117,10 @@ struct BwdCall {
   uint8_t const *mask;
   float *dgamma, *dbeta, *dmean, *dstd, *dX;
   bool accumulate = false;  // dX += instead of dX =
+  // dY not formed yet: it is the sum of `nslices` partial products [nslices][B][H], added in slice order by
+  // the small-batch kernel (the only one that takes them); dY is unused then
+  float const *dy_slices = nullptr;
+  unsigned nslices = 0;
 };
 
 // The single-launch panel kernels (norm_panel_fwd.hip, norm_panel_bwd.hip).  Return 1 when the call was

@@ -118,6 +118,8 @@ __global__ __launch_bounds__(kSmallThreads) void k_small_fwd(SmallFwdArgs a) {
 
 struct SmallBwdArgs {
   float const *x, *dY, *gamma, *beta, *mean, *stdv, *r, *d;
+  float const *dy_slices;  // [nslices][B][H] whose sum is dY, or nullptr
+  unsigned nslices;
   uint8_t const *mask;
   float *dgamma, *dbeta, *dX;
   size_t B, H;
@@ -164,8 +166,19 @@ __global__ __launch_bounds__(kSmallThreads) void k_small_bwd(SmallBwdArgs a) {
     mv[i] = mk;
     if (ok[i]) {
       xv[i] = a.x[off];
-      dy[i] = a.dY[off];
+      if (a.dy_slices == nullptr) dy[i] = a.dY[off];
       if (a.drop_mode == kDropElem) mv[i] = a.mask[off];
+    }
+  }
+  if (a.dy_slices != nullptr) {
+    size_t const plane = a.B * a.H;
+    for (unsigned s = 0; s < a.nslices; ++s) {
+      float t[RPT];
+#pragma unroll
+      for (int i = 0; i < RPT; ++i)
+        t[i] = ok[i] ? a.dy_slices[s * plane + static_cast<size_t>(rg + kSmallGroups * i) * a.H + col] : 0.0f;
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) dy[i] += t[i];
     }
   }
 #pragma unroll
@@ -276,8 +289,12 @@ int small_fwd_try(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c) {
 }
 
 int small_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c) {
-  if (!small_norm_eligible(ctx, B, H) || c.xhat_given || c.dmean != nullptr || c.dstd != nullptr) return 0;
+  if (!small_norm_eligible(ctx, B, H) || c.xhat_given || c.dmean != nullptr || c.dstd != nullptr) {
+    if (c.dy_slices != nullptr) return dlmi_fail(ctx, DLMI_E_INVALID, "small-batch backward: K slices given for a call it cannot take");
+    return 0;
+  }
   SmallBwdArgs a;
+  a.dy_slices = c.dy_slices; a.nslices = c.nslices;
   a.x = c.x; a.dY = c.dY; a.gamma = c.gamma; a.beta = c.beta; a.mean = c.mean; a.stdv = c.stdv; a.r = c.r; a.d = c.d;
   a.mask = c.mask; a.dgamma = c.dgamma; a.dbeta = c.dbeta; a.dX = c.dX;
   a.B = B; a.H = H;

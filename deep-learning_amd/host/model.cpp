@@ -909,6 +909,12 @@ void Model::forward_layers(size_t const B, size_t const end_layer) {
     bool const norm_after = l.Use__Normalization() && !l.use_layer_normalization_before_activation;
     // the GEMM epilogue takes the batch statistics when the normalization follows the GEMM directly
     bool const fused_fc_norm = l.Use__Normalization() && training && !norm_after;
+    // a softmax layer without normalization or dropout (the output layer): product, bias and softmax in one call
+    bool const fused_fc_softmax = softmax && !l.Use__Normalization() && !l.Use__Dropout();
+    if (fused_fc_softmax) {
+      if (dlmi_fc_softmax_fwd(ctx, B, K, H, in, W, bias, l.d_summations, l.d_outputs) != DLMI_OK) { fail("forward_pass: dlmi_fc_softmax_fwd"); return; }
+      continue;
+    }
     if (!fused_fc_norm && dlmi_fc_fwd(ctx, B, K, H, in, W, bias, l.d_summations) != DLMI_OK) { fail("forward_pass: dlmi_fc_fwd"); return; }
     int rc = DLMI_OK;
     if (norm_after) {
@@ -1238,6 +1244,7 @@ void Model::backward_pass(size_t const B) {
   // the entry above) into dZ in place, then hands dZ . W to the entry it reads;
   // a residual block is unwound as a whole.  The gradient with respect to the
   // network input is never formed.
+  bool gradient_done = false;  // this layer's dZ was already formed together with the product of the layer above
   for (size_t li = total_layers - 1; li >= 1; --li) {
     Layer &l = ptr_array_layers[li];
     if (l.in_block) {
@@ -1248,7 +1255,9 @@ void Model::backward_pass(size_t const B) {
     }
     size_t const H = l.n_out;
     int rc = DLMI_OK;
-    if (li + 1 == total_layers) {
+    if (gradient_done) {
+      gradient_done = false;
+    } else if (li + 1 == total_layers) {
       // the output layer's dZ is the seed gradient of compute_error()
     } else if (l.Use__Normalization() && !l.use_layer_normalization_before_activation) {
       // bwp_st.cpp:559-606, 619-632: normalization backward on the activation
@@ -1276,11 +1285,27 @@ void Model::backward_pass(size_t const B) {
     }
     if (rc != DLMI_OK) { fail("backward_pass: layer gradient"); return; }
     // dY = dZ . W, written straight over the (would-be zeroed) buffer of the entry this layer reads
-    if (l.feed_index != 0 &&
-        dlmi_fc_bwd_dx(ctx, B, H, l.n_inp, l.d_errors, impl_->d_params + l.first_connection_index,
-                       ptr_array_layers[l.feed_index].d_errors, 0) != DLMI_OK) {
-      fail("backward_pass: dlmi_fc_bwd_dx");
-      return;
+    if (l.feed_index != 0) {
+      Layer &f = ptr_array_layers[l.feed_index];
+      // the entry below is a plain layer normalized before its activation: its gradient step in the same call
+      // (on a mini-batch the normalization kernel then adds the K slices of the product itself)
+      bool const fuse = l.feed_index + 1 == li && f.type_layer == LAYER::FULLY_CONNECTED && !f.in_block &&
+                        f.Use__Normalization() && f.use_layer_normalization_before_activation;
+      if (fuse) {
+        dlmi_fused_desc d = make_desc(*this, f);
+        if (type_state_propagation != PROPAGATION::TRAINING) d.dropout = DLMI_DROP_NONE;
+        rc = dlmi_fc_bwd_dx_norm_act_bwd(ctx, &d, B, H, l.n_inp, l.d_errors, impl_->d_params + l.first_connection_index,
+                                         f.d_summations, impl_->d_params + f.scale_index, impl_->d_params + f.shift_index,
+                                         f.d_mask, f.d_mean, f.d_std, f.d_r, f.d_d, impl_->d_dparams + f.scale_index,
+                                         impl_->d_dparams + f.shift_index, f.d_errors);
+        gradient_done = true;
+      } else {
+        rc = dlmi_fc_bwd_dx(ctx, B, H, l.n_inp, l.d_errors, impl_->d_params + l.first_connection_index, f.d_errors, 0);
+      }
+      if (rc != DLMI_OK) {
+        fail("backward_pass: dlmi_fc_bwd_dx");
+        return;
+      }
     }
     if (li == 1) break;
   }

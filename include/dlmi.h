@@ -294,6 +294,25 @@ int dlmi_fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, s
                          uint8_t const *mask, float *Z, float *mean, float *std, float *mov_mean,
                          float *mov_std, float *r, float *d, float *y);
 
+/* Z = X W^T + bias and Q = softmax(Z) row by row: the forward of a softmax output layer
+ * (Forward_Pass__FC__Loop + Forward_Pass__Bias__Loop + Forward_Pass__FC_AF__Softmax__Loop,
+ * fwp_st.cpp:4498-4555, 4796-4828) in one call.  Z, Q [B,H].  A layer of at most 16 units on at most
+ * 1024 rows (the reference's 10-way output on a mini-batch) runs as ONE launch, a wavefront per row;
+ * anything else is dlmi_fc_fwd followed by dlmi_softmax_fwd. */
+int dlmi_fc_softmax_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, float const *W,
+                        float const *bias, float *Z, float *Q);
+
+/* Backward of a normalized layer together with the product that brings its upstream gradient:
+ * dY = dZn . Wn (Backward_Pass__FC__Loop, bwp_st.cpp:1009-1045; dZn [B,Hn], Wn [Hn][H]), then
+ * dlmi_fused_norm_act_bwd on dY (bwp_st.cpp:1177-1209, 1284-1366, 1447-1532), result in dX [B,H]
+ * (dgamma, dbeta accumulate).  On a mini-batch (at most 256 rows) whose product runs split over K the
+ * normalization kernel adds the K slices itself and dY is never written; otherwise the two calls run
+ * one after the other with dX as the buffer between them. */
+int dlmi_fc_bwd_dx_norm_act_bwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t Hn, size_t H,
+                                float const *dZn, float const *Wn, float const *x, float const *gamma,
+                                float const *beta, uint8_t const *mask, float const *mean, float const *std,
+                                float const *r, float const *d, float *dgamma, float *dbeta, float *dX);
+
 /* The two forwards above with the identity shortcut of a residual block in the
  * same pass: y = shortcut + (activation output after dropout), shortcut [B,H]
  * (y may alias it).  Saves the separate add and its 12 B/element.  The sum is

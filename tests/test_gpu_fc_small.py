@@ -1,0 +1,116 @@
+"""The narrow-layer kernels (a layer of at most 16 units on a mini-batch: one launch for product + bias
++ softmax, one launch for dW + db) and the backward that takes its upstream gradient as K slices, against
+the tiled-GEMM path of the same library (a context created with DLMI_FC_NARROW=0 / DLMI_NORM_SMALL=0 is the
+twin) and against float64."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_close
+from oracle.binding import ACT
+from test_gpu_norm_panel import dev, make, run_fwd
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def twins(pkg):
+    os.environ["DLMI_FC_NARROW"] = "0"
+    os.environ["DLMI_NORM_SMALL"] = "0"
+    try:
+        plain = pkg.Dlmi(0)
+    finally:
+        del os.environ["DLMI_FC_NARROW"]
+        del os.environ["DLMI_NORM_SMALL"]
+    fast = pkg.Dlmi(0)
+    yield fast, plain
+    fast.close()
+    plain.close()
+
+
+def softmax64(z):
+    e = np.exp(z - z.max(1, keepdims=True))
+    return e / e.sum(1, keepdims=True)
+
+
+@pytest.mark.parametrize("B,K,H", [(128, 512, 10), (1000, 33, 16), (7, 5, 1), (1024, 784, 3), (64, 1, 16), (3, 1000, 2)])
+def test_narrow_forward_with_softmax(twins, pkg, B, K, H):
+    fast, plain = twins
+    rng = np.random.default_rng(B + K + H)
+    X = rng.standard_normal((B, K)).astype(np.float32)
+    W = (rng.standard_normal((H, K)) / np.sqrt(K)).astype(np.float32)
+    b = rng.uniform(-.5, .5, H).astype(np.float32)
+    z64 = X.astype(np.float64) @ W.astype(np.float64).T + b
+    for bias in (b, None):
+        exact = z64 if bias is not None else z64 - b
+        Z, Q = fast.fc_softmax_fwd(dev(X), dev(W), None if bias is None else dev(bias))
+        Zp, Qp = plain.fc_softmax_fwd(dev(X), dev(W), None if bias is None else dev(bias))
+        Zf = fast.fc_fwd(dev(X), dev(W), None if bias is None else dev(bias))
+        assert_close(Z.cpu().numpy(), exact, 1e-4, "Z vs float64", floor=1e-3)
+        assert_close(Q.cpu().numpy(), softmax64(exact), 1e-4, "softmax vs float64")
+        assert_close(Z.cpu().numpy(), Zp.cpu().numpy(), 1e-4, "Z vs tiled GEMM", floor=1e-3)
+        assert_close(Q.cpu().numpy(), Qp.cpu().numpy(), 1e-4, "softmax vs GEMM + softmax leaf")
+        assert torch.equal(Z, Zf), "dlmi_fc_fwd takes the same kernel"
+        # the softmax is the leaf's arithmetic on the same Z
+        assert torch.equal(Q, fast.softmax_fwd(Z))
+        assert np.allclose(Q.cpu().numpy().sum(1), 1.0, atol=1e-6)
+
+
+def test_wider_or_taller_layers_take_the_tiled_path(twins, pkg):
+    fast, plain = twins
+    rng = np.random.default_rng(4)
+    for B, K, H in [(128, 64, 17), (1025, 64, 10)]:
+        X, W = rng.standard_normal((B, K)).astype(np.float32), rng.standard_normal((H, K)).astype(np.float32)
+        Z, Q = fast.fc_softmax_fwd(dev(X), dev(W))
+        Zp, Qp = plain.fc_softmax_fwd(dev(X), dev(W))
+        assert torch.equal(Z, Zp) and torch.equal(Q, Qp)
+
+
+@pytest.mark.parametrize("B,K,H", [(128, 512, 10), (256, 100, 16), (5, 3, 2), (77, 1000, 1), (200, 9, 13)])
+def test_narrow_weight_and_bias_gradient(twins, pkg, B, K, H):
+    fast, plain = twins
+    rng = np.random.default_rng(B * K + H)
+    X = rng.standard_normal((B, K)).astype(np.float32)
+    dZ = rng.standard_normal((B, H)).astype(np.float32)
+    dW64 = dZ.astype(np.float64).T @ X.astype(np.float64)
+    db64 = dZ.astype(np.float64).sum(0)
+    dW, db = fast.fc_bwd_dw(dev(X), dev(dZ), with_bias=True)
+    dWp, dbp = plain.fc_bwd_dw(dev(X), dev(dZ), with_bias=True)
+    assert_close(dW.cpu().numpy(), dW64, 1e-4, "dW vs float64", floor=1e-3)
+    assert_close(db.cpu().numpy(), db64, 1e-5, "db vs float64", floor=1.0)
+    assert_close(dW.cpu().numpy(), dWp.cpu().numpy(), 1e-4, "dW vs tiled GEMM", floor=1e-3)
+    assert_close(db.cpu().numpy(), dbp.cpu().numpy(), 1e-5, "db vs column-sum kernels", floor=1.0)
+    # accumulating on top, and without a bias gradient
+    fast.fc_bwd_dw(dev(X), dev(dZ), dW=dW, db=db, accumulate=True)
+    assert_close(dW.cpu().numpy(), 2 * dW64, 1e-4, "dW accumulated", floor=1e-3)
+    assert_close(db.cpu().numpy(), 2 * db64, 1e-5, "db accumulated", floor=1.0)
+    dW2, none = fast.fc_bwd_dw(dev(X), dev(dZ))
+    assert none is None
+    assert_close(dW2.cpu().numpy(), dW64, 1e-4, "dW alone", floor=1e-3)
+
+
+@pytest.mark.parametrize("B,Hn,H,act,drop", [
+    (128, 512, 512, "RELU", "NONE"),                  # runs split over K: the normalization kernel adds the slices
+    (128, 10, 512, "RELU", "NONE"),                   # K = 10: no split, the two steps run one after the other
+    (200, 300, 36, "ELU", "BERNOULLI_INVERTED"),
+    (256, 1024, 64, "TANH", "BERNOULLI"),
+    (512, 256, 256, "SELU", "NONE"),                  # more rows than the small-batch kernels take
+])
+def test_backward_with_the_product_above_it(twins, pkg, B, Hn, H, act, drop):
+    """dlmi_fc_bwd_dx_norm_act_bwd against dlmi_fc_bwd_dx followed by dlmi_fused_norm_act_bwd on the twin."""
+    fast, plain = twins
+    d = make(B, H, B + Hn + H)
+    rng = np.random.default_rng(B + H)
+    dZn = rng.standard_normal((B, Hn)).astype(np.float32)
+    Wn = (rng.standard_normal((Hn, H)) / np.sqrt(Hn)).astype(np.float32)
+    _, desc, mask, st = run_fwd(plain, pkg, d, act, drop, False, False)
+    dg, db = torch.full((H,), 0.25, device="cuda"), torch.full((H,), -0.5, device="cuda")
+    dX = fast.fc_bwd_dx_fused_bwd(desc, dev(dZn), dev(Wn), dev(d["x"]), dev(d["gamma"]), dev(d["beta"]), st, dg, db, mask=mask)
+    dgp, dbp = torch.full((H,), 0.25, device="cuda"), torch.full((H,), -0.5, device="cuda")
+    dY = plain.fc_bwd_dx(dev(dZn), dev(Wn))
+    dXp = plain.fused_bwd(desc, dev(d["x"]), dev(d["gamma"]), dev(d["beta"]), st, dY, dgp, dbp, mask=mask)
+    assert_close(dX.cpu().numpy(), dXp.cpu().numpy(), 1e-4, "dX", floor=1.0)
+    assert_close(dg.cpu().numpy(), dgp.cpu().numpy(), 1e-4, "dgamma", floor=1.0)
+    assert_close(db.cpu().numpy(), dbp.cpu().numpy(), 1e-4, "dbeta", floor=1.0)
