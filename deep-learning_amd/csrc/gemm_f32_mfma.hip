@@ -456,20 +456,24 @@ static GemmPlan plan_gemm(dlmi_ctx const *ctx, size_t M, size_t N, size_t K) {
   static TileCfg const cfgs[] = {{128, 128, 16}, {256, 128, 16}, {256, 256, 16}, {64, 64, 16}};
   int choice = tile_choice();
   if (choice < 0 || choice >= static_cast<int>(sizeof(cfgs) / sizeof(cfgs[0]))) {
-    // default: the shape with the smallest estimated time = rounds of workgroups
-    // over the CUs x work of one workgroup x workgroups sharing a CU / measured
-    // relative efficiency of the shape (256 x 256 runs one workgroup per CU,
-    // 128-wide shapes two, 64 x 64 four).  A small output picks small tiles: a
-    // workgroup's time is its own MFMA count as long as it has a CU to itself.
+    // default: the shape with the smallest estimated time.  Main loop: rounds of workgroups over the CUs x
+    // work of one workgroup x workgroups sharing a CU / measured relative efficiency of the shape (256 x 256
+    // runs one workgroup per CU, 128-wide shapes two, 64 x 64 four).  Epilogue: storing a tile costs about as
+    // much as 32 k of its main loop, and it is exposed once per CU - workgroups that share a CU or follow each
+    // other on it store while another one multiplies.  (Measured on 65536 x 256 x 256, where the 256 x 256 shape
+    // is one round of 16 K tiles: its 7.4 us of stores are 10 % of the launch; 128-wide tiles run 4 % faster.)
+    // A small output picks small tiles: a workgroup's time is its own MFMA count as long as it has a CU to itself.
     static int const per_cu[] = {2, 2, 1, 4};
     static double const eff[] = {0.95, 0.97, 1.0, 0.8};
+    double const epilogue_k = 32.0;
     double best = 0.0;
     for (int c = 0; c < 4; ++c) {
       size_t const tiles = dlmi_ceil_div(M, cfgs[c].bm) * dlmi_ceil_div(N, cfgs[c].bn);
       size_t const slots = static_cast<size_t>(ctx->num_cu) * per_cu[c];
       size_t const rounds = dlmi_ceil_div(tiles, slots);
       size_t const sharing = dlmi_ceil_div(tiles < slots ? tiles : slots, static_cast<size_t>(ctx->num_cu));
-      double const t = static_cast<double>(rounds) * cfgs[c].bm * cfgs[c].bn * sharing / eff[c];
+      double const per_k = static_cast<double>(cfgs[c].bm) * cfgs[c].bn * sharing;
+      double const t = per_k * (static_cast<double>(rounds) * K / eff[c] + epilogue_k / (rounds * sharing));
       if (c == 0 || t < best) {
         best = t;
         choice = c;
