@@ -13,11 +13,13 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
 #include <limits>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "../../include/dlmi_model.hpp"
@@ -31,9 +33,25 @@ struct Model::Impl {
   float *d_params = nullptr;   // [P]
   float *d_dparams = nullptr;  // [P]
   float *d_mov_mean = nullptr, *d_mov_std = nullptr;  // [units]
-  float *d_input = nullptr;    // [batch, n_in]
+  // Rows handed over as host pointers (forward_pass, compute_error) enter through two slots used in turn:
+  // a pinned staging block and a device block each, filled through a copy stream.  While the kernels of one
+  // pass still read their slot, the rows of the next call are gathered and uploaded into the other one.
+  struct RowSlots {
+    float *h[2] = {nullptr, nullptr};  // pinned staging [batch, width]
+    float *d[2] = {nullptr, nullptr};  // device rows   [batch, width]
+    hipEvent_t uploaded[2] = {nullptr, nullptr};  // copy stream: the slot's last upload has finished
+    hipEvent_t fence[2] = {nullptr, nullptr};     // compute stream: all work enqueued before the other slot's call began
+    bool fenced[2] = {false, false};
+    size_t h_floats = 0;
+    int next = 0;
+  };
+  RowSlots in_rows, tgt_rows;
+  hipStream_t up_stream = nullptr;  // copy stream of the two (default priority)
+  bool slots_alloc(RowSlots &s, size_t floats);
+  void slots_free_device(RowSlots &s);
+  void slots_free_all(RowSlots &s);
+  float const *slots_upload(RowSlots &s, size_t B, size_t width, float const *const *rows, char const *what);
   float *d_input_grad = nullptr;  // [batch, n_in], only when a residual block reads the network input
-  float *d_targets = nullptr;  // [batch, n_out]
   double *d_stats = nullptr;   // { loss sum, correct count }
   // optimizer state [P] each: 0 previous delta, 1 first moment, 2 second moment,
   // 3 second moment hat, 4 regularization mask, 5 previous gradient, 6 step sizes (iRPROP+);
@@ -43,8 +61,6 @@ struct Model::Impl {
   size_t n_errors = 0;               // failed calls so far
   size_t n_loss_values = 0;          // outputs whose loss term has been accumulated since reset_loss()
   size_t all_units = 0;              // normalization units of all entries: the slots a normalized model has
-  float *h_stage = nullptr;    // pinned staging for the row-pointer gather
-  size_t h_stage_floats = 0;
   mutable std::vector<float> out_host;  // get_out() cache
   mutable bool out_valid = false;
   size_t out_batch = 0;
@@ -73,6 +89,12 @@ void dev_free(T *&p) {
   if (p != nullptr) (void)hipFree(p);
   p = nullptr;
 }
+// Rows of at least this many bytes are gathered by several host threads, in pieces of kUploadPiece bytes
+// whose copies start while the next pieces are still being gathered.
+constexpr size_t kParallelGatherBytes = size_t(4) << 20;
+constexpr size_t kUploadPiece = size_t(4) << 20;
+constexpr unsigned kGatherThreads = 8;
+
 bool act_on_path(ACTIVATION::TYPE t) {
   switch (t) {
     case ACTIVATION::ELU: case ACTIVATION::ISRLU: case ACTIVATION::LINEAR: case ACTIVATION::LEAKY_RELU:
@@ -83,6 +105,110 @@ bool act_on_path(ACTIVATION::TYPE t) {
   }
 }
 }  // namespace
+
+// ---- host rows -> device, two slots in turn
+bool Model::Impl::slots_alloc(RowSlots &s, size_t const floats) {
+  for (int k = 0; k < 2; ++k) {
+    if (!dev_alloc(&s.d[k], floats, err)) return false;
+    if (s.uploaded[k] == nullptr && !hip_ok(hipEventCreateWithFlags(&s.uploaded[k], hipEventDisableTiming), err, "hipEventCreate")) return false;
+    if (s.fence[k] == nullptr && !hip_ok(hipEventCreateWithFlags(&s.fence[k], hipEventDisableTiming), err, "hipEventCreate")) return false;
+    s.fenced[k] = false;
+  }
+  s.next = 0;
+  if (floats > s.h_floats) {
+    for (int k = 0; k < 2; ++k) {
+      if (s.h[k] != nullptr) (void)hipHostFree(s.h[k]);
+      s.h[k] = nullptr;
+      void *p = nullptr;
+      if (!hip_ok(hipHostMalloc(&p, (floats ? floats : 1) * sizeof(float), hipHostMallocDefault), err, "hipHostMalloc")) {
+        s.h_floats = 0;
+        return false;
+      }
+      s.h[k] = static_cast<float *>(p);
+    }
+    s.h_floats = floats;
+  }
+  return true;
+}
+
+void Model::Impl::slots_free_device(RowSlots &s) {
+  for (int k = 0; k < 2; ++k) dev_free(s.d[k]);
+}
+
+void Model::Impl::slots_free_all(RowSlots &s) {
+  slots_free_device(s);
+  for (int k = 0; k < 2; ++k) {
+    if (s.h[k] != nullptr) (void)hipHostFree(s.h[k]);
+    if (s.uploaded[k] != nullptr) (void)hipEventDestroy(s.uploaded[k]);
+    if (s.fence[k] != nullptr) (void)hipEventDestroy(s.fence[k]);
+  }
+  s = RowSlots();
+}
+
+// Gathers rows[i][0 .. width) into the next slot's staging block (assign_inputs.cpp:22-40 does this gather
+// into the first layer's values) and uploads it; the compute stream waits for the upload, the host does not.
+// Returns the slot's device rows, nullptr on failure.
+float const *Model::Impl::slots_upload(RowSlots &s, size_t const B, size_t const width, float const *const *const rows,
+                                       char const *const what) {
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone) {
+    err = std::string(what) + ": host rows cannot be handed over while the stream is being recorded";
+    return nullptr;
+  }
+  int const k = s.next;
+  s.next ^= 1;
+  float *const h = s.h[k], *const d = s.d[k];
+  // the staging block is free once its last upload has finished (two calls ago: normally long done)
+  if (!hip_ok(hipEventSynchronize(s.uploaded[k]), err, what)) return nullptr;
+  // the device block is free once the pass that read it has finished: that pass had been enqueued in full
+  // when the previous call (the other slot's) began, which is where this slot's fence was recorded
+  if (s.fenced[k] && !hip_ok(hipStreamWaitEvent(up_stream, s.fence[k], 0), err, what)) return nullptr;
+  if (!hip_ok(hipEventRecord(s.fence[k ^ 1], stream), err, what)) return nullptr;
+  s.fenced[k ^ 1] = true;
+
+  size_t const row_bytes = width * sizeof(float);
+  size_t rows_per_piece = kUploadPiece / (row_bytes ? row_bytes : 1);
+  if (rows_per_piece == 0) rows_per_piece = 1;
+  size_t const npieces = (B + rows_per_piece - 1) / rows_per_piece;
+  hipStream_t const up = up_stream;
+  auto piece = [=](size_t const p) -> hipError_t {
+    size_t const r0 = p * rows_per_piece, r1 = r0 + rows_per_piece < B ? r0 + rows_per_piece : B;
+    for (size_t i = r0; i < r1; ++i) std::memcpy(h + i * width, rows[i], row_bytes);
+    return hipMemcpyAsync(d + r0 * width, h + r0 * width, (r1 - r0) * row_bytes, hipMemcpyHostToDevice, up);
+  };
+  hipError_t first_bad = hipSuccess;
+  unsigned threads = std::thread::hardware_concurrency();
+  if (threads > kGatherThreads) threads = kGatherThreads;
+  if (threads > npieces) threads = static_cast<unsigned>(npieces);
+  if (B * row_bytes < kParallelGatherBytes || threads < 2) {
+    for (size_t p = 0; p < npieces && first_bad == hipSuccess; ++p) first_bad = piece(p);
+  } else {
+    // pieces are handed out in order; a piece's copy starts as soon as it has been gathered, while the
+    // other threads still gather theirs
+    int device = 0;
+    (void)hipGetDevice(&device);
+    std::atomic<size_t> next_piece{0};
+    std::atomic<int> bad{static_cast<int>(hipSuccess)};
+    auto work = [&](bool const set_device) {
+      if (set_device && hipSetDevice(device) != hipSuccess) { bad = static_cast<int>(hipErrorInvalidDevice); return; }
+      for (;;) {
+        size_t const p = next_piece.fetch_add(1);
+        if (p >= npieces) break;
+        hipError_t const e = piece(p);
+        if (e != hipSuccess) bad = static_cast<int>(e);
+      }
+    };
+    std::vector<std::thread> pool;
+    for (unsigned t = 1; t < threads; ++t) pool.emplace_back(work, true);
+    work(false);
+    for (std::thread &t : pool) t.join();
+    first_bad = static_cast<hipError_t>(bad.load());
+  }
+  if (!hip_ok(first_bad, err, what)) return nullptr;
+  if (!hip_ok(hipEventRecord(s.uploaded[k], up_stream), err, what)) return nullptr;
+  if (!hip_ok(hipStreamWaitEvent(stream, s.uploaded[k], 0), err, what)) return nullptr;
+  return d;
+}
 
 Model::Model(void) : impl_(new Impl) {
   real_gen.seed(5489u);
@@ -103,9 +229,11 @@ void Model::clear(void) {
     for (Layer *l = ptr_array_layers; l != ptr_last_layer; ++l) {
       dev_free(l->d_mean); dev_free(l->d_std); dev_free(l->d_r); dev_free(l->d_d); dev_free(l->d_mask);
     }
-  if (impl_->h_stage != nullptr) (void)hipHostFree(impl_->h_stage);
+  if (impl_->up_stream != nullptr) (void)hipStreamSynchronize(impl_->up_stream);
+  impl_->slots_free_all(impl_->in_rows);
+  impl_->slots_free_all(impl_->tgt_rows);
   if (impl_->ctx != nullptr) (void)dlmi_ctx_destroy(impl_->ctx);
-  hipStream_t const stream = impl_->stream;
+  hipStream_t const stream = impl_->stream, up_stream = impl_->up_stream;
   size_t const n_errors = impl_->n_errors;
   Dist::Bernoulli *const masks = bernoulli;
   delete[] ptr_array_layers;
@@ -116,6 +244,7 @@ void Model::clear(void) {
   Impl *const impl = impl_;
   *impl = Impl();
   impl->stream = stream;
+  impl->up_stream = up_stream;
   impl->n_errors = n_errors;
   static_cast<Model_State &>(*this) = Model_State();  // every public member takes its default again
   real_gen.seed(5489u);
@@ -125,6 +254,7 @@ void Model::clear(void) {
 Model::~Model(void) {
   clear();
   if (impl_->stream != nullptr) (void)hipStreamDestroy(impl_->stream);
+  if (impl_->up_stream != nullptr) (void)hipStreamDestroy(impl_->up_stream);
   delete[] bernoulli;
   delete impl_;
 }
@@ -202,6 +332,11 @@ bool Model::compile(size_t const n_layers, size_t const number_recurrent_depth_r
     (void)hipGetLastError();
     impl_->stream = nullptr;
     return fail("compile: no gfx950 device / stream (there is no CPU path)");
+  }
+  if (impl_->up_stream == nullptr && hipStreamCreateWithFlags(&impl_->up_stream, hipStreamNonBlocking) != hipSuccess) {
+    (void)hipGetLastError();
+    impl_->up_stream = nullptr;
+    return fail("compile: no copy stream");
   }
   if (dlmi_ctx_create(&impl_->ctx, 0, impl_->stream) != DLMI_OK)
     return fail("compile: no gfx950 device / context (there is no CPU path)");
@@ -446,8 +581,9 @@ void Model::free_batch(void) {
       dev_free(l->d_block_values);
     }
   dev_free(impl_->d_input_grad);
-  dev_free(impl_->d_input);
-  dev_free(impl_->d_targets);
+  if (impl_->up_stream != nullptr) (void)hipStreamSynchronize(impl_->up_stream);
+  impl_->slots_free_device(impl_->in_rows);
+  impl_->slots_free_device(impl_->tgt_rows);
   impl_->allocated_batch = 0;
 }
 
@@ -477,20 +613,11 @@ bool Model::allocate_batch(size_t const n) {
       return false;
   }
   size_t const n_in = ptr_array_layers[0].n_out, n_o = ptr_array_layers[total_layers - 1].n_out;
-  if (!dev_alloc(&impl_->d_input, n * n_in, err) || !dev_alloc(&impl_->d_targets, n * n_o, err)) return false;
+  if (!impl_->slots_alloc(impl_->in_rows, n * n_in) || !impl_->slots_alloc(impl_->tgt_rows, n * n_o)) return false;
   // a block that reads the network input still sends a gradient through its first
   // layer's normalization (for that layer's scale and shift)
   if (total_layers > 1 && ptr_array_layers[1].type_layer == LAYER::RESIDUAL && !dev_alloc(&impl_->d_input_grad, n * n_in, err))
     return false;
-  size_t const stage = n * (n_in > n_o ? n_in : n_o);
-  if (stage > impl_->h_stage_floats) {
-    if (impl_->h_stage != nullptr) (void)hipHostFree(impl_->h_stage);
-    impl_->h_stage = nullptr;
-    void *p = nullptr;
-    if (!hip_ok(hipHostMalloc(&p, stage * sizeof(float), hipHostMallocDefault), err, "hipHostMalloc")) return false;
-    impl_->h_stage = static_cast<float *>(p);
-    impl_->h_stage_floats = stage;
-  }
   impl_->allocated_batch = n;
   return true;
 }
@@ -499,7 +626,7 @@ bool Model::allocate_batch(size_t const n) {
 // buffers this layout keeps: allocate_batch() above)
 size_t Model::Get__Batch_Sizeof(size_t const batch) const {
   if (ptr_array_layers == nullptr) return 0;
-  size_t floats = ptr_array_layers[0].n_out + ptr_array_layers[total_layers - 1].n_out;  // input rows and targets
+  size_t floats = 2 * (ptr_array_layers[0].n_out + ptr_array_layers[total_layers - 1].n_out);  // input rows and targets, two slots each
   if (total_layers > 1 && ptr_array_layers[1].type_layer == LAYER::RESIDUAL) floats += ptr_array_layers[0].n_out;
   for (size_t i = 1; i < total_layers; ++i) {
     Layer const &l = ptr_array_layers[i];
@@ -869,15 +996,9 @@ void Model::forward_pass(size_t const B, real const *const *const Xm, long long 
   if (in_idx != 0 || out_idx < 2 || out_idx > static_cast<long long>(total_layers)) { fail("forward_pass: a pass starts at the input layer and ends at one of the layers"); return; }
   if (B == 0 || B > impl_->allocated_batch) { fail("forward_pass: batch size exceeds update_mem_batch_size()"); return; }
   size_t const n_in = ptr_array_layers[0].n_out;
-  // assign_inputs.cpp:22-40: gather the row pointers into a dense [B, K] block
-  // (pinned staging buffer: the previous step's copy out of it has completed
-  // once the stream is idle)
-  (void)hipStreamSynchronize(impl_->stream);
-  for (size_t i = 0; i < B; ++i) std::memcpy(impl_->h_stage + i * n_in, Xm[i], n_in * sizeof(float));
-  if (!hip_ok(hipMemcpyAsync(impl_->d_input, impl_->h_stage, B * n_in * sizeof(float), hipMemcpyHostToDevice, impl_->stream),
-              impl_->err, "input upload"))
-    return;
-  impl_->cur_input = impl_->d_input;
+  float const *const d_rows = impl_->slots_upload(impl_->in_rows, B, n_in, Xm, "forward_pass: input upload");
+  if (d_rows == nullptr) { std::string const why = impl_->err; fail(why.c_str()); return; }
+  impl_->cur_input = d_rows;
   forward_layers(B, static_cast<size_t>(out_idx));
 }
 
@@ -1079,12 +1200,9 @@ var const *Model::get_out(size_t const data_index, size_t const) const {
 void Model::compute_error(size_t const B, real const *const *const Ym) {
   if (ptr_array_layers == nullptr || Ym == nullptr || B == 0 || B > impl_->allocated_batch) { fail("compute_error: bad argument"); return; }
   size_t const H = ptr_array_layers[total_layers - 1].n_out;
-  (void)hipStreamSynchronize(impl_->stream);
-  for (size_t i = 0; i < B; ++i) std::memcpy(impl_->h_stage + i * H, Ym[i], H * sizeof(float));
-  if (!hip_ok(hipMemcpyAsync(impl_->d_targets, impl_->h_stage, B * H * sizeof(float), hipMemcpyHostToDevice, impl_->stream),
-              impl_->err, "target upload"))
-    return;
-  seed_error(B, impl_->d_targets);
+  float const *const d_rows = impl_->slots_upload(impl_->tgt_rows, B, H, Ym, "compute_error: target upload");
+  if (d_rows == nullptr) { std::string const why = impl_->err; fail(why.c_str()); return; }
+  seed_error(B, d_rows);
 }
 
 void Model::compute_error_device(size_t const B, float const *d_targets) {
@@ -1142,7 +1260,7 @@ uint64_t Model::launch_signature(void) const {
 #define DLMI_MIX(v) mix(&(v), sizeof(v))
   DLMI_MIX(total_layers); DLMI_MIX(total_parameters); DLMI_MIX(impl_->allocated_batch);
   DLMI_MIX(impl_->d_params); DLMI_MIX(impl_->d_dparams); DLMI_MIX(impl_->d_mov_mean); DLMI_MIX(impl_->d_mov_std);
-  DLMI_MIX(impl_->d_stats); DLMI_MIX(impl_->d_input); DLMI_MIX(impl_->d_input_grad);
+  DLMI_MIX(impl_->d_stats); DLMI_MIX(impl_->in_rows.d[0]); DLMI_MIX(impl_->in_rows.d[1]); DLMI_MIX(impl_->d_input_grad);
   // the context's scratch block, whose address the kernels of a batch are given: a recording made before it grew
   // keeps working (a retired block stays allocated) but is made again, so that every launch uses the same block
   unsigned long long const scratch_generation = dlmi_ctx_scratch_generation(impl_->ctx);

@@ -251,6 +251,27 @@ int dlmi_model_step(dlmi_model *h, int state, size_t B, float const *X, float co
   }
   return m.synchronize() && m.error_count() == errors_before;
 }
+int dlmi_model_steps(dlmi_model *h, int state, size_t n_steps, size_t B, float const *X, float const *Y, int do_backward) {
+  Model &m = h->m;
+  size_t const errors_before = m.error_count();
+  m.type_state_propagation = static_cast<PROPAGATION::TYPE>(state);
+  size_t const K0 = m.ptr_array_layers[0].n_out, Ho = m.Get__Output_Layer()->n_out;
+  std::vector<float const *> Xm(B), Ym(B);
+  for (size_t s = 0; s < n_steps && m.error_count() == errors_before; ++s) {
+    for (size_t i = 0; i < B; ++i) {
+      Xm[i] = X + (s * B + i) * K0;
+      Ym[i] = Y ? Y + (s * B + i) * Ho : nullptr;
+    }
+    m.forward_pass(B, Xm.data());
+    if (do_backward) {
+      m.compute_error(B, Ym.data());
+      m.backward_pass(B);
+      m.update_derivatives(B, m.ptr_array_layers + 1, m.ptr_last_layer);
+      m.merge_mp_derivatives(0, m.total_parameters);
+    }
+  }
+  return m.synchronize() && m.error_count() == errors_before;
+}
 // forward_pass(B, rows of X, 0, end_layer): the layers [1, end_layer) only
 int dlmi_model_forward_to(dlmi_model *h, int state, size_t B, float const *X, size_t end_layer) {
   Model &m = h->m;

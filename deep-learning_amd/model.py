@@ -31,7 +31,7 @@ MODEL_C_ABI_SYMBOLS = [
     "dlmi_model_set_allowable_memory", "dlmi_model_memory", "dlmi_model_create_empty", "dlmi_model_save_params",
     "dlmi_model_save_spec_params", "dlmi_model_load_spec_params", "dlmi_model_load", "dlmi_model_total_layers",
     "dlmi_checkpointer_create", "dlmi_checkpointer_destroy", "dlmi_checkpointer_save", "dlmi_checkpointer_load",
-    "dlmi_model_forward_to", "dlmi_model_lsuv", "dlmi_model_lsuv_trials", "dlmi_model_layer_variance",
+    "dlmi_model_forward_to", "dlmi_model_lsuv", "dlmi_model_lsuv_trials", "dlmi_model_layer_variance", "dlmi_model_steps",
 ]
 
 LAYER_FULLY_CONNECTED, LAYER_RESIDUAL = 3, 9  # v1/data/enum/layer.hpp
@@ -173,6 +173,15 @@ class Model:
             Yp = _ptr(Y)
         self._ok(self.lib.dlmi_model_step(self.h, c_int(state), c_sz(self.B), _ptr(X), Yp, c_int(1 if backward else 0)),
                  "step")
+
+    def steps(self, state, X, Y, batch, backward=True):
+        """len(X) / batch steps on consecutive row blocks, the host waiting only after the last one."""
+        X = np.ascontiguousarray(X, np.float32)
+        Y = np.ascontiguousarray(Y, np.float32)
+        n = X.shape[0] // batch
+        self.B = batch
+        self._ok(self.lib.dlmi_model_steps(self.h, c_int(state), c_sz(n), c_sz(batch), _ptr(X), _ptr(Y),
+                                           c_int(1 if backward else 0)), "steps")
 
     def forward_to(self, state, X, end_layer):
         """forward_pass(B, X, 0, end_layer): layers [1, end_layer) only."""

@@ -89,6 +89,10 @@ void dlmi_model_clear_training_arrays(dlmi_model *m);
 /* type_state_propagation = state; forward_pass(B, rows of X); if do_backward: compute_error(B, rows of Y),
  * backward_pass(B), update_derivatives(B, layers + 1, last_layer).  X [B,K0], Y [B,Hout] dense host arrays. */
 int dlmi_model_step(dlmi_model *m, int state, size_t B, float const *X, float const *Y, int do_backward);
+/* n_steps such steps one behind the other on consecutive row blocks of X [n_steps*B,K0] and Y [n_steps*B,Hout],
+ * the host waiting only after the last one: the rows of a step are gathered and uploaded while the kernels of
+ * the step before it still run (the caller's loop of drivers/driver.cpp:139-160 without a read-back per batch) */
+int dlmi_model_steps(dlmi_model *m, int state, size_t n_steps, size_t B, float const *X, float const *Y, int do_backward);
 /* forward_pass(batch, rows of X, 0, end_layer): only the layers [1, end_layer) run (the partial pass the LSUV
  * initializer uses, lsuv.cpp:131-135) */
 int dlmi_model_forward_to(dlmi_model *m, int state, size_t batch, float const *X, size_t end_layer);

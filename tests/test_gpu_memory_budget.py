@@ -12,7 +12,7 @@ from oracle.binding import ACT, NORM, OPT
 pytestmark = pytest.mark.gpu
 
 WIDTHS = [10, 16, 4]
-PER_EXAMPLE = (10 + 4 + 3 * 16 + 3 * 4) * 4  # input row, target row, Z / output / gradient of both layers
+PER_EXAMPLE = (2 * 10 + 2 * 4 + 3 * 16 + 3 * 4) * 4  # input row and target row (two upload slots each), Z / output / gradient of both layers
 
 
 def build(lib, max_batch, budget=None):
