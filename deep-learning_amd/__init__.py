@@ -36,7 +36,7 @@ STATE = dict(INFERENCE=0, TRAINING=1, UPDATE_BATCH_NORM=2)
 C_ABI_SYMBOLS = [
     "dlmi_ctx_create", "dlmi_ctx_destroy", "dlmi_ctx_set_stream", "dlmi_ctx_synchronize", "dlmi_last_error",
     "dlmi_ctx_compute_units", "dlmi_layer_variance", "dlmi_scale", "dlmi_fc_fwd", "dlmi_fc_bwd_dx", "dlmi_fc_bwd_dw", "dlmi_bias_fwd",
-    "dlmi_norm_fwd_train", "dlmi_norm_fwd_infer", "dlmi_norm_bwd", "dlmi_act_fwd", "dlmi_act_bwd",
+    "dlmi_norm_fwd_train", "dlmi_norm_fwd_infer", "dlmi_norm_bwd", "dlmi_act_fwd", "dlmi_act_fwd_units", "dlmi_act_bwd_units", "dlmi_act_bwd",
     "dlmi_softmax_fwd", "dlmi_dropout_fwd", "dlmi_identity_add", "dlmi_softmax_ce_seed",
     "dlmi_fused_norm_act_fwd", "dlmi_fused_norm_act_bwd", "dlmi_fused_norm_act_infer", "dlmi_fc_norm_act_fwd",
     "dlmi_opt_gd", "dlmi_opt_gd_momentum", "dlmi_opt_adam", "dlmi_zero_padded_identity_fwd", "dlmi_residual_bwd",
@@ -219,6 +219,23 @@ class Dlmi:
         B, H = pre.shape
         dN = out if out is not None else self.empty(B, H)
         self._ck(self.lib.dlmi_act_bwd(self.ctx, c_int(act), c_sz(B), c_sz(H), _p(pre), _p(post), _p(dY), _p(dN)))
+        return dN
+
+    def act_fwd_units(self, types, x):
+        """types: one activation code per unit (host integers)."""
+        self._chk(x)
+        B, H = x.shape
+        t = (c_int * H)(*[int(v) for v in types])
+        y = self.empty(B, H)
+        self._ck(self.lib.dlmi_act_fwd_units(self.ctx, t, c_sz(B), c_sz(H), _p(x), _p(y)))
+        return y
+
+    def act_bwd_units(self, types, pre, post, dY):
+        self._chk(pre, post, dY)
+        B, H = pre.shape
+        t = (c_int * H)(*[int(v) for v in types])
+        dN = self.empty(B, H)
+        self._ck(self.lib.dlmi_act_bwd_units(self.ctx, t, c_sz(B), c_sz(H), _p(pre), _p(post), _p(dY), _p(dN)))
         return dN
 
     def softmax_fwd(self, x):

@@ -59,6 +59,32 @@ __global__ __launch_bounds__(kEwBlock) void k_act_bwd(float const *__restrict__ 
     dN[i] = dY[i] * act_derive<ACT>(pre[i], post[i]);
 }
 
+// ---- the same with one activation type per unit (fwp_st.cpp:4768-4794 takes an array of types, one per
+// unit of the layer; a layer read from a .net file may mix them, load.cpp:4121).  Lanes of a wavefront sit on
+// different units, so the switch diverges where neighbouring units differ; every unit still runs the code of
+// the single-type kernels.
+__device__ __forceinline__ float act_fire_of(int act, float x) {
+  DLMI_DISPATCH_ACT(act, return act_fire<ACT>(x));
+  return x;
+}
+__device__ __forceinline__ float act_derive_of(int act, float x, float q) {
+  DLMI_DISPATCH_ACT(act, return act_derive<ACT>(x, q));
+  return 1.0f;
+}
+__global__ __launch_bounds__(kEwBlock) void k_act_units_fwd(int const *__restrict__ types, float const *__restrict__ x,
+                                                             float *__restrict__ y, size_t H, size_t n) {
+  size_t const stride = static_cast<size_t>(gridDim.x) * kEwBlock;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x; i < n; i += stride)
+    y[i] = act_fire_of(types[i % H], x[i]);
+}
+__global__ __launch_bounds__(kEwBlock) void k_act_units_bwd(int const *__restrict__ types, float const *__restrict__ pre,
+                                                             float const *__restrict__ post, float const *__restrict__ dY,
+                                                             float *__restrict__ dN, size_t H, size_t n) {
+  size_t const stride = static_cast<size_t>(gridDim.x) * kEwBlock;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x; i < n; i += stride)
+    dN[i] = dY[i] * act_derive_of(types[i % H], pre[i], post[i]);
+}
+
 // ---- out = a + b (fwp_st.cpp:5051-5112 with equal widths)
 __global__ __launch_bounds__(kEwBlock) void k_add(float const *__restrict__ a, float const *__restrict__ b,
                                                    float *__restrict__ out, size_t n4, size_t n) {
@@ -374,6 +400,49 @@ int dlmi_act_bwd(dlmi_ctx *ctx, dlmi_activation act, size_t B, size_t H, float c
   DLMI_DISPATCH_ACT(act, hipLaunchKernelGGL((k_act_bwd<ACT>), dim3(grid), dim3(kEwBlock), 0, ctx->stream, pre, post,
                                             dY, dN, n4, n));
   DLMI_LAUNCH_CHECK(ctx, "k_act_bwd");
+  return DLMI_OK;
+}
+
+// The caller's per-unit types, checked on the host and staged in the context's scratch for the kernel.
+static int stage_unit_types(dlmi_ctx *ctx, size_t H, dlmi_activation const *types, int const **d_types) {
+  for (size_t j = 0; j < H; ++j)
+    if (!act_supported(types[j]))
+      return dlmi_fail(ctx, DLMI_E_UNSUPPORTED, "unit %zu: unsupported activation %d", j, static_cast<int>(types[j]));
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(ctx->stream, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone)
+    return dlmi_fail(ctx, DLMI_E_INVALID, "per-unit activation types are copied from the host: not while the stream is being recorded");
+  int const rc = dlmi_scratch_reserve(ctx, H * sizeof(int));
+  if (rc != DLMI_OK) return rc;
+  static_assert(sizeof(dlmi_activation) == sizeof(int), "the enum travels as int");
+  // ordered behind the stream's earlier work (the scratch may still be read), complete for the host on return
+  DLMI_HIP(ctx, hipMemcpyWithStream(dlmi_scratch_data(ctx), types, H * sizeof(int), hipMemcpyHostToDevice, ctx->stream));
+  *d_types = reinterpret_cast<int const *>(dlmi_scratch_data(ctx));
+  return DLMI_OK;
+}
+
+int dlmi_act_fwd_units(dlmi_ctx *ctx, dlmi_activation const *types, size_t B, size_t H, float const *x, float *y) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, types && x && y, "null pointer");
+  size_t const n = B * H;
+  if (n == 0) return DLMI_OK;
+  int const *d_types = nullptr;
+  if (int const rc = stage_unit_types(ctx, H, types, &d_types); rc != DLMI_OK) return rc;
+  hipLaunchKernelGGL(k_act_units_fwd, dim3(ew_grid(ctx, n)), dim3(kEwBlock), 0, ctx->stream, d_types, x, y, H, n);
+  DLMI_LAUNCH_CHECK(ctx, "k_act_units_fwd");
+  return DLMI_OK;
+}
+
+int dlmi_act_bwd_units(dlmi_ctx *ctx, dlmi_activation const *types, size_t B, size_t H, float const *pre,
+                       float const *post, float const *dY, float *dN) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, types && pre && post && dY && dN, "null pointer");
+  size_t const n = B * H;
+  if (n == 0) return DLMI_OK;
+  int const *d_types = nullptr;
+  if (int const rc = stage_unit_types(ctx, H, types, &d_types); rc != DLMI_OK) return rc;
+  hipLaunchKernelGGL(k_act_units_bwd, dim3(ew_grid(ctx, n)), dim3(kEwBlock), 0, ctx->stream, d_types, pre, post, dY,
+                     dN, H, n);
+  DLMI_LAUNCH_CHECK(ctx, "k_act_units_bwd");
   return DLMI_OK;
 }
 

@@ -152,6 +152,12 @@ int dlmi_norm_bwd(dlmi_ctx *ctx, dlmi_norm norm, size_t B, size_t H, float const
  * (v1/ops/activations/functions.hpp:124-220).  y may alias x. */
 int dlmi_act_fwd(dlmi_ctx *ctx, dlmi_activation act, size_t B, size_t H, float const *x, float *y);
 
+/* The same with one type per unit: types[H] on the HOST, as Forward_Pass__FC_AF__Loop takes it
+ * (fwp_st.cpp:4768-4794: `ACTIVATION::TYPE const *ptr_array_type_activations_received`; the units of a layer
+ * read from a .net file may differ, load.cpp:4121).  Every entry must be one of the supported types; the
+ * array is staged in the context's scratch, so not under stream capture. */
+int dlmi_act_fwd_units(dlmi_ctx *ctx, dlmi_activation const *types, size_t B, size_t H, float const *x, float *y);
+
 /* dN = dY * f'(pre, post), with the reference's derivative forms
  * (functions.hpp:41,45,88,92,99,103,107; v1/learner/model.cpp:2594-2651):
  * ELU' = post (x<0), SELU' = scale*(post+alpha) (x<=0), ISRLU' = (post/pre)^3 (x<0),
@@ -159,6 +165,9 @@ int dlmi_act_fwd(dlmi_ctx *ctx, dlmi_activation act, size_t B, size_t H, float c
  * Replaces Backward_Pass__FC__DF__* (bwp_st.cpp:1177-1209).  dN may alias dY. */
 int dlmi_act_bwd(dlmi_ctx *ctx, dlmi_activation act, size_t B, size_t H, float const *pre,
                  float const *post, float const *dY, float *dN);
+/* Per-unit types, as Backward_Pass__FC__DF__Loop takes them (bwp_st.cpp:1177-1209). */
+int dlmi_act_bwd_units(dlmi_ctx *ctx, dlmi_activation const *types, size_t B, size_t H, float const *pre,
+                       float const *post, float const *dY, float *dN);
 
 /* Row-wise softmax (Forward_Pass__FC_AF__Softmax__*, fwp_st.cpp:4796-4828). */
 int dlmi_softmax_fwd(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *y);

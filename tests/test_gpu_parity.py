@@ -96,6 +96,49 @@ def test_activation_special_points(dl, golden_leaves, a):
     assert_close(d, g[f"pts_bwd_{a}"], TE, "bwd " + a)
 
 
+@pytest.mark.parametrize("B,H", [(53, 37), (128, 512), (1, 8)])
+def test_per_unit_activation_types(dl, oracle, golden_leaves, B, H):
+    """One activation type per unit (fwp_st.cpp:4768-4794 takes the array): every column must hold what the
+    single-type leaf gives for that column's type (the same device code: bit-identical) and what the oracle
+    gives for it; the special points of the golden file go through one unit per type."""
+    names = ACTS + ["SIGMOID", "TANH"]
+    rng = np.random.default_rng(B * 131 + H)
+    types = [ACT[names[i]] for i in rng.integers(0, len(names), H)]
+    x = (rng.standard_normal((B, H)) * 3).astype(np.float32)
+    x[0, :] = 0.0
+    dY = rng.standard_normal((B, H)).astype(np.float32)
+    y = dl.act_fwd_units(types, dev(x))
+    dN = dl.act_bwd_units(types, dev(x), y, dev(dY))
+    y, dN = host(y), host(dN)
+    for name in names:
+        cols = [j for j in range(H) if types[j] == ACT[name]]
+        if not cols:
+            continue
+        xs, gs = np.ascontiguousarray(x[:, cols]), np.ascontiguousarray(dY[:, cols])
+        ys = dl.act_fwd(ACT[name], dev(xs))
+        assert np.array_equal(y[:, cols], host(ys)), name
+        assert np.array_equal(dN[:, cols], host(dl.act_bwd(ACT[name], dev(xs), ys, dev(gs)))), name
+        yo = oracle.act_fwd(ACT[name], xs)
+        assert_close(y[:, cols], yo, TE, "per-unit fwd " + name)
+        keep = np.abs(xs) > 1e-6  # the rectifiers' derivatives jump at 0
+        assert_close(np.where(keep, dN[:, cols], 0), np.where(keep, oracle.act_bwd(ACT[name], xs, yo, gs), 0), TE,
+                     "per-unit bwd " + name)
+    g = golden_leaves
+    pts = np.ascontiguousarray(np.repeat(g["pts"].reshape(-1, 1), len(ACTS), axis=1))
+    yp = host(dl.act_fwd_units([ACT[a] for a in ACTS], dev(pts)))
+    for j, a in enumerate(ACTS):
+        assert_close(yp[:, j], g[f"pts_fwd_{a}"].reshape(-1), TE, "special points " + a)
+
+
+def test_per_unit_activation_types_refuse_an_unsupported_type(dl):
+    from deep_learning_amd import DlmiError
+    x = dev(np.zeros((2, 3), np.float32))
+    with pytest.raises(DlmiError, match="unit 1"):
+        dl.act_fwd_units([ACT["RELU"], ACT["SOFTMAX"], ACT["ELU"]], x)
+    with pytest.raises(DlmiError, match="unit 2"):
+        dl.act_bwd_units([ACT["RELU"], ACT["ELU"], 99], x, x, x)
+
+
 # ------------------------------------------------------------------ GEMMs against the oracle
 GEMM_SHAPES = [  # (B, K, H): tile-aligned (fast path) and ragged (guarded path)
     (128, 128, 128), (256, 64, 384), (384, 256, 128), (1, 1, 1), (7, 13, 5), (130, 70, 129), (128, 784, 512),
