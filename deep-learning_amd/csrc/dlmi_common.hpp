@@ -28,6 +28,9 @@ struct dlmi_tuning {
   int fold_fwd = 1;
   int fold_bwd = 2;
   size_t fold_fwd_max_elements = size_t(1) << 20;
+  // ... with the partial sums already there (the product's epilogue wrote them, at most 16 tile rows): the
+  // finalize launch is all that is left to save, which pays up to this many elements
+  size_t fold_fwd_epilogue_max_elements = size_t(1) << 22;
   int fc_narrow = 1;              // layers of at most 16 units on a mini-batch run the narrow-layer kernels (fc_small.hip)
   int norm_small = 1;             // mini-batches (at most 256 rows, 2^20 elements) run the one-launch small-batch kernels
 };
@@ -101,13 +104,17 @@ namespace dlmi {
 int static_scratch_init(dlmi_ctx *ctx);
 // Batch-(re)norm forward tail (finalize + apply) from column-sum partials
 // [2][nchunks][H] that a producer (the GEMM epilogue) already wrote.
-// partial == nullptr: the statistics come from a pass over x.  residual != nullptr:
+// partial == nullptr: the statistics come from a pass over x.  mov_snapshot != nullptr: [2][H], the moving
+// statistics as they were before this step (the producer copied them); with at most kNormFoldChunks chunks the
+// apply pass then does the per-unit arithmetic itself and no finalize kernel runs.  residual != nullptr:
 // y = residual + (activation output after dropout), the identity shortcut of a block.
 int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
                             float const *gamma, float const *beta, uint8_t const *mask, float const *residual,
                             float *mean, float *stdv, float *mov_mean, float *mov_std, float *r, float *d, float *y,
                             float const *partial, unsigned nchunks, float const *slices = nullptr,
-                            unsigned nslices = 0);
+                            unsigned nslices = 0, float const *mov_snapshot = nullptr);
+// Most chunks of partial sums an apply pass adds up itself (its prologue) instead of a finalize kernel.
+constexpr unsigned kNormFoldChunks = 16;
 // Whether a [B, H] tensor runs the small-batch normalization kernels.  Those also accept x as `nslices`
 // partial products [nslices][B][H] still to be added (the slices of a split-K product, passed to
 // fused_fwd_from_partials with x = where the sum is to be stored): a producer may skip its own reduction then.
@@ -122,6 +129,9 @@ size_t norm_scratch_bytes(dlmi_ctx const *ctx, size_t H);
 // scratch they need for [*, H].
 int panel_init(dlmi_ctx *ctx);
 int panel_check(dlmi_ctx *ctx);
+// The context lets go of its stream (destroyed, or given another one), which the caller may destroy next:
+// after the stream's work has completed, the cross-stream ordering of panel launches forgets it.
+void panel_release_stream(dlmi_ctx *ctx);
 size_t panel_scratch_bytes(size_t H);
 // Narrow layers on a mini-batch (fc_small.hip).  narrow_fc_fwd: Z = X W^T + bias and, with Q != nullptr,
 // Q = softmax(Z), one launch; call only when narrow_fc_fwd_eligible.  narrow_dw_try: dW and db in one launch;

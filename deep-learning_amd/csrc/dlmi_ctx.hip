@@ -97,6 +97,7 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
 int dlmi_ctx_destroy(dlmi_ctx *ctx) {
   if (ctx == nullptr) return DLMI_OK;
   (void)hipStreamSynchronize(ctx->stream);
+  dlmi::panel_release_stream(ctx);
   if (ctx->scratch != nullptr) (void)hipFree(ctx->scratch);
   for (int i = 0; i < ctx->n_retired; ++i) (void)hipFree(ctx->retired[i]);
   if (ctx->panel_state != nullptr) (void)hipFree(ctx->panel_state);
@@ -106,6 +107,15 @@ int dlmi_ctx_destroy(dlmi_ctx *ctx) {
 
 int dlmi_ctx_set_stream(dlmi_ctx *ctx, void *stream) {
   if (ctx == nullptr) return DLMI_E_INVALID;
+  if (ctx->stream == static_cast<hipStream_t>(stream)) return DLMI_OK;
+  // the old stream may be destroyed by its owner once the context has let go of it (not while it is being
+  // recorded, which is also when it cannot be waited for)
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(ctx->stream, &capturing) != hipSuccess) (void)hipGetLastError();
+  if (capturing == hipStreamCaptureStatusNone) {
+    DLMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    dlmi::panel_release_stream(ctx);
+  }
   ctx->stream = static_cast<hipStream_t>(stream);
   return DLMI_OK;
 }

@@ -52,6 +52,10 @@ struct GemmArgs {
   size_t k_per_split;  // K range of one blockIdx.z slice (multiple of BK)
   float *split_out;    // when gridDim.z > 1: [splits][M][N] partial products
   float *stats_out;    // optional [2][tiles_m][N]: per tile-row column sums of C and C^2 (gridDim.z == 1)
+  // with stats_out, optional: the first tile row copies two per-column vectors [N] (the moving statistics of the
+  // normalization that follows, before it updates them) to snap_out [2][N]
+  float const *snap_a, *snap_b;
+  float *snap_out;
   int accumulate;      // C += result (only when gridDim.z == 1)
   int a_vec, b_vec;    // operand base and leading dimension allow 16-byte loads (ragged variant)
   unsigned tiles_m, tiles_n;
@@ -366,6 +370,10 @@ void k_gemm_f32(GemmArgs g) {
       if (FAST || col < g.N) {
         g.stats_out[(0 * static_cast<size_t>(g.tiles_m) + tile_m) * g.N + col] = sl[(0 * BN + c) * 2 + 0] + sl[(1 * BN + c) * 2 + 0];
         g.stats_out[(1 * static_cast<size_t>(g.tiles_m) + tile_m) * g.N + col] = sl[(0 * BN + c) * 2 + 1] + sl[(1 * BN + c) * 2 + 1];
+        if (g.snap_out != nullptr && tile_m == 0) {
+          g.snap_out[col] = g.snap_a[col];
+          g.snap_out[g.N + col] = g.snap_b[col];
+        }
       }
     }
   }
@@ -537,7 +545,8 @@ size_t fc_scratch_bytes(dlmi_ctx const *ctx, size_t B, size_t K, size_t H) {
 template <bool AK, bool BKC>
 static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, size_t lda, float const *B, size_t ldb,
                 float *C, float const *bias, int accumulate, unsigned *stats_chunks = nullptr,
-                unsigned *defer_slices = nullptr) {
+                unsigned *defer_slices = nullptr, float const *snap_a = nullptr, float const *snap_b = nullptr,
+                float const **snap_out = nullptr) {
   GemmPlan const plan = plan_gemm(ctx, M, N, K);
   int const choice = plan.choice;
   int const bm = plan.bm, bn = plan.bn, bk = plan.bk;
@@ -545,6 +554,8 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   GemmArgs g;
   g.A = A; g.B = B; g.C = C; g.bias = bias; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldc = N;
   g.accumulate = accumulate; g.split_out = nullptr; g.stats_out = nullptr;
+  g.snap_a = g.snap_b = nullptr; g.snap_out = nullptr;
+  if (snap_out != nullptr) *snap_out = nullptr;
   g.a_vec = (lda % 4 == 0 && dlmi_aligned16(A)) ? 1 : 0;
   g.b_vec = (ldb % 4 == 0 && dlmi_aligned16(B)) ? 1 : 0;
   bool const fast = M % bm == 0 && N % bn == 0 && K % bk == 0 && g.a_vec && g.b_vec;
@@ -565,6 +576,12 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
       int rc = dlmi_scratch_reserve(ctx, 2 * 2 * static_cast<size_t>(chunks_reserved) * N * sizeof(float));
       if (rc != DLMI_OK) return rc;
       g.stats_out = reinterpret_cast<float *>(dlmi_scratch_data(ctx));
+      if (snap_out != nullptr && snap_a != nullptr && snap_b != nullptr) {
+        // the second half of what was reserved: the partial sums fill the first
+        g.snap_a = snap_a; g.snap_b = snap_b;
+        g.snap_out = g.stats_out + 2 * static_cast<size_t>(chunks_reserved) * N;
+        *snap_out = g.snap_out;
+      }
     }
   }
   size_t const kt_per_split = dlmi_ceil_div(ktiles, splits);
@@ -628,7 +645,9 @@ static int fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B,
   unsigned chunks = 0, slices = 0;
   // a mini-batch: the normalization kernel that follows owns whole columns and adds the K slices itself
   bool const defer = small_norm_eligible(ctx, B, H);
-  int rc = gemm<true, true>(ctx, B, H, K, X, K, W, K, Z, nullptr, 0, &chunks, defer ? &slices : nullptr);
+  float const *snapshot = nullptr;  // the moving statistics before this step, copied by the product's epilogue
+  int rc = gemm<true, true>(ctx, B, H, K, X, K, W, K, Z, nullptr, 0, &chunks, defer ? &slices : nullptr, mov_mean, mov_std,
+                            &snapshot);
   if (rc != DLMI_OK) return rc;
   float const *const scratch = reinterpret_cast<float const *>(dlmi_scratch_data(ctx));
   if (slices != 0)
@@ -637,7 +656,7 @@ static int fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B,
   // a small output runs split over K, where no slice sees whole sums: the
   // statistics then come from a pass over Z (nullptr / 0)
   return fused_fwd_from_partials(ctx, desc, B, H, Z, gamma, beta, mask, shortcut, mean, stdv, mov_mean, mov_std, r, d, y,
-                                 chunks != 0 ? scratch : nullptr, chunks);
+                                 chunks != 0 ? scratch : nullptr, chunks, nullptr, 0, snapshot);
 }
 
 int dlmi_fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t K, size_t H, float const *X,

@@ -147,7 +147,7 @@ static ColGeom reduce_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec
 // partial sums): at most kFoldChunks chunks, blocks as narrow as it takes (64, 32 or 16 column groups)
 // to still put a block on most compute units.  False when the shape cannot give both (few units, many
 // rows): the finalize kernel then combines as many chunks as the reduction wants.
-constexpr size_t kFoldChunks = 16;
+constexpr size_t kFoldChunks = kNormFoldChunks;
 static bool fold_geometry(dlmi_ctx const *ctx, size_t B, size_t H, bool vec4, int nplanes, size_t data_bytes,
                           ColGeom *g) {
   int const level = nplanes == 3 ? ctx->tune.fold_bwd : ctx->tune.fold_fwd;
@@ -958,8 +958,14 @@ static int run_fwd_train(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t 
   // data region: [2][H] snapshot of the moving statistics (two-launch scheme), then the partial sums
   size_t const fixed = round_up(3 * H * sizeof(float), 256);
   float *const snap = reinterpret_cast<float *>(sv.data);
+  float const *snap_rd = snap;
   bool fold = false;
-  if (partial == nullptr) {
+  if (partial != nullptr) {
+    // the producer's partial sums and its copy of the moving statistics: few chunks go straight to the apply pass
+    fold = c.snapshot_in != nullptr && nchunks <= kFoldChunks && c.xhat == nullptr && c.nrm == nullptr && c.y != nullptr &&
+           ctx->tune.fold_fwd > 0 && (ctx->tune.fold_fwd > 1 || B * H <= ctx->tune.fold_fwd_epilogue_max_elements);
+    if (fold) snap_rd = c.snapshot_in;
+  } else {
     ColGeom g;
     fold = c.xhat == nullptr && c.nrm == nullptr && c.y != nullptr && fold_geometry(ctx, B, H, vec4, 2, sv.data_bytes, &g);
     if (!fold) g = reduce_geometry(ctx, B, H, vec4, 2, sv.data_bytes);
@@ -999,7 +1005,7 @@ static int run_fwd_train(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t 
   a.mask = c.mask; a.residual = c.residual; a.y = c.y; a.xhat = c.xhat; a.nrm = c.nrm;
   a.B = B; a.H = H; a.rows_per_chunk = ctx->tune.apply_interleave ? 0 : ga.rows_per_chunk; a.tx_log2 = ga.tx_log2;
   a.drop_scale = c.drop_scale;
-  a.fin_partial = fold ? partial : nullptr; a.mov_mean_in = snap; a.mov_std_in = snap + H; a.fin_chunks = nchunks;
+  a.fin_partial = fold ? partial : nullptr; a.mov_mean_in = snap_rd; a.mov_std_in = snap_rd + H; a.fin_chunks = nchunks;
   a.fin = fin;
   dim3 const agrid(ga.grid_x, ga.nchunks);
   if (c.xhat != nullptr || c.nrm != nullptr) {  // un-fused leaf: LINEAR, no dropout by construction
@@ -1147,13 +1153,14 @@ static FwdTrainCall fused_fwd_call(dlmi_fused_desc const *desc, float const *x, 
 int fused_fwd_from_partials(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
                             float const *gamma, float const *beta, uint8_t const *mask, float const *residual,
                             float *mean, float *stdv, float *mov_mean, float *mov_std, float *r, float *d, float *y,
-                            float const *partial, unsigned nchunks, float const *slices, unsigned nslices) {
+                            float const *partial, unsigned nchunks, float const *slices, unsigned nslices,
+                            float const *mov_snapshot) {
   int rc = check_desc(ctx, desc, mask);
   if (rc != DLMI_OK) return rc;
   DLMI_REQUIRE(ctx, x && gamma && beta && mean && stdv && mov_mean && mov_std && r && d && y, "null pointer");
   FwdTrainCall c = fused_fwd_call(desc, x, gamma, beta, mask, mean, stdv, mov_mean, mov_std, r, d, y);
   c.residual = residual;
-  c.partial_in = partial; c.partial_chunks = nchunks;
+  c.partial_in = partial; c.partial_chunks = nchunks; c.snapshot_in = partial != nullptr ? mov_snapshot : nullptr;
   if (nslices > 0) {
     c.slices = slices; c.nslices = nslices; c.z_out = const_cast<float *>(x);
   }

@@ -271,6 +271,16 @@ void panel_launched(dlmi_ctx *ctx) {
   o.recorded = true;
 }
 
+void panel_release_stream(dlmi_ctx *ctx) {
+  std::lock_guard<std::mutex> lock(g_order_mutex);
+  DeviceOrder &o = g_order[ctx->device >= 0 && ctx->device < 64 ? ctx->device : 0];
+  if (!o.recorded || o.stream != ctx->stream) return;
+  // nothing of this stream is still running (the caller synchronized it): a later launch from another stream
+  // has nothing to wait for, and must not touch a stream handle that may be gone by then
+  o.recorded = false;
+  o.stream = nullptr;
+}
+
 // After the stream has been synchronized: did a panel kernel give up?  Then the launch's results are not
 // valid; the state words are cleared and the context stays on the multi-launch path.
 int panel_check(dlmi_ctx *ctx) {

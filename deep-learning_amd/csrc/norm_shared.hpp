@@ -101,6 +101,7 @@ struct FwdTrainCall {
   float *mean, *stdv, *mov_mean, *mov_std, *r, *d, *y, *xhat, *nrm;
   float const *partial_in = nullptr;  // column-sum partials already produced elsewhere ...
   unsigned partial_chunks = 0;        // ... [2][partial_chunks][H]; skips the statistics pass
+  float const *snapshot_in = nullptr;  // ... and the moving statistics before this step [2][H], copied by the same producer
   // x itself not formed yet: it is the sum of `nslices` partial products [nslices][B][H] (split-K slices), to
   // be added in slice order and stored to z_out (== x) by the small-batch kernel, the only one that takes them
   float const *slices = nullptr;

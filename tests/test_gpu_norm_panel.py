@@ -179,3 +179,25 @@ def test_backward_panel_against_float64(twins, pkg):
     assert_close(g["dgamma"], 0.25 + (dn * xh).sum(0), 1e-4, "dgamma", floor=1.0)
     assert_close(g["dbeta"], -0.5 + dn.sum(0), 1e-4, "dbeta", floor=1.0)
     assert np.max(np.abs(g["dx"].astype(np.float64).sum(0))) < 1e-2  # sum_b dX = 0 up to rounding of 4096 terms
+
+
+def test_a_destroyed_stream_is_not_touched_by_the_next_launch(twins, pkg):
+    """Launches of different streams are ordered through the stream of the previous launch.  A model owns its
+    stream and destroys it when it is closed: the next launch, from another stream, must not look at it."""
+    from deep_learning_amd.model import Model
+    from oracle.binding import NORM, STATE
+    panel, _ = twins
+    M = Model(pkg.load_library(), [64, 1024, 4])
+    M.set_layer(1, ACT["RELU"], NORM["BRN"])
+    M.set_layer(2, ACT["SOFTMAX"])
+    M.set_norm_hyper(0.99, 1e-5, 3.0, 5.0)
+    M.prepare(1024)
+    M.glorot_uniform(1)
+    rng = np.random.default_rng(0)
+    Y = np.zeros((1024, 4), np.float32)
+    Y[:, 0] = 1.0
+    M.step(STATE["TRAINING"], rng.standard_normal((1024, 64), dtype=np.float32), Y)  # [1024 x 1024]: a panel launch
+    M.close()
+    d = make(1024, 1024, 3)
+    a, *_ = run_fwd(panel, pkg, d, "RELU", "NONE", False, False)
+    assert np.isfinite(a["y"]).all()
