@@ -97,9 +97,17 @@ struct TileShape {
   }
 };
 
+// How a kernel variant treats the edges of its operands.
+//   kGuarded  any shape and alignment: every piece checked, element by element where it crosses an edge
+//   kFast     M, N, K multiples of the tile, 16-byte aligned operands: no checks at all
+//   kClamped  K a multiple of BK and aligned operands, but M or N ragged (a layer of 784 or 10 units): the loads
+//             of rows beyond the operand are redirected to its last rows (always in bounds, still one 16-byte
+//             load each, so the K loop is the fast one) and their products are dropped by the guarded stores
+enum : int { kGuarded = 0, kFast = 1, kClamped = 2 };
+
 // Global -> registers for one operand tile.  `row0` is the tile's first row
-// (m or n), `k0` its first k.  FAST: whole tile in bounds, 16-byte aligned.
-template <int ROWS, int BK, bool KCONTIG, bool FAST>
+// (m or n), `k0` its first k.
+template <int ROWS, int BK, bool KCONTIG, int MODE>
 __device__ __forceinline__ typename TileShape<ROWS, BK, KCONTIG>::Regs tile_load(float const *__restrict__ P,
                                                                                size_t ld, size_t row0, size_t k0,
                                                                                size_t rows_total, size_t k_end,
@@ -110,10 +118,16 @@ __device__ __forceinline__ typename TileShape<ROWS, BK, KCONTIG>::Regs tile_load
   for (int i = 0; i < T::kPerThread; ++i) {
     int tr, tk;
     T::piece(threadIdx.x + i * kGemmThreads, tr, tk);
-    size_t const row = row0 + tr, k = k0 + tk;
+    size_t row = row0 + tr;
+    size_t const k = k0 + tk;
+    if constexpr (MODE == kClamped) {
+      // a k-contiguous piece lies in one row, the other kind covers 4 consecutive rows (rows_total % 4 == 0)
+      size_t const last = KCONTIG ? rows_total - 1 : rows_total - 4;
+      row = row < last ? row : last;
+    }
     float const *src = KCONTIG ? P + row * ld + k : P + k * ld + row;
     v4f t;
-    if constexpr (FAST) {
+    if constexpr (MODE != kGuarded) {
       (void)vec_ok;
       t = *reinterpret_cast<v4f const *>(src);
     } else {
@@ -183,9 +197,11 @@ __device__ __forceinline__ void sched_spread() {
   }
 }
 
-template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, bool FAST, int WAVES_PER_EU>
+template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int WAVES_PER_EU>
 __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
 void k_gemm_f32(GemmArgs g) {
+  constexpr bool FAST = MODE == kFast;          // no edge anywhere: unguarded stores
+  constexpr bool FAST_LOOP = MODE != kGuarded;  // the scheduled K loop
   using TA = TileShape<BM, BK, A_KCONTIG>;
   using TB = TileShape<BN, BK, B_KCONTIG>;
   constexpr int WM = BM / 2, WN = BN / 2;  // wavefront tile
@@ -257,13 +273,13 @@ void k_gemm_f32(GemmArgs g) {
     // stage and the writes of the next - the first fragments of tile kt+1 are
     // read.  LDS and memory traffic is spread between the MFMAs, so the matrix
     // pipe only waits at the barrier itself.
-    typename TA::Regs ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, k_begin, g.M, k_end, g.a_vec != 0);
-    typename TB::Regs rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, k_begin, g.N, k_end, g.b_vec != 0);
+    typename TA::Regs ra = tile_load<BM, BK, A_KCONTIG, MODE>(g.A, g.lda, m0, k_begin, g.M, k_end, g.a_vec != 0);
+    typename TB::Regs rb = tile_load<BN, BK, B_KCONTIG, MODE>(g.B, g.ldb, n0, k_begin, g.N, k_end, g.b_vec != 0);
     tile_store<BM, BK, A_KCONTIG>(lds, ra);
     tile_store<BN, BK, B_KCONTIG>(lds + TA::kFloats, rb);
     if (ktiles > 1) {
-      ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, k_begin + BK, g.M, k_end, g.a_vec != 0);
-      rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, k_begin + BK, g.N, k_end, g.b_vec != 0);
+      ra = tile_load<BM, BK, A_KCONTIG, MODE>(g.A, g.lda, m0, k_begin + BK, g.M, k_end, g.a_vec != 0);
+      rb = tile_load<BN, BK, B_KCONTIG, MODE>(g.B, g.ldb, n0, k_begin + BK, g.N, k_end, g.b_vec != 0);
     }
     __syncthreads();
     v4f f0a[TM], f0b[TN];
@@ -283,11 +299,11 @@ void k_gemm_f32(GemmArgs g) {
       }
       if constexpr (LOAD) {
         size_t const kn = k_begin + static_cast<size_t>(kt + 2) * BK;
-        ra = tile_load<BM, BK, A_KCONTIG, FAST>(g.A, g.lda, m0, kn, g.M, k_end, g.a_vec != 0);
-        rb = tile_load<BN, BK, B_KCONTIG, FAST>(g.B, g.ldb, n0, kn, g.N, k_end, g.b_vec != 0);
+        ra = tile_load<BM, BK, A_KCONTIG, MODE>(g.A, g.lda, m0, kn, g.M, k_end, g.a_vec != 0);
+        rb = tile_load<BN, BK, B_KCONTIG, MODE>(g.B, g.ldb, n0, kn, g.N, k_end, g.b_vec != 0);
       }
       steps(f1a, f1b, 0, 2);
-      if constexpr (FAST) {
+      if constexpr (FAST_LOOP) {
         sched_spread<NM / 8, 0x100, NFR>();
         sched_spread<NM / 4, 0x200, STORE ? NWR : 0>();
         sched_spread<NM / 4, 0x020, LOAD ? NLD : 0>();
@@ -298,7 +314,7 @@ void k_gemm_f32(GemmArgs g) {
         frags(na, na + TA::kFloats, 0, f0a, f0b);
       }
       steps(f1a, f1b, 2, 4);
-      if constexpr (FAST && STORE) {
+      if constexpr (FAST_LOOP && STORE) {
         sched_group<0x100, NFR>();
         sched_group<0x008, NM / 4>();
       }
@@ -404,16 +420,19 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(float const *__restrict__
 }
 
 // ---------------------------------------------------------------- host side
-template <int BM, int BN, int BK, bool AK, bool BKC, int WPE>
-static int launch_gemm(dlmi_ctx *ctx, GemmArgs g, unsigned splits, bool fast) {
+template <int BM, int BN, int BK, bool AK, bool BKC, int WPE, bool HAS_CLAMPED>
+static int launch_gemm(dlmi_ctx *ctx, GemmArgs g, unsigned splits, int mode) {
   using TA = TileShape<BM, BK, AK>;
   using TB = TileShape<BN, BK, BKC>;
   constexpr size_t lds_bytes = 2 * (TA::kFloats + TB::kFloats) * sizeof(float);
   g.tiles_m = static_cast<unsigned>(dlmi_ceil_div(g.M, BM));
   g.tiles_n = static_cast<unsigned>(dlmi_ceil_div(g.N, BN));
   dim3 const grid(g.tiles_m * g.tiles_n, 1, splits);
-  auto const kfast = k_gemm_f32<BM, BN, BK, AK, BKC, true, WPE>;
-  auto const kslow = k_gemm_f32<BM, BN, BK, AK, BKC, false, WPE>;
+  auto const kfast = k_gemm_f32<BM, BN, BK, AK, BKC, kFast, WPE>;
+  auto const kslow = k_gemm_f32<BM, BN, BK, AK, BKC, kGuarded, WPE>;
+  // the clamped variant exists for the small tiles, which are the ones ragged layers run
+  auto const kclamp = k_gemm_f32<BM, BN, BK, AK, BKC, HAS_CLAMPED ? kClamped : kGuarded, WPE>;
+  if (!HAS_CLAMPED && mode == kClamped) mode = kGuarded;
   // more than 64 KB of LDS has to be asked for once per kernel and device
   static bool attr_set_on[64] = {false};
   bool &attr_set = attr_set_on[ctx->device >= 0 && ctx->device < 64 ? ctx->device : 0];
@@ -422,10 +441,14 @@ static int launch_gemm(dlmi_ctx *ctx, GemmArgs g, unsigned splits, bool fast) {
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     DLMI_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<void const *>(kslow),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+    DLMI_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<void const *>(kclamp),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     attr_set = true;
   }
-  if (fast)
+  if (mode == kFast)
     hipLaunchKernelGGL(kfast, grid, dim3(kGemmThreads), lds_bytes, ctx->stream, g);
+  else if (mode == kClamped)
+    hipLaunchKernelGGL(kclamp, grid, dim3(kGemmThreads), lds_bytes, ctx->stream, g);
   else
     hipLaunchKernelGGL(kslow, grid, dim3(kGemmThreads), lds_bytes, ctx->stream, g);
   DLMI_LAUNCH_CHECK(ctx, "k_gemm_f32");
@@ -558,7 +581,13 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   if (snap_out != nullptr) *snap_out = nullptr;
   g.a_vec = (lda % 4 == 0 && dlmi_aligned16(A)) ? 1 : 0;
   g.b_vec = (ldb % 4 == 0 && dlmi_aligned16(B)) ? 1 : 0;
-  bool const fast = M % bm == 0 && N % bn == 0 && K % bk == 0 && g.a_vec && g.b_vec;
+  int mode = kGuarded;
+  if (K % bk == 0 && g.a_vec && g.b_vec) {
+    if (M % bm == 0 && N % bn == 0)
+      mode = kFast;
+    else if ((AK || M % 4 == 0) && (BKC || N % 4 == 0) && M >= 4 && N >= 4)
+      mode = kClamped;
+  }
   size_t const ktiles = dlmi_ceil_div(K, bk);
   unsigned splits = plan.splits;
   if (splits > 1) {
@@ -590,10 +619,10 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   if (splits > 1) g.split_out = reinterpret_cast<float *>(dlmi_scratch_data(ctx));
   int rc;
   switch (choice) {
-    case 1: rc = launch_gemm<256, 128, 16, AK, BKC, 2>(ctx, g, splits, fast); break;
-    case 2: rc = launch_gemm<256, 256, 16, AK, BKC, 1>(ctx, g, splits, fast); break;
-    case 3: rc = launch_gemm<64, 64, 16, AK, BKC, 4>(ctx, g, splits, fast); break;
-    default: rc = launch_gemm<128, 128, 16, AK, BKC, 2>(ctx, g, splits, fast); break;
+    case 1: rc = launch_gemm<256, 128, 16, AK, BKC, 2, false>(ctx, g, splits, mode); break;
+    case 2: rc = launch_gemm<256, 256, 16, AK, BKC, 1, false>(ctx, g, splits, mode); break;
+    case 3: rc = launch_gemm<64, 64, 16, AK, BKC, 4, true>(ctx, g, splits, mode); break;
+    default: rc = launch_gemm<128, 128, 16, AK, BKC, 2, true>(ctx, g, splits, mode); break;
   }
   if (rc != DLMI_OK) return rc;
   if (defer_slices != nullptr) {
