@@ -142,7 +142,10 @@ def test_per_unit_activation_types_refuse_an_unsupported_type(dl):
 # ------------------------------------------------------------------ GEMMs against the oracle
 GEMM_SHAPES = [  # (B, K, H): tile-aligned (fast path) and ragged (guarded path)
     (128, 128, 128), (256, 64, 384), (384, 256, 128), (1, 1, 1), (7, 13, 5), (130, 70, 129), (128, 784, 512),
-    (128, 512, 10), (33, 1000, 17), (512, 16, 256)]
+    (128, 512, 10), (33, 1000, 17), (512, 16, 256),
+    # ragged M or N behind a K that is a multiple of 16: the clamped variant (rows beyond the operand are loaded
+    # from its last rows and dropped at the store); 18 is not a multiple of 4: back to the guarded one
+    (100, 64, 36), (100, 36, 64), (96, 20, 48), (96, 18, 48), (4, 16, 4), (64, 16, 8), (208, 784, 144), (272, 160, 200)]
 
 
 @pytest.mark.parametrize("B,K,H", GEMM_SHAPES)
