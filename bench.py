@@ -49,6 +49,31 @@ MEASURED_TRAFFIC_BYTES = {
     "c3": {"gemm": (897.8 + 897.3 + 832.8) / 3.0 * MIB, "norm_act": 901.8 * MIB},
     "c2": {"norm_act": 326.4 * MIB},
 }
+# The figures above belong to the kernels as they were when the counters were read: the digest of their
+# sources at that time (`python bench.py --traffic-digest` prints the current one).  When a source has
+# changed since, `traffic` is reported as null instead of a figure that may no longer hold.
+TRAFFIC_SOURCES = ("gemm_f32_mfma.hip", "norm_kernels.hip", "norm_panel_fwd.hip", "norm_panel_bwd.hip",
+                   "norm_panel_common.hpp", "norm_shared.hpp", "activations.hpp", "dlmi_common.hpp")
+TRAFFIC_SOURCES_SHA256 = "ed22eb20d4b82daa51481cd3b8dfce55111d6ae46a1827ff382a8233fbe2ced9"
+
+
+def traffic_sources_digest():
+    import hashlib
+    h = hashlib.sha256()
+    for name in TRAFFIC_SOURCES:
+        with open(os.path.join(ROOT, "deep-learning_amd", "csrc", name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()
+
+
+def measured_traffic(workload, key):
+    """(bytes, source) for the roofline's `traffic`: the profile's figure while the kernels are the measured ones."""
+    v = MEASURED_TRAFFIC_BYTES.get(workload, {}).get(key)
+    if v is None:
+        return None, None
+    if traffic_sources_digest() != TRAFFIC_SOURCES_SHA256:
+        return None, "not reported: the kernel sources have changed since %s was taken" % TRAFFIC_PROFILE
+    return v, TRAFFIC_PROFILE
 
 
 # ---------------------------------------------------------------- helpers
@@ -373,9 +398,9 @@ def run_layer(args, torch, pkg, dl, name, full):
     E = B * H
     t_nf = time_events(torch, step.norm_fwd, 20)
     t_nb = time_events(torch, step.norm_bwd, 20)
+    norm_traffic, norm_traffic_source = measured_traffic(name, "norm_act")
     hbm = {"bound": "hbm", "achieved": 32.0 * E / ((t_nf + t_nb) * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-           "traffic": MEASURED_TRAFFIC_BYTES.get(name, {}).get("norm_act"),
-           "traffic_source": TRAFFIC_PROFILE if name in MEASURED_TRAFFIC_BYTES else None,
+           "traffic": norm_traffic, "traffic_source": norm_traffic_source,
            "kernels": "dlmi_fused_norm_act_fwd + dlmi_fused_norm_act_bwd; `achieved` counts the two-pass accounting "
                       "of 12 + 20 B/element.  Batches of 1024-8192 rows (forward) / 2048-4096 rows (backward) with a "
                       "width that is a multiple of 1024 run the single-launch panel kernels, which read every tensor "
@@ -390,9 +415,9 @@ def run_layer(args, torch, pkg, dl, name, full):
         t_gw = time_events(torch, step.gemm_dw_only, 10)
         flops = 2.0 * B * K * H
         avg = (t_gf + t_gx + t_gw) / 3.0
+        gemm_traffic, gemm_traffic_source = measured_traffic(name, "gemm")
         roof = {"bound": "mfma", "achieved": flops / (avg * 1e-3) / 1e12, "peak": MFMA_FP32_PEAK_TFLOPS,
-                "unit": "TFLOP/s", "traffic": MEASURED_TRAFFIC_BYTES.get(name, {}).get("gemm"),
-                "traffic_source": TRAFFIC_PROFILE if name in MEASURED_TRAFFIC_BYTES else None,
+                "unit": "TFLOP/s", "traffic": gemm_traffic, "traffic_source": gemm_traffic_source,
                 "kernel": "k_gemm_f32 (avg of fwd NT, dX NN, dW TN launches)",
                 "tflops_fwd": flops / (t_gf * 1e-3) / 1e12, "tflops_dx": flops / (t_gx * 1e-3) / 1e12,
                 "tflops_dw": flops / (t_gw * 1e-3) / 1e12}
@@ -686,7 +711,12 @@ def main():
                                                "--steps times and exit without a JSON line")
     ap.add_argument("--shape", default="", help="profiling aid, with --only: B,K,H of the layer to run the part on instead "
                                                 "of a workload's (e.g. 1024,2048,2048: one block of c4)")
+    ap.add_argument("--traffic-digest", action="store_true", help="print the digest of the kernel sources the "
+                                                                  "`traffic` figures are tied to and exit")
     args = ap.parse_args()
+    if args.traffic_digest:
+        print(traffic_sources_digest())
+        return
     args.steps_given = args.steps is not None
     args.steps = 20 if args.steps is None else args.steps
     args.warmup = 3 if args.warmup is None else args.warmup
