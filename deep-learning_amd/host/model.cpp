@@ -17,6 +17,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <exception>
 #include <limits>
 #include <string>
 #include <thread>
@@ -199,7 +200,11 @@ float const *Model::Impl::slots_upload(RowSlots &s, size_t const B, size_t const
       }
     };
     std::vector<std::thread> pool;
-    for (unsigned t = 1; t < threads; ++t) pool.emplace_back(work, true);
+    try {
+      for (unsigned t = 1; t < threads; ++t) pool.emplace_back(work, true);
+    } catch (std::exception const &) {
+      // no more threads to be had: the ones that started and this one share the pieces
+    }
     work(false);
     for (std::thread &t : pool) t.join();
     first_bad = static_cast<hipError_t>(bad.load());
