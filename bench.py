@@ -494,16 +494,44 @@ def run_c4(args, torch, pkg, dl):
     dWs = [torch.empty(H, H, **dev) for _ in range(nblk)]
     dgs, dbs = [zero.clone() for _ in range(nblk)], [zero.clone() for _ in range(nblk)]
     dZ, g = torch.empty(B, H, **dev), torch.empty(B, H, **dev)
+    # The weight gradient of a block depends on nothing that follows it, so it runs on a second stream (a context
+    # of its own: its scratch) beside the chain dX -> normalization backward of the block below -> ...: a product
+    # of this size leaves the matrix pipes idle for 15-20 % of its launch (dispatch, first operands, stores), which
+    # the other stream's product fills (dX + dW of one block: 145 us one after the other, 129 us side by side).
+    # dZ alternates between two buffers; an event per buffer says when the weight gradient has read it.
+    two_streams = args.c4_streams == 2
+    main = torch.cuda.current_stream()
+    side = torch.cuda.Stream() if two_streams else None  # default priority
+    dl_side = pkg.Dlmi(0) if two_streams else None
+    if two_streams:
+        dl_side.set_stream(side)
+    dZs = [dZ, torch.empty(B, H, **dev)] if two_streams else [dZ, dZ]
+    ready = [torch.cuda.Event(), torch.cuda.Event()]
+    read = [torch.cuda.Event(), torch.cuda.Event()]
+    used = [False, False]
 
     def step():
         for i in range(nblk):
             dl.fc_norm_act_fwd(desc, xs[i], Ws[i], one, zero, mm[i], ms[i], mask=mask[i], Z=Zs[i], out=xs[i + 1],
                                stats=stats[i], shortcut=xs[i])
         g.copy_(dOut)
-        for i in reversed(range(nblk)):
-            dl.fused_bwd(desc, Zs[i], one, zero, stats[i], g, dgs[i], dbs[i], mask=mask[i], out=dZ)
-            dl.fc_bwd_dx(dZ, Ws[i], out=g, accumulate=True)  # the shortcut carries g on, the block adds dZ W
-            dl.fc_bwd_dw(xs[i], dZ, dW=dWs[i])
+        for k, i in enumerate(reversed(range(nblk))):
+            b = k & 1
+            if two_streams and used[b]:
+                main.wait_event(read[b])  # the weight gradient two blocks up has read this buffer
+            dl.fused_bwd(desc, Zs[i], one, zero, stats[i], g, dgs[i], dbs[i], mask=mask[i], out=dZs[b])
+            if two_streams:
+                ready[b].record(main)
+            dl.fc_bwd_dx(dZs[b], Ws[i], out=g, accumulate=True)  # the shortcut carries g on, the block adds dZ W
+            if two_streams:
+                side.wait_event(ready[b])
+                dl_side.fc_bwd_dw(xs[i], dZs[b], dW=dWs[i])
+                read[b].record(side)
+                used[b] = True
+            else:
+                dl.fc_bwd_dw(xs[i], dZs[b], dW=dWs[i])
+        if two_streams:
+            main.wait_stream(side)  # the step ends when both streams have
 
     step()
     torch.cuda.synchronize()
@@ -573,7 +601,10 @@ def run_c4(args, torch, pkg, dl):
         parity = parity_block({k: (gpu[k], ref[k]) for k in ref}, 1e-3)
     config = {"workload": "c4: 16 residual blocks x + Dropout(ISRLU(BRN(FC x))), width 2048, batch 1024, "
                           "uint8 keep-mask per element, fwd+bwd", "batch": B, "units": H, "blocks": nblk,
-              "norm": NORM_TEXT, "inputs": "resident in HBM"}
+              "norm": NORM_TEXT, "inputs": "resident in HBM",
+              "streams": "2: weight gradients on a second stream beside the backward chain" if two_streams else "1"}
+    if two_streams:
+        dl_side.close()
     return line(B / (ms_step * 1e-3), ms_step, args.steps, args.warmup, config, roof, hbm, cpu, detail, parity)
 
 
@@ -704,6 +735,8 @@ def main():
                                                             "then take as many as make a sustained load)")
     ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default 3)")
     ap.add_argument("--workload", default="all", choices=["all", "c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--c4-streams", type=int, default=2, choices=[1, 2],
+                    help="workload c4: 2 = the weight gradients run on a second stream beside the backward chain")
     ap.add_argument("--cpu-rows", type=int, default=-1, help="rows of the CPU baseline sample (0 = skip the CPU legs "
                                                              "and the in-run parity check)")
     ap.add_argument("--only", default="", help="profiling aid (layer workloads): run just this part (gemm_fwd, gemm_dx, "

@@ -138,9 +138,9 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
       a.part[((static_cast<size_t>(who.xcd) * npanels + p) * kPanelRanks + who.rank) * kVals + w * kP + c] = t;
     }
   };
-  auto arrive = [&]() {
+  auto arrive = [&](int p) {
     __syncthreads();
-    if (threadIdx.x == 0) panel_count(who.st + 1);
+    if (threadIdx.x == 0) panel_count(panel_arrivals(who, p));
   };
   auto finish = [&](Stage const &s, int p) -> bool {
     size_t const col = col_base + static_cast<size_t>(p) * kP;
@@ -153,7 +153,7 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
           old[i] = __builtin_nontemporal_load(reinterpret_cast<pv4f const *>(a.dX + off0 + static_cast<size_t>(i) * kTY * a.H));
       }
     }
-    if (threadIdx.x == 0 && !panel_wait(who, static_cast<unsigned>(kPanelRanks) * (p + 1))) s_ok = 0;
+    if (threadIdx.x == 0 && !panel_wait(who, p)) s_ok = 0;
     __syncthreads();
     if (!s_ok) return false;
     if (threadIdx.x < kRSplit * kVals) {
@@ -221,7 +221,7 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
   if (npanels > 2) load(b2, 2);
   publish(b0, 0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  arrive();
+  arrive(0);
   if (npanels > 1) publish(b1, 1);
   bool const elem = EXTRA && a.drop_mode == kDropElem;
   auto step = [&](Stage &cur, Stage &s1, Stage &s2, Stage &s3, int p) -> bool {
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
     } else if (p + 1 < npanels) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(RPT) : "memory");
     }
-    if (p + 1 < npanels) arrive();
+    if (p + 1 < npanels) arrive(p + 1);
     if (p + 2 < npanels) publish(s2, p + 2);
     return finish(cur, p);
   };

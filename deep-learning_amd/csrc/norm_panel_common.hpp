@@ -34,8 +34,14 @@ constexpr int kPanelRanks = 32;   // workgroups per XCD
 constexpr int kPanelXcds = 8;
 constexpr int kPanelThreads = 512;
 constexpr int kPanelSpinLimit = 1 << 20;
-// words of the barrier state: [xcd][16] = { rank ticket, arrivals, departures, abort }.  Every word is only
-// ever touched by the workgroups of its own XCD (the L2s of different XCDs are not coherent inside a kernel).
+// words of the barrier state: [xcd][16] = { rank ticket, arrivals at even panels, departures, abort, arrivals
+// at odd panels }.  Every word is only ever touched by the workgroups of its own XCD (the L2s of different XCDs
+// are not coherent inside a kernel).
+// Why two arrival words: a workgroup counts itself in for panel p+1 before it waits for panel p, so one
+// running total could reach 32 (p+1) on the arrivals of the workgroups that are ahead while another has not
+// arrived for p at all (one that started late because its CU was still held by another kernel).  With one word
+// per panel parity an arrival for p+2 can only come from a workgroup that has finished p+1, i.e. after all 32
+// have arrived for p+1 and therefore for p: the first 32 (p/2+1) arrivals on a word are those for panels <= p.
 constexpr int kPanelStateStride = 16;
 constexpr int kPanelStateWords = kPanelXcds * kPanelStateStride;
 
@@ -81,10 +87,13 @@ __device__ __forceinline__ bool panel_enter(unsigned *state, PanelWho &w, unsign
   }
   return true;
 }
-// Thread 0 waits until `target` arrivals have been counted on this XCD.  Returns false after the spin limit.
-__device__ __forceinline__ bool panel_wait(PanelWho const &w, unsigned target) {
+__device__ __forceinline__ unsigned *panel_arrivals(PanelWho const &w, int p) { return w.st + ((p & 1) ? 4 : 1); }
+// Thread 0 waits until all workgroups of this XCD have arrived for panel p.  Returns false after the spin limit.
+__device__ __forceinline__ bool panel_wait(PanelWho const &w, int p) {
+  unsigned const target = static_cast<unsigned>(kPanelRanks) * static_cast<unsigned>(p / 2 + 1);
+  unsigned *const word = panel_arrivals(w, p);
   int spins = 0;
-  while (panel_poll(w.st + 1) < target) {
+  while (panel_poll(word) < target) {
     if (++spins > kPanelSpinLimit || (spins % 1024 == 0 && panel_poll(w.st + 3) != 0)) {
       panel_count(w.st + 3);
       return false;
@@ -101,6 +110,7 @@ __device__ __forceinline__ void panel_leave(PanelWho const &w) {
       w.st[0] = 0;
       w.st[1] = 0;
       w.st[2] = 0;
+      w.st[4] = 0;
     }
   }
 }

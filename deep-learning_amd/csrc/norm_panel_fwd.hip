@@ -82,9 +82,9 @@ __global__ __launch_bounds__(kPanelThreads) void k_fwd_panel(PanelFwdArgs a) {
       snap[p & 1][w][c] = w == 0 ? a.fin.mov_mean[col + c] : a.fin.mov_std[col + c];
     }
   };
-  auto arrive = [&]() {
+  auto arrive = [&](int p) {
     __syncthreads();
-    if (threadIdx.x == 0) panel_count(who.st + 1);
+    if (threadIdx.x == 0) panel_count(panel_arrivals(who, p));
   };
   // wait for the XCD, finish the statistics of panel p and apply them to the rows in registers
   auto finish = [&](pv4f const (&buf)[RPT], int p) -> bool {
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(kPanelThreads) void k_fwd_panel(PanelFwdArgs a) {
     pv4f be = *reinterpret_cast<pv4f const *>(a.beta + col + tx * 4);
     uchar4 um = make_uchar4(1, 1, 1, 1);
     if (a.drop_mode == kDropUnit) um = *reinterpret_cast<uchar4 const *>(a.mask + col + tx * 4);
-    if (threadIdx.x == 0 && !panel_wait(who, static_cast<unsigned>(kPanelRanks) * (p + 1))) s_ok = 0;
+    if (threadIdx.x == 0 && !panel_wait(who, p)) s_ok = 0;
     __syncthreads();
     if (!s_ok) return false;
     {
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(kPanelThreads) void k_fwd_panel(PanelFwdArgs a) {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(RPT) : "memory");  // the partial is older than the RPT loads of panel 1
   else
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  arrive();
+  arrive(0);
   auto step = [&](pv4f (&cur)[RPT], pv4f (&mid)[RPT], pv4f (&nxt)[RPT], int p) -> bool {
     if (p + 1 < npanels) {
       publish(mid, p + 1);
@@ -188,7 +188,7 @@ __global__ __launch_bounds__(kPanelThreads) void k_fwd_panel(PanelFwdArgs a) {
       } else {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       }
-      arrive();
+      arrive(p + 1);
     }
     return finish(cur, p);
   };

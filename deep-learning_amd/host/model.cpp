@@ -16,6 +16,7 @@
 #include <atomic>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <exception>
 #include <limits>
@@ -48,6 +49,19 @@ struct Model::Impl {
   };
   RowSlots in_rows, tgt_rows;
   hipStream_t up_stream = nullptr;  // copy stream of the two (default priority)
+  // The weight gradients of update_derivatives() depend on nothing that follows them in the backward pass, so
+  // they run on a stream (and context: scratch) of their own beside the chain dX -> gradient of the layer below
+  // -> ...: a product of a few GFLOP leaves the matrix pipes idle for 15-20 % of its launch (dispatch, first
+  // operands, stores), which the other stream's kernels fill.  backward_pass() records an event per layer when
+  // that layer's dZ is final; update_derivatives() makes the side stream wait for it, and the compute stream
+  // for the side stream's last product.  DLMI_DW_STREAM=0 keeps everything on the compute stream.
+  hipStream_t dw_stream = nullptr;
+  dlmi_ctx *dw_ctx = nullptr;
+  std::vector<hipEvent_t> dz_ready;  // per layer
+  hipEvent_t dw_done = nullptr;
+  void record_dz_ready(size_t layer) {
+    if (dw_ctx != nullptr && layer < dz_ready.size()) (void)hipEventRecord(dz_ready[layer], stream);
+  }
   bool slots_alloc(RowSlots &s, size_t floats);
   void slots_free_device(RowSlots &s);
   void slots_free_all(RowSlots &s);
@@ -237,8 +251,11 @@ void Model::clear(void) {
   if (impl_->up_stream != nullptr) (void)hipStreamSynchronize(impl_->up_stream);
   impl_->slots_free_all(impl_->in_rows);
   impl_->slots_free_all(impl_->tgt_rows);
+  if (impl_->dw_ctx != nullptr) (void)dlmi_ctx_destroy(impl_->dw_ctx);
+  for (hipEvent_t e : impl_->dz_ready) (void)hipEventDestroy(e);
+  if (impl_->dw_done != nullptr) (void)hipEventDestroy(impl_->dw_done);
   if (impl_->ctx != nullptr) (void)dlmi_ctx_destroy(impl_->ctx);
-  hipStream_t const stream = impl_->stream, up_stream = impl_->up_stream;
+  hipStream_t const stream = impl_->stream, up_stream = impl_->up_stream, dw_stream = impl_->dw_stream;
   size_t const n_errors = impl_->n_errors;
   Dist::Bernoulli *const masks = bernoulli;
   delete[] ptr_array_layers;
@@ -250,6 +267,7 @@ void Model::clear(void) {
   *impl = Impl();
   impl->stream = stream;
   impl->up_stream = up_stream;
+  impl->dw_stream = dw_stream;
   impl->n_errors = n_errors;
   static_cast<Model_State &>(*this) = Model_State();  // every public member takes its default again
   real_gen.seed(5489u);
@@ -260,6 +278,7 @@ Model::~Model(void) {
   clear();
   if (impl_->stream != nullptr) (void)hipStreamDestroy(impl_->stream);
   if (impl_->up_stream != nullptr) (void)hipStreamDestroy(impl_->up_stream);
+  if (impl_->dw_stream != nullptr) (void)hipStreamDestroy(impl_->dw_stream);
   delete[] bernoulli;
   delete impl_;
 }
@@ -281,6 +300,8 @@ bool Model::reserve_for(size_t const batch) {
     Layer &l = ptr_array_layers[i];
     size_t const K = l.type_layer == LAYER::RESIDUAL ? 0 : (l.in_block ? l.n_inp : ptr_array_layers[i - 1].n_out);
     if (dlmi_ctx_reserve_layer(impl_->ctx, batch, K, l.n_out) != DLMI_OK) return fail("reserve_for: dlmi_ctx_reserve_layer");
+    if (impl_->dw_ctx != nullptr && dlmi_ctx_reserve_layer(impl_->dw_ctx, batch, K, l.n_out) != DLMI_OK)
+      return fail("reserve_for: dlmi_ctx_reserve_layer (weight-gradient stream)");
     // normalization after the activation keeps the activation values: the order is a public member that
     // may have been flipped since allocate_batch()
     if (l.type_layer != LAYER::RESIDUAL && !l.in_block && l.Use__Normalization() &&
@@ -345,6 +366,22 @@ bool Model::compile(size_t const n_layers, size_t const number_recurrent_depth_r
   }
   if (dlmi_ctx_create(&impl_->ctx, 0, impl_->stream) != DLMI_OK)
     return fail("compile: no gfx950 device / context (there is no CPU path)");
+  {
+    char const *const e = std::getenv("DLMI_DW_STREAM");
+    bool const side = e == nullptr || std::atoi(e) != 0;
+    if (side && impl_->dw_stream == nullptr && hipStreamCreateWithFlags(&impl_->dw_stream, hipStreamNonBlocking) != hipSuccess) {
+      (void)hipGetLastError();
+      impl_->dw_stream = nullptr;
+    }
+    if (side && impl_->dw_stream != nullptr) {
+      bool ok = dlmi_ctx_create(&impl_->dw_ctx, 0, impl_->dw_stream) == DLMI_OK &&
+                hipEventCreateWithFlags(&impl_->dw_done, hipEventDisableTiming) == hipSuccess;
+      impl_->dz_ready.assign(n_layers, nullptr);
+      for (size_t i = 0; ok && i < n_layers; ++i)
+        ok = hipEventCreateWithFlags(&impl_->dz_ready[i], hipEventDisableTiming) == hipSuccess;
+      if (!ok) return fail("compile: no stream / events for the weight gradients");
+    }
+  }
   type = type_network_received;
   // the reference budgets host memory (model.hpp:2528); here the same number budgets device memory.
   // 0: all of the device's memory.
@@ -1270,6 +1307,8 @@ uint64_t Model::launch_signature(void) const {
   // keeps working (a retired block stays allocated) but is made again, so that every launch uses the same block
   unsigned long long const scratch_generation = dlmi_ctx_scratch_generation(impl_->ctx);
   DLMI_MIX(scratch_generation);
+  unsigned long long const dw_scratch_generation = impl_->dw_ctx != nullptr ? dlmi_ctx_scratch_generation(impl_->dw_ctx) : 0ull;
+  DLMI_MIX(dw_scratch_generation);
   DLMI_MIX(type_loss_function); DLMI_MIX(type_accuracy_function); DLMI_MIX(acc_var);
   DLMI_MIX(normalization_momentum_average); DLMI_MIX(normalization_epsilon);
   DLMI_MIX(batch_renormalization_r_correction_maximum); DLMI_MIX(batch_renormalization_d_correction_maximum);
@@ -1371,7 +1410,9 @@ void Model::backward_pass(size_t const B) {
   for (size_t li = total_layers - 1; li >= 1; --li) {
     Layer &l = ptr_array_layers[li];
     if (l.in_block) {
+      size_t const last_of_block = li;
       if (!backward_block(B, l.block_index)) return;
+      for (size_t k = l.block_index; k <= last_of_block; ++k) impl_->record_dz_ready(k);  // the block's layers at once
       li = l.block_index;
       if (li == 1) break;
       continue;
@@ -1407,6 +1448,7 @@ void Model::backward_pass(size_t const B) {
                         l.d_errors, l.d_errors);
     }
     if (rc != DLMI_OK) { fail("backward_pass: layer gradient"); return; }
+    impl_->record_dz_ready(li);  // this layer's dZ is final: its weight gradient may start
     // dY = dZ . W, written straight over the (would-be zeroed) buffer of the entry this layer reads
     if (l.feed_index != 0) {
       Layer &f = ptr_array_layers[l.feed_index];
@@ -1494,7 +1536,12 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
     fail("update_derivatives: bad argument");
     return;
   }
-  for (Layer *l = first; l != last; ++l) {
+  // from the last layer down: the order in which the backward pass finishes their gradients (every layer adds
+  // into its own part of the gradient array, so the order does not change the sums)
+  bool const side = impl_->dw_ctx != nullptr;
+  dlmi_ctx *const ctx = side ? impl_->dw_ctx : impl_->ctx;
+  for (Layer const *l = last; l != first;) {
+    --l;
     size_t const li = static_cast<size_t>(l - ptr_array_layers);
     if (li == 0 || li >= total_layers || l->type_layer != LAYER::FULLY_CONNECTED) continue;
     // what the weights saw: the feeding entry's outputs, or a block layer's own
@@ -1502,11 +1549,20 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
     float const *in = l->in_block && (l->Use__Normalization() || !l->block_first) ? l->d_block_values : outputs_of(l->feed_index);
     size_t const K = l->n_inp;
     float *db = l->Use__Bias() ? impl_->d_dparams + l->first_bias_connection_index : nullptr;
-    if (dlmi_fc_bwd_dw(impl_->ctx, B, K, l->n_out, in, l->d_errors, impl_->d_dparams + l->first_connection_index, db, 1) != DLMI_OK) {
-      fail("update_derivatives: dlmi_fc_bwd_dw");
+    if (side && !hip_ok(hipStreamWaitEvent(impl_->dw_stream, impl_->dz_ready[li], 0), impl_->err, "update_derivatives: wait for dZ")) {
+      fail("update_derivatives: wait for dZ");
+      return;
+    }
+    if (dlmi_fc_bwd_dw(ctx, B, K, l->n_out, in, l->d_errors, impl_->d_dparams + l->first_connection_index, db, 1) != DLMI_OK) {
+      fail(side ? dlmi_last_error(ctx) : "update_derivatives: dlmi_fc_bwd_dw");
       return;
     }
   }
+  // whatever the compute stream does next (the optimizer step, the next forward pass over the same buffers)
+  // comes after the last weight gradient
+  if (side && (!hip_ok(hipEventRecord(impl_->dw_done, impl_->dw_stream), impl_->err, "update_derivatives: join") ||
+               !hip_ok(hipStreamWaitEvent(impl_->stream, impl_->dw_done, 0), impl_->err, "update_derivatives: join")))
+    fail("update_derivatives: join");
 }
 
 // ---------------------------------------------------------------- optimizer step

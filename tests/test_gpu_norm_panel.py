@@ -201,3 +201,39 @@ def test_a_destroyed_stream_is_not_touched_by_the_next_launch(twins, pkg):
     d = make(1024, 1024, 3)
     a, *_ = run_fwd(panel, pkg, d, "RELU", "NONE", False, False)
     assert np.isfinite(a["y"]).all()
+
+
+def test_panel_kernels_beside_another_kernel(twins, pkg):
+    """A product on another stream holds compute units while a panel kernel starts, so some of its workgroups
+    begin late.  A workgroup counts itself in for panel p+1 before it waits for panel p; with one running
+    arrival total the ones ahead could complete the count for p on their own, and a late workgroup's sums were
+    read before it had stored them.  Arrivals are counted per panel parity now: the results beside a running
+    product must be those of a quiet device, bit for bit."""
+    panel, _ = twins
+    B, H = 4096, 2048
+    d = make(B, H, 77)
+    quiet_f, desc, mask, st = run_fwd(panel, pkg, d, "ELU", "NONE", False, False)
+    quiet_b = run_bwd(panel, pkg, d, desc, mask, st)
+    side = torch.cuda.Stream()
+    other = pkg.Dlmi(0)
+    other.set_stream(side)
+    X = torch.randn(4096, 4096, device="cuda")
+    W = torch.randn(4096, 4096, device="cuda") * 0.01
+    Z = torch.empty(4096, 4096, device="cuda")
+    torch.cuda.synchronize()
+    try:
+        for _ in range(4):
+            for _ in range(3):
+                other.fc_fwd(X, W, None, out=Z)  # 256 x 256 tiles: every compute unit held for about 0.5 ms each
+            busy_f, desc2, mask2, st2 = run_fwd(panel, pkg, d, "ELU", "NONE", False, False)
+            for _ in range(3):
+                other.fc_fwd(X, W, None, out=Z)
+            busy_b = run_bwd(panel, pkg, d, desc, mask, st)
+            torch.cuda.synchronize()
+            for k in quiet_f:
+                assert np.array_equal(quiet_f[k], busy_f[k]), k
+            for k in quiet_b:
+                assert np.array_equal(quiet_b[k], busy_b[k]), k
+    finally:
+        torch.cuda.synchronize()
+        other.close()
