@@ -109,6 +109,10 @@ void dev_free(T *&p) {
 constexpr size_t kParallelGatherBytes = size_t(4) << 20;
 constexpr size_t kUploadPiece = size_t(4) << 20;
 constexpr unsigned kGatherThreads = 8;
+// Input and output rows of a layer, in bytes, up to which its weight gradient runs beside the backward chain.
+constexpr size_t kSideStreamOperandBytes = size_t(32) << 20;
+// ... and the work of the product from which that pays when the launches go through the host.
+constexpr double kSideStreamMinFlop = 5.0e8;
 
 bool act_on_path(ACTIVATION::TYPE t) {
   switch (t) {
@@ -1539,7 +1543,10 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
   // from the last layer down: the order in which the backward pass finishes their gradients (every layer adds
   // into its own part of the gradient array, so the order does not change the sums)
   bool const side = impl_->dw_ctx != nullptr;
-  dlmi_ctx *const ctx = side ? impl_->dw_ctx : impl_->ctx;
+  bool joined = true;  // nothing on the side stream yet
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (side && hipStreamIsCapturing(impl_->stream, &capture) != hipSuccess) (void)hipGetLastError();
+  bool const recording = capture != hipStreamCaptureStatusNone;
   for (Layer const *l = last; l != first;) {
     --l;
     size_t const li = static_cast<size_t>(l - ptr_array_layers);
@@ -1549,18 +1556,29 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
     float const *in = l->in_block && (l->Use__Normalization() || !l->block_first) ? l->d_block_values : outputs_of(l->feed_index);
     size_t const K = l->n_inp;
     float *db = l->Use__Bias() ? impl_->d_dparams + l->first_bias_connection_index : nullptr;
-    if (side && !hip_ok(hipStreamWaitEvent(impl_->dw_stream, impl_->dz_ready[li], 0), impl_->err, "update_derivatives: wait for dZ")) {
+    // Side by side pays while the operands stay in the caches and the products leave room on a CU (1024 x 2048
+    // x 2048: dX + dW 145 us one after the other, 129 us side by side; mini-batches: launch latency hidden).
+    // Products that stream tens of MiB from HBM (65536 x 256 x 256) or fill every CU with one 256 x 256 tile
+    // (8192 x 4096 x 4096) get in each other's way: 12-16 % slower side by side.  Those stay on the compute stream.
+    // A mini-batch's products are too short for the two event calls to pay when every launch goes through the
+    // host (784-512-512-10 on 128 rows: 0.126 -> 0.159 ms per step); recorded into a graph they cost nothing, and
+    // the weight gradients leave the critical path (0.0985 -> 0.091 ms).
+    bool const beside = side && B * (K + l->n_out) * sizeof(float) <= kSideStreamOperandBytes &&
+                        (recording || 2.0 * static_cast<double>(B) * static_cast<double>(K) * static_cast<double>(l->n_out) >= kSideStreamMinFlop);
+    if (beside && !hip_ok(hipStreamWaitEvent(impl_->dw_stream, impl_->dz_ready[li], 0), impl_->err, "update_derivatives: wait for dZ")) {
       fail("update_derivatives: wait for dZ");
       return;
     }
-    if (dlmi_fc_bwd_dw(ctx, B, K, l->n_out, in, l->d_errors, impl_->d_dparams + l->first_connection_index, db, 1) != DLMI_OK) {
-      fail(side ? dlmi_last_error(ctx) : "update_derivatives: dlmi_fc_bwd_dw");
+    if (dlmi_fc_bwd_dw(beside ? impl_->dw_ctx : impl_->ctx, B, K, l->n_out, in, l->d_errors,
+                       impl_->d_dparams + l->first_connection_index, db, 1) != DLMI_OK) {
+      fail("update_derivatives: dlmi_fc_bwd_dw");
       return;
     }
+    joined = joined && !beside;
   }
   // whatever the compute stream does next (the optimizer step, the next forward pass over the same buffers)
   // comes after the last weight gradient
-  if (side && (!hip_ok(hipEventRecord(impl_->dw_done, impl_->dw_stream), impl_->err, "update_derivatives: join") ||
+  if (!joined && (!hip_ok(hipEventRecord(impl_->dw_done, impl_->dw_stream), impl_->err, "update_derivatives: join") ||
                !hip_ok(hipStreamWaitEvent(impl_->stream, impl_->dw_done, 0), impl_->err, "update_derivatives: join")))
     fail("update_derivatives: join");
 }
