@@ -20,9 +20,11 @@
 // except that every XCD receives 32 of the 256 workgroups, which dlmi_ctx_create checks with a probe
 // launch.  Every wait is bounded: a workgroup that does not see its XCD complete within kPanelSpinLimit
 // polls raises the abort word and leaves, the others follow, the host reports the failure at the next
-// dlmi_ctx_synchronize and the context stays on the multi-launch path from then on.  That cannot happen
-// while one panel kernel runs at a time (256 workgroups always fit 256 CUs): launches on different streams
-// of one process are ordered with an event for that reason.
+// dlmi_ctx_synchronize and the context stays on the multi-launch path from then on.  Two panel kernels side
+// by side could starve each other, so launches on different streams of one process are ordered with an
+// event.  Other kernels may hold CUs when a panel kernel starts: its workgroups then start late, the ones
+// already running wait for them (a product lasts milliseconds at most, the limit is about a second), and the
+// arrival words are kept so that being late is harmless (see kPanelStateStride below).
 #ifndef DLMI_NORM_PANEL_COMMON_HPP
 #define DLMI_NORM_PANEL_COMMON_HPP
 
