@@ -1567,12 +1567,13 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
                         (recording || 2.0 * static_cast<double>(B) * static_cast<double>(K) * static_cast<double>(l->n_out) >= kSideStreamMinFlop);
     if (beside && !hip_ok(hipStreamWaitEvent(impl_->dw_stream, impl_->dz_ready[li], 0), impl_->err, "update_derivatives: wait for dZ")) {
       fail("update_derivatives: wait for dZ");
-      return;
+      break;
     }
     if (dlmi_fc_bwd_dw(beside ? impl_->dw_ctx : impl_->ctx, B, K, l->n_out, in, l->d_errors,
                        impl_->d_dparams + l->first_connection_index, db, 1) != DLMI_OK) {
       fail("update_derivatives: dlmi_fc_bwd_dw");
-      return;
+      joined = joined && !beside;  // what was launched beside the chain is still joined below
+      break;
     }
     joined = joined && !beside;
   }
