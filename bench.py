@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|c1|c2|c3|c4|c5]
 
-The default run times workload c3 (BASELINE configuration 3: the one the metric is quoted on) as the
+The default run times workload c3 (configuration 3 of the benchmark: the one the metric is quoted on) as the
 headline and the other four configurations under detail.workloads, each with its step time, the roofline
 of its dominant kernels and the reference's CPU path timed beside it.
 

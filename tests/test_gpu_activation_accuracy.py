@@ -11,7 +11,7 @@ the absolute error of exp stays about 1e-7, so no float evaluation - the referen
 each other by the same amount.  The derivative forms cancel too: tanh' = 1 - q^2 as |q| -> 1 and the
 reference's SELU' = scale * (q + alpha) where q ~ -alpha (x ~ -3.03); there one rounding of q^2 (fused or
 not) already moves the small result by more than 1e-5 of itself.  The test asserts 1e-5 outside those
-zones, bounds the ABSOLUTE error inside them, and prints the measured maxima (recorded in DESIGN.md).
+zones, bounds the ABSOLUTE error inside them, and prints the measured maxima.
 The derivative is taken of the SAME stored output on both sides, as the backward pass does."""
 import numpy as np
 import pytest
