@@ -197,7 +197,7 @@ __device__ __forceinline__ void sched_spread() {
   }
 }
 
-template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int WAVES_PER_EU>
+template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int WAVES_PER_EU, int RST>
 __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
 void k_gemm_f32(GemmArgs g) {
   constexpr bool FAST = MODE == kFast;          // no edge anywhere: unguarded stores
@@ -265,7 +265,7 @@ void k_gemm_f32(GemmArgs g) {
   constexpr int NLD = TA::kPerThread + TB::kPerThread;                       // global loads
 
   if (ktiles > 0) {
-    // Software pipeline over the K tiles: two LDS stages, one register stage.
+    // Software pipeline over the K tiles: two LDS stages, one or two register stages.
     // During tile kt (LDS stage kt&1): tile kt+1, fetched from memory during
     // tile kt-1, moves from registers into the other stage, the global loads of
     // tile kt+2 are issued, and after the barrier - placed three quarters into
@@ -273,20 +273,39 @@ void k_gemm_f32(GemmArgs g) {
     // stage and the writes of the next - the first fragments of tile kt+1 are
     // read.  LDS and memory traffic is spread between the MFMAs, so the matrix
     // pipe only waits at the barrier itself.
-    typename TA::Regs ra = tile_load<BM, BK, A_KCONTIG, MODE>(g.A, g.lda, m0, k_begin, g.M, k_end, g.a_vec != 0);
-    typename TB::Regs rb = tile_load<BN, BK, B_KCONTIG, MODE>(g.B, g.ldb, n0, k_begin, g.N, k_end, g.b_vec != 0);
+    // RST == 2: TWO register stages.  A K tile of a small tile lasts a quarter of a microsecond, less than a
+    // load from the memory side takes, so the loads run three tiles ahead of the MFMAs (tile kt+3 is fetched
+    // during tile kt and moves to LDS during tile kt+2); the stages alternate with the tile's parity.
+    static_assert(RST == 1 || RST == 2, "one or two register stages");
+    auto load_a = [&](int t) {
+      return tile_load<BM, BK, A_KCONTIG, MODE>(g.A, g.lda, m0, k_begin + static_cast<size_t>(t) * BK, g.M, k_end, g.a_vec != 0);
+    };
+    auto load_b = [&](int t) {
+      return tile_load<BN, BK, B_KCONTIG, MODE>(g.B, g.ldb, n0, k_begin + static_cast<size_t>(t) * BK, g.N, k_end, g.b_vec != 0);
+    };
+    typename TA::Regs ra = load_a(0), ra2 = ra;
+    typename TB::Regs rb = load_b(0), rb2 = rb;
     tile_store<BM, BK, A_KCONTIG>(lds, ra);
     tile_store<BN, BK, B_KCONTIG>(lds + TA::kFloats, rb);
+    // one register stage: ra/rb hold tile kt+1 at the start of tile kt.  Two: tile kt+1 is in ra/rb for even
+    // kt and in ra2/rb2 for odd kt, tile kt+2 in the other pair.
     if (ktiles > 1) {
-      ra = tile_load<BM, BK, A_KCONTIG, MODE>(g.A, g.lda, m0, k_begin + BK, g.M, k_end, g.a_vec != 0);
-      rb = tile_load<BN, BK, B_KCONTIG, MODE>(g.B, g.ldb, n0, k_begin + BK, g.N, k_end, g.b_vec != 0);
+      ra = load_a(1);
+      rb = load_b(1);
+    }
+    if constexpr (RST == 2) {
+      if (ktiles > 2) {
+        ra2 = load_a(2);
+        rb2 = load_b(2);
+      }
     }
     __syncthreads();
     v4f f0a[TM], f0b[TN];
     frags(lds, lds + TA::kFloats, 0, f0a, f0b);
 
-    // one K tile; STORE: a next tile exists (in registers), LOAD: one after that exists
-    auto tile_step = [&](int kt, auto store_c, auto load_c) {
+    // one K tile; STORE: a next tile exists (in the registers xa / xb), LOAD: a tile RST further on exists and
+    // is fetched into the same registers
+    auto tile_step = [&](int kt, auto store_c, auto load_c, typename TA::Regs &xa, typename TB::Regs &xb) {
       constexpr bool STORE = decltype(store_c)::value, LOAD = decltype(load_c)::value;
       float const *const sa = lds + (kt & 1) * kStage;
       float *const na = lds + ((kt & 1) ^ 1) * kStage;
@@ -294,13 +313,12 @@ void k_gemm_f32(GemmArgs g) {
       frags(sa, sa + TA::kFloats, 8, f1a, f1b);
       steps(f0a, f0b, 0, 4);
       if constexpr (STORE) {
-        tile_store<BM, BK, A_KCONTIG>(na, ra);
-        tile_store<BN, BK, B_KCONTIG>(na + TA::kFloats, rb);
+        tile_store<BM, BK, A_KCONTIG>(na, xa);
+        tile_store<BN, BK, B_KCONTIG>(na + TA::kFloats, xb);
       }
       if constexpr (LOAD) {
-        size_t const kn = k_begin + static_cast<size_t>(kt + 2) * BK;
-        ra = tile_load<BM, BK, A_KCONTIG, MODE>(g.A, g.lda, m0, kn, g.M, k_end, g.a_vec != 0);
-        rb = tile_load<BN, BK, B_KCONTIG, MODE>(g.B, g.ldb, n0, kn, g.N, k_end, g.b_vec != 0);
+        xa = load_a(kt + 1 + RST);
+        xb = load_b(kt + 1 + RST);
       }
       steps(f1a, f1b, 0, 2);
       if constexpr (FAST_LOOP) {
@@ -322,12 +340,29 @@ void k_gemm_f32(GemmArgs g) {
     using std::false_type;
     using std::true_type;
     int kt = 0;
-    for (; kt + 2 < ktiles; ++kt) tile_step(kt, true_type{}, true_type{});
-    if (kt + 1 < ktiles) {
-      tile_step(kt, true_type{}, false_type{});
-      ++kt;
+    if constexpr (RST == 1) {
+      for (; kt + 2 < ktiles; ++kt) tile_step(kt, true_type{}, true_type{}, ra, rb);
+      if (kt + 1 < ktiles) {
+        tile_step(kt, true_type{}, false_type{}, ra, rb);
+        ++kt;
+      }
+      tile_step(kt, false_type{}, false_type{}, ra, rb);
+    } else {
+      // pairs of tiles while both still fetch (the second of a pair fetches tile kt+4)
+      for (; kt + 4 < ktiles; kt += 2) {
+        tile_step(kt, true_type{}, true_type{}, ra, rb);
+        tile_step(kt + 1, true_type{}, true_type{}, ra2, rb2);
+      }
+      // the last (at most four) tiles: kt is even here
+      for (; kt < ktiles; ++kt) {
+        bool const store = kt + 1 < ktiles, load = kt + 3 < ktiles;
+        typename TA::Regs &xa = (kt & 1) ? ra2 : ra;
+        typename TB::Regs &xb = (kt & 1) ? rb2 : rb;
+        if (load) tile_step(kt, true_type{}, true_type{}, xa, xb);
+        else if (store) tile_step(kt, true_type{}, false_type{}, xa, xb);
+        else tile_step(kt, false_type{}, false_type{}, xa, xb);
+      }
     }
-    tile_step(kt, false_type{}, false_type{});
   }
 
   // ---- epilogue: accumulator register e of lane l holds
@@ -420,7 +455,7 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(float const *__restrict__
 }
 
 // ---------------------------------------------------------------- host side
-template <int BM, int BN, int BK, bool AK, bool BKC, int WPE, bool HAS_CLAMPED>
+template <int BM, int BN, int BK, bool AK, bool BKC, int WPE, bool HAS_CLAMPED, int RST>
 static int launch_gemm(dlmi_ctx *ctx, GemmArgs g, unsigned splits, int mode) {
   using TA = TileShape<BM, BK, AK>;
   using TB = TileShape<BN, BK, BKC>;
@@ -428,10 +463,10 @@ static int launch_gemm(dlmi_ctx *ctx, GemmArgs g, unsigned splits, int mode) {
   g.tiles_m = static_cast<unsigned>(dlmi_ceil_div(g.M, BM));
   g.tiles_n = static_cast<unsigned>(dlmi_ceil_div(g.N, BN));
   dim3 const grid(g.tiles_m * g.tiles_n, 1, splits);
-  auto const kfast = k_gemm_f32<BM, BN, BK, AK, BKC, kFast, WPE>;
-  auto const kslow = k_gemm_f32<BM, BN, BK, AK, BKC, kGuarded, WPE>;
+  auto const kfast = k_gemm_f32<BM, BN, BK, AK, BKC, kFast, WPE, RST>;
+  auto const kslow = k_gemm_f32<BM, BN, BK, AK, BKC, kGuarded, WPE, 1>;
   // the clamped variant exists for the small tiles, which are the ones ragged layers run
-  auto const kclamp = k_gemm_f32<BM, BN, BK, AK, BKC, HAS_CLAMPED ? kClamped : kGuarded, WPE>;
+  auto const kclamp = k_gemm_f32<BM, BN, BK, AK, BKC, HAS_CLAMPED ? kClamped : kGuarded, WPE, HAS_CLAMPED ? RST : 1>;
   if (!HAS_CLAMPED && mode == kClamped) mode = kGuarded;
   // more than 64 KB of LDS has to be asked for once per kernel and device
   static bool attr_set_on[64] = {false};
@@ -619,10 +654,24 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   if (splits > 1) g.split_out = reinterpret_cast<float *>(dlmi_scratch_data(ctx));
   int rc;
   switch (choice) {
-    case 1: rc = launch_gemm<256, 128, 16, AK, BKC, 2, false>(ctx, g, splits, mode); break;
-    case 2: rc = launch_gemm<256, 256, 16, AK, BKC, 1, false>(ctx, g, splits, mode); break;
-    case 3: rc = launch_gemm<64, 64, 16, AK, BKC, 4, true>(ctx, g, splits, mode); break;
-    default: rc = launch_gemm<128, 128, 16, AK, BKC, 2, true>(ctx, g, splits, mode); break;
+    case 1: rc = launch_gemm<256, 128, 16, AK, BKC, 2, false, 1>(ctx, g, splits, mode); break;
+    case 2: rc = launch_gemm<256, 256, 16, AK, BKC, 1, false, 1>(ctx, g, splits, mode); break;
+    // The small tiles keep two register stages on a long reduction: a K tile of 64 x 64 is shorter than a load
+    // takes (1024 x 2048 x 2048: forward 70.9 -> 67.7 us, dX 75.5 -> 69.9 us), and 128 x 128 gains too
+    // (2048 x 2048 x 1024: 69.8 -> 68.5 us; at 8192 x 4096 x 4096 it reaches 145 TFLOP/s with them, 140
+    // without).  A short reduction (16 K tiles) loses 2.5 % to the longer start.
+    case 3:
+      if (kt_per_split >= 32)
+        rc = launch_gemm<64, 64, 16, AK, BKC, 4, true, 2>(ctx, g, splits, mode);
+      else
+        rc = launch_gemm<64, 64, 16, AK, BKC, 4, true, 1>(ctx, g, splits, mode);
+      break;
+    default:
+      if (kt_per_split >= 32)
+        rc = launch_gemm<128, 128, 16, AK, BKC, 2, true, 2>(ctx, g, splits, mode);
+      else
+        rc = launch_gemm<128, 128, 16, AK, BKC, 2, true, 1>(ctx, g, splits, mode);
+      break;
   }
   if (rc != DLMI_OK) return rc;
   if (defer_slices != nullptr) {
