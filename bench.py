@@ -54,7 +54,7 @@ MEASURED_TRAFFIC_BYTES = {
 # changed since, `traffic` is reported as null instead of a figure that may no longer hold.
 TRAFFIC_SOURCES = ("gemm_f32_mfma.hip", "norm_kernels.hip", "norm_panel_fwd.hip", "norm_panel_bwd.hip",
                    "norm_panel_common.hpp", "norm_shared.hpp", "activations.hpp", "dlmi_common.hpp")
-TRAFFIC_SOURCES_SHA256 = "19fa18f268ce7a7d07492c7920092e5d3ac8c488f12e41c4ee02ea6b9c8dc72e"
+TRAFFIC_SOURCES_SHA256 = "702680570f3959e7be429d2bf67fca72e9b824de186086b1f230ed963ab0bd4f"
 
 
 def traffic_sources_digest():
