@@ -11,10 +11,13 @@
 // workgroup (4 wavefronts, 2 x 2) owns a BM x BN tile of C; each wavefront
 // owns (BM/2) x (BN/2) as a grid of 32x32 v_mfma_f32_32x32x2_f32 blocks whose
 // accumulators stay in registers for the whole K loop.  Operand tiles are
-// staged through LDS (two stages, one barrier per K tile) behind a register
-// stage: the global loads run two tiles ahead of the MFMAs, and the LDS writes,
-// the global loads and the fragment reads of a tile are spread between the
-// MFMAs of the previous one with scheduling-group hints.
+// staged through LDS (two stages, one barrier per K tile) behind one register
+// stage (the global loads run two tiles ahead of the MFMAs) or, for the small
+// tiles on a long reduction, two (three tiles ahead); the LDS writes, the
+// global loads and the fragment reads of a tile are spread between the MFMAs
+// of the previous one with scheduling-group hints.  Three edge treatments:
+// none (shapes that are multiples of the tile), clamped rows (ragged M or N),
+// guarded element by element (anything else).
 //
 // The MFMA consumes two k per instruction: lanes 0-31 supply k_lo, lanes 32-63
 // k_hi.  Because the sum over k is order-free inside a tile, the kernel feeds
