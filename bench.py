@@ -54,7 +54,7 @@ MEASURED_TRAFFIC_BYTES = {
 # changed since, `traffic` is reported as null instead of a figure that may no longer hold.
 TRAFFIC_SOURCES = ("gemm_f32_mfma.hip", "norm_kernels.hip", "norm_panel_fwd.hip", "norm_panel_bwd.hip",
                    "norm_panel_common.hpp", "norm_shared.hpp", "activations.hpp", "dlmi_common.hpp")
-TRAFFIC_SOURCES_SHA256 = "6e36cd4465632e28aea18d8e5737b8e21afe7d04a2b484ffbe7ba6864b670030"
+TRAFFIC_SOURCES_SHA256 = "bac12d74dbe0450cca72c0468c1f8a926ba5a3cdf475be4b3daf00067df1171a"
 
 
 def traffic_sources_digest():

@@ -34,7 +34,7 @@ STATE = dict(INFERENCE=0, TRAINING=1, UPDATE_BATCH_NORM=2)
 
 # every symbol include/dlmi.h declares
 C_ABI_SYMBOLS = [
-    "dlmi_ctx_create", "dlmi_ctx_destroy", "dlmi_ctx_set_stream", "dlmi_ctx_synchronize", "dlmi_last_error",
+    "dlmi_gemm_plan", "dlmi_ctx_create", "dlmi_ctx_destroy", "dlmi_ctx_set_stream", "dlmi_ctx_synchronize", "dlmi_last_error",
     "dlmi_ctx_compute_units", "dlmi_layer_variance", "dlmi_scale", "dlmi_fc_fwd", "dlmi_fc_bwd_dx", "dlmi_fc_bwd_dw", "dlmi_bias_fwd",
     "dlmi_norm_fwd_train", "dlmi_norm_fwd_infer", "dlmi_norm_bwd", "dlmi_act_fwd", "dlmi_act_fwd_units", "dlmi_act_bwd_units", "dlmi_act_bwd",
     "dlmi_softmax_fwd", "dlmi_dropout_fwd", "dlmi_identity_add", "dlmi_softmax_ce_seed",

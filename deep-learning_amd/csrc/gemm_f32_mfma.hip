@@ -587,6 +587,12 @@ static GemmPlan plan_gemm(dlmi_ctx const *ctx, size_t M, size_t N, size_t K) {
   return p;
 }
 
+// Register stages of the K loop (see the launch switch in gemm()): two for the small tiles from 32 K tiles per
+// slice on, one otherwise.
+static int gemm_register_stages(int bm, int bn, size_t kt_per_split) {
+  return bm * bn <= 128 * 128 && kt_per_split >= 32 ? 2 : 1;
+}
+
 // Scratch the three products of a layer [B, K] -> [B, H] may ask for (K splits, epilogue statistics).
 size_t fc_scratch_bytes(dlmi_ctx const *ctx, size_t B, size_t K, size_t H) {
   size_t need = 2 * 2 * 64 * H * sizeof(float);  // epilogue statistics: at most B / 64 ... 64 tile rows reserved
@@ -664,13 +670,13 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
     // (2048 x 2048 x 1024: 69.8 -> 68.5 us; at 8192 x 4096 x 4096 it reaches 145 TFLOP/s with them, 140
     // without).  A short reduction (16 K tiles) loses 2.5 % to the longer start.
     case 3:
-      if (kt_per_split >= 32)
+      if (gemm_register_stages(bm, bn, kt_per_split) == 2)
         rc = launch_gemm<64, 64, 16, AK, BKC, 4, true, 2>(ctx, g, splits, mode);
       else
         rc = launch_gemm<64, 64, 16, AK, BKC, 4, true, 1>(ctx, g, splits, mode);
       break;
     default:
-      if (kt_per_split >= 32)
+      if (gemm_register_stages(bm, bn, kt_per_split) == 2)
         rc = launch_gemm<128, 128, 16, AK, BKC, 2, true, 2>(ctx, g, splits, mode);
       else
         rc = launch_gemm<128, 128, 16, AK, BKC, 2, true, 1>(ctx, g, splits, mode);
@@ -699,6 +705,21 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
 using namespace dlmi;
 
 extern "C" {
+
+int dlmi_gemm_plan(int compute_units, size_t M, size_t N, size_t K, int *tile_m, int *tile_n, unsigned *k_slices,
+                   int *register_stages) {
+  if (compute_units <= 0 || M == 0 || N == 0 || K == 0) return DLMI_E_INVALID;
+  dlmi_ctx probe;  // only the CU count enters the plan
+  probe.num_cu = compute_units;
+  GemmPlan const p = plan_gemm(&probe, M, N, K);
+  size_t const ktiles = dlmi_ceil_div(K, p.bk);
+  size_t const kt_per_split = dlmi_ceil_div(ktiles, p.splits);
+  if (tile_m != nullptr) *tile_m = p.bm;
+  if (tile_n != nullptr) *tile_n = p.bn;
+  if (k_slices != nullptr) *k_slices = static_cast<unsigned>(dlmi_ceil_div(ktiles, kt_per_split));
+  if (register_stages != nullptr) *register_stages = gemm_register_stages(p.bm, p.bn, kt_per_split);
+  return DLMI_OK;
+}
 
 int dlmi_fc_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, float const *W, float const *bias,
                 float *Z) {

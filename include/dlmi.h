@@ -85,6 +85,13 @@ int dlmi_ctx_reserve_layer(dlmi_ctx *ctx, size_t B, size_t K, size_t H);
 unsigned long long dlmi_ctx_scratch_generation(dlmi_ctx const *ctx);
 /* Compute units of the context's device (for callers sizing their own work). */
 int dlmi_ctx_compute_units(dlmi_ctx const *ctx);
+/* How a product C[M,N] = A[M,K] . B[K,N] would be launched on a device with `compute_units` CUs: tile shape, K
+ * slices (1 = none; more = partial products plus a fixed-order sum) and register stages of the K loop.  Host
+ * arithmetic only, no device needed: no counterpart in the reference (whose loops have no tiles); for callers and
+ * tests that want to know which kernel variant a layer shape takes.  forward: M = batch, N = units, K = fan-in;
+ * dX: M = batch, N = fan-in, K = units; dW: M = units, N = fan-in, K = batch. */
+int dlmi_gemm_plan(int compute_units, size_t M, size_t N, size_t K, int *tile_m, int *tile_n, unsigned *k_slices,
+                   int *register_stages);
 
 /* ---- fully-connected contractions (fp32 MFMA) ----------------------------- */
 /* Z[b,h] = sum_k X[b,k] * W[h,k] (+ bias[h] if bias != NULL); overwrites Z.
