@@ -510,7 +510,7 @@ def run_c4(args, torch, pkg, dl):
     read = [torch.cuda.Event(), torch.cuda.Event()]
     used = [False, False]
 
-    def step():
+    def step(two_streams=two_streams):
         for i in range(nblk):
             dl.fc_norm_act_fwd(desc, xs[i], Ws[i], one, zero, mm[i], ms[i], mask=mask[i], Z=Zs[i], out=xs[i + 1],
                                stats=stats[i], shortcut=xs[i])
@@ -541,6 +541,7 @@ def run_c4(args, torch, pkg, dl):
     for v in dgs + dbs:
         v.zero_()
     ms_step = time_wall(torch, step, args.steps, args.warmup)
+    ms_one_stream = time_wall(torch, lambda: step(False), args.steps, args.warmup) if two_streams else ms_step
     E = B * H
     t_f = time_events(torch, lambda: dl.fc_fwd(xs[0], Ws[0], None, out=Zs[0]), 20)
     t_x = time_events(torch, lambda: dl.fc_bwd_dx(dZ, Ws[0], out=g), 20)
@@ -563,7 +564,7 @@ def run_c4(args, torch, pkg, dl):
     hbm["frac"] = hbm["achieved"] / hbm["peak"]
     detail = {"ms_gemm_fwd": t_f, "ms_gemm_dx": t_x, "ms_gemm_dw": t_w, "ms_norm_fwd": t_nf, "ms_norm_bwd": t_nb,
               "gemm_ms_per_step": 16 * (t_f + t_x + t_w), "norm_ms_per_step": 16 * (t_nf + t_nb),
-              "calls_per_step": 4 * nblk + 1}
+              "calls_per_step": 4 * nblk + 1, "ms_per_step_one_stream": ms_one_stream}
 
     cpu = parity = None
     if args.cpu_rows != 0:
