@@ -43,7 +43,7 @@ C_ABI_SYMBOLS = [
     "dlmi_opt_adabound", "dlmi_clip_gradient", "dlmi_max_norm_rows", "dlmi_opt_irprop_plus", "dlmi_loss_seed", "dlmi_zero",
     "dlmi_fused_norm_act_fwd_noalloc", "dlmi_fused_norm_act_residual_fwd", "dlmi_fc_norm_act_residual_fwd",
     "dlmi_fc_softmax_fwd", "dlmi_fc_bwd_dx_norm_act_bwd",
-    "dlmi_ctx_reserve_layer", "dlmi_ctx_scratch_generation",
+    "dlmi_ctx_reserve_layer", "dlmi_ctx_scratch_generation", "dlmi_ctx_norm_panel_enabled", "dlmi_ctx_norm_panel_poke",
 ]
 
 
@@ -132,6 +132,14 @@ class Dlmi:
 
     def compute_units(self):
         return self.lib.dlmi_ctx_compute_units(self.ctx)
+
+    def norm_panel_enabled(self):
+        """Whether this context may still launch the single-launch normalization kernels."""
+        return bool(self.lib.dlmi_ctx_norm_panel_enabled(self.ctx))
+
+    def norm_panel_poke(self, xcd, word, value):
+        """Test hook: one word of an XCD's barrier state (see dlmi.h)."""
+        self._ck(self.lib.dlmi_ctx_norm_panel_poke(self.ctx, ctypes.c_uint(xcd), ctypes.c_uint(word), ctypes.c_uint(value)))
 
     # ------------------------------------------------------------ GEMMs
     def fc_fwd(self, X, W, bias=None, out=None):

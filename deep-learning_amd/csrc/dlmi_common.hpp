@@ -53,10 +53,14 @@ struct dlmi_ctx {
   dlmi_tuning tune;
   // single-launch (column panel) normalization kernels: barrier words in device memory, whether this
   // device qualifies (256 CUs, 32 workgroups of a 256-workgroup launch on each of 8 XCDs), and whether
-  // one has been launched since the words were last inspected
+  // a kernel of this context has been recorded into a HIP graph.  A kernel that gives up says so in two words
+  // of pinned host memory (panel_flag_host; the same memory as the device sees it: panel_flag_dev), which the
+  // host reads after every synchronization of the stream.
   unsigned *panel_state = nullptr;
+  unsigned *panel_flag_host = nullptr, *panel_flag_dev = nullptr;
+  int panel_spin_limit = 1 << 20;
   int panel_ok = 0;
-  int panel_used = 0;
+  int panel_in_graph = 0;
   char err[512] = {0};
 };
 
@@ -128,6 +132,7 @@ size_t norm_scratch_bytes(dlmi_ctx const *ctx, size_t H);
 // Column panel kernels (norm_panel_*.hip): set-up at context creation, inspection after a synchronize,
 // scratch they need for [*, H].
 int panel_init(dlmi_ctx *ctx);
+void panel_destroy(dlmi_ctx *ctx);
 int panel_check(dlmi_ctx *ctx);
 // The context lets go of its stream (destroyed, or given another one), which the caller may destroy next:
 // after the stream's work has completed, the cross-stream ordering of panel launches forgets it.

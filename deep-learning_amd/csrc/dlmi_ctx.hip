@@ -86,7 +86,7 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
   if (rc != DLMI_OK) {
     fprintf(stderr, "dlmi: %s\n", ctx->err);
     if (ctx->scratch != nullptr) (void)hipFree(ctx->scratch);
-    if (ctx->panel_state != nullptr) (void)hipFree(ctx->panel_state);
+    dlmi::panel_destroy(ctx);
     delete ctx;
     return rc;
   }
@@ -100,7 +100,7 @@ int dlmi_ctx_destroy(dlmi_ctx *ctx) {
   dlmi::panel_release_stream(ctx);
   if (ctx->scratch != nullptr) (void)hipFree(ctx->scratch);
   for (int i = 0; i < ctx->n_retired; ++i) (void)hipFree(ctx->retired[i]);
-  if (ctx->panel_state != nullptr) (void)hipFree(ctx->panel_state);
+  dlmi::panel_destroy(ctx);
   delete ctx;
   return DLMI_OK;
 }
@@ -147,5 +147,16 @@ unsigned long long dlmi_ctx_scratch_generation(dlmi_ctx const *ctx) {
 char const *dlmi_last_error(dlmi_ctx const *ctx) { return ctx != nullptr ? ctx->err : "null context"; }
 
 int dlmi_ctx_compute_units(dlmi_ctx const *ctx) { return ctx != nullptr ? ctx->num_cu : 0; }
+
+int dlmi_ctx_norm_panel_enabled(dlmi_ctx const *ctx) { return ctx != nullptr && ctx->panel_ok ? 1 : 0; }
+
+int dlmi_ctx_norm_panel_poke(dlmi_ctx *ctx, unsigned xcd, unsigned word, unsigned value) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, ctx->panel_state != nullptr, "this context has no single-launch normalization kernels");
+  DLMI_REQUIRE(ctx, xcd < 8 && word < 16, "no such word");
+  DLMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  DLMI_HIP(ctx, hipMemcpy(ctx->panel_state + xcd * 16 + word, &value, sizeof value, hipMemcpyHostToDevice));
+  return DLMI_OK;
+}
 
 }  // extern "C"

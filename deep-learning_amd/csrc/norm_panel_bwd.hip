@@ -22,7 +22,7 @@ struct PanelBwdArgs {
   size_t B, H;
   float batch_f, batch_scale, drop_scale;
   int drop_mode, drop_bwd_masked, accumulate;
-  unsigned *state;
+  PanelSync sync;
   float *part;  // [xcd][panel][rank][3][kP]
 };
 
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
   __shared__ unsigned s_rank, s_ok;
   PanelWho who;
   if (threadIdx.x == 0) s_ok = 1;
-  if (!panel_enter(a.state, who, &s_rank)) return;
+  if (!panel_enter(a.sync, who, &s_rank)) return;
   int const tx = threadIdx.x % kCG, ty = threadIdx.x / kCG;
   size_t const Hx = a.H / kPanelXcds;
   int const npanels = static_cast<int>(Hx / kP);
@@ -278,10 +278,10 @@ int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4
   a.B = B; a.H = H;
   a.batch_f = static_cast<float>(B); a.batch_scale = 1.0f / static_cast<float>(B); a.drop_scale = c.drop_scale;
   a.drop_mode = c.drop_mode; a.drop_bwd_masked = c.drop_bwd_masked; a.accumulate = c.accumulate ? 1 : 0;
-  a.state = ctx->panel_state;
+  a.sync = panel_sync_of(ctx);
   a.part = static_cast<float *>(scratch);
-  rc = panel_order_launch(ctx);
-  if (rc != DLMI_OK) return rc;
+  rc = panel_admit(ctx);
+  if (rc <= 0) return rc;
   // rows per workgroup = B / 32 = RPT * 2048 / P
   DLMI_DISPATCH_ACT(c.act, {
     if (extra) {

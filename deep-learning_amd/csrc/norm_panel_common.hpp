@@ -18,13 +18,19 @@
 // arrivals).  Which XCD a workgroup runs on is read from the XCC_ID hardware register, its rank among the
 // workgroups of that XCD from a ticket counter in the same L2; nothing is assumed about the dispatch order
 // except that every XCD receives 32 of the 256 workgroups, which dlmi_ctx_create checks with a probe
-// launch.  Every wait is bounded: a workgroup that does not see its XCD complete within kPanelSpinLimit
-// polls raises the abort word and leaves, the others follow, the host reports the failure at the next
-// dlmi_ctx_synchronize and the context stays on the multi-launch path from then on.  Two panel kernels side
-// by side could starve each other, so launches on different streams of one process are ordered with an
-// event.  Other kernels may hold CUs when a panel kernel starts: its workgroups then start late, the ones
-// already running wait for them (a product lasts milliseconds at most, the limit is about a second), and the
-// arrival words are kept so that being late is harmless (see kPanelStateStride below).
+// launch.  Every wait is bounded: a workgroup that does not see its XCD complete within the context's spin
+// limit (kPanelSpinLimit polls unless DLMI_PANEL_SPIN_LIMIT says otherwise) raises the abort word and leaves,
+// the others follow, and the give-up is written to a word of pinned host memory, which the host reads after
+// every synchronization of the context's stream at no cost: dlmi_ctx_synchronize then reports the failure
+// once, clears the barrier words and keeps the context on the multi-launch path from then on.  A launch that
+// finds the words of an earlier give-up still in place (more tickets than workgroups) leaves at once and
+// says so in a second host word, so every call whose results are not valid is reported.  Two panel kernels
+// side by side could starve each other, so launches on different streams of one process are ordered with an
+// event, and once a stream has recorded a panel kernel into a HIP graph (whose replays this library does not
+// see) every other stream of that device takes the multi-launch kernels.  Other kernels may hold CUs when a
+// panel kernel starts: its workgroups then start late, the ones already running wait for them (a product
+// lasts milliseconds at most, the limit is about a second), and the arrival words are kept so that being
+// late is harmless (see kPanelStateStride below).
 #ifndef DLMI_NORM_PANEL_COMMON_HPP
 #define DLMI_NORM_PANEL_COMMON_HPP
 
@@ -75,8 +81,19 @@ __device__ __forceinline__ void panel_count(unsigned *p) {
 struct PanelWho {
   unsigned xcd, rank;
   unsigned *st;
+  unsigned *flag;  // pinned host memory: [0] a wait gave up, [1] a launch found an earlier give-up's words
+  int spin_limit;
 };
-__device__ __forceinline__ bool panel_enter(unsigned *state, PanelWho &w, unsigned *s_rank) {
+// What every panel kernel receives about the barrier besides its operands.
+struct PanelSync {
+  unsigned *state;  // kPanelStateWords words of device memory
+  unsigned *flag;   // two words of pinned host memory
+  int spin_limit;
+};
+__device__ __forceinline__ bool panel_enter(PanelSync const &sy, PanelWho &w, unsigned *s_rank) {
+  unsigned *const state = sy.state;
+  w.flag = sy.flag;
+  w.spin_limit = sy.spin_limit;
   w.xcd = panel_xcc_id();
   if (w.xcd >= static_cast<unsigned>(kPanelXcds)) w.xcd = 0;  // the probe at context creation rules this out
   w.st = state + w.xcd * kPanelStateStride;
@@ -84,7 +101,10 @@ __device__ __forceinline__ bool panel_enter(unsigned *state, PanelWho &w, unsign
   __syncthreads();
   w.rank = *s_rank;
   if (w.rank >= static_cast<unsigned>(kPanelRanks)) {
-    if (threadIdx.x == 0) w.st[3] = 1;
+    if (threadIdx.x == 0) {
+      w.st[3] = 1;
+      *reinterpret_cast<unsigned volatile *>(w.flag + 1) = 1u;
+    }
     return false;
   }
   return true;
@@ -96,8 +116,9 @@ __device__ __forceinline__ bool panel_wait(PanelWho const &w, int p) {
   unsigned *const word = panel_arrivals(w, p);
   int spins = 0;
   while (panel_poll(word) < target) {
-    if (++spins > kPanelSpinLimit || (spins % 1024 == 0 && panel_poll(w.st + 3) != 0)) {
+    if (++spins > w.spin_limit || (spins % 1024 == 0 && panel_poll(w.st + 3) != 0)) {
       panel_count(w.st + 3);
+      *reinterpret_cast<unsigned volatile *>(w.flag) = 1u;
       return false;
     }
   }
@@ -118,8 +139,11 @@ __device__ __forceinline__ void panel_leave(PanelWho const &w) {
 }
 
 // host side (norm_panel_fwd.hip; panel_init / panel_check / panel_scratch_bytes are declared in dlmi_common.hpp)
-int panel_order_launch(dlmi_ctx *ctx);         // before a panel launch: orders it behind the last one of another stream
+// Before a panel launch: 1 = go (ordered behind the last panel kernel of another stream where needed),
+// 0 = this launch must take the multi-launch kernels (see panel_admit), < 0 = failure.
+int panel_admit(dlmi_ctx *ctx);
 void panel_launched(dlmi_ctx *ctx);            // after it
+inline PanelSync panel_sync_of(dlmi_ctx const *ctx) { return PanelSync{ctx->panel_state, ctx->panel_flag_dev, ctx->panel_spin_limit}; }
 
 }  // namespace dlmi
 

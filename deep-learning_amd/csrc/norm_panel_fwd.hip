@@ -27,7 +27,7 @@ struct PanelFwdArgs {
   FwdFinalize fin;
   int drop_mode;
   float drop_scale;
-  unsigned *state;
+  PanelSync sync;
   float *part;  // [xcd][panel][rank][2][kP]
 };
 
@@ -41,7 +41,7 @@ __global__ __launch_bounds__(kPanelThreads) void k_fwd_panel(PanelFwdArgs a) {
   __shared__ unsigned s_rank, s_ok;
   PanelWho who;
   if (threadIdx.x == 0) s_ok = 1;
-  if (!panel_enter(a.state, who, &s_rank)) return;
+  if (!panel_enter(a.sync, who, &s_rank)) return;
   int const tx = threadIdx.x % kCG, ty = threadIdx.x / kCG;
   size_t const Hx = a.H / kPanelXcds;
   int const npanels = static_cast<int>(Hx / kP);
@@ -174,10 +174,10 @@ __global__ __launch_bounds__(kPanelThreads) void k_fwd_panel(PanelFwdArgs a) {
   load(b0, 0);
   if (npanels > 1) load(b1, 1);
   publish(b0, 0);
-  if (npanels > 1)
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(RPT) : "memory");  // the partial is older than the RPT loads of panel 1
-  else
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // The partial of panel 0 was stored AFTER the loads of panel 1 were issued, so a counted wait would let it
+  // pass while still in flight: everything must have completed before this workgroup counts itself in (the
+  // rows of panel 1 are needed by the very next publish anyway).
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   arrive(0);
   auto step = [&](pv4f (&cur)[RPT], pv4f (&mid)[RPT], pv4f (&nxt)[RPT], int p) -> bool {
     if (p + 1 < npanels) {
@@ -209,10 +209,15 @@ __global__ __launch_bounds__(64) void k_panel_probe(unsigned *out) {
 std::mutex g_order_mutex;
 struct DeviceOrder {
   hipEvent_t event = nullptr;
-  hipStream_t stream = nullptr;
+  hipStream_t stream = nullptr;  // the stream of the last panel launch outside a capture
   bool recorded = false;
+  // the stream (and its context) that has recorded a panel kernel into a HIP graph: replays of that graph are
+  // not seen here, so no other stream of the device may launch panel kernels while this owner exists
+  hipStream_t graph_owner = nullptr;
+  dlmi_ctx const *graph_owner_ctx = nullptr;
 };
 DeviceOrder g_order[64];
+DeviceOrder &order_of(dlmi_ctx const *ctx) { return g_order[ctx->device >= 0 && ctx->device < 64 ? ctx->device : 0]; }
 
 template <int ACT, int RPT, bool EXTRA>
 void launch_fwd(dlmi_ctx *ctx, PanelFwdArgs const &a) {
@@ -226,10 +231,20 @@ int panel_init(dlmi_ctx *ctx) {
   char const *e = std::getenv("DLMI_NORM_PANEL");
   if (e != nullptr && std::atoi(e) == 0) return DLMI_OK;
   if (ctx->num_cu != kPanelXcds * kPanelRanks) return DLMI_OK;  // another part or partition mode: multi-launch path
+  // the bound of every wait, in polls; a small value lets a test drive the give-up branch from the host
+  ctx->panel_spin_limit = kPanelSpinLimit;
+  if (char const *l = std::getenv("DLMI_PANEL_SPIN_LIMIT"); l != nullptr && std::atoi(l) > 0) ctx->panel_spin_limit = std::atoi(l);
   void *p = nullptr;
   DLMI_HIP(ctx, hipMalloc(&p, (kPanelStateWords + kPanelXcds * kPanelRanks) * sizeof(unsigned)));
   ctx->panel_state = static_cast<unsigned *>(p);
   DLMI_HIP(ctx, hipMemsetAsync(ctx->panel_state, 0, (kPanelStateWords + kPanelXcds * kPanelRanks) * sizeof(unsigned), ctx->stream));
+  // two words of pinned, device-visible host memory for the give-up reports
+  void *h = nullptr, *hd = nullptr;
+  DLMI_HIP(ctx, hipHostMalloc(&h, 64, hipHostMallocMapped));
+  ctx->panel_flag_host = static_cast<unsigned *>(h);
+  ctx->panel_flag_host[0] = ctx->panel_flag_host[1] = 0;
+  DLMI_HIP(ctx, hipHostGetDevicePointer(&hd, h, 0));
+  ctx->panel_flag_dev = static_cast<unsigned *>(hd);
   unsigned *where = ctx->panel_state + kPanelStateWords;
   hipLaunchKernelGGL(k_panel_probe, dim3(kPanelXcds * kPanelRanks), dim3(64), 0, ctx->stream, where);
   DLMI_LAUNCH_CHECK(ctx, "k_panel_probe");
@@ -244,36 +259,63 @@ int panel_init(dlmi_ctx *ctx) {
   return DLMI_OK;
 }
 
+void panel_destroy(dlmi_ctx *ctx) {
+  if (ctx->panel_state != nullptr) (void)hipFree(ctx->panel_state);
+  if (ctx->panel_flag_host != nullptr) (void)hipHostFree(ctx->panel_flag_host);
+  ctx->panel_state = nullptr;
+  ctx->panel_flag_host = ctx->panel_flag_dev = nullptr;
+  ctx->panel_ok = 0;
+}
+
 // Panel kernels of different streams must not run side by side (each needs all its workgroups resident).
 // As long as one stream launches them, nothing is done.  When a launch comes from another stream than the
-// previous one (outside a stream capture), an event is recorded on the previous stream - behind its last
-// panel kernel - and the new stream waits for it.
+// previous one, an event is recorded on the previous stream - behind its last panel kernel - and the new
+// stream waits for it.  Stream capture: a kernel recorded into a graph runs whenever the graph is replayed,
+// which this library does not see, so no event can order it.  The first stream of a device that records a
+// panel kernel therefore becomes the only one that may launch them at all: while it holds that role, panel
+// launches of any other stream (recorded or not) are refused and take the multi-launch kernels, and it gives
+// the role up when its context is destroyed or given another stream.  A capture on a stream while ANOTHER
+// stream has panel kernels in flight outside a capture is refused as well.
 static bool panel_capturing(hipStream_t s) {
   hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(s, &cs) != hipSuccess) { (void)hipGetLastError(); return true; }
   return cs != hipStreamCaptureStatusNone;
 }
-int panel_order_launch(dlmi_ctx *ctx) {
+int panel_admit(dlmi_ctx *ctx) {
   std::lock_guard<std::mutex> lock(g_order_mutex);
-  DeviceOrder &o = g_order[ctx->device >= 0 && ctx->device < 64 ? ctx->device : 0];
-  if (!o.recorded || o.stream == ctx->stream) return DLMI_OK;
-  if (panel_capturing(ctx->stream) || panel_capturing(o.stream)) return DLMI_OK;
+  DeviceOrder &o = order_of(ctx);
+  if (o.graph_owner_ctx != nullptr && o.graph_owner != ctx->stream) return 0;
+  if (panel_capturing(ctx->stream)) {
+    if (o.recorded && o.stream != ctx->stream) return 0;  // another stream's panel kernels may still be running
+    o.graph_owner = ctx->stream;
+    o.graph_owner_ctx = ctx;
+    return 1;
+  }
+  if (!o.recorded || o.stream == ctx->stream) return 1;
   if (o.event == nullptr) DLMI_HIP(ctx, hipEventCreateWithFlags(&o.event, hipEventDisableTiming));
   DLMI_HIP(ctx, hipEventRecord(o.event, o.stream));
   DLMI_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.event, 0));
-  return DLMI_OK;
+  return 1;
 }
 void panel_launched(dlmi_ctx *ctx) {
-  ctx->panel_used = 1;
   std::lock_guard<std::mutex> lock(g_order_mutex);
-  DeviceOrder &o = g_order[ctx->device >= 0 && ctx->device < 64 ? ctx->device : 0];
+  DeviceOrder &o = order_of(ctx);
+  if (o.graph_owner == ctx->stream && o.graph_owner_ctx == ctx && panel_capturing(ctx->stream)) {
+    ctx->panel_in_graph = 1;
+    return;  // nothing was launched: the kernel runs when the graph does
+  }
   o.stream = ctx->stream;
   o.recorded = true;
 }
 
 void panel_release_stream(dlmi_ctx *ctx) {
   std::lock_guard<std::mutex> lock(g_order_mutex);
-  DeviceOrder &o = g_order[ctx->device >= 0 && ctx->device < 64 ? ctx->device : 0];
+  DeviceOrder &o = order_of(ctx);
+  if (o.graph_owner_ctx == ctx) {
+    // graphs recorded on this stream must not be replayed once the context has let go of it
+    o.graph_owner = nullptr;
+    o.graph_owner_ctx = nullptr;
+  }
   if (!o.recorded || o.stream != ctx->stream) return;
   // nothing of this stream is still running (the caller synchronized it): a later launch from another stream
   // has nothing to wait for, and must not touch a stream handle that may be gone by then
@@ -281,22 +323,23 @@ void panel_release_stream(dlmi_ctx *ctx) {
   o.stream = nullptr;
 }
 
-// After the stream has been synchronized: did a panel kernel give up?  Then the launch's results are not
-// valid; the state words are cleared and the context stays on the multi-launch path.
+// After the stream has been synchronized: did a panel kernel give up, or find the words of an earlier give-up?
+// Then the results of the calls since the last check are not valid; the words are cleared and the context
+// stays on the multi-launch path.  Costs two reads of host memory when nothing happened.
 int panel_check(dlmi_ctx *ctx) {
-  if (!ctx->panel_used || ctx->panel_state == nullptr) return DLMI_OK;
-  ctx->panel_used = 0;
-  unsigned host[kPanelStateWords];
-  DLMI_HIP(ctx, hipMemcpy(host, ctx->panel_state, sizeof host, hipMemcpyDeviceToHost));
-  unsigned bad = 0;
-  for (int x = 0; x < kPanelXcds; ++x) bad |= host[x * kPanelStateStride + 3];
-  if (bad == 0) return DLMI_OK;
+  if (ctx->panel_flag_host == nullptr) return DLMI_OK;
+  unsigned volatile *const flag = ctx->panel_flag_host;
+  unsigned const gave_up = flag[0], found_stale = flag[1];
+  if (gave_up == 0 && found_stale == 0) return DLMI_OK;
+  flag[0] = 0;
+  flag[1] = 0;
   ctx->panel_ok = 0;
   (void)hipMemset(ctx->panel_state, 0, kPanelStateWords * sizeof(unsigned));
   return dlmi_fail(ctx, DLMI_E_HIP,
                    "a single-launch normalization kernel did not see all of its workgroups resident and gave up "
-                   "(another kernel held compute units for a second): the results of that call are not valid; "
-                   "this context uses the multi-launch kernels from now on");
+                   "(another kernel held compute units for too long)%s: the results of the calls since the last "
+                   "synchronization are not valid; this context uses the multi-launch kernels from now on",
+                   found_stale != 0 ? ", and later launches found its barrier words still in place" : "");
 }
 
 size_t panel_scratch_bytes(size_t H) { return static_cast<size_t>(kPanelRanks) * 3 * H * sizeof(float) + 4096; }
@@ -321,10 +364,10 @@ int panel_fwd_try(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c, bool
   a.fin.momentum = c.momentum; a.fin.eps = c.eps; a.fin.r_max = c.r_max; a.fin.d_max = c.d_max;
   a.fin.renorm = c.norm == DLMI_NORM_BATCH_RENORM ? 1 : 0;
   a.drop_mode = c.drop_mode; a.drop_scale = c.drop_scale;
-  a.state = ctx->panel_state;
+  a.sync = panel_sync_of(ctx);
   a.part = static_cast<float *>(scratch);
-  rc = panel_order_launch(ctx);
-  if (rc != DLMI_OK) return rc;
+  rc = panel_admit(ctx);
+  if (rc <= 0) return rc;
   DLMI_DISPATCH_ACT(c.act, {
     if (extra) {
       switch (rpt) {

@@ -73,7 +73,10 @@ bool Driver::make_resident(void) {
   return true;
 }
 
+// Both passes end in a read of the loss sums, which waits for the model's streams: a pass in which a kernel
+// reported a failure there (Model::synchronize) returns HUGE_VAL, like one that could not be set up.
 double Driver::evalt(void) {
+  size_t const errors_before = model.error_count();
   model.reset_loss();
   model.type_state_propagation = PROPAGATION::INFERENCE;
   if (!model.update_mem_batch_size(dataset.n_data)) {
@@ -84,12 +87,14 @@ double Driver::evalt(void) {
   model.n_acc_trial = dataset.n_data * (dataset.seq_w - model.n_time_delay) *
                       (ACCU_FN::CROSS_ENTROPY == model.type_accuracy_function ? size_t(1) : dataset.n_out);
   double const loss = model.get_loss(ENV::NONE);
+  if (model.error_count() != errors_before) return HUGE_VAL;
   model.set_loss(env_type, loss);
   model.set_accu(env_type, model.get_accu(ENV::NONE));
   return loss;
 }
 
 double Driver::train(void) {
+  size_t const errors_before = model.error_count();
   if (model.ptr_array_derivatives_parameters == nullptr) model.clear_training_arrays();
   model.type_state_propagation = PROPAGATION::TRAINING;
   if (!model.update_mem_batch_size(dataset.n_data)) {
@@ -105,6 +110,7 @@ double Driver::train(void) {
   model.n_acc_trial = dataset.n_data * (dataset.seq_w - model.n_time_delay) *
                       (ACCU_FN::CROSS_ENTROPY == model.type_accuracy_function ? size_t(1) : dataset.n_out);
   double const loss = model.get_loss(ENV::NONE);
+  if (model.error_count() != errors_before) return HUGE_VAL;
   model.set_loss(env_type, loss);
   model.set_accu(env_type, model.get_accu(ENV::NONE));
   return loss;
@@ -210,6 +216,9 @@ void Driver::train_st(void) {
   if (irprop) model.loss_rprop_tm1 = model.loss_rprop;
   run_batches(train_rec_, true);
   if (irprop) model.loss_rprop = std::fabs(model.get_loss(v1::ENV::NONE));  // one device-to-host read of the loss sum
+  // gradients of a pass in which a kernel reported a failure are not applied (the wait costs nothing: the loss
+  // is read right after the step anyway)
+  if (!model.synchronize()) return;
   model.Update_Parameter(dataset.n_data, dataset.n_data);
 }
 

@@ -326,8 +326,21 @@ void Model::restore_pass_state(PassState const &s) {
 }
 size_t Model::error_count(void) const { return impl_->n_errors; }
 
+// Waits for both streams.  Every read of results (get_out, get_loss, the download_* calls) comes through here,
+// because this is where a single-launch normalization kernel that gave up its bounded wait is reported: the
+// call fails (once) instead of handing out numbers that are not valid.
 bool Model::synchronize(void) const {
-  return impl_->ctx != nullptr && dlmi_ctx_synchronize(impl_->ctx) == DLMI_OK;
+  if (impl_->ctx == nullptr) return false;
+  bool ok = true;
+  if (impl_->dw_ctx != nullptr && dlmi_ctx_synchronize(impl_->dw_ctx) != DLMI_OK) {
+    ok = false;
+    fail((std::string("synchronize (weight-gradient stream): ") + dlmi_last_error(impl_->dw_ctx)).c_str());
+  }
+  if (dlmi_ctx_synchronize(impl_->ctx) != DLMI_OK) {
+    ok = false;
+    fail("synchronize");
+  }
+  return ok;
 }
 
 // ---------------------------------------------------------------- construction
@@ -956,11 +969,11 @@ bool Model::upload_parameters(void) {
                 impl_->err, "parameter upload");
 }
 bool Model::download_parameters(void) {
-  return hip_ok(hipMemcpy(ptr_array_parameters, impl_->d_params, total_parameters * sizeof(float), hipMemcpyDeviceToHost),
+  return synchronize() && hip_ok(hipMemcpy(ptr_array_parameters, impl_->d_params, total_parameters * sizeof(float), hipMemcpyDeviceToHost),
                 impl_->err, "parameter download");
 }
 bool Model::download_derivatives(void) {
-  return hip_ok(hipMemcpy(ptr_array_derivatives_parameters, impl_->d_dparams, total_parameters * sizeof(float),
+  return synchronize() && hip_ok(hipMemcpy(ptr_array_derivatives_parameters, impl_->d_dparams, total_parameters * sizeof(float),
                           hipMemcpyDeviceToHost), impl_->err, "gradient download");
 }
 bool Model::upload_derivatives(void) {
@@ -976,7 +989,8 @@ bool Model::upload_moving_statistics(void) {
 }
 bool Model::download_moving_statistics(void) {
   size_t const n = total_normalized_units * sizeof(float);
-  return hip_ok(hipMemcpy(ptr_array_normalized_batch_units_means_averages, impl_->d_mov_mean, n, hipMemcpyDeviceToHost),
+  return synchronize() &&
+         hip_ok(hipMemcpy(ptr_array_normalized_batch_units_means_averages, impl_->d_mov_mean, n, hipMemcpyDeviceToHost),
                 impl_->err, "moving mean download") &&
          hip_ok(hipMemcpy(ptr_array_normalized_batch_units_variances_averages, impl_->d_mov_std, n, hipMemcpyDeviceToHost),
                 impl_->err, "moving std download");
@@ -1000,16 +1014,19 @@ bool Model::download_layer(size_t const i, int which, size_t batch, float *out) 
   }
   if (src == nullptr) return fail("download_layer: this entry has no such buffer");
   if (batch > impl_->allocated_batch) return fail("download_layer: batch larger than the allocation");
-  return hip_ok(hipMemcpy(out, src, n * sizeof(float), hipMemcpyDeviceToHost), impl_->err, "layer download");
+  return synchronize() && hip_ok(hipMemcpy(out, src, n * sizeof(float), hipMemcpyDeviceToHost), impl_->err, "layer download");
 }
 
+// not-a-number when the pass behind the sums failed (see synchronize())
 double Model::get_loss_sum(void) const {
   double s[2] = {0, 0};
+  if (!synchronize()) return std::numeric_limits<double>::quiet_NaN();
   (void)hipMemcpy(s, impl_->d_stats, sizeof(s), hipMemcpyDeviceToHost);
   return s[0];
 }
 double Model::get_accuracy_sum(void) const {
   double s[2] = {0, 0};
+  if (!synchronize()) return std::numeric_limits<double>::quiet_NaN();
   (void)hipMemcpy(s, impl_->d_stats, sizeof(s), hipMemcpyDeviceToHost);
   return s[1];
 }
@@ -1235,6 +1252,7 @@ var const *Model::get_out(size_t const data_index, size_t const) const {
   Layer const &o = ptr_array_layers[total_layers - 1];
   if (!impl_->out_valid) {
     impl_->out_host.resize(impl_->out_batch * o.n_out);
+    if (!synchronize()) return nullptr;
     if (!hip_ok(hipMemcpy(impl_->out_host.data(), o.d_outputs, impl_->out_host.size() * sizeof(float),
                           hipMemcpyDeviceToHost), impl_->err, "output download"))
       return nullptr;
@@ -1313,6 +1331,10 @@ uint64_t Model::launch_signature(void) const {
   DLMI_MIX(scratch_generation);
   unsigned long long const dw_scratch_generation = impl_->dw_ctx != nullptr ? dlmi_ctx_scratch_generation(impl_->dw_ctx) : 0ull;
   DLMI_MIX(dw_scratch_generation);
+  // which normalization kernels a layer launches: a recording that holds single-launch kernels is made again once
+  // the context has gone back to the multi-launch ones
+  int const panel_kernels = dlmi_ctx_norm_panel_enabled(impl_->ctx);
+  DLMI_MIX(panel_kernels);
   DLMI_MIX(type_loss_function); DLMI_MIX(type_accuracy_function); DLMI_MIX(acc_var);
   DLMI_MIX(normalization_momentum_average); DLMI_MIX(normalization_epsilon);
   DLMI_MIX(batch_renormalization_r_correction_maximum); DLMI_MIX(batch_renormalization_d_correction_maximum);

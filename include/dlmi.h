@@ -85,6 +85,19 @@ int dlmi_ctx_reserve_layer(dlmi_ctx *ctx, size_t B, size_t K, size_t H);
 unsigned long long dlmi_ctx_scratch_generation(dlmi_ctx const *ctx);
 /* Compute units of the context's device (for callers sizing their own work). */
 int dlmi_ctx_compute_units(dlmi_ctx const *ctx);
+/* The single-launch normalization kernels (one workgroup per compute unit, the 32 of an XCD exchanging column
+ * sums through their L2 behind a bounded wait) have no counterpart in the reference.
+ * dlmi_ctx_synchronize returns DLMI_E_HIP ONCE when such a kernel gave up its wait since the last
+ * synchronization (the results of the calls in between are not valid; the context runs the multi-launch kernels
+ * from then on, and later synchronizations return DLMI_OK again).
+ * dlmi_ctx_norm_panel_enabled: 1 while the context may still launch them, 0 otherwise (device without 8 x 32
+ * compute units, DLMI_NORM_PANEL=0, or after a give-up); callers that record launches key their recordings on it.
+ * dlmi_ctx_norm_panel_poke is a test hook: after synchronizing the stream it writes `value` into word `word`
+ * (0 rank tickets, 1 / 4 arrivals at even / odd panels, 2 departures, 3 abort) of XCD `xcd`'s barrier state, so
+ * that a test can make the next launch's count impossible to complete and, with a small DLMI_PANEL_SPIN_LIMIT
+ * (polls per wait, read at dlmi_ctx_create), drive the give-up branch while every kernel still exits normally. */
+int dlmi_ctx_norm_panel_enabled(dlmi_ctx const *ctx);
+int dlmi_ctx_norm_panel_poke(dlmi_ctx *ctx, unsigned xcd, unsigned word, unsigned value);
 /* How a product C[M,N] = A[M,K] . B[K,N] would be launched on a device with `compute_units` CUs: tile shape, K
  * slices (1 = none; more = partial products plus a fixed-order sum) and register stages of the K loop.  Host
  * arithmetic only, no device needed: no counterpart in the reference (whose loops have no tiles); for callers and

@@ -237,3 +237,160 @@ def test_panel_kernels_beside_another_kernel(twins, pkg):
     finally:
         torch.cuda.synchronize()
         other.close()
+
+
+# ---------------------------------------------------------------- the bounded wait's give-up branch
+def spin_limited(pkg, limit=64):
+    os.environ["DLMI_PANEL_SPIN_LIMIT"] = str(limit)
+    try:
+        return pkg.Dlmi(0)
+    finally:
+        del os.environ["DLMI_PANEL_SPIN_LIMIT"]
+
+
+def test_a_give_up_is_reported_once_and_the_context_falls_back(twins, pkg):
+    """The give-up branch, driven from the host so that every kernel still exits normally: one rank ticket of
+    XCD 0 is taken before the launch, so one of that XCD's 32 workgroups is told it is the 33rd and leaves at
+    once, and the count of the other 31 can never complete; with a spin limit of 64 polls they give up within
+    microseconds.  The synchronization after the call reports it, once; the context then runs the multi-launch
+    kernels (same bits as a context that never had the panel path), and its barrier words are back at zero."""
+    _, plain = twins
+    ctx = spin_limited(pkg)
+    try:
+        assert ctx.norm_panel_enabled()
+        d = make(4096, 1024, 21)
+        good, *_ = run_fwd(ctx, pkg, d, "ELU", "NONE", False, False)  # a normal panel launch first
+        ctx.norm_panel_poke(0, 0, 1)
+        with pytest.raises(pkg.DlmiError, match="gave up"):
+            run_fwd(ctx, pkg, d, "ELU", "NONE", False, False)
+        assert not ctx.norm_panel_enabled()
+        ctx.synchronize()  # reported once
+        again, desc, mask, st = run_fwd(ctx, pkg, d, "ELU", "NONE", False, False)
+        want, *_ = run_fwd(plain, pkg, d, "ELU", "NONE", False, False)
+        for k in want:
+            assert np.array_equal(again[k], want[k]), k
+        for k in ("mean", "std", "r", "d"):
+            assert_close(again[k], good[k], 2e-6, k)
+        # backward: also the multi-launch kernels now
+        a = run_bwd(ctx, pkg, d, desc, mask, st)
+        b = run_bwd(plain, pkg, d, desc, mask, st)
+        for k in a:
+            assert np.array_equal(a[k], b[k]), k
+    finally:
+        ctx.close()
+
+
+def test_a_launch_that_finds_stale_barrier_words_is_reported(pkg):
+    """What a give-up leaves behind (tickets beyond 32) makes every workgroup of a later launch leave at once.
+    That launch says so through the host word, so the call is reported like the give-up itself."""
+    ctx = spin_limited(pkg)
+    try:
+        d = make(2048, 1024, 22)
+        for x in range(8):
+            ctx.norm_panel_poke(x, 0, 32)
+        with pytest.raises(pkg.DlmiError, match="not valid"):
+            run_fwd(ctx, pkg, d, "RELU", "NONE", False, False)
+        assert not ctx.norm_panel_enabled()
+        a, *_ = run_fwd(ctx, pkg, d, "RELU", "NONE", False, False)
+        assert np.isfinite(a["y"]).all()
+    finally:
+        ctx.close()
+
+
+def test_a_give_up_inside_a_model_fails_the_step_and_the_next_one_is_right(pkg):
+    """Through the facade: the step whose normalization kernel gave up returns false (every read of results
+    waits through the context), the model then matches a twin that never used the panel kernels, bit for bit."""
+    import ctypes
+    from deep_learning_amd.model import Model
+    from oracle.binding import NORM, STATE
+    lib = pkg.load_library()
+    lib.dlmi_model_context.restype = ctypes.c_void_p
+
+    def build(env):
+        os.environ.update(env)
+        try:
+            M = Model(lib, [64, 1024, 4])
+        finally:
+            for k in env:
+                del os.environ[k]
+        M.set_layer(1, ACT["ELU"], NORM["BRN"])
+        M.set_layer(2, ACT["SOFTMAX"])
+        M.set_norm_hyper(0.99, 1e-5, 3.0, 5.0)
+        M.prepare(2048)
+        M.glorot_uniform(1)
+        return M
+
+    M, T = build({"DLMI_PANEL_SPIN_LIMIT": "64"}), build({"DLMI_NORM_PANEL": "0"})
+    try:
+        rng = np.random.default_rng(3)
+        X = rng.standard_normal((2048, 64), dtype=np.float32)
+        Y = np.eye(4, dtype=np.float32)[rng.integers(0, 4, 2048)]
+        ctx = ctypes.c_void_p(lib.dlmi_model_context(M.h))
+        assert lib.dlmi_ctx_norm_panel_enabled(ctx) == 1
+        assert lib.dlmi_ctx_norm_panel_poke(ctx, ctypes.c_uint(0), ctypes.c_uint(0), ctypes.c_uint(1)) == 0
+        with pytest.raises(RuntimeError, match="gave up"):
+            M.step(STATE["TRAINING"], X, Y)
+        assert lib.dlmi_ctx_norm_panel_enabled(ctx) == 0
+        # start both from the same state again
+        for m in (M, T):
+            m.clear_training_arrays()
+            mv = m.get_moving()
+            m.set_moving(np.zeros_like(mv[0]), np.ones_like(mv[1]))
+            m.step(STATE["TRAINING"], X, Y)
+        assert np.array_equal(np.array(M.get_dparams()), np.array(T.get_dparams()))
+        assert np.array_equal(np.array(M.layer_buffer(2, 3)), np.array(T.layer_buffer(2, 3)))
+    finally:
+        M.close()
+        T.close()
+
+
+def test_recorded_panel_kernels_keep_other_streams_on_the_multi_launch_path(twins, pkg):
+    """A panel kernel recorded into a HIP graph runs whenever the graph is replayed, where no event of this
+    library can order it against panel kernels of other streams.  The stream that records one therefore becomes
+    the only stream of the device that launches them: another context's call, on another stream, takes the
+    multi-launch kernels (bit-identical to a context without the panel path) while the graph's owner lives, and
+    every replay - with eager work of both contexts between the replays - gives the eager result."""
+    _, plain = twins
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    owner, other = pkg.Dlmi(0), pkg.Dlmi(0)
+    try:
+        owner.set_stream(s1)
+        other.set_stream(s2)
+        B, H = 2048, 1024
+        d = make(B, H, 31)
+        desc = pkg.Dlmi.desc(ACT["ELU"], renorm=True, momentum=0.9, eps=1e-5, r_max=3.0, d_max=5.0)
+        x, ga, be = dev(d["x"]), dev(d["gamma"]), dev(d["beta"])
+        y = torch.empty(B, H, device="cuda")
+        st = {k: torch.empty(H, device="cuda") for k in ("mean", "std", "r", "d")}
+        mm0, ms0 = dev(d["mm"]), dev(d["ms"])
+        mm, ms = mm0.clone(), ms0.clone()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(s1):
+            owner.fused_fwd(desc, x, ga, be, mm, ms, out=y, stats=st)  # eager: a panel launch
+        owner.synchronize()
+        eager = dict(y=y.cpu().numpy(), mean=st["mean"].cpu().numpy(), mov_mean=mm.cpu().numpy())
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s1):
+            owner.fused_fwd(desc, x, ga, be, mm, ms, out=y, stats=st)
+        for _ in range(3):
+            mm.copy_(mm0)
+            ms.copy_(ms0)
+            y.zero_()
+            torch.cuda.synchronize()
+            g.replay()
+            # the other stream's call while the owner's graph may be running: multi-launch kernels
+            with torch.cuda.stream(s2):
+                a, *_ = run_fwd(other, pkg, d, "ELU", "NONE", False, False)
+            torch.cuda.synchronize()
+            owner.synchronize()
+            assert np.array_equal(y.cpu().numpy(), eager["y"])
+            assert np.array_equal(st["mean"].cpu().numpy(), eager["mean"])
+            assert np.array_equal(mm.cpu().numpy(), eager["mov_mean"])
+            b, *_ = run_fwd(plain, pkg, d, "ELU", "NONE", False, False)
+            for k in a:
+                assert np.array_equal(a[k], b[k]), k
+        del g
+    finally:
+        torch.cuda.synchronize()
+        owner.close()
+        other.close()
