@@ -18,7 +18,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libdlmi.so")
+# DLMI_LIBRARY in the environment names another build of the library (tuning runs); the default is the in-tree one
+LIB_PATH = os.environ.get("DLMI_LIBRARY") or os.path.join(_HERE, "lib", "libdlmi.so")
 
 c_sz = ctypes.c_size_t
 c_int = ctypes.c_int
@@ -44,6 +45,7 @@ C_ABI_SYMBOLS = [
     "dlmi_fused_norm_act_fwd_noalloc", "dlmi_fused_norm_act_residual_fwd", "dlmi_fc_norm_act_residual_fwd",
     "dlmi_fc_softmax_fwd", "dlmi_fc_bwd_dx_norm_act_bwd",
     "dlmi_ctx_reserve_layer", "dlmi_ctx_scratch_generation", "dlmi_ctx_norm_panel_enabled", "dlmi_ctx_norm_panel_poke",
+    "dlmi_fc_bwd_dw_grouped", "dlmi_fused_norm_act_bwd_db",
 ]
 
 
@@ -52,6 +54,11 @@ class FusedDesc(ctypes.Structure):
     _fields_ = [("norm", c_int), ("act", c_int), ("dropout", c_int), ("mask_per_element", c_int),
                 ("dropout_bwd", c_int), ("momentum", c_f), ("eps", c_f), ("r_max", c_f), ("d_max", c_f),
                 ("drop_scale", c_f)]
+
+
+class DwProblem(ctypes.Structure):
+    _fields_ = [("B", ctypes.c_size_t), ("K", ctypes.c_size_t), ("H", ctypes.c_size_t), ("Xin", ctypes.c_void_p),
+                ("dZ", ctypes.c_void_p), ("dW", ctypes.c_void_p), ("db", ctypes.c_void_p)]
 
 
 class DlmiError(RuntimeError):
@@ -175,6 +182,15 @@ class Dlmi:
         self._ck(self.lib.dlmi_fc_bwd_dw(self.ctx, c_sz(B), c_sz(K), c_sz(H), _p(Xin), _p(dZ), _p(dW), _p(db),
                                          c_int(1 if accumulate else 0)))
         return dW, db
+
+    def fc_bwd_dw_grouped(self, problems, accumulate=False):
+        """problems: list of (Xin, dZ, dW, db or None); one launch per kernel variant (dlmi_fc_bwd_dw_grouped)."""
+        arr = (DwProblem * len(problems))()
+        for a, (Xin, dZ, dW, db) in zip(arr, problems):
+            self._chk(Xin, dZ, dW, db)
+            a.B, a.K, a.H = Xin.shape[0], Xin.shape[1], dZ.shape[1]
+            a.Xin, a.dZ, a.dW, a.db = _p(Xin), _p(dZ), _p(dW), _p(db)
+        self._ck(self.lib.dlmi_fc_bwd_dw_grouped(self.ctx, c_sz(len(problems)), arr, c_int(1 if accumulate else 0)))
 
     def bias_fwd(self, Z, bias):
         self._chk(Z, bias)
@@ -408,10 +424,17 @@ class Dlmi:
                                                _p(mov_mean), _p(mov_std), _p(s["r"]), _p(s["d"]), _p(y)))
         return Z, y, s
 
-    def fused_bwd(self, desc, x, gamma, beta, stats, dY, dgamma, dbeta, mask=None, out=None):
-        self._chk(x, gamma, beta, dY, dgamma, dbeta, mask, out)
+    def fused_bwd(self, desc, x, gamma, beta, stats, dY, dgamma, dbeta, mask=None, out=None, db=None, accumulate_db=False):
+        """db: also form the bias gradient sum_b dX[b, :] in the pass that writes dX (dlmi_fused_norm_act_bwd_db)."""
+        self._chk(x, gamma, beta, dY, dgamma, dbeta, mask, out, db)
         B, H = x.shape
         dX = out if out is not None else self.empty(B, H)
+        if db is not None:
+            self._ck(self.lib.dlmi_fused_norm_act_bwd_db(
+                self.ctx, ctypes.byref(desc), c_sz(B), c_sz(H), _p(x), _p(gamma), _p(beta), _p(mask), _p(stats["mean"]),
+                _p(stats["std"]), _p(stats["r"]), _p(stats["d"]), _p(dY), _p(dgamma), _p(dbeta), _p(dX), _p(db),
+                c_int(1 if accumulate_db else 0)))
+            return dX
         self._ck(self.lib.dlmi_fused_norm_act_bwd(self.ctx, ctypes.byref(desc), c_sz(B), c_sz(H), _p(x), _p(gamma),
                                                   _p(beta), _p(mask), _p(stats["mean"]), _p(stats["std"]),
                                                   _p(stats["r"]), _p(stats["d"]), _p(dY), _p(dgamma), _p(dbeta),

@@ -201,9 +201,16 @@ __device__ __forceinline__ void sched_spread() {
   }
 }
 
-template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int WAVES_PER_EU, int RST>
-__global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
-void k_gemm_f32(GemmArgs g) {
+// XCD-aware order of a launch's workgroups: the ids that land on one XCD (id % 8) walk one compact eighth of
+// the tiles.
+__device__ __forceinline__ unsigned xcd_order(unsigned id, unsigned ntiles) {
+  return ntiles % kXcds == 0 ? (id % kXcds) * (ntiles / kXcds) + id / kXcds : id;
+}
+
+// One tile of one product: tile number `lid` (in the grouped order below) of K slice `zslice` of `nslices`.
+template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int RST>
+__device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid, unsigned const zslice, unsigned const nslices,
+                                          float *__restrict__ lds) {
   constexpr bool FAST = MODE == kFast;          // no edge anywhere: unguarded stores
   constexpr bool FAST_LOOP = MODE != kGuarded;  // the scheduled K loop
   using TA = TileShape<BM, BK, A_KCONTIG>;
@@ -211,13 +218,9 @@ void k_gemm_f32(GemmArgs g) {
   constexpr int WM = BM / 2, WN = BN / 2;  // wavefront tile
   constexpr int TM = WM / 32, TN = WN / 32;
   static_assert(BK % 8 == 0, "K tile is consumed in groups of 8");
-  extern __shared__ __attribute__((aligned(16))) float lds[];  // 2 stages of (A tile, B tile)
-  constexpr int kStage = TA::kFloats + TB::kFloats;
+  constexpr int kStage = TA::kFloats + TB::kFloats;  // lds: 2 stages of (A tile, B tile)
 
-  // ---- which tile: XCD-aware remap, then grouped ordering -------------------
-  unsigned const ntiles = g.tiles_m * g.tiles_n;
-  unsigned lid = blockIdx.x;
-  if (ntiles % kXcds == 0) lid = (blockIdx.x % kXcds) * (ntiles / kXcds) + blockIdx.x / kXcds;
+  // ---- which tile: walked in groups of 8 rows of tiles -----------------------
   unsigned const per_group = kGroupM * g.tiles_n;
   unsigned const first_m = (lid / per_group) * kGroupM;
   unsigned const gsize = (g.tiles_m - first_m) < kGroupM ? (g.tiles_m - first_m) : kGroupM;
@@ -226,7 +229,7 @@ void k_gemm_f32(GemmArgs g) {
   size_t const m0 = static_cast<size_t>(tile_m) * BM;
   size_t const n0 = static_cast<size_t>(tile_n) * BN;
 
-  size_t const k_begin = blockIdx.z * g.k_per_split;
+  size_t const k_begin = zslice * g.k_per_split;
   size_t const k_end = (k_begin + g.k_per_split < g.K) ? k_begin + g.k_per_split : g.K;
   int const ktiles = static_cast<int>((k_end - k_begin + BK - 1) / BK);
 
@@ -371,8 +374,8 @@ void k_gemm_f32(GemmArgs g) {
 
   // ---- epilogue: accumulator register e of lane l holds
   //      row (e/4)*8 + (l/32)*4 + e%4, column l%32 of its 32x32 block
-  bool const split = gridDim.z > 1;
-  float *const out = split ? g.split_out + static_cast<size_t>(blockIdx.z) * g.M * g.N : g.C;
+  bool const split = nslices > 1;
+  float *const out = split ? g.split_out + static_cast<size_t>(zslice) * g.M * g.N : g.C;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -432,6 +435,49 @@ void k_gemm_f32(GemmArgs g) {
       }
     }
   }
+}
+
+template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int WAVES_PER_EU, int RST>
+__global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
+void k_gemm_f32(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  gemm_tile<BM, BN, BK, A_KCONTIG, B_KCONTIG, MODE, RST>(g, xcd_order(blockIdx.x, g.tiles_m * g.tiles_n), blockIdx.z, gridDim.z, lds);
+}
+
+// Several independent products of one kernel variant in ONE launch (the weight gradients of a network's layers:
+// every layer's dZ exists once the backward pass has run).  The workgroups walk the concatenated tile lists in
+// the XCD-aware order, so each XCD works on whole products and keeps their operands in its L2; a launch of
+// many rounds of tiles runs at the rate of one large product instead of paying every product's start and tail.
+constexpr int kGroupMax = 32;
+struct GemmGroupProblem {
+  float const *A, *B;
+  float *C;
+  unsigned M, N, K;
+  unsigned tiles_n;
+  unsigned tile_end;  // tiles of this and all earlier problems
+};
+struct GemmGroupArgs {
+  GemmGroupProblem p[kGroupMax];
+  unsigned n, total_tiles;
+  int accumulate;
+};
+template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int WAVES_PER_EU, int RST>
+__global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
+void k_gemm_f32_group(GemmGroupArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  unsigned const t = xcd_order(blockIdx.x, a.total_tiles);
+  unsigned pi = 0;
+  while (pi + 1 < a.n && t >= a.p[pi].tile_end) ++pi;
+  GemmGroupProblem const &q = a.p[pi];
+  GemmArgs g;
+  g.A = q.A; g.B = q.B; g.C = q.C; g.bias = nullptr;
+  g.M = q.M; g.N = q.N; g.K = q.K;
+  g.lda = A_KCONTIG ? q.K : q.M; g.ldb = B_KCONTIG ? q.K : q.N; g.ldc = q.N;
+  g.k_per_split = q.K; g.split_out = nullptr; g.stats_out = nullptr;
+  g.snap_a = nullptr; g.snap_b = nullptr; g.snap_out = nullptr;
+  g.accumulate = a.accumulate; g.a_vec = 1; g.b_vec = 1;
+  g.tiles_n = q.tiles_n; g.tiles_m = (q.M + BM - 1) / BM;
+  gemm_tile<BM, BN, BK, A_KCONTIG, B_KCONTIG, kFast, RST>(g, t - (pi == 0 ? 0u : a.p[pi - 1].tile_end), 0u, 1u, lds);
 }
 
 // Fixed-order sum of the split-K partial products (+ bias, + previous C): slice 0, 1, 2, ... as before, with
@@ -588,6 +634,73 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   return DLMI_OK;
 }
 
+// ---- several products in one launch
+struct GroupItem {
+  size_t M, N, K;
+  float const *A, *B;
+  float *C;
+};
+template <int BM, int BN, int BK, bool AK, bool BKC, int WPE, int RST>
+static int launch_group(dlmi_ctx *ctx, GroupItem const *items, size_t n, int accumulate) {
+  using TA = TileShape<BM, BK, AK>;
+  using TB = TileShape<BN, BK, BKC>;
+  constexpr size_t lds_bytes = 2 * (TA::kFloats + TB::kFloats) * sizeof(float);
+  auto const kern = k_gemm_f32_group<BM, BN, BK, AK, BKC, WPE, RST>;
+  static bool attr_set_on[64] = {false};
+  bool &attr_set = attr_set_on[ctx->device >= 0 && ctx->device < 64 ? ctx->device : 0];
+  if (!attr_set) {
+    DLMI_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<void const *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(lds_bytes)));
+    attr_set = true;
+  }
+  for (size_t first = 0; first < n; first += kGroupMax) {
+    GemmGroupArgs a;
+    a.n = static_cast<unsigned>(n - first < static_cast<size_t>(kGroupMax) ? n - first : kGroupMax);
+    a.accumulate = accumulate;
+    unsigned total = 0;
+    for (unsigned i = 0; i < a.n; ++i) {
+      GroupItem const &it = items[first + i];
+      GemmGroupProblem &q = a.p[i];
+      q.A = it.A; q.B = it.B; q.C = it.C;
+      q.M = static_cast<unsigned>(it.M); q.N = static_cast<unsigned>(it.N); q.K = static_cast<unsigned>(it.K);
+      q.tiles_n = static_cast<unsigned>(it.N / BN);
+      total += static_cast<unsigned>(it.M / BM) * q.tiles_n;
+      q.tile_end = total;
+    }
+    for (unsigned i = a.n; i < static_cast<unsigned>(kGroupMax); ++i) a.p[i] = a.p[a.n - 1];
+    a.total_tiles = total;
+    hipLaunchKernelGGL(kern, dim3(total), dim3(kGemmThreads), lds_bytes, ctx->stream, a);
+    DLMI_LAUNCH_CHECK(ctx, "k_gemm_f32_group");
+  }
+  return DLMI_OK;
+}
+
+// Whether a product may join a grouped launch, and which kernel variant it would run there: shapes that are
+// multiples of their tile, 16-byte aligned operands, no K split.  Returns the variant key (tile choice * 4 +
+// register stages), or -1.
+template <bool AK, bool BKC>
+static int group_variant(dlmi_ctx const *ctx, GroupItem const &it) {
+  GemmPlan const plan = plan_gemm(ctx->num_cu, it.M, it.N, it.K);
+  if (plan.splits != 1 || plan.choice == 1) return -1;
+  size_t const lda = AK ? it.K : it.M, ldb = BKC ? it.K : it.N;
+  bool const vec = lda % 4 == 0 && ldb % 4 == 0 && dlmi_aligned16(it.A) && dlmi_aligned16(it.B);
+  if (!vec || it.K % plan.bk != 0 || it.M % plan.bm != 0 || it.N % plan.bn != 0) return -1;
+  if (it.M > 0xffffffffull || it.N > 0xffffffffull || it.K > 0xffffffffull) return -1;
+  int const rst = plan.choice == 2 ? 1 : gemm_register_stages(plan.bm, plan.bn, dlmi_ceil_div(it.K, plan.bk));
+  return plan.choice * 4 + rst;
+}
+template <bool AK, bool BKC>
+static int launch_group_variant(dlmi_ctx *ctx, int variant, GroupItem const *items, size_t n, int accumulate) {
+  switch (variant) {
+    case 0 * 4 + 1: return launch_group<128, 128, 16, AK, BKC, 2, 1>(ctx, items, n, accumulate);
+    case 0 * 4 + 2: return launch_group<128, 128, 16, AK, BKC, 2, 2>(ctx, items, n, accumulate);
+    case 2 * 4 + 1: return launch_group<256, 256, 16, AK, BKC, 1, 1>(ctx, items, n, accumulate);
+    case 3 * 4 + 1: return launch_group<64, 64, 16, AK, BKC, 4, 1>(ctx, items, n, accumulate);
+    case 3 * 4 + 2: return launch_group<64, 64, 16, AK, BKC, 4, 2>(ctx, items, n, accumulate);
+    default: return dlmi_fail(ctx, DLMI_E_INVALID, "no grouped kernel for variant %d", variant);
+  }
+}
+
 }  // namespace dlmi
 
 using namespace dlmi;
@@ -690,6 +803,50 @@ int dlmi_fc_bwd_dw(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin
   if (rc != DLMI_OK || db == nullptr) return rc;
   // db[h] (+)= sum_b dZ[b,h] (update_derivative_fwp_st.cpp:283-302)
   return column_sums(ctx, B, H, dZ, db, accumulate);
+}
+
+int dlmi_fc_bwd_dw_grouped(dlmi_ctx *ctx, size_t n, dlmi_dw_problem const *problems, int accumulate) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, n == 0 || problems != nullptr, "null pointer");
+  // products of one kernel variant share a launch (from two on); everything else goes one by one
+  constexpr size_t kMaxProblems = 256;
+  for (size_t first = 0; first < n; first += kMaxProblems) {
+    size_t const m = n - first < kMaxProblems ? n - first : kMaxProblems;
+    dlmi_dw_problem const *pr = problems + first;
+    int variant[kMaxProblems];
+    GroupItem item[kMaxProblems];
+    for (size_t i = 0; i < m; ++i) {
+      DLMI_REQUIRE(ctx, pr[i].Xin && pr[i].dZ && pr[i].dW, "null pointer");
+      DLMI_REQUIRE(ctx, pr[i].B > 0 && pr[i].K > 0 && pr[i].H > 0, "empty operand");
+      item[i] = GroupItem{pr[i].H, pr[i].K, pr[i].B, pr[i].dZ, pr[i].Xin, pr[i].dW};
+      variant[i] = group_variant<false, false>(ctx, item[i]);  // (a narrow layer is no multiple of a tile: -1)
+    }
+    for (size_t i = 0; i < m; ++i) {
+      if (variant[i] == -2) continue;  // went with an earlier one
+      GroupItem same[kMaxProblems];
+      size_t ns = 0;
+      if (variant[i] >= 0)
+        for (size_t j = i; j < m; ++j)
+          if (variant[j] == variant[i]) same[ns++] = item[j];
+      if (ns >= 2) {
+        int const v = variant[i];
+        for (size_t j = i; j < m; ++j)
+          if (variant[j] == v) variant[j] = -2;
+        int rc = launch_group_variant<false, false>(ctx, v, same, ns, accumulate);
+        if (rc != DLMI_OK) return rc;
+        continue;  // (the bias gradients of grouped products follow below)
+      }
+      int rc = dlmi_fc_bwd_dw(ctx, pr[i].B, pr[i].K, pr[i].H, pr[i].Xin, pr[i].dZ, pr[i].dW, pr[i].db, accumulate);
+      if (rc != DLMI_OK) return rc;
+      variant[i] = -3;  // done, bias gradient included
+    }
+    for (size_t i = 0; i < m; ++i)
+      if (variant[i] == -2 && pr[i].db != nullptr) {
+        int rc = column_sums(ctx, pr[i].B, pr[i].H, pr[i].dZ, pr[i].db, accumulate);
+        if (rc != DLMI_OK) return rc;
+      }
+  }
+  return DLMI_OK;
 }
 
 }  // extern "C"

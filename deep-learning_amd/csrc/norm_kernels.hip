@@ -631,6 +631,7 @@ struct BwdArgs {
   float *dgamma, *dbeta;
   float batch_f, batch_scale;
   float *dX;
+  float *db_partial;  // apply with DBSUM: [apply chunks][H] column sums of the dX rows each block stored
   size_t B, H, rows_per_chunk;
   int tx_log2, drop_bwd_masked;
   float drop_scale;
@@ -788,13 +789,28 @@ __global__ __launch_bounds__(kBlock) void k_bwd_finalize(float const *__restrict
 // Pass 2 of bwp_st.cpp:1508-1531 with the activation derivative recomputed.
 // ACC: dX += instead of dX = (the error array of a layer that also receives a
 // shortcut's gradient, bwp_st.cpp:1112-1175).
-template <int VEC, int ACT, int DROPM, bool XHAT_GIVEN, bool ACC>
+// DBSUM: every block also stores the column sums of the dX rows it wrote (rows of a thread ascending, then the
+// block's row lanes in the fixed order of block_rows_reduce) to db_partial [chunks][H]; a finalize launch adds
+// the chunks: the bias gradient without a second pass over dX.
+template <int VEC, int ACT, int DROPM, bool XHAT_GIVEN, bool ACC, bool DBSUM = false>
 __global__ __launch_bounds__(kBlock) void k_bwd_apply(BwdArgs a) {
+  __shared__ float lds_db[DBSUM ? 4 * kWave * VEC : 1];
   int const TX = 1 << a.tx_log2;
   int const tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> a.tx_log2;
   size_t const col = (static_cast<size_t>(blockIdx.x) * TX + tx) * VEC;
   RowWalk const w = row_walk(a.B, a.rows_per_chunk, a.tx_log2, ty, true);
-  if (col >= a.H || w.count == 0) return;
+  float dbs[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) dbs[i] = 0.0f;
+  if constexpr (DBSUM) {
+    if (col >= a.H || w.count == 0) {  // idle threads still take part in the block's sum
+      block_rows_reduce<VEC>(dbs, TX, lds_db);
+      if (static_cast<int>(threadIdx.x) < TX && col < a.H) store_f<VEC>(a.db_partial + static_cast<size_t>(blockIdx.y) * a.H + col, dbs);
+      return;
+    }
+  } else {
+    if (col >= a.H || w.count == 0) return;
+  }
   UnitConsts<VEC> uc;
   load_unit_consts<VEC, DROPM, XHAT_GIVEN>(a, col, uc);
   float c1[VEC], c2[VEC], c3[VEC];
@@ -855,6 +871,7 @@ __global__ __launch_bounds__(kBlock) void k_bwd_apply(BwdArgs a) {
                                                       uc.be[i], xh);
       dx[i] = dn * c1[i] + (xv[i] - uc.mu[i]) * c2[i] + c3[i];
       if constexpr (ACC) dx[i] += old[i];
+      if constexpr (DBSUM) dbs[i] += dx[i];
     }
     store_f<VEC>(a.dX + off, dx);
   };
@@ -904,6 +921,10 @@ __global__ __launch_bounds__(kBlock) void k_bwd_apply(BwdArgs a) {
     }
     body(off, xv, dy, mv, old);
   }
+  if constexpr (DBSUM) {
+    block_rows_reduce<VEC>(dbs, TX, lds_db);
+    if (static_cast<int>(threadIdx.x) < TX) store_f<VEC>(a.db_partial + static_cast<size_t>(blockIdx.y) * a.H + col, dbs);
+  }
 }
 
 // ---------------------------------------------------------------- host drivers
@@ -927,7 +948,10 @@ static bool use_vec4(size_t H, std::initializer_list<void const *> ptrs) {
 // block: 256 column groups of 4 units) + H, and the 3*H backward coefficients.
 size_t norm_scratch_bytes(dlmi_ctx const *ctx, size_t H) {
   size_t const blocks = static_cast<size_t>(ctx->num_cu) * ctx->tune.reduce_blocks_per_cu;
-  size_t const multi = 3 * sizeof(float) * (blocks * 1024 + 2 * H) + round_up(3 * H * sizeof(float), 256) + 4096;
+  // (+ one plane [apply chunks][H] for the bias-gradient partials of the backward apply pass)
+  size_t const apply_blocks = static_cast<size_t>(ctx->num_cu) * ctx->tune.apply_bwd_blocks_per_cu;
+  size_t const multi = 3 * sizeof(float) * (blocks * 1024 + 2 * H) + round_up(3 * H * sizeof(float), 256) + 4096 +
+                       sizeof(float) * (apply_blocks * 1024 + H) + 256;
   size_t const panel = panel_scratch_bytes(H);
   return multi > panel ? multi : panel;
 }
@@ -1037,9 +1061,11 @@ static int run_fwd_train(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t 
 static int run_bwd(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, BwdCall const &c) {
   bool const vec4 = use_vec4(H, {c.x, c.gamma, c.beta, c.mean, c.stdv, c.r, c.d, c.xhat, c.dY, c.dX, c.dgamma, c.dbeta}) &&
                     (c.drop_mode == kDropNone || (reinterpret_cast<uintptr_t>(c.mask) & 3u) == 0);
-  if (int const took = small_bwd_try(ctx, B, H, c); took != 0) return took < 0 ? took : DLMI_OK;
+  // the one-launch kernels do not form the bias gradient: where it is asked for, a pass over dX follows them
+  auto then_db = [&](int took) { return took < 0 ? took : (c.db != nullptr ? column_sums(ctx, B, H, c.dX, c.db, c.db_accumulate ? 1 : 0) : DLMI_OK); };
+  if (int const took = small_bwd_try(ctx, B, H, c); took != 0) return then_db(took);
   // a few thousand rows, H a multiple of 512: one launch that reads dY and x once
-  if (int const took = panel_bwd_try(ctx, B, H, c, vec4, sv.data, sv.data_bytes); took != 0) return took < 0 ? took : DLMI_OK;
+  if (int const took = panel_bwd_try(ctx, B, H, c, vec4, sv.data, sv.data_bytes); took != 0) return then_db(took);
   ColGeom g;
   bool const fold = !c.xhat_given && c.dmean == nullptr && c.dstd == nullptr &&
                     fold_geometry(ctx, B, H, vec4, 3, sv.data_bytes, &g);
@@ -1092,6 +1118,23 @@ static int run_bwd(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, Bwd
   a.rows_per_chunk = ctx->tune.apply_interleave ? 0 : ga.rows_per_chunk;
   a.tx_log2 = ga.tx_log2;
   dim3 const agrid(ga.grid_x, ga.nchunks);
+  // the bias gradient as a by-product of this pass: block partials behind the reduction's, then one small launch
+  size_t const db_offset = round_up(coef_bytes + static_cast<size_t>(3) * g.nchunks * H * sizeof(float), 256);
+  bool const db_here = c.db != nullptr && vec4 && !c.xhat_given && !c.accumulate &&
+                       db_offset + static_cast<size_t>(ga.nchunks) * H * sizeof(float) <= sv.data_bytes;
+  a.db_partial = db_here ? reinterpret_cast<float *>(sv.data + db_offset) : nullptr;
+  if (db_here) {
+    DLMI_DISPATCH_ACT(c.act, DLMI_DISPATCH_DROP(c.drop_mode, {
+      hipLaunchKernelGGL((k_bwd_apply<4, ACT, DROPM, false, false, true>), agrid, block, 0, ctx->stream, a);
+    }));
+    DLMI_LAUNCH_CHECK(ctx, "k_bwd_apply");
+    int const ftx = finalize_tx_log2(ga.nchunks);
+    dim3 const fgrid(static_cast<unsigned>(dlmi_ceil_div(H / 4, size_t(1) << ftx)));
+    hipLaunchKernelGGL(k_colsum_finalize<4>, fgrid, block, 0, ctx->stream, a.db_partial, ga.nchunks, H, ftx, c.db,
+                       c.db_accumulate ? 1 : 0);
+    DLMI_LAUNCH_CHECK(ctx, "k_colsum_finalize");
+    return DLMI_OK;
+  }
   if (c.xhat_given) {
     if (vec4)
       hipLaunchKernelGGL((k_bwd_apply<4, DLMI_ACT_LINEAR, kDropNone, true, false>), agrid, block, 0, ctx->stream, a);
@@ -1113,7 +1156,7 @@ static int run_bwd(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, Bwd
     }));
   }
   DLMI_LAUNCH_CHECK(ctx, "k_bwd_apply");
-  return DLMI_OK;
+  return c.db != nullptr ? column_sums(ctx, B, H, c.dX, c.db, c.db_accumulate ? 1 : 0) : DLMI_OK;
 }
 
 static int check_desc(dlmi_ctx *ctx, dlmi_fused_desc const *desc, uint8_t const *mask) {
@@ -1329,6 +1372,29 @@ int dlmi_fused_norm_act_bwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
   c.x = x; c.gamma = gamma; c.beta = beta; c.mean = mean; c.stdv = stdv; c.r = r; c.d = d; c.xhat = nullptr;
   c.dY = dY; c.mask = mask;
   c.dgamma = dgamma; c.dbeta = dbeta; c.dmean = nullptr; c.dstd = nullptr; c.dX = dX;
+  ScratchView sv{};
+  rc = ctx_scratch(ctx, H, &sv);
+  if (rc != DLMI_OK) return rc;
+  return run_bwd(ctx, sv, B, H, c);
+}
+
+int dlmi_fused_norm_act_bwd_db(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
+                               float const *gamma, float const *beta, uint8_t const *mask, float const *mean,
+                               float const *stdv, float const *r, float const *d, float const *dY, float *dgamma,
+                               float *dbeta, float *dX, float *db, int accumulate_db) {
+  if (ctx == nullptr || desc == nullptr) return DLMI_E_INVALID;
+  int rc = check_desc(ctx, desc, mask);
+  if (rc != DLMI_OK) return rc;
+  DLMI_REQUIRE(ctx, B > 0 && H > 0, "empty tensor");
+  DLMI_REQUIRE(ctx, x && gamma && beta && mean && stdv && r && d && dY && dgamma && dbeta && dX && db, "null pointer");
+  BwdCall c;
+  c.act = desc->act; c.xhat_given = false; c.drop_mode = drop_mode_of(desc);
+  c.drop_bwd_masked = desc->dropout_bwd == DLMI_DROP_BWD_MASKED ? 1 : 0;
+  c.drop_scale = drop_scale_of(desc);
+  c.x = x; c.gamma = gamma; c.beta = beta; c.mean = mean; c.stdv = stdv; c.r = r; c.d = d; c.xhat = nullptr;
+  c.dY = dY; c.mask = mask;
+  c.dgamma = dgamma; c.dbeta = dbeta; c.dmean = nullptr; c.dstd = nullptr; c.dX = dX;
+  c.db = db; c.db_accumulate = accumulate_db != 0;
   ScratchView sv{};
   rc = ctx_scratch(ctx, H, &sv);
   if (rc != DLMI_OK) return rc;

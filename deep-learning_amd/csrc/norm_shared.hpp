@@ -118,6 +118,10 @@ struct BwdCall {
   uint8_t const *mask;
   float *dgamma, *dbeta, *dmean, *dstd, *dX;
   bool accumulate = false;  // dX += instead of dX =
+  // optional: db[j] (+)= sum over the rows of the dX this call stores (the bias gradient of the layer,
+  // update_derivative_fwp_st.cpp:283-302), formed while dX is written instead of by a pass of its own
+  float *db = nullptr;
+  bool db_accumulate = false;
   // dY not formed yet: it is the sum of `nslices` partial products [nslices][B][H], added in slice order by
   // the small-batch kernel (the only one that takes them); dY is unused then
   float const *dy_slices = nullptr;

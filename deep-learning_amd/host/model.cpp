@@ -1569,6 +1569,7 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
   hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
   if (side && hipStreamIsCapturing(impl_->stream, &capture) != hipSuccess) (void)hipGetLastError();
   bool const recording = capture != hipStreamCaptureStatusNone;
+  std::vector<dlmi_dw_problem> on_stream;
   for (Layer const *l = last; l != first;) {
     --l;
     size_t const li = static_cast<size_t>(l - ptr_array_layers);
@@ -1591,14 +1592,22 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
       fail("update_derivatives: wait for dZ");
       break;
     }
-    if (dlmi_fc_bwd_dw(beside ? impl_->dw_ctx : impl_->ctx, B, K, l->n_out, in, l->d_errors,
+    if (!beside) {
+      // on the compute stream: collected, and issued below as one call, which puts the products that take the
+      // same kernel variant into one launch (every layer's dZ exists by now: drivers/driver.cpp:253-255)
+      on_stream.push_back(dlmi_dw_problem{B, K, l->n_out, in, l->d_errors, impl_->d_dparams + l->first_connection_index, db});
+      continue;
+    }
+    if (dlmi_fc_bwd_dw(impl_->dw_ctx, B, K, l->n_out, in, l->d_errors,
                        impl_->d_dparams + l->first_connection_index, db, 1) != DLMI_OK) {
       fail("update_derivatives: dlmi_fc_bwd_dw");
-      joined = joined && !beside;  // what was launched beside the chain is still joined below
+      joined = false;  // what was launched beside the chain is still joined below
       break;
     }
-    joined = joined && !beside;
+    joined = false;
   }
+  if (!on_stream.empty() && dlmi_fc_bwd_dw_grouped(impl_->ctx, on_stream.size(), on_stream.data(), 1) != DLMI_OK)
+    fail("update_derivatives: dlmi_fc_bwd_dw_grouped");
   // whatever the compute stream does next (the optimizer step, the next forward pass over the same buffers)
   // comes after the last weight gradient
   if (!joined && (!hip_ok(hipEventRecord(impl_->dw_done, impl_->dw_stream), impl_->err, "update_derivatives: join") ||

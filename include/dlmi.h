@@ -130,6 +130,22 @@ int dlmi_fc_bwd_dx(dlmi_ctx *ctx, size_t B, size_t Hn, size_t H, float const *dZ
 int dlmi_fc_bwd_dw(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ,
                    float *dW, float *db, int accumulate);
 
+/* The weight (and bias) gradients of several layers: dlmi_fc_bwd_dw for each problem, with the products that
+ * take the same kernel variant (same tile shape and register stages, shapes that are multiples of the tile, no
+ * K split) issued as ONE launch over the concatenated tile lists.  In the reference update_derivatives runs
+ * after backward_pass has produced every layer's dZ (drivers/driver.cpp:253-255,
+ * update_derivative_fwp_st.cpp:189-281), so the layers' products are independent of each other; a launch of many
+ * rounds of tiles runs at the rate of one large product instead of paying each product's start and tail.
+ * Results are bit-identical to the one-by-one calls.  `problems` is a host array; pointers inside are device. */
+typedef struct {
+  size_t B, K, H;
+  float const *Xin; /* [B, K] */
+  float const *dZ;  /* [B, H] */
+  float *dW;        /* [H, K] */
+  float *db;        /* [H] or NULL */
+} dlmi_dw_problem;
+int dlmi_fc_bwd_dw_grouped(dlmi_ctx *ctx, size_t n, dlmi_dw_problem const *problems, int accumulate);
+
 /* Z[b,h] += bias[h]  (Forward_Pass__Bias__*, fwp_st.cpp:4498-4516). */
 int dlmi_bias_fwd(dlmi_ctx *ctx, size_t B, size_t H, float const *bias, float *Z);
 
@@ -365,6 +381,17 @@ int dlmi_fused_norm_act_bwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
                             uint8_t const *mask, float const *mean, float const *std,
                             float const *r, float const *d, float const *dY, float *dgamma,
                             float *dbeta, float *dX);
+
+/* dlmi_fused_norm_act_bwd that also forms the bias gradient of the layer, db[j] (+)= sum_b dX[b,j]
+ * (Update_Derivative_Bias, update_derivative_fwp_st.cpp:283-302, applied to the dX this call stores): the pass
+ * that writes dX adds up its own rows per block and one small launch adds the blocks, so no second pass reads dX.
+ * (The reference gives a normalized layer no bias, so it never forms this sum there; a benchmark step that
+ * lists db among its gradients does.)  accumulate_db != 0 adds into db. */
+int dlmi_fused_norm_act_bwd_db(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H,
+                               float const *x, float const *gamma, float const *beta,
+                               uint8_t const *mask, float const *mean, float const *std,
+                               float const *r, float const *d, float const *dY, float *dgamma,
+                               float *dbeta, float *dX, float *db, int accumulate_db);
 
 /* Inference-mode tail: y = f(gamma*((x-mov_mean)/mov_std)+beta), then the
  * inference branch of dropout (plain Bernoulli rescales by keep = drop_scale;
