@@ -551,6 +551,11 @@ def run_layer(args, torch, pkg, dl, name, full):
         step()  # every buffer a part reads has been produced once
         ms = time_events(torch, getattr(step, args.only), args.steps, warmup=args.warmup, min_ms=0.0)
         print("%s: %.4f ms per call over %d calls" % (args.only, ms, args.steps), file=sys.stderr)
+        if os.environ.get("DLMI_GEMM_CLOCK") == "1" and args.only.startswith("gemm"):
+            # the engine clock inside the last of those launches, from the kernel's own counters (no profiler)
+            mhz, us = dl.gemm_clock()
+            print("%s: engine clock inside the launch %.0f MHz (first tile's workgroup lived %.1f us)" % (args.only, mhz, us),
+                  file=sys.stderr)
         return None
 
     # ---- one clean step on the fresh inputs: the results the CPU baseline is compared with

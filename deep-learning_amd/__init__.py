@@ -45,7 +45,7 @@ C_ABI_SYMBOLS = [
     "dlmi_fused_norm_act_fwd_noalloc", "dlmi_fused_norm_act_residual_fwd", "dlmi_fc_norm_act_residual_fwd",
     "dlmi_fc_softmax_fwd", "dlmi_fc_bwd_dx_norm_act_bwd",
     "dlmi_ctx_reserve_layer", "dlmi_ctx_scratch_generation", "dlmi_ctx_norm_panel_enabled", "dlmi_ctx_norm_panel_poke",
-    "dlmi_fc_bwd_dw_grouped", "dlmi_fused_norm_act_bwd_db",
+    "dlmi_fc_bwd_dw_grouped", "dlmi_fused_norm_act_bwd_db", "dlmi_ctx_gemm_clock",
 ]
 
 
@@ -139,6 +139,13 @@ class Dlmi:
 
     def compute_units(self):
         return self.lib.dlmi_ctx_compute_units(self.ctx)
+
+    def gemm_clock(self):
+        """(engine clock in MHz, lifetime in us) of the first tile's workgroup of the last product launched; the
+        context must have been created with DLMI_GEMM_CLOCK=1 in the environment."""
+        mhz, us = ctypes.c_double(0), ctypes.c_double(0)
+        self._ck(self.lib.dlmi_ctx_gemm_clock(self.ctx, ctypes.byref(mhz), ctypes.byref(us)))
+        return mhz.value, us.value
 
     def norm_panel_enabled(self):
         """Whether this context may still launch the single-launch normalization kernels."""

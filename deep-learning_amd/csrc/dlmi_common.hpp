@@ -61,6 +61,9 @@ struct dlmi_ctx {
   int panel_spin_limit = 1 << 20;
   int panel_ok = 0;
   int panel_in_graph = 0;
+  // measurement aid (DLMI_GEMM_CLOCK=1 when the context is created): two 64-bit words in which the first tile of
+  // every product launch leaves the engine clock ticks and the 100 MHz reference ticks it spent
+  unsigned long long *gemm_clock = nullptr;
   char err[512] = {0};
 };
 
@@ -106,6 +109,7 @@ int dlmi_scratch_reserve(dlmi_ctx *ctx, size_t bytes);
 namespace dlmi {
 // Finds the device address of the library's fixed scratch array for the context's device (current).
 int static_scratch_init(dlmi_ctx *ctx);
+void static_scratch_release_stream(dlmi_ctx *ctx);
 // Batch-(re)norm forward tail (finalize + apply) from column-sum partials
 // [2][nchunks][H] that a producer (the GEMM epilogue) already wrote.
 // partial == nullptr: the statistics come from a pass over x.  mov_snapshot != nullptr: [2][H], the moving

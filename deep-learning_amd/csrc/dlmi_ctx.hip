@@ -80,6 +80,15 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
   t.fold_bwd = env_level("DLMI_NORM_FOLD_BWD", t.fold_bwd);
   t.norm_small = env_flag("DLMI_NORM_SMALL", t.norm_small);
   t.fc_narrow = env_flag("DLMI_FC_NARROW", t.fc_narrow);
+  if (env_flag("DLMI_GEMM_CLOCK", 0)) {
+    void *p = nullptr;
+    if (hipMalloc(&p, 2 * sizeof(unsigned long long)) == hipSuccess) {
+      ctx->gemm_clock = static_cast<unsigned long long *>(p);
+      (void)hipMemset(p, 0, 2 * sizeof(unsigned long long));
+    } else {
+      (void)hipGetLastError();
+    }
+  }
   int rc = dlmi_scratch_reserve(ctx, size_t(16) << 20);
   if (rc == DLMI_OK) rc = dlmi::static_scratch_init(ctx);
   if (rc == DLMI_OK) rc = dlmi::panel_init(ctx);
@@ -98,9 +107,11 @@ int dlmi_ctx_destroy(dlmi_ctx *ctx) {
   if (ctx == nullptr) return DLMI_OK;
   (void)hipStreamSynchronize(ctx->stream);
   dlmi::panel_release_stream(ctx);
+  dlmi::static_scratch_release_stream(ctx);
   if (ctx->scratch != nullptr) (void)hipFree(ctx->scratch);
   for (int i = 0; i < ctx->n_retired; ++i) (void)hipFree(ctx->retired[i]);
   dlmi::panel_destroy(ctx);
+  if (ctx->gemm_clock != nullptr) (void)hipFree(ctx->gemm_clock);
   delete ctx;
   return DLMI_OK;
 }
@@ -115,6 +126,7 @@ int dlmi_ctx_set_stream(dlmi_ctx *ctx, void *stream) {
   if (capturing == hipStreamCaptureStatusNone) {
     DLMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
     dlmi::panel_release_stream(ctx);
+    dlmi::static_scratch_release_stream(ctx);
   }
   ctx->stream = static_cast<hipStream_t>(stream);
   return DLMI_OK;
@@ -147,6 +159,19 @@ unsigned long long dlmi_ctx_scratch_generation(dlmi_ctx const *ctx) {
 char const *dlmi_last_error(dlmi_ctx const *ctx) { return ctx != nullptr ? ctx->err : "null context"; }
 
 int dlmi_ctx_compute_units(dlmi_ctx const *ctx) { return ctx != nullptr ? ctx->num_cu : 0; }
+
+int dlmi_ctx_gemm_clock(dlmi_ctx *ctx, double *engine_mhz, double *tile_us) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, ctx->gemm_clock != nullptr, "the context was created without DLMI_GEMM_CLOCK=1");
+  DLMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  unsigned long long t[2] = {0, 0};
+  DLMI_HIP(ctx, hipMemcpy(t, ctx->gemm_clock, sizeof t, hipMemcpyDeviceToHost));
+  DLMI_REQUIRE(ctx, t[1] != 0, "no product has been launched yet");
+  double const us = static_cast<double>(t[1]) / 100.0;  // the reference counter runs at 100 MHz
+  if (tile_us != nullptr) *tile_us = us;
+  if (engine_mhz != nullptr) *engine_mhz = static_cast<double>(t[0]) / us;
+  return DLMI_OK;
+}
 
 int dlmi_ctx_norm_panel_enabled(dlmi_ctx const *ctx) { return ctx != nullptr && ctx->panel_ok ? 1 : 0; }
 

@@ -24,8 +24,14 @@
 // k = {s, s+4} (s = 0..3) of every group of 8 instead of {2s, 2s+1}: a lane
 // then needs 4 CONSECUTIVE k of one row, i.e. one ds_read_b128 per 4 MFMAs for
 // either operand (one whose row index is contiguous in memory is transposed on
-// its way into LDS).  Rows are padded by 4 floats so those 16-byte reads hit
-// distinct banks.
+// its way into LDS).  Rows are padded by 4 floats so that those 16-byte reads
+// (served 8 lanes at a time: 8 rows, 20 words apart) hit 32 distinct banks.  The
+// stores into LDS are not conflict-free with that stride - a 16-byte store of a
+// k-contiguous operand puts 4 lanes on a row, and the two rows of an 8-lane group
+// overlap in 4 banks; the 4-byte stores of a transposed operand pair up row groups
+// two apart - both two-way.  A stride that clears the stores (16 or 48 words)
+// would put the reads four-way; the reads are three quarters of the LDS cycles.
+// Counters: conflict cycles / LDS active = 0.33, 0.8 % of wave cycles wait on LDS.
 //
 // Workgroup ids are remapped so that (a) the ids that land on one XCD (id % 8)
 // cover a compact block of tiles and (b) tiles are walked in groups of 8 rows
@@ -60,6 +66,9 @@ struct GemmArgs {
   // normalization that follows, before it updates them) to snap_out [2][N]
   float const *snap_a, *snap_b;
   float *snap_out;
+  // optional: the workgroup of tile 0 / slice 0 stores {engine clock ticks, 100 MHz reference ticks} it spent from
+  // entry to its last store (measurement aid: the engine clock inside this very launch, no profiler attached)
+  unsigned long long *clock_out;
   int accumulate;      // C += result (only when gridDim.z == 1)
   int a_vec, b_vec;    // operand base and leading dimension allow 16-byte loads (ragged variant)
   unsigned tiles_m, tiles_n;
@@ -220,6 +229,12 @@ __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid,
   static_assert(BK % 8 == 0, "K tile is consumed in groups of 8");
   constexpr int kStage = TA::kFloats + TB::kFloats;  // lds: 2 stages of (A tile, B tile)
 
+  bool const clocked = g.clock_out != nullptr && lid == 0 && zslice == 0;
+  unsigned long long c0 = 0, r0 = 0;
+  if (clocked) {
+    c0 = __builtin_amdgcn_s_memtime();
+    r0 = __builtin_amdgcn_s_memrealtime();
+  }
   // ---- which tile: walked in groups of 8 rows of tiles -----------------------
   unsigned const per_group = kGroupM * g.tiles_n;
   unsigned const first_m = (lid / per_group) * kGroupM;
@@ -435,6 +450,10 @@ __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid,
       }
     }
   }
+  if (clocked && threadIdx.x == 0) {
+    g.clock_out[0] = __builtin_amdgcn_s_memtime() - c0;
+    g.clock_out[1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
 }
 
 template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int WAVES_PER_EU, int RST>
@@ -473,7 +492,7 @@ void k_gemm_f32_group(GemmGroupArgs a) {
   g.A = q.A; g.B = q.B; g.C = q.C; g.bias = nullptr;
   g.M = q.M; g.N = q.N; g.K = q.K;
   g.lda = A_KCONTIG ? q.K : q.M; g.ldb = B_KCONTIG ? q.K : q.N; g.ldc = q.N;
-  g.k_per_split = q.K; g.split_out = nullptr; g.stats_out = nullptr;
+  g.k_per_split = q.K; g.split_out = nullptr; g.stats_out = nullptr; g.clock_out = nullptr;
   g.snap_a = nullptr; g.snap_b = nullptr; g.snap_out = nullptr;
   g.accumulate = a.accumulate; g.a_vec = 1; g.b_vec = 1;
   g.tiles_n = q.tiles_n; g.tiles_m = (q.M + BM - 1) / BM;
@@ -556,6 +575,7 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   g.A = A; g.B = B; g.C = C; g.bias = bias; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldc = N;
   g.accumulate = accumulate; g.split_out = nullptr; g.stats_out = nullptr;
   g.snap_a = g.snap_b = nullptr; g.snap_out = nullptr;
+  g.clock_out = ctx->gemm_clock;
   if (snap_out != nullptr) *snap_out = nullptr;
   g.a_vec = (lda % 4 == 0 && dlmi_aligned16(A)) ? 1 : 0;
   g.b_vec = (ldb % 4 == 0 && dlmi_aligned16(B)) ? 1 : 0;

@@ -67,6 +67,16 @@ namespace dlmi {
 constexpr int kMaxDevices = 64;
 static void *g_static_scratch[kMaxDevices] = {nullptr};
 static std::mutex g_static_scratch_mutex;
+// Every call of the entry point that allocates nothing uses the device's one array, so calls from different
+// streams must not overlap.  The stream of the last such call is remembered per device; a call from another stream
+// (outside a stream capture) first makes its stream wait for an event recorded behind that call.  The event is
+// created with the first context of the device, so the entry point itself creates nothing.
+struct StaticScratchOrder {
+  hipEvent_t event = nullptr;
+  hipStream_t stream = nullptr;
+  bool used = false;
+};
+static StaticScratchOrder g_static_order[kMaxDevices];
 
 // Called by dlmi_ctx_create with the context's device current: looks up, once
 // per device, where that device keeps its copy of the static scratch array.
@@ -83,9 +93,42 @@ int static_scratch_init(dlmi_ctx *ctx) {
     }
     g_static_scratch[ctx->device] = p;
   }
+  if (g_static_order[ctx->device].event == nullptr &&
+      hipEventCreateWithFlags(&g_static_order[ctx->device].event, hipEventDisableTiming) != hipSuccess) {
+    (void)hipGetLastError();
+    g_static_order[ctx->device].event = nullptr;  // calls from several streams then race, as documented
+  }
   ctx->static_scratch = static_cast<char *>(g_static_scratch[ctx->device]);
   ctx->static_scratch_bytes = kStaticScratchBytes;
   return DLMI_OK;
+}
+
+static bool stream_capturing(hipStream_t s) {
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &cs) != hipSuccess) { (void)hipGetLastError(); return true; }
+  return cs != hipStreamCaptureStatusNone;
+}
+// Before a call that uses the device's static scratch array: orders it behind the last one of another stream.
+static int static_scratch_order(dlmi_ctx *ctx) {
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  StaticScratchOrder &o = g_static_order[ctx->device];
+  if (o.event != nullptr && o.used && o.stream != ctx->stream && !stream_capturing(ctx->stream) && !stream_capturing(o.stream)) {
+    DLMI_HIP(ctx, hipEventRecord(o.event, o.stream));
+    DLMI_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.event, 0));
+  }
+  o.stream = ctx->stream;
+  o.used = true;
+  return DLMI_OK;
+}
+// The context lets go of its stream (which its owner may destroy next; its work has completed).
+void static_scratch_release_stream(dlmi_ctx *ctx) {
+  if (ctx->device < 0 || ctx->device >= kMaxDevices) return;
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  StaticScratchOrder &o = g_static_order[ctx->device];
+  if (o.used && o.stream == ctx->stream) {
+    o.used = false;
+    o.stream = nullptr;
+  }
 }
 
 constexpr int kBlock = 256;
@@ -1330,6 +1373,8 @@ int dlmi_fused_norm_act_fwd_noalloc(dlmi_ctx *ctx, dlmi_fused_desc const *desc, 
   FwdTrainCall const c = fused_fwd_call(desc, x, gamma, beta, mask, mean, stdv, mov_mean, mov_std, r, d, y);
   // the device's own copy of the file-scope array, by its device address: no hipMalloc, no hipFree, no
   // memset (every partial sum the finalize kernel reads is written by the statistics kernel first)
+  rc = static_scratch_order(ctx);
+  if (rc != DLMI_OK) return rc;
   ScratchView sv{};
   sv.data = ctx->static_scratch;
   sv.data_bytes = ctx->static_scratch_bytes;

@@ -73,6 +73,7 @@ struct Model::Impl {
   // allocated (zeroed; the step sizes filled with rprop_delta_zero) on first use
   float *d_opt[7] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
   float const *cur_input = nullptr;  // [batch, n_in] of the pass in flight: d_input or a caller's device rows
+  bool weights_set = false;          // an initializer has run or parameters have been uploaded
   size_t n_errors = 0;               // failed calls so far
   size_t n_loss_values = 0;          // outputs whose loss term has been accumulated since reset_loss()
   size_t all_units = 0;              // normalization units of all entries: the slots a normalized model has
@@ -526,7 +527,10 @@ bool Model::resize_normalization_slots(bool const present) {
       !dev_alloc(&m.d_mov_std, nu, err))
     return false;
   if (!hip_ok(hipMemsetAsync(m.d_dparams, 0, (P ? P : 1) * sizeof(float), m.stream), err, "memset")) return false;
-  if (!upload_parameters() || !upload_moving_statistics()) return false;
+  bool const weights_were_set = m.weights_set;  // re-sizing the array is no initialization
+  bool const uploaded = upload_parameters() && upload_moving_statistics();
+  m.weights_set = weights_were_set;
+  if (!uploaded) return false;
   return weight_decay == 0.0f || set_weight_decay(weight_decay);  // the regularization mask has the array's length
 }
 
@@ -879,6 +883,11 @@ size_t Model::Get__LSUV_Trials(size_t const li) const { return li < impl_->lsuv_
 bool Model::Initialization__LSUV(size_t const n_data_set, real const *const *const inputs) {
   if (ptr_array_layers == nullptr || inputs == nullptr || n_data_set == 0) return fail("Initialization__LSUV: model not compiled or no data");
   LSUV_Parameters const &p = impl_->lsuv;
+  // The reference starts with layers_initialize_orthogonal (lsuv.cpp:55, orthogonal.cpp:39-172: Eigen's QR), which
+  // is not built here: the loop scales the weights it finds.  Without any, it would scale zeros without a word.
+  if (!impl_->weights_set)
+    return fail("Initialization__LSUV: the orthogonal pre-initialization is not built and no weights have been set: run "
+                "an initializer or upload parameters first");
   // the bias slots, as the pre-initialization would leave them (orthogonal.cpp:62)
   if (!download_parameters()) return false;
   for (size_t li = 1; li < total_layers; ++li) {
@@ -965,6 +974,7 @@ real Model::warm_restarts_decay(void) {
 
 // ---------------------------------------------------------------- buffer movement
 bool Model::upload_parameters(void) {
+  impl_->weights_set = true;
   return hip_ok(hipMemcpy(impl_->d_params, ptr_array_parameters, total_parameters * sizeof(float), hipMemcpyHostToDevice),
                 impl_->err, "parameter upload");
 }

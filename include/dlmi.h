@@ -97,6 +97,13 @@ int dlmi_ctx_compute_units(dlmi_ctx const *ctx);
  * that a test can make the next launch's count impossible to complete and, with a small DLMI_PANEL_SPIN_LIMIT
  * (polls per wait, read at dlmi_ctx_create), drive the give-up branch while every kernel still exits normally. */
 int dlmi_ctx_norm_panel_enabled(dlmi_ctx const *ctx);
+/* Measurement aid, no counterpart in the reference.  A context created with DLMI_GEMM_CLOCK=1 in the environment
+ * has the workgroup of the first tile of every product launch (dlmi_fc_fwd, dlmi_fc_bwd_dx, dlmi_fc_bwd_dw) read the
+ * engine clock counter and the 100 MHz reference counter at its entry and after its last store.
+ * dlmi_ctx_gemm_clock waits for the stream and returns, for the last product launched, the engine clock in MHz
+ * (ticks / time) and that workgroup's lifetime in microseconds: the clock INSIDE the launch, with no profiler
+ * attached.  DLMI_E_INVALID without the environment variable or before the first product. */
+int dlmi_ctx_gemm_clock(dlmi_ctx *ctx, double *engine_mhz, double *tile_us);
 int dlmi_ctx_norm_panel_poke(dlmi_ctx *ctx, unsigned xcd, unsigned word, unsigned value);
 /* How a product C[M,N] = A[M,K] . B[K,N] would be launched on a device with `compute_units` CUs: tile shape, K
  * slices (1 = none; more = partial products plus a fixed-order sum) and register stages of the K loop.  Host
@@ -318,9 +325,11 @@ int dlmi_fused_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B
  * of the context's growable scratch, so the call reaches no hipMalloc, hipFree
  * or memset.  It has no counterpart in the reference.  H is limited to
  * DLMI_NOALLOC_MAX_UNITS units (B is not limited); beyond it the call returns
- * DLMI_E_UNSUPPORTED.  All calls on one GPU share that GPU's array: calls that
- * overlap in time on one GPU (two streams, two contexts) race; calls on one
- * stream are ordered by it. */
+ * DLMI_E_UNSUPPORTED.  All calls on one GPU share that GPU's array: calls on one
+ * stream are ordered by it, and a call from another stream than the previous
+ * one first waits (on the device) for that one through an event made when the
+ * device's first context was created.  Calls recorded into HIP graphs are not
+ * ordered that way: replays that overlap in time on one GPU race. */
 #define DLMI_NOALLOC_MAX_UNITS 65536
 int dlmi_fused_norm_act_fwd_noalloc(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H,
                                     float const *x, float const *gamma, float const *beta,

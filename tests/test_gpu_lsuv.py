@@ -153,3 +153,17 @@ def test_settings_are_checked(lib):
         assert max(t) <= 3 and np.all(np.isfinite(g.get_parameters()))
     finally:
         g.close()
+
+
+def test_lsuv_without_weights_is_refused(lib):
+    """The reference's Initialization__LSUV starts with an orthogonal initialization of its own; this one scales the
+    weights it finds.  On a model whose weights nobody has set it says so instead of scaling zeros."""
+    g = gpu_model(lib, [12, 16, 4], ["RELU", "LINEAR"], ["NONE"])
+    try:
+        X = np.random.default_rng(2).normal(0, 1, (16, 12)).astype(np.float32)
+        with pytest.raises(RuntimeError, match="no weights have been set"):
+            g.lsuv(X)
+        g.glorot_uniform(3)
+        g.lsuv(X)  # an initializer has run: accepted
+    finally:
+        g.close()

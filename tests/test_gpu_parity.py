@@ -452,3 +452,31 @@ def test_softmax_ce_seed(dl, oracle, B, H):
     assert_close(host(dZ), dZo, TE, "seed gradient")
     st = host(stats)
     assert abs(st[0] - loss) <= 1e-5 * max(1.0, abs(loss)) and st[1] == correct
+
+
+@pytest.mark.parametrize("B,K,H", [(1024, 2048, 2048), (4096, 512, 512)])
+def test_products_against_float64_no_worse_than_the_cpu_path(dl, oracle, B, K, H):
+    """The arbitration of the element-wise ("strict") tolerance behind a product: an output that cancels to far
+    below the typical magnitude carries the absolute rounding error of its K terms, so no two summation orders
+    agree on it to 1e-4 of ITSELF.  What can be asked is that the device is no further from the float64 product
+    than the CPU restatement (one chain over k, like the reference's leaves) on the same elements: the
+    root-mean-square error of the device's Z, dX and dW against float64 is at most twice the CPU's."""
+    rng = np.random.default_rng(B + K)
+    X = rng.standard_normal((B, K)).astype(np.float32)
+    lim = (6.0 / (K + H)) ** 0.5
+    W = rng.uniform(-lim, lim, (H, K)).astype(np.float32)
+    dZ = rng.standard_normal((B, H)).astype(np.float32)
+    rows, units = np.arange(0, B, B // 32)[:32], np.arange(0, H, H // 32)[:32]
+    d = lambda a: a.astype(np.float64)
+    rms = lambda a: float(np.sqrt(np.mean(np.square(a))))
+    Zg, dXg = host(dl.fc_fwd(dev(X), dev(W))), host(dl.fc_bwd_dx(dev(dZ), dev(W)))
+    dWg, _ = dl.fc_bwd_dw(dev(X), dev(dZ))
+    dWg = host(dWg)
+    # the CPU side on the slabs only (single thread: one chain per output, the order of the reference's leaves)
+    Zc = oracle.fc_fwd(X[rows], W, 1)
+    dXc = oracle.fc_bwd_dx(dZ[rows], W, nthreads=1)
+    dWc, _ = oracle.fc_bwd_dw(X, np.ascontiguousarray(dZ[:, units]), with_bias=False, nthreads=1)
+    for name, g, c, exact in (("Z", Zg[rows], Zc, d(X[rows]) @ d(W).T), ("dX", dXg[rows], dXc, d(dZ[rows]) @ d(W)),
+                              ("dW", dWg[units], dWc, d(dZ[:, units]).T @ d(X))):
+        eg, ec = rms(g - exact), rms(c - exact)
+        assert eg <= 2.0 * ec + 1e-7 * rms(exact), (name, eg, ec)

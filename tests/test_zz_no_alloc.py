@@ -117,3 +117,45 @@ def test_noalloc_entry_refuses_more_units_than_its_array_holds(dl, pkg):
     a = dl.fused_fwd(desc, x, v(), v() * 0, v() * 0, v(), noalloc=True)[0]
     b = dl.fused_fwd(desc, x, v(), v() * 0, v() * 0, v(), noalloc=False)[0]
     assert torch.equal(a, b)
+
+
+def test_noalloc_calls_from_two_streams_are_ordered(pkg):
+    """Every call on one GPU uses the same fixed array.  Calls from two contexts on two streams, issued
+    alternately without any host wait, would trample each other's partial sums; the library makes a call from
+    another stream than the previous one wait (on the device) for that one.  Results: those of each input alone."""
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    a, b = pkg.Dlmi(0), pkg.Dlmi(0)
+    try:
+        a.set_stream(s1)
+        b.set_stream(s2)
+        desc = pkg.Dlmi.desc(pkg.ACT["ELU"], renorm=True, momentum=0.9)
+        H = 8192  # multi-launch kernels: statistics, finalize and apply all go through the array
+        rng = np.random.default_rng(4)
+        xs = [dev(rng.standard_normal((300 + 40 * i, H)).astype(np.float32) * (1 + i)) for i in range(6)]
+        one, zero = torch.ones(H, device="cuda"), torch.zeros(H, device="cuda")
+
+        def call(ctx, x):
+            y = torch.empty_like(x)
+            st = {k: torch.empty(H, device="cuda") for k in ("mean", "std", "r", "d")}
+            ctx.fused_fwd(desc, x, one, zero, zero.clone(), one.clone(), out=y, stats=st, noalloc=True)
+            return y, st
+
+        torch.cuda.synchronize()
+        want = []
+        for x in xs:
+            with torch.cuda.stream(s1):
+                want.append(call(a, x))
+            torch.cuda.synchronize()
+        for _ in range(5):
+            got = []
+            for i, x in enumerate(xs):  # alternating streams, nothing waits on the host
+                with torch.cuda.stream(s1 if i % 2 == 0 else s2):
+                    got.append(call(a if i % 2 == 0 else b, x))
+            torch.cuda.synchronize()
+            for (y, st), (yw, sw) in zip(got, want):
+                assert torch.equal(y, yw)
+                assert torch.equal(st["mean"], sw["mean"]) and torch.equal(st["std"], sw["std"])
+    finally:
+        torch.cuda.synchronize()
+        a.close()
+        b.close()
