@@ -7,10 +7,15 @@
 // (reference leaves: v1/learner/fwp_st.cpp:4518-4555, bwp_st.cpp:1009-1045,
 //  update_derivative_fwp_st.cpp:246-281 under /root/reference/lib/deep-learning.)
 //
-// One kernel template covers the three operand layouts.  A 256-thread
-// workgroup (4 wavefronts, 2 x 2) owns a BM x BN tile of C; each wavefront
-// owns (BM/2) x (BN/2) as a grid of 32x32 v_mfma_f32_32x32x2_f32 blocks whose
-// accumulators stay in registers for the whole K loop.  Operand tiles are
+// One kernel template covers the three operand layouts.  A workgroup of 4
+// wavefronts (2 x 2) or 8 (4 along M x 2 along N) owns a BM x BN tile of C; each
+// wavefront owns its share as a grid of 32x32 v_mfma_f32_32x32x2_f32 blocks whose
+// accumulators stay in registers for the whole K loop.  Why 8: two 4-wavefront
+// workgroups that share a CU do not advance alike - the scheduler favours the
+// older wavefronts, so one workgroup finishes early and the other runs its last
+// sixth alone, on a matrix pipe it cannot keep fed (measured on 1024 x 2048 x 2048
+// with 64 x 64 tiles: half the workgroups end after 56 us, the other half after
+// 66 us).  Eight wavefronts behind one barrier stay together and share the B tile.  Operand tiles are
 // staged through LDS (two stages, one barrier per K tile) behind one register
 // stage (the global loads run two tiles ahead of the MFMAs) or, for the small
 // tiles on a long reduction, two (three tiles ahead); the LDS writes, the
@@ -48,7 +53,7 @@ namespace dlmi {
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int kGemmThreads = 256;
+constexpr int kGemmThreads = 256;  // of the 4-wavefront workgroups; the 8-wavefront ones have twice as many
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8;
 
@@ -78,13 +83,15 @@ struct GemmArgs {
 // fragments of both operands are 16-byte LDS reads whatever the layout in
 // memory.  An operand whose row (m or n) index is contiguous in memory is
 // transposed on its way into LDS.
-template <int ROWS, int BK, bool KCONTIG>
+template <int ROWS, int BK, bool KCONTIG, int THREADS = kGemmThreads>
 struct TileShape {
   static constexpr int kStride = BK + 4;
   static constexpr int kFloats = ROWS * (BK + 4);
   static constexpr int kVec4 = ROWS * BK / 4;             // 16-byte pieces per tile
-  static constexpr int kPerThread = kVec4 / kGemmThreads;  // pieces per thread
-  static_assert(kVec4 % kGemmThreads == 0, "tile must divide evenly over the workgroup");
+  // pieces per thread; a tile of fewer pieces than threads is moved by the first kVec4 threads (whole wavefronts)
+  static constexpr int kPerThread = kVec4 >= THREADS ? kVec4 / THREADS : 1;
+  static constexpr bool kSomeIdle = kVec4 < THREADS;
+  static_assert(kVec4 % THREADS == 0 || (kVec4 < THREADS && kVec4 % 64 == 0), "tile must divide evenly over the workgroup");
   static_assert(ROWS % 32 == 0 && BK % 8 == 0, "tile shape");
   // the prefetch registers of one thread as ONE vector value (a first-class
   // SSA value: it can neither be spilled to scratch nor be promoted to LDS the
@@ -120,17 +127,24 @@ enum : int { kGuarded = 0, kFast = 1, kClamped = 2 };
 
 // Global -> registers for one operand tile.  `row0` is the tile's first row
 // (m or n), `k0` its first k.
-template <int ROWS, int BK, bool KCONTIG, int MODE>
-__device__ __forceinline__ typename TileShape<ROWS, BK, KCONTIG>::Regs tile_load(float const *__restrict__ P,
-                                                                               size_t ld, size_t row0, size_t k0,
-                                                                               size_t rows_total, size_t k_end,
-                                                                               bool vec_ok) {
-  using T = TileShape<ROWS, BK, KCONTIG>;
+template <int ROWS, int BK, bool KCONTIG, int MODE, int THREADS>
+__device__ __forceinline__ typename TileShape<ROWS, BK, KCONTIG, THREADS>::Regs tile_load(float const *__restrict__ P,
+                                                                                        size_t ld, size_t row0, size_t k0,
+                                                                                        size_t rows_total, size_t k_end,
+                                                                                        bool vec_ok) {
+  using T = TileShape<ROWS, BK, KCONTIG, THREADS>;
   typename T::Regs regs;
+  if constexpr (T::kSomeIdle) {
+    if (static_cast<int>(threadIdx.x) >= T::kVec4) {
+#pragma unroll
+      for (int e = 0; e < 4 * T::kPerThread; ++e) regs[e] = 0.0f;
+      return regs;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < T::kPerThread; ++i) {
     int tr, tk;
-    T::piece(threadIdx.x + i * kGemmThreads, tr, tk);
+    T::piece(threadIdx.x + i * THREADS, tr, tk);
     size_t row = row0 + tr;
     size_t const k = k0 + tk;
     if constexpr (MODE == kClamped) {
@@ -165,14 +179,17 @@ __device__ __forceinline__ typename TileShape<ROWS, BK, KCONTIG>::Regs tile_load
   return regs;
 }
 
-template <int ROWS, int BK, bool KCONTIG>
+template <int ROWS, int BK, bool KCONTIG, int THREADS>
 __device__ __forceinline__ void tile_store(float *__restrict__ lds,
-                                           typename TileShape<ROWS, BK, KCONTIG>::Regs const &regs) {
-  using T = TileShape<ROWS, BK, KCONTIG>;
+                                           typename TileShape<ROWS, BK, KCONTIG, THREADS>::Regs const &regs) {
+  using T = TileShape<ROWS, BK, KCONTIG, THREADS>;
+  if constexpr (T::kSomeIdle) {
+    if (static_cast<int>(threadIdx.x) >= T::kVec4) return;
+  }
 #pragma unroll
   for (int i = 0; i < T::kPerThread; ++i) {
     int tr, tk;
-    T::piece(threadIdx.x + i * kGemmThreads, tr, tk);
+    T::piece(threadIdx.x + i * THREADS, tr, tk);
     if constexpr (KCONTIG) {
       v4f t;
 #pragma unroll
@@ -217,14 +234,15 @@ __device__ __forceinline__ unsigned xcd_order(unsigned id, unsigned ntiles) {
 }
 
 // One tile of one product: tile number `lid` (in the grouped order below) of K slice `zslice` of `nslices`.
-template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int RST>
+template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int RST, int WVM = 2>
 __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid, unsigned const zslice, unsigned const nslices,
                                           float *__restrict__ lds) {
   constexpr bool FAST = MODE == kFast;          // no edge anywhere: unguarded stores
   constexpr bool FAST_LOOP = MODE != kGuarded;  // the scheduled K loop
-  using TA = TileShape<BM, BK, A_KCONTIG>;
-  using TB = TileShape<BN, BK, B_KCONTIG>;
-  constexpr int WM = BM / 2, WN = BN / 2;  // wavefront tile
+  constexpr int THREADS = 128 * WVM;            // WVM wavefronts along M x 2 along N
+  using TA = TileShape<BM, BK, A_KCONTIG, THREADS>;
+  using TB = TileShape<BN, BK, B_KCONTIG, THREADS>;
+  constexpr int WM = BM / WVM, WN = BN / 2;  // wavefront tile
   constexpr int TM = WM / 32, TN = WN / 32;
   static_assert(BK % 8 == 0, "K tile is consumed in groups of 8");
   constexpr int kStage = TA::kFloats + TB::kFloats;  // lds: 2 stages of (A tile, B tile)
@@ -300,15 +318,15 @@ __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid,
     // during tile kt and moves to LDS during tile kt+2); the stages alternate with the tile's parity.
     static_assert(RST == 1 || RST == 2, "one or two register stages");
     auto load_a = [&](int t) {
-      return tile_load<BM, BK, A_KCONTIG, MODE>(g.A, g.lda, m0, k_begin + static_cast<size_t>(t) * BK, g.M, k_end, g.a_vec != 0);
+      return tile_load<BM, BK, A_KCONTIG, MODE, THREADS>(g.A, g.lda, m0, k_begin + static_cast<size_t>(t) * BK, g.M, k_end, g.a_vec != 0);
     };
     auto load_b = [&](int t) {
-      return tile_load<BN, BK, B_KCONTIG, MODE>(g.B, g.ldb, n0, k_begin + static_cast<size_t>(t) * BK, g.N, k_end, g.b_vec != 0);
+      return tile_load<BN, BK, B_KCONTIG, MODE, THREADS>(g.B, g.ldb, n0, k_begin + static_cast<size_t>(t) * BK, g.N, k_end, g.b_vec != 0);
     };
     typename TA::Regs ra = load_a(0), ra2 = ra;
     typename TB::Regs rb = load_b(0), rb2 = rb;
-    tile_store<BM, BK, A_KCONTIG>(lds, ra);
-    tile_store<BN, BK, B_KCONTIG>(lds + TA::kFloats, rb);
+    tile_store<BM, BK, A_KCONTIG, THREADS>(lds, ra);
+    tile_store<BN, BK, B_KCONTIG, THREADS>(lds + TA::kFloats, rb);
     // one register stage: ra/rb hold tile kt+1 at the start of tile kt.  Two: tile kt+1 is in ra/rb for even
     // kt and in ra2/rb2 for odd kt, tile kt+2 in the other pair.
     if (ktiles > 1) {
@@ -335,8 +353,8 @@ __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid,
       frags(sa, sa + TA::kFloats, 8, f1a, f1b);
       steps(f0a, f0b, 0, 4);
       if constexpr (STORE) {
-        tile_store<BM, BK, A_KCONTIG>(na, xa);
-        tile_store<BN, BK, B_KCONTIG>(na + TA::kFloats, xb);
+        tile_store<BM, BK, A_KCONTIG, THREADS>(na, xa);
+        tile_store<BN, BK, B_KCONTIG, THREADS>(na + TA::kFloats, xb);
       }
       if constexpr (LOAD) {
         xa = load_a(kt + 1 + RST);
@@ -438,11 +456,18 @@ __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid,
       }
     }
     __syncthreads();
-    for (int c = threadIdx.x; c < BN; c += kGemmThreads) {
+    for (int c = threadIdx.x; c < BN; c += THREADS) {
       size_t const col = n0 + c;
       if (FAST || col < g.N) {
-        g.stats_out[(0 * static_cast<size_t>(g.tiles_m) + tile_m) * g.N + col] = sl[(0 * BN + c) * 2 + 0] + sl[(1 * BN + c) * 2 + 0];
-        g.stats_out[(1 * static_cast<size_t>(g.tiles_m) + tile_m) * g.N + col] = sl[(0 * BN + c) * 2 + 1] + sl[(1 * BN + c) * 2 + 1];
+        float t1 = sl[(0 * BN + c) * 2 + 0] + sl[(1 * BN + c) * 2 + 0];
+        float t2 = sl[(0 * BN + c) * 2 + 1] + sl[(1 * BN + c) * 2 + 1];
+#pragma unroll
+        for (int w = 2; w < WVM; ++w) {  // the wavefronts stacked along M, top to bottom
+          t1 += sl[(w * BN + c) * 2 + 0];
+          t2 += sl[(w * BN + c) * 2 + 1];
+        }
+        g.stats_out[(0 * static_cast<size_t>(g.tiles_m) + tile_m) * g.N + col] = t1;
+        g.stats_out[(1 * static_cast<size_t>(g.tiles_m) + tile_m) * g.N + col] = t2;
         if (g.snap_out != nullptr && tile_m == 0) {
           g.snap_out[col] = g.snap_a[col];
           g.snap_out[g.N + col] = g.snap_b[col];
@@ -456,11 +481,11 @@ __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid,
   }
 }
 
-template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int WAVES_PER_EU, int RST>
-__global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
+template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int WAVES_PER_EU, int RST, int WVM = 2>
+__global__ __launch_bounds__(128 * WVM) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
 void k_gemm_f32(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  gemm_tile<BM, BN, BK, A_KCONTIG, B_KCONTIG, MODE, RST>(g, xcd_order(blockIdx.x, g.tiles_m * g.tiles_n), blockIdx.z, gridDim.z, lds);
+  gemm_tile<BM, BN, BK, A_KCONTIG, B_KCONTIG, MODE, RST, WVM>(g, xcd_order(blockIdx.x, g.tiles_m * g.tiles_n), blockIdx.z, gridDim.z, lds);
 }
 
 // Several independent products of one kernel variant in ONE launch (the weight gradients of a network's layers:
@@ -524,18 +549,18 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(float const *__restrict__
 }
 
 // ---------------------------------------------------------------- host side
-template <int BM, int BN, int BK, bool AK, bool BKC, int WPE, bool HAS_CLAMPED, int RST>
+template <int BM, int BN, int BK, bool AK, bool BKC, int WPE, bool HAS_CLAMPED, int RST, int WVM = 2>
 static int launch_gemm(dlmi_ctx *ctx, GemmArgs g, unsigned splits, int mode) {
-  using TA = TileShape<BM, BK, AK>;
-  using TB = TileShape<BN, BK, BKC>;
+  using TA = TileShape<BM, BK, AK, 128 * WVM>;
+  using TB = TileShape<BN, BK, BKC, 128 * WVM>;
   constexpr size_t lds_bytes = 2 * (TA::kFloats + TB::kFloats) * sizeof(float);
   g.tiles_m = static_cast<unsigned>(dlmi_ceil_div(g.M, BM));
   g.tiles_n = static_cast<unsigned>(dlmi_ceil_div(g.N, BN));
   dim3 const grid(g.tiles_m * g.tiles_n, 1, splits);
-  auto const kfast = k_gemm_f32<BM, BN, BK, AK, BKC, kFast, WPE, RST>;
-  auto const kslow = k_gemm_f32<BM, BN, BK, AK, BKC, kGuarded, WPE, 1>;
+  auto const kfast = k_gemm_f32<BM, BN, BK, AK, BKC, kFast, WPE, RST, WVM>;
+  auto const kslow = k_gemm_f32<BM, BN, BK, AK, BKC, kGuarded, WPE, 1, WVM>;
   // the clamped variant exists for the small tiles, which are the ones ragged layers run
-  auto const kclamp = k_gemm_f32<BM, BN, BK, AK, BKC, HAS_CLAMPED ? kClamped : kGuarded, WPE, HAS_CLAMPED ? RST : 1>;
+  auto const kclamp = k_gemm_f32<BM, BN, BK, AK, BKC, HAS_CLAMPED ? kClamped : kGuarded, WPE, HAS_CLAMPED ? RST : 1, WVM>;
   if (!HAS_CLAMPED && mode == kClamped) mode = kGuarded;
   // more than 64 KB of LDS has to be asked for once per kernel and device
   static bool attr_set_on[64] = {false};
@@ -550,11 +575,11 @@ static int launch_gemm(dlmi_ctx *ctx, GemmArgs g, unsigned splits, int mode) {
     attr_set = true;
   }
   if (mode == kFast)
-    hipLaunchKernelGGL(kfast, grid, dim3(kGemmThreads), lds_bytes, ctx->stream, g);
+    hipLaunchKernelGGL(kfast, grid, dim3(128 * WVM), lds_bytes, ctx->stream, g);
   else if (mode == kClamped)
-    hipLaunchKernelGGL(kclamp, grid, dim3(kGemmThreads), lds_bytes, ctx->stream, g);
+    hipLaunchKernelGGL(kclamp, grid, dim3(128 * WVM), lds_bytes, ctx->stream, g);
   else
-    hipLaunchKernelGGL(kslow, grid, dim3(kGemmThreads), lds_bytes, ctx->stream, g);
+    hipLaunchKernelGGL(kslow, grid, dim3(128 * WVM), lds_bytes, ctx->stream, g);
   DLMI_LAUNCH_CHECK(ctx, "k_gemm_f32");
   return DLMI_OK;
 }
@@ -628,6 +653,13 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
         rc = launch_gemm<64, 64, 16, AK, BKC, 4, true, 2>(ctx, g, splits, mode);
       else
         rc = launch_gemm<64, 64, 16, AK, BKC, 4, true, 1>(ctx, g, splits, mode);
+      break;
+    // 8 wavefronts (4 along M x 2 along N) behind one barrier, one workgroup per CU, two wavefronts per SIMD
+    case 4:
+      if (gemm_register_stages(bm, bn, kt_per_split) == 2)
+        rc = launch_gemm<128, 128, 16, AK, BKC, 2, false, 2, 4>(ctx, g, splits, mode);
+      else
+        rc = launch_gemm<128, 128, 16, AK, BKC, 2, false, 1, 4>(ctx, g, splits, mode);
       break;
     default:
       if (gemm_register_stages(bm, bn, kt_per_split) == 2)
@@ -707,7 +739,8 @@ static int group_variant(dlmi_ctx const *ctx, GroupItem const &it) {
   if (!vec || it.K % plan.bk != 0 || it.M % plan.bm != 0 || it.N % plan.bn != 0) return -1;
   if (it.M > 0xffffffffull || it.N > 0xffffffffull || it.K > 0xffffffffull) return -1;
   int const rst = plan.choice == 2 ? 1 : gemm_register_stages(plan.bm, plan.bn, dlmi_ceil_div(it.K, plan.bk));
-  return plan.choice * 4 + rst;
+  // (the 8-wavefront 128 x 128 variant is for launches of one workgroup per CU; a group has many per CU)
+  return (plan.choice == 4 ? 0 : plan.choice) * 4 + rst;
 }
 template <bool AK, bool BKC>
 static int launch_group_variant(dlmi_ctx *ctx, int variant, GroupItem const *items, size_t n, int accumulate) {

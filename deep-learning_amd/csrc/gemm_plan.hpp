@@ -12,7 +12,8 @@ namespace dlmi {
 
 // Tile shape and K split of a product, from its shape alone.
 struct GemmPlan {
-  int choice, bm, bn, bk;  // choice: 0 128x128, 1 256x128, 2 256x256, 3 64x64
+  int choice, bm, bn, bk;  // choice: 0 128x128, 1 256x128, 2 256x256, 3 64x64 (4 wavefronts); 4 128x128 (8 wavefronts)
+  int waves;               // wavefronts per workgroup: 4 or 8
   unsigned splits;         // K slices (1: none)
   size_t scratch_bytes;    // partial products of the slices
 };

@@ -20,7 +20,8 @@ static int split_choice() {
   return c;
 }
 
-// Tuning aid: DLMI_GEMM_TILE=<index> forces a tile shape (0: 128x128, 1: 256x128, 2: 256x256, 3: 64x64).
+// Tuning aid: DLMI_GEMM_TILE=<index> forces a tile shape (0: 128x128, 1: 256x128, 2: 256x256, 3: 64x64 with 4
+// wavefronts; 4: 128x128 with 8 wavefronts).
 static int tile_choice() {
   static int const c = [] {
     char const *e = std::getenv("DLMI_GEMM_TILE");
@@ -30,7 +31,7 @@ static int tile_choice() {
 }
 
 GemmPlan plan_gemm(int const num_cu, size_t M, size_t N, size_t K) {
-  static TileCfg const cfgs[] = {{128, 128, 16}, {256, 128, 16}, {256, 256, 16}, {64, 64, 16}};
+  static TileCfg const cfgs[] = {{128, 128, 16}, {256, 128, 16}, {256, 256, 16}, {64, 64, 16}, {128, 128, 16}};
   int choice = tile_choice();
   if (choice < 0 || choice >= static_cast<int>(sizeof(cfgs) / sizeof(cfgs[0]))) {
     // default: the shape with the smallest estimated time.  Main loop: rounds of workgroups over the CUs x
@@ -63,8 +64,20 @@ GemmPlan plan_gemm(int const num_cu, size_t M, size_t N, size_t K) {
   size_t const tiles_128 = dlmi_ceil_div(M, 128) * dlmi_ceil_div(N, 128);
   bool const long_k = tile_choice() < 0 && split_choice() <= 0 && K >= 8192 && tiles_128 * 8 <= static_cast<size_t>(num_cu);
   if (long_k) choice = 0;
+  // 128 x 128 tiles that come to at most one workgroup per CU: four wavefronts would leave every SIMD with one,
+  // which cannot hide its own LDS and memory latencies.  The same tile as 8 wavefronts (4 x 2, each 32 x 64) puts
+  // two on every SIMD (2048 x 2048 x 1024: 68.6 -> 65.9 us).  More than one workgroup per CU is better served by
+  // independent 4-wavefront workgroups, which fill each other's barrier waits (measured: 128 x 64 and 256 x 128
+  // tiles of 8 wavefronts lose 3-6 % against two workgroups of half the tile).  DLMI_GEMM_WAVES8=0 switches it off.
+  static bool const waves8 = [] { char const *e = std::getenv("DLMI_GEMM_WAVES8"); return e == nullptr || std::atoi(e) != 0; }();
+  if (choice == 0 && waves8 && tile_choice() < 0) {
+    size_t const tiles0 = dlmi_ceil_div(M, 128) * dlmi_ceil_div(N, 128);
+    size_t const slices = long_k ? static_cast<size_t>(num_cu) / tiles_128 : 1;
+    if (tiles0 * (slices > 0 ? slices : 1) <= static_cast<size_t>(num_cu)) choice = 4;
+  }
   GemmPlan p;
   p.choice = choice; p.bm = cfgs[choice].bm; p.bn = cfgs[choice].bn; p.bk = cfgs[choice].bk;
+  p.waves = choice >= 4 ? 8 : 4;
   p.splits = 1;
   p.scratch_bytes = 0;
   if (long_k) {
