@@ -61,6 +61,9 @@ struct dlmi_ctx {
   int panel_spin_limit = 1 << 20;
   int panel_ok = 0;
   int panel_in_graph = 0;
+  // one word in device memory, 0 between launches: the ticket by which the blocks of a seed-gradient kernel find
+  // the one that finishes last (block_pairs.hpp)
+  unsigned *pair_ticket = nullptr;
   // measurement aid (DLMI_GEMM_CLOCK=1 when the context is created): two 64-bit words in which the first tile of
   // every product launch leaves the engine clock ticks and the 100 MHz reference ticks it spent
   unsigned long long *gemm_clock = nullptr;
@@ -156,8 +159,6 @@ int fused_bwd_from_slices(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, 
                           float const *gamma, float const *beta, uint8_t const *mask, float const *mean,
                           float const *stdv, float const *r, float const *d, float const *slices, unsigned nslices,
                           float *dgamma, float *dbeta, float *dX);
-// acc[0] += sum_b pairs[2b], acc[1] += sum_b pairs[2b+1] over nblocks per-block pairs, in a fixed order.
-int sum_block_pairs(dlmi_ctx *ctx, double const *pairs, unsigned nblocks, double *acc);
 }  // namespace dlmi
 
 inline bool dlmi_aligned16(void const *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -89,12 +89,25 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
       (void)hipGetLastError();
     }
   }
-  int rc = dlmi_scratch_reserve(ctx, size_t(16) << 20);
+  int rc = DLMI_OK;
+  {
+    void *p = nullptr;
+    if (hipMalloc(&p, 256) == hipSuccess && hipMemset(p, 0, 256) == hipSuccess) {
+      ctx->pair_ticket = static_cast<unsigned *>(p);
+    } else {
+      (void)hipGetLastError();
+      if (p != nullptr) (void)hipFree(p);
+      rc = dlmi_fail(ctx, DLMI_E_HIP, "dlmi_ctx_create: no device memory for the ticket word");
+    }
+  }
+  if (rc == DLMI_OK) rc = dlmi_scratch_reserve(ctx, size_t(16) << 20);
   if (rc == DLMI_OK) rc = dlmi::static_scratch_init(ctx);
   if (rc == DLMI_OK) rc = dlmi::panel_init(ctx);
   if (rc != DLMI_OK) {
     fprintf(stderr, "dlmi: %s\n", ctx->err);
     if (ctx->scratch != nullptr) (void)hipFree(ctx->scratch);
+    if (ctx->pair_ticket != nullptr) (void)hipFree(ctx->pair_ticket);
+    if (ctx->gemm_clock != nullptr) (void)hipFree(ctx->gemm_clock);
     dlmi::panel_destroy(ctx);
     delete ctx;
     return rc;
@@ -112,6 +125,7 @@ int dlmi_ctx_destroy(dlmi_ctx *ctx) {
   for (int i = 0; i < ctx->n_retired; ++i) (void)hipFree(ctx->retired[i]);
   dlmi::panel_destroy(ctx);
   if (ctx->gemm_clock != nullptr) (void)hipFree(ctx->gemm_clock);
+  if (ctx->pair_ticket != nullptr) (void)hipFree(ctx->pair_ticket);
   delete ctx;
   return DLMI_OK;
 }

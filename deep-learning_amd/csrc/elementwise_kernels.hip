@@ -8,6 +8,7 @@
 #include <initializer_list>
 
 #include "activations.hpp"
+#include "block_pairs.hpp"
 #include "dlmi_common.hpp"
 
 namespace dlmi {
@@ -214,11 +215,12 @@ __global__ __launch_bounds__(kEwBlock) void k_softmax(float const *__restrict__ 
 
 // ---- softmax + cross-entropy seed gradient (compute_error_st.cpp:26-131,
 // compute_loss.cpp:88-95, 101-138).  One wavefront per row; the double
-// accumulators are combined with one atomic per block (they are reported
-// metrics, not part of the gradient).
+// accumulators go out as one pair per block, added in a fixed order by the
+// block that finishes last (block_pairs.hpp).
 __global__ __launch_bounds__(kEwBlock) void k_softmax_ce_seed(float const *__restrict__ q, float const *__restrict__ y,
                                                                float *__restrict__ dZ, size_t B, size_t H,
-                                                               double *__restrict__ stats) {
+                                                               double *__restrict__ pairs, double *__restrict__ acc,
+                                                               unsigned *__restrict__ ticket) {
   constexpr float kEps = 0.0000001f;  // data/dtypes.hpp:113
   int const lane = threadIdx.x & 63;
   size_t const row = static_cast<size_t>(blockIdx.x) * (kEwBlock / 64) + threadIdx.x / 64;
@@ -267,41 +269,17 @@ __global__ __launch_bounds__(kEwBlock) void k_softmax_ce_seed(float const *__res
       correct = (target_k == best_k) ? 1.0 : 0.0;
     }
   }
-  if (stats != nullptr) {
+  if (acc != nullptr) {
     __shared__ double sh[2][kEwBlock / 64];
     if (lane == 0) {
       sh[0][threadIdx.x / 64] = loss;
       sh[1][threadIdx.x / 64] = correct;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-      double l = 0.0, c = 0.0;
+    double l = 0.0, c = 0.0;
+    if (threadIdx.x == 0)
       for (int w = 0; w < kEwBlock / 64; ++w) { l += sh[0][w]; c += sh[1][w]; }
-      // one pair per block, added in block order by sum_block_pairs
-      stats[2 * blockIdx.x] = l;
-      stats[2 * blockIdx.x + 1] = c;
-    }
-  }
-}
-
-// acc[0] += sum of pairs[2b], acc[1] += sum of pairs[2b+1] over the blocks b of a seed kernel, in a fixed
-// order: thread t adds blocks t, t+256, ..., then the 256 lane totals are added in lane order.
-__global__ __launch_bounds__(kEwBlock) void k_sum_block_pairs(double const *__restrict__ pairs, unsigned nblocks,
-                                                               double *__restrict__ acc) {
-  __shared__ double sh[2][kEwBlock];
-  double l = 0.0, c = 0.0;
-  for (unsigned b = threadIdx.x; b < nblocks; b += kEwBlock) {
-    l += pairs[2 * b];
-    c += pairs[2 * b + 1];
-  }
-  sh[0][threadIdx.x] = l;
-  sh[1][threadIdx.x] = c;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    double tl = 0.0, tc = 0.0;
-    for (int i = 0; i < kEwBlock; ++i) { tl += sh[0][i]; tc += sh[1][i]; }
-    acc[0] += tl;
-    acc[1] += tc;
+    finish_block_pairs(l, c, pairs, acc, ticket);
   }
 }
 
@@ -361,12 +339,6 @@ __global__ __launch_bounds__(kEwBlock) void k_variance_from_pairs(double const *
 __global__ __launch_bounds__(kEwBlock) void k_scale(float *__restrict__ p, size_t n, float factor) {
   size_t const stride = static_cast<size_t>(gridDim.x) * kEwBlock;
   for (size_t e = static_cast<size_t>(blockIdx.x) * kEwBlock + threadIdx.x; e < n; e += stride) p[e] *= factor;
-}
-
-int sum_block_pairs(dlmi_ctx *ctx, double const *pairs, unsigned nblocks, double *acc) {
-  hipLaunchKernelGGL(k_sum_block_pairs, dim3(1), dim3(kEwBlock), 0, ctx->stream, pairs, nblocks, acc);
-  DLMI_LAUNCH_CHECK(ctx, "k_sum_block_pairs");
-  return DLMI_OK;
 }
 
 }  // namespace dlmi
@@ -607,9 +579,10 @@ int dlmi_softmax_ce_seed(dlmi_ctx *ctx, size_t B, size_t H, float const *q, floa
     if (rc != DLMI_OK) return rc;
     pairs = reinterpret_cast<double *>(dlmi_scratch_data(ctx));
   }
-  hipLaunchKernelGGL(k_softmax_ce_seed, dim3(nblocks), dim3(kEwBlock), 0, ctx->stream, q, y, dZ, B, H, pairs);
+  hipLaunchKernelGGL(k_softmax_ce_seed, dim3(nblocks), dim3(kEwBlock), 0, ctx->stream, q, y, dZ, B, H, pairs, stats,
+                     ctx->pair_ticket);
   DLMI_LAUNCH_CHECK(ctx, "k_softmax_ce_seed");
-  return stats != nullptr ? sum_block_pairs(ctx, pairs, nblocks, stats) : DLMI_OK;
+  return DLMI_OK;
 }
 
 }  // extern "C"

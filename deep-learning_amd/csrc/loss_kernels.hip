@@ -10,9 +10,11 @@
 //   dZ           f'(x, q) * loss_fn_derivative(q, y) compute_error_st.cpp:118-123,
 //                                                   compute_loss.cpp:101-138
 // One wavefront per row (the cross-entropy accuracy needs the row's arg-max);
-// the reported sums are accumulated in double, one atomic per block.  A tiny
+// the reported sums are accumulated in double: one pair per block, added in a
+// fixed order by the block that finishes last (block_pairs.hpp).  A tiny
 // kernel next to the GEMMs: [batch, outputs] elements, 16 B each.
 #include "activations.hpp"
+#include "block_pairs.hpp"
 #include "dlmi_common.hpp"
 
 namespace dlmi {
@@ -26,7 +28,8 @@ template <int ACT>
 __global__ __launch_bounds__(kLossBlock) void k_loss_seed(int loss, int accu, float accu_threshold,
                                                           float const *__restrict__ z, float const *__restrict__ q,
                                                           float const *__restrict__ y, float *__restrict__ dZ, size_t B,
-                                                          size_t H, double *__restrict__ stats) {
+                                                          size_t H, double *__restrict__ pairs, double *__restrict__ acc,
+                                                          unsigned *__restrict__ ticket) {
   int const lane = threadIdx.x & 63;
   size_t const row = static_cast<size_t>(blockIdx.x) * (kLossBlock / 64) + threadIdx.x / 64;
   double lsum = 0.0, asum = 0.0;
@@ -78,21 +81,18 @@ __global__ __launch_bounds__(kLossBlock) void k_loss_seed(int loss, int accu, fl
     }
     if (accu == DLMI_ACCU_CROSS_ENTROPY) asum = (target_k == best_k) ? 1.0 : 0.0;
   }
-  if (stats != nullptr) {
+  if (acc != nullptr) {
     __shared__ double sh[2][kLossBlock / 64];
     if (lane == 0) {
       sh[0][threadIdx.x / 64] = lsum;
       sh[1][threadIdx.x / 64] = asum;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-      double l = 0.0, c = 0.0;
+    double l = 0.0, c = 0.0;
+    if (threadIdx.x == 0)
       for (int w = 0; w < kLossBlock / 64; ++w) { l += sh[0][w]; c += sh[1][w]; }
-      // one pair per block; sum_block_pairs adds them in block order (no atomics: the sums, which iRPROP+
-      // branches on, are the same from run to run)
-      stats[2 * blockIdx.x] = l;
-      stats[2 * blockIdx.x + 1] = c;
-    }
+    // no floating-point atomics: the sums, which iRPROP+ branches on, are the same from run to run
+    finish_block_pairs(l, c, pairs, acc, ticket);
   }
 }
 
@@ -126,9 +126,10 @@ int dlmi_loss_seed(dlmi_ctx *ctx, dlmi_loss loss, dlmi_accuracy accu, float accu
     pairs = reinterpret_cast<double *>(dlmi_scratch_data(ctx));
   }
   DLMI_DISPATCH_ACT(act, hipLaunchKernelGGL((k_loss_seed<ACT>), grid, block, 0, ctx->stream, static_cast<int>(loss),
-                                            static_cast<int>(accu), accu_threshold, zz, q, y, dZ, B, H, pairs));
+                                            static_cast<int>(accu), accu_threshold, zz, q, y, dZ, B, H, pairs, stats,
+                                            ctx->pair_ticket));
   DLMI_LAUNCH_CHECK(ctx, "k_loss_seed");
-  return stats != nullptr ? sum_block_pairs(ctx, pairs, grid.x, stats) : DLMI_OK;
+  return DLMI_OK;
 }
 
 }  // extern "C"

@@ -89,13 +89,16 @@ class Driver {
   bool keep_dataset_on_device = true;
   // true: once a pass has run kernel by kernel (so every buffer exists), train_st and evalt_st
   // record the launches of each mini-batch (forward, seed or loss, backward, weight gradients) into
-  // a HIP graph per mini-batch and replay those in later passes: a small network's epoch is bound by launch
-  // latency, not by its kernels.  The graphs are dropped and recorded again whenever
+  // HIP graphs of batches_per_graph consecutive mini-batches each and replay those in later passes: a small
+  // network's epoch is bound by launch latency, not by its kernels.  The graphs are dropped and recorded again whenever
   // Model::launch_signature() or the data set changes.  Needs the data set resident in HBM.
   // DLMI_RECORD_BATCHES=0 in the environment makes false the default.
   bool record_batches = true;
-  size_t recorded_batches(void) const { return train_rec_.graphs.size(); }        // of train_st
-  size_t recorded_evalt_batches(void) const { return evalt_rec_.graphs.size(); }  // of evalt_st
+  // DLMI_BATCHES_PER_GRAPH in the environment sets another default.
+  size_t batches_per_graph = 64;
+  // mini-batches that replay from a graph
+  size_t recorded_batches(void) const { return train_rec_.n_batches; }        // of train_st
+  size_t recorded_evalt_batches(void) const { return evalt_rec_.n_batches; }  // of evalt_st
 
   Dataset &dataset;
   v1::ENV::TYPE env_type;
@@ -104,7 +107,8 @@ class Driver {
  private:
   bool make_resident(void);
   struct Recorded {
-    std::vector<void *> graphs;  // hipGraphExec_t per mini-batch, empty until recorded
+    std::vector<void *> graphs;  // hipGraphExec_t per batches_per_graph mini-batches, empty until recorded
+    size_t n_batches = 0;        // mini-batches those graphs hold
     uint64_t signature = 0;      // what the graphs were recorded for
     bool warmed_up = false;      // a plain pass has run for that signature
   };

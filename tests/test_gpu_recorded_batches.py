@@ -73,6 +73,22 @@ def test_replays_match_plain_launches_epoch_by_epoch(lib):
         b.close()
 
 
+@pytest.mark.parametrize("per_graph", [1, 3, 4])
+def test_several_minibatches_per_graph(lib, per_graph, monkeypatch):
+    """The driver puts up to batches_per_graph consecutive mini-batches into one graph (read from the
+    environment when the driver is made): one each, a count that leaves a shorter last graph (4 = 3 + 1), and
+    all of them in one graph give the plain launches' results bit for bit."""
+    monkeypatch.setenv("DLMI_BATCHES_PER_GRAPH", str(per_graph))
+    widths = [20, 32, 24, 5]
+    X, Y = data(50, 20, 5)
+    a, b = build(lib, widths), build(lib, widths)
+    try:
+        run_pair(a, b, X, Y, 5, [0, 4, 4, 4, 4])
+    finally:
+        a.close()
+        b.close()
+
+
 def test_regression_output_layer_is_recorded_too(lib):
     from oracle.binding import ACCU, LOSS
     widths = [12, 18, 4]
