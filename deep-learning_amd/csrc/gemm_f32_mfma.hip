@@ -485,7 +485,21 @@ template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int 
 __global__ __launch_bounds__(128 * WVM) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
 void k_gemm_f32(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  gemm_tile<BM, BN, BK, A_KCONTIG, B_KCONTIG, MODE, RST, WVM>(g, xcd_order(blockIdx.x, g.tiles_m * g.tiles_n), blockIdx.z, gridDim.z, lds);
+  unsigned const ntiles = g.tiles_m * g.tiles_n;
+  unsigned lid = xcd_order(blockIdx.x, ntiles), zslice = blockIdx.z;
+  if (gridDim.z % kXcds == 0 && ntiles % kXcds != 0) {
+    // A split product of few tiles (dW of a wide-batch, narrow layer: 2 x 2 tiles, 64 slices): the tiles of one
+    // K slice read the same rows of both operands.  Workgroups go to the XCDs in turn by their linear number
+    // (x fastest, z slowest), which would put a slice's tiles on different XCDs and fetch every operand row once
+    // per tile.  Renumbered so that a slice's tiles are consecutive workgroups of ONE XCD: they run at the same
+    // time and the second and later readers hit that XCD's L2.  Which workgroup computes which (tile, slice)
+    // changes, the sums do not.
+    unsigned const linear = blockIdx.z * ntiles + blockIdx.x;
+    unsigned const on_xcd = linear / kXcds;
+    lid = on_xcd % ntiles;
+    zslice = (on_xcd / ntiles) * kXcds + linear % kXcds;
+  }
+  gemm_tile<BM, BN, BK, A_KCONTIG, B_KCONTIG, MODE, RST, WVM>(g, lid, zslice, gridDim.z, lds);
 }
 
 // Several independent products of one kernel variant in ONE launch (the weight gradients of a network's layers:
