@@ -56,12 +56,14 @@ LAYER_WORKLOADS = {
 MIB = 1024.0 * 1024.0
 TRAFFIC_PROFILE = "profiles/hbm_traffic_pmc.md"
 MEASURED_TRAFFIC_BYTES = {
-    "c3": {"gemm": (897.8 + 897.3 + 832.8) / 3.0 * MIB, "norm_act": 901.8 * MIB},
+    "c3": {"gemm": (898.0 + 897.3 + 832.8) / 3.0 * MIB, "norm_act": 901.9 * MIB},
     "c2": {"norm_act": 326.4 * MIB},
+    "c4": {"gemm": (72.1 + 72.1 + 64.1) / 3.0 * MIB, "norm_act": 73.6 * MIB},
+    "c5": {"gemm": (132.3 + 132.5 + 144.1 + 16.3) / 3.0 * MIB, "norm_act": 516.5 * MIB},
 }
 TRAFFIC_SOURCES = ("gemm_f32_mfma.hip", "norm_kernels.hip", "norm_panel_fwd.hip", "norm_panel_bwd.hip",
                    "norm_panel_common.hpp", "norm_shared.hpp", "activations.hpp")
-TRAFFIC_SOURCES_SHA256 = "unset"
+TRAFFIC_SOURCES_SHA256 = "ae5aaa99cb44be7fa74af3490010b482e8a980bc03e90526f79fdf6f8ca7d476"
 
 
 def traffic_sources_digest():
@@ -745,7 +747,8 @@ def run_c4(args, torch, pkg, dl):
     flops = 2.0 * B * H * H
     avg = (t_f + t_x + t_w) / 3.0
     roof = {"bound": "mfma", "achieved": flops / (avg * 1e-3) / 1e12, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "traffic": None, "kernel": "k_gemm_f32 1024x2048x2048 (avg of fwd, dX, dW; operands cache-resident)"}
+            "traffic": measured_traffic("c4", "gemm"),
+            "kernel": "k_gemm_f32 1024x2048x2048 (avg of fwd, dX, dW; operands cache-resident)"}
     roof["frac"] = roof["achieved"] / roof["peak"]
     ytmp = torch.empty(B, H, **dev)
     t_nf = time_events(torch, lambda: dl.fused_fwd(desc, Zs[0], one, zero, mm[0], ms[0], mask=mask[0], out=ytmp,
@@ -755,7 +758,7 @@ def run_c4(args, torch, pkg, dl):
     # 32 B/element + 3 (mask read by three passes) + 4 (shortcut read by the forward apply pass); the 8 MiB
     # tensors are cache-resident and the chain is bound by launch latency, not by bandwidth
     hbm = {"bound": "hbm", "achieved": 39.0 * E / ((t_nf + t_nb) * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-           "traffic": None}
+           "traffic": measured_traffic("c4", "norm_act")}
     hbm["frac"] = hbm["achieved"] / hbm["peak"]
     bad = gave_up(*ctxs) or bad
     detail = {"ms": {"gemm_fwd": t_f, "gemm_dx": t_x, "gemm_dw": t_w, "norm_fwd": t_nf, "norm_bwd": t_nb,
@@ -982,9 +985,10 @@ def brief(o):
     r, h = o["roofline"], o.get("roofline_norm_act")
     out = {"w": o["config"]["workload"].split(":")[0], "value": o["value"], "ms_per_step": o["ms_per_step"],
            "steps": o["steps"], "warmup": o["warmup"],
-           "roofline": {"bound": r["bound"], "achieved": r["achieved"], "unit": r["unit"], "frac": r["frac"]}}
+           "roofline": {"bound": r["bound"], "achieved": r["achieved"], "unit": r["unit"], "frac": r["frac"],
+                        "traffic": r.get("traffic")}}
     if h is not None and r["bound"] != "hbm":
-        out["norm_act"] = {"achieved": h["achieved"], "frac": h["frac"]}
+        out["norm_act"] = {"achieved": h["achieved"], "frac": h["frac"], "traffic": h.get("traffic")}
     c = o.get("cpu_baseline")
     if c:
         out["cpu"] = {"value": c["value"], "cores": c["cores"], "kind": c["kind"]}
