@@ -372,6 +372,15 @@ class LayerStep:
         counters of a rocprofv3 --pmc run."""
         self.t["y"].copy_(self.t["dY"])
 
+    def strip_fwd(self):
+        """One tensor in, one out, walked like the single-launch normalization kernels walk theirs and nothing
+        else done with the data: the memory floor of the forward kernel's access pattern (measurement aid)."""
+        self.dl.probe_strip_stream(self.t["dY"], self.t["y"])
+
+    def strip_bwd(self):
+        """Two tensors in, one out, same pattern: the memory floor of the backward kernel's."""
+        self.dl.probe_strip_stream(self.t["dY"], self.t["dZ"], x2=self.t["y"])
+
     def parts(self):
         if self.K:
             return [self.fc_norm_fwd, self.norm_bwd_db, self.gemm_dx, self.gemm_dw_only]
@@ -1030,7 +1039,8 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=-1, help="rows of the CPU baseline sample (0 = skip the CPU legs "
                                                              "and the in-run parity check)")
     ap.add_argument("--only", default="", help="profiling aid (layer workloads): run just this part (gemm_fwd, gemm_dx, "
-                                               "gemm_dw, norm_fwd, norm_bwd, fc_norm_fwd, infer_fwd, adam, copy) "
+                                               "gemm_dw, gemm_dw_only, norm_fwd, norm_bwd, norm_bwd_db, fc_norm_fwd, infer_fwd, adam, copy, "
+                                               "strip_fwd, strip_bwd) "
                                                "--steps times and exit without a JSON line")
     ap.add_argument("--shape", default="", help="profiling aid, with --only: B,K,H of the layer to run the part on instead "
                                                 "of a workload's (e.g. 1024,2048,2048: one block of c4)")

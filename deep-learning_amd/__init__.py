@@ -45,7 +45,7 @@ C_ABI_SYMBOLS = [
     "dlmi_fused_norm_act_fwd_noalloc", "dlmi_fused_norm_act_residual_fwd", "dlmi_fc_norm_act_residual_fwd",
     "dlmi_fc_softmax_fwd", "dlmi_fc_bwd_dx_norm_act_bwd",
     "dlmi_ctx_reserve_layer", "dlmi_ctx_scratch_generation", "dlmi_ctx_norm_panel_enabled", "dlmi_ctx_norm_panel_poke",
-    "dlmi_fc_bwd_dw_grouped", "dlmi_fused_norm_act_bwd_db", "dlmi_ctx_gemm_clock",
+    "dlmi_fc_bwd_dw_grouped", "dlmi_fused_norm_act_bwd_db", "dlmi_ctx_gemm_clock", "dlmi_probe_strip_stream",
 ]
 
 
@@ -154,6 +154,13 @@ class Dlmi:
     def norm_panel_poke(self, xcd, word, value):
         """Test hook: one word of an XCD's barrier state (see dlmi.h)."""
         self._ck(self.lib.dlmi_ctx_norm_panel_poke(self.ctx, ctypes.c_uint(xcd), ctypes.c_uint(word), ctypes.c_uint(value)))
+
+    def probe_strip_stream(self, x, y, x2=None):
+        """Measurement aid: y = x (+ x2) streamed in the column panel kernels' access pattern (see dlmi.h)."""
+        self._chk(x, y, x2)
+        B, H = x.shape
+        self._ck(self.lib.dlmi_probe_strip_stream(self.ctx, c_sz(B), c_sz(H), _p(x), _p(x2), _p(y)))
+        return y
 
     # ------------------------------------------------------------ GEMMs
     def fc_fwd(self, X, W, bias=None, out=None):

@@ -104,6 +104,12 @@ int dlmi_ctx_norm_panel_enabled(dlmi_ctx const *ctx);
  * (ticks / time) and that workgroup's lifetime in microseconds: the clock INSIDE the launch, with no profiler
  * attached.  DLMI_E_INVALID without the environment variable or before the first product. */
 int dlmi_ctx_gemm_clock(dlmi_ctx *ctx, double *engine_mhz, double *tile_us);
+/* Measurement aid, no counterpart in the reference.  y = x (x2 == NULL) or y = x + x2 on [B, H] fp32, by 256
+ * workgroups that walk the tensors the way the single-launch normalization kernels do (each XCD its eighth of the
+ * columns in panels of 64, each of its 32 workgroups its 32nd of the rows) and do nothing else with the data: the
+ * time of this launch is the memory floor of that access pattern on the device at hand.  H in multiples of 512, B in
+ * multiples of 4096, 16-byte aligned pointers; DLMI_E_INVALID otherwise. */
+int dlmi_probe_strip_stream(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float const *x2, float *y);
 int dlmi_ctx_norm_panel_poke(dlmi_ctx *ctx, unsigned xcd, unsigned word, unsigned value);
 /* How a product C[M,N] = A[M,K] . B[K,N] would be launched on a device with `compute_units` CUs: tile shape, K
  * slices (1 = none; more = partial products plus a fixed-order sum) and register stages of the K loop.  Host
