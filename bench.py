@@ -131,7 +131,7 @@ def rel_errors(got, exp):
     return a, b
 
 
-def parity_block(pairs, limit, f64=None, extra=None):
+def parity_block(pairs, limit, f64=None, extra=None, ref_rms_floor=None):
     """pairs: name -> (gpu array, cpu array).  The rms-floored error must meet `limit` (1e-4 behind
     reductions and GEMMs, as the parity tests assert); the strict per-element error is reported beside it.
     f64: name -> (gpu slab, its float64 target, cpu slab, its float64 target): the arbitration of the strict
@@ -141,6 +141,10 @@ def parity_block(pairs, limit, f64=None, extra=None):
     tensors of the GPU's root-mean-square error against float64 to the CPU baseline's.  `ok` is judged on the
     ratio (at most 2): the two maxima are single-element errors, whose quotient scatters by more than that
     between two summation orders of equal accuracy.
+    ref_rms_floor: name -> rms error of the reference's OTHER summation order for that tensor (its single-thread
+    leaf, where the timed baseline is its OpenMP path): the baseline error of the ratio is the larger of the two,
+    so the GPU is asked to be no worse than the reference's less accurate own order (`f64.baseline` says which
+    tensors took it).
     Returns (compact block for the line, per-tensor block for the report)."""
     full, ok, worst = {}, True, ("", 0.0, 0.0)
     for k, (g, e) in pairs.items():
@@ -154,17 +158,22 @@ def parity_block(pairs, limit, f64=None, extra=None):
     if f64:
         import numpy as np
         rms = lambda a: float(np.sqrt(np.mean(np.square(np.asarray(a, np.float64)))))
-        g_max, r_max, ratio, worst64 = 0.0, 0.0, 0.0, ""
+        g_max, r_max, ratio, worst64, floored = 0.0, 0.0, 0.0, "", []
         for k, (g, xg, e, xe) in f64.items():
             eg, er = rel_errors(g, xg)[1], rel_errors(e, xe)[1]
             rg, rr = rms(np.asarray(g, np.float64) - xg), rms(np.asarray(e, np.float64) - xe)
-            q = rg / max(rr, 1e-7 * rms(xg), 1e-300)  # a baseline that is exact leaves the float's own rounding
+            floor = (ref_rms_floor or {}).get(k, 0.0)
+            if floor > rr:
+                floored.append(k)
+            q = rg / max(rr, floor, 1e-7 * rms(xg), 1e-300)  # a baseline that is exact leaves the float's own rounding
             full.setdefault(k, {}).update({"strict_gpu_vs_f64": eg, "strict_ref_vs_f64": er, "rms_err_gpu_vs_f64": rg,
                                            "rms_err_ref_vs_f64": rr})
             g_max, r_max = max(g_max, eg), max(r_max, er)
             if q >= ratio:
                 ratio, worst64 = q, k
         out["f64"] = {"gpu": g_max, "ref": r_max, "rms_ratio": ratio, "worst": worst64, "ok": ratio <= 2.0}
+        if floored:
+            out["f64"]["baseline"] = "single-thread order for " + ",".join(floored)
     if extra:
         out.update(extra)
     return out, full
@@ -650,11 +659,13 @@ def run_layer(args, torch, pkg, dl, name, full):
             if name == "c5":
                 cp.inference()
             ref = cp.results()
+            chain = dw_single_chain(h, gpu, ref, B, H, K) if K else None
             parity, per_tensor = parity_block({k: (gpu[k], ref[k]) for k in ref}, 1e-4, layer_f64_slabs(name, h, gpu, ref),
-                                              {"kinks_zeroed": kinks})
+                                              {"kinks_zeroed": kinks},
+                                              {"dW": chain["rms_err_single_chain_vs_f64"]} if chain else None)
             report["parity_tensors"] = per_tensor
-            if K:
-                report["dW_summation_order"] = dw_single_chain(h, gpu, ref, B, H, K)
+            if chain:
+                report["dW_summation_order"] = chain
     config = {"workload": name + ": " + descr, "batch": B, "fan_in": K, "units": H}
     detail["panel_gave_up"] = bad
     del step, t
