@@ -9,11 +9,15 @@
 // faster - the forward kernel's 128 columns reach 5.1 TB/s of actual traffic, 64 columns 3.7 TB/s - but the
 // backward pass holds two values per element; the kernel still beats the multi-launch pair because it moves
 // 12 instead of 20 bytes per element.)
+#include <type_traits>
+
 #include "norm_panel_common.hpp"
 
 namespace dlmi {
 namespace {
 
+
+constexpr int kPanelMaxCols = 1024;  // columns of one XCD whose per-unit constants fit the workgroup's LDS (H <= 8192)
 
 struct PanelBwdArgs {
   float const *x, *dY, *gamma, *beta, *mean, *stdv, *r, *d;
@@ -25,6 +29,54 @@ struct PanelBwdArgs {
   PanelSync sync;
   float *part;  // [xcd][panel][rank][3][kP]
 };
+
+// Loads whose completion this file waits for itself.  A wavefront's loads return in the order they were issued, and
+// the compiler, which must assume the fewest younger loads over every path to a use, would wait for ALL loads in
+// flight before the first use of a panel fetched two steps earlier (it does: vmcnt(0) in the steady state) - the
+// panels just asked for would never be in flight while this one is worked on.  So the bulk loads and the loads of
+// the other workgroups' sums are issued as explicit instructions, invisible to the compiler's bookkeeping, and
+// every use is preceded by an explicit wait that names the number of younger memory operations of the wavefront
+// that may still be outstanding; the registers pass through that wait as in/out operands, so no use can be
+// scheduled before it.
+__device__ __forceinline__ void issue_load(pv4f &dst, float const *p) {
+  asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void issue_load(float &dst, float const *p) {
+  asm volatile("global_load_dword %0, %1, off nt" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void issue_load(unsigned &dst, uint8_t const *p) {  // four mask bytes
+  asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+// the same with a count known at run time (the same in all lanes of a wavefront), 0 .. 47
+template <int N>
+__device__ __forceinline__ void wait_younger_dispatch(int n) {
+  if constexpr (N >= 47) {
+    asm volatile("s_waitcnt vmcnt(47)" ::: "memory");
+  } else {
+    if (n <= N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+    else wait_younger_dispatch<N + 1>(n);
+  }
+}
+__device__ __forceinline__ void wait_younger_n(int n) {
+  wait_younger_dispatch<0>(__builtin_amdgcn_readfirstlane(n < 0 ? 0 : n));
+}
+template <int N>
+__device__ __forceinline__ void wait_younger() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// the wait, with the values it makes usable
+template <int N>
+__device__ __forceinline__ void wait_for(pv4f &a, pv4f &b) {
+  asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_for(float &a) {
+  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_for(unsigned &a) {
+  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(N) : "memory");
+}
 
 // dn of one element, dropout mode at run time (bwd_dn of the multi-launch path, same operations)
 template <int ACT>
@@ -53,7 +105,10 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
   constexpr int kRPer = kPanelRanks / kRSplit;
   __shared__ float sh[3][kTY][kP];       // per-sweep-row sums of the panel being published
   __shared__ float sh2[kRSplit][kVals];  // halves of the rank sum
-  __shared__ float cst[4][7][kP];        // per panel in flight: mean, r/std, d, gamma, beta, std, r
+  // per-unit constants of ALL columns of this XCD (the forward's results), fetched once before the first panel:
+  // mean, r/std, d, gamma, beta, std, r, per-unit keep mask.  A load of them inside a step would return behind
+  // that step's bulk loads (a wavefront's loads return in issue order) and stall the arithmetic on them.
+  __shared__ float cst[8][kPanelMaxCols];
   __shared__ float coef[3][kP];
   __shared__ unsigned s_rank, s_ok;
   PanelWho who;
@@ -65,43 +120,69 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
   size_t const row0 = static_cast<size_t>(who.rank) * (RPT * kTY);
   size_t const col_base = static_cast<size_t>(who.xcd) * Hx;
 
+  auto preload_constants = [&] {
+  for (size_t c = threadIdx.x; c < Hx; c += kPanelThreads) {
+    float const sd = a.stdv[col_base + c], rr = a.r[col_base + c];
+    cst[0][c] = a.mean[col_base + c];
+    cst[1][c] = rr * fast_rcp(sd);
+    cst[2][c] = a.d[col_base + c];
+    cst[3][c] = a.gamma[col_base + c];
+    cst[4][c] = a.beta[col_base + c];
+    cst[5][c] = sd;
+    cst[6][c] = rr;
+    cst[7][c] = a.drop_mode == kDropUnit ? (a.mask[col_base + c] ? 1.0f : 0.0f) : 1.0f;
+  }
+  __syncthreads();
+  };
+
   struct Stage {
     pv4f x[RPT], g[RPT];          // x, and dY until publish() turns it into dn
-    uchar4 m[EXTRA ? RPT : 1];    // per-element keep mask
+    unsigned m[EXTRA ? RPT : 1];  // per-element keep mask, four bytes
   };
+  bool const elem = EXTRA && a.drop_mode == kDropElem;
   auto load = [&](Stage &s, int p) {
     size_t const off0 = (row0 + ty) * a.H + col_base + static_cast<size_t>(p) * kP + tx * 4;
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
       size_t const off = off0 + static_cast<size_t>(i) * kTY * a.H;
-      s.x[i] = __builtin_nontemporal_load(reinterpret_cast<pv4f const *>(a.x + off));
-      s.g[i] = __builtin_nontemporal_load(reinterpret_cast<pv4f const *>(a.dY + off));
+      issue_load(s.x[i], a.x + off);
+      issue_load(s.g[i], a.dY + off);
       if constexpr (EXTRA) {
-        if (a.drop_mode == kDropElem) s.m[i] = *reinterpret_cast<uchar4 const *>(a.mask + off);
+        if (elem) issue_load(s.m[i], a.mask + off);
       }
+    }
+  };
+  // Before the first use of a stage: at most `younger` memory operations of this wavefront that were issued after
+  // the stage's loads may still be outstanding.
+  auto wait_stage = [&](Stage &s, int younger) {
+    wait_younger_n(younger);
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      asm volatile("" : "+v"(s.x[i]), "+v"(s.g[i]));
+      if constexpr (EXTRA) asm volatile("" : "+v"(s.m[i]));
     }
   };
   auto publish = [&](Stage &s, int p) {
     size_t const col = col_base + static_cast<size_t>(p) * kP;
-    // per-unit constants of this thread's 4 columns (the forward's results)
-    pv4f mu = *reinterpret_cast<pv4f const *>(a.mean + col + tx * 4);
-    pv4f sd = *reinterpret_cast<pv4f const *>(a.stdv + col + tx * 4);
-    pv4f rr = *reinterpret_cast<pv4f const *>(a.r + col + tx * 4);
-    pv4f dd = *reinterpret_cast<pv4f const *>(a.d + col + tx * 4);
-    pv4f ga = *reinterpret_cast<pv4f const *>(a.gamma + col + tx * 4);
-    pv4f be = *reinterpret_cast<pv4f const *>(a.beta + col + tx * 4);
-    uchar4 um = make_uchar4(1, 1, 1, 1);
-    if (a.drop_mode == kDropUnit) um = *reinterpret_cast<uchar4 const *>(a.mask + col + tx * 4);
-    pv4f rs;
+    // per-unit constants of this thread's 4 columns
+    int const lc = p * kP + tx * 4;  // column inside this XCD's range
+    pv4f mu, rs, dd, ga, be;
+    unsigned char umv[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) rs[e] = rr[e] * fast_rcp(sd[e]);
-    unsigned char const umv[4] = {um.x, um.y, um.z, um.w};
+    for (int e = 0; e < 4; ++e) {
+      mu[e] = cst[0][lc + e]; rs[e] = cst[1][lc + e]; dd[e] = cst[2][lc + e]; ga[e] = cst[3][lc + e];
+      be[e] = cst[4][lc + e];
+      umv[e] = cst[7][lc + e] != 0.0f ? 1 : 0;
+    }
+    (void)col;
     pv4f s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0}, s2 = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
       unsigned char mv[4] = {umv[0], umv[1], umv[2], umv[3]};
       if constexpr (EXTRA) {
-        if (a.drop_mode == kDropElem) { mv[0] = s.m[i].x; mv[1] = s.m[i].y; mv[2] = s.m[i].z; mv[3] = s.m[i].w; }
+        if (elem) {
+          mv[0] = s.m[i] & 0xffu; mv[1] = (s.m[i] >> 8) & 0xffu; mv[2] = (s.m[i] >> 16) & 0xffu; mv[3] = s.m[i] >> 24;
+        }
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -114,20 +195,12 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
         s.g[i][e] = dn;
       }
     }
-    __syncthreads();  // the previous publish's readers are done with sh
+    // (the previous publish's readers are done with sh: at least one workgroup barrier lies between)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       sh[0][ty][tx * 4 + e] = s0[e];
       sh[1][ty][tx * 4 + e] = s1[e];
       sh[2][ty][tx * 4 + e] = s2[e];
-    }
-    if (ty == 0) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        int const c = tx * 4 + e;
-        cst[p & 3][0][c] = mu[e]; cst[p & 3][1][c] = rs[e]; cst[p & 3][2][c] = dd[e]; cst[p & 3][3][c] = ga[e];
-        cst[p & 3][4][c] = be[e]; cst[p & 3][5][c] = sd[e]; cst[p & 3][6][c] = rr[e];
-      }
     }
     __syncthreads();
     if (threadIdx.x < kVals) {
@@ -142,7 +215,47 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
     __syncthreads();
     if (threadIdx.x == 0) panel_count(panel_arrivals(who, p));
   };
-  auto finish = [&](Stage const &s, int p) -> bool {
+  // ---- the exchange with the other workgroups, one step ahead of its use ------------------------------------
+  // A wavefront's memory operations complete in the order they were issued, so a small load that everything
+  // depends on completes behind every bulk load and every store issued before it.  The exchange is therefore
+  // spread over a step: the count of arrivals for panel p + 1 is asked for at the start of step p and looked
+  // at its end; the other workgroups' sums of p + 1 are then requested, travel while step p + 1 forms the sums
+  // of p + 3, and are added up after that.  Every wait names the younger operations of its wavefront that may
+  // stay in flight (they differ between wavefronts: `stored` ones write a share of the workgroup's sums, `sums`
+  // ones fetch the others' sums, wavefront 0 polls).
+  int const wave_first = static_cast<int>(threadIdx.x & ~63u);
+  bool const stored = wave_first < kVals;             // this wavefront issues the one store of publish()
+  bool const sums = threadIdx.x < kRSplit * kVals;    // whole wavefronts: kRSplit * kVals is a multiple of 64
+  int const extra = sums ? kRPer : 0;                 // its loads of the others' sums
+  int const ld = elem ? 3 * RPT : 2 * RPT;            // bulk loads of a panel per thread
+  int const vc = threadIdx.x % kVals, rs = sums ? threadIdx.x / kVals : 0;
+  float v[kRPer];
+#pragma unroll
+  for (int r = 0; r < kRPer; ++r) v[r] = 0.0f;
+  auto request_sums = [&](int p) {  // every workgroup of this XCD has arrived for panel p
+    float const *pp = a.part + (static_cast<size_t>(who.xcd) * npanels + p) * kPanelRanks * kVals + vc;
+    if (sums) {
+#pragma unroll
+      for (int r = 0; r < kRPer; ++r) issue_load(v[r], pp + static_cast<size_t>(rs * kRPer + r) * kVals);
+    }
+  };
+  unsigned polled = 0;
+  auto poll_issue = [&](int p) {
+    if (threadIdx.x == 0) {
+      unsigned zero = 0;
+      asm volatile("global_atomic_add %0, %1, %2, off sc0" : "=v"(polled) : "v"(panel_arrivals(who, p)), "v"(zero) : "memory");
+    }
+  };
+  auto poll_check = [&](int p, int younger) {
+    if (threadIdx.x == 0) {
+      wait_younger_n(younger);
+      asm volatile("" : "+v"(polled));
+      unsigned const target = static_cast<unsigned>(kPanelRanks) * static_cast<unsigned>(p / 2 + 1);
+      if (polled < target && !panel_wait(who, p)) s_ok = 0;  // somebody is late: poll until it has arrived
+    }
+  };
+  // Finishes panel p from the sums requested a step ago; `younger`: operations issued after that request.
+  auto finish = [&](Stage const &s, int p, int younger) {
     size_t const col = col_base + static_cast<size_t>(p) * kP;
     size_t const off0 = (row0 + ty) * a.H + col + tx * 4;
     pv4f old[EXTRA ? RPT : 1];
@@ -153,18 +266,14 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
           old[i] = __builtin_nontemporal_load(reinterpret_cast<pv4f const *>(a.dX + off0 + static_cast<size_t>(i) * kTY * a.H));
       }
     }
-    if (threadIdx.x == 0 && !panel_wait(who, p)) s_ok = 0;
-    __syncthreads();
-    if (!s_ok) return false;
-    if (threadIdx.x < kRSplit * kVals) {
-      int const vc = threadIdx.x % kVals, rs = threadIdx.x / kVals;
-      float const *pp = a.part + (static_cast<size_t>(who.xcd) * npanels + p) * kPanelRanks * kVals + vc;
-      float v[kRPer];
-#pragma unroll
-      for (int r = 0; r < kRPer; ++r) v[r] = __builtin_nontemporal_load(pp + static_cast<size_t>(rs * kRPer + r) * kVals);
+    if (sums) {
+      wait_younger_n(younger);
       float t = 0.0f;
 #pragma unroll
-      for (int r = 0; r < kRPer; ++r) t += v[r];
+      for (int r = 0; r < kRPer; ++r) {
+        asm volatile("" : "+v"(v[r]));
+        t += v[r];
+      }
       sh2[rs][vc] = t;
     }
     __syncthreads();
@@ -177,10 +286,13 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
         t1 += sh2[j][kP + c];
         t2 += sh2[j][2 * kP + c];
       }
-      float const ga = cst[p & 3][3][c], sd = cst[p & 3][5][c], rr = cst[p & 3][6][c];
-      if (who.rank == 0) {  // accumulating like the reference's derivative array
-        a.dgamma[col + c] += t0;
-        a.dbeta[col + c] += t1;
+      int const lc = p * kP + c;
+      float const ga = cst[3][lc], sd = cst[5][lc], rr = cst[6][lc];
+      if (who.rank == 0) {
+        // accumulating like the reference's derivative array; one addition per unit and launch, by this workgroup
+        // alone, as an atomic without return value so that nothing here waits behind the loads in flight
+        (void)__hip_atomic_fetch_add(a.dgamma + col + c, t0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        (void)__hip_atomic_fetch_add(a.dbeta + col + c, t1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       float const dm = (ga * t1) * (-rr / sd);
       float const ds = (ga * t2) * (-rr / (sd * sd));
@@ -192,7 +304,7 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
     pv4f mu, c1, c2, c3;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      mu[e] = cst[p & 3][0][tx * 4 + e];
+      mu[e] = cst[0][p * kP + tx * 4 + e];
       c1[e] = coef[0][tx * 4 + e];
       c2[e] = coef[1][tx * 4 + e];
       c3[e] = coef[2][tx * 4 + e];
@@ -210,43 +322,66 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
       }
       __builtin_nontemporal_store(out, reinterpret_cast<pv4f *>(a.dX + off0 + static_cast<size_t>(i) * kTY * a.H));
     }
-    return true;
   };
 
-  // Four panels in flight, one step apart (see norm_panel_fwd.hip): loading p+3, sums of p+2 stored,
-  // p+1 counted in at the barrier word, p finished.
-  Stage b0, b1, b2, b3;
+  // Five panels in flight, one step apart: p + 4 loading, p + 3 loaded, sums of p + 2 stored, p + 1 counted in at
+  // the barrier word and its count asked for, p finished.
+  Stage b0, b1, b2, b3, b4;
+  auto clamped = [&](int p) { return p < npanels ? p : npanels - 1; };
   load(b0, 0);
-  if (npanels > 1) load(b1, 1);
-  if (npanels > 2) load(b2, 2);
+  load(b1, clamped(1));
+  preload_constants();  // (its loads are younger than those of panels 0 and 1: waiting for them completes both)
+  wait_stage(b0, ld);  // panel 1's loads are younger
   publish(b0, 0);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  load(b2, clamped(2));
+  load(b3, clamped(3));
+  wait_younger_n(2 * ld);  // the partial of panel 0 is older than the loads of panels 2 and 3
   arrive(0);
-  if (npanels > 1) publish(b1, 1);
-  bool const elem = EXTRA && a.drop_mode == kDropElem;
-  auto step = [&](Stage &cur, Stage &s1, Stage &s2, Stage &s3, int p) -> bool {
-    (void)s1;
-    // loads of panel p+3 first; then the partial of p+1 (stored a step ago) must have reached the L2: it is
-    // older than the RPT stores of dX that ended the last step and than the loads just issued
-    if (p + 3 < npanels) {
-      load(s3, p + 3);
-      if (p + 1 < npanels) {
-        if (elem) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * RPT) : "memory");
-        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * RPT) : "memory");
-      }
-    } else if (p + 1 < npanels) {
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(RPT) : "memory");
+  if (npanels > 1) {
+    wait_stage(b1, 2 * ld);
+    publish(b1, 1);
+  }
+  if (threadIdx.x == 0 && !panel_wait(who, 0)) s_ok = 0;
+  __syncthreads();
+  if (!s_ok) return;
+  request_sums(0);
+  auto step = [&](Stage &cur, Stage &s2, Stage &s4, int p) -> bool {
+    bool const more1 = p + 1 < npanels, more2 = p + 2 < npanels, more4 = p + 4 < npanels;
+    // younger than the store of publish(p + 1) and than the loads of panel p + 2, both issued before them: the
+    // loads of panel p + 3 (if it exists; asked for in the prologue for p = 0), RPT stores of dX (not before the
+    // first step)
+    int const behind = (p == 0 || p + 3 < npanels ? ld : 0) + (p == 0 ? 0 : RPT);
+    if (p > 0) {
+      // the arrivals for panel p, asked for at the start of the last step.  Younger in wavefront 0: the request
+      // for the sums of p - 1 (from the second step on), publish's store, the loads of p + 3, RPT stores of dX
+      poll_check(p, (p >= 2 ? kRPer : 0) + (more1 ? 1 : 0) + (p + 3 < npanels ? ld : 0) + RPT);
     }
-    if (p + 1 < npanels) arrive(p + 1);
-    if (p + 2 < npanels) publish(s2, p + 2);
-    return finish(cur, p);
+    // the partial of p + 1 must have reached the L2 before this workgroup counts itself in (p = 0: only the
+    // request for the sums of panel 0 is younger)
+    if (more1) wait_younger_n(p == 0 ? extra : behind);
+    __syncthreads();
+    if (!s_ok) return false;
+    if (more1) {
+      if (threadIdx.x == 0) panel_count(panel_arrivals(who, p + 1));
+      poll_issue(p + 1);
+    }
+    if (p > 0) request_sums(p);
+    if (more2) {
+      wait_stage(s2, behind + extra);
+      publish(s2, p + 2);
+    }
+    if (more4) load(s4, p + 4);
+    // younger than the request for the sums of p: that store of publish, the loads just issued
+    finish(cur, p, (more4 ? ld : 0) + (stored && more2 ? 1 : 0));
+    return true;
   };
   bool ok = true;
-  for (int p = 0; p < npanels && ok; p += 4) {
-    ok = step(b0, b1, b2, b3, p);
-    if (ok && p + 1 < npanels) ok = step(b1, b2, b3, b0, p + 1);
-    if (ok && p + 2 < npanels) ok = step(b2, b3, b0, b1, p + 2);
-    if (ok && p + 3 < npanels) ok = step(b3, b0, b1, b2, p + 3);
+  for (int p = 0; p < npanels && ok; p += 5) {
+    ok = step(b0, b2, b4, p);
+    if (ok && p + 1 < npanels) ok = step(b1, b3, b0, p + 1);
+    if (ok && p + 2 < npanels) ok = step(b2, b4, b1, p + 2);
+    if (ok && p + 3 < npanels) ok = step(b3, b0, b2, p + 3);
+    if (ok && p + 4 < npanels) ok = step(b4, b1, b3, p + 4);
   }
   if (ok) panel_leave(who);
 }
@@ -260,7 +395,7 @@ void launch_bwd(dlmi_ctx *ctx, PanelBwdArgs const &a) {
 
 int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4, void *scratch, size_t scratch_bytes) {
   if (!ctx->panel_ok || !vec4 || c.xhat_given || c.dmean != nullptr || c.dstd != nullptr) return 0;
-  if (H % 512 != 0) return 0;
+  if (H % 512 != 0 || H / kPanelXcds > static_cast<size_t>(kPanelMaxCols)) return 0;  // the per-unit constants of an XCD's columns live in LDS
   // 8192 rows: four panels of x and dn only fit the registers at 32 columns per panel, and rows cut into
   // 128-byte pieces stream slower than the multi-launch kernels (measured 113 us against 108 us at 8192 x 4096)
   // 1024 rows: no faster than the multi-launch pair in isolation (15 us both) and slower inside a step, where a
