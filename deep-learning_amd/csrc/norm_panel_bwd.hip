@@ -4,8 +4,8 @@
 // kept in registers between the reduction and the apply step instead of being recomputed.
 //
 // Geometry: 512 threads = P/4 column groups of 4 units x 2048/P rows; a workgroup owns B/32 = RPT * 2048/P rows
-// and walks panels of P columns: P = 64 (256 B per row) while four panels of x and dn fit the registers, P = 32
-// for 4096 rows with a per-element mask.  B in {2048, 4096}, H a multiple of 512.  (Wider panels stream
+// and walks panels of P columns: P = 64 (256 B per row) while five panels of x and dn fit the registers, P = 32
+// for 4096 rows with a per-element mask.  B in {2048, 4096}, H a multiple of 512 and at most 8 * kPanelMaxCols.  (Wider panels stream
 // faster - the forward kernel's 128 columns reach 5.1 TB/s of actual traffic, 64 columns 3.7 TB/s - but the
 // backward pass holds two values per element; the kernel still beats the multi-launch pair because it moves
 // 12 instead of 20 bytes per element.)
@@ -29,54 +29,6 @@ struct PanelBwdArgs {
   PanelSync sync;
   float *part;  // [xcd][panel][rank][3][kP]
 };
-
-// Loads whose completion this file waits for itself.  A wavefront's loads return in the order they were issued, and
-// the compiler, which must assume the fewest younger loads over every path to a use, would wait for ALL loads in
-// flight before the first use of a panel fetched two steps earlier (it does: vmcnt(0) in the steady state) - the
-// panels just asked for would never be in flight while this one is worked on.  So the bulk loads and the loads of
-// the other workgroups' sums are issued as explicit instructions, invisible to the compiler's bookkeeping, and
-// every use is preceded by an explicit wait that names the number of younger memory operations of the wavefront
-// that may still be outstanding; the registers pass through that wait as in/out operands, so no use can be
-// scheduled before it.
-__device__ __forceinline__ void issue_load(pv4f &dst, float const *p) {
-  asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst) : "v"(p) : "memory");
-}
-__device__ __forceinline__ void issue_load(float &dst, float const *p) {
-  asm volatile("global_load_dword %0, %1, off nt" : "=v"(dst) : "v"(p) : "memory");
-}
-__device__ __forceinline__ void issue_load(unsigned &dst, uint8_t const *p) {  // four mask bytes
-  asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
-}
-// the same with a count known at run time (the same in all lanes of a wavefront), 0 .. 47
-template <int N>
-__device__ __forceinline__ void wait_younger_dispatch(int n) {
-  if constexpr (N >= 47) {
-    asm volatile("s_waitcnt vmcnt(47)" ::: "memory");
-  } else {
-    if (n <= N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-    else wait_younger_dispatch<N + 1>(n);
-  }
-}
-__device__ __forceinline__ void wait_younger_n(int n) {
-  wait_younger_dispatch<0>(__builtin_amdgcn_readfirstlane(n < 0 ? 0 : n));
-}
-template <int N>
-__device__ __forceinline__ void wait_younger() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-// the wait, with the values it makes usable
-template <int N>
-__device__ __forceinline__ void wait_for(pv4f &a, pv4f &b) {
-  asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_for(float &a) {
-  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(N) : "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_for(unsigned &a) {
-  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(N) : "memory");
-}
 
 // dn of one element, dropout mode at run time (bwd_dn of the multi-launch path, same operations)
 template <int ACT>
@@ -147,8 +99,8 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
       size_t const off = off0 + static_cast<size_t>(i) * kTY * a.H;
       issue_load(s.x[i], a.x + off);
       issue_load(s.g[i], a.dY + off);
-      if constexpr (EXTRA) {
-        if (elem) issue_load(s.m[i], a.mask + off);
+      if constexpr (EXTRA) {  // (always asked for, from a fixed valid address when there is no such mask)
+        issue_load(s.m[i], elem ? a.mask + off : reinterpret_cast<uint8_t const *>(a.gamma));
       }
     }
   };
@@ -218,28 +170,29 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
   // ---- the exchange with the other workgroups, one step ahead of its use ------------------------------------
   // A wavefront's memory operations complete in the order they were issued, so a small load that everything
   // depends on completes behind every bulk load and every store issued before it.  The exchange is therefore
-  // spread over a step: the count of arrivals for panel p + 1 is asked for at the start of step p and looked
-  // at its end; the other workgroups' sums of p + 1 are then requested, travel while step p + 1 forms the sums
-  // of p + 3, and are added up after that.  Every wait names the younger operations of its wavefront that may
+  // spread over a step: the count of arrivals for panel p + 1 is asked for in the middle of step p (the others
+  // have had the first half of the step to count themselves in) and looked at when step p + 1 starts; the other
+  // workgroups' sums of p + 1 are then requested, travel while step p + 1 forms the sums of p + 3, and are added
+  // up after that.  Every wait names the younger operations of its wavefront that may
   // stay in flight (they differ between wavefronts: `stored` ones write a share of the workgroup's sums, `sums`
   // ones fetch the others' sums, wavefront 0 polls).
   int const wave_first = static_cast<int>(threadIdx.x & ~63u);
   bool const stored = wave_first < kVals;             // this wavefront issues the one store of publish()
   bool const sums = threadIdx.x < kRSplit * kVals;    // whole wavefronts: kRSplit * kVals is a multiple of 64
-  int const extra = sums ? kRPer : 0;                 // its loads of the others' sums
-  int const ld = elem ? 3 * RPT : 2 * RPT;            // bulk loads of a panel per thread
+  int const extra = kRPer;                            // a thread's loads of the others' sums
+  int const ld = EXTRA ? 3 * RPT : 2 * RPT;           // bulk loads of a panel per thread
   int const vc = threadIdx.x % kVals, rs = sums ? threadIdx.x / kVals : 0;
   float v[kRPer];
-#pragma unroll
-  for (int r = 0; r < kRPer; ++r) v[r] = 0.0f;
+  // (every thread asks, the ones that do not add anything up for a share that others ask for as well: the
+  // registers have no other definition than the loads' results, and every wavefront issues the same operations)
   auto request_sums = [&](int p) {  // every workgroup of this XCD has arrived for panel p
     float const *pp = a.part + (static_cast<size_t>(who.xcd) * npanels + p) * kPanelRanks * kVals + vc;
-    if (sums) {
 #pragma unroll
-      for (int r = 0; r < kRPer; ++r) issue_load(v[r], pp + static_cast<size_t>(rs * kRPer + r) * kVals);
-    }
+    for (int r = 0; r < kRPer; ++r) issue_load(v[r], pp + static_cast<size_t>(rs * kRPer + r) * kVals);
   };
-  unsigned polled = 0;
+  // (no other definition than the instruction's result: a value merged with another one would be copied at the
+  // merge point, i.e. right behind the instruction, before the result has arrived)
+  unsigned polled;
   auto poll_issue = [&](int p) {
     if (threadIdx.x == 0) {
       unsigned zero = 0;
@@ -266,14 +219,15 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
           old[i] = __builtin_nontemporal_load(reinterpret_cast<pv4f const *>(a.dX + off0 + static_cast<size_t>(i) * kTY * a.H));
       }
     }
+    // every wavefront waits for what it asked for: a register whose load is still in flight must not be given
+    // to another value
+    wait_younger_n(younger);
+#pragma unroll
+    for (int r = 0; r < kRPer; ++r) asm volatile("" : "+v"(v[r]));
     if (sums) {
-      wait_younger_n(younger);
       float t = 0.0f;
 #pragma unroll
-      for (int r = 0; r < kRPer; ++r) {
-        asm volatile("" : "+v"(v[r]));
-        t += v[r];
-      }
+      for (int r = 0; r < kRPer; ++r) t += v[r];
       sh2[rs][vc] = t;
     }
     __syncthreads();
@@ -352,9 +306,9 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
     // first step)
     int const behind = (p == 0 || p + 3 < npanels ? ld : 0) + (p == 0 ? 0 : RPT);
     if (p > 0) {
-      // the arrivals for panel p, asked for at the start of the last step.  Younger in wavefront 0: the request
-      // for the sums of p - 1 (from the second step on), publish's store, the loads of p + 3, RPT stores of dX
-      poll_check(p, (p >= 2 ? kRPer : 0) + (more1 ? 1 : 0) + (p + 3 < npanels ? ld : 0) + RPT);
+      // the arrivals for panel p, asked for in the middle of the last step (the other workgroups had until then
+      // to count themselves in).  Younger in wavefront 0: the loads of p + 3, RPT stores of dX
+      poll_check(p, (p + 3 < npanels ? ld : 0) + RPT);
     }
     // the partial of p + 1 must have reached the L2 before this workgroup counts itself in (p = 0: only the
     // request for the sums of panel 0 is younger)
@@ -363,13 +317,13 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
     if (!s_ok) return false;
     if (more1) {
       if (threadIdx.x == 0) panel_count(panel_arrivals(who, p + 1));
-      poll_issue(p + 1);
     }
     if (p > 0) request_sums(p);
     if (more2) {
       wait_stage(s2, behind + extra);
       publish(s2, p + 2);
     }
+    if (more1) poll_issue(p + 1);
     if (more4) load(s4, p + 4);
     // younger than the request for the sums of p: that store of publish, the loads just issued
     finish(cur, p, (more4 ? ld : 0) + (stored && more2 ? 1 : 0));

@@ -76,6 +76,54 @@ __device__ __forceinline__ void panel_count(unsigned *p) {
   asm volatile("global_atomic_add %0, %1, off" ::"v"(p), "v"(one) : "memory");
 }
 
+// Loads whose completion the panel kernels wait for themselves.  A wavefront's loads return in the order they were issued, and
+// the compiler, which must assume the fewest younger loads over every path to a use, would wait for ALL loads in
+// flight before the first use of a panel fetched two steps earlier (it does: vmcnt(0) in the steady state) - the
+// panels just asked for would never be in flight while this one is worked on.  So the bulk loads and the loads of
+// the other workgroups' sums are issued as explicit instructions, invisible to the compiler's bookkeeping, and
+// every use is preceded by an explicit wait that names the number of younger memory operations of the wavefront
+// that may still be outstanding; the registers pass through that wait as in/out operands, so no use can be
+// scheduled before it.
+__device__ __forceinline__ void issue_load(pv4f &dst, float const *p) {
+  asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void issue_load(float &dst, float const *p) {
+  asm volatile("global_load_dword %0, %1, off nt" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void issue_load(unsigned &dst, uint8_t const *p) {  // four mask bytes
+  asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+// the same with a count known at run time (the same in all lanes of a wavefront), 0 .. 47
+template <int N>
+__device__ __forceinline__ void wait_younger_dispatch(int n) {
+  if constexpr (N >= 47) {
+    asm volatile("s_waitcnt vmcnt(47)" ::: "memory");
+  } else {
+    if (n <= N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+    else wait_younger_dispatch<N + 1>(n);
+  }
+}
+__device__ __forceinline__ void wait_younger_n(int n) {
+  wait_younger_dispatch<0>(__builtin_amdgcn_readfirstlane(n < 0 ? 0 : n));
+}
+template <int N>
+__device__ __forceinline__ void wait_younger() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// the wait, with the values it makes usable
+template <int N>
+__device__ __forceinline__ void wait_for(pv4f &a, pv4f &b) {
+  asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_for(float &a) {
+  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_for(unsigned &a) {
+  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(N) : "memory");
+}
+
 // Entry of a panel kernel: the workgroup's XCD and its rank there.  false: more than 32 workgroups on this
 // XCD (abort word set).
 struct PanelWho {

@@ -151,6 +151,30 @@ def test_backward_panel_equals_multi_launch_to_rounding(twins, pkg, B, H, act, d
     assert_close(a["dbeta"], b["dbeta"], 1e-4, "dbeta", floor=1.0)
 
 
+ALL_ACTS = ["LINEAR", "RELU", "LEAKY_RELU", "ELU", "SELU", "ISRLU", "SIGMOID", "TANH"]
+
+
+@pytest.mark.parametrize("act", ALL_ACTS)
+@pytest.mark.parametrize("B,per_element", [(2048, False), (2048, True), (4096, False), (4096, True)])
+def test_every_backward_panel_kernel_variant(twins, pkg, B, per_element, act):
+    """The backward panel kernel issues its loads as explicit instructions behind explicit waits, which the
+    compiler cannot check: every compiled variant (activation x rows per thread x with / without the per-element
+    mask stream) is therefore run against the multi-launch kernels, over several panels per XCD."""
+    panel, plain = twins
+    H = 1536 if B == 2048 else 1024  # 3 and 2 panels of 64 columns per XCD (4 with the 32-column variant)
+    d = make(B, H, B + len(act))
+    drop = "BERNOULLI_INVERTED" if per_element else "NONE"
+    _, desc, mask, st = run_fwd(plain, pkg, d, act, drop, per_element, False)
+    a = run_bwd(panel, pkg, d, desc, mask, st)
+    b = run_bwd(plain, pkg, d, desc, mask, st)
+    assert_close(a["dx"], b["dx"], 1e-4, f"dX [{B}x{H}] {act}", floor=1.0)
+    assert_close(a["dgamma"], b["dgamma"], 1e-4, "dgamma", floor=1.0)
+    assert_close(a["dbeta"], b["dbeta"], 1e-4, "dbeta", floor=1.0)
+    again = run_bwd(panel, pkg, d, desc, mask, st)
+    for k in a:
+        assert np.array_equal(a[k], again[k]), f"{k}: not reproducible"
+
+
 def test_backward_panel_against_float64(twins, pkg):
     """4096 x 1024, batch renormalization + ELU: dX, dgamma, dbeta from the closed form in float64, and the
     invariant that r-corrected batch normalization removes the column mean of dX."""
