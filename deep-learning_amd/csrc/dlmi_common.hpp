@@ -145,6 +145,8 @@ int panel_check(dlmi_ctx *ctx);
 // after the stream's work has completed, the cross-stream ordering of panel launches forgets it.
 void panel_release_stream(dlmi_ctx *ctx);
 size_t panel_scratch_bytes(size_t H);
+size_t panel_db_offset(size_t H);        // where the backward kernel's bias-gradient partials start in the scratch
+size_t panel_scratch_bytes_db(size_t H);  // scratch of a backward launch that also leaves those partials
 // Narrow layers on a mini-batch (fc_small.hip).  narrow_fc_fwd: Z = X W^T + bias and, with Q != nullptr,
 // Q = softmax(Z), one launch; call only when narrow_fc_fwd_eligible.  narrow_dw_try: dW and db in one launch;
 // returns 1 when launched, 0 when the shape does not qualify, < 0 on failure.

@@ -995,7 +995,7 @@ size_t norm_scratch_bytes(dlmi_ctx const *ctx, size_t H) {
   size_t const apply_blocks = static_cast<size_t>(ctx->num_cu) * ctx->tune.apply_bwd_blocks_per_cu;
   size_t const multi = 3 * sizeof(float) * (blocks * 1024 + 2 * H) + round_up(3 * H * sizeof(float), 256) + 4096 +
                        sizeof(float) * (apply_blocks * 1024 + H) + 256;
-  size_t const panel = panel_scratch_bytes(H);
+  size_t const panel = panel_scratch_bytes_db(H);
   return multi > panel ? multi : panel;
 }
 static int ctx_scratch(dlmi_ctx *ctx, size_t H, ScratchView *v) {
@@ -1108,7 +1108,18 @@ static int run_bwd(dlmi_ctx *ctx, ScratchView const &sv, size_t B, size_t H, Bwd
   auto then_db = [&](int took) { return took < 0 ? took : (c.db != nullptr ? column_sums(ctx, B, H, c.dX, c.db, c.db_accumulate ? 1 : 0) : DLMI_OK); };
   if (int const took = small_bwd_try(ctx, B, H, c); took != 0) return then_db(took);
   // a few thousand rows, H a multiple of 512: one launch that reads dY and x once
-  if (int const took = panel_bwd_try(ctx, B, H, c, vec4, sv.data, sv.data_bytes); took != 0) return then_db(took);
+  float *panel_db = nullptr;
+  unsigned panel_db_rows = 0;
+  if (int const took = panel_bwd_try(ctx, B, H, c, vec4, sv.data, sv.data_bytes, &panel_db, &panel_db_rows); took != 0) {
+    if (took < 0 || panel_db == nullptr) return then_db(took);
+    // the kernel left one row of column sums of dX per workgroup rank: the bias gradient is their sum
+    int const ftx = finalize_tx_log2(panel_db_rows);
+    dim3 const fgrid(static_cast<unsigned>(dlmi_ceil_div(H / 4, size_t(1) << ftx)));
+    hipLaunchKernelGGL(k_colsum_finalize<4>, fgrid, dim3(kBlock), 0, ctx->stream, panel_db, panel_db_rows, H, ftx, c.db,
+                       c.db_accumulate ? 1 : 0);
+    DLMI_LAUNCH_CHECK(ctx, "k_colsum_finalize");
+    return DLMI_OK;
+  }
   ColGeom g;
   bool const fold = !c.xhat_given && c.dmean == nullptr && c.dstd == nullptr &&
                     fold_geometry(ctx, B, H, vec4, 3, sv.data_bytes, &g);

@@ -28,6 +28,7 @@ struct PanelBwdArgs {
   int drop_mode, drop_bwd_masked, accumulate;
   PanelSync sync;
   float *part;  // [xcd][panel][rank][3][kP]
+  float *db_part;  // optional [rank][H]: column sums of the dX rows each workgroup stores (the bias gradient's partials)
 };
 
 // dn of one element, dropout mode at run time (bwd_dn of the multi-launch path, same operations)
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
       coef[2][c] = dm * a.batch_scale;
     }
     __syncthreads();
-    pv4f mu, c1, c2, c3;
+    pv4f mu, c1, c2, c3, colsum = {0, 0, 0, 0};
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       mu[e] = cst[0][p * kP + tx * 4 + e];
@@ -263,18 +264,46 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
       c2[e] = coef[1][tx * 4 + e];
       c3[e] = coef[2][tx * 4 + e];
     }
+    // (the column sums of dX only where they are asked for: one more addition per element)
+    auto apply = [&](auto with_sums) {
 #pragma unroll
-    for (int i = 0; i < RPT; ++i) {
-      pv4f out;
+      for (int i = 0; i < RPT; ++i) {
+        pv4f out;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float dx = s.g[i][e] * c1[e] + (s.x[i][e] - mu[e]) * c2[e] + c3[e];
-        if constexpr (EXTRA) {
-          if (a.accumulate) dx += old[i][e];
+        for (int e = 0; e < 4; ++e) {
+          float dx = s.g[i][e] * c1[e] + (s.x[i][e] - mu[e]) * c2[e] + c3[e];
+          if constexpr (EXTRA) {
+            if (a.accumulate) dx += old[i][e];
+          }
+          out[e] = dx;
+          if constexpr (decltype(with_sums)::value) colsum[e] += dx;
         }
-        out[e] = dx;
+        __builtin_nontemporal_store(out, reinterpret_cast<pv4f *>(a.dX + off0 + static_cast<size_t>(i) * kTY * a.H));
       }
-      __builtin_nontemporal_store(out, reinterpret_cast<pv4f *>(a.dX + off0 + static_cast<size_t>(i) * kTY * a.H));
+    };
+    if (a.db_part != nullptr)
+      apply(std::true_type{});
+    else
+      apply(std::false_type{});
+    if (a.db_part != nullptr) {
+      // column sums of this workgroup's rows of dX, in a fixed order: the rows of a wavefront by lane exchange,
+      // the eight wavefronts through LDS (sh is free: publish's readers are two barriers back)
+#pragma unroll
+      for (int m = kCG; m < 64; m <<= 1) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) colsum[e] += __shfl_xor(colsum[e], m);
+      }
+      if ((threadIdx.x & 63u) < static_cast<unsigned>(kCG)) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sh[0][threadIdx.x / 64][tx * 4 + e] = colsum[e];
+      }
+      __syncthreads();
+      if (threadIdx.x < kP) {
+        float t = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kPanelThreads / 64; ++w) t += sh[0][w][threadIdx.x];
+        a.db_part[static_cast<size_t>(who.rank) * a.H + col + threadIdx.x] = t;
+      }
     }
   };
 
@@ -347,15 +376,16 @@ void launch_bwd(dlmi_ctx *ctx, PanelBwdArgs const &a) {
 
 }  // namespace
 
-int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4, void *scratch, size_t scratch_bytes) {
+int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4, void *scratch, size_t scratch_bytes,
+                  float **db_partials, unsigned *db_rows) {
   if (!ctx->panel_ok || !vec4 || c.xhat_given || c.dmean != nullptr || c.dstd != nullptr) return 0;
   if (H % 512 != 0 || H / kPanelXcds > static_cast<size_t>(kPanelMaxCols)) return 0;  // the per-unit constants of an XCD's columns live in LDS
   // 8192 rows: four panels of x and dn only fit the registers at 32 columns per panel, and rows cut into
   // 128-byte pieces stream slower than the multi-launch kernels (measured 113 us against 108 us at 8192 x 4096)
   // 1024 rows: no faster than the multi-launch pair in isolation (15 us both) and slower inside a step, where a
   // launch that needs every CU at once cannot start into the tail of the kernel before it
-  if (B != 2048 && B != 4096) return 0;
   bool const extra = c.accumulate || c.drop_mode == kDropElem;
+  if (B != 2048 && B != 4096 && !(B == 8192 && !extra)) return 0;
   if (c.drop_mode == kDropElem && (reinterpret_cast<uintptr_t>(c.mask) & 3u) != 0) return 0;
   // the caller's scratch (the context's block, already reserved, or the fixed array of the entry point that
   // allocates nothing): too small for the chunk partials means the multi-launch kernels
@@ -369,6 +399,15 @@ int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4
   a.drop_mode = c.drop_mode; a.drop_bwd_masked = c.drop_bwd_masked; a.accumulate = c.accumulate ? 1 : 0;
   a.sync = panel_sync_of(ctx);
   a.part = static_cast<float *>(scratch);
+  // the bias gradient's partials behind the chunk partials, where the caller asked for them and they fit: one row of
+  // column sums per workgroup rank, added up by the caller's small second launch.  (dX accumulating: the sums must be
+  // those of what ends up in dX, a pass over it follows instead.)
+  size_t const db_offset = panel_db_offset(H);
+  bool const db_here = db_partials != nullptr && c.db != nullptr && !c.accumulate &&
+                       panel_scratch_bytes_db(H) <= scratch_bytes;
+  a.db_part = db_here ? reinterpret_cast<float *>(static_cast<char *>(scratch) + db_offset) : nullptr;
+  if (db_partials != nullptr) *db_partials = a.db_part;
+  if (db_rows != nullptr) *db_rows = static_cast<unsigned>(kPanelRanks);
   rc = panel_admit(ctx);
   if (rc <= 0) return rc;
   // rows per workgroup = B / 32 = RPT * 2048 / P
@@ -381,6 +420,7 @@ int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4
     } else {
       switch (B) {
         case 2048: launch_bwd<ACT, 64, 2, false>(ctx, a); break;
+        case 8192: launch_bwd<ACT, 32, 4, false>(ctx, a); break;
         default: launch_bwd<ACT, 64, 4, false>(ctx, a); break;  // 4096 rows
       }
     }

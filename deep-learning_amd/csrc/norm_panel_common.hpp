@@ -93,18 +93,69 @@ __device__ __forceinline__ void issue_load(float &dst, float const *p) {
 __device__ __forceinline__ void issue_load(unsigned &dst, uint8_t const *p) {  // four mask bytes
   asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
 }
-// the same with a count known at run time (the same in all lanes of a wavefront), 0 .. 47
-template <int N>
-__device__ __forceinline__ void wait_younger_dispatch(int n) {
-  if constexpr (N >= 47) {
-    asm volatile("s_waitcnt vmcnt(47)" ::: "memory");
-  } else {
-    if (n <= N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-    else wait_younger_dispatch<N + 1>(n);
-  }
-}
+// the same with a count known at run time (the same in all lanes of a wavefront), clamped to 0 .. 47: a jump into a
+// table of 48 waits, 8 bytes of code each (a chain of compares would cost several scalar instructions per
+// candidate and a kilobyte of code per wait, and these kernels hold dozens of them)
 __device__ __forceinline__ void wait_younger_n(int n) {
-  wait_younger_dispatch<0>(__builtin_amdgcn_readfirstlane(n < 0 ? 0 : n));
+  int t = __builtin_amdgcn_readfirstlane(n < 0 ? 0 : (n > 47 ? 47 : n));
+  asm volatile("s_getpc_b64 vcc\n"            // the address of the next instruction; the table starts 20 bytes
+               "s_lshl_b32 %0, %0, 3\n"       // (five 4-byte instructions) after it
+               "s_add_u32 %0, %0, 20\n"
+               "s_add_u32 vcc_lo, vcc_lo, %0\n"
+               "s_addc_u32 vcc_hi, vcc_hi, 0\n"
+               "s_setpc_b64 vcc\n"
+               "s_waitcnt vmcnt(0)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(1)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(2)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(3)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(4)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(5)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(6)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(7)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(8)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(9)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(10)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(11)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(12)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(13)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(14)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(15)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(16)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(17)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(18)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(19)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(20)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(21)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(22)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(23)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(24)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(25)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(26)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(27)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(28)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(29)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(30)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(31)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(32)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(33)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(34)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(35)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(36)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(37)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(38)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(39)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(40)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(41)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(42)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(43)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(44)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(45)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(46)\n s_branch .Lwait_done_%=\n"
+               "s_waitcnt vmcnt(47)\n s_branch .Lwait_done_%=\n"
+               ".Lwait_done_%=:\n"
+               : "+s"(t)
+               :
+               : "vcc", "scc", "memory");
 }
 template <int N>
 __device__ __forceinline__ void wait_younger() {

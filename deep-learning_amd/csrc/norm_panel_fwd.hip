@@ -343,6 +343,8 @@ int panel_check(dlmi_ctx *ctx) {
 }
 
 size_t panel_scratch_bytes(size_t H) { return static_cast<size_t>(kPanelRanks) * 3 * H * sizeof(float) + 4096; }
+size_t panel_db_offset(size_t H) { return (panel_scratch_bytes(H) + 255) & ~static_cast<size_t>(255); }
+size_t panel_scratch_bytes_db(size_t H) { return panel_db_offset(H) + static_cast<size_t>(kPanelRanks) * H * sizeof(float); }
 
 int panel_fwd_try(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c, bool vec4, void *scratch, size_t scratch_bytes) {
   if (!ctx->panel_ok || !vec4 || c.partial_in != nullptr || c.xhat != nullptr || c.nrm != nullptr || c.y == nullptr) return 0;

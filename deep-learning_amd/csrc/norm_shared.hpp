@@ -132,7 +132,10 @@ struct BwdCall {
 // launched that way, 0 when the shape or the context does not qualify (the caller goes on with the
 // multi-launch path), a negative DLMI_E_* code on failure.
 int panel_fwd_try(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c, bool vec4, void *scratch, size_t scratch_bytes);
-int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4, void *scratch, size_t scratch_bytes);
+// db_partials / db_rows (optional): receive the [db_rows][H] partial column sums of dX the kernel left for c.db, or
+// nullptr when it left none
+int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4, void *scratch, size_t scratch_bytes,
+                  float **db_partials = nullptr, unsigned *db_rows = nullptr);
 
 
 // The small-batch kernels (norm_small.hip): one launch per direction for at most 256 rows and 2^20 elements.

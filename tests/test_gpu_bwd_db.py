@@ -2,8 +2,9 @@
 pass that writes dX.  dgamma and dbeta must be bit-identical to the plain call and dX equal to the last place or
 two (the two apply kernels are separate instantiations, in which the compiler may contract the same expression
 into fused multiply-adds differently); db must be the column sums of the dX this call stored (float32 sums in another order than numpy's: compared with the float64 sums to the rounding of B terms),
-on every path: multi-launch (the by-product), tall tensors, the single-launch panel and mini-batch kernels and
-ragged widths (a pass over dX after them), with and without accumulation."""
+on every path: multi-launch and single-launch panel kernels (the by-product: per-block / per-workgroup partial sums and
+one small launch), tall tensors, mini-batch kernels and ragged widths (a pass over dX after them), with and without
+accumulation."""
 import numpy as np
 import pytest
 import torch
@@ -16,7 +17,10 @@ pytestmark = pytest.mark.gpu
 CASES = [  # B, H, activation, dropout, per element
     (8192, 512, "ELU", "NONE", False),        # multi-launch, folded finalize
     (65536, 256, "LEAKY_RELU", "NONE", False),  # tall: finalize kernels
-    (2048, 1024, "SELU", "NONE", False),      # single-launch panel kernel, then a pass over dX
+    (2048, 1024, "SELU", "NONE", False),      # single-launch panel kernel, 64-column panels, 2 rows per thread
+    (4096, 1536, "TANH", "NONE", False),      # ... 4 rows per thread, 3 panels per XCD
+    (8192, 1024, "SIGMOID", "NONE", False),   # ... 32-column panels
+    (4096, 1024, "LEAKY_RELU", "BERNOULLI_INVERTED", True),  # ... with the per-element mask stream
     (128, 512, "RELU", "NONE", False),        # mini-batch kernel
     (1000, 250, "TANH", "NONE", False),       # ragged width: no 16-byte path
     (3000, 768, "ISRLU", "BERNOULLI_INVERTED", True),
