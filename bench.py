@@ -56,14 +56,14 @@ LAYER_WORKLOADS = {
 MIB = 1024.0 * 1024.0
 TRAFFIC_PROFILE = "profiles/hbm_traffic_pmc.md"
 MEASURED_TRAFFIC_BYTES = {
-    "c3": {"gemm": (898.0 + 897.3 + 832.8) / 3.0 * MIB, "norm_act": 902.0 * MIB},
-    "c2": {"norm_act": 326.9 * MIB},
+    "c3": {"gemm": (898.0 + 897.3 + 832.8) / 3.0 * MIB, "norm_act": (259.1 + 388.4) * MIB},
+    "c2": {"norm_act": 326.8 * MIB},
     "c4": {"gemm": (72.1 + 72.1 + 64.1) / 3.0 * MIB, "norm_act": 73.6 * MIB},
     "c5": {"gemm": (132.2 + 132.5 + 144.1 + 16.3) / 3.0 * MIB, "norm_act": 516.5 * MIB},
 }
 TRAFFIC_SOURCES = ("gemm_f32_mfma.hip", "norm_kernels.hip", "norm_panel_fwd.hip", "norm_panel_bwd.hip",
                    "norm_panel_common.hpp", "norm_shared.hpp", "activations.hpp")
-TRAFFIC_SOURCES_SHA256 = "3a086e90370083fb9b35ec6547a74917f997a53f65c74f683e965161a5b6f524"
+TRAFFIC_SOURCES_SHA256 = "d3d6757ee6e5be7f050e0cc55b5f250f5d3fd338bede9aacc1285c2ecccab2b5"
 
 
 def traffic_sources_digest():

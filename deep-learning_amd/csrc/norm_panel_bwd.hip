@@ -5,10 +5,12 @@
 //
 // Geometry: 512 threads = P/4 column groups of 4 units x 2048/P rows; a workgroup owns B/32 = RPT * 2048/P rows
 // and walks panels of P columns: P = 64 (256 B per row) while five panels of x and dn fit the registers, P = 32
-// for 4096 rows with a per-element mask.  B in {2048, 4096}, H a multiple of 512 and at most 8 * kPanelMaxCols.  (Wider panels stream
-// faster - the forward kernel's 128 columns reach 5.1 TB/s of actual traffic, 64 columns 3.7 TB/s - but the
-// backward pass holds two values per element; the kernel still beats the multi-launch pair because it moves
-// 12 instead of 20 bytes per element.)
+// for 4096 rows with a per-element mask or an accumulating dX and for 8192 rows.  B in {2048, 4096, 8192}, H a
+// multiple of 512 and at most 8 * kPanelMaxCols.  (32-, 64- and 128-column panels stream alike; the backward pass
+// holds two values per element, so narrower panels buy more of them in flight.  The kernel beats the multi-launch
+// pair because it moves 12 instead of 20 bytes per element.)
+// On request the kernel also leaves the column sums of the dX rows each workgroup stored (the bias gradient of the
+// layer below the normalization, update_derivative_fwp_st.cpp:283-302, as 32 partial rows for a small second launch).
 #include <type_traits>
 
 #include "norm_panel_common.hpp"
@@ -380,8 +382,7 @@ int panel_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c, bool vec4
                   float **db_partials, unsigned *db_rows) {
   if (!ctx->panel_ok || !vec4 || c.xhat_given || c.dmean != nullptr || c.dstd != nullptr) return 0;
   if (H % 512 != 0 || H / kPanelXcds > static_cast<size_t>(kPanelMaxCols)) return 0;  // the per-unit constants of an XCD's columns live in LDS
-  // 8192 rows: four panels of x and dn only fit the registers at 32 columns per panel, and rows cut into
-  // 128-byte pieces stream slower than the multi-launch kernels (measured 113 us against 108 us at 8192 x 4096)
+  // 8192 rows: 32-column panels, and only without a mask stream or an accumulating dX (registers)
   // 1024 rows: no faster than the multi-launch pair in isolation (15 us both) and slower inside a step, where a
   // launch that needs every CU at once cannot start into the tail of the kernel before it
   bool const extra = c.accumulate || c.drop_mode == kDropElem;

@@ -1,4 +1,4 @@
-"""The single-launch (column panel) normalization kernels (forward: 1024 - 8192 rows, backward: 2048 and 4096 rows; the
+"""The single-launch (column panel) normalization kernels (forward: 1024 - 8192 rows, backward: 2048 - 8192 rows; the
 other backward cases below run the multi-launch kernels in both contexts) against the multi-launch path of the same library
 and against the oracle: same per-unit arithmetic, the batch summed in 32 chunks instead of <= 16, so the two
 paths agree to rounding of the column sums (1e-6 relative on the statistics), not bit for bit.  A context
