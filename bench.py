@@ -63,7 +63,7 @@ MEASURED_TRAFFIC_BYTES = {
 }
 TRAFFIC_SOURCES = ("gemm_f32_mfma.hip", "norm_kernels.hip", "norm_panel_fwd.hip", "norm_panel_bwd.hip",
                    "norm_panel_common.hpp", "norm_shared.hpp", "activations.hpp")
-TRAFFIC_SOURCES_SHA256 = "d3d6757ee6e5be7f050e0cc55b5f250f5d3fd338bede9aacc1285c2ecccab2b5"
+TRAFFIC_SOURCES_SHA256 = "08e360334278730f11381c8f34d1b06c3201e0d58c2ffbb844ac6cda7955bf80"
 
 
 def traffic_sources_digest():

@@ -33,6 +33,7 @@ struct dlmi_tuning {
   size_t fold_fwd_epilogue_max_elements = size_t(1) << 22;
   int fc_narrow = 1;              // layers of at most 16 units on a mini-batch run the narrow-layer kernels (fc_small.hip)
   int norm_small = 1;             // mini-batches (at most 256 rows, 2^20 elements) run the one-launch small-batch kernels
+  int narrow_dx_fused = 1;        // ... which also form dY = dZn . Wn below a layer of at most 16 units themselves
 };
 
 struct dlmi_ctx {
@@ -161,6 +162,13 @@ int fused_bwd_from_slices(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, 
                           float const *gamma, float const *beta, uint8_t const *mask, float const *mean,
                           float const *stdv, float const *r, float const *d, float const *slices, unsigned nslices,
                           float *dgamma, float *dbeta, float *dX);
+// The same with dY = dZn [B][Hn] . Wn [Hn][H] of a narrow layer above (Hn <= fused_bwd_narrow_max()), formed inside
+// the small-batch kernel: no product launch at all.
+unsigned fused_bwd_narrow_max();
+int fused_bwd_from_narrow(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
+                          float const *gamma, float const *beta, uint8_t const *mask, float const *mean,
+                          float const *stdv, float const *r, float const *d, float const *dZn, float const *Wn,
+                          size_t Hn, float *dgamma, float *dbeta, float *dX);
 }  // namespace dlmi
 
 inline bool dlmi_aligned16(void const *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -851,6 +851,9 @@ int dlmi_fc_bwd_dx_norm_act_bwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size
   // a mini-batch: the normalization kernel owns whole columns and adds the K slices of dY = dZn . Wn itself
   unsigned slices = 0;
   bool const defer = small_norm_eligible(ctx, B, H);
+  // ... and below a narrow layer (an output layer of a few units) it forms dY itself: no product launch
+  if (defer && Hn <= fused_bwd_narrow_max() && ctx->tune.narrow_dx_fused && x && gamma && beta && mean && stdv && r && d && dgamma && dbeta)
+    return fused_bwd_from_narrow(ctx, desc, B, H, x, gamma, beta, mask, mean, stdv, r, d, dZn, Wn, Hn, dgamma, dbeta, dX);
   int rc = gemm<true, false>(ctx, B, H, Hn, dZn, Hn, Wn, H, dX, nullptr, 0, nullptr, defer ? &slices : nullptr);
   if (rc != DLMI_OK) return rc;
   if (slices != 0)

@@ -1289,6 +1289,28 @@ int fused_bwd_from_slices(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, 
   return took < 0 ? took : DLMI_OK;
 }
 
+unsigned fused_bwd_narrow_max() { return kNarrowMaxUnits; }
+
+int fused_bwd_from_narrow(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,
+                          float const *gamma, float const *beta, uint8_t const *mask, float const *mean,
+                          float const *stdv, float const *r, float const *d, float const *dZn, float const *Wn,
+                          size_t Hn, float *dgamma, float *dbeta, float *dX) {
+  int rc = check_desc(ctx, desc, mask);
+  if (rc != DLMI_OK) return rc;
+  DLMI_REQUIRE(ctx, x && gamma && beta && mean && stdv && r && d && dZn && Wn && dgamma && dbeta && dX, "null pointer");
+  DLMI_REQUIRE(ctx, Hn > 0 && Hn <= kNarrowMaxUnits, "not a narrow layer");
+  BwdCall c;
+  c.act = desc->act; c.xhat_given = false; c.drop_mode = drop_mode_of(desc);
+  c.drop_bwd_masked = desc->dropout_bwd == DLMI_DROP_BWD_MASKED ? 1 : 0;
+  c.drop_scale = drop_scale_of(desc);
+  c.x = x; c.gamma = gamma; c.beta = beta; c.mean = mean; c.stdv = stdv; c.r = r; c.d = d; c.xhat = nullptr;
+  c.dY = nullptr; c.mask = mask; c.narrow_dz = dZn; c.narrow_w = Wn; c.narrow_h = static_cast<unsigned>(Hn);
+  c.dgamma = dgamma; c.dbeta = dbeta; c.dmean = nullptr; c.dstd = nullptr; c.dX = dX;
+  int const took = small_bwd_try(ctx, B, H, c);
+  if (took == 0) return dlmi_fail(ctx, DLMI_E_INVALID, "fused_bwd_from_narrow: not a small-batch shape");
+  return took < 0 ? took : DLMI_OK;
+}
+
 int column_sums(dlmi_ctx *ctx, size_t B, size_t H, float const *x, float *out, int accumulate) {
   if (int const took = small_colsum_try(ctx, B, H, x, out, accumulate); took != 0) return took < 0 ? took : DLMI_OK;
   ScratchView sv{};

@@ -126,7 +126,13 @@ struct BwdCall {
   // the small-batch kernel (the only one that takes them); dY is unused then
   float const *dy_slices = nullptr;
   unsigned nslices = 0;
+  // dY not formed yet: it is the product dZn . Wn of a NARROW layer above (narrow_h <= kNarrowMaxUnits units:
+  // narrow_dz [B][narrow_h], narrow_w [narrow_h][H]), formed by the small-batch kernel itself, unit after unit
+  // (Backward_Pass__FC__Loop, bwp_st.cpp:1009-1045: the sum over the layer's units, here in ascending order); dY is unused then
+  float const *narrow_dz = nullptr, *narrow_w = nullptr;
+  unsigned narrow_h = 0;
 };
+constexpr unsigned kNarrowMaxUnits = 16;
 
 // The single-launch panel kernels (norm_panel_fwd.hip, norm_panel_bwd.hip).  Return 1 when the call was
 // launched that way, 0 when the shape or the context does not qualify (the caller goes on with the

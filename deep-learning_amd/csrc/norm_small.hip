@@ -120,6 +120,8 @@ struct SmallBwdArgs {
   float const *x, *dY, *gamma, *beta, *mean, *stdv, *r, *d;
   float const *dy_slices;  // [nslices][B][H] whose sum is dY, or nullptr
   unsigned nslices;
+  float const *narrow_dz, *narrow_w;  // dY = narrow_dz [B][narrow_h] . narrow_w [narrow_h][H], or nullptr
+  unsigned narrow_h;
   uint8_t const *mask;
   float *dgamma, *dbeta, *dX;
   size_t B, H;
@@ -130,9 +132,21 @@ struct SmallBwdArgs {
 template <int ACT, int RPT>
 __global__ __launch_bounds__(kSmallThreads) void k_small_bwd(SmallBwdArgs a) {
   __shared__ float red[3][kSmallGroups][kSmallCols];
+  __shared__ float ndz[kSmallMaxRows * kNarrowMaxUnits];  // the narrow layer's dZ, all rows
   int const c = threadIdx.x % kSmallCols, rg = threadIdx.x / kSmallCols;
   size_t const col = static_cast<size_t>(blockIdx.x) * kSmallCols + c;
   bool const live = col < a.H;
+  // (all of a thread's loads are asked for before the first one is used: one memory latency, not one per piece)
+  constexpr int kNdzPerThread = static_cast<int>(kSmallMaxRows * kNarrowMaxUnits / kSmallThreads);
+  float ndz_in[kNdzPerThread];
+  unsigned const ndz_count = a.narrow_dz != nullptr ? static_cast<unsigned>(a.B) * a.narrow_h : 0u;
+  if (a.narrow_dz != nullptr) {
+#pragma unroll
+    for (int k = 0; k < kNdzPerThread; ++k) {
+      unsigned const i = threadIdx.x + static_cast<unsigned>(k) * kSmallThreads;
+      ndz_in[k] = i < ndz_count ? a.narrow_dz[i] : 0.0f;
+    }
+  }
   float mu = 0.0f, sd = 1.0f, rr = 1.0f, dd = 0.0f, ga = 1.0f, be = 0.0f;
   uint8_t mk = 1;
   if (live) {
@@ -166,11 +180,32 @@ __global__ __launch_bounds__(kSmallThreads) void k_small_bwd(SmallBwdArgs a) {
     mv[i] = mk;
     if (ok[i]) {
       xv[i] = a.x[off];
-      if (a.dy_slices == nullptr) dy[i] = a.dY[off];
+      if (a.dy_slices == nullptr && a.narrow_dz == nullptr) dy[i] = a.dY[off];
       if (a.drop_mode == kDropElem) mv[i] = a.mask[off];
     }
   }
-  if (a.dy_slices != nullptr) {
+  if (a.narrow_dz != nullptr) {
+    // this column of the narrow layer's weights, then one chain of multiply-adds per row, units ascending
+    float w[kNarrowMaxUnits];
+#pragma unroll
+    for (unsigned u = 0; u < kNarrowMaxUnits; ++u) w[u] = live && u < a.narrow_h ? a.narrow_w[u * a.H + col] : 0.0f;
+#pragma unroll
+    for (int k = 0; k < kNdzPerThread; ++k) {
+      unsigned const i = threadIdx.x + static_cast<unsigned>(k) * kSmallThreads;
+      if (i < ndz_count) ndz[i] = ndz_in[k];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      if (!ok[i]) continue;
+      float const *z = ndz + static_cast<unsigned>(rg + kSmallGroups * i) * a.narrow_h;
+      float t = 0.0f;
+#pragma unroll
+      for (unsigned u = 0; u < kNarrowMaxUnits; ++u)
+        if (u < a.narrow_h) t = fmaf(z[u], w[u], t);
+      dy[i] = t;
+    }
+  } else if (a.dy_slices != nullptr) {
     size_t const plane = a.B * a.H;
     for (unsigned s = 0; s < a.nslices; ++s) {
       float t[RPT];
@@ -290,11 +325,15 @@ int small_fwd_try(dlmi_ctx *ctx, size_t B, size_t H, FwdTrainCall const &c) {
 
 int small_bwd_try(dlmi_ctx *ctx, size_t B, size_t H, BwdCall const &c) {
   if (!small_norm_eligible(ctx, B, H) || c.xhat_given || c.dmean != nullptr || c.dstd != nullptr) {
-    if (c.dy_slices != nullptr) return dlmi_fail(ctx, DLMI_E_INVALID, "small-batch backward: K slices given for a call it cannot take");
+    if (c.dy_slices != nullptr || c.narrow_dz != nullptr)
+      return dlmi_fail(ctx, DLMI_E_INVALID, "small-batch backward: a deferred product given for a call it cannot take");
     return 0;
   }
+  if (c.narrow_dz != nullptr && (c.narrow_h == 0 || c.narrow_h > kNarrowMaxUnits || c.narrow_w == nullptr || c.dy_slices != nullptr))
+    return dlmi_fail(ctx, DLMI_E_INVALID, "small-batch backward: bad narrow product");
   SmallBwdArgs a;
   a.dy_slices = c.dy_slices; a.nslices = c.nslices;
+  a.narrow_dz = c.narrow_dz; a.narrow_w = c.narrow_w; a.narrow_h = c.narrow_h;
   a.x = c.x; a.dY = c.dY; a.gamma = c.gamma; a.beta = c.beta; a.mean = c.mean; a.stdv = c.stdv; a.r = c.r; a.d = c.d;
   a.mask = c.mask; a.dgamma = c.dgamma; a.dbeta = c.dbeta; a.dX = c.dX;
   a.B = B; a.H = H;

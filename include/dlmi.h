@@ -366,8 +366,10 @@ int dlmi_fc_softmax_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const
  * dY = dZn . Wn (Backward_Pass__FC__Loop, bwp_st.cpp:1009-1045; dZn [B,Hn], Wn [Hn][H]), then
  * dlmi_fused_norm_act_bwd on dY (bwp_st.cpp:1177-1209, 1284-1366, 1447-1532), result in dX [B,H]
  * (dgamma, dbeta accumulate).  On a mini-batch (at most 256 rows) whose product runs split over K the
- * normalization kernel adds the K slices itself and dY is never written; otherwise the two calls run
- * one after the other with dX as the buffer between them. */
+ * normalization kernel adds the K slices itself and dY is never written; below a layer of at most 16
+ * units (Hn <= 16, the reference's 10-way output layer) that kernel forms dY itself, one chain of
+ * multiply-adds per element, and no product is launched; otherwise the two calls run one after the other
+ * with dX as the buffer between them. */
 int dlmi_fc_bwd_dx_norm_act_bwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t Hn, size_t H,
                                 float const *dZn, float const *Wn, float const *x, float const *gamma,
                                 float const *beta, uint8_t const *mask, float const *mean, float const *std,

@@ -93,7 +93,11 @@ def test_narrow_weight_and_bias_gradient(twins, pkg, B, K, H):
 
 @pytest.mark.parametrize("B,Hn,H,act,drop", [
     (128, 512, 512, "RELU", "NONE"),                  # runs split over K: the normalization kernel adds the slices
-    (128, 10, 512, "RELU", "NONE"),                   # K = 10: no split, the two steps run one after the other
+    (128, 10, 512, "RELU", "NONE"),                   # a narrow layer above: the normalization kernel forms dY itself
+    (256, 16, 36, "SELU", "BERNOULLI_INVERTED"),      # ... the widest it takes, 8 rows per thread, ragged width
+    (7, 1, 100, "TANH", "NONE"),
+    (33, 3, 8, "LEAKY_RELU", "BERNOULLI"),
+    (128, 17, 512, "RELU", "NONE"),                   # one unit too many: product launch, then the normalization kernel
     (200, 300, 36, "ELU", "BERNOULLI_INVERTED"),
     (256, 1024, 64, "TANH", "BERNOULLI"),
     (512, 256, 256, "SELU", "NONE"),                  # more rows than the small-batch kernels take
