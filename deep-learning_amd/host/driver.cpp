@@ -198,7 +198,7 @@ void Driver::run_batches(Recorded &rec, bool const training) {
       bool ok = hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed) == hipSuccess;
       if (ok) {
         for (size_t i = first; i != end; ++i) one_batch(i, rows_of(i), batch_size_max, resident, training);
-        bool const pass_ok = model.error_count() == before.n_errors;
+        bool const pass_ok = model.join_weight_gradients() && model.error_count() == before.n_errors;
         ok = hipStreamEndCapture(stream, &graph) == hipSuccess && graph != nullptr && pass_ok;
       }
       ok = ok && hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) == hipSuccess;

@@ -59,6 +59,16 @@ struct Model::Impl {
   dlmi_ctx *dw_ctx = nullptr;
   std::vector<hipEvent_t> dz_ready;  // per layer
   hipEvent_t dw_done = nullptr;
+  // The weight gradient of a layer that reads the NETWORK INPUT from rows the caller keeps on the device
+  // (forward_pass_device) is the last product of a training step and nothing of the next step's forward pass
+  // touches what it reads (those rows, the layer's dZ) or writes (its part of the gradient array): the compute
+  // stream does not wait for it at the end of update_derivatives() but where that stops being true
+  // (join_weight_gradients(): before the next seed gradient / backward pass, the optimizer step, a clear or an upload
+  // of the gradient array, any synchronization).  dw_mid: the side stream's products before that last one, which
+  // read layer outputs that the next forward pass overwrites - those the compute stream waits for at once.
+  hipEvent_t dw_mid = nullptr;
+  bool dw_pending = false;          // dw_done is recorded and the compute stream has not waited for it yet
+  bool cur_input_external = false;  // cur_input is the caller's device memory, not an upload slot
   void record_dz_ready(size_t layer) {
     if (dw_ctx != nullptr && layer < dz_ready.size()) (void)hipEventRecord(dz_ready[layer], stream);
   }
@@ -259,6 +269,7 @@ void Model::clear(void) {
   if (impl_->dw_ctx != nullptr) (void)dlmi_ctx_destroy(impl_->dw_ctx);
   for (hipEvent_t e : impl_->dz_ready) (void)hipEventDestroy(e);
   if (impl_->dw_done != nullptr) (void)hipEventDestroy(impl_->dw_done);
+  if (impl_->dw_mid != nullptr) (void)hipEventDestroy(impl_->dw_mid);
   if (impl_->ctx != nullptr) (void)dlmi_ctx_destroy(impl_->ctx);
   hipStream_t const stream = impl_->stream, up_stream = impl_->up_stream, dw_stream = impl_->dw_stream;
   size_t const n_errors = impl_->n_errors;
@@ -321,6 +332,7 @@ Model::PassState Model::pass_state(void) const {
   return PassState{impl_->n_loss_values, impl_->out_batch, impl_->cur_input, impl_->n_errors};
 }
 void Model::restore_pass_state(PassState const &s) {
+  impl_->dw_pending = false;  // (a recording that failed took the side stream's part of it along)
   impl_->n_loss_values = s.n_loss_values;
   impl_->out_batch = s.out_batch;
   impl_->cur_input = s.cur_input;
@@ -330,9 +342,19 @@ size_t Model::error_count(void) const { return impl_->n_errors; }
 // Waits for both streams.  Every read of results (get_out, get_loss, the download_* calls) comes through here,
 // because this is where a single-launch normalization kernel that gave up its bounded wait is reported: the
 // call fails (once) instead of handing out numbers that are not valid.
+bool Model::join_weight_gradients(void) const {
+  if (!impl_->dw_pending) return true;
+  impl_->dw_pending = false;
+  if (!hip_ok(hipStreamWaitEvent(impl_->stream, impl_->dw_done, 0), impl_->err, "join of the weight-gradient stream")) {
+    fail("join of the weight-gradient stream");
+    return false;
+  }
+  return true;
+}
+
 bool Model::synchronize(void) const {
   if (impl_->ctx == nullptr) return false;
-  bool ok = true;
+  bool ok = join_weight_gradients();
   if (impl_->dw_ctx != nullptr && dlmi_ctx_synchronize(impl_->dw_ctx) != DLMI_OK) {
     ok = false;
     fail((std::string("synchronize (weight-gradient stream): ") + dlmi_last_error(impl_->dw_ctx)).c_str());
@@ -393,7 +415,8 @@ bool Model::compile(size_t const n_layers, size_t const number_recurrent_depth_r
     }
     if (side && impl_->dw_stream != nullptr) {
       bool ok = dlmi_ctx_create(&impl_->dw_ctx, 0, impl_->dw_stream) == DLMI_OK &&
-                hipEventCreateWithFlags(&impl_->dw_done, hipEventDisableTiming) == hipSuccess;
+                hipEventCreateWithFlags(&impl_->dw_done, hipEventDisableTiming) == hipSuccess &&
+                hipEventCreateWithFlags(&impl_->dw_mid, hipEventDisableTiming) == hipSuccess;
       impl_->dz_ready.assign(n_layers, nullptr);
       for (size_t i = 0; ok && i < n_layers; ++i)
         ok = hipEventCreateWithFlags(&impl_->dz_ready[i], hipEventDisableTiming) == hipSuccess;
@@ -934,6 +957,7 @@ bool Model::Initialization__LSUV(size_t const n_data_set, real const *const *con
 
 void Model::clear_training_arrays(void) {
   if (impl_->d_dparams == nullptr) return;
+  (void)join_weight_gradients();
   (void)hipMemsetAsync(impl_->d_dparams, 0, total_parameters * sizeof(float), impl_->stream);
   (void)hipMemsetAsync(impl_->d_stats, 0, 2 * sizeof(double), impl_->stream);
   impl_->n_loss_values = 0;
@@ -987,7 +1011,7 @@ bool Model::download_derivatives(void) {
                           hipMemcpyDeviceToHost), impl_->err, "gradient download");
 }
 bool Model::upload_derivatives(void) {
-  return hip_ok(hipMemcpy(impl_->d_dparams, ptr_array_derivatives_parameters, total_parameters * sizeof(float),
+  return synchronize() && hip_ok(hipMemcpy(impl_->d_dparams, ptr_array_derivatives_parameters, total_parameters * sizeof(float),
                           hipMemcpyHostToDevice), impl_->err, "gradient upload");
 }
 bool Model::upload_moving_statistics(void) {
@@ -1072,6 +1096,7 @@ void Model::forward_pass(size_t const B, real const *const *const Xm, long long 
   float const *const d_rows = impl_->slots_upload(impl_->in_rows, B, n_in, Xm, "forward_pass: input upload");
   if (d_rows == nullptr) { std::string const why = impl_->err; fail(why.c_str()); return; }
   impl_->cur_input = d_rows;
+  impl_->cur_input_external = false;
   forward_layers(B, static_cast<size_t>(out_idx));
 }
 
@@ -1079,6 +1104,7 @@ void Model::forward_pass_device(size_t const B, float const *d_inputs) {
   if (ptr_array_layers == nullptr || d_inputs == nullptr) { fail("forward_pass_device: model not compiled or null input"); return; }
   if (B == 0 || B > impl_->allocated_batch) { fail("forward_pass_device: batch size exceeds update_mem_batch_size()"); return; }
   impl_->cur_input = d_inputs;
+  impl_->cur_input_external = true;
   forward_layers(B, total_layers);
 }
 
@@ -1290,6 +1316,7 @@ void Model::compute_loss(size_t const B, real const *const *const Ym) { compute_
 void Model::compute_loss_device(size_t const B, float const *d_targets) { compute_error_device(B, d_targets); }
 
 void Model::seed_error(size_t const B, float const *d_targets) {
+  if (!join_weight_gradients()) return;  // the output layer's dZ is about to be overwritten
   Layer &o = ptr_array_layers[total_layers - 1];
   if (o.type_activation_function == ACTIVATION::SOFTMAX) {
     if (type_loss_function != LOSS_FN::CROSS_ENTROPY || type_accuracy_function != ACCU_FN::CROSS_ENTROPY) {
@@ -1436,6 +1463,7 @@ bool Model::Use__Dropout__Bernoulli__Inverted(void) const {
 
 void Model::backward_pass(size_t const B) {
   if (ptr_array_layers == nullptr || B == 0 || B > impl_->allocated_batch) { fail("backward_pass: bad argument"); return; }
+  if (!join_weight_gradients()) return;  // every layer's dZ is about to be overwritten
   dlmi_ctx *ctx = impl_->ctx;
   // bwp_st.cpp:106-183: from the output layer down to layer 1.  Each plain layer
   // turns the gradient with respect to its outputs (left in its error buffer by
@@ -1574,8 +1602,10 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
   }
   // from the last layer down: the order in which the backward pass finishes their gradients (every layer adds
   // into its own part of the gradient array, so the order does not change the sums)
+  if (!join_weight_gradients()) return;
   bool const side = impl_->dw_ctx != nullptr;
   bool joined = true;  // nothing on the side stream yet
+  bool mid_recorded = false, deferred = false;
   hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
   if (side && hipStreamIsCapturing(impl_->stream, &capture) != hipSuccess) (void)hipGetLastError();
   bool const recording = capture != hipStreamCaptureStatusNone;
@@ -1608,6 +1638,22 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
       on_stream.push_back(dlmi_dw_problem{B, K, l->n_out, in, l->d_errors, impl_->d_dparams + l->first_connection_index, db});
       continue;
     }
+    // the product that reads the caller's input rows may outlast this call (see dw_mid): what was launched
+    // beside the chain before it is marked, and only that is waited for below
+    if (in == impl_->cur_input && impl_->cur_input_external && !deferred) {
+      if (!joined) {
+        if (!hip_ok(hipEventRecord(impl_->dw_mid, impl_->dw_stream), impl_->err, "update_derivatives: mark")) {
+          fail("update_derivatives: mark");
+          break;
+        }
+        mid_recorded = true;
+      }
+      deferred = true;
+    } else if (deferred) {
+      // (a layer order in which another product follows the deferred one: wait for all of them as usual)
+      deferred = false;
+      mid_recorded = false;
+    }
     if (dlmi_fc_bwd_dw(impl_->dw_ctx, B, K, l->n_out, in, l->d_errors,
                        impl_->d_dparams + l->first_connection_index, db, 1) != DLMI_OK) {
       fail("update_derivatives: dlmi_fc_bwd_dw");
@@ -1620,9 +1666,16 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
     fail("update_derivatives: dlmi_fc_bwd_dw_grouped");
   // whatever the compute stream does next (the optimizer step, the next forward pass over the same buffers)
   // comes after the last weight gradient
-  if (!joined && (!hip_ok(hipEventRecord(impl_->dw_done, impl_->dw_stream), impl_->err, "update_derivatives: join") ||
-               !hip_ok(hipStreamWaitEvent(impl_->stream, impl_->dw_done, 0), impl_->err, "update_derivatives: join")))
-    fail("update_derivatives: join");
+  if (!joined) {
+    if (!hip_ok(hipEventRecord(impl_->dw_done, impl_->dw_stream), impl_->err, "update_derivatives: join")) {
+      fail("update_derivatives: join");
+      return;
+    }
+    hipEvent_t const wait_for = deferred ? (mid_recorded ? impl_->dw_mid : nullptr) : impl_->dw_done;
+    if (wait_for != nullptr && !hip_ok(hipStreamWaitEvent(impl_->stream, wait_for, 0), impl_->err, "update_derivatives: join"))
+      fail("update_derivatives: join");
+    impl_->dw_pending = deferred;
+  }
 }
 
 // ---------------------------------------------------------------- optimizer step
@@ -1679,6 +1732,7 @@ real Model::normalized_wd(size_t const batch, size_t const training_size) {
 // adam.cpp:38-54 in float.
 void Model::Update_Parameter(size_t const batch, size_t const training_size) {
   if (impl_->d_params == nullptr) { fail("Update_Parameter: model not compiled"); return; }
+  if (!join_weight_gradients()) return;
   size_t const P = total_parameters;
   Impl &m = *impl_;
   // Every optimizer but iRPROP+ starts by asking the warm-restart schedule for its rate (which may

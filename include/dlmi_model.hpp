@@ -374,6 +374,12 @@ class Model : public Model_State {
   double get_accuracy_sum(void) const; // number of correct arg-max predictions since then
   char const *last_error(void) const;
   bool synchronize(void) const;
+  // No counterpart in the reference.  After update_derivatives() behind forward_pass_device(), the weight
+  // gradient of the layer that reads the network input may still be running on the model's second stream; every
+  // member that reads or overwrites what it uses waits for it by itself.  A caller that records the model's
+  // launches into a HIP graph calls this before it ends the capture (a capture must not end with work forked
+  // off and not joined), and the rows handed to forward_pass_device() must stay unchanged until then.
+  bool join_weight_gradients(void) const;
   // The stream every kernel of this model is launched on (a hipStream_t), and a hash of
   // everything the kernels of one batch take by value or by address (layer settings,
   // hyper-parameters, propagation state, buffer addresses): two batches of the same size

@@ -148,3 +148,41 @@ def test_scratch_that_moves_between_replays_drops_the_recording(lib):
     finally:
         a.close()
         b.close()
+
+
+@pytest.mark.parametrize("widths,max_batch,n", [([20, 32, 24, 5], 16, 50), ([1024, 1024, 512, 10], 256, 600)])
+def test_weight_gradients_beside_the_chain_match_one_stream(lib, widths, max_batch, n):
+    """The weight gradients run on a second stream, and the one of the layer that reads the resident input rows is
+    not waited for until the next pass overwrites what it reads: a twin created with DLMI_DW_STREAM=0 issues every
+    launch on one stream, and parameters, gradients and moving statistics must stay bit-identical epoch after epoch,
+    with plain launches (the wide network's products are large enough to go beside the chain there too) and with
+    recorded mini-batches, with evaluation passes, downloads and an optimizer step between the passes."""
+    import os
+    os.environ["DLMI_DW_STREAM"] = "0"
+    try:
+        one = build(lib, widths, max_batch=max_batch)
+    finally:
+        del os.environ["DLMI_DW_STREAM"]
+    two, rec = build(lib, widths, max_batch=max_batch), build(lib, widths, max_batch=max_batch)
+    X, Y = data(n, widths[0], widths[-1])
+    try:
+        for e in range(5):
+            r1 = one.train_epoch(X, Y, resample_masks=True, record_batches=False)
+            r2 = two.train_epoch(X, Y, resample_masks=True, record_batches=False)
+            r3 = rec.train_epoch(X, Y, resample_masks=True, record_batches=True)
+            assert r2 == r1 and r3[1] == r1[1] and r3[0] == pytest.approx(r1[0], rel=1e-9), f"epoch {e}: {r1} / {r2} / {r3}"
+            p1 = one.get_parameters()
+            assert np.array_equal(p1, two.get_parameters()), f"epoch {e}: parameters (plain launches)"
+            assert np.array_equal(p1, rec.get_parameters()), f"epoch {e}: parameters (recorded)"
+            m1 = one.get_moving()
+            for other in (two, rec):
+                mo = other.get_moving()
+                assert np.array_equal(m1[0], mo[0]) and np.array_equal(m1[1], mo[1]), f"epoch {e}: moving statistics"
+            if e == 2:  # gradients as the last pass left them, before anything clears them
+                assert np.array_equal(one.get_dparams(), two.get_dparams())
+                assert np.array_equal(one.get_dparams(), rec.get_dparams())
+            assert two.evalt(X, Y) == one.evalt(X, Y)
+    finally:
+        one.close()
+        two.close()
+        rec.close()
