@@ -118,7 +118,6 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
     }
   };
   auto publish = [&](Stage &s, int p) {
-    size_t const col = col_base + static_cast<size_t>(p) * kP;
     // per-unit constants of this thread's 4 columns
     int const lc = p * kP + tx * 4;  // column inside this XCD's range
     pv4f mu, rs, dd, ga, be;
@@ -129,7 +128,6 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
       be[e] = cst[4][lc + e];
       umv[e] = cst[7][lc + e] != 0.0f ? 1 : 0;
     }
-    (void)col;
     pv4f s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0}, s2 = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {

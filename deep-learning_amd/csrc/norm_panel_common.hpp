@@ -93,9 +93,10 @@ __device__ __forceinline__ void issue_load(float &dst, float const *p) {
 __device__ __forceinline__ void issue_load(unsigned &dst, uint8_t const *p) {  // four mask bytes
   asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
 }
-// the same with a count known at run time (the same in all lanes of a wavefront), clamped to 0 .. 47: a jump into a
-// table of 48 waits, 8 bytes of code each (a chain of compares would cost several scalar instructions per
-// candidate and a kilobyte of code per wait, and these kernels hold dozens of them)
+// Waits until at most n memory operations of this wavefront are outstanding, i.e. for everything but the n
+// youngest.  n is a run-time value (the same in all lanes), clamped to 0 .. 47 (a smaller count only waits for
+// more): a jump into a table of 48 waits, 8 bytes of code each (a chain of compares would cost several scalar
+// instructions per candidate and a kilobyte of code per wait, and these kernels hold dozens of them)
 __device__ __forceinline__ void wait_younger_n(int n) {
   int t = __builtin_amdgcn_readfirstlane(n < 0 ? 0 : (n > 47 ? 47 : n));
   asm volatile("s_getpc_b64 vcc\n"            // the address of the next instruction; the table starts 20 bytes
@@ -156,23 +157,6 @@ __device__ __forceinline__ void wait_younger_n(int n) {
                : "+s"(t)
                :
                : "vcc", "scc", "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_younger() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-// the wait, with the values it makes usable
-template <int N>
-__device__ __forceinline__ void wait_for(pv4f &a, pv4f &b) {
-  asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_for(float &a) {
-  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(N) : "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_for(unsigned &a) {
-  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(N) : "memory");
 }
 
 // Entry of a panel kernel: the workgroup's XCD and its rank there.  false: more than 32 workgroups on this
