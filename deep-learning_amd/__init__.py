@@ -43,7 +43,7 @@ C_ABI_SYMBOLS = [
     "dlmi_opt_gd", "dlmi_opt_gd_momentum", "dlmi_opt_adam", "dlmi_zero_padded_identity_fwd", "dlmi_residual_bwd",
     "dlmi_opt_adabound", "dlmi_clip_gradient", "dlmi_max_norm_rows", "dlmi_opt_irprop_plus", "dlmi_loss_seed", "dlmi_zero",
     "dlmi_fused_norm_act_fwd_noalloc", "dlmi_fused_norm_act_residual_fwd", "dlmi_fc_norm_act_residual_fwd",
-    "dlmi_fc_softmax_fwd", "dlmi_fc_bwd_dx_norm_act_bwd",
+    "dlmi_fc_softmax_fwd", "dlmi_fc_softmax_ce_fwd", "dlmi_fc_bwd_dx_norm_act_bwd",
     "dlmi_ctx_reserve_layer", "dlmi_ctx_scratch_generation", "dlmi_ctx_norm_panel_enabled", "dlmi_ctx_norm_panel_poke",
     "dlmi_fc_bwd_dw_grouped", "dlmi_fused_norm_act_bwd_db", "dlmi_ctx_gemm_clock", "dlmi_probe_strip_stream",
 ]
@@ -463,6 +463,17 @@ class Dlmi:
         Z, Q = self.empty(B, H), self.empty(B, H)
         self._ck(self.lib.dlmi_fc_softmax_fwd(self.ctx, c_sz(B), c_sz(K), c_sz(H), _p(X), _p(W), _p(bias), _p(Z), _p(Q)))
         return Z, Q
+
+    def fc_softmax_ce_fwd(self, X, W, Y, bias=None, stats=None):
+        """Z = X W^T + bias, Q = softmax(Z), dZ = cross-entropy seed gradient against Y, stats (2 doubles on the
+        device, optional) += (loss sum, correct predictions).  Returns (Z, Q, dZ)."""
+        self._chk(X, W, Y, bias)
+        B, K = X.shape
+        H = W.shape[0]
+        Z, Q, dZ = self.empty(B, H), self.empty(B, H), self.empty(B, H)
+        self._ck(self.lib.dlmi_fc_softmax_ce_fwd(self.ctx, c_sz(B), c_sz(K), c_sz(H), _p(X), _p(W), _p(bias), _p(Y),
+                                                 _p(Z), _p(Q), _p(dZ), _p(stats)))
+        return Z, Q, dZ
 
     def fc_bwd_dx_fused_bwd(self, desc, dZn, Wn, x, gamma, beta, stats, dgamma, dbeta, mask=None):
         """dY = dZn Wn, then the fused normalization backward on dY.  Returns dX."""

@@ -149,11 +149,13 @@ size_t panel_scratch_bytes(size_t H);
 size_t panel_db_offset(size_t H);        // where the backward kernel's bias-gradient partials start in the scratch
 size_t panel_scratch_bytes_db(size_t H);  // scratch of a backward launch that also leaves those partials
 // Narrow layers on a mini-batch (fc_small.hip).  narrow_fc_fwd: Z = X W^T + bias and, with Q != nullptr,
-// Q = softmax(Z), one launch; call only when narrow_fc_fwd_eligible.  narrow_dw_try: dW and db in one launch;
+// Q = softmax(Z), one launch, and with Y != nullptr (targets [B,H]; Q and dZ required) also the cross-entropy seed
+// gradient dZ and stats[0] += loss sum, stats[1] += correct predictions (stats may be nullptr); call only when
+// narrow_fc_fwd_eligible.  narrow_dw_try: dW and db in one launch;
 // returns 1 when launched, 0 when the shape does not qualify, < 0 on failure.
 bool narrow_fc_fwd_eligible(dlmi_ctx const *ctx, size_t B, size_t H);
 int narrow_fc_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, float const *W, float const *bias, float *Z,
-                  float *Q);
+                  float *Q, float const *Y = nullptr, float *dZ = nullptr, double *stats = nullptr);
 int narrow_dw_try(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float *dW, float *db,
                   int accumulate);
 // The fused backward of dlmi_fused_norm_act_bwd whose upstream gradient dY is still `nslices` partial products

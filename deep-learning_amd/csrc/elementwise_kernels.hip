@@ -10,6 +10,7 @@
 #include "activations.hpp"
 #include "block_pairs.hpp"
 #include "dlmi_common.hpp"
+#include "softmax_ce_row.hpp"
 
 namespace dlmi {
 
@@ -221,54 +222,10 @@ __global__ __launch_bounds__(kEwBlock) void k_softmax_ce_seed(float const *__res
                                                                float *__restrict__ dZ, size_t B, size_t H,
                                                                double *__restrict__ pairs, double *__restrict__ acc,
                                                                unsigned *__restrict__ ticket) {
-  constexpr float kEps = 0.0000001f;  // data/dtypes.hpp:113
   int const lane = threadIdx.x & 63;
   size_t const row = static_cast<size_t>(blockIdx.x) * (kEwBlock / 64) + threadIdx.x / 64;
   double loss = 0.0, correct = 0.0;
-  if (row < B) {
-    float const *qi = q + row * H;
-    float const *yi = y + row * H;
-    float const inv_b = static_cast<float>(B);
-    // S = sum_k q_k * dL_k  (dL_k != 0 only where y_k == 1)
-    float s = 0.0f, lsum = 0.0f;
-    float best = -3.402823466e+38f;
-    long long best_k = -1, target_k = static_cast<long long>(H);
-    for (size_t k = lane; k < H; k += 64) {
-      float const qk = qi[k];
-      float const c = qk < kEps ? kEps : (qk > 1.0f - kEps ? 1.0f - kEps : qk);
-      if (yi[k] == 1.0f) {
-        s += qk * ((-1.0f / c) / inv_b);
-        lsum += -(yi[k] * logf(c));
-        target_k = static_cast<long long>(k);  // last k with y == 1 wins below
-      }
-      if (qk >= best) { best = qk; best_k = static_cast<long long>(k); }
-    }
-    for (int off = 32; off > 0; off >>= 1) {
-      s += __shfl_xor(s, off, 64);
-      lsum += __shfl_xor(lsum, off, 64);
-      float const ob = __shfl_xor(best, off, 64);
-      long long const ok = __shfl_xor(best_k, off, 64);
-      // ">=" scan keeps the LAST maximal index (compute_error_st.cpp:62-68)
-      if (ob > best || (ob == best && ok > best_k)) { best = ob; best_k = ok; }
-      long long const ot = __shfl_xor(target_k, off, 64);
-      // the sequential scan keeps the last k with y_k == 1; H means "none"
-      long long const a = target_k == static_cast<long long>(H) ? -1 : target_k;
-      long long const b = ot == static_cast<long long>(H) ? -1 : ot;
-      long long const m = a > b ? a : b;
-      target_k = m < 0 ? static_cast<long long>(H) : m;
-    }
-    for (size_t i = lane; i < H; i += 64) {
-      float const qv = qi[i];
-      float const c = qv < kEps ? kEps : (qv > 1.0f - kEps ? 1.0f - kEps : qv);
-      float const dl = yi[i] == 1.0f ? (-1.0f / c) / inv_b : 0.0f;
-      // sum_k (q_i [i==k] - q_k q_i) dL_k = q_i dL_i - q_i S
-      dZ[row * H + i] = qv * dl - qv * s;
-    }
-    if (lane == 0) {
-      loss = static_cast<double>(lsum);
-      correct = (target_k == best_k) ? 1.0 : 0.0;
-    }
-  }
+  if (row < B) softmax_ce_seed_row(q + row * H, y + row * H, dZ + row * H, H, B, lane, loss, correct);
   if (acc != nullptr) {
     __shared__ double sh[2][kEwBlock / 64];
     if (lane == 0) {

@@ -3,13 +3,18 @@
 // needs a K split, a slice reduction and then separate softmax / bias-gradient launches around it, each
 // of which costs more in launch latency than in work.  Here:
 //   k_narrow_fc_fwd  Z = X W^T + b, optionally Q = softmax(Z), one wavefront per row
-//                    (fwp_st.cpp:4498-4555, 4796-4828);
+//                    (fwp_st.cpp:4498-4555, 4796-4828); optionally also the cross-entropy seed gradient of the row
+//                    against its targets and the loss / accuracy sums (compute_error_st.cpp:26-131,
+//                    compute_loss.cpp:88-95, 101-138): the output layer's forward pass and the start of the
+//                    backward pass in one launch;
 //   k_narrow_dw      dW (+)= dZ^T X and db (+)= column sums of dZ in one launch, a workgroup per 8 columns
 //                    of X for all rows (update_derivative_fwp_st.cpp:246-302).
 // Sums run in a fixed order (no float atomics).  Citations: /root/reference/lib/deep-learning/v1/learner/.
 #include <hip/hip_runtime.h>
 
+#include "block_pairs.hpp"
 #include "dlmi_common.hpp"
+#include "softmax_ce_row.hpp"
 
 namespace dlmi {
 namespace {
@@ -27,10 +32,20 @@ typedef float nv4f __attribute__((ext_vector_type(4)));
 // step are independent, so they are in flight together.  The 64 partial sums of an output are combined with the
 // xor-shuffle tree; lane o then holds output o.  H is a template parameter so that the loops over the outputs
 // unroll without predicates.
-template <int H, int VEC, bool SOFTMAX>
+// What the seed-gradient variant takes besides: targets Y [B,H], the gradient dZ [B,H], and the loss / accuracy
+// accumulators with their per-block pairs and ticket (block_pairs.hpp; acc == nullptr: no sums).
+struct NarrowSeedArgs {
+  float const *Y;
+  float *dZ;
+  double *pairs, *acc;
+  unsigned *ticket;
+};
+
+template <int H, int VEC, bool SOFTMAX, bool SEED = false>
 __global__ __launch_bounds__(kNarrowFwdThreads) void k_narrow_fc_fwd(float const *__restrict__ X, float const *__restrict__ W,
                                                                    float const *__restrict__ bias, float *__restrict__ Z,
-                                                                   float *__restrict__ Q, size_t B, size_t K) {
+                                                                   float *Q, size_t B, size_t K, NarrowSeedArgs sa) {
+  static_assert(!SEED || (SOFTMAX && kNarrowFwdThreads == 64), "the seed variant is one wavefront per workgroup, grid = rows");
   int const lane = threadIdx.x & 63;
   size_t const row = static_cast<size_t>(blockIdx.x) * (kNarrowFwdThreads / 64) + threadIdx.x / 64;
   if (row >= B) return;
@@ -86,6 +101,12 @@ __global__ __launch_bounds__(kNarrowFwdThreads) void k_narrow_fc_fwd(float const
     for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
     s = 1.0f / s;
     if (mine) Q[row * H + lane] = e * s;
+  }
+  if constexpr (SEED) {
+    // (every workgroup of the launch holds a row: the grid is exactly B workgroups of one wavefront)
+    double loss = 0.0, correct = 0.0;
+    softmax_ce_seed_row(Q + row * H, sa.Y + row * H, sa.dZ + row * H, H, B, lane, loss, correct);
+    if (sa.acc != nullptr) finish_block_pairs(loss, correct, sa.pairs, sa.acc, sa.ticket);
   }
 }
 
@@ -144,23 +165,35 @@ bool narrow_fc_fwd_eligible(dlmi_ctx const *ctx, size_t B, size_t H) {
 
 template <int H>
 static void launch_narrow_fwd(dlmi_ctx *ctx, dim3 grid, bool vec, float const *X, float const *W, float const *bias, float *Z,
-                              float *Q, size_t B, size_t K) {
+                              float *Q, size_t B, size_t K, NarrowSeedArgs const &sa) {
   dim3 const block(kNarrowFwdThreads);
-  if (Q != nullptr) {
-    if (vec) hipLaunchKernelGGL((k_narrow_fc_fwd<H, 4, true>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K);
-    else hipLaunchKernelGGL((k_narrow_fc_fwd<H, 1, true>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K);
+  if (sa.Y != nullptr) {
+    if (vec) hipLaunchKernelGGL((k_narrow_fc_fwd<H, 4, true, true>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K, sa);
+    else hipLaunchKernelGGL((k_narrow_fc_fwd<H, 1, true, true>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K, sa);
+  } else if (Q != nullptr) {
+    if (vec) hipLaunchKernelGGL((k_narrow_fc_fwd<H, 4, true>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K, sa);
+    else hipLaunchKernelGGL((k_narrow_fc_fwd<H, 1, true>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K, sa);
   } else {
-    if (vec) hipLaunchKernelGGL((k_narrow_fc_fwd<H, 4, false>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K);
-    else hipLaunchKernelGGL((k_narrow_fc_fwd<H, 1, false>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K);
+    if (vec) hipLaunchKernelGGL((k_narrow_fc_fwd<H, 4, false>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K, sa);
+    else hipLaunchKernelGGL((k_narrow_fc_fwd<H, 1, false>), grid, block, 0, ctx->stream, X, W, bias, Z, Q, B, K, sa);
   }
 }
 
 int narrow_fc_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, float const *W, float const *bias, float *Z,
-                  float *Q) {
+                  float *Q, float const *Y, float *dZ, double *stats) {
   dim3 const grid(static_cast<unsigned>(dlmi_ceil_div(B, static_cast<size_t>(kNarrowFwdThreads / 64))));
   bool const vec = K % 4 == 0 && dlmi_aligned16(X) && dlmi_aligned16(W);
+  NarrowSeedArgs sa{Y, dZ, nullptr, stats, ctx->pair_ticket};
+  if (Y != nullptr) {
+    if (Q == nullptr || dZ == nullptr) return dlmi_fail(ctx, DLMI_E_INVALID, "narrow_fc_fwd: the seed gradient needs Q and dZ");
+    if (stats != nullptr) {
+      int const rc = dlmi_scratch_reserve(ctx, static_cast<size_t>(grid.x) * 2 * sizeof(double));
+      if (rc != DLMI_OK) return rc;
+      sa.pairs = reinterpret_cast<double *>(dlmi_scratch_data(ctx));
+    }
+  }
   switch (H) {
-#define DLMI_NARROW_CASE(n) case n: launch_narrow_fwd<n>(ctx, grid, vec, X, W, bias, Z, Q, B, K); break;
+#define DLMI_NARROW_CASE(n) case n: launch_narrow_fwd<n>(ctx, grid, vec, X, W, bias, Z, Q, B, K, sa); break;
     DLMI_NARROW_CASE(1) DLMI_NARROW_CASE(2) DLMI_NARROW_CASE(3) DLMI_NARROW_CASE(4) DLMI_NARROW_CASE(5)
     DLMI_NARROW_CASE(6) DLMI_NARROW_CASE(7) DLMI_NARROW_CASE(8) DLMI_NARROW_CASE(9) DLMI_NARROW_CASE(10)
     DLMI_NARROW_CASE(11) DLMI_NARROW_CASE(12) DLMI_NARROW_CASE(13) DLMI_NARROW_CASE(14) DLMI_NARROW_CASE(15)
@@ -183,3 +216,13 @@ int narrow_dw_try(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin,
 }
 
 }  // namespace dlmi
+
+extern "C" int dlmi_fc_softmax_ce_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, float const *W,
+                                      float const *bias, float const *Y, float *Z, float *Q, float *dZ, double *stats) {
+  if (ctx == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, X && W && Y && Z && Q && dZ, "null pointer");
+  DLMI_REQUIRE(ctx, B > 0 && K > 0 && H > 0, "empty operand");
+  if (dlmi::narrow_fc_fwd_eligible(ctx, B, H)) return dlmi::narrow_fc_fwd(ctx, B, K, H, X, W, bias, Z, Q, Y, dZ, stats);
+  int const rc = dlmi_fc_softmax_fwd(ctx, B, K, H, X, W, bias, Z, Q);
+  return rc != DLMI_OK ? rc : dlmi_softmax_ce_seed(ctx, B, H, Q, Y, dZ, stats);
+}

@@ -126,8 +126,7 @@ void Driver::one_batch(size_t const i, size_t const batch_size, size_t const bat
                        bool const training) {
   if (resident) {
     float const *const x = d_X_ + i * batch_size_max * dataset.n_inp, *const y = d_Y_ + i * batch_size_max * dataset.n_out;
-    model.forward_pass_device(batch_size, x);
-    if (training) model.compute_error_device(batch_size, y); else model.compute_loss_device(batch_size, y);
+    model.forward_error_device(batch_size, x, y);  // (training and evaluation alike: compute_loss is compute_error)
   } else {
     model.forward_pass(batch_size, dataset.Xm + i * batch_size_max);
     if (training) model.compute_error(batch_size, dataset.Ym + i * batch_size_max);

@@ -68,6 +68,11 @@ struct Model::Impl {
   // read layer outputs that the next forward pass overwrites - those the compute stream waits for at once.
   hipEvent_t dw_mid = nullptr;
   bool dw_pending = false;          // dw_done is recorded and the compute stream has not waited for it yet
+  size_t dw_pending_layer = 0;      // ... for the weight gradient of this layer
+  // forward_error_device(): the targets of the pass in flight, for an output layer that can form the seed gradient
+  // in the launch of its forward pass; whether it did
+  float const *fwd_targets = nullptr;
+  bool fwd_seeded = false;
   bool cur_input_external = false;  // cur_input is the caller's device memory, not an upload slot
   void record_dz_ready(size_t layer) {
     if (dw_ctx != nullptr && layer < dz_ready.size()) (void)hipEventRecord(dz_ready[layer], stream);
@@ -1132,6 +1137,14 @@ void Model::forward_layers(size_t const B, size_t const end_layer) {
     // a softmax layer without normalization or dropout (the output layer): product, bias and softmax in one call
     bool const fused_fc_softmax = softmax && !l.Use__Normalization() && !l.Use__Dropout();
     if (fused_fc_softmax) {
+      // the output layer of a pass that came with its targets: the seed gradient and the loss sums in the same call
+      if (impl_->fwd_targets != nullptr && li + 1 == total_layers && type_loss_function == LOSS_FN::CROSS_ENTROPY &&
+          type_accuracy_function == ACCU_FN::CROSS_ENTROPY) {
+        if (dlmi_fc_softmax_ce_fwd(ctx, B, K, H, in, W, bias, impl_->fwd_targets, l.d_summations, l.d_outputs, l.d_errors,
+                                   impl_->d_stats) != DLMI_OK) { fail("forward_pass: dlmi_fc_softmax_ce_fwd"); return; }
+        impl_->fwd_seeded = true;
+        continue;
+      }
       if (dlmi_fc_softmax_fwd(ctx, B, K, H, in, W, bias, l.d_summations, l.d_outputs) != DLMI_OK) { fail("forward_pass: dlmi_fc_softmax_fwd"); return; }
       continue;
     }
@@ -1308,6 +1321,22 @@ void Model::compute_error(size_t const B, real const *const *const Ym) {
 void Model::compute_error_device(size_t const B, float const *d_targets) {
   if (ptr_array_layers == nullptr || d_targets == nullptr || B == 0 || B > impl_->allocated_batch) { fail("compute_error_device: bad argument"); return; }
   seed_error(B, d_targets);
+}
+
+// forward_pass_device() followed by compute_error_device(), with the output layer's share of both in one call
+// where that layer is a softmax layer under the cross-entropy loss (dlmi_fc_softmax_ce_fwd).
+void Model::forward_error_device(size_t const B, float const *d_inputs, float const *d_targets) {
+  if (ptr_array_layers == nullptr || d_inputs == nullptr || d_targets == nullptr) { fail("forward_error_device: model not compiled or null pointer"); return; }
+  // the output layer's dZ is written during this forward pass: a weight gradient still reading it comes first
+  if (impl_->dw_pending && impl_->dw_pending_layer + 1 == total_layers && !join_weight_gradients()) return;
+  size_t const errors_before = impl_->n_errors;
+  impl_->fwd_targets = d_targets;
+  impl_->fwd_seeded = false;
+  forward_pass_device(B, d_inputs);
+  impl_->fwd_targets = nullptr;
+  if (impl_->n_errors != errors_before) return;
+  if (!impl_->fwd_seeded) { compute_error_device(B, d_targets); return; }
+  impl_->n_loss_values += B * ptr_array_layers[total_layers - 1].n_out;  // as seed_error() counts them
 }
 
 // Loss and accuracy are accumulated by the same kernel that forms the seed
@@ -1641,6 +1670,7 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
     // the product that reads the caller's input rows may outlast this call (see dw_mid): what was launched
     // beside the chain before it is marked, and only that is waited for below
     if (in == impl_->cur_input && impl_->cur_input_external && !deferred) {
+      impl_->dw_pending_layer = li;
       if (!joined) {
         if (!hip_ok(hipEventRecord(impl_->dw_mid, impl_->dw_stream), impl_->err, "update_derivatives: mark")) {
           fail("update_derivatives: mark");

@@ -362,6 +362,16 @@ int dlmi_fc_norm_act_fwd(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, s
 int dlmi_fc_softmax_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, float const *W,
                         float const *bias, float *Z, float *Q);
 
+/* The same and, from the targets Y [B,H], what compute_error does next: the softmax + cross-entropy seed gradient dZ
+ * [B,H] of dlmi_softmax_ce_seed and its loss / accuracy sums in stats (2 doubles on the device, may be NULL)
+ * (compute_error_fwp_st, compute_error_st.cpp:26-131; loss_fn_derivative, compute_loss.cpp:88-95, 101-138).  For a
+ * caller that has the targets at hand when the forward pass reaches the output layer (an epoch driver over a
+ * resident data set): a narrow layer (see above) is ONE launch for product, bias, softmax, seed gradient and sums;
+ * anything else is dlmi_fc_softmax_fwd followed by dlmi_softmax_ce_seed.  Z, Q and dZ hold the same bits as after
+ * those two calls; the sums are the same terms, added block by block in another grouping. */
+int dlmi_fc_softmax_ce_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, float const *W,
+                           float const *bias, float const *Y, float *Z, float *Q, float *dZ, double *stats);
+
 /* Backward of a normalized layer together with the product that brings its upstream gradient:
  * dY = dZn . Wn (Backward_Pass__FC__Loop, bwp_st.cpp:1009-1045; dZn [B,Hn], Wn [Hn][H]), then
  * dlmi_fused_norm_act_bwd on dY (bwp_st.cpp:1177-1209, 1284-1366, 1447-1532), result in dX [B,H]

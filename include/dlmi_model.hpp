@@ -380,6 +380,11 @@ class Model : public Model_State {
   // launches into a HIP graph calls this before it ends the capture (a capture must not end with work forked
   // off and not joined), and the rows handed to forward_pass_device() must stay unchanged until then.
   bool join_weight_gradients(void) const;
+  // No counterpart in the reference: forward_pass_device(batch, d_inputs) followed by
+  // compute_error_device(batch, d_targets) (equally compute_loss_device: the loss sums are the same, the seed gradient
+  // is simply unused) as one call, so that a softmax output layer under the cross-entropy loss forms its outputs, the
+  // seed gradient and the loss / accuracy sums in one launch.  Same results as the two calls.
+  void forward_error_device(size_t const batch, float const *d_inputs, float const *d_targets);
   // The stream every kernel of this model is launched on (a hipStream_t), and a hash of
   // everything the kernels of one batch take by value or by address (layer settings,
   // hyper-parameters, propagation state, buffer addresses): two batches of the same size

@@ -118,3 +118,32 @@ def test_backward_with_the_product_above_it(twins, pkg, B, Hn, H, act, drop):
     assert_close(dX.cpu().numpy(), dXp.cpu().numpy(), 1e-4, "dX", floor=1.0)
     assert_close(dg.cpu().numpy(), dgp.cpu().numpy(), 1e-4, "dgamma", floor=1.0)
     assert_close(db.cpu().numpy(), dbp.cpu().numpy(), 1e-4, "dbeta", floor=1.0)
+
+
+@pytest.mark.parametrize("B,K,H", [(128, 512, 10), (1000, 33, 16), (7, 5, 1), (64, 257, 3), (300, 64, 40)])
+def test_output_layer_forward_with_the_seed_gradient(twins, pkg, B, K, H):
+    """dlmi_fc_softmax_ce_fwd against dlmi_fc_softmax_fwd followed by dlmi_softmax_ce_seed: Z, Q and dZ bit for bit
+    (the seed is formed by the same per-row code), the loss and accuracy sums to the rounding of a double sum in
+    another grouping; the accumulators accumulate, launch after launch; 40 units: the two-call path inside."""
+    fast, _ = twins
+    rng = np.random.default_rng(B * 3 + K + H)
+    X = dev(rng.standard_normal((B, K)).astype(np.float32))
+    W = dev((rng.standard_normal((H, K)) / np.sqrt(K)).astype(np.float32))
+    b = dev(rng.uniform(-.5, .5, H).astype(np.float32))
+    Y = dev(np.eye(H, dtype=np.float32)[rng.integers(0, H, B)])
+    for bias in (b, None):
+        st_two = torch.tensor([0.5, 3.0], dtype=torch.float64, device="cuda")
+        st_one = st_two.clone()
+        Z2, Q2 = fast.fc_softmax_fwd(X, W, bias)
+        dZ2 = fast.softmax_ce_seed(Q2, Y, stats=st_two)
+        for rep in range(2):  # the ticket and the pairs are left ready for the next launch
+            Z1, Q1, dZ1 = fast.fc_softmax_ce_fwd(X, W, Y, bias=bias, stats=st_one)
+            assert torch.equal(Z1, Z2) and torch.equal(Q1, Q2) and torch.equal(dZ1, dZ2)
+        fast.softmax_ce_seed(Q2, Y, stats=st_two)
+        fast.synchronize()
+        a, c = st_one.cpu().numpy(), st_two.cpu().numpy()
+        assert a[1] == c[1], "correct predictions"
+        assert abs(a[0] - c[0]) <= 1e-12 * abs(c[0]), "loss sum"
+    # without accumulators
+    Z1, Q1, dZ1 = fast.fc_softmax_ce_fwd(X, W, Y, bias=b)
+    assert torch.equal(dZ1, fast.softmax_ce_seed(fast.fc_softmax_fwd(X, W, b)[1], Y))
