@@ -63,7 +63,7 @@ MEASURED_TRAFFIC_BYTES = {
 }
 TRAFFIC_SOURCES = ("gemm_f32_mfma.hip", "norm_kernels.hip", "norm_panel_fwd.hip", "norm_panel_bwd.hip",
                    "norm_panel_common.hpp", "norm_shared.hpp", "activations.hpp")
-TRAFFIC_SOURCES_SHA256 = "bbe4f80f634b8f7c90b5e8f1d9e679c5f3f0894f30568908d983e45ce01bdd59"
+TRAFFIC_SOURCES_SHA256 = "55fba464526905c98770ce549eb0c756bafc3d77ba911d4023d15b98ce335554"
 
 
 def traffic_sources_digest():

@@ -75,19 +75,50 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
   size_t const row0 = static_cast<size_t>(who.rank) * (RPT * kTY);
   size_t const col_base = static_cast<size_t>(who.xcd) * Hx;
 
-  auto preload_constants = [&] {
-  for (size_t c = threadIdx.x; c < Hx; c += kPanelThreads) {
-    float const sd = a.stdv[col_base + c], rr = a.r[col_base + c];
-    cst[0][c] = a.mean[col_base + c];
-    cst[1][c] = rr * fast_rcp(sd);
-    cst[2][c] = a.d[col_base + c];
-    cst[3][c] = a.gamma[col_base + c];
-    cst[4][c] = a.beta[col_base + c];
-    cst[5][c] = sd;
-    cst[6][c] = rr;
-    cst[7][c] = a.drop_mode == kDropUnit ? (a.mask[col_base + c] ? 1.0f : 0.0f) : 1.0f;
-  }
-  __syncthreads();
+  // The constants are asked for BEFORE the first panels (they arrive first: a wavefront's loads return in issue
+  // order) and put into LDS once they are there, with the panels' loads still in flight.  A thread fetches the
+  // constants of up to kCstPer columns; a column beyond the XCD's range, or a mask that does not exist, is fetched
+  // from a valid address all the same (no conditional issue, see issue_load) and not used.
+  constexpr int kCstPer = kPanelMaxCols / kPanelThreads;
+  float cin[kCstPer][6];
+  unsigned cmask[kCstPer];
+  auto request_constants = [&] {
+#pragma unroll
+    for (int k = 0; k < kCstPer; ++k) {
+      size_t const c = threadIdx.x + static_cast<size_t>(k) * kPanelThreads;
+      size_t const at = col_base + (c < Hx ? c : 0);
+      issue_load(cin[k][0], a.mean + at);
+      issue_load(cin[k][1], a.stdv + at);
+      issue_load(cin[k][2], a.r + at);
+      issue_load(cin[k][3], a.d + at);
+      issue_load(cin[k][4], a.gamma + at);
+      issue_load(cin[k][5], a.beta + at);
+      // (four mask bytes from the aligned word that holds this column's; without a per-unit mask: any valid word)
+      issue_load(cmask[k], a.drop_mode == kDropUnit ? a.mask + (at & ~static_cast<size_t>(3)) : reinterpret_cast<uint8_t const *>(a.gamma));
+    }
+  };
+  auto store_constants = [&](int younger) {
+    wait_younger_n(younger);
+#pragma unroll
+    for (int k = 0; k < kCstPer; ++k) {
+#pragma unroll
+      for (int j = 0; j < 6; ++j) asm volatile("" : "+v"(cin[k][j]));
+      asm volatile("" : "+v"(cmask[k]));
+      size_t const c = threadIdx.x + static_cast<size_t>(k) * kPanelThreads;
+      if (c < Hx) {
+        float const sd = cin[k][1], rr = cin[k][2];
+        cst[0][c] = cin[k][0];
+        cst[1][c] = rr * fast_rcp(sd);
+        cst[2][c] = cin[k][3];
+        cst[3][c] = cin[k][4];
+        cst[4][c] = cin[k][5];
+        cst[5][c] = sd;
+        cst[6][c] = rr;
+        unsigned const byte = (cmask[k] >> (8u * static_cast<unsigned>((col_base + c) & 3u))) & 0xffu;
+        cst[7][c] = a.drop_mode == kDropUnit ? (byte ? 1.0f : 0.0f) : 1.0f;
+      }
+    }
+    __syncthreads();
   };
 
   struct Stage {
@@ -311,10 +342,11 @@ __global__ __launch_bounds__(kPanelThreads) void k_bwd_panel(PanelBwdArgs a) {
   // the barrier word and its count asked for, p finished.
   Stage b0, b1, b2, b3, b4;
   auto clamped = [&](int p) { return p < npanels ? p : npanels - 1; };
+  request_constants();
   load(b0, 0);
   load(b1, clamped(1));
-  preload_constants();  // (its loads are younger than those of panels 0 and 1: waiting for them completes both)
-  wait_stage(b0, ld);  // panel 1's loads are younger
+  store_constants(2 * ld);  // the loads of panels 0 and 1 are younger
+  wait_stage(b0, ld);       // panel 1's loads are younger
   publish(b0, 0);
   load(b2, clamped(2));
   load(b3, clamped(3));
