@@ -15,6 +15,7 @@
 // best on MI355X).
 struct dlmi_tuning {
   int reduce_tx_cap = 128;        // widest column span of a reduction block, in column groups
+  int reduce_tx_cap_few_units = 16;  // ... when the tensor has at most 64 column groups (256 units)
   int reduce_blocks_per_cu = 1;   // reduction blocks per compute unit
   int reduce_min_rows = 4;        // fewest rows a thread of a reduction block walks
   int apply_fwd_blocks_per_cu = 16;  // blocks per compute unit in the forward apply pass (one read, one write stream)

@@ -69,6 +69,7 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
   ctx->num_cu = prop.multiProcessorCount;
   dlmi_tuning &t = ctx->tune;
   t.reduce_tx_cap = env_knob("DLMI_NORM_REDUCE_TX", t.reduce_tx_cap);
+  t.reduce_tx_cap_few_units = env_knob("DLMI_NORM_REDUCE_TX_FEW_UNITS", t.reduce_tx_cap_few_units);
   t.reduce_blocks_per_cu = env_knob("DLMI_NORM_REDUCE_BLOCKS_PER_CU", t.reduce_blocks_per_cu);
   t.reduce_min_rows = env_knob("DLMI_NORM_REDUCE_MIN_ROWS", t.reduce_min_rows);
   t.apply_fwd_blocks_per_cu = env_knob("DLMI_NORM_APPLY_FWD_BLOCKS_PER_CU", t.apply_fwd_blocks_per_cu);
