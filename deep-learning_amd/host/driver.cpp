@@ -123,18 +123,25 @@ void Driver::evalt_st(void) { run_batches(evalt_rec_, false); }
 // One mini-batch: forward and loss (evaluation), or forward, seed gradient, backward and
 // parameter gradients (training).
 void Driver::one_batch(size_t const i, size_t const batch_size, size_t const batch_size_max, bool const resident,
-                       bool const training) {
+                       bool const training, int const lane) {
   if (resident) {
     float const *const x = d_X_ + i * batch_size_max * dataset.n_inp, *const y = d_Y_ + i * batch_size_max * dataset.n_out;
+    // (lanes: no-ops unless the model has a second set of per-batch buffers, see Model::enable_lanes)
+    (void)model.lane_forward_begin(lane);
     model.forward_error_device(batch_size, x, y);  // (training and evaluation alike: compute_loss is compute_error)
+    (void)model.lane_forward_end();
   } else {
     model.forward_pass(batch_size, dataset.Xm + i * batch_size_max);
     if (training) model.compute_error(batch_size, dataset.Ym + i * batch_size_max);
     else model.compute_loss(batch_size, dataset.Ym + i * batch_size_max);
   }
   if (!training) return;
+  if (resident) (void)model.lane_backward_begin();
   model.backward_pass(batch_size);
   model.update_derivatives(batch_size, model.ptr_array_layers + 1, model.ptr_last_layer);
+  // (the weight gradients stay in this chain: a chain of their own, which would let the next backward pass start
+  // before them, measured slower - 0.067-0.072 against 0.063-0.064 ms per mini-batch of the 784-512-512-10 network)
+  if (resident) (void)model.lane_backward_end();
 }
 
 void Driver::drop_graphs(Recorded &rec) {
@@ -156,10 +163,15 @@ void Driver::run_batches(Recorded &rec, bool const training) {
   // nothing may allocate inside a capture: the scratch of every layer shape and the lazily allocated buffers
   // come first (this can change the scratch generation, which the signature below includes)
   if (resident && record_batches && !recording_failed_ && !model.reserve_for(batch_size_max)) recording_failed_ = true;
+  // mini-batches of a training pass alternate between two sets of buffers, so that the forward pass of one overlaps
+  // the backward pass of the one before (Model::enable_lanes says for which models).  The LAST mini-batch of every
+  // stretch (a graph's worth of mini-batches) runs on lane 0, and every stretch ends with both lanes joined on lane
+  // 0's stream, so that whatever follows finds the model as a single lane would have left it.
+  bool const lanes = training && resident && model.enable_lanes(batch_size_max);
   uint64_t sig = resident && record_batches && !recording_failed_ ? model.launch_signature() : 0;
   if (sig != 0) {
-    uint64_t const extra[5] = {n_data, batch_size_max, reinterpret_cast<uintptr_t>(d_X_), reinterpret_cast<uintptr_t>(d_Y_),
-                               batches_per_graph};
+    uint64_t const extra[6] = {n_data, batch_size_max, reinterpret_cast<uintptr_t>(d_X_), reinterpret_cast<uintptr_t>(d_Y_),
+                               batches_per_graph, lanes ? 1u : 0u};
     for (uint64_t v : extra) sig = (sig ^ v) * 1099511628211ull;
     if (sig == 0) sig = 1;
   }
@@ -176,13 +188,19 @@ void Driver::run_batches(Recorded &rec, bool const training) {
   // pass itself do, see below)
   bool const record = sig != 0 && !replay && rec.warmed_up;
   auto const rows_of = [&](size_t const i) { return i + 1 != n_batch ? batch_size_max : n_data - i * batch_size_max; };
+  // the mini-batches [first, end) one after the other, alternating lanes, the last one on lane 0; then the join
+  auto const stretch = [&](size_t const first, size_t const end) {
+    for (size_t i = first; i != end; ++i)
+      one_batch(i, rows_of(i), batch_size_max, resident, training, lanes ? static_cast<int>((end - 1 - i) & 1u) : 0);
+    return model.lanes_join();
+  };
   for (size_t g = 0; g != n_graphs; ++g) {
     size_t const first = g * per_graph, end = first + per_graph < n_batch ? first + per_graph : n_batch;
     if (replay) {
       if (hipGraphLaunch(static_cast<hipGraphExec_t>(rec.graphs[g]), stream) != hipSuccess) {
         (void)hipGetLastError();
         recording_failed_ = true;  // this pass goes on kernel by kernel, and so do all later ones
-        for (size_t j = first; j != n_batch; ++j) one_batch(j, rows_of(j), batch_size_max, resident, training);
+        (void)stretch(first, n_batch);
         break;
       }
       for (size_t i = first; i != end; ++i) model.account_replayed_batch(rows_of(i), d_X_ + i * batch_size_max * dataset.n_inp);
@@ -196,8 +214,7 @@ void Driver::run_batches(Recorded &rec, bool const training) {
       Model::PassState const before = model.pass_state();
       bool ok = hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed) == hipSuccess;
       if (ok) {
-        for (size_t i = first; i != end; ++i) one_batch(i, rows_of(i), batch_size_max, resident, training);
-        bool const pass_ok = model.join_weight_gradients() && model.error_count() == before.n_errors;
+        bool const pass_ok = stretch(first, end) && model.error_count() == before.n_errors;
         ok = hipStreamEndCapture(stream, &graph) == hipSuccess && graph != nullptr && pass_ok;
       }
       ok = ok && hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) == hipSuccess;
@@ -212,7 +229,7 @@ void Driver::run_batches(Recorded &rec, bool const training) {
       model.restore_pass_state(before);
       recording_failed_ = true;  // nothing of these batches has run yet: fall through to the plain launches
     }
-    for (size_t i = first; i != end; ++i) one_batch(i, rows_of(i), batch_size_max, resident, training);
+    (void)stretch(first, end);
   }
   if (rec.graphs.size() != n_graphs && !rec.graphs.empty()) drop_graphs(rec);  // a partial recording is of no use
   rec.warmed_up = true;

@@ -74,6 +74,21 @@ struct Model::Impl {
   float const *fwd_targets = nullptr;
   bool fwd_seeded = false;
   bool cur_input_external = false;  // cur_input is the caller's device memory, not an upload slot
+  // A second set of the per-batch buffers (layer outputs, gradients, batch statistics) with a stream and a context
+  // (scratch) of its own: the epoch driver runs the mini-batches of a training pass alternately on the two sets, so
+  // that the forward pass of a mini-batch overlaps the backward pass of the one before it (what orders them is in
+  // lane_* below).  The Layer members always point at the CURRENT set; `other` holds the set that is not current.
+  // Outside the driver's pass the model is on lane 0 and the second set is idle.
+  struct LaneSet {
+    std::vector<float *> bufs;  // per layer: summations, outputs, errors, af_values, mean, std, r, d
+    dlmi_ctx *ctx = nullptr;
+    hipStream_t stream = nullptr;
+  };
+  LaneSet other;
+  bool lanes_ready = false;
+  int lane = 0;
+  hipEvent_t f_done[2] = {nullptr, nullptr}, b_done[2] = {nullptr, nullptr}, lane_fork = nullptr;
+  bool f_rec[2] = {false, false}, b_rec[2] = {false, false}, forked = false;
   void record_dz_ready(size_t layer) {
     if (dw_ctx != nullptr && layer < dz_ready.size()) (void)hipEventRecord(dz_ready[layer], stream);
   }
@@ -338,6 +353,8 @@ Model::PassState Model::pass_state(void) const {
 }
 void Model::restore_pass_state(PassState const &s) {
   impl_->dw_pending = false;  // (a recording that failed took the side stream's part of it along)
+  select_lane(0);             // ... and the second lane's
+  impl_->f_rec[0] = impl_->f_rec[1] = impl_->b_rec[0] = impl_->b_rec[1] = impl_->forked = false;
   impl_->n_loss_values = s.n_loss_values;
   impl_->out_batch = s.out_batch;
   impl_->cur_input = s.cur_input;
@@ -357,9 +374,135 @@ bool Model::join_weight_gradients(void) const {
   return true;
 }
 
+// ---- the second set of per-batch buffers (see Impl::LaneSet)
+namespace {
+constexpr size_t kLaneBuffers = 8;         // per layer: summations, outputs, errors, af_values, mean, std, r, d
+constexpr size_t kLaneMaxBatch = 256;      // mini-batches only: that is where launch latency is the bound
+}  // namespace
+
+void Model::free_lanes(void) {
+  Impl &m = *impl_;
+  if (m.lane != 0) select_lane(0);
+  for (float *&p : m.other.bufs) dev_free(p);
+  m.other.bufs.clear();
+  if (m.other.ctx != nullptr) (void)dlmi_ctx_destroy(m.other.ctx);
+  m.other.ctx = nullptr;
+  if (m.other.stream != nullptr) (void)hipStreamDestroy(m.other.stream);
+  m.other.stream = nullptr;
+  for (hipEvent_t *e : {&m.f_done[0], &m.f_done[1], &m.b_done[0], &m.b_done[1], &m.lane_fork}) {
+    if (*e != nullptr) (void)hipEventDestroy(*e);
+    *e = nullptr;
+  }
+  m.lanes_ready = false;
+  m.f_rec[0] = m.f_rec[1] = m.b_rec[0] = m.b_rec[1] = m.forked = false;
+}
+
+bool Model::enable_lanes(size_t const batch) {
+  Impl &m = *impl_;
+  if (m.lanes_ready) return true;
+  static bool const wanted = [] { char const *e = std::getenv("DLMI_LANES"); return e == nullptr || std::atoi(e) != 0; }();
+  if (!wanted || ptr_array_layers == nullptr || m.ctx == nullptr || m.allocated_batch == 0 || batch > m.allocated_batch ||
+      m.allocated_batch > kLaneMaxBatch)
+    return false;
+  for (size_t i = 1; i < total_layers; ++i)
+    if (ptr_array_layers[i].type_layer != LAYER::FULLY_CONNECTED || ptr_array_layers[i].in_block) return false;
+  // the second set counts against the memory the model may take
+  if (maximum_allowable_memory_bytes != 0 &&
+      Get__Sizeof(1, m.allocated_batch) + Get__Batch_Sizeof(m.allocated_batch) > maximum_allowable_memory_bytes)
+    return false;
+  size_t const n = m.allocated_batch;
+  m.other.bufs.assign(total_layers * kLaneBuffers, nullptr);
+  bool ok = hipStreamCreate(&m.other.stream) == hipSuccess && dlmi_ctx_create(&m.other.ctx, 0, m.other.stream) == DLMI_OK;
+  for (hipEvent_t *e : {&m.f_done[0], &m.f_done[1], &m.b_done[0], &m.b_done[1], &m.lane_fork})
+    ok = ok && hipEventCreateWithFlags(e, hipEventDisableTiming) == hipSuccess;
+  for (size_t i = 1; ok && i < total_layers; ++i) {
+    Layer const &l = ptr_array_layers[i];
+    float **b = &m.other.bufs[i * kLaneBuffers];
+    ok = dev_alloc(&b[0], n * l.n_out, m.err) && dev_alloc(&b[1], n * l.n_out, m.err) && dev_alloc(&b[2], n * l.n_out, m.err);
+    if (ok && (l.d_af_values != nullptr || (l.Use__Normalization() && !l.use_layer_normalization_before_activation)))
+      ok = dev_alloc(&b[3], n * l.n_out, m.err);
+    for (int k = 4; ok && k < 8; ++k) ok = dev_alloc(&b[k], l.n_units, m.err);
+    size_t const K = ptr_array_layers[i - 1].n_out;
+    ok = ok && dlmi_ctx_reserve_layer(m.other.ctx, n, K, l.n_out) == DLMI_OK;
+  }
+  if (!ok) {
+    (void)hipGetLastError();
+    free_lanes();
+    return false;
+  }
+  m.lanes_ready = true;
+  return true;
+}
+
+void Model::select_lane(int const k) {
+  Impl &m = *impl_;
+  if (k == m.lane || m.other.bufs.empty()) return;
+  for (size_t i = 1; i < total_layers; ++i) {
+    Layer &l = ptr_array_layers[i];
+    float **b = &m.other.bufs[i * kLaneBuffers];
+    std::swap(l.d_summations, b[0]); std::swap(l.d_outputs, b[1]); std::swap(l.d_errors, b[2]);
+    std::swap(l.d_af_values, b[3]);
+    std::swap(l.d_mean, b[4]); std::swap(l.d_std, b[5]); std::swap(l.d_r, b[6]); std::swap(l.d_d, b[7]);
+  }
+  std::swap(m.ctx, m.other.ctx);
+  std::swap(m.stream, m.other.stream);
+  m.lane = k;
+}
+
+// What orders the two lanes: the forward passes follow each other (moving statistics, the loss sums), the backward
+// passes follow each other (every pass adds to the same gradient array), a lane's own launches follow each other on
+// its stream - and nothing else, so the forward pass of a mini-batch runs beside the backward pass of the one before.
+bool Model::lane_forward_begin(int const k) {
+  Impl &m = *impl_;
+  if (!m.lanes_ready) return true;
+  select_lane(k);
+  bool ok = true;
+  if (k == 1 && !m.forked) {
+    // lane 1 joins what lane 0's stream has been given so far (a capture in progress included)
+    ok = hipEventRecord(m.lane_fork, m.other.stream) == hipSuccess && hipStreamWaitEvent(m.stream, m.lane_fork, 0) == hipSuccess;
+    m.forked = true;
+  }
+  if (ok && m.f_rec[1 - k]) ok = hipStreamWaitEvent(m.stream, m.f_done[1 - k], 0) == hipSuccess;
+  return ok || fail("lane_forward_begin");
+}
+bool Model::lane_forward_end(void) {
+  Impl &m = *impl_;
+  if (!m.lanes_ready) return true;
+  m.f_rec[m.lane] = true;
+  return hipEventRecord(m.f_done[m.lane], m.stream) == hipSuccess || fail("lane_forward_end");
+}
+bool Model::lane_backward_begin(void) {
+  Impl &m = *impl_;
+  if (!m.lanes_ready || !m.b_rec[1 - m.lane]) return true;
+  return hipStreamWaitEvent(m.stream, m.b_done[1 - m.lane], 0) == hipSuccess || fail("lane_backward_begin");
+}
+bool Model::lane_backward_end(void) {
+  Impl &m = *impl_;
+  if (!m.lanes_ready) return true;
+  m.b_rec[m.lane] = true;
+  return hipEventRecord(m.b_done[m.lane], m.stream) == hipSuccess || fail("lane_backward_end");
+}
+// End of a pass (and of a recording): lane 0 current again, and its stream behind everything lane 1 was given.
+bool Model::lanes_join(void) {
+  Impl &m = *impl_;
+  bool ok = join_weight_gradients();
+  if (m.lanes_ready) {
+    select_lane(0);
+    if (m.f_rec[1]) ok = hipStreamWaitEvent(m.stream, m.f_done[1], 0) == hipSuccess && ok;
+    if (m.b_rec[1]) ok = hipStreamWaitEvent(m.stream, m.b_done[1], 0) == hipSuccess && ok;
+    m.f_rec[0] = m.f_rec[1] = m.b_rec[0] = m.b_rec[1] = m.forked = false;
+  }
+  return ok || fail("lanes_join");
+}
+bool Model::lanes_enabled(void) const { return impl_->lanes_ready; }
+
 bool Model::synchronize(void) const {
   if (impl_->ctx == nullptr) return false;
   bool ok = join_weight_gradients();
+  if (impl_->other.ctx != nullptr && dlmi_ctx_synchronize(impl_->other.ctx) != DLMI_OK) {
+    ok = false;
+    fail((std::string("synchronize (second lane): ") + dlmi_last_error(impl_->other.ctx)).c_str());
+  }
   if (impl_->dw_ctx != nullptr && dlmi_ctx_synchronize(impl_->dw_ctx) != DLMI_OK) {
     ok = false;
     fail((std::string("synchronize (weight-gradient stream): ") + dlmi_last_error(impl_->dw_ctx)).c_str());
@@ -665,6 +808,7 @@ bool Model::set_max_batch_size(size_t const n) {
 }
 
 void Model::free_batch(void) {
+  free_lanes();
   if (ptr_array_layers != nullptr)
     for (Layer *l = ptr_array_layers; l != ptr_last_layer; ++l) {
       if (l->d_summations == l->d_outputs) l->d_summations = nullptr;  // one buffer for a layer inside a block
@@ -1369,7 +1513,7 @@ void Model::seed_error(size_t const B, float const *d_targets) {
 }
 
 // ---------------------------------------------------------------- what a recorded batch depends on
-void *Model::native_stream(void) const { return static_cast<void *>(impl_->stream); }
+void *Model::native_stream(void) const { return static_cast<void *>(impl_->lane == 0 ? impl_->stream : impl_->other.stream); }
 void *Model::native_context(void) const { return static_cast<void *>(impl_->ctx); }
 
 void Model::account_replayed_batch(size_t const batch_size, float const *d_inputs) {
@@ -1397,6 +1541,11 @@ uint64_t Model::launch_signature(void) const {
   DLMI_MIX(scratch_generation);
   unsigned long long const dw_scratch_generation = impl_->dw_ctx != nullptr ? dlmi_ctx_scratch_generation(impl_->dw_ctx) : 0ull;
   DLMI_MIX(dw_scratch_generation);
+  // the second set of per-batch buffers, when there is one
+  DLMI_MIX(impl_->lanes_ready);
+  for (float *b : impl_->other.bufs) DLMI_MIX(b);
+  unsigned long long const lane_scratch_generation = impl_->other.ctx != nullptr ? dlmi_ctx_scratch_generation(impl_->other.ctx) : 0ull;
+  DLMI_MIX(lane_scratch_generation);
   // which normalization kernels a layer launches: a recording that holds single-launch kernels is made again once
   // the context has gone back to the multi-launch ones
   int const panel_kernels = dlmi_ctx_norm_panel_enabled(impl_->ctx);
@@ -1632,7 +1781,9 @@ void Model::update_derivatives(size_t const B, Layer *const first, Layer const *
   // from the last layer down: the order in which the backward pass finishes their gradients (every layer adds
   // into its own part of the gradient array, so the order does not change the sums)
   if (!join_weight_gradients()) return;
-  bool const side = impl_->dw_ctx != nullptr;
+  // (two lanes: the other lane's forward pass already fills the gaps the side stream is for, and a recording then
+  // has two streams that wait for each other, not three)
+  bool const side = impl_->dw_ctx != nullptr && !impl_->lanes_ready;
   bool joined = true;  // nothing on the side stream yet
   bool mid_recorded = false, deferred = false;
   hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;

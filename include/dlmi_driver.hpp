@@ -112,7 +112,7 @@ class Driver {
     uint64_t signature = 0;      // what the graphs were recorded for
     bool warmed_up = false;      // a plain pass has run for that signature
   };
-  void one_batch(size_t i, size_t batch_size, size_t batch_size_max, bool resident, bool training);
+  void one_batch(size_t i, size_t batch_size, size_t batch_size_max, bool resident, bool training, int lane = 0);
   void run_batches(Recorded &rec, bool training);
   void drop_graphs(Recorded &rec);
   float *d_X_ = nullptr, *d_Y_ = nullptr;

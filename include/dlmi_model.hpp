@@ -385,6 +385,25 @@ class Model : public Model_State {
   // is simply unused) as one call, so that a softmax output layer under the cross-entropy loss forms its outputs, the
   // seed gradient and the loss / accuracy sums in one launch.  Same results as the two calls.
   void forward_error_device(size_t const batch, float const *d_inputs, float const *d_targets);
+  // No counterpart in the reference: a second set of the per-batch buffers with a stream of its own, for a driver
+  // that runs the mini-batches of a training pass alternately on the two sets ("lanes"), so that the forward pass of
+  // a mini-batch overlaps the backward pass of the one before it.  Networks of plain fully connected layers on
+  // batches of at most 256 rows; false: not such a model, DLMI_LANES=0 in the environment, or no memory for it (the
+  // set counts against maximum_allowable_memory_bytes) - everything below is then a no-op on the one lane.
+  //   lane_forward_begin(k)  makes lane k (0 or 1) current and orders its forward pass behind the other lane's
+  //   lane_forward_end()     after forward_error_device()
+  //   lane_backward_begin()  orders the backward pass behind the other lane's; then backward_pass(),
+  //   lane_backward_end()    update_derivatives() and this
+  //   lanes_join()           end of the pass (before a capture ends, before anything else is asked of the model):
+  //                          lane 0 is current again and its stream waits for everything lane 1 was given
+  // Results are those of the same calls on one lane, bit for bit.
+  bool enable_lanes(size_t const batch);
+  bool lanes_enabled(void) const;
+  bool lane_forward_begin(int const k);
+  bool lane_forward_end(void);
+  bool lane_backward_begin(void);
+  bool lane_backward_end(void);
+  bool lanes_join(void);
   // The stream every kernel of this model is launched on (a hipStream_t), and a hash of
   // everything the kernels of one batch take by value or by address (layer settings,
   // hyper-parameters, propagation state, buffer addresses): two batches of the same size
@@ -446,6 +465,8 @@ class Model : public Model_State {
   int dropout_tail(Layer const &layer, size_t batch, size_t units, float *values);
   float const *outputs_of(size_t index_layer) const;
   void seed_error(size_t batch, float const *d_targets);
+  void free_lanes(void);
+  void select_lane(int const k);
   void free_batch(void);
   bool fail(char const *what) const;
 };

@@ -186,3 +186,47 @@ def test_weight_gradients_beside_the_chain_match_one_stream(lib, widths, max_bat
         one.close()
         two.close()
         rec.close()
+
+
+@pytest.mark.parametrize("widths,max_batch,n", [([20, 32, 24, 5], 16, 50), ([784, 512, 512, 10], 128, 1100), ([30, 40, 7], 8, 8)])
+def test_two_lanes_match_one(lib, widths, max_batch, n):
+    """The driver runs the mini-batches of a training pass alternately on two sets of per-batch buffers, each with a
+    stream of its own, so that a forward pass overlaps the backward pass before it; only forward-after-forward and
+    backward-after-backward are ordered.  A twin created with DLMI_LANES=0 has the one set: parameters, gradients,
+    moving statistics, reports, the outputs of the last mini-batch and evaluation passes must stay bit-identical
+    epoch after epoch, with plain launches and with recorded mini-batches (odd and even numbers of mini-batches, a
+    ragged last one, a single mini-batch)."""
+    import os
+    os.environ["DLMI_LANES"] = "0"
+    try:
+        one = build(lib, widths, max_batch=max_batch)
+    finally:
+        del os.environ["DLMI_LANES"]
+    two, rec = build(lib, widths, max_batch=max_batch), build(lib, widths, max_batch=max_batch)
+    X, Y = data(n, widths[0], widths[-1])
+    try:
+        for e in range(5):
+            r1 = one.train_epoch(X, Y, resample_masks=True, record_batches=False)
+            r2 = two.train_epoch(X, Y, resample_masks=True, record_batches=False)
+            r3 = rec.train_epoch(X, Y, resample_masks=True, record_batches=True)
+            assert r2 == r1 and r3[1] == r1[1] and r3[0] == pytest.approx(r1[0], rel=1e-9), f"epoch {e}: {r1} / {r2} / {r3}"
+            p1 = one.get_parameters()
+            assert np.array_equal(p1, two.get_parameters()), f"epoch {e}: parameters (plain launches)"
+            assert np.array_equal(p1, rec.get_parameters()), f"epoch {e}: parameters (recorded)"
+            m1 = one.get_moving()
+            for other in (two, rec):
+                mo = other.get_moving()
+                assert np.array_equal(m1[0], mo[0]) and np.array_equal(m1[1], mo[1]), f"epoch {e}: moving statistics"
+                assert np.array_equal(one.get_dparams(), other.get_dparams()), f"epoch {e}: gradients"
+                # what the last mini-batch left in the layers: its outputs (its rows), and the batch statistics
+                last_rows = n - (n - 1) // max_batch * max_batch
+                for m in (one, other):
+                    m.B = last_rows
+                assert np.array_equal(one.get_out(), other.get_out()), f"epoch {e}: outputs of the last mini-batch"
+                for k in range(4):
+                    assert np.array_equal(one.layer_vector(1, k), other.layer_vector(1, k)), f"epoch {e}: batch statistic {k}"
+            assert two.evalt(X, Y) == one.evalt(X, Y) and rec.evalt(X, Y) == one.evalt(X, Y)
+    finally:
+        one.close()
+        two.close()
+        rec.close()
