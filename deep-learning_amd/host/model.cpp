@@ -86,6 +86,7 @@ struct Model::Impl {
   };
   LaneSet other;
   bool lanes_ready = false;
+  bool lanes_wanted = true;  // DLMI_LANES, read when the model is compiled
   int lane = 0;
   hipEvent_t f_done[2] = {nullptr, nullptr}, b_done[2] = {nullptr, nullptr}, lane_fork = nullptr;
   bool f_rec[2] = {false, false}, b_rec[2] = {false, false}, forked = false;
@@ -400,8 +401,7 @@ void Model::free_lanes(void) {
 bool Model::enable_lanes(size_t const batch) {
   Impl &m = *impl_;
   if (m.lanes_ready) return true;
-  static bool const wanted = [] { char const *e = std::getenv("DLMI_LANES"); return e == nullptr || std::atoi(e) != 0; }();
-  if (!wanted || ptr_array_layers == nullptr || m.ctx == nullptr || m.allocated_batch == 0 || batch > m.allocated_batch ||
+  if (!m.lanes_wanted || ptr_array_layers == nullptr || m.ctx == nullptr || m.allocated_batch == 0 || batch > m.allocated_batch ||
       m.allocated_batch > kLaneMaxBatch)
     return false;
   for (size_t i = 1; i < total_layers; ++i)
@@ -554,6 +554,10 @@ bool Model::compile(size_t const n_layers, size_t const number_recurrent_depth_r
   }
   if (dlmi_ctx_create(&impl_->ctx, 0, impl_->stream) != DLMI_OK)
     return fail("compile: no gfx950 device / context (there is no CPU path)");
+  {
+    char const *const e = std::getenv("DLMI_LANES");
+    impl_->lanes_wanted = e == nullptr || std::atoi(e) != 0;
+  }
   {
     char const *const e = std::getenv("DLMI_DW_STREAM");
     bool const side = e == nullptr || std::atoi(e) != 0;
