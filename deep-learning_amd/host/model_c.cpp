@@ -181,6 +181,7 @@ void dlmi_model_memory(dlmi_model const *h, size_t *out) {
   out[2] = h->m.Get__Batch_Sizeof(1);
   out[3] = h->m.batch_size;
 }
+int dlmi_model_lanes_enabled(dlmi_model const *h) { return h->m.lanes_enabled() ? 1 : 0; }
 int dlmi_model_set_loss(dlmi_model *h, int loss, int accu, float accu_variance) {
   h->m.set_loss_fn(static_cast<LOSS_FN::TYPE>(loss));
   h->m.set_accu_fn(static_cast<ACCU_FN::TYPE>(accu));

@@ -231,6 +231,10 @@ class Model:
         self.lib.dlmi_model_memory(self.h, out)
         return dict(zip(("budget", "model_bytes", "bytes_per_example", "batch_size"), (int(v) for v in out)))
 
+    def lanes_enabled(self):
+        """Whether the epoch driver runs this model's mini-batches on two sets of per-batch buffers."""
+        return bool(self.lib.dlmi_model_lanes_enabled(self.h))
+
     def set_loss(self, loss, accu, acc_var=0.49):
         """set_loss_fn / set_accu_fn / Set__Accurancy_Variance (after prepare, which selects cross-entropy)."""
         self._ok(self.lib.dlmi_model_set_loss(self.h, c_int(loss), c_int(accu), c_f(acc_var)), "set_loss")

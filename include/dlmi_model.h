@@ -76,6 +76,8 @@ void dlmi_model_loss_accu(dlmi_model *m, size_t n_data, double *out);
  * assigned before dlmi_model_prepare; out[0..3] = that budget, Get__Sizeof(1, 0), Get__Batch_Sizeof(1), batch_size */
 void dlmi_model_set_allowable_memory(dlmi_model *m, size_t bytes);
 void dlmi_model_memory(dlmi_model const *m, size_t *out);
+/* 1 when the epoch driver has given the model its second set of per-batch buffers (Model::enable_lanes) */
+int dlmi_model_lanes_enabled(dlmi_model const *m);
 size_t dlmi_model_total_parameters(dlmi_model const *m);
 size_t dlmi_model_total_normalized_units(dlmi_model const *m);
 /* out[0..5] = first weight index, first bias index, gamma index, beta index, moving-stat index, Use__Bias() */

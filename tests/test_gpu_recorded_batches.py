@@ -230,3 +230,47 @@ def test_two_lanes_match_one(lib, widths, max_batch, n):
         one.close()
         two.close()
         rec.close()
+
+
+def test_which_models_get_a_second_lane(lib):
+    """Plain layers on mini-batches of at most 256 rows, when the memory budget holds a second set of buffers and
+    DLMI_LANES is not 0; everything else trains on the one set (and all of them train: the epoch must succeed)."""
+    import os
+    X, Y = data(40, 20, 5)
+
+    def trained(m):
+        r = m.train_epoch(X, Y)
+        assert np.isfinite(r[0])
+        return m.lanes_enabled()
+
+    m = build(lib, [20, 32, 24, 5])
+    try:
+        assert not m.lanes_enabled()  # only the driver asks for it
+        assert trained(m)
+    finally:
+        m.close()
+    m = build(lib, [20, 32, 24, 5], max_batch=512)  # more rows per mini-batch than launch latency is the bound for
+    try:
+        Xb, Yb = data(1100, 20, 5)
+        assert np.isfinite(m.train_epoch(Xb, Yb)[0]) and not m.lanes_enabled()
+    finally:
+        m.close()
+    os.environ["DLMI_LANES"] = "0"
+    try:
+        m = build(lib, [20, 32, 24, 5])
+    finally:
+        del os.environ["DLMI_LANES"]
+    try:
+        assert not trained(m)
+    finally:
+        m.close()
+    # a budget that holds the model and its one set of buffers, but not a second set
+    m = build(lib, [20, 32, 24, 5])
+    try:
+        mem = m.memory()
+        m.set_allowable_memory(mem["model_bytes"] + mem["bytes_per_example"] * 16 + mem["bytes_per_example"] * 8)
+        assert not trained(m)
+        m.set_allowable_memory(mem["model_bytes"] + mem["bytes_per_example"] * 16 * 4)
+        assert trained(m)
+    finally:
+        m.close()
