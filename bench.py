@@ -63,7 +63,7 @@ MEASURED_TRAFFIC_BYTES = {
 }
 TRAFFIC_SOURCES = ("gemm_f32_mfma.hip", "norm_kernels.hip", "norm_panel_fwd.hip", "norm_panel_bwd.hip",
                    "norm_panel_common.hpp", "norm_shared.hpp", "activations.hpp")
-TRAFFIC_SOURCES_SHA256 = "f6bc68e446a1086cff1edde897ef66cfa09e9cb4961672868bc4125556a7b95e"
+TRAFFIC_SOURCES_SHA256 = "48c05f5183b3d26d214f64b55281dd46a98d5ce2ec0c9634292690bb7012db7f"
 
 
 def traffic_sources_digest():

@@ -34,6 +34,7 @@ struct dlmi_tuning {
   size_t fold_fwd_epilogue_max_elements = size_t(1) << 22;
   int fc_narrow = 1;              // layers of at most 16 units on a mini-batch run the narrow-layer kernels (fc_small.hip)
   int norm_small = 1;             // mini-batches (at most 256 rows, 2^20 elements) run the one-launch small-batch kernels
+  int minibatch_dw = 1;           // weight gradients of a mini-batch (at most 256 rows, 2^20 weights) run the one-block-per-tile kernel of fc_small.hip
   int narrow_dx_fused = 1;        // ... which also form dY = dZn . Wn below a layer of at most 16 units themselves
 };
 
@@ -159,6 +160,10 @@ int narrow_fc_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, f
                   float *Q, float const *Y = nullptr, float *dZ = nullptr, double *stats = nullptr);
 int narrow_dw_try(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float *dW, float *db,
                   int accumulate);
+// The weight gradient of a layer of any width on a mini-batch (fc_small.hip): dW only, the bias gradient is the
+// caller's.  _try: 1 when launched, 0 when the shape or the operands do not qualify, < 0 on failure.
+bool minibatch_dw_eligible(dlmi_ctx const *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float const *dW);
+int minibatch_dw_try(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float *dW, int accumulate);
 // The fused backward of dlmi_fused_norm_act_bwd whose upstream gradient dY is still `nslices` partial products
 // [nslices][B][H] (split-K slices of the dX product above it); small-batch shapes only.
 int fused_bwd_from_slices(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,

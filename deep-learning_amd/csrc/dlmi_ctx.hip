@@ -81,6 +81,7 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
   t.fold_bwd = env_level("DLMI_NORM_FOLD_BWD", t.fold_bwd);
   t.norm_small = env_flag("DLMI_NORM_SMALL", t.norm_small);
   t.narrow_dx_fused = env_flag("DLMI_NARROW_DX_FUSED", t.narrow_dx_fused);
+  t.minibatch_dw = env_flag("DLMI_MINIBATCH_DW", t.minibatch_dw);
   t.fc_narrow = env_flag("DLMI_FC_NARROW", t.fc_narrow);
   if (env_flag("DLMI_GEMM_CLOCK", 0)) {
     void *p = nullptr;

@@ -9,6 +9,12 @@
 //                    backward pass in one launch;
 //   k_narrow_dw      dW (+)= dZ^T X and db (+)= column sums of dZ in one launch, a workgroup per 8 columns
 //                    of X for all rows (update_derivative_fwp_st.cpp:246-302).
+// and for a layer of ANY width on a mini-batch (at most 256 rows):
+//   k_minibatch_dw   dW (+)= dZ^T X, a workgroup per 64 x 64 block of dW: its 64 columns of dZ and of X for all rows
+//                    go into LDS once, the sum over the rows runs on the matrix pipe (v_mfma_f32_16x16x4_f32, the
+//                    rows in ascending groups of four).  The reduction of this product is the batch: a hundred
+//                    rows are eight K tiles of the tiled GEMM, which spends its time starting and draining its
+//                    pipeline (784 x 512 on 128 rows: 12.4 us there, about half of it here).
 // Sums run in a fixed order (no float atomics).  Citations: /root/reference/lib/deep-learning/v1/learner/.
 #include <hip/hip_runtime.h>
 
@@ -203,6 +209,117 @@ int narrow_fc_fwd(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X, f
   }
   DLMI_LAUNCH_CHECK(ctx, "k_narrow_fc_fwd");
   return DLMI_OK;
+}
+
+namespace {
+
+constexpr int kMbTile = 64;      // a workgroup's block of dW: 64 units x 64 inputs
+constexpr int kMbRows = 64;      // batch rows staged at a time (2 x 64 x 80 floats = 40 KB of LDS)
+constexpr int kMbStride = 80;    // floats between staged rows: 16 banks apart, so that the four rows a fragment
+                                 // read touches (two per half wavefront) never share a bank
+constexpr size_t kMbMaxRows = 256;
+constexpr size_t kMbMaxOutputs = size_t(1) << 20;  // H * K: larger layers go to the tiled GEMM
+
+typedef float mv4f __attribute__((ext_vector_type(4)));
+
+// dW[h][k] (+)= sum_b dZ[b][h] X[b][k].  Grid (ceil(K / 64), ceil(H / 64)), 256 threads = 4 wavefronts, each a
+// 32 x 32 quarter of the block as 2 x 2 MFMA tiles of 16 x 16.  H, K multiples of 4, 16-byte aligned operands.
+__global__ __launch_bounds__(256) void k_minibatch_dw(float const *__restrict__ X, float const *__restrict__ dZ,
+                                                       float *__restrict__ dW, unsigned B, unsigned K, unsigned H,
+                                                       int accumulate) {
+  __shared__ float zs[kMbRows * kMbStride];  // dZ[b][h0 .. h0 + 64)
+  __shared__ float xs[kMbRows * kMbStride];  // X [b][k0 .. k0 + 64)
+  unsigned const k0 = blockIdx.x * kMbTile, h0 = blockIdx.y * kMbTile;
+  int const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int const wh = (wave >> 1) * 32, wk = (wave & 1) * 32;  // this wavefront's quarter
+  int const li = lane & 15, lg = lane >> 4;               // position inside a 16 x 16 tile / group of rows
+  mv4f acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = mv4f{0.0f, 0.0f, 0.0f, 0.0f};
+  int const c4 = (threadIdx.x & 15) * 4, r0 = threadIdx.x >> 4;  // staging: 16 threads per row, 16 rows per sweep
+  // The rows go through LDS in passes of kMbRows; the loads of a pass are issued before the pass in front of it is
+  // multiplied, and all of a pass's loads before its first LDS store: one memory latency in all, not one per pass.
+  mv4f vz[kMbRows / 16], vx[kMbRows / 16];
+  auto fetch = [&](unsigned b0) {
+    unsigned const rows = B - b0 < static_cast<unsigned>(kMbRows) ? B - b0 : static_cast<unsigned>(kMbRows);
+#pragma unroll
+    for (int i = 0; i < kMbRows / 16; ++i) {
+      unsigned const r = r0 + 16 * i;
+      bool const row_ok = r < rows;
+      vz[i] = row_ok && h0 + c4 < H ? *reinterpret_cast<mv4f const *>(dZ + static_cast<size_t>(b0 + r) * H + h0 + c4) : mv4f{0, 0, 0, 0};
+      vx[i] = row_ok && k0 + c4 < K ? *reinterpret_cast<mv4f const *>(X + static_cast<size_t>(b0 + r) * K + k0 + c4) : mv4f{0, 0, 0, 0};
+    }
+  };
+  fetch(0);
+  // what is already in dW, asked for now: by the time the sums are formed it is there
+  mv4f was[2][2];
+#pragma unroll
+  for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        unsigned const h = h0 + wh + 16 * ti + 4 * lg + r, k = k0 + wk + 16 * tj + li;
+        was[ti][tj][r] = accumulate && h < H && k < K ? dW[static_cast<size_t>(h) * K + k] : 0.0f;
+      }
+  for (unsigned b0 = 0; b0 < B; b0 += kMbRows) {
+    unsigned const rows = B - b0 < static_cast<unsigned>(kMbRows) ? B - b0 : static_cast<unsigned>(kMbRows);
+    unsigned const rows4 = (rows + 3u) & ~3u;  // the matrix pipe takes rows in fours: the tail is zeros
+    if (b0 != 0) __syncthreads();              // everybody is done with the previous rows
+#pragma unroll
+    for (int i = 0; i < kMbRows / 16; ++i) {
+      unsigned const r = r0 + 16 * i;
+      if (r < rows4) {
+        *reinterpret_cast<mv4f *>(zs + r * kMbStride + c4) = vz[i];
+        *reinterpret_cast<mv4f *>(xs + r * kMbStride + c4) = vx[i];
+      }
+    }
+    __syncthreads();
+    if (b0 + kMbRows < B) fetch(b0 + kMbRows);
+    // A[i][kk] = dZ[b + kk][h0 + wh + 16 ti + i], B[kk][j] = X[b + kk][k0 + wk + 16 tj + j]: lane (li, lg) holds
+    // element (i = li, kk = lg) of A and (kk = lg, j = li) of B
+    float const *zr = zs + lg * kMbStride + wh + li;
+    float const *xr = xs + lg * kMbStride + wk + li;
+    for (unsigned b = 0; b < rows4; b += 4) {
+      float const a0 = zr[b * kMbStride], a1 = zr[b * kMbStride + 16], x0 = xr[b * kMbStride], x1 = xr[b * kMbStride + 16];
+      acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, x0, acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, x1, acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, x0, acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, x1, acc[1][1], 0, 0, 0);
+    }
+  }
+  // D[i = 4 lg + r][j = li] of every tile
+#pragma unroll
+  for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        unsigned const h = h0 + wh + 16 * ti + 4 * lg + r, k = k0 + wk + 16 * tj + li;
+        if (h < H && k < K) {
+          // (was is 0 without accumulation; 0 + x is x bit for bit, up to the sign of a zero sum)
+          dW[static_cast<size_t>(h) * K + k] = accumulate ? was[ti][tj][r] + acc[ti][tj][r] : acc[ti][tj][r];
+        }
+      }
+}
+
+}  // namespace
+
+bool minibatch_dw_eligible(dlmi_ctx const *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float const *dW) {
+  return ctx->tune.minibatch_dw != 0 && B <= kMbMaxRows && H * K <= kMbMaxOutputs && H % 4 == 0 && K % 4 == 0 &&
+         dlmi_aligned16(Xin) && dlmi_aligned16(dZ) && dW != nullptr;
+}
+
+int minibatch_dw_try(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float *dW, int accumulate) {
+  if (!minibatch_dw_eligible(ctx, B, K, H, Xin, dZ, dW)) return 0;
+  dim3 const grid(static_cast<unsigned>(dlmi_ceil_div(K, static_cast<size_t>(kMbTile))),
+                  static_cast<unsigned>(dlmi_ceil_div(H, static_cast<size_t>(kMbTile))));
+  hipLaunchKernelGGL(k_minibatch_dw, grid, dim3(256), 0, ctx->stream, Xin, dZ, dW, static_cast<unsigned>(B),
+                     static_cast<unsigned>(K), static_cast<unsigned>(H), accumulate);
+  DLMI_LAUNCH_CHECK(ctx, "k_minibatch_dw");
+  return 1;
 }
 
 int narrow_dw_try(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float *dW, float *db,

@@ -869,7 +869,10 @@ int dlmi_fc_bwd_dw(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin
   DLMI_REQUIRE(ctx, B > 0 && K > 0 && H > 0, "empty operand");
   // a narrow layer on a mini-batch: dW and db in one launch
   if (int const took = narrow_dw_try(ctx, B, K, H, Xin, dZ, dW, db, accumulate); took != 0) return took < 0 ? took : DLMI_OK;
-  int rc = gemm<false, false>(ctx, H, K, B, dZ, H, Xin, K, dW, nullptr, accumulate);
+  // any layer on a mini-batch: the reduction is the batch, a handful of K tiles; a kernel that stages it whole
+  int rc = minibatch_dw_try(ctx, B, K, H, Xin, dZ, dW, accumulate);
+  if (rc == 0) rc = gemm<false, false>(ctx, H, K, B, dZ, H, Xin, K, dW, nullptr, accumulate);
+  else rc = rc < 0 ? rc : DLMI_OK;
   if (rc != DLMI_OK || db == nullptr) return rc;
   // db[h] (+)= sum_b dZ[b,h] (update_derivative_fwp_st.cpp:283-302)
   return column_sums(ctx, B, H, dZ, db, accumulate);
@@ -890,6 +893,7 @@ int dlmi_fc_bwd_dw_grouped(dlmi_ctx *ctx, size_t n, dlmi_dw_problem const *probl
       DLMI_REQUIRE(ctx, pr[i].B > 0 && pr[i].K > 0 && pr[i].H > 0, "empty operand");
       item[i] = GroupItem{pr[i].H, pr[i].K, pr[i].B, pr[i].dZ, pr[i].Xin, pr[i].dW};
       variant[i] = group_variant<false, false>(ctx, item[i]);  // (a narrow layer is no multiple of a tile: -1)
+      if (minibatch_dw_eligible(ctx, pr[i].B, pr[i].K, pr[i].H, pr[i].Xin, pr[i].dZ, pr[i].dW)) variant[i] = -1;  // its own kernel
     }
     for (size_t i = 0; i < m; ++i) {
       if (variant[i] == -2) continue;  // went with an earlier one

@@ -147,3 +147,40 @@ def test_output_layer_forward_with_the_seed_gradient(twins, pkg, B, K, H):
     # without accumulators
     Z1, Q1, dZ1 = fast.fc_softmax_ce_fwd(X, W, Y, bias=b)
     assert torch.equal(dZ1, fast.softmax_ce_seed(fast.fc_softmax_fwd(X, W, b)[1], Y))
+
+
+@pytest.mark.parametrize("B,K,H", [(128, 784, 512), (128, 512, 512), (256, 64, 64), (1, 4, 20), (7, 100, 36), (130, 68, 132),
+                                   (255, 1000, 24), (64, 2048, 512), (3, 8, 4)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_minibatch_weight_gradient(pkg, B, K, H, accumulate):
+    """dW (+)= dZ^T X of a layer of any width on a mini-batch (k_minibatch_dw: one workgroup per 64 x 64 block of dW,
+    the batch staged in LDS, the sum over the rows on the matrix pipe) against float64 and against the tiled GEMM
+    of the same library (a context created with DLMI_MINIBATCH_DW=0); ragged blocks, batches that are no multiple of
+    four, more than one staging pass; bit-reproducible; the bias gradient behind it unchanged."""
+    os.environ["DLMI_MINIBATCH_DW"] = "0"
+    try:
+        plain = pkg.Dlmi(0)
+    finally:
+        del os.environ["DLMI_MINIBATCH_DW"]
+    fast = pkg.Dlmi(0)
+    try:
+        rng = np.random.default_rng(B + 3 * K + 7 * H)
+        X = rng.standard_normal((B, K)).astype(np.float32)
+        dZ = rng.standard_normal((B, H)).astype(np.float32)
+        dW0 = rng.standard_normal((H, K)).astype(np.float32)
+        db0 = rng.standard_normal(H).astype(np.float32)
+        want = dZ.astype(np.float64).T @ X.astype(np.float64) + (dW0 if accumulate else 0.0)
+        want_db = dZ.astype(np.float64).sum(0) + (db0 if accumulate else 0.0)
+        outs = []
+        for dl in (fast, plain, fast):
+            dW, db = dev(dW0), dev(db0)
+            dl.fc_bwd_dw(dev(X), dev(dZ), dW=dW, db=db, accumulate=accumulate)
+            dl.synchronize()
+            outs.append((dW.cpu().numpy(), db.cpu().numpy()))
+        assert_close(outs[0][0], want, 1e-5, "dW vs float64", floor=1.0)
+        assert_close(outs[0][0], outs[1][0], 1e-5, "dW vs tiled GEMM", floor=1.0)
+        assert_close(outs[0][1], want_db, 1e-5, "db vs float64", floor=1.0)
+        assert np.array_equal(outs[0][0], outs[2][0]) and np.array_equal(outs[0][1], outs[2][1]), "not reproducible"
+    finally:
+        fast.close()
+        plain.close()
