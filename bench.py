@@ -63,7 +63,7 @@ MEASURED_TRAFFIC_BYTES = {
 }
 TRAFFIC_SOURCES = ("gemm_f32_mfma.hip", "norm_kernels.hip", "norm_panel_fwd.hip", "norm_panel_bwd.hip",
                    "norm_panel_common.hpp", "norm_shared.hpp", "activations.hpp")
-TRAFFIC_SOURCES_SHA256 = "48c05f5183b3d26d214f64b55281dd46a98d5ce2ec0c9634292690bb7012db7f"
+TRAFFIC_SOURCES_SHA256 = "2074036494ba3a86470d8887086dadad2e41187338f457107517d6f5bdb77b44"
 
 
 def traffic_sources_digest():

@@ -164,6 +164,14 @@ int narrow_dw_try(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin,
 // caller's.  _try: 1 when launched, 0 when the shape or the operands do not qualify, < 0 on failure.
 bool minibatch_dw_eligible(dlmi_ctx const *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float const *dW);
 int minibatch_dw_try(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float *dW, int accumulate);
+// ... of several layers in one launch (every problem must be minibatch_dw_eligible; same bits as one by one)
+constexpr int kMinibatchDwGroupMax = 8;
+struct MinibatchDwProblem {
+  size_t B, K, H;
+  float const *X, *dZ;
+  float *dW;
+};
+int minibatch_dw_group(dlmi_ctx *ctx, size_t n, MinibatchDwProblem const *problems, int accumulate);
 // The fused backward of dlmi_fused_norm_act_bwd whose upstream gradient dY is still `nslices` partial products
 // [nslices][B][H] (split-K slices of the dX product above it); small-batch shapes only.
 int fused_bwd_from_slices(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,

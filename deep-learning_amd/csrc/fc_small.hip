@@ -224,12 +224,12 @@ typedef float mv4f __attribute__((ext_vector_type(4)));
 
 // dW[h][k] (+)= sum_b dZ[b][h] X[b][k].  Grid (ceil(K / 64), ceil(H / 64)), 256 threads = 4 wavefronts, each a
 // 32 x 32 quarter of the block as 2 x 2 MFMA tiles of 16 x 16.  H, K multiples of 4, 16-byte aligned operands.
-__global__ __launch_bounds__(256) void k_minibatch_dw(float const *__restrict__ X, float const *__restrict__ dZ,
-                                                       float *__restrict__ dW, unsigned B, unsigned K, unsigned H,
-                                                       int accumulate) {
+__device__ __forceinline__ void minibatch_dw_block(float const *__restrict__ X, float const *__restrict__ dZ,
+                                                   float *__restrict__ dW, unsigned B, unsigned K, unsigned H,
+                                                   int accumulate, unsigned block_k, unsigned block_h) {
   __shared__ float zs[kMbRows * kMbStride];  // dZ[b][h0 .. h0 + 64)
   __shared__ float xs[kMbRows * kMbStride];  // X [b][k0 .. k0 + 64)
-  unsigned const k0 = blockIdx.x * kMbTile, h0 = blockIdx.y * kMbTile;
+  unsigned const k0 = block_k * kMbTile, h0 = block_h * kMbTile;
   int const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int const wh = (wave >> 1) * 32, wk = (wave & 1) * 32;  // this wavefront's quarter
   int const li = lane & 15, lg = lane >> 4;               // position inside a 16 x 16 tile / group of rows
@@ -305,7 +305,56 @@ __global__ __launch_bounds__(256) void k_minibatch_dw(float const *__restrict__ 
       }
 }
 
+__global__ __launch_bounds__(256) void k_minibatch_dw(float const *__restrict__ X, float const *__restrict__ dZ,
+                                                       float *__restrict__ dW, unsigned B, unsigned K, unsigned H,
+                                                       int accumulate) {
+  minibatch_dw_block(X, dZ, dW, B, K, H, accumulate, blockIdx.x, blockIdx.y);
+}
+
+// Several such products in one launch (the layers of a network after its backward pass): the workgroups walk the
+// concatenated lists of blocks.  A block's arithmetic is that of the single launch.
+struct MbDwGroupArgs {
+  struct Problem {
+    float const *X, *dZ;
+    float *dW;
+    unsigned B, K, H, blocks_k, block_end;  // block_end: this problem's blocks end before this linear workgroup id
+  };
+  Problem p[kMinibatchDwGroupMax];
+  unsigned n;
+  int accumulate;
+};
+__global__ __launch_bounds__(256) void k_minibatch_dw_group(MbDwGroupArgs a) {
+  unsigned i = 0;
+  while (i + 1 < a.n && blockIdx.x >= a.p[i].block_end) ++i;
+  MbDwGroupArgs::Problem const &q = a.p[i];
+  unsigned const local = blockIdx.x - (i == 0 ? 0u : a.p[i - 1].block_end);
+  minibatch_dw_block(q.X, q.dZ, q.dW, q.B, q.K, q.H, a.accumulate, local % q.blocks_k, local / q.blocks_k);
+}
+
 }  // namespace
+
+int minibatch_dw_group(dlmi_ctx *ctx, size_t n, MinibatchDwProblem const *problems, int accumulate) {
+  for (size_t first = 0; first < n; first += kMinibatchDwGroupMax) {
+    MbDwGroupArgs a;
+    a.n = static_cast<unsigned>(n - first < static_cast<size_t>(kMinibatchDwGroupMax) ? n - first : kMinibatchDwGroupMax);
+    a.accumulate = accumulate;
+    unsigned total = 0;
+    for (unsigned i = 0; i < a.n; ++i) {
+      MinibatchDwProblem const &s = problems[first + i];
+      if (!minibatch_dw_eligible(ctx, s.B, s.K, s.H, s.X, s.dZ, s.dW)) return dlmi_fail(ctx, DLMI_E_INVALID, "minibatch_dw_group: problem %u does not qualify", i);
+      MbDwGroupArgs::Problem &q = a.p[i];
+      q.X = s.X; q.dZ = s.dZ; q.dW = s.dW;
+      q.B = static_cast<unsigned>(s.B); q.K = static_cast<unsigned>(s.K); q.H = static_cast<unsigned>(s.H);
+      q.blocks_k = static_cast<unsigned>(dlmi_ceil_div(s.K, static_cast<size_t>(kMbTile)));
+      total += q.blocks_k * static_cast<unsigned>(dlmi_ceil_div(s.H, static_cast<size_t>(kMbTile)));
+      q.block_end = total;
+    }
+    for (unsigned i = a.n; i < static_cast<unsigned>(kMinibatchDwGroupMax); ++i) a.p[i] = a.p[a.n - 1];
+    hipLaunchKernelGGL(k_minibatch_dw_group, dim3(total), dim3(256), 0, ctx->stream, a);
+    DLMI_LAUNCH_CHECK(ctx, "k_minibatch_dw_group");
+  }
+  return DLMI_OK;
+}
 
 bool minibatch_dw_eligible(dlmi_ctx const *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float const *dW) {
   return ctx->tune.minibatch_dw != 0 && B <= kMbMaxRows && H * K <= kMbMaxOutputs && H % 4 == 0 && K % 4 == 0 &&

@@ -895,6 +895,23 @@ int dlmi_fc_bwd_dw_grouped(dlmi_ctx *ctx, size_t n, dlmi_dw_problem const *probl
       variant[i] = group_variant<false, false>(ctx, item[i]);  // (a narrow layer is no multiple of a tile: -1)
       if (minibatch_dw_eligible(ctx, pr[i].B, pr[i].K, pr[i].H, pr[i].Xin, pr[i].dZ, pr[i].dW)) variant[i] = -1;  // its own kernel
     }
+    // the mini-batch products that are not narrow layers (those bring their bias gradient along in a kernel of
+    // their own): one launch for all of them, from two on
+    {
+      MinibatchDwProblem mb[kMaxProblems];
+      size_t which[kMaxProblems], nmb = 0;
+      for (size_t i = 0; i < m; ++i)
+        if (variant[i] == -1 && pr[i].H > 16 &&
+            minibatch_dw_eligible(ctx, pr[i].B, pr[i].K, pr[i].H, pr[i].Xin, pr[i].dZ, pr[i].dW)) {
+          which[nmb] = i;
+          mb[nmb++] = MinibatchDwProblem{pr[i].B, pr[i].K, pr[i].H, pr[i].Xin, pr[i].dZ, pr[i].dW};
+        }
+      if (nmb >= 2) {
+        int rc = minibatch_dw_group(ctx, nmb, mb, accumulate);
+        if (rc != DLMI_OK) return rc;
+        for (size_t j = 0; j < nmb; ++j) variant[which[j]] = -2;  // done; the bias gradients follow below
+      }
+    }
     for (size_t i = 0; i < m; ++i) {
       if (variant[i] == -2) continue;  // went with an earlier one
       GroupItem same[kMaxProblems];

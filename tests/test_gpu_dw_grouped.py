@@ -32,6 +32,9 @@ MIXES = {
     # split over K go alone
     "mixed": [(256, 512, 256), (256, 256, 512), (128, 784, 512), (128, 512, 10), (8192, 128, 128), (256, 512, 256)],
     "single": [(512, 256, 256)],
+    # the layers of a network on a mini-batch: the products of any width share one launch of the mini-batch kernel
+    # (ragged blocks, a batch that is no multiple of four among them), the narrow output layer goes alone
+    "mini-batch": [(128, 784, 512), (128, 512, 512), (128, 512, 10), (100, 36, 24), (255, 64, 64), (128, 512, 512)],
 }
 
 
