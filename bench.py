@@ -63,7 +63,7 @@ MEASURED_TRAFFIC_BYTES = {
 }
 TRAFFIC_SOURCES = ("gemm_f32_mfma.hip", "norm_kernels.hip", "norm_panel_fwd.hip", "norm_panel_bwd.hip",
                    "norm_panel_common.hpp", "norm_shared.hpp", "activations.hpp")
-TRAFFIC_SOURCES_SHA256 = "2074036494ba3a86470d8887086dadad2e41187338f457107517d6f5bdb77b44"
+TRAFFIC_SOURCES_SHA256 = "4d454462d71e057d77560cbef62f2d1f49c51d9adfcdeb536578b8dace089a08"
 
 
 def traffic_sources_digest():
@@ -305,6 +305,33 @@ def layer_inputs(name):
         t["inf_mean"] = rng.uniform(10, (H,), -1.0, 1.0)
         t["inf_std"] = rng.uniform(11, (H,), 0.5, 2.0)  # the "variance" array holds standard deviations
     return t
+
+
+def workgroup_timeline(dl, step, part):
+    """Profiling aid: when the workgroups of the last product launch started and ended, by the kernel's own stamps."""
+    import ctypes
+    import numpy as np
+    M, N, K = {"gemm_fwd": (step.B, step.H, step.K), "gemm_dx": (step.B, step.K, step.H)}.get(part, (step.H, step.K, step.B))
+    tm, tn, ks, rs = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_uint(0), ctypes.c_int(0)
+    sz = ctypes.c_size_t
+    dl._ck(dl.lib.dlmi_gemm_plan(ctypes.c_int(dl.compute_units()), sz(M), sz(N), sz(K), ctypes.byref(tm), ctypes.byref(tn),
+                                 ctypes.byref(ks), ctypes.byref(rs)))
+    n = min(4096, -(-M // tm.value) * -(-N // tn.value))
+    a = dl.gemm_timeline(n)
+    t0 = a[:, 0].min()
+    start, issued, done = ((a[:, i] - t0) / 100.0 for i in range(3))
+    where = a[:, 3] >> 32 << 16 | (a[:, 3] >> 8 & 0xff)  # XCD, shader engine / array / CU
+    cus = dl.compute_units()
+    out = ["%s %d x %d x %d: %d workgroups of %d x %d (%d K slices) on %d CUs; first start to last acknowledged store %.1f us; "
+           "tile at the matrix peak %.2f us" % (part, M, N, K, n, tm.value, tn.value, ks.value, len(set(where.tolist())),
+                                                done.max(), 2.0 * tm.value * tn.value * K / ks.value / (157.3e12 / cus) * 1e6)]
+    for lo in range(0, n, cus):
+        sl = slice(lo, min(n, lo + cus))
+        out.append("  workgroups %4d..%4d: start %5.1f / %5.1f / %5.1f us, lifetime %5.1f / %5.1f / %5.1f us (min / median / max), "
+                   "last store acknowledged %.2f us after its issue"
+                   % (lo, sl.stop - 1, start[sl].min(), np.median(start[sl]), start[sl].max(), (done - start)[sl].min(),
+                      np.median((done - start)[sl]), (done - start)[sl].max(), np.median((done - issued)[sl])))
+    return "\n".join(out)
 
 
 class LayerStep:
@@ -576,6 +603,7 @@ def run_layer(args, torch, pkg, dl, name, full):
             mhz, us = dl.gemm_clock()
             print("%s: engine clock inside the launch %.0f MHz (first tile's workgroup lived %.1f us)" % (args.only, mhz, us),
                   file=sys.stderr)
+            print(workgroup_timeline(dl, step, args.only), file=sys.stderr)
         return None
 
     # ---- one clean step on the fresh inputs: the results the CPU baseline is compared with

@@ -45,7 +45,7 @@ C_ABI_SYMBOLS = [
     "dlmi_fused_norm_act_fwd_noalloc", "dlmi_fused_norm_act_residual_fwd", "dlmi_fc_norm_act_residual_fwd",
     "dlmi_fc_softmax_fwd", "dlmi_fc_softmax_ce_fwd", "dlmi_fc_bwd_dx_norm_act_bwd",
     "dlmi_ctx_reserve_layer", "dlmi_ctx_scratch_generation", "dlmi_ctx_norm_panel_enabled", "dlmi_ctx_norm_panel_poke",
-    "dlmi_fc_bwd_dw_grouped", "dlmi_fused_norm_act_bwd_db", "dlmi_ctx_gemm_clock", "dlmi_probe_strip_stream",
+    "dlmi_fc_bwd_dw_grouped", "dlmi_fused_norm_act_bwd_db", "dlmi_ctx_gemm_clock", "dlmi_ctx_gemm_timeline", "dlmi_probe_strip_stream",
 ]
 
 
@@ -146,6 +146,14 @@ class Dlmi:
         mhz, us = ctypes.c_double(0), ctypes.c_double(0)
         self._ck(self.lib.dlmi_ctx_gemm_clock(self.ctx, ctypes.byref(mhz), ctypes.byref(us)))
         return mhz.value, us.value
+
+    def gemm_timeline(self, workgroups):
+        """[workgroups, 4] int64: per workgroup of the last product launched the 100 MHz counter at entry, after its
+        last store was issued and after it was acknowledged, and XCC_ID << 32 | HW_ID (DLMI_GEMM_CLOCK=1 contexts)."""
+        import numpy as np
+        buf = (ctypes.c_ulonglong * (4 * workgroups))()
+        self._ck(self.lib.dlmi_ctx_gemm_timeline(self.ctx, buf, ctypes.c_size_t(workgroups)))
+        return np.frombuffer(buf, dtype=np.uint64).reshape(workgroups, 4).astype(np.int64)
 
     def norm_panel_enabled(self):
         """Whether this context may still launch the single-launch normalization kernels."""

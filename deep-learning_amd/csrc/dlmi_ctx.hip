@@ -85,9 +85,9 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
   t.fc_narrow = env_flag("DLMI_FC_NARROW", t.fc_narrow);
   if (env_flag("DLMI_GEMM_CLOCK", 0)) {
     void *p = nullptr;
-    if (hipMalloc(&p, 2 * sizeof(unsigned long long)) == hipSuccess) {
+    if (hipMalloc(&p, (2 + 4 * 4096) * sizeof(unsigned long long)) == hipSuccess) {
       ctx->gemm_clock = static_cast<unsigned long long *>(p);
-      (void)hipMemset(p, 0, 2 * sizeof(unsigned long long));
+      (void)hipMemset(p, 0, (2 + 4 * 4096) * sizeof(unsigned long long));
     } else {
       (void)hipGetLastError();
     }
@@ -187,6 +187,15 @@ int dlmi_ctx_gemm_clock(dlmi_ctx *ctx, double *engine_mhz, double *tile_us) {
   double const us = static_cast<double>(t[1]) / 100.0;  // the reference counter runs at 100 MHz
   if (tile_us != nullptr) *tile_us = us;
   if (engine_mhz != nullptr) *engine_mhz = static_cast<double>(t[0]) / us;
+  return DLMI_OK;
+}
+
+int dlmi_ctx_gemm_timeline(dlmi_ctx *ctx, unsigned long long *out, size_t workgroups) {
+  if (ctx == nullptr || out == nullptr) return DLMI_E_INVALID;
+  DLMI_REQUIRE(ctx, ctx->gemm_clock != nullptr, "the context was created without DLMI_GEMM_CLOCK=1");
+  DLMI_REQUIRE(ctx, workgroups <= 4096, "at most 4096 workgroups are kept");
+  DLMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  DLMI_HIP(ctx, hipMemcpy(out, ctx->gemm_clock + 2, 4 * workgroups * sizeof(unsigned long long), hipMemcpyDeviceToHost));
   return DLMI_OK;
 }
 

@@ -56,6 +56,7 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int kGemmThreads = 256;  // of the 4-wavefront workgroups; the 8-wavefront ones have twice as many
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8;
+constexpr unsigned kClockWgs = 4096;  // workgroups whose time stamps a clocked launch keeps
 
 struct GemmArgs {
   float const *A;
@@ -72,7 +73,10 @@ struct GemmArgs {
   float const *snap_a, *snap_b;
   float *snap_out;
   // optional: the workgroup of tile 0 / slice 0 stores {engine clock ticks, 100 MHz reference ticks} it spent from
-  // entry to its last store (measurement aid: the engine clock inside this very launch, no profiler attached)
+  // entry to its last store (measurement aid: the engine clock inside this very launch, no profiler attached);
+  // behind these two words every workgroup of slice 0 (the first kClockWgs) leaves four more: the 100 MHz counter
+  // at its entry, after its last store was issued and after that store was acknowledged, and where it ran
+  // (XCC_ID << 32 | HW_ID)
   unsigned long long *clock_out;
   int accumulate;      // C += result (only when gridDim.z == 1)
   int a_vec, b_vec;    // operand base and leading dimension allow 16-byte loads (ragged variant)
@@ -499,7 +503,20 @@ void k_gemm_f32(GemmArgs g) {
     lid = on_xcd % ntiles;
     zslice = (on_xcd / ntiles) * kXcds + linear % kXcds;
   }
+  bool const stamp = g.clock_out != nullptr && blockIdx.z == 0 && blockIdx.x < kClockWgs;
+  unsigned long long ts = 0;
+  if (stamp) ts = __builtin_amdgcn_s_memrealtime();
   gemm_tile<BM, BN, BK, A_KCONTIG, B_KCONTIG, MODE, RST, WVM>(g, lid, zslice, gridDim.z, lds);
+  if (stamp && threadIdx.x == 0) {
+    unsigned long long const te = __builtin_amdgcn_s_memrealtime();
+    __builtin_amdgcn_s_waitcnt(0);
+    unsigned long long const td = __builtin_amdgcn_s_memrealtime();
+    unsigned hw, xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    unsigned long long *o = g.clock_out + 2 + 4 * static_cast<size_t>(blockIdx.x);
+    o[0] = ts; o[1] = te; o[2] = td; o[3] = (static_cast<unsigned long long>(xcc) << 32) | hw;
+  }
 }
 
 // Several independent products of one kernel variant in ONE launch (the weight gradients of a network's layers:

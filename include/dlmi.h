@@ -104,6 +104,13 @@ int dlmi_ctx_norm_panel_enabled(dlmi_ctx const *ctx);
  * (ticks / time) and that workgroup's lifetime in microseconds: the clock INSIDE the launch, with no profiler
  * attached.  DLMI_E_INVALID without the environment variable or before the first product. */
 int dlmi_ctx_gemm_clock(dlmi_ctx *ctx, double *engine_mhz, double *tile_us);
+/* Measurement aid, no counterpart in the reference.  In such a context every workgroup of a product launch (K slice 0,
+ * the first 4096 workgroups) also leaves four 64-bit words: the 100 MHz counter at its entry, after its last store
+ * was issued and after that store was acknowledged, and where it ran (XCC_ID << 32 | HW_ID).
+ * dlmi_ctx_gemm_timeline waits for the stream and copies the words of the first `workgroups` workgroups of the last
+ * product launched to `out` [workgroups][4]: which workgroups shared a CU, how long each lived and when the next
+ * one took its place.  DLMI_E_INVALID without the environment variable or for more than 4096 workgroups. */
+int dlmi_ctx_gemm_timeline(dlmi_ctx *ctx, unsigned long long *out, size_t workgroups);
 /* Measurement aid, no counterpart in the reference.  y = x (x2 == NULL) or y = x + x2 on [B, H] fp32, by 256
  * workgroups that walk the tensors the way the single-launch normalization kernels do (each XCD its eighth of the
  * columns in panels of 64, each of its 32 workgroups its 32nd of the rows) and do nothing else with the data: the
