@@ -56,14 +56,14 @@ LAYER_WORKLOADS = {
 MIB = 1024.0 * 1024.0
 TRAFFIC_PROFILE = "profiles/hbm_traffic_pmc.md"
 MEASURED_TRAFFIC_BYTES = {
-    "c3": {"gemm": (898.0 + 897.3 + 832.8) / 3.0 * MIB, "norm_act": (259.1 + 388.4) * MIB},
+    "c3": {"gemm": (898.0 + 898.4 + 832.8) / 3.0 * MIB, "norm_act": (259.1 + 388.4) * MIB},
     "c2": {"norm_act": 326.8 * MIB},
-    "c4": {"gemm": (72.1 + 72.1 + 64.1) / 3.0 * MIB, "norm_act": 73.6 * MIB},
-    "c5": {"gemm": (132.2 + 132.5 + 144.1 + 16.3) / 3.0 * MIB, "norm_act": 513.6 * MIB},
+    "c4": {"gemm": (72.5 + 72.1 + 64.1) / 3.0 * MIB, "norm_act": 73.6 * MIB},
+    "c5": {"gemm": (132.1 + 132.3 + 144.1 + 16.3) / 3.0 * MIB, "norm_act": 513.6 * MIB},
 }
 TRAFFIC_SOURCES = ("gemm_f32_mfma.hip", "norm_kernels.hip", "norm_panel_fwd.hip", "norm_panel_bwd.hip",
                    "norm_panel_common.hpp", "norm_shared.hpp", "activations.hpp")
-TRAFFIC_SOURCES_SHA256 = "4d454462d71e057d77560cbef62f2d1f49c51d9adfcdeb536578b8dace089a08"
+TRAFFIC_SOURCES_SHA256 = "0fa2b2935a546238a0160066cd1b162c3b579a227d62fad1adadb5b2acd3101b"
 
 
 def traffic_sources_digest():

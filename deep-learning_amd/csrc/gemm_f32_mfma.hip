@@ -327,12 +327,15 @@ __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid,
     auto load_b = [&](int t) {
       return tile_load<BN, BK, B_KCONTIG, MODE, THREADS>(g.B, g.ldb, n0, k_begin + static_cast<size_t>(t) * BK, g.N, k_end, g.b_vec != 0);
     };
-    typename TA::Regs ra = load_a(0), ra2 = ra;
-    typename TB::Regs rb = load_b(0), rb2 = rb;
-    tile_store<BM, BK, A_KCONTIG, THREADS>(lds, ra);
-    tile_store<BN, BK, B_KCONTIG, THREADS>(lds + TA::kFloats, rb);
-    // one register stage: ra/rb hold tile kt+1 at the start of tile kt.  Two: tile kt+1 is in ra/rb for even
+    // The loads of the first two (with two register stages: three) K tiles are issued back to back and only
+    // the first is waited for before it goes to LDS: a workgroup's start costs one trip to memory, not two
+    // (the loads of a wavefront return in the order of their issue).
+    // One register stage: ra/rb hold tile kt+1 at the start of tile kt.  Two: tile kt+1 is in ra/rb for even
     // kt and in ra2/rb2 for odd kt, tile kt+2 in the other pair.
+    typename TA::Regs const r0a = load_a(0);
+    typename TB::Regs const r0b = load_b(0);
+    typename TA::Regs ra = {}, ra2 = {};
+    typename TB::Regs rb = {}, rb2 = {};
     if (ktiles > 1) {
       ra = load_a(1);
       rb = load_b(1);
@@ -343,6 +346,8 @@ __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid,
         rb2 = load_b(2);
       }
     }
+    tile_store<BM, BK, A_KCONTIG, THREADS>(lds, r0a);
+    tile_store<BN, BK, B_KCONTIG, THREADS>(lds + TA::kFloats, r0b);
     __syncthreads();
     v4f f0a[TM], f0b[TN];
     frags(lds, lds + TA::kFloats, 0, f0a, f0b);
