@@ -63,7 +63,7 @@ MEASURED_TRAFFIC_BYTES = {
 }
 TRAFFIC_SOURCES = ("gemm_f32_mfma.hip", "norm_kernels.hip", "norm_panel_fwd.hip", "norm_panel_bwd.hip",
                    "norm_panel_common.hpp", "norm_shared.hpp", "activations.hpp")
-TRAFFIC_SOURCES_SHA256 = "0fa2b2935a546238a0160066cd1b162c3b579a227d62fad1adadb5b2acd3101b"
+TRAFFIC_SOURCES_SHA256 = "9f8fa7cae32453e0bb3d8a7ed1e12925231704ccde9c50dc7b97c25851f93a3c"
 
 
 def traffic_sources_digest():

@@ -171,7 +171,16 @@ struct MinibatchDwProblem {
   float const *X, *dZ;
   float *dW;
 };
-int minibatch_dw_group(dlmi_ctx *ctx, size_t n, MinibatchDwProblem const *problems, int accumulate);
+// `narrow`: optionally the weight and bias gradient (db may be null) of one narrow layer (narrow_dw_eligible: at most
+// 16 units, 256 rows) rides along in the first launch, computed as the narrow-layer kernel of its own would
+struct NarrowDwProblem {
+  size_t B, K, H;
+  float const *X, *dZ;
+  float *dW, *db;
+};
+bool narrow_dw_eligible(dlmi_ctx const *ctx, size_t B, size_t H);
+int minibatch_dw_group(dlmi_ctx *ctx, size_t n, MinibatchDwProblem const *problems, int accumulate,
+                       NarrowDwProblem const *narrow = nullptr);
 // The fused backward of dlmi_fused_norm_act_bwd whose upstream gradient dY is still `nslices` partial products
 // [nslices][B][H] (split-K slices of the dX product above it); small-batch shapes only.
 int fused_bwd_from_slices(dlmi_ctx *ctx, dlmi_fused_desc const *desc, size_t B, size_t H, float const *x,

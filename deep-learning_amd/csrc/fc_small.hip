@@ -118,18 +118,22 @@ __global__ __launch_bounds__(kNarrowFwdThreads) void k_narrow_fc_fwd(float const
 
 constexpr int kDwCols = 8, kDwGroups = 32;
 
-// dW[o][j] (+)= sum_b dZ[b][o] X[b][j], db[o] (+)= sum_b dZ[b][o].  B <= 256, H <= 16.
-__global__ __launch_bounds__(kNarrowThreads) void k_narrow_dw(float const *__restrict__ X, float const *__restrict__ dZ,
-                                                               float *__restrict__ dW, float *__restrict__ db, size_t B,
-                                                               size_t K, int H, int accumulate) {
-  constexpr int kStride = kNarrowMaxUnits + 1;
-  __shared__ float dz[kNarrowMaxRowsDw * kStride];
-  __shared__ float red[kDwGroups][kNarrowMaxUnits][kDwCols];
+// dW[o][j] (+)= sum_b dZ[b][o] X[b][j], db[o] (+)= sum_b dZ[b][o].  B <= 256, H <= 16.  Workgroup `block` of
+// ceil(K / 8) forms 8 columns of dW, workgroup 0 also db.  lds: kNarrowDwLds floats.
+constexpr int kNarrowDwStride = kNarrowMaxUnits + 1;
+constexpr int kNarrowDwLds = static_cast<int>(kNarrowMaxRowsDw) * kNarrowDwStride + kDwGroups * kNarrowMaxUnits * kDwCols;
+__device__ __forceinline__ void narrow_dw_block(float const *__restrict__ X, float const *__restrict__ dZ,
+                                                float *__restrict__ dW, float *__restrict__ db, size_t B, size_t K,
+                                                int H, int accumulate, unsigned block, float *__restrict__ lds) {
+  constexpr int kStride = kNarrowDwStride;
+  float *const dz = lds;  // [B][kStride]
+  float (*const red)[kNarrowMaxUnits][kDwCols] =
+      reinterpret_cast<float (*)[kNarrowMaxUnits][kDwCols]>(lds + kNarrowMaxRowsDw * kStride);  // [kDwGroups]
   for (size_t i = threadIdx.x; i < B * static_cast<size_t>(H); i += kNarrowThreads)
     dz[(i / H) * kStride + (i % H)] = dZ[i];
   __syncthreads();
   int const c = threadIdx.x % kDwCols, rg = threadIdx.x / kDwCols;
-  size_t const col = static_cast<size_t>(blockIdx.x) * kDwCols + c;
+  size_t const col = static_cast<size_t>(block) * kDwCols + c;
   float acc[kNarrowMaxUnits];
 #pragma unroll
   for (int o = 0; o < kNarrowMaxUnits; ++o) acc[o] = 0.0f;
@@ -146,7 +150,7 @@ __global__ __launch_bounds__(kNarrowThreads) void k_narrow_dw(float const *__res
   __syncthreads();
   if (static_cast<int>(threadIdx.x) < H * kDwCols) {
     int const o = threadIdx.x / kDwCols, cc = threadIdx.x % kDwCols;
-    size_t const j = static_cast<size_t>(blockIdx.x) * kDwCols + cc;
+    size_t const j = static_cast<size_t>(block) * kDwCols + cc;
     if (j < K) {
       float t = 0.0f;
 #pragma unroll
@@ -155,12 +159,19 @@ __global__ __launch_bounds__(kNarrowThreads) void k_narrow_dw(float const *__res
       *dst = accumulate ? *dst + t : t;
     }
   }
-  if (db != nullptr && blockIdx.x == 0 && static_cast<int>(threadIdx.x) >= kNarrowThreads - H) {
+  if (db != nullptr && block == 0 && static_cast<int>(threadIdx.x) >= kNarrowThreads - H) {
     int const o = kNarrowThreads - 1 - static_cast<int>(threadIdx.x);
     float t = 0.0f;
     for (size_t b = 0; b < B; ++b) t += dz[b * kStride + o];
     db[o] = accumulate ? db[o] + t : t;
   }
+}
+
+__global__ __launch_bounds__(kNarrowThreads) void k_narrow_dw(float const *__restrict__ X, float const *__restrict__ dZ,
+                                                               float *__restrict__ dW, float *__restrict__ db, size_t B,
+                                                               size_t K, int H, int accumulate) {
+  __shared__ float lds[kNarrowDwLds];
+  narrow_dw_block(X, dZ, dW, db, B, K, H, accumulate, blockIdx.x, lds);
 }
 
 }  // namespace
@@ -217,6 +228,7 @@ constexpr int kMbTile = 64;      // a workgroup's block of dW: 64 units x 64 inp
 constexpr int kMbRows = 64;      // batch rows staged at a time (2 x 64 x 80 floats = 40 KB of LDS)
 constexpr int kMbStride = 80;    // floats between staged rows: 16 banks apart, so that the four rows a fragment
                                  // read touches (two per half wavefront) never share a bank
+constexpr int kMbLds = 2 * kMbRows * kMbStride;  // floats of LDS a workgroup stages its rows in
 constexpr size_t kMbMaxRows = 256;
 constexpr size_t kMbMaxOutputs = size_t(1) << 20;  // H * K: larger layers go to the tiled GEMM
 
@@ -226,9 +238,10 @@ typedef float mv4f __attribute__((ext_vector_type(4)));
 // 32 x 32 quarter of the block as 2 x 2 MFMA tiles of 16 x 16.  H, K multiples of 4, 16-byte aligned operands.
 __device__ __forceinline__ void minibatch_dw_block(float const *__restrict__ X, float const *__restrict__ dZ,
                                                    float *__restrict__ dW, unsigned B, unsigned K, unsigned H,
-                                                   int accumulate, unsigned block_k, unsigned block_h) {
-  __shared__ float zs[kMbRows * kMbStride];  // dZ[b][h0 .. h0 + 64)
-  __shared__ float xs[kMbRows * kMbStride];  // X [b][k0 .. k0 + 64)
+                                                   int accumulate, unsigned block_k, unsigned block_h,
+                                                   float *__restrict__ lds) {
+  float *const zs = lds;                        // dZ[b][h0 .. h0 + 64)
+  float *const xs = lds + kMbRows * kMbStride;  // X [b][k0 .. k0 + 64)
   unsigned const k0 = block_k * kMbTile, h0 = block_h * kMbTile;
   int const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int const wh = (wave >> 1) * 32, wk = (wave & 1) * 32;  // this wavefront's quarter
@@ -308,11 +321,14 @@ __device__ __forceinline__ void minibatch_dw_block(float const *__restrict__ X, 
 __global__ __launch_bounds__(256) void k_minibatch_dw(float const *__restrict__ X, float const *__restrict__ dZ,
                                                        float *__restrict__ dW, unsigned B, unsigned K, unsigned H,
                                                        int accumulate) {
-  minibatch_dw_block(X, dZ, dW, B, K, H, accumulate, blockIdx.x, blockIdx.y);
+  __shared__ __attribute__((aligned(16))) float lds[kMbLds];
+  minibatch_dw_block(X, dZ, dW, B, K, H, accumulate, blockIdx.x, blockIdx.y, lds);
 }
 
 // Several such products in one launch (the layers of a network after its backward pass): the workgroups walk the
-// concatenated lists of blocks.  A block's arithmetic is that of the single launch.
+// concatenated lists of blocks.  A block's arithmetic is that of the single launch.  The launch can also carry the
+// weight and bias gradient of ONE narrow layer (at most 16 units: the output layer): the workgroups behind the
+// last block run narrow_dw_block on it, as k_narrow_dw would.
 struct MbDwGroupArgs {
   struct Problem {
     float const *X, *dZ;
@@ -322,18 +338,40 @@ struct MbDwGroupArgs {
   Problem p[kMinibatchDwGroupMax];
   unsigned n;
   int accumulate;
+  // the narrow layer: workgroups [p[n - 1].block_end, gridDim.x); narrow_dW == nullptr: none
+  float const *narrow_X, *narrow_dZ;
+  float *narrow_dW, *narrow_db;
+  unsigned narrow_B, narrow_K, narrow_H;
 };
+constexpr int kMbGroupLds = kMbLds > kNarrowDwLds ? kMbLds : kNarrowDwLds;
+static_assert(kNarrowThreads == 256, "both kinds of workgroup have 256 threads");
 __global__ __launch_bounds__(256) void k_minibatch_dw_group(MbDwGroupArgs a) {
+  __shared__ __attribute__((aligned(16))) float lds[kMbGroupLds];
+  unsigned const mb_blocks = a.p[a.n - 1].block_end;
+  if (blockIdx.x >= mb_blocks) {
+    narrow_dw_block(a.narrow_X, a.narrow_dZ, a.narrow_dW, a.narrow_db, a.narrow_B, a.narrow_K,
+                    static_cast<int>(a.narrow_H), a.accumulate, blockIdx.x - mb_blocks, lds);
+    return;
+  }
   unsigned i = 0;
   while (i + 1 < a.n && blockIdx.x >= a.p[i].block_end) ++i;
   MbDwGroupArgs::Problem const &q = a.p[i];
   unsigned const local = blockIdx.x - (i == 0 ? 0u : a.p[i - 1].block_end);
-  minibatch_dw_block(q.X, q.dZ, q.dW, q.B, q.K, q.H, a.accumulate, local % q.blocks_k, local / q.blocks_k);
+  minibatch_dw_block(q.X, q.dZ, q.dW, q.B, q.K, q.H, a.accumulate, local % q.blocks_k, local / q.blocks_k, lds);
 }
 
 }  // namespace
 
-int minibatch_dw_group(dlmi_ctx *ctx, size_t n, MinibatchDwProblem const *problems, int accumulate) {
+bool narrow_dw_eligible(dlmi_ctx const *ctx, size_t B, size_t H) {
+  return ctx->tune.fc_narrow != 0 && H <= static_cast<size_t>(kNarrowMaxUnits) && B <= kNarrowMaxRowsDw;
+}
+
+int minibatch_dw_group(dlmi_ctx *ctx, size_t n, MinibatchDwProblem const *problems, int accumulate,
+                       NarrowDwProblem const *narrow) {
+  if (n == 0) return dlmi_fail(ctx, DLMI_E_INVALID, "minibatch_dw_group: no problem");
+  if (narrow != nullptr && (!narrow_dw_eligible(ctx, narrow->B, narrow->H) || narrow->X == nullptr ||
+                            narrow->dZ == nullptr || narrow->dW == nullptr || narrow->K == 0))
+    return dlmi_fail(ctx, DLMI_E_INVALID, "minibatch_dw_group: the narrow layer does not qualify");
   for (size_t first = 0; first < n; first += kMinibatchDwGroupMax) {
     MbDwGroupArgs a;
     a.n = static_cast<unsigned>(n - first < static_cast<size_t>(kMinibatchDwGroupMax) ? n - first : kMinibatchDwGroupMax);
@@ -350,6 +388,15 @@ int minibatch_dw_group(dlmi_ctx *ctx, size_t n, MinibatchDwProblem const *proble
       q.block_end = total;
     }
     for (unsigned i = a.n; i < static_cast<unsigned>(kMinibatchDwGroupMax); ++i) a.p[i] = a.p[a.n - 1];
+    a.narrow_X = a.narrow_dZ = nullptr;
+    a.narrow_dW = a.narrow_db = nullptr;
+    a.narrow_B = a.narrow_K = a.narrow_H = 0;
+    if (narrow != nullptr && first == 0) {  // with the first launch
+      a.narrow_X = narrow->X; a.narrow_dZ = narrow->dZ; a.narrow_dW = narrow->dW; a.narrow_db = narrow->db;
+      a.narrow_B = static_cast<unsigned>(narrow->B); a.narrow_K = static_cast<unsigned>(narrow->K);
+      a.narrow_H = static_cast<unsigned>(narrow->H);
+      total += static_cast<unsigned>(dlmi_ceil_div(narrow->K, static_cast<size_t>(kDwCols)));
+    }
     hipLaunchKernelGGL(k_minibatch_dw_group, dim3(total), dim3(256), 0, ctx->stream, a);
     DLMI_LAUNCH_CHECK(ctx, "k_minibatch_dw_group");
   }
@@ -373,7 +420,7 @@ int minibatch_dw_try(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *X
 
 int narrow_dw_try(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ, float *dW, float *db,
                   int accumulate) {
-  if (ctx->tune.fc_narrow == 0 || H > static_cast<size_t>(kNarrowMaxUnits) || B > kNarrowMaxRowsDw) return 0;
+  if (!narrow_dw_eligible(ctx, B, H)) return 0;
   dim3 const grid(static_cast<unsigned>(dlmi_ceil_div(K, static_cast<size_t>(kDwCols))));
   hipLaunchKernelGGL(k_narrow_dw, grid, dim3(kNarrowThreads), 0, ctx->stream, Xin, dZ, dW, db, B, K, static_cast<int>(H),
                      accumulate);

@@ -917,25 +917,34 @@ int dlmi_fc_bwd_dw_grouped(dlmi_ctx *ctx, size_t n, dlmi_dw_problem const *probl
       variant[i] = group_variant<false, false>(ctx, item[i]);  // (a narrow layer is no multiple of a tile: -1)
       if (minibatch_dw_eligible(ctx, pr[i].B, pr[i].K, pr[i].H, pr[i].Xin, pr[i].dZ, pr[i].dW)) variant[i] = -1;  // its own kernel
     }
-    // the mini-batch products that are not narrow layers (those bring their bias gradient along in a kernel of
-    // their own): one launch for all of them, from two on
+    // the mini-batch products that are not narrow layers: one launch for all of them, from two on; the first
+    // narrow layer (at most 16 units: its kernel forms the bias gradient too) rides along in that launch
     {
       MinibatchDwProblem mb[kMaxProblems];
-      size_t which[kMaxProblems], nmb = 0;
-      for (size_t i = 0; i < m; ++i)
+      size_t which[kMaxProblems], nmb = 0, narrow_at = m;
+      for (size_t i = 0; i < m; ++i) {
         if (variant[i] == -1 && pr[i].H > 16 &&
             minibatch_dw_eligible(ctx, pr[i].B, pr[i].K, pr[i].H, pr[i].Xin, pr[i].dZ, pr[i].dW)) {
           which[nmb] = i;
           mb[nmb++] = MinibatchDwProblem{pr[i].B, pr[i].K, pr[i].H, pr[i].Xin, pr[i].dZ, pr[i].dW};
+        } else if (narrow_at == m && pr[i].H <= 16 && narrow_dw_eligible(ctx, pr[i].B, pr[i].H)) {
+          narrow_at = i;
         }
-      if (nmb >= 2) {
-        int rc = minibatch_dw_group(ctx, nmb, mb, accumulate);
+      }
+      if (nmb >= 2 || (nmb == 1 && narrow_at < m)) {
+        NarrowDwProblem nw{};
+        if (narrow_at < m) {
+          dlmi_dw_problem const &q = pr[narrow_at];
+          nw = NarrowDwProblem{q.B, q.K, q.H, q.Xin, q.dZ, q.dW, q.db};
+        }
+        int rc = minibatch_dw_group(ctx, nmb, mb, accumulate, narrow_at < m ? &nw : nullptr);
         if (rc != DLMI_OK) return rc;
         for (size_t j = 0; j < nmb; ++j) variant[which[j]] = -2;  // done; the bias gradients follow below
+        if (narrow_at < m) variant[narrow_at] = -3;                // done, bias gradient included
       }
     }
     for (size_t i = 0; i < m; ++i) {
-      if (variant[i] == -2) continue;  // went with an earlier one
+      if (variant[i] == -2 || variant[i] == -3) continue;  // went with an earlier one
       GroupItem same[kMaxProblems];
       size_t ns = 0;
       if (variant[i] >= 0)

@@ -156,6 +156,8 @@ int dlmi_fc_bwd_dw(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin
  * after backward_pass has produced every layer's dZ (drivers/driver.cpp:253-255,
  * update_derivative_fwp_st.cpp:189-281), so the layers' products are independent of each other; a launch of many
  * rounds of tiles runs at the rate of one large product instead of paying each product's start and tail.
+ * On a mini-batch (at most 256 rows) the layers' products share one launch of the mini-batch kernel whatever their
+ * shapes, and the first layer of at most 16 units (the output layer, with its bias gradient) rides along in it.
  * Results are bit-identical to the one-by-one calls.  `problems` is a host array; pointers inside are device. */
 typedef struct {
   size_t B, K, H;

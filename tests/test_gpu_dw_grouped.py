@@ -33,8 +33,14 @@ MIXES = {
     "mixed": [(256, 512, 256), (256, 256, 512), (128, 784, 512), (128, 512, 10), (8192, 128, 128), (256, 512, 256)],
     "single": [(512, 256, 256)],
     # the layers of a network on a mini-batch: the products of any width share one launch of the mini-batch kernel
-    # (ragged blocks, a batch that is no multiple of four among them), the narrow output layer goes alone
-    "mini-batch": [(128, 784, 512), (128, 512, 512), (128, 512, 10), (100, 36, 24), (255, 64, 64), (128, 512, 512)],
+    # (ragged blocks, a batch that is no multiple of four among them); the first narrow layer (the output layer, with
+    # its bias gradient) rides along in that launch, a second one goes alone
+    "mini-batch": [(128, 784, 512), (128, 512, 512), (128, 512, 10), (100, 36, 24), (255, 64, 64), (128, 512, 512),
+                   (77, 130, 16)],
+    # one hidden layer and the output layer: one launch for both
+    "mini-batch pair": [(128, 784, 512), (128, 512, 10)],
+    # more mini-batch products than one launch of their kernel holds (8), and a narrow layer with the first launch
+    "mini-batch many": [(64, 64, 64)] * 9 + [(64, 64, 3)],
 }
 
 
