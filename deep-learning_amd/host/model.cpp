@@ -24,6 +24,7 @@
 #include <thread>
 #include <vector>
 
+#include "../../include/dlmi_model.h"
 #include "../../include/dlmi_model.hpp"
 
 namespace dlmi {
@@ -267,6 +268,8 @@ float const *Model::Impl::slots_upload(RowSlots &s, size_t const B, size_t const
 
 Model::Model(void) : impl_(new Impl) {
   real_gen.seed(5489u);
+  gaussian_gen.seed(5489u);
+  gaussian_dist.reset();
   bernoulli = new Dist::Bernoulli[1];
 }
 
@@ -308,6 +311,8 @@ void Model::clear(void) {
   impl->n_errors = n_errors;
   static_cast<Model_State &>(*this) = Model_State();  // every public member takes its default again
   real_gen.seed(5489u);
+  gaussian_gen.seed(5489u);
+  gaussian_dist.reset();
   bernoulli = masks;
 }
 
@@ -1025,6 +1030,32 @@ void Model::Initialization__Uniform(real const bias, real const lower_bound, rea
   finish_initialization(*this);
 }
 
+// layers_initialize_orthogonal / weights_initialize_orthogonal (orthogonal.cpp:39-154)
+void Model::weights_initialize_orthogonal(size_t const rows, size_t const cols, real const scale, var *weights) {
+  // weights_initialize_gaussian(weights, weights + rows * cols, 1) (model.cpp:5401-5409)
+  for (size_t i = 0, n = rows * cols; i < n; ++i) weights[i] = gaussian_dist(gaussian_gen);
+  if (dlmi_orthogonal_weights(rows, cols, scale, weights) != 1) fail("weights_initialize_orthogonal: empty layer");
+}
+
+void Model::layers_initialize_orthogonal(bool const pre_initialize, real const bias) {
+  if (ptr_array_layers == nullptr) { fail("layers_initialize_orthogonal: model not compiled"); return; }
+  for (size_t li = 1; li < total_layers; ++li) {
+    Layer const &l = ptr_array_layers[li];
+    if (l.type_layer != LAYER::FULLY_CONNECTED) continue;  // (a RESIDUAL entry has no weights, orthogonal.cpp:48-52)
+    // the gain of the layer's first activation unit (orthogonal.cpp:59), found as the Glorot initializer finds it
+    size_t ga = li;
+    while (ga + 1 < total_layers && (ptr_array_layers[ga].type_layer != LAYER::FULLY_CONNECTED || ptr_array_layers[ga].block_first)) ++ga;
+    weights_initialize_orthogonal(l.n_inp, l.n_out, gain_scale(ptr_array_layers[ga].type_activation_function),
+                                  ptr_array_parameters + l.first_connection_index);
+    for (size_t i = 0; i < l.n_out; ++i) ptr_array_parameters[l.first_bias_connection_index + i] = bias;  // orthogonal.cpp:62
+  }
+  if (pre_initialize) {
+    (void)upload_parameters();
+  } else {
+    finish_initialization(*this);  // orthogonal.cpp:97-104
+  }
+}
+
 // ---------------------------------------------------------------- LSUV
 bool Model::Initialize__LSUV(size_t const max_n_trials, size_t const max_batch_size, real const bias,
                              real const var_target, real const var_tolerance) {
@@ -1059,19 +1090,25 @@ size_t Model::Get__LSUV_Trials(size_t const li) const { return li < impl_->lsuv_
 bool Model::Initialization__LSUV(size_t const n_data_set, real const *const *const inputs) {
   if (ptr_array_layers == nullptr || inputs == nullptr || n_data_set == 0) return fail("Initialization__LSUV: model not compiled or no data");
   LSUV_Parameters const &p = impl_->lsuv;
-  // The reference starts with layers_initialize_orthogonal (lsuv.cpp:55, orthogonal.cpp:39-172: Eigen's QR), which
-  // is not built here: the loop scales the weights it finds.  Without any, it would scale zeros without a word.
-  if (!impl_->weights_set)
-    return fail("Initialization__LSUV: the orthogonal pre-initialization is not built and no weights have been set: run "
-                "an initializer or upload parameters first");
-  // the bias slots, as the pre-initialization would leave them (orthogonal.cpp:62)
-  if (!download_parameters()) return false;
-  for (size_t li = 1; li < total_layers; ++li) {
-    Layer const &l = ptr_array_layers[li];
-    if (l.type_layer != LAYER::FULLY_CONNECTED) continue;
-    for (size_t i = 0; i < l.n_out; ++i) ptr_array_parameters[l.first_bias_connection_index + i] = p.initial_bias;
+  if (lsuv_pre_initialize) {
+    // pre-initialize with orthonormal matrices (lsuv.cpp:55)
+    size_t const errors_at_start = error_count();
+    layers_initialize_orthogonal(true, p.initial_bias);
+    if (error_count() != errors_at_start) return false;
+  } else {
+    // The loop alone scales the weights it finds.  Without any, it would scale zeros without a word.
+    if (!impl_->weights_set)
+      return fail("Initialization__LSUV: no orthogonal pre-initialization was asked for and no weights have been set: run "
+                  "an initializer or upload parameters first");
+    // the bias slots, as the pre-initialization would leave them (orthogonal.cpp:62)
+    if (!download_parameters()) return false;
+    for (size_t li = 1; li < total_layers; ++li) {
+      Layer const &l = ptr_array_layers[li];
+      if (l.type_layer != LAYER::FULLY_CONNECTED) continue;
+      for (size_t i = 0; i < l.n_out; ++i) ptr_array_parameters[l.first_bias_connection_index + i] = p.initial_bias;
+    }
+    if (!upload_parameters()) return false;
   }
-  if (!upload_parameters()) return false;
   size_t const n_data = std::min(p.maximum_batch_size, n_data_set);
   if (!update_mem_batch_size(n_data)) return false;
   size_t const batch_size_max = std::min(batch_size, n_data);

@@ -94,6 +94,15 @@ void dlmi_model_init_uniform(dlmi_model *h, unsigned seed, float bias, float low
   h->m.Initialization__Uniform(bias, lower, upper);
 }
 
+void dlmi_model_seed_gaussian(dlmi_model *h, unsigned seed) {
+  h->m.gaussian_gen.seed(seed);
+  h->m.gaussian_dist.reset();
+}
+void dlmi_model_orthogonal(dlmi_model *h, unsigned seed, float bias) {
+  dlmi_model_seed_gaussian(h, seed);
+  h->m.layers_initialize_orthogonal(false, bias);
+}
+
 // An uncompiled model: what dlmi_model_load() fills.
 dlmi_model *dlmi_model_create_empty(void) { return new dlmi_model; }
 
@@ -286,8 +295,9 @@ int dlmi_model_forward_to(dlmi_model *h, int state, size_t B, float const *X, si
 }
 // Initialize__LSUV(...) then Initialization__LSUV(data set of n_data dense rows)
 int dlmi_model_lsuv(dlmi_model *h, size_t max_n_trials, size_t max_batch_size, float bias, float var_target,
-                    float var_tolerance, size_t n_data, float const *X) {
+                    float var_tolerance, size_t n_data, float const *X, int pre_initialize) {
   Model &m = h->m;
+  m.lsuv_pre_initialize = pre_initialize != 0;
   if (!m.Initialize__LSUV(max_n_trials, max_batch_size, bias, var_target, var_tolerance)) return 0;
   size_t const K0 = m.ptr_array_layers != nullptr ? m.ptr_array_layers[0].n_out : 0;
   std::vector<float const *> Xm(n_data);

@@ -189,11 +189,20 @@ class Model:
         self.B = X.shape[0]
         self._ok(self.lib.dlmi_model_forward_to(self.h, c_int(state), c_sz(self.B), _ptr(X), c_sz(end_layer)), "forward_to")
 
-    def lsuv(self, X, max_n_trials=10, max_batch_size=32, bias=0.0, var_target=1.0, var_tolerance=0.01):
-        """Initialize__LSUV + Initialization__LSUV on the rows of X; returns the scalings applied per layer."""
+    def orthogonal(self, seed, bias=0.0):
+        """gaussian_gen.seed(seed); layers_initialize_orthogonal(false, bias)"""
+        self.lib.dlmi_model_orthogonal(self.h, ctypes.c_uint(seed), c_f(bias))
+
+    def seed_gaussian(self, seed):
+        self.lib.dlmi_model_seed_gaussian(self.h, ctypes.c_uint(seed))
+
+    def lsuv(self, X, max_n_trials=10, max_batch_size=32, bias=0.0, var_target=1.0, var_tolerance=0.01, pre_initialize=True):
+        """Initialize__LSUV + Initialization__LSUV on the rows of X; returns the scalings applied per layer.
+        pre_initialize=False: the scaling loop alone, on the weights the model holds."""
         X = np.ascontiguousarray(X, np.float32)
         self._ok(self.lib.dlmi_model_lsuv(self.h, c_sz(max_n_trials), c_sz(max_batch_size), c_f(bias), c_f(var_target),
-                                          c_f(var_tolerance), c_sz(X.shape[0]), _ptr(X)), "Initialization__LSUV")
+                                          c_f(var_tolerance), c_sz(X.shape[0]), _ptr(X), c_int(1 if pre_initialize else 0)),
+                 "Initialization__LSUV")
         self.lib.dlmi_model_lsuv_trials.restype = c_sz
         return [int(self.lib.dlmi_model_lsuv_trials(self.h, c_sz(l))) for l in range(len(self.widths))]
 

@@ -30,6 +30,17 @@ void dlmi_model_layer_info(dlmi_model const *m, size_t layer, size_t *out);
  * Initialization__Uniform(bias, lower, upper) (uniform.cpp:26-90) */
 void dlmi_model_glorot_uniform(dlmi_model *m, unsigned seed, float bias);
 void dlmi_model_init_uniform(dlmi_model *m, unsigned seed, float bias, float lower, float upper);
+/* gaussian_gen.seed(seed) and a fresh distribution state, then layers_initialize_orthogonal(false, bias)
+ * (v1/ops/initializers/orthogonal.cpp:39-105). */
+void dlmi_model_orthogonal(dlmi_model *m, unsigned seed, float bias);
+/* Only the seeding of the above: what a later dlmi_model_lsuv(..., pre_initialize = 1) draws from. */
+void dlmi_model_seed_gaussian(dlmi_model *m, unsigned seed);
+/* Host arithmetic, no device and no model needed: the second half of Model::weights_initialize_orthogonal
+ * (orthogonal.cpp:132-153).  `weights` [rows * cols] (rows = fan-in, cols = units; the Gaussian draws) is read as a
+ * column-major matrix of max(rows, cols) x min(rows, cols), replaced by Q . sign(diag R) of its column-pivoting QR
+ * factorization, transposed in place when rows >= cols, multiplied by `scale`, and written back as it lies.
+ * Parity with Eigen's ColPivHouseholderQR unpinned; held to LAPACK's geqp3 by the tests.  1 = done, 0 = empty. */
+int dlmi_orthogonal_weights(size_t rows, size_t cols, float scale, float *weights);
 /* Text files of the reference: Model::save_params (`model.net`, v1/learner/save.cpp:190-520), save_spec_params
  * (`model.nn`, :35-188), load_spec_params / load (load.cpp:36, :1243; `load` clears the model first, so it also
  * fills a model from dlmi_model_create_empty()).  Paths are UTF-8.  1 = done, 0 = refused (dlmi_model_last_error). */
@@ -98,12 +109,13 @@ int dlmi_model_steps(dlmi_model *m, int state, size_t n_steps, size_t B, float c
 /* forward_pass(batch, rows of X, 0, end_layer): only the layers [1, end_layer) run (the partial pass the LSUV
  * initializer uses, lsuv.cpp:131-135) */
 int dlmi_model_forward_to(dlmi_model *m, int state, size_t batch, float const *X, size_t end_layer);
-/* Initialize__LSUV + Initialization__LSUV (v1/ops/initializers/lsuv.cpp:27-177) on a data set of n_data dense rows;
- * the weights are scaled from what they hold (the reference's orthogonal start is not part of this).
+/* Initialize__LSUV + Initialization__LSUV (v1/ops/initializers/lsuv.cpp:27-177) on a data set of n_data dense rows.
+ * pre_initialize != 0: as the reference, from the orthogonal initializer (lsuv.cpp:55); 0: the scaling loop alone,
+ * on the weights the model holds (Model::lsuv_pre_initialize).
  * dlmi_model_lsuv_trials: scalings the last run applied to a layer; dlmi_model_layer_variance:
  * Model::get_layer_variance (model.cpp:2813-2858) after the last forward pass. */
 int dlmi_model_lsuv(dlmi_model *m, size_t max_n_trials, size_t max_batch_size, float bias, float var_target,
-                    float var_tolerance, size_t n_data, float const *X);
+                    float var_tolerance, size_t n_data, float const *X, int pre_initialize);
 size_t dlmi_model_lsuv_trials(dlmi_model const *m, size_t layer);
 float dlmi_model_layer_variance(dlmi_model const *m, size_t layer, size_t batch);
 int dlmi_model_download_layer(dlmi_model const *m, size_t layer, int which, size_t batch, float *out);

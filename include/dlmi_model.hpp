@@ -221,6 +221,14 @@ struct Model_State {
   // path is DLMI_DROP_BWD_REFERENCE.
   dlmi_dropout_bwd dropout_backward_mode = DLMI_DROP_BWD_REFERENCE;
   std::mt19937 real_gen;  // weight initializers (the engine inside the reference's Dist::Real real_gen)
+  // The orthogonal initializer's draws: the engine and the distribution object inside the reference's
+  // Dist::Gaussian gaussian (ops/distributions/gaussian.cpp: std::normal_distribution<real> over std::mt19937; the
+  // distribution keeps its spare value from one layer to the next, as there).
+  std::mt19937 gaussian_gen;
+  std::normal_distribution<real> gaussian_dist{0.0f, 1.0f};
+  // false: Initialization__LSUV keeps the weights at hand instead of starting from the orthogonal initializer
+  // (no reference counterpart; see Initialization__LSUV)
+  bool lsuv_pre_initialize = true;
   // Dropout mask generator: `bernoulli[0]`, the one the reference's single-thread Dropout_Bernoulli draws
   // from (model.hpp:3159, allocate.cpp:86-100; clock-seeded there, seed 5489 here until the caller seeds it).
   Dist::Bernoulli *bernoulli = nullptr;
@@ -273,6 +281,16 @@ class Model : public Model_State {
   // (see the definition for the residual cases).
   void initialize_weights_with_glorot_uniform(real const bias = 0.0f);
   void Initialization__Uniform(real const bias = 0.0f, real const lower_bound = -1.0f, real const upper_bound = 1.0f);
+  // Orthogonal initializer (v1/ops/initializers/orthogonal.cpp:39-154), fully-connected layers: a layer's weights
+  // are drawn from N(0, 1) in parameter order (`gaussian_gen`), read as a column-major matrix of max(fan-in, units) x
+  // min(fan-in, units), replaced by Q . sign(diag R) of its column-pivoting QR factorization, transposed in place
+  // when fan-in >= units, multiplied by the gain of the layer's activation and copied back as they lie; every bias
+  // slot is set to `bias`.  pre_initialize == false also does what the other initializers end with (scales / shifts
+  // / moving statistics to 1 / 0 / 0 / 1, training arrays cleared); true is the call LSUV starts with.  The
+  // factorization is this library's own (host, double precision): **parity with Eigen's unpinned** - it is held to
+  // LAPACK's column-pivoting QR, which picks its pivots by the same rule.
+  void layers_initialize_orthogonal(bool const pre_initialize, real const bias = 0.0f);
+  void weights_initialize_orthogonal(size_t const rows, size_t const cols, real const scale, var *weights);
   // LSUV, "all you need is a good init" (v1/ops/initializers/lsuv.cpp:27-177; model.cpp:2813-2858).
   // Initialize__LSUV keeps the settings; Initialization__LSUV then, layer by layer from the first hidden one,
   // forwards up to `maximum_batch_size` rows of the data set through the layers up to that one, measures the
@@ -280,10 +298,11 @@ class Model : public Model_State {
   // sqrt(variance_target / variance) until |variance - target| < tolerance or `maximum_number_trials`
   // scalings are done; the variance of a data set that takes several mini-batches is the SUM of the
   // mini-batch variances, as in the reference.  Forward passes, variance sums (in double) and scalings run on
-  // the device; the host reads one float per trial.  The reference starts from its orthogonal initializer
-  // (orthogonal.cpp:39-172, an Eigen QR that is not available here): here the weights are what the caller
-  // initialized before (a Glorot or uniform start, a loaded file) and only the bias slots are set to
-  // `initial_bias`, as that initializer would.  Afterwards: training arrays cleared, scales / shifts /
+  // the device; the host reads one float per trial.  As in the reference the call starts from the orthogonal
+  // initializer (layers_initialize_orthogonal(true, initial_bias), lsuv.cpp:55).  `lsuv_pre_initialize = false` (no
+  // reference counterpart) keeps the weights the caller initialized before (a Glorot or uniform start, a loaded
+  // file) and only sets the bias slots to `initial_bias`: the scaling loop alone, which is what is pinned bit for
+  // bit to the reference's Initialization__LSUV__Loop.  Afterwards: training arrays cleared, scales / shifts /
   // moving statistics back to 1 / 0 / 0 / 1.  The dataset argument of the reference (get_n_data(),
   // Get__Input_Array()) is passed as its two parts.
   struct LSUV_Parameters {  // model.hpp:224-235

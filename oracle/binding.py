@@ -831,7 +831,7 @@ class ReferenceMLP:
 
     def lsuv(self, X, max_n_trials=10, max_batch_size=32, bias=0.0, var_target=1.0, var_tolerance=0.01):
         """The reference's Initialize__LSUV + Initialization__LSUV__Loop on weights already initialized (its
-        orthogonal pre-initialization needs Eigen and is not built)."""
+        orthogonal pre-initialization is not part of the oracle: the facade has its own, tests/test_orthogonal_weights.py)."""
         X = np.ascontiguousarray(X, np.float32)
         ok = self.lib.dlref_model_lsuv(self.h, c_sz(max_n_trials), c_sz(max_batch_size), c_f(bias), c_f(var_target),
                                        c_f(var_tolerance), c_sz(X.shape[0]), _ptr(X), c_sz(X.shape[1]))

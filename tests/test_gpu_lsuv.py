@@ -34,7 +34,7 @@ def test_device_loop_against_the_oracle(lib, oracle, widths, acts, norms, kw):
         g.set_parameters(p0[:g.P])
         X = np.random.default_rng(1).normal(0, 1, (48, widths[0])).astype(np.float32)
         to = o.lsuv(X, **kw)
-        tg = g.lsuv(X, **kw)
+        tg = g.lsuv(X, pre_initialize=False, **kw)
         assert tg == to
         pg = g.get_parameters()
         nwb = sum(a * b + b for a, b in zip(widths[:-1], widths[1:]))
@@ -131,7 +131,7 @@ def test_residual_network_layers_meet_the_target(lib):
         g.prepare(32)
         g.init_uniform(2, 0.0, -0.3, 0.3)
         X = np.random.default_rng(5).normal(0, 1, (32, 10)).astype(np.float32)
-        trials = g.lsuv(X, var_target=1.5, var_tolerance=1e-3)
+        trials = g.lsuv(X, var_target=1.5, var_tolerance=1e-3, pre_initialize=False)
         assert trials[2] == 0 and all(trials[l] >= 1 for l in (1, 3, 4, 5)) and max(trials) <= 10
         for l in (1, 3, 4, 5):
             g.forward_to(STATE["INFERENCE"], X, l + 1)
@@ -146,24 +146,95 @@ def test_settings_are_checked(lib):
         X = np.zeros((8, 4), np.float32)
         for bad in (dict(max_batch_size=0), dict(var_target=-1.0), dict(var_tolerance=-0.5)):
             with pytest.raises(RuntimeError):
-                g.lsuv(X, **bad)
+                g.lsuv(X, pre_initialize=False, **bad)
         # all-zero inputs: every variance is 0, replaced by epsilon (lsuv.cpp:140), the loop still ends
         g.glorot_uniform(1)
-        t = g.lsuv(X, max_n_trials=3)
+        t = g.lsuv(X, max_n_trials=3, pre_initialize=False)
         assert max(t) <= 3 and np.all(np.isfinite(g.get_parameters()))
     finally:
         g.close()
 
 
-def test_lsuv_without_weights_is_refused(lib):
-    """The reference's Initialization__LSUV starts with an orthogonal initialization of its own; this one scales the
-    weights it finds.  On a model whose weights nobody has set it says so instead of scaling zeros."""
+def test_the_loop_alone_without_weights_is_refused(lib):
+    """With pre_initialize=False the call scales the weights it finds.  On a model whose weights nobody has set it
+    says so instead of scaling zeros."""
     g = gpu_model(lib, [12, 16, 4], ["RELU", "LINEAR"], ["NONE"])
     try:
         X = np.random.default_rng(2).normal(0, 1, (16, 12)).astype(np.float32)
         with pytest.raises(RuntimeError, match="no weights have been set"):
-            g.lsuv(X)
+            g.lsuv(X, pre_initialize=False)
         g.glorot_uniform(3)
-        g.lsuv(X)  # an initializer has run: accepted
+        g.lsuv(X, pre_initialize=False)  # an initializer has run: accepted
     finally:
         g.close()
+
+
+def layer_weights(p, widths):
+    off = 0
+    for a, b in zip(widths[:-1], widths[1:]):
+        yield a, b, p[off:off + a * b]
+        off += a * b
+
+
+def test_orthogonal_initializer(lib):
+    """layers_initialize_orthogonal(false, bias): per layer, the weights as they lie are gain x a matrix with
+    orthonormal columns - max(fan-in, units) x min(fan-in, units), row-major when fan-in >= units (the reference
+    transposes in place), column-major otherwise; biases as given, scales 1, shifts 0, moving statistics 0 / 1,
+    gradients cleared.  The draws continue from layer to layer and repeat for a seed.  (The factorization itself is
+    held to LAPACK's in tests/test_orthogonal_weights.py.)"""
+    widths, acts = [12, 16, 16, 8, 5], ["RELU", "TANH", "LEAKY_RELU", "LINEAR"]
+    gains = [np.sqrt(2.0), 5.0 / 3.0, np.sqrt(2.0 / (1.0 + 0.01 ** 2)), 1.0]
+    g = gpu_model(lib, widths, acts, ["BRN", "NONE", "BN"])
+    h = gpu_model(lib, widths, acts, ["BRN", "NONE", "BN"])
+    try:
+        g.orthogonal(3, bias=0.25)
+        p = g.get_parameters()
+        nw = sum(a * b for a, b in zip(widths[:-1], widths[1:]))
+        nb = sum(widths[1:])
+        for (fan_in, units, w), gain in zip(layer_weights(p, widths), gains):
+            hi, lo = max(fan_in, units), min(fan_in, units)
+            W = (w.reshape(hi, lo) if fan_in >= units else w.reshape(lo, hi).T).astype(np.float64) / gain
+            assert np.max(np.abs(W.T @ W - np.eye(lo))) < 1e-5, (fan_in, units)
+        assert np.all(p[nw:nw + nb] == np.float32(0.25))
+        nu = g.n_units
+        assert np.all(p[nw + nb:nw + nb + nu] == 1.0) and np.all(p[nw + nb + nu:nw + nb + 2 * nu] == 0.0)
+        mm, ms = g.get_moving()
+        assert np.all(mm == 0.0) and np.all(ms == 1.0) and np.all(g.get_dparams() == 0)
+        h.orthogonal(3, bias=0.25)
+        assert np.array_equal(h.get_parameters(), p)
+        h.orthogonal(4, bias=0.25)
+        assert not np.array_equal(h.get_parameters()[:nw], p[:nw])
+        # the second layer's draws follow the first's: a model that starts at the second layer's shape with the
+        # same seed holds other weights there
+        k = gpu_model(lib, widths[1:], acts[1:], ["NONE", "BN"])
+        try:
+            k.orthogonal(3, bias=0.25)
+            assert not np.array_equal(k.get_parameters()[:16 * 16], p[12 * 16:12 * 16 + 16 * 16])
+        finally:
+            k.close()
+    finally:
+        g.close()
+        h.close()
+
+
+def test_lsuv_starts_from_the_orthogonal_initializer(lib):
+    """Initialization__LSUV as the reference runs it (lsuv.cpp:55): on a model whose weights nobody has set, the
+    orthogonal initializer first, then the scaling loop - the same bits as the two steps taken by hand - and every
+    layer's output variance ends within the tolerance of the target."""
+    widths, acts = [20, 32, 24, 6], ["RELU", "TANH", "LINEAR"]
+    a = gpu_model(lib, widths, acts, ["NONE", "NONE"])
+    b = gpu_model(lib, widths, acts, ["NONE", "NONE"])
+    try:
+        X = np.random.default_rng(8).normal(0, 1, (40, 20)).astype(np.float32)
+        a.seed_gaussian(7)
+        ta = a.lsuv(X, bias=0.05, var_tolerance=1e-3)
+        b.orthogonal(7, bias=0.05)
+        tb = b.lsuv(X, bias=0.05, var_tolerance=1e-3, pre_initialize=False)
+        assert ta == tb and max(ta) <= 10
+        assert np.array_equal(a.get_parameters(), b.get_parameters())
+        for l in range(1, len(widths)):
+            a.forward_to(STATE["INFERENCE"], X[:32], l + 1)
+            assert ta[l] == 10 or abs(a.layer_variance(l, 32) - 1.0) < 1e-3, (l, ta)
+    finally:
+        a.close()
+        b.close()
