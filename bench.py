@@ -63,7 +63,7 @@ MEASURED_TRAFFIC_BYTES = {
 }
 TRAFFIC_SOURCES = ("gemm_f32_mfma.hip", "norm_kernels.hip", "norm_panel_fwd.hip", "norm_panel_bwd.hip",
                    "norm_panel_common.hpp", "norm_shared.hpp", "activations.hpp")
-TRAFFIC_SOURCES_SHA256 = "9f8fa7cae32453e0bb3d8a7ed1e12925231704ccde9c50dc7b97c25851f93a3c"
+TRAFFIC_SOURCES_SHA256 = "3f8482c1a956161b8b809770a17f35365877b6bd5396f7d78e2b73a29270ba20"
 
 
 def traffic_sources_digest():

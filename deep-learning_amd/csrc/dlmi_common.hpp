@@ -36,6 +36,7 @@ struct dlmi_tuning {
   int norm_small = 1;             // mini-batches (at most 256 rows, 2^20 elements) run the one-launch small-batch kernels
   int minibatch_dw = 1;           // weight gradients of a mini-batch (at most 256 rows, 2^20 weights) run the one-block-per-tile kernel of fc_small.hip
   int narrow_dx_fused = 1;        // ... which also form dY = dZn . Wn below a layer of at most 16 units themselves
+  int db_in_product = 1;          // a weight gradient split over K forms the bias gradient on its way (no pass over dZ)
 };
 
 struct dlmi_ctx {

@@ -83,6 +83,7 @@ int dlmi_ctx_create(dlmi_ctx **out, int device, void *stream) {
   t.narrow_dx_fused = env_flag("DLMI_NARROW_DX_FUSED", t.narrow_dx_fused);
   t.minibatch_dw = env_flag("DLMI_MINIBATCH_DW", t.minibatch_dw);
   t.fc_narrow = env_flag("DLMI_FC_NARROW", t.fc_narrow);
+  t.db_in_product = env_flag("DLMI_DB_IN_PRODUCT", t.db_in_product);
   if (env_flag("DLMI_GEMM_CLOCK", 0)) {
     void *p = nullptr;
     if (hipMalloc(&p, (2 + 4 * 4096) * sizeof(unsigned long long)) == hipSuccess) {

@@ -81,6 +81,9 @@ struct GemmArgs {
   int accumulate;      // C += result (only when gridDim.z == 1)
   int a_vec, b_vec;    // operand base and leading dimension allow 16-byte loads (ragged variant)
   unsigned tiles_m, tiles_n;
+  // DB variants (a weight gradient dW = dZ^T X split over K): [gridDim.z][M], the sums over this slice's K range of
+  // the A operand's rows - the slice's share of the bias gradient, taken from the registers the A tiles pass through
+  float *db_out;
 };
 
 // LDS tile of either operand: [ROWS][BK+4], k contiguous, so that the MFMA
@@ -238,7 +241,7 @@ __device__ __forceinline__ unsigned xcd_order(unsigned id, unsigned ntiles) {
 }
 
 // One tile of one product: tile number `lid` (in the grouped order below) of K slice `zslice` of `nslices`.
-template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int RST, int WVM = 2>
+template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int RST, int WVM = 2, bool DB = false>
 __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid, unsigned const zslice, unsigned const nslices,
                                           float *__restrict__ lds) {
   constexpr bool FAST = MODE == kFast;          // no edge anywhere: unguarded stores
@@ -302,6 +305,19 @@ __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid,
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
   };
 
+  // DB: every A tile goes through this thread's registers once, on its way to LDS; what it holds of each - 4
+  // consecutive rows at one k - is added up per thread over the K tiles and combined at the end of the tile.
+  static_assert(!DB || (!A_KCONTIG && MODE == kFast), "the bias gradient rides along in the fast weight-gradient variants");
+  bool const db_here = DB && tile_n == 0;  // one column of tiles reports the sums
+  float dbacc[DB ? 4 * TA::kPerThread : 1];
+#pragma unroll
+  for (int e = 0; e < (DB ? 4 * TA::kPerThread : 1); ++e) dbacc[e] = 0.0f;
+  auto db_add = [&](typename TA::Regs const &r) {  // (every workgroup adds: a branch would cut the K loop's schedule in two)
+    if constexpr (DB) {
+#pragma unroll
+      for (int e = 0; e < 4 * TA::kPerThread; ++e) dbacc[e] += r[e];
+    }
+  };
   static_assert(BK == 16, "the pipeline below is written for two K groups per tile");
   constexpr int NM = TM * TN * (BK / 2);                                     // MFMAs per K tile
   constexpr int NFR = TM + TN;                                               // LDS reads per K group
@@ -348,6 +364,7 @@ __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid,
     }
     tile_store<BM, BK, A_KCONTIG, THREADS>(lds, r0a);
     tile_store<BN, BK, B_KCONTIG, THREADS>(lds + TA::kFloats, r0b);
+    db_add(r0a);
     __syncthreads();
     v4f f0a[TM], f0b[TN];
     frags(lds, lds + TA::kFloats, 0, f0a, f0b);
@@ -364,6 +381,7 @@ __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid,
       if constexpr (STORE) {
         tile_store<BM, BK, A_KCONTIG, THREADS>(na, xa);
         tile_store<BN, BK, B_KCONTIG, THREADS>(na + TA::kFloats, xb);
+        db_add(xa);
       }
       if constexpr (LOAD) {
         xa = load_a(kt + 1 + RST);
@@ -484,16 +502,47 @@ __device__ __forceinline__ void gemm_tile(GemmArgs const &g, unsigned const lid,
       }
     }
   }
+  if constexpr (DB) {
+    if (db_here) {
+      // a piece's k is (f & 7) + 8 * kh: the 8 lanes that share a row group first (xor tree), then the halves kh
+      // through LDS, kh = 0 first
+      __syncthreads();  // every wavefront is done reading the operand tiles: reuse that LDS
+#pragma unroll
+      for (int i = 0; i < TA::kPerThread; ++i) {
+        int const f = threadIdx.x + i * THREADS;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = dbacc[4 * i + e];
+          v[e] += __shfl_xor(v[e], 1, 64);
+          v[e] += __shfl_xor(v[e], 2, 64);
+          v[e] += __shfl_xor(v[e], 4, 64);
+        }
+        if ((f & 7) == 0 && (!TA::kSomeIdle || f < TA::kVec4)) {
+          int tr, tk;
+          TA::piece(f, tr, tk);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) lds[(tk >> 3) * BM + tr + e] = v[e];
+        }
+      }
+      __syncthreads();
+      for (int r = threadIdx.x; r < BM; r += THREADS) {
+        float t = lds[r];
+#pragma unroll
+        for (int kh = 1; kh < BK / 8; ++kh) t += lds[kh * BM + r];
+        g.db_out[static_cast<size_t>(zslice) * g.M + m0 + r] = t;
+      }
+    }
+  }
   if (clocked && threadIdx.x == 0) {
     g.clock_out[0] = __builtin_amdgcn_s_memtime() - c0;
     g.clock_out[1] = __builtin_amdgcn_s_memrealtime() - r0;
   }
 }
 
-template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int WAVES_PER_EU, int RST, int WVM = 2>
-__global__ __launch_bounds__(128 * WVM) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
-void k_gemm_f32(GemmArgs g) {
-  extern __shared__ __attribute__((aligned(16))) float lds[];
+// The workgroup of a product launch: which tile and slice it computes, and the time stamps of a clocked launch.
+template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int RST, int WVM, bool DB>
+__device__ __forceinline__ void gemm_workgroup(GemmArgs const &g, float *__restrict__ lds) {
   unsigned const ntiles = g.tiles_m * g.tiles_n;
   unsigned lid = xcd_order(blockIdx.x, ntiles), zslice = blockIdx.z;
   if (gridDim.z % kXcds == 0 && ntiles % kXcds != 0) {
@@ -511,7 +560,7 @@ void k_gemm_f32(GemmArgs g) {
   bool const stamp = g.clock_out != nullptr && blockIdx.z == 0 && blockIdx.x < kClockWgs;
   unsigned long long ts = 0;
   if (stamp) ts = __builtin_amdgcn_s_memrealtime();
-  gemm_tile<BM, BN, BK, A_KCONTIG, B_KCONTIG, MODE, RST, WVM>(g, lid, zslice, gridDim.z, lds);
+  gemm_tile<BM, BN, BK, A_KCONTIG, B_KCONTIG, MODE, RST, WVM, DB>(g, lid, zslice, gridDim.z, lds);
   if (stamp && threadIdx.x == 0) {
     unsigned long long const te = __builtin_amdgcn_s_memrealtime();
     __builtin_amdgcn_s_waitcnt(0);
@@ -522,6 +571,21 @@ void k_gemm_f32(GemmArgs g) {
     unsigned long long *o = g.clock_out + 2 + 4 * static_cast<size_t>(blockIdx.x);
     o[0] = ts; o[1] = te; o[2] = td; o[3] = (static_cast<unsigned long long>(xcc) << 32) | hw;
   }
+}
+
+template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int MODE, int WAVES_PER_EU, int RST, int WVM = 2>
+__global__ __launch_bounds__(128 * WVM) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
+void k_gemm_f32(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  gemm_workgroup<BM, BN, BK, A_KCONTIG, B_KCONTIG, MODE, RST, WVM, false>(g, lds);
+}
+
+// The fast weight-gradient variant whose K slices also leave their shares of the bias gradient (GemmArgs::db_out).
+template <int BM, int BN, int BK, bool A_KCONTIG, bool B_KCONTIG, int WAVES_PER_EU, int RST, int WVM = 2>
+__global__ __launch_bounds__(128 * WVM) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
+void k_gemm_f32_db(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  gemm_workgroup<BM, BN, BK, A_KCONTIG, B_KCONTIG, kFast, RST, WVM, true>(g, lds);
 }
 
 // Several independent products of one kernel variant in ONE launch (the weight gradients of a network's layers:
@@ -553,7 +617,7 @@ void k_gemm_f32_group(GemmGroupArgs a) {
   g.A = q.A; g.B = q.B; g.C = q.C; g.bias = nullptr;
   g.M = q.M; g.N = q.N; g.K = q.K;
   g.lda = A_KCONTIG ? q.K : q.M; g.ldb = B_KCONTIG ? q.K : q.N; g.ldc = q.N;
-  g.k_per_split = q.K; g.split_out = nullptr; g.stats_out = nullptr; g.clock_out = nullptr;
+  g.k_per_split = q.K; g.split_out = nullptr; g.stats_out = nullptr; g.clock_out = nullptr; g.db_out = nullptr;
   g.snap_a = nullptr; g.snap_b = nullptr; g.snap_out = nullptr;
   g.accumulate = a.accumulate; g.a_vec = 1; g.b_vec = 1;
   g.tiles_n = q.tiles_n; g.tiles_m = (q.M + BM - 1) / BM;
@@ -563,10 +627,29 @@ void k_gemm_f32_group(GemmGroupArgs a) {
 // Fixed-order sum of the split-K partial products (+ bias, + previous C): slice 0, 1, 2, ... as before, with
 // the loads of eight slices in flight at a time (one thread per element would otherwise walk the slices one
 // memory latency after the other: 17 us for 64 slices of a 256 x 256 product).
+// db_part != nullptr: also db[m] (+)= the slices' sums [splits][M] of the A operand's rows (the bias gradient that a
+// split weight gradient formed on its way), slice 0 first.
 __global__ __launch_bounds__(256) void k_splitk_reduce(float const *__restrict__ part, unsigned splits, size_t mn,
                                                         size_t N, float const *__restrict__ bias,
-                                                        float *__restrict__ C, int accumulate) {
+                                                        float *__restrict__ C, int accumulate,
+                                                        float const *__restrict__ db_part, float *__restrict__ db,
+                                                        size_t M) {
   size_t const stride = static_cast<size_t>(gridDim.x) * 256;
+  if (db_part != nullptr) {
+    for (size_t m = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; m < M; m += stride) {
+      float s = 0.0f;
+      unsigned z = 0;
+      for (; z + 8 <= splits; z += 8) {  // (eight loads in flight, added in slice order)
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = db_part[(z + u) * M + m];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
+      }
+      for (; z < splits; ++z) s += db_part[z * M + m];
+      db[m] = accumulate ? db[m] + s : s;
+    }
+  }
   for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < mn; i += stride) {
     float s = 0.0f;
     unsigned z = 0;
@@ -585,15 +668,18 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(float const *__restrict__
 }
 
 // ---------------------------------------------------------------- host side
-template <int BM, int BN, int BK, bool AK, bool BKC, int WPE, bool HAS_CLAMPED, int RST, int WVM = 2>
+template <int BM, int BN, int BK, bool AK, bool BKC, int WPE, bool HAS_CLAMPED, int RST, int WVM = 2, bool DB = false>
 static int launch_gemm(dlmi_ctx *ctx, GemmArgs g, unsigned splits, int mode) {
+  if (DB && mode != kFast) return dlmi_fail(ctx, DLMI_E_INVALID, "launch_gemm: the bias-gradient variant is a fast-path kernel");
   using TA = TileShape<BM, BK, AK, 128 * WVM>;
   using TB = TileShape<BN, BK, BKC, 128 * WVM>;
   constexpr size_t lds_bytes = 2 * (TA::kFloats + TB::kFloats) * sizeof(float);
   g.tiles_m = static_cast<unsigned>(dlmi_ceil_div(g.M, BM));
   g.tiles_n = static_cast<unsigned>(dlmi_ceil_div(g.N, BN));
   dim3 const grid(g.tiles_m * g.tiles_n, 1, splits);
-  auto const kfast = k_gemm_f32<BM, BN, BK, AK, BKC, kFast, WPE, RST, WVM>;
+  void (*kfast)(GemmArgs);
+  if constexpr (DB) kfast = k_gemm_f32_db<BM, BN, BK, AK, BKC, WPE, RST, WVM>;
+  else kfast = k_gemm_f32<BM, BN, BK, AK, BKC, kFast, WPE, RST, WVM>;
   auto const kslow = k_gemm_f32<BM, BN, BK, AK, BKC, kGuarded, WPE, 1, WVM>;
   // the clamped variant exists for the small tiles, which are the ones ragged layers run
   auto const kclamp = k_gemm_f32<BM, BN, BK, AK, BKC, HAS_CLAMPED ? kClamped : kGuarded, WPE, HAS_CLAMPED ? RST : 1, WVM>;
@@ -627,7 +713,7 @@ template <bool AK, bool BKC>
 static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, size_t lda, float const *B, size_t ldb,
                 float *C, float const *bias, int accumulate, unsigned *stats_chunks = nullptr,
                 unsigned *defer_slices = nullptr, float const *snap_a = nullptr, float const *snap_b = nullptr,
-                float const **snap_out = nullptr) {
+                float const **snap_out = nullptr, float *db = nullptr, bool *db_done = nullptr) {
   GemmPlan const plan = plan_gemm(ctx->num_cu, M, N, K);
   int const choice = plan.choice;
   int const bm = plan.bm, bn = plan.bn, bk = plan.bk;
@@ -637,6 +723,8 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   g.accumulate = accumulate; g.split_out = nullptr; g.stats_out = nullptr;
   g.snap_a = g.snap_b = nullptr; g.snap_out = nullptr;
   g.clock_out = ctx->gemm_clock;
+  g.db_out = nullptr;
+  if (db_done != nullptr) *db_done = false;
   if (snap_out != nullptr) *snap_out = nullptr;
   g.a_vec = (lda % 4 == 0 && dlmi_aligned16(A)) ? 1 : 0;
   g.b_vec = (ldb % 4 == 0 && dlmi_aligned16(B)) ? 1 : 0;
@@ -650,7 +738,8 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   size_t const ktiles = dlmi_ceil_div(K, bk);
   unsigned splits = plan.splits;
   if (splits > 1) {
-    int rc = dlmi_scratch_reserve(ctx, plan.scratch_bytes);
+    // (room for the slices' shares of a bias gradient behind the partial products)
+    int rc = dlmi_scratch_reserve(ctx, plan.scratch_bytes + static_cast<size_t>(splits) * M * sizeof(float));
     if (rc != DLMI_OK) return rc;
   }
   if (stats_chunks != nullptr) {
@@ -676,6 +765,15 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
   g.k_per_split = kt_per_split * bk;
   splits = static_cast<unsigned>(dlmi_ceil_div(ktiles, kt_per_split));
   if (splits > 1) g.split_out = reinterpret_cast<float *>(dlmi_scratch_data(ctx));
+  // A weight gradient that is split over K and runs the fast 128 x 128 kernels forms the bias gradient on its way:
+  // the slices leave their shares behind the partial products, and the slice sum below adds them up too.  (Such a
+  // product never shares a launch with others, so the grouped entry point takes this same path for it.)
+  bool db_in_product = false;
+  if constexpr (!AK) {
+    db_in_product = db != nullptr && defer_slices == nullptr && splits > 1 && mode == kFast && (choice == 0 || choice == 4) &&
+                    ctx->tune.db_in_product != 0;
+    if (db_in_product) g.db_out = g.split_out + static_cast<size_t>(splits) * M * N;
+  }
   int rc;
   switch (choice) {
     case 1: rc = launch_gemm<256, 128, 16, AK, BKC, 2, false, 1>(ctx, g, splits, mode); break;
@@ -692,12 +790,30 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
       break;
     // 8 wavefronts (4 along M x 2 along N) behind one barrier, one workgroup per CU, two wavefronts per SIMD
     case 4:
+      if constexpr (!AK) {
+        if (db_in_product) {
+          if (gemm_register_stages(bm, bn, kt_per_split) == 2)
+            rc = launch_gemm<128, 128, 16, AK, BKC, 2, false, 2, 4, true>(ctx, g, splits, mode);
+          else
+            rc = launch_gemm<128, 128, 16, AK, BKC, 2, false, 1, 4, true>(ctx, g, splits, mode);
+          break;
+        }
+      }
       if (gemm_register_stages(bm, bn, kt_per_split) == 2)
         rc = launch_gemm<128, 128, 16, AK, BKC, 2, false, 2, 4>(ctx, g, splits, mode);
       else
         rc = launch_gemm<128, 128, 16, AK, BKC, 2, false, 1, 4>(ctx, g, splits, mode);
       break;
     default:
+      if constexpr (!AK) {
+        if (db_in_product) {
+          if (gemm_register_stages(bm, bn, kt_per_split) == 2)
+            rc = launch_gemm<128, 128, 16, AK, BKC, 2, true, 2, 2, true>(ctx, g, splits, mode);
+          else
+            rc = launch_gemm<128, 128, 16, AK, BKC, 2, true, 1, 2, true>(ctx, g, splits, mode);
+          break;
+        }
+      }
       if (gemm_register_stages(bm, bn, kt_per_split) == 2)
         rc = launch_gemm<128, 128, 16, AK, BKC, 2, true, 2>(ctx, g, splits, mode);
       else
@@ -716,8 +832,9 @@ static int gemm(dlmi_ctx *ctx, size_t M, size_t N, size_t K, float const *A, siz
     size_t const cap = static_cast<size_t>(ctx->num_cu) * 16;
     if (blocks > cap) blocks = cap;
     hipLaunchKernelGGL(k_splitk_reduce, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, ctx->stream,
-                       g.split_out, splits, mn, N, bias, C, accumulate);
+                       g.split_out, splits, mn, N, bias, C, accumulate, static_cast<float const *>(g.db_out), db, M);
     DLMI_LAUNCH_CHECK(ctx, "k_splitk_reduce");
+    if (db_in_product && db_done != nullptr) *db_done = true;
   }
   return DLMI_OK;
 }
@@ -893,9 +1010,12 @@ int dlmi_fc_bwd_dw(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin
   if (int const took = narrow_dw_try(ctx, B, K, H, Xin, dZ, dW, db, accumulate); took != 0) return took < 0 ? took : DLMI_OK;
   // any layer on a mini-batch: the reduction is the batch, a handful of K tiles; a kernel that stages it whole
   int rc = minibatch_dw_try(ctx, B, K, H, Xin, dZ, dW, accumulate);
-  if (rc == 0) rc = gemm<false, false>(ctx, H, K, B, dZ, H, Xin, K, dW, nullptr, accumulate);
+  bool db_done = false;  // a product split over K brings the bias gradient along
+  if (rc == 0)
+    rc = gemm<false, false>(ctx, H, K, B, dZ, H, Xin, K, dW, nullptr, accumulate, nullptr, nullptr, nullptr, nullptr, nullptr,
+                            db, &db_done);
   else rc = rc < 0 ? rc : DLMI_OK;
-  if (rc != DLMI_OK || db == nullptr) return rc;
+  if (rc != DLMI_OK || db == nullptr || db_done) return rc;
   // db[h] (+)= sum_b dZ[b,h] (update_derivative_fwp_st.cpp:283-302)
   return column_sums(ctx, B, H, dZ, db, accumulate);
 }

@@ -121,7 +121,9 @@ size_t fc_scratch_bytes(dlmi_ctx const *ctx, size_t B, size_t K, size_t H) {
   if (2 * 2 * rows * H * sizeof(float) > need) need = 2 * 2 * rows * H * sizeof(float);
   size_t const shapes[3][3] = {{B, H, K}, {B, K, H}, {H, K, B}};
   for (auto const &sh : shapes) {
-    size_t const b = plan_gemm(ctx->num_cu, sh[0], sh[1], sh[2]).scratch_bytes;
+    GemmPlan const p = plan_gemm(ctx->num_cu, sh[0], sh[1], sh[2]);
+    // (behind the partial products of a split: the slices' shares of a bias gradient, [splits][M])
+    size_t const b = p.scratch_bytes + (p.splits > 1 ? static_cast<size_t>(p.splits) * sh[0] * sizeof(float) : 0);
     if (b > need) need = b;
   }
   return need;

@@ -145,7 +145,8 @@ int dlmi_fc_bwd_dx(dlmi_ctx *ctx, size_t B, size_t Hn, size_t H, float const *dZ
  * NULL: normalized layers have no bias, v1/learner/model.hpp:708).
  * Replaces Model::Update_Derivative_Weight__FC__* and …__Bias__*
  * (update_derivative_fwp_st.cpp:246-302, update_derivative_fwp_mp.cpp:175-240)
- * together with the thread merge of merge.cpp:76-100.
+ * together with the thread merge of merge.cpp:76-100.  A product that is split over K (few output tiles, a long
+ * batch) forms db on its way, from the rows of dZ it stages; otherwise db takes a pass of its own over dZ.
  * Xin [B,K], dZ [B,H], dW [H,K], db [H]: device. */
 int dlmi_fc_bwd_dw(dlmi_ctx *ctx, size_t B, size_t K, size_t H, float const *Xin, float const *dZ,
                    float *dW, float *db, int accumulate);
