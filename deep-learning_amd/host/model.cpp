@@ -269,7 +269,7 @@ float const *Model::Impl::slots_upload(RowSlots &s, size_t const B, size_t const
 Model::Model(void) : impl_(new Impl) {
   real_gen.seed(5489u);
   gaussian_gen.seed(5489u);
-  gaussian_dist.reset();
+  gaussian_spare_available = false;
   bernoulli = new Dist::Bernoulli[1];
 }
 
@@ -312,7 +312,7 @@ void Model::clear(void) {
   static_cast<Model_State &>(*this) = Model_State();  // every public member takes its default again
   real_gen.seed(5489u);
   gaussian_gen.seed(5489u);
-  gaussian_dist.reset();
+  gaussian_spare_available = false;
   bernoulli = masks;
 }
 
@@ -1031,9 +1031,31 @@ void Model::Initialization__Uniform(real const bias, real const lower_bound, rea
 }
 
 // layers_initialize_orthogonal / weights_initialize_orthogonal (orthogonal.cpp:39-154)
+// std::normal_distribution<real>(0, 1)(mt19937) as libstdc++ computes it (bits/random.tcc: Marsaglia's polar method,
+// the second value of a pair kept for the next call).  The reference's builds (GCC on a target with FMA, which
+// its -march=native release configuration gives on any current host) contract x*x + y*y into fma(x, x, y*y); it
+// is written as one here, so the draws are the same bits whatever this file is compiled for - checked against the
+// compiled reference in tests/test_gpu_lsuv.py.  (2u - 1 and value * 1 + 0 are exact either way.)
+real Model::gaussian_draw(void) {
+  if (gaussian_spare_available) {
+    gaussian_spare_available = false;
+    return gaussian_spare;
+  }
+  real x, y, r2;
+  do {
+    x = 2.0f * std::generate_canonical<real, std::numeric_limits<real>::digits>(gaussian_gen) - 1.0f;
+    y = 2.0f * std::generate_canonical<real, std::numeric_limits<real>::digits>(gaussian_gen) - 1.0f;
+    r2 = std::fma(x, x, y * y);
+  } while (r2 > 1.0f || r2 == 0.0f);
+  real const mult = std::sqrt(-2 * std::log(r2) / r2);
+  gaussian_spare = x * mult;
+  gaussian_spare_available = true;
+  return y * mult;
+}
+
 void Model::weights_initialize_orthogonal(size_t const rows, size_t const cols, real const scale, var *weights) {
   // weights_initialize_gaussian(weights, weights + rows * cols, 1) (model.cpp:5401-5409)
-  for (size_t i = 0, n = rows * cols; i < n; ++i) weights[i] = gaussian_dist(gaussian_gen);
+  for (size_t i = 0, n = rows * cols; i < n; ++i) weights[i] = gaussian_draw();
   if (dlmi_orthogonal_weights(rows, cols, scale, weights) != 1) fail("weights_initialize_orthogonal: empty layer");
 }
 

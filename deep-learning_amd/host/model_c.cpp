@@ -94,9 +94,9 @@ void dlmi_model_init_uniform(dlmi_model *h, unsigned seed, float bias, float low
   h->m.Initialization__Uniform(bias, lower, upper);
 }
 
-void dlmi_model_seed_gaussian(dlmi_model *h, unsigned seed) {
-  h->m.gaussian_gen.seed(seed);
-  h->m.gaussian_dist.reset();
+void dlmi_model_seed_gaussian(dlmi_model *h, unsigned seed) { h->m.gaussian_gen.seed(seed); }
+void dlmi_model_gaussian_draws(dlmi_model *h, size_t n, float *out) {
+  for (size_t i = 0; i < n; ++i) out[i] = h->m.gaussian_draw();
 }
 void dlmi_model_orthogonal(dlmi_model *h, unsigned seed, float bias) {
   dlmi_model_seed_gaussian(h, seed);

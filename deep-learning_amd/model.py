@@ -196,6 +196,11 @@ class Model:
     def seed_gaussian(self, seed):
         self.lib.dlmi_model_seed_gaussian(self.h, ctypes.c_uint(seed))
 
+    def gaussian_draws(self, n):
+        out = np.empty(n, np.float32)
+        self.lib.dlmi_model_gaussian_draws(self.h, c_sz(n), _ptr(out))
+        return out
+
     def lsuv(self, X, max_n_trials=10, max_batch_size=32, bias=0.0, var_target=1.0, var_tolerance=0.01, pre_initialize=True):
         """Initialize__LSUV + Initialization__LSUV on the rows of X; returns the scalings applied per layer.
         pre_initialize=False: the scaling loop alone, on the weights the model holds."""

@@ -33,8 +33,11 @@ void dlmi_model_init_uniform(dlmi_model *m, unsigned seed, float bias, float low
 /* gaussian_gen.seed(seed) and a fresh distribution state, then layers_initialize_orthogonal(false, bias)
  * (v1/ops/initializers/orthogonal.cpp:39-105). */
 void dlmi_model_orthogonal(dlmi_model *m, unsigned seed, float bias);
-/* Only the seeding of the above: what a later dlmi_model_lsuv(..., pre_initialize = 1) draws from. */
+/* Only the seeding of the above (gaussian.seed(seed) of the reference: the engine alone): what a later
+ * dlmi_model_lsuv(..., pre_initialize = 1) draws from.  dlmi_model_gaussian_draws: n draws of N(0, 1) from the
+ * model's generator, as weights_initialize_gaussian takes them (model.cpp:5401-5409; for tests of the stream). */
 void dlmi_model_seed_gaussian(dlmi_model *m, unsigned seed);
+void dlmi_model_gaussian_draws(dlmi_model *m, size_t n, float *out);
 /* Host arithmetic, no device and no model needed: the second half of Model::weights_initialize_orthogonal
  * (orthogonal.cpp:132-153).  `weights` [rows * cols] (rows = fan-in, cols = units; the Gaussian draws) is read as a
  * column-major matrix of max(rows, cols) x min(rows, cols), replaced by Q . sign(diag R) of its column-pivoting QR

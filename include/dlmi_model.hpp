@@ -221,11 +221,14 @@ struct Model_State {
   // path is DLMI_DROP_BWD_REFERENCE.
   dlmi_dropout_bwd dropout_backward_mode = DLMI_DROP_BWD_REFERENCE;
   std::mt19937 real_gen;  // weight initializers (the engine inside the reference's Dist::Real real_gen)
-  // The orthogonal initializer's draws: the engine and the distribution object inside the reference's
-  // Dist::Gaussian gaussian (ops/distributions/gaussian.cpp: std::normal_distribution<real> over std::mt19937; the
-  // distribution keeps its spare value from one layer to the next, as there).
+  // The orthogonal initializer's draws: the engine inside the reference's Dist::Gaussian gaussian
+  // (ops/distributions/gaussian.cpp: std::normal_distribution<real>(0, 1) over std::mt19937) and the state of that
+  // distribution - Marsaglia's polar method makes two values at a time and keeps the spare one for the next call,
+  // from one layer to the next too.  Model::gaussian_draw() is libstdc++'s algorithm written out, with the one
+  // fused multiply-add the reference's builds contract it to (see the definition).
   std::mt19937 gaussian_gen;
-  std::normal_distribution<real> gaussian_dist{0.0f, 1.0f};
+  bool gaussian_spare_available = false;
+  real gaussian_spare = 0.0f;
   // false: Initialization__LSUV keeps the weights at hand instead of starting from the orthogonal initializer
   // (no reference counterpart; see Initialization__LSUV)
   bool lsuv_pre_initialize = true;
@@ -290,6 +293,7 @@ class Model : public Model_State {
   // factorization is this library's own (host, double precision): **parity with Eigen's unpinned** - it is held to
   // LAPACK's column-pivoting QR, which picks its pivots by the same rule.
   void layers_initialize_orthogonal(bool const pre_initialize, real const bias = 0.0f);
+  real gaussian_draw(void);  // one value of N(0, 1): Dist::Gaussian::operator() of the reference
   void weights_initialize_orthogonal(size_t const rows, size_t const cols, real const scale, var *weights);
   // LSUV, "all you need is a good init" (v1/ops/initializers/lsuv.cpp:27-177; model.cpp:2813-2858).
   // Initialize__LSUV keeps the settings; Initialization__LSUV then, layer by layer from the first hidden one,

@@ -809,6 +809,12 @@ class ReferenceMLP:
         """real_gen.seed(seed); Initialization__Uniform(bias, lower, upper)"""
         self.lib.dlref_model_init_uniform(self.h, ctypes.c_uint(seed), c_f(bias), c_f(lower), c_f(upper))
 
+    def gaussian_draws(self, seed, n):
+        """gaussian.seed(seed); weights_initialize_gaussian over n values, variance 1 (model.cpp:5401-5409)"""
+        out = np.empty(n, np.float32)
+        self.lib.dlref_model_gaussian_draws(self.h, ctypes.c_uint(seed), c_sz(n), _ptr(out))
+        return out
+
     def dropout_bernoulli(self, seed=None):
         """[bernoulli[0].seed(seed);] Model::Dropout_Bernoulli() on a single-thread model."""
         ok = self.lib.dlref_model_dropout_bernoulli(self.h, ctypes.c_uint(seed or 0), c_int(int(seed is not None)))

@@ -459,6 +459,14 @@ void dlref_model_init_uniform(void *h, unsigned seed, float bias, float lower, f
   m.Initialization__Uniform(bias, lower, upper);
 }
 
+// The draws the orthogonal initializer starts from (orthogonal.cpp:130; the factorization behind them needs Eigen
+// and is not part of this build): gaussian.seed(seed), weights_initialize_gaussian(out, out + n, 1) (model.cpp:5401-5409).
+void dlref_model_gaussian_draws(void *h, unsigned seed, size_t n, float *out) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  m.gaussian.seed(seed);
+  m.weights_initialize_gaussian(out, out + n, 1.0f);
+}
+
 void dlref_model_destroy(void *h) { delete static_cast<RefModel *>(h); }
 
 int dlref_model_set_activation(void *h, size_t layer, int type) {

@@ -238,3 +238,19 @@ def test_lsuv_starts_from_the_orthogonal_initializer(lib):
     finally:
         a.close()
         b.close()
+
+
+def test_gaussian_draws_are_the_references(lib, reference):
+    """The N(0, 1) draws the orthogonal initializer starts from, against the compiled reference's own
+    gaussian.seed(seed) + weights_initialize_gaussian (model.cpp:5401-5409), bit for bit: an odd count first, so
+    that the distribution's spare value crosses from one call into the next, as it does from layer to layer."""
+    g = gpu_model(lib, [6, 5, 3], ["TANH", "LINEAR"], ["NONE"])
+    r = build(reference.mlp, [6, 5, 3], ["TANH", "LINEAR"], ["NONE"])
+    try:
+        g.seed_gaussian(123)
+        a = np.concatenate([g.gaussian_draws(7), g.gaussian_draws(30)])
+        b = r.gaussian_draws(123, 37)
+        assert np.array_equal(a, b)
+        assert abs(float(a.mean())) < 0.6 and 0.5 < float(a.std()) < 1.6
+    finally:
+        g.close()
