@@ -984,10 +984,23 @@ static void finish_initialization(Model &m) {
   (void)m.upload_moving_statistics();
 }
 
-void Model::initialize_weights_with_glorot_uniform(real const bias) {
-  if (ptr_array_layers == nullptr) { fail("initialize_weights_with_glorot_uniform: model not compiled"); return; }
-  for (size_t li = 1; li < total_layers; ++li) {
-    Layer const &l = ptr_array_layers[li];
+// Initialization__Gaussian__Variance (glorot.cpp:68-88): the standard deviation of the Gaussian form
+static real gaussian_variance(size_t const n_inp, size_t const n_out, ACTIVATION::TYPE const t) {
+  switch (t) {
+    case ACTIVATION::LEAKY_RELU: case ACTIVATION::PARAMETRIC_RELU: case ACTIVATION::RELU: case ACTIVATION::SELU:
+      return std::sqrt(1.0f / static_cast<real>(n_inp));
+    default:
+      return std::sqrt(2.0f / static_cast<real>(n_inp + n_out));
+  }
+}
+
+// What both Glorot initializers walk (glorot.cpp:112-222, 225-359): per fully-connected layer its fan-in, the
+// reference's fan-out and the layer whose activation sets the gain; draw(l, n_inp, n_out, gain layer) fills the
+// weights, the bias slots are set here.
+template <class Draw>
+static void glorot_layers(Model &m, real const bias, bool const first_next_only, Draw const &draw) {
+  for (size_t li = 1; li < m.total_layers; ++li) {
+    Layer const &l = m.ptr_array_layers[li];
     if (l.type_layer != LAYER::FULLY_CONNECTED) continue;
     size_t const n_inp = l.n_inp;
     // fan-out as glorot.cpp:253-268 finds it through next_connected_layers: the
@@ -995,12 +1008,14 @@ void Model::initialize_weights_with_glorot_uniform(real const bias) {
     // entry; for a layer followed by a block the mean of the RESIDUAL entry's
     // width and the block's first layer's; for the output layer the fan-in.
     size_t n_out = n_inp;
-    if (li + 1 != total_layers) {
-      Layer const &nx = ptr_array_layers[li + 1];
-      if (l.in_block && li == l.block_index + ptr_array_layers[l.block_index].block_depth)
-        n_out = ptr_array_layers[l.block_index].n_out;
+    if (li + 1 != m.total_layers) {
+      Layer const &nx = m.ptr_array_layers[li + 1];
+      if (l.in_block && li == l.block_index + m.ptr_array_layers[l.block_index].block_depth)
+        n_out = m.ptr_array_layers[l.block_index].n_out;
       else if (nx.type_layer == LAYER::RESIDUAL)
-        n_out = (nx.n_out + ptr_array_layers[li + 2].n_out) / 2;
+        // (two next connections.  The Gaussian form's loop stops after the first of them and still divides by their
+        // number, glorot.cpp:144-157: half the RESIDUAL entry's width.  Kept.)
+        n_out = first_next_only ? nx.n_out / 2 : (nx.n_out + m.ptr_array_layers[li + 2].n_out) / 2;
       else
         n_out = nx.n_out;
     }
@@ -1008,12 +1023,32 @@ void Model::initialize_weights_with_glorot_uniform(real const bias) {
     // block's first layer has none, and the read lands on the first unit of the
     // next layer that has some: that layer's activation sets the gain.
     size_t ga = li;
-    while (ga + 1 < total_layers && (ptr_array_layers[ga].type_layer != LAYER::FULLY_CONNECTED || ptr_array_layers[ga].block_first)) ++ga;
-    real const v = gain_scale(ptr_array_layers[ga].type_activation_function) * uniform_variance(n_inp, n_out, l.type_activation_function);
+    while (ga + 1 < m.total_layers && (m.ptr_array_layers[ga].type_layer != LAYER::FULLY_CONNECTED || m.ptr_array_layers[ga].block_first)) ++ga;
+    draw(l, n_inp, n_out, m.ptr_array_layers[ga].type_activation_function);
+    for (size_t i = 0; i < l.n_out; ++i) m.ptr_array_parameters[l.first_bias_connection_index + i] = bias;  // model.cpp:5031-5042
+  }
+}
+
+void Model::initialize_weights_with_glorot_uniform(real const bias) {
+  if (ptr_array_layers == nullptr) { fail("initialize_weights_with_glorot_uniform: model not compiled"); return; }
+  glorot_layers(*this, bias, false, [&](Layer const &l, size_t const n_inp, size_t const n_out, ACTIVATION::TYPE const gain_of) {
+    real const v = gain_scale(gain_of) * uniform_variance(n_inp, n_out, l.type_activation_function);
     var *w = ptr_array_parameters + l.first_connection_index;
     for (size_t i = 0, n = l.n_out * n_inp; i < n; ++i) w[i] = uniform_draw(real_gen, -v, v);  // model.cpp:5087-5096
-    for (size_t i = 0; i < l.n_out; ++i) ptr_array_parameters[l.first_bias_connection_index + i] = bias;  // model.cpp:5031-5042
-  }
+  });
+  finish_initialization(*this);
+}
+
+// Initialization__Glorot__Gaussian (glorot.cpp:110-222): N(0, gain * sqrt(2 / (fan_in + fan_out))), rectifier and SELU
+// layers N(0, gain * sqrt(1 / fan_in)); a draw is the standard one times that deviation (plus a mean of 0), as
+// std::normal_distribution scales it (weights_initialize_gaussian, model.cpp:5401-5409).
+void Model::Initialization__Glorot__Gaussian(real const bias) {
+  if (ptr_array_layers == nullptr) { fail("Initialization__Glorot__Gaussian: model not compiled"); return; }
+  glorot_layers(*this, bias, true, [&](Layer const &l, size_t const n_inp, size_t const n_out, ACTIVATION::TYPE const gain_of) {
+    real const v = gain_scale(gain_of) * gaussian_variance(n_inp, n_out, l.type_activation_function);
+    var *w = ptr_array_parameters + l.first_connection_index;
+    for (size_t i = 0, n = l.n_out * n_inp; i < n; ++i) w[i] = gaussian_draw() * v + 0.0f;
+  });
   finish_initialization(*this);
 }
 

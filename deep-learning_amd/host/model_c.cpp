@@ -95,6 +95,10 @@ void dlmi_model_init_uniform(dlmi_model *h, unsigned seed, float bias, float low
 }
 
 void dlmi_model_seed_gaussian(dlmi_model *h, unsigned seed) { h->m.gaussian_gen.seed(seed); }
+void dlmi_model_glorot_gaussian(dlmi_model *h, unsigned seed, float bias) {
+  h->m.gaussian_gen.seed(seed);
+  h->m.Initialization__Glorot__Gaussian(bias);
+}
 void dlmi_model_gaussian_draws(dlmi_model *h, size_t n, float *out) {
   for (size_t i = 0; i < n; ++i) out[i] = h->m.gaussian_draw();
 }

@@ -160,6 +160,10 @@ class Model:
         """real_gen.seed(seed); initialize_weights_with_glorot_uniform(bias)"""
         self.lib.dlmi_model_glorot_uniform(self.h, ctypes.c_uint(seed), c_f(bias))
 
+    def glorot_gaussian(self, seed, bias=0.0):
+        """gaussian_gen.seed(seed); Initialization__Glorot__Gaussian(bias)"""
+        self.lib.dlmi_model_glorot_gaussian(self.h, ctypes.c_uint(seed), c_f(bias))
+
     def init_uniform(self, seed, bias=0.0, lower=-1.0, upper=1.0):
         """real_gen.seed(seed); Initialization__Uniform(bias, lower, upper)"""
         self.lib.dlmi_model_init_uniform(self.h, ctypes.c_uint(seed), c_f(bias), c_f(lower), c_f(upper))

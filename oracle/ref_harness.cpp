@@ -459,6 +459,12 @@ void dlref_model_init_uniform(void *h, unsigned seed, float bias, float lower, f
   m.Initialization__Uniform(bias, lower, upper);
 }
 
+// gaussian.seed(seed); Initialization__Glorot__Gaussian(bias) (glorot.cpp:110-222)
+void dlref_model_glorot_gaussian(void *h, unsigned seed, float bias) {
+  Model &m = static_cast<RefModel *>(h)->model;
+  m.gaussian.seed(seed);
+  m.Initialization__Glorot__Gaussian(bias);
+}
 // The draws the orthogonal initializer starts from (orthogonal.cpp:130; the factorization behind them needs Eigen
 // and is not part of this build): gaussian.seed(seed), weights_initialize_gaussian(out, out + n, 1) (model.cpp:5401-5409).
 void dlref_model_gaussian_draws(void *h, unsigned seed, size_t n, float *out) {

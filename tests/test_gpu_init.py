@@ -61,3 +61,29 @@ def test_same_seed_same_weights_other_seed_other_weights(net_factory):
         return M.get_parameters()
     a, b, c = weights(42), weights(42), weights(43)
     assert np.array_equal(a, b) and not np.array_equal(a, c)
+
+
+@pytest.mark.parametrize("name", [n for n, c in init_cases().items() if c[5] is None])
+def test_gaussian_glorot_against_the_compiled_reference(net_factory, reference, name):
+    """Initialization__Glorot__Gaussian (glorot.cpp:110-222) on the networks of the uniform cases, residual blocks
+    included: the parameter vector after the call is the compiled reference's bit for bit (same walk over the
+    layers, the reference's own Gaussian stream), the tail of the initialization as for the other initializers."""
+    from oracle.binding import ReferenceNet
+    layers, acts, norms, seed, bias, _ = init_cases()[name]
+    M, R = net_factory(layers), ReferenceNet(reference, layers)
+    for m in (M, R):
+        for l in sorted(set(acts) | set(norms)):
+            m.set_layer(l, ACT[acts[l]] if l in acts else 0, NORM[norms.get(l, "NONE")])
+        m.prepare(4)
+    assert [M.P, M.n_units] == [R.P, R.n_units]
+    rng = np.random.default_rng(seed)
+    p0 = rng.uniform(-2, 2, M.P).astype(np.float32)
+    mv = rng.uniform(-2, 2, M.n_units).astype(np.float32), rng.uniform(1, 3, M.n_units).astype(np.float32)
+    for m in (M, R):
+        m.set_parameters(p0)
+        m.set_moving(*mv)
+        m.glorot_gaussian(seed, bias)
+    assert np.array_equal(M.get_parameters(), R.get_parameters())
+    (mm, ms), (rm, rs) = M.get_moving(), R.get_moving()
+    assert np.array_equal(mm, rm) and np.array_equal(ms, rs)
+    assert not np.array_equal(M.get_parameters(), p0)
