@@ -1065,6 +1065,23 @@ void Model::Initialization__Uniform(real const bias, real const lower_bound, rea
   finish_initialization(*this);
 }
 
+// Initialization__Identity / weights_initialize_identity (identity.cpp:25-103): zeros, and a one at [i * units + i]
+// for i below min(fan-in, units) - the reference's own index arithmetic, which is the diagonal of the [units][fan-in]
+// array only where the two are equal; kept as it is.
+void Model::Initialization__Identity(real const bias) {
+  if (ptr_array_layers == nullptr) { fail("Initialization__Identity: model not compiled"); return; }
+  for (size_t li = 1; li < total_layers; ++li) {
+    Layer const &l = ptr_array_layers[li];
+    if (l.type_layer != LAYER::FULLY_CONNECTED) continue;
+    size_t const rows = l.n_inp, cols = l.n_out;
+    var *w = ptr_array_parameters + l.first_connection_index;
+    std::memset(w, 0, rows * cols * sizeof(var));
+    for (size_t i = 0, n = std::min(rows, cols); i < n; ++i) w[i * cols + i] = 1.0f;
+    for (size_t i = 0; i < l.n_out; ++i) ptr_array_parameters[l.first_bias_connection_index + i] = bias;
+  }
+  finish_initialization(*this);
+}
+
 // layers_initialize_orthogonal / weights_initialize_orthogonal (orthogonal.cpp:39-154)
 // std::normal_distribution<real>(0, 1)(mt19937) as libstdc++ computes it (bits/random.tcc: Marsaglia's polar method,
 // the second value of a pair kept for the next call).  The reference's builds (GCC on a target with FMA, which

@@ -95,6 +95,7 @@ void dlmi_model_init_uniform(dlmi_model *h, unsigned seed, float bias, float low
 }
 
 void dlmi_model_seed_gaussian(dlmi_model *h, unsigned seed) { h->m.gaussian_gen.seed(seed); }
+void dlmi_model_init_identity(dlmi_model *h, float bias) { h->m.Initialization__Identity(bias); }
 void dlmi_model_glorot_gaussian(dlmi_model *h, unsigned seed, float bias) {
   h->m.gaussian_gen.seed(seed);
   h->m.Initialization__Glorot__Gaussian(bias);

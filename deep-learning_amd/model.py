@@ -164,6 +164,10 @@ class Model:
         """gaussian_gen.seed(seed); Initialization__Glorot__Gaussian(bias)"""
         self.lib.dlmi_model_glorot_gaussian(self.h, ctypes.c_uint(seed), c_f(bias))
 
+    def init_identity(self, bias=0.0):
+        """Initialization__Identity(bias)"""
+        self.lib.dlmi_model_init_identity(self.h, c_f(bias))
+
     def init_uniform(self, seed, bias=0.0, lower=-1.0, upper=1.0):
         """real_gen.seed(seed); Initialization__Uniform(bias, lower, upper)"""
         self.lib.dlmi_model_init_uniform(self.h, ctypes.c_uint(seed), c_f(bias), c_f(lower), c_f(upper))

@@ -32,6 +32,8 @@ void dlmi_model_glorot_uniform(dlmi_model *m, unsigned seed, float bias);
 void dlmi_model_init_uniform(dlmi_model *m, unsigned seed, float bias, float lower, float upper);
 /* gaussian_gen.seed(seed), then Initialization__Glorot__Gaussian(bias) (glorot.cpp:110-222) */
 void dlmi_model_glorot_gaussian(dlmi_model *m, unsigned seed, float bias);
+/* Initialization__Identity(bias) (identity.cpp:25-103) */
+void dlmi_model_init_identity(dlmi_model *m, float bias);
 /* gaussian_gen.seed(seed) and a fresh distribution state, then layers_initialize_orthogonal(false, bias)
  * (v1/ops/initializers/orthogonal.cpp:39-105). */
 void dlmi_model_orthogonal(dlmi_model *m, unsigned seed, float bias);

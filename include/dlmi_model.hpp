@@ -286,6 +286,8 @@ class Model : public Model_State {
   // The Gaussian form (glorot.cpp:110-222): the same walk, the weights from N(0, gain * sqrt(2 / (fan_in + fan_out)))
   // (rectifier and SELU layers: gain * sqrt(1 / fan_in)), drawn with gaussian_draw() from `gaussian_gen`.
   void Initialization__Glorot__Gaussian(real const bias = 0.0f);
+  // Identity initializer (identity.cpp:25-103): zeros with ones at [i * units + i], i < min(fan-in, units).
+  void Initialization__Identity(real const bias = 0.0f);
   void Initialization__Uniform(real const bias = 0.0f, real const lower_bound = -1.0f, real const upper_bound = 1.0f);
   // Orthogonal initializer (v1/ops/initializers/orthogonal.cpp:39-154), fully-connected layers: a layer's weights
   // are drawn from N(0, 1) in parameter order (`gaussian_gen`), read as a column-major matrix of max(fan-in, units) x

@@ -809,6 +809,10 @@ class ReferenceMLP:
         """real_gen.seed(seed); Initialization__Uniform(bias, lower, upper)"""
         self.lib.dlref_model_init_uniform(self.h, ctypes.c_uint(seed), c_f(bias), c_f(lower), c_f(upper))
 
+    def init_identity(self, bias=0.0):
+        """Initialization__Identity(bias)"""
+        self.lib.dlref_model_init_identity(self.h, c_f(bias))
+
     def glorot_gaussian(self, seed, bias=0.0):
         """gaussian.seed(seed); Initialization__Glorot__Gaussian(bias)"""
         self.lib.dlref_model_glorot_gaussian(self.h, ctypes.c_uint(seed), c_f(bias))

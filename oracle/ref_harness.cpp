@@ -459,6 +459,8 @@ void dlref_model_init_uniform(void *h, unsigned seed, float bias, float lower, f
   m.Initialization__Uniform(bias, lower, upper);
 }
 
+// Initialization__Identity(bias) (identity.cpp:25-103)
+void dlref_model_init_identity(void *h, float bias) { static_cast<RefModel *>(h)->model.Initialization__Identity(bias); }
 // gaussian.seed(seed); Initialization__Glorot__Gaussian(bias) (glorot.cpp:110-222)
 void dlref_model_glorot_gaussian(void *h, unsigned seed, float bias) {
   Model &m = static_cast<RefModel *>(h)->model;

@@ -87,3 +87,10 @@ def test_gaussian_glorot_against_the_compiled_reference(net_factory, reference, 
     (mm, ms), (rm, rs) = M.get_moving(), R.get_moving()
     assert np.array_equal(mm, rm) and np.array_equal(ms, rs)
     assert not np.array_equal(M.get_parameters(), p0)
+    # Initialization__Identity (identity.cpp:25-103) on the same pair: zeros and the reference's ones
+    for m in (M, R):
+        m.set_parameters(p0)
+        m.init_identity(bias)
+    pi = M.get_parameters()
+    assert np.array_equal(pi, R.get_parameters())
+    assert set(np.unique(pi).tolist()) <= {0.0, 1.0, float(np.float32(bias))}
